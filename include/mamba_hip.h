@@ -1,0 +1,113 @@
+/*
+ * C ABI of libmamba_gfx950.so: hand-written HIP kernels (gfx950 / CDNA4) for
+ * Mamba's scan hot path.  Plain pointers and sizes only; no torch types.
+ *
+ * Conventions
+ *  - every pointer is a device pointer unless stated otherwise;
+ *  - the caller owns and allocates every buffer (outputs and workspaces);
+ *    the library never allocates or frees device memory;
+ *  - strides are in ELEMENTS of the tensor's dtype; the sequence (or the
+ *    innermost) dimension must have stride 1 where stated;
+ *  - kernels are launched on `stream` and never synchronise with the host;
+ *  - return value: 0 on success, a negative MAMBA_E_* code otherwise
+ *    (mamba_hip_strerror() gives the text).  Nothing throws.
+ */
+#ifndef MAMBA_HIP_H_
+#define MAMBA_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *mamba_stream_t; /* hipStream_t */
+
+enum {
+  MAMBA_OK = 0,
+  MAMBA_E_BADARG = -1,      /* null pointer / inconsistent sizes */
+  MAMBA_E_UNSUPPORTED = -2, /* valid request this build has no kernel for */
+  MAMBA_E_LAUNCH = -3       /* hipGetLastError() != hipSuccess after launch */
+};
+
+enum { MAMBA_F32 = 0, MAMBA_BF16 = 1, MAMBA_F16 = 2 };
+
+/* mamba_hip_query(what) */
+enum {
+  MAMBA_Q_ABI_VERSION = 0,
+  MAMBA_Q_SCAN_TILE = 1,      /* sequence positions per checkpoint tile of the Mamba-1 scan */
+  MAMBA_Q_MAX_DSTATE = 2,     /* largest d_state the Mamba-1 scan accepts */
+  MAMBA_Q_SSD_MAX_DSTATE = 3, /* largest d_state of the SSD kernels */
+  MAMBA_Q_SSD_MAX_HEADDIM = 4
+};
+
+int mamba_hip_query(int what);
+const char *mamba_hip_strerror(int code);
+
+/* Fills `nbytes` (multiple of 4) of device memory with zero using a kernel, so
+ * that it can be recorded into a HIP graph. */
+int mamba_hip_zero(void *ptr, int64_t nbytes, mamba_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * Mamba-1 selective scan.
+ * Replaces selective_scan_cuda.fwd / .bwd
+ * (reference csrc/selective_scan/selective_scan.cpp:226 and :338, params
+ * struct csrc/selective_scan/selective_scan.h:7 and :52).
+ *
+ *   delta' = softplus(delta + delta_bias)            (each part optional)
+ *   h[t,n] = exp(delta'[t] A[d,n]) h[t-1,n] + delta'[t] B[t,n] u[t]
+ *   y[t]   = sum_n C[t,n] h[t,n] + D[d] u[t]
+ *   out[t] = y[t] * silu(z[t])   (when z != NULL, else y[t])
+ *
+ * u, delta, z, out (and dout, du, ddelta, dz, out_z) are (batch, dim, seqlen)
+ * of `dtype`, seqlen stride 1.  B, C are (batch, ngroups, dstate, seqlen) of
+ * `dtype`, seqlen stride 1; channel d uses group d / (dim / ngroups).
+ * A is (dim, dstate) fp32 contiguous; D, delta_bias are (dim) fp32 or NULL.
+ *
+ * ckpt is (batch, dim, ntiles, dstate) fp32 contiguous with
+ * ntiles = ceil(seqlen / MAMBA_Q_SCAN_TILE): the state h after the last
+ * position of each tile.  ckpt[:, :, ntiles-1, :] is the final state.  The
+ * backward pass re-computes the states inside a tile from ckpt.
+ * ------------------------------------------------------------------------- */
+typedef struct MambaScanParams {
+  int32_t batch, dim, seqlen, dstate, ngroups;
+  int32_t dtype; /* MAMBA_F32 / MAMBA_BF16 / MAMBA_F16 */
+  int32_t delta_softplus;
+  int32_t reserved0;
+
+  const void *u, *delta, *A, *B, *C;
+  const void *D, *z, *delta_bias; /* nullable */
+  void *out;                      /* forward only */
+  float *ckpt;                    /* forward: written; backward: read */
+
+  int64_t u_bs, u_ds;         /* batch / dim stride */
+  int64_t delta_bs, delta_ds;
+  int64_t z_bs, z_ds;
+  int64_t out_bs, out_ds;
+  int64_t B_bs, B_gs, B_ns; /* batch / group / state stride */
+  int64_t C_bs, C_gs, C_ns;
+
+  /* ---- backward only (ignored by mamba1_scan_fwd) ---- */
+  const void *dout;
+  void *du, *ddelta;
+  void *dz;    /* required iff z != NULL; may be a strided view */
+  void *out_z; /* nullable: when set (and z != NULL) the gated output is re-computed into it */
+  /* fp32 accumulators.  dB32, dC32: (batch, ngroups, dstate, seqlen) contiguous,
+   * MUST be zero on entry (kernels add into them).  dA_part: (batch, dim, dstate),
+   * dD_part, ddelta_bias_part: (batch, dim) -- written (not accumulated), the
+   * caller sums them over batch. */
+  float *dB32, *dC32, *dA_part, *dD_part, *ddelta_bias_part;
+  int64_t dout_bs, dout_ds;
+  int64_t du_bs, du_ds;
+  int64_t ddelta_bs, ddelta_ds;
+  int64_t dz_bs, dz_ds;
+  int64_t outz_bs, outz_ds;
+} MambaScanParams;
+
+int mamba1_scan_fwd(const MambaScanParams *p, mamba_stream_t stream);
+int mamba1_scan_bwd(const MambaScanParams *p, mamba_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MAMBA_HIP_H_ */

@@ -1,0 +1,78 @@
+"""ctypes binding of libmamba_gfx950.so (the C ABI declared in include/mamba_hip.h).
+
+The library is the only compute backend: when it is missing, or a call returns
+an error code, a RuntimeError is raised.  There is no CPU or PyTorch fallback.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmamba_gfx950.so")
+
+MAMBA_F32, MAMBA_BF16, MAMBA_F16 = 0, 1, 2
+DTYPE_CODE = {torch.float32: MAMBA_F32, torch.bfloat16: MAMBA_BF16, torch.float16: MAMBA_F16}
+
+c_i32, c_i64, c_vp, c_f32 = ctypes.c_int32, ctypes.c_int64, ctypes.c_void_p, ctypes.c_float
+
+
+class MambaScanParams(ctypes.Structure):
+    _fields_ = (
+        [(n, c_i32) for n in ("batch", "dim", "seqlen", "dstate", "ngroups", "dtype", "delta_softplus", "reserved0")]
+        + [(n, c_vp) for n in ("u", "delta", "A", "B", "C", "D", "z", "delta_bias", "out", "ckpt")]
+        + [(n, c_i64) for n in ("u_bs", "u_ds", "delta_bs", "delta_ds", "z_bs", "z_ds", "out_bs", "out_ds",
+                                "B_bs", "B_gs", "B_ns", "C_bs", "C_gs", "C_ns")]
+        + [(n, c_vp) for n in ("dout", "du", "ddelta", "dz", "out_z", "dB32", "dC32", "dA_part", "dD_part",
+                               "ddelta_bias_part")]
+        + [(n, c_i64) for n in ("dout_bs", "dout_ds", "du_bs", "du_ds", "ddelta_bs", "ddelta_ds", "dz_bs", "dz_ds",
+                                "outz_bs", "outz_ds")]
+    )
+
+
+_lib = None
+
+
+def load():
+    """Loads the shared library once; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -m mamba_amd.build` (hipcc, gfx950). "
+            "mamba_amd has no fallback backend."
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    lib.mamba_hip_query.argtypes = [ctypes.c_int]
+    lib.mamba_hip_query.restype = ctypes.c_int
+    lib.mamba_hip_strerror.argtypes = [ctypes.c_int]
+    lib.mamba_hip_strerror.restype = ctypes.c_char_p
+    lib.mamba_hip_zero.argtypes = [c_vp, c_i64, c_vp]
+    lib.mamba_hip_zero.restype = ctypes.c_int
+    for name in ("mamba1_scan_fwd", "mamba1_scan_bwd"):
+        fn = getattr(lib, name)
+        fn.argtypes = [ctypes.POINTER(MambaScanParams), c_vp]
+        fn.restype = ctypes.c_int
+    _lib = lib
+    return lib
+
+
+def check(rc, what):
+    if rc != 0:
+        msg = load().mamba_hip_strerror(rc).decode()
+        raise RuntimeError(f"{what} failed: {msg} (code {rc})")
+
+
+def ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def current_stream(device):
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def require_gpu(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("mamba_amd kernels need GPU tensors; there is no CPU fallback")

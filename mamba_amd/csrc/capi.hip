@@ -1,0 +1,42 @@
+// Library-level entry points of libmamba_gfx950.so: queries, error strings and
+// a graph-capturable zero fill.
+#include "common.hpp"
+
+namespace {
+__global__ __launch_bounds__(256) void zero_kernel(uint32_t *p, int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = 0u;
+}
+}  // namespace
+
+extern "C" int mamba_hip_query(int what) {
+  switch (what) {
+    case MAMBA_Q_ABI_VERSION: return 1;
+    case MAMBA_Q_SCAN_TILE: return 512;
+    case MAMBA_Q_MAX_DSTATE: return 256;
+    case MAMBA_Q_SSD_MAX_DSTATE: return 256;
+    case MAMBA_Q_SSD_MAX_HEADDIM: return 256;
+    default: return MAMBA_E_BADARG;
+  }
+}
+
+extern "C" const char *mamba_hip_strerror(int code) {
+  switch (code) {
+    case MAMBA_OK: return "success";
+    case MAMBA_E_BADARG: return "bad argument (null pointer or inconsistent sizes)";
+    case MAMBA_E_UNSUPPORTED: return "unsupported shape or dtype for this build";
+    case MAMBA_E_LAUNCH: return "kernel launch failed";
+    default: return "unknown error code";
+  }
+}
+
+extern "C" int mamba_hip_zero(void *ptr, int64_t nbytes, mamba_stream_t stream) {
+  if (nbytes == 0) return MAMBA_OK;
+  if (!ptr || nbytes < 0 || (nbytes & 3) || (reinterpret_cast<uintptr_t>(ptr) & 3)) return MAMBA_E_BADARG;
+  const int64_t n = nbytes / 4;
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(zero_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<uint32_t *>(ptr), n);
+  return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
+}

@@ -1,0 +1,209 @@
+// Device-side helpers shared by the gfx950 kernels: dtype load/store, fast
+// transcendental wrappers, DPP wave64 primitives.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/mamba_hip.h"
+
+#define DEVI __device__ __forceinline__
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+struct bf16_t { uint16_t v; };
+struct f16_t { uint16_t v; };
+
+// ---------------------------------------------------------------- conversions
+DEVI float bf16_lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+DEVI float bf16_hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+DEVI uint32_t f32_to_bf16_bits(float x) {
+  __bf16 b = (__bf16)x;  // round-to-nearest-even; v_cvt_pk_bf16_f32 on gfx950
+  return (uint32_t)__builtin_bit_cast(uint16_t, b);
+}
+DEVI uint32_t pack_bf16(float lo, float hi) {
+  typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+  bf2 r;
+  r.x = (__bf16)lo;
+  r.y = (__bf16)hi;
+  return __builtin_bit_cast(uint32_t, r);
+}
+DEVI float f16_lo(uint32_t w) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu)); }
+DEVI float f16_hi(uint32_t w) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16)); }
+DEVI uint32_t pack_f16(float lo, float hi) {
+  uint32_t a = __builtin_bit_cast(uint16_t, (_Float16)lo);
+  uint32_t b = __builtin_bit_cast(uint16_t, (_Float16)hi);
+  return a | (b << 16);
+}
+
+template <typename T> struct DT;
+template <> struct DT<float> { static constexpr int id = MAMBA_F32; };
+template <> struct DT<bf16_t> { static constexpr int id = MAMBA_BF16; };
+template <> struct DT<f16_t> { static constexpr int id = MAMBA_F16; };
+
+template <typename T> DEVI float ld1(const T *p);
+template <> DEVI float ld1<float>(const float *p) { return *p; }
+template <> DEVI float ld1<bf16_t>(const bf16_t *p) { return __builtin_bit_cast(float, (uint32_t)p->v << 16); }
+template <> DEVI float ld1<f16_t>(const f16_t *p) { return (float)__builtin_bit_cast(_Float16, p->v); }
+
+template <typename T> DEVI void st1(T *p, float x);
+template <> DEVI void st1<float>(float *p, float x) { *p = x; }
+template <> DEVI void st1<bf16_t>(bf16_t *p, float x) { p->v = (uint16_t)f32_to_bf16_bits(x); }
+template <> DEVI void st1<f16_t>(f16_t *p, float x) { p->v = __builtin_bit_cast(uint16_t, (_Float16)x); }
+
+// 8 consecutive elements; p must be 16-byte aligned.
+template <typename T> DEVI void ld8(const T *p, float (&o)[8]);
+template <> DEVI void ld8<float>(const float *p, float (&o)[8]) {
+  f32x4 a = *reinterpret_cast<const f32x4 *>(p);
+  f32x4 b = *reinterpret_cast<const f32x4 *>(p + 4);
+  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+  o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+}
+template <> DEVI void ld8<bf16_t>(const bf16_t *p, float (&o)[8]) {
+  u32x4 a = *reinterpret_cast<const u32x4 *>(p);
+  o[0] = bf16_lo(a.x); o[1] = bf16_hi(a.x); o[2] = bf16_lo(a.y); o[3] = bf16_hi(a.y);
+  o[4] = bf16_lo(a.z); o[5] = bf16_hi(a.z); o[6] = bf16_lo(a.w); o[7] = bf16_hi(a.w);
+}
+template <> DEVI void ld8<f16_t>(const f16_t *p, float (&o)[8]) {
+  u32x4 a = *reinterpret_cast<const u32x4 *>(p);
+  o[0] = f16_lo(a.x); o[1] = f16_hi(a.x); o[2] = f16_lo(a.y); o[3] = f16_hi(a.y);
+  o[4] = f16_lo(a.z); o[5] = f16_hi(a.z); o[6] = f16_lo(a.w); o[7] = f16_hi(a.w);
+}
+template <typename T> DEVI void st8(T *p, const float (&v)[8]);
+template <> DEVI void st8<float>(float *p, const float (&v)[8]) {
+  f32x4 a = {v[0], v[1], v[2], v[3]}, b = {v[4], v[5], v[6], v[7]};
+  *reinterpret_cast<f32x4 *>(p) = a;
+  *reinterpret_cast<f32x4 *>(p + 4) = b;
+}
+template <> DEVI void st8<bf16_t>(bf16_t *p, const float (&v)[8]) {
+  u32x4 a = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7])};
+  *reinterpret_cast<u32x4 *>(p) = a;
+}
+template <> DEVI void st8<f16_t>(f16_t *p, const float (&v)[8]) {
+  u32x4 a = {pack_f16(v[0], v[1]), pack_f16(v[2], v[3]), pack_f16(v[4], v[5]), pack_f16(v[6], v[7])};
+  *reinterpret_cast<u32x4 *>(p) = a;
+}
+
+// 8 elements starting at p[0], of which only the first `nvalid` (0..8) exist;
+// the rest read as `fill`.  VEC: all-or-nothing 16-byte path.
+template <typename T, bool VEC> DEVI void ld8_guard(const T *p, int nvalid, float fill, float (&o)[8]) {
+  if (VEC) {
+    if (nvalid >= 8) {
+      ld8<T>(p, o);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) o[i] = fill;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = (i < nvalid) ? ld1<T>(p + i) : fill;
+  }
+}
+template <typename T, bool VEC> DEVI void st8_guard(T *p, int nvalid, const float (&v)[8]) {
+  if (VEC) {
+    if (nvalid >= 8) st8<T>(p, v);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (i < nvalid) st1<T>(p + i, v[i]);
+  }
+}
+
+// ------------------------------------------------------------------- math
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+DEVI float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }          // v_exp_f32
+DEVI float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * kLog2e); }
+DEVI float fast_log(float x) { return __builtin_amdgcn_logf(x) * kLn2; }     // v_log_f32
+DEVI float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+// softplus with the reference's threshold: x <= 20 ? log1p(exp(x)) : x.
+// log1p(e) for small e is evaluated by its series so that tiny step sizes keep
+// full relative precision.
+DEVI float softplus_f(float x) {
+  float e = fast_exp(fminf(x, 20.f));
+  float big = fast_log(1.f + e);
+  float small = e * (1.f - e * (0.5f - e * (0.33333333f - 0.25f * e)));
+  float r = (e < 0.03f) ? small : big;
+  return x <= 20.f ? r : x;
+}
+DEVI float sigmoid_f(float x) { return fast_rcp(1.f + fast_exp(-x)); }
+
+// ------------------------------------------------------------------- DPP
+// dpp_ctrl encodings of the GFX9 family.
+enum : int {
+  DPP_ROW_SHL = 0x100,
+  DPP_ROW_SHR = 0x110,
+  DPP_WAVE_SHL1 = 0x130,
+  DPP_WAVE_SHR1 = 0x138,
+  DPP_ROW_BCAST15 = 0x142,
+  DPP_ROW_BCAST31 = 0x143
+};
+
+// Lanes whose DPP source does not exist (or whose row is masked off) get `old`.
+template <int CTRL, int ROW_MASK = 0xf> DEVI float dpp_f(float old, float src) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, src), CTRL, ROW_MASK,
+                                         0xf, false));
+}
+DEVI float readlane_f(float x, int lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), lane));
+}
+
+// Inclusive scan over the 64 lanes (lane 0 first) of first-order recurrence
+// segments (a, b) meaning h_out = a * h_in + b.
+DEVI void wave_scan_fwd(float &a, float &b) {
+#define MAMBA_STEP(CTRL, MASK)                   \
+  {                                              \
+    float bp = dpp_f<CTRL, MASK>(0.f, b);        \
+    float ap = dpp_f<CTRL, MASK>(1.f, a);        \
+    b = __builtin_fmaf(a, bp, b);                \
+    a = a * ap;                                  \
+  }
+  MAMBA_STEP(DPP_ROW_SHR + 1, 0xf)
+  MAMBA_STEP(DPP_ROW_SHR + 2, 0xf)
+  MAMBA_STEP(DPP_ROW_SHR + 4, 0xf)
+  MAMBA_STEP(DPP_ROW_SHR + 8, 0xf)
+  MAMBA_STEP(DPP_ROW_BCAST15, 0xa)
+  MAMBA_STEP(DPP_ROW_BCAST31, 0xc)
+#undef MAMBA_STEP
+}
+
+// Inclusive scan in the other direction (lane 63 first): on return lane l
+// holds the composition of lanes l..63, again as h_out = a * h_in + b where
+// h_in enters after lane 63.
+DEVI void wave_scan_rev(float &a, float &b, int lane) {
+#define MAMBA_STEP(N)                                      \
+  {                                                        \
+    float bp = dpp_f<DPP_ROW_SHL + N>(0.f, b);             \
+    float ap = dpp_f<DPP_ROW_SHL + N>(1.f, a);             \
+    b = __builtin_fmaf(a, bp, b);                          \
+    a = a * ap;                                            \
+  }
+  MAMBA_STEP(1)
+  MAMBA_STEP(2)
+  MAMBA_STEP(4)
+  MAMBA_STEP(8)
+#undef MAMBA_STEP
+  // rows 1..3 as whole segments, taken from their first lanes
+  float a1 = readlane_f(a, 16), b1 = readlane_f(b, 16);
+  float a2 = readlane_f(a, 32), b2 = readlane_f(b, 32);
+  float a3 = readlane_f(a, 48), b3 = readlane_f(b, 48);
+  // segment that follows each row: row2 <- row3, row1 <- row2.row3, row0 <- row1.row2.row3
+  float a23 = a2 * a3, b23 = __builtin_fmaf(a2, b3, b2);
+  float a123 = a1 * a23, b123 = __builtin_fmaf(a1, b23, b1);
+  int row = lane >> 4;
+  float an = row == 0 ? a123 : (row == 1 ? a23 : (row == 2 ? a3 : 1.f));
+  float bn = row == 0 ? b123 : (row == 1 ? b23 : (row == 2 ? b3 : 0.f));
+  b = __builtin_fmaf(a, bn, b);
+  a = a * an;
+}
+
+DEVI float wave_sum(float x) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) x += __shfl_xor(x, off, 64);
+  return x;
+}

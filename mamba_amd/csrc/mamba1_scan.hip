@@ -1,0 +1,496 @@
+// Mamba-1 selective scan, forward and backward, for gfx950 (wave64).
+//
+// Work decomposition
+//   * a wave owns R channels of one (batch, group); its 64 lanes hold 64
+//     consecutive 8-step segments of the sequence, i.e. one 512-step tile per
+//     pass.  Lane l loads its 8 items of u/delta/z with one 16-byte access.
+//   * the NW waves of a workgroup walk the tiles together and share the B and
+//     C rows of the tile, staged once per tile in LDS as fp32.
+//   * per state n: an 8-step in-register recurrence per lane, a DPP scan of
+//     the (decay, value) pairs across the 64 lanes, and a carry from the
+//     previous tile kept in LDS.
+//   * the state after every tile is written to `ckpt`; the backward pass walks
+//     the tiles in reverse, restarts each tile from ckpt, and runs the adjoint
+//     recurrence with a lane-reversed scan.  dB/dC are reduced over the
+//     channels of the workgroup in LDS and added to global fp32 buffers once
+//     per tile.
+#include "common.hpp"
+
+namespace {
+
+constexpr int KI = 8;           // items per lane
+constexpr int TILE = 64 * KI;   // sequence positions per tile
+constexpr int NB16 = 16;        // states staged per LDS block
+constexpr int BC_FLOATS = NB16 * TILE;        // one staged tensor
+constexpr int ACC_PITCH = 9;                  // items per lane, padded (bank spread)
+constexpr int ACC_FLOATS = NB16 * 64 * ACC_PITCH;
+constexpr int MAX_DSTATE = 256;
+
+// B or C rows n0..n0+15 of the tile starting at t0 -> LDS as fp32, laid out
+// [n][half][lane][4] so that a lane reads its 8 items with two conflict-free
+// 16-byte LDS loads.
+template <typename T, bool VEC, int NTHREADS>
+DEVI void stage_bc(float *Bs, float *Cs, const T *Bg, int64_t B_ns, const T *Cg, int64_t C_ns, int n0, int N, int t0,
+                   int L, int tid) {
+  for (int unit = tid; unit < 2 * NB16 * 64; unit += NTHREADS) {
+    const int which = unit >> 10, n = (unit >> 6) & 15, j = unit & 63;
+    const int t = t0 + KI * j;
+    const T *src = (which ? Cg + (int64_t)(n0 + n) * C_ns : Bg + (int64_t)(n0 + n) * B_ns) + t;
+    int nvalid = (n0 + n < N) ? min(max(L - t, 0), KI) : 0;
+    float v[8];
+    ld8_guard<T, VEC>(src, nvalid, 0.f, v);
+    float *dst = (which ? Cs : Bs) + n * TILE + j * 4;
+    f32x4 lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
+    *reinterpret_cast<f32x4 *>(dst) = lo;
+    *reinterpret_cast<f32x4 *>(dst + 256) = hi;
+  }
+}
+
+DEVI void lds_ld8(const float *base, int lane, float (&o)[8]) {
+  f32x4 lo = *reinterpret_cast<const f32x4 *>(base + lane * 4);
+  f32x4 hi = *reinterpret_cast<const f32x4 *>(base + 256 + lane * 4);
+  o[0] = lo.x; o[1] = lo.y; o[2] = lo.z; o[3] = lo.w;
+  o[4] = hi.x; o[5] = hi.y; o[6] = hi.z; o[7] = hi.w;
+}
+
+// ------------------------------------------------------------------ forward
+template <typename T, int NW, int R, bool VEC>
+__global__ __launch_bounds__(NW * 64) void scan_fwd_kernel(const MambaScanParams p) {
+  extern __shared__ __align__(16) float smem[];
+  const int N = p.dstate, L = p.seqlen;
+  const int NBLK = (N + NB16 - 1) / NB16, NP = NBLK * NB16;
+  float *Bs = smem;
+  float *Cs = Bs + BC_FLOATS;
+  float *A2s = Cs + BC_FLOATS;       // [NW*R][NP]  A * log2(e)
+  float *hcar = A2s + NW * R * NP;   // [NW*R][NP]  state carried across tiles
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int Dg = p.dim / p.ngroups;
+  const int cblocks = (Dg + NW * R - 1) / (NW * R);
+  const int g = blockIdx.x / cblocks, cb = blockIdx.x % cblocks;
+  const int b = blockIdx.y;
+  const int dbase = g * Dg + cb * NW * R + wave * R;
+  const int dend = (g + 1) * Dg;
+  const int ntiles = (L + TILE - 1) / TILE;
+
+  const T *Bg = (const T *)p.B + b * p.B_bs + g * p.B_gs;
+  const T *Cg = (const T *)p.C + b * p.C_bs + g * p.C_gs;
+  const float *Ag = (const float *)p.A;
+
+  for (int i = lane; i < R * NP; i += 64) {
+    const int r = i / NP, n = i % NP, d = dbase + r;
+    A2s[wave * R * NP + i] = (d < dend && n < N) ? Ag[(int64_t)d * N + n] * kLog2e : 0.f;
+    hcar[wave * R * NP + i] = 0.f;
+  }
+
+  for (int tile = 0; tile < ntiles; ++tile) {
+    const int t0 = tile * TILE, tl = t0 + lane * KI;
+    const int nvalid = min(max(L - tl, 0), KI);
+    for (int r = 0; r < R; ++r) {
+      const int d = dbase + r;
+      const bool valid = d < dend;
+      float u[8], dl[8], du[8], y[8];
+      if (valid) {
+        ld8_guard<T, VEC>((const T *)p.u + b * p.u_bs + d * p.u_ds + tl, nvalid, 0.f, u);
+        ld8_guard<T, VEC>((const T *)p.delta + b * p.delta_bs + d * p.delta_ds + tl, nvalid, 0.f, dl);
+        const float bias = p.delta_bias ? ((const float *)p.delta_bias)[d] : 0.f;
+#pragma unroll
+        for (int i = 0; i < KI; ++i) {
+          float x = dl[i] + bias;
+          if (p.delta_softplus) x = softplus_f(x);
+          dl[i] = (i < nvalid) ? x : 0.f;
+          du[i] = dl[i] * u[i];
+          y[i] = 0.f;
+        }
+      }
+      for (int nb = 0; nb < NBLK; ++nb) {
+        if (NBLK > 1 || r == 0) {
+          __syncthreads();
+          stage_bc<T, VEC, NW * 64>(Bs, Cs, Bg, p.B_ns, Cg, p.C_ns, nb * NB16, N, t0, L, tid);
+          __syncthreads();
+        }
+        if (valid) {
+          const float *A2row = A2s + (wave * R + r) * NP + nb * NB16;
+          float *hrow = hcar + (wave * R + r) * NP + nb * NB16;
+          const int nmax = min(NB16, N - nb * NB16);
+#pragma unroll 2
+          for (int n = 0; n < nmax; ++n) {
+            const float A2 = A2row[n];
+            const float hc = hrow[n];
+            float Bv[8], Cv[8], a[8], hh[8];
+            lds_ld8(Bs + n * TILE, lane, Bv);
+            lds_ld8(Cs + n * TILE, lane, Cv);
+#pragma unroll
+            for (int i = 0; i < KI; ++i) a[i] = fast_exp2(dl[i] * A2);
+            hh[0] = du[0] * Bv[0];
+#pragma unroll
+            for (int i = 1; i < KI; ++i) {
+              hh[i] = __builtin_fmaf(a[i], hh[i - 1], du[i] * Bv[i]);
+              a[i] = a[i] * a[i - 1];  // cumulative decay inside the lane
+            }
+            float sa = a[KI - 1], sb = hh[KI - 1];
+            wave_scan_fwd(sa, sb);
+            const float hend = __builtin_fmaf(sa, hc, sb);  // state after this lane's last item
+            const float hx = dpp_f<DPP_WAVE_SHR1>(hc, hend);  // state entering this lane
+            if (lane == 63) hrow[n] = hend;
+#pragma unroll
+            for (int i = 0; i < KI; ++i) y[i] = __builtin_fmaf(__builtin_fmaf(a[i], hx, hh[i]), Cv[i], y[i]);
+          }
+        }
+      }
+      if (valid) {
+        if (p.D) {
+          const float Dd = ((const float *)p.D)[d];
+#pragma unroll
+          for (int i = 0; i < KI; ++i) y[i] = __builtin_fmaf(Dd, u[i], y[i]);
+        }
+        if (p.z) {
+          float z[8];
+          ld8_guard<T, VEC>((const T *)p.z + b * p.z_bs + d * p.z_ds + tl, nvalid, 0.f, z);
+#pragma unroll
+          for (int i = 0; i < KI; ++i) y[i] *= z[i] * sigmoid_f(z[i]);
+        }
+        st8_guard<T, VEC>((T *)p.out + b * p.out_bs + d * p.out_ds + tl, nvalid, y);
+        float *ck = p.ckpt + (((int64_t)b * p.dim + d) * ntiles + tile) * N;
+        const float *hfin = hcar + (wave * R + r) * NP;
+        for (int n = lane; n < N; n += 64) ck[n] = hfin[n];
+      }
+    }
+  }
+}
+
+// ----------------------------------------------------------------- backward
+template <typename T, int NW, int R, bool VEC>
+__global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams p) {
+  extern __shared__ __align__(16) float smem[];
+  const int N = p.dstate, L = p.seqlen;
+  const int NBLK = (N + NB16 - 1) / NB16, NP = NBLK * NB16;
+  constexpr int WR = NW * R;
+  float *Bs = smem;
+  float *Cs = Bs + BC_FLOATS;
+  float *dBs = Cs + BC_FLOATS;        // [16][64][9]
+  float *dCs = dBs + ACC_FLOATS;
+  float *A1s = dCs + ACC_FLOATS;      // [WR][NP] A
+  float *hcar = A1s + WR * NP;        // state entering the tile (from ckpt)
+  float *gcar = hcar + WR * NP;       // adjoint at the first position of the following tile
+  float *anx = gcar + WR * NP;        // decay at the first position of the following tile
+  float *dAacc = anx + WR * NP;       // [WR][NP]
+  float *dDacc = dAacc + WR * NP;     // [WR]
+  float *dbacc = dDacc + WR;          // [WR]
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int Dg = p.dim / p.ngroups;
+  const int cblocks = (Dg + WR - 1) / WR;
+  const int g = blockIdx.x / cblocks, cb = blockIdx.x % cblocks;
+  const int b = blockIdx.y;
+  const int dbase = g * Dg + cb * WR + wave * R;
+  const int dend = (g + 1) * Dg;
+  const int ntiles = (L + TILE - 1) / TILE;
+  const bool has_z = p.z != nullptr;
+
+  const T *Bg = (const T *)p.B + b * p.B_bs + g * p.B_gs;
+  const T *Cg = (const T *)p.C + b * p.C_bs + g * p.C_gs;
+  const float *Ag = (const float *)p.A;
+  float *dBg = p.dB32 + ((int64_t)b * p.ngroups + g) * N * L;
+  float *dCg = p.dC32 + ((int64_t)b * p.ngroups + g) * N * L;
+
+  for (int i = lane; i < R * NP; i += 64) {
+    const int r = i / NP, n = i % NP, d = dbase + r;
+    const int o = wave * R * NP + i;
+    A1s[o] = (d < dend && n < N) ? Ag[(int64_t)d * N + n] : 0.f;
+    gcar[o] = 0.f;
+    anx[o] = 0.f;
+    dAacc[o] = 0.f;
+  }
+  if (lane < R) {
+    dDacc[wave * R + lane] = 0.f;
+    dbacc[wave * R + lane] = 0.f;
+  }
+
+  for (int tile = ntiles - 1; tile >= 0; --tile) {
+    const int t0 = tile * TILE, tl = t0 + lane * KI;
+    const int nvalid = min(max(L - tl, 0), KI);
+    for (int r = 0; r < R; ++r) {
+      const int d = dbase + r;
+      const bool valid = d < dend;
+      const int row = wave * R + r;
+      float u[8], dl[8], du[8], dy[8], acc[8], dd[8], y[8];
+      float Dd = 0.f;
+      if (valid) {
+        Dd = p.D ? ((const float *)p.D)[d] : 0.f;
+        ld8_guard<T, VEC>((const T *)p.u + b * p.u_bs + d * p.u_ds + tl, nvalid, 0.f, u);
+        ld8_guard<T, VEC>((const T *)p.delta + b * p.delta_bs + d * p.delta_ds + tl, nvalid, 0.f, dl);
+        ld8_guard<T, VEC>((const T *)p.dout + b * p.dout_bs + d * p.dout_ds + tl, nvalid, 0.f, dy);
+        const float bias = p.delta_bias ? ((const float *)p.delta_bias)[d] : 0.f;
+        if (has_z) {
+          float z[8];
+          ld8_guard<T, VEC>((const T *)p.z + b * p.z_bs + d * p.z_ds + tl, nvalid, 0.f, z);
+#pragma unroll
+          for (int i = 0; i < KI; ++i) dy[i] *= z[i] * sigmoid_f(z[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < KI; ++i) {
+          float x = dl[i] + bias;
+          if (p.delta_softplus) x = softplus_f(x);
+          dl[i] = (i < nvalid) ? x : 0.f;
+          du[i] = dl[i] * u[i];
+          acc[i] = 0.f;
+          dd[i] = 0.f;
+          y[i] = 0.f;
+        }
+        // state entering this tile
+        for (int n = lane; n < NP; n += 64) {
+          float v = 0.f;
+          if (tile > 0 && n < N) v = p.ckpt[(((int64_t)b * p.dim + d) * ntiles + tile - 1) * N + n];
+          hcar[row * NP + n] = v;
+        }
+      }
+      for (int nb = 0; nb < NBLK; ++nb) {
+        if (NBLK > 1 || r == 0) {
+          __syncthreads();
+          stage_bc<T, VEC, NW * 64>(Bs, Cs, Bg, p.B_ns, Cg, p.C_ns, nb * NB16, N, t0, L, tid);
+          for (int i = tid; i < 2 * ACC_FLOATS; i += NW * 64) dBs[i] = 0.f;  // dBs and dCs are adjacent
+          __syncthreads();
+        }
+        if (valid) {
+          const float *A1row = A1s + row * NP + nb * NB16;
+          const float *hrow = hcar + row * NP + nb * NB16;
+          float *grow = gcar + row * NP + nb * NB16;
+          float *arow = anx + row * NP + nb * NB16;
+          float *dArow = dAacc + row * NP + nb * NB16;
+          const int nmax = min(NB16, N - nb * NB16);
+          for (int n = 0; n < nmax; ++n) {
+            const float A1 = A1row[n], A2 = A1 * kLog2e;
+            const float hc = hrow[n], gc = grow[n], an = arow[n];
+            float Bv[8], Cv[8], a[8], ac[8], bb[8], h[8];
+            lds_ld8(Bs + n * TILE, lane, Bv);
+            lds_ld8(Cs + n * TILE, lane, Cv);
+#pragma unroll
+            for (int i = 0; i < KI; ++i) {
+              a[i] = fast_exp2(dl[i] * A2);
+              bb[i] = du[i] * Bv[i];
+            }
+            h[0] = bb[0];
+            ac[0] = a[0];
+#pragma unroll
+            for (int i = 1; i < KI; ++i) {
+              h[i] = __builtin_fmaf(a[i], h[i - 1], bb[i]);
+              ac[i] = ac[i - 1] * a[i];
+            }
+            float sa = ac[KI - 1], sb = h[KI - 1];
+            wave_scan_fwd(sa, sb);
+            const float hend = __builtin_fmaf(sa, hc, sb);
+            const float hx = dpp_f<DPP_WAVE_SHR1>(hc, hend);
+#pragma unroll
+            for (int i = 0; i < KI; ++i) h[i] = __builtin_fmaf(ac[i], hx, h[i]);  // true states
+            if (has_z) {
+#pragma unroll
+              for (int i = 0; i < KI; ++i) y[i] = __builtin_fmaf(h[i], Cv[i], y[i]);
+            }
+            // adjoint recurrence g[t] = dy[t] C[t] + a[t+1] g[t+1]
+            const float a_next_lane = dpp_f<DPP_WAVE_SHL1>(an, a[0]);
+            float gg[8], ar[8];
+            gg[KI - 1] = dy[KI - 1] * Cv[KI - 1];
+            ar[KI - 1] = a_next_lane;
+#pragma unroll
+            for (int i = KI - 2; i >= 0; --i) {
+              gg[i] = __builtin_fmaf(a[i + 1], gg[i + 1], dy[i] * Cv[i]);
+              ar[i] = ar[i + 1] * a[i + 1];
+            }
+            float ra = ar[0], rb = gg[0];
+            wave_scan_rev(ra, rb, lane);
+            const float gfirst = __builtin_fmaf(ra, gc, rb);         // adjoint at this lane's first item
+            const float gx = dpp_f<DPP_WAVE_SHL1>(gc, gfirst);       // ... at the next lane's first item
+            if (lane == 0) {
+              grow[n] = gfirst;
+              arow[n] = a[0];
+            }
+            float dAp = 0.f;
+            float *dBl = dBs + (n * 64 + lane) * ACC_PITCH;
+            float *dCl = dCs + (n * 64 + lane) * ACC_PITCH;
+#pragma unroll
+            for (int i = 0; i < KI; ++i) {
+              const float gi = __builtin_fmaf(ar[i], gx, gg[i]);
+              __hip_atomic_fetch_add(dCl + i, dy[i] * h[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+              __hip_atomic_fetch_add(dBl + i, gi * du[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+              acc[i] = __builtin_fmaf(gi, Bv[i], acc[i]);
+              const float w = gi * (h[i] - bb[i]);  // g * a * h[t-1]
+              dd[i] = __builtin_fmaf(A1, w, dd[i]);
+              dAp = __builtin_fmaf(dl[i], w, dAp);
+            }
+            dAp += dpp_f<DPP_ROW_SHR + 1>(0.f, dAp);
+            dAp += dpp_f<DPP_ROW_SHR + 2>(0.f, dAp);
+            dAp += dpp_f<DPP_ROW_SHR + 4>(0.f, dAp);
+            dAp += dpp_f<DPP_ROW_SHR + 8>(0.f, dAp);
+            if ((lane & 15) == 15)
+              __hip_atomic_fetch_add(dArow + n, dAp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          }
+        }
+        if (NBLK > 1 || r == R - 1) {
+          __syncthreads();
+          const int n0 = nb * NB16;
+          for (int i = tid; i < 2 * NB16 * TILE; i += NW * 64) {
+            const int which = i >> 13, n = (i >> 9) & 15, t = i & (TILE - 1);
+            const float v = (which ? dCs : dBs)[(n * 64 + (t >> 3)) * ACC_PITCH + (t & 7)];
+            if (n0 + n < N && t0 + t < L) unsafeAtomicAdd((which ? dCg : dBg) + (int64_t)(n0 + n) * L + t0 + t, v);
+          }
+        }
+      }
+      if (valid) {
+        float draw[8], o[8];
+        ld8_guard<T, VEC>((const T *)p.delta + b * p.delta_bs + d * p.delta_ds + tl, nvalid, 0.f, draw);
+        const float bias = p.delta_bias ? ((const float *)p.delta_bias)[d] : 0.f;
+        float dbs = 0.f, dDs = 0.f;
+#pragma unroll
+        for (int i = 0; i < KI; ++i) o[i] = __builtin_fmaf(dl[i], acc[i], Dd * dy[i]);
+        st8_guard<T, VEC>((T *)p.du + b * p.du_bs + d * p.du_ds + tl, nvalid, o);
+#pragma unroll
+        for (int i = 0; i < KI; ++i) {
+          const float x = draw[i] + bias;
+          float gd = __builtin_fmaf(u[i], acc[i], dd[i]);
+          if (p.delta_softplus && x <= 20.f) gd *= sigmoid_f(x);
+          gd = (i < nvalid) ? gd : 0.f;
+          o[i] = gd;
+          dbs += gd;
+          dDs = __builtin_fmaf(dy[i], u[i], dDs);
+        }
+        st8_guard<T, VEC>((T *)p.ddelta + b * p.ddelta_bs + d * p.ddelta_ds + tl, nvalid, o);
+        if (has_z) {
+          float z[8], dout[8], oz[8];
+          ld8_guard<T, VEC>((const T *)p.z + b * p.z_bs + d * p.z_ds + tl, nvalid, 0.f, z);
+          ld8_guard<T, VEC>((const T *)p.dout + b * p.dout_bs + d * p.dout_ds + tl, nvalid, 0.f, dout);
+#pragma unroll
+          for (int i = 0; i < KI; ++i) {
+            const float yf = __builtin_fmaf(Dd, u[i], y[i]);
+            const float s = sigmoid_f(z[i]);
+            o[i] = dout[i] * yf * s * (1.f + z[i] * (1.f - s));
+            oz[i] = yf * z[i] * s;
+          }
+          st8_guard<T, VEC>((T *)p.dz + b * p.dz_bs + d * p.dz_ds + tl, nvalid, o);
+          if (p.out_z) st8_guard<T, VEC>((T *)p.out_z + b * p.outz_bs + d * p.outz_ds + tl, nvalid, oz);
+        }
+        dbs = wave_sum(dbs);
+        dDs = wave_sum(dDs);
+        if (lane == 0) {
+          dbacc[row] += dbs;
+          dDacc[row] += dDs;
+        }
+      }
+    }
+  }
+  // per-(batch, channel) partial sums; the caller reduces over batch
+  for (int r = 0; r < R; ++r) {
+    const int d = dbase + r;
+    if (d >= dend) continue;
+    const int row = wave * R + r;
+    for (int n = lane; n < N; n += 64) p.dA_part[((int64_t)b * p.dim + d) * N + n] = dAacc[row * NP + n];
+    if (lane == 0) {
+      p.dD_part[(int64_t)b * p.dim + d] = dDacc[row];
+      p.ddelta_bias_part[(int64_t)b * p.dim + d] = dbacc[row];
+    }
+  }
+}
+
+// ------------------------------------------------------------------ launch
+inline bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
+
+struct Cfg {
+  int nw, r;
+};
+
+inline size_t fwd_lds(int nw, int r, int np) { return sizeof(float) * (2 * BC_FLOATS + 2 * nw * r * np); }
+inline size_t bwd_lds(int nw, int r, int np) {
+  return sizeof(float) * (2 * BC_FLOATS + 2 * ACC_FLOATS + 5 * nw * r * np + 2 * nw * r);
+}
+
+template <typename KernelT>
+int launch(KernelT kernel, const MambaScanParams &p, int nw, int r, size_t lds, hipStream_t stream) {
+  const int Dg = p.dim / p.ngroups;
+  const int cblocks = (Dg + nw * r - 1) / (nw * r);
+  if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                          (int)lds) != hipSuccess) {
+    (void)hipGetLastError();
+    return MAMBA_E_LAUNCH;
+  }
+  dim3 grid(p.ngroups * cblocks, p.batch), block(nw * 64);
+  hipLaunchKernelGGL(kernel, grid, block, lds, stream, p);
+  return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
+}
+
+int check_common(const MambaScanParams *p) {
+  if (!p || !p->u || !p->delta || !p->A || !p->B || !p->C || !p->ckpt) return MAMBA_E_BADARG;
+  if (p->batch <= 0 || p->dim <= 0 || p->seqlen <= 0 || p->dstate <= 0 || p->ngroups <= 0) return MAMBA_E_BADARG;
+  if (p->dim % p->ngroups != 0) return MAMBA_E_BADARG;
+  if (p->batch > 65535) return MAMBA_E_UNSUPPORTED;
+  if (p->dstate > MAX_DSTATE) return MAMBA_E_UNSUPPORTED;
+  if (p->dtype != MAMBA_F32 && p->dtype != MAMBA_BF16 && p->dtype != MAMBA_F16) return MAMBA_E_BADARG;
+  return MAMBA_OK;
+}
+
+// 16-byte accesses need every row start aligned and whole 8-item groups.
+bool vec_ok(const MambaScanParams &p, bool bwd) {
+  const int es = p.dtype == MAMBA_F32 ? 4 : 2;
+  const int64_t m = 16 / es;
+  auto ok = [&](const void *ptr, int64_t s0, int64_t s1) { return !ptr || (aligned16(ptr) && s0 % m == 0 && s1 % m == 0); };
+  if (p.seqlen % 8 != 0) return false;
+  bool v = ok(p.u, p.u_bs, p.u_ds) && ok(p.delta, p.delta_bs, p.delta_ds) && ok(p.z, p.z_bs, p.z_ds) &&
+           ok(p.B, p.B_bs, p.B_gs) && p.B_ns % m == 0 && ok(p.C, p.C_bs, p.C_gs) && p.C_ns % m == 0;
+  if (!bwd) return v && ok(p.out, p.out_bs, p.out_ds);
+  return v && ok(p.dout, p.dout_bs, p.dout_ds) && ok(p.du, p.du_bs, p.du_ds) &&
+         ok(p.ddelta, p.ddelta_bs, p.ddelta_ds) && ok(p.dz, p.dz_bs, p.dz_ds) && ok(p.out_z, p.outz_bs, p.outz_ds);
+}
+
+template <typename T, bool BWD> int dispatch(const MambaScanParams &p, hipStream_t stream) {
+  const int np = (p.dstate + NB16 - 1) / NB16 * NB16;
+  const bool vec = vec_ok(p, BWD);
+  const bool small = p.dstate <= NB16;
+  if (!BWD) {
+    if (small) {
+      const size_t lds = fwd_lds(8, 4, np);
+      return vec ? launch(scan_fwd_kernel<T, 8, 4, true>, p, 8, 4, lds, stream)
+                 : launch(scan_fwd_kernel<T, 8, 4, false>, p, 8, 4, lds, stream);
+    }
+    const size_t lds = fwd_lds(8, 1, np);
+    return vec ? launch(scan_fwd_kernel<T, 8, 1, true>, p, 8, 1, lds, stream)
+               : launch(scan_fwd_kernel<T, 8, 1, false>, p, 8, 1, lds, stream);
+  } else {
+    if (small) {
+      const size_t lds = bwd_lds(8, 4, np);
+      return vec ? launch(scan_bwd_kernel<T, 8, 4, true>, p, 8, 4, lds, stream)
+                 : launch(scan_bwd_kernel<T, 8, 4, false>, p, 8, 4, lds, stream);
+    }
+    const size_t lds = bwd_lds(4, 1, np);
+    return vec ? launch(scan_bwd_kernel<T, 4, 1, true>, p, 4, 1, lds, stream)
+               : launch(scan_bwd_kernel<T, 4, 1, false>, p, 4, 1, lds, stream);
+  }
+}
+
+}  // namespace
+
+extern "C" int mamba1_scan_fwd(const MambaScanParams *p, mamba_stream_t stream) {
+  int rc = check_common(p);
+  if (rc != MAMBA_OK) return rc;
+  if (!p->out) return MAMBA_E_BADARG;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (p->dtype) {
+    case MAMBA_F32: return dispatch<float, false>(*p, s);
+    case MAMBA_BF16: return dispatch<bf16_t, false>(*p, s);
+    default: return dispatch<f16_t, false>(*p, s);
+  }
+}
+
+extern "C" int mamba1_scan_bwd(const MambaScanParams *p, mamba_stream_t stream) {
+  int rc = check_common(p);
+  if (rc != MAMBA_OK) return rc;
+  if (!p->dout || !p->du || !p->ddelta || !p->dB32 || !p->dC32 || !p->dA_part || !p->dD_part || !p->ddelta_bias_part)
+    return MAMBA_E_BADARG;
+  if (p->z && !p->dz) return MAMBA_E_BADARG;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (p->dtype) {
+    case MAMBA_F32: return dispatch<float, true>(*p, s);
+    case MAMBA_BF16: return dispatch<bf16_t, true>(*p, s);
+    default: return dispatch<f16_t, true>(*p, s);
+  }
+}

@@ -1,0 +1,209 @@
+"""Mamba-1 selective scan: drop-in for mamba_ssm.ops.selective_scan_interface.
+
+Same names, argument meaning and error behaviour as the reference module
+(mamba_ssm/ops/selective_scan_interface.py:34 SelectiveScanFn, :118
+selective_scan_fn, :196 MambaInnerFn, :386 mamba_inner_fn).  The compute is
+done by the HIP kernels of libmamba_gfx950.so through its C ABI; the functions
+`selective_scan_fwd` / `selective_scan_bwd` below take the place of the
+reference's pybind module `selective_scan_cuda`
+(csrc/selective_scan/selective_scan.cpp:494-497).
+"""
+import torch
+import torch.nn.functional as F
+from einops import rearrange
+
+from mamba_amd import _lib
+
+_FLOAT_TYPES = (torch.float32, torch.bfloat16, torch.float16)
+
+
+def scan_tile():
+    return _lib.load().mamba_hip_query(1)
+
+
+def _check_inputs(u, delta, A, B, C, D, z, delta_bias):
+    """Argument checks of selective_scan.cpp:233-303, before any launch."""
+    _lib.require_gpu(u, delta, A, B, C, D, z, delta_bias)
+    if u.dtype not in _FLOAT_TYPES:
+        raise RuntimeError(f"selective_scan: unsupported input dtype {u.dtype}")
+    if A.is_complex():
+        raise NotImplementedError("selective_scan: complex A is not built in mamba_amd")
+    if A.dtype != torch.float32:
+        raise RuntimeError("selective_scan: A must be float32")
+    if B.dim() < 3 or C.dim() < 3:
+        raise NotImplementedError("selective_scan: input-independent B/C of shape (dim, dstate) is not built in mamba_amd")
+    if u.dim() != 3:
+        raise RuntimeError("selective_scan: u must be (batch, dim, seqlen)")
+    batch, dim, seqlen = u.shape
+    dstate = A.shape[1]
+    if dstate > _lib.load().mamba_hip_query(2):
+        raise RuntimeError("selective_scan only supports state dimension <= 256")
+    if delta.dtype != u.dtype or B.dtype != u.dtype or C.dtype != u.dtype:
+        raise RuntimeError("selective_scan: u, delta, B, C must share one dtype")
+    for name, t in (("u", u), ("delta", delta), ("B", B), ("C", C), ("z", z)):
+        if t is not None and t.stride(-1) != 1:
+            raise RuntimeError(f"selective_scan: {name} must have stride 1 in the last dimension")
+    ngroups = B.shape[1]
+    if tuple(delta.shape) != (batch, dim, seqlen):
+        raise RuntimeError("selective_scan: delta shape mismatch")
+    if tuple(A.shape) != (dim, dstate):
+        raise RuntimeError("selective_scan: A shape mismatch")
+    if tuple(B.shape) != (batch, ngroups, dstate, seqlen) or tuple(C.shape) != (batch, ngroups, dstate, seqlen):
+        raise RuntimeError("selective_scan: B/C must be (batch, ngroups, dstate, seqlen)")
+    if dim % ngroups != 0:
+        raise RuntimeError("selective_scan: dim must be divisible by ngroups")
+    if D is not None and (D.dtype != torch.float32 or tuple(D.shape) != (dim,) or D.stride(-1) != 1):
+        raise RuntimeError("selective_scan: D must be contiguous float32 of shape (dim,)")
+    if delta_bias is not None and (delta_bias.dtype != torch.float32 or tuple(delta_bias.shape) != (dim,)
+                                   or delta_bias.stride(-1) != 1):
+        raise RuntimeError("selective_scan: delta_bias must be contiguous float32 of shape (dim,)")
+    if z is not None and (z.dtype != u.dtype or tuple(z.shape) != (batch, dim, seqlen)):
+        raise RuntimeError("selective_scan: z must match u in dtype and shape")
+    return batch, dim, seqlen, dstate, ngroups
+
+
+def _fill_common(p, u, delta, A, B, C, D, z, delta_bias, delta_softplus, ckpt, dims):
+    batch, dim, seqlen, dstate, ngroups = dims
+    p.batch, p.dim, p.seqlen, p.dstate, p.ngroups = batch, dim, seqlen, dstate, ngroups
+    p.dtype = _lib.DTYPE_CODE[u.dtype]
+    p.delta_softplus = int(bool(delta_softplus))
+    p.u, p.delta, p.A, p.B, p.C = u.data_ptr(), delta.data_ptr(), A.data_ptr(), B.data_ptr(), C.data_ptr()
+    p.D, p.z, p.delta_bias = _lib.ptr(D), _lib.ptr(z), _lib.ptr(delta_bias)
+    p.ckpt = ckpt.data_ptr()
+    p.u_bs, p.u_ds = u.stride(0), u.stride(1)
+    p.delta_bs, p.delta_ds = delta.stride(0), delta.stride(1)
+    if z is not None:
+        p.z_bs, p.z_ds = z.stride(0), z.stride(1)
+    p.B_bs, p.B_gs, p.B_ns = B.stride(0), B.stride(1), B.stride(2)
+    p.C_bs, p.C_gs, p.C_ns = C.stride(0), C.stride(1), C.stride(2)
+
+
+def selective_scan_fwd(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta_softplus=False):
+    """Counterpart of selective_scan_cuda.fwd (selective_scan.cpp:226).
+
+    Returns (out, ckpt): `out` is the gated output y*silu(z) when z is given, else y, in u's
+    dtype; `ckpt` is (batch, dim, ntiles, dstate) fp32, the state after each tile of
+    `scan_tile()` positions (ckpt[:, :, -1] is the last state).  The ungated y is not
+    stored: the backward pass re-computes it.
+    """
+    dims = _check_inputs(u, delta, A, B, C, D, z, delta_bias)
+    batch, dim, seqlen, dstate, _ = dims
+    A = A.contiguous()
+    ntiles = (seqlen + scan_tile() - 1) // scan_tile()
+    out = torch.empty_like(delta)
+    ckpt = torch.empty(batch, dim, ntiles, dstate, device=u.device, dtype=torch.float32)
+    p = _lib.MambaScanParams()
+    _fill_common(p, u, delta, A, B, C, D, z, delta_bias, delta_softplus, ckpt, dims)
+    p.out = out.data_ptr()
+    p.out_bs, p.out_ds = out.stride(0), out.stride(1)
+    with torch.cuda.device(u.device):
+        _lib.check(_lib.load().mamba1_scan_fwd(p, _lib.current_stream(u.device)), "mamba1_scan_fwd")
+    return out, ckpt
+
+
+def selective_scan_bwd(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, dz=None, delta_softplus=False,
+                       recompute_out_z=False):
+    """Counterpart of selective_scan_cuda.bwd (selective_scan.cpp:338).
+
+    `dz` may be a caller-owned strided view (last stride 1) that receives the gate gradient,
+    as MambaInnerFn passes it (selective_scan_interface.py:333-338).
+    Returns (du, ddelta, dA, dB, dC, dD, ddelta_bias, dz, out_z).
+    """
+    dims = _check_inputs(u, delta, A, B, C, D, z, delta_bias)
+    batch, dim, seqlen, dstate, ngroups = dims
+    _lib.require_gpu(dout, ckpt, dz)
+    if dout.dtype != u.dtype or tuple(dout.shape) != (batch, dim, seqlen) or dout.stride(-1) != 1:
+        raise RuntimeError("selective_scan: dout must match u in dtype/shape with stride 1 in the last dimension")
+    A = A.contiguous()
+    dev = u.device
+    du = torch.empty_like(u)
+    ddelta = torch.empty_like(delta)
+    dB32 = torch.zeros(batch, ngroups, dstate, seqlen, device=dev, dtype=torch.float32)
+    dC32 = torch.zeros_like(dB32)
+    dA_part = torch.empty(batch, dim, dstate, device=dev, dtype=torch.float32)
+    dD_part = torch.empty(batch, dim, device=dev, dtype=torch.float32)
+    dbias_part = torch.empty(batch, dim, device=dev, dtype=torch.float32)
+    out_z = None
+    if z is not None:
+        if dz is None:
+            dz = torch.empty_like(z)
+        elif dz.dtype != u.dtype or tuple(dz.shape) != (batch, dim, seqlen) or dz.stride(-1) != 1:
+            raise RuntimeError("selective_scan: dz must match z in dtype/shape with stride 1 in the last dimension")
+        if recompute_out_z:
+            out_z = torch.empty_like(u)
+    else:
+        dz = None
+    p = _lib.MambaScanParams()
+    _fill_common(p, u, delta, A, B, C, D, z, delta_bias, delta_softplus, ckpt, dims)
+    p.dout, p.du, p.ddelta = dout.data_ptr(), du.data_ptr(), ddelta.data_ptr()
+    p.dz, p.out_z = _lib.ptr(dz), _lib.ptr(out_z)
+    p.dB32, p.dC32 = dB32.data_ptr(), dC32.data_ptr()
+    p.dA_part, p.dD_part, p.ddelta_bias_part = dA_part.data_ptr(), dD_part.data_ptr(), dbias_part.data_ptr()
+    p.dout_bs, p.dout_ds = dout.stride(0), dout.stride(1)
+    p.du_bs, p.du_ds = du.stride(0), du.stride(1)
+    p.ddelta_bs, p.ddelta_ds = ddelta.stride(0), ddelta.stride(1)
+    if dz is not None:
+        p.dz_bs, p.dz_ds = dz.stride(0), dz.stride(1)
+    if out_z is not None:
+        p.outz_bs, p.outz_ds = out_z.stride(0), out_z.stride(1)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().mamba1_scan_bwd(p, _lib.current_stream(dev)), "mamba1_scan_bwd")
+    dA = dA_part.sum(0)
+    dD = dD_part.sum(0) if D is not None else None
+    ddelta_bias = dbias_part.sum(0) if delta_bias is not None else None
+    return du, ddelta, dA, dB32.to(B.dtype), dC32.to(C.dtype), dD, ddelta_bias, dz, out_z
+
+
+class SelectiveScanFn(torch.autograd.Function):
+    """autograd wrapper, as the reference's SelectiveScanFn (selective_scan_interface.py:34-93)."""
+
+    @staticmethod
+    def forward(ctx, u, delta, A, B, C, D=None, z=None, delta_bias=None, delta_softplus=False,
+                return_last_state=False):
+        if u.stride(-1) != 1:
+            u = u.contiguous()
+        if delta.stride(-1) != 1:
+            delta = delta.contiguous()
+        if D is not None:
+            D = D.contiguous()
+        if B.stride(-1) != 1:
+            B = B.contiguous()
+        if C.stride(-1) != 1:
+            C = C.contiguous()
+        if z is not None and z.stride(-1) != 1:
+            z = z.contiguous()
+        ctx.squeeze_B = ctx.squeeze_C = False
+        if B.dim() == 3:
+            B = rearrange(B, "b dstate l -> b 1 dstate l")
+            ctx.squeeze_B = True
+        if C.dim() == 3:
+            C = rearrange(C, "b dstate l -> b 1 dstate l")
+            ctx.squeeze_C = True
+        out, ckpt = selective_scan_fwd(u, delta, A, B, C, D, z, delta_bias, delta_softplus)
+        ctx.delta_softplus = delta_softplus
+        ctx.has_z = z is not None
+        ctx.has_D = D is not None
+        ctx.has_bias = delta_bias is not None
+        last_state = ckpt[:, :, -1, :]  # (batch, dim, dstate)
+        ctx.save_for_backward(u, delta, A, B, C, D, z, delta_bias, ckpt)
+        return out if not return_last_state else (out, last_state)
+
+    @staticmethod
+    def backward(ctx, dout, *args):
+        u, delta, A, B, C, D, z, delta_bias, ckpt = ctx.saved_tensors
+        if dout.stride(-1) != 1:
+            dout = dout.contiguous()
+        du, ddelta, dA, dB, dC, dD, ddelta_bias, dz, _ = selective_scan_bwd(
+            u, delta, A, B, C, D, z, delta_bias, dout, ckpt, None, ctx.delta_softplus, False)
+        dB = dB.squeeze(1) if ctx.squeeze_B else dB
+        dC = dC.squeeze(1) if ctx.squeeze_C else dC
+        return (du, ddelta, dA, dB, dC, dD, dz, ddelta_bias, None, None)
+
+
+def selective_scan_fn(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta_softplus=False,
+                      return_last_state=False):
+    """if return_last_state is True, returns (out, last_state)
+    last_state has shape (batch, dim, dstate). The gradient of the last state is not
+    considered in the backward pass (as in the reference, selective_scan_interface.py:118-124).
+    """
+    return SelectiveScanFn.apply(u, delta, A, B, C, D, z, delta_bias, delta_softplus, return_last_state)
