@@ -11,9 +11,10 @@
 //     previous tile kept in LDS.
 //   * the state after every tile is written to `ckpt`; the backward pass walks
 //     the tiles in reverse, restarts each tile from ckpt, and runs the adjoint
-//     recurrence with a lane-reversed scan.  dB/dC are reduced over the
-//     channels of the workgroup in LDS and added to global fp32 buffers once
-//     per tile.
+//     recurrence with a lane-reversed scan.  dB/dC are summed over the
+//     channels of the workgroup in LDS (waves take turns on disjoint state
+//     rows; LDS float atomics are far too slow for this) and added to global
+//     fp32 buffers once per tile.
 #include "common.hpp"
 
 namespace {
@@ -22,8 +23,6 @@ constexpr int KI = 8;           // items per lane
 constexpr int TILE = 64 * KI;   // sequence positions per tile
 constexpr int NB16 = 16;        // states staged per LDS block
 constexpr int BC_FLOATS = NB16 * TILE;        // one staged tensor
-constexpr int ACC_PITCH = 9;                  // items per lane, padded (bank spread)
-constexpr int ACC_FLOATS = NB16 * 64 * ACC_PITCH;
 constexpr int MAX_DSTATE = 256;
 
 // B or C rows n0..n0+15 of the tile starting at t0 -> LDS as fp32, laid out
@@ -44,6 +43,12 @@ DEVI void stage_bc(float *Bs, float *Cs, const T *Bg, int64_t B_ns, const T *Cg,
     *reinterpret_cast<f32x4 *>(dst) = lo;
     *reinterpret_cast<f32x4 *>(dst + 256) = hi;
   }
+}
+
+DEVI void lds_st8(float *base, int lane, const float (&v)[8]) {
+  f32x4 lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
+  *reinterpret_cast<f32x4 *>(base + lane * 4) = lo;
+  *reinterpret_cast<f32x4 *>(base + 256 + lane * 4) = hi;
 }
 
 DEVI void lds_ld8(const float *base, int lane, float (&o)[8]) {
@@ -114,7 +119,6 @@ __global__ __launch_bounds__(NW * 64) void scan_fwd_kernel(const MambaScanParams
           const float *A2row = A2s + (wave * R + r) * NP + nb * NB16;
           float *hrow = hcar + (wave * R + r) * NP + nb * NB16;
           const int nmax = min(NB16, N - nb * NB16);
-#pragma unroll 2
           for (int n = 0; n < nmax; ++n) {
             const float A2 = A2row[n];
             const float hc = hrow[n];
@@ -169,9 +173,9 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
   constexpr int WR = NW * R;
   float *Bs = smem;
   float *Cs = Bs + BC_FLOATS;
-  float *dBs = Cs + BC_FLOATS;        // [16][64][9]
-  float *dCs = dBs + ACC_FLOATS;
-  float *A1s = dCs + ACC_FLOATS;      // [WR][NP] A
+  float *dBs = Cs + BC_FLOATS;        // fp32 sums over the workgroup's channels, same layout as Bs
+  float *dCs = dBs + BC_FLOATS;
+  float *A1s = dCs + BC_FLOATS;       // [WR][NP] A
   float *hcar = A1s + WR * NP;        // state entering the tile (from ckpt)
   float *gcar = hcar + WR * NP;       // adjoint at the first position of the following tile
   float *anx = gcar + WR * NP;        // decay at the first position of the following tile
@@ -251,89 +255,103 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
         if (NBLK > 1 || r == 0) {
           __syncthreads();
           stage_bc<T, VEC, NW * 64>(Bs, Cs, Bg, p.B_ns, Cg, p.C_ns, nb * NB16, N, t0, L, tid);
-          for (int i = tid; i < 2 * ACC_FLOATS; i += NW * 64) dBs[i] = 0.f;  // dBs and dCs are adjacent
+          for (int i = tid; i < 2 * BC_FLOATS; i += NW * 64) dBs[i] = 0.f;  // dBs and dCs are adjacent
           __syncthreads();
         }
-        if (valid) {
+        {
+          // The NW waves add their channels' dB/dC terms into the shared LDS sums without
+          // atomics: in phase ph wave w owns state rows (w + ph) % NPH * NPP .. + NPP - 1,
+          // so no two waves touch a row between two barriers.
+          constexpr int NPP = NB16 / NW > 0 ? NB16 / NW : 1;
+          constexpr int NPH = NB16 / NPP;
+          static_assert(NW <= NPH, "one row slot per wave and phase");
           const float *A1row = A1s + row * NP + nb * NB16;
           const float *hrow = hcar + row * NP + nb * NB16;
           float *grow = gcar + row * NP + nb * NB16;
           float *arow = anx + row * NP + nb * NB16;
           float *dArow = dAacc + row * NP + nb * NB16;
           const int nmax = min(NB16, N - nb * NB16);
-          for (int n = 0; n < nmax; ++n) {
-            const float A1 = A1row[n], A2 = A1 * kLog2e;
-            const float hc = hrow[n], gc = grow[n], an = arow[n];
-            float Bv[8], Cv[8], a[8], ac[8], bb[8], h[8];
-            lds_ld8(Bs + n * TILE, lane, Bv);
-            lds_ld8(Cs + n * TILE, lane, Cv);
+          for (int ph = 0; ph < NPH; ++ph) {
+            const int slot = (wave + ph) % NPH;
+            for (int j = 0; j < NPP; ++j) {
+              const int n = slot * NPP + j;
+              if (!valid || n >= nmax) continue;
+              const float A1 = A1row[n], A2 = A1 * kLog2e;
+              const float hc = hrow[n], gc = grow[n], an = arow[n];
+              float Bv[8], Cv[8], a[8], ac[8], bb[8], h[8];
+              lds_ld8(Bs + n * TILE, lane, Bv);
+              lds_ld8(Cs + n * TILE, lane, Cv);
 #pragma unroll
-            for (int i = 0; i < KI; ++i) {
-              a[i] = fast_exp2(dl[i] * A2);
-              bb[i] = du[i] * Bv[i];
-            }
-            h[0] = bb[0];
-            ac[0] = a[0];
+              for (int i = 0; i < KI; ++i) {
+                a[i] = fast_exp2(dl[i] * A2);
+                bb[i] = du[i] * Bv[i];
+              }
+              h[0] = bb[0];
+              ac[0] = a[0];
 #pragma unroll
-            for (int i = 1; i < KI; ++i) {
-              h[i] = __builtin_fmaf(a[i], h[i - 1], bb[i]);
-              ac[i] = ac[i - 1] * a[i];
-            }
-            float sa = ac[KI - 1], sb = h[KI - 1];
-            wave_scan_fwd(sa, sb);
-            const float hend = __builtin_fmaf(sa, hc, sb);
-            const float hx = dpp_f<DPP_WAVE_SHR1>(hc, hend);
+              for (int i = 1; i < KI; ++i) {
+                h[i] = __builtin_fmaf(a[i], h[i - 1], bb[i]);
+                ac[i] = ac[i - 1] * a[i];
+              }
+              float sa = ac[KI - 1], sb = h[KI - 1];
+              wave_scan_fwd(sa, sb);
+              const float hend = __builtin_fmaf(sa, hc, sb);
+              const float hx = dpp_f<DPP_WAVE_SHR1>(hc, hend);
 #pragma unroll
-            for (int i = 0; i < KI; ++i) h[i] = __builtin_fmaf(ac[i], hx, h[i]);  // true states
-            if (has_z) {
+              for (int i = 0; i < KI; ++i) h[i] = __builtin_fmaf(ac[i], hx, h[i]);  // true states
+              if (has_z) {
 #pragma unroll
-              for (int i = 0; i < KI; ++i) y[i] = __builtin_fmaf(h[i], Cv[i], y[i]);
-            }
-            // adjoint recurrence g[t] = dy[t] C[t] + a[t+1] g[t+1]
-            const float a_next_lane = dpp_f<DPP_WAVE_SHL1>(an, a[0]);
-            float gg[8], ar[8];
-            gg[KI - 1] = dy[KI - 1] * Cv[KI - 1];
-            ar[KI - 1] = a_next_lane;
+                for (int i = 0; i < KI; ++i) y[i] = __builtin_fmaf(h[i], Cv[i], y[i]);
+              }
+              // adjoint recurrence g[t] = dy[t] C[t] + a[t+1] g[t+1]
+              const float a_next_lane = dpp_f<DPP_WAVE_SHL1>(an, a[0]);
+              float gg[8], ar[8];
+              gg[KI - 1] = dy[KI - 1] * Cv[KI - 1];
+              ar[KI - 1] = a_next_lane;
 #pragma unroll
-            for (int i = KI - 2; i >= 0; --i) {
-              gg[i] = __builtin_fmaf(a[i + 1], gg[i + 1], dy[i] * Cv[i]);
-              ar[i] = ar[i + 1] * a[i + 1];
-            }
-            float ra = ar[0], rb = gg[0];
-            wave_scan_rev(ra, rb, lane);
-            const float gfirst = __builtin_fmaf(ra, gc, rb);         // adjoint at this lane's first item
-            const float gx = dpp_f<DPP_WAVE_SHL1>(gc, gfirst);       // ... at the next lane's first item
-            if (lane == 0) {
-              grow[n] = gfirst;
-              arow[n] = a[0];
-            }
-            float dAp = 0.f;
-            float *dBl = dBs + (n * 64 + lane) * ACC_PITCH;
-            float *dCl = dCs + (n * 64 + lane) * ACC_PITCH;
+              for (int i = KI - 2; i >= 0; --i) {
+                gg[i] = __builtin_fmaf(a[i + 1], gg[i + 1], dy[i] * Cv[i]);
+                ar[i] = ar[i + 1] * a[i + 1];
+              }
+              float ra = ar[0], rb = gg[0];
+              wave_scan_rev(ra, rb, lane);
+              const float gfirst = __builtin_fmaf(ra, gc, rb);    // adjoint at this lane's first item
+              const float gx = dpp_f<DPP_WAVE_SHL1>(gc, gfirst);  // ... at the next lane's first item
+              if (lane == 0) {
+                grow[n] = gfirst;
+                arow[n] = a[0];
+              }
+              float dAp = 0.f;
+              float sB[8], sC[8];
+              lds_ld8(dBs + n * TILE, lane, sB);
+              lds_ld8(dCs + n * TILE, lane, sC);
 #pragma unroll
-            for (int i = 0; i < KI; ++i) {
-              const float gi = __builtin_fmaf(ar[i], gx, gg[i]);
-              __hip_atomic_fetch_add(dCl + i, dy[i] * h[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-              __hip_atomic_fetch_add(dBl + i, gi * du[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-              acc[i] = __builtin_fmaf(gi, Bv[i], acc[i]);
-              const float w = gi * (h[i] - bb[i]);  // g * a * h[t-1]
-              dd[i] = __builtin_fmaf(A1, w, dd[i]);
-              dAp = __builtin_fmaf(dl[i], w, dAp);
+              for (int i = 0; i < KI; ++i) {
+                const float gi = __builtin_fmaf(ar[i], gx, gg[i]);
+                sC[i] = __builtin_fmaf(dy[i], h[i], sC[i]);
+                sB[i] = __builtin_fmaf(gi, du[i], sB[i]);
+                acc[i] = __builtin_fmaf(gi, Bv[i], acc[i]);
+                const float w = gi * (h[i] - bb[i]);  // g * a * h[t-1]
+                dd[i] = __builtin_fmaf(A1, w, dd[i]);
+                dAp = __builtin_fmaf(dl[i], w, dAp);
+              }
+              lds_st8(dBs + n * TILE, lane, sB);
+              lds_st8(dCs + n * TILE, lane, sC);
+              dAp += dpp_f<DPP_ROW_SHR + 1>(0.f, dAp);
+              dAp += dpp_f<DPP_ROW_SHR + 2>(0.f, dAp);
+              dAp += dpp_f<DPP_ROW_SHR + 4>(0.f, dAp);
+              dAp += dpp_f<DPP_ROW_SHR + 8>(0.f, dAp);
+              if ((lane & 15) == 15)
+                __hip_atomic_fetch_add(dArow + n, dAp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             }
-            dAp += dpp_f<DPP_ROW_SHR + 1>(0.f, dAp);
-            dAp += dpp_f<DPP_ROW_SHR + 2>(0.f, dAp);
-            dAp += dpp_f<DPP_ROW_SHR + 4>(0.f, dAp);
-            dAp += dpp_f<DPP_ROW_SHR + 8>(0.f, dAp);
-            if ((lane & 15) == 15)
-              __hip_atomic_fetch_add(dArow + n, dAp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            __syncthreads();
           }
         }
         if (NBLK > 1 || r == R - 1) {
-          __syncthreads();
           const int n0 = nb * NB16;
           for (int i = tid; i < 2 * NB16 * TILE; i += NW * 64) {
             const int which = i >> 13, n = (i >> 9) & 15, t = i & (TILE - 1);
-            const float v = (which ? dCs : dBs)[(n * 64 + (t >> 3)) * ACC_PITCH + (t & 7)];
+            const float v = (which ? dCs : dBs)[n * TILE + ((t >> 2) & 1) * 256 + (t >> 3) * 4 + (t & 3)];
             if (n0 + n < N && t0 + t < L) unsafeAtomicAdd((which ? dCg : dBg) + (int64_t)(n0 + n) * L + t0 + t, v);
           }
         }
@@ -402,7 +420,7 @@ struct Cfg {
 
 inline size_t fwd_lds(int nw, int r, int np) { return sizeof(float) * (2 * BC_FLOATS + 2 * nw * r * np); }
 inline size_t bwd_lds(int nw, int r, int np) {
-  return sizeof(float) * (2 * BC_FLOATS + 2 * ACC_FLOATS + 5 * nw * r * np + 2 * nw * r);
+  return sizeof(float) * (4 * BC_FLOATS + 5 * nw * r * np + 2 * nw * r);
 }
 
 template <typename KernelT>
