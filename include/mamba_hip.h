@@ -107,6 +107,44 @@ typedef struct MambaScanParams {
 int mamba1_scan_fwd(const MambaScanParams *p, mamba_stream_t stream);
 int mamba1_scan_bwd(const MambaScanParams *p, mamba_stream_t stream);
 
+/* ------------------------------------------------------------------------- *
+ * Single-token decode: one step of the recurrence, in place on `state`.
+ * Replaces the Triton kernel behind selective_state_update
+ * (reference mamba_ssm/ops/triton/selective_state_update.py:24 kernel, :135
+ * host function):
+ *   dt' = softplus(dt + dt_bias)                (each part optional)
+ *   state[b,h,p,n] = state * exp(A[h,p,n] dt'[b,h,p]) + B[b,g,n] dt' x[b,h,p]
+ *   out[b,h,p] = sum_n state[b,h,p,n] C[b,g,n] + D[h,p] x[b,h,p];  out *= silu(z)
+ * Every tensor is addressed through element strides, so stride-0 (expanded)
+ * dt / A / dt_bias / D are accepted as they are.  Each operand has its own
+ * dtype code (MAMBA_F32/BF16/F16); the arithmetic is fp32.
+ * state_batch_indices (int32, nullable): row of `state` used by batch entry b;
+ * a negative index skips the entry and writes out = 0.
+ * ------------------------------------------------------------------------- */
+typedef struct MambaStepParams {
+  int32_t batch, nheads, dim, dstate, ngroups;
+  int32_t dt_softplus;
+  int32_t state_dtype, x_dtype /* x, z, out */, dt_dtype, dt_bias_dtype, A_dtype, bc_dtype /* B, C */, D_dtype;
+  int32_t reserved0;
+  void *state;
+  const void *x, *dt, *A, *B, *C;
+  const void *D, *z, *dt_bias; /* nullable */
+  void *out;
+  const int32_t *state_batch_indices; /* nullable */
+  int64_t state_bs, state_hs, state_ps, state_ns;
+  int64_t x_bs, x_hs, x_ps;
+  int64_t dt_bs, dt_hs, dt_ps;
+  int64_t dt_bias_hs, dt_bias_ps;
+  int64_t A_hs, A_ps, A_ns;
+  int64_t B_bs, B_gs, B_ns;
+  int64_t C_bs, C_gs, C_ns;
+  int64_t D_hs, D_ps;
+  int64_t z_bs, z_hs, z_ps;
+  int64_t out_bs, out_hs, out_ps;
+} MambaStepParams;
+
+int ssm_state_update(const MambaStepParams *p, mamba_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -30,6 +30,18 @@ class MambaScanParams(ctypes.Structure):
     )
 
 
+class MambaStepParams(ctypes.Structure):
+    _fields_ = (
+        [(n, c_i32) for n in ("batch", "nheads", "dim", "dstate", "ngroups", "dt_softplus", "state_dtype", "x_dtype",
+                              "dt_dtype", "dt_bias_dtype", "A_dtype", "bc_dtype", "D_dtype", "reserved0")]
+        + [(n, c_vp) for n in ("state", "x", "dt", "A", "B", "C", "D", "z", "dt_bias", "out", "state_batch_indices")]
+        + [(n, c_i64) for n in ("state_bs", "state_hs", "state_ps", "state_ns", "x_bs", "x_hs", "x_ps",
+                                "dt_bs", "dt_hs", "dt_ps", "dt_bias_hs", "dt_bias_ps", "A_hs", "A_ps", "A_ns",
+                                "B_bs", "B_gs", "B_ns", "C_bs", "C_gs", "C_ns", "D_hs", "D_ps",
+                                "z_bs", "z_hs", "z_ps", "out_bs", "out_hs", "out_ps")]
+    )
+
+
 _lib = None
 
 
@@ -54,6 +66,8 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = [ctypes.POINTER(MambaScanParams), c_vp]
         fn.restype = ctypes.c_int
+    lib.ssm_state_update.argtypes = [ctypes.POINTER(MambaStepParams), c_vp]
+    lib.ssm_state_update.restype = ctypes.c_int
     _lib = lib
     return lib
 

@@ -101,6 +101,53 @@ def selective_scan_fwd(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta
     return out, ckpt
 
 
+class ScanBwdBuffers:
+    """Outputs and fp32 accumulators of one backward launch (all caller-owned)."""
+
+    def __init__(self, u, delta, B, z, dims, dz=None, recompute_out_z=False):
+        batch, dim, seqlen, dstate, ngroups = dims
+        dev = u.device
+        self.du = torch.empty_like(u)
+        self.ddelta = torch.empty_like(delta)
+        self.dBC32 = torch.empty(2, batch, ngroups, dstate, seqlen, device=dev, dtype=torch.float32)
+        self.dA_part = torch.empty(batch, dim, dstate, device=dev, dtype=torch.float32)
+        self.dD_part = torch.empty(batch, dim, device=dev, dtype=torch.float32)
+        self.dbias_part = torch.empty(batch, dim, device=dev, dtype=torch.float32)
+        self.dz = self.out_z = None
+        if z is not None:
+            self.dz = dz if dz is not None else torch.empty_like(z)
+            if recompute_out_z:
+                self.out_z = torch.empty_like(u)
+
+
+def scan_bwd_zero(bufs, device):
+    """Clears the dB/dC accumulators (the kernel adds into them) with the library's fill kernel."""
+    with torch.cuda.device(device):
+        _lib.check(_lib.load().mamba_hip_zero(bufs.dBC32.data_ptr(), bufs.dBC32.numel() * 4,
+                                              _lib.current_stream(device)), "mamba_hip_zero")
+
+
+def scan_bwd_launch(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, delta_softplus, bufs, dims):
+    """One call of the C ABI's mamba1_scan_bwd on the current stream; bufs.dBC32 must be zero."""
+    p = _lib.MambaScanParams()
+    _fill_common(p, u, delta, A, B, C, D, z, delta_bias, delta_softplus, ckpt, dims)
+    dz, out_z = bufs.dz, bufs.out_z
+    p.dout, p.du, p.ddelta = dout.data_ptr(), bufs.du.data_ptr(), bufs.ddelta.data_ptr()
+    p.dz, p.out_z = _lib.ptr(dz), _lib.ptr(out_z)
+    p.dB32, p.dC32 = bufs.dBC32[0].data_ptr(), bufs.dBC32[1].data_ptr()
+    p.dA_part, p.dD_part = bufs.dA_part.data_ptr(), bufs.dD_part.data_ptr()
+    p.ddelta_bias_part = bufs.dbias_part.data_ptr()
+    p.dout_bs, p.dout_ds = dout.stride(0), dout.stride(1)
+    p.du_bs, p.du_ds = bufs.du.stride(0), bufs.du.stride(1)
+    p.ddelta_bs, p.ddelta_ds = bufs.ddelta.stride(0), bufs.ddelta.stride(1)
+    if dz is not None:
+        p.dz_bs, p.dz_ds = dz.stride(0), dz.stride(1)
+    if out_z is not None:
+        p.outz_bs, p.outz_ds = out_z.stride(0), out_z.stride(1)
+    with torch.cuda.device(u.device):
+        _lib.check(_lib.load().mamba1_scan_bwd(p, _lib.current_stream(u.device)), "mamba1_scan_bwd")
+
+
 def selective_scan_bwd(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, dz=None, delta_softplus=False,
                        recompute_out_z=False):
     """Counterpart of selective_scan_cuda.bwd (selective_scan.cpp:338).
@@ -114,44 +161,18 @@ def selective_scan_bwd(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, dz=None,
     _lib.require_gpu(dout, ckpt, dz)
     if dout.dtype != u.dtype or tuple(dout.shape) != (batch, dim, seqlen) or dout.stride(-1) != 1:
         raise RuntimeError("selective_scan: dout must match u in dtype/shape with stride 1 in the last dimension")
+    if z is not None and dz is not None and (dz.dtype != u.dtype or tuple(dz.shape) != (batch, dim, seqlen)
+                                             or dz.stride(-1) != 1):
+        raise RuntimeError("selective_scan: dz must match z in dtype/shape with stride 1 in the last dimension")
     A = A.contiguous()
-    dev = u.device
-    du = torch.empty_like(u)
-    ddelta = torch.empty_like(delta)
-    dB32 = torch.zeros(batch, ngroups, dstate, seqlen, device=dev, dtype=torch.float32)
-    dC32 = torch.zeros_like(dB32)
-    dA_part = torch.empty(batch, dim, dstate, device=dev, dtype=torch.float32)
-    dD_part = torch.empty(batch, dim, device=dev, dtype=torch.float32)
-    dbias_part = torch.empty(batch, dim, device=dev, dtype=torch.float32)
-    out_z = None
-    if z is not None:
-        if dz is None:
-            dz = torch.empty_like(z)
-        elif dz.dtype != u.dtype or tuple(dz.shape) != (batch, dim, seqlen) or dz.stride(-1) != 1:
-            raise RuntimeError("selective_scan: dz must match z in dtype/shape with stride 1 in the last dimension")
-        if recompute_out_z:
-            out_z = torch.empty_like(u)
-    else:
-        dz = None
-    p = _lib.MambaScanParams()
-    _fill_common(p, u, delta, A, B, C, D, z, delta_bias, delta_softplus, ckpt, dims)
-    p.dout, p.du, p.ddelta = dout.data_ptr(), du.data_ptr(), ddelta.data_ptr()
-    p.dz, p.out_z = _lib.ptr(dz), _lib.ptr(out_z)
-    p.dB32, p.dC32 = dB32.data_ptr(), dC32.data_ptr()
-    p.dA_part, p.dD_part, p.ddelta_bias_part = dA_part.data_ptr(), dD_part.data_ptr(), dbias_part.data_ptr()
-    p.dout_bs, p.dout_ds = dout.stride(0), dout.stride(1)
-    p.du_bs, p.du_ds = du.stride(0), du.stride(1)
-    p.ddelta_bs, p.ddelta_ds = ddelta.stride(0), ddelta.stride(1)
-    if dz is not None:
-        p.dz_bs, p.dz_ds = dz.stride(0), dz.stride(1)
-    if out_z is not None:
-        p.outz_bs, p.outz_ds = out_z.stride(0), out_z.stride(1)
-    with torch.cuda.device(dev):
-        _lib.check(_lib.load().mamba1_scan_bwd(p, _lib.current_stream(dev)), "mamba1_scan_bwd")
-    dA = dA_part.sum(0)
-    dD = dD_part.sum(0) if D is not None else None
-    ddelta_bias = dbias_part.sum(0) if delta_bias is not None else None
-    return du, ddelta, dA, dB32.to(B.dtype), dC32.to(C.dtype), dD, ddelta_bias, dz, out_z
+    bufs = ScanBwdBuffers(u, delta, B, z, dims, dz, recompute_out_z)
+    scan_bwd_zero(bufs, u.device)
+    scan_bwd_launch(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, delta_softplus, bufs, dims)
+    dA = bufs.dA_part.sum(0)
+    dD = bufs.dD_part.sum(0) if D is not None else None
+    ddelta_bias = bufs.dbias_part.sum(0) if delta_bias is not None else None
+    return (bufs.du, bufs.ddelta, dA, bufs.dBC32[0].to(B.dtype), bufs.dBC32[1].to(C.dtype), dD, ddelta_bias,
+            bufs.dz, bufs.out_z)
 
 
 class SelectiveScanFn(torch.autograd.Function):
