@@ -69,8 +69,15 @@ def selective_state_update(state, x, dt, A, B, C, D=None, z=None, dt_bias=None, 
     _lib.require_gpu(state, x, dt, A, B, C, D, z, dt_bias, state_batch_indices)
     if z is not None and z.dtype != x.dtype:
         z = z.to(x.dtype)
-    if C.dtype != B.dtype:
-        C = C.to(B.dtype)
+    # The kernel takes A, D, dt_bias in fp32 and B, C, dt either in x's dtype or in fp32.
+    # (.float() of an fp32 tensor is the tensor itself, so expanded stride-0 views stay views.)
+    A = A.float()
+    D = D.float() if D is not None else None
+    dt_bias = dt_bias.float() if dt_bias is not None else None
+    if B.dtype != x.dtype or C.dtype != x.dtype:
+        B, C = B.float(), C.float()
+    if dt.dtype != x.dtype:
+        dt = dt.float()
     for t in (state, x, dt, A, B, D, dt_bias):
         if t is not None and t.dtype not in _lib.DTYPE_CODE:
             raise RuntimeError(f"selective_state_update: unsupported dtype {t.dtype}")
