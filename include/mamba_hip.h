@@ -145,6 +145,79 @@ typedef struct MambaStepParams {
 
 int ssm_state_update(const MambaStepParams *p, mamba_stream_t stream);
 
+/* ------------------------------------------------------------------------- *
+ * Mamba-2 SSD (chunked state-space-dual scan).
+ * Replaces the Triton kernels launched by _mamba_chunk_scan_combined_fwd / _bwd
+ * (reference mamba_ssm/ops/triton/ssd_combined.py:343 and :397), i.e.
+ * ssd_chunk_state.py (_chunk_cumsum_fwd :718, _chunk_state_fwd :812, ...),
+ * ssd_state_passing.py (:196, :227), ssd_bmm.py (:165, :213) and
+ * ssd_chunk_scan.py (:1259 ...).
+ *
+ * Shapes (b batch, L seqlen, H nheads, P headdim, G ngroups, N dstate,
+ * Q chunk_size, c = nchunks = ceil(L / Q)):
+ *   x, z, out, out_x, dout, dx, dz : (b, L, H, P) of `dtype`, P stride 1
+ *   B, C, dB, dC                   : (b, L, G, N) of `dtype`, N stride 1
+ *   dt, ddt                        : (b, L, H) of `dt_dtype`
+ *   A, dt_bias                     : (H) fp32;  D: (H) or (H, P) fp32 (D_has_hdim)
+ *   seq_idx                        : (b, L) int32, contiguous, nullable
+ *   initial_states                 : (b, H, P, N) fp32 contiguous, nullable
+ * fp32 workspaces, contiguous:
+ *   dt_out, dA_cumsum              : (b, H, c, Q)
+ *   states                         : (b, c, H, P, N)  chunk-local states after
+ *                                    ssd_chunk_state_fwd; state ENTERING each
+ *                                    chunk after ssd_state_passing_fwd (in place)
+ *   final_states                   : (b, H, P, N)
+ *   CB                             : (b, c, G, Q, Q)  only entries s <= l of
+ *                                    row l / column s are defined
+ * ------------------------------------------------------------------------- */
+typedef struct SsdParams {
+  int32_t batch, seqlen, nheads, headdim, dstate, ngroups, chunk_size, nchunks;
+  int32_t dtype, dt_dtype;
+  int32_t dt_softplus, D_has_hdim;
+  float dt_min, dt_max;
+
+  const void *x, *dt, *A, *B, *C;
+  const void *D, *z, *dt_bias;          /* nullable */
+  const float *initial_states;          /* nullable */
+  const int32_t *seq_idx;               /* nullable */
+  void *out;
+  void *out_x;                          /* pre-gate output, written iff z != NULL */
+  float *dt_out, *dA_cumsum, *states, *final_states, *CB;
+
+  int64_t x_bs, x_ls, x_hs;
+  int64_t z_bs, z_ls, z_hs;
+  int64_t out_bs, out_ls, out_hs;       /* out and out_x share strides */
+  int64_t B_bs, B_ls, B_gs;
+  int64_t C_bs, C_ls, C_gs;
+  int64_t dt_bs, dt_ls, dt_hs;
+
+  /* ---- backward only ---- */
+  const void *dout;
+  const float *dfinal_states;           /* nullable, (b, H, P, N) */
+  void *dx, *dz;                        /* `dtype`, contiguous (b, L, H, P) */
+  void *ddt;                            /* `dt_dtype`, contiguous (b, L, H) */
+  void *dB, *dC;                        /* `dtype`, contiguous (b, L, G, N) */
+  float *dA, *ddt_bias;                 /* (H) fp32, zero on entry */
+  float *dD;                            /* (H) or (H, P) fp32, zero on entry */
+  float *dinitial_states;               /* nullable, (b, H, P, N) fp32 */
+  /* fp32 workspaces: */
+  float *dstates;                       /* (b, c, H, P, N) */
+  float *ddA_cumsum;                    /* (b, H, c, Q), zero on entry */
+  float *ddt_out;                       /* (b, H, c, Q), zero on entry */
+  float *dCB;                           /* (b, c, G, Q, Q), zero on entry when H/G > 1 */
+  float *dB32, *dC32;                   /* (b, L, G, N), zero on entry */
+  int64_t dout_bs, dout_ls, dout_hs;
+} SsdParams;
+
+/* forward stages, in launch order */
+int ssd_chunk_cumsum_fwd(const SsdParams *p, mamba_stream_t stream);
+int ssd_chunk_state_fwd(const SsdParams *p, mamba_stream_t stream);
+int ssd_state_passing_fwd(const SsdParams *p, mamba_stream_t stream);
+int ssd_bmm_chunk_fwd(const SsdParams *p, mamba_stream_t stream);
+int ssd_chunk_scan_fwd(const SsdParams *p, mamba_stream_t stream);
+/* all five on `stream` */
+int ssd_combined_fwd(const SsdParams *p, mamba_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -42,6 +42,21 @@ class MambaStepParams(ctypes.Structure):
     )
 
 
+class SsdParams(ctypes.Structure):
+    _fields_ = (
+        [(n, c_i32) for n in ("batch", "seqlen", "nheads", "headdim", "dstate", "ngroups", "chunk_size", "nchunks",
+                              "dtype", "dt_dtype", "dt_softplus", "D_has_hdim")]
+        + [("dt_min", c_f32), ("dt_max", c_f32)]
+        + [(n, c_vp) for n in ("x", "dt", "A", "B", "C", "D", "z", "dt_bias", "initial_states", "seq_idx",
+                               "out", "out_x", "dt_out", "dA_cumsum", "states", "final_states", "CB")]
+        + [(n, c_i64) for n in ("x_bs", "x_ls", "x_hs", "z_bs", "z_ls", "z_hs", "out_bs", "out_ls", "out_hs",
+                                "B_bs", "B_ls", "B_gs", "C_bs", "C_ls", "C_gs", "dt_bs", "dt_ls", "dt_hs")]
+        + [(n, c_vp) for n in ("dout", "dfinal_states", "dx", "dz", "ddt", "dB", "dC", "dA", "ddt_bias", "dD",
+                               "dinitial_states", "dstates", "ddA_cumsum", "ddt_out", "dCB", "dB32", "dC32")]
+        + [(n, c_i64) for n in ("dout_bs", "dout_ls", "dout_hs")]
+    )
+
+
 _lib = None
 
 
@@ -65,6 +80,11 @@ def load():
     for name in ("mamba1_scan_fwd", "mamba1_scan_bwd"):
         fn = getattr(lib, name)
         fn.argtypes = [ctypes.POINTER(MambaScanParams), c_vp]
+        fn.restype = ctypes.c_int
+    for name in ("ssd_chunk_cumsum_fwd", "ssd_chunk_state_fwd", "ssd_state_passing_fwd", "ssd_bmm_chunk_fwd",
+                 "ssd_chunk_scan_fwd", "ssd_combined_fwd"):
+        fn = getattr(lib, name)
+        fn.argtypes = [ctypes.POINTER(SsdParams), c_vp]
         fn.restype = ctypes.c_int
     lib.ssm_state_update.argtypes = [ctypes.POINTER(MambaStepParams), c_vp]
     lib.ssm_state_update.restype = ctypes.c_int

@@ -1,0 +1,130 @@
+// Shared pieces of the SSD kernels: the bf16 MFMA block-GEMM core on LDS tiles
+// and the tile staging helpers.
+//
+// Block GEMM: a 256-thread workgroup (4 waves, 2 x 2) computes a 64 x 64 tile
+// D[m][n] = sum_k A[m][k] * B[n][k] in steps of 32 along k.  Both operand tiles
+// sit in LDS "k-contiguous" ([row][k], padded), which is exactly the register
+// layout v_mfma_f32_16x16x32_bf16 wants for A and for B: lane l supplies row
+// (l % 16) and the 8 k-values 8 * (l / 16) .. + 7 with one 16-byte LDS load.
+// fp32 / fp16 inputs keep their precision by splitting every operand into a
+// bf16 high part and a bf16 remainder and issuing three MFMAs
+// (hi*hi + hi*lo + lo*hi); bf16 inputs need one.
+#pragma once
+#include "common.hpp"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+
+constexpr int GB = 64;         // block tile edge (M and N)
+constexpr int GK = 32;         // k step
+constexpr int GLD = GK + 8;    // LDS row pitch in bf16 (80 bytes: conflict-free 16-byte reads)
+constexpr int GTILE = GB * GLD;
+
+DEVI uint16_t bf16_bits(float x) { return (uint16_t)f32_to_bf16_bits(x); }
+DEVI float bf16_val(uint16_t b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }
+
+template <typename T> DEVI float ldg(const void *base, int64_t idx) { return ld1<T>(static_cast<const T *>(base) + idx); }
+template <typename T> DEVI void stg(void *base, int64_t idx, float v) { st1<T>(static_cast<T *>(base) + idx, v); }
+
+DEVI float ld_dyn(const void *base, int64_t idx, int dtype) {
+  switch (dtype) {
+    case MAMBA_F32: return static_cast<const float *>(base)[idx];
+    case MAMBA_BF16: return ld1<bf16_t>(static_cast<const bf16_t *>(base) + idx);
+    default: return ld1<f16_t>(static_cast<const f16_t *>(base) + idx);
+  }
+}
+DEVI void st_dyn(void *base, int64_t idx, int dtype, float v) {
+  switch (dtype) {
+    case MAMBA_F32: static_cast<float *>(base)[idx] = v; break;
+    case MAMBA_BF16: st1<bf16_t>(static_cast<bf16_t *>(base) + idx, v); break;
+    default: st1<f16_t>(static_cast<f16_t *>(base) + idx, v); break;
+  }
+}
+
+// LDS of one block GEMM: A and B tiles, high and low parts.
+struct GemmLds {
+  uint16_t ah[GTILE], al[GTILE], bh[GTILE], bl[GTILE];
+};
+
+// Fills a 64 x 32 tile from a functor f(row, k) -> float.  K_FAST: consecutive
+// threads walk k (use when the source is contiguous along k), else along rows.
+template <bool SPLIT, bool K_FAST, typename F> DEVI void stage_tile(uint16_t *hi, uint16_t *lo, F f, int tid) {
+#pragma unroll 2
+  for (int idx = tid; idx < GB * GK; idx += 256) {
+    int r, k;
+    if (K_FAST) {
+      k = idx & (GK - 1);
+      r = idx >> 5;
+    } else {
+      r = idx & (GB - 1);
+      k = idx >> 6;
+    }
+    const float v = f(r, k);
+    const uint16_t h = bf16_bits(v);
+    hi[r * GLD + k] = h;
+    if (SPLIT) lo[r * GLD + k] = bf16_bits(v - bf16_val(h));
+  }
+}
+
+struct GemmAcc {
+  f32x4 v[2][2];
+  DEVI void zero() {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) v[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+};
+
+// One 32-deep step.  Wave (wm, wn) of the 2 x 2 grid owns rows 32*wm.. and columns 32*wn...
+template <bool SPLIT> DEVI void mma_step(GemmAcc &acc, const GemmLds &s, int wm, int wn, int lane) {
+  const int i = lane & 15, g = lane >> 4;
+  bf16x8_t a[2], b[2], al[2], bl[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    a[t] = *reinterpret_cast<const bf16x8_t *>(&s.ah[(wm * 32 + t * 16 + i) * GLD + g * 8]);
+    b[t] = *reinterpret_cast<const bf16x8_t *>(&s.bh[(wn * 32 + t * 16 + i) * GLD + g * 8]);
+    if (SPLIT) {
+      al[t] = *reinterpret_cast<const bf16x8_t *>(&s.al[(wm * 32 + t * 16 + i) * GLD + g * 8]);
+      bl[t] = *reinterpret_cast<const bf16x8_t *>(&s.bl[(wn * 32 + t * 16 + i) * GLD + g * 8]);
+    }
+  }
+#pragma unroll
+  for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+    for (int tn = 0; tn < 2; ++tn) {
+      acc.v[tm][tn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[tm], b[tn], acc.v[tm][tn], 0, 0, 0);
+      if (SPLIT) {
+        acc.v[tm][tn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[tm], bl[tn], acc.v[tm][tn], 0, 0, 0);
+        acc.v[tm][tn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al[tm], b[tn], acc.v[tm][tn], 0, 0, 0);
+      }
+    }
+}
+
+// D[m][n] += sum_{k in [k_begin, k_end)} fa(m, k) * fb(n, k) for the block's 64 x 64 tile.
+// fa / fb return 0 outside their valid ranges.  All 256 threads must call.
+template <bool SPLIT, bool A_KFAST, bool B_KFAST, typename FA, typename FB>
+DEVI void block_gemm(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, FA fa, FB fb, int tid) {
+  const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+  for (int k0 = k_begin; k0 < k_end; k0 += GK) {
+    __syncthreads();
+    stage_tile<SPLIT, A_KFAST>(s.ah, s.al, [&](int r, int k) { return fa(r, k0 + k); }, tid);
+    stage_tile<SPLIT, B_KFAST>(s.bh, s.bl, [&](int r, int k) { return fb(r, k0 + k); }, tid);
+    __syncthreads();
+    mma_step<SPLIT>(acc, s, wm, wn, lane);
+  }
+}
+
+// Visits the block tile's accumulator: value = f(m, n, value) with m, n in [0, 64).
+template <typename F> DEVI void acc_foreach(GemmAcc &acc, int tid, F f) {
+  const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+  const int i = lane & 15, g = lane >> 4;
+#pragma unroll
+  for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+    for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        acc.v[tm][tn][r] = f(wm * 32 + tm * 16 + g * 4 + r, wn * 32 + tn * 16 + i, acc.v[tm][tn][r]);
+}
+
+DEVI int cdiv(int a, int b) { return (a + b - 1) / b; }

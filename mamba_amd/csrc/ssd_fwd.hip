@@ -1,0 +1,320 @@
+// Mamba-2 SSD forward for gfx950: chunk_cumsum, chunk_state, state_passing,
+// bmm (C B^T) and chunk_scan.  The three dense contractions run on bf16 MFMA
+// through the block-GEMM core of ssd_common.hpp; the other two are small
+// streaming kernels.
+#include "ssd_common.hpp"
+
+namespace {
+
+// ------------------------------------------------------------ chunk_cumsum
+// One thread per (batch, chunk, head): dt -> (+bias, softplus, clamp), zero past
+// the end of the sequence, and the running sum of dt * A inside the chunk.
+__global__ __launch_bounds__(256) void chunk_cumsum_fwd_kernel(const SsdParams p) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int H = p.nheads, nc = p.nchunks, Q = p.chunk_size;
+  if (idx >= (int64_t)p.batch * nc * H) return;
+  const int h = idx % H, c = (idx / H) % nc, b = idx / ((int64_t)H * nc);
+  const float A = static_cast<const float *>(p.A)[h];
+  const float bias = p.dt_bias ? static_cast<const float *>(p.dt_bias)[h] : 0.f;
+  float *dt_out = p.dt_out + (((int64_t)b * H + h) * nc + c) * Q;
+  float *dA_cs = p.dA_cumsum + (((int64_t)b * H + h) * nc + c) * Q;
+  float run = 0.f;
+  for (int l = 0; l < Q; ++l) {
+    const int t = c * Q + l;
+    float dt = 0.f;
+    if (t < p.seqlen) {
+      dt = ld_dyn(p.dt, b * p.dt_bs + t * p.dt_ls + h * p.dt_hs, p.dt_dtype) + bias;
+      if (p.dt_softplus) dt = softplus_f(dt);
+      dt = fminf(fmaxf(dt, p.dt_min), p.dt_max);
+    }
+    run += dt * A;
+    dt_out[l] = dt;
+    dA_cs[l] = run;
+  }
+}
+
+DEVI bool seq_same(const int32_t *seq, int a, int b) { return seq[a] == seq[b]; }
+
+// --------------------------------------------------------------- bmm (CB)
+// CB[b, c, g, l, s] = sum_n C[l, n] B[s, n] for s-tiles at or below the l-tile,
+// zeroed where seq_idx differs.
+template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bmm_chunk_fwd_kernel(const SsdParams p) {
+  __shared__ GemmLds lds;
+  const int tid = threadIdx.x;
+  const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, G = p.ngroups;
+  // blockIdx.x enumerates the lower-triangular tile pairs (mt >= nt)
+  int mt = 0, rem = blockIdx.x;
+  while (rem > mt) { rem -= mt + 1; ++mt; }
+  const int nt = rem;
+  const int c = blockIdx.y, b = blockIdx.z / G, g = blockIdx.z % G;
+  const int t0 = c * Q;
+  const int64_t Cb = b * p.C_bs + g * p.C_gs, Bb = b * p.B_bs + g * p.B_gs;
+  GemmAcc acc;
+  acc.zero();
+  auto fa = [&](int r, int k) {
+    const int l = mt * GB + r;
+    return (l < Q && t0 + l < L && k < N) ? ldg<T>(p.C, Cb + (int64_t)(t0 + l) * p.C_ls + k) : 0.f;
+  };
+  auto fb = [&](int r, int k) {
+    const int s = nt * GB + r;
+    return (s < Q && t0 + s < L && k < N) ? ldg<T>(p.B, Bb + (int64_t)(t0 + s) * p.B_ls + k) : 0.f;
+  };
+  block_gemm<SPLIT, true, true>(acc, lds, 0, N, fa, fb, tid);
+  float *CB = p.CB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
+  const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
+  acc_foreach(acc, tid, [&](int m, int n, float v) {
+    const int l = mt * GB + m, s = nt * GB + n;
+    if (l < Q && s < Q) {
+      float o = v;
+      if (seq && (t0 + l >= L || t0 + s >= L || seq[l] != seq[s])) o = 0.f;
+      CB[(int64_t)l * Q + s] = o;
+    }
+    return v;
+  });
+}
+
+// ------------------------------------------------------------ chunk_state
+// states[b, c, h, p, n] = sum_s x[s, p] B[s, n] exp(a_last - a_s) dt_s over the
+// positions s of the chunk that belong to the sequence of its last position.
+template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void chunk_state_fwd_kernel(const SsdParams p) {
+  __shared__ GemmLds lds;
+  __shared__ float w[256];
+  const int tid = threadIdx.x;
+  const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads;
+  const int ntn = cdiv(N, GB);
+  const int pt = blockIdx.x / ntn, nt = blockIdx.x % ntn;
+  const int c = blockIdx.y, b = blockIdx.z / H, h = blockIdx.z % H;
+  const int g = h / (H / p.ngroups);
+  const int t0 = c * Q;
+  const int qlim = min(Q, L - t0);
+  const float *dA = p.dA_cumsum + (((int64_t)b * H + h) * p.nchunks + c) * Q;
+  const float *dt = p.dt_out + (((int64_t)b * H + h) * p.nchunks + c) * Q;
+  const float a_last = dA[Q - 1];
+  const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
+  for (int s = tid; s < Q; s += 256) {
+    float v = 0.f;
+    if (s < qlim) {
+      bool ok = true;
+      if (seq) {
+        const int last = seq[qlim - 1];
+        ok = last >= 0 && seq[s] == last;
+      }
+      if (ok) v = fast_exp(fminf(a_last - dA[s], 0.f)) * dt[s];
+    }
+    w[s] = v;
+  }
+  const int64_t xb = b * p.x_bs + h * p.x_hs, Bb = b * p.B_bs + g * p.B_gs;
+  GemmAcc acc;
+  acc.zero();
+  auto fa = [&](int r, int k) {  // (p, s)
+    const int pp = pt * GB + r;
+    return (pp < P && k < qlim) ? ldg<T>(p.x, xb + (int64_t)(t0 + k) * p.x_ls + pp) : 0.f;
+  };
+  auto fb = [&](int r, int k) {  // (n, s)
+    const int n = nt * GB + r;
+    return (n < N && k < qlim) ? ldg<T>(p.B, Bb + (int64_t)(t0 + k) * p.B_ls + n) * w[k] : 0.f;
+  };
+  block_gemm<SPLIT, false, false>(acc, lds, 0, qlim, fa, fb, tid);  // first __syncthreads publishes w
+  float *st = p.states + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
+  acc_foreach(acc, tid, [&](int m, int n, float v) {
+    const int pp = pt * GB + m, nn = nt * GB + n;
+    if (pp < P && nn < N) st[(int64_t)pp * N + nn] = v;
+    return v;
+  });
+}
+
+// ---------------------------------------------------------- state_passing
+// In place over `states`: slot c receives the state ENTERING chunk c; the state
+// after the last chunk goes to final_states.
+__global__ __launch_bounds__(256) void state_passing_fwd_kernel(const SsdParams p) {
+  const int PN = p.headdim * p.dstate, H = p.nheads, nc = p.nchunks, Q = p.chunk_size, L = p.seqlen;
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  const int h = blockIdx.y, b = blockIdx.z;
+  if (e >= PN) return;
+  float s = p.initial_states ? p.initial_states[((int64_t)b * H + h) * PN + e] : 0.f;
+  const float *dA = p.dA_cumsum + ((int64_t)b * H + h) * nc * Q;
+  const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L : nullptr;
+  int seq_prev = 0;
+  for (int c = 0; c < nc; ++c) {
+    float *slot = p.states + (((int64_t)b * nc + c) * H + h) * PN + e;
+    const float local = *slot;
+    *slot = s;
+    float scale = fast_exp(dA[c * Q + Q - 1]);
+    if (seq) {
+      const int seq_new = seq[min((c + 1) * Q, L) - 1];
+      if (seq_new != seq_prev) scale = 0.f;
+      seq_prev = seq_new;
+    }
+    s = __builtin_fmaf(scale, s, local);
+  }
+  p.final_states[((int64_t)b * H + h) * PN + e] = s;
+}
+
+// ------------------------------------------------------------- chunk_scan
+// out[l, p] = exp(a_l) [seq_l == seq before the chunk] sum_n C[l, n] Hc[p, n]
+//           + sum_{s <= l} CB[l, s] exp(a_l - a_s) dt_s x[s, p] + D x[l, p];   out *= silu(z)
+template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void chunk_scan_fwd_kernel(const SsdParams p) {
+  __shared__ GemmLds lds;
+  __shared__ float a_s[256], dt_s[256], rscale[GB];
+  const int tid = threadIdx.x;
+  const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads, G = p.ngroups;
+  const int ntp = cdiv(P, GB);
+  const int mt = blockIdx.x / ntp, pt = blockIdx.x % ntp;
+  const int c = blockIdx.y, b = blockIdx.z / H, h = blockIdx.z % H;
+  const int g = h / (H / G);
+  const int t0 = c * Q;
+  const int qlim = min(Q, L - t0);
+  const float *dA = p.dA_cumsum + (((int64_t)b * H + h) * p.nchunks + c) * Q;
+  const float *dt = p.dt_out + (((int64_t)b * H + h) * p.nchunks + c) * Q;
+  const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
+  for (int s = tid; s < Q; s += 256) {
+    a_s[s] = dA[s];
+    dt_s[s] = dt[s];
+  }
+  if (tid < GB) {
+    const int l = mt * GB + tid;
+    float sc = 0.f;
+    if (l < qlim) {
+      bool ok = true;
+      if (seq) {
+        const int prev = c > 0 ? seq[-1] : 0;
+        ok = seq[l] == prev;
+      }
+      if (ok) sc = fast_exp(dA[l]);
+    }
+    rscale[tid] = sc;
+  }
+  const int64_t xb = b * p.x_bs + h * p.x_hs, Cb = b * p.C_bs + g * p.C_gs;
+  const float *Hc = p.states + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
+  const float *CB = p.CB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
+  GemmAcc acc;
+  acc.zero();
+  {  // carried state -> outputs
+    auto fa = [&](int r, int k) {  // (l, n)
+      const int l = mt * GB + r;
+      return (l < qlim && k < N) ? ldg<T>(p.C, Cb + (int64_t)(t0 + l) * p.C_ls + k) : 0.f;
+    };
+    auto fb = [&](int r, int k) {  // (p, n)
+      const int pp = pt * GB + r;
+      return (pp < P && k < N) ? Hc[(int64_t)pp * N + k] : 0.f;
+    };
+    block_gemm<SPLIT, true, true>(acc, lds, 0, N, fa, fb, tid);
+    acc_foreach(acc, tid, [&](int m, int n, float v) { return v * rscale[m]; });
+  }
+  {  // inside the chunk, causal
+    const int kmax = min((mt + 1) * GB, qlim);
+    auto fa = [&](int r, int k) {  // (l, s)
+      const int l = mt * GB + r;
+      if (l >= qlim || k > l) return 0.f;
+      return CB[(int64_t)l * Q + k] * fast_exp(fminf(a_s[l] - a_s[k], 0.f)) * dt_s[k];
+    };
+    auto fb = [&](int r, int k) {  // (p, s)
+      const int pp = pt * GB + r;
+      return (pp < P && k < qlim) ? ldg<T>(p.x, xb + (int64_t)(t0 + k) * p.x_ls + pp) : 0.f;
+    };
+    block_gemm<SPLIT, true, false>(acc, lds, 0, kmax, fa, fb, tid);
+  }
+  const float *Dp = static_cast<const float *>(p.D);
+  acc_foreach(acc, tid, [&](int m, int n, float v) {
+    const int l = mt * GB + m, pp = pt * GB + n;
+    if (l >= qlim || pp >= P) return v;
+    float o = v;
+    if (Dp) {
+      const float d = p.D_has_hdim ? Dp[h * P + pp] : Dp[h];
+      o = __builtin_fmaf(d, ldg<T>(p.x, xb + (int64_t)(t0 + l) * p.x_ls + pp), o);
+    }
+    const int64_t oi = b * p.out_bs + (int64_t)(t0 + l) * p.out_ls + h * p.out_hs + pp;
+    if (p.z) {
+      stg<T>(p.out_x, oi, o);
+      const float z = ldg<T>(p.z, b * p.z_bs + (int64_t)(t0 + l) * p.z_ls + h * p.z_hs + pp);
+      o *= z * sigmoid_f(z);
+    }
+    stg<T>(p.out, oi, o);
+    return v;
+  });
+}
+
+// ------------------------------------------------------------------ launch
+int check(const SsdParams *p) {
+  if (!p || !p->x || !p->dt || !p->A || !p->B || !p->C) return MAMBA_E_BADARG;
+  if (p->batch <= 0 || p->seqlen <= 0 || p->nheads <= 0 || p->headdim <= 0 || p->dstate <= 0 || p->ngroups <= 0 ||
+      p->chunk_size <= 0)
+    return MAMBA_E_BADARG;
+  if (p->nheads % p->ngroups != 0) return MAMBA_E_BADARG;
+  if (p->nchunks != (p->seqlen + p->chunk_size - 1) / p->chunk_size) return MAMBA_E_BADARG;
+  if (p->chunk_size > 256 || p->dstate > 256 || p->headdim > 256) return MAMBA_E_UNSUPPORTED;
+  if ((int64_t)p->batch * p->nheads > 65535 || p->nchunks > 65535) return MAMBA_E_UNSUPPORTED;
+  if (p->dtype != MAMBA_F32 && p->dtype != MAMBA_BF16 && p->dtype != MAMBA_F16) return MAMBA_E_BADARG;
+  if (p->dt_dtype != MAMBA_F32 && p->dt_dtype != MAMBA_BF16 && p->dt_dtype != MAMBA_F16) return MAMBA_E_BADARG;
+  return MAMBA_OK;
+}
+int launched() { return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH; }
+
+#define SSD_DISPATCH(KERNEL, GRID)                                                                   \
+  switch (p->dtype) {                                                                                \
+    case MAMBA_BF16: hipLaunchKernelGGL((KERNEL<bf16_t, false>), GRID, dim3(256), 0, s, *p); break;  \
+    case MAMBA_F16: hipLaunchKernelGGL((KERNEL<f16_t, true>), GRID, dim3(256), 0, s, *p); break;     \
+    default: hipLaunchKernelGGL((KERNEL<float, true>), GRID, dim3(256), 0, s, *p); break;            \
+  }
+
+}  // namespace
+
+extern "C" int ssd_chunk_cumsum_fwd(const SsdParams *p, mamba_stream_t stream) {
+  int rc = check(p);
+  if (rc) return rc;
+  if (!p->dt_out || !p->dA_cumsum) return MAMBA_E_BADARG;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t n = (int64_t)p->batch * p->nchunks * p->nheads;
+  hipLaunchKernelGGL(chunk_cumsum_fwd_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, *p);
+  return launched();
+}
+
+extern "C" int ssd_bmm_chunk_fwd(const SsdParams *p, mamba_stream_t stream) {
+  int rc = check(p);
+  if (rc) return rc;
+  if (!p->CB) return MAMBA_E_BADARG;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int nt = (p->chunk_size + GB - 1) / GB;
+  dim3 grid(nt * (nt + 1) / 2, p->nchunks, p->batch * p->ngroups);
+  SSD_DISPATCH(bmm_chunk_fwd_kernel, grid)
+  return launched();
+}
+
+extern "C" int ssd_chunk_state_fwd(const SsdParams *p, mamba_stream_t stream) {
+  int rc = check(p);
+  if (rc) return rc;
+  if (!p->states || !p->dt_out || !p->dA_cumsum) return MAMBA_E_BADARG;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  dim3 grid(((p->headdim + GB - 1) / GB) * ((p->dstate + GB - 1) / GB), p->nchunks, p->batch * p->nheads);
+  SSD_DISPATCH(chunk_state_fwd_kernel, grid)
+  return launched();
+}
+
+extern "C" int ssd_state_passing_fwd(const SsdParams *p, mamba_stream_t stream) {
+  int rc = check(p);
+  if (rc) return rc;
+  if (!p->states || !p->final_states || !p->dA_cumsum) return MAMBA_E_BADARG;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  dim3 grid((p->headdim * p->dstate + 255) / 256, p->nheads, p->batch);
+  hipLaunchKernelGGL(state_passing_fwd_kernel, grid, dim3(256), 0, s, *p);
+  return launched();
+}
+
+extern "C" int ssd_chunk_scan_fwd(const SsdParams *p, mamba_stream_t stream) {
+  int rc = check(p);
+  if (rc) return rc;
+  if (!p->states || !p->CB || !p->out || !p->dt_out || !p->dA_cumsum || (p->z && !p->out_x)) return MAMBA_E_BADARG;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  dim3 grid(((p->chunk_size + GB - 1) / GB) * ((p->headdim + GB - 1) / GB), p->nchunks, p->batch * p->nheads);
+  SSD_DISPATCH(chunk_scan_fwd_kernel, grid)
+  return launched();
+}
+
+extern "C" int ssd_combined_fwd(const SsdParams *p, mamba_stream_t stream) {
+  int rc;
+  if ((rc = ssd_chunk_cumsum_fwd(p, stream))) return rc;
+  if ((rc = ssd_chunk_state_fwd(p, stream))) return rc;
+  if ((rc = ssd_state_passing_fwd(p, stream))) return rc;
+  if ((rc = ssd_bmm_chunk_fwd(p, stream))) return rc;
+  return ssd_chunk_scan_fwd(p, stream);
+}

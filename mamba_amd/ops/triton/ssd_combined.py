@@ -1,0 +1,170 @@
+"""Mamba-2 SSD chunked scan: drop-in for mamba_ssm.ops.triton.ssd_combined.
+
+Same entry point, argument meaning, return arity and error behaviour as the reference
+(mamba_ssm/ops/triton/ssd_combined.py:628 mamba_chunk_scan_combined, :596
+MambaChunkScanCombinedFn, :343/:397 the forward/backward orchestration).  The Triton kernels
+are replaced by the HIP kernels behind the C ABI's ssd_* entry points.  The module path keeps
+the reference's `triton` package name so that imports stay source compatible.
+"""
+import math
+
+import torch
+
+from mamba_amd import _lib
+
+
+def _fill_fwd(p, x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, seq_idx, dt_softplus, dt_limit, ws):
+    batch, seqlen, nheads, headdim = x.shape
+    _, _, ngroups, dstate = B.shape
+    p.batch, p.seqlen, p.nheads, p.headdim, p.dstate, p.ngroups = batch, seqlen, nheads, headdim, dstate, ngroups
+    p.chunk_size, p.nchunks = chunk_size, ws["nchunks"]
+    p.dtype, p.dt_dtype = _lib.DTYPE_CODE[x.dtype], _lib.DTYPE_CODE[dt.dtype]
+    p.dt_softplus = int(bool(dt_softplus))
+    p.D_has_hdim = int(D is not None and D.dim() == 2)
+    p.dt_min, p.dt_max = float(dt_limit[0]), float(min(dt_limit[1], 3.0e38))
+    p.x, p.dt, p.A, p.B, p.C = x.data_ptr(), dt.data_ptr(), A.data_ptr(), B.data_ptr(), C.data_ptr()
+    p.D, p.z, p.dt_bias = _lib.ptr(D), _lib.ptr(z), _lib.ptr(dt_bias)
+    p.initial_states, p.seq_idx = _lib.ptr(initial_states), _lib.ptr(seq_idx)
+    p.dt_out, p.dA_cumsum = ws["dt_out"].data_ptr(), ws["dA_cumsum"].data_ptr()
+    p.states, p.final_states, p.CB = ws["states"].data_ptr(), ws["final_states"].data_ptr(), ws["CB"].data_ptr()
+    p.x_bs, p.x_ls, p.x_hs = x.stride(0), x.stride(1), x.stride(2)
+    if z is not None:
+        p.z_bs, p.z_ls, p.z_hs = z.stride(0), z.stride(1), z.stride(2)
+    p.B_bs, p.B_ls, p.B_gs = B.stride(0), B.stride(1), B.stride(2)
+    p.C_bs, p.C_ls, p.C_gs = C.stride(0), C.stride(1), C.stride(2)
+    p.dt_bs, p.dt_ls, p.dt_hs = dt.stride()
+
+
+def _prepare(x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, seq_idx):
+    """Shape checks and layout fixes of ssd_combined.py:344-369, then dtype normalisation."""
+    batch, seqlen, nheads, headdim = x.shape
+    _, _, ngroups, dstate = B.shape
+    assert nheads % ngroups == 0
+    assert B.shape == (batch, seqlen, ngroups, dstate)
+    assert dt.shape == (batch, seqlen, nheads)
+    assert A.shape == (nheads,)
+    assert C.shape == B.shape
+    if z is not None:
+        assert z.shape == x.shape
+    if D is not None:
+        assert D.shape == (nheads, headdim) or D.shape == (nheads,)
+    if seq_idx is not None:
+        assert seq_idx.shape == (batch, seqlen)
+    if initial_states is not None:
+        assert initial_states.shape == (batch, nheads, headdim, dstate)
+    _lib.require_gpu(x, dt, A, B, C, D, z, dt_bias, initial_states, seq_idx)
+    if x.dtype not in _lib.DTYPE_CODE:
+        raise RuntimeError(f"mamba_chunk_scan_combined: unsupported dtype {x.dtype}")
+    lim = _lib.load().mamba_hip_query
+    if chunk_size > 256 or dstate > lim(3) or headdim > lim(4):
+        raise RuntimeError("mamba_chunk_scan_combined: chunk_size, dstate and headdim are limited to 256")
+    if B.stride(-1) != 1:
+        B = B.contiguous()
+    if C.stride(-1) != 1:
+        C = C.contiguous()
+    if x.stride(-1) != 1:
+        x = x.contiguous()
+    if z is not None and z.stride(-1) != 1:
+        z = z.contiguous()
+    B, C = B.to(x.dtype), C.to(x.dtype)
+    z = z.to(x.dtype) if z is not None else None
+    if dt.dtype not in _lib.DTYPE_CODE:
+        dt = dt.float()
+    A = A.float().contiguous()
+    D = D.float().contiguous() if D is not None else None
+    dt_bias = dt_bias.float().contiguous() if dt_bias is not None else None
+    initial_states = initial_states.float().contiguous() if initial_states is not None else None
+    if seq_idx is not None:
+        seq_idx = seq_idx.to(torch.int32).contiguous()
+    return x, dt, A, B, C, D, z, dt_bias, initial_states, seq_idx
+
+
+def _workspace(x, B, chunk_size):
+    batch, seqlen, nheads, headdim = x.shape
+    ngroups, dstate = B.shape[2], B.shape[3]
+    nchunks = math.ceil(seqlen / chunk_size)
+    f32 = dict(device=x.device, dtype=torch.float32)
+    return dict(
+        nchunks=nchunks,
+        dt_out=torch.empty(batch, nheads, nchunks, chunk_size, **f32),
+        dA_cumsum=torch.empty(batch, nheads, nchunks, chunk_size, **f32),
+        states=torch.empty(batch, nchunks, nheads, headdim, dstate, **f32),
+        final_states=torch.empty(batch, nheads, headdim, dstate, **f32),
+        CB=torch.empty(batch, nchunks, ngroups, chunk_size, chunk_size, **f32),
+    )
+
+
+def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initial_states=None,
+                                   seq_idx=None, cu_seqlens=None, dt_softplus=False, dt_limit=(0.0, float("inf")),
+                                   state_dtype=None):
+    """Counterpart of ssd_combined.py:343.  Returns (out, out_x, dt_out, dA_cumsum, states, final_states)
+    where `states[:, c]` is the state entering chunk c, in fp32."""
+    x, dt, A, B, C, D, z, dt_bias, initial_states, seq_idx = _prepare(
+        x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, seq_idx)
+    if cu_seqlens is not None:
+        raise NotImplementedError("return_varlen_states (chunk_state_varlen) is not built in mamba_amd")
+    ws = _workspace(x, B, chunk_size)
+    out = torch.empty_like(x, memory_format=torch.contiguous_format)
+    out_x = torch.empty_like(out) if z is not None else None
+    p = _lib.SsdParams()
+    _fill_fwd(p, x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, seq_idx, dt_softplus, dt_limit, ws)
+    p.out, p.out_x = out.data_ptr(), _lib.ptr(out_x)
+    p.out_bs, p.out_ls, p.out_hs = out.stride(0), out.stride(1), out.stride(2)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().ssd_combined_fwd(p, _lib.current_stream(x.device)), "ssd_combined_fwd")
+    return out, out_x, ws["dt_out"], ws["dA_cumsum"], ws["states"], ws["final_states"]
+
+
+class MambaChunkScanCombinedFn(torch.autograd.Function):
+
+    @staticmethod
+    def forward(ctx, x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initial_states=None, seq_idx=None,
+                cu_seqlens=None, dt_softplus=False, dt_limit=(0.0, float("inf")), return_final_states=False,
+                return_varlen_states=False, state_dtype=None):
+        ctx.dt_dtype = dt.dtype
+        if not return_varlen_states:
+            cu_seqlens = None
+        else:
+            assert cu_seqlens is not None, "cu_seqlens must be provided if return_varlen_states is True"
+        out, out_x, dt_out, dA_cumsum, states, final_states = _mamba_chunk_scan_combined_fwd(
+            x, dt, A, B, C, chunk_size, D=D, z=z, dt_bias=dt_bias, initial_states=initial_states, seq_idx=seq_idx,
+            cu_seqlens=cu_seqlens, dt_softplus=dt_softplus, dt_limit=dt_limit, state_dtype=state_dtype)
+        ctx.save_for_backward(out if z is None else out_x, x, dt, dA_cumsum, A, B, C, D, z, dt_bias, initial_states,
+                              seq_idx)
+        ctx.dt_softplus = dt_softplus
+        ctx.chunk_size = chunk_size
+        ctx.dt_limit = dt_limit
+        ctx.return_final_states = return_final_states
+        ctx.return_varlen_states = return_varlen_states
+        return out if not return_final_states else (out, final_states)
+
+    @staticmethod
+    def backward(ctx, dout, *args):
+        raise NotImplementedError("SSD backward is being built")
+
+
+def mamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initial_states=None,
+                              seq_idx=None, cu_seqlens=None, dt_softplus=False, dt_limit=(0.0, float("inf")),
+                              return_final_states=False, return_varlen_states=False, state_dtype=None):
+    """
+    Argument:
+        x: (batch, seqlen, nheads, headdim)
+        dt: (batch, seqlen, nheads)
+        A: (nheads)
+        B: (batch, seqlen, ngroups, dstate)
+        C: (batch, seqlen, ngroups, dstate)
+        chunk_size: int
+        D: (nheads, headdim) or (nheads,)
+        z: (batch, seqlen, nheads, headdim)
+        dt_bias: (nheads,)
+        initial_states: (batch, nheads, headdim, dstate)
+        seq_idx: (batch, seqlen)
+        cu_seqlens: (num_sequences + 1) or None, only used if return_varlen_states is True
+        dt_softplus: Whether to apply softplus to dt
+        state_dtype: accepted for compatibility; inter-chunk states are kept in fp32
+    Return:
+        out: (batch, seqlen, nheads, headdim) [, final_states (batch, nheads, headdim, dstate) fp32]
+    """
+    return MambaChunkScanCombinedFn.apply(x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, seq_idx,
+                                          cu_seqlens, dt_softplus, dt_limit, return_final_states,
+                                          return_varlen_states, state_dtype)

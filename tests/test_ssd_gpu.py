@@ -1,0 +1,72 @@
+"""GPU parity of the SSD chunked scan (mamba_chunk_scan_combined) against the CPU oracle.
+
+The reference has no test that compares this op with a reference function (its test_ssd.py
+imports the refs but never calls them); the cases below follow the shapes of its generation
+and determinism tests and of the benchmark configurations, with the tolerances the benchmark
+states: fp32 (6e-4, 2e-3), bf16 (3e-2, 5e-2).
+"""
+import pytest
+import torch
+
+from oracle.ssd import ssd_oracle, ssd_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+def _tol(dtype):
+    return (6e-4, 2e-3) if dtype == torch.float32 else ((3e-3, 5e-3) if dtype == torch.float16 else (3e-2, 5e-2))
+
+
+def _close(name, got, ref, rtol, atol):
+    got, ref = got.detach().float().cpu(), ref.detach().float().cpu()
+    err = (got - ref).abs()
+    bound = atol + rtol * ref.abs()
+    assert bool((err <= bound).all()), (
+        f"{name}: max err {err.max().item():.3e}, worst excess {(err - bound).max().item():.3e}, "
+        f"ref max {ref.abs().max().item():.3e}")
+
+
+def _fwd_case(batch, seqlen, nheads, headdim, dstate, ngroups, chunk, dtype, seq_lens=None, has_init=False,
+              has_z=True, has_D=True, D_has_hdim=False, dt_limit=(0.0, float("inf")), seed=0):
+    from mamba_amd.ops.triton.ssd_combined import mamba_chunk_scan_combined
+    t = ssd_inputs(batch, seqlen, nheads, headdim, dstate, ngroups, dtype, seed, has_z=has_z, has_D=has_D,
+                   D_has_hdim=D_has_hdim, seq_lens=seq_lens, has_init=has_init)
+    rtol, atol = _tol(dtype)
+    out_ref, fin_ref = ssd_oracle(t["x"], t["dt"], t["A"], t["B"], t["C"], D=t["D"], z=t["z"], dt_bias=t["dt_bias"],
+                                  initial_states=t["initial_states"], seq_idx=t["seq_idx"], dt_softplus=True,
+                                  dt_limit=dt_limit, return_final_states=True)
+    cu = lambda v: None if v is None else v.cuda()
+    out, fin = mamba_chunk_scan_combined(cu(t["x"]), cu(t["dt"]), cu(t["A"]), cu(t["B"]), cu(t["C"]), chunk,
+                                         D=cu(t["D"]), z=cu(t["z"]), dt_bias=cu(t["dt_bias"]),
+                                         initial_states=cu(t["initial_states"]), seq_idx=cu(t["seq_idx"]),
+                                         dt_softplus=True, dt_limit=dt_limit, return_final_states=True)
+    assert out.dtype == dtype and out.shape == out_ref.shape and fin.dtype == torch.float32
+    _close("out", out, out_ref, rtol, atol)
+    _close("final_states", fin, fin_ref, rtol, atol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("seqlen,chunk", [(256, 64), (300, 128), (1024, 256), (77, 256), (512, 32)])
+def test_ssd_fwd_basic(seqlen, chunk, dtype):
+    _fwd_case(2, seqlen, 4, 64, 32, 2, chunk, dtype)
+
+
+@pytest.mark.parametrize("headdim,dstate,ngroups", [(64, 128, 1), (128, 64, 4), (32, 16, 1), (48, 40, 2), (64, 256, 1)])
+def test_ssd_fwd_shapes(headdim, dstate, ngroups):
+    _fwd_case(1, 384, 4, headdim, dstate, ngroups, 128, torch.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_ssd_fwd_options(dtype):
+    _fwd_case(2, 320, 4, 64, 32, 1, 64, dtype, has_init=True)
+    _fwd_case(2, 320, 4, 64, 32, 1, 64, dtype, has_z=False)
+    _fwd_case(2, 320, 4, 64, 32, 1, 64, dtype, has_D=False)
+    _fwd_case(2, 320, 4, 64, 32, 1, 64, dtype, D_has_hdim=True)
+    _fwd_case(2, 320, 4, 64, 32, 1, 64, dtype, dt_limit=(0.01, 0.05))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_ssd_fwd_packed_sequences(dtype):
+    # sequence boundaries inside chunks, on chunk edges, and a first sequence seeded by initial_states
+    _fwd_case(1, 1024, 8, 64, 64, 8, 256, dtype, seq_lens=[100, 156, 256, 300, 212], has_init=True)
+    _fwd_case(2, 640, 4, 32, 32, 2, 128, dtype, seq_lens=[1, 127, 129, 383], has_init=False)
