@@ -206,6 +206,7 @@ typedef struct SsdParams {
   float *ddt_out;                       /* (b, H, c, Q), zero on entry */
   float *dCB;                           /* (b, c, G, Q, Q), zero on entry when H/G > 1 */
   float *dB32, *dC32;                   /* (b, L, G, N), zero on entry */
+  void *gbuf;                           /* (b, L, H, P) of `dtype`: dout * silu(z); used iff z != NULL */
   int64_t dout_bs, dout_ls, dout_hs;
 } SsdParams;
 
@@ -217,6 +218,31 @@ int ssd_bmm_chunk_fwd(const SsdParams *p, mamba_stream_t stream);
 int ssd_chunk_scan_fwd(const SsdParams *p, mamba_stream_t stream);
 /* all five on `stream` */
 int ssd_combined_fwd(const SsdParams *p, mamba_stream_t stream);
+
+/* Backward.  Inputs: the forward inputs, dout, dfinal_states, the saved pre-gate
+ * output in out_x (z != NULL) or out (z == NULL), and the forward workspaces
+ * dt_out, dA_cumsum, CB, states re-computed by the forward stages 1-4.
+ * ssd_combined_bwd runs, in order:
+ *   ssd_bwd_dz        dz, gbuf = dout silu(z), dD, and the <g, y - D x> part of ddA_cumsum
+ *   ssd_bwd_dstates   dstates[c] = direct gradient of the state entering chunk c
+ *   ssd_state_passing_bwd  reverse recurrence over chunks (in place on dstates -> gradient
+ *                     of the chunk-local states), dinitial_states, ddA_cumsum at chunk ends
+ *   ssd_bwd_dx        dx, ddt_out (direct part) and the matching ddA_cumsum terms
+ *   ssd_bwd_dBC_state state-path parts of dB32 / dC32
+ *   ssd_bwd_dcb       dCB
+ *   ssd_bmm_chunk_bwd dB32 / dC32 += dCB contractions
+ *   ssd_chunk_cumsum_bwd  ddt, dA, ddt_bias from ddA_cumsum and ddt_out
+ * ddA_cumsum holds the gradient with respect to the cumulative sums a_l; the last
+ * stage turns it into the gradient of the per-position dt * A. */
+int ssd_bwd_dz(const SsdParams *p, mamba_stream_t stream);
+int ssd_bwd_dstates(const SsdParams *p, mamba_stream_t stream);
+int ssd_state_passing_bwd(const SsdParams *p, mamba_stream_t stream);
+int ssd_bwd_dx(const SsdParams *p, mamba_stream_t stream);
+int ssd_bwd_dBC_state(const SsdParams *p, mamba_stream_t stream);
+int ssd_bwd_dcb(const SsdParams *p, mamba_stream_t stream);
+int ssd_bmm_chunk_bwd(const SsdParams *p, mamba_stream_t stream);
+int ssd_chunk_cumsum_bwd(const SsdParams *p, mamba_stream_t stream);
+int ssd_combined_bwd(const SsdParams *p, mamba_stream_t stream);
 
 #ifdef __cplusplus
 }

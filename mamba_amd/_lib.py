@@ -52,7 +52,7 @@ class SsdParams(ctypes.Structure):
         + [(n, c_i64) for n in ("x_bs", "x_ls", "x_hs", "z_bs", "z_ls", "z_hs", "out_bs", "out_ls", "out_hs",
                                 "B_bs", "B_ls", "B_gs", "C_bs", "C_ls", "C_gs", "dt_bs", "dt_ls", "dt_hs")]
         + [(n, c_vp) for n in ("dout", "dfinal_states", "dx", "dz", "ddt", "dB", "dC", "dA", "ddt_bias", "dD",
-                               "dinitial_states", "dstates", "ddA_cumsum", "ddt_out", "dCB", "dB32", "dC32")]
+                               "dinitial_states", "dstates", "ddA_cumsum", "ddt_out", "dCB", "dB32", "dC32", "gbuf")]
         + [(n, c_i64) for n in ("dout_bs", "dout_ls", "dout_hs")]
     )
 
@@ -82,7 +82,9 @@ def load():
         fn.argtypes = [ctypes.POINTER(MambaScanParams), c_vp]
         fn.restype = ctypes.c_int
     for name in ("ssd_chunk_cumsum_fwd", "ssd_chunk_state_fwd", "ssd_state_passing_fwd", "ssd_bmm_chunk_fwd",
-                 "ssd_chunk_scan_fwd", "ssd_combined_fwd"):
+                 "ssd_chunk_scan_fwd", "ssd_combined_fwd", "ssd_bwd_dz", "ssd_bwd_dstates",
+                 "ssd_state_passing_bwd", "ssd_bwd_dx", "ssd_bwd_dBC_state", "ssd_bwd_dcb", "ssd_bmm_chunk_bwd",
+                 "ssd_chunk_cumsum_bwd", "ssd_combined_bwd"):
         fn = getattr(lib, name)
         fn.argtypes = [ctypes.POINTER(SsdParams), c_vp]
         fn.restype = ctypes.c_int

@@ -1,0 +1,640 @@
+// Mamba-2 SSD backward for gfx950.  Dense contractions run on the bf16 MFMA
+// block-GEMM core of ssd_common.hpp.
+//
+// Gradient of the decay exponents: every kernel adds its share of dL/da_l (a_l =
+// running sum of dt * A inside the chunk) into ddA_cumsum; the last kernel turns
+// that into dL/d(dt_l A) with a reverse running sum.  The shares are
+//   inside the chunk, w[l, s] = (g_l . x_s) dt_s CB[l, s] exp(a_l - a_s):  + row sums at l,
+//     - column sums at s, both taken from the same fp32 w so that pairs cancel in the
+//     reverse running sum (the shortcut <g_l, y_l> from the stored output does not: its
+//     rounding error is summed coherently over the chunk);
+//   carried state:  + sum_n dC_state[l, n] C[l, n] at l;
+//   chunk state:    - dt_s <x_s, state part of the dx accumulator> at s, + the same at the
+//     chunk end;  state passing:  + scale <G, H> at the chunk end;
+// with g = dout * silu(z).
+#include "ssd_common.hpp"
+
+namespace {
+
+struct View4 {  // (b, L, H, P) tensor, P stride 1
+  const void *ptr;
+  int64_t bs, ls, hs;
+};
+DEVI View4 g_view(const SsdParams &p) {
+  if (p.z) return {p.gbuf, (int64_t)p.seqlen * p.nheads * p.headdim, (int64_t)p.nheads * p.headdim, p.headdim};
+  return {p.dout, p.dout_bs, p.dout_ls, p.dout_hs};
+}
+
+DEVI float *chunk_row(float *base, const SsdParams &p, int b, int h, int c) {
+  return base + (((int64_t)b * p.nheads + h) * p.nchunks + c) * p.chunk_size;
+}
+
+// Sums acc[m][n] * fx(m, n) over n for every row m of the block tile into rows[64] (LDS, zeroed
+// here).  All 256 threads call; rows[] is valid after the trailing barrier.
+template <typename F> DEVI void row_dot(GemmAcc &acc, float *rows, int tid, F fx) {
+  const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+  const int i = lane & 15, g = lane >> 4;
+  __syncthreads();
+  if (tid < GB) rows[tid] = 0.f;
+  __syncthreads();
+#pragma unroll
+  for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int m = wm * 32 + tm * 16 + g * 4 + r;
+      float s = 0.f;
+#pragma unroll
+      for (int tn = 0; tn < 2; ++tn) s += acc.v[tm][tn][r] * fx(m, wn * 32 + tn * 16 + i);
+      s += dpp_f<DPP_ROW_SHR + 1>(0.f, s);
+      s += dpp_f<DPP_ROW_SHR + 2>(0.f, s);
+      s += dpp_f<DPP_ROW_SHR + 4>(0.f, s);
+      s += dpp_f<DPP_ROW_SHR + 8>(0.f, s);
+      if (i == 15) __hip_atomic_fetch_add(&rows[m], s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+  __syncthreads();
+}
+
+// Row sums and column sums of the block tile held in acc, into rows[64] / cols[64] (LDS).
+DEVI void row_col_sums(GemmAcc &acc, float *rows, float *cols, int tid) {
+  const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+  const int i = lane & 15, g = lane >> 4;
+  __syncthreads();
+  if (tid < GB) {
+    rows[tid] = 0.f;
+    cols[tid] = 0.f;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float s = acc.v[tm][0][r] + acc.v[tm][1][r];
+      s += dpp_f<DPP_ROW_SHR + 1>(0.f, s);
+      s += dpp_f<DPP_ROW_SHR + 2>(0.f, s);
+      s += dpp_f<DPP_ROW_SHR + 4>(0.f, s);
+      s += dpp_f<DPP_ROW_SHR + 8>(0.f, s);
+      if (i == 15)
+        __hip_atomic_fetch_add(&rows[wm * 32 + tm * 16 + g * 4 + r], s, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+#pragma unroll
+  for (int tn = 0; tn < 2; ++tn) {
+    float s = 0.f;
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) s += acc.v[tm][tn][r];
+    s += __shfl_xor(s, 16, 64);
+    s += __shfl_xor(s, 32, 64);
+    if (g == 0)
+      __hip_atomic_fetch_add(&cols[wn * 32 + tn * 16 + i], s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  }
+  __syncthreads();
+}
+
+// ------------------------------------------------------------------- dz
+// Per position: dz, g = dout silu(z), dD += g x.
+template <typename T> __global__ __launch_bounds__(256) void bwd_dz_kernel(const SsdParams p) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int L = p.seqlen, H = p.nheads, P = p.headdim;
+  const int h = blockIdx.y, b = blockIdx.z;
+  const float *Dp = static_cast<const float *>(p.D);
+  const void *yptr = p.z ? p.out_x : p.out;
+  float dDacc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < 16; ++j) {
+    const int t = blockIdx.x * 64 + wave + 4 * j;
+    if (t >= L) break;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int pp = lane + 64 * q;
+      if (pp >= P) break;
+      const float dout = ldg<T>(p.dout, b * p.dout_bs + (int64_t)t * p.dout_ls + h * p.dout_hs + pp);
+      const float x = ldg<T>(p.x, b * p.x_bs + (int64_t)t * p.x_ls + h * p.x_hs + pp);
+      float g = dout;
+      if (p.z) {
+        const float y = ldg<T>(yptr, b * p.out_bs + (int64_t)t * p.out_ls + h * p.out_hs + pp);
+        const float z = ldg<T>(p.z, b * p.z_bs + (int64_t)t * p.z_ls + h * p.z_hs + pp);
+        const float sg = sigmoid_f(z);
+        g = dout * z * sg;
+        const int64_t oi = (((int64_t)b * L + t) * H + h) * P + pp;
+        stg<T>(p.dz, oi, dout * y * sg * (1.f + z * (1.f - sg)));
+        stg<T>(p.gbuf, oi, g);
+      }
+      dDacc[q] = __builtin_fmaf(g, x, dDacc[q]);
+    }
+  }
+  if (Dp) {
+    if (p.D_has_hdim) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int pp = lane + 64 * q;
+        if (pp < P) unsafeAtomicAdd(p.dD + h * P + pp, dDacc[q]);
+      }
+    } else {
+      const float s = wave_sum(dDacc[0] + dDacc[1] + dDacc[2] + dDacc[3]);
+      if (lane == 0) unsafeAtomicAdd(p.dD + h, s);
+    }
+  }
+}
+
+// -------------------------------------------------------------- dstates
+// dstates[b, c, h, p, n] = sum_l g[l, p] exp(a_l) [seq_l == seq before the chunk] C[l, n]
+template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dstates_kernel(const SsdParams p) {
+  __shared__ GemmLds lds;
+  __shared__ float rs[256];
+  const int tid = threadIdx.x;
+  const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads;
+  const int ntn = cdiv(N, GB);
+  const int pt = blockIdx.x / ntn, nt = blockIdx.x % ntn;
+  const int c = blockIdx.y, b = blockIdx.z / H, h = blockIdx.z % H;
+  const int g = h / (H / p.ngroups);
+  const int t0 = c * Q, qlim = min(Q, L - t0);
+  const float *dA = chunk_row(p.dA_cumsum, p, b, h, c);
+  const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
+  for (int l = tid; l < Q; l += 256) {
+    float v = 0.f;
+    if (l < qlim) {
+      bool ok = true;
+      if (seq) ok = seq[l] == (c > 0 ? seq[-1] : 0);
+      if (ok) v = fast_exp(dA[l]);
+    }
+    rs[l] = v;
+  }
+  const View4 gv = g_view(p);
+  const int64_t gb = b * gv.bs + h * gv.hs, Cb = b * p.C_bs + g * p.C_gs;
+  GemmAcc acc;
+  acc.zero();
+  auto fa = [&](int r, int k) {  // (p, l)
+    const int pp = pt * GB + r;
+    return (pp < P && k < qlim) ? ldg<T>(gv.ptr, gb + (int64_t)(t0 + k) * gv.ls + pp) : 0.f;
+  };
+  auto fb = [&](int r, int k) {  // (n, l)
+    const int n = nt * GB + r;
+    return (n < N && k < qlim) ? ldg<T>(p.C, Cb + (int64_t)(t0 + k) * p.C_ls + n) * rs[k] : 0.f;
+  };
+  block_gemm<SPLIT, false, false>(acc, lds, 0, qlim, fa, fb, tid);
+  float *ds = p.dstates + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
+  acc_foreach(acc, tid, [&](int m, int n, float v) {
+    const int pp = pt * GB + m, nn = nt * GB + n;
+    if (pp < P && nn < N) ds[(int64_t)pp * N + nn] = v;
+    return v;
+  });
+}
+
+// ---------------------------------------------------- state_passing bwd
+// Reverse recurrence over chunks.  On entry dstates[c] is the direct gradient of the state
+// entering chunk c; on exit it is the gradient of chunk c's local state.
+__global__ __launch_bounds__(256) void state_passing_bwd_kernel(const SsdParams p) {
+  const int PN = p.headdim * p.dstate, H = p.nheads, nc = p.nchunks, Q = p.chunk_size, L = p.seqlen;
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int h = blockIdx.y, b = blockIdx.z;
+  const bool live = e < PN;
+  float G = (live && p.dfinal_states) ? p.dfinal_states[((int64_t)b * H + h) * PN + e] : 0.f;
+  const float *dA = p.dA_cumsum + ((int64_t)b * H + h) * nc * Q;
+  const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L : nullptr;
+  for (int c = nc - 1; c >= 0; --c) {
+    const int64_t off = (((int64_t)b * nc + c) * H + h) * PN + e;
+    float scale = fast_exp(dA[c * Q + Q - 1]);
+    if (seq) {
+      const int end_c = seq[min((c + 1) * Q, L) - 1];
+      const int end_prev = c > 0 ? seq[c * Q - 1] : 0;
+      if (end_c != end_prev) scale = 0.f;
+    }
+    float part = 0.f, direct = 0.f;
+    if (live) {
+      direct = p.dstates[off];
+      p.dstates[off] = G;
+      part = G * p.states[off] * scale;
+    }
+    part = wave_sum(part);
+    if (lane == 0 && part != 0.f) unsafeAtomicAdd(p.ddA_cumsum + (((int64_t)b * H + h) * nc + c) * Q + Q - 1, part);
+    G = __builtin_fmaf(scale, G, direct);
+  }
+  if (live && p.dinitial_states) p.dinitial_states[((int64_t)b * H + h) * PN + e] = G;
+}
+
+// ------------------------------------------------------------------- dx
+// acc[s, p] = exp(a_last - a_s) [s in the chunk's last sequence] sum_n B[s, n] dS[p, n]
+//           + sum_{l >= s} CB[l, s] exp(a_l - a_s) g[l, p]
+// dx = dt_s acc + D g;  ddt_out[s] += <x_s, acc_s>;  chunk-state terms of ddA_cumsum.
+template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_kernel(const SsdParams p) {
+  __shared__ GemmLds lds;
+  __shared__ float a_s[256], dt_s[256], wrow[GB], r1[GB], r2[GB];
+  const int tid = threadIdx.x;
+  const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads, G = p.ngroups;
+  const int ntp = cdiv(P, GB);
+  const int st = blockIdx.x / ntp, pt = blockIdx.x % ntp;
+  const int c = blockIdx.y, b = blockIdx.z / H, h = blockIdx.z % H;
+  const int g = h / (H / G);
+  const int t0 = c * Q, qlim = min(Q, L - t0);
+  const float *dA = chunk_row(p.dA_cumsum, p, b, h, c);
+  const float *dt = chunk_row(p.dt_out, p, b, h, c);
+  const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
+  const float a_last = dA[Q - 1];
+  for (int s = tid; s < Q; s += 256) {
+    a_s[s] = dA[s];
+    dt_s[s] = dt[s];
+  }
+  if (tid < GB) {
+    const int s = st * GB + tid;
+    float v = 0.f;
+    if (s < qlim) {
+      bool ok = true;
+      if (seq) {
+        const int last = seq[qlim - 1];
+        ok = last >= 0 && seq[s] == last;
+      }
+      if (ok) v = fast_exp(fminf(a_last - dA[s], 0.f));
+    }
+    wrow[tid] = v;
+  }
+  const View4 gv = g_view(p);
+  const int64_t gb = b * gv.bs + h * gv.hs, xb = b * p.x_bs + h * p.x_hs, Bb = b * p.B_bs + g * p.B_gs;
+  const float *dS = p.dstates + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
+  const float *CB = p.CB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
+  auto fx = [&](int m, int n) {
+    const int s = st * GB + m, pp = pt * GB + n;
+    return (s < qlim && pp < P) ? ldg<T>(p.x, xb + (int64_t)(t0 + s) * p.x_ls + pp) : 0.f;
+  };
+  GemmAcc acc;
+  acc.zero();
+  {
+    auto fa = [&](int r, int k) {  // (s, n)
+      const int s = st * GB + r;
+      return (s < qlim && k < N) ? ldg<T>(p.B, Bb + (int64_t)(t0 + s) * p.B_ls + k) : 0.f;
+    };
+    auto fb = [&](int r, int k) {  // (p, n)
+      const int pp = pt * GB + r;
+      return (pp < P && k < N) ? dS[(int64_t)pp * N + k] : 0.f;
+    };
+    block_gemm<SPLIT, true, true>(acc, lds, 0, N, fa, fb, tid);
+    acc_foreach(acc, tid, [&](int m, int n, float v) { return v * wrow[m]; });
+    row_dot(acc, r1, tid, fx);  // state-path part of <x_s, acc_s>
+  }
+  {
+    auto fa = [&](int r, int k) {  // (s, l)
+      const int s = st * GB + r;
+      if (s >= qlim || k >= qlim || k < s) return 0.f;
+      return CB[(int64_t)k * Q + s] * fast_exp(fminf(a_s[k] - a_s[s], 0.f));
+    };
+    auto fb = [&](int r, int k) {  // (p, l)
+      const int pp = pt * GB + r;
+      return (pp < P && k < qlim) ? ldg<T>(gv.ptr, gb + (int64_t)(t0 + k) * gv.ls + pp) : 0.f;
+    };
+    block_gemm<SPLIT, false, false>(acc, lds, st * GB, qlim, fa, fb, tid);
+    row_dot(acc, r2, tid, fx);  // full <x_s, acc_s>
+  }
+  if (tid < GB) {
+    const int s = st * GB + tid;
+    if (s < qlim) {
+      unsafeAtomicAdd(chunk_row(p.ddt_out, p, b, h, c) + s, r2[tid]);
+      float *dda = chunk_row(p.ddA_cumsum, p, b, h, c);
+      unsafeAtomicAdd(dda + s, -dt_s[s] * r1[tid]);
+      unsafeAtomicAdd(dda + Q - 1, dt_s[s] * r1[tid]);
+    }
+  }
+  const float *Dp = static_cast<const float *>(p.D);
+  acc_foreach(acc, tid, [&](int m, int n, float v) {
+    const int s = st * GB + m, pp = pt * GB + n;
+    if (s >= qlim || pp >= P) return v;
+    float o = v * dt_s[s];
+    if (Dp) {
+      const float d = p.D_has_hdim ? Dp[h * P + pp] : Dp[h];
+      o = __builtin_fmaf(d, ldg<T>(gv.ptr, gb + (int64_t)(t0 + s) * gv.ls + pp), o);
+    }
+    stg<T>(p.dx, (((int64_t)b * L + t0 + s) * H + h) * P + pp, o);
+    return v;
+  });
+}
+
+// ---------------------------------------------- state-path parts of dB, dC
+// dB32[s, n] += exp(a_last - a_s) dt_s [s in last sequence] sum_p x[s, p] dS[p, n]
+// dC32[l, n] += exp(a_l) [seq_l == seq before the chunk]    sum_p g[l, p] Hc[p, n]
+template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dBC_state_kernel(const SsdParams p) {
+  __shared__ GemmLds lds;
+  __shared__ float wB[GB], wC[GB], rsum[GB];
+  const int tid = threadIdx.x;
+  const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads, G = p.ngroups;
+  const int ntn = cdiv(N, GB);
+  const int st = blockIdx.x / ntn, nt = blockIdx.x % ntn;
+  const int c = blockIdx.y, b = blockIdx.z / H, h = blockIdx.z % H;
+  const int g = h / (H / G);
+  const int t0 = c * Q, qlim = min(Q, L - t0);
+  const float *dA = chunk_row(p.dA_cumsum, p, b, h, c);
+  const float *dt = chunk_row(p.dt_out, p, b, h, c);
+  const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
+  if (tid < GB) {
+    const int s = st * GB + tid;
+    float vb = 0.f, vc = 0.f;
+    if (s < qlim) {
+      bool okb = true, okc = true;
+      if (seq) {
+        const int last = seq[qlim - 1];
+        okb = last >= 0 && seq[s] == last;
+        okc = seq[s] == (c > 0 ? seq[-1] : 0);
+      }
+      if (okb) vb = fast_exp(fminf(dA[Q - 1] - dA[s], 0.f)) * dt[s];
+      if (okc) vc = fast_exp(dA[s]);
+    }
+    wB[tid] = vb;
+    wC[tid] = vc;
+  }
+  const View4 gv = g_view(p);
+  const int64_t gb = b * gv.bs + h * gv.hs, xb = b * p.x_bs + h * p.x_hs;
+  const float *dS = p.dstates + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
+  const float *Hc = p.states + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
+  auto fstate = [&](const float *S) {
+    return [=](int r, int k) {  // (n, p)
+      const int n = nt * GB + r;
+      return (n < N && k < P) ? S[(int64_t)k * N + n] : 0.f;
+    };
+  };
+  {
+    GemmAcc acc;
+    acc.zero();
+    auto fa = [&](int r, int k) {  // (s, p)
+      const int s = st * GB + r;
+      return (s < qlim && k < P) ? ldg<T>(p.x, xb + (int64_t)(t0 + s) * p.x_ls + k) : 0.f;
+    };
+    block_gemm<SPLIT, true, false>(acc, lds, 0, P, fa, fstate(dS), tid);
+    acc_foreach(acc, tid, [&](int m, int n, float v) {
+      const int s = st * GB + m, nn = nt * GB + n;
+      if (s < qlim && nn < N) unsafeAtomicAdd(p.dB32 + (((int64_t)b * L + t0 + s) * G + g) * N + nn, v * wB[m]);
+      return v;
+    });
+  }
+  {
+    GemmAcc acc;
+    acc.zero();
+    auto fa = [&](int r, int k) {  // (l, p)
+      const int l = st * GB + r;
+      return (l < qlim && k < P) ? ldg<T>(gv.ptr, gb + (int64_t)(t0 + l) * gv.ls + k) : 0.f;
+    };
+    block_gemm<SPLIT, true, false>(acc, lds, 0, P, fa, fstate(Hc), tid);
+    acc_foreach(acc, tid, [&](int m, int n, float v) {
+      const int l = st * GB + m, nn = nt * GB + n;
+      const float o = v * wC[m];
+      if (l < qlim && nn < N) unsafeAtomicAdd(p.dC32 + (((int64_t)b * L + t0 + l) * G + g) * N + nn, o);
+      return o;
+    });
+    const int64_t Cb = b * p.C_bs + g * p.C_gs;
+    row_dot(acc, rsum, tid, [&](int m, int n) {
+      const int l = st * GB + m, nn = nt * GB + n;
+      return (l < qlim && nn < N) ? ldg<T>(p.C, Cb + (int64_t)(t0 + l) * p.C_ls + nn) : 0.f;
+    });
+    if (tid < GB && st * GB + tid < qlim)
+      unsafeAtomicAdd(chunk_row(p.ddA_cumsum, p, b, h, c) + st * GB + tid, rsum[tid]);
+  }
+}
+
+// ------------------------------------------------------------------ dCB
+// dCB[b, c, g, l, s] += (sum_p g[l, p] x[s, p]) dt_s exp(a_l - a_s)   for l >= s in one sequence
+template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dcb_kernel(const SsdParams p) {
+  __shared__ GemmLds lds;
+  __shared__ float rows[GB], cols[GB];
+  const int tid = threadIdx.x;
+  const int Q = p.chunk_size, L = p.seqlen, P = p.headdim, H = p.nheads, G = p.ngroups;
+  int lt = 0, rem = blockIdx.x;
+  while (rem > lt) { rem -= lt + 1; ++lt; }
+  const int st = rem;
+  const int c = blockIdx.y, b = blockIdx.z / H, h = blockIdx.z % H;
+  const int g = h / (H / G);
+  const int t0 = c * Q, qlim = min(Q, L - t0);
+  const float *dA = chunk_row(p.dA_cumsum, p, b, h, c);
+  const float *dt = chunk_row(p.dt_out, p, b, h, c);
+  const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
+  const View4 gv = g_view(p);
+  const int64_t gb = b * gv.bs + h * gv.hs, xb = b * p.x_bs + h * p.x_hs;
+  GemmAcc acc;
+  acc.zero();
+  auto fa = [&](int r, int k) {  // (l, p)
+    const int l = lt * GB + r;
+    return (l < qlim && k < P) ? ldg<T>(gv.ptr, gb + (int64_t)(t0 + l) * gv.ls + k) : 0.f;
+  };
+  auto fb = [&](int r, int k) {  // (s, p)
+    const int s = st * GB + r;
+    return (s < qlim && k < P) ? ldg<T>(p.x, xb + (int64_t)(t0 + s) * p.x_ls + k) : 0.f;
+  };
+  block_gemm<SPLIT, true, true>(acc, lds, 0, P, fa, fb, tid);
+  float *dCB = p.dCB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
+  const float *CB = p.CB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
+  // acc <- w[l, s] = dCB_h[l, s] CB[l, s]
+  acc_foreach(acc, tid, [&](int m, int n, float v) {
+    const int l = lt * GB + m, s = st * GB + n;
+    if (l < qlim && s <= l && (!seq || seq[l] == seq[s])) {
+      const float d = v * dt[s] * fast_exp(fminf(dA[l] - dA[s], 0.f));
+      unsafeAtomicAdd(dCB + (int64_t)l * Q + s, d);
+      return d * CB[(int64_t)l * Q + s];
+    }
+    return 0.f;
+  });
+  row_col_sums(acc, rows, cols, tid);
+  if (tid < GB) {
+    float *dda = chunk_row(p.ddA_cumsum, p, b, h, c);
+    const int l = lt * GB + tid, s = st * GB + tid;
+    if (l < qlim && rows[tid] != 0.f) unsafeAtomicAdd(dda + l, rows[tid]);
+    if (s < qlim && cols[tid] != 0.f) unsafeAtomicAdd(dda + s, -cols[tid]);
+  }
+}
+
+// ------------------------------------------------------------- bmm bwd
+// dC32[l, n] += sum_{s <= l} dCB[l, s] B[s, n];   dB32[s, n] += sum_{l >= s} dCB[l, s] C[l, n]
+template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bmm_chunk_bwd_kernel(const SsdParams p) {
+  __shared__ GemmLds lds;
+  const int tid = threadIdx.x;
+  const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, G = p.ngroups;
+  const int ntn = cdiv(N, GB);
+  const int mt = blockIdx.x / ntn, nt = blockIdx.x % ntn;
+  const int c = blockIdx.y, b = blockIdx.z / G, g = blockIdx.z % G;
+  const int t0 = c * Q, qlim = min(Q, L - t0);
+  const float *dCB = p.dCB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
+  const int64_t Cb = b * p.C_bs + g * p.C_gs, Bb = b * p.B_bs + g * p.B_gs;
+  {
+    GemmAcc acc;
+    acc.zero();
+    auto fa = [&](int r, int k) {  // (l, s)
+      const int l = mt * GB + r;
+      return (l < qlim && k <= l) ? dCB[(int64_t)l * Q + k] : 0.f;
+    };
+    auto fb = [&](int r, int k) {  // (n, s)
+      const int n = nt * GB + r;
+      return (n < N && k < qlim) ? ldg<T>(p.B, Bb + (int64_t)(t0 + k) * p.B_ls + n) : 0.f;
+    };
+    block_gemm<SPLIT, true, false>(acc, lds, 0, min((mt + 1) * GB, qlim), fa, fb, tid);
+    acc_foreach(acc, tid, [&](int m, int n, float v) {
+      const int l = mt * GB + m, nn = nt * GB + n;
+      if (l < qlim && nn < N) p.dC32[(((int64_t)b * L + t0 + l) * G + g) * N + nn] += v;
+      return v;
+    });
+  }
+  {
+    GemmAcc acc;
+    acc.zero();
+    auto fa = [&](int r, int k) {  // (s, l)
+      const int s = mt * GB + r;
+      return (s < qlim && k < qlim && k >= s) ? dCB[(int64_t)k * Q + s] : 0.f;
+    };
+    auto fb = [&](int r, int k) {  // (n, l)
+      const int n = nt * GB + r;
+      return (n < N && k < qlim) ? ldg<T>(p.C, Cb + (int64_t)(t0 + k) * p.C_ls + n) : 0.f;
+    };
+    block_gemm<SPLIT, false, false>(acc, lds, mt * GB, qlim, fa, fb, tid);
+    acc_foreach(acc, tid, [&](int m, int n, float v) {
+      const int s = mt * GB + m, nn = nt * GB + n;
+      if (s < qlim && nn < N) p.dB32[(((int64_t)b * L + t0 + s) * G + g) * N + nn] += v;
+      return v;
+    });
+  }
+}
+
+// --------------------------------------------------------- cumsum bwd
+// One thread per (batch, chunk, head): reverse running sum of dL/da -> dL/d(dt A); then
+// the chain through A, the clamp, softplus and the bias.
+__global__ __launch_bounds__(256) void chunk_cumsum_bwd_kernel(const SsdParams p) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int H = p.nheads, nc = p.nchunks, Q = p.chunk_size, L = p.seqlen;
+  if (idx >= (int64_t)p.batch * nc * H) return;
+  const int h = idx % H, c = (idx / H) % nc, b = idx / ((int64_t)H * nc);
+  const float A = static_cast<const float *>(p.A)[h];
+  const float bias = p.dt_bias ? static_cast<const float *>(p.dt_bias)[h] : 0.f;
+  const float *dda = chunk_row(p.ddA_cumsum, p, b, h, c);
+  const float *ddt_out = chunk_row(p.ddt_out, p, b, h, c);
+  const float *dt_out = chunk_row(p.dt_out, p, b, h, c);
+  float run = 0.f, dAsum = 0.f, dbias = 0.f;
+  for (int l = Q - 1; l >= 0; --l) {
+    const int t = c * Q + l;
+    run += dda[l];
+    if (t >= L) continue;
+    float ddt = __builtin_fmaf(run, A, ddt_out[l]);
+    dAsum = __builtin_fmaf(run, dt_out[l], dAsum);
+    const int64_t di = b * p.dt_bs + (int64_t)t * p.dt_ls + h * p.dt_hs;
+    const float raw = ld_dyn(p.dt, di, p.dt_dtype) + bias;
+    const float v = p.dt_softplus ? softplus_f(raw) : raw;
+    if (v < p.dt_min || v > p.dt_max) ddt = 0.f;
+    if (p.dt_softplus && raw <= 20.f) ddt *= sigmoid_f(raw);
+    st_dyn(p.ddt, ((int64_t)b * L + t) * H + h, p.dt_dtype, ddt);
+    dbias += ddt;
+  }
+  unsafeAtomicAdd(p.dA + h, dAsum);
+  if (p.ddt_bias) unsafeAtomicAdd(p.ddt_bias + h, dbias);
+}
+
+int check_bwd(const SsdParams *p) {
+  if (!p || !p->x || !p->dt || !p->A || !p->B || !p->C || !p->dout) return MAMBA_E_BADARG;
+  if (p->batch <= 0 || p->seqlen <= 0 || p->nheads <= 0 || p->headdim <= 0 || p->dstate <= 0 || p->ngroups <= 0 ||
+      p->chunk_size <= 0 || p->nheads % p->ngroups != 0)
+    return MAMBA_E_BADARG;
+  if (p->nchunks != (p->seqlen + p->chunk_size - 1) / p->chunk_size) return MAMBA_E_BADARG;
+  if (p->chunk_size > 256 || p->dstate > 256 || p->headdim > 256) return MAMBA_E_UNSUPPORTED;
+  if ((int64_t)p->batch * p->nheads > 65535 || p->nchunks > 65535) return MAMBA_E_UNSUPPORTED;
+  if (p->dtype != MAMBA_F32 && p->dtype != MAMBA_BF16 && p->dtype != MAMBA_F16) return MAMBA_E_BADARG;
+  if (!p->dt_out || !p->dA_cumsum || !p->states || !p->CB || !p->dstates || !p->ddA_cumsum || !p->ddt_out ||
+      !p->dCB || !p->dB32 || !p->dC32 || !p->dx || !p->ddt || !p->dA)
+    return MAMBA_E_BADARG;
+  if (p->z && (!p->dz || !p->gbuf || !p->out_x)) return MAMBA_E_BADARG;
+  if (!p->z && !p->out) return MAMBA_E_BADARG;
+  if (p->D && !p->dD) return MAMBA_E_BADARG;
+  return MAMBA_OK;
+}
+int launched() { return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH; }
+
+#define SSD_DISPATCH(KERNEL, GRID)                                                                   \
+  switch (p->dtype) {                                                                                \
+    case MAMBA_BF16: hipLaunchKernelGGL((KERNEL<bf16_t, false>), GRID, dim3(256), 0, s, *p); break;  \
+    case MAMBA_F16: hipLaunchKernelGGL((KERNEL<f16_t, true>), GRID, dim3(256), 0, s, *p); break;     \
+    default: hipLaunchKernelGGL((KERNEL<float, true>), GRID, dim3(256), 0, s, *p); break;            \
+  }
+
+inline int tiles(int n) { return (n + GB - 1) / GB; }
+
+}  // namespace
+
+extern "C" int ssd_bwd_dz(const SsdParams *p, mamba_stream_t stream) {
+  int rc = check_bwd(p);
+  if (rc) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  dim3 grid((p->seqlen + 63) / 64, p->nheads, p->batch);
+  switch (p->dtype) {
+    case MAMBA_BF16: hipLaunchKernelGGL(bwd_dz_kernel<bf16_t>, grid, dim3(256), 0, s, *p); break;
+    case MAMBA_F16: hipLaunchKernelGGL(bwd_dz_kernel<f16_t>, grid, dim3(256), 0, s, *p); break;
+    default: hipLaunchKernelGGL(bwd_dz_kernel<float>, grid, dim3(256), 0, s, *p); break;
+  }
+  return launched();
+}
+
+extern "C" int ssd_bwd_dstates(const SsdParams *p, mamba_stream_t stream) {
+  int rc = check_bwd(p);
+  if (rc) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  dim3 grid(tiles(p->headdim) * tiles(p->dstate), p->nchunks, p->batch * p->nheads);
+  SSD_DISPATCH(bwd_dstates_kernel, grid)
+  return launched();
+}
+
+extern "C" int ssd_state_passing_bwd(const SsdParams *p, mamba_stream_t stream) {
+  int rc = check_bwd(p);
+  if (rc) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  dim3 grid((p->headdim * p->dstate + 255) / 256, p->nheads, p->batch);
+  hipLaunchKernelGGL(state_passing_bwd_kernel, grid, dim3(256), 0, s, *p);
+  return launched();
+}
+
+extern "C" int ssd_bwd_dx(const SsdParams *p, mamba_stream_t stream) {
+  int rc = check_bwd(p);
+  if (rc) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  dim3 grid(tiles(p->chunk_size) * tiles(p->headdim), p->nchunks, p->batch * p->nheads);
+  SSD_DISPATCH(bwd_dx_kernel, grid)
+  return launched();
+}
+
+extern "C" int ssd_bwd_dBC_state(const SsdParams *p, mamba_stream_t stream) {
+  int rc = check_bwd(p);
+  if (rc) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  dim3 grid(tiles(p->chunk_size) * tiles(p->dstate), p->nchunks, p->batch * p->nheads);
+  SSD_DISPATCH(bwd_dBC_state_kernel, grid)
+  return launched();
+}
+
+extern "C" int ssd_bwd_dcb(const SsdParams *p, mamba_stream_t stream) {
+  int rc = check_bwd(p);
+  if (rc) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int nt = tiles(p->chunk_size);
+  dim3 grid(nt * (nt + 1) / 2, p->nchunks, p->batch * p->nheads);
+  SSD_DISPATCH(bwd_dcb_kernel, grid)
+  return launched();
+}
+
+extern "C" int ssd_bmm_chunk_bwd(const SsdParams *p, mamba_stream_t stream) {
+  int rc = check_bwd(p);
+  if (rc) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  dim3 grid(tiles(p->chunk_size) * tiles(p->dstate), p->nchunks, p->batch * p->ngroups);
+  SSD_DISPATCH(bmm_chunk_bwd_kernel, grid)
+  return launched();
+}
+
+extern "C" int ssd_chunk_cumsum_bwd(const SsdParams *p, mamba_stream_t stream) {
+  int rc = check_bwd(p);
+  if (rc) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t n = (int64_t)p->batch * p->nchunks * p->nheads;
+  hipLaunchKernelGGL(chunk_cumsum_bwd_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, *p);
+  return launched();
+}
+
+extern "C" int ssd_combined_bwd(const SsdParams *p, mamba_stream_t stream) {
+  int rc;
+  if ((rc = ssd_bwd_dz(p, stream))) return rc;
+  if ((rc = ssd_bwd_dstates(p, stream))) return rc;
+  if ((rc = ssd_state_passing_bwd(p, stream))) return rc;
+  if ((rc = ssd_bwd_dx(p, stream))) return rc;
+  if ((rc = ssd_bwd_dBC_state(p, stream))) return rc;
+  if ((rc = ssd_bwd_dcb(p, stream))) return rc;
+  if ((rc = ssd_bmm_chunk_bwd(p, stream))) return rc;
+  return ssd_chunk_cumsum_bwd(p, stream);
+}

@@ -115,6 +115,78 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
     return out, out_x, ws["dt_out"], ws["dA_cumsum"], ws["states"], ws["final_states"]
 
 
+def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None, z=None, dt_bias=None,
+                                   initial_states=None, dfinal_states=None, seq_idx=None, dt_softplus=False,
+                                   dt_limit=(0.0, float("inf"))):
+    """Counterpart of ssd_combined.py:397.  `out` is the saved pre-gate output (out_x) when z is given,
+    else the forward output.  Returns (dx, ddt, dA, dB, dC, dD, dz, ddt_bias, dinitial_states)."""
+    in_dtypes = (A.dtype, D.dtype if D is not None else None, dt_bias.dtype if dt_bias is not None else None,
+                 initial_states.dtype if initial_states is not None else None, B.dtype, C.dtype)
+    D_shape = D.shape if D is not None else None
+    x, dt, A, B, C, D, z, dt_bias, initial_states, seq_idx = _prepare(
+        x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, seq_idx)
+    batch, seqlen, nheads, headdim = x.shape
+    ngroups, dstate = B.shape[2], B.shape[3]
+    _lib.require_gpu(dout, out, dfinal_states)
+    if dout.stride(-1) != 1:
+        dout = dout.contiguous()
+    dout = dout.to(x.dtype)
+    out = out.to(x.dtype)
+    if out.stride(-1) != 1:
+        out = out.contiguous()
+    dev = x.device
+    ws = _workspace(x, B, chunk_size)
+    nchunks = ws["nchunks"]
+    f32 = dict(device=dev, dtype=torch.float32)
+    dx = torch.empty(batch, seqlen, nheads, headdim, device=dev, dtype=x.dtype)
+    dz = torch.empty_like(dx) if z is not None else None
+    gbuf = torch.empty_like(dx) if z is not None else None
+    ddt = torch.empty(batch, seqlen, nheads, device=dev, dtype=dt.dtype)
+    # one zeroed arena for every accumulator the kernels add into
+    sizes = dict(dA=nheads, ddt_bias=nheads, dD=(D.numel() if D is not None else 0),
+                 ddA_cumsum=batch * nheads * nchunks * chunk_size, ddt_out=batch * nheads * nchunks * chunk_size,
+                 dCB=batch * nchunks * ngroups * chunk_size * chunk_size,
+                 dB32=batch * seqlen * ngroups * dstate, dC32=batch * seqlen * ngroups * dstate)
+    arena = torch.zeros(sum(sizes.values()), **f32)
+    acc, off = {}, 0
+    for k, n in sizes.items():
+        acc[k] = arena[off:off + n]
+        off += n
+    dstates = torch.empty(batch, nchunks, nheads, headdim, dstate, **f32)
+    dinit = torch.empty(batch, nheads, headdim, dstate, **f32) if initial_states is not None else None
+    dfinal = dfinal_states.float().contiguous() if dfinal_states is not None else None
+
+    p = _lib.SsdParams()
+    _fill_fwd(p, x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, seq_idx, dt_softplus, dt_limit, ws)
+    if z is not None:
+        p.out_x = out.data_ptr()
+    else:
+        p.out = out.data_ptr()
+    p.out_bs, p.out_ls, p.out_hs = out.stride(0), out.stride(1), out.stride(2)
+    p.dout, p.dfinal_states = dout.data_ptr(), _lib.ptr(dfinal)
+    p.dout_bs, p.dout_ls, p.dout_hs = dout.stride(0), dout.stride(1), dout.stride(2)
+    p.dx, p.dz, p.ddt, p.gbuf = dx.data_ptr(), _lib.ptr(dz), ddt.data_ptr(), _lib.ptr(gbuf)
+    p.dA, p.ddt_bias = acc["dA"].data_ptr(), acc["ddt_bias"].data_ptr()
+    p.dD = acc["dD"].data_ptr() if D is not None else None
+    p.dinitial_states, p.dstates = _lib.ptr(dinit), dstates.data_ptr()
+    p.ddA_cumsum, p.ddt_out, p.dCB = acc["ddA_cumsum"].data_ptr(), acc["ddt_out"].data_ptr(), acc["dCB"].data_ptr()
+    p.dB32, p.dC32 = acc["dB32"].data_ptr(), acc["dC32"].data_ptr()
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        stream = _lib.current_stream(dev)
+        # re-compute the forward workspaces (the reference does the same, ssd_combined.py:441-448)
+        for stage in ("ssd_chunk_cumsum_fwd", "ssd_chunk_state_fwd", "ssd_state_passing_fwd", "ssd_bmm_chunk_fwd"):
+            _lib.check(getattr(lib, stage)(p, stream), stage)
+        _lib.check(lib.ssd_combined_bwd(p, stream), "ssd_combined_bwd")
+    dA = acc["dA"].to(in_dtypes[0])
+    dD = acc["dD"].view(D_shape).to(in_dtypes[1]) if D is not None else None
+    ddt_bias = acc["ddt_bias"].to(in_dtypes[2]) if dt_bias is not None else None
+    dinit_out = dinit.to(in_dtypes[3]) if dinit is not None else None
+    dB = acc["dB32"].view(batch, seqlen, ngroups, dstate).to(in_dtypes[4])
+    dC = acc["dC32"].view(batch, seqlen, ngroups, dstate).to(in_dtypes[5])
+    return dx, ddt, dA, dB, dC, dD, dz, ddt_bias, dinit_out
+
+
 class MambaChunkScanCombinedFn(torch.autograd.Function):
 
     @staticmethod
@@ -140,7 +212,14 @@ class MambaChunkScanCombinedFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dout, *args):
-        raise NotImplementedError("SSD backward is being built")
+        out, x, dt, dA_cumsum, A, B, C, D, z, dt_bias, initial_states, seq_idx = ctx.saved_tensors
+        assert not ctx.return_varlen_states, "return_varlen_states is not supported in backward"
+        dfinal_states = args[0] if ctx.return_final_states else None
+        dx, ddt, dA, dB, dC, dD, dz, ddt_bias, dinitial_states = _mamba_chunk_scan_combined_bwd(
+            dout, x, dt, A, B, C, out, ctx.chunk_size, D=D, z=z, dt_bias=dt_bias, initial_states=initial_states,
+            dfinal_states=dfinal_states, seq_idx=seq_idx, dt_softplus=ctx.dt_softplus, dt_limit=ctx.dt_limit)
+        return (dx, ddt, dA, dB, dC, None, dD, dz, ddt_bias, dinitial_states, None, None, None, None, None, None,
+                None)
 
 
 def mamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initial_states=None,

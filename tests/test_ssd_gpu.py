@@ -70,3 +70,64 @@ def test_ssd_fwd_packed_sequences(dtype):
     # sequence boundaries inside chunks, on chunk edges, and a first sequence seeded by initial_states
     _fwd_case(1, 1024, 8, 64, 64, 8, 256, dtype, seq_lens=[100, 156, 256, 300, 212], has_init=True)
     _fwd_case(2, 640, 4, 32, 32, 2, 128, dtype, seq_lens=[1, 127, 129, 383], has_init=False)
+
+
+def _bwd_case(batch, seqlen, nheads, headdim, dstate, ngroups, chunk, dtype, seq_lens=None, has_init=False,
+              has_z=True, has_D=True, D_has_hdim=False, dt_limit=(0.0, float("inf")), with_dfinal=True, seed=0,
+              grad_scale=1.0):
+    from mamba_amd.ops.triton.ssd_combined import mamba_chunk_scan_combined
+    t = ssd_inputs(batch, seqlen, nheads, headdim, dstate, ngroups, dtype, seed, has_z=has_z, has_D=has_D,
+                   D_has_hdim=D_has_hdim, seq_lens=seq_lens, has_init=has_init)
+    rtol, atol = _tol(dtype)
+    names = ["x", "dt", "A", "B", "C", "D", "z", "dt_bias", "initial_states"]
+    ref_in = {k: (t[k].clone().requires_grad_() if t[k] is not None else None) for k in names}
+    gpu_in = {k: (t[k].cuda().requires_grad_() if t[k] is not None else None) for k in names}
+    out_ref, fin_ref = ssd_oracle(ref_in["x"], ref_in["dt"], ref_in["A"], ref_in["B"], ref_in["C"], D=ref_in["D"],
+                                  z=ref_in["z"], dt_bias=ref_in["dt_bias"], initial_states=ref_in["initial_states"],
+                                  seq_idx=t["seq_idx"], dt_softplus=True, dt_limit=dt_limit,
+                                  return_final_states=True)
+    cu = lambda v: None if v is None else v.cuda()
+    out, fin = mamba_chunk_scan_combined(gpu_in["x"], gpu_in["dt"], gpu_in["A"], gpu_in["B"], gpu_in["C"], chunk,
+                                         D=gpu_in["D"], z=gpu_in["z"], dt_bias=gpu_in["dt_bias"],
+                                         initial_states=gpu_in["initial_states"], seq_idx=cu(t["seq_idx"]),
+                                         dt_softplus=True, dt_limit=dt_limit, return_final_states=True)
+    _close("out", out, out_ref, rtol, atol)
+    dfin = t["dfinal"] if with_dfinal else torch.zeros_like(t["dfinal"])
+    (out_ref.float() * t["dout"].float()).sum().add((fin_ref * dfin).sum()).backward()
+    (out.float() * t["dout"].cuda().float()).sum().add((fin * dfin.cuda()).sum()).backward()
+    # gradient magnitudes grow with the sequence length; scale the absolute tolerance of the
+    # reduced (weight-like) gradients with their reference magnitude
+    for k in names:
+        if ref_in[k] is None:
+            continue
+        gr, rr = gpu_in[k].grad, ref_in[k].grad
+        assert gr is not None, f"no gradient for {k}"
+        assert gr.dtype == gpu_in[k].dtype and gr.shape == gpu_in[k].shape
+        scale = max(1.0, float(rr.abs().max())) if k in ("A", "D", "dt_bias", "dt") else 1.0
+        _close("d" + k, gr, rr, rtol * 2, atol * 2 * scale * grad_scale)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("seqlen,chunk", [(256, 64), (300, 128), (512, 256), (77, 256)])
+def test_ssd_bwd_basic(seqlen, chunk, dtype):
+    _bwd_case(2, seqlen, 4, 64, 32, 2, chunk, dtype)
+
+
+@pytest.mark.parametrize("headdim,dstate,ngroups", [(64, 128, 1), (128, 64, 4), (32, 16, 1), (48, 40, 2)])
+def test_ssd_bwd_shapes(headdim, dstate, ngroups):
+    _bwd_case(1, 384, 4, headdim, dstate, ngroups, 128, torch.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_ssd_bwd_options(dtype):
+    _bwd_case(2, 320, 4, 64, 32, 1, 64, dtype, has_init=True)
+    _bwd_case(2, 320, 4, 64, 32, 1, 64, dtype, has_z=False)
+    _bwd_case(2, 320, 4, 64, 32, 1, 64, dtype, has_D=False, with_dfinal=False)
+    _bwd_case(2, 320, 4, 64, 32, 1, 64, dtype, D_has_hdim=True)
+    _bwd_case(2, 320, 4, 64, 32, 1, 64, dtype, dt_limit=(0.01, 0.05))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_ssd_bwd_packed_sequences(dtype):
+    _bwd_case(1, 1024, 8, 64, 64, 8, 256, dtype, seq_lens=[100, 156, 256, 300, 212], has_init=True)
+    _bwd_case(2, 640, 4, 32, 32, 2, 128, dtype, seq_lens=[1, 127, 129, 383], has_init=False)
