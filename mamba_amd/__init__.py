@@ -1,0 +1,36 @@
+"""mamba_amd: MI355X-native (gfx950) kernels for Mamba's scan hot path behind the reference's
+operator API.  See mamba_amd.ops.* for the drop-in entry points."""
+import sys
+import types
+
+__version__ = "0.1.0"
+
+
+def install_as_mamba_ssm_ops():
+    """Registers the drop-in modules under the reference's module paths, so that
+    `from mamba_ssm.ops.selective_scan_interface import selective_scan_fn` (and the SSD / decode
+    imports) resolve to this package.  Existing `mamba_ssm` packages are left in place; only the
+    three operator modules are replaced."""
+    from mamba_amd.ops import selective_scan_interface
+    from mamba_amd.ops.triton import selective_state_update, ssd_combined
+
+    def ensure(name):
+        if name not in sys.modules:
+            mod = types.ModuleType(name)
+            mod.__path__ = []
+            sys.modules[name] = mod
+        return sys.modules[name]
+
+    for pkg in ("mamba_ssm", "mamba_ssm.ops", "mamba_ssm.ops.triton"):
+        ensure(pkg)
+    mapping = {
+        "mamba_ssm.ops.selective_scan_interface": selective_scan_interface,
+        "mamba_ssm.ops.triton.ssd_combined": ssd_combined,
+        "mamba_ssm.ops.triton.selective_state_update": selective_state_update,
+    }
+    for name, mod in mapping.items():
+        sys.modules[name] = mod
+        parent, leaf = name.rsplit(".", 1)
+        setattr(sys.modules[parent], leaf, mod)
+    setattr(sys.modules["mamba_ssm"], "ops", sys.modules["mamba_ssm.ops"])
+    setattr(sys.modules["mamba_ssm.ops"], "triton", sys.modules["mamba_ssm.ops.triton"])

@@ -228,3 +228,224 @@ def selective_scan_fn(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta_
     considered in the backward pass (as in the reference, selective_scan_interface.py:118-124).
     """
     return SelectiveScanFn.apply(u, delta, A, B, C, D, z, delta_bias, delta_softplus, return_last_state)
+
+
+def selective_scan_ref(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta_softplus=False,
+                       return_last_state=False):
+    """Plain-PyTorch evaluation of the same recurrence on whatever device the inputs live on (the
+    role of the reference's selective_scan_ref, selective_scan_interface.py:127).  It is a utility
+    for users and is not used by any op of this package."""
+    dtype_in = u.dtype
+    u, delta = u.float(), delta.float()
+    if delta_bias is not None:
+        delta = delta + delta_bias[..., None].float()
+    if delta_softplus:
+        delta = F.softplus(delta)
+    if A.is_complex() or B.dim() < 3 or C.dim() < 3:
+        raise NotImplementedError("selective_scan_ref: complex A / input-independent B, C are not built")
+    dim = A.shape[0]
+    Bf = B.float() if B.dim() == 4 else B.float()[:, None]
+    Cf = C.float() if C.dim() == 4 else C.float()[:, None]
+    Bf = Bf.repeat_interleave(dim // Bf.shape[1], dim=1)
+    Cf = Cf.repeat_interleave(dim // Cf.shape[1], dim=1)
+    state = u.new_zeros(u.shape[0], dim, A.shape[1])
+    ys = []
+    for t in range(u.shape[2]):
+        step = delta[:, :, t, None]
+        state = torch.exp(step * A) * state + step * u[:, :, t, None] * Bf[..., t]
+        ys.append((state * Cf[..., t]).sum(-1))
+    y = torch.stack(ys, dim=2)
+    if D is not None:
+        y = y + u * D[None, :, None]
+    if z is not None:
+        y = y * F.silu(z.float())
+    y = y.to(dtype_in)
+    return y if not return_last_state else (y, state)
+
+
+# --------------------------------------------------------------------------- mamba_inner_fn
+def _causal_conv1d_silu(x, weight, bias):
+    """Depthwise causal convolution (left padding width-1) followed by SiLU: the arithmetic of the
+    un-vendored causal_conv1d package as the reference itself spells it when that package is missing
+    (mamba_ssm/modules/mamba_simple.py:168-169).  x: (b, d, L), weight: (d, w)."""
+    L = x.shape[-1]
+    y = F.conv1d(x, weight.unsqueeze(1), bias, padding=weight.shape[-1] - 1, groups=weight.shape[0])[..., :L]
+    return F.silu(y)
+
+
+def _rms_norm(x, weight, eps):
+    """x * rsqrt(mean(x^2) + eps) * weight over the last dimension (the forward of the reference's
+    rms_norm_forward, selective_scan_interface.py:98-115), in fp32, cast back to x's dtype."""
+    xf = x.float()
+    y = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
+    return y.to(x.dtype)
+
+
+def _norm_over_state(t, weight, eps, L):
+    # (b, 1, n, l) -> rows of n -> back, as selective_scan_interface.py:263-270
+    rows = rearrange(t, "b 1 dstate l -> (b l) dstate", l=L).contiguous()
+    return rearrange(_rms_norm(rows, weight, eps), "(b l) dstate -> b 1 dstate l", l=L).contiguous()
+
+
+class MambaInnerFn(torch.autograd.Function):
+    """conv1d+SiLU -> x_proj -> dt_proj -> selective scan -> out_proj with the reference's layout
+    choreography and recompute-in-backward (selective_scan_interface.py:196-383).  The scan runs on
+    the HIP kernels; the convolution and the projections are torch operators."""
+
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
+    def forward(ctx, xz, conv1d_weight, conv1d_bias, x_proj_weight, delta_proj_weight, out_proj_weight,
+                out_proj_bias, A, B=None, C=None, D=None, delta_bias=None, B_proj_bias=None, C_proj_bias=None,
+                delta_softplus=True, checkpoint_lvl=1, b_rms_weight=None, c_rms_weight=None, dt_rms_weight=None,
+                b_c_dt_rms_eps=1e-6):
+        assert checkpoint_lvl in [0, 1]
+        if A.is_complex():
+            raise NotImplementedError("mamba_inner_fn: complex A is not built in mamba_amd")
+        L = xz.shape[-1]
+        delta_rank = delta_proj_weight.shape[1]
+        d_state = A.shape[-1]
+        if torch.is_autocast_enabled():
+            ac = torch.get_autocast_gpu_dtype()
+            x_proj_weight, delta_proj_weight = x_proj_weight.to(ac), delta_proj_weight.to(ac)
+            out_proj_weight = out_proj_weight.to(ac)
+            out_proj_bias = out_proj_bias.to(ac) if out_proj_bias is not None else None
+        if xz.stride(-1) != 1:
+            xz = xz.contiguous()
+        conv1d_weight = rearrange(conv1d_weight, "d 1 w -> d w")
+        x, z = xz.chunk(2, dim=1)
+        conv1d_bias = conv1d_bias.contiguous() if conv1d_bias is not None else None
+        conv1d_out = _causal_conv1d_silu(x, conv1d_weight, conv1d_bias)
+        # delta keeps d as the slow and L as the fast dimension: what the scan kernel reads
+        x_dbl = F.linear(rearrange(conv1d_out, "b d l -> (b l) d"), x_proj_weight)
+        delta = rearrange(delta_proj_weight @ x_dbl[:, :delta_rank].t(), "d (b l) -> b d l", l=L)
+        ctx.is_variable_B, ctx.is_variable_C = B is None, C is None
+        ctx.B_proj_bias_is_None, ctx.C_proj_bias_is_None = B_proj_bias is None, C_proj_bias is None
+        if B is None:
+            B = x_dbl[:, delta_rank:delta_rank + d_state]
+            if B_proj_bias is not None:
+                B = B + B_proj_bias.to(dtype=B.dtype)
+            B = rearrange(B, "(b l) dstate -> b 1 dstate l", l=L).contiguous()
+        elif B.stride(-1) != 1:
+            B = B.contiguous()
+        if C is None:
+            C = x_dbl[:, -d_state:]
+            if C_proj_bias is not None:
+                C = C + C_proj_bias.to(dtype=C.dtype)
+            C = rearrange(C, "(b l) dstate -> b 1 dstate l", l=L).contiguous()
+        elif C.stride(-1) != 1:
+            C = C.contiguous()
+        if D is not None:
+            D = D.contiguous()
+        if b_rms_weight is not None:
+            B = _norm_over_state(B, b_rms_weight, b_c_dt_rms_eps, L)
+        if c_rms_weight is not None:
+            C = _norm_over_state(C, c_rms_weight, b_c_dt_rms_eps, L)
+        if dt_rms_weight is not None:
+            delta = rearrange(_rms_norm(rearrange(delta, "b d l -> (b l) d").contiguous(), dt_rms_weight,
+                                        b_c_dt_rms_eps), "(b l) d -> b d l", l=L).contiguous()
+        out_z, ckpt = selective_scan_fwd(conv1d_out.contiguous(), delta.contiguous(), A, B, C, D, z, delta_bias,
+                                         delta_softplus)
+        ctx.delta_softplus = delta_softplus
+        ctx.out_proj_bias_is_None = out_proj_bias is None
+        ctx.checkpoint_lvl = checkpoint_lvl
+        ctx.dt_rms_weight, ctx.rms_eps = dt_rms_weight, b_c_dt_rms_eps
+        if checkpoint_lvl >= 1:  # conv1d_out and delta are recomputed in the backward pass
+            conv1d_out, delta = None, None
+        ctx.save_for_backward(xz, conv1d_weight, conv1d_bias, x_dbl, x_proj_weight, delta_proj_weight,
+                              out_proj_weight, conv1d_out, delta, A, B, C, D, delta_bias, ckpt)
+        return F.linear(rearrange(out_z, "b d l -> b l d"), out_proj_weight, out_proj_bias)
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
+    def backward(ctx, dout):
+        (xz, conv1d_weight, conv1d_bias, x_dbl, x_proj_weight, delta_proj_weight, out_proj_weight, conv1d_out,
+         delta, A, B, C, D, delta_bias, ckpt) = ctx.saved_tensors
+        L = xz.shape[-1]
+        delta_rank = delta_proj_weight.shape[1]
+        d_state = A.shape[-1]
+        x, z = xz.chunk(2, dim=1)
+        if dout.stride(-1) != 1:
+            dout = dout.contiguous()
+        # the convolution is differentiated by torch on a local graph (recomputed when checkpointing)
+        with torch.enable_grad():
+            x_leaf = x.detach().requires_grad_()
+            w_leaf = conv1d_weight.detach().requires_grad_()
+            b_leaf = conv1d_bias.detach().requires_grad_() if conv1d_bias is not None else None
+            conv_graph = _causal_conv1d_silu(x_leaf, w_leaf, b_leaf)
+        if ctx.checkpoint_lvl == 1:
+            conv1d_out = conv_graph.detach()
+            delta = rearrange(delta_proj_weight @ x_dbl[:, :delta_rank].t(), "d (b l) -> b d l", l=L)
+            if ctx.dt_rms_weight is not None:
+                delta = rearrange(_rms_norm(rearrange(delta, "b d l -> (b l) d").contiguous(), ctx.dt_rms_weight,
+                                            ctx.rms_eps), "(b l) d -> b d l", l=L).contiguous()
+        dxz = torch.empty_like(xz)
+        dx, dz = dxz.chunk(2, dim=1)
+        dout = rearrange(dout, "b l e -> e (b l)")
+        dout_y = rearrange(out_proj_weight.t() @ dout, "d (b l) -> b d l", l=L)
+        dconv1d_out, ddelta, dA, dB, dC, dD, ddelta_bias, dz, out_z = selective_scan_bwd(
+            conv1d_out.contiguous(), delta.contiguous(), A, B, C, D, z, delta_bias, dout_y.contiguous(), ckpt, dz,
+            ctx.delta_softplus, True)
+        dout_proj_weight = torch.einsum("eB,dB->ed", dout, rearrange(out_z, "b d l -> d (b l)"))
+        dout_proj_bias = dout.sum(dim=1) if not ctx.out_proj_bias_is_None else None
+        dx_dbl = torch.empty_like(x_dbl)
+        dB_proj_bias = dC_proj_bias = None
+        if ctx.is_variable_B:
+            dB = rearrange(dB, "b 1 dstate l -> (b l) dstate").contiguous()
+            dB_proj_bias = dB.sum(0) if not ctx.B_proj_bias_is_None else None
+            dx_dbl[:, delta_rank:delta_rank + d_state] = dB
+            dB = None
+        if ctx.is_variable_C:
+            dC = rearrange(dC, "b 1 dstate l -> (b l) dstate").contiguous()
+            dC_proj_bias = dC.sum(0) if not ctx.C_proj_bias_is_None else None
+            dx_dbl[:, -d_state:] = dC
+            dC = None
+        ddelta = rearrange(ddelta, "b d l -> d (b l)")
+        ddelta_proj_weight = torch.einsum("dB,Br->dr", ddelta, x_dbl[:, :delta_rank])
+        dx_dbl[:, :delta_rank] = torch.einsum("dB,dr->Br", ddelta, delta_proj_weight)
+        dconv1d_out = rearrange(dconv1d_out, "b d l -> d (b l)")
+        dx_proj_weight = torch.einsum("Br,Bd->rd", dx_dbl, rearrange(conv1d_out, "b d l -> (b l) d"))
+        dconv1d_out = torch.addmm(dconv1d_out, x_proj_weight.t(), dx_dbl.t())
+        dconv1d_out = rearrange(dconv1d_out, "d (b l) -> b d l", b=x.shape[0], l=L)
+        leaves = [x_leaf, w_leaf] + ([b_leaf] if b_leaf is not None else [])
+        grads = torch.autograd.grad(conv_graph, leaves, dconv1d_out.to(conv_graph.dtype))
+        dx.copy_(grads[0])
+        dconv1d_weight = rearrange(grads[1], "d w -> d 1 w")
+        dconv1d_bias = grads[2] if b_leaf is not None else None
+        return (dxz, dconv1d_weight, dconv1d_bias, dx_proj_weight, ddelta_proj_weight, dout_proj_weight,
+                dout_proj_bias, dA, dB, dC, dD, ddelta_bias if delta_bias is not None else None,
+                dB_proj_bias, dC_proj_bias, None, None, None, None, None, None)
+
+
+def mamba_inner_fn(xz, conv1d_weight, conv1d_bias, x_proj_weight, delta_proj_weight, out_proj_weight, out_proj_bias,
+                   A, B=None, C=None, D=None, delta_bias=None, B_proj_bias=None, C_proj_bias=None,
+                   delta_softplus=True, checkpoint_lvl=1, b_rms_weight=None, c_rms_weight=None, dt_rms_weight=None,
+                   b_c_dt_rms_eps=1e-6):
+    return MambaInnerFn.apply(xz, conv1d_weight, conv1d_bias, x_proj_weight, delta_proj_weight, out_proj_weight,
+                              out_proj_bias, A, B, C, D, delta_bias, B_proj_bias, C_proj_bias, delta_softplus,
+                              checkpoint_lvl, b_rms_weight, c_rms_weight, dt_rms_weight, b_c_dt_rms_eps)
+
+
+def mamba_inner_ref(xz, conv1d_weight, conv1d_bias, x_proj_weight, delta_proj_weight, out_proj_weight,
+                    out_proj_bias, A, B=None, C=None, D=None, delta_bias=None, B_proj_bias=None, C_proj_bias=None,
+                    delta_softplus=True):
+    """The same block from plain torch operators and selective_scan_ref (the role of the reference's
+    mamba_inner_ref, selective_scan_interface.py:397)."""
+    L = xz.shape[-1]
+    delta_rank = delta_proj_weight.shape[1]
+    d_state = A.shape[-1]
+    x, z = xz.chunk(2, dim=1)
+    x = _causal_conv1d_silu(x, rearrange(conv1d_weight, "d 1 w -> d w"), conv1d_bias)
+    x_dbl = F.linear(rearrange(x, "b d l -> (b l) d"), x_proj_weight)
+    delta = rearrange(delta_proj_weight @ x_dbl[:, :delta_rank].t(), "d (b l) -> b d l", l=L)
+    if B is None:
+        B = x_dbl[:, delta_rank:delta_rank + d_state]
+        if B_proj_bias is not None:
+            B = B + B_proj_bias.to(dtype=B.dtype)
+        B = rearrange(B, "(b l) dstate -> b dstate l", l=L).contiguous()
+    if C is None:
+        C = x_dbl[:, -d_state:]
+        if C_proj_bias is not None:
+            C = C + C_proj_bias.to(dtype=C.dtype)
+        C = rearrange(C, "(b l) dstate -> b dstate l", l=L).contiguous()
+    y = selective_scan_ref(x, delta, A, B, C, D, z=z, delta_bias=delta_bias, delta_softplus=True)
+    return F.linear(rearrange(y, "b d l -> b l d"), out_proj_weight, out_proj_bias)

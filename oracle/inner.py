@@ -1,0 +1,42 @@
+"""Oracle for mamba_inner_fn (test infrastructure, CPU, plain PyTorch).
+
+Restates mamba_inner_ref (reference mamba_ssm/ops/selective_scan_interface.py:397-432): causal
+depthwise conv1d + SiLU, x_proj, dt_proj, selective scan, out_proj.  The convolution is the library
+routine the reference falls back to when the causal_conv1d package is missing
+(mamba_ssm/modules/mamba_simple.py:168-169); the scan is oracle.mamba1.  The reference's own test of
+this block compares two users of the same third-party conv package, so the conv boundary is pinned
+here by the library routine instead (tests/test_oracle_mamba1.py pins the scan).
+"""
+import torch
+import torch.nn.functional as F
+
+from oracle.mamba1 import selective_scan_oracle
+
+
+def mamba_inner_oracle(xz, conv1d_weight, conv1d_bias, x_proj_weight, delta_proj_weight, out_proj_weight,
+                       out_proj_bias, A, D=None, delta_bias=None, B_proj_bias=None, C_proj_bias=None,
+                       compute_dtype=torch.float32):
+    cd = compute_dtype
+    batch, two_d, L = xz.shape
+    d = two_d // 2
+    R, N = delta_proj_weight.shape[1], A.shape[1]
+    x, z = xz.to(cd)[:, :d], xz.to(cd)[:, d:]
+    w = conv1d_weight.to(cd)                                     # (d, 1, width)
+    x = F.silu(F.conv1d(x, w, None if conv1d_bias is None else conv1d_bias.to(cd), padding=w.shape[-1] - 1,
+                        groups=d)[..., :L])
+    x_dbl = x.permute(0, 2, 1).reshape(batch * L, d) @ x_proj_weight.to(cd).t()           # (b l, R + 2N)
+    delta = (delta_proj_weight.to(cd) @ x_dbl[:, :R].t()).reshape(d, batch, L).permute(1, 0, 2)
+    Bm = x_dbl[:, R:R + N]
+    Cm = x_dbl[:, R + N:R + 2 * N]
+    if B_proj_bias is not None:
+        Bm = Bm + B_proj_bias.to(cd)
+    if C_proj_bias is not None:
+        Cm = Cm + C_proj_bias.to(cd)
+    Bm = Bm.reshape(batch, L, N).permute(0, 2, 1)
+    Cm = Cm.reshape(batch, L, N).permute(0, 2, 1)
+    y = selective_scan_oracle(x, delta, A.to(cd), Bm, Cm, None if D is None else D.to(cd), z,
+                              None if delta_bias is None else delta_bias.to(cd), True, compute_dtype=cd)
+    out = y.permute(0, 2, 1) @ out_proj_weight.to(cd).t()
+    if out_proj_bias is not None:
+        out = out + out_proj_bias.to(cd)
+    return out

@@ -1,0 +1,127 @@
+"""Pins the Mamba-1 oracle (oracle/mamba1.py) without the reference: closed forms, library routines,
+brute force and gradcheck, chosen so that a dropped term, a wrong sign/index or a transposed operand
+fails at least one of them."""
+import torch
+import torch.nn.functional as F
+
+from oracle.mamba1 import selective_scan_oracle, scan_inputs
+
+f64 = torch.float64
+
+
+def test_no_decay_reduces_to_cumsum():
+    # A = 0, one state: h_t = sum_{s<=t} delta_s B_s u_s, y = h C + D u
+    g = torch.Generator().manual_seed(0)
+    b, d, L = 2, 3, 37
+    u, delta = torch.randn(b, d, L, generator=g, dtype=f64), torch.rand(b, d, L, generator=g, dtype=f64)
+    B, C = torch.randn(b, 1, L, generator=g, dtype=f64), torch.randn(b, 1, L, generator=g, dtype=f64)
+    D = torch.randn(d, generator=g, dtype=f64)
+    y = selective_scan_oracle(u, delta, torch.zeros(d, 1, dtype=f64), B, C, D, compute_dtype=f64)
+    expect = torch.cumsum(delta * u * B, dim=-1) * C + u * D[None, :, None]
+    assert torch.allclose(y, expect, atol=1e-12)
+
+
+def test_zero_step_leaves_skip_connection():
+    t = scan_inputs(2, 4, 50, 8, dtype=f64)
+    y = selective_scan_oracle(t["u"], torch.zeros_like(t["delta"]), t["A"].double(), t["B"], t["C"], t["D"].double(),
+                              compute_dtype=f64)
+    assert torch.allclose(y, t["u"] * t["D"].double()[None, :, None], atol=1e-12)
+
+
+def test_constant_coefficients_are_a_causal_convolution():
+    # constant delta, B = C = 1: y_t = sum_k delta e^{k delta A} u_{t-k}  -> F.conv1d
+    g = torch.Generator().manual_seed(1)
+    b, d, L, n = 2, 3, 40, 4
+    u = torch.randn(b, d, L, generator=g, dtype=f64)
+    A = -torch.rand(d, n, generator=g, dtype=f64) - 0.1
+    dl = 0.3
+    ones = torch.ones(b, n, L, dtype=f64)
+    y = selective_scan_oracle(u, torch.full((b, d, L), dl, dtype=f64), A, ones, ones, compute_dtype=f64)
+    k = torch.arange(L, dtype=f64)
+    kern = (dl * torch.exp(k[None, None, :] * dl * A[:, :, None])).sum(1)          # (d, L)
+    expect = F.conv1d(F.pad(u, (L - 1, 0)), kern.flip(-1)[:, None, :], groups=d)
+    assert torch.allclose(y, expect, atol=1e-10)
+
+
+def _brute(u, delta, A, B, C, D, z, bias, softplus):
+    b, d, L = u.shape
+    n = A.shape[1]
+    G = B.shape[1]
+    out = torch.zeros(b, d, L, dtype=f64)
+    last = torch.zeros(b, d, n, dtype=f64)
+    for bi in range(b):
+        for di in range(d):
+            gi = di // (d // G)
+            h = [0.0] * n
+            for t in range(L):
+                x = float(delta[bi, di, t]) + (float(bias[di]) if bias is not None else 0.0)
+                if softplus:
+                    x = float(torch.log1p(torch.exp(torch.tensor(x, dtype=f64)))) if x <= 20 else x
+                y = 0.0
+                for ni in range(n):
+                    h[ni] = float(torch.exp(torch.tensor(x * float(A[di, ni]), dtype=f64))) * h[ni] \
+                        + x * float(B[bi, gi, ni, t]) * float(u[bi, di, t])
+                    y += h[ni] * float(C[bi, gi, ni, t])
+                y += float(D[di]) * float(u[bi, di, t])
+                zz = float(z[bi, di, t])
+                out[bi, di, t] = y * zz / (1.0 + float(torch.exp(torch.tensor(-zz, dtype=f64))))
+            last[bi, di] = torch.tensor(h, dtype=f64)
+    return out, last
+
+
+def test_brute_force_with_groups_bias_softplus_gate():
+    t = scan_inputs(2, 4, 9, 3, ngroups=2, dtype=f64, seed=3)
+    A = (-torch.rand(4, 3, dtype=f64) - 0.2)
+    out, last = selective_scan_oracle(t["u"], t["delta"], A, t["B"], t["C"], t["D"].double(), t["z"],
+                                      t["delta_bias"].double() + 3.0, True, True, compute_dtype=f64)
+    eo, el = _brute(t["u"], t["delta"], A, t["B"], t["C"], t["D"].double(), t["z"], t["delta_bias"].double() + 3.0, True)
+    assert torch.allclose(out, eo, atol=1e-10) and torch.allclose(last, el, atol=1e-10)
+
+
+def test_softplus_threshold_matches_library():
+    x = torch.tensor([-30.0, -5.0, 0.0, 19.9, 20.0, 20.1, 50.0], dtype=f64)
+    ones = torch.ones(1, 1, 1, dtype=f64)
+    for v in x:
+        y = selective_scan_oracle(ones, v.reshape(1, 1, 1), torch.zeros(1, 1, dtype=f64), ones, ones,
+                                  delta_softplus=True, compute_dtype=f64)
+        assert torch.allclose(y.flatten()[0], F.softplus(v), atol=1e-12)
+
+
+def test_gradcheck_all_inputs():
+    t = scan_inputs(1, 2, 6, 2, ngroups=1, dtype=f64, seed=5)
+    A = (-torch.rand(2, 2, dtype=f64) - 0.2).requires_grad_()
+    ins = [t[k].double().clone().requires_grad_() for k in ("u", "delta")] + [A] + \
+          [t[k].double().clone().requires_grad_() for k in ("B", "C", "D", "z", "delta_bias")]
+    fn = lambda *a: selective_scan_oracle(*a, delta_softplus=True, compute_dtype=f64)
+    assert torch.autograd.gradcheck(fn, ins, eps=1e-6, atol=1e-6)
+
+
+def test_gradient_invariants():
+    t = scan_inputs(2, 4, 20, 3, ngroups=2, dtype=f64, seed=7)
+    ins = {k: (v.double().clone().requires_grad_() if v is not None else None) for k, v in t.items()}
+    out = selective_scan_oracle(ins["u"], ins["delta"], ins["A"], ins["B"], ins["C"], ins["D"], ins["z"],
+                                ins["delta_bias"], True, compute_dtype=f64)
+    out.backward(t["dout"].double())
+    # without softplus the bias gradient is the sum of the delta gradient; with it both share the chain factor
+    assert torch.allclose(ins["delta_bias"].grad, ins["delta"].grad.sum((0, 2)), atol=1e-10)
+    # channels of a group share B, C: per-channel runs add up
+    tot = torch.zeros_like(ins["B"].grad)
+    for d in range(4):
+        sub = {k: t[k].double().clone() for k in ("u", "delta", "z", "dout")}
+        Bd = t["B"].double().clone().requires_grad_()
+        o = selective_scan_oracle(sub["u"][:, d:d + 1], sub["delta"][:, d:d + 1], t["A"].double()[d:d + 1],
+                                  Bd[:, d // 2:d // 2 + 1], t["C"].double()[:, d // 2:d // 2 + 1],
+                                  t["D"].double()[d:d + 1], sub["z"][:, d:d + 1], t["delta_bias"].double()[d:d + 1],
+                                  True, compute_dtype=f64)
+        o.backward(sub["dout"][:, d:d + 1])
+        tot += Bd.grad
+    assert torch.allclose(tot, ins["B"].grad, atol=1e-10)
+
+
+def test_output_dtype_and_fp32_agreement():
+    t = scan_inputs(1, 8, 64, 16, dtype=torch.bfloat16, seed=9)
+    y32 = selective_scan_oracle(t["u"], t["delta"], t["A"], t["B"], t["C"], t["D"], t["z"], t["delta_bias"], True)
+    y64 = selective_scan_oracle(t["u"], t["delta"], t["A"], t["B"], t["C"], t["D"], t["z"], t["delta_bias"], True,
+                                compute_dtype=f64)
+    assert y32.dtype == torch.bfloat16
+    assert torch.allclose(y32.float(), y64.float(), rtol=2e-2, atol=2e-2)
