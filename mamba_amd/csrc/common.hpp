@@ -202,6 +202,55 @@ DEVI void wave_scan_rev(float &a, float &b, int lane) {
   a = a * an;
 }
 
+// The same two scans for two independent recurrences at once, with the DPP operand folded
+// into the multiply / multiply-add (v_fmac_f32_dpp, v_mul_f32_dpp).  Lanes without a DPP source
+// are left unwritten, which is the identity of the scan.  Interleaving the two chains keeps the
+// two wait states the hardware wants between a VALU write and a DPP read of the same register.
+#define MAMBA_DPP2(CTRL)                                                       \
+  "v_fmac_f32_dpp %1, %1, %0 " CTRL " bank_mask:0xf\n\t"                      \
+  "v_fmac_f32_dpp %3, %3, %2 " CTRL " bank_mask:0xf\n\t"                      \
+  "v_mul_f32_dpp %0, %0, %0 " CTRL " bank_mask:0xf\n\t"                       \
+  "v_mul_f32_dpp %2, %2, %2 " CTRL " bank_mask:0xf\n\t"
+
+DEVI void wave_scan_fwd2(float &a0, float &b0, float &a1, float &b1) {
+  asm volatile("s_nop 1\n\t"
+               MAMBA_DPP2("row_shr:1 row_mask:0xf")
+               MAMBA_DPP2("row_shr:2 row_mask:0xf")
+               MAMBA_DPP2("row_shr:4 row_mask:0xf")
+               MAMBA_DPP2("row_shr:8 row_mask:0xf")
+               MAMBA_DPP2("row_bcast:15 row_mask:0xa")
+               MAMBA_DPP2("row_bcast:31 row_mask:0xc")
+               "s_nop 1\n\t"
+               : "+v"(a0), "+v"(b0), "+v"(a1), "+v"(b1));
+}
+
+// rows only (16 lanes each), towards lane 0 of the row
+DEVI void row_scan_rev2(float &a0, float &b0, float &a1, float &b1) {
+  asm volatile("s_nop 1\n\t"
+               MAMBA_DPP2("row_shl:1 row_mask:0xf")
+               MAMBA_DPP2("row_shl:2 row_mask:0xf")
+               MAMBA_DPP2("row_shl:4 row_mask:0xf")
+               MAMBA_DPP2("row_shl:8 row_mask:0xf")
+               "s_nop 1\n\t"
+               : "+v"(a0), "+v"(b0), "+v"(a1), "+v"(b1));
+}
+#undef MAMBA_DPP2
+
+// Completes a lane-reversed scan whose rows have been scanned by row_scan_rev2: appends to every
+// row the composition of the rows after it.
+DEVI void wave_scan_rev_finish(float &a, float &b, int lane) {
+  float a1 = readlane_f(a, 16), b1 = readlane_f(b, 16);
+  float a2 = readlane_f(a, 32), b2 = readlane_f(b, 32);
+  float a3 = readlane_f(a, 48), b3 = readlane_f(b, 48);
+  float a23 = a2 * a3, b23 = __builtin_fmaf(a2, b3, b2);
+  float a123 = a1 * a23, b123 = __builtin_fmaf(a1, b23, b1);
+  int row = lane >> 4;
+  float an = row == 0 ? a123 : (row == 1 ? a23 : (row == 2 ? a3 : 1.f));
+  float bn = row == 0 ? b123 : (row == 1 ? b23 : (row == 2 ? b3 : 0.f));
+  b = __builtin_fmaf(a, bn, b);
+  a = a * an;
+}
+
 DEVI float wave_sum(float x) {
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) x += __shfl_xor(x, off, 64);

@@ -119,27 +119,37 @@ __global__ __launch_bounds__(NW * 64) void scan_fwd_kernel(const MambaScanParams
           const float *A2row = A2s + (wave * R + r) * NP + nb * NB16;
           float *hrow = hcar + (wave * R + r) * NP + nb * NB16;
           const int nmax = min(NB16, N - nb * NB16);
-          for (int n = 0; n < nmax; ++n) {
-            const float A2 = A2row[n];
-            const float hc = hrow[n];
-            float Bv[8], Cv[8], a[8], hh[8];
-            lds_ld8(Bs + n * TILE, lane, Bv);
-            lds_ld8(Cs + n * TILE, lane, Cv);
+          // two states per iteration: their wave scans are interleaved (padded rows are inert:
+          // A = 0, B = C = 0)
+          for (int n = 0; n < nmax; n += 2) {
+            float a[2][8], hh[2][8], Cv[2][8], hc[2];
 #pragma unroll
-            for (int i = 0; i < KI; ++i) a[i] = fast_exp2(dl[i] * A2);
-            hh[0] = du[0] * Bv[0];
+            for (int q = 0; q < 2; ++q) {
+              const float A2 = A2row[n + q];
+              hc[q] = hrow[n + q];
+              float Bv[8];
+              lds_ld8(Bs + (n + q) * TILE, lane, Bv);
+              lds_ld8(Cs + (n + q) * TILE, lane, Cv[q]);
 #pragma unroll
-            for (int i = 1; i < KI; ++i) {
-              hh[i] = __builtin_fmaf(a[i], hh[i - 1], du[i] * Bv[i]);
-              a[i] = a[i] * a[i - 1];  // cumulative decay inside the lane
+              for (int i = 0; i < KI; ++i) a[q][i] = fast_exp2(dl[i] * A2);
+              hh[q][0] = du[0] * Bv[0];
+#pragma unroll
+              for (int i = 1; i < KI; ++i) {
+                hh[q][i] = __builtin_fmaf(a[q][i], hh[q][i - 1], du[i] * Bv[i]);
+                a[q][i] = a[q][i] * a[q][i - 1];  // cumulative decay inside the lane
+              }
             }
-            float sa = a[KI - 1], sb = hh[KI - 1];
-            wave_scan_fwd(sa, sb);
-            const float hend = __builtin_fmaf(sa, hc, sb);  // state after this lane's last item
-            const float hx = dpp_f<DPP_WAVE_SHR1>(hc, hend);  // state entering this lane
-            if (lane == 63) hrow[n] = hend;
+            float sa0 = a[0][KI - 1], sb0 = hh[0][KI - 1], sa1 = a[1][KI - 1], sb1 = hh[1][KI - 1];
+            wave_scan_fwd2(sa0, sb0, sa1, sb1);
+            const float hend[2] = {__builtin_fmaf(sa0, hc[0], sb0), __builtin_fmaf(sa1, hc[1], sb1)};
 #pragma unroll
-            for (int i = 0; i < KI; ++i) y[i] = __builtin_fmaf(__builtin_fmaf(a[i], hx, hh[i]), Cv[i], y[i]);
+            for (int q = 0; q < 2; ++q) {
+              const float hx = dpp_f<DPP_WAVE_SHR1>(hc[q], hend[q]);  // state entering this lane
+              if (lane == 63) hrow[n + q] = hend[q];                  // state after the tile
+#pragma unroll
+              for (int i = 0; i < KI; ++i)
+                y[i] = __builtin_fmaf(__builtin_fmaf(a[q][i], hx, hh[q][i]), Cv[q][i], y[i]);
+            }
           }
         }
       }
@@ -271,78 +281,94 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
           float *arow = anx + row * NP + nb * NB16;
           float *dArow = dAacc + row * NP + nb * NB16;
           const int nmax = min(NB16, N - nb * NB16);
+          static_assert(NPP % 2 == 0, "states are processed in pairs");
           for (int ph = 0; ph < NPH; ++ph) {
             const int slot = (wave + ph) % NPH;
-            for (int j = 0; j < NPP; ++j) {
+            for (int j = 0; j < NPP; j += 2) {
               const int n = slot * NPP + j;
               if (!valid || n >= nmax) continue;
-              const float A1 = A1row[n], A2 = A1 * kLog2e;
-              const float hc = hrow[n], gc = grow[n], an = arow[n];
-              float Bv[8], Cv[8], a[8], ac[8], bb[8], h[8];
-              lds_ld8(Bs + n * TILE, lane, Bv);
-              lds_ld8(Cs + n * TILE, lane, Cv);
+              float A1[2], hc[2], gc[2], an[2];
+              float Bv[2][8], Cv[2][8], a[2][8], ac[2][8], bb[2][8], h[2][8];
 #pragma unroll
-              for (int i = 0; i < KI; ++i) {
-                a[i] = fast_exp2(dl[i] * A2);
-                bb[i] = du[i] * Bv[i];
-              }
-              h[0] = bb[0];
-              ac[0] = a[0];
+              for (int q = 0; q < 2; ++q) {
+                A1[q] = A1row[n + q];
+                hc[q] = hrow[n + q];
+                gc[q] = grow[n + q];
+                an[q] = arow[n + q];
+                lds_ld8(Bs + (n + q) * TILE, lane, Bv[q]);
+                lds_ld8(Cs + (n + q) * TILE, lane, Cv[q]);
+                const float A2 = A1[q] * kLog2e;
 #pragma unroll
-              for (int i = 1; i < KI; ++i) {
-                h[i] = __builtin_fmaf(a[i], h[i - 1], bb[i]);
-                ac[i] = ac[i - 1] * a[i];
-              }
-              float sa = ac[KI - 1], sb = h[KI - 1];
-              wave_scan_fwd(sa, sb);
-              const float hend = __builtin_fmaf(sa, hc, sb);
-              const float hx = dpp_f<DPP_WAVE_SHR1>(hc, hend);
+                for (int i = 0; i < KI; ++i) {
+                  a[q][i] = fast_exp2(dl[i] * A2);
+                  bb[q][i] = du[i] * Bv[q][i];
+                }
+                h[q][0] = bb[q][0];
+                ac[q][0] = a[q][0];
 #pragma unroll
-              for (int i = 0; i < KI; ++i) h[i] = __builtin_fmaf(ac[i], hx, h[i]);  // true states
-              if (has_z) {
+                for (int i = 1; i < KI; ++i) {
+                  h[q][i] = __builtin_fmaf(a[q][i], h[q][i - 1], bb[q][i]);
+                  ac[q][i] = ac[q][i - 1] * a[q][i];
+                }
+              }
+              float sa0 = ac[0][KI - 1], sb0 = h[0][KI - 1], sa1 = ac[1][KI - 1], sb1 = h[1][KI - 1];
+              wave_scan_fwd2(sa0, sb0, sa1, sb1);
+              const float hend[2] = {__builtin_fmaf(sa0, hc[0], sb0), __builtin_fmaf(sa1, hc[1], sb1)};
+              float gg[2][8], ar[2][8];
 #pragma unroll
-                for (int i = 0; i < KI; ++i) y[i] = __builtin_fmaf(h[i], Cv[i], y[i]);
-              }
-              // adjoint recurrence g[t] = dy[t] C[t] + a[t+1] g[t+1]
-              const float a_next_lane = dpp_f<DPP_WAVE_SHL1>(an, a[0]);
-              float gg[8], ar[8];
-              gg[KI - 1] = dy[KI - 1] * Cv[KI - 1];
-              ar[KI - 1] = a_next_lane;
+              for (int q = 0; q < 2; ++q) {
+                const float hx = dpp_f<DPP_WAVE_SHR1>(hc[q], hend[q]);
 #pragma unroll
-              for (int i = KI - 2; i >= 0; --i) {
-                gg[i] = __builtin_fmaf(a[i + 1], gg[i + 1], dy[i] * Cv[i]);
-                ar[i] = ar[i + 1] * a[i + 1];
-              }
-              float ra = ar[0], rb = gg[0];
-              wave_scan_rev(ra, rb, lane);
-              const float gfirst = __builtin_fmaf(ra, gc, rb);    // adjoint at this lane's first item
-              const float gx = dpp_f<DPP_WAVE_SHL1>(gc, gfirst);  // ... at the next lane's first item
-              if (lane == 0) {
-                grow[n] = gfirst;
-                arow[n] = a[0];
-              }
-              float dAp = 0.f;
-              float sB[8], sC[8];
-              lds_ld8(dBs + n * TILE, lane, sB);
-              lds_ld8(dCs + n * TILE, lane, sC);
+                for (int i = 0; i < KI; ++i) h[q][i] = __builtin_fmaf(ac[q][i], hx, h[q][i]);  // true states
+                if (has_z) {
 #pragma unroll
-              for (int i = 0; i < KI; ++i) {
-                const float gi = __builtin_fmaf(ar[i], gx, gg[i]);
-                sC[i] = __builtin_fmaf(dy[i], h[i], sC[i]);
-                sB[i] = __builtin_fmaf(gi, du[i], sB[i]);
-                acc[i] = __builtin_fmaf(gi, Bv[i], acc[i]);
-                const float w = gi * (h[i] - bb[i]);  // g * a * h[t-1]
-                dd[i] = __builtin_fmaf(A1, w, dd[i]);
-                dAp = __builtin_fmaf(dl[i], w, dAp);
+                  for (int i = 0; i < KI; ++i) y[i] = __builtin_fmaf(h[q][i], Cv[q][i], y[i]);
+                }
+                // adjoint recurrence g[t] = dy[t] C[t] + a[t+1] g[t+1]
+                const float a_next_lane = dpp_f<DPP_WAVE_SHL1>(an[q], a[q][0]);
+                gg[q][KI - 1] = dy[KI - 1] * Cv[q][KI - 1];
+                ar[q][KI - 1] = a_next_lane;
+#pragma unroll
+                for (int i = KI - 2; i >= 0; --i) {
+                  gg[q][i] = __builtin_fmaf(a[q][i + 1], gg[q][i + 1], dy[i] * Cv[q][i]);
+                  ar[q][i] = ar[q][i + 1] * a[q][i + 1];
+                }
               }
-              lds_st8(dBs + n * TILE, lane, sB);
-              lds_st8(dCs + n * TILE, lane, sC);
-              dAp += dpp_f<DPP_ROW_SHR + 1>(0.f, dAp);
-              dAp += dpp_f<DPP_ROW_SHR + 2>(0.f, dAp);
-              dAp += dpp_f<DPP_ROW_SHR + 4>(0.f, dAp);
-              dAp += dpp_f<DPP_ROW_SHR + 8>(0.f, dAp);
-              if ((lane & 15) == 15)
-                __hip_atomic_fetch_add(dArow + n, dAp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+              float ra0 = ar[0][0], rb0 = gg[0][0], ra1 = ar[1][0], rb1 = gg[1][0];
+              row_scan_rev2(ra0, rb0, ra1, rb1);
+              wave_scan_rev_finish(ra0, rb0, lane);
+              wave_scan_rev_finish(ra1, rb1, lane);
+              const float gfirst[2] = {__builtin_fmaf(ra0, gc[0], rb0), __builtin_fmaf(ra1, gc[1], rb1)};
+#pragma unroll
+              for (int q = 0; q < 2; ++q) {
+                const float gx = dpp_f<DPP_WAVE_SHL1>(gc[q], gfirst[q]);  // adjoint at the next lane's first item
+                if (lane == 0) {
+                  grow[n + q] = gfirst[q];
+                  arow[n + q] = a[q][0];
+                }
+                float dAp = 0.f;
+                float sB[8], sC[8];
+                lds_ld8(dBs + (n + q) * TILE, lane, sB);
+                lds_ld8(dCs + (n + q) * TILE, lane, sC);
+#pragma unroll
+                for (int i = 0; i < KI; ++i) {
+                  const float gi = __builtin_fmaf(ar[q][i], gx, gg[q][i]);
+                  sC[i] = __builtin_fmaf(dy[i], h[q][i], sC[i]);
+                  sB[i] = __builtin_fmaf(gi, du[i], sB[i]);
+                  acc[i] = __builtin_fmaf(gi, Bv[q][i], acc[i]);
+                  const float w = gi * (h[q][i] - bb[q][i]);  // g * a * h[t-1]
+                  dd[i] = __builtin_fmaf(A1[q], w, dd[i]);
+                  dAp = __builtin_fmaf(dl[i], w, dAp);
+                }
+                lds_st8(dBs + (n + q) * TILE, lane, sB);
+                lds_st8(dCs + (n + q) * TILE, lane, sC);
+                dAp += dpp_f<DPP_ROW_SHR + 1>(0.f, dAp);
+                dAp += dpp_f<DPP_ROW_SHR + 2>(0.f, dAp);
+                dAp += dpp_f<DPP_ROW_SHR + 4>(0.f, dAp);
+                dAp += dpp_f<DPP_ROW_SHR + 8>(0.f, dAp);
+                if ((lane & 15) == 15)
+                  __hip_atomic_fetch_add(dArow + n + q, dAp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+              }
             }
             __syncthreads();
           }
