@@ -53,12 +53,35 @@ def cpu_baseline(seqlen, dstate, full_dim):
                       f"{dt:.1f} s, scaled by {dim}/{full_dim}"}
 
 
+def copy_calibration(dev):
+    """Runs mamba_hip_copy (one 16-byte element per thread) over 1 GiB: 1 GiB read + 1 GiB written."""
+    import torch
+    from mamba_amd import _lib
+    nbytes = 1 << 30
+    src = torch.empty(nbytes, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    lib = _lib.load()
+    stream = _lib.current_stream(dev)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    for i in range(6):
+        if i == 1:
+            ev[0].record()
+        _lib.check(lib.mamba_hip_copy(dst.data_ptr(), src.data_ptr(), nbytes, stream), "mamba_hip_copy")
+    ev[1].record()
+    torch.cuda.synchronize()
+    ms = ev[0].elapsed_time(ev[1]) / 5
+    print(json.dumps({"kernel": "copy_kernel", "bytes_read": nbytes, "bytes_written": nbytes, "ms": ms,
+                      "GB/s": 2 * nbytes / ms / 1e6}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run the library's plain copy kernel over 1 GiB (yardstick for HBM counters)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (the scan has no cross-GPU exchange step); "
@@ -73,6 +96,9 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
+    if args.copy_calibration:
+        copy_calibration(dev)
+        return
     batch, dim, seqlen, dstate = 8, 5120, 4096, 16
     dtype = torch.bfloat16
     t = make_inputs(batch, dim, seqlen, dstate, dtype, dev)

@@ -48,6 +48,11 @@ const char *mamba_hip_strerror(int code);
  * that it can be recorded into a HIP graph. */
 int mamba_hip_zero(void *ptr, int64_t nbytes, mamba_stream_t stream);
 
+/* Plain device-to-device copy of `nbytes` (multiple of 16, 16-byte aligned pointers), one 16-byte
+ * element per thread.  It is the streaming yardstick the profiles are calibrated against: its HBM
+ * traffic is exactly 2 * nbytes. */
+int mamba_hip_copy(void *dst, const void *src, int64_t nbytes, mamba_stream_t stream);
+
 /* ------------------------------------------------------------------------- *
  * Mamba-1 selective scan.
  * Replaces selective_scan_cuda.fwd / .bwd

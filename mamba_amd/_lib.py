@@ -77,6 +77,8 @@ def load():
     lib.mamba_hip_strerror.restype = ctypes.c_char_p
     lib.mamba_hip_zero.argtypes = [c_vp, c_i64, c_vp]
     lib.mamba_hip_zero.restype = ctypes.c_int
+    lib.mamba_hip_copy.argtypes = [c_vp, c_vp, c_i64, c_vp]
+    lib.mamba_hip_copy.restype = ctypes.c_int
     for name in ("mamba1_scan_fwd", "mamba1_scan_bwd"):
         fn = getattr(lib, name)
         fn.argtypes = [ctypes.POINTER(MambaScanParams), c_vp]

@@ -7,7 +7,23 @@ __global__ __launch_bounds__(256) void zero_kernel(uint32_t *p, int64_t n) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = 0u;
 }
+__global__ __launch_bounds__(256) void copy_kernel(const u32x4 *__restrict__ src, u32x4 *__restrict__ dst, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) dst[i] = src[i];
+}
 }  // namespace
+
+extern "C" int mamba_hip_copy(void *dst, const void *src, int64_t nbytes, mamba_stream_t stream) {
+  if (nbytes == 0) return MAMBA_OK;
+  if (!dst || !src || nbytes < 0 || (nbytes & 15) || (reinterpret_cast<uintptr_t>(dst) & 15) ||
+      (reinterpret_cast<uintptr_t>(src) & 15))
+    return MAMBA_E_BADARG;
+  const int64_t n = nbytes / 16;
+  if ((n + 255) / 256 > 0x7fffffff) return MAMBA_E_UNSUPPORTED;
+  hipLaunchKernelGGL(copy_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const u32x4 *>(src), static_cast<u32x4 *>(dst), n);
+  return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
+}
 
 extern "C" int mamba_hip_query(int what) {
   switch (what) {

@@ -86,6 +86,39 @@ template <> DEVI void st8<f16_t>(f16_t *p, const float (&v)[8]) {
   *reinterpret_cast<u32x4 *>(p) = a;
 }
 
+// 8 values kept in registers in the storage format of T (exact round trip for values that were
+// loaded from T): 4 registers for 16-bit types, 8 for fp32.
+template <typename T> struct Pack8 {
+  u32x4 w;
+  DEVI void pack(const float (&v)[8]) {
+    if constexpr (DT<T>::id == MAMBA_BF16) {
+      w = u32x4{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7])};
+    } else {
+      w = u32x4{pack_f16(v[0], v[1]), pack_f16(v[2], v[3]), pack_f16(v[4], v[5]), pack_f16(v[6], v[7])};
+    }
+  }
+  DEVI void unpack(float (&o)[8]) const {
+    if constexpr (DT<T>::id == MAMBA_BF16) {
+      o[0] = bf16_lo(w.x); o[1] = bf16_hi(w.x); o[2] = bf16_lo(w.y); o[3] = bf16_hi(w.y);
+      o[4] = bf16_lo(w.z); o[5] = bf16_hi(w.z); o[6] = bf16_lo(w.w); o[7] = bf16_hi(w.w);
+    } else {
+      o[0] = f16_lo(w.x); o[1] = f16_hi(w.x); o[2] = f16_lo(w.y); o[3] = f16_hi(w.y);
+      o[4] = f16_lo(w.z); o[5] = f16_hi(w.z); o[6] = f16_lo(w.w); o[7] = f16_hi(w.w);
+    }
+  }
+};
+template <> struct Pack8<float> {
+  float v[8];
+  DEVI void pack(const float (&x)[8]) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = x[i];
+  }
+  DEVI void unpack(float (&o)[8]) const {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = v[i];
+  }
+};
+
 // 8 elements starting at p[0], of which only the first `nvalid` (0..8) exist;
 // the rest read as `fill`.  VEC: all-or-nothing 16-byte path.
 template <typename T, bool VEC> DEVI void ld8_guard(const T *p, int nvalid, float fill, float (&o)[8]) {

@@ -231,16 +231,21 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
       const bool valid = d < dend;
       const int row = wave * R + r;
       float u[8], dl[8], du[8], dy[8], acc[8], dd[8], y[8];
+      // raw delta, z and dout stay in registers in their storage format for the epilogue
+      Pack8<T> draw_k, z_k, dout_k;
       float Dd = 0.f;
       if (valid) {
         Dd = p.D ? ((const float *)p.D)[d] : 0.f;
         ld8_guard<T, VEC>((const T *)p.u + b * p.u_bs + d * p.u_ds + tl, nvalid, 0.f, u);
         ld8_guard<T, VEC>((const T *)p.delta + b * p.delta_bs + d * p.delta_ds + tl, nvalid, 0.f, dl);
         ld8_guard<T, VEC>((const T *)p.dout + b * p.dout_bs + d * p.dout_ds + tl, nvalid, 0.f, dy);
+        draw_k.pack(dl);
+        dout_k.pack(dy);
         const float bias = p.delta_bias ? ((const float *)p.delta_bias)[d] : 0.f;
         if (has_z) {
           float z[8];
           ld8_guard<T, VEC>((const T *)p.z + b * p.z_bs + d * p.z_ds + tl, nvalid, 0.f, z);
+          z_k.pack(z);
 #pragma unroll
           for (int i = 0; i < KI; ++i) dy[i] *= z[i] * sigmoid_f(z[i]);
         }
@@ -384,7 +389,7 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
       }
       if (valid) {
         float draw[8], o[8];
-        ld8_guard<T, VEC>((const T *)p.delta + b * p.delta_bs + d * p.delta_ds + tl, nvalid, 0.f, draw);
+        draw_k.unpack(draw);
         const float bias = p.delta_bias ? ((const float *)p.delta_bias)[d] : 0.f;
         float dbs = 0.f, dDs = 0.f;
 #pragma unroll
@@ -403,8 +408,8 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
         st8_guard<T, VEC>((T *)p.ddelta + b * p.ddelta_bs + d * p.ddelta_ds + tl, nvalid, o);
         if (has_z) {
           float z[8], dout[8], oz[8];
-          ld8_guard<T, VEC>((const T *)p.z + b * p.z_bs + d * p.z_ds + tl, nvalid, 0.f, z);
-          ld8_guard<T, VEC>((const T *)p.dout + b * p.dout_bs + d * p.dout_ds + tl, nvalid, 0.f, dout);
+          z_k.unpack(z);
+          dout_k.unpack(dout);
 #pragma unroll
           for (int i = 0; i < KI; ++i) {
             const float yf = __builtin_fmaf(Dd, u[i], y[i]);
