@@ -489,35 +489,62 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bmm_chu
 }
 
 // --------------------------------------------------------- cumsum bwd
-// One thread per (batch, chunk, head): reverse running sum of dL/da -> dL/d(dt A); then
-// the chain through A, the clamp, softplus and the bias.
+// One workgroup per (batch, chunk, 16 heads); thread tid handles position Q-1-tid, so that the
+// reverse running sum of dL/da over the chunk (-> dL/d(dt A)) is a forward wave scan.  Then the
+// chain through A, the clamp, softplus and the bias; dA and ddt_bias are reduced per workgroup.
+constexpr int CS_HT = 16;
+
+DEVI float wave_incl_sum(float x) {
+  x += dpp_f<DPP_ROW_SHR + 1>(0.f, x);
+  x += dpp_f<DPP_ROW_SHR + 2>(0.f, x);
+  x += dpp_f<DPP_ROW_SHR + 4>(0.f, x);
+  x += dpp_f<DPP_ROW_SHR + 8>(0.f, x);
+  x += dpp_f<DPP_ROW_BCAST15, 0xa>(0.f, x);
+  x += dpp_f<DPP_ROW_BCAST31, 0xc>(0.f, x);
+  return x;
+}
+
 __global__ __launch_bounds__(256) void chunk_cumsum_bwd_kernel(const SsdParams p) {
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int H = p.nheads, nc = p.nchunks, Q = p.chunk_size, L = p.seqlen;
-  if (idx >= (int64_t)p.batch * nc * H) return;
-  const int h = idx % H, c = (idx / H) % nc, b = idx / ((int64_t)H * nc);
-  const float A = static_cast<const float *>(p.A)[h];
-  const float bias = p.dt_bias ? static_cast<const float *>(p.dt_bias)[h] : 0.f;
-  const float *dda = chunk_row(p.ddA_cumsum, p, b, h, c);
-  const float *ddt_out = chunk_row(p.ddt_out, p, b, h, c);
-  const float *dt_out = chunk_row(p.dt_out, p, b, h, c);
-  float run = 0.f, dAsum = 0.f, dbias = 0.f;
-  for (int l = Q - 1; l >= 0; --l) {
-    const int t = c * Q + l;
-    run += dda[l];
-    if (t >= L) continue;
-    float ddt = __builtin_fmaf(run, A, ddt_out[l]);
-    dAsum = __builtin_fmaf(run, dt_out[l], dAsum);
-    const int64_t di = b * p.dt_bs + (int64_t)t * p.dt_ls + h * p.dt_hs;
-    const float raw = ld_dyn(p.dt, di, p.dt_dtype) + bias;
-    const float v = p.dt_softplus ? softplus_f(raw) : raw;
-    if (v < p.dt_min || v > p.dt_max) ddt = 0.f;
-    if (p.dt_softplus && raw <= 20.f) ddt *= sigmoid_f(raw);
-    st_dyn(p.ddt, ((int64_t)b * L + t) * H + h, p.dt_dtype, ddt);
-    dbias += ddt;
+  __shared__ float wtot[4][CS_HT];
+  const int H = p.nheads, Q = p.chunk_size, L = p.seqlen;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l = Q - 1 - tid;
+  const int c = blockIdx.x, h0 = blockIdx.y * CS_HT, b = blockIdx.z;
+  const int t = c * Q + l;
+  const bool inq = l >= 0, live = inq && t < L;
+  float run[CS_HT];
+#pragma unroll
+  for (int i = 0; i < CS_HT; ++i) {
+    const int h = h0 + i;
+    const float v = (h < H && inq) ? chunk_row(p.ddA_cumsum, p, b, h, c)[l] : 0.f;
+    run[i] = wave_incl_sum(v);
+    if (lane == 63) wtot[wave][i] = run[i];
   }
-  unsafeAtomicAdd(p.dA + h, dAsum);
-  if (p.ddt_bias) unsafeAtomicAdd(p.ddt_bias + h, dbias);
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < CS_HT; ++i) {
+    const int h = h0 + i;
+    float r = run[i];
+    for (int w = 0; w < wave; ++w) r += wtot[w][i];
+    float dAterm = 0.f, ddt = 0.f;
+    if (h < H && live) {
+      const float A = static_cast<const float *>(p.A)[h];
+      const float bias = p.dt_bias ? static_cast<const float *>(p.dt_bias)[h] : 0.f;
+      ddt = __builtin_fmaf(r, A, chunk_row(p.ddt_out, p, b, h, c)[l]);
+      dAterm = r * chunk_row(p.dt_out, p, b, h, c)[l];
+      const float raw = ld_dyn(p.dt, b * p.dt_bs + (int64_t)t * p.dt_ls + h * p.dt_hs, p.dt_dtype) + bias;
+      const float v = p.dt_softplus ? softplus_f(raw) : raw;
+      if (v < p.dt_min || v > p.dt_max) ddt = 0.f;
+      if (p.dt_softplus && raw <= 20.f) ddt *= sigmoid_f(raw);
+      st_dyn(p.ddt, ((int64_t)b * L + t) * H + h, p.dt_dtype, ddt);
+    }
+    dAterm = wave_sum(dAterm);
+    ddt = wave_sum(ddt);
+    if (lane == 0 && h < H) {
+      unsafeAtomicAdd(p.dA + h, dAterm);
+      if (p.ddt_bias) unsafeAtomicAdd(p.ddt_bias + h, ddt);
+    }
+  }
 }
 
 int check_bwd(const SsdParams *p) {
@@ -622,8 +649,8 @@ extern "C" int ssd_chunk_cumsum_bwd(const SsdParams *p, mamba_stream_t stream) {
   int rc = check_bwd(p);
   if (rc) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int64_t n = (int64_t)p->batch * p->nchunks * p->nheads;
-  hipLaunchKernelGGL(chunk_cumsum_bwd_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, *p);
+  dim3 grid(p->nchunks, (p->nheads + CS_HT - 1) / CS_HT, p->batch);
+  hipLaunchKernelGGL(chunk_cumsum_bwd_kernel, grid, dim3(256), 0, s, *p);
   return launched();
 }
 

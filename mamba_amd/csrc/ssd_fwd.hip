@@ -7,29 +7,58 @@
 namespace {
 
 // ------------------------------------------------------------ chunk_cumsum
-// One thread per (batch, chunk, head): dt -> (+bias, softplus, clamp), zero past
-// the end of the sequence, and the running sum of dt * A inside the chunk.
+// One workgroup per (batch, chunk, 16 heads); thread = position inside the chunk, so loads of
+// dt (head-contiguous) are 16 consecutive elements per thread and the stores of dt_out / dA_cumsum
+// (position-contiguous) are coalesced.  dt -> (+bias, softplus, clamp), zero past the end of the
+// sequence; dA_cumsum = running sum of dt * A over the chunk (wave DPP scan + cross-wave offsets).
+constexpr int CS_HT = 16;
+
+DEVI float wave_incl_sum(float x) {
+  x += dpp_f<DPP_ROW_SHR + 1>(0.f, x);
+  x += dpp_f<DPP_ROW_SHR + 2>(0.f, x);
+  x += dpp_f<DPP_ROW_SHR + 4>(0.f, x);
+  x += dpp_f<DPP_ROW_SHR + 8>(0.f, x);
+  x += dpp_f<DPP_ROW_BCAST15, 0xa>(0.f, x);
+  x += dpp_f<DPP_ROW_BCAST31, 0xc>(0.f, x);
+  return x;
+}
+
 __global__ __launch_bounds__(256) void chunk_cumsum_fwd_kernel(const SsdParams p) {
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  __shared__ float wtot[4][CS_HT];
   const int H = p.nheads, nc = p.nchunks, Q = p.chunk_size;
-  if (idx >= (int64_t)p.batch * nc * H) return;
-  const int h = idx % H, c = (idx / H) % nc, b = idx / ((int64_t)H * nc);
-  const float A = static_cast<const float *>(p.A)[h];
-  const float bias = p.dt_bias ? static_cast<const float *>(p.dt_bias)[h] : 0.f;
-  float *dt_out = p.dt_out + (((int64_t)b * H + h) * nc + c) * Q;
-  float *dA_cs = p.dA_cumsum + (((int64_t)b * H + h) * nc + c) * Q;
-  float run = 0.f;
-  for (int l = 0; l < Q; ++l) {
-    const int t = c * Q + l;
-    float dt = 0.f;
-    if (t < p.seqlen) {
-      dt = ld_dyn(p.dt, b * p.dt_bs + t * p.dt_ls + h * p.dt_hs, p.dt_dtype) + bias;
-      if (p.dt_softplus) dt = softplus_f(dt);
-      dt = fminf(fmaxf(dt, p.dt_min), p.dt_max);
+  const int l = threadIdx.x, lane = l & 63, wave = l >> 6;
+  const int c = blockIdx.x, h0 = blockIdx.y * CS_HT, b = blockIdx.z;
+  const int t = c * Q + l;
+  const bool live = l < Q && t < p.seqlen;
+  float dtv[CS_HT], cs[CS_HT];
+#pragma unroll
+  for (int i = 0; i < CS_HT; ++i) {
+    const int h = h0 + i;
+    float dt = 0.f, A = 0.f;
+    if (h < H) {
+      A = static_cast<const float *>(p.A)[h];
+      if (live) {
+        dt = ld_dyn(p.dt, b * p.dt_bs + (int64_t)t * p.dt_ls + h * p.dt_hs, p.dt_dtype);
+        if (p.dt_bias) dt += static_cast<const float *>(p.dt_bias)[h];
+        if (p.dt_softplus) dt = softplus_f(dt);
+        dt = fminf(fmaxf(dt, p.dt_min), p.dt_max);
+      }
     }
-    run += dt * A;
-    dt_out[l] = dt;
-    dA_cs[l] = run;
+    dtv[i] = dt;
+    cs[i] = wave_incl_sum(dt * A);
+    if (lane == 63) wtot[wave][i] = cs[i];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < CS_HT; ++i) {
+    const int h = h0 + i;
+    float off = 0.f;
+    for (int w = 0; w < wave; ++w) off += wtot[w][i];
+    if (h < H && l < Q) {
+      const int64_t o = (((int64_t)b * H + h) * nc + c) * Q + l;
+      p.dt_out[o] = dtv[i];
+      p.dA_cumsum[o] = cs[i] + off;
+    }
   }
 }
 
@@ -264,8 +293,8 @@ extern "C" int ssd_chunk_cumsum_fwd(const SsdParams *p, mamba_stream_t stream) {
   if (rc) return rc;
   if (!p->dt_out || !p->dA_cumsum) return MAMBA_E_BADARG;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int64_t n = (int64_t)p->batch * p->nchunks * p->nheads;
-  hipLaunchKernelGGL(chunk_cumsum_fwd_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, *p);
+  dim3 grid(p->nchunks, (p->nheads + CS_HT - 1) / CS_HT, p->batch);
+  hipLaunchKernelGGL(chunk_cumsum_fwd_kernel, grid, dim3(256), 0, s, *p);
   return launched();
 }
 
