@@ -221,7 +221,12 @@ int ssd_chunk_state_fwd(const SsdParams *p, mamba_stream_t stream);
 int ssd_state_passing_fwd(const SsdParams *p, mamba_stream_t stream);
 int ssd_bmm_chunk_fwd(const SsdParams *p, mamba_stream_t stream);
 int ssd_chunk_scan_fwd(const SsdParams *p, mamba_stream_t stream);
-/* all five on `stream` */
+/* chunk_scan with the C B^T contraction fused in (CB is neither read nor written): bf16,
+ * headdim 32/64, dstate 64/128, chunk_size 64/128/256, 16-byte aligned rows.
+ * ssd_chunk_scan_fwd_fused_supported returns 1 when it applies. */
+int ssd_chunk_scan_fwd_fused_supported(const SsdParams *p);
+int ssd_chunk_scan_fwd_fused(const SsdParams *p, mamba_stream_t stream);
+/* cumsum, chunk_state, state_passing, then the fused scan when supported, else bmm + chunk_scan */
 int ssd_combined_fwd(const SsdParams *p, mamba_stream_t stream);
 
 /* Backward.  Inputs: the forward inputs, dout, dfinal_states, the saved pre-gate

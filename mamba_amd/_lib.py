@@ -84,12 +84,14 @@ def load():
         fn.argtypes = [ctypes.POINTER(MambaScanParams), c_vp]
         fn.restype = ctypes.c_int
     for name in ("ssd_chunk_cumsum_fwd", "ssd_chunk_state_fwd", "ssd_state_passing_fwd", "ssd_bmm_chunk_fwd",
-                 "ssd_chunk_scan_fwd", "ssd_combined_fwd", "ssd_bwd_dz", "ssd_bwd_dstates",
+                 "ssd_chunk_scan_fwd", "ssd_combined_fwd", "ssd_chunk_scan_fwd_fused", "ssd_bwd_dz", "ssd_bwd_dstates",
                  "ssd_state_passing_bwd", "ssd_bwd_dx", "ssd_bwd_dBC_state", "ssd_bwd_dcb", "ssd_bmm_chunk_bwd",
                  "ssd_chunk_cumsum_bwd", "ssd_combined_bwd"):
         fn = getattr(lib, name)
         fn.argtypes = [ctypes.POINTER(SsdParams), c_vp]
         fn.restype = ctypes.c_int
+    lib.ssd_chunk_scan_fwd_fused_supported.argtypes = [ctypes.POINTER(SsdParams)]
+    lib.ssd_chunk_scan_fwd_fused_supported.restype = ctypes.c_int
     lib.ssm_state_update.argtypes = [ctypes.POINTER(MambaStepParams), c_vp]
     lib.ssm_state_update.restype = ctypes.c_int
     _lib = lib

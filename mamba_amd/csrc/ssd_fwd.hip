@@ -344,6 +344,7 @@ extern "C" int ssd_combined_fwd(const SsdParams *p, mamba_stream_t stream) {
   if ((rc = ssd_chunk_cumsum_fwd(p, stream))) return rc;
   if ((rc = ssd_chunk_state_fwd(p, stream))) return rc;
   if ((rc = ssd_state_passing_fwd(p, stream))) return rc;
+  if (ssd_chunk_scan_fwd_fused_supported(p)) return ssd_chunk_scan_fwd_fused(p, stream);
   if ((rc = ssd_bmm_chunk_fwd(p, stream))) return rc;
   return ssd_chunk_scan_fwd(p, stream);
 }

@@ -1,0 +1,340 @@
+// SSD chunk_scan forward, fused with the C B^T contraction, for bf16 on gfx950.
+//
+// One workgroup (8 waves) computes the whole (chunk_size x headdim) output tile of one
+// (batch, chunk, head).  It is organised like a causal attention forward pass whose softmax
+// is replaced by the decay mask:
+//     S^T[s, l] = sum_n B[s, n] C[l, n]                       (MFMA; C rows live in registers)
+//     M^T[s, l] = S^T[s, l] * dt_s * exp(a_l - a_s)   (s <= l, same sequence)
+//     y^T[p, l] += sum_s X^T[p, s] M^T[s, l]                 (MFMA)
+// plus the carried state  y^T[p, l] += exp(a_l) sum_n H[p, n] C[l, n].
+// Working on the transposes makes the accumulator layout of the first MFMA (4 consecutive s per
+// lane for one l) equal to the B-operand layout of the second one, so M never leaves registers
+// and CB never goes to memory.  The k index of the second MFMA is permuted accordingly when X
+// is staged (transposed) into LDS.  For positions more than one 16-tile apart the decay is
+// factored as exp(a_l - a_end) * exp(a_end - a_s) with a_end the last a of the s tile (both
+// exponents <= 0), so the inner loop has one multiply per element instead of an exponential;
+// diagonal tiles use the exact form.  Each wave owns a balanced set of 16-row l tiles
+// (tile i paired with tile QT-1-i) so that the causal work is the same for all waves.
+#include "ssd_common.hpp"
+
+namespace {
+
+DEVI f32x4 mfma_bf16(bf16x8_t a, bf16x8_t b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+DEVI bf16x8_t ld_frag(const uint16_t *p) { return *reinterpret_cast<const bf16x8_t *>(p); }
+
+// l tile k (0 .. LT-1) of wave w, QT tiles in all, NWV waves
+template <int QT, int NWV> DEVI int l_tile(int w, int k) {
+  constexpr int LT = QT / NWV;
+  if (LT == 1) return w;
+  constexpr int HALF = LT / 2;
+  return k < HALF ? HALF * w + k : QT - 1 - (HALF * w + (k - HALF));
+}
+
+template <int PT, int NK, int QT, int NWV>
+__global__ __launch_bounds__(64 * NWV) void chunk_scan_fwd_fused_kernel(const SsdParams p) {
+  constexpr int P = 16 * PT, N = 32 * NK, Q = 16 * QT, LT = QT / NWV, NSB = Q / 32, NT = 64 * NWV;
+  static_assert(LT >= 1 && LT * NWV == QT, "l tiles divide evenly over the waves");
+  constexpr int BP = N + 8;  // LDS pitch of a B row / H row (bf16): 16-byte aligned, bank-spread
+  constexpr int XP = 40;     // LDS pitch of an X^T row (32 k values + pad)
+  constexpr int YP = P + 8;  // fp32 pitch of the epilogue's per-wave transpose patch
+  struct Stage {
+    uint16_t Bs[2][32 * BP];
+    uint16_t Xs[2][P * XP];
+    uint16_t Hs[P * BP];
+  };
+  union __align__(16) Shared {
+    Stage st;                       // main loop
+    float ypatch[NWV * 16 * YP];    // epilogue (the staging buffers are dead by then)
+  };
+  __shared__ Shared shm;
+  auto &Bs = shm.st.Bs;
+  auto &Xs = shm.st.Xs;
+  auto &Hs = shm.st.Hs;
+  __shared__ float a2_s[Q], dt_s[Q], cs_s[Q], rs_s[Q];
+  __shared__ int seq_s[Q];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int j = lane & 15, g = lane >> 4;
+  const int H = p.nheads, G = p.ngroups, L = p.seqlen;
+  const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int grp = h / (H / G);
+  const int t0 = c * Q;
+  const int qlim = min(Q, L - t0);
+  const bf16_t *xg = static_cast<const bf16_t *>(p.x) + b * p.x_bs + h * p.x_hs;
+  const bf16_t *Bg = static_cast<const bf16_t *>(p.B) + b * p.B_bs + grp * p.B_gs;
+  const bf16_t *Cg = static_cast<const bf16_t *>(p.C) + b * p.C_bs + grp * p.C_gs;
+  const bool has_seq = p.seq_idx != nullptr;
+
+  // ---- per-position scalars of this (batch, head, chunk)
+  {
+    const float *dA = p.dA_cumsum + (((int64_t)b * H + h) * p.nchunks + c) * Q;
+    const float *dt = p.dt_out + (((int64_t)b * H + h) * p.nchunks + c) * Q;
+    const int32_t *seq = has_seq ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
+    for (int s = tid; s < Q; s += NT) {
+      const float a = dA[s];
+      const float aend = dA[(s | 15)];
+      a2_s[s] = a * kLog2e;
+      dt_s[s] = dt[s];
+      cs_s[s] = dt[s] * fast_exp(aend - a);
+      bool ok = s < qlim;
+      int id = 0;
+      if (has_seq) {
+        id = s < qlim ? seq[s] : -2;
+        ok = ok && id == (c > 0 ? seq[-1] : 0);
+      }
+      seq_s[s] = id;
+      rs_s[s] = ok ? fast_exp(a) : 0.f;
+    }
+  }
+
+  // ---- staging helpers (global -> registers -> LDS), one s block of 32 positions
+  constexpr int BCH = (32 * N / 8 + NT - 1) / NT;    // 16-byte chunks of B per thread
+  // X tasks: 4 consecutive positions x 8 consecutive p (four 16-byte loads, eight 8-byte
+  // transposed LDS stores); 8 * P / 8 tasks per block, taken by the first threads
+  constexpr int XTASKS = 8 * (P / 8);
+  static_assert(XTASKS <= NT, "one X task per thread at most");
+  struct XRegs { u32x4 v[4]; };
+  u32x4 bregs[2][BCH];
+  XRegs xregs[2];  // two blocks in flight: global loads run two blocks ahead
+  auto load_block = [&](int sb, u32x4 (&breg)[BCH], XRegs &xreg) {
+#pragma unroll
+    for (int q = 0; q < BCH; ++q) {
+      const int id = tid + q * NT, r = id / (N / 8), c8 = id % (N / 8);
+      const int s = sb * 32 + r;
+      breg[q] = u32x4{0, 0, 0, 0};
+      if (id < 32 * N / 8 && s < qlim) breg[q] = *reinterpret_cast<const u32x4 *>(Bg + (int64_t)(t0 + s) * p.B_ls + c8 * 8);
+    }
+    if (tid < XTASKS) {
+      const int q4 = tid / (P / 8), p8 = tid % (P / 8);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int s = sb * 32 + q4 * 4 + e;
+        xreg.v[e] = u32x4{0, 0, 0, 0};
+        if (s < qlim) xreg.v[e] = *reinterpret_cast<const u32x4 *>(xg + (int64_t)(t0 + s) * p.x_ls + p8 * 8);
+      }
+    }
+  };
+  auto store_block = [&](int buf, const u32x4 (&breg)[BCH], const XRegs &xreg) {
+#pragma unroll
+    for (int q = 0; q < BCH; ++q) {
+      const int id = tid + q * NT, r = id / (N / 8), c8 = id % (N / 8);
+      if (id < 32 * N / 8) *reinterpret_cast<u32x4 *>(&Bs[buf][r * BP + c8 * 8]) = breg[q];
+    }
+    if (tid < XTASKS) {
+      const int q4 = tid / (P / 8), p8 = tid % (P / 8);
+      // k slots of positions 4 q4 .. 4 q4 + 3 inside the 32-block: the second MFMA's lane group gq
+      // holds positions 4 gq .. 4 gq + 3 of both 16-tiles.  The 8-element group is XOR-swizzled
+      // with p8 so that the transposing stores spread over the banks.
+      const int pos = (((q4 & 3) ^ (p8 & 3)) << 3) + ((q4 >> 2) << 2);
+      const uint32_t w[4][4] = {{xreg.v[0].x, xreg.v[0].y, xreg.v[0].z, xreg.v[0].w},
+                                {xreg.v[1].x, xreg.v[1].y, xreg.v[1].z, xreg.v[1].w},
+                                {xreg.v[2].x, xreg.v[2].y, xreg.v[2].z, xreg.v[2].w},
+                                {xreg.v[3].x, xreg.v[3].y, xreg.v[3].z, xreg.v[3].w}};
+#pragma unroll
+      for (int pp = 0; pp < 8; ++pp) {  // p = p8 * 8 + pp: element pp of each of the 4 positions
+        const int d = pp >> 1;
+        uint32_t lo, hi;
+        if (pp & 1) {
+          lo = (w[0][d] >> 16) | (w[1][d] & 0xffff0000u);
+          hi = (w[2][d] >> 16) | (w[3][d] & 0xffff0000u);
+        } else {
+          lo = (w[0][d] & 0xffffu) | (w[1][d] << 16);
+          hi = (w[2][d] & 0xffffu) | (w[3][d] << 16);
+        }
+        *reinterpret_cast<u32x2 *>(&Xs[buf][(p8 * 8 + pp) * XP + pos]) = u32x2{lo, hi};
+      }
+    }
+  };
+
+  load_block(0, bregs[0], xregs[0]);
+  if (NSB > 1) load_block(1, bregs[1], xregs[1]);
+  // carried state, fp32 -> bf16, rows p, k = n
+  {
+    const float *Hc = p.states + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
+    for (int id = tid; id < P * N / 8; id += NT) {
+      const int pp = id / (N / 8), c8 = id % (N / 8);
+      const f32x4 v0 = *reinterpret_cast<const f32x4 *>(Hc + (int64_t)pp * N + c8 * 8);
+      const f32x4 v1 = *reinterpret_cast<const f32x4 *>(Hc + (int64_t)pp * N + c8 * 8 + 4);
+      u32x4 o = {pack_bf16(v0.x, v0.y), pack_bf16(v0.z, v0.w), pack_bf16(v1.x, v1.y), pack_bf16(v1.z, v1.w)};
+      *reinterpret_cast<u32x4 *>(&Hs[pp * BP + c8 * 8]) = o;
+    }
+  }
+  // C rows of this wave's l tiles: B operand of both contractions (col l = j, k = n)
+  bf16x8_t Cf[LT][NK];
+#pragma unroll
+  for (int k = 0; k < LT; ++k) {
+    const int l = l_tile<QT, NWV>(wave, k) * 16 + j;
+#pragma unroll
+    for (int kk = 0; kk < NK; ++kk) {
+      u32x4 v = {0, 0, 0, 0};
+      if (l < qlim) v = *reinterpret_cast<const u32x4 *>(Cg + (int64_t)(t0 + l) * p.C_ls + kk * 32 + g * 8);
+      Cf[k][kk] = __builtin_bit_cast(bf16x8_t, v);
+    }
+  }
+  store_block(0, bregs[0], xregs[0]);
+  __syncthreads();
+
+  f32x4 acc[LT][PT];
+  // ---- carried state: y^T[p, l] = rs_l * sum_n H[p, n] C[l, n]
+#pragma unroll
+  for (int k = 0; k < LT; ++k) {
+#pragma unroll
+    for (int pt = 0; pt < PT; ++pt) {
+      f32x4 v = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < NK; ++kk) v = mfma_bf16(ld_frag(&Hs[(pt * 16 + j) * BP + kk * 32 + g * 8]), Cf[k][kk], v);
+      acc[k][pt] = v * rs_s[l_tile<QT, NWV>(wave, k) * 16 + j];
+    }
+  }
+
+  // ---- inside the chunk
+#pragma unroll
+  for (int sb = 0; sb < NSB; ++sb) {
+    const int buf = sb & 1;
+    if (sb + 2 < NSB) load_block(sb + 2, bregs[sb & 1], xregs[sb & 1]);
+#pragma unroll
+    for (int k = 0; k < LT; ++k) {
+      const int lt = l_tile<QT, NWV>(wave, k);
+      if (lt * 16 + 15 < sb * 32) continue;  // every position of the block is after the tile
+      const int l = lt * 16 + j;
+      const float al2 = a2_s[l];
+      const int lid = seq_s[l];
+      float m[8];
+#pragma unroll
+      for (int h2 = 0; h2 < 2; ++h2) {
+        const int st = 2 * sb + h2;
+        if (st > lt) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) m[h2 * 4 + r] = 0.f;
+          continue;
+        }
+        f32x4 S = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < NK; ++kk)
+          S = mfma_bf16(ld_frag(&Bs[buf][(h2 * 16 + j) * BP + kk * 32 + g * 8]), Cf[k][kk], S);
+        const int s0 = st * 16 + 4 * g;
+        if (st < lt) {
+          const float rl = fast_exp2(al2 - a2_s[st * 16 + 15]);
+          const f32x4 cs = *reinterpret_cast<const f32x4 *>(&cs_s[s0]);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) m[h2 * 4 + r] = S[r] * cs[r] * rl;
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int s = s0 + r;
+            m[h2 * 4 + r] = s <= l ? S[r] * dt_s[s] * fast_exp2(fminf(al2 - a2_s[s], 0.f)) : 0.f;
+          }
+        }
+        if (has_seq) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (seq_s[s0 + r] != lid) m[h2 * 4 + r] = 0.f;
+        }
+      }
+      const u32x4 mp = {pack_bf16(m[0], m[1]), pack_bf16(m[2], m[3]), pack_bf16(m[4], m[5]), pack_bf16(m[6], m[7])};
+      const bf16x8_t Mf = __builtin_bit_cast(bf16x8_t, mp);
+#pragma unroll
+      for (int pt = 0; pt < PT; ++pt)
+        acc[k][pt] = mfma_bf16(ld_frag(&Xs[buf][(pt * 16 + j) * XP + ((g ^ ((pt * 2 + (j >> 3)) & 3)) << 3)]), Mf,
+                               acc[k][pt]);
+    }
+    if (sb + 1 < NSB) store_block(buf ^ 1, bregs[(sb + 1) & 1], xregs[(sb + 1) & 1]);
+    __syncthreads();
+  }
+
+  // ---- epilogue: + D x, pre-gate copy, gate.  Each wave transposes its 16-row tiles through a
+  // private LDS patch so that x / z loads and out / out_x stores are 16-byte pieces of
+  // contiguous rows (the accumulator layout itself would scatter 8-byte pieces over 16 rows).
+  float *Ys = shm.ypatch + wave * 16 * YP;
+  const float *Dp = static_cast<const float *>(p.D);
+  const bf16_t *zg = p.z ? static_cast<const bf16_t *>(p.z) + b * p.z_bs + h * p.z_hs : nullptr;
+  bf16_t *og = static_cast<bf16_t *>(p.out) + b * p.out_bs + h * p.out_hs;
+  bf16_t *oxg = p.z ? static_cast<bf16_t *>(p.out_x) + b * p.out_bs + h * p.out_hs : nullptr;
+#pragma unroll
+  for (int k = 0; k < LT; ++k) {
+    const int ltile = l_tile<QT, NWV>(wave, k);
+#pragma unroll
+    for (int pt = 0; pt < PT; ++pt) *reinterpret_cast<f32x4 *>(&Ys[j * YP + pt * 16 + 4 * g]) = acc[k][pt];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // 16 rows x P/8 chunks of 8 columns
+#pragma unroll
+    for (int q = 0; q < (16 * P / 8 + 63) / 64; ++q) {
+      const int id = lane + q * 64, rr = id / (P / 8), c8 = id % (P / 8);
+      const int l = ltile * 16 + rr;
+      if (id >= 16 * P / 8 || l >= qlim) continue;
+      const f32x4 y0 = *reinterpret_cast<const f32x4 *>(&Ys[rr * YP + c8 * 8]);
+      const f32x4 y1 = *reinterpret_cast<const f32x4 *>(&Ys[rr * YP + c8 * 8 + 4]);
+      float v[8] = {y0.x, y0.y, y0.z, y0.w, y1.x, y1.y, y1.z, y1.w};
+      if (Dp) {
+        float xf[8];
+        ld8<bf16_t>(xg + (int64_t)(t0 + l) * p.x_ls + c8 * 8, xf);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = __builtin_fmaf(p.D_has_hdim ? Dp[h * P + c8 * 8 + e] : Dp[h], xf[e], v[e]);
+      }
+      const int64_t oi = (int64_t)(t0 + l) * p.out_ls + c8 * 8;
+      if (zg) {
+        st8<bf16_t>(oxg + oi, v);
+        float zf[8];
+        ld8<bf16_t>(zg + (int64_t)(t0 + l) * p.z_ls + c8 * 8, zf);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] *= zf[e] * sigmoid_f(zf[e]);
+      }
+      st8<bf16_t>(og + oi, v);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+bool aligned(const void *ptr, int a) { return (reinterpret_cast<uintptr_t>(ptr) % a) == 0; }
+
+template <int PT, int NK> int launch_q(const SsdParams &p, hipStream_t s) {
+  dim3 grid(p.nchunks, p.nheads, p.batch);
+  switch (p.chunk_size) {
+    case 256: hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 16, 8>), grid, dim3(512), 0, s, p); break;
+    case 128: hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 8, 8>), grid, dim3(512), 0, s, p); break;
+    case 64: hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 4, 4>), grid, dim3(256), 0, s, p); break;
+    default: return MAMBA_E_UNSUPPORTED;
+  }
+  return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
+}
+
+template <int PT> int launch_n(const SsdParams &p, hipStream_t s) {
+  switch (p.dstate) {
+    case 64: return launch_q<PT, 2>(p, s);
+    case 128: return launch_q<PT, 4>(p, s);
+    default: return MAMBA_E_UNSUPPORTED;
+  }
+}
+
+}  // namespace
+
+// 1 if ssd_chunk_scan_fwd_fused has a kernel for this problem, else 0.
+extern "C" int ssd_chunk_scan_fwd_fused_supported(const SsdParams *p) {
+  if (!p || p->dtype != MAMBA_BF16) return 0;
+  if (p->headdim != 32 && p->headdim != 64) return 0;
+  if (p->dstate != 64 && p->dstate != 128) return 0;
+  if (p->chunk_size != 64 && p->chunk_size != 128 && p->chunk_size != 256) return 0;
+  // 16-byte pieces of rows everywhere
+  if (!aligned(p->x, 16) || !aligned(p->B, 16) || !aligned(p->C, 16) || !aligned(p->out, 16)) return 0;
+  if (p->x_bs % 8 || p->x_ls % 8 || p->x_hs % 8 || p->B_bs % 8 || p->B_ls % 8 || p->B_gs % 8 || p->C_bs % 8 ||
+      p->C_ls % 8 || p->C_gs % 8)
+    return 0;
+  if (p->out_bs % 8 || p->out_ls % 8 || p->out_hs % 8) return 0;
+  if (p->z && (!aligned(p->z, 16) || !aligned(p->out_x, 16) || p->z_bs % 8 || p->z_ls % 8 || p->z_hs % 8)) return 0;
+  if (p->batch > 65535 || p->nheads > 65535) return 0;
+  return 1;
+}
+
+extern "C" int ssd_chunk_scan_fwd_fused(const SsdParams *p, mamba_stream_t stream) {
+  if (!p || !p->x || !p->B || !p->C || !p->states || !p->out || !p->dt_out || !p->dA_cumsum || (p->z && !p->out_x))
+    return MAMBA_E_BADARG;
+  if (!ssd_chunk_scan_fwd_fused_supported(p)) return MAMBA_E_UNSUPPORTED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return p->headdim == 64 ? launch_n<4>(*p, s) : launch_n<2>(*p, s);
+}

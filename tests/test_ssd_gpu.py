@@ -56,6 +56,20 @@ def test_ssd_fwd_shapes(headdim, dstate, ngroups):
     _fwd_case(1, 384, 4, headdim, dstate, ngroups, 128, torch.float32)
 
 
+@pytest.mark.parametrize("headdim,dstate,chunk,seqlen", [
+    (64, 128, 256, 1024), (64, 64, 128, 300), (32, 128, 64, 200), (64, 128, 256, 77), (32, 64, 256, 513),
+    (64, 128, 128, 640)])
+def test_ssd_fwd_fused_scan_shapes(headdim, dstate, chunk, seqlen):
+    # bf16 shapes served by the fused C B^T + scan kernel, full and partial last chunks
+    _fwd_case(2, seqlen, 4, headdim, dstate, 2, chunk, torch.bfloat16, has_init=True)
+    _fwd_case(1, seqlen, 4, headdim, dstate, 1, chunk, torch.bfloat16, has_z=False, D_has_hdim=True)
+
+
+def test_ssd_fwd_fused_scan_packed():
+    _fwd_case(1, 1024, 4, 64, 128, 2, 256, torch.bfloat16, seq_lens=[300, 212, 100, 156, 256], has_init=True)
+    _fwd_case(1, 700, 4, 32, 64, 1, 128, torch.bfloat16, seq_lens=[1, 127, 129, 443])
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_ssd_fwd_options(dtype):
     _fwd_case(2, 320, 4, 64, 32, 1, 64, dtype, has_init=True)
