@@ -164,15 +164,19 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dst
   const int64_t gb = b * gv.bs + h * gv.hs, Cb = b * p.C_bs + g * p.C_gs;
   GemmAcc acc;
   acc.zero();
-  auto fa = [&](int r, int k) {  // (p, l)
-    const int pp = pt * GB + r;
-    return (pp < P && k < qlim) ? ldg<T>(gv.ptr, gb + (int64_t)(t0 + k) * gv.ls + pp) : 0.f;
-  };
-  auto fb = [&](int r, int k) {  // (n, l)
-    const int n = nt * GB + r;
-    return (n < N && k < qlim) ? ldg<T>(p.C, Cb + (int64_t)(t0 + k) * p.C_ls + n) * rs[k] : 0.f;
-  };
-  block_gemm<SPLIT, false, false>(acc, lds, 0, qlim, fa, fb, tid);
+  // A = g^T (rows p, k = position), B = (C rs)^T (rows n, k = position)
+  const T *ga = static_cast<const T *>(gv.ptr) + gb + (int64_t)t0 * gv.ls + pt * GB;
+  const T *Ca = static_cast<const T *>(p.C) + Cb + (int64_t)t0 * p.C_ls + nt * GB;
+  const bool va = rows_aligned16(ga, gv.ls), vb = rows_aligned16(Ca, p.C_ls);
+  block_gemm_staged<SPLIT>(
+      acc, lds, 0, qlim,
+      [&](int k0) {
+        if (tid < 128) stage_rc<SPLIT, T>(lds.ah, lds.al, ga, gv.ls, P - pt * GB, k0, qlim, nullptr, nullptr, va, tid);
+      },
+      [&](int k0) {
+        if (tid >= 128) stage_rc<SPLIT, T>(lds.bh, lds.bl, Ca, p.C_ls, N - nt * GB, k0, qlim, rs, nullptr, vb, tid - 128);
+      },
+      tid);
   float *ds = p.dstates + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
   acc_foreach(acc, tid, [&](int m, int n, float v) {
     const int pp = pt * GB + m, nn = nt * GB + n;
@@ -260,15 +264,15 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
   GemmAcc acc;
   acc.zero();
   {
-    auto fa = [&](int r, int k) {  // (s, n)
-      const int s = st * GB + r;
-      return (s < qlim && k < N) ? ldg<T>(p.B, Bb + (int64_t)(t0 + s) * p.B_ls + k) : 0.f;
-    };
-    auto fb = [&](int r, int k) {  // (p, n)
-      const int pp = pt * GB + r;
-      return (pp < P && k < N) ? dS[(int64_t)pp * N + k] : 0.f;
-    };
-    block_gemm<SPLIT, true, true>(acc, lds, 0, N, fa, fb, tid);
+    // A = B rows (s, k = n), B = dS rows (p, k = n): both k-contiguous
+    const T *Ba = static_cast<const T *>(p.B) + Bb + (int64_t)(t0 + st * GB) * p.B_ls;
+    const float *dSa = dS + (int64_t)pt * GB * N;
+    const bool va = rows_aligned16(Ba, p.B_ls), vb = rows_aligned16(dSa, N);
+    block_gemm_staged<SPLIT>(
+        acc, lds, 0, N,
+        [&](int k0) { stage_kc<SPLIT, T>(lds.ah, lds.al, Ba, p.B_ls, qlim - st * GB, k0, N, nullptr, nullptr, va, tid); },
+        [&](int k0) { stage_kc<SPLIT, float>(lds.bh, lds.bl, dSa, N, P - pt * GB, k0, N, nullptr, nullptr, vb, tid); },
+        tid);
     acc_foreach(acc, tid, [&](int m, int n, float v) { return v * wrow[m]; });
     row_dot(acc, r1, tid, fx);  // state-path part of <x_s, acc_s>
   }
@@ -278,11 +282,15 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
       if (s >= qlim || k >= qlim || k < s) return 0.f;
       return CB[(int64_t)k * Q + s] * fast_exp(fminf(a_s[k] - a_s[s], 0.f));
     };
-    auto fb = [&](int r, int k) {  // (p, l)
-      const int pp = pt * GB + r;
-      return (pp < P && k < qlim) ? ldg<T>(gv.ptr, gb + (int64_t)(t0 + k) * gv.ls + pp) : 0.f;
-    };
-    block_gemm<SPLIT, false, false>(acc, lds, st * GB, qlim, fa, fb, tid);
+    const T *ga = static_cast<const T *>(gv.ptr) + gb + (int64_t)t0 * gv.ls + pt * GB;
+    const bool vb = rows_aligned16(ga, gv.ls);
+    block_gemm_staged<SPLIT>(
+        acc, lds, st * GB, qlim,
+        [&](int k0) { stage_tile<SPLIT, false>(lds.ah, lds.al, [&](int r, int k) { return fa(r, k0 + k); }, tid); },
+        [&](int k0) {
+          if (tid < 128) stage_rc<SPLIT, T>(lds.bh, lds.bl, ga, gv.ls, P - pt * GB, k0, qlim, nullptr, nullptr, vb, tid);
+        },
+        tid);
     row_dot(acc, r2, tid, fx);  // full <x_s, acc_s>
   }
   if (tid < GB) {
@@ -344,20 +352,24 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dBC
   const int64_t gb = b * gv.bs + h * gv.hs, xb = b * p.x_bs + h * p.x_hs;
   const float *dS = p.dstates + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
   const float *Hc = p.states + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
-  auto fstate = [&](const float *S) {
-    return [=](int r, int k) {  // (n, p)
-      const int n = nt * GB + r;
-      return (n < N && k < P) ? S[(int64_t)k * N + n] : 0.f;
-    };
+  // A = x or g rows (position, k = p): k-contiguous; B = state rows n, k = p: row-contiguous fp32
+  const bool vs = rows_aligned16(dS + nt * GB, N) && rows_aligned16(Hc + nt * GB, N);
+  auto run = [&](GemmAcc &acc, const T *a_base, int64_t a_ls, const float *S) {
+    const T *aa = a_base + (int64_t)(t0 + st * GB) * a_ls;
+    const bool va = rows_aligned16(aa, a_ls);
+    block_gemm_staged<SPLIT>(
+        acc, lds, 0, P,
+        [&](int k0) { stage_kc<SPLIT, T>(lds.ah, lds.al, aa, a_ls, qlim - st * GB, k0, P, nullptr, nullptr, va, tid); },
+        [&](int k0) {
+          if (tid < 128)
+            stage_rc<SPLIT, float>(lds.bh, lds.bl, S + nt * GB, N, N - nt * GB, k0, P, nullptr, nullptr, vs, tid);
+        },
+        tid);
   };
   {
     GemmAcc acc;
     acc.zero();
-    auto fa = [&](int r, int k) {  // (s, p)
-      const int s = st * GB + r;
-      return (s < qlim && k < P) ? ldg<T>(p.x, xb + (int64_t)(t0 + s) * p.x_ls + k) : 0.f;
-    };
-    block_gemm<SPLIT, true, false>(acc, lds, 0, P, fa, fstate(dS), tid);
+    run(acc, static_cast<const T *>(p.x) + xb, p.x_ls, dS);
     acc_foreach(acc, tid, [&](int m, int n, float v) {
       const int s = st * GB + m, nn = nt * GB + n;
       if (s < qlim && nn < N) unsafeAtomicAdd(p.dB32 + (((int64_t)b * L + t0 + s) * G + g) * N + nn, v * wB[m]);
@@ -367,11 +379,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dBC
   {
     GemmAcc acc;
     acc.zero();
-    auto fa = [&](int r, int k) {  // (l, p)
-      const int l = st * GB + r;
-      return (l < qlim && k < P) ? ldg<T>(gv.ptr, gb + (int64_t)(t0 + l) * gv.ls + k) : 0.f;
-    };
-    block_gemm<SPLIT, true, false>(acc, lds, 0, P, fa, fstate(Hc), tid);
+    run(acc, static_cast<const T *>(gv.ptr) + gb, gv.ls, Hc);
     acc_foreach(acc, tid, [&](int m, int n, float v) {
       const int l = st * GB + m, nn = nt * GB + n;
       const float o = v * wC[m];
@@ -408,15 +416,15 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dcb
   const int64_t gb = b * gv.bs + h * gv.hs, xb = b * p.x_bs + h * p.x_hs;
   GemmAcc acc;
   acc.zero();
-  auto fa = [&](int r, int k) {  // (l, p)
-    const int l = lt * GB + r;
-    return (l < qlim && k < P) ? ldg<T>(gv.ptr, gb + (int64_t)(t0 + l) * gv.ls + k) : 0.f;
-  };
-  auto fb = [&](int r, int k) {  // (s, p)
-    const int s = st * GB + r;
-    return (s < qlim && k < P) ? ldg<T>(p.x, xb + (int64_t)(t0 + s) * p.x_ls + k) : 0.f;
-  };
-  block_gemm<SPLIT, true, true>(acc, lds, 0, P, fa, fb, tid);
+  // A = g rows (l, k = p), B = x rows (s, k = p): both k-contiguous
+  const T *ga = static_cast<const T *>(gv.ptr) + gb + (int64_t)(t0 + lt * GB) * gv.ls;
+  const T *xa = static_cast<const T *>(p.x) + xb + (int64_t)(t0 + st * GB) * p.x_ls;
+  const bool va = rows_aligned16(ga, gv.ls), vb = rows_aligned16(xa, p.x_ls);
+  block_gemm_staged<SPLIT>(
+      acc, lds, 0, P,
+      [&](int k0) { stage_kc<SPLIT, T>(lds.ah, lds.al, ga, gv.ls, qlim - lt * GB, k0, P, nullptr, nullptr, va, tid); },
+      [&](int k0) { stage_kc<SPLIT, T>(lds.bh, lds.bl, xa, p.x_ls, qlim - st * GB, k0, P, nullptr, nullptr, vb, tid); },
+      tid);
   float *dCB = p.dCB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
   const float *CB = p.CB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
   // acc <- w[l, s] = dCB_h[l, s] CB[l, s]
@@ -453,15 +461,19 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bmm_chu
   {
     GemmAcc acc;
     acc.zero();
-    auto fa = [&](int r, int k) {  // (l, s)
-      const int l = mt * GB + r;
-      return (l < qlim && k <= l) ? dCB[(int64_t)l * Q + k] : 0.f;
-    };
-    auto fb = [&](int r, int k) {  // (n, s)
-      const int n = nt * GB + r;
-      return (n < N && k < qlim) ? ldg<T>(p.B, Bb + (int64_t)(t0 + k) * p.B_ls + n) : 0.f;
-    };
-    block_gemm<SPLIT, true, false>(acc, lds, 0, min((mt + 1) * GB, qlim), fa, fb, tid);
+    // dCB is zero above the diagonal (never written), so no mask is needed here.
+    // A = dCB rows (l, k = s): k-contiguous fp32; B = B^T (rows n, k = s): row-contiguous
+    const float *da = dCB + (int64_t)mt * GB * Q;
+    const T *Ba = static_cast<const T *>(p.B) + Bb + (int64_t)t0 * p.B_ls + nt * GB;
+    const bool va = rows_aligned16(da, Q), vb = rows_aligned16(Ba, p.B_ls);
+    const int kend = min((mt + 1) * GB, qlim);
+    block_gemm_staged<SPLIT>(
+        acc, lds, 0, kend,
+        [&](int k0) { stage_kc<SPLIT, float>(lds.ah, lds.al, da, Q, qlim - mt * GB, k0, kend, nullptr, nullptr, va, tid); },
+        [&](int k0) {
+          if (tid < 128) stage_rc<SPLIT, T>(lds.bh, lds.bl, Ba, p.B_ls, N - nt * GB, k0, kend, nullptr, nullptr, vb, tid);
+        },
+        tid);
     acc_foreach(acc, tid, [&](int m, int n, float v) {
       const int l = mt * GB + m, nn = nt * GB + n;
       if (l < qlim && nn < N) p.dC32[(((int64_t)b * L + t0 + l) * G + g) * N + nn] += v;
@@ -471,15 +483,20 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bmm_chu
   {
     GemmAcc acc;
     acc.zero();
-    auto fa = [&](int r, int k) {  // (s, l)
-      const int s = mt * GB + r;
-      return (s < qlim && k < qlim && k >= s) ? dCB[(int64_t)k * Q + s] : 0.f;
-    };
-    auto fb = [&](int r, int k) {  // (n, l)
-      const int n = nt * GB + r;
-      return (n < N && k < qlim) ? ldg<T>(p.C, Cb + (int64_t)(t0 + k) * p.C_ls + n) : 0.f;
-    };
-    block_gemm<SPLIT, false, false>(acc, lds, mt * GB, qlim, fa, fb, tid);
+    // A = dCB^T (rows s, k = l): row-contiguous fp32; B = C^T (rows n, k = l): row-contiguous
+    const float *da = dCB + mt * GB;
+    const T *Ca = static_cast<const T *>(p.C) + Cb + (int64_t)t0 * p.C_ls + nt * GB;
+    const bool va = rows_aligned16(da, Q), vb = rows_aligned16(Ca, p.C_ls);
+    block_gemm_staged<SPLIT>(
+        acc, lds, mt * GB, qlim,
+        [&](int k0) {
+          if (tid < 128) stage_rc<SPLIT, float>(lds.ah, lds.al, da, Q, qlim - mt * GB, k0, qlim, nullptr, nullptr, va, tid);
+        },
+        [&](int k0) {
+          if (tid >= 128)
+            stage_rc<SPLIT, T>(lds.bh, lds.bl, Ca, p.C_ls, N - nt * GB, k0, qlim, nullptr, nullptr, vb, tid - 128);
+        },
+        tid);
     acc_foreach(acc, tid, [&](int m, int n, float v) {
       const int s = mt * GB + m, nn = nt * GB + n;
       if (s < qlim && nn < N) p.dB32[(((int64_t)b * L + t0 + s) * G + g) * N + nn] += v;

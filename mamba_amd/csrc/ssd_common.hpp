@@ -45,6 +45,106 @@ struct GemmLds {
   uint16_t ah[GTILE], al[GTILE], bh[GTILE], bl[GTILE];
 };
 
+// Offset of element (row, k) inside a staged 64 x 32 tile.  The four 8-element k groups of a row
+// are XOR-swizzled with (row / 8): 16-byte fragment reads stay conflict-free and the transposing
+// stores of row-contiguous sources (8 lanes writing rows 8 apart) no longer pile on one bank.
+DEVI int tile_off(int r, int k) { return r * GLD + ((((k >> 3) ^ (r >> 3)) & 3) << 3) + (k & 7); }
+
+template <bool SPLIT> DEVI void put8(uint16_t *hi, uint16_t *lo, int off, const float (&v)[8]) {
+  uint32_t h[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) h[e] = pack_bf16(v[2 * e], v[2 * e + 1]);
+  *reinterpret_cast<u32x4 *>(hi + off) = u32x4{h[0], h[1], h[2], h[3]};
+  if (SPLIT) {
+    uint32_t l[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      l[e] = pack_bf16(v[2 * e] - bf16_lo(h[e]), v[2 * e + 1] - bf16_hi(h[e]));
+    *reinterpret_cast<u32x4 *>(lo + off) = u32x4{l[0], l[1], l[2], l[3]};
+  }
+}
+
+// Vectorised staging of a k-contiguous source: element (r, k) at base[r * rstride + k].  All 256
+// threads take part (8 consecutive k each).  rows_valid / k_valid bound the source; kscale
+// (indexed by absolute k) and rscale (by tile row) are optional multipliers.  `vec` promises
+// 16-byte aligned rows (base and rstride), else every element is loaded on its own.
+template <bool SPLIT, typename S>
+DEVI void stage_kc(uint16_t *hi, uint16_t *lo, const S *base, int64_t rstride, int rows_valid, int k0, int k_valid,
+                   const float *kscale, const float *rscale, bool vec, int tid) {
+  const int r = tid >> 2, k8 = (tid & 3) * 8;
+  float v[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = 0.f;
+  if (r < rows_valid && k0 + k8 < k_valid) {
+    const S *src = base + (int64_t)r * rstride + k0 + k8;
+    if (vec && k0 + k8 + 8 <= k_valid) {
+      ld8<S>(src, v);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (k0 + k8 + e < k_valid) v[e] = ld1<S>(src + e);
+    }
+    if (kscale) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] *= kscale[k0 + k8 + e];
+    }
+    if (rscale) {
+      const float rs = rscale[r];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] *= rs;
+    }
+  }
+  put8<SPLIT>(hi, lo, tile_off(r, k8), v);
+}
+
+// Vectorised staging of a row-contiguous source: element (r, k) at base[k * kstride + r].  128
+// tasks (t = 0..127): 2 consecutive k x 8 consecutive rows, stored transposed as 4-byte pairs.
+template <bool SPLIT, typename S>
+DEVI void stage_rc(uint16_t *hi, uint16_t *lo, const S *base, int64_t kstride, int rows_valid, int k0, int k_valid,
+                   const float *kscale, const float *rscale, bool vec, int t) {
+  const int k2 = (t >> 3) * 2, r8 = (t & 7) * 8;
+  float v[2][8];
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const int k = k0 + k2 + q;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[q][e] = 0.f;
+    if (k < k_valid && r8 < rows_valid) {
+      const S *src = base + (int64_t)k * kstride + r8;
+      if (vec && r8 + 8 <= rows_valid) {
+        ld8<S>(src, v[q]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (r8 + e < rows_valid) v[q][e] = ld1<S>(src + e);
+      }
+      if (kscale) {
+        const float ks = kscale[k];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[q][e] *= ks;
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    float a = v[0][e], b = v[1][e];
+    if (rscale) {
+      const float rs = rscale[r8 + e];
+      a *= rs;
+      b *= rs;
+    }
+    const int off = tile_off(r8 + e, k2);
+    const uint32_t h = pack_bf16(a, b);
+    *reinterpret_cast<uint32_t *>(hi + off) = h;
+    if (SPLIT) *reinterpret_cast<uint32_t *>(lo + off) = pack_bf16(a - bf16_lo(h), b - bf16_hi(h));
+  }
+}
+
+template <typename S> DEVI bool rows_aligned16(const S *base, int64_t stride) {
+  constexpr int m = 16 / sizeof(S);
+  return (reinterpret_cast<uintptr_t>(base) & 15) == 0 && stride % m == 0;
+}
+
 // Fills a 64 x 32 tile from a functor f(row, k) -> float.  K_FAST: consecutive
 // threads walk k (use when the source is contiguous along k), else along rows.
 template <bool SPLIT, bool K_FAST, typename F> DEVI void stage_tile(uint16_t *hi, uint16_t *lo, F f, int tid) {
@@ -60,8 +160,8 @@ template <bool SPLIT, bool K_FAST, typename F> DEVI void stage_tile(uint16_t *hi
     }
     const float v = f(r, k);
     const uint16_t h = bf16_bits(v);
-    hi[r * GLD + k] = h;
-    if (SPLIT) lo[r * GLD + k] = bf16_bits(v - bf16_val(h));
+    hi[tile_off(r, k)] = h;
+    if (SPLIT) lo[tile_off(r, k)] = bf16_bits(v - bf16_val(h));
   }
 }
 
@@ -81,11 +181,12 @@ template <bool SPLIT> DEVI void mma_step(GemmAcc &acc, const GemmLds &s, int wm,
   bf16x8_t a[2], b[2], al[2], bl[2];
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
-    a[t] = *reinterpret_cast<const bf16x8_t *>(&s.ah[(wm * 32 + t * 16 + i) * GLD + g * 8]);
-    b[t] = *reinterpret_cast<const bf16x8_t *>(&s.bh[(wn * 32 + t * 16 + i) * GLD + g * 8]);
+    const int oa = tile_off(wm * 32 + t * 16 + i, g * 8), ob = tile_off(wn * 32 + t * 16 + i, g * 8);
+    a[t] = *reinterpret_cast<const bf16x8_t *>(&s.ah[oa]);
+    b[t] = *reinterpret_cast<const bf16x8_t *>(&s.bh[ob]);
     if (SPLIT) {
-      al[t] = *reinterpret_cast<const bf16x8_t *>(&s.al[(wm * 32 + t * 16 + i) * GLD + g * 8]);
-      bl[t] = *reinterpret_cast<const bf16x8_t *>(&s.bl[(wn * 32 + t * 16 + i) * GLD + g * 8]);
+      al[t] = *reinterpret_cast<const bf16x8_t *>(&s.al[oa]);
+      bl[t] = *reinterpret_cast<const bf16x8_t *>(&s.bl[ob]);
     }
   }
 #pragma unroll
@@ -109,6 +210,20 @@ DEVI void block_gemm(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, FA fa, FB
     __syncthreads();
     stage_tile<SPLIT, A_KFAST>(s.ah, s.al, [&](int r, int k) { return fa(r, k0 + k); }, tid);
     stage_tile<SPLIT, B_KFAST>(s.bh, s.bl, [&](int r, int k) { return fb(r, k0 + k); }, tid);
+    __syncthreads();
+    mma_step<SPLIT>(acc, s, wm, wn, lane);
+  }
+}
+
+// Same with caller-supplied stagers: stage_a(k0) / stage_b(k0) fill the A / B tile for the k step
+// starting at k0 (all 256 threads call both).
+template <bool SPLIT, typename SA, typename SB>
+DEVI void block_gemm_staged(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, SA stage_a, SB stage_b, int tid) {
+  const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+  for (int k0 = k_begin; k0 < k_end; k0 += GK) {
+    __syncthreads();
+    stage_a(k0);
+    stage_b(k0);
     __syncthreads();
     mma_step<SPLIT>(acc, s, wm, wn, lane);
   }

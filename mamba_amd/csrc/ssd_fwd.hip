@@ -80,15 +80,15 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bmm_chu
   const int64_t Cb = b * p.C_bs + g * p.C_gs, Bb = b * p.B_bs + g * p.B_gs;
   GemmAcc acc;
   acc.zero();
-  auto fa = [&](int r, int k) {
-    const int l = mt * GB + r;
-    return (l < Q && t0 + l < L && k < N) ? ldg<T>(p.C, Cb + (int64_t)(t0 + l) * p.C_ls + k) : 0.f;
-  };
-  auto fb = [&](int r, int k) {
-    const int s = nt * GB + r;
-    return (s < Q && t0 + s < L && k < N) ? ldg<T>(p.B, Bb + (int64_t)(t0 + s) * p.B_ls + k) : 0.f;
-  };
-  block_gemm<SPLIT, true, true>(acc, lds, 0, N, fa, fb, tid);
+  const int qlim = min(Q, L - t0);
+  const T *Ca = static_cast<const T *>(p.C) + Cb + (int64_t)(t0 + mt * GB) * p.C_ls;
+  const T *Ba = static_cast<const T *>(p.B) + Bb + (int64_t)(t0 + nt * GB) * p.B_ls;
+  const bool va = rows_aligned16(Ca, p.C_ls), vb = rows_aligned16(Ba, p.B_ls);
+  block_gemm_staged<SPLIT>(
+      acc, lds, 0, N,
+      [&](int k0) { stage_kc<SPLIT, T>(lds.ah, lds.al, Ca, p.C_ls, qlim - mt * GB, k0, N, nullptr, nullptr, va, tid); },
+      [&](int k0) { stage_kc<SPLIT, T>(lds.bh, lds.bl, Ba, p.B_ls, qlim - nt * GB, k0, N, nullptr, nullptr, vb, tid); },
+      tid);
   float *CB = p.CB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
   const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
   acc_foreach(acc, tid, [&](int m, int n, float v) {
@@ -135,15 +135,20 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void chunk_s
   const int64_t xb = b * p.x_bs + h * p.x_hs, Bb = b * p.B_bs + g * p.B_gs;
   GemmAcc acc;
   acc.zero();
-  auto fa = [&](int r, int k) {  // (p, s)
-    const int pp = pt * GB + r;
-    return (pp < P && k < qlim) ? ldg<T>(p.x, xb + (int64_t)(t0 + k) * p.x_ls + pp) : 0.f;
-  };
-  auto fb = [&](int r, int k) {  // (n, s)
-    const int n = nt * GB + r;
-    return (n < N && k < qlim) ? ldg<T>(p.B, Bb + (int64_t)(t0 + k) * p.B_ls + n) * w[k] : 0.f;
-  };
-  block_gemm<SPLIT, false, false>(acc, lds, 0, qlim, fa, fb, tid);  // first __syncthreads publishes w
+  // A = x^T (rows p, k = position), B = (B w)^T (rows n, k = position): both row-contiguous sources
+  const T *xa = static_cast<const T *>(p.x) + xb + (int64_t)t0 * p.x_ls + pt * GB;
+  const T *Ba = static_cast<const T *>(p.B) + Bb + (int64_t)t0 * p.B_ls + nt * GB;
+  const bool va = rows_aligned16(xa, p.x_ls), vb = rows_aligned16(Ba, p.B_ls);
+  block_gemm_staged<SPLIT>(  // the first barrier inside publishes w
+      acc, lds, 0, qlim,
+      [&](int k0) {
+        if (tid < 128) stage_rc<SPLIT, T>(lds.ah, lds.al, xa, p.x_ls, P - pt * GB, k0, qlim, nullptr, nullptr, va, tid);
+      },
+      [&](int k0) {
+        if (tid >= 128)
+          stage_rc<SPLIT, T>(lds.bh, lds.bl, Ba, p.B_ls, N - nt * GB, k0, qlim, w, nullptr, vb, tid - 128);
+      },
+      tid);
   float *st = p.states + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
   acc_foreach(acc, tid, [&](int m, int n, float v) {
     const int pp = pt * GB + m, nn = nt * GB + n;
