@@ -25,6 +25,10 @@ DEVI View4 g_view(const SsdParams &p) {
   return {p.dout, p.dout_bs, p.dout_ls, p.dout_hs};
 }
 
+// The heads of a group are spread over this many workgroups (each sums ~8 heads in registers and
+// adds its partial result atomically).
+__host__ __device__ inline int head_splits(int heads_per_group) { return (heads_per_group + 7) / 8; }
+
 DEVI float *chunk_row(float *base, const SsdParams &p, int b, int h, int c) {
   return base + (((int64_t)b * p.nheads + h) * p.nchunks + c) * p.chunk_size;
 }
@@ -317,8 +321,11 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
 }
 
 // ---------------------------------------------- state-path parts of dB, dC
-// dB32[s, n] += exp(a_last - a_s) dt_s [s in last sequence] sum_p x[s, p] dS[p, n]
-// dC32[l, n] += exp(a_l) [seq_l == seq before the chunk]    sum_p g[l, p] Hc[p, n]
+// dB32[s, n] = sum_{h in group} exp(a_last - a_s) dt_s [s in last sequence] sum_p x[s, p] dS[p, n]
+// dC32[l, n] = sum_{h in group} exp(a_l) [seq_l == seq before the chunk]    sum_p g[l, p] Hc[p, n]
+// One workgroup per (batch, chunk, group, 64 x 64 tile) loops over the heads of the group and keeps
+// both sums in registers (no atomics); the per-head row factor is folded into the A operand.
+// The carried-state share of ddA_cumsum, sum_n dC_h[l, n] C[l, n], is taken per head on the way.
 template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dBC_state_kernel(const SsdParams p) {
   __shared__ GemmLds lds;
   __shared__ float wB[GB], wC[GB], rsum[GB];
@@ -326,78 +333,84 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dBC
   const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads, G = p.ngroups;
   const int ntn = cdiv(N, GB);
   const int st = blockIdx.x / ntn, nt = blockIdx.x % ntn;
-  const int c = blockIdx.y, b = blockIdx.z / H, h = blockIdx.z % H;
-  const int g = h / (H / G);
+  const int hpg = H / G, nsplit = head_splits(hpg);
+  const int c = blockIdx.y, bg = blockIdx.z / nsplit, hs = blockIdx.z % nsplit, b = bg / G, g = bg % G;
   const int t0 = c * Q, qlim = min(Q, L - t0);
-  const float *dA = chunk_row(p.dA_cumsum, p, b, h, c);
-  const float *dt = chunk_row(p.dt_out, p, b, h, c);
   const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
-  if (tid < GB) {
-    const int s = st * GB + tid;
-    float vb = 0.f, vc = 0.f;
-    if (s < qlim) {
-      bool okb = true, okc = true;
-      if (seq) {
-        const int last = seq[qlim - 1];
-        okb = last >= 0 && seq[s] == last;
-        okc = seq[s] == (c > 0 ? seq[-1] : 0);
-      }
-      if (okb) vb = fast_exp(fminf(dA[Q - 1] - dA[s], 0.f)) * dt[s];
-      if (okc) vc = fast_exp(dA[s]);
-    }
-    wB[tid] = vb;
-    wC[tid] = vc;
-  }
   const View4 gv = g_view(p);
-  const int64_t gb = b * gv.bs + h * gv.hs, xb = b * p.x_bs + h * p.x_hs;
-  const float *dS = p.dstates + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
-  const float *Hc = p.states + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
-  // A = x or g rows (position, k = p): k-contiguous; B = state rows n, k = p: row-contiguous fp32
-  const bool vs = rows_aligned16(dS + nt * GB, N) && rows_aligned16(Hc + nt * GB, N);
-  auto run = [&](GemmAcc &acc, const T *a_base, int64_t a_ls, const float *S) {
-    const T *aa = a_base + (int64_t)(t0 + st * GB) * a_ls;
-    const bool va = rows_aligned16(aa, a_ls);
-    block_gemm_staged<SPLIT>(
-        acc, lds, 0, P,
-        [&](int k0) { stage_kc<SPLIT, T>(lds.ah, lds.al, aa, a_ls, qlim - st * GB, k0, P, nullptr, nullptr, va, tid); },
-        [&](int k0) {
-          if (tid < 128)
-            stage_rc<SPLIT, float>(lds.bh, lds.bl, S + nt * GB, N, N - nt * GB, k0, P, nullptr, nullptr, vs, tid);
-        },
-        tid);
-  };
-  {
-    GemmAcc acc;
-    acc.zero();
-    run(acc, static_cast<const T *>(p.x) + xb, p.x_ls, dS);
-    acc_foreach(acc, tid, [&](int m, int n, float v) {
-      const int s = st * GB + m, nn = nt * GB + n;
-      if (s < qlim && nn < N) unsafeAtomicAdd(p.dB32 + (((int64_t)b * L + t0 + s) * G + g) * N + nn, v * wB[m]);
-      return v;
-    });
-  }
-  {
-    GemmAcc acc;
-    acc.zero();
-    run(acc, static_cast<const T *>(gv.ptr) + gb, gv.ls, Hc);
-    acc_foreach(acc, tid, [&](int m, int n, float v) {
-      const int l = st * GB + m, nn = nt * GB + n;
-      const float o = v * wC[m];
-      if (l < qlim && nn < N) unsafeAtomicAdd(p.dC32 + (((int64_t)b * L + t0 + l) * G + g) * N + nn, o);
-      return o;
-    });
-    const int64_t Cb = b * p.C_bs + g * p.C_gs;
-    row_dot(acc, rsum, tid, [&](int m, int n) {
+  const int64_t Cb = b * p.C_bs + g * p.C_gs;
+  GemmAcc accB, accC;
+  accB.zero();
+  accC.zero();
+  for (int hh = hs; hh < hpg; hh += nsplit) {
+    const int h = g * hpg + hh;
+    const float *dA = chunk_row(p.dA_cumsum, p, b, h, c);
+    const float *dt = chunk_row(p.dt_out, p, b, h, c);
+    __syncthreads();  // previous head's wB / wC / rsum readers are done
+    if (tid < GB) {
+      const int s = st * GB + tid;
+      float vb = 0.f, vc = 0.f;
+      if (s < qlim) {
+        bool okb = true, okc = true;
+        if (seq) {
+          const int last = seq[qlim - 1];
+          okb = last >= 0 && seq[s] == last;
+          okc = seq[s] == (c > 0 ? seq[-1] : 0);
+        }
+        if (okb) vb = fast_exp(fminf(dA[Q - 1] - dA[s], 0.f)) * dt[s];
+        if (okc) vc = fast_exp(dA[s]);
+      }
+      wB[tid] = vb;
+      wC[tid] = vc;
+    }
+    const int64_t gb = b * gv.bs + h * gv.hs, xb = b * p.x_bs + h * p.x_hs;
+    const float *dS = p.dstates + (((int64_t)b * p.nchunks + c) * H + h) * P * N + nt * GB;
+    const float *Hc = p.states + (((int64_t)b * p.nchunks + c) * H + h) * P * N + nt * GB;
+    const bool vs = rows_aligned16(dS, N) && rows_aligned16(Hc, N);
+    // A = (w x) or (w g) rows (position, k = p): k-contiguous; B = state rows n, k = p: row-contiguous fp32
+    auto run = [&](GemmAcc &acc, const T *a_base, int64_t a_ls, const float *w, const float *S) {
+      const T *aa = a_base + (int64_t)(t0 + st * GB) * a_ls;
+      const bool va = rows_aligned16(aa, a_ls);
+      block_gemm_staged<SPLIT>(  // the first barrier inside publishes wB / wC
+          acc, lds, 0, P,
+          [&](int k0) { stage_kc<SPLIT, T>(lds.ah, lds.al, aa, a_ls, qlim - st * GB, k0, P, nullptr, w, va, tid); },
+          [&](int k0) {
+            if (tid < 128) stage_rc<SPLIT, float>(lds.bh, lds.bl, S, N, N - nt * GB, k0, P, nullptr, nullptr, vs, tid);
+          },
+          tid);
+    };
+    run(accB, static_cast<const T *>(p.x) + xb, p.x_ls, wB, dS);
+    GemmAcc accH;
+    accH.zero();
+    run(accH, static_cast<const T *>(gv.ptr) + gb, gv.ls, wC, Hc);
+    row_dot(accH, rsum, tid, [&](int m, int n) {
       const int l = st * GB + m, nn = nt * GB + n;
       return (l < qlim && nn < N) ? ldg<T>(p.C, Cb + (int64_t)(t0 + l) * p.C_ls + nn) : 0.f;
     });
     if (tid < GB && st * GB + tid < qlim)
       unsafeAtomicAdd(chunk_row(p.ddA_cumsum, p, b, h, c) + st * GB + tid, rsum[tid]);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) accC.v[i][j] += accH.v[i][j];
   }
+  acc_foreach(accB, tid, [&](int m, int n, float v) {
+    const int s = st * GB + m, nn = nt * GB + n;
+    if (s < qlim && nn < N) unsafeAtomicAdd(p.dB32 + (((int64_t)b * L + t0 + s) * G + g) * N + nn, v);
+    return v;
+  });
+  acc_foreach(accC, tid, [&](int m, int n, float v) {
+    const int l = st * GB + m, nn = nt * GB + n;
+    if (l < qlim && nn < N) unsafeAtomicAdd(p.dC32 + (((int64_t)b * L + t0 + l) * G + g) * N + nn, v);
+    return v;
+  });
 }
 
 // ------------------------------------------------------------------ dCB
-// dCB[b, c, g, l, s] += (sum_p g[l, p] x[s, p]) dt_s exp(a_l - a_s)   for l >= s in one sequence
+// dCB[b, c, g, l, s] = sum_{h in group} (sum_p g[l, p] x[s, p]) dt_s exp(a_l - a_s)   for l >= s in
+// one sequence.  One workgroup per (batch, chunk, group, lower-triangular 64 x 64 tile pair) loops
+// over the heads of the group with the sum in registers.  Per head, w = (head's term) * CB gives
+// the in-chunk share of ddA_cumsum: + row sums at l, - column sums at s.
 template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dcb_kernel(const SsdParams p) {
   __shared__ GemmLds lds;
   __shared__ float rows[GB], cols[GB];
@@ -406,44 +419,64 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dcb
   int lt = 0, rem = blockIdx.x;
   while (rem > lt) { rem -= lt + 1; ++lt; }
   const int st = rem;
-  const int c = blockIdx.y, b = blockIdx.z / H, h = blockIdx.z % H;
-  const int g = h / (H / G);
+  const int hpg = H / G, nsplit = head_splits(hpg);
+  const int c = blockIdx.y, bg = blockIdx.z / nsplit, hs = blockIdx.z % nsplit, b = bg / G, g = bg % G;
   const int t0 = c * Q, qlim = min(Q, L - t0);
-  const float *dA = chunk_row(p.dA_cumsum, p, b, h, c);
-  const float *dt = chunk_row(p.dt_out, p, b, h, c);
   const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
   const View4 gv = g_view(p);
-  const int64_t gb = b * gv.bs + h * gv.hs, xb = b * p.x_bs + h * p.x_hs;
-  GemmAcc acc;
-  acc.zero();
-  // A = g rows (l, k = p), B = x rows (s, k = p): both k-contiguous
-  const T *ga = static_cast<const T *>(gv.ptr) + gb + (int64_t)(t0 + lt * GB) * gv.ls;
-  const T *xa = static_cast<const T *>(p.x) + xb + (int64_t)(t0 + st * GB) * p.x_ls;
-  const bool va = rows_aligned16(ga, gv.ls), vb = rows_aligned16(xa, p.x_ls);
-  block_gemm_staged<SPLIT>(
-      acc, lds, 0, P,
-      [&](int k0) { stage_kc<SPLIT, T>(lds.ah, lds.al, ga, gv.ls, qlim - lt * GB, k0, P, nullptr, nullptr, va, tid); },
-      [&](int k0) { stage_kc<SPLIT, T>(lds.bh, lds.bl, xa, p.x_ls, qlim - st * GB, k0, P, nullptr, nullptr, vb, tid); },
-      tid);
   float *dCB = p.dCB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
   const float *CB = p.CB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
-  // acc <- w[l, s] = dCB_h[l, s] CB[l, s]
-  acc_foreach(acc, tid, [&](int m, int n, float v) {
-    const int l = lt * GB + m, s = st * GB + n;
-    if (l < qlim && s <= l && (!seq || seq[l] == seq[s])) {
-      const float d = v * dt[s] * fast_exp(fminf(dA[l] - dA[s], 0.f));
-      unsafeAtomicAdd(dCB + (int64_t)l * Q + s, d);
-      return d * CB[(int64_t)l * Q + s];
+  GemmAcc sum;
+  sum.zero();
+  for (int hh = hs; hh < hpg; hh += nsplit) {
+    const int h = g * hpg + hh;
+    const float *dA = chunk_row(p.dA_cumsum, p, b, h, c);
+    const float *dt = chunk_row(p.dt_out, p, b, h, c);
+    const int64_t gb = b * gv.bs + h * gv.hs, xb = b * p.x_bs + h * p.x_hs;
+    GemmAcc acc;
+    acc.zero();
+    // A = g rows (l, k = p), B = x rows (s, k = p): both k-contiguous
+    const T *ga = static_cast<const T *>(gv.ptr) + gb + (int64_t)(t0 + lt * GB) * gv.ls;
+    const T *xa = static_cast<const T *>(p.x) + xb + (int64_t)(t0 + st * GB) * p.x_ls;
+    const bool va = rows_aligned16(ga, gv.ls), vb = rows_aligned16(xa, p.x_ls);
+    block_gemm_staged<SPLIT>(
+        acc, lds, 0, P,
+        [&](int k0) { stage_kc<SPLIT, T>(lds.ah, lds.al, ga, gv.ls, qlim - lt * GB, k0, P, nullptr, nullptr, va, tid); },
+        [&](int k0) { stage_kc<SPLIT, T>(lds.bh, lds.bl, xa, p.x_ls, qlim - st * GB, k0, P, nullptr, nullptr, vb, tid); },
+        tid);
+    // acc <- this head's dCB term; sum += it; acc <- w[l, s] = term * CB[l, s]
+    {
+      const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+      const int i = lane & 15, gq = lane >> 4;
+#pragma unroll
+      for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int l = lt * GB + wm * 32 + tm * 16 + gq * 4 + r, s = st * GB + wn * 32 + tn * 16 + i;
+            float d = 0.f, w = 0.f;
+            if (l < qlim && s <= l && (!seq || seq[l] == seq[s])) {
+              d = acc.v[tm][tn][r] * dt[s] * fast_exp(fminf(dA[l] - dA[s], 0.f));
+              w = d * CB[(int64_t)l * Q + s];
+            }
+            sum.v[tm][tn][r] += d;
+            acc.v[tm][tn][r] = w;
+          }
     }
-    return 0.f;
-  });
-  row_col_sums(acc, rows, cols, tid);
-  if (tid < GB) {
-    float *dda = chunk_row(p.ddA_cumsum, p, b, h, c);
-    const int l = lt * GB + tid, s = st * GB + tid;
-    if (l < qlim && rows[tid] != 0.f) unsafeAtomicAdd(dda + l, rows[tid]);
-    if (s < qlim && cols[tid] != 0.f) unsafeAtomicAdd(dda + s, -cols[tid]);
+    row_col_sums(acc, rows, cols, tid);
+    if (tid < GB) {
+      float *dda = chunk_row(p.ddA_cumsum, p, b, h, c);
+      const int l = lt * GB + tid, s = st * GB + tid;
+      if (l < qlim && rows[tid] != 0.f) unsafeAtomicAdd(dda + l, rows[tid]);
+      if (s < qlim && cols[tid] != 0.f) unsafeAtomicAdd(dda + s, -cols[tid]);
+    }
   }
+  acc_foreach(sum, tid, [&](int m, int n, float v) {
+    const int l = lt * GB + m, s = st * GB + n;
+    if (l < Q && s < Q && v != 0.f) unsafeAtomicAdd(dCB + (int64_t)l * Q + s, v);  // dCB starts zeroed
+    return v;
+  });
 }
 
 // ------------------------------------------------------------- bmm bwd
@@ -638,7 +671,8 @@ extern "C" int ssd_bwd_dBC_state(const SsdParams *p, mamba_stream_t stream) {
   int rc = check_bwd(p);
   if (rc) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  dim3 grid(tiles(p->chunk_size) * tiles(p->dstate), p->nchunks, p->batch * p->nheads);
+  dim3 grid(tiles(p->chunk_size) * tiles(p->dstate), p->nchunks,
+            p->batch * p->ngroups * head_splits(p->nheads / p->ngroups));
   SSD_DISPATCH(bwd_dBC_state_kernel, grid)
   return launched();
 }
@@ -648,7 +682,7 @@ extern "C" int ssd_bwd_dcb(const SsdParams *p, mamba_stream_t stream) {
   if (rc) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int nt = tiles(p->chunk_size);
-  dim3 grid(nt * (nt + 1) / 2, p->nchunks, p->batch * p->nheads);
+  dim3 grid(nt * (nt + 1) / 2, p->nchunks, p->batch * p->ngroups * head_splits(p->nheads / p->ngroups));
   SSD_DISPATCH(bwd_dcb_kernel, grid)
   return launched();
 }
