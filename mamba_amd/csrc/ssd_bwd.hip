@@ -97,46 +97,96 @@ DEVI void row_col_sums(GemmAcc &acc, float *rows, float *cols, int tid) {
 }
 
 // ------------------------------------------------------------------- dz
-// Per position: dz, g = dout silu(z), dD += g x.
+// Per position: dz, g = dout silu(z), dD += g x.  A lane owns 8 consecutive p of one position
+// (16-byte accesses when the rows allow it); a workgroup covers 64 positions of one (batch, head).
 template <typename T> __global__ __launch_bounds__(256) void bwd_dz_kernel(const SsdParams p) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tid = threadIdx.x;
   const int L = p.seqlen, H = p.nheads, P = p.headdim;
   const int h = blockIdx.y, b = blockIdx.z;
+  const int pchunks = (P + 7) / 8;                 // 8-wide column groups per row
   const float *Dp = static_cast<const float *>(p.D);
   const void *yptr = p.z ? p.out_x : p.out;
-  float dDacc[4] = {0.f, 0.f, 0.f, 0.f};
-  for (int j = 0; j < 16; ++j) {
-    const int t = blockIdx.x * 64 + wave + 4 * j;
+  const bool vec = P % 8 == 0 && rows_aligned16(static_cast<const T *>(p.dout) + b * p.dout_bs + h * p.dout_hs, p.dout_ls) &&
+                   rows_aligned16(static_cast<const T *>(p.x) + b * p.x_bs + h * p.x_hs, p.x_ls) &&
+                   (!p.z || (rows_aligned16(static_cast<const T *>(p.z) + b * p.z_bs + h * p.z_hs, p.z_ls) &&
+                             rows_aligned16(static_cast<const T *>(yptr) + b * p.out_bs + h * p.out_hs, p.out_ls)));
+  // every thread keeps one column group (tid % pchunks is fixed when 256 % pchunks == 0; otherwise
+  // the partial dD sums are flushed per task)
+  const bool fixed_cols = 256 % pchunks == 0;
+  float dDacc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  const int ntask = 64 * pchunks;
+  for (int task = tid; task < ntask; task += 256) {
+    const int t = blockIdx.x * 64 + task / pchunks, c8 = (task % pchunks) * 8;
     if (t >= L) break;
+    const int nv = min(8, P - c8);
+    float dout[8], x[8], g[8];
+    const T *dop = static_cast<const T *>(p.dout) + b * p.dout_bs + (int64_t)t * p.dout_ls + h * p.dout_hs + c8;
+    const T *xp = static_cast<const T *>(p.x) + b * p.x_bs + (int64_t)t * p.x_ls + h * p.x_hs + c8;
+    if (vec) {
+      ld8<T>(dop, dout);
+      ld8<T>(xp, x);
+    } else {
+      ld8_guard<T, false>(dop, nv, 0.f, dout);
+      ld8_guard<T, false>(xp, nv, 0.f, x);
+    }
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int pp = lane + 64 * q;
-      if (pp >= P) break;
-      const float dout = ldg<T>(p.dout, b * p.dout_bs + (int64_t)t * p.dout_ls + h * p.dout_hs + pp);
-      const float x = ldg<T>(p.x, b * p.x_bs + (int64_t)t * p.x_ls + h * p.x_hs + pp);
-      float g = dout;
-      if (p.z) {
-        const float y = ldg<T>(yptr, b * p.out_bs + (int64_t)t * p.out_ls + h * p.out_hs + pp);
-        const float z = ldg<T>(p.z, b * p.z_bs + (int64_t)t * p.z_ls + h * p.z_hs + pp);
-        const float sg = sigmoid_f(z);
-        g = dout * z * sg;
-        const int64_t oi = (((int64_t)b * L + t) * H + h) * P + pp;
-        stg<T>(p.dz, oi, dout * y * sg * (1.f + z * (1.f - sg)));
-        stg<T>(p.gbuf, oi, g);
+    for (int e = 0; e < 8; ++e) g[e] = dout[e];
+    if (p.z) {
+      float y[8], z[8], dz[8];
+      const T *yp = static_cast<const T *>(yptr) + b * p.out_bs + (int64_t)t * p.out_ls + h * p.out_hs + c8;
+      const T *zp = static_cast<const T *>(p.z) + b * p.z_bs + (int64_t)t * p.z_ls + h * p.z_hs + c8;
+      if (vec) {
+        ld8<T>(yp, y);
+        ld8<T>(zp, z);
+      } else {
+        ld8_guard<T, false>(yp, nv, 0.f, y);
+        ld8_guard<T, false>(zp, nv, 0.f, z);
       }
-      dDacc[q] = __builtin_fmaf(g, x, dDacc[q]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float sg = sigmoid_f(z[e]);
+        g[e] = dout[e] * z[e] * sg;
+        dz[e] = dout[e] * y[e] * sg * (1.f + z[e] * (1.f - sg));
+      }
+      const int64_t oi = (((int64_t)b * L + t) * H + h) * P + c8;
+      if (vec) {
+        st8<T>(static_cast<T *>(p.dz) + oi, dz);
+        st8<T>(static_cast<T *>(p.gbuf) + oi, g);
+      } else {
+        st8_guard<T, false>(static_cast<T *>(p.dz) + oi, nv, dz);
+        st8_guard<T, false>(static_cast<T *>(p.gbuf) + oi, nv, g);
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) dDacc[e] = __builtin_fmaf(g[e], x[e], dDacc[e]);
+    if (Dp && !fixed_cols) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if (e < nv) unsafeAtomicAdd(p.dD + (p.D_has_hdim ? h * P + c8 + e : h), dDacc[e]);
+        dDacc[e] = 0.f;
+      }
     }
   }
-  if (Dp) {
-    if (p.D_has_hdim) {
+  if (Dp && fixed_cols) {
+    __shared__ float red[256 * 9];                 // row stride 9: conflict-free column reads
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int pp = lane + 64 * q;
-        if (pp < P) unsafeAtomicAdd(p.dD + h * P + pp, dDacc[q]);
+    for (int e = 0; e < 8; ++e) red[tid * 9 + e] = dDacc[e];
+    __syncthreads();
+    if (p.D_has_hdim) {
+      // column c of the head: threads with tid % pchunks == c / 8 hold its partial sums
+      if (tid < P) {
+        float sacc = 0.f;
+        for (int r = tid / 8; r < 256; r += pchunks) sacc += red[r * 9 + (tid & 7)];
+        unsafeAtomicAdd(p.dD + h * P + tid, sacc);
       }
-    } else {
-      const float s = wave_sum(dDacc[0] + dDacc[1] + dDacc[2] + dDacc[3]);
-      if (lane == 0) unsafeAtomicAdd(p.dD + h, s);
+    } else if (tid < 64) {
+      float sacc = 0.f;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sacc += red[(tid * 4 + r) * 9 + e];
+      sacc = wave_sum(sacc);
+      if (tid == 0) unsafeAtomicAdd(p.dD + h, sacc);
     }
   }
 }

@@ -15,7 +15,7 @@
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 
 constexpr int GB = 64;         // block tile edge (M and N)
-constexpr int GK = 32;         // k step
+constexpr int GK = 32;         // k step (one MFMA k-slice per barrier pair; 64 measured slower)
 constexpr int GLD = GK + 8;    // LDS row pitch in bf16 (80 bytes: conflict-free 16-byte reads)
 constexpr int GTILE = GB * GLD;
 
@@ -45,10 +45,10 @@ struct GemmLds {
   uint16_t ah[GTILE], al[GTILE], bh[GTILE], bl[GTILE];
 };
 
-// Offset of element (row, k) inside a staged 64 x 32 tile.  The four 8-element k groups of a row
+// Offset of element (row, k) inside a staged 64 x GK tile.  The 8-element k groups of a row
 // are XOR-swizzled with (row / 8): 16-byte fragment reads stay conflict-free and the transposing
 // stores of row-contiguous sources (8 lanes writing rows 8 apart) no longer pile on one bank.
-DEVI int tile_off(int r, int k) { return r * GLD + ((((k >> 3) ^ (r >> 3)) & 3) << 3) + (k & 7); }
+DEVI int tile_off(int r, int k) { return r * GLD + ((((k >> 3) ^ (r >> 3)) & (GK / 8 - 1)) << 3) + (k & 7); }
 
 template <bool SPLIT> DEVI void put8(uint16_t *hi, uint16_t *lo, int off, const float (&v)[8]) {
   uint32_t h[4];
@@ -71,7 +71,10 @@ template <bool SPLIT> DEVI void put8(uint16_t *hi, uint16_t *lo, int off, const 
 template <bool SPLIT, typename S>
 DEVI void stage_kc(uint16_t *hi, uint16_t *lo, const S *base, int64_t rstride, int rows_valid, int k0, int k_valid,
                    const float *kscale, const float *rscale, bool vec, int tid) {
-  const int r = tid >> 2, k8 = (tid & 3) * 8;
+  constexpr int KG = GK / 8;  // 8-element groups per row
+#pragma unroll
+  for (int task = tid; task < GB * KG; task += 256) {
+  const int r = task / KG, k8 = (task % KG) * 8;
   float v[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) v[e] = 0.f;
@@ -95,14 +98,18 @@ DEVI void stage_kc(uint16_t *hi, uint16_t *lo, const S *base, int64_t rstride, i
     }
   }
   put8<SPLIT>(hi, lo, tile_off(r, k8), v);
+  }
 }
 
-// Vectorised staging of a row-contiguous source: element (r, k) at base[k * kstride + r].  128
-// tasks (t = 0..127): 2 consecutive k x 8 consecutive rows, stored transposed as 4-byte pairs.
+// Vectorised staging of a row-contiguous source: element (r, k) at base[k * kstride + r].  Tasks
+// are 2 consecutive k x 8 consecutive rows, stored transposed as 4-byte pairs; the 128 threads
+// t = 0..127 of the calling half of the workgroup share the GK / 2 * 8 tasks.
 template <bool SPLIT, typename S>
 DEVI void stage_rc(uint16_t *hi, uint16_t *lo, const S *base, int64_t kstride, int rows_valid, int k0, int k_valid,
                    const float *kscale, const float *rscale, bool vec, int t) {
-  const int k2 = (t >> 3) * 2, r8 = (t & 7) * 8;
+#pragma unroll
+  for (int task = t; task < (GK / 2) * 8; task += 128) {
+  const int k2 = (task >> 3) * 2, r8 = (task & 7) * 8;
   float v[2][8];
 #pragma unroll
   for (int q = 0; q < 2; ++q) {
@@ -138,6 +145,7 @@ DEVI void stage_rc(uint16_t *hi, uint16_t *lo, const S *base, int64_t kstride, i
     *reinterpret_cast<uint32_t *>(hi + off) = h;
     if (SPLIT) *reinterpret_cast<uint32_t *>(lo + off) = pack_bf16(a - bf16_lo(h), b - bf16_hi(h));
   }
+  }
 }
 
 template <typename S> DEVI bool rows_aligned16(const S *base, int64_t stride) {
@@ -152,11 +160,11 @@ template <bool SPLIT, bool K_FAST, typename F> DEVI void stage_tile(uint16_t *hi
   for (int idx = tid; idx < GB * GK; idx += 256) {
     int r, k;
     if (K_FAST) {
-      k = idx & (GK - 1);
-      r = idx >> 5;
+      k = idx % GK;
+      r = idx / GK;
     } else {
-      r = idx & (GB - 1);
-      k = idx >> 6;
+      r = idx % GB;
+      k = idx / GB;
     }
     const float v = f(r, k);
     const uint16_t h = bf16_bits(v);
@@ -178,10 +186,12 @@ struct GemmAcc {
 // One 32-deep step.  Wave (wm, wn) of the 2 x 2 grid owns rows 32*wm.. and columns 32*wn...
 template <bool SPLIT> DEVI void mma_step(GemmAcc &acc, const GemmLds &s, int wm, int wn, int lane) {
   const int i = lane & 15, g = lane >> 4;
+#pragma unroll
+  for (int ks = 0; ks < GK / 32; ++ks) {
   bf16x8_t a[2], b[2], al[2], bl[2];
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
-    const int oa = tile_off(wm * 32 + t * 16 + i, g * 8), ob = tile_off(wn * 32 + t * 16 + i, g * 8);
+    const int oa = tile_off(wm * 32 + t * 16 + i, ks * 32 + g * 8), ob = tile_off(wn * 32 + t * 16 + i, ks * 32 + g * 8);
     a[t] = *reinterpret_cast<const bf16x8_t *>(&s.ah[oa]);
     b[t] = *reinterpret_cast<const bf16x8_t *>(&s.bh[ob]);
     if (SPLIT) {
@@ -199,6 +209,7 @@ template <bool SPLIT> DEVI void mma_step(GemmAcc &acc, const GemmLds &s, int wm,
         acc.v[tm][tn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al[tm], b[tn], acc.v[tm][tn], 0, 0, 0);
       }
     }
+  }
 }
 
 // D[m][n] += sum_{k in [k_begin, k_end)} fa(m, k) * fb(n, k) for the block's 64 x 64 tile.
