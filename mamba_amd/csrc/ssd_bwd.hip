@@ -278,7 +278,7 @@ __global__ __launch_bounds__(256) void state_passing_bwd_kernel(const SsdParams 
 // dx = dt_s acc + D g;  ddt_out[s] += <x_s, acc_s>;  chunk-state terms of ddA_cumsum.
 template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_kernel(const SsdParams p) {
   __shared__ GemmLds lds;
-  __shared__ float a_s[256], dt_s[256], wrow[GB], r1[GB], r2[GB];
+  __shared__ float a_s[256], dt_s[256], kdec[256], rdec[GB], wrow[GB];
   const int tid = threadIdx.x;
   const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads, G = p.ngroups;
   const int ntp = cdiv(P, GB);
@@ -290,12 +290,18 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
   const float *dt = chunk_row(p.dt_out, p, b, h, c);
   const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
   const float a_last = dA[Q - 1];
+  // Below the diagonal block exp(a_l - a_s) = exp(a_l - a_ref) exp(a_ref - a_s) with a_ref taken
+  // at the tile's last row: both factors are <= 1, so the rank-1 form cannot overflow.
+  const float a_ref = dA[min((st + 1) * GB, qlim) - 1];
   for (int s = tid; s < Q; s += 256) {
-    a_s[s] = dA[s];
+    const float a = dA[s];
+    a_s[s] = a;
     dt_s[s] = dt[s];
+    kdec[s] = fast_exp(fminf(a - a_ref, 0.f));
   }
   if (tid < GB) {
     const int s = st * GB + tid;
+    rdec[tid] = s < qlim ? fast_exp(fminf(a_ref - dA[s], 0.f)) : 0.f;
     float v = 0.f;
     if (s < qlim) {
       bool ok = true;
@@ -311,24 +317,19 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
   const int64_t gb = b * gv.bs + h * gv.hs, xb = b * p.x_bs + h * p.x_hs, Bb = b * p.B_bs + g * p.B_gs;
   const float *dS = p.dstates + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
   const float *CB = p.CB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
-  auto fx = [&](int m, int n) {
-    const int s = st * GB + m, pp = pt * GB + n;
-    return (s < qlim && pp < P) ? ldg<T>(p.x, xb + (int64_t)(t0 + s) * p.x_ls + pp) : 0.f;
-  };
-  GemmAcc acc;
-  acc.zero();
+  GemmAcc acc1, acc2;  // carried-state part, in-chunk part
+  acc1.zero();
+  acc2.zero();
   {
     // A = B rows (s, k = n), B = dS rows (p, k = n): both k-contiguous
     const T *Ba = static_cast<const T *>(p.B) + Bb + (int64_t)(t0 + st * GB) * p.B_ls;
     const float *dSa = dS + (int64_t)pt * GB * N;
     const bool va = rows_aligned16(Ba, p.B_ls), vb = rows_aligned16(dSa, N);
     block_gemm_staged<SPLIT>(
-        acc, lds, 0, N,
+        acc1, lds, 0, N,
         [&](int k0) { stage_kc<SPLIT, T>(lds.ah, lds.al, Ba, p.B_ls, qlim - st * GB, k0, N, nullptr, nullptr, va, tid); },
         [&](int k0) { stage_kc<SPLIT, float>(lds.bh, lds.bl, dSa, N, P - pt * GB, k0, N, nullptr, nullptr, vb, tid); },
         tid);
-    acc_foreach(acc, tid, [&](int m, int n, float v) { return v * wrow[m]; });
-    row_dot(acc, r1, tid, fx);  // state-path part of <x_s, acc_s>
   }
   {
     auto fa = [&](int r, int k) {  // (s, l)
@@ -338,36 +339,75 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
     };
     const T *ga = static_cast<const T *>(gv.ptr) + gb + (int64_t)t0 * gv.ls + pt * GB;
     const bool vb = rows_aligned16(ga, gv.ls);
+    const float *CBa = CB + st * GB;  // A rows s are contiguous in the source, k = l strides by Q
+    const bool va = rows_aligned16(CBa, Q);
     block_gemm_staged<SPLIT>(
-        acc, lds, st * GB, qlim,
-        [&](int k0) { stage_tile<SPLIT, false>(lds.ah, lds.al, [&](int r, int k) { return fa(r, k0 + k); }, tid); },
+        acc2, lds, st * GB, qlim,
+        [&](int k0) {
+          if (k0 < (st + 1) * GB)  // diagonal block: causal mask and the exact decay
+            stage_tile<SPLIT, false>(lds.ah, lds.al, [&](int r, int k) { return fa(r, k0 + k); }, tid);
+          else if (tid >= 128)
+            stage_rc<SPLIT, float>(lds.ah, lds.al, CBa, Q, qlim - st * GB, k0, qlim, kdec, rdec, va, tid - 128);
+        },
         [&](int k0) {
           if (tid < 128) stage_rc<SPLIT, T>(lds.bh, lds.bl, ga, gv.ls, P - pt * GB, k0, qlim, nullptr, nullptr, vb, tid);
         },
         tid);
-    row_dot(acc, r2, tid, fx);  // full <x_s, acc_s>
   }
-  if (tid < GB) {
-    const int s = st * GB + tid;
-    if (s < qlim) {
-      unsafeAtomicAdd(chunk_row(p.ddt_out, p, b, h, c) + s, r2[tid]);
-      float *dda = chunk_row(p.ddA_cumsum, p, b, h, c);
-      unsafeAtomicAdd(dda + s, -dt_s[s] * r1[tid]);
-      unsafeAtomicAdd(dda + Q - 1, dt_s[s] * r1[tid]);
-    }
+  // Epilogue with rows in threads: thread t owns position s = tile row t / 4 and 16 consecutive p.
+  float v1[16], v2[16];
+  acc_to_rows(acc1, lds, tid, v1);
+  acc_to_rows(acc2, lds, tid, v2);
+  {
+    const float w = wrow[tid >> 2];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) v1[e] *= w;
   }
+  const int s = st * GB + (tid >> 2), p0 = pt * GB + (tid & 3) * 16;
+  const bool row_ok = s < qlim;
+  const T *xr = static_cast<const T *>(p.x) + xb + (int64_t)(t0 + s) * p.x_ls + p0;
+  const T *gr = static_cast<const T *>(gv.ptr) + gb + (int64_t)(t0 + s) * gv.ls + p0;
+  T *dxr = static_cast<T *>(p.dx) + (((int64_t)b * L + t0 + s) * H + h) * P + p0;
+  const bool vec = P % 8 == 0 && rows_aligned16(static_cast<const T *>(p.x) + xb, p.x_ls) &&
+                   rows_aligned16(static_cast<const T *>(gv.ptr) + gb, gv.ls) &&
+                   (reinterpret_cast<uintptr_t>(p.dx) & 15) == 0;
   const float *Dp = static_cast<const float *>(p.D);
-  acc_foreach(acc, tid, [&](int m, int n, float v) {
-    const int s = st * GB + m, pp = pt * GB + n;
-    if (s >= qlim || pp >= P) return v;
-    float o = v * dt_s[s];
-    if (Dp) {
-      const float d = p.D_has_hdim ? Dp[h * P + pp] : Dp[h];
-      o = __builtin_fmaf(d, ldg<T>(gv.ptr, gb + (int64_t)(t0 + s) * gv.ls + pp), o);
+  float q1 = 0.f, q2 = 0.f;
+  const float dts = dt_s[min(s, Q - 1)];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int nv = row_ok ? max(0, min(8, P - p0 - 8 * j)) : 0;
+    float xv[8], gvv[8], o[8];
+    if (vec) {
+      ld8_guard<T, true>(xr + 8 * j, nv, 0.f, xv);
+      ld8_guard<T, true>(gr + 8 * j, Dp ? nv : 0, 0.f, gvv);
+    } else {
+      ld8_guard<T, false>(xr + 8 * j, nv, 0.f, xv);
+      ld8_guard<T, false>(gr + 8 * j, Dp ? nv : 0, 0.f, gvv);
     }
-    stg<T>(p.dx, (((int64_t)b * L + t0 + s) * H + h) * P + pp, o);
-    return v;
-  });
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float a1 = v1[8 * j + e], a = a1 + v2[8 * j + e];
+      q1 = __builtin_fmaf(xv[e], a1, q1);
+      q2 = __builtin_fmaf(xv[e], a, q2);
+      float d = 0.f;
+      if (Dp) d = p.D_has_hdim ? Dp[h * P + min(p0 + 8 * j + e, P - 1)] : Dp[h];
+      o[e] = __builtin_fmaf(d, gvv[e], a * dts);
+    }
+    if (vec) st8_guard<T, true>(dxr + 8 * j, nv, o);
+    else st8_guard<T, false>(dxr + 8 * j, nv, o);
+  }
+  // <x_s, acc_s> over the row's four threads
+  q1 += __shfl_xor(q1, 1, 64);
+  q1 += __shfl_xor(q1, 2, 64);
+  q2 += __shfl_xor(q2, 1, 64);
+  q2 += __shfl_xor(q2, 2, 64);
+  if ((tid & 3) == 0 && row_ok) {
+    unsafeAtomicAdd(chunk_row(p.ddt_out, p, b, h, c) + s, q2);
+    float *dda = chunk_row(p.ddA_cumsum, p, b, h, c);
+    unsafeAtomicAdd(dda + s, -dts * q1);      // chunk-state terms: -dt_s <x_s, acc1_s> at s ...
+    unsafeAtomicAdd(dda + Q - 1, dts * q1);   // ... and + at the chunk end
+  }
 }
 
 // ---------------------------------------------- state-path parts of dB, dC
@@ -378,8 +418,10 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
 // The carried-state share of ddA_cumsum, sum_n dC_h[l, n] C[l, n], is taken per head on the way.
 template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dBC_state_kernel(const SsdParams p) {
   __shared__ GemmLds lds;
-  __shared__ float wB[GB], wC[GB], rsum[GB];
+  __shared__ float wB[2][GB], wC[2][GB];  // per-head row factors, double-buffered over the head loop
   const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+  const int i = lane & 15, gq = lane >> 4;
   const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads, G = p.ngroups;
   const int ntn = cdiv(N, GB);
   const int st = blockIdx.x / ntn, nt = blockIdx.x % ntn;
@@ -389,14 +431,27 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dBC
   const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
   const View4 gv = g_view(p);
   const int64_t Cb = b * p.C_bs + g * p.C_gs;
+  // C at this lane's 16 accumulator positions (shared by the heads of the group)
+  float cr[2][2][4];
+#pragma unroll
+  for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+    for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int l = st * GB + wm * 32 + tm * 16 + gq * 4 + r, nn = nt * GB + wn * 32 + tn * 16 + i;
+        cr[tm][tn][r] = (l < qlim && nn < N) ? ldg<T>(p.C, Cb + (int64_t)(t0 + l) * p.C_ls + nn) : 0.f;
+      }
   GemmAcc accB, accC;
   accB.zero();
   accC.zero();
-  for (int hh = hs; hh < hpg; hh += nsplit) {
+  int par = 0;
+  for (int hh = hs; hh < hpg; hh += nsplit, par ^= 1) {
     const int h = g * hpg + hh;
     const float *dA = chunk_row(p.dA_cumsum, p, b, h, c);
     const float *dt = chunk_row(p.dt_out, p, b, h, c);
-    __syncthreads();  // previous head's wB / wC / rsum readers are done
+    // published by the first barrier inside the GEMM; the buffer written here was last read two
+    // iterations ago
     if (tid < GB) {
       const int s = st * GB + tid;
       float vb = 0.f, vc = 0.f;
@@ -410,8 +465,8 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dBC
         if (okb) vb = fast_exp(fminf(dA[Q - 1] - dA[s], 0.f)) * dt[s];
         if (okc) vc = fast_exp(dA[s]);
       }
-      wB[tid] = vb;
-      wC[tid] = vc;
+      wB[par][tid] = vb;
+      wC[par][tid] = vc;
     }
     const int64_t gb = b * gv.bs + h * gv.hs, xb = b * p.x_bs + h * p.x_hs;
     const float *dS = p.dstates + (((int64_t)b * p.nchunks + c) * H + h) * P * N + nt * GB;
@@ -421,7 +476,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dBC
     auto run = [&](GemmAcc &acc, const T *a_base, int64_t a_ls, const float *w, const float *S) {
       const T *aa = a_base + (int64_t)(t0 + st * GB) * a_ls;
       const bool va = rows_aligned16(aa, a_ls);
-      block_gemm_staged<SPLIT>(  // the first barrier inside publishes wB / wC
+      block_gemm_staged<SPLIT>(
           acc, lds, 0, P,
           [&](int k0) { stage_kc<SPLIT, T>(lds.ah, lds.al, aa, a_ls, qlim - st * GB, k0, P, nullptr, w, va, tid); },
           [&](int k0) {
@@ -429,20 +484,28 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dBC
           },
           tid);
     };
-    run(accB, static_cast<const T *>(p.x) + xb, p.x_ls, wB, dS);
+    run(accB, static_cast<const T *>(p.x) + xb, p.x_ls, wB[par], dS);
     GemmAcc accH;
     accH.zero();
-    run(accH, static_cast<const T *>(gv.ptr) + gb, gv.ls, wC, Hc);
-    row_dot(accH, rsum, tid, [&](int m, int n) {
-      const int l = st * GB + m, nn = nt * GB + n;
-      return (l < qlim && nn < N) ? ldg<T>(p.C, Cb + (int64_t)(t0 + l) * p.C_ls + nn) : 0.f;
-    });
-    if (tid < GB && st * GB + tid < qlim)
-      unsafeAtomicAdd(chunk_row(p.ddA_cumsum, p, b, h, c) + st * GB + tid, rsum[tid]);
+    run(accH, static_cast<const T *>(gv.ptr) + gb, gv.ls, wC[par], Hc);
+    // carried-state share of ddA_cumsum: sum_n dC_h[l, n] C[l, n]
+    float *dda = chunk_row(p.ddA_cumsum, p, b, h, c);
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) accC.v[i][j] += accH.v[i][j];
+      for (int r = 0; r < 4; ++r) {
+        float rs = accH.v[tm][0][r] * cr[tm][0][r] + accH.v[tm][1][r] * cr[tm][1][r];
+        rs += dpp_f<DPP_ROW_SHR + 1>(0.f, rs);
+        rs += dpp_f<DPP_ROW_SHR + 2>(0.f, rs);
+        rs += dpp_f<DPP_ROW_SHR + 4>(0.f, rs);
+        rs += dpp_f<DPP_ROW_SHR + 8>(0.f, rs);
+        const int l = st * GB + wm * 32 + tm * 16 + gq * 4 + r;
+        if (i == 15 && l < qlim && rs != 0.f) unsafeAtomicAdd(dda + l, rs);
+      }
+#pragma unroll
+    for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) accC.v[ii][j] += accH.v[ii][j];
   }
   acc_foreach(accB, tid, [&](int m, int n, float v) {
     const int s = st * GB + m, nn = nt * GB + n;
@@ -463,8 +526,10 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dBC
 // the in-chunk share of ddA_cumsum: + row sums at l, - column sums at s.
 template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dcb_kernel(const SsdParams p) {
   __shared__ GemmLds lds;
-  __shared__ float rows[GB], cols[GB];
+  __shared__ float hA_l[2][GB], hA_s[2][GB], hdt[2][GB];  // per-head rows, double-buffered over the head loop
   const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+  const int i = lane & 15, gq = lane >> 4;
   const int Q = p.chunk_size, L = p.seqlen, P = p.headdim, H = p.nheads, G = p.ngroups;
   int lt = 0, rem = blockIdx.x;
   while (rem > lt) { rem -= lt + 1; ++lt; }
@@ -476,12 +541,33 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dcb
   const View4 gv = g_view(p);
   float *dCB = p.dCB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
   const float *CB = p.CB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
+  // This lane's 16 accumulator positions: CB there (the same for every head) and the causal /
+  // same-sequence mask, kept as zeros in cbr and a bit per position.
+  float cbr[2][2][4];
+  uint32_t live = 0;
+#pragma unroll
+  for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+    for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int l = lt * GB + wm * 32 + tm * 16 + gq * 4 + r, s = st * GB + wn * 32 + tn * 16 + i;
+        const bool ok = l < qlim && s <= l && (!seq || seq[l] == seq[s]);
+        cbr[tm][tn][r] = ok ? CB[(int64_t)l * Q + s] : 0.f;
+        live |= (uint32_t)ok << ((tm * 2 + tn) * 4 + r);
+      }
   GemmAcc sum;
   sum.zero();
-  for (int hh = hs; hh < hpg; hh += nsplit) {
+  int par = 0;
+  for (int hh = hs; hh < hpg; hh += nsplit, par ^= 1) {
     const int h = g * hpg + hh;
     const float *dA = chunk_row(p.dA_cumsum, p, b, h, c);
     const float *dt = chunk_row(p.dt_out, p, b, h, c);
+    // published by the barriers inside the GEMM; the buffer written here was last read two
+    // iterations ago
+    if (tid < GB) hA_l[par][tid] = lt * GB + tid < Q ? dA[lt * GB + tid] : 0.f;
+    else if (tid < 2 * GB) hA_s[par][tid - GB] = st * GB + tid - GB < Q ? dA[st * GB + tid - GB] : 0.f;
+    else if (tid < 3 * GB) hdt[par][tid - 2 * GB] = st * GB + tid - 2 * GB < Q ? dt[st * GB + tid - 2 * GB] : 0.f;
     const int64_t gb = b * gv.bs + h * gv.hs, xb = b * p.x_bs + h * p.x_hs;
     GemmAcc acc;
     acc.zero();
@@ -494,32 +580,42 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dcb
         [&](int k0) { stage_kc<SPLIT, T>(lds.ah, lds.al, ga, gv.ls, qlim - lt * GB, k0, P, nullptr, nullptr, va, tid); },
         [&](int k0) { stage_kc<SPLIT, T>(lds.bh, lds.bl, xa, p.x_ls, qlim - st * GB, k0, P, nullptr, nullptr, vb, tid); },
         tid);
-    // acc <- this head's dCB term; sum += it; acc <- w[l, s] = term * CB[l, s]
-    {
-      const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
-      const int i = lane & 15, gq = lane >> 4;
+    // d = this head's dCB term (added to sum); w = d * CB, whose row / column sums go to ddA
+    float *dda = chunk_row(p.ddA_cumsum, p, b, h, c);
+    float a_s[2], dt_s[2], csum[2] = {0.f, 0.f};
 #pragma unroll
-      for (int tm = 0; tm < 2; ++tm)
-#pragma unroll
-        for (int tn = 0; tn < 2; ++tn)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int l = lt * GB + wm * 32 + tm * 16 + gq * 4 + r, s = st * GB + wn * 32 + tn * 16 + i;
-            float d = 0.f, w = 0.f;
-            if (l < qlim && s <= l && (!seq || seq[l] == seq[s])) {
-              d = acc.v[tm][tn][r] * dt[s] * fast_exp(fminf(dA[l] - dA[s], 0.f));
-              w = d * CB[(int64_t)l * Q + s];
-            }
-            sum.v[tm][tn][r] += d;
-            acc.v[tm][tn][r] = w;
-          }
+    for (int tn = 0; tn < 2; ++tn) {
+      a_s[tn] = hA_s[par][wn * 32 + tn * 16 + i];
+      dt_s[tn] = hdt[par][wn * 32 + tn * 16 + i];
     }
-    row_col_sums(acc, rows, cols, tid);
-    if (tid < GB) {
-      float *dda = chunk_row(p.ddA_cumsum, p, b, h, c);
-      const int l = lt * GB + tid, s = st * GB + tid;
-      if (l < qlim && rows[tid] != 0.f) unsafeAtomicAdd(dda + l, rows[tid]);
-      if (s < qlim && cols[tid] != 0.f) unsafeAtomicAdd(dda + s, -cols[tid]);
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = wm * 32 + tm * 16 + gq * 4 + r;
+        const float a_l = hA_l[par][m];
+        float rsum = 0.f;
+#pragma unroll
+        for (int tn = 0; tn < 2; ++tn) {
+          float d = acc.v[tm][tn][r] * dt_s[tn] * fast_exp(fminf(a_l - a_s[tn], 0.f));
+          d = (live >> ((tm * 2 + tn) * 4 + r)) & 1 ? d : 0.f;
+          sum.v[tm][tn][r] += d;
+          const float w = d * cbr[tm][tn][r];
+          rsum += w;
+          csum[tn] += w;
+        }
+        rsum += dpp_f<DPP_ROW_SHR + 1>(0.f, rsum);
+        rsum += dpp_f<DPP_ROW_SHR + 2>(0.f, rsum);
+        rsum += dpp_f<DPP_ROW_SHR + 4>(0.f, rsum);
+        rsum += dpp_f<DPP_ROW_SHR + 8>(0.f, rsum);
+        if (i == 15 && rsum != 0.f) unsafeAtomicAdd(dda + lt * GB + m, rsum);
+      }
+#pragma unroll
+    for (int tn = 0; tn < 2; ++tn) {
+      float cs = csum[tn];
+      cs += __shfl_xor(cs, 16, 64);
+      cs += __shfl_xor(cs, 32, 64);
+      if (gq == 0 && cs != 0.f) unsafeAtomicAdd(dda + st * GB + wn * 32 + tn * 16 + i, -cs);
     }
   }
   acc_foreach(sum, tid, [&](int m, int n, float v) {

@@ -253,4 +253,30 @@ template <typename F> DEVI void acc_foreach(GemmAcc &acc, int tid, F f) {
         acc.v[tm][tn][r] = f(wm * 32 + tm * 16 + g * 4 + r, wn * 32 + tn * 16 + i, acc.v[tm][tn][r]);
 }
 
+// Re-lays the block tile from the MFMA accumulator layout to rows: thread t receives row t / 4,
+// columns 16 * (t % 4) .. + 15.  Goes through LDS in the storage of the GEMM tiles (free once the
+// leading barrier is passed).  All 256 threads call.
+DEVI void acc_to_rows(const GemmAcc &acc, GemmLds &s, int tid, float (&o)[16]) {
+  constexpr int PLD = GB + 4;
+  static_assert(sizeof(GemmLds) >= GB * PLD * sizeof(float), "row patch must fit in the GEMM tiles");
+  float *patch = reinterpret_cast<float *>(&s);
+  const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+  const int i = lane & 15, g = lane >> 4;
+  __syncthreads();
+#pragma unroll
+  for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+    for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        patch[(wm * 32 + tm * 16 + g * 4 + r) * PLD + wn * 32 + tn * 16 + i] = acc.v[tm][tn][r];
+  __syncthreads();
+  const float *src = patch + (tid >> 2) * PLD + (tid & 3) * 16;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const f32x4 v = *reinterpret_cast<const f32x4 *>(src + 4 * q);
+    o[4 * q] = v.x; o[4 * q + 1] = v.y; o[4 * q + 2] = v.z; o[4 * q + 3] = v.w;
+  }
+}
+
 DEVI int cdiv(int a, int b) { return (a + b - 1) / b; }
