@@ -6,6 +6,12 @@ Mamba-1 benchmark configuration (batch 8, d_inner 5120, seqlen 4096, d_state 16,
 activations, fp32 A/D/delta_bias/state), inputs resident in HBM.  Prints ONE JSON line.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+
+Side workloads (each prints its own JSON line; they are not the headline metric):
+  python bench.py --workload ssd      Mamba-2 mamba_chunk_scan_combined fwd+bwd (batch 4, 80 heads x 64,
+                                      seqlen 4096, d_state 128, chunk 256, bf16)
+  python bench.py --workload decode   selective_state_update (batch 256, 80 heads x 64, d_state 128)
+  python bench.py --copy-calibration  the library's plain copy kernel over 1 GiB
 """
 import argparse
 import json
@@ -18,6 +24,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch read off the FETCH_SIZE / WRITE_SIZE counters (scaled by the copy yardstick),
+# from the *_hbm_counters.txt summaries under profiles/; they describe the kernels as committed there.
+TRAFFIC = {"scan_bwd_kernel": 1399.3e6 + 1680.7e6, "scan_fwd_kernel": 1032.6e6 + 357.4e6,
+           "chunk_scan_fwd_fused_kernel": 557.8e6 + 335.5e6, "state_update_kernel": 683.1e6 + 673.7e6}
 
 
 def make_inputs(batch, dim, seqlen, dstate, dtype, device, seed=0):
@@ -74,12 +84,130 @@ def copy_calibration(dev):
                       "GB/s": 2 * nbytes / ms / 1e6}))
 
 
+def event_ms(fn, n, pre=None):
+    """Average HIP-event time of fn() on torch's current stream (where the library launches);
+    pre() runs outside the event pair."""
+    import torch
+    if pre:
+        pre()
+    fn()
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+    for a, b in ev:
+        if pre:
+            pre()
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    return sum(a.elapsed_time(b) for a, b in ev) / n
+
+
+def bench_ssd(dev, steps, warmup):
+    """Mamba-2 SSD: mamba_chunk_scan_combined forward + backward; the roofline entry is the fused
+    C B^T + chunk_scan forward kernel, which is HBM-bound (65 flop per byte against 312 at the ridge)."""
+    import torch
+    from mamba_amd import _lib
+    from mamba_amd.ops.triton import ssd_combined as sc
+    batch, L, H, P, N, G, Q = 4, 4096, 80, 64, 128, 1, 256
+    bf = torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(0)
+    rn = lambda *s: torch.randn(*s, device=dev, generator=g)
+    x, z = (rn(batch, L, H, P).to(bf).requires_grad_() for _ in range(2))
+    B, C = (rn(batch, L, G, N).to(bf).requires_grad_() for _ in range(2))
+    dt = rn(batch, L, H).to(bf).requires_grad_()
+    A = (-(1 + 15 * torch.rand(H, device=dev, generator=g))).requires_grad_()
+    D = torch.rand(H, device=dev, generator=g).requires_grad_()
+    dtb = (torch.rand(H, device=dev, generator=g) - 4).requires_grad_()
+    dout = rn(batch, L, H, P).to(bf)
+    leaves = (x, z, B, C, dt, A, D, dtb)
+
+    def fwd():
+        return sc.mamba_chunk_scan_combined(x, dt, A, B, C, Q, D=D, z=z, dt_bias=dtb, dt_softplus=True)
+
+    def step():
+        for v in leaves:
+            v.grad = None
+        fwd().backward(dout)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / steps
+    with torch.no_grad():
+        fwd_ms = event_ms(fwd, max(5, min(steps, 50)))
+        # the fused scan kernel alone, on the buffers of one forward pass
+        lib = _lib.load()
+        a = sc._prepare(x, dt, A, B, C, Q, D, z, dtb, None, None)
+        ws = sc._workspace(a[0], a[3], Q)
+        out, out_x = torch.empty_like(a[0]), torch.empty_like(a[0])
+        p = _lib.SsdParams()
+        sc._fill_fwd(p, a[0], a[1], a[2], a[3], a[4], Q, a[5], a[6], a[7], None, None, True, (0.0, float("inf")), ws)
+        p.out, p.out_x = out.data_ptr(), out_x.data_ptr()
+        p.out_bs, p.out_ls, p.out_hs = out.stride(0), out.stride(1), out.stride(2)
+        stream = _lib.current_stream(dev)
+        _lib.check(lib.ssd_combined_fwd(p, stream), "ssd_combined_fwd")   # fills dA_cumsum and the chunk states
+        scan_ms = event_ms(lambda: _lib.check(lib.ssd_chunk_scan_fwd_fused(p, stream), "ssd_chunk_scan_fwd_fused"),
+                           max(5, min(steps, 50)))
+    nc = L // Q
+    flops = batch * nc * (H * (Q * Q * P + 2 * Q * N * P) + G * Q * Q * N)   # causal halves counted once
+    nbytes = 2 * (4 * batch * L * H * P + 2 * batch * L * G * N) + 4 * batch * nc * H * P * N  # x z out out_x B C states
+    print(json.dumps({
+        "metric": "SSD mamba_chunk_scan_combined fwd+bwd tokens/s at 1 GPU", "value": batch * L / sec,
+        "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": sec * 1e3,
+        "fwd_ms": fwd_ms, "higher_is_better": True, "dtype": "bf16 in/out, fp32 accumulation", "data": "synthetic",
+        "config": {"workload": f"Mamba-2 SSD fwd+bwd: batch {batch}, seqlen {L}, {H} heads x {P}, d_state {N}, "
+                               f"{G} group, chunk {Q}, bf16 (BASELINE configs[2])"},
+        "roofline": {"bound": "hbm", "kernel": "chunk_scan_fwd_fused_kernel", "achieved": nbytes / scan_ms / 1e6,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / scan_ms / 1e6 / HBM_PEAK_GBS,
+                     "traffic": TRAFFIC["chunk_scan_fwd_fused_kernel"], "kernel_ms": scan_ms, "algorithmic_bytes": nbytes,
+                     "algorithmic_flops": flops, "mfma_tflops": flops / scan_ms / 1e9,
+                     "mfma_frac_of_bf16_peak": flops / scan_ms / 1e9 / 2500.0}}))
+
+
+def bench_decode(dev, steps, warmup):
+    """Decode: one selective_state_update call per step; the state (fp32) is read and written once."""
+    import torch
+    from mamba_amd.ops.triton.selective_state_update import selective_state_update
+    batch, H, P, N, G = 256, 80, 64, 128, 1
+    bf = torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(0)
+    rn = lambda *s: torch.randn(*s, device=dev, generator=g)
+    state = 0.1 * rn(batch, H, P, N)
+    x, z = rn(batch, H, P).to(bf), rn(batch, H, P).to(bf)
+    dt = rn(batch, H).to(bf)[:, :, None].expand(batch, H, P)
+    A = (-(1 + 15 * torch.rand(H, device=dev, generator=g)))[:, None, None].expand(H, P, N)
+    D = torch.rand(H, device=dev, generator=g)[:, None].expand(H, P)
+    dtb = (torch.rand(H, device=dev, generator=g) - 4)[:, None].expand(H, P)
+    B, C = rn(batch, G, N).to(bf), rn(batch, G, N).to(bf)
+    fn = lambda: selective_state_update(state, x, dt, A, B, C, D=D, z=z, dt_bias=dtb, dt_softplus=True)
+    for _ in range(warmup):
+        fn()
+    ms = event_ms(fn, max(steps, 5))
+    nbytes = 2 * state.numel() * 4 + 2 * (3 * x.numel() + 2 * B.numel()) + 2 * batch * H
+    print(json.dumps({
+        "metric": "decode selective_state_update tokens/s at 1 GPU", "value": batch / ms * 1e3, "unit": "tokens/s",
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": ms, "higher_is_better": True,
+        "dtype": "fp32 state, bf16 x/z/B/C/dt", "data": "synthetic",
+        "config": {"workload": f"selective_state_update: batch {batch}, {H} heads x {P}, d_state {N}, {G} group, "
+                               "tied A/dt/D per head (BASELINE configs[3])"},
+        "roofline": {"bound": "hbm", "kernel": "state_update_kernel", "achieved": nbytes / ms / 1e6,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / ms / 1e6 / HBM_PEAK_GBS,
+                     "traffic": TRAFFIC["state_update_kernel"],
+                     "kernel_ms": ms, "algorithmic_bytes": nbytes}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--workload", choices=("mamba1", "ssd", "decode"), default="mamba1")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run the library's plain copy kernel over 1 GiB (yardstick for HBM counters)")
     args = ap.parse_args()
@@ -98,6 +226,12 @@ def main():
     torch.cuda.set_device(dev)
     if args.copy_calibration:
         copy_calibration(dev)
+        return
+    if args.workload == "ssd":
+        bench_ssd(dev, args.steps, args.warmup)
+        return
+    if args.workload == "decode":
+        bench_decode(dev, args.steps, args.warmup)
         return
     batch, dim, seqlen, dstate = 8, 5120, 4096, 16
     dtype = torch.bfloat16
@@ -134,25 +268,9 @@ def main():
         fwd = lambda: selective_scan_fwd(d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["z"],
                                          d["delta_bias"], True)
 
-        def kernel_ms(fn, n, pre=None):
-            # the library launches on torch's current stream, which is where these events are recorded
-            if pre:
-                pre()
-            fn()
-            torch.cuda.synchronize()
-            ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
-            for a, b in ev:
-                if pre:
-                    pre()
-                a.record()
-                fn()
-                b.record()
-            torch.cuda.synchronize()
-            return sum(a.elapsed_time(b) for a, b in ev) / n
-
         n = max(5, min(args.steps, 50))
-        bwd_ms = kernel_ms(bwd, n, bwd_pre)
-        fwd_ms = kernel_ms(fwd, n)
+        bwd_ms = event_ms(bwd, n, bwd_pre)
+        fwd_ms = event_ms(fwd, n)
     es = 2  # bf16
     E = batch * dim * seqlen * es
     BC = batch * dstate * seqlen * es
@@ -160,7 +278,7 @@ def main():
     fwd_bytes = 4 * E + 2 * BC   # reads u, delta, z, B, C; writes out
     achieved = bwd_bytes / (bwd_ms * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": "scan_bwd_kernel", "achieved": achieved, "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": TRAFFIC["scan_bwd_kernel"],
                 "kernel_ms": bwd_ms, "algorithmic_bytes": bwd_bytes,
                 "fwd_kernel_ms": fwd_ms, "fwd_achieved": fwd_bytes / (fwd_ms * 1e-3) / 1e9,
                 "fwd_bwd_frac": (fwd_bytes + bwd_bytes) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS}
