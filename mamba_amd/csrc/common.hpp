@@ -284,6 +284,17 @@ DEVI void wave_scan_rev_finish(float &a, float &b, int lane) {
   a = a * an;
 }
 
+// Sum over the 64 lanes by DPP adds; only lane 63 holds the full sum on return.
+DEVI float wave_sum_to_last(float x) {
+  x += dpp_f<DPP_ROW_SHR + 1>(0.f, x);
+  x += dpp_f<DPP_ROW_SHR + 2>(0.f, x);
+  x += dpp_f<DPP_ROW_SHR + 4>(0.f, x);
+  x += dpp_f<DPP_ROW_SHR + 8>(0.f, x);
+  x += dpp_f<DPP_ROW_BCAST15, 0xa>(0.f, x);
+  x += dpp_f<DPP_ROW_BCAST31, 0xc>(0.f, x);
+  return x;
+}
+
 DEVI float wave_sum(float x) {
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) x += __shfl_xor(x, off, 64);

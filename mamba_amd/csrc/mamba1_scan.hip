@@ -270,7 +270,8 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
         if (NBLK > 1 || r == 0) {
           __syncthreads();
           stage_bc<T, VEC, NW * 64>(Bs, Cs, Bg, p.B_ns, Cg, p.C_ns, nb * NB16, N, t0, L, tid);
-          for (int i = tid; i < 2 * BC_FLOATS; i += NW * 64) dBs[i] = 0.f;  // dBs and dCs are adjacent
+          for (int i = tid * 4; i < 2 * BC_FLOATS; i += NW * 256)  // dBs and dCs are adjacent
+            *reinterpret_cast<f32x4 *>(dBs + i) = f32x4{0.f, 0.f, 0.f, 0.f};
           __syncthreads();
         }
         {
@@ -367,12 +368,8 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
                 }
                 lds_st8(dBs + (n + q) * TILE, lane, sB);
                 lds_st8(dCs + (n + q) * TILE, lane, sC);
-                dAp += dpp_f<DPP_ROW_SHR + 1>(0.f, dAp);
-                dAp += dpp_f<DPP_ROW_SHR + 2>(0.f, dAp);
-                dAp += dpp_f<DPP_ROW_SHR + 4>(0.f, dAp);
-                dAp += dpp_f<DPP_ROW_SHR + 8>(0.f, dAp);
-                if ((lane & 15) == 15)
-                  __hip_atomic_fetch_add(dArow + n + q, dAp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                dAp = wave_sum_to_last(dAp);
+                if (lane == 63) dArow[n + q] += dAp;  // the row belongs to this wave alone
               }
             }
             __syncthreads();
@@ -420,9 +417,9 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
           st8_guard<T, VEC>((T *)p.dz + b * p.dz_bs + d * p.dz_ds + tl, nvalid, o);
           if (p.out_z) st8_guard<T, VEC>((T *)p.out_z + b * p.outz_bs + d * p.outz_ds + tl, nvalid, oz);
         }
-        dbs = wave_sum(dbs);
-        dDs = wave_sum(dDs);
-        if (lane == 0) {
+        dbs = wave_sum_to_last(dbs);
+        dDs = wave_sum_to_last(dDs);
+        if (lane == 63) {
           dbacc[row] += dbs;
           dDacc[row] += dDs;
         }
