@@ -287,16 +287,17 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
           float *arow = anx + row * NP + nb * NB16;
           float *dArow = dAacc + row * NP + nb * NB16;
           const int nmax = min(NB16, N - nb * NB16);
-          static_assert(NPP % 2 == 0, "states are processed in pairs");
+          constexpr int Q = NPP >= 2 ? 2 : 1;  // states per step; two keep two scan chains in flight
+          static_assert(NPP % Q == 0, "whole steps per phase");
           for (int ph = 0; ph < NPH; ++ph) {
             const int slot = (wave + ph) % NPH;
-            for (int j = 0; j < NPP; j += 2) {
+            for (int j = 0; j < NPP; j += Q) {
               const int n = slot * NPP + j;
               if (!valid || n >= nmax) continue;
-              float A1[2], hc[2], gc[2], an[2];
-              float Bv[2][8], Cv[2][8], a[2][8], ac[2][8], bb[2][8], h[2][8];
+              float A1[Q], hc[Q], gc[Q], an[Q];
+              float Bv[Q][8], Cv[Q][8], a[Q][8], ac[Q][8], bb[Q][8], h[Q][8];
 #pragma unroll
-              for (int q = 0; q < 2; ++q) {
+              for (int q = 0; q < Q; ++q) {
                 A1[q] = A1row[n + q];
                 hc[q] = hrow[n + q];
                 gc[q] = grow[n + q];
@@ -317,12 +318,19 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
                   ac[q][i] = ac[q][i - 1] * a[q][i];
                 }
               }
-              float sa0 = ac[0][KI - 1], sb0 = h[0][KI - 1], sa1 = ac[1][KI - 1], sb1 = h[1][KI - 1];
-              wave_scan_fwd2(sa0, sb0, sa1, sb1);
-              const float hend[2] = {__builtin_fmaf(sa0, hc[0], sb0), __builtin_fmaf(sa1, hc[1], sb1)};
-              float gg[2][8], ar[2][8];
+              float sa[Q], sb[Q], hend[Q];
 #pragma unroll
-              for (int q = 0; q < 2; ++q) {
+              for (int q = 0; q < Q; ++q) {
+                sa[q] = ac[q][KI - 1];
+                sb[q] = h[q][KI - 1];
+              }
+              if constexpr (Q == 2) wave_scan_fwd2(sa[0], sb[0], sa[1], sb[1]);
+              else wave_scan_fwd(sa[0], sb[0]);
+#pragma unroll
+              for (int q = 0; q < Q; ++q) hend[q] = __builtin_fmaf(sa[q], hc[q], sb[q]);
+              float gg[Q][8], ar[Q][8];
+#pragma unroll
+              for (int q = 0; q < Q; ++q) {
                 const float hx = dpp_f<DPP_WAVE_SHR1>(hc[q], hend[q]);
 #pragma unroll
                 for (int i = 0; i < KI; ++i) h[q][i] = __builtin_fmaf(ac[q][i], hx, h[q][i]);  // true states
@@ -340,13 +348,23 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
                   ar[q][i] = ar[q][i + 1] * a[q][i + 1];
                 }
               }
-              float ra0 = ar[0][0], rb0 = gg[0][0], ra1 = ar[1][0], rb1 = gg[1][0];
-              row_scan_rev2(ra0, rb0, ra1, rb1);
-              wave_scan_rev_finish(ra0, rb0, lane);
-              wave_scan_rev_finish(ra1, rb1, lane);
-              const float gfirst[2] = {__builtin_fmaf(ra0, gc[0], rb0), __builtin_fmaf(ra1, gc[1], rb1)};
+              float ra[Q], rb[Q], gfirst[Q];
 #pragma unroll
-              for (int q = 0; q < 2; ++q) {
+              for (int q = 0; q < Q; ++q) {
+                ra[q] = ar[q][0];
+                rb[q] = gg[q][0];
+              }
+              if constexpr (Q == 2) {
+                row_scan_rev2(ra[0], rb[0], ra[1], rb[1]);
+                wave_scan_rev_finish(ra[0], rb[0], lane);
+                wave_scan_rev_finish(ra[1], rb[1], lane);
+              } else {
+                wave_scan_rev(ra[0], rb[0], lane);
+              }
+#pragma unroll
+              for (int q = 0; q < Q; ++q) gfirst[q] = __builtin_fmaf(ra[q], gc[q], rb[q]);
+#pragma unroll
+              for (int q = 0; q < Q; ++q) {
                 const float gx = dpp_f<DPP_WAVE_SHL1>(gc[q], gfirst[q]);  // adjoint at the next lane's first item
                 if (lane == 0) {
                   grow[n + q] = gfirst[q];
