@@ -32,10 +32,14 @@ template <int QT, int NWV> DEVI int l_tile(int w, int k) {
   return k < HALF ? HALF * w + k : QT - 1 - (HALF * w + (k - HALF));
 }
 
-template <int PT, int NK, int QT, int NWV>
-__global__ __launch_bounds__(64 * NWV) void chunk_scan_fwd_fused_kernel(const SsdParams p) {
-  constexpr int P = 16 * PT, N = 32 * NK, Q = 16 * QT, LT = QT / NWV, NSB = Q / 32, NT = 64 * NWV;
+// NWV waves share the l tiles of one (batch, chunk, head); they are spread over SPLIT workgroups
+// of NWV / SPLIT waves each (the pairing of tile i with tile QT-1-i keeps the workgroups balanced
+// as well).  Smaller workgroups let several of them, at different stages, share a CU.
+template <int PT, int NK, int QT, int NWV, int SPLIT>
+__global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(const SsdParams p) {
+  constexpr int P = 16 * PT, N = 32 * NK, Q = 16 * QT, LT = QT / NWV, NSB = Q / 32, NWG = NWV / SPLIT, NT = 64 * NWG;
   static_assert(LT >= 1 && LT * NWV == QT, "l tiles divide evenly over the waves");
+  static_assert(NWG * SPLIT == NWV, "waves divide evenly over the workgroups");
   constexpr int BP = N + 8;  // LDS pitch of a B row / H row (bf16): 16-byte aligned, bank-spread
   constexpr int XP = 40;     // LDS pitch of an X^T row (32 k values + pad)
   constexpr int YP = P + 8;  // fp32 pitch of the epilogue's per-wave transpose patch
@@ -46,7 +50,7 @@ __global__ __launch_bounds__(64 * NWV) void chunk_scan_fwd_fused_kernel(const Ss
   };
   union __align__(16) Shared {
     Stage st;                       // main loop
-    float ypatch[NWV * 16 * YP];    // epilogue (the staging buffers are dead by then)
+    float ypatch[NWG * 16 * YP];    // epilogue (the staging buffers are dead by then)
   };
   __shared__ Shared shm;
   auto &Bs = shm.st.Bs;
@@ -56,10 +60,18 @@ __global__ __launch_bounds__(64 * NWV) void chunk_scan_fwd_fused_kernel(const Ss
   __shared__ int seq_s[Q];
 
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lwave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave inside this workgroup
   const int j = lane & 15, g = lane >> 4;
   const int H = p.nheads, G = p.ngroups, L = p.seqlen;
-  const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  // heads vary fastest over the grid: workgroups in flight together then read and write whole
+  // (position, all heads) rows of x, z and out between them
+  const int h = blockIdx.x, c = blockIdx.y / SPLIT, part = blockIdx.y % SPLIT, b = blockIdx.z;
+  const int wave = part * NWG + lwave;  // wave among the NWV that share the chunk
+  // s blocks this workgroup needs: up to its last l tile
+  int last_tile = 0;
+#pragma unroll
+  for (int k = 0; k < LT; ++k) last_tile = max(last_tile, l_tile<QT, NWV>(part * NWG, k));
+  const int nsb = SPLIT == 1 ? NSB : min(NSB, (last_tile * 16 + 15) / 32 + 1);
   const int grp = h / (H / G);
   const int t0 = c * Q;
   const int qlim = min(Q, L - t0);
@@ -150,7 +162,7 @@ __global__ __launch_bounds__(64 * NWV) void chunk_scan_fwd_fused_kernel(const Ss
   };
 
   load_block(0, bregs[0], xregs[0]);
-  if (NSB > 1) load_block(1, bregs[1], xregs[1]);
+  if (nsb > 1) load_block(1, bregs[1], xregs[1]);
   // carried state, fp32 -> bf16, rows p, k = n
   {
     const float *Hc = p.states + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
@@ -190,11 +202,35 @@ __global__ __launch_bounds__(64 * NWV) void chunk_scan_fwd_fused_kernel(const Ss
     }
   }
 
+  // The epilogue's x (for D) and z rows are fetched a few blocks before the main loop ends, so
+  // that their latency is covered by the remaining blocks.
+  constexpr int EQ = (16 * P / 8 + 63) / 64;  // 16-byte chunks per lane of one 16 x P tile
+  const float *Dp = static_cast<const float *>(p.D);
+  const bf16_t *zg = p.z ? static_cast<const bf16_t *>(p.z) + b * p.z_bs + h * p.z_hs : nullptr;
+  u32x4 xe[LT][EQ], ze[LT][EQ];
+  auto epilogue_prefetch = [&]() {
+#pragma unroll
+    for (int k = 0; k < LT; ++k)
+#pragma unroll
+      for (int q = 0; q < EQ; ++q) {
+        const int id = lane + q * 64, rr = id / (P / 8), c8 = id % (P / 8);
+        const int l = l_tile<QT, NWV>(wave, k) * 16 + rr;
+        xe[k][q] = u32x4{0, 0, 0, 0};
+        ze[k][q] = u32x4{0, 0, 0, 0};
+        if (id < 16 * P / 8 && l < qlim) {
+          if (Dp) xe[k][q] = *reinterpret_cast<const u32x4 *>(xg + (int64_t)(t0 + l) * p.x_ls + c8 * 8);
+          if (zg) ze[k][q] = *reinterpret_cast<const u32x4 *>(zg + (int64_t)(t0 + l) * p.z_ls + c8 * 8);
+        }
+      }
+  };
+
   // ---- inside the chunk
 #pragma unroll
   for (int sb = 0; sb < NSB; ++sb) {
     const int buf = sb & 1;
-    if (sb + 2 < NSB) load_block(sb + 2, bregs[sb & 1], xregs[sb & 1]);
+    if (SPLIT > 1 && sb >= nsb) break;
+    if (sb == max(nsb - 3, 0)) epilogue_prefetch();
+    if (sb + 2 < nsb) load_block(sb + 2, bregs[sb & 1], xregs[sb & 1]);
 #pragma unroll
     for (int k = 0; k < LT; ++k) {
       const int lt = l_tile<QT, NWV>(wave, k);
@@ -241,16 +277,14 @@ __global__ __launch_bounds__(64 * NWV) void chunk_scan_fwd_fused_kernel(const Ss
         acc[k][pt] = mfma_bf16(ld_frag(&Xs[buf][(pt * 16 + j) * XP + ((g ^ ((pt * 2 + (j >> 3)) & 3)) << 3)]), Mf,
                                acc[k][pt]);
     }
-    if (sb + 1 < NSB) store_block(buf ^ 1, bregs[(sb + 1) & 1], xregs[(sb + 1) & 1]);
+    if (sb + 1 < nsb) store_block(buf ^ 1, bregs[(sb + 1) & 1], xregs[(sb + 1) & 1]);
     __syncthreads();
   }
 
   // ---- epilogue: + D x, pre-gate copy, gate.  Each wave transposes its 16-row tiles through a
   // private LDS patch so that x / z loads and out / out_x stores are 16-byte pieces of
   // contiguous rows (the accumulator layout itself would scatter 8-byte pieces over 16 rows).
-  float *Ys = shm.ypatch + wave * 16 * YP;
-  const float *Dp = static_cast<const float *>(p.D);
-  const bf16_t *zg = p.z ? static_cast<const bf16_t *>(p.z) + b * p.z_bs + h * p.z_hs : nullptr;
+  float *Ys = shm.ypatch + lwave * 16 * YP;
   bf16_t *og = static_cast<bf16_t *>(p.out) + b * p.out_bs + h * p.out_hs;
   bf16_t *oxg = p.z ? static_cast<bf16_t *>(p.out_x) + b * p.out_bs + h * p.out_hs : nullptr;
 #pragma unroll
@@ -263,7 +297,7 @@ __global__ __launch_bounds__(64 * NWV) void chunk_scan_fwd_fused_kernel(const Ss
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     // 16 rows x P/8 chunks of 8 columns
 #pragma unroll
-    for (int q = 0; q < (16 * P / 8 + 63) / 64; ++q) {
+    for (int q = 0; q < EQ; ++q) {
       const int id = lane + q * 64, rr = id / (P / 8), c8 = id % (P / 8);
       const int l = ltile * 16 + rr;
       if (id >= 16 * P / 8 || l >= qlim) continue;
@@ -271,16 +305,18 @@ __global__ __launch_bounds__(64 * NWV) void chunk_scan_fwd_fused_kernel(const Ss
       const f32x4 y1 = *reinterpret_cast<const f32x4 *>(&Ys[rr * YP + c8 * 8 + 4]);
       float v[8] = {y0.x, y0.y, y0.z, y0.w, y1.x, y1.y, y1.z, y1.w};
       if (Dp) {
-        float xf[8];
-        ld8<bf16_t>(xg + (int64_t)(t0 + l) * p.x_ls + c8 * 8, xf);
+        const u32x4 xw = xe[k][q];
+        const float xf[8] = {bf16_lo(xw.x), bf16_hi(xw.x), bf16_lo(xw.y), bf16_hi(xw.y),
+                             bf16_lo(xw.z), bf16_hi(xw.z), bf16_lo(xw.w), bf16_hi(xw.w)};
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] = __builtin_fmaf(p.D_has_hdim ? Dp[h * P + c8 * 8 + e] : Dp[h], xf[e], v[e]);
       }
       const int64_t oi = (int64_t)(t0 + l) * p.out_ls + c8 * 8;
       if (zg) {
         st8<bf16_t>(oxg + oi, v);
-        float zf[8];
-        ld8<bf16_t>(zg + (int64_t)(t0 + l) * p.z_ls + c8 * 8, zf);
+        const u32x4 zw = ze[k][q];
+        const float zf[8] = {bf16_lo(zw.x), bf16_hi(zw.x), bf16_lo(zw.y), bf16_hi(zw.y),
+                             bf16_lo(zw.z), bf16_hi(zw.z), bf16_lo(zw.w), bf16_hi(zw.w)};
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] *= zf[e] * sigmoid_f(zf[e]);
       }
@@ -291,14 +327,20 @@ __global__ __launch_bounds__(64 * NWV) void chunk_scan_fwd_fused_kernel(const Ss
   }
 }
 
+#ifndef FUSED_SPLIT
+#define FUSED_SPLIT 1
+#endif
 bool aligned(const void *ptr, int a) { return (reinterpret_cast<uintptr_t>(ptr) % a) == 0; }
 
 template <int PT, int NK> int launch_q(const SsdParams &p, hipStream_t s) {
-  dim3 grid(p.nchunks, p.nheads, p.batch);
+  dim3 grid(p.nheads, p.nchunks, p.batch);
   switch (p.chunk_size) {
-    case 256: hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 16, 8>), grid, dim3(512), 0, s, p); break;
-    case 128: hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 8, 8>), grid, dim3(512), 0, s, p); break;
-    case 64: hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 4, 4>), grid, dim3(256), 0, s, p); break;
+    case 256:
+      grid.y *= FUSED_SPLIT;
+      hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 16, 8, FUSED_SPLIT>), grid, dim3(512 / FUSED_SPLIT), 0, s, p);
+      break;
+    case 128: hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 8, 8, 1>), grid, dim3(512), 0, s, p); break;
+    case 64: hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 4, 4, 1>), grid, dim3(256), 0, s, p); break;
     default: return MAMBA_E_UNSUPPORTED;
   }
   return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
