@@ -337,7 +337,7 @@ template <int PT, int NK> int launch_q(const SsdParams &p, hipStream_t s) {
   switch (p.chunk_size) {
     case 256:
       grid.y *= FUSED_SPLIT;
-      hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 16, 8, FUSED_SPLIT>), grid, dim3(512 / FUSED_SPLIT), 0, s, p);
+      hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 16, 16, FUSED_SPLIT>), grid, dim3(1024 / FUSED_SPLIT), 0, s, p);
       break;
     case 128: hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 8, 8, 1>), grid, dim3(512), 0, s, p); break;
     case 64: hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 4, 4, 1>), grid, dim3(256), 0, s, p); break;
