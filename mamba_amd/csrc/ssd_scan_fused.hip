@@ -70,7 +70,8 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
   // s blocks this workgroup needs: up to its last l tile
   int last_tile = 0;
 #pragma unroll
-  for (int k = 0; k < LT; ++k) last_tile = max(last_tile, l_tile<QT, NWV>(part * NWG, k));
+  for (int k = 0; k < LT; ++k)
+    last_tile = max(last_tile, max(l_tile<QT, NWV>(part * NWG, k), l_tile<QT, NWV>(part * NWG + NWG - 1, k)));
   const int nsb = SPLIT == 1 ? NSB : min(NSB, (last_tile * 16 + 15) / 32 + 1);
   const int grp = h / (H / G);
   const int t0 = c * Q;
