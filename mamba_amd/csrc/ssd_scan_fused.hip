@@ -81,28 +81,6 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
   const bf16_t *Cg = static_cast<const bf16_t *>(p.C) + b * p.C_bs + grp * p.C_gs;
   const bool has_seq = p.seq_idx != nullptr;
 
-  // ---- per-position scalars of this (batch, head, chunk)
-  {
-    const float *dA = p.dA_cumsum + (((int64_t)b * H + h) * p.nchunks + c) * Q;
-    const float *dt = p.dt_out + (((int64_t)b * H + h) * p.nchunks + c) * Q;
-    const int32_t *seq = has_seq ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
-    for (int s = tid; s < Q; s += NT) {
-      const float a = dA[s];
-      const float aend = dA[(s | 15)];
-      a2_s[s] = a * kLog2e;
-      dt_s[s] = dt[s];
-      cs_s[s] = dt[s] * fast_exp(aend - a);
-      bool ok = s < qlim;
-      int id = 0;
-      if (has_seq) {
-        id = s < qlim ? seq[s] : -2;
-        ok = ok && id == (c > 0 ? seq[-1] : 0);
-      }
-      seq_s[s] = id;
-      rs_s[s] = ok ? fast_exp(a) : 0.f;
-    }
-  }
-
   // ---- staging helpers (global -> registers -> LDS), one s block of 32 positions
   constexpr int BCH = (32 * N / 8 + NT - 1) / NT;    // 16-byte chunks of B per thread
   // X tasks: 4 consecutive positions x 8 consecutive p (four 16-byte loads, eight 8-byte
@@ -162,19 +140,10 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
     }
   };
 
+  // Prologue: every global load is issued before anything waits, so the workgroup pays one
+  // memory latency: the first two s blocks, the wave's C rows, the carried state, the scalars.
   load_block(0, bregs[0], xregs[0]);
   if (nsb > 1) load_block(1, bregs[1], xregs[1]);
-  // carried state, fp32 -> bf16, rows p, k = n
-  {
-    const float *Hc = p.states + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
-    for (int id = tid; id < P * N / 8; id += NT) {
-      const int pp = id / (N / 8), c8 = id % (N / 8);
-      const f32x4 v0 = *reinterpret_cast<const f32x4 *>(Hc + (int64_t)pp * N + c8 * 8);
-      const f32x4 v1 = *reinterpret_cast<const f32x4 *>(Hc + (int64_t)pp * N + c8 * 8 + 4);
-      u32x4 o = {pack_bf16(v0.x, v0.y), pack_bf16(v0.z, v0.w), pack_bf16(v1.x, v1.y), pack_bf16(v1.z, v1.w)};
-      *reinterpret_cast<u32x4 *>(&Hs[pp * BP + c8 * 8]) = o;
-    }
-  }
   // C rows of this wave's l tiles: B operand of both contractions (col l = j, k = n)
   bf16x8_t Cf[LT][NK];
 #pragma unroll
@@ -186,6 +155,50 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
       if (l < qlim) v = *reinterpret_cast<const u32x4 *>(Cg + (int64_t)(t0 + l) * p.C_ls + kk * 32 + g * 8);
       Cf[k][kk] = __builtin_bit_cast(bf16x8_t, v);
     }
+  }
+  // carried state, fp32 -> bf16, rows p, k = n
+  constexpr int HCH = (P * N / 8 + NT - 1) / NT;
+  f32x4 hraw[HCH][2];
+  {
+    const float *Hc = p.states + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
+#pragma unroll
+    for (int q = 0; q < HCH; ++q) {
+      const int id = tid + q * NT;
+      hraw[q][0] = hraw[q][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (id < P * N / 8) {
+        hraw[q][0] = *reinterpret_cast<const f32x4 *>(Hc + (int64_t)id * 8);
+        hraw[q][1] = *reinterpret_cast<const f32x4 *>(Hc + (int64_t)id * 8 + 4);
+      }
+    }
+  }
+  // ---- per-position scalars of this (batch, head, chunk)
+  {
+    const float *dA = p.dA_cumsum + (((int64_t)b * H + h) * p.nchunks + c) * Q;
+    const float *dt = p.dt_out + (((int64_t)b * H + h) * p.nchunks + c) * Q;
+    const int32_t *seq = has_seq ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
+    for (int s = tid; s < Q; s += NT) {
+      const float a = dA[s];
+      const float aend = dA[(s | 15)];
+      a2_s[s] = a * kLog2e;
+      dt_s[s] = dt[s];
+      cs_s[s] = dt[s] * fast_exp(aend - a);
+      bool ok = s < qlim;
+      int id = 0;
+      if (has_seq) {
+        id = s < qlim ? seq[s] : -2;
+        ok = ok && id == (c > 0 ? seq[-1] : 0);
+      }
+      seq_s[s] = id;
+      rs_s[s] = ok ? fast_exp(a) : 0.f;
+    }
+  }
+
+#pragma unroll
+  for (int q = 0; q < HCH; ++q) {
+    const int id = tid + q * NT, pp = id / (N / 8), c8 = id % (N / 8);
+    const f32x4 v0 = hraw[q][0], v1 = hraw[q][1];
+    const u32x4 o = {pack_bf16(v0.x, v0.y), pack_bf16(v0.z, v0.w), pack_bf16(v1.x, v1.y), pack_bf16(v1.z, v1.w)};
+    if (id < P * N / 8) *reinterpret_cast<u32x4 *>(&Hs[pp * BP + c8 * 8]) = o;
   }
   store_block(0, bregs[0], xregs[0]);
   __syncthreads();
