@@ -282,8 +282,10 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
   const int tid = threadIdx.x;
   const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads, G = p.ngroups;
   const int ntp = cdiv(P, GB);
-  const int st = blockIdx.x / ntp, pt = blockIdx.x % ntp;
-  const int c = blockIdx.y, b = blockIdx.z / H, h = blockIdx.z % H;
+  const Block3 blk = xcd_block();
+  const int nst = gridDim.x / ntp;
+  const int st = blk.x % nst, pt = blk.x / nst;  // the s tiles of a (chunk, head) share dS and CB
+  const int c = blk.y, b = blk.z / H, h = blk.z % H;
   const int g = h / (H / G);
   const int t0 = c * Q, qlim = min(Q, L - t0);
   const float *dA = chunk_row(p.dA_cumsum, p, b, h, c);
@@ -424,9 +426,11 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dBC
   const int i = lane & 15, gq = lane >> 4;
   const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads, G = p.ngroups;
   const int ntn = cdiv(N, GB);
-  const int st = blockIdx.x / ntn, nt = blockIdx.x % ntn;
+  const Block3 blk = xcd_block();
+  const int nst = gridDim.x / ntn;
+  const int st = blk.x % nst, nt = blk.x / nst;  // the s tiles of a chunk share the state tiles
   const int hpg = H / G, nsplit = head_splits(hpg);
-  const int c = blockIdx.y, bg = blockIdx.z / nsplit, hs = blockIdx.z % nsplit, b = bg / G, g = bg % G;
+  const int c = blk.y, bg = blk.z / nsplit, hs = blk.z % nsplit, b = bg / G, g = bg % G;
   const int t0 = c * Q, qlim = min(Q, L - t0);
   const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
   const View4 gv = g_view(p);
@@ -531,11 +535,12 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dcb
   const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
   const int i = lane & 15, gq = lane >> 4;
   const int Q = p.chunk_size, L = p.seqlen, P = p.headdim, H = p.nheads, G = p.ngroups;
-  int lt = 0, rem = blockIdx.x;
+  const Block3 blk = xcd_block();
+  int lt = 0, rem = blk.x;
   while (rem > lt) { rem -= lt + 1; ++lt; }
   const int st = rem;
   const int hpg = H / G, nsplit = head_splits(hpg);
-  const int c = blockIdx.y, bg = blockIdx.z / nsplit, hs = blockIdx.z % nsplit, b = bg / G, g = bg % G;
+  const int c = blk.y, bg = blk.z / nsplit, hs = blk.z % nsplit, b = bg / G, g = bg % G;
   const int t0 = c * Q, qlim = min(Q, L - t0);
   const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
   const View4 gv = g_view(p);

@@ -280,3 +280,17 @@ DEVI void acc_to_rows(const GemmAcc &acc, GemmLds &s, int tid, float (&o)[16]) {
 }
 
 DEVI int cdiv(int a, int b) { return (a + b - 1) / b; }
+
+// Logical block coordinates.  The hardware deals consecutive workgroup ids to the 8 XCDs in turn,
+// and every XCD has its own L2; this remap gives each XCD one contiguous range of logical ids, so
+// that neighbours along x (tiles that share operands) run at about the same time behind one L2.
+struct Block3 {
+  int x, y, z;
+};
+DEVI Block3 xcd_block() {
+  const int nx = gridDim.x, ny = gridDim.y, total = nx * ny * gridDim.z;
+  const int pid = blockIdx.x + nx * (blockIdx.y + ny * blockIdx.z);
+  const int per = total / 8;
+  const int lid = pid < per * 8 ? (pid % 8) * per + pid / 8 : pid;
+  return {lid % nx, (lid / nx) % ny, lid / (nx * ny)};
+}
