@@ -228,12 +228,18 @@ int ssd_chunk_scan_fwd_fused_supported(const SsdParams *p);
 int ssd_chunk_scan_fwd_fused(const SsdParams *p, mamba_stream_t stream);
 /* cumsum, chunk_state, state_passing, then the fused scan when supported, else bmm + chunk_scan */
 int ssd_combined_fwd(const SsdParams *p, mamba_stream_t stream);
+/* Packed batch (p->batch == 1): the state after the last position of each of the nseq sequences
+ * [cu_seqlens[i], cu_seqlens[i+1]) into varlen_states (nseq, H, P, N) fp32.  Needs dt_out,
+ * dA_cumsum and states (entering each chunk) of a forward pass whose seq_idx matches cu_seqlens.
+ * Replaces chunk_state_varlen, mamba_ssm/ops/triton/ssd_chunk_state.py:1018. */
+int ssd_chunk_state_varlen(const SsdParams *p, const int32_t *cu_seqlens, int nseq, float *varlen_states,
+                           mamba_stream_t stream);
 
 /* Backward.  Inputs: the forward inputs, dout, dfinal_states, the saved pre-gate
  * output in out_x (z != NULL) or out (z == NULL), and the forward workspaces
  * dt_out, dA_cumsum, CB, states re-computed by the forward stages 1-4.
  * ssd_combined_bwd runs, in order:
- *   ssd_bwd_dz        dz, gbuf = dout silu(z), dD, and the <g, y - D x> part of ddA_cumsum
+ *   ssd_bwd_dz        dz, gbuf = dout silu(z), dD
  *   ssd_bwd_dstates   dstates[c] = direct gradient of the state entering chunk c
  *   ssd_state_passing_bwd  reverse recurrence over chunks (in place on dstates -> gradient
  *                     of the chunk-local states), dinitial_states, ddA_cumsum at chunk ends

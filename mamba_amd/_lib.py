@@ -90,6 +90,8 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = [ctypes.POINTER(SsdParams), c_vp]
         fn.restype = ctypes.c_int
+    lib.ssd_chunk_state_varlen.argtypes = [ctypes.POINTER(SsdParams), c_vp, ctypes.c_int, c_vp, c_vp]
+    lib.ssd_chunk_state_varlen.restype = ctypes.c_int
     lib.ssd_chunk_scan_fwd_fused_supported.argtypes = [ctypes.POINTER(SsdParams)]
     lib.ssd_chunk_scan_fwd_fused_supported.restype = ctypes.c_int
     lib.ssm_state_update.argtypes = [ctypes.POINTER(MambaStepParams), c_vp]

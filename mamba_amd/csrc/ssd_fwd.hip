@@ -157,6 +157,62 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void chunk_s
   });
 }
 
+// ---------------------------------------------------- chunk_state_varlen
+// Packed batch (batch 1): state at the last position of every sequence i = [cu[i], cu[i+1]).
+// out[i, h, p, n] = sum_{k in the last chunk, k >= start} x[k, p] B[k, n] exp(a_end - a_k) dt_k
+//                 + exp(a_end) states[c, h, p, n] if the sequence began before that chunk,
+// with `states` the state entering each chunk.  Empty sequences give zeros.
+template <typename T, bool SPLIT>
+__global__ __launch_bounds__(256) void chunk_state_varlen_kernel(const SsdParams p, const int32_t *cu, float *out) {
+  __shared__ GemmLds lds;
+  __shared__ float w[256];
+  const int tid = threadIdx.x;
+  const int Q = p.chunk_size, N = p.dstate, P = p.headdim, H = p.nheads;
+  const int ntn = cdiv(N, GB);
+  const int pt = blockIdx.x / ntn, nt = blockIdx.x % ntn;
+  const int i = blockIdx.y, h = blockIdx.z;
+  const int g = h / (H / p.ngroups);
+  const int start = cu[i], end = min(cu[i + 1], p.seqlen);
+  float *dst = out + ((int64_t)i * H + h) * P * N;
+  GemmAcc acc;
+  acc.zero();
+  if (end > start) {
+    const int c = (end - 1) / Q, t0 = c * Q;
+    const int kstart = max(start - t0, 0), kend = end - t0;
+    const float *dA = p.dA_cumsum + ((int64_t)h * p.nchunks + c) * Q;
+    const float *dt = p.dt_out + ((int64_t)h * p.nchunks + c) * Q;
+    const float a_end = dA[kend - 1];
+    for (int k = tid; k < Q; k += 256)
+      w[k] = (k >= kstart && k < kend) ? fast_exp(fminf(a_end - dA[k], 0.f)) * dt[k] : 0.f;
+    const T *xa = static_cast<const T *>(p.x) + h * p.x_hs + (int64_t)t0 * p.x_ls + pt * GB;
+    const T *Ba = static_cast<const T *>(p.B) + g * p.B_gs + (int64_t)t0 * p.B_ls + nt * GB;
+    const bool va = rows_aligned16(xa, p.x_ls), vb = rows_aligned16(Ba, p.B_ls);
+    block_gemm_staged<SPLIT>(  // the first barrier inside publishes w
+        acc, lds, kstart / GK * GK, kend,
+        [&](int k0) {
+          if (tid < 128) stage_rc<SPLIT, T>(lds.ah, lds.al, xa, p.x_ls, P - pt * GB, k0, kend, nullptr, nullptr, va, tid);
+        },
+        [&](int k0) {
+          if (tid >= 128)
+            stage_rc<SPLIT, T>(lds.bh, lds.bl, Ba, p.B_ls, N - nt * GB, k0, kend, w, nullptr, vb, tid - 128);
+        },
+        tid);
+    if (start < t0) {
+      const float *Hc = p.states + ((int64_t)c * H + h) * P * N;
+      const float sc = fast_exp(a_end);
+      acc_foreach(acc, tid, [&](int m, int n, float v) {
+        const int pp = pt * GB + m, nn = nt * GB + n;
+        return (pp < P && nn < N) ? __builtin_fmaf(sc, Hc[(int64_t)pp * N + nn], v) : v;
+      });
+    }
+  }
+  acc_foreach(acc, tid, [&](int m, int n, float v) {
+    const int pp = pt * GB + m, nn = nt * GB + n;
+    if (pp < P && nn < N) dst[(int64_t)pp * N + nn] = v;
+    return v;
+  });
+}
+
 // ---------------------------------------------------------- state_passing
 // In place over `states`: slot c receives the state ENTERING chunk c; the state
 // after the last chunk goes to final_states.
@@ -321,6 +377,29 @@ extern "C" int ssd_chunk_state_fwd(const SsdParams *p, mamba_stream_t stream) {
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid(((p->headdim + GB - 1) / GB) * ((p->dstate + GB - 1) / GB), p->nchunks, p->batch * p->nheads);
   SSD_DISPATCH(chunk_state_fwd_kernel, grid)
+  return launched();
+}
+
+extern "C" int ssd_chunk_state_varlen(const SsdParams *p, const int32_t *cu_seqlens, int nseq, float *varlen_states,
+                                      mamba_stream_t stream) {
+  int rc = check(p);
+  if (rc) return rc;
+  if (!p->states || !p->dt_out || !p->dA_cumsum || !cu_seqlens || !varlen_states) return MAMBA_E_BADARG;
+  if (p->batch != 1 || nseq < 0 || nseq > 65535) return MAMBA_E_BADARG;
+  if (nseq == 0) return MAMBA_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  dim3 grid(((p->headdim + GB - 1) / GB) * ((p->dstate + GB - 1) / GB), nseq, p->nheads);
+  switch (p->dtype) {
+    case MAMBA_BF16:
+      hipLaunchKernelGGL((chunk_state_varlen_kernel<bf16_t, false>), grid, dim3(256), 0, s, *p, cu_seqlens, varlen_states);
+      break;
+    case MAMBA_F16:
+      hipLaunchKernelGGL((chunk_state_varlen_kernel<f16_t, true>), grid, dim3(256), 0, s, *p, cu_seqlens, varlen_states);
+      break;
+    default:
+      hipLaunchKernelGGL((chunk_state_varlen_kernel<float, true>), grid, dim3(256), 0, s, *p, cu_seqlens, varlen_states);
+      break;
+  }
   return launched();
 }
 

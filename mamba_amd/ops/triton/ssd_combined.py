@@ -98,11 +98,17 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
                                    seq_idx=None, cu_seqlens=None, dt_softplus=False, dt_limit=(0.0, float("inf")),
                                    state_dtype=None):
     """Counterpart of ssd_combined.py:343.  Returns (out, out_x, dt_out, dA_cumsum, states, final_states)
-    where `states[:, c]` is the state entering chunk c, in fp32."""
+    where `states[:, c]` is the state entering chunk c, in fp32; with cu_seqlens a seventh element,
+    varlen_states (nseq, nheads, headdim, dstate): the state at the end of every packed sequence
+    (ssd_combined.py:390-394), in state_dtype, else C's dtype, as the reference returns it."""
+    state_out_dtype = state_dtype if state_dtype is not None else C.dtype
     x, dt, A, B, C, D, z, dt_bias, initial_states, seq_idx = _prepare(
         x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, seq_idx)
     if cu_seqlens is not None:
-        raise NotImplementedError("return_varlen_states (chunk_state_varlen) is not built in mamba_amd")
+        assert x.shape[0] == 1, "passing cu_seqlens to get the varlen states is only supported if batch dimension is 1"
+        assert cu_seqlens.dim() == 1 and cu_seqlens.numel() >= 1
+        _lib.require_gpu(cu_seqlens)
+        cu_seqlens = cu_seqlens.to(torch.int32).contiguous()
     ws = _workspace(x, B, chunk_size)
     out = torch.empty_like(x, memory_format=torch.contiguous_format)
     out_x = torch.empty_like(out) if z is not None else None
@@ -112,6 +118,13 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
     p.out_bs, p.out_ls, p.out_hs = out.stride(0), out.stride(1), out.stride(2)
     with torch.cuda.device(x.device):
         _lib.check(_lib.load().ssd_combined_fwd(p, _lib.current_stream(x.device)), "ssd_combined_fwd")
+        if cu_seqlens is not None:
+            nseq = cu_seqlens.numel() - 1
+            varlen = torch.empty(nseq, x.shape[2], x.shape[3], B.shape[3], device=x.device, dtype=torch.float32)
+            _lib.check(_lib.load().ssd_chunk_state_varlen(p, cu_seqlens.data_ptr(), nseq, varlen.data_ptr(),
+                                                          _lib.current_stream(x.device)), "ssd_chunk_state_varlen")
+            return (out, out_x, ws["dt_out"], ws["dA_cumsum"], ws["states"], ws["final_states"],
+                    varlen.to(state_out_dtype))
     return out, out_x, ws["dt_out"], ws["dA_cumsum"], ws["states"], ws["final_states"]
 
 
@@ -198,7 +211,7 @@ class MambaChunkScanCombinedFn(torch.autograd.Function):
             cu_seqlens = None
         else:
             assert cu_seqlens is not None, "cu_seqlens must be provided if return_varlen_states is True"
-        out, out_x, dt_out, dA_cumsum, states, final_states = _mamba_chunk_scan_combined_fwd(
+        out, out_x, dt_out, dA_cumsum, states, final_states, *rest = _mamba_chunk_scan_combined_fwd(
             x, dt, A, B, C, chunk_size, D=D, z=z, dt_bias=dt_bias, initial_states=initial_states, seq_idx=seq_idx,
             cu_seqlens=cu_seqlens, dt_softplus=dt_softplus, dt_limit=dt_limit, state_dtype=state_dtype)
         ctx.save_for_backward(out if z is None else out_x, x, dt, dA_cumsum, A, B, C, D, z, dt_bias, initial_states,
@@ -208,7 +221,10 @@ class MambaChunkScanCombinedFn(torch.autograd.Function):
         ctx.dt_limit = dt_limit
         ctx.return_final_states = return_final_states
         ctx.return_varlen_states = return_varlen_states
-        return out if not return_final_states else (out, final_states)
+        if not return_varlen_states:
+            return out if not return_final_states else (out, final_states)
+        varlen_states = rest[0]
+        return (out, varlen_states) if not return_final_states else (out, final_states, varlen_states)
 
     @staticmethod
     def backward(ctx, dout, *args):

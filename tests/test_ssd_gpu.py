@@ -145,3 +145,44 @@ def test_ssd_bwd_options(dtype):
 def test_ssd_bwd_packed_sequences(dtype):
     _bwd_case(1, 1024, 8, 64, 64, 8, 256, dtype, seq_lens=[100, 156, 256, 300, 212], has_init=True)
     _bwd_case(2, 640, 4, 32, 32, 2, 128, dtype, seq_lens=[1, 127, 129, 383], has_init=False)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("seq_lens", [[100, 156, 256, 1, 299, 212], [300, 84, 128, 512]])
+def test_ssd_varlen_states(seq_lens, dtype):
+    """return_varlen_states: the state at the end of every packed sequence equals the final state of
+    that sequence run alone through the oracle.  Boundaries inside chunks, on chunk edges, length 1.
+    Only sequence 0 sees initial_states (ssd_state_passing.py:71-79), and, as in the reference
+    (ssd_chunk_state.py:700-706 adds the carried state only when the sequence began before its last
+    chunk), not when it ends inside the first chunk."""
+    from mamba_amd.ops.triton.ssd_combined import mamba_chunk_scan_combined
+    chunk = 128
+    total = sum(seq_lens)
+    t = ssd_inputs(1, total, 4, 64, 32, 2, dtype, 3, seq_lens=seq_lens, has_init=True)
+    rtol, atol = _tol(dtype)
+    cu_seqlens = torch.tensor([0] + list(torch.tensor(seq_lens).cumsum(0)), dtype=torch.int32)
+    refs, start = [], 0
+    for i, n in enumerate(seq_lens):
+        sl = slice(start, start + n)
+        seeded = i == 0 and n > chunk
+        _, fin = ssd_oracle(t["x"][:, sl], t["dt"][:, sl], t["A"], t["B"][:, sl], t["C"][:, sl], D=t["D"],
+                            z=t["z"][:, sl], dt_bias=t["dt_bias"],
+                            initial_states=t["initial_states"] if seeded else None, dt_softplus=True,
+                            return_final_states=True)
+        refs.append(fin[0])
+        start += n
+    ref = torch.stack(refs)
+    cu = lambda v: None if v is None else v.cuda()
+    out, fin, varlen = mamba_chunk_scan_combined(
+        cu(t["x"]), cu(t["dt"]), cu(t["A"]), cu(t["B"]), cu(t["C"]), chunk, D=cu(t["D"]), z=cu(t["z"]),
+        dt_bias=cu(t["dt_bias"]), initial_states=cu(t["initial_states"]), seq_idx=cu(t["seq_idx"]),
+        cu_seqlens=cu_seqlens.cuda(), dt_softplus=True, return_final_states=True, return_varlen_states=True)
+    assert varlen.shape == ref.shape and varlen.dtype == dtype
+    _close("varlen_states", varlen, ref, rtol, atol)
+    _close("final_states", fin, ref[-1:], rtol, atol)
+    out2, varlen2 = mamba_chunk_scan_combined(
+        cu(t["x"]), cu(t["dt"]), cu(t["A"]), cu(t["B"]), cu(t["C"]), chunk, D=cu(t["D"]), z=cu(t["z"]),
+        dt_bias=cu(t["dt_bias"]), initial_states=cu(t["initial_states"]), seq_idx=cu(t["seq_idx"]),
+        cu_seqlens=cu_seqlens.cuda(), dt_softplus=True, return_varlen_states=True, state_dtype=torch.float32)
+    assert varlen2.dtype == torch.float32 and torch.equal(out, out2)
+    _close("varlen_states fp32", varlen2, ref, rtol, atol)
