@@ -68,6 +68,10 @@ int mamba_hip_copy(void *dst, const void *src, int64_t nbytes, mamba_stream_t st
  * of `dtype`, seqlen stride 1.  B, C are (batch, ngroups, dstate, seqlen) of
  * `dtype`, seqlen stride 1; channel d uses group d / (dim / ngroups).
  * A is (dim, dstate) fp32 contiguous; D, delta_bias are (dim) fp32 or NULL.
+ * With bc_const bit 0 (bit 1) set, B (C) is instead a contiguous (dim, dstate) fp32
+ * matrix used at every position (the reference's is_variable_B / is_variable_C false,
+ * csrc/selective_scan/selective_scan.cpp:254-255); its strides are ignored and
+ * ngroups describes the other operand (1 when both are matrices).
  *
  * ckpt is (batch, dim, ntiles, dstate) fp32 contiguous with
  * ntiles = ceil(seqlen / MAMBA_Q_SCAN_TILE): the state h after the last
@@ -78,7 +82,7 @@ typedef struct MambaScanParams {
   int32_t batch, dim, seqlen, dstate, ngroups;
   int32_t dtype; /* MAMBA_F32 / MAMBA_BF16 / MAMBA_F16 */
   int32_t delta_softplus;
-  int32_t reserved0;
+  int32_t bc_const; /* bit 0: B is an input-independent (dim, dstate) fp32 matrix; bit 1: C likewise */
 
   const void *u, *delta, *A, *B, *C;
   const void *D, *z, *delta_bias; /* nullable */
@@ -100,7 +104,8 @@ typedef struct MambaScanParams {
   /* fp32 accumulators.  dB32, dC32: (batch, ngroups, dstate, seqlen) contiguous,
    * MUST be zero on entry (kernels add into them).  dA_part: (batch, dim, dstate),
    * dD_part, ddelta_bias_part: (batch, dim) -- written (not accumulated), the
-   * caller sums them over batch. */
+   * caller sums them over batch.  For an input-independent B (C), dB32 (dC32) is
+   * instead (batch, dim, dstate) partials, written like dA_part. */
   float *dB32, *dC32, *dA_part, *dD_part, *ddelta_bias_part;
   int64_t dout_bs, dout_ds;
   int64_t du_bs, du_ds;

@@ -28,10 +28,12 @@ constexpr int MAX_DSTATE = 256;
 // B or C rows n0..n0+15 of the tile starting at t0 -> LDS as fp32, laid out
 // [n][half][lane][4] so that a lane reads its 8 items with two conflict-free
 // 16-byte LDS loads.
-template <typename T, bool VEC, int NTHREADS>
+// BC: bit 0 set = B is not staged (input-independent), bit 1 = C likewise.
+template <typename T, bool VEC, int NTHREADS, int BC>
 DEVI void stage_bc(float *Bs, float *Cs, const T *Bg, int64_t B_ns, const T *Cg, int64_t C_ns, int n0, int N, int t0,
                    int L, int tid) {
-  for (int unit = tid; unit < 2 * NB16 * 64; unit += NTHREADS) {
+  constexpr int FIRST = (BC & 1) ? NB16 * 64 : 0, LAST = (BC & 2) ? NB16 * 64 : 2 * NB16 * 64;
+  for (int unit = FIRST + tid; unit < LAST; unit += NTHREADS) {
     const int which = unit >> 10, n = (unit >> 6) & 15, j = unit & 63;
     const int t = t0 + KI * j;
     const T *src = (which ? Cg + (int64_t)(n0 + n) * C_ns : Bg + (int64_t)(n0 + n) * B_ns) + t;
@@ -58,8 +60,23 @@ DEVI void lds_ld8(const float *base, int lane, float (&o)[8]) {
   o[4] = hi.x; o[5] = hi.y; o[6] = hi.z; o[7] = hi.w;
 }
 
+// The 8 items of B (or C) for state n of channel d: from the staged tile, or, when the operand is an
+// input-independent (dim, dstate) fp32 matrix, its one value for every position (0 for padded states).
+template <int CONST>
+DEVI void load_bc(float (&v)[8], const float *staged, const void *mat, int d, int N, int n_abs, int n_loc, int lane) {
+  if constexpr (CONST != 0) {
+    const float c = n_abs < N ? static_cast<const float *>(mat)[(int64_t)d * N + n_abs] : 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = c;
+  } else {
+    lds_ld8(staged + n_loc * TILE, lane, v);
+  }
+}
+
 // ------------------------------------------------------------------ forward
-template <typename T, int NW, int R, bool VEC>
+// BC: bit 0 = B is an input-independent (dim, dstate) fp32 matrix, bit 1 = C likewise
+// (selective_scan_fwd_kernel.cuh:74 kIsVariableB / kIsVariableC false).
+template <typename T, int NW, int R, bool VEC, int BC>
 __global__ __launch_bounds__(NW * 64) void scan_fwd_kernel(const MambaScanParams p) {
   extern __shared__ __align__(16) float smem[];
   const int N = p.dstate, L = p.seqlen;
@@ -110,9 +127,9 @@ __global__ __launch_bounds__(NW * 64) void scan_fwd_kernel(const MambaScanParams
         }
       }
       for (int nb = 0; nb < NBLK; ++nb) {
-        if (NBLK > 1 || r == 0) {
+        if (BC != 3 && (NBLK > 1 || r == 0)) {
           __syncthreads();
-          stage_bc<T, VEC, NW * 64>(Bs, Cs, Bg, p.B_ns, Cg, p.C_ns, nb * NB16, N, t0, L, tid);
+          stage_bc<T, VEC, NW * 64, BC>(Bs, Cs, Bg, p.B_ns, Cg, p.C_ns, nb * NB16, N, t0, L, tid);
           __syncthreads();
         }
         if (valid) {
@@ -128,8 +145,8 @@ __global__ __launch_bounds__(NW * 64) void scan_fwd_kernel(const MambaScanParams
               const float A2 = A2row[n + q];
               hc[q] = hrow[n + q];
               float Bv[8];
-              lds_ld8(Bs + (n + q) * TILE, lane, Bv);
-              lds_ld8(Cs + (n + q) * TILE, lane, Cv[q]);
+              load_bc<BC & 1>(Bv, Bs, p.B, d, N, nb * NB16 + n + q, n + q, lane);
+              load_bc<BC & 2>(Cv[q], Cs, p.C, d, N, nb * NB16 + n + q, n + q, lane);
 #pragma unroll
               for (int i = 0; i < KI; ++i) a[q][i] = fast_exp2(dl[i] * A2);
               hh[q][0] = du[0] * Bv[0];
@@ -175,7 +192,7 @@ __global__ __launch_bounds__(NW * 64) void scan_fwd_kernel(const MambaScanParams
 }
 
 // ----------------------------------------------------------------- backward
-template <typename T, int NW, int R, bool VEC>
+template <typename T, int NW, int R, bool VEC, int BC>
 __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams p) {
   extern __shared__ __align__(16) float smem[];
   const int N = p.dstate, L = p.seqlen;
@@ -192,6 +209,8 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
   float *dAacc = anx + WR * NP;       // [WR][NP]
   float *dDacc = dAacc + WR * NP;     // [WR]
   float *dbacc = dDacc + WR;          // [WR]
+  float *dBcacc = dbacc + WR;         // [WR][NP] gradients of input-independent B / C
+  float *dCcacc = dBcacc + WR * NP;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -217,6 +236,8 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
     gcar[o] = 0.f;
     anx[o] = 0.f;
     dAacc[o] = 0.f;
+    dBcacc[o] = 0.f;
+    dCcacc[o] = 0.f;
   }
   if (lane < R) {
     dDacc[wave * R + lane] = 0.f;
@@ -267,9 +288,9 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
         }
       }
       for (int nb = 0; nb < NBLK; ++nb) {
-        if (NBLK > 1 || r == 0) {
+        if (BC != 3 && (NBLK > 1 || r == 0)) {
           __syncthreads();
-          stage_bc<T, VEC, NW * 64>(Bs, Cs, Bg, p.B_ns, Cg, p.C_ns, nb * NB16, N, t0, L, tid);
+          stage_bc<T, VEC, NW * 64, BC>(Bs, Cs, Bg, p.B_ns, Cg, p.C_ns, nb * NB16, N, t0, L, tid);
           for (int i = tid * 4; i < 2 * BC_FLOATS; i += NW * 256)  // dBs and dCs are adjacent
             *reinterpret_cast<f32x4 *>(dBs + i) = f32x4{0.f, 0.f, 0.f, 0.f};
           __syncthreads();
@@ -302,8 +323,8 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
                 hc[q] = hrow[n + q];
                 gc[q] = grow[n + q];
                 an[q] = arow[n + q];
-                lds_ld8(Bs + (n + q) * TILE, lane, Bv[q]);
-                lds_ld8(Cs + (n + q) * TILE, lane, Cv[q]);
+                load_bc<BC & 1>(Bv[q], Bs, p.B, d, N, nb * NB16 + n + q, n + q, lane);
+                load_bc<BC & 2>(Cv[q], Cs, p.C, d, N, nb * NB16 + n + q, n + q, lane);
                 const float A2 = A1[q] * kLog2e;
 #pragma unroll
                 for (int i = 0; i < KI; ++i) {
@@ -370,32 +391,43 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
                   grow[n + q] = gfirst[q];
                   arow[n + q] = a[q][0];
                 }
-                float dAp = 0.f;
+                float dAp = 0.f, dBp = 0.f, dCp = 0.f;
                 float sB[8], sC[8];
-                lds_ld8(dBs + (n + q) * TILE, lane, sB);
-                lds_ld8(dCs + (n + q) * TILE, lane, sC);
+                if constexpr (!(BC & 1)) lds_ld8(dBs + (n + q) * TILE, lane, sB);
+                if constexpr (!(BC & 2)) lds_ld8(dCs + (n + q) * TILE, lane, sC);
 #pragma unroll
                 for (int i = 0; i < KI; ++i) {
                   const float gi = __builtin_fmaf(ar[q][i], gx, gg[q][i]);
-                  sC[i] = __builtin_fmaf(dy[i], h[q][i], sC[i]);
-                  sB[i] = __builtin_fmaf(gi, du[i], sB[i]);
+                  if constexpr (BC & 2) dCp = __builtin_fmaf(dy[i], h[q][i], dCp);
+                  else sC[i] = __builtin_fmaf(dy[i], h[q][i], sC[i]);
+                  if constexpr (BC & 1) dBp = __builtin_fmaf(gi, du[i], dBp);
+                  else sB[i] = __builtin_fmaf(gi, du[i], sB[i]);
                   acc[i] = __builtin_fmaf(gi, Bv[q][i], acc[i]);
                   const float w = gi * (h[q][i] - bb[q][i]);  // g * a * h[t-1]
                   dd[i] = __builtin_fmaf(A1[q], w, dd[i]);
                   dAp = __builtin_fmaf(dl[i], w, dAp);
                 }
-                lds_st8(dBs + (n + q) * TILE, lane, sB);
-                lds_st8(dCs + (n + q) * TILE, lane, sC);
+                if constexpr (!(BC & 1)) lds_st8(dBs + (n + q) * TILE, lane, sB);
+                if constexpr (!(BC & 2)) lds_st8(dCs + (n + q) * TILE, lane, sC);
                 dAp = wave_sum_to_last(dAp);
                 if (lane == 63) dArow[n + q] += dAp;  // the row belongs to this wave alone
+                if constexpr (BC & 1) {
+                  dBp = wave_sum_to_last(dBp);
+                  if (lane == 63) dBcacc[row * NP + nb * NB16 + n + q] += dBp;
+                }
+                if constexpr (BC & 2) {
+                  dCp = wave_sum_to_last(dCp);
+                  if (lane == 63) dCcacc[row * NP + nb * NB16 + n + q] += dCp;
+                }
               }
             }
             __syncthreads();
           }
         }
-        if (NBLK > 1 || r == R - 1) {
+        if (BC != 3 && (NBLK > 1 || r == R - 1)) {
           const int n0 = nb * NB16;
-          for (int i = tid; i < 2 * NB16 * TILE; i += NW * 64) {
+          constexpr int FIRST = (BC & 1) ? NB16 * TILE : 0, LAST = (BC & 2) ? NB16 * TILE : 2 * NB16 * TILE;
+          for (int i = FIRST + tid; i < LAST; i += NW * 64) {
             const int which = i >> 13, n = (i >> 9) & 15, t = i & (TILE - 1);
             const float v = (which ? dCs : dBs)[n * TILE + ((t >> 2) & 1) * 256 + (t >> 3) * 4 + (t & 3)];
             if (n0 + n < N && t0 + t < L) unsafeAtomicAdd((which ? dCg : dBg) + (int64_t)(n0 + n) * L + t0 + t, v);
@@ -449,7 +481,11 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
     const int d = dbase + r;
     if (d >= dend) continue;
     const int row = wave * R + r;
-    for (int n = lane; n < N; n += 64) p.dA_part[((int64_t)b * p.dim + d) * N + n] = dAacc[row * NP + n];
+    for (int n = lane; n < N; n += 64) {
+      p.dA_part[((int64_t)b * p.dim + d) * N + n] = dAacc[row * NP + n];
+      if constexpr (BC & 1) p.dB32[((int64_t)b * p.dim + d) * N + n] = dBcacc[row * NP + n];
+      if constexpr (BC & 2) p.dC32[((int64_t)b * p.dim + d) * N + n] = dCcacc[row * NP + n];
+    }
     if (lane == 0) {
       p.dD_part[(int64_t)b * p.dim + d] = dDacc[row];
       p.ddelta_bias_part[(int64_t)b * p.dim + d] = dbacc[row];
@@ -466,7 +502,7 @@ struct Cfg {
 
 inline size_t fwd_lds(int nw, int r, int np) { return sizeof(float) * (2 * BC_FLOATS + 2 * nw * r * np); }
 inline size_t bwd_lds(int nw, int r, int np) {
-  return sizeof(float) * (4 * BC_FLOATS + 5 * nw * r * np + 2 * nw * r);
+  return sizeof(float) * (4 * BC_FLOATS + 7 * nw * r * np + 2 * nw * r);
 }
 
 template <typename KernelT>
@@ -499,35 +535,45 @@ bool vec_ok(const MambaScanParams &p, bool bwd) {
   const int64_t m = 16 / es;
   auto ok = [&](const void *ptr, int64_t s0, int64_t s1) { return !ptr || (aligned16(ptr) && s0 % m == 0 && s1 % m == 0); };
   if (p.seqlen % 8 != 0) return false;
-  bool v = ok(p.u, p.u_bs, p.u_ds) && ok(p.delta, p.delta_bs, p.delta_ds) && ok(p.z, p.z_bs, p.z_ds) &&
-           ok(p.B, p.B_bs, p.B_gs) && p.B_ns % m == 0 && ok(p.C, p.C_bs, p.C_gs) && p.C_ns % m == 0;
+  bool v = ok(p.u, p.u_bs, p.u_ds) && ok(p.delta, p.delta_bs, p.delta_ds) && ok(p.z, p.z_bs, p.z_ds);
+  if (!(p.bc_const & 1)) v = v && ok(p.B, p.B_bs, p.B_gs) && p.B_ns % m == 0;
+  if (!(p.bc_const & 2)) v = v && ok(p.C, p.C_bs, p.C_gs) && p.C_ns % m == 0;
   if (!bwd) return v && ok(p.out, p.out_bs, p.out_ds);
   return v && ok(p.dout, p.dout_bs, p.dout_ds) && ok(p.du, p.du_bs, p.du_ds) &&
          ok(p.ddelta, p.ddelta_bs, p.ddelta_ds) && ok(p.dz, p.dz_bs, p.dz_ds) && ok(p.out_z, p.outz_bs, p.outz_ds);
 }
 
-template <typename T, bool BWD> int dispatch(const MambaScanParams &p, hipStream_t stream) {
+template <typename T, bool BWD, int BC> int dispatch_bc(const MambaScanParams &p, hipStream_t stream) {
   const int np = (p.dstate + NB16 - 1) / NB16 * NB16;
   const bool vec = vec_ok(p, BWD);
   const bool small = p.dstate <= NB16;
   if (!BWD) {
     if (small) {
       const size_t lds = fwd_lds(8, 4, np);
-      return vec ? launch(scan_fwd_kernel<T, 8, 4, true>, p, 8, 4, lds, stream)
-                 : launch(scan_fwd_kernel<T, 8, 4, false>, p, 8, 4, lds, stream);
+      return vec ? launch(scan_fwd_kernel<T, 8, 4, true, BC>, p, 8, 4, lds, stream)
+                 : launch(scan_fwd_kernel<T, 8, 4, false, BC>, p, 8, 4, lds, stream);
     }
     const size_t lds = fwd_lds(8, 1, np);
-    return vec ? launch(scan_fwd_kernel<T, 8, 1, true>, p, 8, 1, lds, stream)
-               : launch(scan_fwd_kernel<T, 8, 1, false>, p, 8, 1, lds, stream);
+    return vec ? launch(scan_fwd_kernel<T, 8, 1, true, BC>, p, 8, 1, lds, stream)
+               : launch(scan_fwd_kernel<T, 8, 1, false, BC>, p, 8, 1, lds, stream);
   } else {
     if (small) {
       const size_t lds = bwd_lds(8, 4, np);
-      return vec ? launch(scan_bwd_kernel<T, 8, 4, true>, p, 8, 4, lds, stream)
-                 : launch(scan_bwd_kernel<T, 8, 4, false>, p, 8, 4, lds, stream);
+      return vec ? launch(scan_bwd_kernel<T, 8, 4, true, BC>, p, 8, 4, lds, stream)
+                 : launch(scan_bwd_kernel<T, 8, 4, false, BC>, p, 8, 4, lds, stream);
     }
     const size_t lds = bwd_lds(4, 1, np);
-    return vec ? launch(scan_bwd_kernel<T, 4, 1, true>, p, 4, 1, lds, stream)
-               : launch(scan_bwd_kernel<T, 4, 1, false>, p, 4, 1, lds, stream);
+    return vec ? launch(scan_bwd_kernel<T, 4, 1, true, BC>, p, 4, 1, lds, stream)
+               : launch(scan_bwd_kernel<T, 4, 1, false, BC>, p, 4, 1, lds, stream);
+  }
+}
+
+template <typename T, bool BWD> int dispatch(const MambaScanParams &p, hipStream_t stream) {
+  switch (p.bc_const & 3) {
+    case 0: return dispatch_bc<T, BWD, 0>(p, stream);
+    case 1: return dispatch_bc<T, BWD, 1>(p, stream);
+    case 2: return dispatch_bc<T, BWD, 2>(p, stream);
+    default: return dispatch_bc<T, BWD, 3>(p, stream);
   }
 }
 

@@ -8,6 +8,8 @@ done by the HIP kernels of libmamba_gfx950.so through its C ABI; the functions
 reference's pybind module `selective_scan_cuda`
 (csrc/selective_scan/selective_scan.cpp:494-497).
 """
+import math
+
 import torch
 import torch.nn.functional as F
 from einops import rearrange
@@ -30,26 +32,40 @@ def _check_inputs(u, delta, A, B, C, D, z, delta_bias):
         raise NotImplementedError("selective_scan: complex A is not built in mamba_amd")
     if A.dtype != torch.float32:
         raise RuntimeError("selective_scan: A must be float32")
-    if B.dim() < 3 or C.dim() < 3:
-        raise NotImplementedError("selective_scan: input-independent B/C of shape (dim, dstate) is not built in mamba_amd")
     if u.dim() != 3:
         raise RuntimeError("selective_scan: u must be (batch, dim, seqlen)")
     batch, dim, seqlen = u.shape
     dstate = A.shape[1]
     if dstate > _lib.load().mamba_hip_query(2):
         raise RuntimeError("selective_scan only supports state dimension <= 256")
-    if delta.dtype != u.dtype or B.dtype != u.dtype or C.dtype != u.dtype:
-        raise RuntimeError("selective_scan: u, delta, B, C must share one dtype")
-    for name, t in (("u", u), ("delta", delta), ("B", B), ("C", C), ("z", z)):
+    if delta.dtype != u.dtype:
+        raise RuntimeError("selective_scan: u and delta must share one dtype")
+    for name, t in (("u", u), ("delta", delta), ("z", z)):
         if t is not None and t.stride(-1) != 1:
             raise RuntimeError(f"selective_scan: {name} must have stride 1 in the last dimension")
-    ngroups = B.shape[1]
+    # B / C: (batch, ngroups, dstate, seqlen) in u's dtype, or an input-independent (dim, dstate)
+    # matrix in A's dtype (selective_scan.cpp:254-259, :268-277)
+    ngroups = 1
+    for name, t in (("B", B), ("C", C)):
+        if t.dim() == 4:
+            ngroups = t.shape[1]
+    for name, t in (("B", B), ("C", C)):
+        if t.dim() == 2:
+            if t.dtype != torch.float32 or tuple(t.shape) != (dim, dstate) or not t.is_contiguous():
+                raise RuntimeError(f"selective_scan: input-independent {name} must be contiguous float32 (dim, dstate)")
+        elif t.dim() == 4:
+            if t.dtype != u.dtype:
+                raise RuntimeError(f"selective_scan: {name} must have u's dtype")
+            if t.stride(-1) != 1:
+                raise RuntimeError(f"selective_scan: {name} must have stride 1 in the last dimension")
+            if tuple(t.shape) != (batch, ngroups, dstate, seqlen):
+                raise RuntimeError("selective_scan: B/C must be (batch, ngroups, dstate, seqlen)")
+        else:
+            raise RuntimeError(f"selective_scan: {name} must be (batch, ngroups, dstate, seqlen) or (dim, dstate)")
     if tuple(delta.shape) != (batch, dim, seqlen):
         raise RuntimeError("selective_scan: delta shape mismatch")
     if tuple(A.shape) != (dim, dstate):
         raise RuntimeError("selective_scan: A shape mismatch")
-    if tuple(B.shape) != (batch, ngroups, dstate, seqlen) or tuple(C.shape) != (batch, ngroups, dstate, seqlen):
-        raise RuntimeError("selective_scan: B/C must be (batch, ngroups, dstate, seqlen)")
     if dim % ngroups != 0:
         raise RuntimeError("selective_scan: dim must be divisible by ngroups")
     if D is not None and (D.dtype != torch.float32 or tuple(D.shape) != (dim,) or D.stride(-1) != 1):
@@ -74,8 +90,11 @@ def _fill_common(p, u, delta, A, B, C, D, z, delta_bias, delta_softplus, ckpt, d
     p.delta_bs, p.delta_ds = delta.stride(0), delta.stride(1)
     if z is not None:
         p.z_bs, p.z_ds = z.stride(0), z.stride(1)
-    p.B_bs, p.B_gs, p.B_ns = B.stride(0), B.stride(1), B.stride(2)
-    p.C_bs, p.C_gs, p.C_ns = C.stride(0), C.stride(1), C.stride(2)
+    p.bc_const = (1 if B.dim() == 2 else 0) | (2 if C.dim() == 2 else 0)
+    if B.dim() == 4:
+        p.B_bs, p.B_gs, p.B_ns = B.stride(0), B.stride(1), B.stride(2)
+    if C.dim() == 4:
+        p.C_bs, p.C_gs, p.C_ns = C.stride(0), C.stride(1), C.stride(2)
 
 
 def selective_scan_fwd(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta_softplus=False):
@@ -104,12 +123,19 @@ def selective_scan_fwd(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta
 class ScanBwdBuffers:
     """Outputs and fp32 accumulators of one backward launch (all caller-owned)."""
 
-    def __init__(self, u, delta, B, z, dims, dz=None, recompute_out_z=False):
+    def __init__(self, u, delta, B, z, dims, dz=None, recompute_out_z=False, C=None):
         batch, dim, seqlen, dstate, ngroups = dims
         dev = u.device
         self.du = torch.empty_like(u)
         self.ddelta = torch.empty_like(delta)
-        self.dBC32 = torch.empty(2, batch, ngroups, dstate, seqlen, device=dev, dtype=torch.float32)
+        # one fp32 arena: per operand (batch, ngroups, dstate, seqlen) sums the kernel adds into, or
+        # (batch, dim, dstate) per-batch partials when the operand is an input-independent matrix
+        shapes = [(batch, dim, dstate) if (t is not None and t.dim() == 2) else (batch, ngroups, dstate, seqlen)
+                  for t in (B, C)]
+        sizes = [math.prod(sh) for sh in shapes]
+        self.dBC32 = torch.empty(sum(sizes), device=dev, dtype=torch.float32)
+        self.dB32 = self.dBC32[:sizes[0]].view(shapes[0])
+        self.dC32 = self.dBC32[sizes[0]:].view(shapes[1])
         self.dA_part = torch.empty(batch, dim, dstate, device=dev, dtype=torch.float32)
         self.dD_part = torch.empty(batch, dim, device=dev, dtype=torch.float32)
         self.dbias_part = torch.empty(batch, dim, device=dev, dtype=torch.float32)
@@ -134,7 +160,7 @@ def scan_bwd_launch(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, delta_softp
     dz, out_z = bufs.dz, bufs.out_z
     p.dout, p.du, p.ddelta = dout.data_ptr(), bufs.du.data_ptr(), bufs.ddelta.data_ptr()
     p.dz, p.out_z = _lib.ptr(dz), _lib.ptr(out_z)
-    p.dB32, p.dC32 = bufs.dBC32[0].data_ptr(), bufs.dBC32[1].data_ptr()
+    p.dB32, p.dC32 = bufs.dB32.data_ptr(), bufs.dC32.data_ptr()
     p.dA_part, p.dD_part = bufs.dA_part.data_ptr(), bufs.dD_part.data_ptr()
     p.ddelta_bias_part = bufs.dbias_part.data_ptr()
     p.dout_bs, p.dout_ds = dout.stride(0), dout.stride(1)
@@ -165,14 +191,15 @@ def selective_scan_bwd(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, dz=None,
                                              or dz.stride(-1) != 1):
         raise RuntimeError("selective_scan: dz must match z in dtype/shape with stride 1 in the last dimension")
     A = A.contiguous()
-    bufs = ScanBwdBuffers(u, delta, B, z, dims, dz, recompute_out_z)
+    bufs = ScanBwdBuffers(u, delta, B, z, dims, dz, recompute_out_z, C=C)
     scan_bwd_zero(bufs, u.device)
     scan_bwd_launch(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, delta_softplus, bufs, dims)
     dA = bufs.dA_part.sum(0)
     dD = bufs.dD_part.sum(0) if D is not None else None
     ddelta_bias = bufs.dbias_part.sum(0) if delta_bias is not None else None
-    return (bufs.du, bufs.ddelta, dA, bufs.dBC32[0].to(B.dtype), bufs.dBC32[1].to(C.dtype), dD, ddelta_bias,
-            bufs.dz, bufs.out_z)
+    dB = bufs.dB32.sum(0) if B.dim() == 2 else bufs.dB32.to(B.dtype)
+    dC = bufs.dC32.sum(0) if C.dim() == 2 else bufs.dC32.to(C.dtype)
+    return (bufs.du, bufs.ddelta, dA, dB, dC, dD, ddelta_bias, bufs.dz, bufs.out_z)
 
 
 class SelectiveScanFn(torch.autograd.Function):
@@ -187,9 +214,9 @@ class SelectiveScanFn(torch.autograd.Function):
             delta = delta.contiguous()
         if D is not None:
             D = D.contiguous()
-        if B.stride(-1) != 1:
+        if B.stride(-1) != 1 or B.dim() == 2:
             B = B.contiguous()
-        if C.stride(-1) != 1:
+        if C.stride(-1) != 1 or C.dim() == 2:
             C = C.contiguous()
         if z is not None and z.stride(-1) != 1:
             z = z.contiguous()
@@ -241,13 +268,19 @@ def selective_scan_ref(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta
         delta = delta + delta_bias[..., None].float()
     if delta_softplus:
         delta = F.softplus(delta)
-    if A.is_complex() or B.dim() < 3 or C.dim() < 3:
-        raise NotImplementedError("selective_scan_ref: complex A / input-independent B, C are not built")
+    if A.is_complex():
+        raise NotImplementedError("selective_scan_ref: complex A is not built")
     dim = A.shape[0]
-    Bf = B.float() if B.dim() == 4 else B.float()[:, None]
-    Cf = C.float() if C.dim() == 4 else C.float()[:, None]
-    Bf = Bf.repeat_interleave(dim // Bf.shape[1], dim=1)
-    Cf = Cf.repeat_interleave(dim // Cf.shape[1], dim=1)
+
+    def per_channel(t):  # -> (batch or 1, dim, dstate, L or 1)
+        if t.dim() == 2:
+            return t.float()[None, :, :, None]
+        t = t.float() if t.dim() == 4 else t.float()[:, None]
+        return t.repeat_interleave(dim // t.shape[1], dim=1)
+
+    Bf, Cf = per_channel(B), per_channel(C)
+    Bf = Bf.expand(-1, -1, -1, u.shape[2]) if Bf.shape[-1] == 1 else Bf
+    Cf = Cf.expand(-1, -1, -1, u.shape[2]) if Cf.shape[-1] == 1 else Cf
     state = u.new_zeros(u.shape[0], dim, A.shape[1])
     ys = []
     for t in range(u.shape[2]):

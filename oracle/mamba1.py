@@ -6,7 +6,8 @@ Restates selective_scan_ref (reference mamba_ssm/ops/selective_scan_interface.py
     y_t = <h_t, C_t> + D u_t                            (:176-188)
     out = y * silu(z), cast back to the input dtype     (:189-192)
 B, C of shape (batch, ngroups, dstate, L) are shared by the dim/ngroups channels of a
-group (:169-172).  Gradients come from torch.autograd through this function, which is how
+group (:169-172); an input-independent B or C is a (dim, dstate) matrix used at every
+position (:163-166, :177-178).  Gradients come from torch.autograd through this function, which is how
 the reference's own test obtains them (tests/ops/test_selective_scan.py:119-121).
 Pinned by tests/test_oracle_mamba1.py.
 """
@@ -16,7 +17,7 @@ import torch.nn.functional as F
 
 def selective_scan_oracle(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta_softplus=False,
                           return_last_state=False, compute_dtype=torch.float32):
-    """u, delta, z: (b, d, L); A: (d, n); B, C: (b, n, L) or (b, g, n, L); D, delta_bias: (d,)."""
+    """u, delta, z: (b, d, L); A: (d, n); B, C: (b, n, L), (b, g, n, L) or (d, n); D, delta_bias: (d,)."""
     dtype_in = u.dtype
     cd = compute_dtype
     u = u.to(cd)
@@ -30,12 +31,15 @@ def selective_scan_oracle(u, delta, A, B, C, D=None, z=None, delta_bias=None, de
     A = A.to(cd)
     B = B.to(cd)
     C = C.to(cd)
-    if B.dim() == 3:
-        B = B[:, None]
-    if C.dim() == 3:
-        C = C[:, None]
-    B = B.repeat_interleave(dim // B.shape[1], dim=1)  # (b, d, n, L)
-    C = C.repeat_interleave(dim // C.shape[1], dim=1)
+    def per_channel(t):  # -> (b or 1, d, n, L)
+        if t.dim() == 2:
+            return t[None, :, :, None].expand(1, dim, n, L)
+        if t.dim() == 3:
+            t = t[:, None]
+        return t.repeat_interleave(dim // t.shape[1], dim=1)
+
+    B = per_channel(B)
+    C = per_channel(C)
     h = torch.zeros(batch, dim, n, dtype=cd, device=u.device)
     ys = []
     for t in range(L):

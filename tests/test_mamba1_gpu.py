@@ -31,7 +31,7 @@ def _close(name, got, ref, rtol, atol):
 
 
 def _run_case(batch, dim, dstate, seqlen, itype, groups, has_z=True, has_D=True, has_bias=True,
-              softplus=True, reference_style=True, seed=0):
+              softplus=True, reference_style=True, seed=0, var_B=True, var_C=True):
     from mamba_amd.ops.selective_scan_interface import selective_scan_fn
     dev = "cuda"
     rtol, atol, rtolw, atolw = _tols(itype)
@@ -39,8 +39,9 @@ def _run_case(batch, dim, dstate, seqlen, itype, groups, has_z=True, has_D=True,
     if reference_style:  # distributions of tests/ops/test_selective_scan.py:56-90
         A = -0.5 * torch.rand(dim, dstate, generator=g)
         Bshape = (batch, dstate, seqlen) if groups == 0 else (batch, groups, dstate, seqlen)
-        B = torch.randn(*Bshape, generator=g).to(itype)
-        C = torch.randn(*Bshape, generator=g).to(itype)
+        # input-independent B / C are fp32 (dim, dstate) matrices (tests/ops/test_selective_scan.py:64-79)
+        B = torch.randn(*Bshape, generator=g).to(itype) if var_B else torch.randn(dim, dstate, generator=g)
+        C = torch.randn(*Bshape, generator=g).to(itype) if var_C else torch.randn(dim, dstate, generator=g)
         D = torch.randn(dim, generator=g) if has_D else None
         z = torch.randn(batch, dim, seqlen, generator=g).to(itype) if has_z else None
         delta_bias = 0.5 * torch.rand(dim, generator=g) if has_bias else None
@@ -73,8 +74,8 @@ def _run_case(batch, dim, dstate, seqlen, itype, groups, has_z=True, has_D=True,
     _close("du", gr("u"), rr("u"), rtol * 2, atol * 2)
     _close("ddelta", gr("delta"), rr("delta"), rtol * 5, atol * 10)
     _close("dA", gr("A"), rr("A"), rtolw, atolw * 5)
-    _close("dB", gr("B"), rr("B"), rtol, atol)
-    _close("dC", gr("C"), rr("C"), rtol, atol)
+    _close("dB", gr("B"), rr("B"), rtol if var_B else rtolw, atol if var_B else atolw)
+    _close("dC", gr("C"), rr("C"), rtol if var_C else rtolw, atol if var_C else atolw)
     if has_D:
         _close("dD", gr("D"), rr("D"), rtolw, atolw)
     if has_z:
@@ -83,7 +84,7 @@ def _run_case(batch, dim, dstate, seqlen, itype, groups, has_z=True, has_D=True,
         _close("ddelta_bias", gr("delta_bias"), rr("delta_bias"), rtolw, atolw)
     for k in ("u", "delta", "B", "C", "z"):
         if gpu_in[k] is not None:
-            assert gr(k).dtype == itype and gr(k).shape == gpu_in[k].shape
+            assert gr(k).dtype == gpu_in[k].dtype and gr(k).shape == gpu_in[k].shape
     assert gr("A").dtype == torch.float32
 
 
@@ -117,3 +118,13 @@ def test_selective_scan_dstate(dstate):
 def test_selective_scan_benchmark_distribution(itype):
     # the benchmark's value distributions (A = -(1..16), softplus^-1 bias) on a slice of its shape
     _run_case(2, 96, 16, 2048, itype, 1, reference_style=False)
+
+
+@pytest.mark.parametrize("itype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("var_B,var_C", [(False, True), (True, False), (False, False)])
+def test_selective_scan_input_independent_B_C(var_B, var_C, itype):
+    # is_variable_B / is_variable_C of tests/ops/test_selective_scan.py:30-33: (dim, dstate) fp32 matrices;
+    # several tiles, a ragged tail, more channels than one workgroup holds, dstate above one LDS block
+    _run_case(2, 4, 8, 1024, itype, 2, var_B=var_B, var_C=var_C)
+    _run_case(2, 40, 16, 700, itype, 1, var_B=var_B, var_C=var_C, has_z=False)
+    _run_case(1, 6, 24, 300, itype, 1, var_B=var_B, var_C=var_C, has_bias=False)

@@ -125,3 +125,32 @@ def test_output_dtype_and_fp32_agreement():
                                 compute_dtype=f64)
     assert y32.dtype == torch.bfloat16
     assert torch.allclose(y32.float(), y64.float(), rtol=2e-2, atol=2e-2)
+
+
+def test_input_independent_B_C_matrices():
+    # B, C of shape (dim, dstate): brute force on a tiny case, and equality with the per-position form
+    # in which every channel is its own group and the matrix is repeated along batch and length
+    g = torch.Generator().manual_seed(5)
+    b, d, L, n = 2, 3, 9, 2
+    u, delta = torch.randn(b, d, L, generator=g, dtype=f64), torch.rand(b, d, L, generator=g, dtype=f64)
+    A = -torch.rand(d, n, generator=g, dtype=f64)
+    Bm, Cm = torch.randn(d, n, generator=g, dtype=f64), torch.randn(d, n, generator=g, dtype=f64)
+    Bv = torch.randn(b, 1, n, L, generator=g, dtype=f64)
+    y = selective_scan_oracle(u, delta, A, Bm, Cm, compute_dtype=f64)
+    expect = torch.zeros(b, d, L, dtype=f64)
+    for bi in range(b):
+        for di in range(d):
+            h = [0.0] * n
+            for t in range(L):
+                for k in range(n):
+                    h[k] = float(torch.exp(delta[bi, di, t] * A[di, k])) * h[k] + float(delta[bi, di, t] * Bm[di, k] * u[bi, di, t])
+                expect[bi, di, t] = sum(h[k] * float(Cm[di, k]) for k in range(n))
+    assert torch.allclose(y, expect, atol=1e-12)
+    rep = lambda m: m[None, :, :, None].expand(b, d, n, L).contiguous()
+    assert torch.allclose(y, selective_scan_oracle(u, delta, A, rep(Bm), rep(Cm), compute_dtype=f64), atol=1e-12)
+    # mixed: matrix B with per-position C and the reverse
+    y1 = selective_scan_oracle(u, delta, A, Bm, Bv, compute_dtype=f64)
+    assert torch.allclose(y1, selective_scan_oracle(u, delta, A, rep(Bm), Bv.expand(b, d, n, L).contiguous(),
+                                                    compute_dtype=f64), atol=1e-12)
+    y2 = selective_scan_oracle(u, delta, A, Bv, Cm, compute_dtype=f64)
+    assert torch.allclose(y2, selective_scan_oracle(u, delta, A, Bv, rep(Cm), compute_dtype=f64), atol=1e-12)
