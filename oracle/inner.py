@@ -15,7 +15,9 @@ from oracle.mamba1 import selective_scan_oracle
 
 def mamba_inner_oracle(xz, conv1d_weight, conv1d_bias, x_proj_weight, delta_proj_weight, out_proj_weight,
                        out_proj_bias, A, D=None, delta_bias=None, B_proj_bias=None, C_proj_bias=None,
-                       compute_dtype=torch.float32):
+                       compute_dtype=torch.float32, B=None, C=None):
+    """B / C given: input-independent (dim, dstate) matrices instead of the x_proj slices (:415-430);
+    x_proj_weight then only carries the rows of the slices that are still projected."""
     cd = compute_dtype
     batch, two_d, L = xz.shape
     d = two_d // 2
@@ -26,14 +28,20 @@ def mamba_inner_oracle(xz, conv1d_weight, conv1d_bias, x_proj_weight, delta_proj
                         groups=d)[..., :L])
     x_dbl = x.permute(0, 2, 1).reshape(batch * L, d) @ x_proj_weight.to(cd).t()           # (b l, R + 2N)
     delta = (delta_proj_weight.to(cd) @ x_dbl[:, :R].t()).reshape(d, batch, L).permute(1, 0, 2)
-    Bm = x_dbl[:, R:R + N]
-    Cm = x_dbl[:, R + N:R + 2 * N]
-    if B_proj_bias is not None:
-        Bm = Bm + B_proj_bias.to(cd)
-    if C_proj_bias is not None:
-        Cm = Cm + C_proj_bias.to(cd)
-    Bm = Bm.reshape(batch, L, N).permute(0, 2, 1)
-    Cm = Cm.reshape(batch, L, N).permute(0, 2, 1)
+    if B is None:
+        Bm = x_dbl[:, R:R + N]
+        if B_proj_bias is not None:
+            Bm = Bm + B_proj_bias.to(cd)
+        Bm = Bm.reshape(batch, L, N).permute(0, 2, 1)
+    else:
+        Bm = B.to(cd)
+    if C is None:
+        Cm = x_dbl[:, x_dbl.shape[1] - N:]
+        if C_proj_bias is not None:
+            Cm = Cm + C_proj_bias.to(cd)
+        Cm = Cm.reshape(batch, L, N).permute(0, 2, 1)
+    else:
+        Cm = C.to(cd)
     y = selective_scan_oracle(x, delta, A.to(cd), Bm, Cm, None if D is None else D.to(cd), z,
                               None if delta_bias is None else delta_bias.to(cd), True, compute_dtype=cd)
     out = y.permute(0, 2, 1) @ out_proj_weight.to(cd).t()

@@ -63,6 +63,40 @@ def test_mamba_inner_fn(L, with_bias):
             f"d{k}: max err {(got - ref).abs().max().item():.3e}, ref max {ref.abs().max().item():.3e}"
 
 
+@pytest.mark.parametrize("given", ["B", "C", "BC"])
+def test_mamba_inner_fn_given_B_C(given):
+    """B and / or C passed in as input-independent (dim, dstate) matrices
+    (selective_scan_interface.py:386 B=, C=; is_variable_B / is_variable_C false)."""
+    from mamba_amd.ops.selective_scan_interface import mamba_inner_fn
+    g = torch.Generator().manual_seed(1)
+    batch, dim, dstate, dt_rank, d_model, L = 2, 256, 8, 16, 128, 300
+    p = _params(batch, dim, L, dstate, dt_rank, d_model, g, False)
+    nproj = dt_rank + dstate * (("B" not in given) + ("C" not in given))
+    p["x_proj_weight"] = p["x_proj_weight"][:nproj].contiguous()
+    p["B"] = torch.randn(dim, dstate, generator=g) if "B" in given else None
+    p["C"] = torch.randn(dim, dstate, generator=g) if "C" in given else None
+    ref_in = {k: (v.clone().requires_grad_() if v is not None else None) for k, v in p.items()}
+    gpu_in = {k: (v.cuda().requires_grad_() if v is not None else None) for k, v in p.items()}
+    order = ["xz", "conv1d_weight", "conv1d_bias", "x_proj_weight", "delta_proj_weight", "out_proj_weight",
+             "out_proj_bias", "A"]
+    out_ref = mamba_inner_oracle(*[ref_in[k] for k in order], D=ref_in["D"], delta_bias=ref_in["delta_bias"],
+                                 B=ref_in["B"], C=ref_in["C"])
+    out = mamba_inner_fn(*[gpu_in[k] for k in order], gpu_in["B"], gpu_in["C"], gpu_in["D"],
+                         delta_bias=gpu_in["delta_bias"], delta_softplus=True)
+    scale = float(out_ref.abs().max())
+    assert torch.allclose(out.cpu(), out_ref, rtol=6e-4, atol=2e-3 * max(1.0, scale))
+    dout = torch.randn(out_ref.shape, generator=g)
+    out_ref.backward(dout)
+    out.backward(dout.cuda())
+    for k, v in ref_in.items():
+        if v is None:
+            continue
+        got, ref = gpu_in[k].grad.cpu(), v.grad
+        s = max(1.0, float(ref.abs().max()))
+        assert torch.allclose(got, ref, rtol=5e-3, atol=5e-3 * s), \
+            f"d{k}: max err {(got - ref).abs().max().item():.3e}, ref max {ref.abs().max().item():.3e}"
+
+
 def test_install_as_mamba_ssm_ops():
     import importlib
     import mamba_amd
