@@ -57,8 +57,12 @@ constexpr int UNR = SSU_UNR;  // row passes per wave
 // TS: state dtype.  TX: dtype of x, z, out.  TB: dtype of B, C.  TD: dtype of dt.
 // A, D and dt_bias are fp32.  lpr = lanes per row (power of two, dstate <= 4 * lpr).
 // Addressing: the (batch, head) part of every address is wave-uniform 64-bit scalar math; the
-// per-lane part is a 32-bit element offset that advances by a uniform step per row pass, so the
-// vector ALU does no 64-bit multiplies (they would cost more than the streaming itself).
+// per-lane part is a 32-bit element offset, so the vector ALU does no 64-bit multiplies (they would
+// cost more than the streaming itself).
+// Every global load of the wave sits in one branch-free block ahead of the first use: rows and
+// states past the end are read from clamped (valid) addresses and masked afterwards, and absent
+// optional operands read a stand-in address with a zero weight.  A load under a branch would make
+// the compiler wait for all earlier loads at that point, which serialises the memory round trips.
 template <typename TS, typename TX, typename TB, typename TD, bool VEC>
 __global__ __launch_bounds__(256) void state_update_kernel(const MambaStepParams p, int lpr_log2) {
   const int lane = threadIdx.x & 63;
@@ -84,111 +88,115 @@ __global__ __launch_bounds__(256) void state_update_kernel(const MambaStepParams
   const int N = p.dstate;
   const int n0 = sub * 4;
   const int nlane = min(max(N - n0, 0), 4);
+  const int n0c = VEC ? min(n0, N - 4) : n0;  // clamped start of this lane's 4 states (VEC: N % 4 == 0)
   const int row0 = p_begin + rsel;
   // wave-uniform bases
   TS *state = static_cast<TS *>(p.state) + sb * p.state_bs + h * p.state_hs;
   const TX *xp = static_cast<const TX *>(p.x) + b * p.x_bs + h * p.x_hs;
-  const TX *zp = p.z ? static_cast<const TX *>(p.z) + b * p.z_bs + h * p.z_hs : nullptr;
   const TD *dtp = static_cast<const TD *>(p.dt) + b * p.dt_bs + h * p.dt_hs;
-  const float *dtb = p.dt_bias ? static_cast<const float *>(p.dt_bias) + h * p.dt_bias_hs : nullptr;
-  const float *Dp = p.D ? static_cast<const float *>(p.D) + h * p.D_hs : nullptr;
   const float *Ap = static_cast<const float *>(p.A) + h * p.A_hs;
   const TB *Bp = static_cast<const TB *>(p.B) + b * p.B_bs + g * p.B_gs;
   const TB *Cp = static_cast<const TB *>(p.C) + b * p.C_bs + g * p.C_gs;
+  // optional operands: a stand-in pointer of the right type, stride 0 and weight 0 when absent
+  const bool has_z = p.z != nullptr, has_D = p.D != nullptr, has_dtb = p.dt_bias != nullptr;
+  const TX *zp = has_z ? static_cast<const TX *>(p.z) + b * p.z_bs + h * p.z_hs : xp;
+  const float *dtb = has_dtb ? static_cast<const float *>(p.dt_bias) + h * p.dt_bias_hs : Ap;
+  const float *Dp = has_D ? static_cast<const float *>(p.D) + h * p.D_hs : Ap;
   // 32-bit strides (the host checks that the per-head extents fit)
   const int s_ps = (int)p.state_ps, s_ns = (int)p.state_ns, x_ps = (int)p.x_ps, dt_ps = (int)p.dt_ps;
-  const int dtb_ps = (int)p.dt_bias_ps, A_ps = (int)p.A_ps, A_ns = (int)p.A_ns;
+  const int dtb_ps = has_dtb ? (int)p.dt_bias_ps : 0, A_ps = (int)p.A_ps, A_ns = (int)p.A_ns;
   const int B_ns = (int)p.B_ns, C_ns = (int)p.C_ns;
+  const int z_ps = has_z ? (int)p.z_ps : 0, D_ps = has_D ? (int)p.D_ps : 0, out_ps = (int)p.out_ps;
+  const bool A_per_row = A_ps != 0;
+  const bool dt_per_row = dt_ps != 0 || dtb_ps != 0;
 
-  // 1. the long-latency traffic first
-  float s[UNR][4], xs[UNR], dts[UNR];
-  int nv[UNR];
-  int soff = row0 * s_ps + n0 * s_ns, xoff = row0 * x_ps, dtoff = row0 * dt_ps, dtboff = row0 * dtb_ps;
+  // 1. all loads
+  float s[UNR][4], xs[UNR], dts[UNR], dtbs[UNR], zs[UNR], Ds[UNR], Arow[UNR][4];
+  bool live[UNR];
 #pragma unroll
   for (int k = 0; k < UNR; ++k) {
     const int row = row0 + k * rpp;
-    nv[k] = row < p.dim ? nlane : 0;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) s[k][i] = 0.f;
-    xs[k] = 0.f;
-    dts[k] = 0.f;
-    if (nv[k] > 0) {
-      ld_state4<TS, VEC>(state + soff, s_ns, nv[k], s[k]);
-      xs[k] = ld1<TX>(xp + xoff);
-      dts[k] = ld1<TD>(dtp + dtoff);
-      if (dtb) dts[k] += dtb[dtboff];
+    live[k] = row < p.dim && nlane > 0;
+    const int rc = min(row, p.dim - 1);
+    if constexpr (VEC) {
+      ld_state4<TS, true>(state + rc * s_ps + n0c * s_ns, s_ns, 4, s[k]);
+    } else {
+      ld_state4<TS, false>(state + rc * s_ps + n0 * s_ns, s_ns, live[k] ? nlane : 0, s[k]);
     }
-    soff += rpp * s_ps;
-    xoff += rpp * x_ps;
-    dtoff += rpp * dt_ps;
-    dtboff += rpp * dtb_ps;
+    xs[k] = ld1<TX>(xp + rc * x_ps);
+    dts[k] = ld1<TD>(dtp + rc * dt_ps);
+    dtbs[k] = dtb[rc * dtb_ps];
+    zs[k] = ld1<TX>(zp + rc * z_ps);
+    Ds[k] = Dp[rc * D_ps];
   }
-  // 2. operands shared by the rows of this wave
   float Bv[4], Cv[4], Av[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const bool ok = i < nlane;
-    Bv[i] = ok ? ld1<TB>(Bp + (n0 + i) * B_ns) : 0.f;
-    Cv[i] = ok ? ld1<TB>(Cp + (n0 + i) * C_ns) : 0.f;
-    Av[i] = ok ? Ap[(n0 + i) * A_ns] * kLog2e : 0.f;
+    const int nc = min(n0 + i, N - 1);
+    Bv[i] = ld1<TB>(Bp + nc * B_ns);
+    Cv[i] = ld1<TB>(Cp + nc * C_ns);
+    Av[i] = Ap[nc * A_ns];
   }
-  const bool A_per_row = A_ps != 0;
-  const bool dt_per_row = dt_ps != 0 || (dtb && dtb_ps != 0);
-  // per-head step size and decay, used as they are when dt and A do not depend on the row
-  float dt_head = dts[0];
+  if (A_per_row) {  // uniform; the block holds loads only
+#pragma unroll
+    for (int k = 0; k < UNR; ++k) {
+      const int rc = min(row0 + k * rpp, p.dim - 1);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) Arow[k][i] = Ap[rc * A_ps + min(n0 + i, N - 1) * A_ns];
+    }
+  }
+  // 2. masks and per-head values
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const bool ok = i < nlane;
+    Bv[i] = ok ? Bv[i] : 0.f;
+    Cv[i] = ok ? Cv[i] : 0.f;
+    Av[i] *= kLog2e;
+  }
+  const float w_dtb = has_dtb ? 1.f : 0.f, w_D = has_D ? 1.f : 0.f;
+  const bool per_row = A_per_row || dt_per_row;
+  float dt_head = __builtin_fmaf(w_dtb, dtbs[0], dts[0]);
   if (p.dt_softplus) dt_head = softplus_f(dt_head);
   float dA_head[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) dA_head[i] = fast_exp2(Av[i] * dt_head);
-  const bool per_row = A_per_row || dt_per_row;
 
   float outs[UNR];
-  soff = row0 * s_ps + n0 * s_ns;
-  int aoff = row0 * A_ps + n0 * A_ns;
 #pragma unroll
   for (int k = 0; k < UNR; ++k) {
-    float out = 0.f;
-    if (nv[k] > 0) {
-      float dt = dt_head;
-      float dA[4];
-      if (per_row) {
-        dt = dts[k];
-        if (p.dt_softplus) dt = softplus_f(dt);
+    float dt = dt_head;
+    float dA[4];
+    if (per_row) {
+      dt = __builtin_fmaf(w_dtb, dtbs[k], dts[k]);
+      if (p.dt_softplus) dt = softplus_f(dt);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          float a = Av[i];
-          if (A_per_row && i < nv[k]) a = Ap[aoff + i * A_ns] * kLog2e;
-          dA[i] = fast_exp2(a * dt);
-        }
-      } else {
+      for (int i = 0; i < 4; ++i) dA[i] = fast_exp2((A_per_row ? Arow[k][i] * kLog2e : Av[i]) * dt);
+    } else {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) dA[i] = dA_head[i];
-      }
-      const float dtx = dt * xs[k];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        s[k][i] = __builtin_fmaf(s[k][i], dA[i], Bv[i] * dtx);
-        out = __builtin_fmaf(s[k][i], Cv[i], out);
-      }
-      st_state4<TS, VEC>(state + soff, s_ns, nv[k], s[k]);
+      for (int i = 0; i < 4; ++i) dA[i] = dA_head[i];
     }
-    outs[k] = out;
-    soff += rpp * s_ps;
-    aoff += rpp * A_ps;
+    const float dtx = dt * xs[k];
+    float out = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      s[k][i] = __builtin_fmaf(s[k][i], dA[i], Bv[i] * dtx);
+      out = __builtin_fmaf(s[k][i], Cv[i], out);
+    }
+    outs[k] = live[k] ? out : 0.f;
+    if (live[k]) {
+      const int row = row0 + k * rpp;
+      st_state4<TS, VEC>(state + row * s_ps + n0 * s_ns, s_ns, nlane, s[k]);
+    }
   }
   // 3. sum over the lanes of each row, then the skip connection and the gate
-  const int z_ps = (int)p.z_ps, D_ps = (int)p.D_ps, out_ps = (int)p.out_ps;
 #pragma unroll
   for (int k = 0; k < UNR; ++k) {
     const int row = row0 + k * rpp;
     float out = outs[k];
     for (int off = lpr >> 1; off >= 1; off >>= 1) out += __shfl_xor(out, off, 64);
     if (row < p.dim && sub == 0) {
-      if (Dp) out = __builtin_fmaf(xs[k], Dp[row * D_ps], out);
-      if (zp) {
-        const float z = ld1<TX>(zp + row * z_ps);
-        out *= z * sigmoid_f(z);
-      }
+      out = __builtin_fmaf(xs[k] * w_D, Ds[k], out);
+      if (has_z) out *= zs[k] * sigmoid_f(zs[k]);
       st1<TX>(outp + row * out_ps, out);
     }
   }
