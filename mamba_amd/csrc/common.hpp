@@ -90,6 +90,8 @@ template <> DEVI void st8<f16_t>(f16_t *p, const float (&v)[8]) {
 // loaded from T): 4 registers for 16-bit types, 8 for fp32.
 template <typename T> struct Pack8 {
   u32x4 w;
+  DEVI void load(const T *p) { w = *reinterpret_cast<const u32x4 *>(p); }  // 16-byte aligned
+  DEVI void zero() { w = u32x4{0, 0, 0, 0}; }
   DEVI void pack(const float (&v)[8]) {
     if constexpr (DT<T>::id == MAMBA_BF16) {
       w = u32x4{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7])};
@@ -109,6 +111,15 @@ template <typename T> struct Pack8 {
 };
 template <> struct Pack8<float> {
   float v[8];
+  DEVI void load(const float *p) {
+    const f32x4 a = *reinterpret_cast<const f32x4 *>(p), b = *reinterpret_cast<const f32x4 *>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  }
+  DEVI void zero() {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = 0.f;
+  }
   DEVI void pack(const float (&x)[8]) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) v[i] = x[i];

@@ -33,17 +33,58 @@ template <typename T, bool VEC, int NTHREADS, int BC>
 DEVI void stage_bc(float *Bs, float *Cs, const T *Bg, int64_t B_ns, const T *Cg, int64_t C_ns, int n0, int N, int t0,
                    int L, int tid) {
   constexpr int FIRST = (BC & 1) ? NB16 * 64 : 0, LAST = (BC & 2) ? NB16 * 64 : 2 * NB16 * 64;
-  for (int unit = FIRST + tid; unit < LAST; unit += NTHREADS) {
-    const int which = unit >> 10, n = (unit >> 6) & 15, j = unit & 63;
-    const int t = t0 + KI * j;
-    const T *src = (which ? Cg + (int64_t)(n0 + n) * C_ns : Bg + (int64_t)(n0 + n) * B_ns) + t;
-    int nvalid = (n0 + n < N) ? min(max(L - t, 0), KI) : 0;
+  if constexpr (BC == 3) {
+    return;  // nothing is staged
+  } else if constexpr (VEC) {
+    // all loads first, from clamped (valid) addresses, then the masked LDS stores: a load under
+    // a branch, or converted right away, would make every load wait for the one before
+    constexpr int UNITS = (LAST - FIRST) / NTHREADS;
+    static_assert(UNITS * NTHREADS == LAST - FIRST, "whole units per thread");
+    Pack8<T> raw[UNITS];
+#pragma unroll
+    for (int q = 0; q < UNITS; ++q) {
+      const int unit = FIRST + tid + q * NTHREADS;
+      const int which = unit >> 10, n = min(n0 + ((unit >> 6) & 15), N - 1), t = min(t0 + KI * (unit & 63), L - KI);
+      raw[q].load((which ? Cg + (int64_t)n * C_ns : Bg + (int64_t)n * B_ns) + t);
+    }
+#pragma unroll
+    for (int q = 0; q < UNITS; ++q) {
+      const int unit = FIRST + tid + q * NTHREADS;
+      const int which = unit >> 10, n = (unit >> 6) & 15, j = unit & 63;
+      float v[8];
+      raw[q].unpack(v);
+      const bool ok = n0 + n < N && t0 + KI * j < L;
+      float *dst = (which ? Cs : Bs) + n * TILE + j * 4;
+      const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+      const f32x4 lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
+      *reinterpret_cast<f32x4 *>(dst) = ok ? lo : zero;
+      *reinterpret_cast<f32x4 *>(dst + 256) = ok ? hi : zero;
+    }
+  } else {
+    for (int unit = FIRST + tid; unit < LAST; unit += NTHREADS) {
+      const int which = unit >> 10, n = (unit >> 6) & 15, j = unit & 63;
+      const int t = t0 + KI * j;
+      const T *src = (which ? Cg + (int64_t)(n0 + n) * C_ns : Bg + (int64_t)(n0 + n) * B_ns) + t;
+      int nvalid = (n0 + n < N) ? min(max(L - t, 0), KI) : 0;
+      float v[8];
+      ld8_guard<T, false>(src, nvalid, 0.f, v);
+      float *dst = (which ? Cs : Bs) + n * TILE + j * 4;
+      f32x4 lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
+      *reinterpret_cast<f32x4 *>(dst) = lo;
+      *reinterpret_cast<f32x4 *>(dst + 256) = hi;
+    }
+  }
+}
+
+// The 8 items of one (batch, channel) row owned by this lane, as stored: VEC reads 16 bytes from a
+// clamped position (the caller masks lanes past the end), else element by element.
+template <typename T, bool VEC> DEVI void load_items(Pack8<T> &k, const T *row, int tl, int L, int nvalid) {
+  if constexpr (VEC) {
+    k.load(row + min(tl, L - KI));
+  } else {
     float v[8];
-    ld8_guard<T, VEC>(src, nvalid, 0.f, v);
-    float *dst = (which ? Cs : Bs) + n * TILE + j * 4;
-    f32x4 lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
-    *reinterpret_cast<f32x4 *>(dst) = lo;
-    *reinterpret_cast<f32x4 *>(dst + 256) = hi;
+    ld8_guard<T, false>(row + tl, nvalid, 0.f, v);
+    k.pack(v);
   }
 }
 
@@ -113,15 +154,21 @@ __global__ __launch_bounds__(NW * 64) void scan_fwd_kernel(const MambaScanParams
       const int d = dbase + r;
       const bool valid = d < dend;
       float u[8], dl[8], du[8], y[8];
+      Pack8<T> ku, kd, kz;  // raw rows: every load is issued before the first conversion
+      kz.zero();
       if (valid) {
-        ld8_guard<T, VEC>((const T *)p.u + b * p.u_bs + d * p.u_ds + tl, nvalid, 0.f, u);
-        ld8_guard<T, VEC>((const T *)p.delta + b * p.delta_bs + d * p.delta_ds + tl, nvalid, 0.f, dl);
+        load_items<T, VEC>(ku, (const T *)p.u + b * p.u_bs + d * p.u_ds, tl, L, nvalid);
+        load_items<T, VEC>(kd, (const T *)p.delta + b * p.delta_bs + d * p.delta_ds, tl, L, nvalid);
+        if (p.z) load_items<T, VEC>(kz, (const T *)p.z + b * p.z_bs + d * p.z_ds, tl, L, nvalid);
         const float bias = p.delta_bias ? ((const float *)p.delta_bias)[d] : 0.f;
+        ku.unpack(u);
+        kd.unpack(dl);
 #pragma unroll
         for (int i = 0; i < KI; ++i) {
           float x = dl[i] + bias;
           if (p.delta_softplus) x = softplus_f(x);
           dl[i] = (i < nvalid) ? x : 0.f;
+          u[i] = (i < nvalid) ? u[i] : 0.f;
           du[i] = dl[i] * u[i];
           y[i] = 0.f;
         }
@@ -178,7 +225,7 @@ __global__ __launch_bounds__(NW * 64) void scan_fwd_kernel(const MambaScanParams
         }
         if (p.z) {
           float z[8];
-          ld8_guard<T, VEC>((const T *)p.z + b * p.z_bs + d * p.z_ds + tl, nvalid, 0.f, z);
+          kz.unpack(z);
 #pragma unroll
           for (int i = 0; i < KI; ++i) y[i] *= z[i] * sigmoid_f(z[i]);
         }
@@ -244,6 +291,24 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
     dbacc[wave * R + lane] = 0.f;
   }
 
+  // The rows of the next (tile, channel) are fetched while the current one is computed.
+  struct Rows {
+    Pack8<T> u, delta, dout, z;
+  };
+  auto fetch_rows = [&](Rows &k, int tile, int r) {
+    const int d = dbase + r, tl = tile * TILE + lane * KI;
+    const int nvalid = min(max(L - tl, 0), KI);
+    k.z.zero();
+    if (d < dend) {
+      load_items<T, VEC>(k.u, (const T *)p.u + b * p.u_bs + d * p.u_ds, tl, L, nvalid);
+      load_items<T, VEC>(k.delta, (const T *)p.delta + b * p.delta_bs + d * p.delta_ds, tl, L, nvalid);
+      load_items<T, VEC>(k.dout, (const T *)p.dout + b * p.dout_bs + d * p.dout_ds, tl, L, nvalid);
+      if (has_z) load_items<T, VEC>(k.z, (const T *)p.z + b * p.z_bs + d * p.z_ds, tl, L, nvalid);
+    }
+  };
+  Rows nxt;
+  fetch_rows(nxt, ntiles - 1, 0);
+
   for (int tile = ntiles - 1; tile >= 0; --tile) {
     const int t0 = tile * TILE, tl = t0 + lane * KI;
     const int nvalid = min(max(L - tl, 0), KI);
@@ -253,20 +318,26 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
       const int row = wave * R + r;
       float u[8], dl[8], du[8], dy[8], acc[8], dd[8], y[8];
       // raw delta, z and dout stay in registers in their storage format for the epilogue
-      Pack8<T> draw_k, z_k, dout_k;
+      const Rows cur = nxt;
+      Pack8<T> draw_k = cur.delta, z_k = cur.z, dout_k = cur.dout;
+      if (r + 1 < R) fetch_rows(nxt, tile, r + 1);
+      else if (tile > 0) fetch_rows(nxt, tile - 1, 0);
       float Dd = 0.f;
       if (valid) {
         Dd = p.D ? ((const float *)p.D)[d] : 0.f;
-        ld8_guard<T, VEC>((const T *)p.u + b * p.u_bs + d * p.u_ds + tl, nvalid, 0.f, u);
-        ld8_guard<T, VEC>((const T *)p.delta + b * p.delta_bs + d * p.delta_ds + tl, nvalid, 0.f, dl);
-        ld8_guard<T, VEC>((const T *)p.dout + b * p.dout_bs + d * p.dout_ds + tl, nvalid, 0.f, dy);
-        draw_k.pack(dl);
-        dout_k.pack(dy);
+        const Pack8<T> u_k = cur.u;
         const float bias = p.delta_bias ? ((const float *)p.delta_bias)[d] : 0.f;
+        u_k.unpack(u);
+        draw_k.unpack(dl);
+        dout_k.unpack(dy);
+#pragma unroll
+        for (int i = 0; i < KI; ++i) {  // lanes past the end read a clamped position: mask them
+          u[i] = (i < nvalid) ? u[i] : 0.f;
+          dy[i] = (i < nvalid) ? dy[i] : 0.f;
+        }
         if (has_z) {
           float z[8];
-          ld8_guard<T, VEC>((const T *)p.z + b * p.z_bs + d * p.z_ds + tl, nvalid, 0.f, z);
-          z_k.pack(z);
+          z_k.unpack(z);
 #pragma unroll
           for (int i = 0; i < KI; ++i) dy[i] *= z[i] * sigmoid_f(z[i]);
         }
