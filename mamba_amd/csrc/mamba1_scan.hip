@@ -294,12 +294,15 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
   // The rows of the next (tile, channel) are fetched while the current one is computed.
   struct Rows {
     Pack8<T> u, delta, dout, z;
+    float ck;  // checkpointed state n = lane entering the tile (when the padded state count fits a wave)
   };
   auto fetch_rows = [&](Rows &k, int tile, int r) {
     const int d = dbase + r, tl = tile * TILE + lane * KI;
     const int nvalid = min(max(L - tl, 0), KI);
     k.z.zero();
+    k.ck = 0.f;
     if (d < dend) {
+      if (NP <= 64 && tile > 0 && lane < N) k.ck = p.ckpt[(((int64_t)b * p.dim + d) * ntiles + tile - 1) * N + lane];
       load_items<T, VEC>(k.u, (const T *)p.u + b * p.u_bs + d * p.u_ds, tl, L, nvalid);
       load_items<T, VEC>(k.delta, (const T *)p.delta + b * p.delta_bs + d * p.delta_ds, tl, L, nvalid);
       load_items<T, VEC>(k.dout, (const T *)p.dout + b * p.dout_bs + d * p.dout_ds, tl, L, nvalid);
@@ -352,10 +355,14 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
           y[i] = 0.f;
         }
         // state entering this tile
-        for (int n = lane; n < NP; n += 64) {
-          float v = 0.f;
-          if (tile > 0 && n < N) v = p.ckpt[(((int64_t)b * p.dim + d) * ntiles + tile - 1) * N + n];
-          hcar[row * NP + n] = v;
+        if (NP <= 64) {
+          if (lane < NP) hcar[row * NP + lane] = cur.ck;
+        } else {
+          for (int n = lane; n < NP; n += 64) {
+            float v = 0.f;
+            if (tile > 0 && n < N) v = p.ckpt[(((int64_t)b * p.dim + d) * ntiles + tile - 1) * N + n];
+            hcar[row * NP + n] = v;
+          }
         }
       }
       for (int nb = 0; nb < NBLK; ++nb) {
