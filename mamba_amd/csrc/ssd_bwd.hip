@@ -222,14 +222,10 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dst
   const T *ga = static_cast<const T *>(gv.ptr) + gb + (int64_t)t0 * gv.ls + pt * GB;
   const T *Ca = static_cast<const T *>(p.C) + Cb + (int64_t)t0 * p.C_ls + nt * GB;
   const bool va = rows_aligned16(ga, gv.ls), vb = rows_aligned16(Ca, p.C_ls);
-  block_gemm_staged<SPLIT>(
+  block_gemm_pipe<SPLIT>(
       acc, lds, 0, qlim,
-      [&](int k0) {
-        if (tid < 128) stage_rc<SPLIT, T>(lds.ah, lds.al, ga, gv.ls, P - pt * GB, k0, qlim, nullptr, nullptr, va, tid);
-      },
-      [&](int k0) {
-        if (tid >= 128) stage_rc<SPLIT, T>(lds.bh, lds.bl, Ca, p.C_ls, N - nt * GB, k0, qlim, rs, nullptr, vb, tid - 128);
-      },
+      RcStager<SPLIT, T>(lds.ah, lds.al, ga, gv.ls, P - pt * GB, qlim, nullptr, nullptr, va, tid, tid < 128),
+      RcStager<SPLIT, T>(lds.bh, lds.bl, Ca, p.C_ls, N - nt * GB, qlim, rs, nullptr, vb, tid - 128, tid >= 128),
       tid);
   float *ds = p.dstates + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
   acc_foreach(acc, tid, [&](int m, int n, float v) {
@@ -327,10 +323,10 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
     const T *Ba = static_cast<const T *>(p.B) + Bb + (int64_t)(t0 + st * GB) * p.B_ls;
     const float *dSa = dS + (int64_t)pt * GB * N;
     const bool va = rows_aligned16(Ba, p.B_ls), vb = rows_aligned16(dSa, N);
-    block_gemm_staged<SPLIT>(
+    block_gemm_pipe<SPLIT>(
         acc1, lds, 0, N,
-        [&](int k0) { stage_kc<SPLIT, T>(lds.ah, lds.al, Ba, p.B_ls, qlim - st * GB, k0, N, nullptr, nullptr, va, tid); },
-        [&](int k0) { stage_kc<SPLIT, float>(lds.bh, lds.bl, dSa, N, P - pt * GB, k0, N, nullptr, nullptr, vb, tid); },
+        KcStager<SPLIT, T>(lds.ah, lds.al, Ba, p.B_ls, qlim - st * GB, N, nullptr, nullptr, va, tid),
+        KcStager<SPLIT, float>(lds.bh, lds.bl, dSa, N, P - pt * GB, N, nullptr, nullptr, vb, tid),
         tid);
   }
   {
@@ -343,17 +339,13 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
     const bool vb = rows_aligned16(ga, gv.ls);
     const float *CBa = CB + st * GB;  // A rows s are contiguous in the source, k = l strides by Q
     const bool va = rows_aligned16(CBa, Q);
-    block_gemm_staged<SPLIT>(
+    block_gemm_pipe<SPLIT>(
         acc2, lds, st * GB, qlim,
-        [&](int k0) {
-          if (k0 < (st + 1) * GB)  // diagonal block: causal mask and the exact decay
-            stage_tile<SPLIT, false>(lds.ah, lds.al, [&](int r, int k) { return fa(r, k0 + k); }, tid);
-          else if (tid >= 128)
-            stage_rc<SPLIT, float>(lds.ah, lds.al, CBa, Q, qlim - st * GB, k0, qlim, kdec, rdec, va, tid - 128);
-        },
-        [&](int k0) {
-          if (tid < 128) stage_rc<SPLIT, T>(lds.bh, lds.bl, ga, gv.ls, P - pt * GB, k0, qlim, nullptr, nullptr, vb, tid);
-        },
+        // diagonal block: causal mask and the exact decay; below it CB^T with the rank-1 decays
+        diag_stager<SPLIT>(lds.ah, lds.al, fa, (st + 1) * GB, tid,
+                           RcStager<SPLIT, float>(lds.ah, lds.al, CBa, Q, qlim - st * GB, qlim, kdec, rdec, va, tid - 128,
+                                                  tid >= 128)),
+        RcStager<SPLIT, T>(lds.bh, lds.bl, ga, gv.ls, P - pt * GB, qlim, nullptr, nullptr, vb, tid, tid < 128),
         tid);
   }
   // Epilogue with rows in threads: thread t owns position s = tile row t / 4 and 16 consecutive p.
@@ -480,12 +472,10 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dBC
     auto run = [&](GemmAcc &acc, const T *a_base, int64_t a_ls, const float *w, const float *S) {
       const T *aa = a_base + (int64_t)(t0 + st * GB) * a_ls;
       const bool va = rows_aligned16(aa, a_ls);
-      block_gemm_staged<SPLIT>(
+      block_gemm_pipe<SPLIT>(
           acc, lds, 0, P,
-          [&](int k0) { stage_kc<SPLIT, T>(lds.ah, lds.al, aa, a_ls, qlim - st * GB, k0, P, nullptr, w, va, tid); },
-          [&](int k0) {
-            if (tid < 128) stage_rc<SPLIT, float>(lds.bh, lds.bl, S, N, N - nt * GB, k0, P, nullptr, nullptr, vs, tid);
-          },
+          KcStager<SPLIT, T>(lds.ah, lds.al, aa, a_ls, qlim - st * GB, P, nullptr, w, va, tid),
+          RcStager<SPLIT, float>(lds.bh, lds.bl, S, N, N - nt * GB, P, nullptr, nullptr, vs, tid, tid < 128),
           tid);
     };
     run(accB, static_cast<const T *>(p.x) + xb, p.x_ls, wB[par], dS);
@@ -580,10 +570,10 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dcb
     const T *ga = static_cast<const T *>(gv.ptr) + gb + (int64_t)(t0 + lt * GB) * gv.ls;
     const T *xa = static_cast<const T *>(p.x) + xb + (int64_t)(t0 + st * GB) * p.x_ls;
     const bool va = rows_aligned16(ga, gv.ls), vb = rows_aligned16(xa, p.x_ls);
-    block_gemm_staged<SPLIT>(
+    block_gemm_pipe<SPLIT>(
         acc, lds, 0, P,
-        [&](int k0) { stage_kc<SPLIT, T>(lds.ah, lds.al, ga, gv.ls, qlim - lt * GB, k0, P, nullptr, nullptr, va, tid); },
-        [&](int k0) { stage_kc<SPLIT, T>(lds.bh, lds.bl, xa, p.x_ls, qlim - st * GB, k0, P, nullptr, nullptr, vb, tid); },
+        KcStager<SPLIT, T>(lds.ah, lds.al, ga, gv.ls, qlim - lt * GB, P, nullptr, nullptr, va, tid),
+        KcStager<SPLIT, T>(lds.bh, lds.bl, xa, p.x_ls, qlim - st * GB, P, nullptr, nullptr, vb, tid),
         tid);
     // d = this head's dCB term (added to sum); w = d * CB, whose row / column sums go to ddA
     float *dda = chunk_row(p.ddA_cumsum, p, b, h, c);
@@ -651,12 +641,10 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bmm_chu
     const T *Ba = static_cast<const T *>(p.B) + Bb + (int64_t)t0 * p.B_ls + nt * GB;
     const bool va = rows_aligned16(da, Q), vb = rows_aligned16(Ba, p.B_ls);
     const int kend = min((mt + 1) * GB, qlim);
-    block_gemm_staged<SPLIT>(
+    block_gemm_pipe<SPLIT>(
         acc, lds, 0, kend,
-        [&](int k0) { stage_kc<SPLIT, float>(lds.ah, lds.al, da, Q, qlim - mt * GB, k0, kend, nullptr, nullptr, va, tid); },
-        [&](int k0) {
-          if (tid < 128) stage_rc<SPLIT, T>(lds.bh, lds.bl, Ba, p.B_ls, N - nt * GB, k0, kend, nullptr, nullptr, vb, tid);
-        },
+        KcStager<SPLIT, float>(lds.ah, lds.al, da, Q, qlim - mt * GB, kend, nullptr, nullptr, va, tid),
+        RcStager<SPLIT, T>(lds.bh, lds.bl, Ba, p.B_ls, N - nt * GB, kend, nullptr, nullptr, vb, tid, tid < 128),
         tid);
     acc_foreach(acc, tid, [&](int m, int n, float v) {
       const int l = mt * GB + m, nn = nt * GB + n;
@@ -671,15 +659,10 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bmm_chu
     const float *da = dCB + mt * GB;
     const T *Ca = static_cast<const T *>(p.C) + Cb + (int64_t)t0 * p.C_ls + nt * GB;
     const bool va = rows_aligned16(da, Q), vb = rows_aligned16(Ca, p.C_ls);
-    block_gemm_staged<SPLIT>(
+    block_gemm_pipe<SPLIT>(
         acc, lds, mt * GB, qlim,
-        [&](int k0) {
-          if (tid < 128) stage_rc<SPLIT, float>(lds.ah, lds.al, da, Q, qlim - mt * GB, k0, qlim, nullptr, nullptr, va, tid);
-        },
-        [&](int k0) {
-          if (tid >= 128)
-            stage_rc<SPLIT, T>(lds.bh, lds.bl, Ca, p.C_ls, N - nt * GB, k0, qlim, nullptr, nullptr, vb, tid - 128);
-        },
+        RcStager<SPLIT, float>(lds.ah, lds.al, da, Q, qlim - mt * GB, qlim, nullptr, nullptr, va, tid, tid < 128),
+        RcStager<SPLIT, T>(lds.bh, lds.bl, Ca, p.C_ls, N - nt * GB, qlim, nullptr, nullptr, vb, tid - 128, tid >= 128),
         tid);
     acc_foreach(acc, tid, [&](int m, int n, float v) {
       const int s = mt * GB + m, nn = nt * GB + n;

@@ -64,29 +64,44 @@ template <bool SPLIT> DEVI void put8(uint16_t *hi, uint16_t *lo, int off, const 
   }
 }
 
-// Vectorised staging of a k-contiguous source: element (r, k) at base[r * rstride + k].  All 256
-// threads take part (8 consecutive k each).  rows_valid / k_valid bound the source; kscale
-// (indexed by absolute k) and rscale (by tile row) are optional multipliers.  `vec` promises
-// 16-byte aligned rows (base and rstride), else every element is loaded on its own.
-template <bool SPLIT, typename S>
-DEVI void stage_kc(uint16_t *hi, uint16_t *lo, const S *base, int64_t rstride, int rows_valid, int k0, int k_valid,
-                   const float *kscale, const float *rscale, bool vec, int tid) {
-  constexpr int KG = GK / 8;  // 8-element groups per row
+// ---- staging split into a fetch (global -> registers) and a commit (registers -> LDS) half, so
+// that the loads of the next k step are in flight while the current one is multiplied.
+// Both stagers take one task per thread with the 32-wide k step.
+static_assert(GK == 32, "one staging task per thread");
+
+// k-contiguous source: element (r, k) at base[r * rstride + k]; thread t takes row t / 4, 8 k values.
+template <bool SPLIT, typename S> struct KcStager {
+  uint16_t *hi, *lo;
+  const S *base;
+  int64_t rstride;
+  int rows_valid, k_valid;
+  const float *kscale, *rscale;  // optional multipliers, by absolute k / by tile row
+  bool vec;                      // rows are 16-byte aligned
+  int t;
+  Pack8<S> q;
+  DEVI KcStager(uint16_t *hi_, uint16_t *lo_, const S *base_, int64_t rstride_, int rows_valid_, int k_valid_,
+                const float *kscale_, const float *rscale_, bool vec_, int t_)
+      : hi(hi_), lo(lo_), base(base_), rstride(rstride_), rows_valid(rows_valid_), k_valid(k_valid_), kscale(kscale_),
+        rscale(rscale_), vec(vec_), t(t_) {}
+  DEVI void fetch(int k0) {
+    const int r = t >> 2, k = k0 + (t & 3) * 8;
+    q.zero();
+    if (r < rows_valid && k < k_valid) {
+      const S *src = base + (int64_t)r * rstride + k;
+      if (vec && k + 8 <= k_valid) {
+        q.load(src);
+      } else {
+        float v[8];
 #pragma unroll
-  for (int task = tid; task < GB * KG; task += 256) {
-  const int r = task / KG, k8 = (task % KG) * 8;
-  float v[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) v[e] = 0.f;
-  if (r < rows_valid && k0 + k8 < k_valid) {
-    const S *src = base + (int64_t)r * rstride + k0 + k8;
-    if (vec && k0 + k8 + 8 <= k_valid) {
-      ld8<S>(src, v);
-    } else {
-#pragma unroll
-      for (int e = 0; e < 8; ++e)
-        if (k0 + k8 + e < k_valid) v[e] = ld1<S>(src + e);
+        for (int e = 0; e < 8; ++e) v[e] = k + e < k_valid ? ld1<S>(src + e) : 0.f;
+        q.pack(v);
+      }
     }
+  }
+  DEVI void commit(int k0) {
+    const int r = t >> 2, k8 = (t & 3) * 8;
+    float v[8];
+    q.unpack(v);
     if (kscale) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) v[e] *= kscale[k0 + k8 + e];
@@ -96,57 +111,74 @@ DEVI void stage_kc(uint16_t *hi, uint16_t *lo, const S *base, int64_t rstride, i
 #pragma unroll
       for (int e = 0; e < 8; ++e) v[e] *= rs;
     }
+    put8<SPLIT>(hi, lo, tile_off(r, k8), v);
   }
-  put8<SPLIT>(hi, lo, tile_off(r, k8), v);
-  }
-}
+};
 
-// Vectorised staging of a row-contiguous source: element (r, k) at base[k * kstride + r].  Tasks
-// are 2 consecutive k x 8 consecutive rows, stored transposed as 4-byte pairs; the 128 threads
-// t = 0..127 of the calling half of the workgroup share the GK / 2 * 8 tasks.
-template <bool SPLIT, typename S>
-DEVI void stage_rc(uint16_t *hi, uint16_t *lo, const S *base, int64_t kstride, int rows_valid, int k0, int k_valid,
-                   const float *kscale, const float *rscale, bool vec, int t) {
+// row-contiguous source: element (r, k) at base[k * kstride + r]; 128 threads take part (t = 0..127,
+// `active` false for the others): 2 consecutive k x 8 consecutive rows each, stored transposed.
+template <bool SPLIT, typename S> struct RcStager {
+  uint16_t *hi, *lo;
+  const S *base;
+  int64_t kstride;
+  int rows_valid, k_valid;
+  const float *kscale, *rscale;
+  bool vec;
+  int t;
+  bool active;
+  Pack8<S> q[2];
+  DEVI RcStager(uint16_t *hi_, uint16_t *lo_, const S *base_, int64_t kstride_, int rows_valid_, int k_valid_,
+                const float *kscale_, const float *rscale_, bool vec_, int t_, bool active_)
+      : hi(hi_), lo(lo_), base(base_), kstride(kstride_), rows_valid(rows_valid_), k_valid(k_valid_), kscale(kscale_),
+        rscale(rscale_), vec(vec_), t(t_), active(active_) {}
+  DEVI void fetch(int k0) {
+    if (!active) return;
+    const int k2 = (t >> 3) * 2, r8 = (t & 7) * 8;
 #pragma unroll
-  for (int task = t; task < (GK / 2) * 8; task += 128) {
-  const int k2 = (task >> 3) * 2, r8 = (task & 7) * 8;
-  float v[2][8];
+    for (int j = 0; j < 2; ++j) {
+      const int k = k0 + k2 + j;
+      q[j].zero();
+      if (k < k_valid && r8 < rows_valid) {
+        const S *src = base + (int64_t)k * kstride + r8;
+        if (vec && r8 + 8 <= rows_valid) {
+          q[j].load(src);
+        } else {
+          float v[8];
 #pragma unroll
-  for (int q = 0; q < 2; ++q) {
-    const int k = k0 + k2 + q;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) v[q][e] = 0.f;
-    if (k < k_valid && r8 < rows_valid) {
-      const S *src = base + (int64_t)k * kstride + r8;
-      if (vec && r8 + 8 <= rows_valid) {
-        ld8<S>(src, v[q]);
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (r8 + e < rows_valid) v[q][e] = ld1<S>(src + e);
+          for (int e = 0; e < 8; ++e) v[e] = r8 + e < rows_valid ? ld1<S>(src + e) : 0.f;
+          q[j].pack(v);
+        }
       }
+    }
+  }
+  DEVI void commit(int k0) {
+    if (!active) return;
+    const int k2 = (t >> 3) * 2, r8 = (t & 7) * 8;
+    float v[2][8];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      q[j].unpack(v[j]);
       if (kscale) {
-        const float ks = kscale[k];
+        const float ks = kscale[k0 + k2 + j];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[q][e] *= ks;
+        for (int e = 0; e < 8; ++e) v[j][e] *= ks;
       }
     }
-  }
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    float a = v[0][e], b = v[1][e];
-    if (rscale) {
-      const float rs = rscale[r8 + e];
-      a *= rs;
-      b *= rs;
+    for (int e = 0; e < 8; ++e) {
+      float a = v[0][e], b = v[1][e];
+      if (rscale) {
+        const float rs = rscale[r8 + e];
+        a *= rs;
+        b *= rs;
+      }
+      const int off = tile_off(r8 + e, k2);
+      const uint32_t h = pack_bf16(a, b);
+      *reinterpret_cast<uint32_t *>(hi + off) = h;
+      if (SPLIT) *reinterpret_cast<uint32_t *>(lo + off) = pack_bf16(a - bf16_lo(h), b - bf16_hi(h));
     }
-    const int off = tile_off(r8 + e, k2);
-    const uint32_t h = pack_bf16(a, b);
-    *reinterpret_cast<uint32_t *>(hi + off) = h;
-    if (SPLIT) *reinterpret_cast<uint32_t *>(lo + off) = pack_bf16(a - bf16_lo(h), b - bf16_hi(h));
   }
-  }
-}
+};
 
 template <typename S> DEVI bool rows_aligned16(const S *base, int64_t stride) {
   constexpr int m = 16 / sizeof(S);
@@ -226,18 +258,51 @@ DEVI void block_gemm(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, FA fa, FB
   }
 }
 
-// Same with caller-supplied stagers: stage_a(k0) / stage_b(k0) fill the A / B tile for the k step
-// starting at k0 (all 256 threads call both).
+// Software-pipelined form: sa / sb are stager objects with fetch(k0) (global -> registers) and
+// commit(k0) (registers -> LDS tile).  The fetch of step k0 + 32 is issued before the MFMAs of step
+// k0, so its latency hides behind them and behind the next barrier.
 template <bool SPLIT, typename SA, typename SB>
-DEVI void block_gemm_staged(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, SA stage_a, SB stage_b, int tid) {
+DEVI void block_gemm_pipe(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, SA &&sa, SB &&sb, int tid) {
   const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+  if (k_begin >= k_end) return;
+  sa.fetch(k_begin);
+  sb.fetch(k_begin);
   for (int k0 = k_begin; k0 < k_end; k0 += GK) {
     __syncthreads();
-    stage_a(k0);
-    stage_b(k0);
+    sa.commit(k0);
+    sb.commit(k0);
     __syncthreads();
+    if (k0 + GK < k_end) {
+      sa.fetch(k0 + GK);
+      sb.fetch(k0 + GK);
+    }
     mma_step<SPLIT>(acc, s, wm, wn, lane);
   }
+}
+
+// Stager for a causal operand: k steps below `diag_end` are filled from a functor f(row, k)
+// (exact masked form, nothing to fetch), the others by the wrapped vectorised stager.
+template <bool SPLIT, typename F, typename Inner> struct DiagStager {
+  uint16_t *hi, *lo;
+  F f;
+  int diag_end, tid;
+  Inner inner;
+  DEVI DiagStager(uint16_t *hi_, uint16_t *lo_, F f_, int diag_end_, int tid_, Inner inner_)
+      : hi(hi_), lo(lo_), f(f_), diag_end(diag_end_), tid(tid_), inner(inner_) {}
+  DEVI void fetch(int k0) {
+    if (k0 >= diag_end) inner.fetch(k0);
+  }
+  DEVI void commit(int k0) {
+    if (k0 < diag_end) {
+      stage_tile<SPLIT, false>(hi, lo, [&](int r, int k) { return f(r, k0 + k); }, tid);
+    } else {
+      inner.commit(k0);
+    }
+  }
+};
+template <bool SPLIT, typename F, typename Inner>
+DEVI DiagStager<SPLIT, F, Inner> diag_stager(uint16_t *hi, uint16_t *lo, F f, int diag_end, int tid, Inner inner) {
+  return DiagStager<SPLIT, F, Inner>(hi, lo, f, diag_end, tid, inner);
 }
 
 // Visits the block tile's accumulator: value = f(m, n, value) with m, n in [0, 64).

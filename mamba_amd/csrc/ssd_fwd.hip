@@ -84,10 +84,10 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bmm_chu
   const T *Ca = static_cast<const T *>(p.C) + Cb + (int64_t)(t0 + mt * GB) * p.C_ls;
   const T *Ba = static_cast<const T *>(p.B) + Bb + (int64_t)(t0 + nt * GB) * p.B_ls;
   const bool va = rows_aligned16(Ca, p.C_ls), vb = rows_aligned16(Ba, p.B_ls);
-  block_gemm_staged<SPLIT>(
+  block_gemm_pipe<SPLIT>(
       acc, lds, 0, N,
-      [&](int k0) { stage_kc<SPLIT, T>(lds.ah, lds.al, Ca, p.C_ls, qlim - mt * GB, k0, N, nullptr, nullptr, va, tid); },
-      [&](int k0) { stage_kc<SPLIT, T>(lds.bh, lds.bl, Ba, p.B_ls, qlim - nt * GB, k0, N, nullptr, nullptr, vb, tid); },
+      KcStager<SPLIT, T>(lds.ah, lds.al, Ca, p.C_ls, qlim - mt * GB, N, nullptr, nullptr, va, tid),
+      KcStager<SPLIT, T>(lds.bh, lds.bl, Ba, p.B_ls, qlim - nt * GB, N, nullptr, nullptr, vb, tid),
       tid);
   float *CB = p.CB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
   const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
@@ -139,15 +139,10 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void chunk_s
   const T *xa = static_cast<const T *>(p.x) + xb + (int64_t)t0 * p.x_ls + pt * GB;
   const T *Ba = static_cast<const T *>(p.B) + Bb + (int64_t)t0 * p.B_ls + nt * GB;
   const bool va = rows_aligned16(xa, p.x_ls), vb = rows_aligned16(Ba, p.B_ls);
-  block_gemm_staged<SPLIT>(  // the first barrier inside publishes w
+  block_gemm_pipe<SPLIT>(  // the first barrier inside publishes w
       acc, lds, 0, qlim,
-      [&](int k0) {
-        if (tid < 128) stage_rc<SPLIT, T>(lds.ah, lds.al, xa, p.x_ls, P - pt * GB, k0, qlim, nullptr, nullptr, va, tid);
-      },
-      [&](int k0) {
-        if (tid >= 128)
-          stage_rc<SPLIT, T>(lds.bh, lds.bl, Ba, p.B_ls, N - nt * GB, k0, qlim, w, nullptr, vb, tid - 128);
-      },
+      RcStager<SPLIT, T>(lds.ah, lds.al, xa, p.x_ls, P - pt * GB, qlim, nullptr, nullptr, va, tid, tid < 128),
+      RcStager<SPLIT, T>(lds.bh, lds.bl, Ba, p.B_ls, N - nt * GB, qlim, w, nullptr, vb, tid - 128, tid >= 128),
       tid);
   float *st = p.states + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
   acc_foreach(acc, tid, [&](int m, int n, float v) {
@@ -187,15 +182,10 @@ __global__ __launch_bounds__(256) void chunk_state_varlen_kernel(const SsdParams
     const T *xa = static_cast<const T *>(p.x) + h * p.x_hs + (int64_t)t0 * p.x_ls + pt * GB;
     const T *Ba = static_cast<const T *>(p.B) + g * p.B_gs + (int64_t)t0 * p.B_ls + nt * GB;
     const bool va = rows_aligned16(xa, p.x_ls), vb = rows_aligned16(Ba, p.B_ls);
-    block_gemm_staged<SPLIT>(  // the first barrier inside publishes w
+    block_gemm_pipe<SPLIT>(  // the first barrier inside publishes w
         acc, lds, kstart / GK * GK, kend,
-        [&](int k0) {
-          if (tid < 128) stage_rc<SPLIT, T>(lds.ah, lds.al, xa, p.x_ls, P - pt * GB, k0, kend, nullptr, nullptr, va, tid);
-        },
-        [&](int k0) {
-          if (tid >= 128)
-            stage_rc<SPLIT, T>(lds.bh, lds.bl, Ba, p.B_ls, N - nt * GB, k0, kend, w, nullptr, vb, tid - 128);
-        },
+        RcStager<SPLIT, T>(lds.ah, lds.al, xa, p.x_ls, P - pt * GB, kend, nullptr, nullptr, va, tid, tid < 128),
+        RcStager<SPLIT, T>(lds.bh, lds.bl, Ba, p.B_ls, N - nt * GB, kend, w, nullptr, vb, tid - 128, tid >= 128),
         tid);
     if (start < t0) {
       const float *Hc = p.states + ((int64_t)c * H + h) * P * N;
