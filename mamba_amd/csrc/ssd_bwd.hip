@@ -676,7 +676,6 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bmm_chu
 // One workgroup per (batch, chunk, 16 heads); thread tid handles position Q-1-tid, so that the
 // reverse running sum of dL/da over the chunk (-> dL/d(dt A)) is a forward wave scan.  Then the
 // chain through A, the clamp, softplus and the bias; dA and ddt_bias are reduced per workgroup.
-constexpr int CS_HT = 16;
 
 DEVI float wave_incl_sum(float x) {
   x += dpp_f<DPP_ROW_SHR + 1>(0.f, x);
@@ -688,45 +687,66 @@ DEVI float wave_incl_sum(float x) {
   return x;
 }
 
+constexpr int CSB_HT = 4;  // heads per workgroup in the backward kernel (more, smaller workgroups)
+
 __global__ __launch_bounds__(256) void chunk_cumsum_bwd_kernel(const SsdParams p) {
-  __shared__ float wtot[4][CS_HT];
+  __shared__ float wtot[4][CSB_HT], part[2][4][CSB_HT];
   const int H = p.nheads, Q = p.chunk_size, L = p.seqlen;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l = Q - 1 - tid;
-  const int c = blockIdx.x, h0 = blockIdx.y * CS_HT, b = blockIdx.z;
+  const int c = blockIdx.x, h0 = blockIdx.y * CSB_HT, b = blockIdx.z;
   const int t = c * Q + l;
   const bool inq = l >= 0, live = inq && t < L;
-  float run[CS_HT];
+  const int lc = max(l, 0), tc = min(c * Q + lc, L - 1);  // clamped: every load below is unconditional
+  // all loads first
+  float g[CSB_HT], o[CSB_HT], d[CSB_HT], raw[CSB_HT], A[CSB_HT], bias[CSB_HT];
 #pragma unroll
-  for (int i = 0; i < CS_HT; ++i) {
-    const int h = h0 + i;
-    const float v = (h < H && inq) ? chunk_row(p.ddA_cumsum, p, b, h, c)[l] : 0.f;
-    run[i] = wave_incl_sum(v);
+  for (int i = 0; i < CSB_HT; ++i) {
+    const int h = min(h0 + i, H - 1);
+    g[i] = chunk_row(p.ddA_cumsum, p, b, h, c)[lc];
+    o[i] = chunk_row(p.ddt_out, p, b, h, c)[lc];
+    d[i] = chunk_row(p.dt_out, p, b, h, c)[lc];
+    raw[i] = ld_dyn(p.dt, b * p.dt_bs + (int64_t)tc * p.dt_ls + h * p.dt_hs, p.dt_dtype);
+    A[i] = static_cast<const float *>(p.A)[h];
+    bias[i] = p.dt_bias ? static_cast<const float *>(p.dt_bias)[h] : 0.f;
+  }
+  float run[CSB_HT];
+#pragma unroll
+  for (int i = 0; i < CSB_HT; ++i) {
+    run[i] = wave_incl_sum((h0 + i < H && inq) ? g[i] : 0.f);
     if (lane == 63) wtot[wave][i] = run[i];
   }
   __syncthreads();
 #pragma unroll
-  for (int i = 0; i < CS_HT; ++i) {
+  for (int i = 0; i < CSB_HT; ++i) {
     const int h = h0 + i;
     float r = run[i];
     for (int w = 0; w < wave; ++w) r += wtot[w][i];
     float dAterm = 0.f, ddt = 0.f;
     if (h < H && live) {
-      const float A = static_cast<const float *>(p.A)[h];
-      const float bias = p.dt_bias ? static_cast<const float *>(p.dt_bias)[h] : 0.f;
-      ddt = __builtin_fmaf(r, A, chunk_row(p.ddt_out, p, b, h, c)[l]);
-      dAterm = r * chunk_row(p.dt_out, p, b, h, c)[l];
-      const float raw = ld_dyn(p.dt, b * p.dt_bs + (int64_t)t * p.dt_ls + h * p.dt_hs, p.dt_dtype) + bias;
-      const float v = p.dt_softplus ? softplus_f(raw) : raw;
+      ddt = __builtin_fmaf(r, A[i], o[i]);
+      dAterm = r * d[i];
+      const float x = raw[i] + bias[i];
+      const float v = p.dt_softplus ? softplus_f(x) : x;
       if (v < p.dt_min || v > p.dt_max) ddt = 0.f;
-      if (p.dt_softplus && raw <= 20.f) ddt *= sigmoid_f(raw);
+      if (p.dt_softplus && x <= 20.f) ddt *= sigmoid_f(x);
       st_dyn(p.ddt, ((int64_t)b * L + t) * H + h, p.dt_dtype, ddt);
     }
-    dAterm = wave_sum(dAterm);
-    ddt = wave_sum(ddt);
-    if (lane == 0 && h < H) {
-      unsafeAtomicAdd(p.dA + h, dAterm);
-      if (p.ddt_bias) unsafeAtomicAdd(p.ddt_bias + h, ddt);
+    dAterm = wave_sum_to_last(dAterm);
+    ddt = wave_sum_to_last(ddt);
+    if (lane == 63) {
+      part[0][wave][i] = dAterm;
+      part[1][wave][i] = ddt;
+    }
+  }
+  // one atomic per workgroup and head: adds to one address serialise in L2
+  __syncthreads();
+  if (tid < 2 * CSB_HT) {
+    const int which = tid / CSB_HT, i = tid % CSB_HT, h = h0 + i;
+    const float v = part[which][0][i] + part[which][1][i] + part[which][2][i] + part[which][3][i];
+    if (h < H) {
+      if (which == 0) unsafeAtomicAdd(p.dA + h, v);
+      else if (p.ddt_bias) unsafeAtomicAdd(p.ddt_bias + h, v);
     }
   }
 }
@@ -834,7 +854,7 @@ extern "C" int ssd_chunk_cumsum_bwd(const SsdParams *p, mamba_stream_t stream) {
   int rc = check_bwd(p);
   if (rc) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  dim3 grid(p->nchunks, (p->nheads + CS_HT - 1) / CS_HT, p->batch);
+  dim3 grid(p->nchunks, (p->nheads + CSB_HT - 1) / CSB_HT, p->batch);
   hipLaunchKernelGGL(chunk_cumsum_bwd_kernel, grid, dim3(256), 0, s, *p);
   return launched();
 }
