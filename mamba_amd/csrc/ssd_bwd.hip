@@ -238,34 +238,86 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dst
 // ---------------------------------------------------- state_passing bwd
 // Reverse recurrence over chunks.  On entry dstates[c] is the direct gradient of the state
 // entering chunk c; on exit it is the gradient of chunk c's local state.
-__global__ __launch_bounds__(256) void state_passing_bwd_kernel(const SsdParams p) {
+// A thread owns W consecutive elements; the direct gradients and states of the next SPB_PF chunks
+// are always in flight (the serial recurrence only needs them one chunk at a time, and the
+// compiler cannot hoist the loads over the in-place stores by itself).
+constexpr int SPB_PF = 4;
+
+template <int W> struct VecG;
+template <> struct VecG<1> {
+  float v[1];
+  DEVI void load(const float *p) { v[0] = *p; }
+  DEVI void store(float *p) const { *p = v[0]; }
+};
+template <> struct VecG<4> {
+  float v[4];
+  DEVI void load(const float *p) {
+    const f32x4 t = *reinterpret_cast<const f32x4 *>(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+  }
+  DEVI void store(float *p) const { *reinterpret_cast<f32x4 *>(p) = f32x4{v[0], v[1], v[2], v[3]}; }
+};
+
+template <int W> __global__ __launch_bounds__(256) void state_passing_bwd_kernel(const SsdParams p) {
   const int PN = p.headdim * p.dstate, H = p.nheads, nc = p.nchunks, Q = p.chunk_size, L = p.seqlen;
-  const int e = blockIdx.x * 256 + threadIdx.x;
+  const int e = (blockIdx.x * 256 + threadIdx.x) * W;
   const int lane = threadIdx.x & 63;
   const int h = blockIdx.y, b = blockIdx.z;
   const bool live = e < PN;
-  float G = (live && p.dfinal_states) ? p.dfinal_states[((int64_t)b * H + h) * PN + e] : 0.f;
+  const int ec = live ? e : 0;  // clamped: idle threads read valid memory and add nothing
+  VecG<W> G;
+#pragma unroll
+  for (int i = 0; i < W; ++i) G.v[i] = 0.f;
+  if (live && p.dfinal_states) G.load(p.dfinal_states + ((int64_t)b * H + h) * PN + e);
   const float *dA = p.dA_cumsum + ((int64_t)b * H + h) * nc * Q;
   const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L : nullptr;
-  for (int c = nc - 1; c >= 0; --c) {
-    const int64_t off = (((int64_t)b * nc + c) * H + h) * PN + e;
+  auto offset = [&](int c) { return (((int64_t)b * nc + c) * H + h) * PN + ec; };
+  auto decay = [&](int c) {
     float scale = fast_exp(dA[c * Q + Q - 1]);
     if (seq) {
       const int end_c = seq[min((c + 1) * Q, L) - 1];
       const int end_prev = c > 0 ? seq[c * Q - 1] : 0;
       if (end_c != end_prev) scale = 0.f;
     }
-    float part = 0.f, direct = 0.f;
-    if (live) {
-      direct = p.dstates[off];
-      p.dstates[off] = G;
-      part = G * p.states[off] * scale;
+    return scale;
+  };
+  VecG<W> direct[SPB_PF], state[SPB_PF];
+  float scale[SPB_PF];
+#pragma unroll
+  for (int j = 0; j < SPB_PF; ++j) {
+    const int c = nc - 1 - j;
+    if (c >= 0) {
+      direct[j].load(p.dstates + offset(c));
+      state[j].load(p.states + offset(c));
+      scale[j] = decay(c);
     }
-    part = wave_sum(part);
-    if (lane == 0 && part != 0.f) unsafeAtomicAdd(p.ddA_cumsum + (((int64_t)b * H + h) * nc + c) * Q + Q - 1, part);
-    G = __builtin_fmaf(scale, G, direct);
   }
-  if (live && p.dinitial_states) p.dinitial_states[((int64_t)b * H + h) * PN + e] = G;
+  for (int c0 = nc - 1; c0 >= 0; c0 -= SPB_PF) {
+#pragma unroll
+    for (int j = 0; j < SPB_PF; ++j) {
+      const int c = c0 - j;
+      if (c < 0) break;
+      if (live) G.store(p.dstates + offset(c));
+      const VecG<W> dir = direct[j], st = state[j];
+      const float sc = scale[j];
+      if (c - SPB_PF >= 0) {
+        direct[j].load(p.dstates + offset(c - SPB_PF));
+        state[j].load(p.states + offset(c - SPB_PF));
+        scale[j] = decay(c - SPB_PF);
+      }
+      float part = 0.f;
+#pragma unroll
+      for (int i = 0; i < W; ++i) {
+        part = __builtin_fmaf(G.v[i], st.v[i], part);
+        G.v[i] = __builtin_fmaf(sc, G.v[i], dir.v[i]);
+      }
+      part = live ? part * sc : 0.f;
+      part = wave_sum_to_last(part);
+      if (lane == 63 && part != 0.f)
+        unsafeAtomicAdd(p.ddA_cumsum + (((int64_t)b * H + h) * nc + c) * Q + Q - 1, part);
+    }
+  }
+  if (live && p.dinitial_states) G.store(p.dinitial_states + ((int64_t)b * H + h) * PN + e);
 }
 
 // ------------------------------------------------------------------- dx
@@ -807,8 +859,15 @@ extern "C" int ssd_state_passing_bwd(const SsdParams *p, mamba_stream_t stream) 
   int rc = check_bwd(p);
   if (rc) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  dim3 grid((p->headdim * p->dstate + 255) / 256, p->nheads, p->batch);
-  hipLaunchKernelGGL(state_passing_bwd_kernel, grid, dim3(256), 0, s, *p);
+  const int PN = p->headdim * p->dstate;
+  auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+  if (PN % 4 == 0 && al16(p->states) && al16(p->dstates) && al16(p->dfinal_states) && al16(p->dinitial_states)) {
+    dim3 grid((PN / 4 + 255) / 256, p->nheads, p->batch);
+    hipLaunchKernelGGL(state_passing_bwd_kernel<4>, grid, dim3(256), 0, s, *p);
+  } else {
+    dim3 grid((PN + 255) / 256, p->nheads, p->batch);
+    hipLaunchKernelGGL(state_passing_bwd_kernel<1>, grid, dim3(256), 0, s, *p);
+  }
   return launched();
 }
 

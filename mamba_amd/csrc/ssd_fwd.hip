@@ -205,29 +205,72 @@ __global__ __launch_bounds__(256) void chunk_state_varlen_kernel(const SsdParams
 
 // ---------------------------------------------------------- state_passing
 // In place over `states`: slot c receives the state ENTERING chunk c; the state
-// after the last chunk goes to final_states.
-__global__ __launch_bounds__(256) void state_passing_fwd_kernel(const SsdParams p) {
+// after the last chunk goes to final_states.  A thread owns W consecutive elements of the
+// (headdim x dstate) state; the chunk loop is a serial recurrence, so the local states of the
+// next SP_PF chunks are always in flight (the compiler cannot hoist those loads over the in-place
+// stores by itself).
+constexpr int SP_PF = 4;
+
+template <int W> struct VecF;
+template <> struct VecF<1> {
+  float v[1];
+  DEVI void load(const float *p) { v[0] = *p; }
+  DEVI void store(float *p) const { *p = v[0]; }
+};
+template <> struct VecF<4> {
+  float v[4];
+  DEVI void load(const float *p) {
+    const f32x4 t = *reinterpret_cast<const f32x4 *>(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+  }
+  DEVI void store(float *p) const { *reinterpret_cast<f32x4 *>(p) = f32x4{v[0], v[1], v[2], v[3]}; }
+};
+
+template <int W> __global__ __launch_bounds__(256) void state_passing_fwd_kernel(const SsdParams p) {
   const int PN = p.headdim * p.dstate, H = p.nheads, nc = p.nchunks, Q = p.chunk_size, L = p.seqlen;
-  const int e = blockIdx.x * 256 + threadIdx.x;
+  const int e = (blockIdx.x * 256 + threadIdx.x) * W;
   const int h = blockIdx.y, b = blockIdx.z;
   if (e >= PN) return;
-  float s = p.initial_states ? p.initial_states[((int64_t)b * H + h) * PN + e] : 0.f;
+  VecF<W> s;
+#pragma unroll
+  for (int i = 0; i < W; ++i) s.v[i] = 0.f;
+  if (p.initial_states) s.load(p.initial_states + ((int64_t)b * H + h) * PN + e);
   const float *dA = p.dA_cumsum + ((int64_t)b * H + h) * nc * Q;
   const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L : nullptr;
-  int seq_prev = 0;
-  for (int c = 0; c < nc; ++c) {
-    float *slot = p.states + (((int64_t)b * nc + c) * H + h) * PN + e;
-    const float local = *slot;
-    *slot = s;
+  auto slot = [&](int c) { return p.states + (((int64_t)b * nc + c) * H + h) * PN + e; };
+  auto decay = [&](int c) {  // carried-state factor of chunk c: 0 across a sequence boundary
     float scale = fast_exp(dA[c * Q + Q - 1]);
     if (seq) {
-      const int seq_new = seq[min((c + 1) * Q, L) - 1];
+      const int seq_new = seq[min((c + 1) * Q, L) - 1], seq_prev = c > 0 ? seq[c * Q - 1] : 0;
       if (seq_new != seq_prev) scale = 0.f;
-      seq_prev = seq_new;
     }
-    s = __builtin_fmaf(scale, s, local);
+    return scale;
+  };
+  VecF<W> local[SP_PF];
+  float scale[SP_PF];
+#pragma unroll
+  for (int j = 0; j < SP_PF; ++j)
+    if (j < nc) {
+      local[j].load(slot(j));
+      scale[j] = decay(j);
+    }
+  for (int c0 = 0; c0 < nc; c0 += SP_PF) {
+#pragma unroll
+    for (int j = 0; j < SP_PF; ++j) {
+      const int c = c0 + j;
+      if (c >= nc) break;
+      s.store(slot(c));
+      const VecF<W> loc = local[j];
+      const float sc = scale[j];
+      if (c + SP_PF < nc) {
+        local[j].load(slot(c + SP_PF));
+        scale[j] = decay(c + SP_PF);
+      }
+#pragma unroll
+      for (int i = 0; i < W; ++i) s.v[i] = __builtin_fmaf(sc, s.v[i], loc.v[i]);
+    }
   }
-  p.final_states[((int64_t)b * H + h) * PN + e] = s;
+  s.store(p.final_states + ((int64_t)b * H + h) * PN + e);
 }
 
 // ------------------------------------------------------------- chunk_scan
@@ -398,8 +441,15 @@ extern "C" int ssd_state_passing_fwd(const SsdParams *p, mamba_stream_t stream) 
   if (rc) return rc;
   if (!p->states || !p->final_states || !p->dA_cumsum) return MAMBA_E_BADARG;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  dim3 grid((p->headdim * p->dstate + 255) / 256, p->nheads, p->batch);
-  hipLaunchKernelGGL(state_passing_fwd_kernel, grid, dim3(256), 0, s, *p);
+  const int PN = p->headdim * p->dstate;
+  auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+  if (PN % 4 == 0 && al16(p->states) && al16(p->final_states) && al16(p->initial_states)) {
+    dim3 grid((PN / 4 + 255) / 256, p->nheads, p->batch);
+    hipLaunchKernelGGL(state_passing_fwd_kernel<4>, grid, dim3(256), 0, s, *p);
+  } else {
+    dim3 grid((PN + 255) / 256, p->nheads, p->batch);
+    hipLaunchKernelGGL(state_passing_fwd_kernel<1>, grid, dim3(256), 0, s, *p);
+  }
   return launched();
 }
 
