@@ -400,6 +400,27 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
         RcStager<SPLIT, T>(lds.bh, lds.bl, ga, gv.ls, P - pt * GB, qlim, nullptr, nullptr, vb, tid, tid < 128),
         tid);
   }
+  // The epilogue's x and g rows (thread t: position s = tile row t / 4, 16 consecutive p) are
+  // fetched before the accumulators are re-laid, so that they arrive during that exchange (any
+  // earlier and the extra live registers cost a wave of occupancy).
+  const int s = st * GB + (tid >> 2), p0 = pt * GB + (tid & 3) * 16;
+  const bool row_ok = s < qlim;
+  const T *xr = static_cast<const T *>(p.x) + xb + (int64_t)(t0 + s) * p.x_ls + p0;
+  const T *gr = static_cast<const T *>(gv.ptr) + gb + (int64_t)(t0 + s) * gv.ls + p0;
+  const bool vec = P % 8 == 0 && rows_aligned16(static_cast<const T *>(p.x) + xb, p.x_ls) &&
+                   rows_aligned16(static_cast<const T *>(gv.ptr) + gb, gv.ls) &&
+                   (reinterpret_cast<uintptr_t>(p.dx) & 15) == 0;
+  const float *Dp = static_cast<const float *>(p.D);
+  Pack8<T> xk[2], gk[2];
+  if (vec) {
+    const int sc = min(s, qlim - 1) - s;  // row clamp, as an offset from s
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int pc = min(p0 + 8 * j, P - 8) - p0;  // column clamp; clamped pieces are masked below
+      xk[j].load(xr + (int64_t)sc * p.x_ls + pc);
+      gk[j].load(gr + (int64_t)sc * gv.ls + pc);
+    }
+  }
   // Epilogue with rows in threads: thread t owns position s = tile row t / 4 and 16 consecutive p.
   float v1[16], v2[16];
   acc_to_rows(acc1, lds, tid, v1);
@@ -409,15 +430,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
 #pragma unroll
     for (int e = 0; e < 16; ++e) v1[e] *= w;
   }
-  const int s = st * GB + (tid >> 2), p0 = pt * GB + (tid & 3) * 16;
-  const bool row_ok = s < qlim;
-  const T *xr = static_cast<const T *>(p.x) + xb + (int64_t)(t0 + s) * p.x_ls + p0;
-  const T *gr = static_cast<const T *>(gv.ptr) + gb + (int64_t)(t0 + s) * gv.ls + p0;
   T *dxr = static_cast<T *>(p.dx) + (((int64_t)b * L + t0 + s) * H + h) * P + p0;
-  const bool vec = P % 8 == 0 && rows_aligned16(static_cast<const T *>(p.x) + xb, p.x_ls) &&
-                   rows_aligned16(static_cast<const T *>(gv.ptr) + gb, gv.ls) &&
-                   (reinterpret_cast<uintptr_t>(p.dx) & 15) == 0;
-  const float *Dp = static_cast<const float *>(p.D);
   float q1 = 0.f, q2 = 0.f;
   const float dts = dt_s[min(s, Q - 1)];
 #pragma unroll
@@ -425,8 +438,12 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
     const int nv = row_ok ? max(0, min(8, P - p0 - 8 * j)) : 0;
     float xv[8], gvv[8], o[8];
     if (vec) {
-      ld8_guard<T, true>(xr + 8 * j, nv, 0.f, xv);
-      ld8_guard<T, true>(gr + 8 * j, Dp ? nv : 0, 0.f, gvv);
+      xk[j].unpack(xv);
+      gk[j].unpack(gvv);
+      if (nv < 8) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) xv[e] = gvv[e] = 0.f;
+      }
     } else {
       ld8_guard<T, false>(xr + 8 * j, nv, 0.f, xv);
       ld8_guard<T, false>(gr + 8 * j, Dp ? nv : 0, 0.f, gvv);
@@ -448,12 +465,15 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
   q1 += __shfl_xor(q1, 2, 64);
   q2 += __shfl_xor(q2, 1, 64);
   q2 += __shfl_xor(q2, 2, 64);
-  if ((tid & 3) == 0 && row_ok) {
+  const bool lead = (tid & 3) == 0 && row_ok;
+  float *dda = chunk_row(p.ddA_cumsum, p, b, h, c);
+  if (lead) {
     unsafeAtomicAdd(chunk_row(p.ddt_out, p, b, h, c) + s, q2);
-    float *dda = chunk_row(p.ddA_cumsum, p, b, h, c);
-    unsafeAtomicAdd(dda + s, -dts * q1);      // chunk-state terms: -dt_s <x_s, acc1_s> at s ...
-    unsafeAtomicAdd(dda + Q - 1, dts * q1);   // ... and + at the chunk end
+    unsafeAtomicAdd(dda + s, -dts * q1);  // chunk-state terms: -dt_s <x_s, acc1_s> at s ...
   }
+  // ... and + at the chunk end: one address for the whole tile, so one atomic per wave
+  const float endsum = wave_sum_to_last(lead ? dts * q1 : 0.f);
+  if ((tid & 63) == 63) unsafeAtomicAdd(dda + Q - 1, endsum);
 }
 
 // ---------------------------------------------- state-path parts of dB, dC
