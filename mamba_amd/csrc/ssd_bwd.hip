@@ -382,10 +382,10 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
         tid);
   }
   {
-    auto fa = [&](int r, int k) {  // (s, l)
+    // exact decay and causal mask for the diagonal 64 x 64 block: multiplier of CB[l = k, s]
+    auto fa = [&](int r, int k) {
       const int s = st * GB + r;
-      if (s >= qlim || k >= qlim || k < s) return 0.f;
-      return CB[(int64_t)k * Q + s] * fast_exp(fminf(a_s[k] - a_s[s], 0.f));
+      return (s < qlim && k < qlim && k >= s) ? fast_exp(fminf(a_s[min(k, Q - 1)] - a_s[min(s, Q - 1)], 0.f)) : 0.f;
     };
     const T *ga = static_cast<const T *>(gv.ptr) + gb + (int64_t)t0 * gv.ls + pt * GB;
     const bool vb = rows_aligned16(ga, gv.ls);
@@ -394,7 +394,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
     block_gemm_pipe<SPLIT>(
         acc2, lds, st * GB, qlim,
         // diagonal block: causal mask and the exact decay; below it CB^T with the rank-1 decays
-        diag_stager<SPLIT>(lds.ah, lds.al, fa, (st + 1) * GB, tid,
+        diag_stager<SPLIT>(fa, (st + 1) * GB,
                            RcStager<SPLIT, float>(lds.ah, lds.al, CBa, Q, qlim - st * GB, qlim, kdec, rdec, va, tid - 128,
                                                   tid >= 128)),
         RcStager<SPLIT, T>(lds.bh, lds.bl, ga, gv.ls, P - pt * GB, qlim, nullptr, nullptr, vb, tid, tid < 128),

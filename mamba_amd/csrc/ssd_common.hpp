@@ -151,6 +151,22 @@ template <bool SPLIT, typename S> struct RcStager {
       }
     }
   }
+  // commit with a multiplier per element, f(tile row, absolute k), instead of the scale vectors
+  template <typename F> DEVI void commit_each(int k0, F f) {
+    if (!active) return;
+    const int k2 = (t >> 3) * 2, r8 = (t & 7) * 8;
+    float v[2][8];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) q[j].unpack(v[j]);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float a = v[0][e] * f(r8 + e, k0 + k2), b = v[1][e] * f(r8 + e, k0 + k2 + 1);
+      const int off = tile_off(r8 + e, k2);
+      const uint32_t h = pack_bf16(a, b);
+      *reinterpret_cast<uint32_t *>(hi + off) = h;
+      if (SPLIT) *reinterpret_cast<uint32_t *>(lo + off) = pack_bf16(a - bf16_lo(h), b - bf16_hi(h));
+    }
+  }
   DEVI void commit(int k0) {
     if (!active) return;
     const int k2 = (t >> 3) * 2, r8 = (t & 7) * 8;
@@ -280,29 +296,22 @@ DEVI void block_gemm_pipe(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, SA &
   }
 }
 
-// Stager for a causal operand: k steps below `diag_end` are filled from a functor f(row, k)
-// (exact masked form, nothing to fetch), the others by the wrapped vectorised stager.
+// Stager for a causal operand on top of a row-contiguous stager: k steps below `diag_end` take an
+// exact per-element multiplier f(tile row, k) (mask and decay), the others the stager's rank-1
+// scale vectors.  Either way the loads go through the same fetch.
 template <bool SPLIT, typename F, typename Inner> struct DiagStager {
-  uint16_t *hi, *lo;
   F f;
-  int diag_end, tid;
+  int diag_end;
   Inner inner;
-  DEVI DiagStager(uint16_t *hi_, uint16_t *lo_, F f_, int diag_end_, int tid_, Inner inner_)
-      : hi(hi_), lo(lo_), f(f_), diag_end(diag_end_), tid(tid_), inner(inner_) {}
-  DEVI void fetch(int k0) {
-    if (k0 >= diag_end) inner.fetch(k0);
-  }
+  DEVI DiagStager(F f_, int diag_end_, Inner inner_) : f(f_), diag_end(diag_end_), inner(inner_) {}
+  DEVI void fetch(int k0) { inner.fetch(k0); }
   DEVI void commit(int k0) {
-    if (k0 < diag_end) {
-      stage_tile<SPLIT, false>(hi, lo, [&](int r, int k) { return f(r, k0 + k); }, tid);
-    } else {
-      inner.commit(k0);
-    }
+    if (k0 < diag_end) inner.commit_each(k0, f);
+    else inner.commit(k0);
   }
 };
-template <bool SPLIT, typename F, typename Inner>
-DEVI DiagStager<SPLIT, F, Inner> diag_stager(uint16_t *hi, uint16_t *lo, F f, int diag_end, int tid, Inner inner) {
-  return DiagStager<SPLIT, F, Inner>(hi, lo, f, diag_end, tid, inner);
+template <bool SPLIT, typename F, typename Inner> DEVI DiagStager<SPLIT, F, Inner> diag_stager(F f, int diag_end, Inner inner) {
+  return DiagStager<SPLIT, F, Inner>(f, diag_end, inner);
 }
 
 // Visits the block tile's accumulator: value = f(m, n, value) with m, n in [0, 64).
