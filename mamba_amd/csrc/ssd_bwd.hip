@@ -482,9 +482,10 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
 // One workgroup per (batch, chunk, group, 64 x 64 tile) loops over the heads of the group and keeps
 // both sums in registers (no atomics); the per-head row factor is folded into the A operand.
 // The carried-state share of ddA_cumsum, sum_n dC_h[l, n] C[l, n], is taken per head on the way.
-template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dBC_state_kernel(const SsdParams p) {
+template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_dBC_state_kernel(const SsdParams p) {
+  constexpr int MAXH = 8;  // heads per workgroup (head_splits keeps it at or below 8)
   __shared__ GemmLds lds;
-  __shared__ float wB[2][GB], wC[2][GB];  // per-head row factors, double-buffered over the head loop
+  __shared__ float wB[MAXH][GB], wC[MAXH][GB];  // per-head row factors
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
   const int i = lane & 15, gq = lane >> 4;
@@ -495,94 +496,126 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dBC
   const int st = blk.x % nst, nt = blk.x / nst;  // the s tiles of a chunk share the state tiles
   const int hpg = H / G, nsplit = head_splits(hpg);
   const int c = blk.y, bg = blk.z / nsplit, hs = blk.z % nsplit, b = bg / G, g = bg % G;
+  const int nh = hs < hpg ? (hpg - hs + nsplit - 1) / nsplit : 0;  // heads hs, hs + nsplit, ...
   const int t0 = c * Q, qlim = min(Q, L - t0);
   const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
   const View4 gv = g_view(p);
-  const int64_t Cb = b * p.C_bs + g * p.C_gs;
-  // C at this lane's 16 accumulator positions (shared by the heads of the group)
-  float cr[2][2][4];
-#pragma unroll
-  for (int tm = 0; tm < 2; ++tm)
-#pragma unroll
-    for (int tn = 0; tn < 2; ++tn)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int l = st * GB + wm * 32 + tm * 16 + gq * 4 + r, nn = nt * GB + wn * 32 + tn * 16 + i;
-        cr[tm][tn][r] = (l < qlim && nn < N) ? ldg<T>(p.C, Cb + (int64_t)(t0 + l) * p.C_ls + nn) : 0.f;
+  // row factors of every head of this workgroup (published by the first barrier of the GEMM)
+  for (int idx = tid; idx < nh * GB; idx += 256) {
+    const int hl = idx / GB, r = idx % GB, s = st * GB + r, h = g * hpg + hs + hl * nsplit;
+    float vb = 0.f, vc = 0.f;
+    if (s < qlim) {
+      const float *dA = chunk_row(p.dA_cumsum, p, b, h, c);
+      bool okb = true, okc = true;
+      if (seq) {
+        const int last = seq[qlim - 1];
+        okb = last >= 0 && seq[s] == last;
+        okc = seq[s] == (c > 0 ? seq[-1] : 0);
       }
-  GemmAcc accB, accC;
-  accB.zero();
-  accC.zero();
-  int par = 0;
-  for (int hh = hs; hh < hpg; hh += nsplit, par ^= 1) {
-    const int h = g * hpg + hh;
-    const float *dA = chunk_row(p.dA_cumsum, p, b, h, c);
-    const float *dt = chunk_row(p.dt_out, p, b, h, c);
-    // published by the first barrier inside the GEMM; the buffer written here was last read two
-    // iterations ago
-    if (tid < GB) {
-      const int s = st * GB + tid;
-      float vb = 0.f, vc = 0.f;
-      if (s < qlim) {
-        bool okb = true, okc = true;
-        if (seq) {
-          const int last = seq[qlim - 1];
-          okb = last >= 0 && seq[s] == last;
-          okc = seq[s] == (c > 0 ? seq[-1] : 0);
-        }
-        if (okb) vb = fast_exp(fminf(dA[Q - 1] - dA[s], 0.f)) * dt[s];
-        if (okc) vc = fast_exp(dA[s]);
-      }
-      wB[par][tid] = vb;
-      wC[par][tid] = vc;
+      if (okb) vb = fast_exp(fminf(dA[Q - 1] - dA[s], 0.f)) * chunk_row(p.dt_out, p, b, h, c)[s];
+      if (okc) vc = fast_exp(dA[s]);
     }
-    const int64_t gb = b * gv.bs + h * gv.hs, xb = b * p.x_bs + h * p.x_hs;
-    const float *dS = p.dstates + (((int64_t)b * p.nchunks + c) * H + h) * P * N + nt * GB;
-    const float *Hc = p.states + (((int64_t)b * p.nchunks + c) * H + h) * P * N + nt * GB;
-    const bool vs = rows_aligned16(dS, N) && rows_aligned16(Hc, N);
-    // A = (w x) or (w g) rows (position, k = p): k-contiguous; B = state rows n, k = p: row-contiguous fp32
-    auto run = [&](GemmAcc &acc, const T *a_base, int64_t a_ls, const float *w, const float *S) {
-      const T *aa = a_base + (int64_t)(t0 + st * GB) * a_ls;
-      const bool va = rows_aligned16(aa, a_ls);
-      block_gemm_pipe<SPLIT>(
-          acc, lds, 0, P,
-          KcStager<SPLIT, T>(lds.ah, lds.al, aa, a_ls, qlim - st * GB, P, nullptr, w, va, tid),
-          RcStager<SPLIT, float>(lds.bh, lds.bl, S, N, N - nt * GB, P, nullptr, nullptr, vs, tid, tid < 128),
-          tid);
-    };
-    run(accB, static_cast<const T *>(p.x) + xb, p.x_ls, wB[par], dS);
-    GemmAcc accH;
-    accH.zero();
-    run(accH, static_cast<const T *>(gv.ptr) + gb, gv.ls, wC[par], Hc);
-    // carried-state share of ddA_cumsum: sum_n dC_h[l, n] C[l, n]
-    float *dda = chunk_row(p.ddA_cumsum, p, b, h, c);
+    wB[hl][r] = vb;
+    wC[hl][r] = vc;
+  }
+  // The k axis of both products concatenates the heads (k = (head, p)), so each runs as one
+  // pipelined GEMM: A = (w x) or (w g) rows (position, k = p), k-contiguous; B = state rows n,
+  // k = p: row-contiguous fp32.
+  const int seg_k = cdiv(P, GK) * GK;
+  auto state_off = [&](int hl) {
+    return (((int64_t)b * p.nchunks + c) * H + g * hpg + hs + hl * nsplit) * P * N + nt * GB;
+  };
+  {  // dB32 += (wB x)^T-rows times dS
+    GemmAcc accB;
+    accB.zero();
+    block_gemm_pipe<SPLIT>(
+        accB, lds, 0, nh * seg_k,
+        seg_stager(KcStager<SPLIT, T>(lds.ah, lds.al, nullptr, p.x_ls, qlim - st * GB, P, nullptr, nullptr, false, tid),
+                   [&](KcStager<SPLIT, T> &q, int hl) {
+                     q.base = static_cast<const T *>(p.x) + b * p.x_bs + (g * hpg + hs + hl * nsplit) * p.x_hs +
+                              (int64_t)(t0 + st * GB) * p.x_ls;
+                     q.vec = rows_aligned16(q.base, p.x_ls);
+                     q.rscale = wB[hl];
+                   },
+                   seg_k),
+        seg_stager(RcStager<SPLIT, float>(lds.bh, lds.bl, nullptr, N, N - nt * GB, P, nullptr, nullptr, false, tid,
+                                          tid < 128),
+                   [&](RcStager<SPLIT, float> &q, int hl) {
+                     q.base = p.dstates + state_off(hl);
+                     q.vec = rows_aligned16(q.base, N);
+                   },
+                   seg_k),
+        tid);
+    acc_foreach(accB, tid, [&](int m, int n, float v) {
+      const int s = st * GB + m, nn = nt * GB + n;
+      if (s < qlim && nn < N) unsafeAtomicAdd(p.dB32 + (((int64_t)b * L + t0 + s) * G + g) * N + nn, v);
+      return v;
+    });
+  }
+  {  // dC32 += (wC g) rows times H, and per head the carried-state share of ddA_cumsum
+    const int64_t Cb = b * p.C_bs + g * p.C_gs;
+    // C at this lane's 16 accumulator positions (shared by the heads of the group)
+    float cr[2][2][4];
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float rs = accH.v[tm][0][r] * cr[tm][0][r] + accH.v[tm][1][r] * cr[tm][1][r];
-        rs += dpp_f<DPP_ROW_SHR + 1>(0.f, rs);
-        rs += dpp_f<DPP_ROW_SHR + 2>(0.f, rs);
-        rs += dpp_f<DPP_ROW_SHR + 4>(0.f, rs);
-        rs += dpp_f<DPP_ROW_SHR + 8>(0.f, rs);
-        const int l = st * GB + wm * 32 + tm * 16 + gq * 4 + r;
-        if (i == 15 && l < qlim && rs != 0.f) unsafeAtomicAdd(dda + l, rs);
-      }
+      for (int tn = 0; tn < 2; ++tn)
 #pragma unroll
-    for (int ii = 0; ii < 2; ++ii)
+        for (int r = 0; r < 4; ++r) {
+          const int l = st * GB + wm * 32 + tm * 16 + gq * 4 + r, nn = nt * GB + wn * 32 + tn * 16 + i;
+          cr[tm][tn][r] = (l < qlim && nn < N) ? ldg<T>(p.C, Cb + (int64_t)(t0 + l) * p.C_ls + nn) : 0.f;
+        }
+    GemmAcc accC, accH;
+    accC.zero();
+    accH.zero();
+    block_gemm_pipe<SPLIT>(
+        accH, lds, 0, nh * seg_k,
+        seg_stager(KcStager<SPLIT, T>(lds.ah, lds.al, nullptr, gv.ls, qlim - st * GB, P, nullptr, nullptr, false, tid),
+                   [&](KcStager<SPLIT, T> &q, int hl) {
+                     q.base = static_cast<const T *>(gv.ptr) + b * gv.bs + (g * hpg + hs + hl * nsplit) * gv.hs +
+                              (int64_t)(t0 + st * GB) * gv.ls;
+                     q.vec = rows_aligned16(q.base, gv.ls);
+                     q.rscale = wC[hl];
+                   },
+                   seg_k),
+        seg_stager(RcStager<SPLIT, float>(lds.bh, lds.bl, nullptr, N, N - nt * GB, P, nullptr, nullptr, false, tid,
+                                          tid < 128),
+                   [&](RcStager<SPLIT, float> &q, int hl) {
+                     q.base = p.states + state_off(hl);
+                     q.vec = rows_aligned16(q.base, N);
+                   },
+                   seg_k),
+        tid, [&](int k0) {
+          if ((k0 + GK) % seg_k != 0) return;
+          // a head is complete: sum_n dC_h[l, n] C[l, n] goes to its ddA_cumsum row, dC_h to the sum
+          const int h = g * hpg + hs + (k0 / seg_k) * nsplit;
+          float *dda = chunk_row(p.ddA_cumsum, p, b, h, c);
 #pragma unroll
-      for (int j = 0; j < 2; ++j) accC.v[ii][j] += accH.v[ii][j];
+          for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              float rs = accH.v[tm][0][r] * cr[tm][0][r] + accH.v[tm][1][r] * cr[tm][1][r];
+              rs += dpp_f<DPP_ROW_SHR + 1>(0.f, rs);
+              rs += dpp_f<DPP_ROW_SHR + 2>(0.f, rs);
+              rs += dpp_f<DPP_ROW_SHR + 4>(0.f, rs);
+              rs += dpp_f<DPP_ROW_SHR + 8>(0.f, rs);
+              const int l = st * GB + wm * 32 + tm * 16 + gq * 4 + r;
+              if (i == 15 && l < qlim && rs != 0.f) unsafeAtomicAdd(dda + l, rs);
+            }
+#pragma unroll
+          for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              accC.v[ii][j] += accH.v[ii][j];
+              accH.v[ii][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+        });
+    acc_foreach(accC, tid, [&](int m, int n, float v) {
+      const int l = st * GB + m, nn = nt * GB + n;
+      if (l < qlim && nn < N) unsafeAtomicAdd(p.dC32 + (((int64_t)b * L + t0 + l) * G + g) * N + nn, v);
+      return v;
+    });
   }
-  acc_foreach(accB, tid, [&](int m, int n, float v) {
-    const int s = st * GB + m, nn = nt * GB + n;
-    if (s < qlim && nn < N) unsafeAtomicAdd(p.dB32 + (((int64_t)b * L + t0 + s) * G + g) * N + nn, v);
-    return v;
-  });
-  acc_foreach(accC, tid, [&](int m, int n, float v) {
-    const int l = st * GB + m, nn = nt * GB + n;
-    if (l < qlim && nn < N) unsafeAtomicAdd(p.dC32 + (((int64_t)b * L + t0 + l) * G + g) * N + nn, v);
-    return v;
-  });
 }
 
 // ------------------------------------------------------------------ dCB

@@ -277,8 +277,8 @@ DEVI void block_gemm(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, FA fa, FB
 // Software-pipelined form: sa / sb are stager objects with fetch(k0) (global -> registers) and
 // commit(k0) (registers -> LDS tile).  The fetch of step k0 + 32 is issued before the MFMAs of step
 // k0, so its latency hides behind them and behind the next barrier.
-template <bool SPLIT, typename SA, typename SB>
-DEVI void block_gemm_pipe(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, SA &&sa, SB &&sb, int tid) {
+template <bool SPLIT, typename SA, typename SB, typename AFTER>
+DEVI void block_gemm_pipe(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, SA &&sa, SB &&sb, int tid, AFTER after_step) {
   const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
   if (k_begin >= k_end) return;
   sa.fetch(k_begin);
@@ -293,7 +293,32 @@ DEVI void block_gemm_pipe(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, SA &
       sb.fetch(k0 + GK);
     }
     mma_step<SPLIT>(acc, s, wm, wn, lane);
+    after_step(k0);  // e.g. to consume and clear the accumulator at segment ends
   }
+}
+template <bool SPLIT, typename SA, typename SB>
+DEVI void block_gemm_pipe(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, SA &&sa, SB &&sb, int tid) {
+  block_gemm_pipe<SPLIT>(acc, s, k_begin, k_end, sa, sb, tid, [](int) {});
+}
+
+// A k axis made of equal segments (one per head, say), each `seg_k` long (a multiple of the k step):
+// before the first fetch of segment i, point(inner, i) re-targets the wrapped stager; inside a
+// segment the wrapped stager sees k relative to the segment start.  The pipeline then runs through
+// all segments without draining.
+template <typename Inner, typename PT> struct SegStager {
+  Inner inner;
+  PT point;
+  int seg_k;
+  DEVI SegStager(Inner inner_, PT point_, int seg_k_) : inner(inner_), point(point_), seg_k(seg_k_) {}
+  DEVI void fetch(int k0) {
+    const int seg = k0 / seg_k, kk = k0 - seg * seg_k;
+    if (kk == 0) point(inner, seg);
+    inner.fetch(kk);
+  }
+  DEVI void commit(int k0) { inner.commit(k0 % seg_k); }
+};
+template <typename Inner, typename PT> DEVI SegStager<Inner, PT> seg_stager(Inner inner, PT point, int seg_k) {
+  return SegStager<Inner, PT>(inner, point, seg_k);
 }
 
 // Stager for a causal operand on top of a row-contiguous stager: k steps below `diag_end` take an
