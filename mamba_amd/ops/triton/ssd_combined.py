@@ -79,16 +79,27 @@ def _prepare(x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, seq_idx)
     return x, dt, A, B, C, D, z, dt_bias, initial_states, seq_idx
 
 
-def _workspace(x, B, chunk_size):
+def _workspace(x, B, chunk_size, forward_state=None):
+    """fp32 workspaces of the forward stages; forward_state = (dt_out, dA_cumsum, states) re-uses the
+    ones a forward pass has filled."""
     batch, seqlen, nheads, headdim = x.shape
     ngroups, dstate = B.shape[2], B.shape[3]
     nchunks = math.ceil(seqlen / chunk_size)
     f32 = dict(device=x.device, dtype=torch.float32)
+    if forward_state is not None:
+        dt_out, dA_cumsum, states = forward_state
+        assert dt_out.shape == (batch, nheads, nchunks, chunk_size) and dA_cumsum.shape == dt_out.shape
+        assert states.shape == (batch, nchunks, nheads, headdim, dstate)
+        assert all(t.dtype == torch.float32 and t.is_contiguous() for t in forward_state)
+    else:
+        dt_out = torch.empty(batch, nheads, nchunks, chunk_size, **f32)
+        dA_cumsum = torch.empty(batch, nheads, nchunks, chunk_size, **f32)
+        states = torch.empty(batch, nchunks, nheads, headdim, dstate, **f32)
     return dict(
         nchunks=nchunks,
-        dt_out=torch.empty(batch, nheads, nchunks, chunk_size, **f32),
-        dA_cumsum=torch.empty(batch, nheads, nchunks, chunk_size, **f32),
-        states=torch.empty(batch, nchunks, nheads, headdim, dstate, **f32),
+        dt_out=dt_out,
+        dA_cumsum=dA_cumsum,
+        states=states,
         final_states=torch.empty(batch, nheads, headdim, dstate, **f32),
         CB=torch.empty(batch, nchunks, ngroups, chunk_size, chunk_size, **f32),
     )
@@ -130,9 +141,11 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
 
 def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None, z=None, dt_bias=None,
                                    initial_states=None, dfinal_states=None, seq_idx=None, dt_softplus=False,
-                                   dt_limit=(0.0, float("inf"))):
+                                   dt_limit=(0.0, float("inf")), saved=None):
     """Counterpart of ssd_combined.py:397.  `out` is the saved pre-gate output (out_x) when z is given,
-    else the forward output.  Returns (dx, ddt, dA, dB, dC, dD, dz, ddt_bias, dinitial_states)."""
+    else the forward output.  `saved` = (dt_out, dA_cumsum, states) of the forward pass skips their
+    re-computation (the reference always re-computes them, ssd_combined.py:441-448).
+    Returns (dx, ddt, dA, dB, dC, dD, dz, ddt_bias, dinitial_states)."""
     in_dtypes = (A.dtype, D.dtype if D is not None else None, dt_bias.dtype if dt_bias is not None else None,
                  initial_states.dtype if initial_states is not None else None, B.dtype, C.dtype)
     D_shape = D.shape if D is not None else None
@@ -148,7 +161,7 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
     if out.stride(-1) != 1:
         out = out.contiguous()
     dev = x.device
-    ws = _workspace(x, B, chunk_size)
+    ws = _workspace(x, B, chunk_size, forward_state=saved)
     nchunks = ws["nchunks"]
     f32 = dict(device=dev, dtype=torch.float32)
     dx = torch.empty(batch, seqlen, nheads, headdim, device=dev, dtype=x.dtype)
@@ -187,8 +200,11 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
     lib = _lib.load()
     with torch.cuda.device(dev):
         stream = _lib.current_stream(dev)
-        # re-compute the forward workspaces (the reference does the same, ssd_combined.py:441-448)
-        for stage in ("ssd_chunk_cumsum_fwd", "ssd_chunk_state_fwd", "ssd_state_passing_fwd", "ssd_bmm_chunk_fwd"):
+        # forward workspaces: kept from the forward pass, or re-computed as the reference does
+        # (ssd_combined.py:441-448); CB is always re-computed (the fused forward never forms it)
+        stages = ("ssd_bmm_chunk_fwd",) if saved is not None else (
+            "ssd_chunk_cumsum_fwd", "ssd_chunk_state_fwd", "ssd_state_passing_fwd", "ssd_bmm_chunk_fwd")
+        for stage in stages:
             _lib.check(getattr(lib, stage)(p, stream), stage)
         _lib.check(lib.ssd_combined_bwd(p, stream), "ssd_combined_bwd")
     dA = acc["dA"].to(in_dtypes[0])
@@ -198,6 +214,11 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
     dB = acc["dB32"].view(batch, seqlen, ngroups, dstate).to(in_dtypes[4])
     dC = acc["dC32"].view(batch, seqlen, ngroups, dstate).to(in_dtypes[5])
     return dx, ddt, dA, dB, dC, dD, dz, ddt_bias, dinit_out
+
+
+# Keep the forward pass's fp32 workspaces for the backward pass (288 GB of HBM make the memory cheap;
+# the re-computation costs ~7 % of a forward + backward step).  False restores the reference's behaviour.
+KEEP_FORWARD_STATE = True
 
 
 class MambaChunkScanCombinedFn(torch.autograd.Function):
@@ -214,8 +235,13 @@ class MambaChunkScanCombinedFn(torch.autograd.Function):
         out, out_x, dt_out, dA_cumsum, states, final_states, *rest = _mamba_chunk_scan_combined_fwd(
             x, dt, A, B, C, chunk_size, D=D, z=z, dt_bias=dt_bias, initial_states=initial_states, seq_idx=seq_idx,
             cu_seqlens=cu_seqlens, dt_softplus=dt_softplus, dt_limit=dt_limit, state_dtype=state_dtype)
+        # with KEEP_FORWARD_STATE the fp32 dt, cumulative decay and chunk states of the forward pass
+        # stay alive for the backward pass (batch*nchunks*nheads*headdim*dstate*4 bytes) instead of
+        # being re-computed there as in the reference (ssd_combined.py:441-448)
+        keep = (dt_out, states) if KEEP_FORWARD_STATE else ()
+        ctx.kept = len(keep) > 0
         ctx.save_for_backward(out if z is None else out_x, x, dt, dA_cumsum, A, B, C, D, z, dt_bias, initial_states,
-                              seq_idx)
+                              seq_idx, *keep)
         ctx.dt_softplus = dt_softplus
         ctx.chunk_size = chunk_size
         ctx.dt_limit = dt_limit
@@ -228,12 +254,14 @@ class MambaChunkScanCombinedFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dout, *args):
-        out, x, dt, dA_cumsum, A, B, C, D, z, dt_bias, initial_states, seq_idx = ctx.saved_tensors
+        out, x, dt, dA_cumsum, A, B, C, D, z, dt_bias, initial_states, seq_idx, *kept = ctx.saved_tensors
         assert not ctx.return_varlen_states, "return_varlen_states is not supported in backward"
         dfinal_states = args[0] if ctx.return_final_states else None
+        saved = (kept[0], dA_cumsum, kept[1]) if ctx.kept else None
         dx, ddt, dA, dB, dC, dD, dz, ddt_bias, dinitial_states = _mamba_chunk_scan_combined_bwd(
             dout, x, dt, A, B, C, out, ctx.chunk_size, D=D, z=z, dt_bias=dt_bias, initial_states=initial_states,
-            dfinal_states=dfinal_states, seq_idx=seq_idx, dt_softplus=ctx.dt_softplus, dt_limit=ctx.dt_limit)
+            dfinal_states=dfinal_states, seq_idx=seq_idx, dt_softplus=ctx.dt_softplus, dt_limit=ctx.dt_limit,
+            saved=saved)
         return (dx, ddt, dA, dB, dC, None, dD, dz, ddt_bias, dinitial_states, None, None, None, None, None, None,
                 None)
 

@@ -147,6 +147,30 @@ def test_ssd_bwd_packed_sequences(dtype):
     _bwd_case(2, 640, 4, 32, 32, 2, 128, dtype, seq_lens=[1, 127, 129, 383], has_init=False)
 
 
+def test_ssd_bwd_recompute_mode_matches_kept_state():
+    """Backward from the kept forward workspaces and backward with the reference's re-computation
+    (ssd_combined.py:441-448) give the same gradients, bit for bit."""
+    from mamba_amd.ops.triton import ssd_combined as sc
+    t = ssd_inputs(2, 600, 4, 64, 64, 2, torch.bfloat16, 5, seq_lens=None, has_init=True)
+    names = ["x", "dt", "A", "B", "C", "D", "z", "dt_bias", "initial_states"]
+    grads = []
+    for keep in (True, False):
+        old, sc.KEEP_FORWARD_STATE = sc.KEEP_FORWARD_STATE, keep
+        try:
+            g = {k: t[k].cuda().requires_grad_() for k in names}
+            out, fin = sc.mamba_chunk_scan_combined(g["x"], g["dt"], g["A"], g["B"], g["C"], 128, D=g["D"], z=g["z"],
+                                                    dt_bias=g["dt_bias"], initial_states=g["initial_states"],
+                                                    dt_softplus=True, return_final_states=True)
+            (out.float().square().sum() + fin.sum()).backward()
+            grads.append({k: g[k].grad.clone() for k in names})
+        finally:
+            sc.KEEP_FORWARD_STATE = old
+    for k in ("x", "z", "initial_states"):  # written once per element: deterministic
+        assert torch.equal(grads[0][k], grads[1][k]), k
+    for k in ("dt", "A", "B", "C", "D", "dt_bias"):  # sums of float atomics: order-dependent rounding
+        assert torch.allclose(grads[0][k].float(), grads[1][k].float(), rtol=2e-2, atol=1e-2), k
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("seq_lens", [[100, 156, 256, 1, 299, 212], [300, 84, 128, 512]])
 def test_ssd_varlen_states(seq_lens, dtype):
