@@ -112,3 +112,33 @@ def selective_state_update(state, x, dt, A, B, C, D=None, z=None, dt_bias=None, 
     if not has_heads:
         out = out.squeeze(1)
     return out
+
+
+def selective_state_update_ref(state, x, dt, A, B, C, D=None, z=None, dt_bias=None, dt_softplus=False):
+    """One decode step from plain torch operators, in place on `state`, on whatever device the
+    inputs live on (the role of the reference's selective_state_update_ref,
+    selective_state_update.py:224).  A utility for users; no op of this package calls it.
+    Shapes as selective_state_update, with or without the head dimension."""
+    import torch.nn.functional as F
+    has_heads = state.dim() > 3
+    if not has_heads:
+        state, x, dt, A, B, C = state[:, None], x[:, None], dt[:, None], A[None], B[:, None], C[:, None]
+        D = D[None] if D is not None else None
+        z = z[:, None] if z is not None else None
+        dt_bias = dt_bias[None] if dt_bias is not None else None
+    nheads, ngroups = state.shape[1], B.shape[1]
+    step = dt.float() + (dt_bias.float() if dt_bias is not None else 0.0)
+    if dt_softplus:
+        step = F.softplus(step)
+    Bh = B.float().repeat_interleave(nheads // ngroups, dim=1)       # (batch, nheads, dstate)
+    Ch = C.float().repeat_interleave(nheads // ngroups, dim=1)
+    decay = torch.exp(step[..., None] * A.float())                  # (batch, nheads, dim, dstate)
+    new_state = state.float() * decay + (step * x.float())[..., None] * Bh[:, :, None, :]
+    state.copy_(new_state)
+    out = (new_state * Ch[:, :, None, :]).sum(-1)
+    if D is not None:
+        out = out + x.float() * D.float()
+    if z is not None:
+        out = out * F.silu(z.float())
+    out = out.to(x.dtype)
+    return out if has_heads else out.squeeze(1)

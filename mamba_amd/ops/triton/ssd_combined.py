@@ -291,3 +291,236 @@ def mamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bia
     return MambaChunkScanCombinedFn.apply(x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, seq_idx,
                                           cu_seqlens, dt_softplus, dt_limit, return_final_states,
                                           return_varlen_states, state_dtype)
+
+
+def mamba_chunk_scan(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, dt_softplus=False):
+    """The stage-by-stage entry point of the reference (ssd_combined.py:651): same result as
+    mamba_chunk_scan_combined with these arguments, and served by the same kernels here."""
+    return mamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=D, z=z, dt_bias=dt_bias, dt_softplus=dt_softplus)
+
+
+def ssd_chunk_scan_combined_ref(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, dt_softplus=False):
+    """The same operator from plain torch operators on whatever device the inputs live on (the role
+    of the reference's ssd_chunk_scan_combined_ref, ssd_combined.py:687).  A utility for users; no op
+    of this package calls it.  Evaluated as the per-position recurrence in fp32 (chunk_size does not
+    change the result and is only accepted for signature compatibility)."""
+    import torch.nn.functional as F
+    batch, seqlen, nheads, headdim = x.shape
+    ngroups = B.shape[2]
+    step = dt.float() + (dt_bias.float() if dt_bias is not None else 0.0)
+    if dt_softplus:
+        step = F.softplus(step)
+    decay = torch.exp(step * A.float())                                      # (batch, seqlen, nheads)
+    Bh = B.float().repeat_interleave(nheads // ngroups, dim=2)
+    Ch = C.float().repeat_interleave(nheads // ngroups, dim=2)
+    xf = x.float()
+    state = xf.new_zeros(batch, nheads, headdim, B.shape[3])
+    ys = []
+    for t in range(seqlen):
+        state = state * decay[:, t, :, None, None] + (step[:, t, :, None] * xf[:, t])[..., None] * Bh[:, t, :, None, :]
+        ys.append((state * Ch[:, t, :, None, :]).sum(-1))
+    y = torch.stack(ys, dim=1)
+    if D is not None:
+        y = y + xf * (D.float()[..., None] if D.dim() == 1 else D.float())
+    if z is not None:
+        y = y * F.silu(z.float())
+    return y.to(x.dtype)
+
+
+def ssd_selective_scan(x, dt, A, B, C, D=None, z=None, dt_bias=None, dt_softplus=False,
+                       dt_limit=(0.0, float("inf"))):
+    """The SSD operator evaluated by the Mamba-1 selective scan kernels (ssd_combined.py:728): every
+    (head, headdim) pair becomes a channel whose states all decay with the head's A.
+    x, z: (batch, seqlen, nheads, headdim); dt: (batch, seqlen, nheads[, headdim]); A: (nheads) or
+    (nheads * headdim, dstate); B, C: (batch, seqlen, ngroups, dstate); D: (nheads[, headdim])."""
+    import torch.nn.functional as F
+    from mamba_amd.ops.selective_scan_interface import selective_scan_fn
+    batch, seqlen, nheads, headdim = x.shape
+    dstate = B.shape[3]
+    chan = lambda t: t.reshape(batch, seqlen, nheads * headdim).transpose(1, 2)      # -> (b, h*p, l)
+    dtc = dt if dt.dim() == 4 else dt[..., None].expand(batch, seqlen, nheads, headdim)
+    u, delta = chan(x), chan(dtc)
+    Af = (A.float()[:, None, None].expand(nheads, headdim, dstate).reshape(nheads * headdim, dstate)
+          if A.dim() == 1 else A.float())
+    Bc, Cc = B.permute(0, 2, 3, 1), C.permute(0, 2, 3, 1)                            # (b, g, n, l)
+    Dc = None
+    if D is not None:
+        Dc = (D.reshape(-1) if D.dim() == 2 else D[:, None].expand(nheads, headdim).reshape(-1)).float().contiguous()
+    zc = chan(z) if z is not None else None
+    bias = None
+    if dt_bias is not None:
+        bias = (dt_bias if dt_bias.dim() == 2 else dt_bias[:, None].expand(nheads, headdim)).reshape(-1).float()
+    if dt_limit != (0.0, float("inf")):
+        if bias is not None:
+            delta = delta + bias[:, None]
+        if dt_softplus:
+            delta = F.softplus(delta)
+        delta = delta.clamp(min=dt_limit[0], max=dt_limit[1]).to(x.dtype)
+        bias, dt_softplus = None, False
+    out = selective_scan_fn(u.contiguous(), delta.to(x.dtype).contiguous(), Af.contiguous(), Bc.contiguous(),
+                            Cc.contiguous(), D=Dc, z=zc.contiguous() if zc is not None else None,
+                            delta_bias=bias.contiguous() if bias is not None else None,
+                            delta_softplus=bool(dt_softplus))
+    return out.transpose(1, 2).reshape(batch, seqlen, nheads, headdim)
+
+
+def _causal_conv1d(xBC, weight, bias, activation, seq_idx=None):
+    """Depthwise causal convolution over (batch, seqlen, channels) with optional SiLU: the arithmetic
+    of the un-vendored causal_conv1d package as the reference spells it when the package is missing
+    (mamba_ssm/modules/mamba2.py:230-234).  With seq_idx, taps that reach into another sequence of a
+    packed batch contribute nothing."""
+    import torch.nn.functional as F
+    width = weight.shape[-1]
+    if seq_idx is None:
+        y = F.conv1d(xBC.transpose(1, 2), weight.unsqueeze(1), bias, padding=width - 1,
+                     groups=weight.shape[0])[..., :xBC.shape[1]].transpose(1, 2)
+    else:
+        y = xBC * weight[:, width - 1]
+        for k in range(1, width):
+            shifted = F.pad(xBC, (0, 0, k, 0))[:, :xBC.shape[1]]
+            same = F.pad(seq_idx, (k, 0), value=-1)[:, :xBC.shape[1]] == seq_idx
+            y = y + torch.where(same[..., None], shifted, torch.zeros_like(shifted)) * weight[:, width - 1 - k]
+        if bias is not None:
+            y = y + bias
+    return F.silu(y) if activation in ("silu", "swish") else y
+
+
+def _gated_rms_norm(x, weight, z, eps, group_size, norm_before_gate):
+    """RMSNorm over groups of `group_size` channels with the SiLU gate before or after it
+    (mamba_ssm/ops/triton/layernorm_gated.py:18 with bias None), computed in fp32."""
+    import torch.nn.functional as F
+    dtype = x.dtype
+    x, z = x.float(), z.float()
+    if not norm_before_gate:
+        x = x * F.silu(z)
+    xg = x.reshape(*x.shape[:-1], x.shape[-1] // group_size, group_size)
+    xg = xg * torch.rsqrt(xg.square().mean(dim=-1, keepdim=True) + eps)
+    out = xg.reshape(x.shape) * weight.float()
+    if norm_before_gate:
+        out = out * F.silu(z)
+    return out.to(dtype)
+
+
+def mamba_split_conv1d_scan_combined(zxbcdt, conv1d_weight, conv1d_bias, dt_bias, A, D, chunk_size,
+                                     initial_states=None, seq_idx=None, dt_limit=(0.0, float("inf")),
+                                     return_final_states=False, activation="silu", rmsnorm_weight=None,
+                                     rmsnorm_eps=1e-6, outproj_weight=None, outproj_bias=None, headdim=None,
+                                     ngroups=1, norm_before_gate=True, state_dtype=None):
+    """The Mamba-2 block body after in_proj (ssd_combined.py:983, forward :824-899): split, causal
+    conv1d + SiLU on xBC, the chunked scan on the HIP kernels, gate or gated RMSNorm, out_proj.
+    The convolution, the norm and the projection are torch operators and their gradients come from
+    autograd; the scan's come from MambaChunkScanCombinedFn.
+        zxbcdt: (batch, seqlen, 2 * d_nonssm + 2 * dim + 2 * ngroups * dstate + nheads), dim = nheads * headdim
+        conv1d_weight: (dim + 2 * ngroups * dstate, width); conv1d_bias: (dim + 2 * ngroups * dstate,)
+        dt_bias, A: (nheads,); D: (nheads, headdim) or (nheads,) (then headdim must be given)
+        rmsnorm_weight: (dim,); outproj_weight: (out_dim, d_nonssm + dim); outproj_bias: (out_dim,)
+        norm_before_gate: True computes RMSNorm(y) * silu(z), False RMSNorm(y * silu(z))
+    Returns out, or (out, final_states) with return_final_states."""
+    import torch.nn.functional as F
+    assert activation in [None, "silu", "swish"]
+    if D.dim() == 1:
+        assert headdim is not None
+        nheads, = D.shape
+    else:
+        nheads, headdim = D.shape
+    batch, seqlen, _ = zxbcdt.shape
+    dim = nheads * headdim
+    assert nheads % ngroups == 0
+    dstate = (conv1d_weight.shape[0] - dim) // ngroups // 2
+    d_nonssm = (zxbcdt.shape[-1] - 2 * dim - 2 * ngroups * dstate - nheads) // 2
+    assert d_nonssm >= 0
+    assert zxbcdt.shape == (batch, seqlen, 2 * d_nonssm + 2 * dim + 2 * ngroups * dstate + nheads)
+    assert dt_bias.shape == (nheads,) and A.shape == (nheads,)
+    if conv1d_weight.dim() == 3:
+        conv1d_weight = conv1d_weight.squeeze(1)
+    zx0, z, xBC, dt = torch.split(zxbcdt, [2 * d_nonssm, dim, dim + 2 * ngroups * dstate, nheads], dim=-1)
+    xBC = _causal_conv1d(xBC, conv1d_weight, conv1d_bias, activation, seq_idx)
+    x, B, C = torch.split(xBC, [dim, ngroups * dstate, ngroups * dstate], dim=-1)
+    x = x.reshape(batch, seqlen, nheads, headdim)
+    B = B.reshape(batch, seqlen, ngroups, dstate)
+    C = C.reshape(batch, seqlen, ngroups, dstate)
+    z = z.reshape(batch, seqlen, nheads, headdim)
+    res = mamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=D, z=z if rmsnorm_weight is None else None,
+                                    dt_bias=dt_bias, initial_states=initial_states, seq_idx=seq_idx, dt_softplus=True,
+                                    dt_limit=dt_limit, return_final_states=return_final_states, state_dtype=state_dtype)
+    y, final_states = res if return_final_states else (res, None)
+    y = y.reshape(batch, seqlen, dim)
+    if rmsnorm_weight is not None:
+        y = _gated_rms_norm(y, rmsnorm_weight, z.reshape(batch, seqlen, dim), rmsnorm_eps, dim // ngroups,
+                            norm_before_gate)
+    if d_nonssm > 0:
+        gate, up = zx0.chunk(2, dim=-1)
+        y = torch.cat([(F.silu(gate.float()) * up.float()).to(y.dtype), y], dim=-1)
+    if outproj_weight is not None:
+        if torch.is_autocast_enabled():
+            ac = torch.get_autocast_gpu_dtype()
+            y, outproj_weight = y.to(ac), outproj_weight.to(ac)
+            outproj_bias = outproj_bias.to(ac) if outproj_bias is not None else None
+        y = F.linear(y, outproj_weight, outproj_bias)
+    else:
+        assert outproj_bias is None
+    return y if not return_final_states else (y, final_states)
+
+
+def mamba_conv1d_scan_ref(xBC, conv1d_weight, conv1d_bias, dt, A, chunk_size, D=None, z=None, dt_bias=None,
+                          dt_softplus=False, dt_limit=(0.0, float("inf")), activation="silu", headdim=None, ngroups=1):
+    """Convolution + scan through ssd_selective_scan (the role of ssd_combined.py:779).
+    xBC: (batch, seqlen, dim + 2 * ngroups * dstate); returns (batch, seqlen, dim)."""
+    batch, seqlen, nheads = dt.shape[:3]
+    assert nheads % ngroups == 0
+    if z is not None:
+        dim = z.shape[-1]
+        assert dim % nheads == 0
+        headdim = dim // nheads
+    else:
+        if D.dim() == 1:
+            assert headdim is not None
+        else:
+            headdim = D.shape[1]
+        dim = nheads * headdim
+    if conv1d_weight.dim() == 3:
+        conv1d_weight = conv1d_weight.squeeze(1)
+    xBC = _causal_conv1d(xBC, conv1d_weight, conv1d_bias, activation)
+    dstate = (xBC.shape[-1] - dim) // ngroups // 2
+    x, B, C = torch.split(xBC, [dim, ngroups * dstate, ngroups * dstate], dim=-1)
+    out = ssd_selective_scan(x.reshape(batch, seqlen, nheads, headdim), dt.to(x.dtype), A,
+                             B.reshape(batch, seqlen, ngroups, dstate), C.reshape(batch, seqlen, ngroups, dstate),
+                             D=D.float() if D is not None else None,
+                             z=z.reshape(batch, seqlen, nheads, headdim) if z is not None else None,
+                             dt_bias=dt_bias, dt_softplus=dt_softplus, dt_limit=dt_limit)
+    return out.reshape(batch, seqlen, dim)
+
+
+def mamba_split_conv1d_scan_ref(zxbcdt, conv1d_weight, conv1d_bias, dt_bias, A, D, chunk_size,
+                                dt_limit=(0.0, float("inf")), activation="silu", rmsnorm_weight=None, rmsnorm_eps=1e-6,
+                                outproj_weight=None, outproj_bias=None, headdim=None, ngroups=1,
+                                norm_before_gate=True):
+    """mamba_split_conv1d_scan_combined with the scan routed through ssd_selective_scan (the role
+    of ssd_combined.py:1006); no d_nonssm part, no packed sequences."""
+    import torch.nn.functional as F
+    if D.dim() == 1:
+        assert headdim is not None
+        nheads, = D.shape
+    else:
+        nheads, headdim = D.shape
+    assert nheads % ngroups == 0
+    batch, seqlen, _ = zxbcdt.shape
+    dim = nheads * headdim
+    dstate = (zxbcdt.shape[-1] - 2 * dim - nheads) // ngroups // 2
+    assert zxbcdt.shape == (batch, seqlen, 2 * dim + 2 * ngroups * dstate + nheads)
+    assert dt_bias.shape == (nheads,) and A.shape == (nheads,)
+    if conv1d_weight.dim() == 3:
+        conv1d_weight = conv1d_weight.squeeze(1)
+    z, xBC, dt = torch.split(zxbcdt, [dim, dim + 2 * ngroups * dstate, nheads], dim=-1)
+    xBC = _causal_conv1d(xBC, conv1d_weight, conv1d_bias, activation)
+    x, B, C = torch.split(xBC, [dim, ngroups * dstate, ngroups * dstate], dim=-1)
+    z4 = z.reshape(batch, seqlen, nheads, headdim)
+    y = ssd_selective_scan(x.reshape(batch, seqlen, nheads, headdim), dt.to(x.dtype), A,
+                           B.reshape(batch, seqlen, ngroups, dstate), C.reshape(batch, seqlen, ngroups, dstate),
+                           D=D.float(), z=z4 if rmsnorm_weight is None else None, dt_bias=dt_bias, dt_softplus=True,
+                           dt_limit=dt_limit).reshape(batch, seqlen, dim)
+    if rmsnorm_weight is not None:
+        y = _gated_rms_norm(y, rmsnorm_weight, z, rmsnorm_eps, dim // ngroups, norm_before_gate)
+    if outproj_weight is not None:
+        y = F.linear(y, outproj_weight, outproj_bias)
+    return y
