@@ -73,6 +73,13 @@ int mamba_hip_copy(void *dst, const void *src, int64_t nbytes, mamba_stream_t st
  * csrc/selective_scan/selective_scan.cpp:254-255); its strides are ignored and
  * ngroups describes the other operand (1 when both are matrices).
  *
+ * With a_complex set (the reference's complex64 A, selective_scan.cpp:236,:312) the state is
+ * complex: A is (dim, dstate, 2) fp32 (re, im); per-position B, C are (batch, ngroups, dstate,
+ * 2 * seqlen) of `dtype` with (re, im) pairs interleaved along the last axis; input-independent
+ * B, C are (dim, dstate, 2) fp32; out = 2 Re <h, C> (+ D u, gate); ckpt gains a trailing
+ * dimension of 2, and so do dA_part and the dB32 / dC32 of input-independent operands, while the
+ * dB32 / dC32 of per-position operands are (batch, ngroups, dstate, 2 * seqlen).
+ *
  * ckpt is (batch, dim, ntiles, dstate) fp32 contiguous with
  * ntiles = ceil(seqlen / MAMBA_Q_SCAN_TILE): the state h after the last
  * position of each tile.  ckpt[:, :, ntiles-1, :] is the final state.  The
@@ -83,6 +90,8 @@ typedef struct MambaScanParams {
   int32_t dtype; /* MAMBA_F32 / MAMBA_BF16 / MAMBA_F16 */
   int32_t delta_softplus;
   int32_t bc_const; /* bit 0: B is an input-independent (dim, dstate) fp32 matrix; bit 1: C likewise */
+  int32_t a_complex; /* 1: complex A (see above) */
+  int32_t reserved0;
 
   const void *u, *delta, *A, *B, *C;
   const void *D, *z, *delta_bias; /* nullable */

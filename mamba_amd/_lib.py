@@ -19,7 +19,7 @@ c_i32, c_i64, c_vp, c_f32 = ctypes.c_int32, ctypes.c_int64, ctypes.c_void_p, cty
 
 class MambaScanParams(ctypes.Structure):
     _fields_ = (
-        [(n, c_i32) for n in ("batch", "dim", "seqlen", "dstate", "ngroups", "dtype", "delta_softplus", "bc_const")]
+        [(n, c_i32) for n in ("batch", "dim", "seqlen", "dstate", "ngroups", "dtype", "delta_softplus", "bc_const", "a_complex", "reserved0")]
         + [(n, c_vp) for n in ("u", "delta", "A", "B", "C", "D", "z", "delta_bias", "out", "ckpt")]
         + [(n, c_i64) for n in ("u_bs", "u_ds", "delta_bs", "delta_ds", "z_bs", "z_ds", "out_bs", "out_ds",
                                 "B_bs", "B_gs", "B_ns", "C_bs", "C_gs", "C_ns")]

@@ -657,11 +657,14 @@ template <typename T, bool BWD> int dispatch(const MambaScanParams &p, hipStream
 
 }  // namespace
 
+int mamba1_scan_complex(const MambaScanParams *p, hipStream_t s, bool bwd);  // mamba1_scan_complex.hip
+
 extern "C" int mamba1_scan_fwd(const MambaScanParams *p, mamba_stream_t stream) {
   int rc = check_common(p);
   if (rc != MAMBA_OK) return rc;
   if (!p->out) return MAMBA_E_BADARG;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (p->a_complex) return mamba1_scan_complex(p, s, false);
   switch (p->dtype) {
     case MAMBA_F32: return dispatch<float, false>(*p, s);
     case MAMBA_BF16: return dispatch<bf16_t, false>(*p, s);
@@ -676,6 +679,7 @@ extern "C" int mamba1_scan_bwd(const MambaScanParams *p, mamba_stream_t stream) 
     return MAMBA_E_BADARG;
   if (p->z && !p->dz) return MAMBA_E_BADARG;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (p->a_complex) return mamba1_scan_complex(p, s, true);
   switch (p->dtype) {
     case MAMBA_F32: return dispatch<float, true>(*p, s);
     case MAMBA_BF16: return dispatch<bf16_t, true>(*p, s);

@@ -28,10 +28,9 @@ def _check_inputs(u, delta, A, B, C, D, z, delta_bias):
     _lib.require_gpu(u, delta, A, B, C, D, z, delta_bias)
     if u.dtype not in _FLOAT_TYPES:
         raise RuntimeError(f"selective_scan: unsupported input dtype {u.dtype}")
-    if A.is_complex():
-        raise NotImplementedError("selective_scan: complex A is not built in mamba_amd")
-    if A.dtype != torch.float32:
-        raise RuntimeError("selective_scan: A must be float32")
+    is_complex = A.is_complex()
+    if A.dtype not in (torch.float32, torch.complex64):
+        raise RuntimeError("selective_scan: A must be float32 or complex64")
     if u.dim() != 3:
         raise RuntimeError("selective_scan: u must be (batch, dim, seqlen)")
     batch, dim, seqlen = u.shape
@@ -49,17 +48,20 @@ def _check_inputs(u, delta, A, B, C, D, z, delta_bias):
     for name, t in (("B", B), ("C", C)):
         if t.dim() == 4:
             ngroups = t.shape[1]
+    # with a complex A the matrices are complex64 and the per-position operands carry (re, im)
+    # pairs along a last axis of length 2 * seqlen (selective_scan.cpp:258-259, :268-277)
     for name, t in (("B", B), ("C", C)):
         if t.dim() == 2:
-            if t.dtype != torch.float32 or tuple(t.shape) != (dim, dstate) or not t.is_contiguous():
-                raise RuntimeError(f"selective_scan: input-independent {name} must be contiguous float32 (dim, dstate)")
+            if t.dtype != A.dtype or tuple(t.shape) != (dim, dstate) or not t.is_contiguous():
+                raise RuntimeError(f"selective_scan: input-independent {name} must be contiguous (dim, dstate) of A's dtype")
         elif t.dim() == 4:
             if t.dtype != u.dtype:
                 raise RuntimeError(f"selective_scan: {name} must have u's dtype")
             if t.stride(-1) != 1:
                 raise RuntimeError(f"selective_scan: {name} must have stride 1 in the last dimension")
-            if tuple(t.shape) != (batch, ngroups, dstate, seqlen):
-                raise RuntimeError("selective_scan: B/C must be (batch, ngroups, dstate, seqlen)")
+            if tuple(t.shape) != (batch, ngroups, dstate, seqlen * (2 if is_complex else 1)):
+                raise RuntimeError("selective_scan: B/C must be (batch, ngroups, dstate, seqlen), "
+                                   "or (..., 2 * seqlen) with a complex A")
         else:
             raise RuntimeError(f"selective_scan: {name} must be (batch, ngroups, dstate, seqlen) or (dim, dstate)")
     if tuple(delta.shape) != (batch, dim, seqlen):
@@ -83,6 +85,7 @@ def _fill_common(p, u, delta, A, B, C, D, z, delta_bias, delta_softplus, ckpt, d
     p.batch, p.dim, p.seqlen, p.dstate, p.ngroups = batch, dim, seqlen, dstate, ngroups
     p.dtype = _lib.DTYPE_CODE[u.dtype]
     p.delta_softplus = int(bool(delta_softplus))
+    p.a_complex = int(A.is_complex())
     p.u, p.delta, p.A, p.B, p.C = u.data_ptr(), delta.data_ptr(), A.data_ptr(), B.data_ptr(), C.data_ptr()
     p.D, p.z, p.delta_bias = _lib.ptr(D), _lib.ptr(z), _lib.ptr(delta_bias)
     p.ckpt = ckpt.data_ptr()
@@ -110,7 +113,8 @@ def selective_scan_fwd(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta
     A = A.contiguous()
     ntiles = (seqlen + scan_tile() - 1) // scan_tile()
     out = torch.empty_like(delta)
-    ckpt = torch.empty(batch, dim, ntiles, dstate, device=u.device, dtype=torch.float32)
+    ckpt = torch.empty((batch, dim, ntiles, dstate) + ((2,) if A.is_complex() else ()), device=u.device,
+                       dtype=torch.float32)
     p = _lib.MambaScanParams()
     _fill_common(p, u, delta, A, B, C, D, z, delta_bias, delta_softplus, ckpt, dims)
     p.out = out.data_ptr()
@@ -123,20 +127,22 @@ def selective_scan_fwd(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta
 class ScanBwdBuffers:
     """Outputs and fp32 accumulators of one backward launch (all caller-owned)."""
 
-    def __init__(self, u, delta, B, z, dims, dz=None, recompute_out_z=False, C=None):
+    def __init__(self, u, delta, B, z, dims, dz=None, recompute_out_z=False, C=None, complex_A=False):
         batch, dim, seqlen, dstate, ngroups = dims
         dev = u.device
         self.du = torch.empty_like(u)
         self.ddelta = torch.empty_like(delta)
         # one fp32 arena: per operand (batch, ngroups, dstate, seqlen) sums the kernel adds into, or
-        # (batch, dim, dstate) per-batch partials when the operand is an input-independent matrix
-        shapes = [(batch, dim, dstate) if (t is not None and t.dim() == 2) else (batch, ngroups, dstate, seqlen)
-                  for t in (B, C)]
+        # (batch, dim, dstate) per-batch partials when the operand is an input-independent matrix;
+        # with a complex A every entry is a (re, im) pair
+        two = 2 if complex_A else 1
+        shapes = [(batch, dim, dstate * two) if (t is not None and t.dim() == 2)
+                  else (batch, ngroups, dstate, seqlen * two) for t in (B, C)]
         sizes = [math.prod(sh) for sh in shapes]
         self.dBC32 = torch.empty(sum(sizes), device=dev, dtype=torch.float32)
         self.dB32 = self.dBC32[:sizes[0]].view(shapes[0])
         self.dC32 = self.dBC32[sizes[0]:].view(shapes[1])
-        self.dA_part = torch.empty(batch, dim, dstate, device=dev, dtype=torch.float32)
+        self.dA_part = torch.empty(batch, dim, dstate * two, device=dev, dtype=torch.float32)
         self.dD_part = torch.empty(batch, dim, device=dev, dtype=torch.float32)
         self.dbias_part = torch.empty(batch, dim, device=dev, dtype=torch.float32)
         self.dz = self.out_z = None
@@ -191,14 +197,16 @@ def selective_scan_bwd(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, dz=None,
                                              or dz.stride(-1) != 1):
         raise RuntimeError("selective_scan: dz must match z in dtype/shape with stride 1 in the last dimension")
     A = A.contiguous()
-    bufs = ScanBwdBuffers(u, delta, B, z, dims, dz, recompute_out_z, C=C)
+    cplx = A.is_complex()
+    bufs = ScanBwdBuffers(u, delta, B, z, dims, dz, recompute_out_z, C=C, complex_A=cplx)
     scan_bwd_zero(bufs, u.device)
     scan_bwd_launch(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, delta_softplus, bufs, dims)
-    dA = bufs.dA_part.sum(0)
+    as_A = (lambda t: torch.view_as_complex(t.reshape(dim, dstate, 2))) if cplx else (lambda t: t)
+    dA = as_A(bufs.dA_part.sum(0))
     dD = bufs.dD_part.sum(0) if D is not None else None
     ddelta_bias = bufs.dbias_part.sum(0) if delta_bias is not None else None
-    dB = bufs.dB32.sum(0) if B.dim() == 2 else bufs.dB32.to(B.dtype)
-    dC = bufs.dC32.sum(0) if C.dim() == 2 else bufs.dC32.to(C.dtype)
+    dB = as_A(bufs.dB32.sum(0)) if B.dim() == 2 else bufs.dB32.to(B.dtype)
+    dC = as_A(bufs.dC32.sum(0)) if C.dim() == 2 else bufs.dC32.to(C.dtype)
     return (bufs.du, bufs.ddelta, dA, dB, dC, dD, ddelta_bias, bufs.dz, bufs.out_z)
 
 
@@ -232,7 +240,9 @@ class SelectiveScanFn(torch.autograd.Function):
         ctx.has_z = z is not None
         ctx.has_D = D is not None
         ctx.has_bias = delta_bias is not None
-        last_state = ckpt[:, :, -1, :]  # (batch, dim, dstate)
+        last_state = ckpt[:, :, -1]  # (batch, dim, dstate)
+        if A.is_complex():
+            last_state = torch.view_as_complex(last_state)
         ctx.save_for_backward(u, delta, A, B, C, D, z, delta_bias, ckpt)
         return out if not return_last_state else (out, last_state)
 
@@ -268,25 +278,25 @@ def selective_scan_ref(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta
         delta = delta + delta_bias[..., None].float()
     if delta_softplus:
         delta = F.softplus(delta)
-    if A.is_complex():
-        raise NotImplementedError("selective_scan_ref: complex A is not built")
-    dim = A.shape[0]
+    dim, L = A.shape[0], u.shape[2]
+    cplx = A.is_complex()
 
-    def per_channel(t):  # -> (batch or 1, dim, dstate, L or 1)
+    def per_channel(t):  # -> (batch or 1, dim, dstate, L), complex when A is
         if t.dim() == 2:
-            return t.float()[None, :, :, None]
+            return (t if cplx else t.float())[None, :, :, None].expand(1, dim, A.shape[1], L)
         t = t.float() if t.dim() == 4 else t.float()[:, None]
+        if cplx:  # (re, im) pairs interleaved along the last axis
+            t = torch.view_as_complex(t.reshape(*t.shape[:-1], L, 2).contiguous())
         return t.repeat_interleave(dim // t.shape[1], dim=1)
 
     Bf, Cf = per_channel(B), per_channel(C)
-    Bf = Bf.expand(-1, -1, -1, u.shape[2]) if Bf.shape[-1] == 1 else Bf
-    Cf = Cf.expand(-1, -1, -1, u.shape[2]) if Cf.shape[-1] == 1 else Cf
-    state = u.new_zeros(u.shape[0], dim, A.shape[1])
+    state = torch.zeros(u.shape[0], dim, A.shape[1], device=u.device, dtype=A.dtype)
     ys = []
-    for t in range(u.shape[2]):
+    for t in range(L):
         step = delta[:, :, t, None]
         state = torch.exp(step * A) * state + step * u[:, :, t, None] * Bf[..., t]
-        ys.append((state * Cf[..., t]).sum(-1))
+        yt = (state * Cf[..., t]).sum(-1)
+        ys.append(2 * yt.real if cplx else yt)
     y = torch.stack(ys, dim=2)
     if D is not None:
         y = y + u * D[None, :, None]
@@ -332,11 +342,13 @@ class MambaInnerFn(torch.autograd.Function):
                 delta_softplus=True, checkpoint_lvl=1, b_rms_weight=None, c_rms_weight=None, dt_rms_weight=None,
                 b_c_dt_rms_eps=1e-6):
         assert checkpoint_lvl in [0, 1]
-        if A.is_complex():
-            raise NotImplementedError("mamba_inner_fn: complex A is not built in mamba_amd")
         L = xz.shape[-1]
         delta_rank = delta_proj_weight.shape[1]
-        d_state = A.shape[-1]
+        # x_proj emits (re, im) pairs per state when A is complex (selective_scan_interface.py:207)
+        d_state = A.shape[-1] * (1 if not A.is_complex() else 2)
+        pack = ("(b l) dstate -> b 1 dstate l" if not A.is_complex()
+                else "(b l) (dstate two) -> b 1 dstate (l two)")
+        pack_kw = dict(l=L) if not A.is_complex() else dict(l=L, two=2)
         if torch.is_autocast_enabled():
             ac = torch.get_autocast_gpu_dtype()
             x_proj_weight, delta_proj_weight = x_proj_weight.to(ac), delta_proj_weight.to(ac)
@@ -357,14 +369,14 @@ class MambaInnerFn(torch.autograd.Function):
             B = x_dbl[:, delta_rank:delta_rank + d_state]
             if B_proj_bias is not None:
                 B = B + B_proj_bias.to(dtype=B.dtype)
-            B = rearrange(B, "(b l) dstate -> b 1 dstate l", l=L).contiguous()
+            B = rearrange(B, pack, **pack_kw).contiguous()
         elif B.stride(-1) != 1:
             B = B.contiguous()
         if C is None:
             C = x_dbl[:, -d_state:]
             if C_proj_bias is not None:
                 C = C + C_proj_bias.to(dtype=C.dtype)
-            C = rearrange(C, "(b l) dstate -> b 1 dstate l", l=L).contiguous()
+            C = rearrange(C, pack, **pack_kw).contiguous()
         elif C.stride(-1) != 1:
             C = C.contiguous()
         if D is not None:
@@ -395,7 +407,10 @@ class MambaInnerFn(torch.autograd.Function):
          delta, A, B, C, D, delta_bias, ckpt) = ctx.saved_tensors
         L = xz.shape[-1]
         delta_rank = delta_proj_weight.shape[1]
-        d_state = A.shape[-1]
+        d_state = A.shape[-1] * (1 if not A.is_complex() else 2)
+        unpack = ("b 1 dstate l -> (b l) dstate" if not A.is_complex()
+                  else "b 1 dstate (l two) -> (b l) (dstate two)")
+        unpack_kw = dict() if not A.is_complex() else dict(two=2)
         x, z = xz.chunk(2, dim=1)
         if dout.stride(-1) != 1:
             dout = dout.contiguous()
@@ -423,12 +438,12 @@ class MambaInnerFn(torch.autograd.Function):
         dx_dbl = torch.empty_like(x_dbl)
         dB_proj_bias = dC_proj_bias = None
         if ctx.is_variable_B:
-            dB = rearrange(dB, "b 1 dstate l -> (b l) dstate").contiguous()
+            dB = rearrange(dB, unpack, **unpack_kw).contiguous()
             dB_proj_bias = dB.sum(0) if not ctx.B_proj_bias_is_None else None
             dx_dbl[:, delta_rank:delta_rank + d_state] = dB
             dB = None
         if ctx.is_variable_C:
-            dC = rearrange(dC, "b 1 dstate l -> (b l) dstate").contiguous()
+            dC = rearrange(dC, unpack, **unpack_kw).contiguous()
             dC_proj_bias = dC.sum(0) if not ctx.C_proj_bias_is_None else None
             dx_dbl[:, -d_state:] = dC
             dC = None
@@ -465,7 +480,9 @@ def mamba_inner_ref(xz, conv1d_weight, conv1d_bias, x_proj_weight, delta_proj_we
     mamba_inner_ref, selective_scan_interface.py:397)."""
     L = xz.shape[-1]
     delta_rank = delta_proj_weight.shape[1]
-    d_state = A.shape[-1]
+    d_state = A.shape[-1] * (1 if not A.is_complex() else 2)
+    pack = "(b l) dstate -> b dstate l" if not A.is_complex() else "(b l) (dstate two) -> b dstate (l two)"
+    pack_kw = dict(l=L) if not A.is_complex() else dict(l=L, two=2)
     x, z = xz.chunk(2, dim=1)
     x = _causal_conv1d_silu(x, rearrange(conv1d_weight, "d 1 w -> d w"), conv1d_bias)
     x_dbl = F.linear(rearrange(x, "b d l -> (b l) d"), x_proj_weight)
@@ -474,11 +491,11 @@ def mamba_inner_ref(xz, conv1d_weight, conv1d_bias, x_proj_weight, delta_proj_we
         B = x_dbl[:, delta_rank:delta_rank + d_state]
         if B_proj_bias is not None:
             B = B + B_proj_bias.to(dtype=B.dtype)
-        B = rearrange(B, "(b l) dstate -> b dstate l", l=L).contiguous()
+        B = rearrange(B, pack, **pack_kw).contiguous()
     if C is None:
         C = x_dbl[:, -d_state:]
         if C_proj_bias is not None:
             C = C + C_proj_bias.to(dtype=C.dtype)
-        C = rearrange(C, "(b l) dstate -> b dstate l", l=L).contiguous()
+        C = rearrange(C, pack, **pack_kw).contiguous()
     y = selective_scan_ref(x, delta, A, B, C, D, z=z, delta_bias=delta_bias, delta_softplus=True)
     return F.linear(rearrange(y, "b d l -> b l d"), out_proj_weight, out_proj_bias)

@@ -21,7 +21,14 @@ def mamba_inner_oracle(xz, conv1d_weight, conv1d_bias, x_proj_weight, delta_proj
     cd = compute_dtype
     batch, two_d, L = xz.shape
     d = two_d // 2
-    R, N = delta_proj_weight.shape[1], A.shape[1]
+    R = delta_proj_weight.shape[1]
+    N = A.shape[1] * (2 if A.is_complex() else 1)   # x_proj emits (re, im) pairs per state (:207, :255-258)
+
+    def pack(m):  # (b l, N) -> (b, n, L) or, complex, (b, n, 2 L) with interleaved pairs
+        if not A.is_complex():
+            return m.reshape(batch, L, N).permute(0, 2, 1)
+        return m.reshape(batch, L, N // 2, 2).permute(0, 2, 1, 3).reshape(batch, N // 2, 2 * L)
+
     x, z = xz.to(cd)[:, :d], xz.to(cd)[:, d:]
     w = conv1d_weight.to(cd)                                     # (d, 1, width)
     x = F.silu(F.conv1d(x, w, None if conv1d_bias is None else conv1d_bias.to(cd), padding=w.shape[-1] - 1,
@@ -32,17 +39,17 @@ def mamba_inner_oracle(xz, conv1d_weight, conv1d_bias, x_proj_weight, delta_proj
         Bm = x_dbl[:, R:R + N]
         if B_proj_bias is not None:
             Bm = Bm + B_proj_bias.to(cd)
-        Bm = Bm.reshape(batch, L, N).permute(0, 2, 1)
+        Bm = pack(Bm)
     else:
-        Bm = B.to(cd)
+        Bm = B if B.is_complex() else B.to(cd)
     if C is None:
         Cm = x_dbl[:, x_dbl.shape[1] - N:]
         if C_proj_bias is not None:
             Cm = Cm + C_proj_bias.to(cd)
-        Cm = Cm.reshape(batch, L, N).permute(0, 2, 1)
+        Cm = pack(Cm)
     else:
-        Cm = C.to(cd)
-    y = selective_scan_oracle(x, delta, A.to(cd), Bm, Cm, None if D is None else D.to(cd), z,
+        Cm = C if C.is_complex() else C.to(cd)
+    y = selective_scan_oracle(x, delta, A if A.is_complex() else A.to(cd), Bm, Cm, None if D is None else D.to(cd), z,
                               None if delta_bias is None else delta_bias.to(cd), True, compute_dtype=cd)
     out = y.permute(0, 2, 1) @ out_proj_weight.to(cd).t()
     if out_proj_bias is not None:

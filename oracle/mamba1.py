@@ -7,7 +7,9 @@ Restates selective_scan_ref (reference mamba_ssm/ops/selective_scan_interface.py
     out = y * silu(z), cast back to the input dtype     (:189-192)
 B, C of shape (batch, ngroups, dstate, L) are shared by the dim/ngroups channels of a
 group (:169-172); an input-independent B or C is a (dim, dstate) matrix used at every
-position (:163-166, :177-178).  Gradients come from torch.autograd through this function, which is how
+position (:163-166, :177-178).  With a complex A (:150-158) the state, A and the matrices B, C are
+complex, per-position B, C carry (re, im) pairs interleaved along their last axis (length 2L,
+:152-157), and the output is twice the real part of <h, C> (:186-187).  Gradients come from torch.autograd through this function, which is how
 the reference's own test obtains them (tests/ops/test_selective_scan.py:119-121).
 Pinned by tests/test_oracle_mamba1.py.
 """
@@ -28,9 +30,21 @@ def selective_scan_oracle(u, delta, A, B, C, D=None, z=None, delta_bias=None, de
         delta = F.softplus(delta)
     batch, dim, L = u.shape
     n = A.shape[1]
-    A = A.to(cd)
-    B = B.to(cd)
-    C = C.to(cd)
+    is_complex = A.is_complex()
+    if is_complex:
+        ccd = torch.complex64 if cd == torch.float32 else torch.complex128
+        A = A.to(ccd)
+
+        def as_complex(t):  # per-position operands: (..., 2L) real pairs -> (..., L) complex
+            if t.is_complex():
+                return t.to(ccd)
+            return torch.view_as_complex(t.to(cd).reshape(*t.shape[:-1], L, 2).contiguous())
+
+        B, C = as_complex(B), as_complex(C)
+    else:
+        A = A.to(cd)
+        B = B.to(cd)
+        C = C.to(cd)
     def per_channel(t):  # -> (b or 1, d, n, L)
         if t.dim() == 2:
             return t[None, :, :, None].expand(1, dim, n, L)
@@ -40,12 +54,13 @@ def selective_scan_oracle(u, delta, A, B, C, D=None, z=None, delta_bias=None, de
 
     B = per_channel(B)
     C = per_channel(C)
-    h = torch.zeros(batch, dim, n, dtype=cd, device=u.device)
+    h = torch.zeros(batch, dim, n, dtype=A.dtype, device=u.device)
     ys = []
     for t in range(L):
         dt = delta[:, :, t, None]                              # (b, d, 1)
         h = torch.exp(dt * A[None]) * h + (dt * u[:, :, t, None]) * B[:, :, :, t]
-        ys.append((h * C[:, :, :, t]).sum(-1))
+        yt = (h * C[:, :, :, t]).sum(-1)
+        ys.append(2 * yt.real if is_complex else yt)
     y = torch.stack(ys, dim=2)
     if D is not None:
         y = y + u * D.to(cd)[None, :, None]

@@ -21,27 +21,38 @@ def _tols(itype):
     return rtol, atol, rtolw, atolw
 
 
-def _close(name, got, ref, rtol, atol):
-    got, ref = got.detach().float().cpu(), ref.detach().float().cpu()
+def _close(name, got, ref, rtol, atol, floor=0.0):
+    """|got - ref| <= atol + rtol |ref| (+ floor * max |ref|: the fp32 summation-order noise of a
+    reduction over batch * seqlen terms, for tensors whose entries differ by orders of magnitude)."""
+    got, ref = got.detach().cpu(), ref.detach().cpu()
+    if ref.is_complex():
+        assert got.is_complex()
+        got, ref = torch.view_as_real(got), torch.view_as_real(ref)
+    got, ref = got.float(), ref.float()
     err = (got - ref).abs()
-    bound = atol + rtol * ref.abs()
+    bound = atol + rtol * ref.abs() + floor * ref.abs().max()
     assert bool((err <= bound).all()), (
         f"{name}: max err {err.max().item():.3e}, worst excess {(err - bound).max().item():.3e}, "
         f"ref max {ref.abs().max().item():.3e}")
 
 
 def _run_case(batch, dim, dstate, seqlen, itype, groups, has_z=True, has_D=True, has_bias=True,
-              softplus=True, reference_style=True, seed=0, var_B=True, var_C=True):
+              softplus=True, reference_style=True, seed=0, var_B=True, var_C=True, complex_A=False):
     from mamba_amd.ops.selective_scan_interface import selective_scan_fn
     dev = "cuda"
     rtol, atol, rtolw, atolw = _tols(itype)
     g = torch.Generator().manual_seed(seed)
     if reference_style:  # distributions of tests/ops/test_selective_scan.py:56-90
         A = -0.5 * torch.rand(dim, dstate, generator=g)
-        Bshape = (batch, dstate, seqlen) if groups == 0 else (batch, groups, dstate, seqlen)
-        # input-independent B / C are fp32 (dim, dstate) matrices (tests/ops/test_selective_scan.py:64-79)
-        B = torch.randn(*Bshape, generator=g).to(itype) if var_B else torch.randn(dim, dstate, generator=g)
-        C = torch.randn(*Bshape, generator=g).to(itype) if var_C else torch.randn(dim, dstate, generator=g)
+        two = 2 if complex_A else 1
+        Bshape = (batch, dstate, seqlen * two) if groups == 0 else (batch, groups, dstate, seqlen * two)
+        # input-independent B / C are (dim, dstate) matrices of A's dtype (tests/ops/test_selective_scan.py:64-79)
+        mat = lambda: (torch.complex(torch.randn(dim, dstate, generator=g), torch.randn(dim, dstate, generator=g))
+                       if complex_A else torch.randn(dim, dstate, generator=g))
+        if complex_A:  # wtype complex64 (tests/ops/test_selective_scan.py:59: A = -0.5 * rand, complex)
+            A = torch.complex(A, 2.0 * torch.randn(dim, dstate, generator=g))
+        B = torch.randn(*Bshape, generator=g).to(itype) if var_B else mat()
+        C = torch.randn(*Bshape, generator=g).to(itype) if var_C else mat()
         D = torch.randn(dim, generator=g) if has_D else None
         z = torch.randn(batch, dim, seqlen, generator=g).to(itype) if has_z else None
         delta_bias = 0.5 * torch.rand(dim, generator=g) if has_bias else None
@@ -73,7 +84,7 @@ def _run_case(batch, dim, dstate, seqlen, itype, groups, has_z=True, has_D=True,
     # per-gradient tolerances of tests/ops/test_selective_scan.py:135-147
     _close("du", gr("u"), rr("u"), rtol * 2, atol * 2)
     _close("ddelta", gr("delta"), rr("delta"), rtol * 5, atol * 10)
-    _close("dA", gr("A"), rr("A"), rtolw, atolw * 5)
+    _close("dA", gr("A"), rr("A"), rtolw, atolw * 5, floor=3e-5 if complex_A else 0.0)
     _close("dB", gr("B"), rr("B"), rtol if var_B else rtolw, atol if var_B else atolw)
     _close("dC", gr("C"), rr("C"), rtol if var_C else rtolw, atol if var_C else atolw)
     if has_D:
@@ -85,7 +96,7 @@ def _run_case(batch, dim, dstate, seqlen, itype, groups, has_z=True, has_D=True,
     for k in ("u", "delta", "B", "C", "z"):
         if gpu_in[k] is not None:
             assert gr(k).dtype == gpu_in[k].dtype and gr(k).shape == gpu_in[k].shape
-    assert gr("A").dtype == torch.float32
+    assert gr("A").dtype == (torch.complex64 if complex_A else torch.float32)
 
 
 @pytest.mark.parametrize("groups", [0, 1, 2])
@@ -128,3 +139,11 @@ def test_selective_scan_input_independent_B_C(var_B, var_C, itype):
     _run_case(2, 4, 8, 1024, itype, 2, var_B=var_B, var_C=var_C)
     _run_case(2, 40, 16, 700, itype, 1, var_B=var_B, var_C=var_C, has_z=False)
     _run_case(1, 6, 24, 300, itype, 1, var_B=var_B, var_C=var_C, has_bias=False)
+
+
+@pytest.mark.parametrize("itype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("var_B,var_C", [(True, True), (False, True), (True, False), (False, False)])
+def test_selective_scan_complex_A(var_B, var_C, itype):
+    # wtype complex64 of tests/ops/test_selective_scan.py:17: complex state, (re, im)-interleaved B / C
+    _run_case(2, 4, 8, 1024, itype, 2, var_B=var_B, var_C=var_C, complex_A=True)
+    _run_case(1, 6, 5, 300, itype, 1, var_B=var_B, var_C=var_C, complex_A=True, has_z=False, has_bias=False)

@@ -97,6 +97,43 @@ def test_mamba_inner_fn_given_B_C(given):
             f"d{k}: max err {(got - ref).abs().max().item():.3e}, ref max {ref.abs().max().item():.3e}"
 
 
+def test_mamba_inner_fn_complex_A():
+    """Complex A: x_proj emits (re, im) pairs per state for B and C
+    (selective_scan_interface.py:207, :255-258, :268-271)."""
+    from mamba_amd.ops.selective_scan_interface import mamba_inner_fn, mamba_inner_ref
+    g = torch.Generator().manual_seed(2)
+    batch, dim, dstate, dt_rank, d_model, L = 2, 128, 4, 8, 64, 200
+    p = _params(batch, dim, L, 2 * dstate, dt_rank, d_model, g, True)   # 2 * dstate projected columns each
+    p["A"] = torch.complex(-0.5 * torch.rand(dim, dstate, generator=g), torch.randn(dim, dstate, generator=g))
+    ref_in = {k: (v.clone().requires_grad_() if v is not None else None) for k, v in p.items()}
+    gpu_in = {k: (v.cuda().requires_grad_() if v is not None else None) for k, v in p.items()}
+    order = ["xz", "conv1d_weight", "conv1d_bias", "x_proj_weight", "delta_proj_weight", "out_proj_weight",
+             "out_proj_bias", "A"]
+    out_ref = mamba_inner_oracle(*[ref_in[k] for k in order], D=ref_in["D"], delta_bias=ref_in["delta_bias"],
+                                 B_proj_bias=ref_in["B_proj_bias"], C_proj_bias=ref_in["C_proj_bias"])
+    out = mamba_inner_fn(*[gpu_in[k] for k in order], None, None, gpu_in["D"], delta_bias=gpu_in["delta_bias"],
+                         B_proj_bias=gpu_in["B_proj_bias"], C_proj_bias=gpu_in["C_proj_bias"], delta_softplus=True)
+    scale = max(1.0, float(out_ref.detach().abs().max()))
+    assert torch.allclose(out.cpu(), out_ref, rtol=6e-4, atol=2e-3 * scale)
+    with torch.no_grad():
+        out2 = mamba_inner_ref(*[gpu_in[k].detach() for k in order], None, None, gpu_in["D"].detach(),
+                               delta_bias=gpu_in["delta_bias"].detach(), B_proj_bias=gpu_in["B_proj_bias"].detach(),
+                               C_proj_bias=gpu_in["C_proj_bias"].detach())
+    assert torch.allclose(out, out2, rtol=6e-4, atol=2e-3 * scale)
+    dout = torch.randn(out_ref.shape, generator=g)
+    out_ref.backward(dout)
+    out.backward(dout.cuda())
+    for k, v in ref_in.items():
+        if v is None:
+            continue
+        got, ref = gpu_in[k].grad.cpu(), v.grad
+        if ref.is_complex():
+            got, ref = torch.view_as_real(got), torch.view_as_real(ref)
+        s = max(1.0, float(ref.abs().max()))
+        assert torch.allclose(got, ref, rtol=5e-3, atol=5e-3 * s), \
+            f"d{k}: max err {(got - ref).abs().max().item():.3e}, ref max {ref.abs().max().item():.3e}"
+
+
 def test_install_as_mamba_ssm_ops():
     import importlib
     import mamba_amd

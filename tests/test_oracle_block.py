@@ -127,3 +127,21 @@ def test_exported_torch_utilities_match_the_oracles():
     for nbg in (True, False):
         assert torch.allclose(_gated_rms_norm(xn, wn, zn, 1e-5, 8, nbg),
                               gated_rms_norm_oracle(xn, wn, zn, 1e-5, 8, nbg).float(), atol=1e-5)
+
+
+def test_selective_scan_ref_utility_matches_the_oracle_real_and_complex():
+    from mamba_amd.ops.selective_scan_interface import selective_scan_ref
+    from oracle.mamba1 import selective_scan_oracle
+    g = torch.Generator().manual_seed(9)
+    b, d, L, n = 2, 4, 30, 3
+    u, delta, z = (torch.randn(b, d, L, generator=g) for _ in range(3))
+    D, bias = torch.randn(d, generator=g), torch.rand(d, generator=g)
+    for cplx in (False, True):
+        A = -torch.rand(d, n, generator=g)
+        if cplx:
+            A = torch.complex(A, torch.randn(d, n, generator=g))
+        Bv = torch.randn(b, 2, n, L * (2 if cplx else 1), generator=g)
+        Cm = torch.complex(torch.randn(d, n, generator=g), torch.randn(d, n, generator=g)) if cplx else torch.randn(d, n, generator=g)
+        got, st = selective_scan_ref(u, delta, A, Bv, Cm, D, z, bias, True, return_last_state=True)
+        ref, st_ref = selective_scan_oracle(u, delta, A, Bv, Cm, D, z, bias, True, return_last_state=True)
+        assert torch.allclose(got, ref, atol=1e-5) and torch.allclose(st, st_ref, atol=1e-5)

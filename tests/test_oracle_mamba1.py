@@ -154,3 +154,36 @@ def test_input_independent_B_C_matrices():
                                                     compute_dtype=f64), atol=1e-12)
     y2 = selective_scan_oracle(u, delta, A, Bv, Cm, compute_dtype=f64)
     assert torch.allclose(y2, selective_scan_oracle(u, delta, A, Bv, rep(Cm), compute_dtype=f64), atol=1e-12)
+
+
+def test_complex_A_brute_force_rotation_and_gradcheck():
+    # complex A: brute force with Python complex numbers; a pure rotation (Re A = 0) keeps |h| when the
+    # input stops; gradcheck through the complex recurrence for every input
+    g = torch.Generator().manual_seed(6)
+    b, d, L, n = 2, 2, 7, 3
+    u, delta = torch.randn(b, d, L, generator=g, dtype=f64), torch.rand(b, d, L, generator=g, dtype=f64)
+    A = torch.complex(-torch.rand(d, n, generator=g, dtype=f64), 3 * torch.randn(d, n, generator=g, dtype=f64))
+    Bv = torch.randn(b, 1, n, 2 * L, generator=g, dtype=f64)     # (re, im) interleaved along the last axis
+    Cm = torch.complex(torch.randn(d, n, generator=g, dtype=f64), torch.randn(d, n, generator=g, dtype=f64))
+    y, last = selective_scan_oracle(u, delta, A, Bv, Cm, compute_dtype=f64, return_last_state=True)
+    import cmath
+    expect = torch.zeros(b, d, L, dtype=f64)
+    for bi in range(b):
+        for di in range(d):
+            h = [0j] * n
+            for t in range(L):
+                for k in range(n):
+                    Bk = complex(float(Bv[bi, 0, k, 2 * t]), float(Bv[bi, 0, k, 2 * t + 1]))
+                    h[k] = cmath.exp(float(delta[bi, di, t]) * complex(A[di, k])) * h[k] + float(delta[bi, di, t] * u[bi, di, t]) * Bk
+                expect[bi, di, t] = 2 * sum((h[k] * complex(Cm[di, k])).real for k in range(n))
+            for k in range(n):
+                assert abs(complex(last[bi, di, k]) - h[k]) < 1e-12
+    assert torch.allclose(y, expect, atol=1e-12)
+    rot = torch.complex(torch.zeros(1, 1, dtype=f64), torch.full((1, 1), 0.7, dtype=f64))
+    uu = torch.zeros(1, 1, 6, dtype=f64)
+    uu[0, 0, 0] = 1.0
+    _, hl = selective_scan_oracle(uu, torch.ones(1, 1, 6, dtype=f64), rot, torch.ones(1, 1, dtype=f64) + 0j,
+                                  torch.ones(1, 1, dtype=f64) + 0j, compute_dtype=f64, return_last_state=True)
+    assert abs(complex(hl[0, 0, 0]) - cmath.exp(1j * 5 * 0.7)) < 1e-12   # unit modulus, phase 5 steps x 0.7
+    ins = [t.clone().requires_grad_() for t in (u[:1, :, :5], delta[:1, :, :5], A, Bv[:1, :, :, :10], Cm)]
+    assert torch.autograd.gradcheck(lambda *a: selective_scan_oracle(*a, compute_dtype=f64), ins, atol=1e-6)
