@@ -44,13 +44,13 @@ def make_inputs(batch, dim, seqlen, dstate, dtype, device, seed=0):
 
 def cpu_baseline(seqlen, dstate, full_dim):
     """Oracle (a PyTorch restatement of the reference's selective_scan_ref) forward + backward on the
-    host cores, on a batch-1 / 64-channel slice of the workload; channels and batch rows are independent
-    in the scan, so tokens/s is scaled by (64 / full_dim)."""
+    host cores, on a batch-1 / 128-channel slice of the workload; channels and batch rows are independent
+    in the scan, so tokens/s is scaled by (128 / full_dim)."""
     import torch
     from oracle.mamba1 import selective_scan_oracle, scan_inputs
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
-    dim = 256
+    dim = 128
     t = scan_inputs(1, dim, seqlen, dstate, 1, torch.bfloat16, seed=0)
     ins = {k: (v.clone().requires_grad_() if (v is not None and k != "dout") else v) for k, v in t.items()}
     t0 = time.perf_counter()

@@ -170,3 +170,48 @@ def test_decode_benchmark_shape():
                                  dt_bias=ex(bg[:, None], nheads, headdim), dt_softplus=True)
     _check(state_g, state_ref, 3e-4, 1e-3, "state")
     _check(out, out_ref, 1e-2, 1e-1, "out")
+
+
+def test_decode_step_inside_a_hip_graph():
+    """The decode step is what mamba_ssm/utils/generation.py:342-379 captures in a graph: capture one
+    step, replay it several times with eager work in between, and compare every replay with the same
+    sequence of eager steps (the op allocates nothing the graph does not own and never synchronises)."""
+    from mamba_amd.ops.triton.selective_state_update import selective_state_update
+    g = torch.Generator().manual_seed(0)
+    batch, H, P, N = 4, 8, 64, 64
+    dev = "cuda"
+    state0 = torch.randn(batch, H, P, N, generator=g).to(dev)
+    A = (-torch.rand(H, generator=g) - 1.0).to(dev)[:, None, None].expand(H, P, N)
+    D = torch.randn(H, generator=g).to(dev)[:, None].expand(H, P)
+    dtb = torch.rand(H, generator=g).to(dev)[:, None].expand(H, P)
+    steps = [dict(x=torch.randn(batch, H, P, generator=g).to(dev).bfloat16(),
+                  z=torch.randn(batch, H, P, generator=g).to(dev).bfloat16(),
+                  dt=torch.randn(batch, H, generator=g).to(dev).bfloat16(),
+                  B=torch.randn(batch, 1, N, generator=g).to(dev).bfloat16(),
+                  C=torch.randn(batch, 1, N, generator=g).to(dev).bfloat16()) for _ in range(4)]
+    call = lambda st, s: selective_state_update(st, s["x"], s["dt"][:, :, None].expand(batch, H, P), A, s["B"], s["C"],
+                                                D=D, z=s["z"], dt_bias=dtb, dt_softplus=True)
+    eager_state, eager_out = state0.clone(), []
+    for s in steps:
+        eager_out.append(call(eager_state, s).clone())
+    # static buffers of the captured step
+    gstate = state0.clone()
+    buf = {k: v.clone() for k, v in steps[0].items()}
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call(gstate, buf)                      # warm-up on the side stream
+    torch.cuda.current_stream().wait_stream(side)
+    gstate.copy_(state0)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        gout = call(gstate, buf)
+    gstate.copy_(state0)
+    for i, s in enumerate(steps):
+        for k in buf:
+            buf[k].copy_(s[k])
+        graph.replay()
+        torch.cuda.synchronize()
+        scratch = torch.randn(1024, device=dev).sum().item()   # eager work between replays
+        assert torch.equal(gout, eager_out[i]), f"replay {i}"
+    assert torch.equal(gstate, eager_state)
