@@ -161,7 +161,7 @@ def bench_ssd(dev, steps, warmup):
         "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": sec * 1e3,
         "fwd_ms": fwd_ms, "higher_is_better": True, "dtype": "bf16 in/out, fp32 accumulation", "data": "synthetic",
         "config": {"workload": f"Mamba-2 SSD fwd+bwd: batch {batch}, seqlen {L}, {H} heads x {P}, d_state {N}, "
-                               f"{G} group, chunk {Q}, bf16 (BASELINE configs[2])"},
+                               f"{G} group, chunk {Q}, bf16 (benchmark configuration 2)"},
         "roofline": {"bound": "hbm", "kernel": "chunk_scan_fwd_fused_kernel", "achieved": nbytes / scan_ms / 1e6,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / scan_ms / 1e6 / HBM_PEAK_GBS,
                      "traffic": TRAFFIC["chunk_scan_fwd_fused_kernel"], "kernel_ms": scan_ms, "algorithmic_bytes": nbytes,
@@ -194,7 +194,7 @@ def bench_decode(dev, steps, warmup):
         "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": ms, "higher_is_better": True,
         "dtype": "fp32 state, bf16 x/z/B/C/dt", "data": "synthetic",
         "config": {"workload": f"selective_state_update: batch {batch}, {H} heads x {P}, d_state {N}, {G} group, "
-                               "tied A/dt/D per head (BASELINE configs[3])"},
+                               "tied A/dt/D per head (benchmark configuration 3)"},
         "roofline": {"bound": "hbm", "kernel": "state_update_kernel", "achieved": nbytes / ms / 1e6,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / ms / 1e6 / HBM_PEAK_GBS,
                      "traffic": TRAFFIC["state_update_kernel"],
@@ -289,7 +289,7 @@ def main():
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16 in/out, fp32 state and accumulation", "data": "synthetic",
         "config": {"workload": "Mamba-1 selective_scan_fn fwd+bwd: batch 8, d_inner 5120, seqlen 4096, d_state 16, "
-                               "bf16 u/delta/B/C/z, fp32 A/D/delta_bias (BASELINE configs[1])",
+                               "bf16 u/delta/B/C/z, fp32 A/D/delta_bias (benchmark configuration 1)",
                    "global_batch": batch, "seq_len": seqlen},
         "roofline": roofline,
     }
