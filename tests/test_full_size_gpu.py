@@ -120,3 +120,47 @@ def test_decode_benchmark_configuration_full_size():
     _close("state", gstate[rows], rstate, 6e-4, 2e-3)
     untouched = torch.ones(batch, dtype=torch.bool)
     assert gstate.shape == state.shape and bool(torch.isfinite(gstate).all())
+
+
+def test_ssd_packed_long_configuration_full_size():
+    """Benchmark configuration 4: one batch row of 32768 positions packing 16 sequences (lengths in
+    [512, 4096]), 64 heads in 8 groups, initial states, final states.  A sequence in the middle of the
+    pack and the last one are compared, for two heads of different groups, with the oracle run on
+    that sequence alone (packed == separate is what the oracle's own tests pin)."""
+    from mamba_amd.ops.triton.ssd_combined import mamba_chunk_scan_combined
+    L, H, P, N, G, Q = 32768, 64, 64, 128, 8, 256
+    gen = torch.Generator().manual_seed(4)
+    lens = torch.randint(512, 4097, (16,), generator=gen).float()
+    lens = (lens / lens.sum() * L).long()
+    lens[-1] += L - lens.sum()
+    lens = [int(v) for v in lens]
+    t = ssd_inputs(1, L, H, P, N, G, torch.bfloat16, 4, seq_lens=lens, has_init=True)
+    names = ["x", "dt", "A", "B", "C", "D", "z", "dt_bias", "initial_states"]
+    g = {k: t[k].cuda().requires_grad_() for k in names}
+    out, fin = mamba_chunk_scan_combined(g["x"], g["dt"], g["A"], g["B"], g["C"], Q, D=g["D"], z=g["z"],
+                                         dt_bias=g["dt_bias"], initial_states=g["initial_states"],
+                                         seq_idx=t["seq_idx"].cuda(), dt_softplus=True, return_final_states=True)
+    dout, dfin = t["dout"].cuda(), t["dfinal"].cuda()
+    (out.float() * dout.float()).sum().add((fin * dfin).sum()).backward()
+    heads = [0, 63]
+    groups = [h // (H // G) for h in heads]
+    starts = [0]
+    for n in lens:
+        starts.append(starts[-1] + n)
+    for which in (7, 15):
+        sl = slice(starts[which], starts[which + 1])
+        for h, grp in zip(heads, groups):
+            r = dict(x=t["x"][:, sl, h:h + 1].clone().requires_grad_(), dt=t["dt"][:, sl, h:h + 1].clone().requires_grad_(),
+                     z=t["z"][:, sl, h:h + 1].clone().requires_grad_())
+            ref, rfin = ssd_oracle(r["x"], r["dt"], t["A"][h:h + 1], t["B"][:, sl, grp:grp + 1], t["C"][:, sl, grp:grp + 1],
+                                   D=t["D"][h:h + 1], z=r["z"], dt_bias=t["dt_bias"][h:h + 1], dt_softplus=True,
+                                   return_final_states=True)
+            loss = (ref.float() * t["dout"][:, sl, h:h + 1].float()).sum()
+            if which == 15:
+                loss = loss + (rfin * t["dfinal"][:, h:h + 1]).sum()
+                _close(f"final_states h{h}", fin[:, h:h + 1], rfin, 3e-2, 5e-2)
+            loss.backward()
+            _close(f"out seq{which} h{h}", out[:, sl, h:h + 1], ref, 3e-2, 5e-2)
+            _close(f"dx seq{which} h{h}", g["x"].grad[:, sl, h:h + 1], r["x"].grad, 3e-2, 5e-2, floor=4e-3)
+            _close(f"dz seq{which} h{h}", g["z"].grad[:, sl, h:h + 1], r["z"].grad, 3e-2, 5e-2, floor=4e-3)
+            _close(f"ddt seq{which} h{h}", g["dt"].grad[:, sl, h:h + 1], r["dt"].grad, 6e-2, 2e-1, floor=4e-3)
