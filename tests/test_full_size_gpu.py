@@ -23,6 +23,18 @@ def _close(name, got, ref, rtol, atol, floor=0.0):
     assert bool((err <= bound).all()), f"{name}: max err {err.max().item():.3e}, ref max {ref.abs().max().item():.3e}"
 
 
+def test_mamba1_plumbing_configuration_full_size():
+    """Configuration 0 (batch 2, 1536 channels, 2048 steps, 16 states, fp32, forward only): small
+    enough for the oracle to run whole, so every output entry and the last state are compared."""
+    from mamba_amd.ops.selective_scan_interface import selective_scan_fn
+    t = scan_inputs(2, 1536, 2048, 16, 1, torch.float32, 0)
+    names = ("u", "delta", "A", "B", "C", "D", "z", "delta_bias")
+    out, last = selective_scan_fn(*[t[k].cuda() for k in names], True, True)
+    ref, rlast = selective_scan_oracle(*[t[k] for k in names], True, True)
+    _close("out", out, ref, 6e-4, 2e-3)
+    _close("last_state", last, rlast, 6e-4, 2e-3)
+
+
 def test_mamba1_benchmark_configuration_full_size():
     from mamba_amd.ops.selective_scan_interface import selective_scan_fn
     batch, dim, L, N = 8, 5120, 4096, 16
