@@ -118,7 +118,7 @@ DEVI void load_bc(float (&v)[8], const float *staged, const void *mat, int d, in
 // BC: bit 0 = B is an input-independent (dim, dstate) fp32 matrix, bit 1 = C likewise
 // (selective_scan_fwd_kernel.cuh:74 kIsVariableB / kIsVariableC false).
 template <typename T, int NW, int R, bool VEC, int BC>
-__global__ __launch_bounds__(NW * 64) void scan_fwd_kernel(const MambaScanParams p) {
+__global__ __launch_bounds__(NW * 64, 4) void scan_fwd_kernel(const MambaScanParams p) {
   extern __shared__ __align__(16) float smem[];
   const int N = p.dstate, L = p.seqlen;
   const int NBLK = (N + NB16 - 1) / NB16, NP = NBLK * NB16;
@@ -153,7 +153,7 @@ __global__ __launch_bounds__(NW * 64) void scan_fwd_kernel(const MambaScanParams
     for (int r = 0; r < R; ++r) {
       const int d = dbase + r;
       const bool valid = d < dend;
-      float u[8], dl[8], du[8], y[8];
+      float u[8], dl[8], du[8], y[8], dsum = 0.f;
       Pack8<T> ku, kd, kz;  // raw rows: every load is issued before the first conversion
       kz.zero();
       if (valid) {
@@ -172,6 +172,8 @@ __global__ __launch_bounds__(NW * 64) void scan_fwd_kernel(const MambaScanParams
           du[i] = dl[i] * u[i];
           y[i] = 0.f;
         }
+#pragma unroll
+        for (int i = 0; i < KI; ++i) dsum += dl[i];
       }
       for (int nb = 0; nb < NBLK; ++nb) {
         if (BC != 3 && (NBLK > 1 || r == 0)) {
@@ -186,7 +188,11 @@ __global__ __launch_bounds__(NW * 64) void scan_fwd_kernel(const MambaScanParams
           // two states per iteration: their wave scans are interleaved (padded rows are inert:
           // A = 0, B = C = 0)
           for (int n = 0; n < nmax; n += 2) {
-            float a[2][8], hh[2][8], Cv[2][8], hc[2];
+            // Pass 1 runs the lane's 8 steps from a zero state to get the lane's (decay, value) pair;
+            // the decay over the lane is one exp of the summed delta instead of 7 products. Pass 2
+            // reruns the 8 steps from the state the wave scan gives this lane.
+            float a[2][8], bb[2][8], Cv[2][8], hc[2];
+            float sa[2], sb[2];
 #pragma unroll
             for (int q = 0; q < 2; ++q) {
               const float A2 = A2row[n + q];
@@ -194,25 +200,28 @@ __global__ __launch_bounds__(NW * 64) void scan_fwd_kernel(const MambaScanParams
               float Bv[8];
               load_bc<BC & 1>(Bv, Bs, p.B, d, N, nb * NB16 + n + q, n + q, lane);
               load_bc<BC & 2>(Cv[q], Cs, p.C, d, N, nb * NB16 + n + q, n + q, lane);
+              sa[q] = fast_exp2(dsum * A2);
 #pragma unroll
-              for (int i = 0; i < KI; ++i) a[q][i] = fast_exp2(dl[i] * A2);
-              hh[q][0] = du[0] * Bv[0];
-#pragma unroll
-              for (int i = 1; i < KI; ++i) {
-                hh[q][i] = __builtin_fmaf(a[q][i], hh[q][i - 1], du[i] * Bv[i]);
-                a[q][i] = a[q][i] * a[q][i - 1];  // cumulative decay inside the lane
+              for (int i = 0; i < KI; ++i) {
+                a[q][i] = fast_exp2(dl[i] * A2);
+                bb[q][i] = du[i] * Bv[i];
               }
+              float hl = bb[q][0];
+#pragma unroll
+              for (int i = 1; i < KI; ++i) hl = __builtin_fmaf(a[q][i], hl, bb[q][i]);
+              sb[q] = hl;
             }
-            float sa0 = a[0][KI - 1], sb0 = hh[0][KI - 1], sa1 = a[1][KI - 1], sb1 = hh[1][KI - 1];
-            wave_scan_fwd2(sa0, sb0, sa1, sb1);
-            const float hend[2] = {__builtin_fmaf(sa0, hc[0], sb0), __builtin_fmaf(sa1, hc[1], sb1)};
+            wave_scan_fwd2(sa[0], sb[0], sa[1], sb[1]);
+            const float hend[2] = {__builtin_fmaf(sa[0], hc[0], sb[0]), __builtin_fmaf(sa[1], hc[1], sb[1])};
 #pragma unroll
             for (int q = 0; q < 2; ++q) {
-              const float hx = dpp_f<DPP_WAVE_SHR1>(hc[q], hend[q]);  // state entering this lane
-              if (lane == 63) hrow[n + q] = hend[q];                  // state after the tile
+              float h = dpp_f<DPP_WAVE_SHR1>(hc[q], hend[q]);  // state entering this lane
+              if (lane == 63) hrow[n + q] = hend[q];           // state after the tile
 #pragma unroll
-              for (int i = 0; i < KI; ++i)
-                y[i] = __builtin_fmaf(__builtin_fmaf(a[q][i], hx, hh[q][i]), Cv[q][i], y[i]);
+              for (int i = 0; i < KI; ++i) {
+                h = __builtin_fmaf(a[q][i], h, bb[q][i]);
+                y[i] = __builtin_fmaf(h, Cv[q][i], y[i]);
+              }
             }
           }
         }
