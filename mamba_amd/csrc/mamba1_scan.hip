@@ -328,7 +328,7 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
       const int d = dbase + r;
       const bool valid = d < dend;
       const int row = wave * R + r;
-      float u[8], dl[8], du[8], dy[8], acc[8], dd[8], y[8];
+      float u[8], dl[8], du[8], dy[8], acc[8], dd[8], y[8], dsum = 0.f, dtail = 0.f;
       // raw delta, z and dout stay in registers in their storage format for the epilogue
       const Rows cur = nxt;
       Pack8<T> draw_k = cur.delta, z_k = cur.z, dout_k = cur.dout;
@@ -363,6 +363,10 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
           dd[i] = 0.f;
           y[i] = 0.f;
         }
+        dtail = 0.f;
+#pragma unroll
+        for (int i = 1; i < KI; ++i) dtail += dl[i];
+        dsum = dtail + dl[0];
         // state entering this tile
         if (NP <= 64) {
           if (lane < NP) hcar[row * NP + lane] = cur.ck;
@@ -402,8 +406,12 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
             for (int j = 0; j < NPP; j += Q) {
               const int n = slot * NPP + j;
               if (!valid || n >= nmax) continue;
+              // Forward states: pass 1 runs the lane's 8 steps from zero for the lane's (decay, value)
+              // pair, the decay being one exp of the summed delta; pass 2 reruns them from the state
+              // the wave scan gives this lane. The adjoint is handled the same way in reverse.
               float A1[Q], hc[Q], gc[Q], an[Q];
-              float Bv[Q][8], Cv[Q][8], a[Q][8], ac[Q][8], bb[Q][8], h[Q][8];
+              float Bv[Q][8], Cv[Q][8], a[Q][8], bb[Q][8], h[Q][8];
+              float sa[Q], sb[Q], hend[Q];
 #pragma unroll
               for (int q = 0; q < Q; ++q) {
                 A1[q] = A1row[n + q];
@@ -413,54 +421,43 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
                 load_bc<BC & 1>(Bv[q], Bs, p.B, d, N, nb * NB16 + n + q, n + q, lane);
                 load_bc<BC & 2>(Cv[q], Cs, p.C, d, N, nb * NB16 + n + q, n + q, lane);
                 const float A2 = A1[q] * kLog2e;
+                sa[q] = fast_exp2(dsum * A2);
 #pragma unroll
                 for (int i = 0; i < KI; ++i) {
                   a[q][i] = fast_exp2(dl[i] * A2);
                   bb[q][i] = du[i] * Bv[q][i];
                 }
-                h[q][0] = bb[q][0];
-                ac[q][0] = a[q][0];
+                float hl = bb[q][0];
 #pragma unroll
-                for (int i = 1; i < KI; ++i) {
-                  h[q][i] = __builtin_fmaf(a[q][i], h[q][i - 1], bb[q][i]);
-                  ac[q][i] = ac[q][i - 1] * a[q][i];
-                }
-              }
-              float sa[Q], sb[Q], hend[Q];
-#pragma unroll
-              for (int q = 0; q < Q; ++q) {
-                sa[q] = ac[q][KI - 1];
-                sb[q] = h[q][KI - 1];
+                for (int i = 1; i < KI; ++i) hl = __builtin_fmaf(a[q][i], hl, bb[q][i]);
+                sb[q] = hl;
               }
               if constexpr (Q == 2) wave_scan_fwd2(sa[0], sb[0], sa[1], sb[1]);
               else wave_scan_fwd(sa[0], sb[0]);
 #pragma unroll
               for (int q = 0; q < Q; ++q) hend[q] = __builtin_fmaf(sa[q], hc[q], sb[q]);
-              float gg[Q][8], ar[Q][8];
+              float ra[Q], rb[Q], gfirst[Q], a_next_lane[Q];
 #pragma unroll
               for (int q = 0; q < Q; ++q) {
-                const float hx = dpp_f<DPP_WAVE_SHR1>(hc[q], hend[q]);
+                float hp = dpp_f<DPP_WAVE_SHR1>(hc[q], hend[q]);
 #pragma unroll
-                for (int i = 0; i < KI; ++i) h[q][i] = __builtin_fmaf(ac[q][i], hx, h[q][i]);  // true states
+                for (int i = 0; i < KI; ++i) {
+                  hp = __builtin_fmaf(a[q][i], hp, bb[q][i]);
+                  h[q][i] = hp;  // true states
+                }
                 if (has_z) {
 #pragma unroll
                   for (int i = 0; i < KI; ++i) y[i] = __builtin_fmaf(h[q][i], Cv[q][i], y[i]);
                 }
-                // adjoint recurrence g[t] = dy[t] C[t] + a[t+1] g[t+1]
-                const float a_next_lane = dpp_f<DPP_WAVE_SHL1>(an[q], a[q][0]);
-                gg[q][KI - 1] = dy[KI - 1] * Cv[q][KI - 1];
-                ar[q][KI - 1] = a_next_lane;
+                // adjoint recurrence g[t] = dy[t] C[t] + a[t+1] g[t+1]; Cv becomes dy * C
+                a_next_lane[q] = dpp_f<DPP_WAVE_SHL1>(an[q], a[q][0]);
 #pragma unroll
-                for (int i = KI - 2; i >= 0; --i) {
-                  gg[q][i] = __builtin_fmaf(a[q][i + 1], gg[q][i + 1], dy[i] * Cv[q][i]);
-                  ar[q][i] = ar[q][i + 1] * a[q][i + 1];
-                }
-              }
-              float ra[Q], rb[Q], gfirst[Q];
+                for (int i = 0; i < KI; ++i) Cv[q][i] *= dy[i];
+                float gl = Cv[q][KI - 1];
 #pragma unroll
-              for (int q = 0; q < Q; ++q) {
-                ra[q] = ar[q][0];
-                rb[q] = gg[q][0];
+                for (int i = KI - 2; i >= 0; --i) gl = __builtin_fmaf(a[q][i + 1], gl, Cv[q][i]);
+                ra[q] = fast_exp2(dtail * (A1[q] * kLog2e)) * a_next_lane[q];
+                rb[q] = gl;
               }
               if constexpr (Q == 2) {
                 row_scan_rev2(ra[0], rb[0], ra[1], rb[1]);
@@ -482,9 +479,11 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
                 float sB[8], sC[8];
                 if constexpr (!(BC & 1)) lds_ld8(dBs + (n + q) * TILE, lane, sB);
                 if constexpr (!(BC & 2)) lds_ld8(dCs + (n + q) * TILE, lane, sC);
+                float gi = gx, an_i = a_next_lane[q];
 #pragma unroll
-                for (int i = 0; i < KI; ++i) {
-                  const float gi = __builtin_fmaf(ar[q][i], gx, gg[q][i]);
+                for (int i = KI - 1; i >= 0; --i) {
+                  gi = __builtin_fmaf(an_i, gi, Cv[q][i]);
+                  an_i = a[q][i];
                   if constexpr (BC & 2) dCp = __builtin_fmaf(dy[i], h[q][i], dCp);
                   else sC[i] = __builtin_fmaf(dy[i], h[q][i], sC[i]);
                   if constexpr (BC & 1) dBp = __builtin_fmaf(gi, du[i], dBp);
