@@ -199,8 +199,9 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dst
   const int tid = threadIdx.x;
   const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads;
   const int ntn = cdiv(N, GB);
-  const int pt = blockIdx.x / ntn, nt = blockIdx.x % ntn;
-  const int c = blockIdx.y, b = blockIdx.z / H, h = blockIdx.z % H;
+  const Block3 blk = xcd_block();  // the tiles of one (chunk, head) share its x / g rows: same L2
+  const int pt = blk.x / ntn, nt = blk.x % ntn;
+  const int c = blk.y, b = blk.z / H, h = blk.z % H;
   const int g = h / (H / p.ngroups);
   const int t0 = c * Q, qlim = min(Q, L - t0);
   const float *dA = chunk_row(p.dA_cumsum, p, b, h, c);
@@ -330,10 +331,13 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
   const int tid = threadIdx.x;
   const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads, G = p.ngroups;
   const int ntp = cdiv(P, GB);
-  const Block3 blk = xcd_block();
+  // Logical order: s tile fastest (the tiles of a (chunk, head) share dS and g), then head (the heads
+  // of a chunk share CB and B), then chunk, then batch, behind one L2 at a time.
+  int lid = xcd_linear_block();
   const int nst = gridDim.x / ntp;
-  const int st = blk.x % nst, pt = blk.x / nst;  // the s tiles of a (chunk, head) share dS and CB
-  const int c = blk.y, b = blk.z / H, h = blk.z % H;
+  const int st = lid % nst, pt = (lid / nst) % ntp;
+  lid /= gridDim.x;
+  const int h = lid % H, c = (lid / H) % p.nchunks, b = lid / (H * p.nchunks);
   const int g = h / (H / G);
   const int t0 = c * Q, qlim = min(Q, L - t0);
   const float *dA = chunk_row(p.dA_cumsum, p, b, h, c);

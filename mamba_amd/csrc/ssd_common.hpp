@@ -386,10 +386,14 @@ DEVI int cdiv(int a, int b) { return (a + b - 1) / b; }
 struct Block3 {
   int x, y, z;
 };
-DEVI Block3 xcd_block() {
+DEVI int xcd_linear_block() {
   const int nx = gridDim.x, ny = gridDim.y, total = nx * ny * gridDim.z;
   const int pid = blockIdx.x + nx * (blockIdx.y + ny * blockIdx.z);
   const int per = total / 8;
-  const int lid = pid < per * 8 ? (pid % 8) * per + pid / 8 : pid;
+  return pid < per * 8 ? (pid % 8) * per + pid / 8 : pid;
+}
+DEVI Block3 xcd_block() {
+  const int nx = gridDim.x, ny = gridDim.y;
+  const int lid = xcd_linear_block();
   return {lid % nx, (lid / nx) % ny, lid / (nx * ny)};
 }

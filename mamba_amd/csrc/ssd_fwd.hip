@@ -111,8 +111,9 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void chunk_s
   const int tid = threadIdx.x;
   const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads;
   const int ntn = cdiv(N, GB);
-  const int pt = blockIdx.x / ntn, nt = blockIdx.x % ntn;
-  const int c = blockIdx.y, b = blockIdx.z / H, h = blockIdx.z % H;
+  const Block3 blk = xcd_block();  // the tiles of one (chunk, head) share its x / g rows: same L2
+  const int pt = blk.x / ntn, nt = blk.x % ntn;
+  const int c = blk.y, b = blk.z / H, h = blk.z % H;
   const int g = h / (H / p.ngroups);
   const int t0 = c * Q;
   const int qlim = min(Q, L - t0);
