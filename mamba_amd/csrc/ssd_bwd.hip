@@ -225,8 +225,8 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dst
   const bool va = rows_aligned16(ga, gv.ls), vb = rows_aligned16(Ca, p.C_ls);
   block_gemm_pipe<SPLIT>(
       acc, lds, 0, qlim,
-      RcStager<SPLIT, T>(lds.ah, lds.al, ga, gv.ls, P - pt * GB, qlim, nullptr, nullptr, va, tid, tid < 128),
-      RcStager<SPLIT, T>(lds.bh, lds.bl, Ca, p.C_ls, N - nt * GB, qlim, rs, nullptr, vb, tid - 128, tid >= 128),
+      TrStager<SPLIT, T>(lds.ah, lds.al, ga, gv.ls, P - pt * GB, qlim, nullptr, nullptr, va, tid),
+      TrStager<SPLIT, T>(lds.bh, lds.bl, Ca, p.C_ls, N - nt * GB, qlim, rs, nullptr, vb, tid),
       tid);
   float *ds = p.dstates + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
   acc_foreach(acc, tid, [&](int m, int n, float v) {
@@ -399,9 +399,8 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
         acc2, lds, st * GB, qlim,
         // diagonal block: causal mask and the exact decay; below it CB^T with the rank-1 decays
         diag_stager<SPLIT>(fa, (st + 1) * GB,
-                           RcStager<SPLIT, float>(lds.ah, lds.al, CBa, Q, qlim - st * GB, qlim, kdec, rdec, va, tid - 128,
-                                                  tid >= 128)),
-        RcStager<SPLIT, T>(lds.bh, lds.bl, ga, gv.ls, P - pt * GB, qlim, nullptr, nullptr, vb, tid, tid < 128),
+                           TrStager<SPLIT, float>(lds.ah, lds.al, CBa, Q, qlim - st * GB, qlim, kdec, rdec, va, tid)),
+        TrStager<SPLIT, T>(lds.bh, lds.bl, ga, gv.ls, P - pt * GB, qlim, nullptr, nullptr, vb, tid),
         tid);
   }
   // The epilogue's x and g rows (thread t: position s = tile row t / 4, 16 consecutive p) are
@@ -542,9 +541,8 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_
                      q.rscale = wB[hl];
                    },
                    seg_k),
-        seg_stager(RcStager<SPLIT, float>(lds.bh, lds.bl, nullptr, N, N - nt * GB, P, nullptr, nullptr, false, tid,
-                                          tid < 128),
-                   [&](RcStager<SPLIT, float> &q, int hl) {
+        seg_stager(TrStager<SPLIT, float>(lds.bh, lds.bl, nullptr, N, N - nt * GB, P, nullptr, nullptr, false, tid),
+                   [&](TrStager<SPLIT, float> &q, int hl) {
                      q.base = p.dstates + state_off(hl);
                      q.vec = rows_aligned16(q.base, N);
                    },
@@ -582,9 +580,8 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_
                      q.rscale = wC[hl];
                    },
                    seg_k),
-        seg_stager(RcStager<SPLIT, float>(lds.bh, lds.bl, nullptr, N, N - nt * GB, P, nullptr, nullptr, false, tid,
-                                          tid < 128),
-                   [&](RcStager<SPLIT, float> &q, int hl) {
+        seg_stager(TrStager<SPLIT, float>(lds.bh, lds.bl, nullptr, N, N - nt * GB, P, nullptr, nullptr, false, tid),
+                   [&](TrStager<SPLIT, float> &q, int hl) {
                      q.base = p.states + state_off(hl);
                      q.vec = rows_aligned16(q.base, N);
                    },
@@ -753,7 +750,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bmm_chu
     block_gemm_pipe<SPLIT>(
         acc, lds, 0, kend,
         KcStager<SPLIT, float>(lds.ah, lds.al, da, Q, qlim - mt * GB, kend, nullptr, nullptr, va, tid),
-        RcStager<SPLIT, T>(lds.bh, lds.bl, Ba, p.B_ls, N - nt * GB, kend, nullptr, nullptr, vb, tid, tid < 128),
+        TrStager<SPLIT, T>(lds.bh, lds.bl, Ba, p.B_ls, N - nt * GB, kend, nullptr, nullptr, vb, tid),
         tid);
     acc_foreach(acc, tid, [&](int m, int n, float v) {
       const int l = mt * GB + m, nn = nt * GB + n;
@@ -770,8 +767,8 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bmm_chu
     const bool va = rows_aligned16(da, Q), vb = rows_aligned16(Ca, p.C_ls);
     block_gemm_pipe<SPLIT>(
         acc, lds, mt * GB, qlim,
-        RcStager<SPLIT, float>(lds.ah, lds.al, da, Q, qlim - mt * GB, qlim, nullptr, nullptr, va, tid, tid < 128),
-        RcStager<SPLIT, T>(lds.bh, lds.bl, Ca, p.C_ls, N - nt * GB, qlim, nullptr, nullptr, vb, tid - 128, tid >= 128),
+        TrStager<SPLIT, float>(lds.ah, lds.al, da, Q, qlim - mt * GB, qlim, nullptr, nullptr, va, tid),
+        TrStager<SPLIT, T>(lds.bh, lds.bl, Ca, p.C_ls, N - nt * GB, qlim, nullptr, nullptr, vb, tid),
         tid);
     acc_foreach(acc, tid, [&](int m, int n, float v) {
       const int s = mt * GB + m, nn = nt * GB + n;

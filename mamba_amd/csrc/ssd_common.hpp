@@ -11,6 +11,7 @@
 // (hi*hi + hi*lo + lo*hi); bf16 inputs need one.
 #pragma once
 #include "common.hpp"
+#include <type_traits>
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 
@@ -50,27 +51,45 @@ struct GemmLds {
 // stores of row-contiguous sources (8 lanes writing rows 8 apart) no longer pile on one bank.
 DEVI int tile_off(int r, int k) { return r * GLD + ((((k >> 3) ^ (r >> 3)) & (GK / 8 - 1)) << 3) + (k & 7); }
 
-template <bool SPLIT> DEVI void put8(uint16_t *hi, uint16_t *lo, int off, const float (&v)[8]) {
+// Packs 8 floats to bf16 (plus the bf16 remainders when SPLIT) and stores them with 16-byte LDS
+// writes; `ok` false stores zeros instead (the mask is applied to the packed words).
+template <bool SPLIT> DEVI void put8(uint16_t *hi, uint16_t *lo, int off, const float (&v)[8], bool ok = true) {
   uint32_t h[4];
 #pragma unroll
   for (int e = 0; e < 4; ++e) h[e] = pack_bf16(v[2 * e], v[2 * e + 1]);
-  *reinterpret_cast<u32x4 *>(hi + off) = u32x4{h[0], h[1], h[2], h[3]};
   if (SPLIT) {
     uint32_t l[4];
 #pragma unroll
-    for (int e = 0; e < 4; ++e)
+    for (int e = 0; e < 4; ++e) {
       l[e] = pack_bf16(v[2 * e] - bf16_lo(h[e]), v[2 * e + 1] - bf16_hi(h[e]));
+      l[e] = ok ? l[e] : 0u;
+    }
     *reinterpret_cast<u32x4 *>(lo + off) = u32x4{l[0], l[1], l[2], l[3]};
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) h[e] = ok ? h[e] : 0u;
+  *reinterpret_cast<u32x4 *>(hi + off) = u32x4{h[0], h[1], h[2], h[3]};
+}
+
+// A register slot that already holds 8 bf16 values goes to LDS as it is.
+template <bool SPLIT, typename S> constexpr bool kRawCopy = !SPLIT && DT<S>::id == MAMBA_BF16;
+template <typename S> DEVI void put_raw(uint16_t *hi, int off, const Pack8<S> &q, bool ok) {
+  if constexpr (DT<S>::id == MAMBA_BF16) {
+    *reinterpret_cast<u32x4 *>(hi + off) = u32x4{ok ? q.w.x : 0u, ok ? q.w.y : 0u, ok ? q.w.z : 0u, ok ? q.w.w : 0u};
   }
 }
 
 // ---- staging split into a fetch (global -> registers) and a commit (registers -> LDS) half, so
 // that the loads of the next k step are in flight while the current one is multiplied.
-// Both stagers take one task per thread with the 32-wide k step.
+// FAST is the path on which every thread's task is a whole, 16-byte aligned group of 8 elements:
+// its loads are issued unguarded from clamped (always valid) addresses and masked at commit, which
+// keeps branches away from the loads.  The guarded path (ragged or unaligned operands) takes any
+// shape.  Both stagers take one task per thread with the 32-wide k step.
 static_assert(GK == 32, "one staging task per thread");
 
 // k-contiguous source: element (r, k) at base[r * rstride + k]; thread t takes row t / 4, 8 k values.
 template <bool SPLIT, typename S> struct KcStager {
+  static constexpr bool transposed = false;
   uint16_t *hi, *lo;
   const S *base;
   int64_t rstride;
@@ -83,23 +102,35 @@ template <bool SPLIT, typename S> struct KcStager {
                 const float *kscale_, const float *rscale_, bool vec_, int t_)
       : hi(hi_), lo(lo_), base(base_), rstride(rstride_), rows_valid(rows_valid_), k_valid(k_valid_), kscale(kscale_),
         rscale(rscale_), vec(vec_), t(t_) {}
-  DEVI void fetch(int k0) {
+  DEVI bool fast() const { return vec && k_valid >= 8 && k_valid % 8 == 0 && rows_valid >= 1; }
+  template <bool FAST> DEVI void fetch(int k0) {
     const int r = t >> 2, k = k0 + (t & 3) * 8;
-    q.zero();
-    if (r < rows_valid && k < k_valid) {
-      const S *src = base + (int64_t)r * rstride + k;
-      if (vec && k + 8 <= k_valid) {
-        q.load(src);
-      } else {
-        float v[8];
+    if constexpr (FAST) {
+      q.load(base + (int64_t)min(r, rows_valid - 1) * rstride + min(k, k_valid - 8));
+    } else {
+      q.zero();
+      if (r < rows_valid && k < k_valid) {
+        const S *src = base + (int64_t)r * rstride + k;
+        if (vec && k + 8 <= k_valid) {
+          q.load(src);
+        } else {
+          float v[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = k + e < k_valid ? ld1<S>(src + e) : 0.f;
-        q.pack(v);
+          for (int e = 0; e < 8; ++e) v[e] = k + e < k_valid ? ld1<S>(src + e) : 0.f;
+          q.pack(v);
+        }
       }
     }
   }
-  DEVI void commit(int k0) {
+  template <bool FAST> DEVI void commit(int k0) {
     const int r = t >> 2, k8 = (t & 3) * 8;
+    const bool ok = !FAST || (r < rows_valid && k0 + k8 < k_valid);
+    if constexpr (kRawCopy<SPLIT, S>) {
+      if (!kscale && !rscale) {
+        put_raw<S>(hi, tile_off(r, k8), q, ok);
+        return;
+      }
+    }
     float v[8];
     q.unpack(v);
     if (kscale) {
@@ -111,13 +142,19 @@ template <bool SPLIT, typename S> struct KcStager {
 #pragma unroll
       for (int e = 0; e < 8; ++e) v[e] *= rs;
     }
-    put8<SPLIT>(hi, lo, tile_off(r, k8), v);
+    put8<SPLIT>(hi, lo, tile_off(r, k8), v, ok);
   }
 };
 
-// row-contiguous source: element (r, k) at base[k * kstride + r]; 128 threads take part (t = 0..127,
-// `active` false for the others): 2 consecutive k x 8 consecutive rows each, stored transposed.
-template <bool SPLIT, typename S> struct RcStager {
+// Row-contiguous source kept as it lies: element (r, k) at base[k * kstride + r] goes to LDS as
+// [k][r] (pitch TLD), and the MFMA fragments are read with the transposing LDS load.  Thread t takes
+// k = t / 8 and 8 consecutive rows: one 16-byte load, one 16-byte LDS store, no per-element shuffling.
+constexpr int TLD = GB + 16;  // [k][r] pitch in bf16 (160 bytes: the 4 rows of a transposing read hit disjoint banks)
+static_assert(GK * TLD <= GTILE, "the [k][r] tile fits the operand's LDS array");
+DEVI int tr_off(int k, int r) { return k * TLD + r; }
+
+template <bool SPLIT, typename S> struct TrStager {
+  static constexpr bool transposed = true;
   uint16_t *hi, *lo;
   const S *base;
   int64_t kstride;
@@ -125,74 +162,64 @@ template <bool SPLIT, typename S> struct RcStager {
   const float *kscale, *rscale;
   bool vec;
   int t;
-  bool active;
-  Pack8<S> q[2];
-  DEVI RcStager(uint16_t *hi_, uint16_t *lo_, const S *base_, int64_t kstride_, int rows_valid_, int k_valid_,
-                const float *kscale_, const float *rscale_, bool vec_, int t_, bool active_)
+  Pack8<S> q;
+  DEVI TrStager(uint16_t *hi_, uint16_t *lo_, const S *base_, int64_t kstride_, int rows_valid_, int k_valid_,
+                const float *kscale_, const float *rscale_, bool vec_, int t_)
       : hi(hi_), lo(lo_), base(base_), kstride(kstride_), rows_valid(rows_valid_), k_valid(k_valid_), kscale(kscale_),
-        rscale(rscale_), vec(vec_), t(t_), active(active_) {}
-  DEVI void fetch(int k0) {
-    if (!active) return;
-    const int k2 = (t >> 3) * 2, r8 = (t & 7) * 8;
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int k = k0 + k2 + j;
-      q[j].zero();
+        rscale(rscale_), vec(vec_), t(t_) {}
+  DEVI bool fast() const { return vec && rows_valid >= 8 && rows_valid % 8 == 0 && k_valid >= 1; }
+  template <bool FAST> DEVI void fetch(int k0) {
+    const int k = k0 + (t >> 3), r8 = (t & 7) * 8;
+    if constexpr (FAST) {
+      q.load(base + (int64_t)min(k, k_valid - 1) * kstride + min(r8, rows_valid - 8));
+    } else {
+      q.zero();
       if (k < k_valid && r8 < rows_valid) {
         const S *src = base + (int64_t)k * kstride + r8;
         if (vec && r8 + 8 <= rows_valid) {
-          q[j].load(src);
+          q.load(src);
         } else {
           float v[8];
 #pragma unroll
           for (int e = 0; e < 8; ++e) v[e] = r8 + e < rows_valid ? ld1<S>(src + e) : 0.f;
-          q[j].pack(v);
+          q.pack(v);
         }
       }
     }
   }
-  // commit with a multiplier per element, f(tile row, absolute k), instead of the scale vectors
-  template <typename F> DEVI void commit_each(int k0, F f) {
-    if (!active) return;
-    const int k2 = (t >> 3) * 2, r8 = (t & 7) * 8;
-    float v[2][8];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) q[j].unpack(v[j]);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float a = v[0][e] * f(r8 + e, k0 + k2), b = v[1][e] * f(r8 + e, k0 + k2 + 1);
-      const int off = tile_off(r8 + e, k2);
-      const uint32_t h = pack_bf16(a, b);
-      *reinterpret_cast<uint32_t *>(hi + off) = h;
-      if (SPLIT) *reinterpret_cast<uint32_t *>(lo + off) = pack_bf16(a - bf16_lo(h), b - bf16_hi(h));
-    }
+  template <bool FAST> DEVI bool task_ok(int k0) const {
+    return !FAST || (k0 + (t >> 3) < k_valid && (t & 7) * 8 < rows_valid);
   }
-  DEVI void commit(int k0) {
-    if (!active) return;
-    const int k2 = (t >> 3) * 2, r8 = (t & 7) * 8;
-    float v[2][8];
+  // commit with a multiplier per element, f(tile row, absolute k), instead of the scale vectors
+  template <bool FAST, typename F> DEVI void commit_each(int k0, F f) {
+    const int kk = t >> 3, r8 = (t & 7) * 8;
+    float v[8];
+    q.unpack(v);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      q[j].unpack(v[j]);
-      if (kscale) {
-        const float ks = kscale[k0 + k2 + j];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[j][e] *= ks;
+    for (int e = 0; e < 8; ++e) v[e] *= f(r8 + e, k0 + kk);
+    put8<SPLIT>(hi, lo, tr_off(kk, r8), v, task_ok<FAST>(k0));
+  }
+  template <bool FAST> DEVI void commit(int k0) {
+    const int kk = t >> 3, r8 = (t & 7) * 8;
+    const bool ok = task_ok<FAST>(k0);
+    if constexpr (kRawCopy<SPLIT, S>) {
+      if (!kscale && !rscale) {
+        put_raw<S>(hi, tr_off(kk, r8), q, ok);
+        return;
       }
     }
+    float v[8];
+    q.unpack(v);
+    if (kscale) {
+      const float ks = kscale[k0 + kk];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      float a = v[0][e], b = v[1][e];
-      if (rscale) {
-        const float rs = rscale[r8 + e];
-        a *= rs;
-        b *= rs;
-      }
-      const int off = tile_off(r8 + e, k2);
-      const uint32_t h = pack_bf16(a, b);
-      *reinterpret_cast<uint32_t *>(hi + off) = h;
-      if (SPLIT) *reinterpret_cast<uint32_t *>(lo + off) = pack_bf16(a - bf16_lo(h), b - bf16_hi(h));
+      for (int e = 0; e < 8; ++e) v[e] *= ks;
     }
+    if (rscale) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] *= rscale[r8 + e];
+    }
+    put8<SPLIT>(hi, lo, tr_off(kk, r8), v, ok);
   }
 };
 
@@ -231,20 +258,38 @@ struct GemmAcc {
   }
 };
 
+// MFMA fragment of a staged tile: rows row0 .. row0 + 15, lane (i, g) gets row row0 + i, k = 8 g .. 8 g + 7.
+// From a [row][k] tile that is one 16-byte load.  From a [k][row] tile (TR) it is two transposing
+// loads: in each, the 16 lanes of a k group read the 4 x 16 block of rows k .. k + 3 (lane i: row
+// k + i / 4, 4 columns from 4 (i % 4)) and the hardware hands lane i column i of the 4 rows.
+typedef short i16x4_t __attribute__((ext_vector_type(4)));
+template <bool TR> DEVI bf16x8_t load_frag(const uint16_t *tile, int row0, int i, int g) {
+  if constexpr (!TR) {
+    return *reinterpret_cast<const bf16x8_t *>(&tile[tile_off(row0 + i, g * 8)]);
+  } else {
+    typedef __attribute__((address_space(3))) i16x4_t *lds_ptr;
+    const uint16_t *src = tile + tr_off(g * 8 + (i >> 2), row0 + 4 * (i & 3));
+    const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)src);
+    const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(src + 4 * TLD));
+    typedef short i16x8_t __attribute__((ext_vector_type(8)));
+    const i16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8_t, both);
+  }
+}
+
 // One 32-deep step.  Wave (wm, wn) of the 2 x 2 grid owns rows 32*wm.. and columns 32*wn...
-template <bool SPLIT> DEVI void mma_step(GemmAcc &acc, const GemmLds &s, int wm, int wn, int lane) {
+template <bool SPLIT, bool ATR = false, bool BTR = false>
+DEVI void mma_step(GemmAcc &acc, const GemmLds &s, int wm, int wn, int lane) {
+  static_assert(GK == 32, "one MFMA k-slice per step");
   const int i = lane & 15, g = lane >> 4;
-#pragma unroll
-  for (int ks = 0; ks < GK / 32; ++ks) {
   bf16x8_t a[2], b[2], al[2], bl[2];
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
-    const int oa = tile_off(wm * 32 + t * 16 + i, ks * 32 + g * 8), ob = tile_off(wn * 32 + t * 16 + i, ks * 32 + g * 8);
-    a[t] = *reinterpret_cast<const bf16x8_t *>(&s.ah[oa]);
-    b[t] = *reinterpret_cast<const bf16x8_t *>(&s.bh[ob]);
+    a[t] = load_frag<ATR>(s.ah, wm * 32 + t * 16, i, g);
+    b[t] = load_frag<BTR>(s.bh, wn * 32 + t * 16, i, g);
     if (SPLIT) {
-      al[t] = *reinterpret_cast<const bf16x8_t *>(&s.al[oa]);
-      bl[t] = *reinterpret_cast<const bf16x8_t *>(&s.bl[ob]);
+      al[t] = load_frag<ATR>(s.al, wm * 32 + t * 16, i, g);
+      bl[t] = load_frag<BTR>(s.bl, wn * 32 + t * 16, i, g);
     }
   }
 #pragma unroll
@@ -257,7 +302,6 @@ template <bool SPLIT> DEVI void mma_step(GemmAcc &acc, const GemmLds &s, int wm,
         acc.v[tm][tn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al[tm], b[tn], acc.v[tm][tn], 0, 0, 0);
       }
     }
-  }
 }
 
 // D[m][n] += sum_{k in [k_begin, k_end)} fa(m, k) * fb(n, k) for the block's 64 x 64 tile.
@@ -274,27 +318,36 @@ DEVI void block_gemm(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, FA fa, FB
   }
 }
 
-// Software-pipelined form: sa / sb are stager objects with fetch(k0) (global -> registers) and
-// commit(k0) (registers -> LDS tile).  The fetch of step k0 + 32 is issued before the MFMAs of step
-// k0, so its latency hides behind them and behind the next barrier.
-template <bool SPLIT, typename SA, typename SB, typename AFTER>
-DEVI void block_gemm_pipe(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, SA &&sa, SB &&sb, int tid, AFTER after_step) {
+// Software-pipelined form: sa / sb are stager objects with fetch<FAST>(k0) (global -> registers)
+// and commit<FAST>(k0) (registers -> LDS tile).  The fetch of step k0 + 32 is issued before the MFMAs
+// of step k0, so its latency hides behind them and behind the next barrier.  On the FAST path the
+// fetch past the last step re-reads the last step instead (never committed), which keeps the loop
+// free of branches around loads.
+template <bool SPLIT, bool FAST, typename SA, typename SB, typename AFTER>
+DEVI void block_gemm_run(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, SA &sa, SB &sb, int tid, AFTER &after_step) {
+  constexpr bool ATR = SA::transposed, BTR = SB::transposed;
   const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
-  if (k_begin >= k_end) return;
-  sa.fetch(k_begin);
-  sb.fetch(k_begin);
-  for (int k0 = k_begin; k0 < k_end; k0 += GK) {
+  const int k_last = k_begin + (k_end - k_begin - 1) / GK * GK;
+  sa.template fetch<FAST>(k_begin);
+  sb.template fetch<FAST>(k_begin);
+  for (int k0 = k_begin; k0 <= k_last; k0 += GK) {
     __syncthreads();
-    sa.commit(k0);
-    sb.commit(k0);
+    sa.template commit<FAST>(k0);
+    sb.template commit<FAST>(k0);
     __syncthreads();
-    if (k0 + GK < k_end) {
-      sa.fetch(k0 + GK);
-      sb.fetch(k0 + GK);
+    if (FAST || k0 + GK <= k_last) {
+      sa.template fetch<FAST>(min(k0 + GK, k_last));
+      sb.template fetch<FAST>(min(k0 + GK, k_last));
     }
-    mma_step<SPLIT>(acc, s, wm, wn, lane);
+    mma_step<SPLIT, ATR, BTR>(acc, s, wm, wn, lane);
     after_step(k0);  // e.g. to consume and clear the accumulator at segment ends
   }
+}
+template <bool SPLIT, typename SA, typename SB, typename AFTER>
+DEVI void block_gemm_pipe(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, SA &&sa, SB &&sb, int tid, AFTER after_step) {
+  if (k_begin >= k_end) return;
+  if (sa.fast() && sb.fast()) block_gemm_run<SPLIT, true>(acc, s, k_begin, k_end, sa, sb, tid, after_step);
+  else block_gemm_run<SPLIT, false>(acc, s, k_begin, k_end, sa, sb, tid, after_step);
 }
 template <bool SPLIT, typename SA, typename SB>
 DEVI void block_gemm_pipe(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, SA &&sa, SB &&sb, int tid) {
@@ -304,18 +357,21 @@ DEVI void block_gemm_pipe(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, SA &
 // A k axis made of equal segments (one per head, say), each `seg_k` long (a multiple of the k step):
 // before the first fetch of segment i, point(inner, i) re-targets the wrapped stager; inside a
 // segment the wrapped stager sees k relative to the segment start.  The pipeline then runs through
-// all segments without draining.
+// all segments without draining.  The constructor points at segment 0, whose alignment stands for
+// all segments when the fast path is chosen.
 template <typename Inner, typename PT> struct SegStager {
+  static constexpr bool transposed = Inner::transposed;
   Inner inner;
   PT point;
   int seg_k;
-  DEVI SegStager(Inner inner_, PT point_, int seg_k_) : inner(inner_), point(point_), seg_k(seg_k_) {}
-  DEVI void fetch(int k0) {
+  DEVI SegStager(Inner inner_, PT point_, int seg_k_) : inner(inner_), point(point_), seg_k(seg_k_) { point(inner, 0); }
+  DEVI bool fast() const { return inner.fast(); }
+  template <bool FAST> DEVI void fetch(int k0) {
     const int seg = k0 / seg_k, kk = k0 - seg * seg_k;
     if (kk == 0) point(inner, seg);
-    inner.fetch(kk);
+    inner.template fetch<FAST>(kk);
   }
-  DEVI void commit(int k0) { inner.commit(k0 % seg_k); }
+  template <bool FAST> DEVI void commit(int k0) { inner.template commit<FAST>(k0 % seg_k); }
 };
 template <typename Inner, typename PT> DEVI SegStager<Inner, PT> seg_stager(Inner inner, PT point, int seg_k) {
   return SegStager<Inner, PT>(inner, point, seg_k);
@@ -325,14 +381,16 @@ template <typename Inner, typename PT> DEVI SegStager<Inner, PT> seg_stager(Inne
 // exact per-element multiplier f(tile row, k) (mask and decay), the others the stager's rank-1
 // scale vectors.  Either way the loads go through the same fetch.
 template <bool SPLIT, typename F, typename Inner> struct DiagStager {
+  static constexpr bool transposed = Inner::transposed;
   F f;
   int diag_end;
   Inner inner;
   DEVI DiagStager(F f_, int diag_end_, Inner inner_) : f(f_), diag_end(diag_end_), inner(inner_) {}
-  DEVI void fetch(int k0) { inner.fetch(k0); }
-  DEVI void commit(int k0) {
-    if (k0 < diag_end) inner.commit_each(k0, f);
-    else inner.commit(k0);
+  DEVI bool fast() const { return inner.fast(); }
+  template <bool FAST> DEVI void fetch(int k0) { inner.template fetch<FAST>(k0); }
+  template <bool FAST> DEVI void commit(int k0) {
+    if (k0 < diag_end) inner.template commit_each<FAST>(k0, f);
+    else inner.template commit<FAST>(k0);
   }
 };
 template <bool SPLIT, typename F, typename Inner> DEVI DiagStager<SPLIT, F, Inner> diag_stager(F f, int diag_end, Inner inner) {

@@ -142,8 +142,8 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void chunk_s
   const bool va = rows_aligned16(xa, p.x_ls), vb = rows_aligned16(Ba, p.B_ls);
   block_gemm_pipe<SPLIT>(  // the first barrier inside publishes w
       acc, lds, 0, qlim,
-      RcStager<SPLIT, T>(lds.ah, lds.al, xa, p.x_ls, P - pt * GB, qlim, nullptr, nullptr, va, tid, tid < 128),
-      RcStager<SPLIT, T>(lds.bh, lds.bl, Ba, p.B_ls, N - nt * GB, qlim, w, nullptr, vb, tid - 128, tid >= 128),
+      TrStager<SPLIT, T>(lds.ah, lds.al, xa, p.x_ls, P - pt * GB, qlim, nullptr, nullptr, va, tid),
+      TrStager<SPLIT, T>(lds.bh, lds.bl, Ba, p.B_ls, N - nt * GB, qlim, w, nullptr, vb, tid),
       tid);
   float *st = p.states + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
   acc_foreach(acc, tid, [&](int m, int n, float v) {
@@ -185,8 +185,8 @@ __global__ __launch_bounds__(256) void chunk_state_varlen_kernel(const SsdParams
     const bool va = rows_aligned16(xa, p.x_ls), vb = rows_aligned16(Ba, p.B_ls);
     block_gemm_pipe<SPLIT>(  // the first barrier inside publishes w
         acc, lds, kstart / GK * GK, kend,
-        RcStager<SPLIT, T>(lds.ah, lds.al, xa, p.x_ls, P - pt * GB, kend, nullptr, nullptr, va, tid, tid < 128),
-        RcStager<SPLIT, T>(lds.bh, lds.bl, Ba, p.B_ls, N - nt * GB, kend, w, nullptr, vb, tid - 128, tid >= 128),
+        TrStager<SPLIT, T>(lds.ah, lds.al, xa, p.x_ls, P - pt * GB, kend, nullptr, nullptr, va, tid),
+        TrStager<SPLIT, T>(lds.bh, lds.bl, Ba, p.B_ls, N - nt * GB, kend, w, nullptr, vb, tid),
         tid);
     if (start < t0) {
       const float *Hc = p.states + ((int64_t)c * H + h) * P * N;
