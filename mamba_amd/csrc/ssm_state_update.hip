@@ -63,7 +63,11 @@ constexpr int UNR = SSU_UNR;  // row passes per wave
 // states past the end are read from clamped (valid) addresses and masked afterwards, and absent
 // optional operands read a stand-in address with a zero weight.  A load under a branch would make
 // the compiler wait for all earlier loads at that point, which serialises the memory round trips.
-template <typename TS, typename TX, typename TB, typename TD, bool VEC>
+// SHARE (with VEC): B and C are contiguous and aligned, so a lane's 4 values are one load each, and
+// the wave has at most 64 rows, so lane j loads the per-row scalars (x, dt, dt_bias, z, D) of row j
+// once and the lanes of a row pick them up through the LDS crossbar: 15 vector-memory instructions
+// per wave instead of 36 for the same 4 KB of state.
+template <typename TS, typename TX, typename TB, typename TD, bool VEC, bool SHARE>
 __global__ __launch_bounds__(256) void state_update_kernel(const MambaStepParams p, int lpr_log2) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -123,19 +127,42 @@ __global__ __launch_bounds__(256) void state_update_kernel(const MambaStepParams
     } else {
       ld_state4<TS, false>(state + rc * s_ps + n0 * s_ns, s_ns, live[k] ? nlane : 0, s[k]);
     }
-    xs[k] = ld1<TX>(xp + rc * x_ps);
-    dts[k] = ld1<TD>(dtp + rc * dt_ps);
-    dtbs[k] = dtb[rc * dtb_ps];
-    zs[k] = ld1<TX>(zp + rc * z_ps);
-    Ds[k] = Dp[rc * D_ps];
+    if constexpr (!SHARE) {
+      xs[k] = ld1<TX>(xp + rc * x_ps);
+      dts[k] = ld1<TD>(dtp + rc * dt_ps);
+      dtbs[k] = dtb[rc * dtb_ps];
+      zs[k] = ld1<TX>(zp + rc * z_ps);
+      Ds[k] = Dp[rc * D_ps];
+    }
   }
   float Bv[4], Cv[4], Av[4];
+  float x_j = 0.f, dt_j = 0.f, dtb_j = 0.f, z_j = 0.f, D_j = 0.f;  // SHARE: the scalars of row p_begin + lane
+  if constexpr (SHARE) {
+    const int rj = min(p_begin + lane, p.dim - 1);
+    x_j = ld1<TX>(xp + rj * x_ps);
+    dt_j = ld1<TD>(dtp + rj * dt_ps);
+    dtb_j = dtb[rj * dtb_ps];
+    z_j = ld1<TX>(zp + rj * z_ps);
+    D_j = Dp[rj * D_ps];
+    ld_state4<TB, true>(Bp + n0c, 1, 4, Bv);
+    ld_state4<TB, true>(Cp + n0c, 1, 4, Cv);
+  }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int nc = min(n0 + i, N - 1);
-    Bv[i] = ld1<TB>(Bp + nc * B_ns);
-    Cv[i] = ld1<TB>(Cp + nc * C_ns);
-    Av[i] = Ap[nc * A_ns];
+    if constexpr (!SHARE) {
+      Bv[i] = ld1<TB>(Bp + nc * B_ns);
+      Cv[i] = ld1<TB>(Cp + nc * C_ns);
+    }
+    if (!SHARE || i == 0) Av[i] = Ap[nc * A_ns];
+  }
+  if constexpr (SHARE) {  // one A per head (stride 0 along the states) needs no further loads
+    if (A_ns != 0) {
+#pragma unroll
+      for (int i = 1; i < 4; ++i) Av[i] = Ap[min(n0 + i, N - 1) * A_ns];
+    } else {
+      Av[1] = Av[2] = Av[3] = Av[0];
+    }
   }
   if (A_per_row) {  // uniform; the block holds loads only
 #pragma unroll
@@ -146,6 +173,17 @@ __global__ __launch_bounds__(256) void state_update_kernel(const MambaStepParams
     }
   }
   // 2. masks and per-head values
+  if constexpr (SHARE) {
+#pragma unroll
+    for (int k = 0; k < UNR; ++k) {
+      const int src = rsel + k * rpp;  // the lane that holds this row's scalars
+      xs[k] = __shfl(x_j, src, 64);
+      dts[k] = __shfl(dt_j, src, 64);
+      dtbs[k] = __shfl(dtb_j, src, 64);
+      zs[k] = __shfl(z_j, src, 64);
+      Ds[k] = __shfl(D_j, src, 64);
+    }
+  }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const bool ok = i < nlane;
@@ -208,7 +246,19 @@ int launch(const MambaStepParams &p, hipStream_t stream) {
   while ((4 << lpr_log2) < p.dstate) ++lpr_log2;  // dstate <= 256 -> lpr <= 64
   const int rows_per_block = 4 * (64 >> lpr_log2) * UNR;
   dim3 grid((p.dim + rows_per_block - 1) / rows_per_block, p.nheads, p.batch), block(256);
-  hipLaunchKernelGGL((state_update_kernel<TS, TX, TB, TD, VEC>), grid, block, 0, stream, p, lpr_log2);
+  if constexpr (VEC) {
+    // the shared loads need contiguous, aligned B / C rows and at most 64 rows per wave
+    const int64_t eb = sizeof(TB), ab = 4 * eb;
+    const bool share = (64 >> lpr_log2) * UNR <= 64 && p.B_ns == 1 && p.C_ns == 1 &&
+                       reinterpret_cast<uintptr_t>(p.B) % ab == 0 && reinterpret_cast<uintptr_t>(p.C) % ab == 0 &&
+                       (p.B_bs * eb) % ab == 0 && (p.B_gs * eb) % ab == 0 && (p.C_bs * eb) % ab == 0 &&
+                       (p.C_gs * eb) % ab == 0;
+    if (share) {
+      hipLaunchKernelGGL((state_update_kernel<TS, TX, TB, TD, true, true>), grid, block, 0, stream, p, lpr_log2);
+      return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
+    }
+  }
+  hipLaunchKernelGGL((state_update_kernel<TS, TX, TB, TD, VEC, false>), grid, block, 0, stream, p, lpr_log2);
   return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
 }
 
