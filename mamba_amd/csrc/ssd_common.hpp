@@ -304,6 +304,109 @@ DEVI void mma_step(GemmAcc &acc, const GemmLds &s, int wm, int wn, int lane) {
     }
 }
 
+// ---- wide variant: a 64 x 128 tile per workgroup, 32 x 64 per wave, both operands row-contiguous
+// ([k][row] in LDS).  Per MFMA it moves three quarters of the LDS and global bytes of the 64 x 64 core.
+constexpr int WB = 128;          // columns of the wide tile
+constexpr int WLD = WB + 16;     // [k][row] pitch of the wide operand (288 bytes)
+template <bool SPLIT> struct GemmLdsWide {
+  uint16_t ah[GK * TLD], al[SPLIT ? GK * TLD : 8], bh[GK * WLD], bl[SPLIT ? GK * WLD : 8];
+};
+struct GemmAccWide {
+  f32x4 v[2][4];
+  DEVI void zero() {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+};
+template <int PITCH> DEVI bf16x8_t load_frag_tr(const uint16_t *tile, int row0, int i, int g) {
+  typedef __attribute__((address_space(3))) i16x4_t *lds_ptr;
+  typedef short i16x8_t __attribute__((ext_vector_type(8)));
+  const uint16_t *src = tile + (g * 8 + (i >> 2)) * PITCH + row0 + 4 * (i & 3);
+  const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)src);
+  const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(src + 4 * PITCH));
+  return __builtin_bit_cast(bf16x8_t, (i16x8_t)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+// Stages ROWS rows x 32 k of a row-contiguous operand (element (r, k) at base[k * kstride + r]) as
+// [k][r]: thread t takes k = t / 8 and, per 64 rows, 8 consecutive rows from 8 (t % 8).  The operand
+// must be 16-byte aligned with rows_valid a multiple of 8 and k_valid a multiple of 32 (the caller
+// checks); rows past rows_valid re-read the last rows and are zeroed.
+template <bool SPLIT, typename S, int ROWS> struct WideTrStager {
+  static constexpr int NT = ROWS / 64, PITCH = ROWS + 16;
+  uint16_t *hi, *lo;
+  const S *base;
+  int64_t kstride;
+  int rows_valid;
+  const float *kscale;
+  int t;
+  Pack8<S> q[NT];
+  DEVI WideTrStager(uint16_t *hi_, uint16_t *lo_, const S *base_, int64_t kstride_, int rows_valid_, const float *kscale_, int t_)
+      : hi(hi_), lo(lo_), base(base_), kstride(kstride_), rows_valid(rows_valid_), kscale(kscale_), t(t_) {}
+  DEVI void fetch(int k0) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+      q[j].load(base + (int64_t)(k0 + (t >> 3)) * kstride + min((t & 7) * 8 + 64 * j, rows_valid - 8));
+  }
+  DEVI void commit(int k0) {
+    const int kk = t >> 3;
+    const float ks = kscale ? kscale[k0 + kk] : 1.f;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const int r8 = (t & 7) * 8 + 64 * j, off = kk * PITCH + r8;
+      if (r8 >= rows_valid) {
+        const float zero[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        put8<SPLIT>(hi, lo, off, zero);
+      } else if (kRawCopy<SPLIT, S> && !kscale) {
+        put_raw<S>(hi, off, q[j], true);
+      } else {
+        float v[8];
+        q[j].unpack(v);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] *= ks;
+        put8<SPLIT>(hi, lo, off, v);
+      }
+    }
+  }
+};
+// acc[m][n] += sum_k A[m][k] B[n][k] over k in [0, k_end), k_end a multiple of 32.
+template <bool SPLIT, typename SA, typename SB>
+DEVI void block_gemm_wide(GemmAccWide &acc, GemmLdsWide<SPLIT> &s, int k_end, SA &sa, SB &sb, int tid) {
+  const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+  const int i = lane & 15, g = lane >> 4;
+  sa.fetch(0);
+  sb.fetch(0);
+  for (int k0 = 0; k0 < k_end; k0 += GK) {
+    __syncthreads();
+    sa.commit(k0);
+    sb.commit(k0);
+    __syncthreads();
+    sa.fetch(min(k0 + GK, k_end - GK));
+    sb.fetch(min(k0 + GK, k_end - GK));
+    bf16x8_t a[2], b[4], al[2], bl[4];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      a[t] = load_frag_tr<TLD>(s.ah, wm * 32 + t * 16, i, g);
+      if (SPLIT) al[t] = load_frag_tr<TLD>(s.al, wm * 32 + t * 16, i, g);
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      b[t] = load_frag_tr<WLD>(s.bh, wn * 64 + t * 16, i, g);
+      if (SPLIT) bl[t] = load_frag_tr<WLD>(s.bl, wn * 64 + t * 16, i, g);
+    }
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < 4; ++tn) {
+        acc.v[tm][tn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[tm], b[tn], acc.v[tm][tn], 0, 0, 0);
+        if (SPLIT) {
+          acc.v[tm][tn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[tm], bl[tn], acc.v[tm][tn], 0, 0, 0);
+          acc.v[tm][tn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al[tm], b[tn], acc.v[tm][tn], 0, 0, 0);
+        }
+      }
+  }
+}
+
 // D[m][n] += sum_{k in [k_begin, k_end)} fa(m, k) * fb(n, k) for the block's 64 x 64 tile.
 // fa / fb return 0 outside their valid ranges.  All 256 threads must call.
 template <bool SPLIT, bool A_KFAST, bool B_KFAST, typename FA, typename FB>

@@ -153,6 +153,56 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void chunk_s
   });
 }
 
+// The same product with a 64 x 128 tile per workgroup, for whole 128-state blocks of aligned operands
+// and chunks that are whole k steps.
+template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void chunk_state_fwd_wide_kernel(const SsdParams p) {
+  __shared__ GemmLdsWide<SPLIT> lds;
+  __shared__ float w[256];
+  const int tid = threadIdx.x;
+  const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads;
+  const int ntn = N / WB;
+  const Block3 blk = xcd_block();
+  const int pt = blk.x / ntn, nt = blk.x % ntn;
+  const int c = blk.y, b = blk.z / H, h = blk.z % H;
+  const int g = h / (H / p.ngroups);
+  const int t0 = c * Q;
+  const int qlim = min(Q, L - t0);
+  const float *dA = p.dA_cumsum + (((int64_t)b * H + h) * p.nchunks + c) * Q;
+  const float *dt = p.dt_out + (((int64_t)b * H + h) * p.nchunks + c) * Q;
+  const float a_last = dA[Q - 1];
+  const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
+  for (int s = tid; s < Q; s += 256) {
+    float v = 0.f;
+    if (s < qlim) {
+      bool ok = true;
+      if (seq) {
+        const int last = seq[qlim - 1];
+        ok = last >= 0 && seq[s] == last;
+      }
+      if (ok) v = fast_exp(fminf(a_last - dA[s], 0.f)) * dt[s];
+    }
+    w[s] = v;
+  }
+  const T *xa = static_cast<const T *>(p.x) + b * p.x_bs + h * p.x_hs + (int64_t)t0 * p.x_ls + pt * GB;
+  const T *Ba = static_cast<const T *>(p.B) + b * p.B_bs + g * p.B_gs + (int64_t)t0 * p.B_ls + nt * WB;
+  GemmAccWide acc;
+  acc.zero();
+  WideTrStager<SPLIT, T, 64> sa(lds.ah, lds.al, xa, p.x_ls, P - pt * GB, nullptr, tid);
+  WideTrStager<SPLIT, T, WB> sb(lds.bh, lds.bl, Ba, p.B_ls, WB, w, tid);
+  block_gemm_wide<SPLIT>(acc, lds, qlim, sa, sb, tid);  // the first barrier inside publishes w
+  float *st = p.states + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
+  const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1, i = lane & 15, gq = lane >> 4;
+#pragma unroll
+  for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int pp = pt * GB + wm * 32 + tm * 16 + gq * 4 + r;
+      if (pp >= P) continue;
+#pragma unroll
+      for (int tn = 0; tn < 4; ++tn) st[(int64_t)pp * N + nt * WB + wn * 64 + tn * 16 + i] = acc.v[tm][tn][r];
+    }
+}
+
 // ---------------------------------------------------- chunk_state_varlen
 // Packed batch (batch 1): state at the last position of every sequence i = [cu[i], cu[i+1]).
 // out[i, h, p, n] = sum_{k in the last chunk, k >= start} x[k, p] B[k, n] exp(a_end - a_k) dt_k
@@ -409,6 +459,20 @@ extern "C" int ssd_chunk_state_fwd(const SsdParams *p, mamba_stream_t stream) {
   if (rc) return rc;
   if (!p->states || !p->dt_out || !p->dA_cumsum) return MAMBA_E_BADARG;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  {
+    // whole 128-state blocks, 16-byte aligned x / B rows, headdim in whole groups of 8, whole k steps
+    const int64_t es = p->dtype == MAMBA_F32 ? 4 : 2, m = 16 / es;
+    const int last = p->seqlen - (p->nchunks - 1) * p->chunk_size;
+    const bool wide = p->dstate % WB == 0 && p->headdim % 8 == 0 && p->chunk_size % GK == 0 && last % GK == 0 &&
+                      reinterpret_cast<uintptr_t>(p->x) % 16 == 0 && reinterpret_cast<uintptr_t>(p->B) % 16 == 0 &&
+                      p->x_bs % m == 0 && p->x_ls % m == 0 && p->x_hs % m == 0 && p->B_bs % m == 0 &&
+                      p->B_ls % m == 0 && p->B_gs % m == 0;
+    if (wide) {
+      dim3 grid(((p->headdim + GB - 1) / GB) * (p->dstate / WB), p->nchunks, p->batch * p->nheads);
+      SSD_DISPATCH(chunk_state_fwd_wide_kernel, grid)
+      return launched();
+    }
+  }
   dim3 grid(((p->headdim + GB - 1) / GB) * ((p->dstate + GB - 1) / GB), p->nchunks, p->batch * p->nheads);
   SSD_DISPATCH(chunk_state_fwd_kernel, grid)
   return launched();
