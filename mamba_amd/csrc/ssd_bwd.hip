@@ -236,6 +236,42 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dst
   });
 }
 
+// The same product with a 64 x 128 tile per workgroup (whole 128-state blocks, aligned operands,
+// chunks that are whole k steps).
+template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dstates_wide_kernel(const SsdParams p) {
+  __shared__ GemmLdsWide<SPLIT> lds;
+  __shared__ float rs[256];
+  const int tid = threadIdx.x;
+  const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads;
+  const int ntn = N / WB;
+  const Block3 blk = xcd_block();
+  const int pt = blk.x / ntn, nt = blk.x % ntn;
+  const int c = blk.y, b = blk.z / H, h = blk.z % H;
+  const int g = h / (H / p.ngroups);
+  const int t0 = c * Q, qlim = min(Q, L - t0);
+  const float *dA = chunk_row(p.dA_cumsum, p, b, h, c);
+  const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
+  for (int l = tid; l < Q; l += 256) {
+    float v = 0.f;
+    if (l < qlim) {
+      bool ok = true;
+      if (seq) ok = seq[l] == (c > 0 ? seq[-1] : 0);
+      if (ok) v = fast_exp(dA[l]);
+    }
+    rs[l] = v;
+  }
+  const View4 gv = g_view(p);
+  const T *ga = static_cast<const T *>(gv.ptr) + b * gv.bs + h * gv.hs + (int64_t)t0 * gv.ls + pt * GB;
+  const T *Ca = static_cast<const T *>(p.C) + b * p.C_bs + g * p.C_gs + (int64_t)t0 * p.C_ls + nt * WB;
+  GemmAccWide acc;
+  acc.zero();
+  WideTrStager<SPLIT, T, 64> sa(lds.ah, lds.al, ga, gv.ls, P - pt * GB, nullptr, tid);
+  WideTrStager<SPLIT, T, WB> sb(lds.bh, lds.bl, Ca, p.C_ls, WB, rs, tid);
+  block_gemm_wide<SPLIT>(acc, lds, qlim, sa, sb, tid);  // the first barrier inside publishes rs
+  float *ds = p.dstates + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
+  store_wide(acc, ds + (int64_t)pt * GB * N + nt * WB, N, P - pt * GB, tid);
+}
+
 // ---------------------------------------------------- state_passing bwd
 // Reverse recurrence over chunks.  On entry dstates[c] is the direct gradient of the state
 // entering chunk c; on exit it is the gradient of chunk c's local state.
@@ -904,6 +940,17 @@ extern "C" int ssd_bwd_dstates(const SsdParams *p, mamba_stream_t stream) {
   int rc = check_bwd(p);
   if (rc) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  {
+    const bool g_ok = p->z ? (p->headdim % 8 == 0 && reinterpret_cast<uintptr_t>(p->gbuf) % 16 == 0)
+                           : wide_operand_ok(p->dout, p->dtype, p->dout_bs, p->dout_ls, p->dout_hs);
+    const bool wide = p->dstate % WB == 0 && p->headdim % 8 == 0 && whole_k_steps(p) && g_ok &&
+                      wide_operand_ok(p->C, p->dtype, p->C_bs, p->C_ls, p->C_gs);
+    if (wide) {
+      dim3 grid(tiles(p->headdim) * (p->dstate / WB), p->nchunks, p->batch * p->nheads);
+      SSD_DISPATCH(bwd_dstates_wide_kernel, grid)
+      return launched();
+    }
+  }
   dim3 grid(tiles(p->headdim) * tiles(p->dstate), p->nchunks, p->batch * p->nheads);
   SSD_DISPATCH(bwd_dstates_kernel, grid)
   return launched();

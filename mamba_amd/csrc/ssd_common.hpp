@@ -407,6 +407,30 @@ DEVI void block_gemm_wide(GemmAccWide &acc, GemmLdsWide<SPLIT> &s, int k_end, SA
   }
 }
 
+// Stores the wide tile as fp32 rows of dst (the tile's origin, row pitch ld); rows >= rows_valid are skipped.
+DEVI void store_wide(const GemmAccWide &acc, float *dst, int64_t ld, int rows_valid, int tid) {
+  const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1, i = lane & 15, g = lane >> 4;
+#pragma unroll
+  for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int m = wm * 32 + tm * 16 + g * 4 + r;
+      if (m >= rows_valid) continue;
+#pragma unroll
+      for (int tn = 0; tn < 4; ++tn) dst[(int64_t)m * ld + wn * 64 + tn * 16 + i] = acc.v[tm][tn][r];
+    }
+}
+// Host side: a (batch, position, head/group, row) operand can feed WideTrStager.
+inline bool wide_operand_ok(const void *ptr, int dtype, int64_t s0, int64_t s1, int64_t s2) {
+  const int64_t m = dtype == MAMBA_F32 ? 4 : 8;
+  return reinterpret_cast<uintptr_t>(ptr) % 16 == 0 && s0 % m == 0 && s1 % m == 0 && s2 % m == 0;
+}
+// Host side: every chunk is a whole number of k steps.
+inline bool whole_k_steps(const SsdParams *p) {
+  const int last = p->seqlen - (p->nchunks - 1) * p->chunk_size;
+  return p->chunk_size % GK == 0 && last % GK == 0;
+}
+
 // D[m][n] += sum_{k in [k_begin, k_end)} fa(m, k) * fb(n, k) for the block's 64 x 64 tile.
 // fa / fb return 0 outside their valid ranges.  All 256 threads must call.
 template <bool SPLIT, bool A_KFAST, bool B_KFAST, typename FA, typename FB>

@@ -191,16 +191,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void chunk_s
   WideTrStager<SPLIT, T, WB> sb(lds.bh, lds.bl, Ba, p.B_ls, WB, w, tid);
   block_gemm_wide<SPLIT>(acc, lds, qlim, sa, sb, tid);  // the first barrier inside publishes w
   float *st = p.states + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
-  const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1, i = lane & 15, gq = lane >> 4;
-#pragma unroll
-  for (int tm = 0; tm < 2; ++tm)
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int pp = pt * GB + wm * 32 + tm * 16 + gq * 4 + r;
-      if (pp >= P) continue;
-#pragma unroll
-      for (int tn = 0; tn < 4; ++tn) st[(int64_t)pp * N + nt * WB + wn * 64 + tn * 16 + i] = acc.v[tm][tn][r];
-    }
+  store_wide(acc, st + (int64_t)pt * GB * N + nt * WB, N, P - pt * GB, tid);
 }
 
 // ---------------------------------------------------- chunk_state_varlen
@@ -461,12 +452,9 @@ extern "C" int ssd_chunk_state_fwd(const SsdParams *p, mamba_stream_t stream) {
   hipStream_t s = static_cast<hipStream_t>(stream);
   {
     // whole 128-state blocks, 16-byte aligned x / B rows, headdim in whole groups of 8, whole k steps
-    const int64_t es = p->dtype == MAMBA_F32 ? 4 : 2, m = 16 / es;
-    const int last = p->seqlen - (p->nchunks - 1) * p->chunk_size;
-    const bool wide = p->dstate % WB == 0 && p->headdim % 8 == 0 && p->chunk_size % GK == 0 && last % GK == 0 &&
-                      reinterpret_cast<uintptr_t>(p->x) % 16 == 0 && reinterpret_cast<uintptr_t>(p->B) % 16 == 0 &&
-                      p->x_bs % m == 0 && p->x_ls % m == 0 && p->x_hs % m == 0 && p->B_bs % m == 0 &&
-                      p->B_ls % m == 0 && p->B_gs % m == 0;
+    const bool wide = p->dstate % WB == 0 && p->headdim % 8 == 0 && whole_k_steps(p) &&
+                      wide_operand_ok(p->x, p->dtype, p->x_bs, p->x_ls, p->x_hs) &&
+                      wide_operand_ok(p->B, p->dtype, p->B_bs, p->B_ls, p->B_gs);
     if (wide) {
       dim3 grid(((p->headdim + GB - 1) / GB) * (p->dstate / WB), p->nchunks, p->batch * p->nheads);
       SSD_DISPATCH(chunk_state_fwd_wide_kernel, grid)
