@@ -521,7 +521,8 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
 // One workgroup per (batch, chunk, group, 64 x 64 tile) loops over the heads of the group and keeps
 // both sums in registers (no atomics); the per-head row factor is folded into the A operand.
 // The carried-state share of ddA_cumsum, sum_n dC_h[l, n] C[l, n], is taken per head on the way.
-template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_dBC_state_kernel(const SsdParams p) {
+// PARTS: bit 0 = the dB product, bit 1 = the dC product.
+template <typename T, bool SPLIT, int PARTS> DEVI void dBC_state_body(const SsdParams &p) {
   constexpr int MAXH = 8;  // heads per workgroup (head_splits keeps it at or below 8)
   __shared__ GemmLds lds;
   __shared__ float wB[MAXH][GB], wC[MAXH][GB];  // per-head row factors
@@ -564,7 +565,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_
   auto state_off = [&](int hl) {
     return (((int64_t)b * p.nchunks + c) * H + g * hpg + hs + hl * nsplit) * P * N + nt * GB;
   };
-  {  // dB32 += (wB x)^T-rows times dS
+  if constexpr ((PARTS & 1) != 0) {  // dB32 += (wB x)^T-rows times dS
     GemmAcc accB;
     accB.zero();
     block_gemm_pipe<SPLIT>(
@@ -590,7 +591,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_
       return v;
     });
   }
-  {  // dC32 += (wC g) rows times H, and per head the carried-state share of ddA_cumsum
+  if constexpr ((PARTS & 2) != 0) {  // dC32 += (wC g) rows times H, and per head the carried-state share of ddA_cumsum
     const int64_t Cb = b * p.C_bs + g * p.C_gs;
     // C at this lane's 16 accumulator positions (shared by the heads of the group)
     float cr[2][2][4];
@@ -653,6 +654,73 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_
       return v;
     });
   }
+}
+
+template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_dBC_state_kernel(const SsdParams p) {
+  dBC_state_body<T, SPLIT, 3>(p);
+}
+template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_dC_state_kernel(const SsdParams p) {
+  dBC_state_body<T, SPLIT, 2>(p);
+}
+
+// The dB product alone with a 64 x 128 tile per workgroup (whole 128-state blocks, headdim in whole
+// k steps, aligned x): k runs through (head, p) as above.
+template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dB_state_wide_kernel(const SsdParams p) {
+  constexpr int MAXH = 8;
+  __shared__ GemmLdsWide<SPLIT> lds;
+  __shared__ float wB[MAXH][GB];
+  const int tid = threadIdx.x;
+  const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads, G = p.ngroups;
+  const int ntn = N / WB;
+  const Block3 blk = xcd_block();
+  const int nst = gridDim.x / ntn;
+  const int st = blk.x % nst, nt = blk.x / nst;
+  const int hpg = H / G, nsplit = head_splits(hpg);
+  const int c = blk.y, bg = blk.z / nsplit, hs = blk.z % nsplit, b = bg / G, g = bg % G;
+  const int nh = hs < hpg ? (hpg - hs + nsplit - 1) / nsplit : 0;
+  const int t0 = c * Q, qlim = min(Q, L - t0);
+  if (st * GB >= qlim || nh == 0) return;
+  const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
+  for (int idx = tid; idx < nh * GB; idx += 256) {
+    const int hl = idx / GB, r = idx % GB, s = st * GB + r, h = g * hpg + hs + hl * nsplit;
+    float vb = 0.f;
+    if (s < qlim) {
+      const float *dA = chunk_row(p.dA_cumsum, p, b, h, c);
+      bool okb = true;
+      if (seq) {
+        const int last = seq[qlim - 1];
+        okb = last >= 0 && seq[s] == last;
+      }
+      if (okb) vb = fast_exp(fminf(dA[Q - 1] - dA[s], 0.f)) * chunk_row(p.dt_out, p, b, h, c)[s];
+    }
+    wB[hl][r] = vb;
+  }
+  GemmAccWide accB;
+  accB.zero();
+  auto sa = seg_stager(KcStager<SPLIT, T>(lds.ah, lds.al, nullptr, p.x_ls, qlim - st * GB, P, nullptr, nullptr, true, tid),
+                       [&](KcStager<SPLIT, T> &q, int hl) {
+                         q.base = static_cast<const T *>(p.x) + b * p.x_bs + (g * hpg + hs + hl * nsplit) * p.x_hs +
+                                  (int64_t)(t0 + st * GB) * p.x_ls;
+                         q.rscale = wB[hl];
+                       },
+                       P);
+  auto sb = seg_stager(WideTrStager<SPLIT, float, WB>(lds.bh, lds.bl, nullptr, N, WB, nullptr, tid),
+                       [&](WideTrStager<SPLIT, float, WB> &q, int hl) {
+                         q.base = p.dstates + (((int64_t)b * p.nchunks + c) * H + g * hpg + hs + hl * nsplit) * P * N + nt * WB;
+                       },
+                       P);
+  block_gemm_wide<SPLIT>(accB, lds, nh * P, sa, sb, tid);  // the first barrier inside publishes wB
+  const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1, i = lane & 15, gq = lane >> 4;
+#pragma unroll
+  for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int s = st * GB + wm * 32 + tm * 16 + gq * 4 + r;
+      if (s >= qlim) continue;
+      float *row = p.dB32 + (((int64_t)b * L + t0 + s) * G + g) * N + nt * WB + wn * 64 + i;
+#pragma unroll
+      for (int tn = 0; tn < 4; ++tn) unsafeAtomicAdd(row + tn * 16, accB.v[tm][tn][r]);
+    }
 }
 
 // ------------------------------------------------------------------ dCB
@@ -985,8 +1053,17 @@ extern "C" int ssd_bwd_dBC_state(const SsdParams *p, mamba_stream_t stream) {
   int rc = check_bwd(p);
   if (rc) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  dim3 grid(tiles(p->chunk_size) * tiles(p->dstate), p->nchunks,
-            p->batch * p->ngroups * head_splits(p->nheads / p->ngroups));
+  const int zdim = p->batch * p->ngroups * head_splits(p->nheads / p->ngroups);
+  dim3 grid(tiles(p->chunk_size) * tiles(p->dstate), p->nchunks, zdim);
+  // whole 128-state blocks, headdim in whole k steps, aligned x rows: the dB product runs on wide tiles
+  const bool wide = p->dstate % WB == 0 && p->headdim % GK == 0 &&
+                    wide_operand_ok(p->x, p->dtype, p->x_bs, p->x_ls, p->x_hs);
+  if (wide) {
+    dim3 gridw(tiles(p->chunk_size) * (p->dstate / WB), p->nchunks, zdim);
+    SSD_DISPATCH(bwd_dB_state_wide_kernel, gridw)
+    SSD_DISPATCH(bwd_dC_state_kernel, grid)
+    return launched();
+  }
   SSD_DISPATCH(bwd_dBC_state_kernel, grid)
   return launched();
 }

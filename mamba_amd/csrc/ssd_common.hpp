@@ -309,7 +309,7 @@ DEVI void mma_step(GemmAcc &acc, const GemmLds &s, int wm, int wn, int lane) {
 constexpr int WB = 128;          // columns of the wide tile
 constexpr int WLD = WB + 16;     // [k][row] pitch of the wide operand (288 bytes)
 template <bool SPLIT> struct GemmLdsWide {
-  uint16_t ah[GK * TLD], al[SPLIT ? GK * TLD : 8], bh[GK * WLD], bl[SPLIT ? GK * WLD : 8];
+  uint16_t ah[GTILE], al[SPLIT ? GTILE : 8], bh[GK * WLD], bl[SPLIT ? GK * WLD : 8];
 };
 struct GemmAccWide {
   f32x4 v[2][4];
@@ -343,12 +343,14 @@ template <bool SPLIT, typename S, int ROWS> struct WideTrStager {
   Pack8<S> q[NT];
   DEVI WideTrStager(uint16_t *hi_, uint16_t *lo_, const S *base_, int64_t kstride_, int rows_valid_, const float *kscale_, int t_)
       : hi(hi_), lo(lo_), base(base_), kstride(kstride_), rows_valid(rows_valid_), kscale(kscale_), t(t_) {}
-  DEVI void fetch(int k0) {
+  static constexpr bool transposed = true;
+  DEVI bool fast() const { return true; }
+  template <bool FAST = true> DEVI void fetch(int k0) {
 #pragma unroll
     for (int j = 0; j < NT; ++j)
       q[j].load(base + (int64_t)(k0 + (t >> 3)) * kstride + min((t & 7) * 8 + 64 * j, rows_valid - 8));
   }
-  DEVI void commit(int k0) {
+  template <bool FAST = true> DEVI void commit(int k0) {
     const int kk = t >> 3;
     const float ks = kscale ? kscale[k0 + kk] : 1.f;
 #pragma unroll
@@ -369,25 +371,28 @@ template <bool SPLIT, typename S, int ROWS> struct WideTrStager {
     }
   }
 };
-// acc[m][n] += sum_k A[m][k] B[n][k] over k in [0, k_end), k_end a multiple of 32.
+// acc[m][n] += sum_k A[m][k] B[n][k] over k in [0, k_end), k_end a multiple of 32.  The A stager is
+// a 64-row stager of either layout on its fast path, the B stager a 128-row WideTrStager (possibly
+// inside a SegStager).
 template <bool SPLIT, typename SA, typename SB>
 DEVI void block_gemm_wide(GemmAccWide &acc, GemmLdsWide<SPLIT> &s, int k_end, SA &sa, SB &sb, int tid) {
+  constexpr bool ATR = SA::transposed;
   const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
   const int i = lane & 15, g = lane >> 4;
-  sa.fetch(0);
-  sb.fetch(0);
+  sa.template fetch<true>(0);
+  sb.template fetch<true>(0);
   for (int k0 = 0; k0 < k_end; k0 += GK) {
     __syncthreads();
-    sa.commit(k0);
-    sb.commit(k0);
+    sa.template commit<true>(k0);
+    sb.template commit<true>(k0);
     __syncthreads();
-    sa.fetch(min(k0 + GK, k_end - GK));
-    sb.fetch(min(k0 + GK, k_end - GK));
+    sa.template fetch<true>(min(k0 + GK, k_end - GK));
+    sb.template fetch<true>(min(k0 + GK, k_end - GK));
     bf16x8_t a[2], b[4], al[2], bl[4];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      a[t] = load_frag_tr<TLD>(s.ah, wm * 32 + t * 16, i, g);
-      if (SPLIT) al[t] = load_frag_tr<TLD>(s.al, wm * 32 + t * 16, i, g);
+      a[t] = load_frag<ATR>(s.ah, wm * 32 + t * 16, i, g);
+      if (SPLIT) al[t] = load_frag<ATR>(s.al, wm * 32 + t * 16, i, g);
     }
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
