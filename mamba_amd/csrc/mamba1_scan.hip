@@ -410,7 +410,7 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
               // pair, the decay being one exp of the summed delta; pass 2 reruns them from the state
               // the wave scan gives this lane. The adjoint is handled the same way in reverse.
               float A1[Q], hc[Q], gc[Q], an[Q];
-              float Bv[Q][8], Cv[Q][8], a[Q][8], bb[Q][8], h[Q][8];
+              float Cv[Q][8], a[Q][8], bb[Q][8], h[Q][8];
               float sa[Q], sb[Q], hend[Q];
 #pragma unroll
               for (int q = 0; q < Q; ++q) {
@@ -418,14 +418,15 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
                 hc[q] = hrow[n + q];
                 gc[q] = grow[n + q];
                 an[q] = arow[n + q];
-                load_bc<BC & 1>(Bv[q], Bs, p.B, d, N, nb * NB16 + n + q, n + q, lane);
+                float Bv[8];  // read again for the last loop: 16 registers fewer held through the scans
+                load_bc<BC & 1>(Bv, Bs, p.B, d, N, nb * NB16 + n + q, n + q, lane);
                 load_bc<BC & 2>(Cv[q], Cs, p.C, d, N, nb * NB16 + n + q, n + q, lane);
                 const float A2 = A1[q] * kLog2e;
                 sa[q] = fast_exp2(dsum * A2);
 #pragma unroll
                 for (int i = 0; i < KI; ++i) {
                   a[q][i] = fast_exp2(dl[i] * A2);
-                  bb[q][i] = du[i] * Bv[q][i];
+                  bb[q][i] = du[i] * Bv[i];
                 }
                 float hl = bb[q][0];
 #pragma unroll
@@ -476,7 +477,8 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
                   arow[n + q] = a[q][0];
                 }
                 float dAp = 0.f, dBp = 0.f, dCp = 0.f;
-                float sB[8], sC[8];
+                float sB[8], sC[8], Bv[8];
+                load_bc<BC & 1>(Bv, Bs, p.B, d, N, nb * NB16 + n + q, n + q, lane);
                 if constexpr (!(BC & 1)) lds_ld8(dBs + (n + q) * TILE, lane, sB);
                 if constexpr (!(BC & 2)) lds_ld8(dCs + (n + q) * TILE, lane, sC);
                 float gi = gx, an_i = a_next_lane[q];
@@ -488,7 +490,7 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
                   else sC[i] = __builtin_fmaf(dy[i], h[q][i], sC[i]);
                   if constexpr (BC & 1) dBp = __builtin_fmaf(gi, du[i], dBp);
                   else sB[i] = __builtin_fmaf(gi, du[i], sB[i]);
-                  acc[i] = __builtin_fmaf(gi, Bv[q][i], acc[i]);
+                  acc[i] = __builtin_fmaf(gi, Bv[i], acc[i]);
                   const float w = gi * (h[q][i] - bb[q][i]);  // g * a * h[t-1]
                   dd[i] = __builtin_fmaf(A1[q], w, dd[i]);
                   dAp = __builtin_fmaf(dl[i], w, dAp);
