@@ -132,6 +132,14 @@ def test_ssd_bwd_shapes(headdim, dstate, ngroups):
     _bwd_case(1, 384, 4, headdim, dstate, ngroups, 128, torch.float32)
 
 
+@pytest.mark.parametrize("headdim,dstate,ngroups,dtype", [
+    (32, 128, 1, torch.bfloat16), (128, 256, 2, torch.float32), (16, 128, 1, torch.bfloat16), (96, 128, 1, torch.float32)])
+def test_ssd_bwd_wide_tiles(headdim, dstate, ngroups, dtype):
+    # whole 128-state blocks and whole 32-position steps: chunk states, their gradients and the
+    # state part of dB run on 64 x 128 tiles, with head dimensions below, at and above one tile
+    _bwd_case(2, 512, 4, headdim, dstate, ngroups, 128, dtype, has_init=True)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_ssd_bwd_options(dtype):
     _bwd_case(2, 320, 4, 64, 32, 1, 64, dtype, has_init=True)
