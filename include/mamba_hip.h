@@ -274,6 +274,46 @@ int ssd_bmm_chunk_bwd(const SsdParams *p, mamba_stream_t stream);
 int ssd_chunk_cumsum_bwd(const SsdParams *p, mamba_stream_t stream);
 int ssd_combined_bwd(const SsdParams *p, mamba_stream_t stream);
 
+/* ------------------------------------------------------------------------- *
+ * Depthwise causal 1-D convolution in front of the scans.  The reference calls the
+ * separate causal_conv1d package for it (causal_conv1d_fn / causal_conv1d_cuda:
+ * call sites mamba_ssm/ops/selective_scan_interface.py:224,:307,
+ * mamba_ssm/ops/triton/ssd_combined.py:845,:920, mamba_ssm/modules/mamba2.py:236) and
+ * falls back to nn.Conv1d(groups = channels, padding = width - 1)[..., :L]
+ * (mamba_ssm/modules/mamba_simple.py:168-169):
+ *   out[b, c, l] = act(bias[c] + sum_k weight[c, k] x[b, c, l - (width - 1) + k])
+ * with x = 0 before position 0 and, when seq_idx is given, for taps whose position
+ * has another sequence id than l.  x, out, dout, dx are of `dtype` and addressed through
+ * (batch, channel, position) element strides; either the position stride or the
+ * channel stride of all of them must be 1 (the two layouts of the callers).  weight
+ * (dim, width), bias (dim), dweight, dbias are fp32 contiguous; dweight and dbias MUST be
+ * zero on entry (the kernels add into them).  width is 2, 3 or 4.
+ * The backward pass re-computes the pre-activation from x.
+ * ------------------------------------------------------------------------- */
+typedef struct CausalConvParams {
+  int32_t batch, dim, seqlen, width;
+  int32_t dtype; /* MAMBA_F32 / MAMBA_BF16 / MAMBA_F16 */
+  int32_t silu;  /* 1: SiLU after the convolution */
+  int32_t reserved0, reserved1;
+  const void *x;
+  const float *weight;
+  const float *bias;      /* nullable */
+  const int32_t *seq_idx; /* nullable, (batch, seqlen) contiguous */
+  void *out;              /* forward only */
+  int64_t x_bs, x_cs, x_ls; /* batch / channel / position stride */
+  int64_t out_bs, out_cs, out_ls;
+  /* ---- backward only ---- */
+  const void *dout;
+  void *dx;
+  float *dweight;
+  float *dbias; /* nullable */
+  int64_t dout_bs, dout_cs, dout_ls;
+  int64_t dx_bs, dx_cs, dx_ls;
+} CausalConvParams;
+
+int causal_conv1d_fwd(const CausalConvParams *p, mamba_stream_t stream);
+int causal_conv1d_bwd(const CausalConvParams *p, mamba_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -57,6 +57,16 @@ class SsdParams(ctypes.Structure):
     )
 
 
+class CausalConvParams(ctypes.Structure):
+    _fields_ = (
+        [(n, c_i32) for n in ("batch", "dim", "seqlen", "width", "dtype", "silu", "reserved0", "reserved1")]
+        + [(n, c_vp) for n in ("x", "weight", "bias", "seq_idx", "out")]
+        + [(n, c_i64) for n in ("x_bs", "x_cs", "x_ls", "out_bs", "out_cs", "out_ls")]
+        + [(n, c_vp) for n in ("dout", "dx", "dweight", "dbias")]
+        + [(n, c_i64) for n in ("dout_bs", "dout_cs", "dout_ls", "dx_bs", "dx_cs", "dx_ls")]
+    )
+
+
 _lib = None
 
 
@@ -96,6 +106,10 @@ def load():
     lib.ssd_chunk_scan_fwd_fused_supported.restype = ctypes.c_int
     lib.ssm_state_update.argtypes = [ctypes.POINTER(MambaStepParams), c_vp]
     lib.ssm_state_update.restype = ctypes.c_int
+    for name in ("causal_conv1d_fwd", "causal_conv1d_bwd"):
+        fn = getattr(lib, name)
+        fn.argtypes = [ctypes.POINTER(CausalConvParams), c_vp]
+        fn.restype = ctypes.c_int
     _lib = lib
     return lib
 

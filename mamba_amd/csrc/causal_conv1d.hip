@@ -1,0 +1,428 @@
+// Depthwise causal 1-D convolution (kernel width 2..4) with optional SiLU, forward and backward, for
+// gfx950.  It is the convolution in front of both scans (the reference calls the separate
+// causal_conv1d package for it: mamba_ssm/ops/selective_scan_interface.py:224,
+// mamba_ssm/ops/triton/ssd_combined.py:845); the arithmetic is
+//   out[b, c, l] = act(bias[c] + sum_k w[c, k] x[b, c, l - (W-1) + k]),  x = 0 before the sequence,
+// and with seq_idx a tap that reaches into another sequence of a packed row contributes nothing.
+// Both memory layouts of the callers are served without a transpose:
+//   * position-contiguous rows (batch, channel, position): a thread owns 8 consecutive positions of
+//     one row (16-byte accesses) and reads the 3-position halo from the neighbouring chunk;
+//   * channel-contiguous rows (batch, position, channel): a thread owns 8 consecutive channels and
+//     walks a run of positions with the previous taps in registers, so every element is read once.
+// The backward pass re-computes the pre-activation from x instead of storing it.
+#include "common.hpp"
+
+namespace {
+
+constexpr int MAXW = 4;
+
+DEVI float dsilu(float pre) {  // d/dpre silu(pre)
+  const float s = sigmoid_f(pre);
+  return s * (1.f + pre * (1.f - s));
+}
+DEVI float silu_f(float v) { return v * sigmoid_f(v); }
+
+// Taps right-aligned in 4 slots: slot 3 multiplies x[l], slot 0 multiplies x[l - 3].
+DEVI void load_taps(const CausalConvParams &p, int c, float (&w)[MAXW], float &bias) {
+#pragma unroll
+  for (int k = 0; k < MAXW; ++k) {
+    const int j = k - (MAXW - p.width);
+    w[k] = j >= 0 ? p.weight[(int64_t)c * p.width + j] : 0.f;
+  }
+  bias = p.bias ? p.bias[c] : 0.f;
+}
+
+// ------------------------------------------------------------------ position-contiguous rows
+// Element j of win[] is position l0 - 3 + j; positions outside [0, L) read as 0.
+template <typename T, bool VEC, int NWIN> DEVI void load_window(const T *row, int l0, int L, float (&win)[NWIN]) {
+  static_assert(NWIN == 11 || NWIN == 19, "3 halo positions, 8 own, optionally 8 following");
+  if constexpr (VEC) {  // l0 is a multiple of 8, L a multiple of 8, the row 16-byte aligned
+    Pack8<T> prev, cur, next;
+    prev.load(row + max(l0 - 8, 0));
+    cur.load(row + l0);
+    if (NWIN == 19) next.load(row + min(l0 + 8, L - 8));
+    float a[8], c[8];
+    prev.unpack(a);
+    cur.unpack(c);
+#pragma unroll
+    for (int j = 0; j < 3; ++j) win[j] = l0 >= 8 ? a[5 + j] : 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) win[3 + j] = c[j];
+    if constexpr (NWIN == 19) {
+      float n[8];
+      next.unpack(n);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) win[11 + j] = l0 + 8 < L ? n[j] : 0.f;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < NWIN; ++j) {
+      const int l = l0 - 3 + j;
+      win[j] = (l >= 0 && l < L) ? ld1<T>(row + l) : 0.f;
+    }
+  }
+}
+template <int NWIN> DEVI void load_ids(const int32_t *seq, int l0, int L, int (&ids)[NWIN]) {
+#pragma unroll
+  for (int j = 0; j < NWIN; ++j) {
+    const int l = l0 - 3 + j;
+    ids[j] = (l >= 0 && l < L) ? seq[l] : -0x7fffffff;
+  }
+}
+
+template <typename T, bool VEC> __global__ __launch_bounds__(256) void conv_rows_fwd_kernel(const CausalConvParams p) {
+  const int L = p.seqlen, c = blockIdx.y, b = blockIdx.z;
+  const int l0 = (blockIdx.x * 256 + threadIdx.x) * 8;
+  if (l0 >= L) return;
+  float w[MAXW], bias;
+  load_taps(p, c, w, bias);
+  float win[11];
+  load_window<T, VEC, 11>(static_cast<const T *>(p.x) + b * p.x_bs + c * p.x_cs, l0, L, win);
+  int ids[11];
+  if (p.seq_idx) load_ids<11>(p.seq_idx + (int64_t)b * L, l0, L, ids);
+  float o[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    float v = bias;
+#pragma unroll
+    for (int k = 0; k < MAXW; ++k) {
+      float t = win[i + k];
+      if (p.seq_idx && ids[i + k] != ids[i + 3]) t = 0.f;
+      v = __builtin_fmaf(w[k], t, v);
+    }
+    o[i] = p.silu ? silu_f(v) : v;
+  }
+  st8_guard<T, VEC>(static_cast<T *>(p.out) + b * p.out_bs + c * p.out_cs + l0, min(8, L - l0), o);
+}
+
+template <typename T, bool VEC> __global__ __launch_bounds__(256) void conv_rows_bwd_kernel(const CausalConvParams p) {
+  const int L = p.seqlen, c = blockIdx.y, b = blockIdx.z;
+  const int l0 = (blockIdx.x * 256 + threadIdx.x) * 8;
+  float dw[MAXW] = {0.f, 0.f, 0.f, 0.f}, db = 0.f;
+  if (l0 < L) {
+    float w[MAXW], bias;
+    load_taps(p, c, w, bias);
+    float xw[19], gw[19];  // x and dout at positions l0 - 3 .. l0 + 15 (dout's halo is not used)
+    load_window<T, VEC, 19>(static_cast<const T *>(p.x) + b * p.x_bs + c * p.x_cs, l0, L, xw);
+    load_window<T, VEC, 19>(static_cast<const T *>(p.dout) + b * p.dout_bs + c * p.dout_cs, l0, L, gw);
+    int ids[19];
+    if (p.seq_idx) load_ids<19>(p.seq_idx + (int64_t)b * L, l0, L, ids);
+    // gradient of the pre-activation at positions l0 .. l0 + 10 (own 8 and the 3 that still see them)
+    float dpre[11];
+#pragma unroll
+    for (int j = 0; j < 11; ++j) {
+      float v = bias;
+#pragma unroll
+      for (int k = 0; k < MAXW; ++k) {
+        float t = xw[j + k];
+        if (p.seq_idx && ids[j + k] != ids[j + 3]) t = 0.f;
+        v = __builtin_fmaf(w[k], t, v);
+      }
+      const float g = gw[j + 3];
+      dpre[j] = l0 + j < L ? (p.silu ? g * dsilu(v) : g) : 0.f;
+    }
+    float o[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float v = 0.f;
+#pragma unroll
+      for (int k = 0; k < MAXW; ++k) {  // x[l] enters out[l + 3 - k] through tap k
+        float t = dpre[i + 3 - k];
+        if (p.seq_idx && ids[i + 3 + 3 - k] != ids[i + 3]) t = 0.f;
+        v = __builtin_fmaf(w[k], t, v);
+      }
+      o[i] = v;
+#pragma unroll
+      for (int k = 0; k < MAXW; ++k) {
+        float t = xw[i + k];
+        if (p.seq_idx && ids[i + k] != ids[i + 3]) t = 0.f;
+        dw[k] = __builtin_fmaf(dpre[i], t, dw[k]);
+      }
+      db += dpre[i];
+    }
+    st8_guard<T, VEC>(static_cast<T *>(p.dx) + b * p.dx_bs + c * p.dx_cs + l0, min(8, L - l0), o);
+  }
+  // one atomic per wave and tap
+#pragma unroll
+  for (int k = 0; k < MAXW; ++k) dw[k] = wave_sum_to_last(dw[k]);
+  db = wave_sum_to_last(db);
+  if ((threadIdx.x & 63) == 63) {
+#pragma unroll
+    for (int k = 0; k < MAXW; ++k) {
+      const int j = k - (MAXW - p.width);
+      if (j >= 0 && dw[k] != 0.f) unsafeAtomicAdd(p.dweight + (int64_t)c * p.width + j, dw[k]);
+    }
+    if (p.dbias && db != 0.f) unsafeAtomicAdd(p.dbias + c, db);
+  }
+}
+
+// ------------------------------------------------------------------ channel-contiguous rows
+constexpr int RUN = 32;   // positions per thread
+constexpr int NRUN = 4;   // runs per workgroup (256 threads = 64 channel groups x 4 runs)
+
+template <typename T, bool VEC> DEVI void load_ch8(const T *p, int nvalid, float (&o)[8]) {
+  if constexpr (VEC) ld8<T>(p, o);
+  else ld8_guard<T, false>(p, nvalid, 0.f, o);
+}
+
+template <typename T, bool VEC> __global__ __launch_bounds__(256) void conv_cl_fwd_kernel(const CausalConvParams p) {
+  const int L = p.seqlen, b = blockIdx.z;
+  const int cg = threadIdx.x & 63, run = threadIdx.x >> 6;
+  const int c0 = (blockIdx.x * 64 + cg) * 8;
+  if (c0 >= p.dim) return;
+  const int nch = min(8, p.dim - c0);
+  const int lbeg = (blockIdx.y * NRUN + run) * RUN, lend = min(lbeg + RUN, L);
+  if (lbeg >= L) return;
+  float w[8][MAXW], bias[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) load_taps(p, min(c0 + e, p.dim - 1), w[e], bias[e]);
+  const T *xb = static_cast<const T *>(p.x) + b * p.x_bs + c0;
+  T *ob = static_cast<T *>(p.out) + b * p.out_bs + c0;
+  const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L : nullptr;
+  float xw[3][8];  // x at l - 3, l - 2, l - 1
+  int idw[3] = {-0x7fffffff, -0x7fffffff, -0x7fffffff};
+#pragma unroll
+  for (int j = 0; j < 3; ++j) {
+    const int l = lbeg - 3 + j;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) xw[j][e] = 0.f;
+    if (l >= 0) {
+      load_ch8<T, VEC>(xb + (int64_t)l * p.x_ls, nch, xw[j]);
+      if (seq) idw[j] = seq[l];
+    }
+  }
+  for (int l4 = lbeg; l4 < lend; l4 += 4) {
+    float xin[4][8];
+    int idn[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {  // the loads of four positions first
+      const int l = min(l4 + u, L - 1);
+      load_ch8<T, VEC>(xb + (int64_t)l * p.x_ls, nch, xin[u]);
+      idn[u] = seq ? seq[l] : 0;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int l = l4 + u;
+      if (l >= lend) break;
+      float o[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float v = __builtin_fmaf(w[e][3], xin[u][e], bias[e]);
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+          float t = xw[j][e];
+          if (seq && idw[j] != idn[u]) t = 0.f;
+          v = __builtin_fmaf(w[e][j], t, v);
+        }
+        o[e] = p.silu ? silu_f(v) : v;
+      }
+      st8_guard<T, VEC>(ob + (int64_t)l * p.out_ls, nch, o);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        xw[0][e] = xw[1][e];
+        xw[1][e] = xw[2][e];
+        xw[2][e] = xin[u][e];
+      }
+      idw[0] = idw[1];
+      idw[1] = idw[2];
+      idw[2] = idn[u];
+    }
+  }
+}
+
+template <typename T, bool VEC> __global__ __launch_bounds__(256) void conv_cl_bwd_kernel(const CausalConvParams p) {
+  __shared__ float red[NRUN - 1][64][8 * (MAXW + 1)];
+  const int L = p.seqlen, b = blockIdx.z;
+  const int cg = threadIdx.x & 63, run = threadIdx.x >> 6;
+  const int c0 = (blockIdx.x * 64 + cg) * 8;
+  const int nch = max(0, min(8, p.dim - c0));
+  const int lbeg = (blockIdx.y * NRUN + run) * RUN, lend = min(lbeg + RUN, L);
+  float dw[8][MAXW], db[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    db[e] = 0.f;
+#pragma unroll
+    for (int k = 0; k < MAXW; ++k) dw[e][k] = 0.f;
+  }
+  if (nch > 0 && lbeg < L) {
+    float w[8][MAXW], bias[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) load_taps(p, min(c0 + e, p.dim - 1), w[e], bias[e]);
+    const T *xb = static_cast<const T *>(p.x) + b * p.x_bs + c0;
+    const T *gb = static_cast<const T *>(p.dout) + b * p.dout_bs + c0;
+    T *dxb = static_cast<T *>(p.dx) + b * p.dx_bs + c0;
+    const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L : nullptr;
+    // Walk down from lend + 2: the first three steps only rebuild dpre at the positions after the run.
+    const int ltop = min(lend + 2, L - 1);
+    float xw[4][8];   // x at l - 3 .. l
+    float dp[4][8];   // dpre at l .. l + 3
+    int idx[7];       // sequence ids at l - 3 .. l + 3
+#pragma unroll
+    for (int j = 0; j < 7; ++j) {
+      const int l = ltop - 3 + j;
+      idx[j] = (seq && l >= 0 && l < L) ? seq[l] : -0x7fffffff;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int l = ltop - 3 + j;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) xw[j][e] = dp[j][e] = 0.f;
+      if (l >= 0) load_ch8<T, VEC>(xb + (int64_t)l * p.x_ls, nch, xw[j]);
+    }
+    for (int l = ltop; l >= lbeg; --l) {
+      float g[8], xnew[8];
+      load_ch8<T, VEC>(gb + (int64_t)l * p.dout_ls, nch, g);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) xnew[e] = 0.f;
+      if (l - 4 >= 0) load_ch8<T, VEC>(xb + (int64_t)(l - 4) * p.x_ls, nch, xnew);
+      const int idnew = (seq && l - 4 >= 0) ? seq[l - 4] : -0x7fffffff;
+      // dpre at l
+      float dcur[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float v = bias[e];
+#pragma unroll
+        for (int k = 0; k < MAXW; ++k) {
+          float t = xw[k][e];
+          if (seq && idx[k] != idx[3]) t = 0.f;
+          v = __builtin_fmaf(w[e][k], t, v);
+        }
+        dcur[e] = p.silu ? g[e] * dsilu(v) : g[e];
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        dp[3][e] = dp[2][e];
+        dp[2][e] = dp[1][e];
+        dp[1][e] = dp[0][e];
+        dp[0][e] = dcur[e];
+      }
+      if (l < lend) {
+        float o[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          float v = 0.f;
+#pragma unroll
+          for (int k = 0; k < MAXW; ++k) {  // x[l] enters out[l + 3 - k] through tap k
+            float t = dp[3 - k][e];
+            if (seq && idx[3 + 3 - k] != idx[3]) t = 0.f;
+            v = __builtin_fmaf(w[e][k], t, v);
+          }
+          o[e] = v;
+#pragma unroll
+          for (int k = 0; k < MAXW; ++k) {
+            float t = xw[k][e];
+            if (seq && idx[k] != idx[3]) t = 0.f;
+            dw[e][k] = __builtin_fmaf(dcur[e], t, dw[e][k]);
+          }
+          db[e] += dcur[e];
+        }
+        st8_guard<T, VEC>(dxb + (int64_t)l * p.dx_ls, nch, o);
+      }
+      // slide both windows one position down
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        xw[3][e] = xw[2][e];
+        xw[2][e] = xw[1][e];
+        xw[1][e] = xw[0][e];
+        xw[0][e] = xnew[e];
+      }
+#pragma unroll
+      for (int j = 6; j > 0; --j) idx[j] = idx[j - 1];
+      idx[0] = idnew;
+    }
+  }
+  // the four runs of a channel group are summed in LDS, then one atomic per channel and tap
+  if (run > 0) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+#pragma unroll
+      for (int k = 0; k < MAXW; ++k) red[run - 1][cg][e * (MAXW + 1) + k] = dw[e][k];
+      red[run - 1][cg][e * (MAXW + 1) + MAXW] = db[e];
+    }
+  }
+  __syncthreads();
+  if (run == 0 && nch > 0) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      if (e >= nch) break;
+#pragma unroll
+      for (int k = 0; k < MAXW; ++k) {
+        float v = dw[e][k];
+#pragma unroll
+        for (int r = 0; r < NRUN - 1; ++r) v += red[r][cg][e * (MAXW + 1) + k];
+        const int j = k - (MAXW - p.width);
+        if (j >= 0 && v != 0.f) unsafeAtomicAdd(p.dweight + (int64_t)(c0 + e) * p.width + j, v);
+      }
+      float v = db[e];
+#pragma unroll
+      for (int r = 0; r < NRUN - 1; ++r) v += red[r][cg][e * (MAXW + 1) + MAXW];
+      if (p.dbias && v != 0.f) unsafeAtomicAdd(p.dbias + c0 + e, v);
+    }
+  }
+}
+
+// ------------------------------------------------------------------ launch
+int check(const CausalConvParams *p, bool bwd) {
+  if (!p || !p->x || !p->weight) return MAMBA_E_BADARG;
+  if (p->batch <= 0 || p->dim <= 0 || p->seqlen <= 0) return MAMBA_E_BADARG;
+  if (p->width < 2 || p->width > MAXW) return MAMBA_E_UNSUPPORTED;
+  if (p->dtype != MAMBA_F32 && p->dtype != MAMBA_BF16 && p->dtype != MAMBA_F16) return MAMBA_E_BADARG;
+  if (p->batch > 65535) return MAMBA_E_UNSUPPORTED;
+  if (!bwd && !p->out) return MAMBA_E_BADARG;
+  if (bwd && (!p->dout || !p->dx || !p->dweight)) return MAMBA_E_BADARG;
+  if (p->x_ls != 1 && p->x_cs != 1) return MAMBA_E_UNSUPPORTED;
+  return MAMBA_OK;
+}
+
+bool al16(const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; }
+
+template <typename T> int launch_conv(const CausalConvParams &p, bool bwd, hipStream_t s) {
+  const int64_t m = 16 / sizeof(T);
+  const bool rows = p.x_ls == 1 && (bwd ? p.dout_ls == 1 && p.dx_ls == 1 : p.out_ls == 1);
+  auto ok = [&](const void *q, int64_t a, int64_t b2) { return al16(q) && a % m == 0 && b2 % m == 0; };
+  if (rows) {
+    if (p.dim > 65535) return MAMBA_E_UNSUPPORTED;
+    const bool vec = p.seqlen % 8 == 0 && ok(p.x, p.x_bs, p.x_cs) &&
+                     (bwd ? ok(p.dout, p.dout_bs, p.dout_cs) && ok(p.dx, p.dx_bs, p.dx_cs) : ok(p.out, p.out_bs, p.out_cs));
+    dim3 grid((p.seqlen + 2047) / 2048, p.dim, p.batch);
+    if (bwd) {
+      if (vec) hipLaunchKernelGGL((conv_rows_bwd_kernel<T, true>), grid, dim3(256), 0, s, p);
+      else hipLaunchKernelGGL((conv_rows_bwd_kernel<T, false>), grid, dim3(256), 0, s, p);
+    } else {
+      if (vec) hipLaunchKernelGGL((conv_rows_fwd_kernel<T, true>), grid, dim3(256), 0, s, p);
+      else hipLaunchKernelGGL((conv_rows_fwd_kernel<T, false>), grid, dim3(256), 0, s, p);
+    }
+  } else {
+    const bool cl = p.x_cs == 1 && (bwd ? p.dout_cs == 1 && p.dx_cs == 1 : p.out_cs == 1);
+    if (!cl) return MAMBA_E_UNSUPPORTED;
+    const bool vec = p.dim % 8 == 0 && ok(p.x, p.x_bs, p.x_ls) &&
+                     (bwd ? ok(p.dout, p.dout_bs, p.dout_ls) && ok(p.dx, p.dx_bs, p.dx_ls) : ok(p.out, p.out_bs, p.out_ls));
+    const int ygrid = (p.seqlen + RUN * NRUN - 1) / (RUN * NRUN);
+    if (ygrid > 65535) return MAMBA_E_UNSUPPORTED;
+    dim3 grid((p.dim + 511) / 512, ygrid, p.batch);
+    if (bwd) {
+      if (vec) hipLaunchKernelGGL((conv_cl_bwd_kernel<T, true>), grid, dim3(256), 0, s, p);
+      else hipLaunchKernelGGL((conv_cl_bwd_kernel<T, false>), grid, dim3(256), 0, s, p);
+    } else {
+      if (vec) hipLaunchKernelGGL((conv_cl_fwd_kernel<T, true>), grid, dim3(256), 0, s, p);
+      else hipLaunchKernelGGL((conv_cl_fwd_kernel<T, false>), grid, dim3(256), 0, s, p);
+    }
+  }
+  return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
+}
+
+int dispatch(const CausalConvParams *p, bool bwd, mamba_stream_t stream) {
+  int rc = check(p, bwd);
+  if (rc != MAMBA_OK) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (p->dtype) {
+    case MAMBA_F32: return launch_conv<float>(*p, bwd, s);
+    case MAMBA_BF16: return launch_conv<bf16_t>(*p, bwd, s);
+    default: return launch_conv<f16_t>(*p, bwd, s);
+  }
+}
+
+}  // namespace
+
+extern "C" int causal_conv1d_fwd(const CausalConvParams *p, mamba_stream_t stream) { return dispatch(p, false, stream); }
+extern "C" int causal_conv1d_bwd(const CausalConvParams *p, mamba_stream_t stream) { return dispatch(p, true, stream); }

@@ -15,6 +15,7 @@ import torch.nn.functional as F
 from einops import rearrange
 
 from mamba_amd import _lib
+from mamba_amd.ops.causal_conv1d import causal_conv1d_bwd, causal_conv1d_fwd
 
 _FLOAT_TYPES = (torch.float32, torch.bfloat16, torch.float16)
 
@@ -359,7 +360,7 @@ class MambaInnerFn(torch.autograd.Function):
         conv1d_weight = rearrange(conv1d_weight, "d 1 w -> d w")
         x, z = xz.chunk(2, dim=1)
         conv1d_bias = conv1d_bias.contiguous() if conv1d_bias is not None else None
-        conv1d_out = _causal_conv1d_silu(x, conv1d_weight, conv1d_bias)
+        conv1d_out = causal_conv1d_fwd(x, conv1d_weight, conv1d_bias, activation="silu")
         # delta keeps d as the slow and L as the fast dimension: what the scan kernel reads
         x_dbl = F.linear(rearrange(conv1d_out, "b d l -> (b l) d"), x_proj_weight)
         delta = rearrange(delta_proj_weight @ x_dbl[:, :delta_rank].t(), "d (b l) -> b d l", l=L)
@@ -414,14 +415,8 @@ class MambaInnerFn(torch.autograd.Function):
         x, z = xz.chunk(2, dim=1)
         if dout.stride(-1) != 1:
             dout = dout.contiguous()
-        # the convolution is differentiated by torch on a local graph (recomputed when checkpointing)
-        with torch.enable_grad():
-            x_leaf = x.detach().requires_grad_()
-            w_leaf = conv1d_weight.detach().requires_grad_()
-            b_leaf = conv1d_bias.detach().requires_grad_() if conv1d_bias is not None else None
-            conv_graph = _causal_conv1d_silu(x_leaf, w_leaf, b_leaf)
-        if ctx.checkpoint_lvl == 1:
-            conv1d_out = conv_graph.detach()
+        if ctx.checkpoint_lvl == 1:  # the convolution output and delta are re-computed
+            conv1d_out = causal_conv1d_fwd(x, conv1d_weight, conv1d_bias, activation="silu")
             delta = rearrange(delta_proj_weight @ x_dbl[:, :delta_rank].t(), "d (b l) -> b d l", l=L)
             if ctx.dt_rms_weight is not None:
                 delta = rearrange(_rms_norm(rearrange(delta, "b d l -> (b l) d").contiguous(), ctx.dt_rms_weight,
@@ -454,11 +449,10 @@ class MambaInnerFn(torch.autograd.Function):
         dx_proj_weight = torch.einsum("Br,Bd->rd", dx_dbl, rearrange(conv1d_out, "b d l -> (b l) d"))
         dconv1d_out = torch.addmm(dconv1d_out, x_proj_weight.t(), dx_dbl.t())
         dconv1d_out = rearrange(dconv1d_out, "d (b l) -> b d l", b=x.shape[0], l=L)
-        leaves = [x_leaf, w_leaf] + ([b_leaf] if b_leaf is not None else [])
-        grads = torch.autograd.grad(conv_graph, leaves, dconv1d_out.to(conv_graph.dtype))
-        dx.copy_(grads[0])
-        dconv1d_weight = rearrange(grads[1], "d w -> d 1 w")
-        dconv1d_bias = grads[2] if b_leaf is not None else None
+        # the convolution's backward kernel re-computes the pre-activation from x and writes dx in place
+        _, dconv1d_weight, dconv1d_bias = causal_conv1d_bwd(x, conv1d_weight, conv1d_bias, dconv1d_out.to(x.dtype),
+                                                            activation="silu", dx=dx)
+        dconv1d_weight = rearrange(dconv1d_weight, "d w -> d 1 w")
         return (dxz, dconv1d_weight, dconv1d_bias, dx_proj_weight, ddelta_proj_weight, dout_proj_weight,
                 dout_proj_bias, dA, dB, dC, dD, ddelta_bias if delta_bias is not None else None,
                 dB_proj_bias, dC_proj_bias, None, None, None, None, None, None)

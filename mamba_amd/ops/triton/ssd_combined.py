@@ -11,6 +11,7 @@ import math
 import torch
 
 from mamba_amd import _lib
+from mamba_amd.ops.causal_conv1d import causal_conv1d_fn
 
 
 def _fill_fwd(p, x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, seq_idx, dt_softplus, dt_limit, ws):
@@ -407,9 +408,9 @@ def mamba_split_conv1d_scan_combined(zxbcdt, conv1d_weight, conv1d_bias, dt_bias
                                      rmsnorm_eps=1e-6, outproj_weight=None, outproj_bias=None, headdim=None,
                                      ngroups=1, norm_before_gate=True, state_dtype=None):
     """The Mamba-2 block body after in_proj (ssd_combined.py:983, forward :824-899): split, causal
-    conv1d + SiLU on xBC, the chunked scan on the HIP kernels, gate or gated RMSNorm, out_proj.
-    The convolution, the norm and the projection are torch operators and their gradients come from
-    autograd; the scan's come from MambaChunkScanCombinedFn.
+    conv1d + SiLU on xBC and the chunked scan on the HIP kernels, gate or gated RMSNorm, out_proj.
+    The norm and the projection are torch operators and their gradients come from autograd; the
+    convolution's and the scan's come from CausalConv1dFn and MambaChunkScanCombinedFn.
         zxbcdt: (batch, seqlen, 2 * d_nonssm + 2 * dim + 2 * ngroups * dstate + nheads), dim = nheads * headdim
         conv1d_weight: (dim + 2 * ngroups * dstate, width); conv1d_bias: (dim + 2 * ngroups * dstate,)
         dt_bias, A: (nheads,); D: (nheads, headdim) or (nheads,) (then headdim must be given)
@@ -434,7 +435,9 @@ def mamba_split_conv1d_scan_combined(zxbcdt, conv1d_weight, conv1d_bias, dt_bias
     if conv1d_weight.dim() == 3:
         conv1d_weight = conv1d_weight.squeeze(1)
     zx0, z, xBC, dt = torch.split(zxbcdt, [2 * d_nonssm, dim, dim + 2 * ngroups * dstate, nheads], dim=-1)
-    xBC = _causal_conv1d(xBC, conv1d_weight, conv1d_bias, activation, seq_idx)
+    # the HIP convolution reads the channel-contiguous slice as it lies and returns a dense (b, l, c) tensor
+    xBC = causal_conv1d_fn(xBC.transpose(1, 2), conv1d_weight, conv1d_bias, seq_idx=seq_idx,
+                           activation=activation).transpose(1, 2)
     x, B, C = torch.split(xBC, [dim, ngroups * dstate, ngroups * dstate], dim=-1)
     x = x.reshape(batch, seqlen, nheads, headdim)
     B = B.reshape(batch, seqlen, ngroups, dstate)

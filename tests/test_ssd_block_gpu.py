@@ -30,7 +30,9 @@ def _block_inputs(batch, L, nheads, headdim, dstate, ngroups, d_nonssm, d_out, s
         conv1d_weight=(0.5 * r(dim + 2 * ngroups * dstate, width)).to(dtype),
         conv1d_bias=(0.1 * r(dim + 2 * ngroups * dstate)).to(dtype),
         dt_bias=torch.rand(nheads, generator=g) - 4.0, A=-(1.0 + 15.0 * torch.rand(nheads, generator=g)),
-        D=torch.rand(nheads, generator=g), rmsnorm_weight=(1.0 + 0.1 * r(dim)).to(dtype),
+        # D away from 0: with a tiny skip term the scan output right after a sequence start is ~0 for a
+        # whole norm group, and 1 / rms then multiplies every rounding difference by hundreds
+        D=0.5 + torch.rand(nheads, generator=g), rmsnorm_weight=(1.0 + 0.1 * r(dim)).to(dtype),
         outproj_weight=(0.2 * r(d_out, d_nonssm + dim)).to(dtype), outproj_bias=(0.1 * r(d_out)).to(dtype))
 
 
