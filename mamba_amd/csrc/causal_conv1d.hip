@@ -269,66 +269,77 @@ template <typename T, bool VEC> __global__ __launch_bounds__(256) void conv_cl_b
       for (int e = 0; e < 8; ++e) xw[j][e] = dp[j][e] = 0.f;
       if (l >= 0) load_ch8<T, VEC>(xb + (int64_t)l * p.x_ls, nch, xw[j]);
     }
-    for (int l = ltop; l >= lbeg; --l) {
-      float g[8], xnew[8];
-      load_ch8<T, VEC>(gb + (int64_t)l * p.dout_ls, nch, g);
+    for (int l4 = ltop; l4 >= lbeg; l4 -= 4) {
+      // the loads of four steps first (dout at l4 .. l4 - 3, x at l4 - 4 .. l4 - 7): the stores of dx in
+      // between would otherwise keep the compiler from moving them up
+      float g4[4][8], x4[4][8];
+      int id4[4];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) xnew[e] = 0.f;
-      if (l - 4 >= 0) load_ch8<T, VEC>(xb + (int64_t)(l - 4) * p.x_ls, nch, xnew);
-      const int idnew = (seq && l - 4 >= 0) ? seq[l - 4] : -0x7fffffff;
-      // dpre at l
-      float dcur[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        float v = bias[e];
-#pragma unroll
-        for (int k = 0; k < MAXW; ++k) {
-          float t = xw[k][e];
-          if (seq && idx[k] != idx[3]) t = 0.f;
-          v = __builtin_fmaf(w[e][k], t, v);
-        }
-        dcur[e] = p.silu ? g[e] * dsilu(v) : g[e];
+      for (int u = 0; u < 4; ++u) {
+        const int l = l4 - u;
+        load_ch8<T, VEC>(gb + (int64_t)max(l, 0) * p.dout_ls, nch, g4[u]);
+        load_ch8<T, VEC>(xb + (int64_t)max(l - 4, 0) * p.x_ls, nch, x4[u]);
+        id4[u] = (seq && l - 4 >= 0) ? seq[l - 4] : -0x7fffffff;
       }
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        dp[3][e] = dp[2][e];
-        dp[2][e] = dp[1][e];
-        dp[1][e] = dp[0][e];
-        dp[0][e] = dcur[e];
-      }
-      if (l < lend) {
-        float o[8];
+      for (int u = 0; u < 4; ++u) {
+        const int l = l4 - u;
+        if (l < lbeg) break;
+        // dpre at l
+        float dcur[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          float v = 0.f;
-#pragma unroll
-          for (int k = 0; k < MAXW; ++k) {  // x[l] enters out[l + 3 - k] through tap k
-            float t = dp[3 - k][e];
-            if (seq && idx[3 + 3 - k] != idx[3]) t = 0.f;
-            v = __builtin_fmaf(w[e][k], t, v);
-          }
-          o[e] = v;
+          float v = bias[e];
 #pragma unroll
           for (int k = 0; k < MAXW; ++k) {
             float t = xw[k][e];
             if (seq && idx[k] != idx[3]) t = 0.f;
-            dw[e][k] = __builtin_fmaf(dcur[e], t, dw[e][k]);
+            v = __builtin_fmaf(w[e][k], t, v);
           }
-          db[e] += dcur[e];
+          dcur[e] = p.silu ? g4[u][e] * dsilu(v) : g4[u][e];
         }
-        st8_guard<T, VEC>(dxb + (int64_t)l * p.dx_ls, nch, o);
-      }
-      // slide both windows one position down
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        xw[3][e] = xw[2][e];
-        xw[2][e] = xw[1][e];
-        xw[1][e] = xw[0][e];
-        xw[0][e] = xnew[e];
-      }
+        for (int e = 0; e < 8; ++e) {
+          dp[3][e] = dp[2][e];
+          dp[2][e] = dp[1][e];
+          dp[1][e] = dp[0][e];
+          dp[0][e] = dcur[e];
+        }
+        if (l < lend) {
+          float o[8];
 #pragma unroll
-      for (int j = 6; j > 0; --j) idx[j] = idx[j - 1];
-      idx[0] = idnew;
+          for (int e = 0; e < 8; ++e) {
+            float v = 0.f;
+#pragma unroll
+            for (int k = 0; k < MAXW; ++k) {  // x[l] enters out[l + 3 - k] through tap k
+              float t = dp[3 - k][e];
+              if (seq && idx[3 + 3 - k] != idx[3]) t = 0.f;
+              v = __builtin_fmaf(w[e][k], t, v);
+            }
+            o[e] = v;
+#pragma unroll
+            for (int k = 0; k < MAXW; ++k) {
+              float t = xw[k][e];
+              if (seq && idx[k] != idx[3]) t = 0.f;
+              dw[e][k] = __builtin_fmaf(dcur[e], t, dw[e][k]);
+            }
+            db[e] += dcur[e];
+          }
+          st8_guard<T, VEC>(dxb + (int64_t)l * p.dx_ls, nch, o);
+        }
+        // slide both windows one position down
+        const bool has = l - 4 >= 0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          xw[3][e] = xw[2][e];
+          xw[2][e] = xw[1][e];
+          xw[1][e] = xw[0][e];
+          xw[0][e] = has ? x4[u][e] : 0.f;
+        }
+#pragma unroll
+        for (int j = 6; j > 0; --j) idx[j] = idx[j - 1];
+        idx[0] = id4[u];
+      }
     }
   }
   // the four runs of a channel group are summed in LDS, then one atomic per channel and tap
