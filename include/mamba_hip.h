@@ -314,6 +314,50 @@ typedef struct CausalConvParams {
 int causal_conv1d_fwd(const CausalConvParams *p, mamba_stream_t stream);
 int causal_conv1d_bwd(const CausalConvParams *p, mamba_stream_t stream);
 
+/* -------------------------------------------------------------------------
+ * Gated LayerNorm / RMSNorm over groups of channels: the epilogue of the Mamba-2 block between
+ * the chunked scan and the output projection.  Replaces the Triton launches of
+ * mamba_ssm/ops/triton/layernorm_gated.py:108 (_layer_norm_fwd) and :271 (_layer_norm_bwd),
+ * called from mamba_ssm/modules/mamba2.py:242 and mamba_ssm/ops/triton/ssd_combined.py:872-874.
+ *   x' = norm_before_gate ? x : x * silu(z);   y = (x' - mean) * rstd * weight + bias;
+ *   out = norm_before_gate ? y * silu(z) : y;  statistics per (row, group), mean = 0 when is_rms.
+ * x, z, out, dy, dx, dz are (rows, dim) with unit channel stride and the given row strides, all
+ * of `dtype`; weight / bias are fp32 (dim); mean / rstd are fp32 (rows, dim / group_size), written
+ * by the forward call and read by the backward call (mean may be null when is_rms).
+ * Backward: dw_part / db_part are caller-provided fp32 (nparts, dim) workspaces (any nparts in
+ * 1..65536; a team of 8 .. 1024 threads, the smallest power of two with 16 * threads >= group_size (128
+ * skipped), works on each (group, part), and a few thousand teams fill the GPU); dweight / dbias are
+ * overwritten with their sums.  group_size <= 32768.
+ * ------------------------------------------------------------------------- */
+typedef struct NormGatedParams {
+  int32_t rows, dim, group_size;
+  int32_t dtype; /* MAMBA_F32 / MAMBA_BF16 / MAMBA_F16 */
+  int32_t is_rms;
+  int32_t norm_before_gate;
+  int32_t nparts; /* backward only */
+  float eps;
+  const void *x;
+  const void *z; /* nullable: no gate */
+  const float *weight;
+  const float *bias; /* nullable */
+  void *out;         /* forward only */
+  float *mean;       /* nullable when is_rms */
+  float *rstd;
+  int64_t x_rs, z_rs, out_rs;
+  /* ---- backward only ---- */
+  const void *dy;
+  void *dx;
+  void *dz; /* null iff z is null */
+  float *dweight;
+  float *dbias; /* null iff bias is null */
+  float *dw_part;
+  float *db_part; /* null iff bias is null */
+  int64_t dy_rs, dx_rs, dz_rs;
+} NormGatedParams;
+
+int norm_gated_fwd(const NormGatedParams *p, mamba_stream_t stream);
+int norm_gated_bwd(const NormGatedParams *p, mamba_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -10,9 +10,9 @@ def install_as_mamba_ssm_ops():
     """Registers the drop-in modules under the reference's module paths, so that
     `from mamba_ssm.ops.selective_scan_interface import selective_scan_fn` (and the SSD / decode
     imports) resolve to this package.  Existing `mamba_ssm` packages are left in place; only the
-    three operator modules are replaced."""
+    operator modules are replaced."""
     from mamba_amd.ops import selective_scan_interface
-    from mamba_amd.ops.triton import selective_state_update, ssd_combined
+    from mamba_amd.ops.triton import layernorm_gated, selective_state_update, ssd_combined
 
     def ensure(name):
         if name not in sys.modules:
@@ -27,6 +27,7 @@ def install_as_mamba_ssm_ops():
         "mamba_ssm.ops.selective_scan_interface": selective_scan_interface,
         "mamba_ssm.ops.triton.ssd_combined": ssd_combined,
         "mamba_ssm.ops.triton.selective_state_update": selective_state_update,
+        "mamba_ssm.ops.triton.layernorm_gated": layernorm_gated,
     }
     for name, mod in mapping.items():
         sys.modules[name] = mod

@@ -67,6 +67,17 @@ class CausalConvParams(ctypes.Structure):
     )
 
 
+class NormGatedParams(ctypes.Structure):
+    _fields_ = (
+        [(n, c_i32) for n in ("rows", "dim", "group_size", "dtype", "is_rms", "norm_before_gate", "nparts")]
+        + [("eps", ctypes.c_float)]
+        + [(n, c_vp) for n in ("x", "z", "weight", "bias", "out", "mean", "rstd")]
+        + [(n, c_i64) for n in ("x_rs", "z_rs", "out_rs")]
+        + [(n, c_vp) for n in ("dy", "dx", "dz", "dweight", "dbias", "dw_part", "db_part")]
+        + [(n, c_i64) for n in ("dy_rs", "dx_rs", "dz_rs")]
+    )
+
+
 _lib = None
 
 
@@ -109,6 +120,10 @@ def load():
     for name in ("causal_conv1d_fwd", "causal_conv1d_bwd"):
         fn = getattr(lib, name)
         fn.argtypes = [ctypes.POINTER(CausalConvParams), c_vp]
+        fn.restype = ctypes.c_int
+    for name in ("norm_gated_fwd", "norm_gated_bwd"):
+        fn = getattr(lib, name)
+        fn.argtypes = [ctypes.POINTER(NormGatedParams), c_vp]
         fn.restype = ctypes.c_int
     _lib = lib
     return lib

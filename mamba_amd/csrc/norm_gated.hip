@@ -5,12 +5,14 @@
 //   x' = norm_before_gate ? x : x * silu(z)
 //   y  = (x' - mean) * rstd * w + b          mean = 0 for RMSNorm, statistics per (row, group)
 //   out = norm_before_gate ? y * silu(z) : y
-// A team of 64, 256 or 1024 threads owns one (row, group) at a time and keeps it in registers, 8
+// A team of 8 to 1024 threads owns one (row, group) at a time and keeps it in registers, 8
 // consecutive channels per thread and step, so x, z and dy are read once and out / dx / dz written
 // once.  A team walks rows r = part, part + nparts, ... of one group; the backward pass keeps the
 // team's sums for dweight / dbias in registers over that walk, stores one partial row per part, and
 // a second kernel adds the parts.
 #include "common.hpp"
+
+#include <type_traits>
 
 namespace {
 
@@ -19,14 +21,19 @@ DEVI float silu_g(float z, float &sig) {
   return z * sig;
 }
 
+// Sums over the TEAM threads that share a (row, group): lanes of one wave by xor shuffles, waves of
+// a workgroup through LDS.
 template <int TEAM> struct TeamSum {
   static constexpr int NW = TEAM / 64;
   float *red;  // LDS: 2 slots x NW x 2 floats
   int slot = 0;
   DEVI explicit TeamSum(float *lds) : red(lds) {}
   DEVI void sum2(float &a, float &b) {
-    a = wave_sum(a);
-    b = wave_sum(b);
+#pragma unroll
+    for (int off = (TEAM < 64 ? TEAM : 64) / 2; off >= 1; off >>= 1) {
+      a += __shfl_xor(a, off, 64);
+      b += __shfl_xor(b, off, 64);
+    }
     if constexpr (NW > 1) {
       const int wave = threadIdx.x >> 6;
       float *s = red + slot * NW * 2;
@@ -47,37 +54,62 @@ template <int TEAM> struct TeamSum {
   }
 };
 
+// Neighbouring teams take neighbouring groups of the same rows, so that a wave of small teams still
+// reads one contiguous stretch of a row.
 struct Item {
   int group, part, col;  // col: first channel of this thread's step 0 inside the group
   bool live;
 };
 template <int TEAM> DEVI Item my_item(const NormGatedParams &p, int nparts) {
   constexpr int WGT = TEAM < 256 ? 256 : TEAM;
+  const int ngroups = p.dim / p.group_size;
   const int team = blockIdx.x * (WGT / TEAM) + threadIdx.x / TEAM;
   Item it;
-  it.part = team % nparts;
-  it.group = team / nparts;
+  it.group = team % ngroups;
+  it.part = team / ngroups;
   it.col = (threadIdx.x % TEAM) * 8;
-  it.live = it.group < p.dim / p.group_size;
+  it.live = it.part < nparts;
   return it;
 }
 
-template <typename T, bool VEC, int K, int TEAM>
-DEVI void load_row(const T *row, int col, int gs, float (&v)[K][8]) {
+// K steps of 8 channels of one row, as loaded (16 bytes per step when VEC): the next row is fetched
+// into this form while the current one is worked on, at half the registers of its fp32 values.
+struct F8 {
+  float f[8];
+};
+template <typename T, bool VEC, int K, int TEAM> struct RowBuf {
+  using Slot = std::conditional_t<VEC, Pack8<T>, F8>;
+  Slot s[K];
+  DEVI void fetch(const T *row, int col, int gs) {
 #pragma unroll
-  for (int k = 0; k < K; ++k) {
-    const int c = col + k * TEAM * 8;
-    const int nv = min(max(gs - c, 0), 8);
-    if (VEC) {
-      if (nv == 8) ld8<T>(row + c, v[k]);
-      else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[k][e] = 0.f;
+    for (int k = 0; k < K; ++k) {
+      const int c = col + k * TEAM * 8;
+      const int nv = min(max(gs - c, 0), 8);
+      if constexpr (VEC) {
+        if (nv == 8) s[k].load(row + c);
+        else s[k].zero();
+      } else {
+        ld8_guard<T, false>(row + c, nv, 0.f, s[k].f);
       }
-    } else {
-      ld8_guard<T, false>(row + c, nv, 0.f, v[k]);
     }
   }
+  DEVI void get(float (&v)[K][8]) const {
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      if constexpr (VEC) s[k].unpack(v[k]);
+      else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[k][e] = s[k].f[e];
+      }
+    }
+  }
+};
+
+template <typename T, bool VEC, int K, int TEAM>
+DEVI void load_row(const T *row, int col, int gs, float (&v)[K][8]) {
+  RowBuf<T, VEC, K, TEAM> b;
+  b.fetch(row, col, gs);
+  b.get(v);
 }
 template <typename T, bool VEC, int K, int TEAM>
 DEVI void store_row(T *row, int col, int gs, const float (&v)[K][8]) {
@@ -91,7 +123,7 @@ DEVI void store_row(T *row, int col, int gs, const float (&v)[K][8]) {
 
 template <typename T, int TEAM, int K, bool VEC>
 __global__ __launch_bounds__(TEAM < 256 ? 256 : TEAM) void norm_fwd_kernel(const NormGatedParams p, int nparts) {
-  __shared__ float lds[2 * (TEAM / 64) * 2];
+  __shared__ float lds[TEAM >= 128 ? 2 * (TEAM / 64) * 2 : 1];
   TeamSum<TEAM> ts(lds);
   const Item it = my_item<TEAM>(p, nparts);
   if (!it.live) return;  // whole teams only; a team of more than one wave is a whole workgroup
@@ -104,11 +136,20 @@ __global__ __launch_bounds__(TEAM < 256 ? 256 : TEAM) void norm_fwd_kernel(const
   const T *zp = p.z ? static_cast<const T *>(p.z) + g0 : nullptr;
   T *op = static_cast<T *>(p.out) + g0;
   const float inv_n = 1.f / (float)gs;
+  RowBuf<T, VEC, K, TEAM> bx, bz;
+  if (it.part < p.rows) {
+    bx.fetch(xp + it.part * p.x_rs, it.col, gs);
+    if (zp) bz.fetch(zp + it.part * p.z_rs, it.col, gs);
+  }
   for (int r = it.part; r < p.rows; r += nparts) {
     float x[K][8], sz[K][8];
-    load_row<T, VEC, K, TEAM>(xp + r * p.x_rs, it.col, gs, x);
+    bx.get(x);
+    if (zp) bz.get(sz);
+    if (r + nparts < p.rows) {
+      bx.fetch(xp + (r + nparts) * p.x_rs, it.col, gs);
+      if (zp) bz.fetch(zp + (r + nparts) * p.z_rs, it.col, gs);
+    }
     if (zp) {
-      load_row<T, VEC, K, TEAM>(zp + r * p.z_rs, it.col, gs, sz);
 #pragma unroll
       for (int k = 0; k < K; ++k)
 #pragma unroll
@@ -159,7 +200,7 @@ __global__ __launch_bounds__(TEAM < 256 ? 256 : TEAM) void norm_fwd_kernel(const
 
 template <typename T, int TEAM, int K, bool VEC>
 __global__ __launch_bounds__(TEAM < 256 ? 256 : TEAM) void norm_bwd_kernel(const NormGatedParams p) {
-  __shared__ float lds[2 * (TEAM / 64) * 2];
+  __shared__ float lds[TEAM >= 128 ? 2 * (TEAM / 64) * 2 : 1];
   TeamSum<TEAM> ts(lds);
   const int nparts = p.nparts;
   const Item it = my_item<TEAM>(p, nparts);
@@ -180,11 +221,23 @@ __global__ __launch_bounds__(TEAM < 256 ? 256 : TEAM) void norm_bwd_kernel(const
   T *dzp = p.z ? static_cast<T *>(p.dz) + g0 : nullptr;
   const float inv_n = 1.f / (float)gs;
   const bool gate_after = zp && p.norm_before_gate, gate_before = zp && !p.norm_before_gate;
+  RowBuf<T, VEC, K, TEAM> bx, bg, bz;
+  if (it.part < p.rows) {
+    bx.fetch(xp + it.part * p.x_rs, it.col, gs);
+    bg.fetch(gp + it.part * p.dy_rs, it.col, gs);
+    if (zp) bz.fetch(zp + it.part * p.z_rs, it.col, gs);
+  }
   for (int r = it.part; r < p.rows; r += nparts) {
     float x[K][8], z[K][8], g[K][8];
-    load_row<T, VEC, K, TEAM>(xp + r * p.x_rs, it.col, gs, x);
-    load_row<T, VEC, K, TEAM>(gp + r * p.dy_rs, it.col, gs, g);
-    if (zp) load_row<T, VEC, K, TEAM>(zp + r * p.z_rs, it.col, gs, z);
+    bx.get(x);
+    bg.get(g);
+    if (zp) bz.get(z);
+    const RowBuf<T, VEC, K, TEAM> xkeep = bx;  // x itself is needed again when the gate comes first
+    if (r + nparts < p.rows) {
+      bx.fetch(xp + (r + nparts) * p.x_rs, it.col, gs);
+      bg.fetch(gp + (r + nparts) * p.dy_rs, it.col, gs);
+      if (zp) bz.fetch(zp + (r + nparts) * p.z_rs, it.col, gs);
+    }
     const float mean = p.is_rms ? 0.f : p.mean[(int64_t)r * ngroups + it.group];
     const float rstd = p.rstd[(int64_t)r * ngroups + it.group];
     float c1 = 0.f, c2 = 0.f;
@@ -218,8 +271,8 @@ __global__ __launch_bounds__(TEAM < 256 ? 256 : TEAM) void norm_bwd_kernel(const
     c1 *= inv_n;
     c2 = p.is_rms ? 0.f : c2 * inv_n;
     if (gate_before) {
-      float xr[K][8];  // x itself is needed again: dz = dx' * x * dsilu(z)
-      load_row<T, VEC, K, TEAM>(xp + r * p.x_rs, it.col, gs, xr);
+      float xr[K][8];  // dz = dx' * x * dsilu(z), dx = dx' * silu(z)
+      xkeep.get(xr);
 #pragma unroll
       for (int k = 0; k < K; ++k)
 #pragma unroll
@@ -301,20 +354,26 @@ template <typename T, int TEAM, int K, bool VEC> int launch(const NormGatedParam
   return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
 }
 
+// The smallest team that holds the group in at most two steps of 8 channels per thread (more steps
+// cost registers, hence waves in flight); only groups beyond 16384 channels take 3 or 4 steps.
 template <typename T, int TEAM, bool VEC> int pick_k(const NormGatedParams &p, bool bwd, hipStream_t st) {
   const int k = (p.group_size + TEAM * 8 - 1) / (TEAM * 8);
-  switch (k) {
-    case 1: return launch<T, TEAM, 1, VEC>(p, bwd, st);
-    case 2: return launch<T, TEAM, 2, VEC>(p, bwd, st);
-    case 3: return launch<T, TEAM, 3, VEC>(p, bwd, st);
-    case 4: return launch<T, TEAM, 4, VEC>(p, bwd, st);
-    default: return MAMBA_E_UNSUPPORTED;
+  if (k == 1) return launch<T, TEAM, 1, VEC>(p, bwd, st);
+  if (k == 2) return launch<T, TEAM, 2, VEC>(p, bwd, st);
+  if constexpr (TEAM == 1024) {
+    if (k == 3) return launch<T, TEAM, 3, VEC>(p, bwd, st);
+    if (k == 4) return launch<T, TEAM, 4, VEC>(p, bwd, st);
   }
+  return MAMBA_E_UNSUPPORTED;
 }
 
 template <typename T, bool VEC> int pick_team(const NormGatedParams &p, bool bwd, hipStream_t st) {
+  if (p.group_size <= 128) return pick_k<T, 8, VEC>(p, bwd, st);
+  if (p.group_size <= 256) return pick_k<T, 16, VEC>(p, bwd, st);
+  if (p.group_size <= 512) return pick_k<T, 32, VEC>(p, bwd, st);
   if (p.group_size <= 1024) return pick_k<T, 64, VEC>(p, bwd, st);
-  if (p.group_size <= 8192) return pick_k<T, 256, VEC>(p, bwd, st);
+  if (p.group_size <= 4096) return pick_k<T, 256, VEC>(p, bwd, st);
+  if (p.group_size <= 8192) return pick_k<T, 512, VEC>(p, bwd, st);
   return pick_k<T, 1024, VEC>(p, bwd, st);
 }
 

@@ -12,6 +12,7 @@ import torch
 
 from mamba_amd import _lib
 from mamba_amd.ops.causal_conv1d import causal_conv1d_fn
+from mamba_amd.ops.triton.layernorm_gated import rmsnorm_fn
 
 
 def _fill_fwd(p, x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, seq_idx, dt_softplus, dt_limit, ws):
@@ -408,9 +409,9 @@ def mamba_split_conv1d_scan_combined(zxbcdt, conv1d_weight, conv1d_bias, dt_bias
                                      rmsnorm_eps=1e-6, outproj_weight=None, outproj_bias=None, headdim=None,
                                      ngroups=1, norm_before_gate=True, state_dtype=None):
     """The Mamba-2 block body after in_proj (ssd_combined.py:983, forward :824-899): split, causal
-    conv1d + SiLU on xBC and the chunked scan on the HIP kernels, gate or gated RMSNorm, out_proj.
-    The norm and the projection are torch operators and their gradients come from autograd; the
-    convolution's and the scan's come from CausalConv1dFn and MambaChunkScanCombinedFn.
+    conv1d + SiLU on xBC, the chunked scan and the gate or gated RMSNorm on the HIP kernels, out_proj.
+    The projection is a torch GEMM; the gradients of the convolution, the scan and the norm come from
+    CausalConv1dFn, MambaChunkScanCombinedFn and LayerNormFn, chained by autograd.
         zxbcdt: (batch, seqlen, 2 * d_nonssm + 2 * dim + 2 * ngroups * dstate + nheads), dim = nheads * headdim
         conv1d_weight: (dim + 2 * ngroups * dstate, width); conv1d_bias: (dim + 2 * ngroups * dstate,)
         dt_bias, A: (nheads,); D: (nheads, headdim) or (nheads,) (then headdim must be given)
@@ -449,8 +450,9 @@ def mamba_split_conv1d_scan_combined(zxbcdt, conv1d_weight, conv1d_bias, dt_bias
     y, final_states = res if return_final_states else (res, None)
     y = y.reshape(batch, seqlen, dim)
     if rmsnorm_weight is not None:
-        y = _gated_rms_norm(y, rmsnorm_weight, z.reshape(batch, seqlen, dim), rmsnorm_eps, dim // ngroups,
-                            norm_before_gate)
+        # reads z where it lies inside zxbcdt (unit channel stride, row stride of the whole projection)
+        y = rmsnorm_fn(y, rmsnorm_weight, None, z=z.reshape(batch, seqlen, dim), eps=rmsnorm_eps,
+                       group_size=dim // ngroups, norm_before_gate=norm_before_gate)
     if d_nonssm > 0:
         gate, up = zx0.chunk(2, dim=-1)
         y = torch.cat([(F.silu(gate.float()) * up.float()).to(y.dtype), y], dim=-1)

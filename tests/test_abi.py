@@ -38,7 +38,7 @@ def test_query_and_strerror():
     assert b"unsupported" in lib.mamba_hip_strerror(-2)
 
 
-@pytest.mark.parametrize("name", ["MambaScanParams", "MambaStepParams", "SsdParams"])
+@pytest.mark.parametrize("name", ["MambaScanParams", "MambaStepParams", "SsdParams", "CausalConvParams", "NormGatedParams"])
 def test_ctypes_structs_match_c_layout(name):
     cls = getattr(_lib, name)
     fields = [f[0] for f in cls._fields_]
@@ -66,6 +66,9 @@ def test_null_and_inconsistent_arguments_are_rejected_before_launch():
     assert lib.ssd_combined_fwd(ctypes.byref(q), None) == -1
     assert lib.ssd_combined_bwd(ctypes.byref(q), None) == -1
     assert lib.mamba_hip_zero(None, 16, None) == -1
+    assert lib.causal_conv1d_fwd(ctypes.byref(_lib.CausalConvParams()), None) == -1
+    assert lib.norm_gated_fwd(ctypes.byref(_lib.NormGatedParams()), None) == -1
+    assert lib.norm_gated_bwd(ctypes.byref(_lib.NormGatedParams()), None) == -1
 
 
 def test_host_ops_refuse_cpu_tensors():
