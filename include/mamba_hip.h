@@ -315,6 +315,57 @@ int causal_conv1d_fwd(const CausalConvParams *p, mamba_stream_t stream);
 int causal_conv1d_bwd(const CausalConvParams *p, mamba_stream_t stream);
 
 /* -------------------------------------------------------------------------
+ * Causal conv1d, decode step: with xn = [conv_state, x] along the position axis,
+ *   out[b, c, t] = act(bias[c] + sum_k weight[c, k] * xn[b, c, state_len + t - (width-1) + k]),
+ *   conv_state[b, c, :] <- the last state_len positions of xn      (in place)
+ * Replaces the causal_conv1d package's causal_conv1d_update as the reference calls it
+ * (mamba_ssm/modules/mamba2.py:298-304, mamba_ssm/modules/mamba_simple.py:223-229) and the
+ * roll + insert + dot it falls back to (mamba2.py:291-296).
+ * x, out: (batch, dim, seqlen) of `dtype`, any strides; conv_state: (rows, dim, state_len) of
+ * `state_dtype`, any strides, state_len >= width - 1; conv_state_indices (nullable): int32 (batch,),
+ * row of conv_state per batch entry; outside [0, state_rows) = padding entry (state untouched,
+ * out = 0).
+ * ------------------------------------------------------------------------- */
+typedef struct CausalConvUpdateParams {
+  int32_t batch, dim, seqlen, width, state_len;
+  int32_t dtype, state_dtype;
+  int32_t silu;
+  int32_t state_rows; /* rows of conv_state; an index outside [0, state_rows) is a padding entry */
+  int32_t reserved;
+  const void *x;
+  void *conv_state;
+  const float *weight;
+  const float *bias; /* nullable */
+  void *out;
+  const int32_t *conv_state_indices; /* nullable */
+  int64_t x_bs, x_cs, x_ls;
+  int64_t out_bs, out_cs, out_ls;
+  int64_t state_bs, state_cs, state_ls;
+} CausalConvUpdateParams;
+
+int causal_conv1d_update(const CausalConvUpdateParams *p, mamba_stream_t stream);
+
+/* -------------------------------------------------------------------------
+ * Convolution states of the sequences of one packed row:
+ *   states[s, c, j] = x[cu_seqlens[s+1] - state_len + j, c], 0 before the start of sequence s.
+ * Replaces causal_conv1d.causal_conv1d_varlen.causal_conv1d_varlen_states as called at
+ * mamba_ssm/modules/mamba2.py:225-227 (per sequence it is the F.pad of :221).
+ * x: (total, dim); cu_seqlens: int32 (nseq + 1); states: (nseq, dim, state_len); all of `dtype`.
+ * ------------------------------------------------------------------------- */
+typedef struct CausalConvVarlenParams {
+  int32_t nseq, dim, total, state_len;
+  int32_t dtype;
+  int32_t reserved;
+  const void *x;
+  const int32_t *cu_seqlens;
+  void *states;
+  int64_t x_ls, x_cs;
+  int64_t states_bs, states_cs, states_ls;
+} CausalConvVarlenParams;
+
+int causal_conv1d_varlen_states(const CausalConvVarlenParams *p, mamba_stream_t stream);
+
+/* -------------------------------------------------------------------------
  * Gated LayerNorm / RMSNorm over groups of channels: the epilogue of the Mamba-2 block between
  * the chunked scan and the output projection.  Replaces the Triton launches of
  * mamba_ssm/ops/triton/layernorm_gated.py:108 (_layer_norm_fwd) and :271 (_layer_norm_bwd),

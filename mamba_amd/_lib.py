@@ -67,6 +67,23 @@ class CausalConvParams(ctypes.Structure):
     )
 
 
+class CausalConvUpdateParams(ctypes.Structure):
+    _fields_ = (
+        [(n, c_i32) for n in ("batch", "dim", "seqlen", "width", "state_len", "dtype", "state_dtype", "silu",
+                                "state_rows", "reserved")]
+        + [(n, c_vp) for n in ("x", "conv_state", "weight", "bias", "out", "conv_state_indices")]
+        + [(n, c_i64) for n in ("x_bs", "x_cs", "x_ls", "out_bs", "out_cs", "out_ls", "state_bs", "state_cs", "state_ls")]
+    )
+
+
+class CausalConvVarlenParams(ctypes.Structure):
+    _fields_ = (
+        [(n, c_i32) for n in ("nseq", "dim", "total", "state_len", "dtype", "reserved")]
+        + [(n, c_vp) for n in ("x", "cu_seqlens", "states")]
+        + [(n, c_i64) for n in ("x_ls", "x_cs", "states_bs", "states_cs", "states_ls")]
+    )
+
+
 class NormGatedParams(ctypes.Structure):
     _fields_ = (
         [(n, c_i32) for n in ("rows", "dim", "group_size", "dtype", "is_rms", "norm_before_gate", "nparts")]
@@ -121,6 +138,10 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = [ctypes.POINTER(CausalConvParams), c_vp]
         fn.restype = ctypes.c_int
+    lib.causal_conv1d_update.argtypes = [ctypes.POINTER(CausalConvUpdateParams), c_vp]
+    lib.causal_conv1d_update.restype = ctypes.c_int
+    lib.causal_conv1d_varlen_states.argtypes = [ctypes.POINTER(CausalConvVarlenParams), c_vp]
+    lib.causal_conv1d_varlen_states.restype = ctypes.c_int
     for name in ("norm_gated_fwd", "norm_gated_bwd"):
         fn = getattr(lib, name)
         fn.argtypes = [ctypes.POINTER(NormGatedParams), c_vp]

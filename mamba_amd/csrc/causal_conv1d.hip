@@ -372,6 +372,68 @@ template <typename T, bool VEC> __global__ __launch_bounds__(256) void conv_cl_b
   }
 }
 
+// ------------------------------------------------------------------ decode step
+// One thread per (batch entry, channel): with xn = [conv_state, x] along the position axis,
+//   out[t] = act(bias + sum_k w[k] xn[state_len + t - (W-1) + k]),  conv_state <- last state_len of xn
+// (what the reference spells, for one new position and state_len = W, as roll + insert + dot:
+// mamba_ssm/modules/mamba2.py:291-296).  The shift runs in place in ascending order, which is safe
+// because every entry is written from a higher index of the same thread's own row.
+template <typename T, typename S> __global__ __launch_bounds__(256) void conv_update_kernel(const CausalConvUpdateParams p) {
+  const int c = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
+  if (c >= p.dim) return;
+  const T *x = static_cast<const T *>(p.x) + b * p.x_bs + c * p.x_cs;
+  T *out = static_cast<T *>(p.out) + b * p.out_bs + c * p.out_cs;
+  const int slot = p.conv_state_indices ? p.conv_state_indices[b] : b;
+  if (slot < 0 || slot >= p.state_rows) {  // padding entry of the batch: no state, zero output
+    for (int t = 0; t < p.seqlen; ++t) st1<T>(out + t * p.out_ls, 0.f);
+    return;
+  }
+  S *st = static_cast<S *>(p.conv_state) + slot * p.state_bs + c * p.state_cs;
+  float w[MAXW], bias;
+#pragma unroll
+  for (int k = 0; k < MAXW; ++k) {
+    const int j = k - (MAXW - p.width);
+    w[k] = j >= 0 ? p.weight[(int64_t)c * p.width + j] : 0.f;
+  }
+  bias = p.bias ? p.bias[c] : 0.f;
+  const int SL = p.state_len;
+  float win[MAXW];  // win[0..2]: the three positions before the next output, win[3]: the new one
+#pragma unroll
+  for (int i = 0; i < MAXW - 1; ++i) {
+    const int j = SL - (MAXW - 1) + i;
+    win[i] = j >= 0 ? ld1<S>(st + j * p.state_ls) : 0.f;
+  }
+  for (int j = 0; j < SL; ++j) {
+    const int src = j + p.seqlen;
+    const float v = src < SL ? ld1<S>(st + src * p.state_ls) : ld1<T>(x + (src - SL) * p.x_ls);
+    st1<S>(st + j * p.state_ls, v);
+  }
+  for (int t = 0; t < p.seqlen; ++t) {
+    win[3] = ld1<T>(x + t * p.x_ls);
+    float v = bias;
+#pragma unroll
+    for (int k = 0; k < MAXW; ++k) v = __builtin_fmaf(w[k], win[k], v);
+    st1<T>(out + t * p.out_ls, p.silu ? silu_f(v) : v);
+    win[0] = win[1];
+    win[1] = win[2];
+    win[2] = win[3];
+  }
+}
+
+// states[s, c, j] = x[cu_seqlens[s + 1] - state_len + j, c], zero where that position lies before
+// the start of sequence s: the convolution state each sequence of a packed row leaves behind.
+template <typename T> __global__ __launch_bounds__(256) void conv_varlen_states_kernel(const CausalConvVarlenParams p) {
+  const int c = blockIdx.x * 256 + threadIdx.x, s = blockIdx.y;
+  if (c >= p.dim) return;
+  const int beg = p.cu_seqlens[s], end = p.cu_seqlens[s + 1];
+  const T *x = static_cast<const T *>(p.x) + c * p.x_cs;
+  T *o = static_cast<T *>(p.states) + s * p.states_bs + c * p.states_cs;
+  for (int j = 0; j < p.state_len; ++j) {
+    const int l = end - p.state_len + j;
+    st1<T>(o + j * p.states_ls, l >= beg && l >= 0 && l < p.total ? ld1<T>(x + l * p.x_ls) : 0.f);
+  }
+}
+
 // ------------------------------------------------------------------ launch
 int check(const CausalConvParams *p, bool bwd) {
   if (!p || !p->x || !p->weight) return MAMBA_E_BADARG;
@@ -433,7 +495,49 @@ int dispatch(const CausalConvParams *p, bool bwd, mamba_stream_t stream) {
   }
 }
 
+template <typename T> int launch_update(const CausalConvUpdateParams &p, hipStream_t s) {
+  dim3 grid((p.dim + 255) / 256, p.batch);
+  switch (p.state_dtype) {
+    case MAMBA_F32: hipLaunchKernelGGL((conv_update_kernel<T, float>), grid, dim3(256), 0, s, p); break;
+    case MAMBA_BF16: hipLaunchKernelGGL((conv_update_kernel<T, bf16_t>), grid, dim3(256), 0, s, p); break;
+    case MAMBA_F16: hipLaunchKernelGGL((conv_update_kernel<T, f16_t>), grid, dim3(256), 0, s, p); break;
+    default: return MAMBA_E_BADARG;
+  }
+  return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
+}
+
 }  // namespace
 
 extern "C" int causal_conv1d_fwd(const CausalConvParams *p, mamba_stream_t stream) { return dispatch(p, false, stream); }
 extern "C" int causal_conv1d_bwd(const CausalConvParams *p, mamba_stream_t stream) { return dispatch(p, true, stream); }
+
+extern "C" int causal_conv1d_update(const CausalConvUpdateParams *p, mamba_stream_t stream) {
+  if (!p || !p->x || !p->conv_state || !p->weight || !p->out) return MAMBA_E_BADARG;
+  if (p->batch <= 0 || p->dim <= 0 || p->seqlen <= 0 || p->state_len < 0) return MAMBA_E_BADARG;
+  if (p->width < 2 || p->width > MAXW) return MAMBA_E_UNSUPPORTED;
+  if (p->state_len < p->width - 1 || p->state_rows <= 0) return MAMBA_E_BADARG;
+  if (!p->conv_state_indices && p->state_rows < p->batch) return MAMBA_E_BADARG;
+  if (p->batch > 65535) return MAMBA_E_UNSUPPORTED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (p->dtype) {
+    case MAMBA_F32: return launch_update<float>(*p, s);
+    case MAMBA_BF16: return launch_update<bf16_t>(*p, s);
+    case MAMBA_F16: return launch_update<f16_t>(*p, s);
+    default: return MAMBA_E_BADARG;
+  }
+}
+
+extern "C" int causal_conv1d_varlen_states(const CausalConvVarlenParams *p, mamba_stream_t stream) {
+  if (!p || !p->x || !p->cu_seqlens || !p->states) return MAMBA_E_BADARG;
+  if (p->nseq <= 0 || p->dim <= 0 || p->total < 0 || p->state_len <= 0) return MAMBA_E_BADARG;
+  if (p->nseq > 65535) return MAMBA_E_UNSUPPORTED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  dim3 grid((p->dim + 255) / 256, p->nseq);
+  switch (p->dtype) {
+    case MAMBA_F32: hipLaunchKernelGGL((conv_varlen_states_kernel<float>), grid, dim3(256), 0, s, *p); break;
+    case MAMBA_BF16: hipLaunchKernelGGL((conv_varlen_states_kernel<bf16_t>), grid, dim3(256), 0, s, *p); break;
+    case MAMBA_F16: hipLaunchKernelGGL((conv_varlen_states_kernel<f16_t>), grid, dim3(256), 0, s, *p); break;
+    default: return MAMBA_E_BADARG;
+  }
+  return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
+}

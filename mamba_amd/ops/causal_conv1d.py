@@ -127,3 +127,84 @@ def causal_conv1d_fn(x, weight, bias=None, seq_idx=None, initial_states=None, re
     if initial_states is not None or return_final_states or final_states_out is not None:
         raise NotImplementedError("causal_conv1d_fn: streaming conv states are not supported")
     return CausalConv1dFn.apply(x, weight, bias, seq_idx, activation)
+
+
+def causal_conv1d_update(x, conv_state, weight, bias=None, activation=None, cache_seqlens=None,
+                         conv_state_indices=None):
+    """Decode step (the package's causal_conv1d_update as called at mamba_ssm/modules/mamba2.py:298,
+    mamba_ssm/modules/mamba_simple.py:223).
+        x: (batch, dim) or (batch, dim, seqlen): the new position(s)
+        conv_state: (rows, dim, state_len), state_len >= width - 1, updated in place to the last
+            state_len positions of [conv_state, x]
+        weight: (dim, width); bias: (dim,)
+        conv_state_indices: (batch,) int32, row of conv_state per batch entry (negative: padding)
+    Returns out with x's shape and dtype."""
+    if cache_seqlens is not None:
+        raise NotImplementedError("causal_conv1d_update: circular-buffer states (cache_seqlens) are not supported")
+    if activation not in (None, "silu", "swish"):
+        raise NotImplementedError("activation must be None, silu, or swish")
+    _lib.require_gpu(x, conv_state, weight, bias, conv_state_indices)
+    squeeze = x.dim() == 2
+    if squeeze:
+        x = x.unsqueeze(-1)
+    batch, dim, seqlen = x.shape
+    width = weight.shape[1]
+    if x.dtype not in _lib.DTYPE_CODE or conv_state.dtype not in _lib.DTYPE_CODE:
+        raise RuntimeError("causal_conv1d_update: x and conv_state must be fp32, fp16 or bf16")
+    if weight.shape[0] != dim or not 2 <= width <= 4:
+        raise RuntimeError("causal_conv1d_update: weight must be (dim, width) with width between 2 and 4")
+    if conv_state.dim() != 3 or conv_state.shape[1] != dim or conv_state.shape[2] < width - 1:
+        raise RuntimeError("causal_conv1d_update: conv_state must be (rows, dim, state_len >= width - 1)")
+    if conv_state_indices is None:
+        if conv_state.shape[0] != batch:
+            raise RuntimeError("causal_conv1d_update: conv_state must have one row per batch entry")
+    else:
+        if tuple(conv_state_indices.shape) != (batch,) or conv_state_indices.dtype != torch.int32:
+            raise RuntimeError("causal_conv1d_update: conv_state_indices must be (batch,) int32")
+        conv_state_indices = conv_state_indices.contiguous()
+    if bias is not None and tuple(bias.shape) != (dim,):
+        raise RuntimeError("causal_conv1d_update: bias must be (dim,)")
+    out = torch.empty_like(x)
+    if batch == 0:
+        return out.squeeze(-1) if squeeze else out
+    w32 = weight.detach().float().contiguous()
+    b32 = bias.detach().float().contiguous() if bias is not None else None
+    p = _lib.CausalConvUpdateParams()
+    p.batch, p.dim, p.seqlen, p.width, p.state_len = batch, dim, seqlen, width, conv_state.shape[2]
+    p.dtype, p.state_dtype = _lib.DTYPE_CODE[x.dtype], _lib.DTYPE_CODE[conv_state.dtype]
+    p.silu, p.state_rows = int(activation in ("silu", "swish")), conv_state.shape[0]
+    p.x, p.conv_state, p.weight, p.bias, p.out = x.data_ptr(), conv_state.data_ptr(), w32.data_ptr(), _lib.ptr(b32), out.data_ptr()
+    p.conv_state_indices = _lib.ptr(conv_state_indices)
+    p.x_bs, p.x_cs, p.x_ls = _strides_bcl(x)
+    p.out_bs, p.out_cs, p.out_ls = _strides_bcl(out)
+    p.state_bs, p.state_cs, p.state_ls = _strides_bcl(conv_state)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().causal_conv1d_update(p, _lib.current_stream(x.device)), "causal_conv1d_update")
+    return out.squeeze(-1) if squeeze else out
+
+
+def causal_conv1d_varlen_states(x, cu_seqlens, state_len):
+    """Convolution state left by each sequence of a packed row (the package's
+    causal_conv1d_varlen_states as called at mamba_ssm/modules/mamba2.py:225).
+        x: (total, dim); cu_seqlens: (nseq + 1,) int32 starting at 0
+    Returns (nseq, dim, state_len), channel-contiguous: the last state_len positions of each
+    sequence, zero-filled on the left where the sequence is shorter."""
+    _lib.require_gpu(x, cu_seqlens)
+    if x.dim() != 2 or x.dtype not in _lib.DTYPE_CODE:
+        raise RuntimeError("causal_conv1d_varlen_states: x must be (total, dim) in fp32, fp16 or bf16")
+    if cu_seqlens.dim() != 1 or cu_seqlens.dtype != torch.int32 or cu_seqlens.numel() < 1:
+        raise RuntimeError("causal_conv1d_varlen_states: cu_seqlens must be (nseq + 1,) int32")
+    total, dim = x.shape
+    nseq = cu_seqlens.numel() - 1
+    states = torch.empty(nseq, state_len, dim, dtype=x.dtype, device=x.device).transpose(1, 2)
+    if nseq == 0 or state_len == 0:
+        return states
+    cu_seqlens = cu_seqlens.contiguous()
+    p = _lib.CausalConvVarlenParams()
+    p.nseq, p.dim, p.total, p.state_len, p.dtype = nseq, dim, total, state_len, _lib.DTYPE_CODE[x.dtype]
+    p.x, p.cu_seqlens, p.states = x.data_ptr(), cu_seqlens.data_ptr(), states.data_ptr()
+    p.x_ls, p.x_cs = x.stride(0), x.stride(1)
+    p.states_bs, p.states_cs, p.states_ls = _strides_bcl(states)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().causal_conv1d_varlen_states(p, _lib.current_stream(x.device)), "causal_conv1d_varlen_states")
+    return states

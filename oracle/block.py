@@ -35,6 +35,35 @@ def causal_conv1d_oracle(x, weight, bias=None, activation="silu", seq_idx=None):
     return F.silu(y) if activation in ("silu", "swish") else y
 
 
+def causal_conv1d_update_oracle(x, conv_state, weight, bias=None, activation="silu"):
+    """Decode step of the convolution: x (batch, dim, seqlen), conv_state (batch, dim, state_len),
+    weight (dim, width).  Returns (out, new_state); generalises the roll + insert + dot of reference
+    mamba_ssm/modules/mamba2.py:291-296 (one new position, state_len = width) to seqlen new positions
+    and any state_len >= width - 1 by running the full convolution over [conv_state, x]."""
+    batch, dim, seqlen = x.shape
+    state_len, width = conv_state.shape[2], weight.shape[1]
+    xn = torch.cat([conv_state.to(x.dtype), x], dim=-1)
+    out = torch.zeros_like(x)
+    for t in range(seqlen):
+        for k in range(width):
+            out[:, :, t] += weight[:, k] * xn[:, :, state_len + t - (width - 1) + k]
+    if bias is not None:
+        out = out + bias[None, :, None]
+    if activation in ("silu", "swish"):
+        out = F.silu(out)
+    return out, xn[:, :, xn.shape[2] - state_len:]
+
+
+def causal_conv1d_varlen_states_oracle(x, cu_seqlens, state_len):
+    """x: (total, dim).  Per sequence the F.pad(x_seq^T, (state_len - len, 0)) of reference
+    mamba_ssm/modules/mamba2.py:219-221: the last state_len positions, zero-filled on the left."""
+    out = []
+    for s in range(len(cu_seqlens) - 1):
+        seq = x[int(cu_seqlens[s]):int(cu_seqlens[s + 1])].transpose(0, 1)
+        out.append(F.pad(seq, (state_len - seq.shape[1], 0)))
+    return torch.stack(out)
+
+
 def gated_rms_norm_oracle(x, weight, z, eps, group_size, norm_before_gate):
     x, z, weight = x.double(), z.double(), weight.double()
     if not norm_before_gate:

@@ -38,7 +38,8 @@ def test_query_and_strerror():
     assert b"unsupported" in lib.mamba_hip_strerror(-2)
 
 
-@pytest.mark.parametrize("name", ["MambaScanParams", "MambaStepParams", "SsdParams", "CausalConvParams", "NormGatedParams"])
+@pytest.mark.parametrize("name", ["MambaScanParams", "MambaStepParams", "SsdParams", "CausalConvParams", "CausalConvUpdateParams",
+                                  "CausalConvVarlenParams", "NormGatedParams"])
 def test_ctypes_structs_match_c_layout(name):
     cls = getattr(_lib, name)
     fields = [f[0] for f in cls._fields_]

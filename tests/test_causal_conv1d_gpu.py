@@ -3,7 +3,7 @@ by tests/test_oracle_block.py against F.conv1d), forward and every gradient, bot
 import pytest
 import torch
 
-from oracle.block import causal_conv1d_oracle
+from oracle.block import causal_conv1d_oracle, causal_conv1d_update_oracle, causal_conv1d_varlen_states_oracle
 
 pytestmark = pytest.mark.gpu
 
@@ -81,3 +81,64 @@ def test_causal_conv1d_strided_view():
     ref = causal_conv1d_oracle(full[:, :, 16:64].float(), w.float(), None, "silu")
     out = causal_conv1d_fn(full.cuda()[:, :, 16:64].transpose(1, 2), w.cuda(), None, activation="silu")
     _close("out", out.transpose(1, 2), ref, 3e-2, 5e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("channel_last_state", [False, True])
+@pytest.mark.parametrize("width,state_len,seqlen", [(4, 4, 1), (4, 3, 1), (3, 3, 1), (2, 1, 1), (4, 7, 3), (4, 4, 6), (2, 5, 2)])
+def test_causal_conv1d_update(width, state_len, seqlen, channel_last_state, dtype):
+    from mamba_amd.ops.causal_conv1d import causal_conv1d_update
+    g = torch.Generator().manual_seed(width * 100 + state_len * 10 + seqlen)
+    batch, dim = 3, 200
+    x = torch.randn(batch, dim, seqlen, generator=g).to(dtype)
+    state = torch.randn(batch, dim, state_len, generator=g).to(dtype)
+    w = (torch.randn(dim, width, generator=g) * 0.5).to(dtype)
+    bias = torch.randn(dim, generator=g).to(dtype)
+    rtol, atol = _tol(dtype)
+    ref, new_ref = causal_conv1d_update_oracle(x.float(), state.float(), w.float(), bias.float(), "silu")
+    sg = state.cuda()
+    if channel_last_state:  # the layout the Mamba-2 module allocates (mamba_ssm/modules/mamba2.py:333-335)
+        sg = sg.transpose(1, 2).contiguous().transpose(1, 2)
+    xg = x.cuda() if seqlen > 1 else x.cuda()[:, :, 0]
+    out = causal_conv1d_update(xg, sg, w.cuda(), bias.cuda(), "silu")
+    assert out.shape == xg.shape and out.dtype == dtype
+    _close("out", out.reshape(batch, dim, seqlen), ref, rtol, atol)
+    assert torch.equal(sg.cpu(), new_ref.to(dtype))  # the state only moves values
+
+
+def test_causal_conv1d_update_steps_match_the_sequence_kernel_and_indices():
+    from mamba_amd.ops.causal_conv1d import causal_conv1d_fn, causal_conv1d_update
+    g = torch.Generator().manual_seed(3)
+    batch, dim, L, width = 4, 96, 9, 4
+    x = torch.randn(batch, dim, L, generator=g).to(torch.bfloat16).cuda()
+    w = (torch.randn(dim, width, generator=g) * 0.5).cuda()
+    bias = torch.randn(dim, generator=g).cuda()
+    full = causal_conv1d_fn(x, w, bias, activation="silu")
+    # states live in a pool of 7 rows; entry 2 of the batch is padding
+    pool = torch.zeros(7, dim, width, dtype=torch.bfloat16, device="cuda")
+    idx = torch.tensor([5, 0, -1, 3], dtype=torch.int32, device="cuda")
+    untouched = pool.clone()
+    for t in range(L):
+        out = causal_conv1d_update(x[:, :, t], pool, w, bias, "silu", conv_state_indices=idx)
+        keep = [0, 1, 3]
+        _close(f"step {t}", out[keep], full[keep, :, t], 3e-2, 5e-2)
+        assert float(out[2].abs().max()) == 0.0
+    assert torch.equal(pool[[1, 2, 4, 6]], untouched[[1, 2, 4, 6]])
+    assert torch.equal(pool[5], x[0, :, L - width:])
+    with pytest.raises(NotImplementedError):
+        causal_conv1d_update(x[:, :, 0], pool[:4], w, bias, "silu", cache_seqlens=idx)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_causal_conv1d_varlen_states(dtype):
+    from mamba_amd.ops.causal_conv1d import causal_conv1d_varlen_states
+    g = torch.Generator().manual_seed(4)
+    lens = [5, 1, 2, 300, 4, 3]
+    total, dim = sum(lens), 520
+    x = torch.randn(total, dim + 8, generator=g).to(dtype)[:, :dim]          # rows of a wider buffer
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    for state_len in (3, 4):
+        ref = causal_conv1d_varlen_states_oracle(x, cu, state_len)
+        got = causal_conv1d_varlen_states(x.cuda(), cu.cuda(), state_len)
+        assert got.shape == (len(lens), dim, state_len) and got.stride(1) == 1
+        assert torch.equal(got.cpu(), ref)

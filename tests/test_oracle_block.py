@@ -3,7 +3,8 @@ host modules export next to the operators; none of this needs a GPU."""
 import torch
 import torch.nn.functional as F
 
-from oracle.block import causal_conv1d_oracle, gated_rms_norm_oracle, split_conv1d_scan_oracle
+from oracle.block import (causal_conv1d_oracle, causal_conv1d_update_oracle, causal_conv1d_varlen_states_oracle,
+                          gated_rms_norm_oracle, split_conv1d_scan_oracle)
 from oracle.ssd import ssd_oracle, ssd_inputs
 from oracle.step import selective_state_update_oracle
 
@@ -145,3 +146,40 @@ def test_selective_scan_ref_utility_matches_the_oracle_real_and_complex():
         got, st = selective_scan_ref(u, delta, A, Bv, Cm, D, z, bias, True, return_last_state=True)
         ref, st_ref = selective_scan_oracle(u, delta, A, Bv, Cm, D, z, bias, True, return_last_state=True)
         assert torch.allclose(got, ref, atol=1e-5) and torch.allclose(st, st_ref, atol=1e-5)
+
+
+def test_conv_update_is_the_roll_insert_dot_and_continues_the_full_convolution():
+    g = torch.Generator().manual_seed(5)
+    batch, dim, width = 2, 6, 4
+    wt = torch.randn(dim, width, generator=g, dtype=torch.float64)
+    bias = torch.randn(dim, generator=g, dtype=torch.float64)
+    state = torch.randn(batch, dim, width, generator=g, dtype=torch.float64)
+    x = torch.randn(batch, dim, 1, generator=g, dtype=torch.float64)
+    out, new = causal_conv1d_update_oracle(x, state, wt, bias, "silu")
+    # the reference's own spelling for one new position (mamba_ssm/modules/mamba2.py:291-296)
+    rolled = torch.roll(state, shifts=-1, dims=-1)
+    rolled[:, :, -1] = x[:, :, 0]
+    assert torch.allclose(new, rolled)
+    assert torch.allclose(out[:, :, 0], F.silu((rolled * wt).sum(-1) + bias), atol=1e-12)
+    # steps over a sequence == the full causal convolution of that sequence; state_len = width - 1 and longer
+    seq = torch.randn(batch, 11, dim, generator=g, dtype=torch.float64)
+    full = causal_conv1d_oracle(seq, wt, bias, "silu")
+    for state_len, chunk in ((3, 1), (3, 4), (7, 2), (5, 11)):
+        st = torch.zeros(batch, dim, state_len, dtype=torch.float64)
+        outs = []
+        for t0 in range(0, 11, chunk):
+            o, st = causal_conv1d_update_oracle(seq[:, t0:t0 + chunk].transpose(1, 2), st, wt, bias, "silu")
+            outs.append(o)
+        assert torch.allclose(torch.cat(outs, dim=-1).transpose(1, 2), full, atol=1e-12)
+        keep = min(state_len, 11)
+        assert torch.allclose(st[:, :, state_len - keep:], seq[:, 11 - keep:].transpose(1, 2))
+
+
+def test_varlen_states_are_the_tails_of_the_sequences():
+    x = torch.arange(10 * 3, dtype=torch.float64).reshape(10, 3) + 1
+    cu = torch.tensor([0, 2, 7, 10], dtype=torch.int32)
+    st = causal_conv1d_varlen_states_oracle(x, cu, 4)
+    assert st.shape == (3, 3, 4)
+    assert torch.equal(st[0, 0], torch.tensor([0, 0, x[0, 0], x[1, 0]], dtype=torch.float64))
+    assert torch.equal(st[1, 2], x[3:7, 2])
+    assert torch.equal(st[2, 1], torch.tensor([0, x[7, 1], x[8, 1], x[9, 1]], dtype=torch.float64))
