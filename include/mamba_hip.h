@@ -409,6 +409,52 @@ typedef struct NormGatedParams {
 int norm_gated_fwd(const NormGatedParams *p, mamba_stream_t stream);
 int norm_gated_bwd(const NormGatedParams *p, mamba_stream_t stream);
 
+/* -------------------------------------------------------------------------
+ * LayerNorm / RMSNorm of (x + residual) with the sum handed on: the norm in front of every mixer
+ * of the reference's Block (mamba_ssm/modules/block.py:57-66).  Replaces the Triton launches of
+ * mamba_ssm/ops/triton/layer_norm.py:291 (_layer_norm_fwd) and :589 (_layer_norm_bwd) for the
+ * arguments the Block uses (residual, prenorm, residual_in_fp32; no dropout, rowscale or second
+ * branch).
+ *   forward:  s = x + residual;  residual_out = s;  out = (s - mean) * rstd * weight + bias
+ *   backward: dx = d_norm(dy) + dresidual, written as dx (dtype) and dresidual_in (res_dtype)
+ * x, out, dy, dx are (rows, dim) of `dtype`; residual, residual_out, dresidual, dresidual_in of
+ * `res_dtype` (equal to dtype, or fp32); unit channel stride, row strides given.  In the backward
+ * call `x` is the summed input the forward call wrote (residual_out, or x itself when there was
+ * neither a residual nor a residual_out), of res_dtype.  weight / bias fp32 (dim); mean / rstd fp32
+ * (rows), mean nullable when is_rms.  dw_part / db_part: fp32 (nparts, dim) workspaces, any nparts
+ * in 1..65536; dweight / dbias are overwritten with the sums.  dim <= 32768.
+ * ------------------------------------------------------------------------- */
+typedef struct NormResidualParams {
+  int32_t rows, dim;
+  int32_t dtype, res_dtype;
+  int32_t is_rms;
+  int32_t nparts; /* backward only */
+  float eps;
+  int32_t reserved;
+  const void *x;
+  const void *residual; /* forward, nullable */
+  const float *weight;
+  const float *bias;  /* nullable */
+  void *out;          /* forward only */
+  void *residual_out; /* forward, nullable */
+  float *mean;        /* nullable when is_rms */
+  float *rstd;
+  int64_t x_rs, residual_rs, out_rs, residual_out_rs;
+  /* ---- backward only ---- */
+  const void *dy;
+  const void *dresidual; /* nullable */
+  void *dx;
+  void *dresidual_in; /* nullable */
+  float *dweight;
+  float *dbias; /* null iff bias is null */
+  float *dw_part;
+  float *db_part; /* null iff bias is null */
+  int64_t dy_rs, dresidual_rs, dx_rs, dresidual_in_rs;
+} NormResidualParams;
+
+int norm_residual_fwd(const NormResidualParams *p, mamba_stream_t stream);
+int norm_residual_bwd(const NormResidualParams *p, mamba_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

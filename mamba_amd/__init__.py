@@ -12,7 +12,7 @@ def install_as_mamba_ssm_ops():
     imports) resolve to this package.  Existing `mamba_ssm` packages are left in place; only the
     operator modules are replaced."""
     from mamba_amd.ops import selective_scan_interface
-    from mamba_amd.ops.triton import layernorm_gated, selective_state_update, ssd_combined
+    from mamba_amd.ops.triton import layer_norm, layernorm_gated, selective_state_update, ssd_combined
 
     def ensure(name):
         if name not in sys.modules:
@@ -28,6 +28,7 @@ def install_as_mamba_ssm_ops():
         "mamba_ssm.ops.triton.ssd_combined": ssd_combined,
         "mamba_ssm.ops.triton.selective_state_update": selective_state_update,
         "mamba_ssm.ops.triton.layernorm_gated": layernorm_gated,
+        "mamba_ssm.ops.triton.layer_norm": layer_norm,
     }
     for name, mod in mapping.items():
         sys.modules[name] = mod

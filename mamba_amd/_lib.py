@@ -95,6 +95,17 @@ class NormGatedParams(ctypes.Structure):
     )
 
 
+class NormResidualParams(ctypes.Structure):
+    _fields_ = (
+        [(n, c_i32) for n in ("rows", "dim", "dtype", "res_dtype", "is_rms", "nparts")]
+        + [("eps", ctypes.c_float), ("reserved", c_i32)]
+        + [(n, c_vp) for n in ("x", "residual", "weight", "bias", "out", "residual_out", "mean", "rstd")]
+        + [(n, c_i64) for n in ("x_rs", "residual_rs", "out_rs", "residual_out_rs")]
+        + [(n, c_vp) for n in ("dy", "dresidual", "dx", "dresidual_in", "dweight", "dbias", "dw_part", "db_part")]
+        + [(n, c_i64) for n in ("dy_rs", "dresidual_rs", "dx_rs", "dresidual_in_rs")]
+    )
+
+
 _lib = None
 
 
@@ -145,6 +156,10 @@ def load():
     for name in ("norm_gated_fwd", "norm_gated_bwd"):
         fn = getattr(lib, name)
         fn.argtypes = [ctypes.POINTER(NormGatedParams), c_vp]
+        fn.restype = ctypes.c_int
+    for name in ("norm_residual_fwd", "norm_residual_bwd"):
+        fn = getattr(lib, name)
+        fn.argtypes = [ctypes.POINTER(NormResidualParams), c_vp]
         fn.restype = ctypes.c_int
     _lib = lib
     return lib

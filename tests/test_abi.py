@@ -39,7 +39,7 @@ def test_query_and_strerror():
 
 
 @pytest.mark.parametrize("name", ["MambaScanParams", "MambaStepParams", "SsdParams", "CausalConvParams", "CausalConvUpdateParams",
-                                  "CausalConvVarlenParams", "NormGatedParams"])
+                                  "CausalConvVarlenParams", "NormGatedParams", "NormResidualParams"])
 def test_ctypes_structs_match_c_layout(name):
     cls = getattr(_lib, name)
     fields = [f[0] for f in cls._fields_]
