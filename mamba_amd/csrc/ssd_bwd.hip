@@ -728,7 +728,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dB_
 // one sequence.  One workgroup per (batch, chunk, group, lower-triangular 64 x 64 tile pair) loops
 // over the heads of the group with the sum in registers.  Per head, w = (head's term) * CB gives
 // the in-chunk share of ddA_cumsum: + row sums at l, - column sums at s.
-template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dcb_kernel(const SsdParams p) {
+template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_dcb_kernel(const SsdParams p) {
   __shared__ GemmLds lds;
   __shared__ float hA_l[2][GB], hA_s[2][GB], hdt[2][GB];  // per-head rows, double-buffered over the head loop
   const int tid = threadIdx.x;
@@ -761,68 +761,85 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dcb
         cbr[tm][tn][r] = ok ? CB[(int64_t)l * Q + s] : 0.f;
         live |= (uint32_t)ok << ((tm * 2 + tn) * 4 + r);
       }
-  GemmAcc sum;
+  GemmAcc sum, acc;
   sum.zero();
-  int par = 0;
-  for (int hh = hs; hh < hpg; hh += nsplit, par ^= 1) {
-    const int h = g * hpg + hh;
+  acc.zero();
+  // One pipeline over the heads of this workgroup: k runs over (head, p), a head's product is
+  // finished, weighted and added to the sum at its last k step, and the loads of the next head are
+  // already in flight then.
+  const int nh = (hpg - hs + nsplit - 1) / nsplit;
+  const int seg_k = (P + GK - 1) / GK * GK;
+  auto load_rows = [&](int hl) {  // rows of head hl into buffer hl & 1; published by the next step's barriers
+    const int h = g * hpg + hs + hl * nsplit, par = hl & 1;
     const float *dA = chunk_row(p.dA_cumsum, p, b, h, c);
     const float *dt = chunk_row(p.dt_out, p, b, h, c);
-    // published by the barriers inside the GEMM; the buffer written here was last read two
-    // iterations ago
     if (tid < GB) hA_l[par][tid] = lt * GB + tid < Q ? dA[lt * GB + tid] : 0.f;
     else if (tid < 2 * GB) hA_s[par][tid - GB] = st * GB + tid - GB < Q ? dA[st * GB + tid - GB] : 0.f;
     else if (tid < 3 * GB) hdt[par][tid - 2 * GB] = st * GB + tid - 2 * GB < Q ? dt[st * GB + tid - 2 * GB] : 0.f;
-    const int64_t gb = b * gv.bs + h * gv.hs, xb = b * p.x_bs + h * p.x_hs;
-    GemmAcc acc;
-    acc.zero();
-    // A = g rows (l, k = p), B = x rows (s, k = p): both k-contiguous
-    const T *ga = static_cast<const T *>(gv.ptr) + gb + (int64_t)(t0 + lt * GB) * gv.ls;
-    const T *xa = static_cast<const T *>(p.x) + xb + (int64_t)(t0 + st * GB) * p.x_ls;
-    const bool va = rows_aligned16(ga, gv.ls), vb = rows_aligned16(xa, p.x_ls);
-    block_gemm_pipe<SPLIT>(
-        acc, lds, 0, P,
-        KcStager<SPLIT, T>(lds.ah, lds.al, ga, gv.ls, qlim - lt * GB, P, nullptr, nullptr, va, tid),
-        KcStager<SPLIT, T>(lds.bh, lds.bl, xa, p.x_ls, qlim - st * GB, P, nullptr, nullptr, vb, tid),
-        tid);
-    // d = this head's dCB term (added to sum); w = d * CB, whose row / column sums go to ddA
-    float *dda = chunk_row(p.ddA_cumsum, p, b, h, c);
-    float a_s[2], dt_s[2], csum[2] = {0.f, 0.f};
-#pragma unroll
-    for (int tn = 0; tn < 2; ++tn) {
-      a_s[tn] = hA_s[par][wn * 32 + tn * 16 + i];
-      dt_s[tn] = hdt[par][wn * 32 + tn * 16 + i];
-    }
-#pragma unroll
-    for (int tm = 0; tm < 2; ++tm)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int m = wm * 32 + tm * 16 + gq * 4 + r;
-        const float a_l = hA_l[par][m];
-        float rsum = 0.f;
+  };
+  load_rows(0);
+  // A = g rows (l, k = p), B = x rows (s, k = p): both k-contiguous
+  block_gemm_pipe<SPLIT>(
+      acc, lds, 0, nh * seg_k,
+      seg_stager(KcStager<SPLIT, T>(lds.ah, lds.al, nullptr, gv.ls, qlim - lt * GB, P, nullptr, nullptr, false, tid),
+                 [&](KcStager<SPLIT, T> &q, int hl) {
+                   q.base = static_cast<const T *>(gv.ptr) + b * gv.bs + (g * hpg + hs + hl * nsplit) * gv.hs +
+                            (int64_t)(t0 + lt * GB) * gv.ls;
+                   q.vec = rows_aligned16(q.base, gv.ls);
+                 },
+                 seg_k),
+      seg_stager(KcStager<SPLIT, T>(lds.bh, lds.bl, nullptr, p.x_ls, qlim - st * GB, P, nullptr, nullptr, false, tid),
+                 [&](KcStager<SPLIT, T> &q, int hl) {
+                   q.base = static_cast<const T *>(p.x) + b * p.x_bs + (g * hpg + hs + hl * nsplit) * p.x_hs +
+                            (int64_t)(t0 + st * GB) * p.x_ls;
+                   q.vec = rows_aligned16(q.base, p.x_ls);
+                 },
+                 seg_k),
+      tid, [&](int k0) {
+        const int hl = k0 / seg_k;
+        // the buffer written here was last read one step ago, before this step's barriers
+        if (k0 % seg_k == 0 && hl + 1 < nh) load_rows(hl + 1);
+        if ((k0 + GK) % seg_k != 0) return;
+        const int h = g * hpg + hs + hl * nsplit, par = hl & 1;
+        // d = this head's dCB term (added to sum); w = d * CB, whose row / column sums go to ddA
+        float *dda = chunk_row(p.ddA_cumsum, p, b, h, c);
+        float a_s[2], dt_s[2], csum[2] = {0.f, 0.f};
 #pragma unroll
         for (int tn = 0; tn < 2; ++tn) {
-          float d = acc.v[tm][tn][r] * dt_s[tn] * fast_exp(fminf(a_l - a_s[tn], 0.f));
-          d = (live >> ((tm * 2 + tn) * 4 + r)) & 1 ? d : 0.f;
-          sum.v[tm][tn][r] += d;
-          const float w = d * cbr[tm][tn][r];
-          rsum += w;
-          csum[tn] += w;
+          a_s[tn] = hA_s[par][wn * 32 + tn * 16 + i];
+          dt_s[tn] = hdt[par][wn * 32 + tn * 16 + i];
         }
-        rsum += dpp_f<DPP_ROW_SHR + 1>(0.f, rsum);
-        rsum += dpp_f<DPP_ROW_SHR + 2>(0.f, rsum);
-        rsum += dpp_f<DPP_ROW_SHR + 4>(0.f, rsum);
-        rsum += dpp_f<DPP_ROW_SHR + 8>(0.f, rsum);
-        if (i == 15 && rsum != 0.f) unsafeAtomicAdd(dda + lt * GB + m, rsum);
-      }
 #pragma unroll
-    for (int tn = 0; tn < 2; ++tn) {
-      float cs = csum[tn];
-      cs += __shfl_xor(cs, 16, 64);
-      cs += __shfl_xor(cs, 32, 64);
-      if (gq == 0 && cs != 0.f) unsafeAtomicAdd(dda + st * GB + wn * 32 + tn * 16 + i, -cs);
-    }
-  }
+        for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int m = wm * 32 + tm * 16 + gq * 4 + r;
+            const float a_l = hA_l[par][m];
+            float rsum = 0.f;
+#pragma unroll
+            for (int tn = 0; tn < 2; ++tn) {
+              float d = acc.v[tm][tn][r] * dt_s[tn] * fast_exp(fminf(a_l - a_s[tn], 0.f));
+              d = (live >> ((tm * 2 + tn) * 4 + r)) & 1 ? d : 0.f;
+              acc.v[tm][tn][r] = 0.f;
+              sum.v[tm][tn][r] += d;
+              const float w = d * cbr[tm][tn][r];
+              rsum += w;
+              csum[tn] += w;
+            }
+            rsum += dpp_f<DPP_ROW_SHR + 1>(0.f, rsum);
+            rsum += dpp_f<DPP_ROW_SHR + 2>(0.f, rsum);
+            rsum += dpp_f<DPP_ROW_SHR + 4>(0.f, rsum);
+            rsum += dpp_f<DPP_ROW_SHR + 8>(0.f, rsum);
+            if (i == 15 && rsum != 0.f) unsafeAtomicAdd(dda + lt * GB + m, rsum);
+          }
+#pragma unroll
+        for (int tn = 0; tn < 2; ++tn) {
+          float cs = csum[tn];
+          cs += __shfl_xor(cs, 16, 64);
+          cs += __shfl_xor(cs, 32, 64);
+          if (gq == 0 && cs != 0.f) unsafeAtomicAdd(dda + st * GB + wn * 32 + tn * 16 + i, -cs);
+        }
+      });
   acc_foreach(sum, tid, [&](int m, int n, float v) {
     const int l = lt * GB + m, s = st * GB + n;
     if (l < Q && s < Q && v != 0.f) unsafeAtomicAdd(dCB + (int64_t)l * Q + s, v);  // dCB starts zeroed
