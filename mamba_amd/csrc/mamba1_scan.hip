@@ -248,8 +248,19 @@ __global__ __launch_bounds__(NW * 64, 4) void scan_fwd_kernel(const MambaScanPar
 }
 
 // ----------------------------------------------------------------- backward
+// Row starts of one channel of the workgroup, kept in LDS: every (tile, channel) step needs nine
+// addresses, and as scalars next to the loop state they did not fit the scalar registers (each step
+// then re-read some 250 spilled scalars through v_readlane).
+template <typename T> struct BwdRow {
+  const T *u, *delta, *dout, *z;
+  T *du, *ddelta, *dz, *out_z;
+  const float *ckpt;  // checkpoint of tile 0 of this channel
+  float D, bias;
+};
+
 template <typename T, int NW, int R, bool VEC, int BC>
 __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams p) {
+  static_assert(sizeof(BwdRow<T>) == 80, "the host side sizes the LDS table with 80 bytes per channel");
   extern __shared__ __align__(16) float smem[];
   const int N = p.dstate, L = p.seqlen;
   const int NBLK = (N + NB16 - 1) / NB16, NP = NBLK * NB16;
@@ -267,6 +278,7 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
   float *dbacc = dDacc + WR;          // [WR]
   float *dBcacc = dbacc + WR;         // [WR][NP] gradients of input-independent B / C
   float *dCcacc = dBcacc + WR * NP;
+  BwdRow<T> *rows = reinterpret_cast<BwdRow<T> *>(dCcacc + WR * NP);  // [WR]
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -278,6 +290,22 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
   const int dend = (g + 1) * Dg;
   const int ntiles = (L + TILE - 1) / TILE;
   const bool has_z = p.z != nullptr;
+  if (lane < R) {  // each wave fills and reads only its own rows
+    const int d = min(dbase + lane, dend - 1);
+    BwdRow<T> q;
+    q.u = (const T *)p.u + b * p.u_bs + d * p.u_ds;
+    q.delta = (const T *)p.delta + b * p.delta_bs + d * p.delta_ds;
+    q.dout = (const T *)p.dout + b * p.dout_bs + d * p.dout_ds;
+    q.z = has_z ? (const T *)p.z + b * p.z_bs + d * p.z_ds : nullptr;
+    q.du = (T *)p.du + b * p.du_bs + d * p.du_ds;
+    q.ddelta = (T *)p.ddelta + b * p.ddelta_bs + d * p.ddelta_ds;
+    q.dz = has_z ? (T *)p.dz + b * p.dz_bs + d * p.dz_ds : nullptr;
+    q.out_z = (has_z && p.out_z) ? (T *)p.out_z + b * p.outz_bs + d * p.outz_ds : nullptr;
+    q.ckpt = p.ckpt + ((int64_t)b * p.dim + d) * ntiles * N;
+    q.D = p.D ? ((const float *)p.D)[d] : 0.f;
+    q.bias = p.delta_bias ? ((const float *)p.delta_bias)[d] : 0.f;
+    rows[wave * R + lane] = q;
+  }
 
   const T *Bg = (const T *)p.B + b * p.B_bs + g * p.B_gs;
   const T *Cg = (const T *)p.C + b * p.C_bs + g * p.C_gs;
@@ -311,11 +339,12 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
     k.z.zero();
     k.ck = 0.f;
     if (d < dend) {
-      if (NP <= 64 && tile > 0 && lane < N) k.ck = p.ckpt[(((int64_t)b * p.dim + d) * ntiles + tile - 1) * N + lane];
-      load_items<T, VEC>(k.u, (const T *)p.u + b * p.u_bs + d * p.u_ds, tl, L, nvalid);
-      load_items<T, VEC>(k.delta, (const T *)p.delta + b * p.delta_bs + d * p.delta_ds, tl, L, nvalid);
-      load_items<T, VEC>(k.dout, (const T *)p.dout + b * p.dout_bs + d * p.dout_ds, tl, L, nvalid);
-      if (has_z) load_items<T, VEC>(k.z, (const T *)p.z + b * p.z_bs + d * p.z_ds, tl, L, nvalid);
+      const BwdRow<T> &q = rows[wave * R + r];
+      if (NP <= 64 && tile > 0 && lane < N) k.ck = q.ckpt[(int64_t)(tile - 1) * N + lane];
+      load_items<T, VEC>(k.u, q.u, tl, L, nvalid);
+      load_items<T, VEC>(k.delta, q.delta, tl, L, nvalid);
+      load_items<T, VEC>(k.dout, q.dout, tl, L, nvalid);
+      if (has_z) load_items<T, VEC>(k.z, q.z, tl, L, nvalid);
     }
   };
   Rows nxt;
@@ -336,9 +365,9 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
       else if (tile > 0) fetch_rows(nxt, tile - 1, 0);
       float Dd = 0.f;
       if (valid) {
-        Dd = p.D ? ((const float *)p.D)[d] : 0.f;
+        Dd = rows[row].D;
         const Pack8<T> u_k = cur.u;
-        const float bias = p.delta_bias ? ((const float *)p.delta_bias)[d] : 0.f;
+        const float bias = rows[row].bias;
         u_k.unpack(u);
         draw_k.unpack(dl);
         dout_k.unpack(dy);
@@ -373,7 +402,7 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
         } else {
           for (int n = lane; n < NP; n += 64) {
             float v = 0.f;
-            if (tile > 0 && n < N) v = p.ckpt[(((int64_t)b * p.dim + d) * ntiles + tile - 1) * N + n];
+            if (tile > 0 && n < N) v = rows[row].ckpt[(int64_t)(tile - 1) * N + n];
             hcar[row * NP + n] = v;
           }
         }
@@ -525,11 +554,12 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
       if (valid) {
         float draw[8], o[8];
         draw_k.unpack(draw);
-        const float bias = p.delta_bias ? ((const float *)p.delta_bias)[d] : 0.f;
+        const BwdRow<T> q = rows[row];
+        const float bias = q.bias;
         float dbs = 0.f, dDs = 0.f;
 #pragma unroll
         for (int i = 0; i < KI; ++i) o[i] = __builtin_fmaf(dl[i], acc[i], Dd * dy[i]);
-        st8_guard<T, VEC>((T *)p.du + b * p.du_bs + d * p.du_ds + tl, nvalid, o);
+        st8_guard<T, VEC>(q.du + tl, nvalid, o);
 #pragma unroll
         for (int i = 0; i < KI; ++i) {
           const float x = draw[i] + bias;
@@ -540,7 +570,7 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
           dbs += gd;
           dDs = __builtin_fmaf(dy[i], u[i], dDs);
         }
-        st8_guard<T, VEC>((T *)p.ddelta + b * p.ddelta_bs + d * p.ddelta_ds + tl, nvalid, o);
+        st8_guard<T, VEC>(q.ddelta + tl, nvalid, o);
         if (has_z) {
           float z[8], dout[8], oz[8];
           z_k.unpack(z);
@@ -552,8 +582,8 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
             o[i] = dout[i] * yf * s * (1.f + z[i] * (1.f - s));
             oz[i] = yf * z[i] * s;
           }
-          st8_guard<T, VEC>((T *)p.dz + b * p.dz_bs + d * p.dz_ds + tl, nvalid, o);
-          if (p.out_z) st8_guard<T, VEC>((T *)p.out_z + b * p.outz_bs + d * p.outz_ds + tl, nvalid, oz);
+          st8_guard<T, VEC>(q.dz + tl, nvalid, o);
+          if (q.out_z) st8_guard<T, VEC>(q.out_z + tl, nvalid, oz);
         }
         dbs = wave_sum_to_last(dbs);
         dDs = wave_sum_to_last(dDs);
@@ -590,7 +620,7 @@ struct Cfg {
 
 inline size_t fwd_lds(int nw, int r, int np) { return sizeof(float) * (2 * BC_FLOATS + 2 * nw * r * np); }
 inline size_t bwd_lds(int nw, int r, int np) {
-  return sizeof(float) * (4 * BC_FLOATS + 7 * nw * r * np + 2 * nw * r);
+  return sizeof(float) * (4 * BC_FLOATS + 7 * nw * r * np + 2 * nw * r) + (size_t)nw * r * 80;  // + BwdRow per channel
 }
 
 template <typename KernelT>
