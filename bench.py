@@ -11,6 +11,11 @@ Side workloads (each prints its own JSON line; they are not the headline metric)
   python bench.py --workload ssd      Mamba-2 mamba_chunk_scan_combined fwd+bwd (batch 4, 80 heads x 64,
                                       seqlen 4096, d_state 128, chunk 256, bf16)
   python bench.py --workload decode   selective_state_update (batch 256, 80 heads x 64, d_state 128)
+  python bench.py --workload varlen   the same operator on one packed row of 16 sequences, 32768 positions,
+                                      64 heads, 8 groups, initial and final states (benchmark configuration 4)
+  python bench.py --workload inner    mamba_inner_fn fwd+bwd (conv, projections, scan; d_model 2560)
+  python bench.py --workload block    mamba_split_conv1d_scan_combined fwd+bwd (conv, SSD scan, gated norm,
+                                      out_proj; d_model 2560)
   python bench.py --copy-calibration  the library's plain copy kernel over 1 GiB
 """
 import argparse
@@ -201,13 +206,172 @@ def bench_decode(dev, steps, warmup):
                      "kernel_ms": ms, "algorithmic_bytes": nbytes}}))
 
 
+def _timed(step, steps, warmup):
+    import torch
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def bench_varlen(dev, steps, warmup):
+    """Configuration 4: one packed row of 16 sequences (lengths uniform in [512, 4096], rescaled to sum to
+    32768), seq_idx, nonzero initial states, final states returned; forward + backward."""
+    import torch
+    from mamba_amd.ops.triton import ssd_combined as sc
+    batch, L, H, P, N, G, Q, nseq = 1, 32768, 64, 64, 128, 8, 256, 16
+    bf = torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(0)
+    rn = lambda *s: torch.randn(*s, device=dev, generator=g)
+    x, z = (rn(batch, L, H, P).to(bf).requires_grad_() for _ in range(2))
+    B, C = (rn(batch, L, G, N).to(bf).requires_grad_() for _ in range(2))
+    dt = rn(batch, L, H).to(bf).requires_grad_()
+    A = (-(1 + 15 * torch.rand(H, device=dev, generator=g))).requires_grad_()
+    D = torch.rand(H, device=dev, generator=g).requires_grad_()
+    dtb = (torch.rand(H, device=dev, generator=g) - 4).requires_grad_()
+    init = (0.1 * rn(batch, H, P, N)).requires_grad_()
+    dout = rn(batch, L, H, P).to(bf)
+    lens = torch.randint(512, 4097, (nseq,), generator=torch.Generator().manual_seed(0)).double()
+    lens = (lens / lens.sum() * L).long()
+    lens[-1] += L - lens.sum()
+    seq_idx = torch.cat([torch.full((int(n),), i, dtype=torch.int32) for i, n in enumerate(lens)])[None].to(dev)
+    leaves = (x, z, B, C, dt, A, D, dtb, init)
+
+    def fwd():
+        return sc.mamba_chunk_scan_combined(x, dt, A, B, C, Q, D=D, z=z, dt_bias=dtb, initial_states=init,
+                                            seq_idx=seq_idx, dt_softplus=True, return_final_states=True)
+
+    def step():
+        for v in leaves:
+            v.grad = None
+        fwd()[0].backward(dout)
+
+    sec = _timed(step, steps, warmup)
+    with torch.no_grad():
+        fwd_ms = event_ms(fwd, max(5, min(steps, 50)))
+    nbytes = 2 * (5 * batch * L * H * P + 4 * batch * L * G * N)   # x z dout in, dx dz out, B C in, dB dC out (bf16)
+    print(json.dumps({
+        "metric": "SSD mamba_chunk_scan_combined packed varlen fwd+bwd tokens/s at 1 GPU", "value": batch * L / sec,
+        "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": sec * 1e3,
+        "fwd_ms": fwd_ms, "higher_is_better": True, "dtype": "bf16 in/out, fp32 accumulation", "data": "synthetic",
+        "config": {"workload": f"Mamba-2 SSD fwd+bwd, packed: 1 row of {nseq} sequences, {L} positions, {H} heads x {P}, "
+                               f"d_state {N}, {G} groups, chunk {Q}, initial + final states (benchmark configuration 4)"},
+        "roofline": {"bound": "hbm", "kernel": "whole step", "achieved": nbytes / sec / 1e9, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": nbytes / sec / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes": nbytes}}))
+
+
+def bench_inner(dev, steps, warmup):
+    """mamba_inner_fn forward + backward: conv1d + SiLU, x_proj, dt_proj, selective scan, out_proj."""
+    import torch
+    from mamba_amd.ops.selective_scan_interface import mamba_inner_fn
+    from mamba_amd.ops.causal_conv1d import causal_conv1d_fwd
+    batch, L, dm, di, N, W = 8, 4096, 2560, 5120, 16, 4
+    R = math.ceil(dm / 16)
+    bf = torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(0)
+    rn = lambda *s: torch.randn(*s, device=dev, generator=g)
+    xz = rn(batch, 2 * di, L).to(bf).requires_grad_()
+    conv_w = (0.3 * rn(di, 1, W)).to(bf).requires_grad_()
+    conv_b = (0.1 * rn(di)).to(bf).requires_grad_()
+    x_proj = (rn(R + 2 * N, di) / math.sqrt(di)).to(bf).requires_grad_()
+    dt_proj = (rn(di, R) / math.sqrt(R)).to(bf).requires_grad_()
+    out_proj = (rn(dm, di) / math.sqrt(di)).to(bf).requires_grad_()
+    A = (-torch.arange(1, N + 1, device=dev, dtype=torch.float32)[None].repeat(di, 1)).requires_grad_()
+    D = torch.ones(di, device=dev).requires_grad_()
+    dtb = (torch.rand(di, device=dev, generator=g) - 4).requires_grad_()
+    dout = rn(batch, L, dm).to(bf)
+    leaves = (xz, conv_w, conv_b, x_proj, dt_proj, out_proj, A, D, dtb)
+
+    def fwd():
+        return mamba_inner_fn(xz, conv_w, conv_b, x_proj, dt_proj, out_proj, None, A, None, None, D,
+                              delta_bias=dtb, delta_softplus=True)
+
+    def step():
+        for v in leaves:
+            v.grad = None
+        fwd().backward(dout)
+
+    sec = _timed(step, steps, warmup)
+    with torch.no_grad():
+        fwd_ms = event_ms(fwd, max(5, min(steps, 50)))
+        xin = xz[:, :di]
+        cw = conv_w.squeeze(1)
+        conv_ms = event_ms(lambda: causal_conv1d_fwd(xin, cw, conv_b, activation="silu"), max(5, min(steps, 50)))
+    nbytes = 2 * 2 * batch * di * L   # the convolution reads x and writes its output once
+    print(json.dumps({
+        "metric": "mamba_inner_fn fwd+bwd tokens/s at 1 GPU", "value": batch * L / sec, "unit": "tokens/s",
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": sec * 1e3, "fwd_ms": fwd_ms,
+        "higher_is_better": True, "dtype": "bf16 in/out, fp32 state and accumulation", "data": "synthetic",
+        "config": {"workload": f"mamba_inner_fn fwd+bwd: batch {batch}, seqlen {L}, d_model {dm}, d_inner {di}, "
+                               f"d_state {N}, dt_rank {R}, conv width {W}"},
+        "roofline": {"bound": "hbm", "kernel": "conv_rows_fwd_kernel", "achieved": nbytes / conv_ms / 1e6,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / conv_ms / 1e6 / HBM_PEAK_GBS,
+                     "traffic": None, "kernel_ms": conv_ms, "algorithmic_bytes": nbytes}}))
+
+
+def bench_block(dev, steps, warmup):
+    """mamba_split_conv1d_scan_combined forward + backward: the Mamba-2 block body after in_proj."""
+    import torch
+    from mamba_amd.ops.triton.ssd_combined import mamba_split_conv1d_scan_combined
+    from mamba_amd.ops.triton.layernorm_gated import _layer_norm_fwd
+    batch, L, H, P, N, G, Q, W = 4, 4096, 80, 64, 128, 1, 256, 4
+    dim = H * P
+    dm = dim // 2
+    width = 2 * dim + 2 * G * N + H
+    bf = torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(0)
+    rn = lambda *s: torch.randn(*s, device=dev, generator=g)
+    zxbcdt = (0.5 * rn(batch, L, width)).to(bf).requires_grad_()
+    conv_w = (0.3 * rn(dim + 2 * G * N, W)).requires_grad_()
+    conv_b = (0.1 * rn(dim + 2 * G * N)).requires_grad_()
+    dtb = (torch.rand(H, device=dev, generator=g) - 4).requires_grad_()
+    A = (-(1 + 15 * torch.rand(H, device=dev, generator=g))).requires_grad_()
+    D = torch.rand(H, device=dev, generator=g).requires_grad_()
+    norm_w = torch.ones(dim, device=dev).requires_grad_()
+    out_w = (rn(dm, dim) / math.sqrt(dim)).to(bf).requires_grad_()
+    dout = rn(batch, L, dm).to(bf)
+    leaves = (zxbcdt, conv_w, conv_b, dtb, A, D, norm_w, out_w)
+
+    def fwd():
+        return mamba_split_conv1d_scan_combined(zxbcdt, conv_w, conv_b, dtb, A, D, Q, rmsnorm_weight=norm_w,
+                                                outproj_weight=out_w, headdim=P, ngroups=G, norm_before_gate=False)
+
+    def step():
+        for v in leaves:
+            v.grad = None
+        fwd().backward(dout)
+
+    sec = _timed(step, steps, warmup)
+    with torch.no_grad():
+        fwd_ms = event_ms(fwd, max(5, min(steps, 50)))
+        y = rn(batch * L, dim).to(bf)
+        zz = rn(batch * L, dim).to(bf)
+        norm_ms = event_ms(lambda: _layer_norm_fwd(y, norm_w, None, 1e-6, z=zz, group_size=dim // G,
+                                                   norm_before_gate=False, is_rms_norm=True), max(5, min(steps, 50)))
+    nbytes = 3 * 2 * batch * L * dim   # the gated norm reads y and z and writes its output once
+    print(json.dumps({
+        "metric": "mamba_split_conv1d_scan_combined fwd+bwd tokens/s at 1 GPU", "value": batch * L / sec,
+        "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": sec * 1e3, "fwd_ms": fwd_ms,
+        "higher_is_better": True, "dtype": "bf16 in/out, fp32 accumulation", "data": "synthetic",
+        "config": {"workload": f"Mamba-2 block body fwd+bwd: batch {batch}, seqlen {L}, {H} heads x {P}, d_state {N}, "
+                               f"{G} group, chunk {Q}, conv width {W}, gated RMSNorm, out_proj to {dm}"},
+        "roofline": {"bound": "hbm", "kernel": "norm_fwd_kernel", "achieved": nbytes / norm_ms / 1e6,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / norm_ms / 1e6 / HBM_PEAK_GBS,
+                     "traffic": None, "kernel_ms": norm_ms, "algorithmic_bytes": nbytes}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--workload", choices=("mamba1", "ssd", "decode"), default="mamba1")
+    ap.add_argument("--workload", choices=("mamba1", "ssd", "decode", "varlen", "inner", "block"), default="mamba1")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run the library's plain copy kernel over 1 GiB (yardstick for HBM counters)")
     args = ap.parse_args()
@@ -232,6 +396,9 @@ def main():
         return
     if args.workload == "decode":
         bench_decode(dev, args.steps, args.warmup)
+        return
+    if args.workload in ("varlen", "inner", "block"):
+        {"varlen": bench_varlen, "inner": bench_inner, "block": bench_block}[args.workload](dev, args.steps, args.warmup)
         return
     batch, dim, seqlen, dstate = 8, 5120, 4096, 16
     dtype = torch.bfloat16

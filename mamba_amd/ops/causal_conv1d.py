@@ -52,15 +52,19 @@ def _check(x, weight, bias, seq_idx, activation):
         raise RuntimeError("causal_conv1d: seq_idx must be (batch, seqlen) int32")
 
 
-def causal_conv1d_fwd(x, weight, bias=None, seq_idx=None, activation=None):
-    """One call of the C ABI's causal_conv1d_fwd; out is dense in x's layout."""
+def causal_conv1d_fwd(x, weight, bias=None, seq_idx=None, activation=None, out=None):
+    """One call of the C ABI's causal_conv1d_fwd; out is dense in x's layout unless the caller brings
+    one (same shape and dtype, unit stride on the axis where x has it)."""
     _check(x, weight, bias, seq_idx, activation)
     if not _usable(x):
         x = x.contiguous()
     seq_idx = seq_idx.contiguous() if seq_idx is not None else None
     w32 = weight.detach().float().contiguous()
     b32 = bias.detach().float().contiguous() if bias is not None else None
-    out = _like_layout(x)
+    if out is None:
+        out = _like_layout(x)
+    elif out.shape != x.shape or out.dtype != x.dtype or out.stride(2 if x.stride(2) == 1 else 1) != 1:
+        raise RuntimeError("causal_conv1d: out must match x in shape, dtype and layout")
     p = _lib.CausalConvParams()
     _fill(p, x, w32, b32, seq_idx, activation)
     p.out = out.data_ptr()

@@ -331,6 +331,22 @@ def _norm_over_state(t, weight, eps, L):
     return rearrange(_rms_norm(rows, weight, eps), "(b l) dstate -> b 1 dstate l", l=L).contiguous()
 
 
+def _channel_major(x):
+    """An empty (batch, dim, seqlen) tensor like x whose memory order is (dim, batch, seqlen)."""
+    b, d, L = x.shape
+    return torch.empty(d, b, L, dtype=x.dtype, device=x.device).permute(1, 0, 2)
+
+
+def _as_matrix(t):
+    """(batch, dim, seqlen) -> (dim, batch * seqlen): a view when t is channel-major, else a copy."""
+    return t.permute(1, 0, 2).reshape(t.shape[1], -1)
+
+
+def _from_matrix(m, L):
+    """(dim, batch * seqlen) -> the (batch, dim, seqlen) view of the same memory."""
+    return m.view(m.shape[0], -1, L).permute(1, 0, 2)
+
+
 class MambaInnerFn(torch.autograd.Function):
     """conv1d+SiLU -> x_proj -> dt_proj -> selective scan -> out_proj with the reference's layout
     choreography and recompute-in-backward (selective_scan_interface.py:196-383).  The scan runs on
@@ -360,10 +376,12 @@ class MambaInnerFn(torch.autograd.Function):
         conv1d_weight = rearrange(conv1d_weight, "d 1 w -> d w")
         x, z = xz.chunk(2, dim=1)
         conv1d_bias = conv1d_bias.contiguous() if conv1d_bias is not None else None
-        conv1d_out = causal_conv1d_fwd(x, conv1d_weight, conv1d_bias, activation="silu")
-        # delta keeps d as the slow and L as the fast dimension: what the scan kernel reads
-        x_dbl = F.linear(rearrange(conv1d_out, "b d l -> (b l) d"), x_proj_weight)
-        delta = rearrange(delta_proj_weight @ x_dbl[:, :delta_rank].t(), "d (b l) -> b d l", l=L)
+        # Every (batch, dim, seqlen) intermediate lives in memory as (dim, batch, seqlen): the kernels take
+        # batch and channel strides as they come, and the projections then see (dim, batch * seqlen)
+        # matrices and their transposes without a copy.
+        conv1d_out = causal_conv1d_fwd(x, conv1d_weight, conv1d_bias, activation="silu", out=_channel_major(x))
+        x_dbl = F.linear(_as_matrix(conv1d_out).t(), x_proj_weight)        # (b l) x (rank + 2 n)
+        delta = _from_matrix(delta_proj_weight @ x_dbl[:, :delta_rank].t(), L)
         ctx.is_variable_B, ctx.is_variable_C = B is None, C is None
         ctx.B_proj_bias_is_None, ctx.C_proj_bias_is_None = B_proj_bias is None, C_proj_bias is None
         if B is None:
@@ -389,8 +407,7 @@ class MambaInnerFn(torch.autograd.Function):
         if dt_rms_weight is not None:
             delta = rearrange(_rms_norm(rearrange(delta, "b d l -> (b l) d").contiguous(), dt_rms_weight,
                                         b_c_dt_rms_eps), "(b l) d -> b d l", l=L).contiguous()
-        out_z, ckpt = selective_scan_fwd(conv1d_out.contiguous(), delta.contiguous(), A, B, C, D, z, delta_bias,
-                                         delta_softplus)
+        out_z, ckpt = selective_scan_fwd(conv1d_out, delta, A, B, C, D, z, delta_bias, delta_softplus)
         ctx.delta_softplus = delta_softplus
         ctx.out_proj_bias_is_None = out_proj_bias is None
         ctx.checkpoint_lvl = checkpoint_lvl
@@ -399,7 +416,8 @@ class MambaInnerFn(torch.autograd.Function):
             conv1d_out, delta = None, None
         ctx.save_for_backward(xz, conv1d_weight, conv1d_bias, x_dbl, x_proj_weight, delta_proj_weight,
                               out_proj_weight, conv1d_out, delta, A, B, C, D, delta_bias, ckpt)
-        return F.linear(rearrange(out_z, "b d l -> b l d"), out_proj_weight, out_proj_bias)
+        out = F.linear(_as_matrix(out_z).t(), out_proj_weight, out_proj_bias)   # out_z has delta's layout
+        return out.view(xz.shape[0], L, -1)
 
     @staticmethod
     @torch.amp.custom_bwd(device_type="cuda")
@@ -416,19 +434,19 @@ class MambaInnerFn(torch.autograd.Function):
         if dout.stride(-1) != 1:
             dout = dout.contiguous()
         if ctx.checkpoint_lvl == 1:  # the convolution output and delta are re-computed
-            conv1d_out = causal_conv1d_fwd(x, conv1d_weight, conv1d_bias, activation="silu")
-            delta = rearrange(delta_proj_weight @ x_dbl[:, :delta_rank].t(), "d (b l) -> b d l", l=L)
+            conv1d_out = causal_conv1d_fwd(x, conv1d_weight, conv1d_bias, activation="silu", out=_channel_major(x))
+            delta = _from_matrix(delta_proj_weight @ x_dbl[:, :delta_rank].t(), L)
             if ctx.dt_rms_weight is not None:
                 delta = rearrange(_rms_norm(rearrange(delta, "b d l -> (b l) d").contiguous(), ctx.dt_rms_weight,
                                             ctx.rms_eps), "(b l) d -> b d l", l=L).contiguous()
         dxz = torch.empty_like(xz)
         dx, dz = dxz.chunk(2, dim=1)
-        dout = rearrange(dout, "b l e -> e (b l)")
-        dout_y = rearrange(out_proj_weight.t() @ dout, "d (b l) -> b d l", l=L)
+        dout = dout.reshape(-1, dout.shape[-1]).t()                                  # e x (b l)
+        dout_y = _from_matrix(out_proj_weight.t() @ dout, L)
+        # du, ddelta and out_z come back in the layouts of u and delta
         dconv1d_out, ddelta, dA, dB, dC, dD, ddelta_bias, dz, out_z = selective_scan_bwd(
-            conv1d_out.contiguous(), delta.contiguous(), A, B, C, D, z, delta_bias, dout_y.contiguous(), ckpt, dz,
-            ctx.delta_softplus, True)
-        dout_proj_weight = torch.einsum("eB,dB->ed", dout, rearrange(out_z, "b d l -> d (b l)"))
+            conv1d_out, delta, A, B, C, D, z, delta_bias, dout_y, ckpt, dz, ctx.delta_softplus, True)
+        dout_proj_weight = dout @ _as_matrix(out_z).t()
         dout_proj_bias = dout.sum(dim=1) if not ctx.out_proj_bias_is_None else None
         dx_dbl = torch.empty_like(x_dbl)
         dB_proj_bias = dC_proj_bias = None
@@ -442,13 +460,12 @@ class MambaInnerFn(torch.autograd.Function):
             dC_proj_bias = dC.sum(0) if not ctx.C_proj_bias_is_None else None
             dx_dbl[:, -d_state:] = dC
             dC = None
-        ddelta = rearrange(ddelta, "b d l -> d (b l)")
-        ddelta_proj_weight = torch.einsum("dB,Br->dr", ddelta, x_dbl[:, :delta_rank])
-        dx_dbl[:, :delta_rank] = torch.einsum("dB,dr->Br", ddelta, delta_proj_weight)
-        dconv1d_out = rearrange(dconv1d_out, "b d l -> d (b l)")
-        dx_proj_weight = torch.einsum("Br,Bd->rd", dx_dbl, rearrange(conv1d_out, "b d l -> (b l) d"))
-        dconv1d_out = torch.addmm(dconv1d_out, x_proj_weight.t(), dx_dbl.t())
-        dconv1d_out = rearrange(dconv1d_out, "d (b l) -> b d l", b=x.shape[0], l=L)
+        ddelta = _as_matrix(ddelta)
+        ddelta_proj_weight = ddelta @ x_dbl[:, :delta_rank]
+        dx_dbl[:, :delta_rank] = ddelta.t() @ delta_proj_weight
+        dx_proj_weight = dx_dbl.t() @ _as_matrix(conv1d_out).t()
+        dconv1d_mat = _as_matrix(dconv1d_out)            # the scan's own du buffer: add the x_proj path in place
+        dconv1d_out = _from_matrix(dconv1d_mat.addmm_(x_proj_weight.t(), dx_dbl.t()), L)
         # the convolution's backward kernel re-computes the pre-activation from x and writes dx in place
         _, dconv1d_weight, dconv1d_bias = causal_conv1d_bwd(x, conv1d_weight, conv1d_bias, dconv1d_out.to(x.dtype),
                                                             activation="silu", dx=dx)
