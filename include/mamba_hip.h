@@ -213,7 +213,7 @@ typedef struct SsdParams {
   /* ---- backward only ---- */
   const void *dout;
   const float *dfinal_states;           /* nullable, (b, H, P, N) */
-  void *dx, *dz;                        /* `dtype`, contiguous (b, L, H, P) */
+  void *dx, *dz;                        /* `dtype`, (b, L, H, P): dz contiguous, dx with the strides below */
   void *ddt;                            /* `dt_dtype`, contiguous (b, L, H) */
   void *dB, *dC;                        /* `dtype`, contiguous (b, L, G, N) */
   float *dA, *ddt_bias;                 /* (H) fp32, zero on entry */
@@ -227,6 +227,7 @@ typedef struct SsdParams {
   float *dB32, *dC32;                   /* (b, L, G, N), zero on entry */
   void *gbuf;                           /* (b, L, H, P) of `dtype`: dout * silu(z); used iff z != NULL */
   int64_t dout_bs, dout_ls, dout_hs;
+  int64_t dx_bs, dx_ls, dx_hs;          /* dx may be a slice of a wider buffer; unit headdim stride */
 } SsdParams;
 
 /* forward stages, in launch order */

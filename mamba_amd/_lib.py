@@ -53,7 +53,7 @@ class SsdParams(ctypes.Structure):
                                 "B_bs", "B_ls", "B_gs", "C_bs", "C_ls", "C_gs", "dt_bs", "dt_ls", "dt_hs")]
         + [(n, c_vp) for n in ("dout", "dfinal_states", "dx", "dz", "ddt", "dB", "dC", "dA", "ddt_bias", "dD",
                                "dinitial_states", "dstates", "ddA_cumsum", "ddt_out", "dCB", "dB32", "dC32", "gbuf")]
-        + [(n, c_i64) for n in ("dout_bs", "dout_ls", "dout_hs")]
+        + [(n, c_i64) for n in ("dout_bs", "dout_ls", "dout_hs", "dx_bs", "dx_ls", "dx_hs")]
     )
 
 

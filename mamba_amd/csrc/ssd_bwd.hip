@@ -448,7 +448,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
   const T *gr = static_cast<const T *>(gv.ptr) + gb + (int64_t)(t0 + s) * gv.ls + p0;
   const bool vec = P % 8 == 0 && rows_aligned16(static_cast<const T *>(p.x) + xb, p.x_ls) &&
                    rows_aligned16(static_cast<const T *>(gv.ptr) + gb, gv.ls) &&
-                   (reinterpret_cast<uintptr_t>(p.dx) & 15) == 0;
+                   rows_aligned16(static_cast<T *>(p.dx) + b * p.dx_bs + h * p.dx_hs, p.dx_ls);
   const float *Dp = static_cast<const float *>(p.D);
   Pack8<T> xk[2], gk[2];
   if (vec) {
@@ -469,7 +469,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
 #pragma unroll
     for (int e = 0; e < 16; ++e) v1[e] *= w;
   }
-  T *dxr = static_cast<T *>(p.dx) + (((int64_t)b * L + t0 + s) * H + h) * P + p0;
+  T *dxr = static_cast<T *>(p.dx) + b * p.dx_bs + (int64_t)(t0 + s) * p.dx_ls + h * p.dx_hs + p0;
   float q1 = 0.f, q2 = 0.f;
   const float dts = dt_s[min(s, Q - 1)];
 #pragma unroll
@@ -1060,6 +1060,7 @@ extern "C" int ssd_state_passing_bwd(const SsdParams *p, mamba_stream_t stream) 
 extern "C" int ssd_bwd_dx(const SsdParams *p, mamba_stream_t stream) {
   int rc = check_bwd(p);
   if (rc) return rc;
+  if (p->dx_ls < (int64_t)p->headdim || p->dx_hs < (int64_t)p->headdim) return MAMBA_E_BADARG;  // strides not filled in
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid(tiles(p->chunk_size) * tiles(p->headdim), p->nchunks, p->batch * p->nheads);
   SSD_DISPATCH(bwd_dx_kernel, grid)

@@ -143,10 +143,12 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
 
 def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None, z=None, dt_bias=None,
                                    initial_states=None, dfinal_states=None, seq_idx=None, dt_softplus=False,
-                                   dt_limit=(0.0, float("inf")), saved=None):
+                                   dt_limit=(0.0, float("inf")), saved=None, dx=None, ddt=None, dB=None, dC=None):
     """Counterpart of ssd_combined.py:397.  `out` is the saved pre-gate output (out_x) when z is given,
     else the forward output.  `saved` = (dt_out, dA_cumsum, states) of the forward pass skips their
-    re-computation (the reference always re-computes them, ssd_combined.py:441-448).
+    re-computation (the reference always re-computes them, ssd_combined.py:441-448).  dx, ddt, dB, dC may
+    be caller-owned views (slices of a wider gradient buffer, unit stride in the last dimension), as the
+    reference's fused block function passes them (ssd_combined.py:934-944).
     Returns (dx, ddt, dA, dB, dC, dD, dz, ddt_bias, dinitial_states)."""
     in_dtypes = (A.dtype, D.dtype if D is not None else None, dt_bias.dtype if dt_bias is not None else None,
                  initial_states.dtype if initial_states is not None else None, B.dtype, C.dtype)
@@ -166,9 +168,13 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
     ws = _workspace(x, B, chunk_size, forward_state=saved)
     nchunks = ws["nchunks"]
     f32 = dict(device=dev, dtype=torch.float32)
-    dx = torch.empty(batch, seqlen, nheads, headdim, device=dev, dtype=x.dtype)
-    dz = torch.empty_like(dx) if z is not None else None
-    gbuf = torch.empty_like(dx) if z is not None else None
+    if dx is None:
+        dx = torch.empty(batch, seqlen, nheads, headdim, device=dev, dtype=x.dtype)
+    else:
+        assert dx.shape == x.shape and dx.dtype == x.dtype and dx.stride(-1) == 1 and dx.is_cuda
+    dz = torch.empty(batch, seqlen, nheads, headdim, device=dev, dtype=x.dtype) if z is not None else None
+    gbuf = torch.empty_like(dz) if z is not None else None
+    ddt_out_view = ddt
     ddt = torch.empty(batch, seqlen, nheads, device=dev, dtype=dt.dtype)
     # one zeroed arena for every accumulator the kernels add into
     sizes = dict(dA=nheads, ddt_bias=nheads, dD=(D.numel() if D is not None else 0),
@@ -194,6 +200,7 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
     p.dout, p.dfinal_states = dout.data_ptr(), _lib.ptr(dfinal)
     p.dout_bs, p.dout_ls, p.dout_hs = dout.stride(0), dout.stride(1), dout.stride(2)
     p.dx, p.dz, p.ddt, p.gbuf = dx.data_ptr(), _lib.ptr(dz), ddt.data_ptr(), _lib.ptr(gbuf)
+    p.dx_bs, p.dx_ls, p.dx_hs = dx.stride(0), dx.stride(1), dx.stride(2)
     p.dA, p.ddt_bias = acc["dA"].data_ptr(), acc["ddt_bias"].data_ptr()
     p.dD = acc["dD"].data_ptr() if D is not None else None
     p.dinitial_states, p.dstates = _lib.ptr(dinit), dstates.data_ptr()
@@ -213,8 +220,12 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
     dD = acc["dD"].view(D_shape).to(in_dtypes[1]) if D is not None else None
     ddt_bias = acc["ddt_bias"].to(in_dtypes[2]) if dt_bias is not None else None
     dinit_out = dinit.to(in_dtypes[3]) if dinit is not None else None
-    dB = acc["dB32"].view(batch, seqlen, ngroups, dstate).to(in_dtypes[4])
-    dC = acc["dC32"].view(batch, seqlen, ngroups, dstate).to(in_dtypes[5])
+    dB32 = acc["dB32"].view(batch, seqlen, ngroups, dstate)
+    dC32 = acc["dC32"].view(batch, seqlen, ngroups, dstate)
+    dB = dB32.to(in_dtypes[4]) if dB is None else dB.copy_(dB32)     # the copy is the cast
+    dC = dC32.to(in_dtypes[5]) if dC is None else dC.copy_(dC32)
+    if ddt_out_view is not None:
+        ddt = ddt_out_view.copy_(ddt)
     return dx, ddt, dA, dB, dC, dD, dz, ddt_bias, dinit_out
 
 
@@ -403,68 +414,163 @@ def _gated_rms_norm(x, weight, z, eps, group_size, norm_before_gate):
     return out.to(dtype)
 
 
+class MambaSplitConv1dScanCombinedFn(torch.autograd.Function):
+    """The Mamba-2 block body as one autograd node (ssd_combined.py:822): the backward pass writes the
+    gradients of z, xBC and dt straight into their slices of one dzxbcdt buffer (norm, convolution and
+    scan kernels take the slices' strides), and the scan writes dx into its slice of the buffer the
+    convolution's backward pass reads, so no concatenation is left."""
+
+    @staticmethod
+    def forward(ctx, zxbcdt, conv1d_weight, conv1d_bias, dt_bias, A, D, chunk_size, initial_states=None, seq_idx=None,
+                dt_limit=(0.0, float("inf")), return_final_states=False, activation="silu", rmsnorm_weight=None,
+                rmsnorm_eps=1e-6, outproj_weight=None, outproj_bias=None, headdim=None, ngroups=1,
+                norm_before_gate=True, state_dtype=None):
+        import torch.nn.functional as F
+        from mamba_amd.ops.causal_conv1d import causal_conv1d_fwd
+        from mamba_amd.ops.triton.layernorm_gated import _layer_norm_fwd
+        assert activation in [None, "silu", "swish"]
+        if D.dim() == 1:
+            assert headdim is not None
+            nheads, = D.shape
+        else:
+            nheads, headdim = D.shape
+        batch, seqlen, _ = zxbcdt.shape
+        dim = nheads * headdim
+        assert nheads % ngroups == 0
+        dstate = (conv1d_weight.shape[0] - dim) // ngroups // 2
+        d_nonssm = (zxbcdt.shape[-1] - 2 * dim - 2 * ngroups * dstate - nheads) // 2
+        assert d_nonssm >= 0
+        assert zxbcdt.shape == (batch, seqlen, 2 * d_nonssm + 2 * dim + 2 * ngroups * dstate + nheads)
+        assert dt_bias.shape == (nheads,) and A.shape == (nheads,)
+        ctx.conv_w_3d = conv1d_weight.dim() == 3
+        conv_w = conv1d_weight.squeeze(1) if ctx.conv_w_3d else conv1d_weight
+        if zxbcdt.stride(-1) != 1:
+            zxbcdt = zxbcdt.contiguous()
+        zx0, z, xBC, dt = torch.split(zxbcdt, [2 * d_nonssm, dim, dim + 2 * ngroups * dstate, nheads], dim=-1)
+        # the convolution reads the channel-contiguous slice as it lies and returns a dense (b, l, c) tensor
+        xBC_conv = causal_conv1d_fwd(xBC.transpose(1, 2), conv_w, conv1d_bias, seq_idx=seq_idx,
+                                     activation=activation).transpose(1, 2)
+        x, B, C = torch.split(xBC_conv, [dim, ngroups * dstate, ngroups * dstate], dim=-1)
+        x = x.reshape(batch, seqlen, nheads, headdim)
+        B = B.reshape(batch, seqlen, ngroups, dstate)
+        C = C.reshape(batch, seqlen, ngroups, dstate)
+        z4 = z.reshape(batch, seqlen, nheads, headdim)
+        gate_in_scan = rmsnorm_weight is None
+        out, out_x, dt_out, dA_cumsum, states, final_states = _mamba_chunk_scan_combined_fwd(
+            x, dt, A, B, C, chunk_size, D=D, z=z4 if gate_in_scan else None, dt_bias=dt_bias,
+            initial_states=initial_states, seq_idx=seq_idx, dt_softplus=True, dt_limit=dt_limit, state_dtype=state_dtype)
+        y = out.view(batch, seqlen, dim)
+        rstd = None
+        if not gate_in_scan:
+            # reads z where it lies inside zxbcdt (unit channel stride, row stride of the whole projection)
+            y, _, rstd = _layer_norm_fwd(out.view(batch * seqlen, dim), rmsnorm_weight, None, rmsnorm_eps,
+                                         z=z.reshape(batch * seqlen, dim), group_size=dim // ngroups,
+                                         norm_before_gate=norm_before_gate, is_rms_norm=True)
+            y = y.view(batch, seqlen, dim)
+        if d_nonssm > 0:
+            gate, up = zx0.chunk(2, dim=-1)
+            y = torch.cat([(F.silu(gate.float()) * up.float()).to(y.dtype), y], dim=-1)
+        ctx.autocast = None
+        if outproj_weight is not None:
+            w, bias = outproj_weight, outproj_bias
+            if torch.is_autocast_enabled():
+                ctx.autocast = torch.get_autocast_gpu_dtype()
+                y, w = y.to(ctx.autocast), w.to(ctx.autocast)
+                bias = bias.to(ctx.autocast) if bias is not None else None
+            res = F.linear(y, w, bias)
+        else:
+            assert outproj_bias is None
+            res = y
+        # the scan's backward pass wants its pre-gate output: out_x when the gate ran inside the scan
+        ctx.save_for_backward(zxbcdt, conv_w, conv1d_bias, xBC_conv, out_x if gate_in_scan else out,
+                              dt_out, dA_cumsum, states, A, D, dt_bias, initial_states, seq_idx, rmsnorm_weight, rstd,
+                              outproj_weight, outproj_bias, y if outproj_weight is not None else None)
+        ctx.dims = (batch, seqlen, nheads, headdim, ngroups, dstate, d_nonssm)
+        ctx.chunk_size, ctx.dt_limit, ctx.activation = chunk_size, dt_limit, activation
+        ctx.rmsnorm_eps, ctx.norm_before_gate = rmsnorm_eps, norm_before_gate
+        ctx.return_final_states = return_final_states
+        return res if not return_final_states else (res, final_states)
+
+    @staticmethod
+    def backward(ctx, dout, *args):
+        import torch.nn.functional as F
+        from mamba_amd.ops.causal_conv1d import causal_conv1d_bwd
+        from mamba_amd.ops.triton.layernorm_gated import _layer_norm_bwd
+        (zxbcdt, conv_w, conv_b, xBC_conv, scan_out, dt_out, dA_cumsum, states, A, D, dt_bias, initial_states, seq_idx,
+         rmsnorm_weight, rstd, outproj_weight, outproj_bias, y_proj) = ctx.saved_tensors
+        batch, seqlen, nheads, headdim, ngroups, dstate, d_nonssm = ctx.dims
+        dim = nheads * headdim
+        dfinal_states = args[0] if ctx.return_final_states else None
+        gate_in_scan = rmsnorm_weight is None
+        zx0, z, xBC, dt = torch.split(zxbcdt, [2 * d_nonssm, dim, dim + 2 * ngroups * dstate, nheads], dim=-1)
+        dzxbcdt = torch.empty_like(zxbcdt)
+        dzx0, dz, dxBC, ddt = torch.split(dzxbcdt, [2 * d_nonssm, dim, dim + 2 * ngroups * dstate, nheads], dim=-1)
+        doutproj_weight = doutproj_bias = None
+        if outproj_weight is not None:
+            w = outproj_weight if ctx.autocast is None else outproj_weight.to(ctx.autocast)
+            dout2 = dout.reshape(-1, dout.shape[-1]).to(w.dtype)
+            dy_cat = (dout2 @ w).view(batch, seqlen, d_nonssm + dim)
+            doutproj_weight = (dout2.t() @ y_proj.reshape(-1, d_nonssm + dim)).to(outproj_weight.dtype)
+            doutproj_bias = dout2.sum(0).to(outproj_bias.dtype) if outproj_bias is not None else None
+        else:
+            dy_cat = dout
+        if dy_cat.stride(-1) != 1:
+            dy_cat = dy_cat.contiguous()
+        dy_cat = dy_cat.to(zxbcdt.dtype)
+        if d_nonssm > 0:  # SwiGLU of the part that bypasses the scan (k_activations.py:42)
+            gate, up = (t.float() for t in zx0.chunk(2, dim=-1))
+            d0 = dy_cat[..., :d_nonssm].float()
+            sg = torch.sigmoid(gate)
+            dzx0[..., :d_nonssm] = d0 * up * sg * (1 + gate * (1 - sg))
+            dzx0[..., d_nonssm:] = d0 * gate * sg
+        dy = dy_cat[..., d_nonssm:]
+        drmsnorm_weight = None
+        if not gate_in_scan:
+            dy2, drmsnorm_weight, _, _ = _layer_norm_bwd(
+                dy.reshape(batch * seqlen, dim), scan_out.view(batch * seqlen, dim), rmsnorm_weight, None,
+                ctx.rmsnorm_eps, None, rstd, z=z.reshape(batch * seqlen, dim), group_size=dim // ngroups,
+                norm_before_gate=ctx.norm_before_gate, is_rms_norm=True, dz=dz.view(batch * seqlen, dim))
+            dy = dy2.view(batch, seqlen, dim)
+        x, B, C = torch.split(xBC_conv, [dim, ngroups * dstate, ngroups * dstate], dim=-1)
+        dxBC_conv = torch.empty_like(xBC_conv)
+        dx, dB, dC = torch.split(dxBC_conv, [dim, ngroups * dstate, ngroups * dstate], dim=-1)
+        _, _, dA, _, _, dD, dz_scan, ddt_bias, dinitial_states = _mamba_chunk_scan_combined_bwd(
+            dy.reshape(batch, seqlen, nheads, headdim), x.reshape(batch, seqlen, nheads, headdim), dt, A,
+            B.reshape(batch, seqlen, ngroups, dstate), C.reshape(batch, seqlen, ngroups, dstate), scan_out, ctx.chunk_size,
+            D=D, z=z.reshape(batch, seqlen, nheads, headdim) if gate_in_scan else None, dt_bias=dt_bias,
+            initial_states=initial_states, dfinal_states=dfinal_states, seq_idx=seq_idx, dt_softplus=True,
+            dt_limit=ctx.dt_limit, saved=(dt_out, dA_cumsum, states),
+            dx=dx.view(batch, seqlen, nheads, headdim), ddt=ddt, dB=dB.view(batch, seqlen, ngroups, dstate),
+            dC=dC.view(batch, seqlen, ngroups, dstate))
+        if gate_in_scan:
+            dz.copy_(dz_scan.view(batch, seqlen, dim))
+        # the convolution's backward kernel re-computes its pre-activation from xBC and writes into the xBC slice
+        _, dconv_w, dconv_b = causal_conv1d_bwd(xBC.transpose(1, 2), conv_w, conv_b, dxBC_conv.transpose(1, 2),
+                                                seq_idx=seq_idx, activation=ctx.activation, dx=dxBC.transpose(1, 2))
+        if ctx.conv_w_3d:
+            dconv_w = dconv_w.unsqueeze(1)
+        return (dzxbcdt, dconv_w, dconv_b, ddt_bias, dA, dD, None, dinitial_states, None, None, None, None,
+                drmsnorm_weight, None, doutproj_weight, doutproj_bias, None, None, None, None)
+
+
 def mamba_split_conv1d_scan_combined(zxbcdt, conv1d_weight, conv1d_bias, dt_bias, A, D, chunk_size,
                                      initial_states=None, seq_idx=None, dt_limit=(0.0, float("inf")),
                                      return_final_states=False, activation="silu", rmsnorm_weight=None,
                                      rmsnorm_eps=1e-6, outproj_weight=None, outproj_bias=None, headdim=None,
                                      ngroups=1, norm_before_gate=True, state_dtype=None):
-    """The Mamba-2 block body after in_proj (ssd_combined.py:983, forward :824-899): split, causal
-    conv1d + SiLU on xBC, the chunked scan and the gate or gated RMSNorm on the HIP kernels, out_proj.
-    The projection is a torch GEMM; the gradients of the convolution, the scan and the norm come from
-    CausalConv1dFn, MambaChunkScanCombinedFn and LayerNormFn, chained by autograd.
+    """The Mamba-2 block body after in_proj (ssd_combined.py:983): split, causal conv1d + SiLU on xBC, the
+    chunked scan and the gate or gated RMSNorm on the HIP kernels, SwiGLU of the non-SSM part and out_proj
+    (torch GEMM), as one autograd node.
         zxbcdt: (batch, seqlen, 2 * d_nonssm + 2 * dim + 2 * ngroups * dstate + nheads), dim = nheads * headdim
         conv1d_weight: (dim + 2 * ngroups * dstate, width); conv1d_bias: (dim + 2 * ngroups * dstate,)
         dt_bias, A: (nheads,); D: (nheads, headdim) or (nheads,) (then headdim must be given)
         rmsnorm_weight: (dim,); outproj_weight: (out_dim, d_nonssm + dim); outproj_bias: (out_dim,)
         norm_before_gate: True computes RMSNorm(y) * silu(z), False RMSNorm(y * silu(z))
     Returns out, or (out, final_states) with return_final_states."""
-    import torch.nn.functional as F
-    assert activation in [None, "silu", "swish"]
-    if D.dim() == 1:
-        assert headdim is not None
-        nheads, = D.shape
-    else:
-        nheads, headdim = D.shape
-    batch, seqlen, _ = zxbcdt.shape
-    dim = nheads * headdim
-    assert nheads % ngroups == 0
-    dstate = (conv1d_weight.shape[0] - dim) // ngroups // 2
-    d_nonssm = (zxbcdt.shape[-1] - 2 * dim - 2 * ngroups * dstate - nheads) // 2
-    assert d_nonssm >= 0
-    assert zxbcdt.shape == (batch, seqlen, 2 * d_nonssm + 2 * dim + 2 * ngroups * dstate + nheads)
-    assert dt_bias.shape == (nheads,) and A.shape == (nheads,)
-    if conv1d_weight.dim() == 3:
-        conv1d_weight = conv1d_weight.squeeze(1)
-    zx0, z, xBC, dt = torch.split(zxbcdt, [2 * d_nonssm, dim, dim + 2 * ngroups * dstate, nheads], dim=-1)
-    # the HIP convolution reads the channel-contiguous slice as it lies and returns a dense (b, l, c) tensor
-    xBC = causal_conv1d_fn(xBC.transpose(1, 2), conv1d_weight, conv1d_bias, seq_idx=seq_idx,
-                           activation=activation).transpose(1, 2)
-    x, B, C = torch.split(xBC, [dim, ngroups * dstate, ngroups * dstate], dim=-1)
-    x = x.reshape(batch, seqlen, nheads, headdim)
-    B = B.reshape(batch, seqlen, ngroups, dstate)
-    C = C.reshape(batch, seqlen, ngroups, dstate)
-    z = z.reshape(batch, seqlen, nheads, headdim)
-    res = mamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=D, z=z if rmsnorm_weight is None else None,
-                                    dt_bias=dt_bias, initial_states=initial_states, seq_idx=seq_idx, dt_softplus=True,
-                                    dt_limit=dt_limit, return_final_states=return_final_states, state_dtype=state_dtype)
-    y, final_states = res if return_final_states else (res, None)
-    y = y.reshape(batch, seqlen, dim)
-    if rmsnorm_weight is not None:
-        # reads z where it lies inside zxbcdt (unit channel stride, row stride of the whole projection)
-        y = rmsnorm_fn(y, rmsnorm_weight, None, z=z.reshape(batch, seqlen, dim), eps=rmsnorm_eps,
-                       group_size=dim // ngroups, norm_before_gate=norm_before_gate)
-    if d_nonssm > 0:
-        gate, up = zx0.chunk(2, dim=-1)
-        y = torch.cat([(F.silu(gate.float()) * up.float()).to(y.dtype), y], dim=-1)
-    if outproj_weight is not None:
-        if torch.is_autocast_enabled():
-            ac = torch.get_autocast_gpu_dtype()
-            y, outproj_weight = y.to(ac), outproj_weight.to(ac)
-            outproj_bias = outproj_bias.to(ac) if outproj_bias is not None else None
-        y = F.linear(y, outproj_weight, outproj_bias)
-    else:
-        assert outproj_bias is None
-    return y if not return_final_states else (y, final_states)
+    return MambaSplitConv1dScanCombinedFn.apply(zxbcdt, conv1d_weight, conv1d_bias, dt_bias, A, D, chunk_size,
+                                                initial_states, seq_idx, dt_limit, return_final_states, activation,
+                                                rmsnorm_weight, rmsnorm_eps, outproj_weight, outproj_bias, headdim,
+                                                ngroups, norm_before_gate, state_dtype)
 
 
 def mamba_conv1d_scan_ref(xBC, conv1d_weight, conv1d_bias, dt, A, chunk_size, D=None, z=None, dt_bias=None,

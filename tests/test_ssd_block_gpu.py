@@ -75,6 +75,45 @@ def test_mamba_split_conv1d_scan_combined(norm, nbg, d_nonssm, packed, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("norm", [False, True])
+def test_block_without_projection_with_states_and_3d_conv_weight(norm, dtype):
+    """No out_proj, initial states, a gradient arriving through the final states, and the convolution weight
+    in nn.Conv1d's (channels, 1, width) shape."""
+    from mamba_amd.ops.triton.ssd_combined import mamba_split_conv1d_scan_combined
+    batch, L, nheads, headdim, dstate, ngroups, chunk = 2, 200, 4, 32, 16, 1, 64
+    t = _block_inputs(batch, L, nheads, headdim, dstate, ngroups, 8, 24, 21, dtype)
+    t.pop("outproj_weight")
+    t.pop("outproj_bias")
+    g = torch.Generator().manual_seed(8)
+    t["initial_states"] = 0.3 * torch.randn(batch, nheads, headdim, dstate, generator=g)
+    rtol, atol = _tol(dtype)
+    names = list(t)
+    ref_in = {k: t[k].float().clone().requires_grad_() for k in names}
+    gpu_in = {k: t[k].cuda().requires_grad_() for k in names}
+    w3 = gpu_in["conv1d_weight"].detach().unsqueeze(1).clone().requires_grad_()
+    kw = dict(headdim=headdim, ngroups=ngroups, norm_before_gate=False)
+    out_ref, fin_ref = split_conv1d_scan_oracle(
+        ref_in["zxbcdt"], ref_in["conv1d_weight"], ref_in["conv1d_bias"], ref_in["dt_bias"], ref_in["A"], ref_in["D"],
+        initial_states=ref_in["initial_states"], rmsnorm_weight=ref_in["rmsnorm_weight"] if norm else None, **kw)
+    out, fin = mamba_split_conv1d_scan_combined(
+        gpu_in["zxbcdt"], w3, gpu_in["conv1d_bias"], gpu_in["dt_bias"], gpu_in["A"], gpu_in["D"], chunk,
+        initial_states=gpu_in["initial_states"], return_final_states=True,
+        rmsnorm_weight=gpu_in["rmsnorm_weight"] if norm else None, **kw)
+    _close("out", out, out_ref, rtol, atol)
+    _close("final_states", fin, fin_ref, rtol, atol)
+    dout = torch.randn(out_ref.shape, generator=g)
+    dfin = torch.randn(fin_ref.shape, generator=g)
+    ((out_ref * dout).sum() + (fin_ref * dfin).sum()).backward()
+    torch.autograd.backward([out, fin], [dout.to(dtype).cuda(), dfin.cuda()])
+    assert w3.grad.shape == w3.shape
+    _close("dconv1d_weight", w3.grad.squeeze(1), ref_in["conv1d_weight"].grad, 5 * rtol, 5 * atol)
+    for k in names:
+        if k == "conv1d_weight" or (k == "rmsnorm_weight" and not norm):
+            continue
+        _close("d" + k, gpu_in[k].grad, ref_in[k].grad, 5 * rtol, 5 * atol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_ssd_selective_scan_and_chunk_scan_wrappers(dtype):
     from mamba_amd.ops.triton.ssd_combined import ssd_selective_scan, mamba_chunk_scan, ssd_chunk_scan_combined_ref
     t = ssd_inputs(2, 300, 4, 32, 16, 2, dtype, 13)
