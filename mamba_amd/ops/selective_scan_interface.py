@@ -367,7 +367,7 @@ class MambaInnerFn(torch.autograd.Function):
                 else "(b l) (dstate two) -> b 1 dstate (l two)")
         pack_kw = dict(l=L) if not A.is_complex() else dict(l=L, two=2)
         if torch.is_autocast_enabled():
-            ac = torch.get_autocast_gpu_dtype()
+            ac = torch.get_autocast_dtype("cuda")
             x_proj_weight, delta_proj_weight = x_proj_weight.to(ac), delta_proj_weight.to(ac)
             out_proj_weight = out_proj_weight.to(ac)
             out_proj_bias = out_proj_bias.to(ac) if out_proj_bias is not None else None

@@ -234,7 +234,7 @@ def layer_norm_linear_fn(x, norm_weight, norm_bias, linear_weight, linear_bias, 
                         residual_in_fp32=residual_in_fp32, is_rms_norm=is_rms_norm)
     y, residual_out = res if prenorm else (res, None)
     if torch.is_autocast_enabled():
-        ac = torch.get_autocast_gpu_dtype()
+        ac = torch.get_autocast_dtype("cuda")
         y, linear_weight = y.to(ac), linear_weight.to(ac)
         linear_bias = linear_bias.to(ac) if linear_bias is not None else None
     out = F.linear(y.to(linear_weight.dtype), linear_weight, linear_bias)

@@ -474,7 +474,7 @@ class MambaSplitConv1dScanCombinedFn(torch.autograd.Function):
         if outproj_weight is not None:
             w, bias = outproj_weight, outproj_bias
             if torch.is_autocast_enabled():
-                ctx.autocast = torch.get_autocast_gpu_dtype()
+                ctx.autocast = torch.get_autocast_dtype("cuda")
                 y, w = y.to(ctx.autocast), w.to(ctx.autocast)
                 bias = bias.to(ctx.autocast) if bias is not None else None
             res = F.linear(y, w, bias)
