@@ -426,14 +426,17 @@ def main():
     # Dominant kernel (the backward scan) alone, HIP events on the launch stream.
     with torch.no_grad():
         d = {k: v.detach() for k, v in leaves.items()}
-        _, ckpt = selective_scan_fwd(d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["z"], d["delta_bias"], True)
+        keep = ssi.KEEP_LANE_STATES   # the timed kernels are the ones a training step launches
+        _, ckpt, lanes = selective_scan_fwd(d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["z"], d["delta_bias"],
+                                            True, lane_states=True)
+        lanes = lanes if keep else None
         dims = (batch, dim, seqlen, dstate, 1)
         bufs = ssi.ScanBwdBuffers(d["u"], d["delta"], d["B"], d["z"], dims)
         bwd_pre = lambda: ssi.scan_bwd_zero(bufs, dev)  # outside the event pair
         bwd = lambda: ssi.scan_bwd_launch(d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["z"],
-                                          d["delta_bias"], t["dout"], ckpt, True, bufs, dims)
+                                          d["delta_bias"], t["dout"], ckpt, True, bufs, dims, lanes)
         fwd = lambda: selective_scan_fwd(d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["z"],
-                                         d["delta_bias"], True)
+                                         d["delta_bias"], True, lane_states=keep)
 
         n = max(5, min(args.steps, 50))
         bwd_ms = event_ms(bwd, n, bwd_pre)

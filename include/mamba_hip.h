@@ -121,6 +121,11 @@ typedef struct MambaScanParams {
   int64_t ddelta_bs, ddelta_ds;
   int64_t dz_bs, dz_ds;
   int64_t outz_bs, outz_ds;
+  /* Optional (real A only): (batch, dim, ntiles, dstate, 64) fp32, the state entering each lane's
+   * 8 positions of a tile.  The forward call writes it when non-null; the backward call, when
+   * non-null, starts its re-computation of the states from it instead of re-running the scan over
+   * the tile (about a tenth of its instructions). */
+  float *lane_state;
 } MambaScanParams;
 
 int mamba1_scan_fwd(const MambaScanParams *p, mamba_stream_t stream);

@@ -27,6 +27,7 @@ class MambaScanParams(ctypes.Structure):
                                "ddelta_bias_part")]
         + [(n, c_i64) for n in ("dout_bs", "dout_ds", "du_bs", "du_ds", "ddelta_bs", "ddelta_ds", "dz_bs", "dz_ds",
                                 "outz_bs", "outz_ds")]
+        + [("lane_state", c_vp)]
     )
 
 

@@ -156,6 +156,8 @@ __global__ __launch_bounds__(NW * 64, 4) void scan_fwd_kernel(const MambaScanPar
       float u[8], dl[8], du[8], y[8], dsum = 0.f;
       Pack8<T> ku, kd, kz;  // raw rows: every load is issued before the first conversion
       kz.zero();
+      // lane states of this (tile, channel), when the caller keeps them for the backward pass
+      float *lanes = (p.lane_state && valid) ? p.lane_state + (((int64_t)b * p.dim + d) * ntiles + tile) * N * 64 : nullptr;
       if (valid) {
         load_items<T, VEC>(ku, (const T *)p.u + b * p.u_bs + d * p.u_ds, tl, L, nvalid);
         load_items<T, VEC>(kd, (const T *)p.delta + b * p.delta_bs + d * p.delta_ds, tl, L, nvalid);
@@ -217,6 +219,7 @@ __global__ __launch_bounds__(NW * 64, 4) void scan_fwd_kernel(const MambaScanPar
             for (int q = 0; q < 2; ++q) {
               float h = dpp_f<DPP_WAVE_SHR1>(hc[q], hend[q]);  // state entering this lane
               if (lane == 63) hrow[n + q] = hend[q];           // state after the tile
+              if (lanes && nb * NB16 + n + q < N) lanes[(nb * NB16 + n + q) * 64 + lane] = h;
 #pragma unroll
               for (int i = 0; i < KI; ++i) {
                 h = __builtin_fmaf(a[q][i], h, bb[q][i]);
@@ -254,11 +257,13 @@ __global__ __launch_bounds__(NW * 64, 4) void scan_fwd_kernel(const MambaScanPar
 template <typename T> struct BwdRow {
   const T *u, *delta, *dout, *z;
   T *du, *ddelta, *dz, *out_z;
-  const float *ckpt;  // checkpoint of tile 0 of this channel
+  const float *ckpt;  // tile 0 of this channel: the tile checkpoints, or with LS the lane states
   float D, bias;
 };
 
-template <typename T, int NW, int R, bool VEC, int BC>
+// LS: the forward pass left the state entering every lane's 8 positions (lane_state); the states of a
+// tile are then re-computed from those directly, without the lane-local pass and the wave scan.
+template <typename T, int NW, int R, bool VEC, int BC, bool LS>
 __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams p) {
   static_assert(sizeof(BwdRow<T>) == 80, "the host side sizes the LDS table with 80 bytes per channel");
   extern __shared__ __align__(16) float smem[];
@@ -301,7 +306,7 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
     q.ddelta = (T *)p.ddelta + b * p.ddelta_bs + d * p.ddelta_ds;
     q.dz = has_z ? (T *)p.dz + b * p.dz_bs + d * p.dz_ds : nullptr;
     q.out_z = (has_z && p.out_z) ? (T *)p.out_z + b * p.outz_bs + d * p.outz_ds : nullptr;
-    q.ckpt = p.ckpt + ((int64_t)b * p.dim + d) * ntiles * N;
+    q.ckpt = LS ? p.lane_state + ((int64_t)b * p.dim + d) * ntiles * N * 64 : p.ckpt + ((int64_t)b * p.dim + d) * ntiles * N;
     q.D = p.D ? ((const float *)p.D)[d] : 0.f;
     q.bias = p.delta_bias ? ((const float *)p.delta_bias)[d] : 0.f;
     rows[wave * R + lane] = q;
@@ -329,18 +334,31 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
   }
 
   // The rows of the next (tile, channel) are fetched while the current one is computed.
+  constexpr int NPP = NB16 / NW > 0 ? NB16 / NW : 1;  // state rows per wave and phase (see the state loop)
+  constexpr int NPH = NB16 / NPP;
+  constexpr int Q = NPP >= 2 ? 2 : 1;                 // states per step; two keep two scan chains in flight
   struct Rows {
     Pack8<T> u, delta, dout, z;
-    float ck;  // checkpointed state n = lane entering the tile (when the padded state count fits a wave)
+    float ck;     // !LS: checkpointed state n = lane entering the tile (when the padded state count fits a wave)
+    float h0[Q];  // LS: lane states of the first step's states
+  };
+  // lane states of step (nb, ph, j) of a (tile, channel): rows past N read a clamped row and are never used
+  auto lane_states = [&](const float *tile_base, int nb, int ph, int j, float (&o)[Q]) {
+    const int n = nb * NB16 + ((wave + ph) % NPH) * NPP + j;
+#pragma unroll
+    for (int q = 0; q < Q; ++q) o[q] = tile_base[(int64_t)min(n + q, N - 1) * 64 + lane];
   };
   auto fetch_rows = [&](Rows &k, int tile, int r) {
     const int d = dbase + r, tl = tile * TILE + lane * KI;
     const int nvalid = min(max(L - tl, 0), KI);
     k.z.zero();
     k.ck = 0.f;
+#pragma unroll
+    for (int q = 0; q < Q; ++q) k.h0[q] = 0.f;
     if (d < dend) {
       const BwdRow<T> &q = rows[wave * R + r];
-      if (NP <= 64 && tile > 0 && lane < N) k.ck = q.ckpt[(int64_t)(tile - 1) * N + lane];
+      if constexpr (LS) lane_states(q.ckpt + (int64_t)tile * N * 64, 0, 0, 0, k.h0);
+      else if (NP <= 64 && tile > 0 && lane < N) k.ck = q.ckpt[(int64_t)(tile - 1) * N + lane];
       load_items<T, VEC>(k.u, q.u, tl, L, nvalid);
       load_items<T, VEC>(k.delta, q.delta, tl, L, nvalid);
       load_items<T, VEC>(k.dout, q.dout, tl, L, nvalid);
@@ -360,6 +378,9 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
       float u[8], dl[8], du[8], dy[8], acc[8], dd[8], y[8], dsum = 0.f, dtail = 0.f;
       // raw delta, z and dout stay in registers in their storage format for the epilogue
       const Rows cur = nxt;
+      float hnext[Q];  // LS: lane states of the step about to run
+#pragma unroll
+      for (int q = 0; q < Q; ++q) hnext[q] = cur.h0[q];
       Pack8<T> draw_k = cur.delta, z_k = cur.z, dout_k = cur.dout;
       if (r + 1 < R) fetch_rows(nxt, tile, r + 1);
       else if (tile > 0) fetch_rows(nxt, tile - 1, 0);
@@ -397,7 +418,8 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
         for (int i = 1; i < KI; ++i) dtail += dl[i];
         dsum = dtail + dl[0];
         // state entering this tile
-        if (NP <= 64) {
+        if constexpr (LS) {
+        } else if (NP <= 64) {
           if (lane < NP) hcar[row * NP + lane] = cur.ck;
         } else {
           for (int n = lane; n < NP; n += 64) {
@@ -419,8 +441,6 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
           // The NW waves add their channels' dB/dC terms into the shared LDS sums without
           // atomics: in phase ph wave w owns state rows (w + ph) % NPH * NPP .. + NPP - 1,
           // so no two waves touch a row between two barriers.
-          constexpr int NPP = NB16 / NW > 0 ? NB16 / NW : 1;
-          constexpr int NPH = NB16 / NPP;
           static_assert(NW <= NPH, "one row slot per wave and phase");
           const float *A1row = A1s + row * NP + nb * NB16;
           const float *hrow = hcar + row * NP + nb * NB16;
@@ -428,12 +448,22 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
           float *arow = anx + row * NP + nb * NB16;
           float *dArow = dAacc + row * NP + nb * NB16;
           const int nmax = min(NB16, N - nb * NB16);
-          constexpr int Q = NPP >= 2 ? 2 : 1;  // states per step; two keep two scan chains in flight
           static_assert(NPP % Q == 0, "whole steps per phase");
           for (int ph = 0; ph < NPH; ++ph) {
             const int slot = (wave + ph) % NPH;
             for (int j = 0; j < NPP; j += Q) {
               const int n = slot * NPP + j;
+              float hin[Q];
+              if constexpr (LS) {
+                // this step's lane states arrived during the previous step (the first step's with the rows);
+                // the next step's are requested now
+#pragma unroll
+                for (int q = 0; q < Q; ++q) hin[q] = hnext[q];
+                int j2 = j + Q, ph2 = ph, nb2 = nb;
+                if (j2 >= NPP) { j2 = 0; ++ph2; }
+                if (ph2 >= NPH) { ph2 = 0; ++nb2; }
+                if (valid && nb2 < NBLK) lane_states(rows[row].ckpt + (int64_t)tile * N * 64, nb2, ph2, j2, hnext);
+              }
               if (!valid || n >= nmax) continue;
               // Forward states: pass 1 runs the lane's 8 steps from zero for the lane's (decay, value)
               // pair, the decay being one exp of the summed delta; pass 2 reruns them from the state
@@ -444,32 +474,38 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
 #pragma unroll
               for (int q = 0; q < Q; ++q) {
                 A1[q] = A1row[n + q];
-                hc[q] = hrow[n + q];
+                hc[q] = LS ? 0.f : hrow[n + q];
                 gc[q] = grow[n + q];
                 an[q] = arow[n + q];
                 float Bv[8];  // read again for the last loop: 16 registers fewer held through the scans
                 load_bc<BC & 1>(Bv, Bs, p.B, d, N, nb * NB16 + n + q, n + q, lane);
                 load_bc<BC & 2>(Cv[q], Cs, p.C, d, N, nb * NB16 + n + q, n + q, lane);
                 const float A2 = A1[q] * kLog2e;
-                sa[q] = fast_exp2(dsum * A2);
 #pragma unroll
                 for (int i = 0; i < KI; ++i) {
                   a[q][i] = fast_exp2(dl[i] * A2);
                   bb[q][i] = du[i] * Bv[i];
                 }
-                float hl = bb[q][0];
+                if constexpr (!LS) {
+                  sa[q] = fast_exp2(dsum * A2);
+                  float hl = bb[q][0];
 #pragma unroll
-                for (int i = 1; i < KI; ++i) hl = __builtin_fmaf(a[q][i], hl, bb[q][i]);
-                sb[q] = hl;
+                  for (int i = 1; i < KI; ++i) hl = __builtin_fmaf(a[q][i], hl, bb[q][i]);
+                  sb[q] = hl;
+                }
               }
-              if constexpr (Q == 2) wave_scan_fwd2(sa[0], sb[0], sa[1], sb[1]);
-              else wave_scan_fwd(sa[0], sb[0]);
+              if constexpr (!LS) {
+                if constexpr (Q == 2) wave_scan_fwd2(sa[0], sb[0], sa[1], sb[1]);
+                else wave_scan_fwd(sa[0], sb[0]);
 #pragma unroll
-              for (int q = 0; q < Q; ++q) hend[q] = __builtin_fmaf(sa[q], hc[q], sb[q]);
+                for (int q = 0; q < Q; ++q) hend[q] = __builtin_fmaf(sa[q], hc[q], sb[q]);
+              }
               float ra[Q], rb[Q], gfirst[Q], a_next_lane[Q];
 #pragma unroll
               for (int q = 0; q < Q; ++q) {
-                float hp = dpp_f<DPP_WAVE_SHR1>(hc[q], hend[q]);
+                float hp;
+                if constexpr (LS) hp = hin[q];
+                else hp = dpp_f<DPP_WAVE_SHR1>(hc[q], hend[q]);
 #pragma unroll
                 for (int i = 0; i < KI; ++i) {
                   hp = __builtin_fmaf(a[q][i], hp, bb[q][i]);
@@ -677,12 +713,18 @@ template <typename T, bool BWD, int BC> int dispatch_bc(const MambaScanParams &p
   } else {
     if (small) {
       const size_t lds = bwd_lds(8, 4, np);
-      return vec ? launch(scan_bwd_kernel<T, 8, 4, true, BC>, p, 8, 4, lds, stream)
-                 : launch(scan_bwd_kernel<T, 8, 4, false, BC>, p, 8, 4, lds, stream);
+      if (p.lane_state)
+        return vec ? launch(scan_bwd_kernel<T, 8, 4, true, BC, true>, p, 8, 4, lds, stream)
+                   : launch(scan_bwd_kernel<T, 8, 4, false, BC, true>, p, 8, 4, lds, stream);
+      return vec ? launch(scan_bwd_kernel<T, 8, 4, true, BC, false>, p, 8, 4, lds, stream)
+                 : launch(scan_bwd_kernel<T, 8, 4, false, BC, false>, p, 8, 4, lds, stream);
     }
     const size_t lds = bwd_lds(4, 1, np);
-    return vec ? launch(scan_bwd_kernel<T, 4, 1, true, BC>, p, 4, 1, lds, stream)
-               : launch(scan_bwd_kernel<T, 4, 1, false, BC>, p, 4, 1, lds, stream);
+    if (p.lane_state)
+      return vec ? launch(scan_bwd_kernel<T, 4, 1, true, BC, true>, p, 4, 1, lds, stream)
+                 : launch(scan_bwd_kernel<T, 4, 1, false, BC, true>, p, 4, 1, lds, stream);
+    return vec ? launch(scan_bwd_kernel<T, 4, 1, true, BC, false>, p, 4, 1, lds, stream)
+               : launch(scan_bwd_kernel<T, 4, 1, false, BC, false>, p, 4, 1, lds, stream);
   }
 }
 

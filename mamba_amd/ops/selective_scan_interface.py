@@ -101,13 +101,21 @@ def _fill_common(p, u, delta, A, B, C, D, z, delta_bias, delta_softplus, ckpt, d
         p.C_bs, p.C_gs, p.C_ns = C.stride(0), C.stride(1), C.stride(2)
 
 
-def selective_scan_fwd(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta_softplus=False):
+# Keep the state entering every lane's 8 positions from the forward pass for the backward pass
+# (batch * dim * seqlen / 8 * dstate * 4 bytes: 1.3 GB at batch 8, dim 5120, seqlen 4096, dstate 16).  The
+# backward kernel then skips its own scan over each tile, about a tenth of its instructions.  False
+# makes it re-run that scan and keeps only the per-tile checkpoints.
+KEEP_LANE_STATES = True
+
+
+def selective_scan_fwd(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta_softplus=False, lane_states=False):
     """Counterpart of selective_scan_cuda.fwd (selective_scan.cpp:226).
 
-    Returns (out, ckpt): `out` is the gated output y*silu(z) when z is given, else y, in u's
-    dtype; `ckpt` is (batch, dim, ntiles, dstate) fp32, the state after each tile of
-    `scan_tile()` positions (ckpt[:, :, -1] is the last state).  The ungated y is not
-    stored: the backward pass re-computes it.
+    Returns (out, ckpt), or (out, ckpt, lanes) with lane_states=True: `out` is the gated output
+    y*silu(z) when z is given, else y, in u's dtype; `ckpt` is (batch, dim, ntiles, dstate) fp32, the
+    state after each tile of `scan_tile()` positions (ckpt[:, :, -1] is the last state); `lanes` is
+    (batch, dim, ntiles, dstate, 64) fp32, the state entering each lane's 8 positions (None with a
+    complex A).  The ungated y is not stored: the backward pass re-computes it.
     """
     dims = _check_inputs(u, delta, A, B, C, D, z, delta_bias)
     batch, dim, seqlen, dstate, _ = dims
@@ -120,9 +128,13 @@ def selective_scan_fwd(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta
     _fill_common(p, u, delta, A, B, C, D, z, delta_bias, delta_softplus, ckpt, dims)
     p.out = out.data_ptr()
     p.out_bs, p.out_ds = out.stride(0), out.stride(1)
+    lanes = None
+    if lane_states and not A.is_complex():
+        lanes = torch.empty((batch, dim, ntiles, dstate, 64), device=u.device, dtype=torch.float32)
+        p.lane_state = lanes.data_ptr()
     with torch.cuda.device(u.device):
         _lib.check(_lib.load().mamba1_scan_fwd(p, _lib.current_stream(u.device)), "mamba1_scan_fwd")
-    return out, ckpt
+    return (out, ckpt, lanes) if lane_states else (out, ckpt)
 
 
 class ScanBwdBuffers:
@@ -160,10 +172,11 @@ def scan_bwd_zero(bufs, device):
                                               _lib.current_stream(device)), "mamba_hip_zero")
 
 
-def scan_bwd_launch(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, delta_softplus, bufs, dims):
+def scan_bwd_launch(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, delta_softplus, bufs, dims, lanes=None):
     """One call of the C ABI's mamba1_scan_bwd on the current stream; bufs.dBC32 must be zero."""
     p = _lib.MambaScanParams()
     _fill_common(p, u, delta, A, B, C, D, z, delta_bias, delta_softplus, ckpt, dims)
+    p.lane_state = _lib.ptr(lanes)
     dz, out_z = bufs.dz, bufs.out_z
     p.dout, p.du, p.ddelta = dout.data_ptr(), bufs.du.data_ptr(), bufs.ddelta.data_ptr()
     p.dz, p.out_z = _lib.ptr(dz), _lib.ptr(out_z)
@@ -182,11 +195,12 @@ def scan_bwd_launch(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, delta_softp
 
 
 def selective_scan_bwd(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, dz=None, delta_softplus=False,
-                       recompute_out_z=False):
+                       recompute_out_z=False, lanes=None):
     """Counterpart of selective_scan_cuda.bwd (selective_scan.cpp:338).
 
     `dz` may be a caller-owned strided view (last stride 1) that receives the gate gradient,
-    as MambaInnerFn passes it (selective_scan_interface.py:333-338).
+    as MambaInnerFn passes it (selective_scan_interface.py:333-338).  `lanes` is the third result of
+    selective_scan_fwd(..., lane_states=True), or None to re-run the scan over each tile.
     Returns (du, ddelta, dA, dB, dC, dD, ddelta_bias, dz, out_z).
     """
     dims = _check_inputs(u, delta, A, B, C, D, z, delta_bias)
@@ -201,7 +215,14 @@ def selective_scan_bwd(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, dz=None,
     cplx = A.is_complex()
     bufs = ScanBwdBuffers(u, delta, B, z, dims, dz, recompute_out_z, C=C, complex_A=cplx)
     scan_bwd_zero(bufs, u.device)
-    scan_bwd_launch(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, delta_softplus, bufs, dims)
+    if lanes is not None:
+        _lib.require_gpu(lanes)
+        ntiles = (seqlen + scan_tile() - 1) // scan_tile()
+        if cplx or lanes.dtype != torch.float32 or tuple(lanes.shape) != (batch, dim, ntiles, dstate, 64) \
+                or not lanes.is_contiguous():
+            raise RuntimeError("selective_scan: lanes must be the contiguous fp32 (batch, dim, ntiles, dstate, 64) "
+                               "tensor of the forward call (real A only)")
+    scan_bwd_launch(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, delta_softplus, bufs, dims, lanes)
     as_A = (lambda t: torch.view_as_complex(t.reshape(dim, dstate, 2))) if cplx else (lambda t: t)
     dA = as_A(bufs.dA_part.sum(0))
     dD = bufs.dD_part.sum(0) if D is not None else None
@@ -236,7 +257,9 @@ class SelectiveScanFn(torch.autograd.Function):
         if C.dim() == 3:
             C = rearrange(C, "b dstate l -> b 1 dstate l")
             ctx.squeeze_C = True
-        out, ckpt = selective_scan_fwd(u, delta, A, B, C, D, z, delta_bias, delta_softplus)
+        keep = KEEP_LANE_STATES and any(ctx.needs_input_grad)
+        out, ckpt, lanes = selective_scan_fwd(u, delta, A, B, C, D, z, delta_bias, delta_softplus, lane_states=keep) \
+            if keep else (*selective_scan_fwd(u, delta, A, B, C, D, z, delta_bias, delta_softplus), None)
         ctx.delta_softplus = delta_softplus
         ctx.has_z = z is not None
         ctx.has_D = D is not None
@@ -244,16 +267,16 @@ class SelectiveScanFn(torch.autograd.Function):
         last_state = ckpt[:, :, -1]  # (batch, dim, dstate)
         if A.is_complex():
             last_state = torch.view_as_complex(last_state)
-        ctx.save_for_backward(u, delta, A, B, C, D, z, delta_bias, ckpt)
+        ctx.save_for_backward(u, delta, A, B, C, D, z, delta_bias, ckpt, lanes)
         return out if not return_last_state else (out, last_state)
 
     @staticmethod
     def backward(ctx, dout, *args):
-        u, delta, A, B, C, D, z, delta_bias, ckpt = ctx.saved_tensors
+        u, delta, A, B, C, D, z, delta_bias, ckpt, lanes = ctx.saved_tensors
         if dout.stride(-1) != 1:
             dout = dout.contiguous()
         du, ddelta, dA, dB, dC, dD, ddelta_bias, dz, _ = selective_scan_bwd(
-            u, delta, A, B, C, D, z, delta_bias, dout, ckpt, None, ctx.delta_softplus, False)
+            u, delta, A, B, C, D, z, delta_bias, dout, ckpt, None, ctx.delta_softplus, False, lanes=lanes)
         dB = dB.squeeze(1) if ctx.squeeze_B else dB
         dC = dC.squeeze(1) if ctx.squeeze_C else dC
         return (du, ddelta, dA, dB, dC, dD, dz, ddelta_bias, None, None)
@@ -407,7 +430,10 @@ class MambaInnerFn(torch.autograd.Function):
         if dt_rms_weight is not None:
             delta = rearrange(_rms_norm(rearrange(delta, "b d l -> (b l) d").contiguous(), dt_rms_weight,
                                         b_c_dt_rms_eps), "(b l) d -> b d l", l=L).contiguous()
-        out_z, ckpt = selective_scan_fwd(conv1d_out, delta, A, B, C, D, z, delta_bias, delta_softplus)
+        out_z, ckpt, lanes = selective_scan_fwd(conv1d_out, delta, A, B, C, D, z, delta_bias, delta_softplus,
+                                                lane_states=True)
+        if not KEEP_LANE_STATES:
+            lanes = None
         ctx.delta_softplus = delta_softplus
         ctx.out_proj_bias_is_None = out_proj_bias is None
         ctx.checkpoint_lvl = checkpoint_lvl
@@ -415,7 +441,7 @@ class MambaInnerFn(torch.autograd.Function):
         if checkpoint_lvl >= 1:  # conv1d_out and delta are recomputed in the backward pass
             conv1d_out, delta = None, None
         ctx.save_for_backward(xz, conv1d_weight, conv1d_bias, x_dbl, x_proj_weight, delta_proj_weight,
-                              out_proj_weight, conv1d_out, delta, A, B, C, D, delta_bias, ckpt)
+                              out_proj_weight, conv1d_out, delta, A, B, C, D, delta_bias, ckpt, lanes)
         out = F.linear(_as_matrix(out_z).t(), out_proj_weight, out_proj_bias)   # out_z has delta's layout
         return out.view(xz.shape[0], L, -1)
 
@@ -423,7 +449,7 @@ class MambaInnerFn(torch.autograd.Function):
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, dout):
         (xz, conv1d_weight, conv1d_bias, x_dbl, x_proj_weight, delta_proj_weight, out_proj_weight, conv1d_out,
-         delta, A, B, C, D, delta_bias, ckpt) = ctx.saved_tensors
+         delta, A, B, C, D, delta_bias, ckpt, lanes) = ctx.saved_tensors
         L = xz.shape[-1]
         delta_rank = delta_proj_weight.shape[1]
         d_state = A.shape[-1] * (1 if not A.is_complex() else 2)
@@ -445,7 +471,7 @@ class MambaInnerFn(torch.autograd.Function):
         dout_y = _from_matrix(out_proj_weight.t() @ dout, L)
         # du, ddelta and out_z come back in the layouts of u and delta
         dconv1d_out, ddelta, dA, dB, dC, dD, ddelta_bias, dz, out_z = selective_scan_bwd(
-            conv1d_out, delta, A, B, C, D, z, delta_bias, dout_y, ckpt, dz, ctx.delta_softplus, True)
+            conv1d_out, delta, A, B, C, D, z, delta_bias, dout_y, ckpt, dz, ctx.delta_softplus, True, lanes=lanes)
         dout_proj_weight = dout @ _as_matrix(out_z).t()
         dout_proj_bias = dout.sum(dim=1) if not ctx.out_proj_bias_is_None else None
         dx_dbl = torch.empty_like(x_dbl)
