@@ -31,7 +31,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch read off the FETCH_SIZE / WRITE_SIZE counters (scaled by the copy yardstick),
 # from the *_hbm_counters.txt summaries under profiles/; they describe the kernels as committed there.
-TRAFFIC = {"scan_bwd_kernel": 1399.2e6 + 1680.7e6, "scan_fwd_kernel": 1043.6e6 + 360.3e6,
+TRAFFIC = {"scan_bwd_kernel": 2719.6e6 + 1686.0e6, "scan_fwd_kernel": 1098.0e6 + 1709.5e6,
            "chunk_scan_fwd_fused_kernel": 591.1e6 + 335.5e6, "state_update_kernel": 683.1e6 + 673.7e6}
 
 
