@@ -426,7 +426,7 @@ def main():
     # Dominant kernel (the backward scan) alone, HIP events on the launch stream.
     with torch.no_grad():
         d = {k: v.detach() for k, v in leaves.items()}
-        keep = ssi.KEEP_LANE_STATES   # the timed kernels are the ones a training step launches
+        keep = ssi._keep_lane_states(d["u"], d["A"])   # the timed kernels are the ones a training step launches
         _, ckpt, lanes = selective_scan_fwd(d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["z"], d["delta_bias"],
                                             True, lane_states=True)
         lanes = lanes if keep else None

@@ -106,12 +106,20 @@ def _fill_common(p, u, delta, A, B, C, D, z, delta_bias, delta_softplus, ckpt, d
 # backward kernel then skips its own scan over each tile, about a tenth of its instructions.  False
 # makes it re-run that scan and keeps only the per-tile checkpoints.
 KEEP_LANE_STATES = True
+KEEP_LANE_STATES_MAX_BYTES = 16 << 30   # above this size per call the buffer is not kept
 
 
-def selective_scan_fwd(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta_softplus=False, lane_states=False):
+def _keep_lane_states(u, A):
+    batch, dim, seqlen = u.shape
+    ntiles = (seqlen + scan_tile() - 1) // scan_tile()
+    return (KEEP_LANE_STATES and not A.is_complex()
+            and batch * dim * ntiles * A.shape[1] * 64 * 4 <= KEEP_LANE_STATES_MAX_BYTES)
+
+
+def selective_scan_fwd(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta_softplus=False, lane_states=None):
     """Counterpart of selective_scan_cuda.fwd (selective_scan.cpp:226).
 
-    Returns (out, ckpt), or (out, ckpt, lanes) with lane_states=True: `out` is the gated output
+    Returns (out, ckpt), or (out, ckpt, lanes) when lane_states is True or False (lanes None if False): `out` is the gated output
     y*silu(z) when z is given, else y, in u's dtype; `ckpt` is (batch, dim, ntiles, dstate) fp32, the
     state after each tile of `scan_tile()` positions (ckpt[:, :, -1] is the last state); `lanes` is
     (batch, dim, ntiles, dstate, 64) fp32, the state entering each lane's 8 positions (None with a
@@ -134,7 +142,7 @@ def selective_scan_fwd(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta
         p.lane_state = lanes.data_ptr()
     with torch.cuda.device(u.device):
         _lib.check(_lib.load().mamba1_scan_fwd(p, _lib.current_stream(u.device)), "mamba1_scan_fwd")
-    return (out, ckpt, lanes) if lane_states else (out, ckpt)
+    return (out, ckpt, lanes) if lane_states is not None else (out, ckpt)
 
 
 class ScanBwdBuffers:
@@ -257,9 +265,8 @@ class SelectiveScanFn(torch.autograd.Function):
         if C.dim() == 3:
             C = rearrange(C, "b dstate l -> b 1 dstate l")
             ctx.squeeze_C = True
-        keep = KEEP_LANE_STATES and any(ctx.needs_input_grad)
-        out, ckpt, lanes = selective_scan_fwd(u, delta, A, B, C, D, z, delta_bias, delta_softplus, lane_states=keep) \
-            if keep else (*selective_scan_fwd(u, delta, A, B, C, D, z, delta_bias, delta_softplus), None)
+        keep = _keep_lane_states(u, A) and any(ctx.needs_input_grad)
+        out, ckpt, lanes = selective_scan_fwd(u, delta, A, B, C, D, z, delta_bias, delta_softplus, lane_states=keep)
         ctx.delta_softplus = delta_softplus
         ctx.has_z = z is not None
         ctx.has_D = D is not None
@@ -431,9 +438,7 @@ class MambaInnerFn(torch.autograd.Function):
             delta = rearrange(_rms_norm(rearrange(delta, "b d l -> (b l) d").contiguous(), dt_rms_weight,
                                         b_c_dt_rms_eps), "(b l) d -> b d l", l=L).contiguous()
         out_z, ckpt, lanes = selective_scan_fwd(conv1d_out, delta, A, B, C, D, z, delta_bias, delta_softplus,
-                                                lane_states=True)
-        if not KEEP_LANE_STATES:
-            lanes = None
+                                                lane_states=_keep_lane_states(conv1d_out, A))
         ctx.delta_softplus = delta_softplus
         ctx.out_proj_bias_is_None = out_proj_bias is None
         ctx.checkpoint_lvl = checkpoint_lvl
