@@ -111,3 +111,54 @@ def test_mamba1_layer_prefill_then_decode(dtype, rtol, atol):
                                        dt_bias=dt_bias, dt_softplus=True)
             outs.append(y)
         _close("decode", torch.stack(outs, dim=2), full[:, :, L0:], rtol, atol)
+
+
+def test_mamba2_packed_prefill_then_one_decode_step_per_sequence():
+    """Variable-length inference (mamba2.py:216-228, :255-262): three sequences packed into one row are prefilled
+    with seq_idx / cu_seqlens, the per-sequence scan and convolution states land in a pool of state rows, and one
+    more token per sequence is decoded as a batch through the pool indices; each must equal position len_i of a
+    one-pass call on that sequence alone."""
+    from mamba_amd.ops.causal_conv1d import causal_conv1d_fn, causal_conv1d_update, causal_conv1d_varlen_states
+    from mamba_amd.ops.triton.selective_state_update import selective_state_update
+    from mamba_amd.ops.triton.ssd_combined import mamba_chunk_scan_combined
+    g = torch.Generator().manual_seed(2)
+    r = lambda *s: torch.randn(*s, generator=g)
+    lens, nheads, headdim, N, ngroups, W, chunk = [70, 33, 129], 4, 32, 16, 1, 4, 64
+    dim, total = nheads * headdim, sum(lens)
+    conv_dim = dim + 2 * ngroups * N
+    conv_w, conv_b = (0.4 * r(conv_dim, W)).cuda(), (0.1 * r(conv_dim)).cuda()
+    dt_bias, A, D = (r(nheads) * 0.5 - 1).cuda(), (-(0.5 + torch.rand(nheads, generator=g))).cuda(), torch.rand(nheads, generator=g).cuda()
+    # inputs after in_proj, one token more than the prefill per sequence
+    seqs = [dict(xBC=r(n + 1, conv_dim).cuda(), dt=r(n + 1, nheads).cuda()) for n in lens]
+
+    def scan(xBC, dt, **kw):
+        xc = causal_conv1d_fn(xBC.transpose(0, 1)[None], conv_w, conv_b, activation="silu", seq_idx=kw.get("seq_idx"))[0].transpose(0, 1)
+        xs, B, C = torch.split(xc, [dim, ngroups * N, ngroups * N], dim=-1)
+        return mamba_chunk_scan_combined(xs.reshape(1, -1, nheads, headdim), dt[None], A, B.reshape(1, -1, ngroups, N),
+                                         C.reshape(1, -1, ngroups, N), chunk, D=D, dt_bias=dt_bias, dt_softplus=True, **kw)
+
+    with torch.no_grad():
+        want = torch.stack([scan(s["xBC"], s["dt"])[0, -1] for s in seqs])                 # (nseq, h, p): the extra token
+        xBC_pack = torch.cat([s["xBC"][:-1] for s in seqs])
+        dt_pack = torch.cat([s["dt"][:-1] for s in seqs])
+        cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32, device="cuda")
+        seq_idx = torch.cat([torch.full((n,), i, dtype=torch.int32) for i, n in enumerate(lens)])[None].cuda()
+        _, varlen_states = scan(xBC_pack, dt_pack, seq_idx=seq_idx, cu_seqlens=cu, return_varlen_states=True)
+        assert varlen_states.shape == (3, nheads, headdim, N)
+        # pools of 5 state rows; the three sequences live in rows 4, 0, 2
+        rows = torch.tensor([4, 0, 2], dtype=torch.int32, device="cuda")
+        ssm_pool = torch.zeros(5, nheads, headdim, N, device="cuda")
+        conv_pool = torch.zeros(5, conv_dim, W, device="cuda")
+        ssm_pool[rows.long()] = varlen_states.float()
+        conv_pool[rows.long()] = causal_conv1d_varlen_states(xBC_pack, cu, W)
+        xBC_new = torch.stack([s["xBC"][-1] for s in seqs])
+        dt_new = torch.stack([s["dt"][-1] for s in seqs])
+        xc = causal_conv1d_update(xBC_new, conv_pool, conv_w, conv_b, "silu", conv_state_indices=rows)
+        xs, B, C = torch.split(xc, [dim, ngroups * N, ngroups * N], dim=-1)
+        got = selective_state_update(
+            ssm_pool, xs.reshape(3, nheads, headdim), dt_new[:, :, None].expand(3, nheads, headdim),
+            A[:, None, None].expand(nheads, headdim, N), B.reshape(3, ngroups, N), C.reshape(3, ngroups, N),
+            D=D[:, None].expand(nheads, headdim), dt_bias=dt_bias[:, None].expand(nheads, headdim), dt_softplus=True,
+            state_batch_indices=rows)
+        _close("decode after packed prefill", got, want, 2e-3, 2e-3)
+        assert float(ssm_pool[[1, 3]].abs().max()) == 0.0 and float(conv_pool[[1, 3]].abs().max()) == 0.0
