@@ -42,7 +42,7 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
   static_assert(NWG * SPLIT == NWV, "waves divide evenly over the workgroups");
   constexpr int BP = N + 8;  // LDS pitch of a B row / H row (bf16): 16-byte aligned, bank-spread
   constexpr int XP = 40;     // LDS pitch of an X^T row (32 k values + pad)
-  constexpr int YP = P + 8;  // fp32 pitch of the epilogue's per-wave transpose patch
+  constexpr int YP = P + 4;  // fp32 pitch of the epilogue's per-wave transpose patch (rows 4 banks apart)
   struct Stage {
     uint16_t Bs[2][32 * BP];
     uint16_t Xs[2][P * XP];
@@ -117,9 +117,10 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
     if (tid < XTASKS) {
       const int q4 = tid / (P / 8), p8 = tid % (P / 8);
       // k slots of positions 4 q4 .. 4 q4 + 3 inside the 32-block: the second MFMA's lane group gq
-      // holds positions 4 gq .. 4 gq + 3 of both 16-tiles.  The 8-element group is XOR-swizzled
-      // with p8 so that the transposing stores spread over the banks.
-      const int pos = (((q4 & 3) ^ (p8 & 3)) << 3) + ((q4 >> 2) << 2);
+      // holds positions 4 gq .. 4 gq + 3 of both 16-tiles.  The 8-element group is XOR-swizzled with the
+      // row's 16-tile index: the stores spread over the banks, and the 16 rows a quarter wave reads
+      // together share one swizzle, so their 16-byte pieces fall into 16 different bank groups.
+      const int pos = (((q4 & 3) ^ ((p8 >> 1) & 3)) << 3) + ((q4 >> 2) << 2);
       const uint32_t w[4][4] = {{xreg.v[0].x, xreg.v[0].y, xreg.v[0].z, xreg.v[0].w},
                                 {xreg.v[1].x, xreg.v[1].y, xreg.v[1].z, xreg.v[1].w},
                                 {xreg.v[2].x, xreg.v[2].y, xreg.v[2].z, xreg.v[2].w},
@@ -288,8 +289,7 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
       const bf16x8_t Mf = __builtin_bit_cast(bf16x8_t, mp);
 #pragma unroll
       for (int pt = 0; pt < PT; ++pt)
-        acc[k][pt] = mfma_bf16(ld_frag(&Xs[buf][(pt * 16 + j) * XP + ((g ^ ((pt * 2 + (j >> 3)) & 3)) << 3)]), Mf,
-                               acc[k][pt]);
+        acc[k][pt] = mfma_bf16(ld_frag(&Xs[buf][(pt * 16 + j) * XP + ((g ^ (pt & 3)) << 3)]), Mf, acc[k][pt]);
     }
     if (sb + 1 < nsb) store_block(buf ^ 1, bregs[(sb + 1) & 1], xregs[(sb + 1) & 1]);
     __syncthreads();
