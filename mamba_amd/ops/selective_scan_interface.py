@@ -348,11 +348,10 @@ def _causal_conv1d_silu(x, weight, bias):
 
 
 def _rms_norm(x, weight, eps):
-    """x * rsqrt(mean(x^2) + eps) * weight over the last dimension (the forward of the reference's
-    rms_norm_forward, selective_scan_interface.py:98-115), in fp32, cast back to x's dtype."""
-    xf = x.float()
-    y = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
-    return y.to(x.dtype)
+    """x * rsqrt(mean(x^2) + eps) * weight over the last dimension of contiguous rows: the reference's
+    rms_norm_forward (selective_scan_interface.py:98-115), on the HIP norm kernel."""
+    from mamba_amd.ops.triton.layer_norm import _layer_norm_fwd
+    return _layer_norm_fwd(x, weight, None, eps, is_rms_norm=True)[0]
 
 
 def _norm_over_state(t, weight, eps, L):

@@ -15,9 +15,14 @@ from oracle.mamba1 import selective_scan_oracle
 
 def mamba_inner_oracle(xz, conv1d_weight, conv1d_bias, x_proj_weight, delta_proj_weight, out_proj_weight,
                        out_proj_bias, A, D=None, delta_bias=None, B_proj_bias=None, C_proj_bias=None,
-                       compute_dtype=torch.float32, B=None, C=None):
+                       compute_dtype=torch.float32, B=None, C=None, b_rms_weight=None, c_rms_weight=None,
+                       dt_rms_weight=None, b_c_dt_rms_eps=1e-6):
     """B / C given: input-independent (dim, dstate) matrices instead of the x_proj slices (:415-430);
-    x_proj_weight then only carries the rows of the slices that are still projected."""
+    x_proj_weight then only carries the rows of the slices that are still projected.
+    b / c / dt_rms_weight: RMSNorm of the projected B and C rows over the states and of delta over the
+    channels before the scan (MambaInnerFn.forward, :263-274).  The reference's backward pass treats these
+    norms as the identity (it hands the scan's dB / dC / ddelta straight to the projections and returns no
+    gradient for the norm weights, :283-383), so they are written here with a straight-through gradient."""
     cd = compute_dtype
     batch, two_d, L = xz.shape
     d = two_d // 2
@@ -49,6 +54,16 @@ def mamba_inner_oracle(xz, conv1d_weight, conv1d_bias, x_proj_weight, delta_proj
         Cm = pack(Cm)
     else:
         Cm = C if C.is_complex() else C.to(cd)
+    def rms_st(t, w, dim):  # value of the norm, gradient of the identity
+        n = t * torch.rsqrt(t.pow(2).mean(dim, keepdim=True) + b_c_dt_rms_eps) * w
+        return t + (n - t).detach()
+
+    if b_rms_weight is not None:
+        Bm = rms_st(Bm, b_rms_weight.to(cd)[None, :, None], 1)
+    if c_rms_weight is not None:
+        Cm = rms_st(Cm, c_rms_weight.to(cd)[None, :, None], 1)
+    if dt_rms_weight is not None:
+        delta = rms_st(delta, dt_rms_weight.to(cd)[None, :, None], 1)
     y = selective_scan_oracle(x, delta, A if A.is_complex() else A.to(cd), Bm, Cm, None if D is None else D.to(cd), z,
                               None if delta_bias is None else delta_bias.to(cd), True, compute_dtype=cd)
     out = y.permute(0, 2, 1) @ out_proj_weight.to(cd).t()

@@ -142,3 +142,38 @@ def test_install_as_mamba_ssm_ops():
     from mamba_ssm.ops.triton.ssd_combined import mamba_chunk_scan_combined  # noqa: F401
     from mamba_ssm.ops.triton.selective_state_update import selective_state_update  # noqa: F401
     assert m.selective_scan_fn.__module__.startswith("mamba_amd")
+
+
+@pytest.mark.parametrize("which", ["b", "c", "dt", "all"])
+def test_mamba_inner_fn_rms_norms(which):
+    """b / c / dt_rms_weight (selective_scan_interface.py:263-274): the value of the norms in the forward pass;
+    in the backward pass the reference hands gradients straight through them, and so do the oracle and this."""
+    from mamba_amd.ops.selective_scan_interface import mamba_inner_fn
+    g = torch.Generator().manual_seed(4)
+    batch, dim, dstate, dt_rank, d_model, L = 2, 128, 8, 16, 96, 200
+    p = _params(batch, dim, L, dstate, dt_rank, d_model, g, False)
+    rms = dict(b_rms_weight=1 + 0.2 * torch.randn(dstate, generator=g) if which in ("b", "all") else None,
+               c_rms_weight=1 + 0.2 * torch.randn(dstate, generator=g) if which in ("c", "all") else None,
+               dt_rms_weight=0.3 + 0.1 * torch.rand(dim, generator=g) if which in ("dt", "all") else None)
+    ref_in = {k: (v.clone().requires_grad_() if v is not None else None) for k, v in p.items()}
+    gpu_in = {k: (v.cuda().requires_grad_() if v is not None else None) for k, v in p.items()}
+    order = ["xz", "conv1d_weight", "conv1d_bias", "x_proj_weight", "delta_proj_weight", "out_proj_weight",
+             "out_proj_bias", "A"]
+    out_ref = mamba_inner_oracle(*[ref_in[k] for k in order], D=ref_in["D"], delta_bias=ref_in["delta_bias"],
+                                 b_c_dt_rms_eps=1e-5, **rms)
+    out = mamba_inner_fn(*[gpu_in[k] for k in order], None, None, gpu_in["D"], delta_bias=gpu_in["delta_bias"],
+                         delta_softplus=True, b_c_dt_rms_eps=1e-5,
+                         **{k: (v.cuda() if v is not None else None) for k, v in rms.items()})
+    scale = float(out_ref.abs().max())
+    assert torch.allclose(out.cpu(), out_ref, rtol=6e-4, atol=2e-3 * max(1.0, scale)), \
+        f"max err {(out.cpu() - out_ref).abs().max().item():.3e} (scale {scale:.2e})"
+    dout = torch.randn(out_ref.shape, generator=g)
+    out_ref.backward(dout)
+    out.backward(dout.cuda())
+    for k, v in ref_in.items():
+        if v is None:
+            continue
+        got, ref = gpu_in[k].grad.cpu(), v.grad
+        s = max(1.0, float(ref.abs().max()))
+        assert torch.allclose(got, ref, rtol=5e-3, atol=5e-3 * s), \
+            f"d{k}: max err {(got - ref).abs().max().item():.3e}, ref max {ref.abs().max().item():.3e}"

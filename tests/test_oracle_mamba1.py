@@ -187,3 +187,47 @@ def test_complex_A_brute_force_rotation_and_gradcheck():
     assert abs(complex(hl[0, 0, 0]) - cmath.exp(1j * 5 * 0.7)) < 1e-12   # unit modulus, phase 5 steps x 0.7
     ins = [t.clone().requires_grad_() for t in (u[:1, :, :5], delta[:1, :, :5], A, Bv[:1, :, :, :10], Cm)]
     assert torch.autograd.gradcheck(lambda *a: selective_scan_oracle(*a, compute_dtype=f64), ins, atol=1e-6)
+
+
+def test_inner_oracle_rms_options_against_library_norm_and_straight_through_gradient():
+    """mamba_inner_oracle's b / c / dt RMSNorms: values against F.rms_norm applied by hand between the same
+    stages, gradients as the reference's backward pass has them (identity through the norms, none for their
+    weights)."""
+    import torch.nn.functional as F
+    from oracle.inner import mamba_inner_oracle
+    g = torch.Generator().manual_seed(3)
+    r = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64)
+    batch, d, L, N, R, dm = 2, 6, 11, 4, 3, 5
+    xz, cw, cb = r(batch, 2 * d, L), r(d, 1, 3), r(d)
+    xp, dp, op = r(R + 2 * N, d) * 0.5, r(d, R) * 0.5, r(dm, d)
+    A, D, dbias = -torch.rand(d, N, generator=g, dtype=torch.float64), r(d), r(d) * 0.3
+    wb, wc, wdt = 1 + 0.3 * r(N), 1 + 0.3 * r(N), 0.5 + torch.rand(d, generator=g, dtype=torch.float64)
+    kw = dict(D=D, delta_bias=dbias, compute_dtype=torch.float64)
+    got = mamba_inner_oracle(xz, cw, cb, xp, dp, op, None, A, b_rms_weight=wb, c_rms_weight=wc, dt_rms_weight=wdt,
+                             b_c_dt_rms_eps=1e-5, **kw)
+    # by hand: the same stages with the library norm in between
+    x, z = xz[:, :d], xz[:, d:]
+    xc = F.silu(F.conv1d(x, cw, cb, padding=2, groups=d)[..., :L])
+    x_dbl = xc.permute(0, 2, 1).reshape(batch * L, d) @ xp.t()
+    delta = (dp @ x_dbl[:, :R].t()).reshape(d, batch, L).permute(1, 2, 0)            # (b, l, d)
+    delta = F.rms_norm(delta, (d,), wdt, 1e-5).permute(0, 2, 1)
+    Bm = F.rms_norm(x_dbl[:, R:R + N], (N,), wb, 1e-5).reshape(batch, L, N).permute(0, 2, 1)
+    Cm = F.rms_norm(x_dbl[:, R + N:], (N,), wc, 1e-5).reshape(batch, L, N).permute(0, 2, 1)
+    y = selective_scan_oracle(xc, delta, A, Bm, Cm, D, z, dbias, True, compute_dtype=torch.float64)
+    assert torch.allclose(got, y.permute(0, 2, 1) @ op.t(), atol=1e-10)
+    # straight-through: the gradient equals that of a run whose norms are frozen multipliers
+    xp1 = xp.clone().requires_grad_()
+    wb1 = wb.clone().requires_grad_()
+    out = mamba_inner_oracle(xz, cw, cb, xp1, dp, op, None, A, b_rms_weight=wb1, b_c_dt_rms_eps=1e-5, **kw)
+    out.sum().backward()
+    assert wb1.grad is None or float(wb1.grad.abs().max()) == 0.0
+    xp2 = xp.clone().requires_grad_()
+    x_dbl2 = xc.permute(0, 2, 1).reshape(batch * L, d) @ xp2.t()
+    Braw = x_dbl2[:, R:R + N]
+    Bst = Braw + (F.rms_norm(Braw, (N,), wb, 1e-5) - Braw).detach()
+    delta2 = (dp @ x_dbl2[:, :R].t()).reshape(d, batch, L).permute(1, 0, 2)
+    y2 = selective_scan_oracle(xc, delta2, A, Bst.reshape(batch, L, N).permute(0, 2, 1),
+                               x_dbl2[:, R + N:].reshape(batch, L, N).permute(0, 2, 1), D, z, dbias, True,
+                               compute_dtype=torch.float64)
+    (y2.permute(0, 2, 1) @ op.t()).sum().backward()
+    assert torch.allclose(xp1.grad, xp2.grad, atol=1e-9)
