@@ -218,3 +218,9 @@ def test_ssd_varlen_states(seq_lens, dtype):
         cu_seqlens=cu_seqlens.cuda(), dt_softplus=True, return_varlen_states=True, state_dtype=torch.float32)
     assert varlen2.dtype == torch.float32 and torch.equal(out, out2)
     _close("varlen_states fp32", varlen2, ref, rtol, atol)
+
+
+@pytest.mark.parametrize("seqlen,chunk", [(300, 64), (512, 256)])
+def test_ssd_bwd_fp16(seqlen, chunk):
+    _bwd_case(2, seqlen, 4, 64, 64, 2, chunk, torch.float16, has_init=True, seed=12)
+    _bwd_case(1, seqlen, 2, 32, 128, 1, chunk, torch.float16, seq_lens=[seqlen // 3, seqlen - seqlen // 3], seed=13)
