@@ -94,8 +94,15 @@ def _layer_norm_fwd(x, weight, bias, eps, z=None, out=None, group_size=None, nor
 
 
 def _layer_norm_bwd(dy, x, weight, bias, eps, mean, rstd, z=None, group_size=None, norm_before_gate=True,
-                    is_rms_norm=False, dz=None):
-    """Returns (dx, dweight, dbias, dz); dweight / dbias in the dtype of weight / bias."""
+                    is_rms_norm=False, recompute_output=False, dz=None, out=None):
+    """Returns (dx, dweight, dbias, dz), plus the forward output with recompute_output (a second launch of the
+    forward kernel here; the reference's backward kernel writes it on the side, layernorm_gated.py:271);
+    dweight / dbias in the dtype of weight / bias."""
+    if recompute_output:
+        y = _layer_norm_fwd(x, weight, bias, eps, z=z, out=out, group_size=group_size,
+                            norm_before_gate=norm_before_gate, is_rms_norm=is_rms_norm)[0]
+        return (*_layer_norm_bwd(dy, x, weight, bias, eps, mean, rstd, z, group_size, norm_before_gate, is_rms_norm,
+                                 False, dz), y)
     group_size = _check(x, weight, bias, z, group_size)
     _lib.require_gpu(dy, rstd, mean)
     M, N = x.shape

@@ -118,3 +118,16 @@ def test_module_and_empty():
     assert xe.grad.shape == (0, 9, 256) and float(we.grad.abs().max()) == 0.0
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         rmsnorm_fn(x.cpu(), m.weight.cpu(), None)
+
+
+def test_backward_with_recomputed_output():
+    from mamba_amd.ops.triton.layernorm_gated import _layer_norm_bwd, _layer_norm_fwd
+    g = torch.Generator().manual_seed(9)
+    x, z, dy = (torch.randn(37, 256, generator=g).cuda() for _ in range(3))
+    w = (1 + 0.1 * torch.randn(256, generator=g)).cuda()
+    y, _, rstd = _layer_norm_fwd(x, w, None, 1e-5, z=z, group_size=64, norm_before_gate=False, is_rms_norm=True)
+    plain = _layer_norm_bwd(dy, x, w, None, 1e-5, None, rstd, z, 64, False, True)
+    again = _layer_norm_bwd(dy, x, w, None, 1e-5, None, rstd, z, 64, False, True, recompute_output=True)
+    assert len(again) == 5 and torch.equal(again[4], y)
+    for a, b in zip(plain, again[:4]):
+        assert (a is None and b is None) or torch.equal(a, b)
