@@ -347,11 +347,18 @@ def _causal_conv1d_silu(x, weight, bias):
     return F.silu(y)
 
 
-def _rms_norm(x, weight, eps):
-    """x * rsqrt(mean(x^2) + eps) * weight over the last dimension of contiguous rows: the reference's
-    rms_norm_forward (selective_scan_interface.py:98-115), on the HIP norm kernel."""
+def rms_norm_forward(x, weight, bias, eps=1e-6, is_rms_norm=True):
+    """RMSNorm (or LayerNorm) of the rows of x, (rows, dim), on the HIP norm kernel; no autograd
+    (selective_scan_interface.py:98-115)."""
     from mamba_amd.ops.triton.layer_norm import _layer_norm_fwd
-    return _layer_norm_fwd(x, weight, None, eps, is_rms_norm=True)[0]
+    if x.stride(-1) != 1:
+        x = x.contiguous()
+    return _layer_norm_fwd(x, weight.contiguous(), bias.contiguous() if bias is not None else None, eps,
+                           is_rms_norm=is_rms_norm)[0]
+
+
+def _rms_norm(x, weight, eps):
+    return rms_norm_forward(x, weight, None, eps)
 
 
 def _norm_over_state(t, weight, eps, L):

@@ -226,6 +226,17 @@ class RMSNorm(torch.nn.Module):
                            residual_in_fp32=residual_in_fp32)
 
 
+class LayerNormLinearFn:
+    """Name of the reference's fused autograd function (layer_norm.py:985); `apply` takes its arguments in
+    the same order and chains LayerNormFn with a torch GEMM."""
+
+    @staticmethod
+    def apply(x, norm_weight, norm_bias, linear_weight, linear_bias, residual=None, eps=1e-6, prenorm=False,
+              residual_in_fp32=False, is_rms_norm=False):
+        return layer_norm_linear_fn(x, norm_weight, norm_bias, linear_weight, linear_bias, residual, eps, prenorm,
+                                    residual_in_fp32, is_rms_norm)
+
+
 def layer_norm_linear_fn(x, norm_weight, norm_bias, linear_weight, linear_bias, residual=None, eps=1e-6,
                          prenorm=False, residual_in_fp32=False, is_rms_norm=False):
     """Norm on the HIP kernels followed by a torch GEMM (layer_norm.py:1092 keeps only the norm's input
