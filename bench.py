@@ -68,8 +68,9 @@ def cpu_baseline(seqlen, dstate, full_dim):
                       f"{dt:.1f} s, scaled by {dim}/{full_dim}"}
 
 
-def copy_calibration(dev):
-    """Runs mamba_hip_copy (one 16-byte element per thread) over 1 GiB: 1 GiB read + 1 GiB written."""
+def measured_copy(dev):
+    """Runs mamba_hip_copy (one 16-byte element per thread) over 1 GiB: 1 GiB read + 1 GiB written.
+    Returns (ms per launch, GB/s): the streaming rate this GPU sustains, beside the published peak."""
     import torch
     from mamba_amd import _lib
     nbytes = 1 << 30
@@ -85,8 +86,41 @@ def copy_calibration(dev):
     ev[1].record()
     torch.cuda.synchronize()
     ms = ev[0].elapsed_time(ev[1]) / 5
-    print(json.dumps({"kernel": "copy_kernel", "bytes_read": nbytes, "bytes_written": nbytes, "ms": ms,
-                      "GB/s": 2 * nbytes / ms / 1e6}))
+    return ms, 2 * nbytes / ms / 1e6
+
+
+def copy_calibration(dev):
+    ms, gbs = measured_copy(dev)
+    print(json.dumps({"kernel": "copy_kernel", "bytes_read": 1 << 30, "bytes_written": 1 << 30, "ms": ms, "GB/s": gbs}))
+
+
+def measured_mfma(dev):
+    """TFLOP/s of mamba_hip_mfma_probe: independent bf16 MFMA chains on register operands, 8 workgroups per CU."""
+    import torch
+    from mamba_amd import _lib
+    lib = _lib.load()
+    stream = _lib.current_stream(dev)
+    sink = torch.zeros(1, device=dev)
+    blocks = 8 * torch.cuda.get_device_properties(dev).multi_processor_count
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    flops = 0
+    for i in range(4):
+        if i == 1:
+            ev[0].record()
+        flops = lib.mamba_hip_mfma_probe(sink.data_ptr(), 4096, blocks, stream)
+        if flops <= 0:
+            _lib.check(int(flops), "mamba_hip_mfma_probe")
+    ev[1].record()
+    torch.cuda.synchronize()
+    return flops / (ev[0].elapsed_time(ev[1]) / 3) / 1e9
+
+
+def vs_measured_copy(roofline, dev):
+    """Adds the streaming-copy rate measured in this run and the kernel's fraction of it."""
+    _, gbs = measured_copy(dev)
+    roofline["measured_copy_gbs"] = gbs
+    roofline["frac_of_measured_copy"] = roofline["achieved"] / gbs
+    return roofline
 
 
 def event_ms(fn, n, pre=None):
@@ -159,6 +193,7 @@ def bench_ssd(dev, steps, warmup):
         scan_ms = event_ms(lambda: _lib.check(lib.ssd_chunk_scan_fwd_fused(p, stream), "ssd_chunk_scan_fwd_fused"),
                            max(5, min(steps, 50)))
     nc = L // Q
+    mfma_tflops = measured_mfma(dev)
     flops = batch * nc * (H * (Q * Q * P + 2 * Q * N * P) + G * Q * Q * N)   # causal halves counted once
     nbytes = 2 * (4 * batch * L * H * P + 2 * batch * L * G * N) + 4 * batch * nc * H * P * N  # x z out out_x B C states
     print(json.dumps({
@@ -167,11 +202,13 @@ def bench_ssd(dev, steps, warmup):
         "fwd_ms": fwd_ms, "higher_is_better": True, "dtype": "bf16 in/out, fp32 accumulation", "data": "synthetic",
         "config": {"workload": f"Mamba-2 SSD fwd+bwd: batch {batch}, seqlen {L}, {H} heads x {P}, d_state {N}, "
                                f"{G} group, chunk {Q}, bf16 (benchmark configuration 2)"},
-        "roofline": {"bound": "hbm", "kernel": "chunk_scan_fwd_fused_kernel", "achieved": nbytes / scan_ms / 1e6,
+        "roofline": vs_measured_copy({"bound": "hbm", "kernel": "chunk_scan_fwd_fused_kernel", "achieved": nbytes / scan_ms / 1e6,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / scan_ms / 1e6 / HBM_PEAK_GBS,
                      "traffic": TRAFFIC["chunk_scan_fwd_fused_kernel"], "kernel_ms": scan_ms, "algorithmic_bytes": nbytes,
                      "algorithmic_flops": flops, "mfma_tflops": flops / scan_ms / 1e9,
-                     "mfma_frac_of_bf16_peak": flops / scan_ms / 1e9 / 2500.0}}))
+                     "mfma_frac_of_bf16_peak": flops / scan_ms / 1e9 / 2500.0,
+                     "measured_mfma_tflops": mfma_tflops,
+                     "mfma_frac_of_measured": flops / scan_ms / 1e9 / mfma_tflops}, dev)}))
 
 
 def bench_decode(dev, steps, warmup):
@@ -200,10 +237,10 @@ def bench_decode(dev, steps, warmup):
         "dtype": "fp32 state, bf16 x/z/B/C/dt", "data": "synthetic",
         "config": {"workload": f"selective_state_update: batch {batch}, {H} heads x {P}, d_state {N}, {G} group, "
                                "tied A/dt/D per head (benchmark configuration 3)"},
-        "roofline": {"bound": "hbm", "kernel": "state_update_kernel", "achieved": nbytes / ms / 1e6,
+        "roofline": vs_measured_copy({"bound": "hbm", "kernel": "state_update_kernel", "achieved": nbytes / ms / 1e6,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / ms / 1e6 / HBM_PEAK_GBS,
                      "traffic": TRAFFIC["state_update_kernel"],
-                     "kernel_ms": ms, "algorithmic_bytes": nbytes}}))
+                     "kernel_ms": ms, "algorithmic_bytes": nbytes}, dev)}))
 
 
 def _timed(step, steps, warmup):
@@ -260,9 +297,9 @@ def bench_varlen(dev, steps, warmup):
         "fwd_ms": fwd_ms, "higher_is_better": True, "dtype": "bf16 in/out, fp32 accumulation", "data": "synthetic",
         "config": {"workload": f"Mamba-2 SSD fwd+bwd, packed: 1 row of {nseq} sequences, {L} positions, {H} heads x {P}, "
                                f"d_state {N}, {G} groups, chunk {Q}, initial + final states (benchmark configuration 4)"},
-        "roofline": {"bound": "hbm", "kernel": "whole step", "achieved": nbytes / sec / 1e9, "peak": HBM_PEAK_GBS,
+        "roofline": vs_measured_copy({"bound": "hbm", "kernel": "whole step", "achieved": nbytes / sec / 1e9, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": nbytes / sec / 1e9 / HBM_PEAK_GBS, "traffic": None,
-                     "algorithmic_bytes": nbytes}}))
+                     "algorithmic_bytes": nbytes}, dev)}))
 
 
 def bench_inner(dev, steps, warmup):
@@ -309,9 +346,9 @@ def bench_inner(dev, steps, warmup):
         "higher_is_better": True, "dtype": "bf16 in/out, fp32 state and accumulation", "data": "synthetic",
         "config": {"workload": f"mamba_inner_fn fwd+bwd: batch {batch}, seqlen {L}, d_model {dm}, d_inner {di}, "
                                f"d_state {N}, dt_rank {R}, conv width {W}"},
-        "roofline": {"bound": "hbm", "kernel": "conv_rows_fwd_kernel", "achieved": nbytes / conv_ms / 1e6,
+        "roofline": vs_measured_copy({"bound": "hbm", "kernel": "conv_rows_fwd_kernel", "achieved": nbytes / conv_ms / 1e6,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / conv_ms / 1e6 / HBM_PEAK_GBS,
-                     "traffic": None, "kernel_ms": conv_ms, "algorithmic_bytes": nbytes}}))
+                     "traffic": None, "kernel_ms": conv_ms, "algorithmic_bytes": nbytes}, dev)}))
 
 
 def bench_block(dev, steps, warmup):
@@ -360,9 +397,9 @@ def bench_block(dev, steps, warmup):
         "higher_is_better": True, "dtype": "bf16 in/out, fp32 accumulation", "data": "synthetic",
         "config": {"workload": f"Mamba-2 block body fwd+bwd: batch {batch}, seqlen {L}, {H} heads x {P}, d_state {N}, "
                                f"{G} group, chunk {Q}, conv width {W}, gated RMSNorm, out_proj to {dm}"},
-        "roofline": {"bound": "hbm", "kernel": "norm_fwd_kernel", "achieved": nbytes / norm_ms / 1e6,
+        "roofline": vs_measured_copy({"bound": "hbm", "kernel": "norm_fwd_kernel", "achieved": nbytes / norm_ms / 1e6,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / norm_ms / 1e6 / HBM_PEAK_GBS,
-                     "traffic": None, "kernel_ms": norm_ms, "algorithmic_bytes": nbytes}}))
+                     "traffic": None, "kernel_ms": norm_ms, "algorithmic_bytes": nbytes}, dev)}))
 
 
 def main():
@@ -452,6 +489,7 @@ def main():
                 "kernel_ms": bwd_ms, "algorithmic_bytes": bwd_bytes,
                 "fwd_kernel_ms": fwd_ms, "fwd_achieved": fwd_bytes / (fwd_ms * 1e-3) / 1e9,
                 "fwd_bwd_frac": (fwd_bytes + bwd_bytes) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    vs_measured_copy(roofline, dev)
 
     result = {
         "metric": "scan fwd+bwd tokens/s at 1 GPU; achieved HBM GB/s and % bf16 MFMA peak",

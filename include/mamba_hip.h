@@ -53,6 +53,12 @@ int mamba_hip_zero(void *ptr, int64_t nbytes, mamba_stream_t stream);
  * traffic is exactly 2 * nbytes. */
 int mamba_hip_copy(void *dst, const void *src, int64_t nbytes, mamba_stream_t stream);
 
+/* Measurement yardstick for the GEMM kernels: launches `blocks` workgroups of 4 waves, each wave running
+ * `iters` rounds of eight independent v_mfma_f32_16x16x32_bf16 on register operands (no LDS, no memory).
+ * Returns the floating-point operations of the launch (> 0), or an error code (< 0).  `sink` is one float
+ * of device memory that is never written. */
+int64_t mamba_hip_mfma_probe(float *sink, int iters, int blocks, mamba_stream_t stream);
+
 /* ------------------------------------------------------------------------- *
  * Mamba-1 selective scan.
  * Replaces selective_scan_cuda.fwd / .bwd

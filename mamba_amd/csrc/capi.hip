@@ -11,7 +11,35 @@ __global__ __launch_bounds__(256) void copy_kernel(const u32x4 *__restrict__ src
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i < n) dst[i] = src[i];
 }
+// Eight independent chains of v_mfma_f32_16x16x32_bf16 per wave on register operands: the rate the matrix
+// cores sustain with nothing else in the way (no LDS, no memory), as a yardstick for the GEMM kernels.
+typedef __bf16 probe_bf16x8 __attribute__((ext_vector_type(8)));
+__global__ __launch_bounds__(256) void mfma_probe_kernel(float *sink, int iters) {
+  const int lane = threadIdx.x & 63;
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  const s16x8 ai = {(short)(0x3f80 + lane), 0x3f80, 0x3f00, 0x3e80, 0x3f80, 0x3f00, 0x3e80, 0x3f80};
+  const s16x8 bi = {0x3f80, (short)(0x3f00 + lane), 0x3f80, 0x3e80, 0x3f00, 0x3f80, 0x3e80, 0x3f00};
+  const probe_bf16x8 a = __builtin_bit_cast(probe_bf16x8, ai), b = __builtin_bit_cast(probe_bf16x8, bi);
+  f32x4 acc[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[j], 0, 0, 0);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) s += acc[j].x + acc[j].y + acc[j].z + acc[j].w;
+  if (s == -1.f) sink[0] = s;  // never true: keeps the loop alive
+}
 }  // namespace
+
+extern "C" int64_t mamba_hip_mfma_probe(float *sink, int iters, int blocks, mamba_stream_t stream) {
+  if (!sink || iters <= 0 || blocks <= 0) return MAMBA_E_BADARG;
+  hipLaunchKernelGGL(mfma_probe_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), sink, iters);
+  if (hipGetLastError() != hipSuccess) return MAMBA_E_LAUNCH;
+  return (int64_t)blocks * 4 * iters * 8 * (2LL * 16 * 16 * 32);  // flops of this launch
+}
 
 extern "C" int mamba_hip_copy(void *dst, const void *src, int64_t nbytes, mamba_stream_t stream) {
   if (nbytes == 0) return MAMBA_OK;

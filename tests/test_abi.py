@@ -19,7 +19,7 @@ HEADER = os.path.join(ROOT, "include", "mamba_hip.h")
 def _declared_functions():
     src = open(HEADER).read()
     src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
-    return sorted(set(re.findall(r"^\s*(?:const\s+char\s*\*|int)\s*(\w+)\s*\(", src, flags=re.M)))
+    return sorted(set(re.findall(r"^\s*(?:const\s+char\s*\*|int64_t|int)\s*(\w+)\s*\(", src, flags=re.M)))
 
 
 def test_library_exports_every_declared_symbol():
