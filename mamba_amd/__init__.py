@@ -15,7 +15,8 @@ def install_as_mamba_ssm_ops(causal_conv1d=True):
     mamba_ssm/modules/mamba_simple.py:15-18) resolves to this package's convolution as well, so those
     modules take their fused paths instead of falling back to nn.Conv1d."""
     from mamba_amd.ops import selective_scan_interface
-    from mamba_amd.ops.triton import layer_norm, layernorm_gated, selective_state_update, ssd_combined
+    from mamba_amd.ops.triton import (layer_norm, layernorm_gated, selective_state_update, ssd_bmm, ssd_chunk_scan,
+                                      ssd_chunk_state, ssd_combined, ssd_state_passing)
 
     def ensure(name):
         if name not in sys.modules:
@@ -29,6 +30,10 @@ def install_as_mamba_ssm_ops(causal_conv1d=True):
     mapping = {
         "mamba_ssm.ops.selective_scan_interface": selective_scan_interface,
         "mamba_ssm.ops.triton.ssd_combined": ssd_combined,
+        "mamba_ssm.ops.triton.ssd_chunk_state": ssd_chunk_state,
+        "mamba_ssm.ops.triton.ssd_state_passing": ssd_state_passing,
+        "mamba_ssm.ops.triton.ssd_bmm": ssd_bmm,
+        "mamba_ssm.ops.triton.ssd_chunk_scan": ssd_chunk_scan,
         "mamba_ssm.ops.triton.selective_state_update": selective_state_update,
         "mamba_ssm.ops.triton.layernorm_gated": layernorm_gated,
         "mamba_ssm.ops.triton.layer_norm": layer_norm,
