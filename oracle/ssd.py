@@ -28,9 +28,10 @@ def dt_pipeline(dt, dt_bias=None, dt_softplus=False, dt_limit=(0.0, float("inf")
         dt = dt + dt_bias.to(compute_dtype)
     if dt_softplus:
         dt = F.softplus(dt)
-    if dt_limit != (0.0, float("inf")):
-        dt = dt.clamp(min=dt_limit[0], max=dt_limit[1])
-    return dt
+    # The reference's kernel clamps even at the default limits (0, inf), so a negative dt without softplus
+    # becomes 0 (ssd_chunk_state.py:80); its torch reference (ssd_combined.py:706-710) has no clamp.
+    # The kernel's behaviour is the one restated here.
+    return dt.clamp(min=dt_limit[0], max=dt_limit[1])
 
 
 def ssd_oracle(x, dt, A, B, C, D=None, z=None, dt_bias=None, initial_states=None, seq_idx=None,

@@ -224,3 +224,26 @@ def test_ssd_varlen_states(seq_lens, dtype):
 def test_ssd_bwd_fp16(seqlen, chunk):
     _bwd_case(2, seqlen, 4, 64, 64, 2, chunk, torch.float16, has_init=True, seed=12)
     _bwd_case(1, seqlen, 2, 32, 128, 1, chunk, torch.float16, seq_lens=[seqlen // 3, seqlen - seqlen // 3], seed=13)
+
+
+def test_ssd_negative_dt_without_softplus_is_clamped():
+    """Without softplus a raw dt can be negative; the reference's kernels clamp it to dt_limit's lower bound 0
+    (ssd_chunk_state.py:80) and pass no gradient through the clamped positions (ssd_chunk_state.py:147-160)."""
+    from mamba_amd.ops.triton.ssd_combined import mamba_chunk_scan_combined
+    t = ssd_inputs(2, 200, 4, 32, 64, 2, torch.float32, seed=21)
+    t["dt"] = 0.05 * torch.randn(2, 200, 4, generator=torch.Generator().manual_seed(1))
+    assert 0.3 < (t["dt"] < 0).float().mean() < 0.7
+    names = ["x", "dt", "A", "B", "C", "D", "z"]
+    ref_in = {k: t[k].clone().requires_grad_() for k in names}
+    gpu_in = {k: t[k].cuda().requires_grad_() for k in names}
+    out_ref = ssd_oracle(ref_in["x"], ref_in["dt"], ref_in["A"], ref_in["B"], ref_in["C"], D=ref_in["D"], z=ref_in["z"])
+    out = mamba_chunk_scan_combined(gpu_in["x"], gpu_in["dt"], gpu_in["A"], gpu_in["B"], gpu_in["C"], 64,
+                                    D=gpu_in["D"], z=gpu_in["z"])
+    rtol, atol = _tol(torch.float32)
+    _close("out", out, out_ref, rtol, atol)
+    (out_ref * t["dout"]).sum().backward()
+    (out * t["dout"].cuda()).sum().backward()
+    assert bool((gpu_in["dt"].grad[gpu_in["dt"] < 0] == 0).all())
+    for k in names:
+        scale = max(1.0, float(ref_in[k].grad.abs().max())) if k in ("A", "D", "dt") else 1.0
+        _close("d" + k, gpu_in[k].grad, ref_in[k].grad, rtol * 2, atol * 2 * scale)
