@@ -443,8 +443,9 @@ class MambaInnerFn(torch.autograd.Function):
         if dt_rms_weight is not None:
             delta = rearrange(_rms_norm(rearrange(delta, "b d l -> (b l) d").contiguous(), dt_rms_weight,
                                         b_c_dt_rms_eps), "(b l) d -> b d l", l=L).contiguous()
+        keep = _keep_lane_states(conv1d_out, A) and any(ctx.needs_input_grad)
         out_z, ckpt, lanes = selective_scan_fwd(conv1d_out, delta, A, B, C, D, z, delta_bias, delta_softplus,
-                                                lane_states=_keep_lane_states(conv1d_out, A))
+                                                lane_states=keep)
         ctx.delta_softplus = delta_softplus
         ctx.out_proj_bias_is_None = out_proj_bias is None
         ctx.checkpoint_lvl = checkpoint_lvl
