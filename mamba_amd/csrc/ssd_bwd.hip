@@ -723,6 +723,119 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dB_
     }
 }
 
+// The dC product alone with a 64 x 128 tile per workgroup (same conditions, aligned g rows); the row sums
+// of the tile against C after each head give the heads' ddA_cumsum rows.
+template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_dC_state_wide_kernel(const SsdParams p) {
+  constexpr int MAXH = 8;
+  __shared__ GemmLdsWide<SPLIT> lds;
+  __shared__ float wC[MAXH][GB];
+  __shared__ float dda_s[2][MAXH][GB];  // the running ddA_cumsum row sums after each head, per half of the tile's columns, flushed at the end:
+                                        // a global atomic per head would sit in the memory queue in front of the next loads
+  const int tid = threadIdx.x;
+  const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads, G = p.ngroups;
+  const int ntn = N / WB;
+  const Block3 blk = xcd_block();
+  const int nst = gridDim.x / ntn;
+  const int st = blk.x % nst, nt = blk.x / nst;
+  const int hpg = H / G, nsplit = head_splits(hpg);
+  const int c = blk.y, bg = blk.z / nsplit, hs = blk.z % nsplit, b = bg / G, g = bg % G;
+  const int nh = hs < hpg ? (hpg - hs + nsplit - 1) / nsplit : 0;
+  const int t0 = c * Q, qlim = min(Q, L - t0);
+  if (st * GB >= qlim || nh == 0) return;
+  const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
+  const View4 gv = g_view(p);
+  for (int idx = tid; idx < nh * GB; idx += 256) {
+    const int hl = idx / GB, r = idx % GB, s = st * GB + r, h = g * hpg + hs + hl * nsplit;
+    float vc = 0.f;
+    if (s < qlim) {
+      const bool okc = !seq || seq[s] == (c > 0 ? seq[-1] : 0);
+      if (okc) vc = fast_exp(chunk_row(p.dA_cumsum, p, b, h, c)[s]);
+    }
+    wC[hl][r] = vc;
+  }
+  const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1, i = lane & 15, gq = lane >> 4;
+  // C at this lane's 32 accumulator positions (shared by the heads of the group); 16-bit inputs stay packed in
+  // pairs, which keeps the kernel at four workgroups per CU without spills
+  constexpr bool PK = sizeof(T) == 2;
+  const int64_t Cb = b * p.C_bs + g * p.C_gs;
+  uint32_t crp[2][2][4] = {};
+  float crf[2][4][4];
+#pragma unroll
+  for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int l = st * GB + wm * 32 + tm * 16 + gq * 4 + r;
+#pragma unroll
+      for (int tn = 0; tn < 4; ++tn) {
+        const int64_t at = Cb + (int64_t)(t0 + l) * p.C_ls + nt * WB + wn * 64 + tn * 16 + i;
+        if constexpr (PK) {
+          const uint32_t raw = l < qlim ? (uint32_t) reinterpret_cast<const uint16_t *>(p.C)[at] : 0u;
+          crp[tm][tn >> 1][r] |= raw << (16 * (tn & 1));
+        } else {
+          crf[tm][tn][r] = l < qlim ? ldg<T>(p.C, at) : 0.f;
+        }
+      }
+    }
+  auto cr = [&](int tm, int tn, int r) -> float {
+    if constexpr (PK) {
+      const uint32_t w = crp[tm][tn >> 1][r];
+      if constexpr (DT<T>::id == MAMBA_BF16) return (tn & 1) ? bf16_hi(w) : bf16_lo(w);
+      else return (tn & 1) ? f16_hi(w) : f16_lo(w);
+    } else {
+      return crf[tm][tn][r];
+    }
+  };
+  // One accumulator runs through the heads (at most 8 per workgroup); a head's share of the row sums is the
+  // difference of the running row sums after it and after the head before.
+  GemmAccWide acc;
+  acc.zero();
+  auto sa = seg_stager(KcStager<SPLIT, T>(lds.ah, lds.al, nullptr, gv.ls, qlim - st * GB, P, nullptr, nullptr, true, tid),
+                       [&](KcStager<SPLIT, T> &q, int hl) {
+                         q.base = static_cast<const T *>(gv.ptr) + b * gv.bs + (g * hpg + hs + hl * nsplit) * gv.hs +
+                                  (int64_t)(t0 + st * GB) * gv.ls;
+                         q.rscale = wC[hl];
+                       },
+                       P);
+  auto sb = seg_stager(WideTrStager<SPLIT, float, WB>(lds.bh, lds.bl, nullptr, N, WB, nullptr, tid),
+                       [&](WideTrStager<SPLIT, float, WB> &q, int hl) {
+                         q.base = p.states + (((int64_t)b * p.nchunks + c) * H + g * hpg + hs + hl * nsplit) * P * N + nt * WB;
+                       },
+                       P);
+  block_gemm_wide<SPLIT>(acc, lds, nh * P, sa, sb, tid, [&](int k0) {  // the first barrier inside publishes wC
+    if ((k0 + GK) % P != 0) return;
+    const int hl = k0 / P;
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float rs = 0.f;
+#pragma unroll
+        for (int tn = 0; tn < 4; ++tn) rs = __builtin_fmaf(acc.v[tm][tn][r], cr(tm, tn, r), rs);
+        rs += dpp_f<DPP_ROW_SHR + 1>(0.f, rs);
+        rs += dpp_f<DPP_ROW_SHR + 2>(0.f, rs);
+        rs += dpp_f<DPP_ROW_SHR + 4>(0.f, rs);
+        rs += dpp_f<DPP_ROW_SHR + 8>(0.f, rs);
+        if (i == 15) dda_s[wn][hl][wm * 32 + tm * 16 + gq * 4 + r] = rs;
+      }
+  });
+  __syncthreads();
+  for (int idx = tid; idx < nh * GB; idx += 256) {
+    const int hl = idx / GB, r = idx % GB, l = st * GB + r;
+    const float d = dda_s[0][hl][r] + dda_s[1][hl][r] - (hl > 0 ? dda_s[0][hl - 1][r] + dda_s[1][hl - 1][r] : 0.f);
+    if (l < qlim && d != 0.f) unsafeAtomicAdd(chunk_row(p.ddA_cumsum, p, b, g * hpg + hs + hl * nsplit, c) + l, d);
+  }
+#pragma unroll
+  for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int l = st * GB + wm * 32 + tm * 16 + gq * 4 + r;
+      if (l >= qlim) continue;
+      float *row = p.dC32 + (((int64_t)b * L + t0 + l) * G + g) * N + nt * WB + wn * 64 + i;
+#pragma unroll
+      for (int tn = 0; tn < 4; ++tn) unsafeAtomicAdd(row + tn * 16, acc.v[tm][tn][r]);
+    }
+}
+
 // ------------------------------------------------------------------ dCB
 // dCB[b, c, g, l, s] = sum_{h in group} (sum_p g[l, p] x[s, p]) dt_s exp(a_l - a_s)   for l >= s in
 // one sequence.  One workgroup per (batch, chunk, group, lower-triangular 64 x 64 tile pair) loops
@@ -1078,8 +1191,14 @@ extern "C" int ssd_bwd_dBC_state(const SsdParams *p, mamba_stream_t stream) {
                     wide_operand_ok(p->x, p->dtype, p->x_bs, p->x_ls, p->x_hs);
   if (wide) {
     dim3 gridw(tiles(p->chunk_size) * (p->dstate / WB), p->nchunks, zdim);
+    const bool g_ok = p->z ? (p->headdim % 8 == 0 && reinterpret_cast<uintptr_t>(p->gbuf) % 16 == 0)
+                           : wide_operand_ok(p->dout, p->dtype, p->dout_bs, p->dout_ls, p->dout_hs);
+    if (g_ok) {
+      SSD_DISPATCH(bwd_dC_state_wide_kernel, gridw)
+    } else {
+      SSD_DISPATCH(bwd_dC_state_kernel, grid)
+    }
     SSD_DISPATCH(bwd_dB_state_wide_kernel, gridw)
-    SSD_DISPATCH(bwd_dC_state_kernel, grid)
     return launched();
   }
   SSD_DISPATCH(bwd_dBC_state_kernel, grid)
@@ -1119,8 +1238,10 @@ extern "C" int ssd_combined_bwd(const SsdParams *p, mamba_stream_t stream) {
   if ((rc = ssd_bwd_dz(p, stream))) return rc;
   if ((rc = ssd_bwd_dstates(p, stream))) return rc;
   if ((rc = ssd_state_passing_bwd(p, stream))) return rc;
-  if ((rc = ssd_bwd_dx(p, stream))) return rc;
+  // dC reads the forward states, which the state-passing kernel has just read, and dB and dx the dstates it has just
+  // written: in this order each finds them in the last-level cache
   if ((rc = ssd_bwd_dBC_state(p, stream))) return rc;
+  if ((rc = ssd_bwd_dx(p, stream))) return rc;
   if ((rc = ssd_bwd_dcb(p, stream))) return rc;
   if ((rc = ssd_bmm_chunk_bwd(p, stream))) return rc;
   return ssd_chunk_cumsum_bwd(p, stream);

@@ -374,8 +374,8 @@ template <bool SPLIT, typename S, int ROWS> struct WideTrStager {
 // acc[m][n] += sum_k A[m][k] B[n][k] over k in [0, k_end), k_end a multiple of 32.  The A stager is
 // a 64-row stager of either layout on its fast path, the B stager a 128-row WideTrStager (possibly
 // inside a SegStager).
-template <bool SPLIT, typename SA, typename SB>
-DEVI void block_gemm_wide(GemmAccWide &acc, GemmLdsWide<SPLIT> &s, int k_end, SA &sa, SB &sb, int tid) {
+template <bool SPLIT, typename SA, typename SB, typename AFTER>
+DEVI void block_gemm_wide(GemmAccWide &acc, GemmLdsWide<SPLIT> &s, int k_end, SA &sa, SB &sb, int tid, AFTER after_step) {
   constexpr bool ATR = SA::transposed;
   const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
   const int i = lane & 15, g = lane >> 4;
@@ -409,7 +409,12 @@ DEVI void block_gemm_wide(GemmAccWide &acc, GemmLdsWide<SPLIT> &s, int k_end, SA
           acc.v[tm][tn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al[tm], b[tn], acc.v[tm][tn], 0, 0, 0);
         }
       }
+    after_step(k0);
   }
+}
+template <bool SPLIT, typename SA, typename SB>
+DEVI void block_gemm_wide(GemmAccWide &acc, GemmLdsWide<SPLIT> &s, int k_end, SA &sa, SB &sb, int tid) {
+  block_gemm_wide<SPLIT>(acc, s, k_end, sa, sb, tid, [](int) {});
 }
 
 // Stores the wide tile as fp32 rows of dst (the tile's origin, row pitch ld); rows >= rows_valid are skipped.
