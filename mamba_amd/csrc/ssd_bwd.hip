@@ -844,6 +844,10 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_
 template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_dcb_kernel(const SsdParams p) {
   __shared__ GemmLds lds;
   __shared__ float hA_l[2][GB], hA_s[2][GB], hdt[2][GB];  // per-head rows, double-buffered over the head loop
+  // the heads' ddA_cumsum shares (row sums per column half, column sums per row half), flushed at the end: a
+  // global atomic per head would sit in the memory queue in front of the next head's loads
+  constexpr int MAXH = 8;  // heads per workgroup (head_splits keeps it at or below 8)
+  __shared__ float rs_s[2][MAXH][GB], cs_s[2][MAXH][GB];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
   const int i = lane & 15, gq = lane >> 4;
@@ -913,9 +917,8 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_
         // the buffer written here was last read one step ago, before this step's barriers
         if (k0 % seg_k == 0 && hl + 1 < nh) load_rows(hl + 1);
         if ((k0 + GK) % seg_k != 0) return;
-        const int h = g * hpg + hs + hl * nsplit, par = hl & 1;
+        const int par = hl & 1;
         // d = this head's dCB term (added to sum); w = d * CB, whose row / column sums go to ddA
-        float *dda = chunk_row(p.ddA_cumsum, p, b, h, c);
         float a_s[2], dt_s[2], csum[2] = {0.f, 0.f};
 #pragma unroll
         for (int tn = 0; tn < 2; ++tn) {
@@ -943,16 +946,24 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_
             rsum += dpp_f<DPP_ROW_SHR + 2>(0.f, rsum);
             rsum += dpp_f<DPP_ROW_SHR + 4>(0.f, rsum);
             rsum += dpp_f<DPP_ROW_SHR + 8>(0.f, rsum);
-            if (i == 15 && rsum != 0.f) unsafeAtomicAdd(dda + lt * GB + m, rsum);
+            if (i == 15) rs_s[wn][hl][m] = rsum;
           }
 #pragma unroll
         for (int tn = 0; tn < 2; ++tn) {
           float cs = csum[tn];
           cs += __shfl_xor(cs, 16, 64);
           cs += __shfl_xor(cs, 32, 64);
-          if (gq == 0 && cs != 0.f) unsafeAtomicAdd(dda + st * GB + wn * 32 + tn * 16 + i, -cs);
+          if (gq == 0) cs_s[wm][hl][wn * 32 + tn * 16 + i] = cs;
         }
       });
+  __syncthreads();
+  for (int idx = tid; idx < nh * GB; idx += 256) {
+    const int hl = idx / GB, r = idx % GB;
+    float *dda = chunk_row(p.ddA_cumsum, p, b, g * hpg + hs + hl * nsplit, c);
+    const float row = rs_s[0][hl][r] + rs_s[1][hl][r], col = cs_s[0][hl][r] + cs_s[1][hl][r];
+    if (lt * GB + r < Q && row != 0.f) unsafeAtomicAdd(dda + lt * GB + r, row);
+    if (st * GB + r < Q && col != 0.f) unsafeAtomicAdd(dda + st * GB + r, -col);
+  }
   acc_foreach(sum, tid, [&](int m, int n, float v) {
     const int l = lt * GB + m, s = st * GB + n;
     if (l < Q && s < Q && v != 0.f) unsafeAtomicAdd(dCB + (int64_t)l * Q + s, v);  // dCB starts zeroed
