@@ -526,6 +526,8 @@ template <typename T, bool SPLIT, int PARTS> DEVI void dBC_state_body(const SsdP
   constexpr int MAXH = 8;  // heads per workgroup (head_splits keeps it at or below 8)
   __shared__ GemmLds lds;
   __shared__ float wB[MAXH][GB], wC[MAXH][GB];  // per-head row factors
+  // the heads' ddA_cumsum shares per half of the tile's columns, added to global memory once at the end
+  __shared__ float dda_s[(PARTS & 2) ? 2 : 1][(PARTS & 2) ? MAXH : 1][GB];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
   const int i = lane & 15, gq = lane >> 4;
@@ -626,8 +628,6 @@ template <typename T, bool SPLIT, int PARTS> DEVI void dBC_state_body(const SsdP
         tid, [&](int k0) {
           if ((k0 + GK) % seg_k != 0) return;
           // a head is complete: sum_n dC_h[l, n] C[l, n] goes to its ddA_cumsum row, dC_h to the sum
-          const int h = g * hpg + hs + (k0 / seg_k) * nsplit;
-          float *dda = chunk_row(p.ddA_cumsum, p, b, h, c);
 #pragma unroll
           for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
@@ -637,8 +637,7 @@ template <typename T, bool SPLIT, int PARTS> DEVI void dBC_state_body(const SsdP
               rs += dpp_f<DPP_ROW_SHR + 2>(0.f, rs);
               rs += dpp_f<DPP_ROW_SHR + 4>(0.f, rs);
               rs += dpp_f<DPP_ROW_SHR + 8>(0.f, rs);
-              const int l = st * GB + wm * 32 + tm * 16 + gq * 4 + r;
-              if (i == 15 && l < qlim && rs != 0.f) unsafeAtomicAdd(dda + l, rs);
+              if (i == 15) dda_s[wn][k0 / seg_k][wm * 32 + tm * 16 + gq * 4 + r] = rs;
             }
 #pragma unroll
           for (int ii = 0; ii < 2; ++ii)
@@ -653,6 +652,12 @@ template <typename T, bool SPLIT, int PARTS> DEVI void dBC_state_body(const SsdP
       if (l < qlim && nn < N) unsafeAtomicAdd(p.dC32 + (((int64_t)b * L + t0 + l) * G + g) * N + nn, v);
       return v;
     });
+    __syncthreads();
+    for (int idx = tid; idx < nh * GB; idx += 256) {
+      const int hl = idx / GB, r = idx % GB, l = st * GB + r;
+      const float d = dda_s[0][hl][r] + dda_s[1][hl][r];
+      if (l < qlim && d != 0.f) unsafeAtomicAdd(chunk_row(p.ddA_cumsum, p, b, g * hpg + hs + hl * nsplit, c) + l, d);
+    }
   }
 }
 
