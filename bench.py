@@ -107,7 +107,7 @@ def measured_mfma(dev):
     for i in range(4):
         if i == 1:
             ev[0].record()
-        flops = lib.mamba_hip_mfma_probe(sink.data_ptr(), 4096, blocks, stream)
+        flops = lib.mamba_hip_mfma_probe(sink.data_ptr(), 512, blocks, stream)
         if flops <= 0:
             _lib.check(int(flops), "mamba_hip_mfma_probe")
     ev[1].record()
