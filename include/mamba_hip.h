@@ -148,14 +148,15 @@ int mamba1_scan_bwd(const MambaScanParams *p, mamba_stream_t stream);
  * Every tensor is addressed through element strides, so stride-0 (expanded)
  * dt / A / dt_bias / D are accepted as they are.  Each operand has its own
  * dtype code (MAMBA_F32/BF16/F16); the arithmetic is fp32.
+ * `state` has state_rows rows (>= batch when state_batch_indices is null: entry b uses row b).
  * state_batch_indices (int32, nullable): row of `state` used by batch entry b;
- * a negative index skips the entry and writes out = 0.
+ * an index outside [0, state_rows) is a padding entry: its state is untouched and out = 0.
  * ------------------------------------------------------------------------- */
 typedef struct MambaStepParams {
   int32_t batch, nheads, dim, dstate, ngroups;
   int32_t dt_softplus;
   int32_t state_dtype, x_dtype /* x, z, out */, dt_dtype, dt_bias_dtype, A_dtype, bc_dtype /* B, C */, D_dtype;
-  int32_t reserved0;
+  int32_t state_rows; /* rows of `state` (its leading extent) */
   void *state;
   const void *x, *dt, *A, *B, *C;
   const void *D, *z, *dt_bias; /* nullable */

@@ -34,7 +34,7 @@ class MambaScanParams(ctypes.Structure):
 class MambaStepParams(ctypes.Structure):
     _fields_ = (
         [(n, c_i32) for n in ("batch", "nheads", "dim", "dstate", "ngroups", "dt_softplus", "state_dtype", "x_dtype",
-                              "dt_dtype", "dt_bias_dtype", "A_dtype", "bc_dtype", "D_dtype", "reserved0")]
+                              "dt_dtype", "dt_bias_dtype", "A_dtype", "bc_dtype", "D_dtype", "state_rows")]
         + [(n, c_vp) for n in ("state", "x", "dt", "A", "B", "C", "D", "z", "dt_bias", "out", "state_batch_indices")]
         + [(n, c_i64) for n in ("state_bs", "state_hs", "state_ps", "state_ns", "x_bs", "x_hs", "x_ps",
                                 "dt_bs", "dt_hs", "dt_ps", "dt_bias_hs", "dt_bias_ps", "A_hs", "A_ps", "A_ns",

@@ -82,7 +82,7 @@ __global__ __launch_bounds__(256) void state_update_kernel(const MambaStepParams
   int64_t sb = b;
   if (p.state_batch_indices) {
     const int idx = p.state_batch_indices[b];
-    if (idx < 0) {  // padding entry: no state update, zero output
+    if (idx < 0 || idx >= p.state_rows) {  // padding entry: no state update, zero output
       const int row = p_begin + lane;
       if (lane < rpp * UNR && row < p.dim) st1<TX>(outp + row * (int)p.out_ps, 0.f);
       return;
@@ -301,6 +301,8 @@ extern "C" int ssm_state_update(const MambaStepParams *p, mamba_stream_t stream)
   if (!p || !p->state || !p->x || !p->dt || !p->A || !p->B || !p->C || !p->out) return MAMBA_E_BADARG;
   if (p->batch <= 0 || p->nheads <= 0 || p->dim <= 0 || p->dstate <= 0 || p->ngroups <= 0) return MAMBA_E_BADARG;
   if (p->nheads % p->ngroups != 0) return MAMBA_E_BADARG;
+  // rows of `state`: without indices entry b uses row b; with them, an index outside [0, state_rows) is padding
+  if (p->state_rows <= 0 || (!p->state_batch_indices && p->state_rows < p->batch)) return MAMBA_E_BADARG;
   if (!dtype_ok(p->state_dtype) || !dtype_ok(p->x_dtype) || !dtype_ok(p->dt_dtype) || !dtype_ok(p->bc_dtype))
     return MAMBA_E_BADARG;
   // the small per-head operands are fp32 (the host side converts them)

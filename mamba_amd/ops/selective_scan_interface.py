@@ -105,7 +105,7 @@ def _fill_common(p, u, delta, A, B, C, D, z, delta_bias, delta_softplus, ckpt, d
 # (batch * dim * seqlen / 8 * dstate * 4 bytes: 1.3 GB at batch 8, dim 5120, seqlen 4096, dstate 16).  The
 # backward kernel then skips its own scan over each tile, about a tenth of its instructions.  False
 # makes it re-run that scan and keeps only the per-tile checkpoints.
-KEEP_LANE_STATES = True
+KEEP_LANE_STATES = False
 KEEP_LANE_STATES_MAX_BYTES = 16 << 30   # above this size per call the buffer is not kept
 
 

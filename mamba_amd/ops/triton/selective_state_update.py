@@ -23,7 +23,8 @@ def selective_state_update(state, x, dt, A, B, C, D=None, z=None, dt_bias=None, 
         D: (dim,) or (nheads, dim)
         z: (batch, dim) or (batch, nheads, dim)
         dt_bias: (dim,) or (nheads, dim)
-        state_batch_indices: (batch,) int32, row of `state` per batch entry; negative = padding
+        state_batch_indices: (batch,) int32, row of `state` per batch entry; an index outside
+            [0, state.shape[0]) is a padding entry (state untouched, out = 0)
     Return:
         out: (batch, dim) or (batch, nheads, dim)
     """
@@ -46,8 +47,11 @@ def selective_state_update(state, x, dt, A, B, C, D=None, z=None, dt_bias=None, 
         z = z.unsqueeze(1)
     if dt_bias is not None and dt_bias.dim() == 1:
         dt_bias = dt_bias.unsqueeze(0)
-    _, nheads, dim, dstate = state.shape
+    state_rows, nheads, dim, dstate = state.shape
     batch = x.shape[0]
+    if state_batch_indices is None and state_rows < batch:
+        raise RuntimeError(f"selective_state_update: state has {state_rows} rows for a batch of {batch} "
+                           "and no state_batch_indices")
     assert x.shape == (batch, nheads, dim)
     assert dt.shape == x.shape
     assert A.shape == (nheads, dim, dstate)
@@ -86,6 +90,7 @@ def selective_state_update(state, x, dt, A, B, C, D=None, z=None, dt_bias=None, 
     p = _lib.MambaStepParams()
     p.batch, p.nheads, p.dim, p.dstate, p.ngroups = batch, nheads, dim, dstate, ngroups
     p.dt_softplus = int(bool(dt_softplus))
+    p.state_rows = state_rows
     code = _lib.DTYPE_CODE
     p.state_dtype, p.x_dtype, p.dt_dtype = code[state.dtype], code[x.dtype], code[dt.dtype]
     p.A_dtype, p.bc_dtype = code[A.dtype], code[B.dtype]

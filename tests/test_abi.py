@@ -87,6 +87,22 @@ def test_host_ops_refuse_cpu_tensors():
                                   torch.randn(1, 8, 1, 4), torch.randn(1, 8, 1, 4), 4)
 
 
+def test_decode_step_refuses_a_state_with_fewer_rows_than_the_batch():
+    from mamba_amd.ops.triton.selective_state_update import selective_state_update
+    with pytest.raises(RuntimeError, match="rows"):   # checked before anything touches a device
+        selective_state_update(torch.zeros(2, 2, 4), torch.randn(3, 2), torch.randn(3, 2), -torch.ones(2, 4),
+                               torch.randn(3, 4), torch.randn(3, 4))
+    lib = _lib.load()
+    s = _lib.MambaStepParams()
+    for f in ("state", "x", "dt", "A", "B", "C", "out"):
+        setattr(s, f, 256)            # non-null stand-ins: the size checks below run before any launch
+    s.batch, s.nheads, s.dim, s.dstate, s.ngroups = 3, 1, 2, 4, 1
+    s.state_rows = 2
+    assert lib.ssm_state_update(ctypes.byref(s), None) == -1      # row b of a 2-row state for b = 2
+    s.state_rows = 0
+    assert lib.ssm_state_update(ctypes.byref(s), None) == -1
+
+
 def test_shape_errors_match_the_reference_behaviour():
     from mamba_amd.ops.triton.ssd_combined import mamba_chunk_scan_combined
     with pytest.raises(AssertionError):   # nheads % ngroups, ssd_combined.py:346

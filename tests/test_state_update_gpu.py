@@ -112,6 +112,31 @@ def test_selective_state_update_with_heads(with_indices, dim, dstate, ngroups, h
         assert float(out[1].abs().max()) == 0.0
 
 
+def test_index_past_the_state_rows_is_a_padding_entry():
+    """An index >= state.shape[0] must not be written through: the entry is skipped like a negative one."""
+    from mamba_amd.ops.triton.selective_state_update import selective_state_update
+    g = torch.Generator().manual_seed(5)
+    rows, batch, nheads, headdim, dstate = 3, 4, 2, 64, 16
+    state = torch.randn(rows, nheads, headdim, dstate, generator=g)
+    guard = torch.zeros(8, nheads, headdim, dstate)           # memory behind the state, must stay zero
+    buf = torch.cat([state, guard]).cuda()
+    state_g = buf[:rows]
+    x = torch.randn(batch, nheads, headdim, generator=g)
+    dt = torch.rand(batch, nheads, headdim, generator=g)
+    A = -torch.rand(nheads, headdim, dstate, generator=g)
+    B = torch.randn(batch, 1, dstate, generator=g)
+    C = torch.randn(batch, 1, dstate, generator=g)
+    idx = torch.tensor([2, 3, -1, 0], dtype=torch.int32)     # 3 == rows: out of range
+    state_ref = state.clone()
+    ok = torch.tensor([0, 3])
+    out_ref = selective_state_update_oracle(state_ref, x, dt, A, B, C, state_batch_indices=torch.where(idx >= rows, -1, idx))
+    out = selective_state_update(state_g, x.cuda(), dt.cuda(), A.cuda(), B.cuda(), C.cuda(), state_batch_indices=idx.cuda())
+    _check(state_g, state_ref, 1e-4, 1e-4, "state")
+    _check(out[ok], out_ref[ok], 1e-4, 1e-4, "out")
+    assert float(out[1].abs().max()) == 0.0 and float(out[2].abs().max()) == 0.0
+    assert float(buf[rows:].abs().max()) == 0.0
+
+
 def test_decode_steps_equal_scan():
     """T decode steps reproduce a length-T selective scan (the invariant of the reference's
     tests/test_generation.py:34-43), checked end to end on the GPU ops."""
