@@ -137,6 +137,21 @@ typedef struct MambaScanParams {
 int mamba1_scan_fwd(const MambaScanParams *p, mamba_stream_t stream);
 int mamba1_scan_bwd(const MambaScanParams *p, mamba_stream_t stream);
 
+/* No counterpart in the reference.  For callers that cannot allocate device memory -- code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc: mamba1_scan_fwd with the tile
+ * checkpoints kept in a fixed buffer inside the library (MAMBA_NOALLOC_SCRATCH_BYTES per GPU, held until
+ * the process ends) instead of a caller workspace.  p->ckpt and p->lane_state are ignored; `last_state`
+ * (nullable) is (batch, dim, dstate) fp32 contiguous ((batch, dim, dstate, 2) with a complex A) and
+ * receives the state after the last position.  Allocates and frees nothing.  Requests whose checkpoints
+ * batch * dim * ceil(seqlen / MAMBA_Q_SCAN_TILE) * dstate (* 2 if complex) * 4 bytes exceed the buffer
+ * return MAMBA_E_UNSUPPORTED.  Every call on a GPU uses that GPU's one buffer: calls that overlap on one
+ * GPU (two streams, two threads) race and must be serialised by the caller.  The buffer's address is
+ * looked up on the first call on a device; mamba_hip_init() does that ahead of time for the current
+ * device (call it before capturing a graph). */
+#define MAMBA_NOALLOC_SCRATCH_BYTES (32 << 20)
+int mamba_hip_init(void);
+int mamba1_scan_fwd_noalloc(const MambaScanParams *p, float *last_state, mamba_stream_t stream);
+
 /* ------------------------------------------------------------------------- *
  * Single-token decode: one step of the recurrence, in place on `state`.
  * Replaces the Triton kernel behind selective_state_update

@@ -754,6 +754,68 @@ extern "C" int mamba1_scan_fwd(const MambaScanParams *p, mamba_stream_t stream) 
   }
 }
 
+// ----------------------------------------------------- forward without a caller workspace
+// The tile checkpoints of mamba1_scan_fwd_noalloc live in this array instead of a caller buffer.
+// Host code never uses the array's name as an address: the device address is looked up once per
+// device with hipGetSymbolAddress and kept in g_scratch_ptr.
+constexpr int64_t SCRATCH_FLOATS = (int64_t)MAMBA_NOALLOC_SCRATCH_BYTES / 4;
+constexpr int SCRATCH_MAX_DEVICES = 64;
+static __device__ __align__(256) float scratch[SCRATCH_FLOATS];
+static float *g_scratch_ptr[SCRATCH_MAX_DEVICES];  // per device, null until resolved
+
+namespace {
+// Device address of `scratch` on the current device (resolved on first use), or null on failure.
+float *scratch_for_current_device() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= SCRATCH_MAX_DEVICES) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  float *ptr = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+  if (ptr) return ptr;
+  if (hipGetSymbolAddress(reinterpret_cast<void **>(&ptr), HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  __atomic_store_n(&g_scratch_ptr[dev], ptr, __ATOMIC_RELEASE);
+  return ptr;
+}
+
+// last_state[b, d, :] = ckpt[b, d, ntiles - 1, :]; `width` floats per (b, d) row (dstate, or 2 * dstate
+// for a complex state).
+__global__ __launch_bounds__(256) void gather_last_state_kernel(const float *__restrict__ ckpt, float *__restrict__ last,
+                                                                int64_t rows, int ntiles, int width) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= rows * width) return;
+  const int64_t row = i / width;
+  const int n = (int)(i - row * width);
+  last[i] = ckpt[(row * ntiles + (ntiles - 1)) * width + n];
+}
+}  // namespace
+
+extern "C" int mamba_hip_init(void) { return scratch_for_current_device() ? MAMBA_OK : MAMBA_E_LAUNCH; }
+
+extern "C" int mamba1_scan_fwd_noalloc(const MambaScanParams *p, float *last_state, mamba_stream_t stream) {
+  if (!p) return MAMBA_E_BADARG;
+  if (p->batch <= 0 || p->dim <= 0 || p->seqlen <= 0 || p->dstate <= 0) return MAMBA_E_BADARG;
+  const int ntiles = (p->seqlen + TILE - 1) / TILE;
+  const int width = p->dstate * (p->a_complex ? 2 : 1);
+  const int64_t rows = (int64_t)p->batch * p->dim;
+  if (rows * ntiles > SCRATCH_FLOATS / width) return MAMBA_E_UNSUPPORTED;  // checkpoints beyond the fixed buffer
+  float *ws = scratch_for_current_device();
+  if (!ws) return MAMBA_E_LAUNCH;
+  MambaScanParams q = *p;
+  q.ckpt = ws;
+  q.lane_state = nullptr;
+  const int rc = mamba1_scan_fwd(&q, stream);
+  if (rc != MAMBA_OK || !last_state) return rc;
+  const int64_t n = rows * width;
+  if ((n + 255) / 256 > 0x7fffffff) return MAMBA_E_UNSUPPORTED;
+  hipLaunchKernelGGL(gather_last_state_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), ws, last_state, rows, ntiles, width);
+  return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
+}
+
 extern "C" int mamba1_scan_bwd(const MambaScanParams *p, mamba_stream_t stream) {
   int rc = check_common(p);
   if (rc != MAMBA_OK) return rc;
