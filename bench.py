@@ -463,17 +463,13 @@ def main():
     # Dominant kernel (the backward scan) alone, HIP events on the launch stream.
     with torch.no_grad():
         d = {k: v.detach() for k, v in leaves.items()}
-        keep = ssi._keep_lane_states(d["u"], d["A"])   # the timed kernels are the ones a training step launches
-        _, ckpt, lanes = selective_scan_fwd(d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["z"], d["delta_bias"],
-                                            True, lane_states=True)
-        lanes = lanes if keep else None
+        _, ckpt = selective_scan_fwd(d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["z"], d["delta_bias"], True)
         dims = (batch, dim, seqlen, dstate, 1)
-        bufs = ssi.ScanBwdBuffers(d["u"], d["delta"], d["B"], d["z"], dims)
-        bwd_pre = lambda: ssi.scan_bwd_zero(bufs, dev)  # outside the event pair
-        bwd = lambda: ssi.scan_bwd_launch(d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["z"],
-                                          d["delta_bias"], t["dout"], ckpt, True, bufs, dims, lanes)
-        fwd = lambda: selective_scan_fwd(d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["z"],
-                                         d["delta_bias"], True, lane_states=keep)
+        bwd_args = (d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["z"], d["delta_bias"], t["dout"], ckpt, True, dims)
+        bufs = ssi.scan_bwd_launch(*bwd_args)
+        bwd_pre = None
+        bwd = lambda: ssi.scan_bwd_launch(*bwd_args, bufs=bufs)   # the scan kernel and its two small reduce kernels
+        fwd = lambda: selective_scan_fwd(d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["z"], d["delta_bias"], True)
 
         n = max(5, min(args.steps, 50))
         bwd_ms = event_ms(bwd, n, bwd_pre)

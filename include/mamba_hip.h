@@ -38,7 +38,8 @@ enum {
   MAMBA_Q_SCAN_TILE = 1,      /* sequence positions per checkpoint tile of the Mamba-1 scan */
   MAMBA_Q_MAX_DSTATE = 2,     /* largest d_state the Mamba-1 scan accepts */
   MAMBA_Q_SSD_MAX_DSTATE = 3, /* largest d_state of the SSD kernels */
-  MAMBA_Q_SSD_MAX_HEADDIM = 4
+  MAMBA_Q_SSD_MAX_HEADDIM = 4,
+  MAMBA_Q_SCAN_TILE_COMPLEX = 5 /* the same for a complex A */
 };
 
 int mamba_hip_query(int what);
@@ -87,9 +88,12 @@ int64_t mamba_hip_mfma_probe(float *sink, int iters, int blocks, mamba_stream_t 
  * dB32 / dC32 of per-position operands are (batch, ngroups, dstate, 2 * seqlen).
  *
  * ckpt is (batch, dim, ntiles, dstate) fp32 contiguous with
- * ntiles = ceil(seqlen / MAMBA_Q_SCAN_TILE): the state h after the last
- * position of each tile.  ckpt[:, :, ntiles-1, :] is the final state.  The
+ * ntiles = ceil(seqlen / MAMBA_Q_SCAN_TILE) (MAMBA_Q_SCAN_TILE_COMPLEX with a complex A): the
+ * state h after the last position of each tile.  ckpt[:, :, ntiles-1, :] is the final state.  The
  * backward pass re-computes the states inside a tile from ckpt.
+ *
+ * Backward: no float atomics are used for a real A, so every gradient repeats bit for bit from run to
+ * run (the reference's deterministic mode, mamba_ssm/utils/determinism.py:21-27, is the only mode).
  * ------------------------------------------------------------------------- */
 typedef struct MambaScanParams {
   int32_t batch, dim, seqlen, dstate, ngroups;
@@ -116,34 +120,36 @@ typedef struct MambaScanParams {
   void *du, *ddelta;
   void *dz;    /* required iff z != NULL; may be a strided view */
   void *out_z; /* nullable: when set (and z != NULL) the gated output is re-computed into it */
-  /* fp32 accumulators.  dB32, dC32: (batch, ngroups, dstate, seqlen) contiguous,
-   * MUST be zero on entry (kernels add into them).  dA_part: (batch, dim, dstate),
-   * dD_part, ddelta_bias_part: (batch, dim) -- written (not accumulated), the
-   * caller sums them over batch.  For an input-independent B (C), dB32 (dC32) is
-   * instead (batch, dim, dstate) partials, written like dA_part. */
+  /* fp32 workspaces, contents ignored on entry.  dB32, dC32: (batch, ngroups, nparts, dstate, seqlen)
+   * contiguous and 16-byte aligned, nparts = mamba1_scan_bwd_nparts(p): one partial sum per workgroup,
+   * which the call then adds up in a fixed order into dB / dC below (with a complex A: nparts = 1 and
+   * a last axis of 2 * seqlen).  dA_part: (batch, dim, dstate), dD_part, ddelta_bias_part:
+   * (batch, dim) -- written, the caller sums them over batch.  For an input-independent B (C),
+   * dB32 (dC32) is instead (batch, dim, dstate) partials, written like dA_part, and dB (dC) is unused. */
   float *dB32, *dC32, *dA_part, *dD_part, *ddelta_bias_part;
   int64_t dout_bs, dout_ds;
   int64_t du_bs, du_ds;
   int64_t ddelta_bs, ddelta_ds;
   int64_t dz_bs, dz_ds;
   int64_t outz_bs, outz_ds;
-  /* Optional (real A only): (batch, dim, ntiles, dstate, 64) fp32, the state entering each lane's
-   * 8 positions of a tile.  The forward call writes it when non-null; the backward call, when
-   * non-null, starts its re-computation of the states from it instead of re-running the scan over
-   * the tile (about a tenth of its instructions). */
-  float *lane_state;
+  /* gradients of per-position B and C: (batch, ngroups, dstate, seqlen) of `dtype`, contiguous
+   * ((..., 2 * seqlen) with a complex A) */
+  void *dB, *dC;
 } MambaScanParams;
 
 int mamba1_scan_fwd(const MambaScanParams *p, mamba_stream_t stream);
 int mamba1_scan_bwd(const MambaScanParams *p, mamba_stream_t stream);
+/* Number of per-workgroup partials the backward call writes into dB32 / dC32 for these sizes on the
+ * current device (> 0), or an error code.  Uses batch, dim, seqlen, dstate, ngroups, bc_const, a_complex. */
+int mamba1_scan_bwd_nparts(const MambaScanParams *p);
 
 /* No counterpart in the reference.  For callers that cannot allocate device memory -- code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc: mamba1_scan_fwd with the tile
  * checkpoints kept in a fixed buffer inside the library (MAMBA_NOALLOC_SCRATCH_BYTES per GPU, held until
- * the process ends) instead of a caller workspace.  p->ckpt and p->lane_state are ignored; `last_state`
+ * the process ends) instead of a caller workspace.  p->ckpt is ignored; `last_state`
  * (nullable) is (batch, dim, dstate) fp32 contiguous ((batch, dim, dstate, 2) with a complex A) and
  * receives the state after the last position.  Allocates and frees nothing.  Requests whose checkpoints
- * batch * dim * ceil(seqlen / MAMBA_Q_SCAN_TILE) * dstate (* 2 if complex) * 4 bytes exceed the buffer
+ * batch * dim * ceil(seqlen / tile) * dstate (* 2 if complex) * 4 bytes exceed the buffer
  * return MAMBA_E_UNSUPPORTED.  Every call on a GPU uses that GPU's one buffer: calls that overlap on one
  * GPU (two streams, two threads) race and must be serialised by the caller.  The buffer's address is
  * looked up on the first call on a device; mamba_hip_init() does that ahead of time for the current

@@ -9,7 +9,8 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libmamba_gfx950.so")
+# MAMBA_AMD_LIB names another build of the same library (same C ABI) to load instead of the in-tree one
+LIB_PATH = os.environ.get("MAMBA_AMD_LIB") or os.path.join(_HERE, "libmamba_gfx950.so")
 
 MAMBA_F32, MAMBA_BF16, MAMBA_F16 = 0, 1, 2
 DTYPE_CODE = {torch.float32: MAMBA_F32, torch.bfloat16: MAMBA_BF16, torch.float16: MAMBA_F16}
@@ -27,7 +28,7 @@ class MambaScanParams(ctypes.Structure):
                                "ddelta_bias_part")]
         + [(n, c_i64) for n in ("dout_bs", "dout_ds", "du_bs", "du_ds", "ddelta_bs", "ddelta_ds", "dz_bs", "dz_ds",
                                 "outz_bs", "outz_ds")]
-        + [("lane_state", c_vp)]
+        + [("dB", c_vp), ("dC", c_vp)]
     )
 
 
@@ -133,6 +134,8 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = [ctypes.POINTER(MambaScanParams), c_vp]
         fn.restype = ctypes.c_int
+    lib.mamba1_scan_bwd_nparts.argtypes = [ctypes.POINTER(MambaScanParams)]
+    lib.mamba1_scan_bwd_nparts.restype = ctypes.c_int
     lib.mamba1_scan_fwd_noalloc.argtypes = [ctypes.POINTER(MambaScanParams), c_vp, c_vp]
     lib.mamba1_scan_fwd_noalloc.restype = ctypes.c_int
     lib.mamba_hip_init.argtypes = []

@@ -55,8 +55,9 @@ extern "C" int mamba_hip_copy(void *dst, const void *src, int64_t nbytes, mamba_
 
 extern "C" int mamba_hip_query(int what) {
   switch (what) {
-    case MAMBA_Q_ABI_VERSION: return 4;
-    case MAMBA_Q_SCAN_TILE: return 512;
+    case MAMBA_Q_ABI_VERSION: return 5;
+    case MAMBA_Q_SCAN_TILE: return 128;
+    case MAMBA_Q_SCAN_TILE_COMPLEX: return 512;
     case MAMBA_Q_MAX_DSTATE: return 256;
     case MAMBA_Q_SSD_MAX_DSTATE: return 256;
     case MAMBA_Q_SSD_MAX_HEADDIM: return 256;

@@ -268,6 +268,17 @@ DEVI void wave_scan_fwd2(float &a0, float &b0, float &a1, float &b1) {
                : "+v"(a0), "+v"(b0), "+v"(a1), "+v"(b1));
 }
 
+// rows only (16 lanes each), towards lane 15 of the row: an inclusive scan per row
+DEVI void row_scan_fwd2(float &a0, float &b0, float &a1, float &b1) {
+  asm volatile("s_nop 1\n\t"
+               MAMBA_DPP2("row_shr:1 row_mask:0xf")
+               MAMBA_DPP2("row_shr:2 row_mask:0xf")
+               MAMBA_DPP2("row_shr:4 row_mask:0xf")
+               MAMBA_DPP2("row_shr:8 row_mask:0xf")
+               "s_nop 1\n\t"
+               : "+v"(a0), "+v"(b0), "+v"(a1), "+v"(b1));
+}
+
 // rows only (16 lanes each), towards lane 0 of the row
 DEVI void row_scan_rev2(float &a0, float &b0, float &a1, float &b1) {
   asm volatile("s_nop 1\n\t"
@@ -303,6 +314,15 @@ DEVI float wave_sum_to_last(float x) {
   x += dpp_f<DPP_ROW_SHR + 8>(0.f, x);
   x += dpp_f<DPP_ROW_BCAST15, 0xa>(0.f, x);
   x += dpp_f<DPP_ROW_BCAST31, 0xc>(0.f, x);
+  return x;
+}
+
+// Sum over each row of 16 lanes; only the last lane of a row holds its sum on return.
+DEVI float row_sum_to_last(float x) {
+  x += dpp_f<DPP_ROW_SHR + 1>(0.f, x);
+  x += dpp_f<DPP_ROW_SHR + 2>(0.f, x);
+  x += dpp_f<DPP_ROW_SHR + 4>(0.f, x);
+  x += dpp_f<DPP_ROW_SHR + 8>(0.f, x);
   return x;
 }
 

@@ -1,78 +1,72 @@
 // Mamba-1 selective scan, forward and backward, for gfx950 (wave64).
 //
 // Work decomposition
-//   * a wave owns R channels of one (batch, group); its 64 lanes hold 64
-//     consecutive 8-step segments of the sequence, i.e. one 512-step tile per
-//     pass.  Lane l loads its 8 items of u/delta/z with one 16-byte access.
-//   * the NW waves of a workgroup walk the tiles together and share the B and
-//     C rows of the tile, staged once per tile in LDS as fp32.
-//   * per state n: an 8-step in-register recurrence per lane, a DPP scan of
-//     the (decay, value) pairs across the 64 lanes, and a carry from the
-//     previous tile kept in LDS.
-//   * the state after every tile is written to `ckpt`; the backward pass walks
-//     the tiles in reverse, restarts each tile from ckpt, and runs the adjoint
-//     recurrence with a lane-reversed scan.  dB/dC are summed over the
-//     channels of the workgroup in LDS (waves take turns on disjoint state
-//     rows; LDS float atomics are far too slow for this) and added to global
-//     fp32 buffers once per tile.
+//   * a wave owns 4 channels of one (batch, group) at a time, one per DPP row of 16 lanes; the 16
+//     lanes of a row hold 16 consecutive 8-step segments of the sequence, i.e. one 128-step tile
+//     per pass.  A lane loads its 8 items of u/delta/z with one 16-byte access.  Every cross-lane
+//     step of the scans then stays inside a DPP row (row_shr / row_shl), which is the cheap kind.
+//   * the 8 waves of a workgroup walk the tiles together and share the B and C rows of the tile,
+//     staged once per tile in LDS as fp32; a backward workgroup takes several passes of 32 channels
+//     over a tile.
+//   * per state n: an 8-step in-register recurrence per lane, a row scan of the (decay, value)
+//     pairs across the 16 lanes, and a carry from the previous tile kept in LDS.
+//   * the state after every tile is written to `ckpt`; the backward pass walks the tiles in
+//     reverse, restarts each tile from ckpt, and runs the adjoint recurrence with a reversed row
+//     scan.  dB/dC are summed over the channels of the workgroup in LDS (waves take turns on
+//     disjoint state rows; LDS float atomics are far too slow for this), written once per tile as
+//     one partial per workgroup, and summed over the workgroups in a fixed order by a second
+//     kernel: no float atomics anywhere, so every gradient repeats bit for bit.
 #include "common.hpp"
 
 namespace {
 
-constexpr int KI = 8;           // items per lane
-constexpr int TILE = 64 * KI;   // sequence positions per tile
-constexpr int NB16 = 16;        // states staged per LDS block
-constexpr int BC_FLOATS = NB16 * TILE;        // one staged tensor
+constexpr int KI = 8;             // items per lane
+constexpr int RL = 16;            // lanes per channel (one DPP row)
+constexpr int ROWS = 4;           // channels per wave
+constexpr int TILE = RL * KI;     // sequence positions per tile
+constexpr int TILE_COMPLEX = 512; // tile of the complex kernels (mamba1_scan_complex.hip)
+constexpr int NB16 = 16;          // states staged per LDS block
+constexpr int NWAVES = 8;
+constexpr int NTHREADS = NWAVES * 64;
+constexpr int PASS_CH = NWAVES * ROWS;         // channels of a workgroup per pass
+constexpr int BC_FLOATS = NB16 * TILE;         // one staged operand
+constexpr int ACC_PITCH = TILE * ROWS;         // floats per state row of a dB / dC accumulator
+constexpr int ACC_FLOATS = NB16 * ACC_PITCH;   // one accumulator: [n][half][lane][4]
 constexpr int MAX_DSTATE = 256;
+constexpr int MAX_PASSES = 8;
 
-// B or C rows n0..n0+15 of the tile starting at t0 -> LDS as fp32, laid out
-// [n][half][lane][4] so that a lane reads its 8 items with two conflict-free
-// 16-byte LDS loads.
+// B or C rows n0..n0+15 of the tile starting at t0 -> LDS as fp32, laid out [n][half][c][4] (c = the
+// lane's place in its row) so that a lane reads its 8 items with two 16-byte LDS loads.
 // BC: bit 0 set = B is not staged (input-independent), bit 1 = C likewise.
-template <typename T, bool VEC, int NTHREADS, int BC>
+template <typename T, bool VEC, int BC>
 DEVI void stage_bc(float *Bs, float *Cs, const T *Bg, int64_t B_ns, const T *Cg, int64_t C_ns, int n0, int N, int t0,
                    int L, int tid) {
-  constexpr int FIRST = (BC & 1) ? NB16 * 64 : 0, LAST = (BC & 2) ? NB16 * 64 : 2 * NB16 * 64;
+  constexpr int FIRST = (BC & 1) ? NB16 * RL : 0, LAST = (BC & 2) ? NB16 * RL : 2 * NB16 * RL;
   if constexpr (BC == 3) {
     return;  // nothing is staged
-  } else if constexpr (VEC) {
-    // all loads first, from clamped (valid) addresses, then the masked LDS stores: a load under
-    // a branch, or converted right away, would make every load wait for the one before
-    constexpr int UNITS = (LAST - FIRST) / NTHREADS;
-    static_assert(UNITS * NTHREADS == LAST - FIRST, "whole units per thread");
-    Pack8<T> raw[UNITS];
-#pragma unroll
-    for (int q = 0; q < UNITS; ++q) {
-      const int unit = FIRST + tid + q * NTHREADS;
-      const int which = unit >> 10, n = min(n0 + ((unit >> 6) & 15), N - 1), t = min(t0 + KI * (unit & 63), L - KI);
-      raw[q].load((which ? Cg + (int64_t)n * C_ns : Bg + (int64_t)n * B_ns) + t);
-    }
-#pragma unroll
-    for (int q = 0; q < UNITS; ++q) {
-      const int unit = FIRST + tid + q * NTHREADS;
-      const int which = unit >> 10, n = (unit >> 6) & 15, j = unit & 63;
-      float v[8];
-      raw[q].unpack(v);
-      const bool ok = n0 + n < N && t0 + KI * j < L;
-      float *dst = (which ? Cs : Bs) + n * TILE + j * 4;
-      const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-      const f32x4 lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
-      *reinterpret_cast<f32x4 *>(dst) = ok ? lo : zero;
-      *reinterpret_cast<f32x4 *>(dst + 256) = ok ? hi : zero;
-    }
   } else {
-    for (int unit = FIRST + tid; unit < LAST; unit += NTHREADS) {
-      const int which = unit >> 10, n = (unit >> 6) & 15, j = unit & 63;
+    const int unit = FIRST + tid;  // one 8-item unit per thread: 2 operands x 16 states x 16 segments
+    if (unit >= LAST) return;
+    const int which = unit >> 8, n = (unit >> 4) & 15, j = unit & 15;
+    float v[8];
+    if constexpr (VEC) {
+      // from a clamped (valid) address, masked afterwards
+      Pack8<T> raw;
+      const int nc = min(n0 + n, N - 1), t = min(t0 + KI * j, L - KI);
+      raw.load((which ? Cg + (int64_t)nc * C_ns : Bg + (int64_t)nc * B_ns) + t);
+      raw.unpack(v);
+      const bool ok = n0 + n < N && t0 + KI * j < L;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = ok ? v[i] : 0.f;
+    } else {
       const int t = t0 + KI * j;
       const T *src = (which ? Cg + (int64_t)(n0 + n) * C_ns : Bg + (int64_t)(n0 + n) * B_ns) + t;
-      int nvalid = (n0 + n < N) ? min(max(L - t, 0), KI) : 0;
-      float v[8];
+      const int nvalid = (n0 + n < N) ? min(max(L - t, 0), KI) : 0;
       ld8_guard<T, false>(src, nvalid, 0.f, v);
-      float *dst = (which ? Cs : Bs) + n * TILE + j * 4;
-      f32x4 lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
-      *reinterpret_cast<f32x4 *>(dst) = lo;
-      *reinterpret_cast<f32x4 *>(dst + 256) = hi;
     }
+    float *dst = (which ? Cs : Bs) + n * TILE + j * 4;
+    *reinterpret_cast<f32x4 *>(dst) = f32x4{v[0], v[1], v[2], v[3]};
+    *reinterpret_cast<f32x4 *>(dst + 4 * RL) = f32x4{v[4], v[5], v[6], v[7]};
   }
 }
 
@@ -88,15 +82,14 @@ template <typename T, bool VEC> DEVI void load_items(Pack8<T> &k, const T *row, 
   }
 }
 
-DEVI void lds_st8(float *base, int lane, const float (&v)[8]) {
-  f32x4 lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
-  *reinterpret_cast<f32x4 *>(base + lane * 4) = lo;
-  *reinterpret_cast<f32x4 *>(base + 256 + lane * 4) = hi;
+// 8 floats of a [half][slot][4] LDS row: a slot's two 16-byte halves lie HALF_STRIDE floats apart
+template <int HALF_STRIDE> DEVI void lds_st8(float *base, int slot, const float (&v)[8]) {
+  *reinterpret_cast<f32x4 *>(base + slot * 4) = f32x4{v[0], v[1], v[2], v[3]};
+  *reinterpret_cast<f32x4 *>(base + HALF_STRIDE + slot * 4) = f32x4{v[4], v[5], v[6], v[7]};
 }
-
-DEVI void lds_ld8(const float *base, int lane, float (&o)[8]) {
-  f32x4 lo = *reinterpret_cast<const f32x4 *>(base + lane * 4);
-  f32x4 hi = *reinterpret_cast<const f32x4 *>(base + 256 + lane * 4);
+template <int HALF_STRIDE> DEVI void lds_ld8(const float *base, int slot, float (&o)[8]) {
+  const f32x4 lo = *reinterpret_cast<const f32x4 *>(base + slot * 4);
+  const f32x4 hi = *reinterpret_cast<const f32x4 *>(base + HALF_STRIDE + slot * 4);
   o[0] = lo.x; o[1] = lo.y; o[2] = lo.z; o[3] = lo.w;
   o[4] = hi.x; o[5] = hi.y; o[6] = hi.z; o[7] = hi.w;
 }
@@ -104,291 +97,284 @@ DEVI void lds_ld8(const float *base, int lane, float (&o)[8]) {
 // The 8 items of B (or C) for state n of channel d: from the staged tile, or, when the operand is an
 // input-independent (dim, dstate) fp32 matrix, its one value for every position (0 for padded states).
 template <int CONST>
-DEVI void load_bc(float (&v)[8], const float *staged, const void *mat, int d, int N, int n_abs, int n_loc, int lane) {
+DEVI void load_bc(float (&v)[8], const float *staged, const void *mat, int d, int N, int n_abs, int n_loc, int c) {
   if constexpr (CONST != 0) {
-    const float c = n_abs < N ? static_cast<const float *>(mat)[(int64_t)d * N + n_abs] : 0.f;
+    const float x = n_abs < N ? static_cast<const float *>(mat)[(int64_t)d * N + n_abs] : 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = c;
+    for (int i = 0; i < 8; ++i) v[i] = x;
   } else {
-    lds_ld8(staged + n_loc * TILE, lane, v);
+    lds_ld8<4 * RL>(staged + n_loc * TILE, c, v);
   }
+}
+
+// Where a workgroup's channels lie: workgroup cb of group g takes `passes` passes of PASS_CH channels.
+struct Geo {
+  int g, cb, b, Dg, dend, ntiles, cblocks;
+};
+DEVI Geo geometry(const MambaScanParams &p, int passes) {
+  Geo q;
+  q.Dg = p.dim / p.ngroups;
+  q.cblocks = (q.Dg + PASS_CH * passes - 1) / (PASS_CH * passes);
+  q.g = blockIdx.x / q.cblocks;
+  q.cb = blockIdx.x % q.cblocks;
+  q.b = blockIdx.y;
+  q.dend = (q.g + 1) * q.Dg;
+  q.ntiles = (p.seqlen + TILE - 1) / TILE;
+  return q;
 }
 
 // ------------------------------------------------------------------ forward
 // BC: bit 0 = B is an input-independent (dim, dstate) fp32 matrix, bit 1 = C likewise
 // (selective_scan_fwd_kernel.cuh:74 kIsVariableB / kIsVariableC false).
-template <typename T, int NW, int R, bool VEC, int BC>
-__global__ __launch_bounds__(NW * 64, 4) void scan_fwd_kernel(const MambaScanParams p) {
+template <typename T, bool VEC, int BC>
+__global__ __launch_bounds__(NTHREADS, 4) void scan_fwd_kernel(const MambaScanParams p, const int passes) {
   extern __shared__ __align__(16) float smem[];
   const int N = p.dstate, L = p.seqlen;
   const int NBLK = (N + NB16 - 1) / NB16, NP = NBLK * NB16;
   float *Bs = smem;
   float *Cs = Bs + BC_FLOATS;
-  float *A2s = Cs + BC_FLOATS;       // [NW*R][NP]  A * log2(e)
-  float *hcar = A2s + NW * R * NP;   // [NW*R][NP]  state carried across tiles
+  float *A2s = Cs + BC_FLOATS;                 // [passes * PASS_CH][NP]  A * log2(e)
+  float *hcar = A2s + passes * PASS_CH * NP;   // [passes * PASS_CH][NP]  state carried across tiles
 
-  const int tid = threadIdx.x, lane = tid & 63;
+  const int tid = threadIdx.x, lane = tid & 63, c = lane & (RL - 1), rsel = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int Dg = p.dim / p.ngroups;
-  const int cblocks = (Dg + NW * R - 1) / (NW * R);
-  const int g = blockIdx.x / cblocks, cb = blockIdx.x % cblocks;
-  const int b = blockIdx.y;
-  const int dbase = g * Dg + cb * NW * R + wave * R;
-  const int dend = (g + 1) * Dg;
-  const int ntiles = (L + TILE - 1) / TILE;
-
-  const T *Bg = (const T *)p.B + b * p.B_bs + g * p.B_gs;
-  const T *Cg = (const T *)p.C + b * p.C_bs + g * p.C_gs;
+  const Geo q = geometry(p, passes);
+  const int b = q.b;
+  const int chl = wave * ROWS + rsel;  // this lane's channel within a pass
+  const T *Bg = (const T *)p.B + b * p.B_bs + q.g * p.B_gs;
+  const T *Cg = (const T *)p.C + b * p.C_bs + q.g * p.C_gs;
   const float *Ag = (const float *)p.A;
+  const int d0 = q.g * q.Dg + q.cb * passes * PASS_CH;  // first channel of the workgroup
 
-  for (int i = lane; i < R * NP; i += 64) {
-    const int r = i / NP, n = i % NP, d = dbase + r;
-    A2s[wave * R * NP + i] = (d < dend && n < N) ? Ag[(int64_t)d * N + n] * kLog2e : 0.f;
-    hcar[wave * R * NP + i] = 0.f;
+  for (int i = tid; i < passes * PASS_CH * NP; i += NTHREADS) {
+    const int ch = i / NP, n = i % NP, d = d0 + ch;
+    A2s[i] = (d < q.dend && n < N) ? Ag[(int64_t)d * N + n] * kLog2e : 0.f;
+    hcar[i] = 0.f;
   }
+  __syncthreads();
 
-  for (int tile = 0; tile < ntiles; ++tile) {
-    const int t0 = tile * TILE, tl = t0 + lane * KI;
-    const int nvalid = min(max(L - tl, 0), KI);
-    for (int r = 0; r < R; ++r) {
-      const int d = dbase + r;
-      const bool valid = d < dend;
+  for (int tile = 0; tile < q.ntiles; ++tile) {
+    const int t0 = tile * TILE, tl = t0 + c * KI;
+    for (int r = 0; r < passes; ++r) {
+      if (d0 + r * PASS_CH >= q.dend) break;  // the whole pass lies past the group (the same in every wave)
+      const int chw = r * PASS_CH + chl;
+      const bool valid = d0 + chw < q.dend;
+      const int d = min(d0 + chw, q.dend - 1);
+      const int nvalid = valid ? min(max(L - tl, 0), KI) : 0;
       float u[8], dl[8], du[8], y[8], dsum = 0.f;
       Pack8<T> ku, kd, kz;  // raw rows: every load is issued before the first conversion
       kz.zero();
-      // lane states of this (tile, channel), when the caller keeps them for the backward pass
-      float *lanes = (p.lane_state && valid) ? p.lane_state + (((int64_t)b * p.dim + d) * ntiles + tile) * N * 64 : nullptr;
-      if (valid) {
-        load_items<T, VEC>(ku, (const T *)p.u + b * p.u_bs + d * p.u_ds, tl, L, nvalid);
-        load_items<T, VEC>(kd, (const T *)p.delta + b * p.delta_bs + d * p.delta_ds, tl, L, nvalid);
-        if (p.z) load_items<T, VEC>(kz, (const T *)p.z + b * p.z_bs + d * p.z_ds, tl, L, nvalid);
-        const float bias = p.delta_bias ? ((const float *)p.delta_bias)[d] : 0.f;
-        ku.unpack(u);
-        kd.unpack(dl);
+      load_items<T, VEC>(ku, (const T *)p.u + b * p.u_bs + d * p.u_ds, tl, L, nvalid);
+      load_items<T, VEC>(kd, (const T *)p.delta + b * p.delta_bs + d * p.delta_ds, tl, L, nvalid);
+      if (p.z) load_items<T, VEC>(kz, (const T *)p.z + b * p.z_bs + d * p.z_ds, tl, L, nvalid);
+      const float bias = p.delta_bias ? ((const float *)p.delta_bias)[d] : 0.f;
+      ku.unpack(u);
+      kd.unpack(dl);
 #pragma unroll
-        for (int i = 0; i < KI; ++i) {
-          float x = dl[i] + bias;
-          if (p.delta_softplus) x = softplus_f(x);
-          dl[i] = (i < nvalid) ? x : 0.f;
-          u[i] = (i < nvalid) ? u[i] : 0.f;
-          du[i] = dl[i] * u[i];
-          y[i] = 0.f;
-        }
-#pragma unroll
-        for (int i = 0; i < KI; ++i) dsum += dl[i];
+      for (int i = 0; i < KI; ++i) {
+        float x = dl[i] + bias;
+        if (p.delta_softplus) x = softplus_f(x);
+        dl[i] = (i < nvalid) ? x : 0.f;
+        u[i] = (i < nvalid) ? u[i] : 0.f;
+        du[i] = dl[i] * u[i];
+        y[i] = 0.f;
       }
+#pragma unroll
+      for (int i = 0; i < KI; ++i) dsum += dl[i];
       for (int nb = 0; nb < NBLK; ++nb) {
         if (BC != 3 && (NBLK > 1 || r == 0)) {
           __syncthreads();
-          stage_bc<T, VEC, NW * 64, BC>(Bs, Cs, Bg, p.B_ns, Cg, p.C_ns, nb * NB16, N, t0, L, tid);
+          stage_bc<T, VEC, BC>(Bs, Cs, Bg, p.B_ns, Cg, p.C_ns, nb * NB16, N, t0, L, tid);
           __syncthreads();
         }
-        if (valid) {
-          const float *A2row = A2s + (wave * R + r) * NP + nb * NB16;
-          float *hrow = hcar + (wave * R + r) * NP + nb * NB16;
-          const int nmax = min(NB16, N - nb * NB16);
-          // two states per iteration: their wave scans are interleaved (padded rows are inert:
-          // A = 0, B = C = 0)
-          for (int n = 0; n < nmax; n += 2) {
-            // Pass 1 runs the lane's 8 steps from a zero state to get the lane's (decay, value) pair;
-            // the decay over the lane is one exp of the summed delta instead of 7 products. Pass 2
-            // reruns the 8 steps from the state the wave scan gives this lane.
-            float a[2][8], bb[2][8], Cv[2][8], hc[2];
-            float sa[2], sb[2];
+        const float *A2row = A2s + chw * NP + nb * NB16;
+        float *hrow = hcar + chw * NP + nb * NB16;
+        const int nmax = min(NB16, N - nb * NB16);
+        // two states per iteration: their row scans are interleaved (padded rows are inert:
+        // A = 0, B = C = 0)
+        for (int n = 0; n < nmax; n += 2) {
+          // Pass 1 runs the lane's 8 steps from a zero state to get the lane's (decay, value) pair;
+          // the decay over the lane is one exp of the summed delta instead of 7 products. Pass 2
+          // reruns the 8 steps from the state the row scan gives this lane.
+          float a[2][8], bb[2][8], Cv[2][8], hc[2];
+          float sa[2], sb[2];
 #pragma unroll
-            for (int q = 0; q < 2; ++q) {
-              const float A2 = A2row[n + q];
-              hc[q] = hrow[n + q];
-              float Bv[8];
-              load_bc<BC & 1>(Bv, Bs, p.B, d, N, nb * NB16 + n + q, n + q, lane);
-              load_bc<BC & 2>(Cv[q], Cs, p.C, d, N, nb * NB16 + n + q, n + q, lane);
-              sa[q] = fast_exp2(dsum * A2);
+          for (int s = 0; s < 2; ++s) {
+            const float A2 = A2row[n + s];
+            hc[s] = hrow[n + s];
+            float Bv[8];
+            load_bc<BC & 1>(Bv, Bs, p.B, d, N, nb * NB16 + n + s, n + s, c);
+            load_bc<BC & 2>(Cv[s], Cs, p.C, d, N, nb * NB16 + n + s, n + s, c);
+            sa[s] = fast_exp2(dsum * A2);
 #pragma unroll
-              for (int i = 0; i < KI; ++i) {
-                a[q][i] = fast_exp2(dl[i] * A2);
-                bb[q][i] = du[i] * Bv[i];
-              }
-              float hl = bb[q][0];
-#pragma unroll
-              for (int i = 1; i < KI; ++i) hl = __builtin_fmaf(a[q][i], hl, bb[q][i]);
-              sb[q] = hl;
+            for (int i = 0; i < KI; ++i) {
+              a[s][i] = fast_exp2(dl[i] * A2);
+              bb[s][i] = du[i] * Bv[i];
             }
-            wave_scan_fwd2(sa[0], sb[0], sa[1], sb[1]);
-            const float hend[2] = {__builtin_fmaf(sa[0], hc[0], sb[0]), __builtin_fmaf(sa[1], hc[1], sb[1])};
+            float hl = bb[s][0];
 #pragma unroll
-            for (int q = 0; q < 2; ++q) {
-              float h = dpp_f<DPP_WAVE_SHR1>(hc[q], hend[q]);  // state entering this lane
-              if (lane == 63) hrow[n + q] = hend[q];           // state after the tile
-              if (lanes && nb * NB16 + n + q < N) lanes[(nb * NB16 + n + q) * 64 + lane] = h;
+            for (int i = 1; i < KI; ++i) hl = __builtin_fmaf(a[s][i], hl, bb[s][i]);
+            sb[s] = hl;
+          }
+          row_scan_fwd2(sa[0], sb[0], sa[1], sb[1]);
+          const float hend[2] = {__builtin_fmaf(sa[0], hc[0], sb[0]), __builtin_fmaf(sa[1], hc[1], sb[1])};
 #pragma unroll
-              for (int i = 0; i < KI; ++i) {
-                h = __builtin_fmaf(a[q][i], h, bb[q][i]);
-                y[i] = __builtin_fmaf(h, Cv[q][i], y[i]);
-              }
+          for (int s = 0; s < 2; ++s) {
+            float h = dpp_f<DPP_ROW_SHR + 1>(hc[s], hend[s]);  // state entering this lane
+            if (c == RL - 1) hrow[n + s] = hend[s];            // state after the tile
+#pragma unroll
+            for (int i = 0; i < KI; ++i) {
+              h = __builtin_fmaf(a[s][i], h, bb[s][i]);
+              y[i] = __builtin_fmaf(h, Cv[s][i], y[i]);
             }
           }
         }
       }
-      if (valid) {
-        if (p.D) {
-          const float Dd = ((const float *)p.D)[d];
+      if (p.D) {
+        const float Dd = ((const float *)p.D)[d];
 #pragma unroll
-          for (int i = 0; i < KI; ++i) y[i] = __builtin_fmaf(Dd, u[i], y[i]);
-        }
-        if (p.z) {
-          float z[8];
-          kz.unpack(z);
+        for (int i = 0; i < KI; ++i) y[i] = __builtin_fmaf(Dd, u[i], y[i]);
+      }
+      if (p.z) {
+        float z[8];
+        kz.unpack(z);
 #pragma unroll
-          for (int i = 0; i < KI; ++i) y[i] *= z[i] * sigmoid_f(z[i]);
-        }
-        st8_guard<T, VEC>((T *)p.out + b * p.out_bs + d * p.out_ds + tl, nvalid, y);
-        float *ck = p.ckpt + (((int64_t)b * p.dim + d) * ntiles + tile) * N;
-        const float *hfin = hcar + (wave * R + r) * NP;
-        for (int n = lane; n < N; n += 64) ck[n] = hfin[n];
+        for (int i = 0; i < KI; ++i) y[i] *= z[i] * sigmoid_f(z[i]);
+      }
+      st8_guard<T, VEC>((T *)p.out + b * p.out_bs + d * p.out_ds + tl, nvalid, y);
+      if (valid) {  // a row's own lanes wrote its slots of hcar: no other wave touches them
+        float *ck = p.ckpt + (((int64_t)b * p.dim + d) * q.ntiles + tile) * N;
+        const float *hfin = hcar + chw * NP;
+        for (int n = c; n < N; n += RL) ck[n] = hfin[n];
       }
     }
   }
 }
 
 // ----------------------------------------------------------------- backward
-// Row starts of one channel of the workgroup, kept in LDS: every (tile, channel) step needs nine
-// addresses, and as scalars next to the loop state they did not fit the scalar registers (each step
-// then re-read some 250 spilled scalars through v_readlane).
+// Row starts of one channel of the workgroup, kept in LDS: every (tile, pass) step needs nine
+// addresses per lane, and as kernel arguments next to the loop state they did not fit the scalar
+// registers (each step then re-read hundreds of spilled scalars through v_readlane).
 template <typename T> struct BwdRow {
   const T *u, *delta, *dout, *z;
   T *du, *ddelta, *dz, *out_z;
-  const float *ckpt;  // tile 0 of this channel: the tile checkpoints, or with LS the lane states
+  const float *ckpt;  // tile 0 of this channel
   float D, bias;
 };
 
-// LS: the forward pass left the state entering every lane's 8 positions (lane_state); the states of a
-// tile are then re-computed from those directly, without the lane-local pass and the wave scan.
-template <typename T, int NW, int R, bool VEC, int BC, bool LS>
-__global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams p) {
-  static_assert(sizeof(BwdRow<T>) == 80, "the host side sizes the LDS table with 80 bytes per channel");
+// `passes` passes of PASS_CH channels per tile; the dB / dC sums of all of them leave once per tile as
+// partial number (workgroup's place in its group), or after every pass and block when the states come
+// in blocks of 16 (the host side then asks for one pass).
+template <typename T, bool VEC, int BC>
+__global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParams p, const int passes) {
   extern __shared__ __align__(16) float smem[];
   const int N = p.dstate, L = p.seqlen;
   const int NBLK = (N + NB16 - 1) / NB16, NP = NBLK * NB16;
-  constexpr int WR = NW * R;
+  const int WCH = passes * PASS_CH;
   float *Bs = smem;
   float *Cs = Bs + BC_FLOATS;
-  float *dBs = Cs + BC_FLOATS;        // fp32 sums over the workgroup's channels, same layout as Bs
-  float *dCs = dBs + BC_FLOATS;
-  float *A1s = dCs + BC_FLOATS;       // [WR][NP] A
-  float *hcar = A1s + WR * NP;        // state entering the tile (from ckpt)
-  float *gcar = hcar + WR * NP;       // adjoint at the first position of the following tile
-  float *anx = gcar + WR * NP;        // decay at the first position of the following tile
-  float *dAacc = anx + WR * NP;       // [WR][NP]
-  float *dDacc = dAacc + WR * NP;     // [WR]
-  float *dbacc = dDacc + WR;          // [WR]
-  float *dBcacc = dbacc + WR;         // [WR][NP] gradients of input-independent B / C
-  float *dCcacc = dBcacc + WR * NP;
-  BwdRow<T> *rows = reinterpret_cast<BwdRow<T> *>(dCcacc + WR * NP);  // [WR]
+  float *dBs = Cs + BC_FLOATS;        // fp32 sums over the workgroup's channels: [n][half][lane][4]
+  float *dCs = dBs + ACC_FLOATS;
+  float *hcar = dCs + ACC_FLOATS;     // [PASS_CH][NP] state entering the tile (from ckpt), per pass
+  float *A1s = hcar + PASS_CH * NP;   // [WCH][NP] A
+  float *gcar = A1s + WCH * NP;       // adjoint at the first position of the following tile
+  float *anx = gcar + WCH * NP;       // decay at the first position of the following tile
+  float *dAacc = anx + WCH * NP;      // [WCH][NP]
+  float *dDacc = dAacc + WCH * NP;    // [WCH]
+  float *dbacc = dDacc + WCH;         // [WCH]
+  BwdRow<T> *rows = reinterpret_cast<BwdRow<T> *>(dbacc + WCH);  // [WCH]
+  float *dBcacc = reinterpret_cast<float *>(rows + WCH);  // [WCH][NP] gradients of input-independent B / C (BC != 0)
+  float *dCcacc = dBcacc + WCH * NP;
+  static_assert(sizeof(BwdRow<T>) == 80, "the host side sizes the LDS table with 80 bytes per channel");
 
-  const int tid = threadIdx.x, lane = tid & 63;
+  const int tid = threadIdx.x, lane = tid & 63, c = lane & (RL - 1), rsel = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int Dg = p.dim / p.ngroups;
-  const int cblocks = (Dg + WR - 1) / WR;
-  const int g = blockIdx.x / cblocks, cb = blockIdx.x % cblocks;
-  const int b = blockIdx.y;
-  const int dbase = g * Dg + cb * WR + wave * R;
-  const int dend = (g + 1) * Dg;
-  const int ntiles = (L + TILE - 1) / TILE;
+  const Geo q = geometry(p, passes);
+  const int b = q.b;
+  const int chl = wave * ROWS + rsel;
+  const int d0 = q.g * q.Dg + q.cb * WCH;
+  const int ntiles = q.ntiles;
   const bool has_z = p.z != nullptr;
-  if (lane < R) {  // each wave fills and reads only its own rows
-    const int d = min(dbase + lane, dend - 1);
-    BwdRow<T> q;
-    q.u = (const T *)p.u + b * p.u_bs + d * p.u_ds;
-    q.delta = (const T *)p.delta + b * p.delta_bs + d * p.delta_ds;
-    q.dout = (const T *)p.dout + b * p.dout_bs + d * p.dout_ds;
-    q.z = has_z ? (const T *)p.z + b * p.z_bs + d * p.z_ds : nullptr;
-    q.du = (T *)p.du + b * p.du_bs + d * p.du_ds;
-    q.ddelta = (T *)p.ddelta + b * p.ddelta_bs + d * p.ddelta_ds;
-    q.dz = has_z ? (T *)p.dz + b * p.dz_bs + d * p.dz_ds : nullptr;
-    q.out_z = (has_z && p.out_z) ? (T *)p.out_z + b * p.outz_bs + d * p.outz_ds : nullptr;
-    q.ckpt = LS ? p.lane_state + ((int64_t)b * p.dim + d) * ntiles * N * 64 : p.ckpt + ((int64_t)b * p.dim + d) * ntiles * N;
-    q.D = p.D ? ((const float *)p.D)[d] : 0.f;
-    q.bias = p.delta_bias ? ((const float *)p.delta_bias)[d] : 0.f;
-    rows[wave * R + lane] = q;
-  }
 
-  const T *Bg = (const T *)p.B + b * p.B_bs + g * p.B_gs;
-  const T *Cg = (const T *)p.C + b * p.C_bs + g * p.C_gs;
+  const T *Bg = (const T *)p.B + b * p.B_bs + q.g * p.B_gs;
+  const T *Cg = (const T *)p.C + b * p.C_bs + q.g * p.C_gs;
   const float *Ag = (const float *)p.A;
-  float *dBg = p.dB32 + ((int64_t)b * p.ngroups + g) * N * L;
-  float *dCg = p.dC32 + ((int64_t)b * p.ngroups + g) * N * L;
+  // partials of this workgroup: (batch, ngroups, nparts, dstate, seqlen), nparts = cblocks (x passes when NBLK > 1)
+  const int per_wg = NBLK > 1 ? passes : 1;
+  const int64_t part0 = ((int64_t)b * p.ngroups + q.g) * (q.cblocks * per_wg) + (int64_t)q.cb * per_wg;
 
-  for (int i = lane; i < R * NP; i += 64) {
-    const int r = i / NP, n = i % NP, d = dbase + r;
-    const int o = wave * R * NP + i;
-    A1s[o] = (d < dend && n < N) ? Ag[(int64_t)d * N + n] : 0.f;
-    gcar[o] = 0.f;
-    anx[o] = 0.f;
-    dAacc[o] = 0.f;
-    dBcacc[o] = 0.f;
-    dCcacc[o] = 0.f;
+  for (int i = tid; i < WCH * NP; i += NTHREADS) {
+    const int ch = i / NP, n = i % NP, d = d0 + ch;
+    A1s[i] = (d < q.dend && n < N) ? Ag[(int64_t)d * N + n] : 0.f;
+    gcar[i] = 0.f;
+    anx[i] = 0.f;
+    dAacc[i] = 0.f;
+    if constexpr (BC != 0) {
+      dBcacc[i] = 0.f;
+      dCcacc[i] = 0.f;
+    }
   }
-  if (lane < R) {
-    dDacc[wave * R + lane] = 0.f;
-    dbacc[wave * R + lane] = 0.f;
+  for (int i = tid; i < WCH; i += NTHREADS) {
+    dDacc[i] = 0.f;
+    dbacc[i] = 0.f;
+    const int d = min(d0 + i, q.dend - 1);  // channels past the group stand on its last one; their lanes are masked
+    BwdRow<T> w;
+    w.u = (const T *)p.u + b * p.u_bs + d * p.u_ds;
+    w.delta = (const T *)p.delta + b * p.delta_bs + d * p.delta_ds;
+    w.dout = (const T *)p.dout + b * p.dout_bs + d * p.dout_ds;
+    w.z = has_z ? (const T *)p.z + b * p.z_bs + d * p.z_ds : nullptr;
+    w.du = (T *)p.du + b * p.du_bs + d * p.du_ds;
+    w.ddelta = (T *)p.ddelta + b * p.ddelta_bs + d * p.ddelta_ds;
+    w.dz = has_z ? (T *)p.dz + b * p.dz_bs + d * p.dz_ds : nullptr;
+    w.out_z = (has_z && p.out_z) ? (T *)p.out_z + b * p.outz_bs + d * p.outz_ds : nullptr;
+    w.ckpt = p.ckpt + ((int64_t)b * p.dim + d) * ntiles * N;
+    w.D = p.D ? ((const float *)p.D)[d] : 0.f;
+    w.bias = p.delta_bias ? ((const float *)p.delta_bias)[d] : 0.f;
+    rows[i] = w;
   }
+  __syncthreads();
 
-  // The rows of the next (tile, channel) are fetched while the current one is computed.
-  constexpr int NPP = NB16 / NW > 0 ? NB16 / NW : 1;  // state rows per wave and phase (see the state loop)
+  constexpr int NPP = NB16 / NWAVES;  // state rows per wave and phase (see the state loop)
   constexpr int NPH = NB16 / NPP;
-  constexpr int Q = NPP >= 2 ? 2 : 1;                 // states per step; two keep two scan chains in flight
+  static_assert(NPP == 2 && NPH == NWAVES, "two states per step, one row slot per wave and phase");
+  // The rows of the next (tile, pass) are fetched while the current one is computed.
   struct Rows {
     Pack8<T> u, delta, dout, z;
-    float ck;     // !LS: checkpointed state n = lane entering the tile (when the padded state count fits a wave)
-    float h0[Q];  // LS: lane states of the first step's states
-  };
-  // lane states of step (nb, ph, j) of a (tile, channel): rows past N read a clamped row and are never used
-  auto lane_states = [&](const float *tile_base, int nb, int ph, int j, float (&o)[Q]) {
-    const int n = nb * NB16 + ((wave + ph) % NPH) * NPP + j;
-#pragma unroll
-    for (int q = 0; q < Q; ++q) o[q] = tile_base[(int64_t)min(n + q, N - 1) * 64 + lane];
+    float ck;  // checkpointed state n = c entering the tile (when the padded state count is 16)
   };
   auto fetch_rows = [&](Rows &k, int tile, int r) {
-    const int d = dbase + r, tl = tile * TILE + lane * KI;
+    const BwdRow<T> &w = rows[r * PASS_CH + chl];
+    const int tl = tile * TILE + c * KI;
     const int nvalid = min(max(L - tl, 0), KI);
     k.z.zero();
     k.ck = 0.f;
-#pragma unroll
-    for (int q = 0; q < Q; ++q) k.h0[q] = 0.f;
-    if (d < dend) {
-      const BwdRow<T> &q = rows[wave * R + r];
-      if constexpr (LS) lane_states(q.ckpt + (int64_t)tile * N * 64, 0, 0, 0, k.h0);
-      else if (NP <= 64 && tile > 0 && lane < N) k.ck = q.ckpt[(int64_t)(tile - 1) * N + lane];
-      load_items<T, VEC>(k.u, q.u, tl, L, nvalid);
-      load_items<T, VEC>(k.delta, q.delta, tl, L, nvalid);
-      load_items<T, VEC>(k.dout, q.dout, tl, L, nvalid);
-      if (has_z) load_items<T, VEC>(k.z, q.z, tl, L, nvalid);
-    }
+    if (NBLK == 1 && tile > 0) k.ck = w.ckpt[(int64_t)(tile - 1) * N + min(c, N - 1)];
+    load_items<T, VEC>(k.u, w.u, tl, L, nvalid);
+    load_items<T, VEC>(k.delta, w.delta, tl, L, nvalid);
+    load_items<T, VEC>(k.dout, w.dout, tl, L, nvalid);
+    if (has_z) load_items<T, VEC>(k.z, w.z, tl, L, nvalid);
   };
+  int npass = 0;  // passes that hold at least one channel of the group (the same in every wave)
+  while (npass < passes && d0 + npass * PASS_CH < q.dend) ++npass;
   Rows nxt;
   fetch_rows(nxt, ntiles - 1, 0);
 
   for (int tile = ntiles - 1; tile >= 0; --tile) {
-    const int t0 = tile * TILE, tl = t0 + lane * KI;
-    const int nvalid = min(max(L - tl, 0), KI);
-    for (int r = 0; r < R; ++r) {
-      const int d = dbase + r;
-      const bool valid = d < dend;
-      const int row = wave * R + r;
+    const int t0 = tile * TILE, tl = t0 + c * KI;
+    for (int r = 0; r < npass; ++r) {
+      const int chw = r * PASS_CH + chl;
+      const bool valid = d0 + chw < q.dend;
+      const int d = min(d0 + chw, q.dend - 1);
+      const int nvalid = valid ? min(max(L - tl, 0), KI) : 0;
       float u[8], dl[8], du[8], dy[8], acc[8], dd[8], y[8], dsum = 0.f, dtail = 0.f;
       // raw delta, z and dout stay in registers in their storage format for the epilogue
       const Rows cur = nxt;
-      float hnext[Q];  // LS: lane states of the step about to run
-#pragma unroll
-      for (int q = 0; q < Q; ++q) hnext[q] = cur.h0[q];
       Pack8<T> draw_k = cur.delta, z_k = cur.z, dout_k = cur.dout;
-      if (r + 1 < R) fetch_rows(nxt, tile, r + 1);
+      if (r + 1 < npass) fetch_rows(nxt, tile, r + 1);
       else if (tile > 0) fetch_rows(nxt, tile - 1, 0);
-      float Dd = 0.f;
-      if (valid) {
-        Dd = rows[row].D;
+      const float Dd = rows[chw].D, bias = rows[chw].bias;
+      {
         const Pack8<T> u_k = cur.u;
-        const float bias = rows[row].bias;
         u_k.unpack(u);
         draw_k.unpack(dl);
         dout_k.unpack(dy);
@@ -413,200 +399,217 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
           dd[i] = 0.f;
           y[i] = 0.f;
         }
-        dtail = 0.f;
 #pragma unroll
         for (int i = 1; i < KI; ++i) dtail += dl[i];
         dsum = dtail + dl[0];
-        // state entering this tile
-        if constexpr (LS) {
-        } else if (NP <= 64) {
-          if (lane < NP) hcar[row * NP + lane] = cur.ck;
+        // state entering this tile (a row's own lanes write and read its slots)
+        if (NBLK == 1) {
+          hcar[chl * NP + c] = c < N ? cur.ck : 0.f;
         } else {
-          for (int n = lane; n < NP; n += 64) {
+          for (int n = c; n < NP; n += RL) {
             float v = 0.f;
-            if (tile > 0 && n < N) v = rows[row].ckpt[(int64_t)(tile - 1) * N + n];
-            hcar[row * NP + n] = v;
+            if (tile > 0 && n < N) v = rows[chw].ckpt[(int64_t)(tile - 1) * N + n];
+            hcar[chl * NP + n] = v;
           }
         }
       }
       for (int nb = 0; nb < NBLK; ++nb) {
         if (BC != 3 && (NBLK > 1 || r == 0)) {
           __syncthreads();
-          stage_bc<T, VEC, NW * 64, BC>(Bs, Cs, Bg, p.B_ns, Cg, p.C_ns, nb * NB16, N, t0, L, tid);
-          for (int i = tid * 4; i < 2 * BC_FLOATS; i += NW * 256)  // dBs and dCs are adjacent
+          stage_bc<T, VEC, BC>(Bs, Cs, Bg, p.B_ns, Cg, p.C_ns, nb * NB16, N, t0, L, tid);
+          for (int i = tid * 4; i < 2 * ACC_FLOATS; i += NTHREADS * 4)  // dBs and dCs are adjacent
             *reinterpret_cast<f32x4 *>(dBs + i) = f32x4{0.f, 0.f, 0.f, 0.f};
           __syncthreads();
         }
         {
-          // The NW waves add their channels' dB/dC terms into the shared LDS sums without
-          // atomics: in phase ph wave w owns state rows (w + ph) % NPH * NPP .. + NPP - 1,
-          // so no two waves touch a row between two barriers.
-          static_assert(NW <= NPH, "one row slot per wave and phase");
-          const float *A1row = A1s + row * NP + nb * NB16;
-          const float *hrow = hcar + row * NP + nb * NB16;
-          float *grow = gcar + row * NP + nb * NB16;
-          float *arow = anx + row * NP + nb * NB16;
-          float *dArow = dAacc + row * NP + nb * NB16;
-          const int nmax = min(NB16, N - nb * NB16);
-          static_assert(NPP % Q == 0, "whole steps per phase");
-          for (int ph = 0; ph < NPH; ++ph) {
-            const int slot = (wave + ph) % NPH;
-            for (int j = 0; j < NPP; j += Q) {
-              const int n = slot * NPP + j;
-              float hin[Q];
-              if constexpr (LS) {
-                // this step's lane states arrived during the previous step (the first step's with the rows);
-                // the next step's are requested now
+          // The 8 waves add their channels' dB/dC terms into the shared LDS sums without atomics: between
+          // two workgroup barriers every wave adds into another pair of state rows, and the 4 channels of a
+          // wave have their own slots of a row.  A phase has two halves, the states and adjoints of the pair
+          // (vector ALU work) and the sums (LDS traffic).  Waves 4-7 meet the barrier at the end of a phase;
+          // waves 0-3 meet the same barrier between their two halves, so they run half a phase behind and
+          // the two waves of a SIMD are never in the same half: one computes while the other waits for LDS.
+          // Between barriers j and j + 1 waves 0-3 add the sums of phase j into rows (w + j) % 8 * 2, + 1 and
+          // waves 4-7 those of phase j + 1 into rows (w + j) % 8 * 2, + 1 (their rows run one phase behind):
+          // eight different pairs.
+          const bool early = wave < NWAVES / 2;
+          const int slot_shift = early ? 0 : NPH - 1;
+          const float *A1row = A1s + chw * NP + nb * NB16;
+          const float *hrow = hcar + chl * NP + nb * NB16;
+          float *grow = gcar + chw * NP + nb * NB16;
+          float *arow = anx + chw * NP + nb * NB16;
+          float *dArow = dAacc + chw * NP + nb * NB16;
+          // the LDS operands of a phase's two states: A, the carries, the B and C rows
+          struct Operands {
+            float A1[2], hc[2], gc[2], an[2], Bv[2][8], Cv[2][8];
+          };
+          auto fetch_operands = [&](Operands &o, int ph) {
+            const int n = ((wave + ph + slot_shift) % NPH) * NPP;
 #pragma unroll
-                for (int q = 0; q < Q; ++q) hin[q] = hnext[q];
-                int j2 = j + Q, ph2 = ph, nb2 = nb;
-                if (j2 >= NPP) { j2 = 0; ++ph2; }
-                if (ph2 >= NPH) { ph2 = 0; ++nb2; }
-                if (valid && nb2 < NBLK) lane_states(rows[row].ckpt + (int64_t)tile * N * 64, nb2, ph2, j2, hnext);
-              }
-              if (!valid || n >= nmax) continue;
+            for (int s = 0; s < 2; ++s) {
+              o.A1[s] = A1row[n + s];
+              o.hc[s] = hrow[n + s];
+              o.gc[s] = grow[n + s];
+              o.an[s] = arow[n + s];
+              load_bc<BC & 1>(o.Bv[s], Bs, p.B, d, N, nb * NB16 + n + s, n + s, c);
+              load_bc<BC & 2>(o.Cv[s], Cs, p.C, d, N, nb * NB16 + n + s, n + s, c);
+            }
+          };
+          Operands ops;
+          fetch_operands(ops, 0);
+          for (int ph = 0; ph < NPH; ++ph) {
+            const int n = ((wave + ph + slot_shift) % NPH) * NPP;
+            constexpr bool active = true;  // padded states run on zeros (A = B = C = 0)
+            float A1[2], gc[2], an[2];
+            float Cv[2][8], a[2][8], bb[2][8], h[2][8];
+            float gfirst[2], a_next_lane[2];
+            if (active) {
               // Forward states: pass 1 runs the lane's 8 steps from zero for the lane's (decay, value)
               // pair, the decay being one exp of the summed delta; pass 2 reruns them from the state
-              // the wave scan gives this lane. The adjoint is handled the same way in reverse.
-              float A1[Q], hc[Q], gc[Q], an[Q];
-              float Cv[Q][8], a[Q][8], bb[Q][8], h[Q][8];
-              float sa[Q], sb[Q], hend[Q];
+              // the row scan gives this lane. The adjoint is handled the same way in reverse.
+              float hc[2], sa[2], sb[2], hend[2];
 #pragma unroll
-              for (int q = 0; q < Q; ++q) {
-                A1[q] = A1row[n + q];
-                hc[q] = LS ? 0.f : hrow[n + q];
-                gc[q] = grow[n + q];
-                an[q] = arow[n + q];
-                float Bv[8];  // read again for the last loop: 16 registers fewer held through the scans
-                load_bc<BC & 1>(Bv, Bs, p.B, d, N, nb * NB16 + n + q, n + q, lane);
-                load_bc<BC & 2>(Cv[q], Cs, p.C, d, N, nb * NB16 + n + q, n + q, lane);
-                const float A2 = A1[q] * kLog2e;
+              for (int s = 0; s < 2; ++s) {
+                A1[s] = ops.A1[s];
+                hc[s] = ops.hc[s];
+                gc[s] = ops.gc[s];
+                an[s] = ops.an[s];
+                const float A2 = A1[s] * kLog2e;
 #pragma unroll
                 for (int i = 0; i < KI; ++i) {
-                  a[q][i] = fast_exp2(dl[i] * A2);
-                  bb[q][i] = du[i] * Bv[i];
+                  Cv[s][i] = ops.Cv[s][i];
+                  a[s][i] = fast_exp2(dl[i] * A2);
+                  bb[s][i] = du[i] * ops.Bv[s][i];
                 }
-                if constexpr (!LS) {
-                  sa[q] = fast_exp2(dsum * A2);
-                  float hl = bb[q][0];
+                sa[s] = fast_exp2(dsum * A2);
+                float hl = bb[s][0];
 #pragma unroll
-                  for (int i = 1; i < KI; ++i) hl = __builtin_fmaf(a[q][i], hl, bb[q][i]);
-                  sb[q] = hl;
-                }
+                for (int i = 1; i < KI; ++i) hl = __builtin_fmaf(a[s][i], hl, bb[s][i]);
+                sb[s] = hl;
               }
-              if constexpr (!LS) {
-                if constexpr (Q == 2) wave_scan_fwd2(sa[0], sb[0], sa[1], sb[1]);
-                else wave_scan_fwd(sa[0], sb[0]);
+              row_scan_fwd2(sa[0], sb[0], sa[1], sb[1]);
 #pragma unroll
-                for (int q = 0; q < Q; ++q) hend[q] = __builtin_fmaf(sa[q], hc[q], sb[q]);
-              }
-              float ra[Q], rb[Q], gfirst[Q], a_next_lane[Q];
+              for (int s = 0; s < 2; ++s) hend[s] = __builtin_fmaf(sa[s], hc[s], sb[s]);
+              float ra[2], rb[2];
 #pragma unroll
-              for (int q = 0; q < Q; ++q) {
-                float hp;
-                if constexpr (LS) hp = hin[q];
-                else hp = dpp_f<DPP_WAVE_SHR1>(hc[q], hend[q]);
+              for (int s = 0; s < 2; ++s) {
+                float hp = dpp_f<DPP_ROW_SHR + 1>(hc[s], hend[s]);
 #pragma unroll
                 for (int i = 0; i < KI; ++i) {
-                  hp = __builtin_fmaf(a[q][i], hp, bb[q][i]);
-                  h[q][i] = hp;  // true states
+                  hp = __builtin_fmaf(a[s][i], hp, bb[s][i]);
+                  h[s][i] = hp;  // true states
                 }
                 if (has_z) {
 #pragma unroll
-                  for (int i = 0; i < KI; ++i) y[i] = __builtin_fmaf(h[q][i], Cv[q][i], y[i]);
+                  for (int i = 0; i < KI; ++i) y[i] = __builtin_fmaf(h[s][i], Cv[s][i], y[i]);
                 }
                 // adjoint recurrence g[t] = dy[t] C[t] + a[t+1] g[t+1]; Cv becomes dy * C
-                a_next_lane[q] = dpp_f<DPP_WAVE_SHL1>(an[q], a[q][0]);
+                a_next_lane[s] = dpp_f<DPP_ROW_SHL + 1>(an[s], a[s][0]);
 #pragma unroll
-                for (int i = 0; i < KI; ++i) Cv[q][i] *= dy[i];
-                float gl = Cv[q][KI - 1];
+                for (int i = 0; i < KI; ++i) Cv[s][i] *= dy[i];
+                float gl = Cv[s][KI - 1];
 #pragma unroll
-                for (int i = KI - 2; i >= 0; --i) gl = __builtin_fmaf(a[q][i + 1], gl, Cv[q][i]);
-                ra[q] = fast_exp2(dtail * (A1[q] * kLog2e)) * a_next_lane[q];
-                rb[q] = gl;
+                for (int i = KI - 2; i >= 0; --i) gl = __builtin_fmaf(a[s][i + 1], gl, Cv[s][i]);
+                ra[s] = fast_exp2(dtail * (A1[s] * kLog2e)) * a_next_lane[s];
+                rb[s] = gl;
               }
-              if constexpr (Q == 2) {
-                row_scan_rev2(ra[0], rb[0], ra[1], rb[1]);
-                wave_scan_rev_finish(ra[0], rb[0], lane);
-                wave_scan_rev_finish(ra[1], rb[1], lane);
-              } else {
-                wave_scan_rev(ra[0], rb[0], lane);
-              }
+              row_scan_rev2(ra[0], rb[0], ra[1], rb[1]);
 #pragma unroll
-              for (int q = 0; q < Q; ++q) gfirst[q] = __builtin_fmaf(ra[q], gc[q], rb[q]);
+              for (int s = 0; s < 2; ++s) gfirst[s] = __builtin_fmaf(ra[s], gc[s], rb[s]);
+            }
+            if (early) __syncthreads();  // the early waves meet the others here, between the two halves
+            if (active) {
 #pragma unroll
-              for (int q = 0; q < Q; ++q) {
-                const float gx = dpp_f<DPP_WAVE_SHL1>(gc[q], gfirst[q]);  // adjoint at the next lane's first item
-                if (lane == 0) {
-                  grow[n + q] = gfirst[q];
-                  arow[n + q] = a[q][0];
+              for (int s = 0; s < 2; ++s) {
+                const float gx = dpp_f<DPP_ROW_SHL + 1>(gc[s], gfirst[s]);  // adjoint at the next lane's first item
+                if (c == 0) {
+                  grow[n + s] = gfirst[s];
+                  arow[n + s] = a[s][0];
                 }
                 float dAp = 0.f, dBp = 0.f, dCp = 0.f;
                 float sB[8], sC[8], Bv[8];
-                load_bc<BC & 1>(Bv, Bs, p.B, d, N, nb * NB16 + n + q, n + q, lane);
-                if constexpr (!(BC & 1)) lds_ld8(dBs + (n + q) * TILE, lane, sB);
-                if constexpr (!(BC & 2)) lds_ld8(dCs + (n + q) * TILE, lane, sC);
-                float gi = gx, an_i = a_next_lane[q];
+                load_bc<BC & 1>(Bv, Bs, p.B, d, N, nb * NB16 + n + s, n + s, c);
+                if constexpr (!(BC & 1)) lds_ld8<4 * 64>(dBs + (n + s) * ACC_PITCH, lane, sB);
+                if constexpr (!(BC & 2)) lds_ld8<4 * 64>(dCs + (n + s) * ACC_PITCH, lane, sC);
+                float gi = gx, an_i = a_next_lane[s];
 #pragma unroll
                 for (int i = KI - 1; i >= 0; --i) {
-                  gi = __builtin_fmaf(an_i, gi, Cv[q][i]);
-                  an_i = a[q][i];
-                  if constexpr (BC & 2) dCp = __builtin_fmaf(dy[i], h[q][i], dCp);
-                  else sC[i] = __builtin_fmaf(dy[i], h[q][i], sC[i]);
+                  gi = __builtin_fmaf(an_i, gi, Cv[s][i]);
+                  an_i = a[s][i];
+                  if constexpr (BC & 2) dCp = __builtin_fmaf(dy[i], h[s][i], dCp);
+                  else sC[i] = __builtin_fmaf(dy[i], h[s][i], sC[i]);
                   if constexpr (BC & 1) dBp = __builtin_fmaf(gi, du[i], dBp);
                   else sB[i] = __builtin_fmaf(gi, du[i], sB[i]);
                   acc[i] = __builtin_fmaf(gi, Bv[i], acc[i]);
-                  const float w = gi * (h[q][i] - bb[q][i]);  // g * a * h[t-1]
-                  dd[i] = __builtin_fmaf(A1[q], w, dd[i]);
+                  const float w = gi * (h[s][i] - bb[s][i]);  // g * a * h[t-1]
+                  dd[i] = __builtin_fmaf(A1[s], w, dd[i]);
                   dAp = __builtin_fmaf(dl[i], w, dAp);
                 }
-                if constexpr (!(BC & 1)) lds_st8(dBs + (n + q) * TILE, lane, sB);
-                if constexpr (!(BC & 2)) lds_st8(dCs + (n + q) * TILE, lane, sC);
-                dAp = wave_sum_to_last(dAp);
-                if (lane == 63) dArow[n + q] += dAp;  // the row belongs to this wave alone
+                if constexpr (!(BC & 1)) lds_st8<4 * 64>(dBs + (n + s) * ACC_PITCH, lane, sB);
+                if constexpr (!(BC & 2)) lds_st8<4 * 64>(dCs + (n + s) * ACC_PITCH, lane, sC);
+                dAp = row_sum_to_last(dAp);
+                if (c == RL - 1) dArow[n + s] += dAp;  // the slot belongs to this row alone
                 if constexpr (BC & 1) {
-                  dBp = wave_sum_to_last(dBp);
-                  if (lane == 63) dBcacc[row * NP + nb * NB16 + n + q] += dBp;
+                  dBp = row_sum_to_last(dBp);
+                  if (c == RL - 1) dBcacc[chw * NP + nb * NB16 + n + s] += dBp;
                 }
                 if constexpr (BC & 2) {
-                  dCp = wave_sum_to_last(dCp);
-                  if (lane == 63) dCcacc[row * NP + nb * NB16 + n + q] += dCp;
+                  dCp = row_sum_to_last(dCp);
+                  if (c == RL - 1) dCcacc[chw * NP + nb * NB16 + n + s] += dCp;
                 }
               }
             }
-            __syncthreads();
+            if (ph + 1 < NPH) fetch_operands(ops, ph + 1);
+            if (!early) __syncthreads();
           }
         }
-        if (BC != 3 && (NBLK > 1 || r == R - 1)) {
+        if (BC != 3 && (NBLK > 1 || r == npass - 1)) {
+          __syncthreads();  // waves 0-3 add their last sums after the last barrier of the phases
+          // One partial per workgroup: the sum over the 4 channel slots of every (state, position), written
+          // with plain stores (positions past the end and padded states are skipped).
           const int n0 = nb * NB16;
-          constexpr int FIRST = (BC & 1) ? NB16 * TILE : 0, LAST = (BC & 2) ? NB16 * TILE : 2 * NB16 * TILE;
-          for (int i = FIRST + tid; i < LAST; i += NW * 64) {
-            const int which = i >> 13, n = (i >> 9) & 15, t = i & (TILE - 1);
-            const float v = (which ? dCs : dBs)[n * TILE + ((t >> 2) & 1) * 256 + (t >> 3) * 4 + (t & 3)];
-            if (n0 + n < N && t0 + t < L) unsafeAtomicAdd((which ? dCg : dBg) + (int64_t)(n0 + n) * L + t0 + t, v);
+          const int64_t part = part0 + (NBLK > 1 ? r : 0);
+          constexpr int FIRST = (BC & 1) ? NB16 * TILE / 4 : 0, LAST = (BC & 2) ? NB16 * TILE / 4 : 2 * NB16 * TILE / 4;
+          for (int o = FIRST + tid; o < LAST; o += NTHREADS) {
+            const int which = o >> 9, n = (o >> 5) & 15, q4 = o & 31;  // positions 4 q4 .. 4 q4 + 3 of state n
+            const float *src = (which ? dCs : dBs) + n * ACC_PITCH + (q4 & 1) * 256 + (q4 >> 1) * 4;
+            f32x4 v = *reinterpret_cast<const f32x4 *>(src);
+#pragma unroll
+            for (int k = 1; k < ROWS; ++k) {
+              const f32x4 w = *reinterpret_cast<const f32x4 *>(src + k * RL * 4);
+              v.x += w.x; v.y += w.y; v.z += w.z; v.w += w.w;
+            }
+            const int t = t0 + 4 * q4;
+            if (n0 + n >= N || t >= L) continue;
+            float *dst = (which ? p.dC32 : p.dB32) + (part * N + n0 + n) * L + t;
+            if (VEC) {
+              *reinterpret_cast<f32x4 *>(dst) = v;
+            } else {
+              dst[0] = v.x;
+              if (t + 1 < L) dst[1] = v.y;
+              if (t + 2 < L) dst[2] = v.z;
+              if (t + 3 < L) dst[3] = v.w;
+            }
           }
         }
       }
-      if (valid) {
+      {
         float draw[8], o[8];
         draw_k.unpack(draw);
-        const BwdRow<T> q = rows[row];
-        const float bias = q.bias;
+        const BwdRow<T> w = rows[chw];
         float dbs = 0.f, dDs = 0.f;
 #pragma unroll
         for (int i = 0; i < KI; ++i) o[i] = __builtin_fmaf(dl[i], acc[i], Dd * dy[i]);
-        st8_guard<T, VEC>(q.du + tl, nvalid, o);
+        st8_guard<T, VEC>(w.du + tl, nvalid, o);
 #pragma unroll
         for (int i = 0; i < KI; ++i) {
-          const float x = draw[i] + bias;
           float gd = __builtin_fmaf(u[i], acc[i], dd[i]);
-          if (p.delta_softplus && x <= 20.f) gd *= sigmoid_f(x);
+          if (p.delta_softplus) gd *= sigmoid_f(draw[i] + bias);  // (above the softplus threshold of 20 it rounds to 1)
           gd = (i < nvalid) ? gd : 0.f;
           o[i] = gd;
           dbs += gd;
           dDs = __builtin_fmaf(dy[i], u[i], dDs);
         }
-        st8_guard<T, VEC>(q.ddelta + tl, nvalid, o);
+        st8_guard<T, VEC>(w.ddelta + tl, nvalid, o);
         if (has_z) {
           float z[8], dout[8], oz[8];
           z_k.unpack(z);
@@ -618,31 +621,64 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
             o[i] = dout[i] * yf * s * (1.f + z[i] * (1.f - s));
             oz[i] = yf * z[i] * s;
           }
-          st8_guard<T, VEC>(q.dz + tl, nvalid, o);
-          if (q.out_z) st8_guard<T, VEC>(q.out_z + tl, nvalid, oz);
+          st8_guard<T, VEC>(w.dz + tl, nvalid, o);
+          if (w.out_z) st8_guard<T, VEC>(w.out_z + tl, nvalid, oz);
         }
-        dbs = wave_sum_to_last(dbs);
-        dDs = wave_sum_to_last(dDs);
-        if (lane == 63) {
-          dbacc[row] += dbs;
-          dDacc[row] += dDs;
+        dbs = row_sum_to_last(dbs);
+        dDs = row_sum_to_last(dDs);
+        if (c == RL - 1) {
+          dbacc[chw] += dbs;
+          dDacc[chw] += dDs;
         }
       }
     }
   }
+  __syncthreads();
   // per-(batch, channel) partial sums; the caller reduces over batch
-  for (int r = 0; r < R; ++r) {
-    const int d = dbase + r;
-    if (d >= dend) continue;
-    const int row = wave * R + r;
-    for (int n = lane; n < N; n += 64) {
-      p.dA_part[((int64_t)b * p.dim + d) * N + n] = dAacc[row * NP + n];
-      if constexpr (BC & 1) p.dB32[((int64_t)b * p.dim + d) * N + n] = dBcacc[row * NP + n];
-      if constexpr (BC & 2) p.dC32[((int64_t)b * p.dim + d) * N + n] = dCcacc[row * NP + n];
+  for (int i = tid; i < WCH * N; i += NTHREADS) {
+    const int ch = i / N, n = i % N, d = d0 + ch;
+    if (d >= q.dend) continue;
+    p.dA_part[((int64_t)b * p.dim + d) * N + n] = dAacc[ch * NP + n];
+    if constexpr (BC & 1) p.dB32[((int64_t)b * p.dim + d) * N + n] = dBcacc[ch * NP + n];
+    if constexpr (BC & 2) p.dC32[((int64_t)b * p.dim + d) * N + n] = dCcacc[ch * NP + n];
+  }
+  for (int ch = tid; ch < WCH; ch += NTHREADS) {
+    const int d = d0 + ch;
+    if (d >= q.dend) continue;
+    p.dD_part[(int64_t)b * p.dim + d] = dDacc[ch];
+    p.ddelta_bias_part[(int64_t)b * p.dim + d] = dbacc[ch];
+  }
+}
+
+// out[row, e] = sum over parts of part[row, part, e], in the order of the parts, converted to T; one
+// thread per 4 consecutive elements e of the row's `row_len`.
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void reduce_parts_kernel(const float *__restrict__ parts, T *__restrict__ out,
+                                                           int64_t rows, int nparts, int64_t row_len) {
+  const int64_t quad = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t per_row = (row_len + 3) / 4;
+  if (quad >= rows * per_row) return;
+  const int64_t row = quad / per_row, e = (quad - row * per_row) * 4;
+  const float *src = parts + row * nparts * row_len + e;
+  T *dst = out + row * row_len + e;
+  if (VEC) {
+    f32x4 v = *reinterpret_cast<const f32x4 *>(src);
+    for (int k = 1; k < nparts; ++k) {
+      const f32x4 w = *reinterpret_cast<const f32x4 *>(src + (int64_t)k * row_len);
+      v.x += w.x; v.y += w.y; v.z += w.z; v.w += w.w;
     }
-    if (lane == 0) {
-      p.dD_part[(int64_t)b * p.dim + d] = dDacc[row];
-      p.ddelta_bias_part[(int64_t)b * p.dim + d] = dbacc[row];
+    if constexpr (DT<T>::id == MAMBA_F32) {
+      *reinterpret_cast<f32x4 *>(dst) = v;
+    } else if constexpr (DT<T>::id == MAMBA_BF16) {
+      *reinterpret_cast<u32x2 *>(dst) = u32x2{pack_bf16(v.x, v.y), pack_bf16(v.z, v.w)};
+    } else {
+      *reinterpret_cast<u32x2 *>(dst) = u32x2{pack_f16(v.x, v.y), pack_f16(v.z, v.w)};
+    }
+  } else {
+    for (int i = 0; i < 4 && e + i < row_len; ++i) {
+      float v = src[i];
+      for (int k = 1; k < nparts; ++k) v += src[(int64_t)k * row_len + i];
+      st1<T>(dst + i, v);
     }
   }
 }
@@ -650,26 +686,66 @@ __global__ __launch_bounds__(NW * 64) void scan_bwd_kernel(const MambaScanParams
 // ------------------------------------------------------------------ launch
 inline bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
 
-struct Cfg {
-  int nw, r;
-};
+inline size_t fwd_lds(int passes, int np) { return sizeof(float) * (2 * BC_FLOATS + 2 * passes * PASS_CH * np); }
+inline size_t bwd_lds(int passes, int np, int bc) {
+  const int wch = passes * PASS_CH;
+  return sizeof(float) * (2 * BC_FLOATS + 2 * ACC_FLOATS + PASS_CH * np + (bc ? 6 : 4) * wch * np + 2 * wch) +
+         (size_t)wch * 80;  // + BwdRow per channel
+}
+constexpr size_t LDS_LIMIT = 160 * 1024;
 
-inline size_t fwd_lds(int nw, int r, int np) { return sizeof(float) * (2 * BC_FLOATS + 2 * nw * r * np); }
-inline size_t bwd_lds(int nw, int r, int np) {
-  return sizeof(float) * (4 * BC_FLOATS + 7 * nw * r * np + 2 * nw * r) + (size_t)nw * r * 80;  // + BwdRow per channel
+int compute_units() {
+  static int cus = 0;
+  if (cus > 0) return cus;
+  int dev = 0, n = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+    (void)hipGetLastError();
+    return 256;  // not cached: asked again on the next call
+  }
+  cus = n;
+  return n;
+}
+
+// Passes of PASS_CH channels a backward workgroup takes per tile.  More passes mean fewer, larger
+// partials of dB / dC; the count is chosen so that the workgroups still fill whole rounds over the
+// compute units (one workgroup per unit): the smallest rounds * passes wins, ties go to more passes.
+int bwd_passes(const MambaScanParams &p) {
+  const int np = (p.dstate + NB16 - 1) / NB16 * NB16;
+  if (np > NB16) return 1;  // states in blocks: the sums leave after every block
+  const int Dg = p.dim / p.ngroups, cus = compute_units();
+  int best = 1;
+  int64_t best_cost = -1;
+  for (int r = 1; r <= MAX_PASSES; ++r) {
+    if (bwd_lds(r, np, p.bc_const & 3) > LDS_LIMIT) break;
+    if (r > 1 && (r - 1) * PASS_CH >= Dg) break;
+    const int64_t wgs = (int64_t)p.batch * p.ngroups * ((Dg + PASS_CH * r - 1) / (PASS_CH * r));
+    const int64_t cost = (wgs + cus - 1) / cus * r;
+    if (best_cost < 0 || cost <= best_cost) {
+      best_cost = cost;
+      best = r;
+    }
+  }
+  return best;
+}
+
+int bwd_nparts(const MambaScanParams &p) {
+  const int Dg = p.dim / p.ngroups, r = bwd_passes(p);
+  return (Dg + PASS_CH * r - 1) / (PASS_CH * r) * (p.dstate > NB16 ? r : 1);
 }
 
 template <typename KernelT>
-int launch(KernelT kernel, const MambaScanParams &p, int nw, int r, size_t lds, hipStream_t stream) {
+int launch(KernelT kernel, const MambaScanParams &p, int passes, size_t lds, hipStream_t stream) {
   const int Dg = p.dim / p.ngroups;
-  const int cblocks = (Dg + nw * r - 1) / (nw * r);
+  const int cblocks = (Dg + PASS_CH * passes - 1) / (PASS_CH * passes);
+  if (lds > LDS_LIMIT) return MAMBA_E_UNSUPPORTED;
   if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                           (int)lds) != hipSuccess) {
     (void)hipGetLastError();
     return MAMBA_E_LAUNCH;
   }
-  dim3 grid(p.ngroups * cblocks, p.batch), block(nw * 64);
-  hipLaunchKernelGGL(kernel, grid, block, lds, stream, p);
+  dim3 grid(p.ngroups * cblocks, p.batch), block(NTHREADS);
+  hipLaunchKernelGGL(kernel, grid, block, lds, stream, p, passes);
   return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
 }
 
@@ -693,39 +769,48 @@ bool vec_ok(const MambaScanParams &p, bool bwd) {
   if (!(p.bc_const & 1)) v = v && ok(p.B, p.B_bs, p.B_gs) && p.B_ns % m == 0;
   if (!(p.bc_const & 2)) v = v && ok(p.C, p.C_bs, p.C_gs) && p.C_ns % m == 0;
   if (!bwd) return v && ok(p.out, p.out_bs, p.out_ds);
+  if (!(p.bc_const & 1)) v = v && aligned16(p.dB32);
+  if (!(p.bc_const & 2)) v = v && aligned16(p.dC32);
   return v && ok(p.dout, p.dout_bs, p.dout_ds) && ok(p.du, p.du_bs, p.du_ds) &&
          ok(p.ddelta, p.ddelta_bs, p.ddelta_ds) && ok(p.dz, p.dz_bs, p.dz_ds) && ok(p.out_z, p.outz_bs, p.outz_ds);
+}
+
+template <typename T>
+int reduce_parts(const float *parts, void *out, int64_t rows, int nparts, int64_t row_len, hipStream_t stream) {
+  const int64_t quads = rows * ((row_len + 3) / 4);
+  if ((quads + 255) / 256 > 0x7fffffff) return MAMBA_E_UNSUPPORTED;
+  const dim3 grid((unsigned)((quads + 255) / 256)), block(256);
+  T *o = static_cast<T *>(out);
+  if (row_len % 4 == 0 && aligned16(parts) && aligned16(out))
+    hipLaunchKernelGGL((reduce_parts_kernel<T, true>), grid, block, 0, stream, parts, o, rows, nparts, row_len);
+  else
+    hipLaunchKernelGGL((reduce_parts_kernel<T, false>), grid, block, 0, stream, parts, o, rows, nparts, row_len);
+  return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
+}
+
+// dB / dC of per-position operands: the partials summed in a fixed order into the outputs
+template <typename T> int reduce_dBC(const MambaScanParams &p, int nparts, hipStream_t stream) {
+  const int64_t rows = (int64_t)p.batch * p.ngroups;
+  const int64_t row_len = (int64_t)p.dstate * p.seqlen * (p.a_complex ? 2 : 1);
+  int rc = MAMBA_OK;
+  if (!(p.bc_const & 1)) rc = reduce_parts<T>(p.dB32, p.dB, rows, nparts, row_len, stream);
+  if (rc == MAMBA_OK && !(p.bc_const & 2)) rc = reduce_parts<T>(p.dC32, p.dC, rows, nparts, row_len, stream);
+  return rc;
 }
 
 template <typename T, bool BWD, int BC> int dispatch_bc(const MambaScanParams &p, hipStream_t stream) {
   const int np = (p.dstate + NB16 - 1) / NB16 * NB16;
   const bool vec = vec_ok(p, BWD);
-  const bool small = p.dstate <= NB16;
   if (!BWD) {
-    if (small) {
-      const size_t lds = fwd_lds(8, 4, np);
-      return vec ? launch(scan_fwd_kernel<T, 8, 4, true, BC>, p, 8, 4, lds, stream)
-                 : launch(scan_fwd_kernel<T, 8, 4, false, BC>, p, 8, 4, lds, stream);
-    }
-    const size_t lds = fwd_lds(8, 1, np);
-    return vec ? launch(scan_fwd_kernel<T, 8, 1, true, BC>, p, 8, 1, lds, stream)
-               : launch(scan_fwd_kernel<T, 8, 1, false, BC>, p, 8, 1, lds, stream);
-  } else {
-    if (small) {
-      const size_t lds = bwd_lds(8, 4, np);
-      if (p.lane_state)
-        return vec ? launch(scan_bwd_kernel<T, 8, 4, true, BC, true>, p, 8, 4, lds, stream)
-                   : launch(scan_bwd_kernel<T, 8, 4, false, BC, true>, p, 8, 4, lds, stream);
-      return vec ? launch(scan_bwd_kernel<T, 8, 4, true, BC, false>, p, 8, 4, lds, stream)
-                 : launch(scan_bwd_kernel<T, 8, 4, false, BC, false>, p, 8, 4, lds, stream);
-    }
-    const size_t lds = bwd_lds(4, 1, np);
-    if (p.lane_state)
-      return vec ? launch(scan_bwd_kernel<T, 4, 1, true, BC, true>, p, 4, 1, lds, stream)
-                 : launch(scan_bwd_kernel<T, 4, 1, false, BC, true>, p, 4, 1, lds, stream);
-    return vec ? launch(scan_bwd_kernel<T, 4, 1, true, BC, false>, p, 4, 1, lds, stream)
-               : launch(scan_bwd_kernel<T, 4, 1, false, BC, false>, p, 4, 1, lds, stream);
+    const size_t lds = fwd_lds(1, np);
+    return vec ? launch(scan_fwd_kernel<T, true, BC>, p, 1, lds, stream)
+               : launch(scan_fwd_kernel<T, false, BC>, p, 1, lds, stream);
   }
+  const int passes = bwd_passes(p);
+  const size_t lds = bwd_lds(passes, np, BC);
+  const int rc = vec ? launch(scan_bwd_kernel<T, true, BC>, p, passes, lds, stream)
+                     : launch(scan_bwd_kernel<T, false, BC>, p, passes, lds, stream);
+  return rc != MAMBA_OK ? rc : reduce_dBC<T>(p, bwd_nparts(p), stream);
 }
 
 template <typename T, bool BWD> int dispatch(const MambaScanParams &p, hipStream_t stream) {
@@ -798,7 +883,8 @@ extern "C" int mamba_hip_init(void) { return scratch_for_current_device() ? MAMB
 extern "C" int mamba1_scan_fwd_noalloc(const MambaScanParams *p, float *last_state, mamba_stream_t stream) {
   if (!p) return MAMBA_E_BADARG;
   if (p->batch <= 0 || p->dim <= 0 || p->seqlen <= 0 || p->dstate <= 0) return MAMBA_E_BADARG;
-  const int ntiles = (p->seqlen + TILE - 1) / TILE;
+  const int tile = p->a_complex ? TILE_COMPLEX : TILE;
+  const int ntiles = (p->seqlen + tile - 1) / tile;
   const int width = p->dstate * (p->a_complex ? 2 : 1);
   const int64_t rows = (int64_t)p->batch * p->dim;
   if (rows * ntiles > SCRATCH_FLOATS / width) return MAMBA_E_UNSUPPORTED;  // checkpoints beyond the fixed buffer
@@ -806,7 +892,6 @@ extern "C" int mamba1_scan_fwd_noalloc(const MambaScanParams *p, float *last_sta
   if (!ws) return MAMBA_E_LAUNCH;
   MambaScanParams q = *p;
   q.ckpt = ws;
-  q.lane_state = nullptr;
   const int rc = mamba1_scan_fwd(&q, stream);
   if (rc != MAMBA_OK || !last_state) return rc;
   const int64_t n = rows * width;
@@ -816,14 +901,35 @@ extern "C" int mamba1_scan_fwd_noalloc(const MambaScanParams *p, float *last_sta
   return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
 }
 
+extern "C" int mamba1_scan_bwd_nparts(const MambaScanParams *p) {
+  if (!p || p->batch <= 0 || p->dim <= 0 || p->seqlen <= 0 || p->dstate <= 0 || p->ngroups <= 0 ||
+      p->dim % p->ngroups != 0)
+    return MAMBA_E_BADARG;
+  if (p->dstate > MAX_DSTATE) return MAMBA_E_UNSUPPORTED;
+  return p->a_complex ? 1 : bwd_nparts(*p);
+}
+
 extern "C" int mamba1_scan_bwd(const MambaScanParams *p, mamba_stream_t stream) {
   int rc = check_common(p);
   if (rc != MAMBA_OK) return rc;
   if (!p->dout || !p->du || !p->ddelta || !p->dB32 || !p->dC32 || !p->dA_part || !p->dD_part || !p->ddelta_bias_part)
     return MAMBA_E_BADARG;
+  if ((!(p->bc_const & 1) && !p->dB) || (!(p->bc_const & 2) && !p->dC)) return MAMBA_E_BADARG;
   if (p->z && !p->dz) return MAMBA_E_BADARG;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (p->a_complex) return mamba1_scan_complex(p, s, true);
+  if (p->a_complex) {
+    // the complex kernels add their dB / dC terms into one fp32 copy with atomics: clear it, run, convert
+    const int64_t bytes = (int64_t)p->batch * p->ngroups * p->dstate * 2 * p->seqlen * 4;
+    if (!(p->bc_const & 1)) rc = mamba_hip_zero(p->dB32, bytes, stream);
+    if (rc == MAMBA_OK && !(p->bc_const & 2)) rc = mamba_hip_zero(p->dC32, bytes, stream);
+    if (rc == MAMBA_OK) rc = mamba1_scan_complex(p, s, true);
+    if (rc != MAMBA_OK) return rc;
+    switch (p->dtype) {
+      case MAMBA_F32: return reduce_dBC<float>(*p, 1, s);
+      case MAMBA_BF16: return reduce_dBC<bf16_t>(*p, 1, s);
+      default: return reduce_dBC<f16_t>(*p, 1, s);
+    }
+  }
   switch (p->dtype) {
     case MAMBA_F32: return dispatch<float, true>(*p, s);
     case MAMBA_BF16: return dispatch<bf16_t, true>(*p, s);

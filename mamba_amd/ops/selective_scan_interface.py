@@ -20,8 +20,9 @@ from mamba_amd.ops.causal_conv1d import causal_conv1d_bwd, causal_conv1d_fwd
 _FLOAT_TYPES = (torch.float32, torch.bfloat16, torch.float16)
 
 
-def scan_tile():
-    return _lib.load().mamba_hip_query(1)
+def scan_tile(complex_A=False):
+    """Positions per checkpoint tile of the scan (MAMBA_Q_SCAN_TILE / MAMBA_Q_SCAN_TILE_COMPLEX)."""
+    return _lib.load().mamba_hip_query(5 if complex_A else 1)
 
 
 def _check_inputs(u, delta, A, B, C, D, z, delta_bias):
@@ -101,34 +102,18 @@ def _fill_common(p, u, delta, A, B, C, D, z, delta_bias, delta_softplus, ckpt, d
         p.C_bs, p.C_gs, p.C_ns = C.stride(0), C.stride(1), C.stride(2)
 
 
-# Keep the state entering every lane's 8 positions from the forward pass for the backward pass
-# (batch * dim * seqlen / 8 * dstate * 4 bytes: 1.3 GB at batch 8, dim 5120, seqlen 4096, dstate 16).  The
-# backward kernel then skips its own scan over each tile, about a tenth of its instructions.  False
-# makes it re-run that scan and keeps only the per-tile checkpoints.
-KEEP_LANE_STATES = False
-KEEP_LANE_STATES_MAX_BYTES = 16 << 30   # above this size per call the buffer is not kept
-
-
-def _keep_lane_states(u, A):
-    batch, dim, seqlen = u.shape
-    ntiles = (seqlen + scan_tile() - 1) // scan_tile()
-    return (KEEP_LANE_STATES and not A.is_complex()
-            and batch * dim * ntiles * A.shape[1] * 64 * 4 <= KEEP_LANE_STATES_MAX_BYTES)
-
-
-def selective_scan_fwd(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta_softplus=False, lane_states=None):
+def selective_scan_fwd(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta_softplus=False):
     """Counterpart of selective_scan_cuda.fwd (selective_scan.cpp:226).
 
-    Returns (out, ckpt), or (out, ckpt, lanes) when lane_states is True or False (lanes None if False): `out` is the gated output
-    y*silu(z) when z is given, else y, in u's dtype; `ckpt` is (batch, dim, ntiles, dstate) fp32, the
-    state after each tile of `scan_tile()` positions (ckpt[:, :, -1] is the last state); `lanes` is
-    (batch, dim, ntiles, dstate, 64) fp32, the state entering each lane's 8 positions (None with a
-    complex A).  The ungated y is not stored: the backward pass re-computes it.
+    Returns (out, ckpt): `out` is the gated output y*silu(z) when z is given, else y, in u's dtype;
+    `ckpt` is (batch, dim, ntiles, dstate) fp32, the state after each tile of `scan_tile()` positions
+    (ckpt[:, :, -1] is the last state).  The ungated y is not stored: the backward pass re-computes it.
     """
     dims = _check_inputs(u, delta, A, B, C, D, z, delta_bias)
     batch, dim, seqlen, dstate, _ = dims
     A = A.contiguous()
-    ntiles = (seqlen + scan_tile() - 1) // scan_tile()
+    tile = scan_tile(A.is_complex())
+    ntiles = (seqlen + tile - 1) // tile
     out = torch.empty_like(delta)
     ckpt = torch.empty((batch, dim, ntiles, dstate) + ((2,) if A.is_complex() else ()), device=u.device,
                        dtype=torch.float32)
@@ -136,33 +121,26 @@ def selective_scan_fwd(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta
     _fill_common(p, u, delta, A, B, C, D, z, delta_bias, delta_softplus, ckpt, dims)
     p.out = out.data_ptr()
     p.out_bs, p.out_ds = out.stride(0), out.stride(1)
-    lanes = None
-    if lane_states and not A.is_complex():
-        lanes = torch.empty((batch, dim, ntiles, dstate, 64), device=u.device, dtype=torch.float32)
-        p.lane_state = lanes.data_ptr()
     with torch.cuda.device(u.device):
         _lib.check(_lib.load().mamba1_scan_fwd(p, _lib.current_stream(u.device)), "mamba1_scan_fwd")
-    return (out, ckpt, lanes) if lane_states is not None else (out, ckpt)
+    return out, ckpt
 
 
 class ScanBwdBuffers:
-    """Outputs and fp32 accumulators of one backward launch (all caller-owned)."""
+    """Outputs and fp32 workspaces of one backward launch (all caller-owned).  `nparts` is
+    mamba1_scan_bwd_nparts for the launch's sizes."""
 
-    def __init__(self, u, delta, B, z, dims, dz=None, recompute_out_z=False, C=None, complex_A=False):
+    def __init__(self, u, delta, B, z, dims, dz=None, recompute_out_z=False, C=None, complex_A=False, nparts=1):
         batch, dim, seqlen, dstate, ngroups = dims
         dev = u.device
         self.du = torch.empty_like(u)
         self.ddelta = torch.empty_like(delta)
-        # one fp32 arena: per operand (batch, ngroups, dstate, seqlen) sums the kernel adds into, or
-        # (batch, dim, dstate) per-batch partials when the operand is an input-independent matrix;
-        # with a complex A every entry is a (re, im) pair
+        # per operand: (batch, ngroups, nparts, dstate, seqlen) partial sums, one per workgroup, which the
+        # call adds up into dB / dC in the operand's dtype; or (batch, dim, dstate) per-batch partials
+        # when the operand is an input-independent matrix; with a complex A every entry is a (re, im) pair
         two = 2 if complex_A else 1
-        shapes = [(batch, dim, dstate * two) if (t is not None and t.dim() == 2)
-                  else (batch, ngroups, dstate, seqlen * two) for t in (B, C)]
-        sizes = [math.prod(sh) for sh in shapes]
-        self.dBC32 = torch.empty(sum(sizes), device=dev, dtype=torch.float32)
-        self.dB32 = self.dBC32[:sizes[0]].view(shapes[0])
-        self.dC32 = self.dBC32[sizes[0]:].view(shapes[1])
+        self.dB32, self.dB = self._operand(B, batch, dim, ngroups, nparts, dstate, seqlen, two, dev)
+        self.dC32, self.dC = self._operand(C, batch, dim, ngroups, nparts, dstate, seqlen, two, dev)
         self.dA_part = torch.empty(batch, dim, dstate * two, device=dev, dtype=torch.float32)
         self.dD_part = torch.empty(batch, dim, device=dev, dtype=torch.float32)
         self.dbias_part = torch.empty(batch, dim, device=dev, dtype=torch.float32)
@@ -172,23 +150,32 @@ class ScanBwdBuffers:
             if recompute_out_z:
                 self.out_z = torch.empty_like(u)
 
+    @staticmethod
+    def _operand(t, batch, dim, ngroups, nparts, dstate, seqlen, two, dev):
+        if t is not None and t.dim() == 2:
+            return torch.empty(batch, dim, dstate * two, device=dev, dtype=torch.float32), None
+        part = torch.empty(batch, ngroups, nparts, dstate, seqlen * two, device=dev, dtype=torch.float32)
+        return part, torch.empty(batch, ngroups, dstate, seqlen * two, device=dev, dtype=t.dtype)
 
-def scan_bwd_zero(bufs, device):
-    """Clears the dB/dC accumulators (the kernel adds into them) with the library's fill kernel."""
-    with torch.cuda.device(device):
-        _lib.check(_lib.load().mamba_hip_zero(bufs.dBC32.data_ptr(), bufs.dBC32.numel() * 4,
-                                              _lib.current_stream(device)), "mamba_hip_zero")
 
-
-def scan_bwd_launch(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, delta_softplus, bufs, dims, lanes=None):
-    """One call of the C ABI's mamba1_scan_bwd on the current stream; bufs.dBC32 must be zero."""
+def scan_bwd_launch(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, delta_softplus, dims, dz=None,
+                    recompute_out_z=False, bufs=None):
+    """One call of the C ABI's mamba1_scan_bwd on the current stream; returns its buffers (allocated
+    here unless the ScanBwdBuffers of an earlier call with the same sizes are passed in)."""
     p = _lib.MambaScanParams()
     _fill_common(p, u, delta, A, B, C, D, z, delta_bias, delta_softplus, ckpt, dims)
-    p.lane_state = _lib.ptr(lanes)
+    lib = _lib.load()
+    if bufs is None:
+        with torch.cuda.device(u.device):
+            nparts = lib.mamba1_scan_bwd_nparts(p)
+        if nparts <= 0:
+            _lib.check(nparts or -1, "mamba1_scan_bwd_nparts")
+        bufs = ScanBwdBuffers(u, delta, B, z, dims, dz, recompute_out_z, C=C, complex_A=A.is_complex(), nparts=nparts)
     dz, out_z = bufs.dz, bufs.out_z
     p.dout, p.du, p.ddelta = dout.data_ptr(), bufs.du.data_ptr(), bufs.ddelta.data_ptr()
     p.dz, p.out_z = _lib.ptr(dz), _lib.ptr(out_z)
     p.dB32, p.dC32 = bufs.dB32.data_ptr(), bufs.dC32.data_ptr()
+    p.dB, p.dC = _lib.ptr(bufs.dB), _lib.ptr(bufs.dC)
     p.dA_part, p.dD_part = bufs.dA_part.data_ptr(), bufs.dD_part.data_ptr()
     p.ddelta_bias_part = bufs.dbias_part.data_ptr()
     p.dout_bs, p.dout_ds = dout.stride(0), dout.stride(1)
@@ -199,17 +186,18 @@ def scan_bwd_launch(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, delta_softp
     if out_z is not None:
         p.outz_bs, p.outz_ds = out_z.stride(0), out_z.stride(1)
     with torch.cuda.device(u.device):
-        _lib.check(_lib.load().mamba1_scan_bwd(p, _lib.current_stream(u.device)), "mamba1_scan_bwd")
+        _lib.check(lib.mamba1_scan_bwd(p, _lib.current_stream(u.device)), "mamba1_scan_bwd")
+    return bufs
 
 
 def selective_scan_bwd(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, dz=None, delta_softplus=False,
-                       recompute_out_z=False, lanes=None):
+                       recompute_out_z=False):
     """Counterpart of selective_scan_cuda.bwd (selective_scan.cpp:338).
 
     `dz` may be a caller-owned strided view (last stride 1) that receives the gate gradient,
-    as MambaInnerFn passes it (selective_scan_interface.py:333-338).  `lanes` is the third result of
-    selective_scan_fwd(..., lane_states=True), or None to re-run the scan over each tile.
-    Returns (du, ddelta, dA, dB, dC, dD, ddelta_bias, dz, out_z).
+    as MambaInnerFn passes it (selective_scan_interface.py:333-338).
+    Returns (du, ddelta, dA, dB, dC, dD, ddelta_bias, dz, out_z).  No float atomics are involved: the
+    same inputs give the same bits every time.
     """
     dims = _check_inputs(u, delta, A, B, C, D, z, delta_bias)
     batch, dim, seqlen, dstate, ngroups = dims
@@ -221,22 +209,17 @@ def selective_scan_bwd(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, dz=None,
         raise RuntimeError("selective_scan: dz must match z in dtype/shape with stride 1 in the last dimension")
     A = A.contiguous()
     cplx = A.is_complex()
-    bufs = ScanBwdBuffers(u, delta, B, z, dims, dz, recompute_out_z, C=C, complex_A=cplx)
-    scan_bwd_zero(bufs, u.device)
-    if lanes is not None:
-        _lib.require_gpu(lanes)
-        ntiles = (seqlen + scan_tile() - 1) // scan_tile()
-        if cplx or lanes.dtype != torch.float32 or tuple(lanes.shape) != (batch, dim, ntiles, dstate, 64) \
-                or not lanes.is_contiguous():
-            raise RuntimeError("selective_scan: lanes must be the contiguous fp32 (batch, dim, ntiles, dstate, 64) "
-                               "tensor of the forward call (real A only)")
-    scan_bwd_launch(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, delta_softplus, bufs, dims, lanes)
+    tile = scan_tile(cplx)
+    want = (batch, dim, (seqlen + tile - 1) // tile, dstate) + ((2,) if cplx else ())
+    if ckpt.dtype != torch.float32 or tuple(ckpt.shape) != want or not ckpt.is_contiguous():
+        raise RuntimeError(f"selective_scan: ckpt must be the contiguous fp32 {want} tensor of the forward call")
+    bufs = scan_bwd_launch(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, delta_softplus, dims, dz, recompute_out_z)
     as_A = (lambda t: torch.view_as_complex(t.reshape(dim, dstate, 2))) if cplx else (lambda t: t)
     dA = as_A(bufs.dA_part.sum(0))
     dD = bufs.dD_part.sum(0) if D is not None else None
     ddelta_bias = bufs.dbias_part.sum(0) if delta_bias is not None else None
-    dB = as_A(bufs.dB32.sum(0)) if B.dim() == 2 else bufs.dB32.to(B.dtype)
-    dC = as_A(bufs.dC32.sum(0)) if C.dim() == 2 else bufs.dC32.to(C.dtype)
+    dB = as_A(bufs.dB32.sum(0)) if B.dim() == 2 else bufs.dB
+    dC = as_A(bufs.dC32.sum(0)) if C.dim() == 2 else bufs.dC
     return (bufs.du, bufs.ddelta, dA, dB, dC, dD, ddelta_bias, bufs.dz, bufs.out_z)
 
 
@@ -265,8 +248,7 @@ class SelectiveScanFn(torch.autograd.Function):
         if C.dim() == 3:
             C = rearrange(C, "b dstate l -> b 1 dstate l")
             ctx.squeeze_C = True
-        keep = _keep_lane_states(u, A) and any(ctx.needs_input_grad)
-        out, ckpt, lanes = selective_scan_fwd(u, delta, A, B, C, D, z, delta_bias, delta_softplus, lane_states=keep)
+        out, ckpt = selective_scan_fwd(u, delta, A, B, C, D, z, delta_bias, delta_softplus)
         ctx.delta_softplus = delta_softplus
         ctx.has_z = z is not None
         ctx.has_D = D is not None
@@ -274,16 +256,16 @@ class SelectiveScanFn(torch.autograd.Function):
         last_state = ckpt[:, :, -1]  # (batch, dim, dstate)
         if A.is_complex():
             last_state = torch.view_as_complex(last_state)
-        ctx.save_for_backward(u, delta, A, B, C, D, z, delta_bias, ckpt, lanes)
+        ctx.save_for_backward(u, delta, A, B, C, D, z, delta_bias, ckpt)
         return out if not return_last_state else (out, last_state)
 
     @staticmethod
     def backward(ctx, dout, *args):
-        u, delta, A, B, C, D, z, delta_bias, ckpt, lanes = ctx.saved_tensors
+        u, delta, A, B, C, D, z, delta_bias, ckpt = ctx.saved_tensors
         if dout.stride(-1) != 1:
             dout = dout.contiguous()
         du, ddelta, dA, dB, dC, dD, ddelta_bias, dz, _ = selective_scan_bwd(
-            u, delta, A, B, C, D, z, delta_bias, dout, ckpt, None, ctx.delta_softplus, False, lanes=lanes)
+            u, delta, A, B, C, D, z, delta_bias, dout, ckpt, None, ctx.delta_softplus, False)
         dB = dB.squeeze(1) if ctx.squeeze_B else dB
         dC = dC.squeeze(1) if ctx.squeeze_C else dC
         return (du, ddelta, dA, dB, dC, dD, dz, ddelta_bias, None, None)
@@ -443,9 +425,7 @@ class MambaInnerFn(torch.autograd.Function):
         if dt_rms_weight is not None:
             delta = rearrange(_rms_norm(rearrange(delta, "b d l -> (b l) d").contiguous(), dt_rms_weight,
                                         b_c_dt_rms_eps), "(b l) d -> b d l", l=L).contiguous()
-        keep = _keep_lane_states(conv1d_out, A) and any(ctx.needs_input_grad)
-        out_z, ckpt, lanes = selective_scan_fwd(conv1d_out, delta, A, B, C, D, z, delta_bias, delta_softplus,
-                                                lane_states=keep)
+        out_z, ckpt = selective_scan_fwd(conv1d_out, delta, A, B, C, D, z, delta_bias, delta_softplus)
         ctx.delta_softplus = delta_softplus
         ctx.out_proj_bias_is_None = out_proj_bias is None
         ctx.checkpoint_lvl = checkpoint_lvl
@@ -453,7 +433,7 @@ class MambaInnerFn(torch.autograd.Function):
         if checkpoint_lvl >= 1:  # conv1d_out and delta are recomputed in the backward pass
             conv1d_out, delta = None, None
         ctx.save_for_backward(xz, conv1d_weight, conv1d_bias, x_dbl, x_proj_weight, delta_proj_weight,
-                              out_proj_weight, conv1d_out, delta, A, B, C, D, delta_bias, ckpt, lanes)
+                              out_proj_weight, conv1d_out, delta, A, B, C, D, delta_bias, ckpt)
         out = F.linear(_as_matrix(out_z).t(), out_proj_weight, out_proj_bias)   # out_z has delta's layout
         return out.view(xz.shape[0], L, -1)
 
@@ -461,7 +441,7 @@ class MambaInnerFn(torch.autograd.Function):
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, dout):
         (xz, conv1d_weight, conv1d_bias, x_dbl, x_proj_weight, delta_proj_weight, out_proj_weight, conv1d_out,
-         delta, A, B, C, D, delta_bias, ckpt, lanes) = ctx.saved_tensors
+         delta, A, B, C, D, delta_bias, ckpt) = ctx.saved_tensors
         L = xz.shape[-1]
         delta_rank = delta_proj_weight.shape[1]
         d_state = A.shape[-1] * (1 if not A.is_complex() else 2)
@@ -483,7 +463,7 @@ class MambaInnerFn(torch.autograd.Function):
         dout_y = _from_matrix(out_proj_weight.t() @ dout, L)
         # du, ddelta and out_z come back in the layouts of u and delta
         dconv1d_out, ddelta, dA, dB, dC, dD, ddelta_bias, dz, out_z = selective_scan_bwd(
-            conv1d_out, delta, A, B, C, D, z, delta_bias, dout_y, ckpt, dz, ctx.delta_softplus, True, lanes=lanes)
+            conv1d_out, delta, A, B, C, D, z, delta_bias, dout_y, ckpt, dz, ctx.delta_softplus, True)
         dout_proj_weight = dout @ _as_matrix(out_z).t()
         dout_proj_bias = dout.sum(dim=1) if not ctx.out_proj_bias_is_None else None
         dx_dbl = torch.empty_like(x_dbl)

@@ -32,7 +32,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_query_and_strerror():
     lib = _lib.load()
-    assert lib.mamba_hip_query(0) >= 1 and lib.mamba_hip_query(1) == 512
+    assert lib.mamba_hip_query(0) >= 5 and lib.mamba_hip_query(1) == 128 and lib.mamba_hip_query(5) == 512
     assert lib.mamba_hip_query(999) < 0
     assert b"success" in lib.mamba_hip_strerror(0)
     assert b"unsupported" in lib.mamba_hip_strerror(-2)

@@ -147,37 +147,3 @@ def test_selective_scan_complex_A(var_B, var_C, itype):
     # wtype complex64 of tests/ops/test_selective_scan.py:17: complex state, (re, im)-interleaved B / C
     _run_case(2, 4, 8, 1024, itype, 2, var_B=var_B, var_C=var_C, complex_A=True)
     _run_case(1, 6, 5, 300, itype, 1, var_B=var_B, var_C=var_C, complex_A=True, has_z=False, has_bias=False)
-
-
-@pytest.mark.parametrize("dstate,seqlen,var_B", [(16, 1500, True), (40, 700, True), (5, 512, False)])
-def test_backward_without_lane_states(dstate, seqlen, var_B, monkeypatch):
-    """The backward kernel's two ways to the states of a tile: from the lane states the forward pass
-    left (the default), or by re-running the scan over the tile when they were not kept."""
-    from mamba_amd.ops import selective_scan_interface as ssi
-    monkeypatch.setattr(ssi, "KEEP_LANE_STATES", False)
-    _run_case(2, 48, dstate, seqlen, torch.float32, 1, var_B=var_B, seed=31)
-    # both ways agree closely on the same inputs
-    g = torch.Generator().manual_seed(32)
-    batch, dim = 2, 40
-    u = torch.randn(batch, dim, seqlen, generator=g).cuda()
-    delta = (0.5 * torch.rand(batch, dim, seqlen, generator=g)).cuda()
-    A = (-0.5 * torch.rand(dim, dstate, generator=g)).cuda()
-    B = torch.randn(batch, 1, dstate, seqlen, generator=g).cuda()
-    C = torch.randn(batch, 1, dstate, seqlen, generator=g).cuda()
-    z = torch.randn(batch, dim, seqlen, generator=g).cuda()
-    dout = torch.randn(batch, dim, seqlen, generator=g).cuda()
-    out, ckpt, lanes = ssi.selective_scan_fwd(u, delta, A, B, C, None, z, None, True, lane_states=True)
-    out2, ckpt2 = ssi.selective_scan_fwd(u, delta, A, B, C, None, z, None, True)
-    assert torch.equal(out, out2) and torch.equal(ckpt, ckpt2)
-    ntiles = (seqlen + ssi.scan_tile() - 1) // ssi.scan_tile()
-    assert lanes.shape == (batch, dim, ntiles, dstate, 64)
-    # lane 0 of a tile holds the state entering the tile: zero for the first, the checkpoint after that
-    assert float(lanes[:, :, 0, :, 0].abs().max()) == 0.0
-    if ntiles > 1:
-        assert torch.equal(lanes[:, :, 1:, :, 0], ckpt[:, :, :-1])
-    with_l = ssi.selective_scan_bwd(u, delta, A, B, C, None, z, None, dout, ckpt, None, True, False, lanes=lanes)
-    without = ssi.selective_scan_bwd(u, delta, A, B, C, None, z, None, dout, ckpt, None, True, False)
-    for name, a, b in zip(("du", "ddelta", "dA", "dB", "dC"), with_l, without):
-        _close(name, a, b, 1e-4, 1e-4 * max(1.0, float(b.abs().max())))
-    with pytest.raises(RuntimeError, match="lanes"):
-        ssi.selective_scan_bwd(u, delta, A, B, C, None, z, None, dout, ckpt, None, True, False, lanes=lanes[:, :, :, :, :32])
