@@ -5,12 +5,15 @@ A step is one forward + backward pass of selective_scan_fn over one synthetic ba
 Mamba-1 benchmark configuration (batch 8, d_inner 5120, seqlen 4096, d_state 16, bf16
 activations, fp32 A/D/delta_bias/state), inputs resident in HBM.  Prints ONE JSON line.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extra]
+
+The line also carries, under "extra", the SSD (configuration 2), decode (configuration 3) and packed-SSD
+(configuration 4) workloads timed in the same run, and under "cpu_baseline" the oracle on the host cores.
 
 Side workloads (each prints its own JSON line; they are not the headline metric):
   python bench.py --workload ssd      Mamba-2 mamba_chunk_scan_combined fwd+bwd (batch 4, 80 heads x 64,
                                       seqlen 4096, d_state 128, chunk 256, bf16)
-  python bench.py --workload decode   selective_state_update (batch 256, 80 heads x 64, d_state 128)
+  python bench.py --workload decode [--batch B]   selective_state_update, 1000 consecutive steps (batch 256, 80 heads x 64, d_state 128)
   python bench.py --workload varlen   the same operator on one packed row of 16 sequences, 32768 positions,
                                       64 heads, 8 groups, initial and final states (benchmark configuration 4)
   python bench.py --workload inner    mamba_inner_fn fwd+bwd (conv, projections, scan; d_model 2560)
@@ -29,10 +32,33 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch read off the FETCH_SIZE / WRITE_SIZE counters (scaled by the copy yardstick),
-# from the *_hbm_counters.txt summaries under profiles/; they describe the kernels as committed there.
-TRAFFIC = {"scan_bwd_kernel": 2719.6e6 + 1686.0e6, "scan_fwd_kernel": 1098.0e6 + 1709.5e6,
-           "chunk_scan_fwd_fused_kernel": 591.1e6 + 335.5e6, "state_update_kernel": 683.1e6 + 673.7e6}
+PROFILES = os.path.join(ROOT, "profiles")
+
+
+def profile_traffic(filename, kernel):
+    """HBM bytes per launch of `kernel` as the FETCH_SIZE / WRITE_SIZE counter runs measured them: the row of
+    that kernel in profiles/<filename> (columns ... read MB (scaled), written MB (scaled)).  None when the
+    summary or the row is missing, e.g. after a kernel was renamed and before the counters were taken again."""
+    try:
+        for line in open(os.path.join(PROFILES, filename)):
+            cols = line.split()
+            if len(cols) >= 5 and cols[0].startswith(kernel):
+                return (float(cols[-2]) + float(cols[-1])) * 1e6
+    except (OSError, ValueError):
+        pass
+    return None
+
+
+def profile_counter(filename, kernel, counter):
+    """Average per-launch value of one hardware counter from profiles/<filename> (lines `kernel counter value`)."""
+    try:
+        for line in open(os.path.join(PROFILES, filename)):
+            cols = line.split()
+            if len(cols) == 3 and cols[0].startswith(kernel) and cols[1] == counter:
+                return float(cols[2])
+    except (OSError, ValueError):
+        pass
+    return None
 
 
 def make_inputs(batch, dim, seqlen, dstate, dtype, device, seed=0):
@@ -47,25 +73,45 @@ def make_inputs(batch, dim, seqlen, dstate, dtype, device, seed=0):
         D=torch.ones(dim, device=device), delta_bias=dt + torch.log(-torch.expm1(-dt)))
 
 
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(seqlen, dstate, full_dim):
-    """Oracle (a PyTorch restatement of the reference's selective_scan_ref) forward + backward on the
-    host cores, on a batch-1 / 128-channel slice of the workload; channels and batch rows are independent
-    in the scan, so tokens/s is scaled by (128 / full_dim)."""
+    """Oracle (a PyTorch restatement of the reference's selective_scan_ref) on the host cores, forward alone and
+    forward + backward, median of 3 each, on a batch-1 / 32-channel slice of the workload; channels and batch
+    rows are independent in the scan, so tokens/s is scaled by (32 / full_dim)."""
+    import statistics
     import torch
     from oracle.mamba1 import selective_scan_oracle, scan_inputs
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
-    dim = 128
+    dim = 32
     t = scan_inputs(1, dim, seqlen, dstate, 1, torch.bfloat16, seed=0)
-    ins = {k: (v.clone().requires_grad_() if (v is not None and k != "dout") else v) for k, v in t.items()}
-    t0 = time.perf_counter()
-    out = selective_scan_oracle(ins["u"], ins["delta"], ins["A"], ins["B"], ins["C"], ins["D"], ins["z"],
-                                ins["delta_bias"], True)
-    out.backward(ins["dout"])
-    dt = time.perf_counter() - t0
-    return {"value": seqlen * (dim / full_dim) / dt, "unit": "tokens/s", "cores": cores, "kind": "port",
-            "sample": f"oracle fwd+bwd, batch 1 x {dim} of {full_dim} channels x seqlen {seqlen}, "
-                      f"{dt:.1f} s, scaled by {dim}/{full_dim}"}
+    names = ("u", "delta", "A", "B", "C", "D", "z", "delta_bias")
+
+    def run(backward):
+        ins = {k: (t[k].clone().requires_grad_(backward) if t[k] is not None else None) for k in names}
+        t0 = time.perf_counter()
+        with torch.set_grad_enabled(backward):
+            out = selective_scan_oracle(*[ins[k] for k in names], True)
+            if backward:
+                out.backward(t["dout"])
+        return time.perf_counter() - t0
+
+    fwd = statistics.median(run(False) for _ in range(3))
+    both = statistics.median(run(True) for _ in range(3))
+    scale = dim / full_dim
+    return {"value": seqlen * scale / both, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "fwd_only_value": seqlen * scale / fwd, "cpu": cpu_model(),
+            "sample": f"oracle, batch 1 x {dim} of {full_dim} channels x seqlen {seqlen}, median of 3: forward "
+                      f"{fwd:.2f} s, forward + backward {both:.2f} s, scaled by {dim}/{full_dim}"}
 
 
 def measured_copy(dev):
@@ -113,6 +159,28 @@ def measured_mfma(dev):
     ev[1].record()
     torch.cuda.synchronize()
     return flops / (ev[0].elapsed_time(ev[1]) / 3) / 1e9
+
+
+def measured_valu(dev):
+    """Per-lane v_fma_f32 instructions per second of mamba_hip_valu_probe (16 independent chains per lane,
+    8 workgroups of 4 waves per CU), in T/s."""
+    import torch
+    from mamba_amd import _lib
+    lib = _lib.load()
+    stream = _lib.current_stream(dev)
+    sink = torch.zeros(1, device=dev)
+    blocks = 8 * torch.cuda.get_device_properties(dev).multi_processor_count
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    n = 0
+    for i in range(4):
+        if i == 1:
+            ev[0].record()
+        n = lib.mamba_hip_valu_probe(sink.data_ptr(), 2048, blocks, stream)
+        if n <= 0:
+            _lib.check(int(n), "mamba_hip_valu_probe")
+    ev[1].record()
+    torch.cuda.synchronize()
+    return n / (ev[0].elapsed_time(ev[1]) / 3) / 1e9
 
 
 def vs_measured_copy(roofline, dev):
@@ -196,7 +264,7 @@ def bench_ssd(dev, steps, warmup):
     mfma_tflops = measured_mfma(dev)
     flops = batch * nc * (H * (Q * Q * P + 2 * Q * N * P) + G * Q * Q * N)   # causal halves counted once
     nbytes = 2 * (4 * batch * L * H * P + 2 * batch * L * G * N) + 4 * batch * nc * H * P * N  # x z out out_x B C states
-    print(json.dumps({
+    return ({
         "metric": "SSD mamba_chunk_scan_combined fwd+bwd tokens/s at 1 GPU", "value": batch * L / sec,
         "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": sec * 1e3,
         "fwd_ms": fwd_ms, "higher_is_better": True, "dtype": "bf16 in/out, fp32 accumulation", "data": "synthetic",
@@ -204,43 +272,63 @@ def bench_ssd(dev, steps, warmup):
                                f"{G} group, chunk {Q}, bf16 (benchmark configuration 2)"},
         "roofline": vs_measured_copy({"bound": "hbm", "kernel": "chunk_scan_fwd_fused_kernel", "achieved": nbytes / scan_ms / 1e6,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / scan_ms / 1e6 / HBM_PEAK_GBS,
-                     "traffic": TRAFFIC["chunk_scan_fwd_fused_kernel"], "kernel_ms": scan_ms, "algorithmic_bytes": nbytes,
+                     "traffic": profile_traffic("ssd_combined_b4_l4096_h80_p64_n128_q256_bf16_hbm_counters.txt", "chunk_scan_fwd_fused_kernel"),
+                     "kernel_ms": scan_ms, "algorithmic_bytes": nbytes,
                      "algorithmic_flops": flops, "mfma_tflops": flops / scan_ms / 1e9,
                      "mfma_frac_of_bf16_peak": flops / scan_ms / 1e9 / 2500.0,
+                     # the kernel moves `algorithmic_bytes` for `algorithmic_flops`: at the HBM peak that caps it at
+                     "flop_per_byte": flops / nbytes, "mfma_cap_from_hbm_tflops": flops / nbytes * HBM_PEAK_GBS / 1e3,
                      "measured_mfma_tflops": mfma_tflops,
-                     "mfma_frac_of_measured": flops / scan_ms / 1e9 / mfma_tflops}, dev)}))
+                     "mfma_frac_of_measured": flops / scan_ms / 1e9 / mfma_tflops}, dev)})
 
 
-def bench_decode(dev, steps, warmup):
-    """Decode: one selective_state_update call per step; the state (fp32) is read and written once."""
+def bench_decode(dev, steps, warmup, batch=256):
+    """Decode: `steps` consecutive selective_state_update calls in place on one state (fp32), the inputs of
+    step i taken from a ring of 8 pre-generated sets; the state is read and written once per step."""
     import torch
     from mamba_amd.ops.triton.selective_state_update import selective_state_update
-    batch, H, P, N, G = 256, 80, 64, 128, 1
+    H, P, N, G = 80, 64, 128, 1
     bf = torch.bfloat16
     g = torch.Generator(device=dev).manual_seed(0)
     rn = lambda *s: torch.randn(*s, device=dev, generator=g)
     state = 0.1 * rn(batch, H, P, N)
-    x, z = rn(batch, H, P).to(bf), rn(batch, H, P).to(bf)
-    dt = rn(batch, H).to(bf)[:, :, None].expand(batch, H, P)
+    ring = [dict(x=rn(batch, H, P).to(bf), z=rn(batch, H, P).to(bf),
+                 dt=rn(batch, H).to(bf)[:, :, None].expand(batch, H, P),
+                 B=rn(batch, G, N).to(bf), C=rn(batch, G, N).to(bf)) for _ in range(8)]
     A = (-(1 + 15 * torch.rand(H, device=dev, generator=g)))[:, None, None].expand(H, P, N)
     D = torch.rand(H, device=dev, generator=g)[:, None].expand(H, P)
     dtb = (torch.rand(H, device=dev, generator=g) - 4)[:, None].expand(H, P)
-    B, C = rn(batch, G, N).to(bf), rn(batch, G, N).to(bf)
-    fn = lambda: selective_state_update(state, x, dt, A, B, C, D=D, z=z, dt_bias=dtb, dt_softplus=True)
-    for _ in range(warmup):
-        fn()
-    ms = event_ms(fn, max(steps, 5))
-    nbytes = 2 * state.numel() * 4 + 2 * (3 * x.numel() + 2 * B.numel()) + 2 * batch * H
-    print(json.dumps({
-        "metric": "decode selective_state_update tokens/s at 1 GPU", "value": batch / ms * 1e3, "unit": "tokens/s",
-        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": ms, "higher_is_better": True,
-        "dtype": "fp32 state, bf16 x/z/B/C/dt", "data": "synthetic",
+
+    def one(i):
+        r = ring[i & 7]
+        return selective_state_update(state, r["x"], r["dt"], A, r["B"], r["C"], D=D, z=r["z"], dt_bias=dtb,
+                                      dt_softplus=True)
+
+    for i in range(warmup):
+        one(i)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev[0].record()
+    for i in range(steps):
+        one(i)
+    ev[1].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) / steps * 1e3
+    ms = ev[0].elapsed_time(ev[1]) / steps
+    x = ring[0]["x"]
+    nbytes = 2 * state.numel() * 4 + 2 * (3 * x.numel() + 2 * ring[0]["B"].numel()) + 2 * batch * H
+    return ({
+        "metric": "decode selective_state_update tokens/s at 1 GPU", "value": batch / wall_ms * 1e3, "unit": "tokens/s",
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": wall_ms, "event_ms_per_step": ms,
+        "higher_is_better": True, "dtype": "fp32 state, bf16 x/z/B/C/dt", "data": "synthetic",
+        "state_finite": bool(torch.isfinite(state).all()),
         "config": {"workload": f"selective_state_update: batch {batch}, {H} heads x {P}, d_state {N}, {G} group, "
-                               "tied A/dt/D per head (benchmark configuration 3)"},
+                               f"tied A/dt/D per head, {steps} consecutive in-place steps (benchmark configuration 3)"},
         "roofline": vs_measured_copy({"bound": "hbm", "kernel": "state_update_kernel", "achieved": nbytes / ms / 1e6,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / ms / 1e6 / HBM_PEAK_GBS,
-                     "traffic": TRAFFIC["state_update_kernel"],
-                     "kernel_ms": ms, "algorithmic_bytes": nbytes}, dev)}))
+                     "traffic": profile_traffic("state_update_b256_h80_p64_n128_bf16_hbm_counters.txt", "state_update_kernel") if batch == 256 else None,
+                     "kernel_ms": ms, "algorithmic_bytes": nbytes}, dev)})
 
 
 def _timed(step, steps, warmup):
@@ -291,7 +379,7 @@ def bench_varlen(dev, steps, warmup):
     with torch.no_grad():
         fwd_ms = event_ms(fwd, max(5, min(steps, 50)))
     nbytes = 2 * (5 * batch * L * H * P + 4 * batch * L * G * N)   # x z dout in, dx dz out, B C in, dB dC out (bf16)
-    print(json.dumps({
+    return ({
         "metric": "SSD mamba_chunk_scan_combined packed varlen fwd+bwd tokens/s at 1 GPU", "value": batch * L / sec,
         "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": sec * 1e3,
         "fwd_ms": fwd_ms, "higher_is_better": True, "dtype": "bf16 in/out, fp32 accumulation", "data": "synthetic",
@@ -299,7 +387,7 @@ def bench_varlen(dev, steps, warmup):
                                f"d_state {N}, {G} groups, chunk {Q}, initial + final states (benchmark configuration 4)"},
         "roofline": vs_measured_copy({"bound": "hbm", "kernel": "whole step", "achieved": nbytes / sec / 1e9, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": nbytes / sec / 1e9 / HBM_PEAK_GBS, "traffic": None,
-                     "algorithmic_bytes": nbytes}, dev)}))
+                     "algorithmic_bytes": nbytes}, dev)})
 
 
 def bench_inner(dev, steps, warmup):
@@ -340,7 +428,7 @@ def bench_inner(dev, steps, warmup):
         cw = conv_w.squeeze(1)
         conv_ms = event_ms(lambda: causal_conv1d_fwd(xin, cw, conv_b, activation="silu"), max(5, min(steps, 50)))
     nbytes = 2 * 2 * batch * di * L   # the convolution reads x and writes its output once
-    print(json.dumps({
+    return ({
         "metric": "mamba_inner_fn fwd+bwd tokens/s at 1 GPU", "value": batch * L / sec, "unit": "tokens/s",
         "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": sec * 1e3, "fwd_ms": fwd_ms,
         "higher_is_better": True, "dtype": "bf16 in/out, fp32 state and accumulation", "data": "synthetic",
@@ -348,7 +436,7 @@ def bench_inner(dev, steps, warmup):
                                f"d_state {N}, dt_rank {R}, conv width {W}"},
         "roofline": vs_measured_copy({"bound": "hbm", "kernel": "conv_rows_fwd_kernel", "achieved": nbytes / conv_ms / 1e6,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / conv_ms / 1e6 / HBM_PEAK_GBS,
-                     "traffic": None, "kernel_ms": conv_ms, "algorithmic_bytes": nbytes}, dev)}))
+                     "traffic": None, "kernel_ms": conv_ms, "algorithmic_bytes": nbytes}, dev)})
 
 
 def bench_block(dev, steps, warmup):
@@ -391,7 +479,7 @@ def bench_block(dev, steps, warmup):
         norm_ms = event_ms(lambda: _layer_norm_fwd(y, norm_w, None, 1e-6, z=zz, group_size=dim // G,
                                                    norm_before_gate=False, is_rms_norm=True), max(5, min(steps, 50)))
     nbytes = 3 * 2 * batch * L * dim   # the gated norm reads y and z and writes its output once
-    print(json.dumps({
+    return ({
         "metric": "mamba_split_conv1d_scan_combined fwd+bwd tokens/s at 1 GPU", "value": batch * L / sec,
         "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": sec * 1e3, "fwd_ms": fwd_ms,
         "higher_is_better": True, "dtype": "bf16 in/out, fp32 accumulation", "data": "synthetic",
@@ -399,44 +487,14 @@ def bench_block(dev, steps, warmup):
                                f"{G} group, chunk {Q}, conv width {W}, gated RMSNorm, out_proj to {dm}"},
         "roofline": vs_measured_copy({"bound": "hbm", "kernel": "norm_fwd_kernel", "achieved": nbytes / norm_ms / 1e6,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / norm_ms / 1e6 / HBM_PEAK_GBS,
-                     "traffic": None, "kernel_ms": norm_ms, "algorithmic_bytes": nbytes}, dev)}))
+                     "traffic": None, "kernel_ms": norm_ms, "algorithmic_bytes": nbytes}, dev)})
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--workload", choices=("mamba1", "ssd", "decode", "varlen", "inner", "block"), default="mamba1")
-    ap.add_argument("--copy-calibration", action="store_true",
-                    help="only run the library's plain copy kernel over 1 GiB (yardstick for HBM counters)")
-    args = ap.parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build measures one GPU only (the scan has no cross-GPU exchange step); "
-              "run with --gpus 1", file=sys.stderr)
-        sys.exit(2)
-
+def bench_mamba1(dev, steps, warmup):
+    """The headline workload: selective_scan_fn forward + backward at benchmark configuration 1."""
     import torch
     from mamba_amd.ops import selective_scan_interface as ssi
     from mamba_amd.ops.selective_scan_interface import selective_scan_fn, selective_scan_fwd
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        sys.exit(2)
-    dev = torch.device("cuda", 0)
-    torch.cuda.set_device(dev)
-    if args.copy_calibration:
-        copy_calibration(dev)
-        return
-    if args.workload == "ssd":
-        bench_ssd(dev, args.steps, args.warmup)
-        return
-    if args.workload == "decode":
-        bench_decode(dev, args.steps, args.warmup)
-        return
-    if args.workload in ("varlen", "inner", "block"):
-        {"varlen": bench_varlen, "inner": bench_inner, "block": bench_block}[args.workload](dev, args.steps, args.warmup)
-        return
     batch, dim, seqlen, dstate = 8, 5120, 4096, 16
     dtype = torch.bfloat16
     t = make_inputs(batch, dim, seqlen, dstate, dtype, dev)
@@ -449,30 +507,29 @@ def main():
                                 z=leaves["z"], delta_bias=leaves["delta_bias"], delta_softplus=True)
         out.backward(t["dout"])
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed / args.steps * 1e3
-    tokens_per_s = batch * seqlen / (elapsed / args.steps)
+    ms_per_step = elapsed / steps * 1e3
+    tokens_per_s = batch * seqlen / (elapsed / steps)
 
-    # Dominant kernel (the backward scan) alone, HIP events on the launch stream.
+    # Dominant kernel (the backward scan, with the two small kernels that add up its dB / dC partials) alone,
+    # HIP events on the launch stream.
     with torch.no_grad():
         d = {k: v.detach() for k, v in leaves.items()}
         _, ckpt = selective_scan_fwd(d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["z"], d["delta_bias"], True)
         dims = (batch, dim, seqlen, dstate, 1)
         bwd_args = (d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["z"], d["delta_bias"], t["dout"], ckpt, True, dims)
         bufs = ssi.scan_bwd_launch(*bwd_args)
-        bwd_pre = None
-        bwd = lambda: ssi.scan_bwd_launch(*bwd_args, bufs=bufs)   # the scan kernel and its two small reduce kernels
+        bwd = lambda: ssi.scan_bwd_launch(*bwd_args, bufs=bufs)
         fwd = lambda: selective_scan_fwd(d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["z"], d["delta_bias"], True)
-
-        n = max(5, min(args.steps, 50))
-        bwd_ms = event_ms(bwd, n, bwd_pre)
+        n = max(5, min(steps, 50))
+        bwd_ms = event_ms(bwd, n)
         fwd_ms = event_ms(fwd, n)
     es = 2  # bf16
     E = batch * dim * seqlen * es
@@ -480,16 +537,37 @@ def main():
     bwd_bytes = 7 * E + 4 * BC   # reads u, delta, z, dout, B, C; writes du, ddelta, dz, dB, dC
     fwd_bytes = 4 * E + 2 * BC   # reads u, delta, z, B, C; writes out
     achieved = bwd_bytes / (bwd_ms * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "kernel": "scan_bwd_kernel", "achieved": achieved, "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": TRAFFIC["scan_bwd_kernel"],
+    prof = "mamba1_scan_b8_d5120_l4096_n16_bf16"
+    roofline = {"bound": "hbm", "kernel": "scan_bwd_kernel (+ reduce_parts_kernel x 2)", "achieved": achieved,
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                "traffic": profile_traffic(prof + "_hbm_counters.txt", "scan_bwd_kernel"),
                 "kernel_ms": bwd_ms, "algorithmic_bytes": bwd_bytes,
                 "fwd_kernel_ms": fwd_ms, "fwd_achieved": fwd_bytes / (fwd_ms * 1e-3) / 1e9,
+                "fwd_traffic": profile_traffic(prof + "_hbm_counters.txt", "scan_fwd_kernel"),
                 "fwd_bwd_frac": (fwd_bytes + bwd_bytes) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS}
     vs_measured_copy(roofline, dev)
-
-    result = {
+    # The binding resource of both scan kernels is fp32 vector-ALU issue, not HBM: instruction slots per
+    # (position, channel, state) from the hardware counters of the committed profile (a transcendental
+    # takes two slots), times the elements of this launch, over the event time, beside the rate a bare
+    # v_fma_f32 loop reaches in this run.
+    elems = batch * dim * seqlen * dstate
+    probe = measured_valu(dev)
+    valu = {"unit": "T lane-instruction slots/s", "measured_fma_probe": probe,
+            "nominal_peak": 256 * 4 * 16 * 2.4e9 / 1e12, "element_states": elems}
+    for name, ms in (("bwd", bwd_ms), ("fwd", fwd_ms)):
+        kern = "scan_%s_kernel" % name
+        insts = profile_counter(prof + "_valu_counters.txt", kern, "SQ_INSTS_VALU")
+        trans = profile_counter(prof + "_valu_counters.txt", kern, "SQ_INSTS_VALU_TRANS_F32")
+        if insts is None or trans is None:
+            valu[name] = None
+            continue
+        slots = (insts + trans) * 64 / elems
+        valu[name] = {"slots_per_element_state": slots, "achieved": slots * elems / (ms * 1e-3) / 1e12,
+                      "frac_of_probe": slots * elems / (ms * 1e-3) / 1e12 / probe}
+    roofline["valu"] = valu
+    return {
         "metric": "scan fwd+bwd tokens/s at 1 GPU; achieved HBM GB/s and % bf16 MFMA peak",
-        "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16 in/out, fp32 state and accumulation", "data": "synthetic",
         "config": {"workload": "Mamba-1 selective_scan_fn fwd+bwd: batch 8, d_inner 5120, seqlen 4096, d_state 16, "
@@ -497,8 +575,57 @@ def main():
                    "global_batch": batch, "seq_len": seqlen},
         "roofline": roofline,
     }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true",
+                    help="headline workload only: leave out the SSD, decode and packed-SSD lines under `extra`")
+    ap.add_argument("--workload", choices=("mamba1", "ssd", "decode", "varlen", "inner", "block"), default="mamba1")
+    ap.add_argument("--batch", type=int, default=256, help="batch of --workload decode")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run the library's plain copy kernel over 1 GiB (yardstick for HBM counters)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only (the scan has no cross-GPU exchange step); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    if args.copy_calibration:
+        copy_calibration(dev)
+        return
+    if args.workload == "decode":
+        print(json.dumps(bench_decode(dev, max(args.steps, 1000), args.warmup, args.batch)))
+        return
+    if args.workload != "mamba1":
+        fn = {"ssd": bench_ssd, "varlen": bench_varlen, "inner": bench_inner, "block": bench_block}[args.workload]
+        print(json.dumps(fn(dev, args.steps, args.warmup)))
+        return
+    result = bench_mamba1(dev, args.steps, args.warmup)
+    if not args.no_extra:
+        # the other benchmark configurations, timed in the same run (each entry is the line its own
+        # --workload prints): configuration 2 (SSD, with the MFMA figures), 3 (decode, 1000 consecutive
+        # steps) and 4 (packed SSD)
+        keep = ("value", "unit", "ms_per_step", "fwd_ms", "event_ms_per_step", "steps", "config", "roofline")
+        extra = {}
+        for name, fn in (("ssd", lambda: bench_ssd(dev, args.steps, args.warmup)),
+                         ("decode", lambda: bench_decode(dev, 1000, 10)),
+                         ("varlen", lambda: bench_varlen(dev, args.steps, args.warmup))):
+            r = fn()
+            extra[name] = {k: r[k] for k in keep if k in r}
+        result["extra"] = extra
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(seqlen, dstate, dim)
+        result["cpu_baseline"] = cpu_baseline(4096, 16, 5120)
     print(json.dumps(result))
 
 

@@ -60,6 +60,11 @@ int mamba_hip_copy(void *dst, const void *src, int64_t nbytes, mamba_stream_t st
  * of device memory that is never written. */
 int64_t mamba_hip_mfma_probe(float *sink, int iters, int blocks, mamba_stream_t stream);
 
+/* Measurement yardstick for the scan kernels, whose time is fp32 vector-ALU issue: launches `blocks` workgroups of
+ * 4 waves, each lane running `iters` rounds of 64 v_fma_f32 in sixteen independent chains on register operands.
+ * Returns the per-lane instructions of the launch (> 0), or an error code (< 0).  `sink` as above. */
+int64_t mamba_hip_valu_probe(float *sink, int iters, int blocks, mamba_stream_t stream);
+
 /* ------------------------------------------------------------------------- *
  * Mamba-1 selective scan.
  * Replaces selective_scan_cuda.fwd / .bwd

@@ -167,6 +167,8 @@ def load():
         fn.restype = ctypes.c_int
     lib.mamba_hip_mfma_probe.argtypes = [c_vp, ctypes.c_int, ctypes.c_int, c_vp]
     lib.mamba_hip_mfma_probe.restype = ctypes.c_int64
+    lib.mamba_hip_valu_probe.argtypes = [c_vp, ctypes.c_int, ctypes.c_int, c_vp]
+    lib.mamba_hip_valu_probe.restype = ctypes.c_int64
     for name in ("norm_residual_fwd", "norm_residual_bwd"):
         fn = getattr(lib, name)
         fn.argtypes = [ctypes.POINTER(NormResidualParams), c_vp]

@@ -32,7 +32,33 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(float *sink, int iters)
   for (int j = 0; j < 8; ++j) s += acc[j].x + acc[j].y + acc[j].z + acc[j].w;
   if (s == -1.f) sink[0] = s;  // never true: keeps the loop alive
 }
+// Sixteen independent chains of v_fma_f32 per lane on register operands: the rate at which the vector ALUs
+// issue fp32 instructions with nothing else in the way, as a yardstick for the scan kernels.
+__global__ __launch_bounds__(256) void valu_probe_kernel(float *sink, int iters) {
+  float a[16];
+#pragma unroll
+  for (int j = 0; j < 16; ++j) a[j] = 1.f + 0.001f * (float)((threadIdx.x + j) & 31);
+  const float m = 0.99999f, c = 1e-6f;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+#pragma unroll
+      for (int j = 0; j < 16; ++j) a[j] = __builtin_fmaf(a[j], m, c);
+    }
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) s += a[j];
+  if (s == -1.f) sink[0] = s;  // never true: keeps the loop alive
+}
 }  // namespace
+
+extern "C" int64_t mamba_hip_valu_probe(float *sink, int iters, int blocks, mamba_stream_t stream) {
+  if (!sink || iters <= 0 || blocks <= 0) return MAMBA_E_BADARG;
+  hipLaunchKernelGGL(valu_probe_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), sink, iters);
+  if (hipGetLastError() != hipSuccess) return MAMBA_E_LAUNCH;
+  return (int64_t)blocks * 256 * iters * 64;  // per-lane fma instructions of this launch
+}
 
 extern "C" int64_t mamba_hip_mfma_probe(float *sink, int iters, int blocks, mamba_stream_t stream) {
   if (!sink || iters <= 0 || blocks <= 0) return MAMBA_E_BADARG;
@@ -53,11 +79,13 @@ extern "C" int mamba_hip_copy(void *dst, const void *src, int64_t nbytes, mamba_
   return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
 }
 
+int mamba1_scan_tile(bool a_complex);  // mamba1_scan.hip
+
 extern "C" int mamba_hip_query(int what) {
   switch (what) {
     case MAMBA_Q_ABI_VERSION: return 5;
-    case MAMBA_Q_SCAN_TILE: return 128;
-    case MAMBA_Q_SCAN_TILE_COMPLEX: return 512;
+    case MAMBA_Q_SCAN_TILE: return mamba1_scan_tile(false);
+    case MAMBA_Q_SCAN_TILE_COMPLEX: return mamba1_scan_tile(true);
     case MAMBA_Q_MAX_DSTATE: return 256;
     case MAMBA_Q_SSD_MAX_DSTATE: return 256;
     case MAMBA_Q_SSD_MAX_HEADDIM: return 256;

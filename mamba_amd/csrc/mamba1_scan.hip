@@ -826,6 +826,8 @@ template <typename T, bool BWD> int dispatch(const MambaScanParams &p, hipStream
 
 int mamba1_scan_complex(const MambaScanParams *p, hipStream_t s, bool bwd);  // mamba1_scan_complex.hip
 
+int mamba1_scan_tile(bool a_complex) { return a_complex ? TILE_COMPLEX : TILE; }  // positions per checkpoint tile
+
 extern "C" int mamba1_scan_fwd(const MambaScanParams *p, mamba_stream_t stream) {
   int rc = check_common(p);
   if (rc != MAMBA_OK) return rc;
