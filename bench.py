@@ -331,6 +331,83 @@ def bench_decode(dev, steps, warmup, batch=256):
                      "kernel_ms": ms, "algorithmic_bytes": nbytes}, dev)})
 
 
+def bench_decode_step(dev, steps, warmup, batch):
+    """One generated token of a Mamba-2 layer's mixer core, as the reference's step() runs it
+    (mamba_ssm/modules/mamba2.py:298-336): causal_conv1d_update over the x/B/C channels, then
+    selective_state_update.  Reports wall time per token of the two launches eager and replayed from a
+    captured HIP graph, and of each kernel alone in a graph: a single fused kernel cannot be faster than
+    the state update alone, so `graph_two_launches - graph_state_update_only` bounds what fusing saves,
+    and `eager - graph` is the host side's share (argument checks + parameter fill through ctypes)."""
+    import torch
+    from mamba_amd.ops.causal_conv1d import causal_conv1d_update
+    from mamba_amd.ops.triton.selective_state_update import selective_state_update, mamba2_decode_step
+    H, P, N, G, W = 80, 64, 128, 1, 4
+    dim, conv_dim = H * P, H * P + 2 * G * N
+    bf = torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(0)
+    rn = lambda *s: torch.randn(*s, device=dev, generator=g)
+    ssm_state = 0.1 * rn(batch, H, P, N)
+    conv_state = rn(batch, W, conv_dim).to(bf).transpose(1, 2)   # channel-contiguous, as the reference allocates it
+    conv_w, conv_b = (0.4 * rn(conv_dim, W)).to(bf), (0.1 * rn(conv_dim)).to(bf)
+    xBC, z, dt = rn(batch, conv_dim).to(bf), rn(batch, H, P).to(bf), rn(batch, H).to(bf)
+    A = (-(1 + 15 * torch.rand(H, device=dev, generator=g)))[:, None, None].expand(H, P, N)
+    D = torch.rand(H, device=dev, generator=g)[:, None].expand(H, P)
+    dtb = (torch.rand(H, device=dev, generator=g) - 4)[:, None].expand(H, P)
+    xc0 = rn(batch, conv_dim).to(bf)
+    Ah, Dh, dtbh = A[:, 0, 0].contiguous(), D[:, 0].contiguous(), dtb[:, 0].contiguous()
+
+    def fused():
+        return mamba2_decode_step(ssm_state, conv_state, xBC, dt, Ah, conv_w, conv_b, D=Dh, z=z, dt_bias=dtbh, ngroups=G,
+                                  fuse=True)
+
+    def conv():
+        return causal_conv1d_update(xBC, conv_state, conv_w, conv_b, "silu")
+
+    def ssm(xc):
+        xs, B, C = torch.split(xc, [dim, G * N, G * N], dim=-1)
+        return selective_state_update(ssm_state, xs.reshape(batch, H, P), dt[:, :, None].expand(batch, H, P), A,
+                                      B.reshape(batch, G, N), C.reshape(batch, G, N), D=D, z=z, dt_bias=dtb,
+                                      dt_softplus=True)
+
+    variants = {"two_launches": lambda: ssm(conv()), "fused": fused, "state_update_only": lambda: ssm(xc0),
+                "conv_update_only": conv}
+
+    def wall(fn, n):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n * 1e6
+
+    out = {}
+    with torch.no_grad():
+        for name, fn in variants.items():
+            for _ in range(warmup):
+                fn()
+            out["eager_us_" + name] = wall(fn, steps)
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                fn()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for _ in range(10):   # ten tokens per replay, so that the replay's own launch cost is shared
+                    fn()
+            graph.replay()
+            out["graph_us_" + name] = wall(graph.replay, max(steps // 10, 20)) / 10
+    out["fusion_bound_us"] = out["graph_us_two_launches"] - out["graph_us_state_update_only"]
+    out["fused_gain_us"] = out["graph_us_two_launches"] - out["graph_us_fused"]
+    out["host_share_us"] = out["eager_us_two_launches"] - out["graph_us_two_launches"]
+    return {"metric": "decode step (conv update + state update) wall time per token", "unit": "us", "batch": batch,
+            "value": out["graph_us_two_launches"], "higher_is_better": False, "steps": steps, "n_gpus": 1,
+            "config": {"workload": f"causal_conv1d_update ({conv_dim} channels, width {W}) + selective_state_update: "
+                                   f"batch {batch}, {H} heads x {P}, d_state {N}, bf16 inputs, fp32 state"},
+            **out}
+
+
 def _timed(step, steps, warmup):
     import torch
     for _ in range(warmup):
@@ -585,7 +662,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true",
                     help="headline workload only: leave out the SSD, decode and packed-SSD lines under `extra`")
-    ap.add_argument("--workload", choices=("mamba1", "ssd", "decode", "varlen", "inner", "block"), default="mamba1")
+    ap.add_argument("--workload", choices=("mamba1", "ssd", "decode", "decode_step", "varlen", "inner", "block"), default="mamba1")
     ap.add_argument("--batch", type=int, default=256, help="batch of --workload decode")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run the library's plain copy kernel over 1 GiB (yardstick for HBM counters)")
@@ -606,6 +683,9 @@ def main():
         return
     if args.workload == "decode":
         print(json.dumps(bench_decode(dev, max(args.steps, 1000), args.warmup, args.batch)))
+        return
+    if args.workload == "decode_step":
+        print(json.dumps(bench_decode_step(dev, max(args.steps, 200), args.warmup, args.batch)))
         return
     if args.workload != "mamba1":
         fn = {"ssd": bench_ssd, "varlen": bench_varlen, "inner": bench_inner, "block": bench_block}[args.workload]

@@ -203,6 +203,42 @@ typedef struct MambaStepParams {
 int ssm_state_update(const MambaStepParams *p, mamba_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
+ * One generated token of a Mamba-2 mixer in ONE launch: the decode step of the depthwise convolution
+ * over the x / B / C channels followed by the state update, i.e. the pair of calls
+ *   xBC = causal_conv1d_update(xBC, conv_state, conv_weight, conv_bias, activation)
+ *   y   = selective_state_update(ssm_state, x, dt, A, B, C, D, z, dt_bias, dt_softplus=True)
+ * of the reference's step() (mamba_ssm/modules/mamba2.py:298-336).  At generation batches of 1-8 the two
+ * kernels are launch-bound; fused, the step is one kernel that reads each state once.
+ *   xBC        : (batch, conv_dim) of ssm.x_dtype, channels contiguous, conv_dim = nheads * dim + 2 * ngroups * dstate,
+ *                laid out [x (nheads * dim) | B (ngroups * dstate) | C (ngroups * dstate)]
+ *   conv_state : (conv_state_rows >= batch, conv_dim, state_len) of ssm.x_dtype through element strides, updated in place
+ *                to the last state_len positions of [conv_state, xBC]; width - 1 <= state_len <= 4
+ *   conv_weight: (conv_dim, width) fp32 contiguous; conv_bias: (conv_dim) fp32, nullable; width 2..4
+ *   sync       : int32 (mamba2_decode_step_sync_ints(p)), all zero on entry and again on return (the workgroups of a
+ *                (batch entry, group) count themselves off here; the last one shifts the conv state of the group's
+ *                shared B / C channels once every other one has read it).  Calls that share `sync` must not overlap.
+ * `ssm` describes the state update as for ssm_state_update; its x, B, C pointers and strides are ignored (the
+ * convolution's outputs take their place), dt / A / dt_bias / D must be per head (stride 0 along dim and dstate:
+ * the tie_hdim form of the reference's step), bc_dtype = x_dtype, and state_batch_indices must be null.
+ * Returns MAMBA_E_UNSUPPORTED for anything outside this form (the caller then makes the two calls).
+ * ------------------------------------------------------------------------- */
+typedef struct MambaDecodeStepParams {
+  MambaStepParams ssm;
+  int32_t conv_dim, width, state_len, silu;
+  int32_t conv_state_rows, reserved;
+  const void *xBC;
+  void *conv_state;
+  const float *conv_weight;
+  const float *conv_bias; /* nullable */
+  int32_t *sync;
+  int64_t xBC_bs;
+  int64_t cs_bs, cs_cs, cs_ls; /* conv_state strides: row, channel, position */
+} MambaDecodeStepParams;
+
+int64_t mamba2_decode_step_sync_ints(const MambaDecodeStepParams *p); /* needs ssm.batch, nheads, ngroups, dim, dstate */
+int mamba2_decode_step(const MambaDecodeStepParams *p, mamba_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
  * Mamba-2 SSD (chunked state-space-dual scan).
  * Replaces the Triton kernels launched by _mamba_chunk_scan_combined_fwd / _bwd
  * (reference mamba_ssm/ops/triton/ssd_combined.py:343 and :397), i.e.
@@ -380,6 +416,8 @@ typedef struct CausalConvUpdateParams {
   int64_t x_bs, x_cs, x_ls;
   int64_t out_bs, out_cs, out_ls;
   int64_t state_bs, state_cs, state_ls;
+  const int32_t *cache_seqlens; /* nullable; (batch): conv_state is a circular buffer, entry b has seen cache_seqlens[b]
+                                   positions, position t lives in slot t % state_len; nothing is shifted */
 } CausalConvUpdateParams;
 
 int causal_conv1d_update(const CausalConvUpdateParams *p, mamba_stream_t stream);

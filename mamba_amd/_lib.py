@@ -44,6 +44,15 @@ class MambaStepParams(ctypes.Structure):
     )
 
 
+class MambaDecodeStepParams(ctypes.Structure):
+    _fields_ = (
+        [("ssm", MambaStepParams)]
+        + [(n, c_i32) for n in ("conv_dim", "width", "state_len", "silu", "conv_state_rows", "reserved")]
+        + [(n, c_vp) for n in ("xBC", "conv_state", "conv_weight", "conv_bias", "sync")]
+        + [(n, c_i64) for n in ("xBC_bs", "cs_bs", "cs_cs", "cs_ls")]
+    )
+
+
 class SsdParams(ctypes.Structure):
     _fields_ = (
         [(n, c_i32) for n in ("batch", "seqlen", "nheads", "headdim", "dstate", "ngroups", "chunk_size", "nchunks",
@@ -75,6 +84,7 @@ class CausalConvUpdateParams(ctypes.Structure):
                                 "state_rows", "reserved")]
         + [(n, c_vp) for n in ("x", "conv_state", "weight", "bias", "out", "conv_state_indices")]
         + [(n, c_i64) for n in ("x_bs", "x_cs", "x_ls", "out_bs", "out_cs", "out_ls", "state_bs", "state_cs", "state_ls")]
+        + [("cache_seqlens", c_vp)]
     )
 
 
@@ -153,6 +163,10 @@ def load():
     lib.ssd_chunk_scan_fwd_fused_supported.restype = ctypes.c_int
     lib.ssm_state_update.argtypes = [ctypes.POINTER(MambaStepParams), c_vp]
     lib.ssm_state_update.restype = ctypes.c_int
+    lib.mamba2_decode_step.argtypes = [ctypes.POINTER(MambaDecodeStepParams), c_vp]
+    lib.mamba2_decode_step.restype = ctypes.c_int
+    lib.mamba2_decode_step_sync_ints.argtypes = [ctypes.POINTER(MambaDecodeStepParams)]
+    lib.mamba2_decode_step_sync_ints.restype = ctypes.c_int64
     for name in ("causal_conv1d_fwd", "causal_conv1d_bwd"):
         fn = getattr(lib, name)
         fn.argtypes = [ctypes.POINTER(CausalConvParams), c_vp]

@@ -398,15 +398,25 @@ template <typename T, typename S> __global__ __launch_bounds__(256) void conv_up
   bias = p.bias ? p.bias[c] : 0.f;
   const int SL = p.state_len;
   float win[MAXW];  // win[0..2]: the three positions before the next output, win[3]: the new one
+  if (p.cache_seqlens) {
+    // circular buffer: position t of the sequence lives in slot t mod SL; taps the filter does not use stay 0
+    const int len = p.cache_seqlens[b];
+    auto slot_of = [&](int t) { return ((t % SL) + SL) % SL; };
 #pragma unroll
-  for (int i = 0; i < MAXW - 1; ++i) {
-    const int j = SL - (MAXW - 1) + i;
-    win[i] = j >= 0 ? ld1<S>(st + j * p.state_ls) : 0.f;
-  }
-  for (int j = 0; j < SL; ++j) {
-    const int src = j + p.seqlen;
-    const float v = src < SL ? ld1<S>(st + src * p.state_ls) : ld1<T>(x + (src - SL) * p.x_ls);
-    st1<S>(st + j * p.state_ls, v);
+    for (int i = 0; i < MAXW - 1; ++i)
+      win[i] = i >= MAXW - p.width ? ld1<S>(st + slot_of(len - (MAXW - 1) + i) * p.state_ls) : 0.f;
+    for (int t = 0; t < p.seqlen; ++t) st1<S>(st + slot_of(len + t) * p.state_ls, ld1<T>(x + t * p.x_ls));
+  } else {
+#pragma unroll
+    for (int i = 0; i < MAXW - 1; ++i) {
+      const int j = SL - (MAXW - 1) + i;
+      win[i] = j >= 0 ? ld1<S>(st + j * p.state_ls) : 0.f;
+    }
+    for (int j = 0; j < SL; ++j) {
+      const int src = j + p.seqlen;
+      const float v = src < SL ? ld1<S>(st + src * p.state_ls) : ld1<T>(x + (src - SL) * p.x_ls);
+      st1<S>(st + j * p.state_ls, v);
+    }
   }
   for (int t = 0; t < p.seqlen; ++t) {
     win[3] = ld1<T>(x + t * p.x_ls);

@@ -295,6 +295,245 @@ template <typename TS> int dispatch_x(const MambaStepParams &p, hipStream_t s) {
 
 bool dtype_ok(int d) { return d == MAMBA_F32 || d == MAMBA_BF16 || d == MAMBA_F16; }
 
+// ------------------------------------------------------------------ fused decode step
+// causal_conv1d_update over the x / B / C channels and the state update in one launch (the pair of calls
+// of the reference's Mamba2.step, mamba_ssm/modules/mamba2.py:298-336).  Same decomposition as
+// state_update_kernel; on top of it
+//   * lane j of a wave convolves the x channel of the wave's row j, shifts that channel's conv state in
+//     place (no other wave reads it) and hands the value to the lanes of the row;
+//   * every workgroup convolves the B and C channels of its head's group from the OLD conv state (re-done
+//     per workgroup: a few cached loads per thread, shared through LDS) -- so nobody may shift those shared
+//     channels until every workgroup of the batch entry has read them.  Workgroups count themselves off in
+//     `sync` when their loads are done; the one that arrives last shifts the B / C channels and puts the
+//     counters back to zero.  Nobody waits.
+// The convolution's outputs are rounded to the activation dtype as the separate kernel's stored output is,
+// so the fused step and the two calls give the same bits.
+DEVI float silu_act(float v) { return v * sigmoid_f(v); }
+template <typename T> DEVI float round_to(float x) {
+  if constexpr (DT<T>::id == MAMBA_F32) return x;
+  else if constexpr (DT<T>::id == MAMBA_BF16) return __builtin_bit_cast(float, f32_to_bf16_bits(x) << 16);
+  else return (float)(_Float16)x;
+}
+
+constexpr int CW = 4;  // widest filter, longest conv state
+constexpr int SYNC_FAN = 16;  // arrivals per counter
+
+// taps sv[0..2] = the conv state's last three positions (0 where the state is shorter), xn the new value,
+// w[0..3] the filter right-aligned in 4 taps
+DEVI float conv_tap(const float (&sv)[3], float xn, const float (&w)[4], float bias, bool silu) {
+  float v = bias;
+  v = __builtin_fmaf(w[0], sv[0], v);
+  v = __builtin_fmaf(w[1], sv[1], v);
+  v = __builtin_fmaf(w[2], sv[2], v);
+  v = __builtin_fmaf(w[3], xn, v);
+  return silu ? silu_act(v) : v;
+}
+
+// this thread's conv state taps and filter of channel c (element loads from valid addresses)
+template <typename TX>
+DEVI void conv_loads(const MambaDecodeStepParams &q, const TX *cstate, const TX *xBC, int c, float (&sv)[3], float &xn,
+                     float (&w)[4], float &bias) {
+  const int SL = q.state_len, W = q.width, cs_cs = (int)q.cs_cs, cs_ls = (int)q.cs_ls;
+#pragma unroll
+  for (int i = 0; i < 3; ++i) {
+    const int j = SL - 3 + i;
+    const float v = ld1<TX>(cstate + c * cs_cs + max(j, 0) * cs_ls);
+    sv[i] = j >= 0 ? v : 0.f;
+  }
+  xn = ld1<TX>(xBC + c);
+  if (W == CW) {
+    const f32x4 wq = *reinterpret_cast<const f32x4 *>(q.conv_weight + (int64_t)c * CW);
+    w[0] = wq.x; w[1] = wq.y; w[2] = wq.z; w[3] = wq.w;
+  } else {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int j = k - (CW - W);
+      const float v = q.conv_weight[(int64_t)c * W + max(j, 0)];
+      w[k] = j >= 0 ? v : 0.f;
+    }
+  }
+  bias = q.conv_bias ? q.conv_bias[c] : 0.f;
+}
+// conv state of one channel after the step: the old positions moved down by one, the new value last
+template <typename TX> DEVI void conv_shift(TX *st, int SL, int cs_ls, const float (&sv)[3], float xn) {
+  st1<TX>(st + (SL - 1) * cs_ls, xn);
+  if (SL > 1) st1<TX>(st + (SL - 2) * cs_ls, sv[2]);
+  if (SL > 2) st1<TX>(st + (SL - 3) * cs_ls, sv[1]);
+  if (SL > 3) st1<TX>(st + (SL - 4) * cs_ls, sv[0]);
+}
+
+template <typename TS, typename TX, typename TD>
+__global__ __launch_bounds__(256) void decode_step_fused_kernel(const MambaDecodeStepParams q, int lpr_log2) {
+  const MambaStepParams &p = q.ssm;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int G = p.ngroups, N = p.dstate, hpg = p.nheads / G;
+  const int g = h / hpg;
+  const int lpr = 1 << lpr_log2, rpp = 64 >> lpr_log2;
+  const int sub = lane & (lpr - 1), rsel = lane >> lpr_log2;
+  const int p_begin = (blockIdx.x * 4 + wave) * rpp * UNR;  // may lie past the head's rows: such a wave loads from
+  const int SL = q.state_len;                               // clamped rows like any other and stores nothing
+  const int cs_cs = (int)q.cs_cs, cs_ls = (int)q.cs_ls;
+  TX *cstate = static_cast<TX *>(q.conv_state) + b * q.cs_bs;
+  const TX *xBC = static_cast<const TX *>(q.xBC) + b * q.xBC_bs;
+  const int c_B0 = p.nheads * p.dim + g * N, c_C0 = c_B0 + G * N;  // first B / C channel of this group
+  __shared__ __align__(16) float bc_lds[2 * 256];
+  __shared__ int s_last;
+
+  const int n0 = sub * 4;
+  const int nlane = min(max(N - n0, 0), 4);
+  const int n0c = min(n0, N - 4);  // the host requires N % 4 == 0
+  const int row0 = p_begin + rsel;
+  TS *state = static_cast<TS *>(p.state) + (int64_t)b * p.state_bs + h * p.state_hs;
+  const int s_ps = (int)p.state_ps;
+  const bool has_z = p.z != nullptr, has_D = p.D != nullptr, has_dtb = p.dt_bias != nullptr;
+  const TX *zp = has_z ? static_cast<const TX *>(p.z) + b * p.z_bs + h * p.z_hs : xBC;
+  const int z_ps = has_z ? (int)p.z_ps : 0;
+
+  // 1. every load of the thread, branch-free, from clamped addresses: the state rows first
+  float s[UNR][4];
+  bool live[UNR];
+#pragma unroll
+  for (int k = 0; k < UNR; ++k) {
+    const int row = row0 + k * rpp;
+    live[k] = row < p.dim && nlane > 0;
+    ld_state4<TS, true>(state + min(row, p.dim - 1) * s_ps + n0c, 1, 4, s[k]);
+  }
+  // the x channel of row p_begin + lane
+  const int rj = min(p_begin + lane, p.dim - 1);
+  const bool mine = lane < rpp * UNR && p_begin + lane < p.dim;
+  const int cx = h * p.dim + rj;
+  float xsv[3], xw[4], xn, xbias;
+  conv_loads<TX>(q, cstate, xBC, cx, xsv, xn, xw, xbias);
+  const float z_j = ld1<TX>(zp + rj * z_ps);
+  // the B / C channels of this head's group: thread t takes channels t and t + 256 of the 2 N (B first, then C)
+  constexpr int BCI = 2;  // 2 N <= 512
+  float bsv[BCI][3], bw[BCI][4], bxn[BCI], bbias[BCI];
+  int bc_c[BCI];
+#pragma unroll
+  for (int it = 0; it < BCI; ++it) {
+    const int t = min((int)threadIdx.x + it * 256, 2 * N - 1);
+    bc_c[it] = t < N ? c_B0 + t : c_C0 + (t - N);
+    conv_loads<TX>(q, cstate, xBC, bc_c[it], bsv[it], bxn[it], bw[it], bbias[it]);
+  }
+  // per head: dt, dt_bias, A, D
+  const float dt_raw = ld1<TD>(static_cast<const TD *>(p.dt) + b * p.dt_bs + h * p.dt_hs);
+  const float dtb = has_dtb ? static_cast<const float *>(p.dt_bias)[h * p.dt_bias_hs] : 0.f;
+  const float A2 = static_cast<const float *>(p.A)[h * p.A_hs] * kLog2e;
+  const float Dh = has_D ? static_cast<const float *>(p.D)[h * p.D_hs] : 0.f;
+
+  // 2. convolutions: B / C once per workgroup, shared through LDS
+#pragma unroll
+  for (int it = 0; it < BCI; ++it) {
+    const int t = (int)threadIdx.x + it * 256;
+    if (t < 2 * N) bc_lds[t] = round_to<TX>(conv_tap(bsv[it], bxn[it], bw[it], bbias[it], q.silu));
+  }
+  const float x_j = round_to<TX>(conv_tap(xsv, xn, xw, xbias, q.silu));
+  if (mine) conv_shift<TX>(cstate + cx * cs_cs, SL, cs_ls, xsv, xn);  // no other thread reads this channel
+  __syncthreads();
+  float Bv[4], Cv[4];
+  {
+    const f32x4 bq = *reinterpret_cast<const f32x4 *>(bc_lds + n0c), cq = *reinterpret_cast<const f32x4 *>(bc_lds + N + n0c);
+    Bv[0] = bq.x; Bv[1] = bq.y; Bv[2] = bq.z; Bv[3] = bq.w;
+    Cv[0] = cq.x; Cv[1] = cq.y; Cv[2] = cq.z; Cv[3] = cq.w;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool ok = i < nlane;
+      Bv[i] = ok ? Bv[i] : 0.f;
+      Cv[i] = ok ? Cv[i] : 0.f;
+    }
+  }
+  // 3. the state update
+  float dt = dt_raw + dtb;
+  if (p.dt_softplus) dt = softplus_f(dt);
+  const float dA = fast_exp2(A2 * dt);
+  float outs[UNR], xs[UNR], zs[UNR];
+#pragma unroll
+  for (int k = 0; k < UNR; ++k) {
+    const int src = rsel + k * rpp;  // the lane that holds this row's scalars
+    xs[k] = __shfl(x_j, src, 64);
+    zs[k] = __shfl(z_j, src, 64);
+    const float dtx = dt * xs[k];
+    float out = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      s[k][i] = __builtin_fmaf(s[k][i], dA, Bv[i] * dtx);
+      out = __builtin_fmaf(s[k][i], Cv[i], out);
+    }
+    outs[k] = live[k] ? out : 0.f;
+    if (live[k]) st_state4<TS, true>(state + (row0 + k * rpp) * s_ps + n0, 1, nlane, s[k]);
+  }
+  TX *outp = static_cast<TX *>(p.out) + b * p.out_bs + h * p.out_hs;
+#pragma unroll
+  for (int k = 0; k < UNR; ++k) {
+    const int row = row0 + k * rpp;
+    float out = outs[k];
+    for (int off = lpr >> 1; off >= 1; off >>= 1) out += __shfl_xor(out, off, 64);
+    if (row < p.dim && sub == 0) {
+      out = __builtin_fmaf(xs[k], Dh, out);
+      if (has_z) out *= zs[k] * sigmoid_f(zs[k]);
+      st1<TX>(outp + row * (int)p.out_ps, out);
+    }
+  }
+  // 4. count this workgroup off among those of its (batch entry, group), in two levels so that no counter sees
+  // more than SYNC_FAN arrivals (atomics to one address serialise); the last one shifts the conv state of the
+  // group's B / C channels, which it still holds in registers.  Relaxed atomics are enough: the loads of the old
+  // conv state have returned (their values went into LDS before the barrier above), and the last workgroup's stores
+  // follow its own arrival in program order; acquire / release at device scope would write back and invalidate
+  // the L2 at every arrival.
+  if (threadIdx.x == 0) {
+    const int nwg = (int)gridDim.x * hpg, wg = (h - g * hpg) * (int)gridDim.x + (int)blockIdx.x;
+    const int ngrp = (nwg + SYNC_FAN - 1) / SYNC_FAN, grp = wg / SYNC_FAN;
+    const int in_grp = min(SYNC_FAN, nwg - grp * SYNC_FAN);
+    int *cnt = q.sync + ((int64_t)b * G + g) * (ngrp + 1);
+    int last = 0;
+    if (__hip_atomic_fetch_add(cnt + 1 + grp, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == in_grp - 1) {
+      __hip_atomic_store(cnt + 1 + grp, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (__hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ngrp - 1) {
+        __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        last = 1;
+      }
+    }
+    s_last = last;
+  }
+  __syncthreads();
+  if (!s_last) return;
+#pragma unroll
+  for (int it = 0; it < BCI; ++it) {
+    if ((int)threadIdx.x + it * 256 < 2 * N) conv_shift<TX>(cstate + bc_c[it] * cs_cs, SL, cs_ls, bsv[it], bxn[it]);
+  }
+}
+
+int fused_grid_x(const MambaStepParams &p, int *lpr_log2_out) {
+  int lpr_log2 = 0;
+  while ((4 << lpr_log2) < p.dstate) ++lpr_log2;
+  if (lpr_log2_out) *lpr_log2_out = lpr_log2;
+  const int rows_per_block = 4 * (64 >> lpr_log2) * UNR;
+  return (p.dim + rows_per_block - 1) / rows_per_block;
+}
+
+template <typename TS, typename TX, typename TD> int launch_fused(const MambaDecodeStepParams &q, hipStream_t stream) {
+  const MambaStepParams &p = q.ssm;
+  int lpr_log2 = 0;
+  dim3 grid(fused_grid_x(p, &lpr_log2), p.nheads, p.batch), block(256);
+  hipLaunchKernelGGL((decode_step_fused_kernel<TS, TX, TD>), grid, block, 0, stream, q, lpr_log2);
+  return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
+}
+
+template <typename TS, typename TX> int fused_dt(const MambaDecodeStepParams &q, hipStream_t s) {
+  if (q.ssm.dt_dtype == MAMBA_F32) return launch_fused<TS, TX, float>(q, s);
+  if (q.ssm.dt_dtype != DT<TX>::id) return MAMBA_E_UNSUPPORTED;
+  return launch_fused<TS, TX, TX>(q, s);
+}
+template <typename TS> int fused_x(const MambaDecodeStepParams &q, hipStream_t s) {
+  switch (q.ssm.x_dtype) {
+    case MAMBA_F32: return fused_dt<TS, float>(q, s);
+    case MAMBA_BF16: return fused_dt<TS, bf16_t>(q, s);
+    default: return fused_dt<TS, f16_t>(q, s);
+  }
+}
+
 }  // namespace
 
 extern "C" int ssm_state_update(const MambaStepParams *p, mamba_stream_t stream) {
@@ -324,5 +563,50 @@ extern "C" int ssm_state_update(const MambaStepParams *p, mamba_stream_t stream)
     case MAMBA_F32: return dispatch_x<float>(*p, s);
     case MAMBA_BF16: return dispatch_x<bf16_t>(*p, s);
     default: return dispatch_x<f16_t>(*p, s);
+  }
+}
+
+extern "C" int64_t mamba2_decode_step_sync_ints(const MambaDecodeStepParams *q) {
+  if (!q || q->ssm.batch <= 0 || q->ssm.nheads <= 0 || q->ssm.dim <= 0 || q->ssm.dstate <= 0) return MAMBA_E_BADARG;
+  if (q->ssm.ngroups <= 0 || q->ssm.nheads % q->ssm.ngroups != 0) return MAMBA_E_BADARG;
+  const int nwg = fused_grid_x(q->ssm, nullptr) * (q->ssm.nheads / q->ssm.ngroups);  // per (batch entry, group)
+  return (int64_t)q->ssm.batch * q->ssm.ngroups * ((nwg + SYNC_FAN - 1) / SYNC_FAN + 1);
+}
+
+extern "C" int mamba2_decode_step(const MambaDecodeStepParams *q, mamba_stream_t stream) {
+  if (!q) return MAMBA_E_BADARG;
+  const MambaStepParams *p = &q->ssm;
+  if (!p->state || !p->dt || !p->A || !p->out || !q->xBC || !q->conv_state || !q->conv_weight || !q->sync)
+    return MAMBA_E_BADARG;
+  if (p->batch <= 0 || p->nheads <= 0 || p->dim <= 0 || p->dstate <= 0 || p->ngroups <= 0) return MAMBA_E_BADARG;
+  if (p->nheads % p->ngroups != 0) return MAMBA_E_BADARG;
+  if (q->conv_dim != p->nheads * p->dim + 2 * p->ngroups * p->dstate) return MAMBA_E_BADARG;
+  if (p->state_rows < p->batch || q->conv_state_rows < p->batch) return MAMBA_E_BADARG;
+  if (!dtype_ok(p->state_dtype) || !dtype_ok(p->x_dtype) || !dtype_ok(p->dt_dtype)) return MAMBA_E_BADARG;
+  // the form served here; anything else is for the two separate calls
+  if (p->state_batch_indices) return MAMBA_E_UNSUPPORTED;
+  if (reinterpret_cast<uintptr_t>(q->conv_weight) % 16 != 0) return MAMBA_E_UNSUPPORTED;
+  if (q->width < 2 || q->width > CW || q->state_len < q->width - 1 || q->state_len > CW) return MAMBA_E_UNSUPPORTED;
+  if (p->A_dtype != MAMBA_F32 || (p->D && p->D_dtype != MAMBA_F32) || (p->dt_bias && p->dt_bias_dtype != MAMBA_F32))
+    return MAMBA_E_UNSUPPORTED;
+  if (p->dt_ps != 0 || p->A_ps != 0 || p->A_ns != 0 || (p->dt_bias && p->dt_bias_ps != 0) || (p->D && p->D_ps != 0))
+    return MAMBA_E_UNSUPPORTED;
+  if (p->batch > 65535 || p->nheads > 65535 || p->dstate > 256 || p->dstate % 4 != 0) return MAMBA_E_UNSUPPORTED;
+  {
+    const int es = p->state_dtype == MAMBA_F32 ? 4 : 2;
+    const int64_t vb = 4 * es;
+    if (p->state_ns != 1 || reinterpret_cast<uintptr_t>(p->state) % vb != 0 || (p->state_bs * es) % vb != 0 ||
+        (p->state_hs * es) % vb != 0 || (p->state_ps * es) % vb != 0)
+      return MAMBA_E_UNSUPPORTED;
+    auto big = [&](int64_t a) { return (a < 0 ? -a : a) >= (int64_t(1) << 30); };
+    if (big(p->state_ps * p->dim + p->dstate) || big(p->z_ps * p->dim) || big(p->out_ps * p->dim) ||
+        big(q->cs_cs * q->conv_dim + q->cs_ls * q->state_len))
+      return MAMBA_E_UNSUPPORTED;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (p->state_dtype) {
+    case MAMBA_F32: return fused_x<float>(*q, s);
+    case MAMBA_BF16: return fused_x<bf16_t>(*q, s);
+    default: return fused_x<f16_t>(*q, s);
   }
 }

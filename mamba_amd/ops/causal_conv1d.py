@@ -126,11 +126,44 @@ def causal_conv1d_fn(x, weight, bias=None, seq_idx=None, initial_states=None, re
                      final_states_out=None, activation=None):
     """x: (batch, dim, seqlen), position- or channel-contiguous; weight: (dim, width); bias: (dim,);
     seq_idx: (batch, seqlen) int32; activation: None, "silu" or "swish".  out: (batch, dim, seqlen) in
-    x's layout.  Streaming states (initial_states / return_final_states) belong to the decode path of
-    the separate package and are not served here."""
-    if initial_states is not None or return_final_states or final_states_out is not None:
-        raise NotImplementedError("causal_conv1d_fn: streaming conv states are not supported")
-    return CausalConv1dFn.apply(x, weight, bias, seq_idx, activation)
+    x's layout.
+    Streaming (the causal_conv1d package's arguments of the same names):
+        initial_states: (batch, dim, width - 1), the positions in front of x; the output is that of the
+            convolution over [initial_states, x], cut to x's positions (not together with seq_idx)
+        return_final_states: also return (batch, dim, width - 1), the last width - 1 positions of
+            [initial_states, x] (zero-filled on the left when there are fewer); no gradient flows through them
+        final_states_out: a tensor to receive them
+    The streaming form runs the same kernel over the joined row (one extra copy of x)."""
+    if initial_states is None and not return_final_states and final_states_out is None:
+        return CausalConv1dFn.apply(x, weight, bias, seq_idx, activation)
+    width = weight.shape[1]
+    batch, dim, seqlen = x.shape
+    joined = x
+    if initial_states is not None:
+        if seq_idx is not None:
+            raise RuntimeError("causal_conv1d_fn: initial_states cannot be combined with seq_idx")
+        if tuple(initial_states.shape) != (batch, dim, width - 1):
+            raise RuntimeError("causal_conv1d_fn: initial_states must be (batch, dim, width - 1)")
+        _lib.require_gpu(x, initial_states)
+        if x.stride(1) == 1 and x.stride(2) != 1:   # keep a channel-contiguous row channel-contiguous
+            joined = torch.cat([initial_states.to(x.dtype).transpose(1, 2), x.transpose(1, 2)], dim=1).transpose(1, 2)
+        else:
+            joined = torch.cat([initial_states.to(x.dtype), x], dim=2)
+        out = CausalConv1dFn.apply(joined, weight, bias, None, activation)[:, :, width - 1:]
+    else:
+        out = CausalConv1dFn.apply(x, weight, bias, seq_idx, activation)
+    if not return_final_states and final_states_out is None:
+        return out
+    with torch.no_grad():
+        tail = joined[:, :, max(joined.shape[2] - (width - 1), 0):]
+        if tail.shape[2] < width - 1:
+            tail = torch.nn.functional.pad(tail, (width - 1 - tail.shape[2], 0))
+        if final_states_out is not None:
+            final_states_out.copy_(tail)
+            final = final_states_out
+        else:
+            final = tail.clone()
+    return out, final
 
 
 def causal_conv1d_update(x, conv_state, weight, bias=None, activation=None, cache_seqlens=None,
@@ -142,9 +175,10 @@ def causal_conv1d_update(x, conv_state, weight, bias=None, activation=None, cach
             state_len positions of [conv_state, x]
         weight: (dim, width); bias: (dim,)
         conv_state_indices: (batch,) int32, row of conv_state per batch entry (negative: padding)
+        cache_seqlens: (batch,) int32; when given, conv_state is a circular buffer: entry b has seen
+            cache_seqlens[b] positions, position t lives in slot t % state_len, the new ones are written to
+            their slots and nothing is shifted (the causal_conv1d package's argument of the same name)
     Returns out with x's shape and dtype."""
-    if cache_seqlens is not None:
-        raise NotImplementedError("causal_conv1d_update: circular-buffer states (cache_seqlens) are not supported")
     if activation not in (None, "silu", "swish"):
         raise NotImplementedError("activation must be None, silu, or swish")
     _lib.require_gpu(x, conv_state, weight, bias, conv_state_indices)
@@ -166,6 +200,11 @@ def causal_conv1d_update(x, conv_state, weight, bias=None, activation=None, cach
         if tuple(conv_state_indices.shape) != (batch,) or conv_state_indices.dtype != torch.int32:
             raise RuntimeError("causal_conv1d_update: conv_state_indices must be (batch,) int32")
         conv_state_indices = conv_state_indices.contiguous()
+    if cache_seqlens is not None:
+        _lib.require_gpu(cache_seqlens)
+        if tuple(cache_seqlens.shape) != (batch,) or cache_seqlens.dtype != torch.int32:
+            raise RuntimeError("causal_conv1d_update: cache_seqlens must be (batch,) int32")
+        cache_seqlens = cache_seqlens.contiguous()
     if bias is not None and tuple(bias.shape) != (dim,):
         raise RuntimeError("causal_conv1d_update: bias must be (dim,)")
     out = torch.empty_like(x)
@@ -179,6 +218,7 @@ def causal_conv1d_update(x, conv_state, weight, bias=None, activation=None, cach
     p.silu, p.state_rows = int(activation in ("silu", "swish")), conv_state.shape[0]
     p.x, p.conv_state, p.weight, p.bias, p.out = x.data_ptr(), conv_state.data_ptr(), w32.data_ptr(), _lib.ptr(b32), out.data_ptr()
     p.conv_state_indices = _lib.ptr(conv_state_indices)
+    p.cache_seqlens = _lib.ptr(cache_seqlens)
     p.x_bs, p.x_cs, p.x_ls = _strides_bcl(x)
     p.out_bs, p.out_cs, p.out_ls = _strides_bcl(out)
     p.state_bs, p.state_cs, p.state_ls = _strides_bcl(conv_state)

@@ -271,12 +271,27 @@ class SelectiveScanFn(torch.autograd.Function):
         return (du, ddelta, dA, dB, dC, dD, dz, ddelta_bias, None, None)
 
 
+MAX_GRID_BATCH = 65535  # batch rows per launch of the scan kernels
+
+
 def selective_scan_fn(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta_softplus=False,
                       return_last_state=False):
     """if return_last_state is True, returns (out, last_state)
     last_state has shape (batch, dim, dstate). The gradient of the last state is not
     considered in the backward pass (as in the reference, selective_scan_interface.py:118-124).
     """
+    if u.shape[0] > MAX_GRID_BATCH:
+        # the kernels index the batch with one 16-bit grid coordinate: larger batches go in slices (batch rows
+        # are independent; autograd adds up the gradients of the shared A, D, delta_bias and constant B / C)
+        outs = []
+        for i in range(0, u.shape[0], MAX_GRID_BATCH):
+            sl = slice(i, i + MAX_GRID_BATCH)
+            cut = lambda t: t if t is None or t.dim() == 2 else t[sl]
+            outs.append(selective_scan_fn(u[sl], delta[sl], A, cut(B), cut(C), D, None if z is None else z[sl],
+                                          delta_bias, delta_softplus, return_last_state))
+        if return_last_state:
+            return torch.cat([o[0] for o in outs]), torch.cat([o[1] for o in outs])
+        return torch.cat(outs)
     return SelectiveScanFn.apply(u, delta, A, B, C, D, z, delta_bias, delta_softplus, return_last_state)
 
 

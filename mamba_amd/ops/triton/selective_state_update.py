@@ -119,6 +119,119 @@ def selective_state_update(state, x, dt, A, B, C, D=None, z=None, dt_bias=None, 
     return out
 
 
+_SYNC = {}  # (device index, size) -> zeroed int32 counters of mamba2_decode_step (left zero by every call)
+
+E_UNSUPPORTED = -2
+FUSE_MAX_BATCH = 16  # largest batch for which mamba2_decode_step picks the fused kernel by itself
+
+
+def mamba2_decode_step(ssm_state, conv_state, xBC, dt, A, conv_weight, conv_bias=None, D=None, z=None, dt_bias=None,
+                       ngroups=1, activation="silu", dt_softplus=True, fuse=None):
+    """One generated token of a Mamba-2 mixer core: the two calls of the reference's step()
+    (mamba_ssm/modules/mamba2.py:298-336)
+
+        xBC = causal_conv1d_update(xBC, conv_state, conv_weight, conv_bias, activation)
+        x, B, C = split(xBC, [nheads * headdim, ngroups * dstate, ngroups * dstate])
+        y = selective_state_update(ssm_state, x, dt, A, B, C, D, z, dt_bias, dt_softplus)
+
+    as ONE kernel launch where the library serves the form (per-head dt / A / dt_bias / D, conv state of at most
+    4 positions, no state indices), otherwise as those two calls.  Both give the same bits.
+        ssm_state: (batch, nheads, headdim, dstate), updated in place
+        conv_state: (batch, conv_dim, state_len), updated in place; conv_dim = nheads * headdim + 2 * ngroups * dstate
+        xBC: (batch, conv_dim); dt: (batch, nheads); A, dt_bias, D: (nheads,); z: (batch, nheads, headdim)
+        conv_weight: (conv_dim, width); conv_bias: (conv_dim,)
+        fuse: None = one launch where served, False = always the two calls, True = one launch or an error
+    Returns y: (batch, nheads, headdim) in xBC's dtype."""
+    from mamba_amd.ops.causal_conv1d import causal_conv1d_update
+    _, nheads, headdim, dstate = ssm_state.shape
+    batch = xBC.shape[0]
+    conv_dim = nheads * headdim + 2 * ngroups * dstate
+    if tuple(xBC.shape) != (batch, conv_dim):
+        raise RuntimeError(f"mamba2_decode_step: xBC must be (batch, {conv_dim})")
+    if ssm_state.shape[0] < batch:
+        raise RuntimeError("mamba2_decode_step: ssm_state has fewer rows than the batch")
+    if conv_state.dim() != 3 or conv_state.shape[0] < batch or conv_state.shape[1] != conv_dim:
+        raise RuntimeError("mamba2_decode_step: conv_state must be (rows >= batch, conv_dim, state_len)")
+    if tuple(dt.shape) != (batch, nheads) or tuple(A.shape) != (nheads,):
+        raise RuntimeError("mamba2_decode_step: dt must be (batch, nheads) and A (nheads,)")
+    _lib.require_gpu(ssm_state, conv_state, xBC, dt, A, conv_weight, conv_bias, D, z, dt_bias)
+
+    def two_calls():
+        xc = causal_conv1d_update(xBC, conv_state, conv_weight, conv_bias, activation)
+        x, B, C = torch.split(xc, [nheads * headdim, ngroups * dstate, ngroups * dstate], dim=-1)
+        ex = lambda t: None if t is None else t[:, None].expand(nheads, headdim)
+        return selective_state_update(
+            ssm_state, x.reshape(batch, nheads, headdim), dt[:, :, None].expand(batch, nheads, headdim),
+            A[:, None, None].expand(nheads, headdim, dstate), B.reshape(batch, ngroups, dstate),
+            C.reshape(batch, ngroups, dstate), D=ex(D), z=z, dt_bias=ex(dt_bias), dt_softplus=dt_softplus)
+
+    width, state_len = conv_weight.shape[1], conv_state.shape[2]
+    code = _lib.DTYPE_CODE
+    fusable = (activation in (None, "silu", "swish") and xBC.dtype in code and conv_state.dtype == xBC.dtype
+               and ssm_state.dtype in code and 2 <= width <= 4 and width - 1 <= state_len <= 4 and dstate % 4 == 0
+               and xBC.stride(1) == 1 and ssm_state.stride(3) == 1 and (z is None or z.dtype == xBC.dtype))
+    explicit = fuse is True
+    if fuse is None:
+        # Measured (80 heads x 64, 128 states, one MI355X): replayed from a captured graph the fused kernel takes as
+        # long as the two launches at batch 1 (12 us) and 2-16 us longer above (its ordered hand-over of the shared
+        # B / C conv state costs what the second launch costs); called eagerly it saves one host call (27 us against
+        # 47 us per token up to batch ~16, after which kernel time decides).
+        fuse = fusable and batch <= FUSE_MAX_BATCH and not torch.cuda.is_current_stream_capturing()
+        if not fuse:
+            return two_calls()
+    if fuse is False:
+        return two_calls()
+    if not fusable:
+        raise RuntimeError("mamba2_decode_step: this form is not served by the fused kernel")
+    A32 = A.float()
+    D32 = D.float() if D is not None else None
+    dtb32 = dt_bias.float() if dt_bias is not None else None
+    if dt.dtype != xBC.dtype:
+        dt = dt.float()
+    w32 = conv_weight.detach().float().contiguous()
+    b32 = conv_bias.detach().float().contiguous() if conv_bias is not None else None
+    out = torch.empty(batch, nheads, headdim, dtype=xBC.dtype, device=xBC.device)
+    q = _lib.MambaDecodeStepParams()
+    p = q.ssm
+    p.batch, p.nheads, p.dim, p.dstate, p.ngroups = batch, nheads, headdim, dstate, ngroups
+    nsync = int(_lib.load().mamba2_decode_step_sync_ints(q))
+    if nsync <= 0:
+        _lib.check(nsync or -1, "mamba2_decode_step_sync_ints")
+    key = (xBC.device.index, nsync)
+    sync = _SYNC.get(key)
+    if sync is None:
+        sync = _SYNC[key] = torch.zeros(nsync, dtype=torch.int32, device=xBC.device)
+    p.dt_softplus, p.state_rows = int(bool(dt_softplus)), ssm_state.shape[0]
+    p.state_dtype, p.x_dtype, p.dt_dtype, p.bc_dtype = code[ssm_state.dtype], code[xBC.dtype], code[dt.dtype], code[xBC.dtype]
+    p.A_dtype = code[A32.dtype]
+    p.D_dtype = code[D32.dtype] if D32 is not None else 0
+    p.dt_bias_dtype = code[dtb32.dtype] if dtb32 is not None else 0
+    p.state, p.dt, p.A, p.out = ssm_state.data_ptr(), dt.data_ptr(), A32.data_ptr(), out.data_ptr()
+    p.D, p.z, p.dt_bias = _lib.ptr(D32), _lib.ptr(z), _lib.ptr(dtb32)
+    p.state_bs, p.state_hs, p.state_ps, p.state_ns = ssm_state.stride()
+    p.dt_bs, p.dt_hs = dt.stride()
+    p.A_hs = A32.stride(0)
+    if dtb32 is not None:
+        p.dt_bias_hs = dtb32.stride(0)
+    if D32 is not None:
+        p.D_hs = D32.stride(0)
+    if z is not None:
+        p.z_bs, p.z_hs, p.z_ps = z.stride()
+    p.out_bs, p.out_hs, p.out_ps = out.stride()
+    q.conv_dim, q.width, q.state_len = conv_dim, width, state_len
+    q.silu, q.conv_state_rows = int(activation in ("silu", "swish")), conv_state.shape[0]
+    q.xBC, q.conv_state, q.conv_weight, q.conv_bias = xBC.data_ptr(), conv_state.data_ptr(), w32.data_ptr(), _lib.ptr(b32)
+    q.sync = sync.data_ptr()
+    q.xBC_bs = xBC.stride(0)
+    q.cs_bs, q.cs_cs, q.cs_ls = conv_state.stride()
+    with torch.cuda.device(xBC.device):
+        rc = _lib.load().mamba2_decode_step(q, _lib.current_stream(xBC.device))
+    if rc == E_UNSUPPORTED and not explicit:
+        return two_calls()
+    _lib.check(rc, "mamba2_decode_step")
+    return out
+
+
 def selective_state_update_ref(state, x, dt, A, B, C, D=None, z=None, dt_bias=None, dt_softplus=False):
     """One decode step from plain torch operators, in place on `state`, on whatever device the
     inputs live on (the role of the reference's selective_state_update_ref,

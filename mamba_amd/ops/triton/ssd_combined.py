@@ -279,6 +279,9 @@ class MambaChunkScanCombinedFn(torch.autograd.Function):
                 None)
 
 
+MAX_GRID_ROWS = 65535  # (batch, head) pairs per launch of the SSD kernels
+
+
 def mamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initial_states=None,
                               seq_idx=None, cu_seqlens=None, dt_softplus=False, dt_limit=(0.0, float("inf")),
                               return_final_states=False, return_varlen_states=False, state_dtype=None):
@@ -301,6 +304,22 @@ def mamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bia
     Return:
         out: (batch, seqlen, nheads, headdim) [, final_states (batch, nheads, headdim, dstate) fp32]
     """
+    batch, nheads = x.shape[0], x.shape[2]
+    rows = MAX_GRID_ROWS // max(nheads, 1)
+    if batch > rows >= 1 and not return_varlen_states:
+        # the kernels index (batch, head) pairs with one 16-bit grid coordinate: larger batches go in slices
+        # (batch rows are independent; autograd adds up the gradients of the shared A, D, dt_bias)
+        outs = []
+        for i in range(0, batch, rows):
+            sl = slice(i, i + rows)
+            cut = lambda t: None if t is None else t[sl]
+            outs.append(mamba_chunk_scan_combined(x[sl], dt[sl], A, B[sl], C[sl], chunk_size, D=D, z=cut(z), dt_bias=dt_bias,
+                                                  initial_states=cut(initial_states), seq_idx=cut(seq_idx),
+                                                  dt_softplus=dt_softplus, dt_limit=dt_limit,
+                                                  return_final_states=return_final_states, state_dtype=state_dtype))
+        if return_final_states:
+            return torch.cat([o[0] for o in outs]), torch.cat([o[1] for o in outs])
+        return torch.cat(outs)
     return MambaChunkScanCombinedFn.apply(x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, seq_idx,
                                           cu_seqlens, dt_softplus, dt_limit, return_final_states,
                                           return_varlen_states, state_dtype)

@@ -38,7 +38,7 @@ def test_query_and_strerror():
     assert b"unsupported" in lib.mamba_hip_strerror(-2)
 
 
-@pytest.mark.parametrize("name", ["MambaScanParams", "MambaStepParams", "SsdParams", "CausalConvParams", "CausalConvUpdateParams",
+@pytest.mark.parametrize("name", ["MambaScanParams", "MambaStepParams", "MambaDecodeStepParams", "SsdParams", "CausalConvParams", "CausalConvUpdateParams",
                                   "CausalConvVarlenParams", "NormGatedParams", "NormResidualParams"])
 def test_ctypes_structs_match_c_layout(name):
     cls = getattr(_lib, name)
@@ -63,6 +63,7 @@ def test_null_and_inconsistent_arguments_are_rejected_before_launch():
     assert lib.mamba1_scan_fwd(ctypes.byref(p), None) == -1          # null pointers
     s = _lib.MambaStepParams()
     assert lib.ssm_state_update(ctypes.byref(s), None) == -1
+    assert lib.mamba2_decode_step(ctypes.byref(_lib.MambaDecodeStepParams()), None) == -1
     q = _lib.SsdParams()
     assert lib.ssd_combined_fwd(ctypes.byref(q), None) == -1
     assert lib.ssd_combined_bwd(ctypes.byref(q), None) == -1

@@ -125,8 +125,8 @@ def test_causal_conv1d_update_steps_match_the_sequence_kernel_and_indices():
         assert float(out[2].abs().max()) == 0.0
     assert torch.equal(pool[[1, 2, 4, 6]], untouched[[1, 2, 4, 6]])
     assert torch.equal(pool[5], x[0, :, L - width:])
-    with pytest.raises(NotImplementedError):
-        causal_conv1d_update(x[:, :, 0], pool[:4], w, bias, "silu", cache_seqlens=idx)
+    with pytest.raises(RuntimeError):   # cache_seqlens must be int32 of the batch's length
+        causal_conv1d_update(x[:, :, 0], pool[:4], w, bias, "silu", cache_seqlens=idx[:2])
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -142,3 +142,76 @@ def test_causal_conv1d_varlen_states(dtype):
         got = causal_conv1d_varlen_states(x.cuda(), cu.cuda(), state_len)
         assert got.shape == (len(lens), dim, state_len) and got.stride(1) == 1
         assert torch.equal(got.cpu(), ref)
+
+
+@pytest.mark.parametrize("channel_last", [False, True])
+@pytest.mark.parametrize("width,seqlen", [(4, 64), (3, 17), (4, 2), (2, 1)])
+def test_causal_conv1d_streaming_states(width, seqlen, channel_last):
+    """initial_states / return_final_states: a row cut in two and convolved piece by piece, the second piece
+    starting from the first one's final states, equals the row convolved whole (outputs and every gradient);
+    checked against F.conv1d over the joined row."""
+    import torch.nn.functional as F
+    from mamba_amd.ops.causal_conv1d import causal_conv1d_fn
+    g = torch.Generator().manual_seed(width * 100 + seqlen)
+    batch, dim = 2, 24
+    x = torch.randn(batch, dim, seqlen, generator=g)
+    init = torch.randn(batch, dim, width - 1, generator=g)
+    w, bias = 0.5 * torch.randn(dim, width, generator=g), torch.randn(dim, generator=g)
+    dout = torch.randn(batch, dim, seqlen, generator=g)
+    xr, ir, wr, br = (t.clone().requires_grad_() for t in (x, init, w, bias))
+    ref = F.silu(F.conv1d(torch.cat([ir, xr], dim=2), wr[:, None, :], br, groups=dim))
+    (ref * dout).sum().backward()
+    lay = (lambda t: t.cuda().transpose(1, 2).contiguous().transpose(1, 2)) if channel_last else (lambda t: t.cuda())
+    xg, ig = lay(x).requires_grad_(), lay(init).requires_grad_()
+    wg, bg = w.cuda().requires_grad_(), bias.cuda().requires_grad_()
+    out, fin = causal_conv1d_fn(xg, wg, bg, initial_states=ig, return_final_states=True, activation="silu")
+    (out * dout.cuda()).sum().backward()
+    _close("out", out, ref, 6e-4, 2e-3)
+    _close("final_states", fin, torch.cat([init, x], dim=2)[:, :, -(width - 1):], 0, 0)
+    for name, a, b in (("dx", xg.grad, xr.grad), ("dinitial_states", ig.grad, ir.grad), ("dweight", wg.grad, wr.grad),
+                       ("dbias", bg.grad, br.grad)):
+        _close(name, a, b, 6e-4, 2e-3)
+    # without initial states the final states are the row's own tail, zero-filled on the left
+    out2, fin2 = causal_conv1d_fn(xg.detach(), wg.detach(), bg.detach(), return_final_states=True, activation="silu")
+    want = F.pad(x, (max(width - 1 - seqlen, 0), 0))[:, :, -(width - 1):]
+    _close("final_states without initial", fin2, want, 0, 0)
+    buf = torch.empty(batch, dim, width - 1, device="cuda")
+    causal_conv1d_fn(xg.detach(), wg.detach(), bg.detach(), final_states_out=buf, activation="silu")
+    _close("final_states_out", buf, want, 0, 0)
+
+
+@pytest.mark.parametrize("width,state_len", [(4, 4), (4, 7), (3, 2), (2, 5)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_causal_conv1d_update_circular_buffer(width, state_len, dtype):
+    """cache_seqlens: the conv state as a circular buffer.  Tokens fed one at a time (and two at a time) through
+    the circular form must equal the shifting form fed the same tokens, at every step and for batch entries
+    that stand at different positions."""
+    from mamba_amd.ops.causal_conv1d import causal_conv1d_update
+    g = torch.Generator().manual_seed(width * 10 + state_len)
+    batch, dim, steps = 3, 40, 11
+    w, bias = (0.5 * torch.randn(dim, width, generator=g)).to(dtype).cuda(), torch.randn(dim, generator=g).to(dtype).cuda()
+    xs = torch.randn(steps, batch, dim, generator=g).to(dtype).cuda()
+    start = torch.tensor([0, 5, 9], dtype=torch.int32)       # positions the entries have already seen
+    shift_state = torch.zeros(batch, dim, state_len, dtype=dtype, device="cuda")
+    ring_state = torch.zeros(batch, dim, state_len, dtype=dtype, device="cuda")
+    lens = start.clone().cuda()
+    for t in range(steps):
+        want = causal_conv1d_update(xs[t], shift_state, w, bias, "silu")
+        got = causal_conv1d_update(xs[t], ring_state, w, bias, "silu", cache_seqlens=lens)
+        assert torch.equal(got, want), f"step {t}"
+        lens += 1
+    # the ring holds the same last positions, rotated by each entry's own count
+    for b in range(batch):
+        n = int(lens[b])
+        for k in range(min(state_len, steps)):
+            assert torch.equal(ring_state[b, :, (n - 1 - k) % state_len], shift_state[b, :, state_len - 1 - k])
+    # two tokens per call
+    ring2 = torch.zeros_like(ring_state)
+    shift2 = torch.zeros_like(shift_state)
+    lens2 = start.clone().cuda()
+    for t in range(0, steps - 1, 2):
+        pair = xs[t:t + 2].permute(1, 2, 0).contiguous()      # (batch, dim, 2)
+        want = causal_conv1d_update(pair, shift2, w, bias, "silu")
+        got = causal_conv1d_update(pair, ring2, w, bias, "silu", cache_seqlens=lens2)
+        assert torch.equal(got, want), f"pair at {t}"
+        lens2 += 2
