@@ -1,9 +1,9 @@
 """Run-to-run reproducibility (the reference's tests/test_determinism.py:186-211 asks for bitwise equality in
-its deterministic mode and 1e-2 agreement with the default mode).  Here: every forward operator, the decode step
-and the norm backward passes use no float atomics and must repeat bit for bit; the scan / conv backward passes
-sum dB, dC, ddt, dA, dD and the conv weight gradient with float atomics, so their repeats must agree to
-rounding noise of the sums (far inside the reference's 1e-2) but not bit for bit.  There is no deterministic
-mode for those yet."""
+its deterministic mode and 1e-2 agreement with the default mode).  Here: every forward operator, the decode step,
+the norm backward passes and the Mamba-1 scan's backward pass (real A) use no float atomics and must repeat bit
+for bit in the one mode there is; the SSD and conv backward passes still sum dB, dC, ddt, dA, dD and the conv
+weight gradient with float atomics, so their repeats must agree to rounding noise of the sums (far inside the
+reference's 1e-2) but not bit for bit."""
 import pytest
 import torch
 
@@ -106,7 +106,10 @@ def test_scan_backward_repeats_to_rounding_noise():
                                   z=leaves["z"], dt_bias=leaves["dt_bias"], dt_softplus=True).backward(t["dout"])
         return [leaves[k].grad for k in names]
 
-    for fn in (mamba1, ssd):
+    a, b = _twice(mamba1)   # per-workgroup partial sums added up in a fixed order: every gradient repeats exactly
+    for ga, gb in zip(a, b):
+        assert torch.equal(ga, gb)
+    for fn in (ssd,):
         a, b = _twice(fn)
         # a 16-bit gradient may flip its last bit (2^-8 of the element); fp32 sums differ by summation order only.
         # Both are inside the reference's det-vs-default bound of 1e-2.
