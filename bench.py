@@ -245,6 +245,19 @@ def bench_ssd(dev, steps, warmup):
         step()
     torch.cuda.synchronize()
     sec = (time.perf_counter() - t0) / steps
+    # the same step in the deterministic mode (integer atomics on fixed-point terms in the backward pass)
+    from mamba_amd.utils.determinism import set_deterministic_mode
+    set_deterministic_mode(True)
+    try:
+        step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(max(3, steps // 4)):
+            step()
+        torch.cuda.synchronize()
+        det_sec = (time.perf_counter() - t0) / max(3, steps // 4)
+    finally:
+        set_deterministic_mode(None)
     with torch.no_grad():
         fwd_ms = event_ms(fwd, max(5, min(steps, 50)))
         # the fused scan kernel alone, on the buffers of one forward pass
@@ -267,7 +280,8 @@ def bench_ssd(dev, steps, warmup):
     return ({
         "metric": "SSD mamba_chunk_scan_combined fwd+bwd tokens/s at 1 GPU", "value": batch * L / sec,
         "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": sec * 1e3,
-        "fwd_ms": fwd_ms, "higher_is_better": True, "dtype": "bf16 in/out, fp32 accumulation", "data": "synthetic",
+        "fwd_ms": fwd_ms, "deterministic_ms_per_step": det_sec * 1e3, "higher_is_better": True,
+        "dtype": "bf16 in/out, fp32 accumulation", "data": "synthetic",
         "config": {"workload": f"Mamba-2 SSD fwd+bwd: batch {batch}, seqlen {L}, {H} heads x {P}, d_state {N}, "
                                f"{G} group, chunk {Q}, bf16 (benchmark configuration 2)"},
         "roofline": vs_measured_copy({"bound": "hbm", "kernel": "chunk_scan_fwd_fused_kernel", "achieved": nbytes / scan_ms / 1e6,
@@ -696,7 +710,8 @@ def main():
         # the other benchmark configurations, timed in the same run (each entry is the line its own
         # --workload prints): configuration 2 (SSD, with the MFMA figures), 3 (decode, 1000 consecutive
         # steps) and 4 (packed SSD)
-        keep = ("value", "unit", "ms_per_step", "fwd_ms", "event_ms_per_step", "steps", "config", "roofline")
+        keep = ("value", "unit", "ms_per_step", "fwd_ms", "deterministic_ms_per_step", "event_ms_per_step", "steps",
+                "config", "roofline")
         extra = {}
         for name, fn in (("ssd", lambda: bench_ssd(dev, args.steps, args.warmup)),
                          ("decode", lambda: bench_decode(dev, 1000, 10)),

@@ -302,6 +302,16 @@ typedef struct SsdParams {
   void *gbuf;                           /* (b, L, H, P) of `dtype`: dout * silu(z); used iff z != NULL */
   int64_t dout_bs, dout_ls, dout_hs;
   int64_t dx_bs, dx_ls, dx_hs;          /* dx may be a slice of a wider buffer; unit headdim stride */
+  /* ---- deterministic backward (all null: float atomics, whose order changes the last bits from run to run) ----
+   * det_scale: device, {s, 1 / s} with s a power of two chosen by the caller from the size of the upstream gradients
+   * (2^30 / 2^floor(log2(max |dout|)) keeps ~9 decimal digits below that maximum and 9 above it).  Every term of a
+   * sum that several workgroups share is multiplied by s, rounded to an integer and added with a 64-bit integer
+   * atomic into the sum's shadow; integer adds are associative, so the sum does not depend on their order.  The
+   * shadows have the shapes of dD, ddA_cumsum, ddt_out, dCB, dB32, dC32, dA, ddt_bias and are zero on entry;
+   * ssd_combined_bwd converts each into its float buffer (ssd_det_convert) before that buffer's first reader runs.
+   * Counterpart of the reference's deterministic mode, mamba_ssm/utils/determinism.py:21-27. */
+  const float *det_scale;
+  int64_t *det_dD, *det_ddA_cumsum, *det_ddt_out, *det_dCB, *det_dB, *det_dC, *det_dA, *det_ddt_bias;
 } SsdParams;
 
 /* forward stages, in launch order */
@@ -340,6 +350,9 @@ int ssd_chunk_state_varlen(const SsdParams *p, const int32_t *cu_seqlens, int ns
  * ddA_cumsum holds the gradient with respect to the cumulative sums a_l; the last
  * stage turns it into the gradient of the per-position dt * A. */
 int ssd_bwd_dz(const SsdParams *p, mamba_stream_t stream);
+/* dst[i] = shadow[i] / s for i < n (det_scale = {s, 1 / s} on the device): the step between the stages of a
+ * deterministic backward pass that ssd_combined_bwd inserts by itself */
+int ssd_det_convert(const int64_t *shadow, float *dst, int64_t n, const float *det_scale, mamba_stream_t stream);
 int ssd_bwd_dstates(const SsdParams *p, mamba_stream_t stream);
 int ssd_state_passing_bwd(const SsdParams *p, mamba_stream_t stream);
 int ssd_bwd_dx(const SsdParams *p, mamba_stream_t stream);
@@ -384,6 +397,10 @@ typedef struct CausalConvParams {
   float *dbias; /* nullable */
   int64_t dout_bs, dout_cs, dout_ls;
   int64_t dx_bs, dx_cs, dx_ls;
+  /* deterministic backward (all null: float atomics): fixed-point scale {s, 1 / s} on the device and int64 shadows
+   * of dweight (dim, width) and dbias (dim), zero on entry; the caller converts them with ssd_det_convert */
+  const float *det_scale;
+  int64_t *det_dweight, *det_dbias;
 } CausalConvParams;
 
 int causal_conv1d_fwd(const CausalConvParams *p, mamba_stream_t stream);

@@ -65,6 +65,8 @@ class SsdParams(ctypes.Structure):
         + [(n, c_vp) for n in ("dout", "dfinal_states", "dx", "dz", "ddt", "dB", "dC", "dA", "ddt_bias", "dD",
                                "dinitial_states", "dstates", "ddA_cumsum", "ddt_out", "dCB", "dB32", "dC32", "gbuf")]
         + [(n, c_i64) for n in ("dout_bs", "dout_ls", "dout_hs", "dx_bs", "dx_ls", "dx_hs")]
+        + [(n, c_vp) for n in ("det_scale", "det_dD", "det_ddA_cumsum", "det_ddt_out", "det_dCB", "det_dB", "det_dC",
+                               "det_dA", "det_ddt_bias")]
     )
 
 
@@ -75,6 +77,7 @@ class CausalConvParams(ctypes.Structure):
         + [(n, c_i64) for n in ("x_bs", "x_cs", "x_ls", "out_bs", "out_cs", "out_ls")]
         + [(n, c_vp) for n in ("dout", "dx", "dweight", "dbias")]
         + [(n, c_i64) for n in ("dout_bs", "dout_cs", "dout_ls", "dx_bs", "dx_cs", "dx_ls")]
+        + [(n, c_vp) for n in ("det_scale", "det_dweight", "det_dbias")]
     )
 
 
@@ -157,6 +160,8 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = [ctypes.POINTER(SsdParams), c_vp]
         fn.restype = ctypes.c_int
+    lib.ssd_det_convert.argtypes = [c_vp, c_vp, c_i64, c_vp, c_vp]
+    lib.ssd_det_convert.restype = ctypes.c_int
     lib.ssd_chunk_state_varlen.argtypes = [ctypes.POINTER(SsdParams), c_vp, ctypes.c_int, c_vp, c_vp]
     lib.ssd_chunk_state_varlen.restype = ctypes.c_int
     lib.ssd_chunk_scan_fwd_fused_supported.argtypes = [ctypes.POINTER(SsdParams)]

@@ -22,6 +22,19 @@ DEVI float dsilu(float pre) {  // d/dpre silu(pre)
 }
 DEVI float silu_f(float v) { return v * sigmoid_f(v); }
 
+// Shared sums (dweight, dbias): float atomics, or -- deterministic mode, p.det_scale set -- 64-bit integer atomics
+// on terms scaled to a fixed point, whose result does not depend on the order of the adds (see SsdParams).
+DEVI void conv_acc_add(const CausalConvParams &p, float *dst, int64_t *shadow, int64_t idx, float v) {
+  if (p.det_scale) {
+    const float q = fminf(fmaxf(v * p.det_scale[0], -9.0e18f), 9.0e18f);
+    __hip_atomic_fetch_add(reinterpret_cast<unsigned long long *>(shadow + idx),
+                           static_cast<unsigned long long>(static_cast<long long>(__builtin_rintf(q))), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+  } else {
+    unsafeAtomicAdd(dst + idx, v);
+  }
+}
+
 // Taps right-aligned in 4 slots: slot 3 multiplies x[l], slot 0 multiplies x[l - 3].
 DEVI void load_taps(const CausalConvParams &p, int c, float (&w)[MAXW], float &bias) {
 #pragma unroll
@@ -150,9 +163,9 @@ template <typename T, bool VEC> __global__ __launch_bounds__(256) void conv_rows
 #pragma unroll
     for (int k = 0; k < MAXW; ++k) {
       const int j = k - (MAXW - p.width);
-      if (j >= 0 && dw[k] != 0.f) unsafeAtomicAdd(p.dweight + (int64_t)c * p.width + j, dw[k]);
+      if (j >= 0 && dw[k] != 0.f) conv_acc_add(p, p.dweight, p.det_dweight, (int64_t)c * p.width + j, dw[k]);
     }
-    if (p.dbias && db != 0.f) unsafeAtomicAdd(p.dbias + c, db);
+    if (p.dbias && db != 0.f) conv_acc_add(p, p.dbias, p.det_dbias, c, db);
   }
 }
 
@@ -362,12 +375,12 @@ template <typename T, bool VEC> __global__ __launch_bounds__(256) void conv_cl_b
 #pragma unroll
         for (int r = 0; r < NRUN - 1; ++r) v += red[r][cg][e * (MAXW + 1) + k];
         const int j = k - (MAXW - p.width);
-        if (j >= 0 && v != 0.f) unsafeAtomicAdd(p.dweight + (int64_t)(c0 + e) * p.width + j, v);
+        if (j >= 0 && v != 0.f) conv_acc_add(p, p.dweight, p.det_dweight, (int64_t)(c0 + e) * p.width + j, v);
       }
       float v = db[e];
 #pragma unroll
       for (int r = 0; r < NRUN - 1; ++r) v += red[r][cg][e * (MAXW + 1) + MAXW];
-      if (p.dbias && v != 0.f) unsafeAtomicAdd(p.dbias + c0 + e, v);
+      if (p.dbias && v != 0.f) conv_acc_add(p, p.dbias, p.det_dbias, c0 + e, v);
     }
   }
 }
@@ -453,6 +466,7 @@ int check(const CausalConvParams *p, bool bwd) {
   if (p->batch > 65535) return MAMBA_E_UNSUPPORTED;
   if (!bwd && !p->out) return MAMBA_E_BADARG;
   if (bwd && (!p->dout || !p->dx || !p->dweight)) return MAMBA_E_BADARG;
+  if (bwd && p->det_scale && (!p->det_dweight || (p->dbias && !p->det_dbias))) return MAMBA_E_BADARG;
   if (p->x_ls != 1 && p->x_cs != 1) return MAMBA_E_UNSUPPORTED;
   return MAMBA_OK;
 }

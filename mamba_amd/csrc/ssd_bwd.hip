@@ -32,6 +32,31 @@ __host__ __device__ inline int head_splits(int heads_per_group) { return (heads_
 DEVI float *chunk_row(float *base, const SsdParams &p, int b, int h, int c) {
   return base + (((int64_t)b * p.nheads + h) * p.nchunks + c) * p.chunk_size;
 }
+DEVI int64_t chunk_off(const SsdParams &p, int b, int h, int c) {
+  return (((int64_t)b * p.nheads + h) * p.nchunks + c) * p.chunk_size;
+}
+
+// Sums that several workgroups add into one address.  Default: float atomics (the order of the adds, hence the
+// last bits of the sum, changes from run to run).  Deterministic mode (p.det_scale set): the term is scaled by a
+// power of two common to the whole call, rounded to an integer and added with a 64-bit integer atomic into the
+// shadow of the buffer; integer addition is associative, so the sum is the same in every order, and
+// det_convert_kernel turns the shadow into the float buffer before its first reader runs.
+DEVI float det_scale_of(const SsdParams &p) { return p.det_scale ? p.det_scale[0] : 0.f; }
+DEVI void acc_add(float *dst, int64_t *shadow, int64_t idx, float v, float dsc) {
+  if (dsc != 0.f) {
+    const float q = fminf(fmaxf(v * dsc, -9.0e18f), 9.0e18f);
+    __hip_atomic_fetch_add(reinterpret_cast<unsigned long long *>(shadow + idx),
+                           static_cast<unsigned long long>(static_cast<long long>(__builtin_rintf(q))), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+  } else {
+    unsafeAtomicAdd(dst + idx, v);
+  }
+}
+__global__ __launch_bounds__(256) void det_convert_kernel(const int64_t *__restrict__ src, float *__restrict__ dst, int64_t n,
+                                                          const float *__restrict__ scale) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) dst[i] = (float)((double)src[i] * (double)scale[1]);
+}
 
 // Sums acc[m][n] * fx(m, n) over n for every row m of the block tile into rows[64] (LDS, zeroed
 // here).  All 256 threads call; rows[] is valid after the trailing barrier.
@@ -162,7 +187,7 @@ template <typename T> __global__ __launch_bounds__(256) void bwd_dz_kernel(const
     if (Dp && !fixed_cols) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        if (e < nv) unsafeAtomicAdd(p.dD + (p.D_has_hdim ? h * P + c8 + e : h), dDacc[e]);
+        if (e < nv) acc_add(p.dD, p.det_dD, p.D_has_hdim ? h * P + c8 + e : h, dDacc[e], det_scale_of(p));
         dDacc[e] = 0.f;
       }
     }
@@ -177,7 +202,7 @@ template <typename T> __global__ __launch_bounds__(256) void bwd_dz_kernel(const
       if (tid < P) {
         float sacc = 0.f;
         for (int r = tid / 8; r < 256; r += pchunks) sacc += red[r * 9 + (tid & 7)];
-        unsafeAtomicAdd(p.dD + h * P + tid, sacc);
+        acc_add(p.dD, p.det_dD, h * P + tid, sacc, det_scale_of(p));
       }
     } else if (tid < 64) {
       float sacc = 0.f;
@@ -186,7 +211,7 @@ template <typename T> __global__ __launch_bounds__(256) void bwd_dz_kernel(const
 #pragma unroll
         for (int e = 0; e < 8; ++e) sacc += red[(tid * 4 + r) * 9 + e];
       sacc = wave_sum(sacc);
-      if (tid == 0) unsafeAtomicAdd(p.dD + h, sacc);
+      if (tid == 0) acc_add(p.dD, p.det_dD, h, sacc, det_scale_of(p));
     }
   }
 }
@@ -351,7 +376,7 @@ template <int W> __global__ __launch_bounds__(256) void state_passing_bwd_kernel
       part = live ? part * sc : 0.f;
       part = wave_sum_to_last(part);
       if (lane == 63 && part != 0.f)
-        unsafeAtomicAdd(p.ddA_cumsum + (((int64_t)b * H + h) * nc + c) * Q + Q - 1, part);
+        acc_add(p.ddA_cumsum, p.det_ddA_cumsum, (((int64_t)b * H + h) * nc + c) * Q + Q - 1, part, det_scale_of(p));
     }
   }
   if (live && p.dinitial_states) G.store(p.dinitial_states + ((int64_t)b * H + h) * PN + e);
@@ -505,14 +530,15 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
   q2 += __shfl_xor(q2, 1, 64);
   q2 += __shfl_xor(q2, 2, 64);
   const bool lead = (tid & 3) == 0 && row_ok;
-  float *dda = chunk_row(p.ddA_cumsum, p, b, h, c);
+  const int64_t row_off = chunk_off(p, b, h, c);
+  const float dsc = det_scale_of(p);
   if (lead) {
-    unsafeAtomicAdd(chunk_row(p.ddt_out, p, b, h, c) + s, q2);
-    unsafeAtomicAdd(dda + s, -dts * q1);  // chunk-state terms: -dt_s <x_s, acc1_s> at s ...
+    acc_add(p.ddt_out, p.det_ddt_out, row_off + s, q2, dsc);
+    acc_add(p.ddA_cumsum, p.det_ddA_cumsum, row_off + s, -dts * q1, dsc);  // chunk-state terms: -dt_s <x_s, acc1_s> at s ...
   }
   // ... and + at the chunk end: one address for the whole tile, so one atomic per wave
   const float endsum = wave_sum_to_last(lead ? dts * q1 : 0.f);
-  if ((tid & 63) == 63) unsafeAtomicAdd(dda + Q - 1, endsum);
+  if ((tid & 63) == 63) acc_add(p.ddA_cumsum, p.det_ddA_cumsum, row_off + Q - 1, endsum, dsc);
 }
 
 // ---------------------------------------------- state-path parts of dB, dC
@@ -589,7 +615,7 @@ template <typename T, bool SPLIT, int PARTS> DEVI void dBC_state_body(const SsdP
         tid);
     acc_foreach(accB, tid, [&](int m, int n, float v) {
       const int s = st * GB + m, nn = nt * GB + n;
-      if (s < qlim && nn < N) unsafeAtomicAdd(p.dB32 + (((int64_t)b * L + t0 + s) * G + g) * N + nn, v);
+      if (s < qlim && nn < N) acc_add(p.dB32, p.det_dB, (((int64_t)b * L + t0 + s) * G + g) * N + nn, v, det_scale_of(p));
       return v;
     });
   }
@@ -649,14 +675,15 @@ template <typename T, bool SPLIT, int PARTS> DEVI void dBC_state_body(const SsdP
         });
     acc_foreach(accC, tid, [&](int m, int n, float v) {
       const int l = st * GB + m, nn = nt * GB + n;
-      if (l < qlim && nn < N) unsafeAtomicAdd(p.dC32 + (((int64_t)b * L + t0 + l) * G + g) * N + nn, v);
+      if (l < qlim && nn < N) acc_add(p.dC32, p.det_dC, (((int64_t)b * L + t0 + l) * G + g) * N + nn, v, det_scale_of(p));
       return v;
     });
     __syncthreads();
     for (int idx = tid; idx < nh * GB; idx += 256) {
       const int hl = idx / GB, r = idx % GB, l = st * GB + r;
       const float d = dda_s[0][hl][r] + dda_s[1][hl][r];
-      if (l < qlim && d != 0.f) unsafeAtomicAdd(chunk_row(p.ddA_cumsum, p, b, g * hpg + hs + hl * nsplit, c) + l, d);
+      if (l < qlim && d != 0.f)
+        acc_add(p.ddA_cumsum, p.det_ddA_cumsum, chunk_off(p, b, g * hpg + hs + hl * nsplit, c) + l, d, det_scale_of(p));
     }
   }
 }
@@ -722,9 +749,9 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dB_
     for (int r = 0; r < 4; ++r) {
       const int s = st * GB + wm * 32 + tm * 16 + gq * 4 + r;
       if (s >= qlim) continue;
-      float *row = p.dB32 + (((int64_t)b * L + t0 + s) * G + g) * N + nt * WB + wn * 64 + i;
+      const int64_t row = (((int64_t)b * L + t0 + s) * G + g) * N + nt * WB + wn * 64 + i;
 #pragma unroll
-      for (int tn = 0; tn < 4; ++tn) unsafeAtomicAdd(row + tn * 16, accB.v[tm][tn][r]);
+      for (int tn = 0; tn < 4; ++tn) acc_add(p.dB32, p.det_dB, row + tn * 16, accB.v[tm][tn][r], det_scale_of(p));
     }
 }
 
@@ -827,7 +854,8 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_
   for (int idx = tid; idx < nh * GB; idx += 256) {
     const int hl = idx / GB, r = idx % GB, l = st * GB + r;
     const float d = dda_s[0][hl][r] + dda_s[1][hl][r] - (hl > 0 ? dda_s[0][hl - 1][r] + dda_s[1][hl - 1][r] : 0.f);
-    if (l < qlim && d != 0.f) unsafeAtomicAdd(chunk_row(p.ddA_cumsum, p, b, g * hpg + hs + hl * nsplit, c) + l, d);
+    if (l < qlim && d != 0.f)
+      acc_add(p.ddA_cumsum, p.det_ddA_cumsum, chunk_off(p, b, g * hpg + hs + hl * nsplit, c) + l, d, det_scale_of(p));
   }
 #pragma unroll
   for (int tm = 0; tm < 2; ++tm)
@@ -835,9 +863,9 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_
     for (int r = 0; r < 4; ++r) {
       const int l = st * GB + wm * 32 + tm * 16 + gq * 4 + r;
       if (l >= qlim) continue;
-      float *row = p.dC32 + (((int64_t)b * L + t0 + l) * G + g) * N + nt * WB + wn * 64 + i;
+      const int64_t row = (((int64_t)b * L + t0 + l) * G + g) * N + nt * WB + wn * 64 + i;
 #pragma unroll
-      for (int tn = 0; tn < 4; ++tn) unsafeAtomicAdd(row + tn * 16, acc.v[tm][tn][r]);
+      for (int tn = 0; tn < 4; ++tn) acc_add(p.dC32, p.det_dC, row + tn * 16, acc.v[tm][tn][r], det_scale_of(p));
     }
 }
 
@@ -866,7 +894,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_
   const int t0 = c * Q, qlim = min(Q, L - t0);
   const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
   const View4 gv = g_view(p);
-  float *dCB = p.dCB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
+  const int64_t dCB_off = (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
   const float *CB = p.CB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
   // This lane's 16 accumulator positions: CB there (the same for every head) and the causal /
   // same-sequence mask, kept as zeros in cbr and a bit per position.
@@ -964,14 +992,14 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_
   __syncthreads();
   for (int idx = tid; idx < nh * GB; idx += 256) {
     const int hl = idx / GB, r = idx % GB;
-    float *dda = chunk_row(p.ddA_cumsum, p, b, g * hpg + hs + hl * nsplit, c);
+    const int64_t dda = chunk_off(p, b, g * hpg + hs + hl * nsplit, c);
     const float row = rs_s[0][hl][r] + rs_s[1][hl][r], col = cs_s[0][hl][r] + cs_s[1][hl][r];
-    if (lt * GB + r < Q && row != 0.f) unsafeAtomicAdd(dda + lt * GB + r, row);
-    if (st * GB + r < Q && col != 0.f) unsafeAtomicAdd(dda + st * GB + r, -col);
+    if (lt * GB + r < Q && row != 0.f) acc_add(p.ddA_cumsum, p.det_ddA_cumsum, dda + lt * GB + r, row, det_scale_of(p));
+    if (st * GB + r < Q && col != 0.f) acc_add(p.ddA_cumsum, p.det_ddA_cumsum, dda + st * GB + r, -col, det_scale_of(p));
   }
   acc_foreach(sum, tid, [&](int m, int n, float v) {
     const int l = lt * GB + m, s = st * GB + n;
-    if (l < Q && s < Q && v != 0.f) unsafeAtomicAdd(dCB + (int64_t)l * Q + s, v);  // dCB starts zeroed
+    if (l < Q && s < Q && v != 0.f) acc_add(p.dCB, p.det_dCB, dCB_off + (int64_t)l * Q + s, v, det_scale_of(p));  // dCB starts zeroed
     return v;
   });
 }
@@ -1101,8 +1129,8 @@ __global__ __launch_bounds__(256) void chunk_cumsum_bwd_kernel(const SsdParams p
     const int which = tid / CSB_HT, i = tid % CSB_HT, h = h0 + i;
     const float v = part[which][0][i] + part[which][1][i] + part[which][2][i] + part[which][3][i];
     if (h < H) {
-      if (which == 0) unsafeAtomicAdd(p.dA + h, v);
-      else if (p.ddt_bias) unsafeAtomicAdd(p.ddt_bias + h, v);
+      if (which == 0) acc_add(p.dA, p.det_dA, h, v, det_scale_of(p));
+      else if (p.ddt_bias) acc_add(p.ddt_bias, p.det_ddt_bias, h, v, det_scale_of(p));
     }
   }
 }
@@ -1249,8 +1277,45 @@ extern "C" int ssd_chunk_cumsum_bwd(const SsdParams *p, mamba_stream_t stream) {
   return launched();
 }
 
+extern "C" int ssd_det_convert(const int64_t *shadow, float *dst, int64_t n, const float *det_scale, mamba_stream_t stream) {
+  if (n == 0) return MAMBA_OK;
+  if (!shadow || !dst || !det_scale || n < 0 || (n + 255) / 256 > 0x7fffffff) return MAMBA_E_BADARG;
+  hipLaunchKernelGGL(det_convert_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     shadow, dst, n, det_scale);
+  return launched();
+}
+
 extern "C" int ssd_combined_bwd(const SsdParams *p, mamba_stream_t stream) {
   int rc;
+  if (p && p->det_scale) {
+    // deterministic mode: every shared sum goes through its integer shadow
+    if (!p->det_ddA_cumsum || !p->det_ddt_out || !p->det_dCB || !p->det_dB || !p->det_dC || !p->det_dA ||
+        (p->D && !p->det_dD) || (p->ddt_bias && !p->det_ddt_bias))
+      return MAMBA_E_BADARG;
+    const int64_t rows = (int64_t)p->batch * p->nheads * p->nchunks * p->chunk_size;
+    const int64_t bc = (int64_t)p->batch * p->seqlen * p->ngroups * p->dstate;
+    const int64_t cb = (int64_t)p->batch * p->nchunks * p->ngroups * p->chunk_size * p->chunk_size;
+    if ((rc = ssd_bwd_dz(p, stream))) return rc;
+    if ((rc = ssd_bwd_dstates(p, stream))) return rc;
+    if ((rc = ssd_state_passing_bwd(p, stream))) return rc;
+    if ((rc = ssd_bwd_dBC_state(p, stream))) return rc;
+    if ((rc = ssd_bwd_dx(p, stream))) return rc;
+    if ((rc = ssd_bwd_dcb(p, stream))) return rc;
+    // every term of these sums is in: shadows -> the float buffers their readers take
+    if ((rc = ssd_det_convert(p->det_dCB, p->dCB, cb, p->det_scale, stream))) return rc;
+    if ((rc = ssd_det_convert(p->det_dB, p->dB32, bc, p->det_scale, stream))) return rc;
+    if ((rc = ssd_det_convert(p->det_dC, p->dC32, bc, p->det_scale, stream))) return rc;
+    if ((rc = ssd_det_convert(p->det_ddA_cumsum, p->ddA_cumsum, rows, p->det_scale, stream))) return rc;
+    if ((rc = ssd_det_convert(p->det_ddt_out, p->ddt_out, rows, p->det_scale, stream))) return rc;
+    if (p->D && (rc = ssd_det_convert(p->det_dD, p->dD, p->D_has_hdim ? (int64_t)p->nheads * p->headdim : p->nheads,
+                                      p->det_scale, stream)))
+      return rc;
+    if ((rc = ssd_bmm_chunk_bwd(p, stream))) return rc;  // one workgroup per output tile: plain adds
+    if ((rc = ssd_chunk_cumsum_bwd(p, stream))) return rc;
+    if ((rc = ssd_det_convert(p->det_dA, p->dA, p->nheads, p->det_scale, stream))) return rc;
+    if (p->ddt_bias) return ssd_det_convert(p->det_ddt_bias, p->ddt_bias, p->nheads, p->det_scale, stream);
+    return MAMBA_OK;
+  }
   if ((rc = ssd_bwd_dz(p, stream))) return rc;
   if ((rc = ssd_bwd_dstates(p, stream))) return rc;
   if ((rc = ssd_state_passing_bwd(p, stream))) return rc;

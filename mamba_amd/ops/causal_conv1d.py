@@ -9,6 +9,7 @@ There is no CPU or PyTorch fallback: CPU tensors raise.
 import torch
 
 from mamba_amd import _lib
+from mamba_amd.utils.determinism import fixed_point_scale, use_deterministic_mode
 
 
 def _strides_bcl(t):
@@ -102,8 +103,21 @@ def causal_conv1d_bwd(x, weight, bias, dout, seq_idx=None, activation=None, dx=N
     p.dout, p.dx, p.dweight, p.dbias = dout.data_ptr(), dx.data_ptr(), dw32.data_ptr(), _lib.ptr(db32)
     p.dout_bs, p.dout_cs, p.dout_ls = _strides_bcl(dout)
     p.dx_bs, p.dx_cs, p.dx_ls = _strides_bcl(dx)
+    det = use_deterministic_mode()
+    if det:
+        # integer shadows of the two shared sums and the call's fixed-point scale (mamba_amd/utils/determinism.py)
+        sw = torch.zeros(w32.numel(), dtype=torch.int64, device=x.device)
+        sb = torch.zeros(b32.numel(), dtype=torch.int64, device=x.device) if b32 is not None else None
+        scale = fixed_point_scale(dout)
+        p.det_scale, p.det_dweight, p.det_dbias = scale.data_ptr(), sw.data_ptr(), _lib.ptr(sb)
     with torch.cuda.device(x.device):
-        _lib.check(_lib.load().causal_conv1d_bwd(p, _lib.current_stream(x.device)), "causal_conv1d_bwd")
+        lib, stream = _lib.load(), _lib.current_stream(x.device)
+        _lib.check(lib.causal_conv1d_bwd(p, stream), "causal_conv1d_bwd")
+        if det:
+            _lib.check(lib.ssd_det_convert(sw.data_ptr(), dw32.data_ptr(), sw.numel(), scale.data_ptr(), stream), "ssd_det_convert")
+            if sb is not None:
+                _lib.check(lib.ssd_det_convert(sb.data_ptr(), db32.data_ptr(), sb.numel(), scale.data_ptr(), stream),
+                           "ssd_det_convert")
     return dx, dw32.to(weight.dtype), (db32.to(bias.dtype) if bias is not None else None)
 
 

@@ -13,6 +13,7 @@ import torch
 from mamba_amd import _lib
 from mamba_amd.ops.causal_conv1d import causal_conv1d_fn
 from mamba_amd.ops.triton.layernorm_gated import rmsnorm_fn
+from mamba_amd.utils.determinism import fixed_point_scale, use_deterministic_mode
 
 
 def _fill_fwd(p, x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, seq_idx, dt_softplus, dt_limit, ws):
@@ -206,6 +207,16 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
     p.dinitial_states, p.dstates = _lib.ptr(dinit), dstates.data_ptr()
     p.ddA_cumsum, p.ddt_out, p.dCB = acc["ddA_cumsum"].data_ptr(), acc["ddt_out"].data_ptr(), acc["dCB"].data_ptr()
     p.dB32, p.dC32 = acc["dB32"].data_ptr(), acc["dC32"].data_ptr()
+    if use_deterministic_mode():
+        # integer shadows of the shared sums, laid out like the float arena, and the call's fixed-point scale
+        shadow = torch.zeros(sum(sizes.values()), device=dev, dtype=torch.int64)
+        det_scale = fixed_point_scale(dout, dfinal)
+        p.det_scale = det_scale.data_ptr()
+        off = 0
+        for k, n in sizes.items():
+            field = {"dB32": "det_dB", "dC32": "det_dC"}.get(k, "det_" + k)
+            setattr(p, field, shadow[off:off + n].data_ptr() if n else None)
+            off += n
     lib = _lib.load()
     with torch.cuda.device(dev):
         stream = _lib.current_stream(dev)

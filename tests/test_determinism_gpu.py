@@ -115,3 +115,91 @@ def test_scan_backward_repeats_to_rounding_noise():
         # Both are inside the reference's det-vs-default bound of 1e-2.
         noise = [(_noise(ga, gb), ga.dtype) for ga, gb in zip(a, b)]
         assert all(n < (1e-2 if dt != torch.float32 else 1e-3) for n, dt in noise), (fn.__name__, noise)
+
+
+@pytest.fixture
+def deterministic_mode():
+    from mamba_amd.utils.determinism import set_deterministic_mode
+    set_deterministic_mode(True)
+    yield
+    set_deterministic_mode(None)
+
+
+def _ssd_grads(t, names, chunk, **kw):
+    from mamba_amd.ops.triton.ssd_combined import mamba_chunk_scan_combined
+    leaves = {k: t[k].clone().requires_grad_() for k in names if t.get(k) is not None}
+    res = mamba_chunk_scan_combined(leaves["x"], leaves["dt"], leaves["A"], leaves["B"], leaves["C"], chunk,
+                                    D=leaves.get("D"), z=leaves.get("z"), dt_bias=leaves.get("dt_bias"),
+                                    initial_states=leaves.get("initial_states"), dt_softplus=True, **kw)
+    if isinstance(res, tuple):
+        (res[0].float() * t["dout"].float()).sum().add((res[1] * t["dfinal"]).sum()).backward()
+    else:
+        res.backward(t["dout"])
+    return {k: v.grad for k, v in leaves.items()}
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("headdim,dstate,ngroups,d_hdim", [(64, 128, 1, False), (128, 64, 2, True), (64, 64, 8, False)])
+def test_ssd_backward_deterministic_mode(deterministic_mode, headdim, dstate, ngroups, d_hdim, dtype):
+    """The reference's requirement for its deterministic mode (tests/test_determinism.py:186-211): five runs give
+    the same bits for every gradient, and the result is within 1e-2 of the default mode's."""
+    from mamba_amd.utils.determinism import set_deterministic_mode
+    names = ("x", "dt", "A", "B", "C", "D", "z", "dt_bias", "initial_states")
+    t = {k: (v.cuda() if torch.is_tensor(v) else v)
+         for k, v in ssd_inputs(2, 640, 16, headdim, dstate, ngroups, dtype, 7, D_has_hdim=d_hdim, has_init=True).items()}
+    runs = [_ssd_grads(t, names, 256, return_final_states=True) for _ in range(5)]
+    for r in runs[1:]:
+        for k in runs[0]:
+            assert torch.equal(runs[0][k], r[k]), k
+    set_deterministic_mode(False)
+    default = _ssd_grads(t, names, 256, return_final_states=True)
+    for k in default:
+        assert torch.allclose(default[k].float(), runs[0][k].float(), rtol=1e-2, atol=1e-2), k
+
+
+def test_ssd_backward_deterministic_mode_packed(deterministic_mode):
+    names = ("x", "dt", "A", "B", "C", "D", "z", "dt_bias", "initial_states")
+    t = {k: (v.cuda() if torch.is_tensor(v) else v)
+         for k, v in ssd_inputs(1, 1024, 8, 64, 128, 4, torch.bfloat16, 8, seq_lens=[300, 500, 224], has_init=True).items()}
+    runs = [_ssd_grads(t, names, 128, seq_idx=t["seq_idx"], return_final_states=True) for _ in range(3)]
+    for r in runs[1:]:
+        for k in runs[0]:
+            assert torch.equal(runs[0][k], r[k]), k
+
+
+def test_conv_and_block_backward_deterministic_mode(deterministic_mode):
+    from mamba_amd.ops.causal_conv1d import causal_conv1d_fn
+    from mamba_amd.ops.triton.ssd_combined import mamba_split_conv1d_scan_combined
+    g = torch.Generator().manual_seed(3)
+    r = lambda *s: torch.randn(*s, generator=g).cuda()
+    for channel_last in (False, True):
+        x = r(2, 2048, 512).bfloat16()
+        x = x.transpose(1, 2) if channel_last else x.transpose(1, 2).contiguous()
+        w, bias, dout = 0.5 * r(512, 4), r(512), r(2, 512, 2048).bfloat16()
+
+        def conv():
+            leaves = [x.clone().requires_grad_(), w.clone().requires_grad_(), bias.clone().requires_grad_()]
+            causal_conv1d_fn(*leaves, activation="silu").backward(dout if not channel_last else dout.transpose(1, 2).contiguous().transpose(1, 2))
+            return [t.grad for t in leaves]
+        a, b = _twice(conv)
+        for ga, gb in zip(a, b):
+            assert torch.equal(ga, gb)
+    # the whole Mamba-2 block body
+    batch, L, H, P, N, G, W, dm = 2, 512, 8, 64, 64, 1, 4, 256
+    d_inner, conv_dim = H * P, H * P + 2 * G * N
+    zxbcdt = r(batch, L, 2 * d_inner + 2 * G * N + H).bfloat16()
+    params = dict(conv_w=0.4 * r(conv_dim, W), conv_b=0.1 * r(conv_dim), dt_bias=r(H) - 3, A=-(1 + torch.rand(H, generator=g)).cuda(),
+                  D=torch.rand(H, generator=g).cuda(), norm_w=1 + 0.1 * r(d_inner), out_w=0.05 * r(dm, d_inner).bfloat16())
+    dout = r(batch, L, dm).bfloat16()
+
+    def block():
+        lv = {k: v.clone().requires_grad_() for k, v in params.items()}
+        zx = zxbcdt.clone().requires_grad_()
+        out = mamba_split_conv1d_scan_combined(zx, lv["conv_w"], lv["conv_b"], lv["dt_bias"], lv["A"], lv["D"], 128,
+                                               activation="silu", rmsnorm_weight=lv["norm_w"], rmsnorm_eps=1e-5,
+                                               outproj_weight=lv["out_w"], headdim=P, ngroups=G, norm_before_gate=False)
+        out.backward(dout)
+        return [zx.grad] + [v.grad for v in lv.values()]
+    a, b = _twice(block)
+    for ga, gb in zip(a, b):
+        assert torch.equal(ga, gb)
