@@ -62,7 +62,7 @@ def _chunk_scan_fwd(cb, x, dt, dA_cumsum, C, states, D=None, z=None, seq_idx=Non
 
 
 class ChunkScanFn(torch.autograd.Function):
-    """Forward of ssd_chunk_scan.py:1764 ChunkScanFn."""
+    """ssd_chunk_scan.py:1764 ChunkScanFn."""
 
     @staticmethod
     def forward(ctx, B, C, x, dt, dA_cumsum, prev_states, D=None, z=None):
@@ -71,12 +71,15 @@ class ChunkScanFn(torch.autograd.Function):
         assert B.shape == C.shape and B.shape[:2] == (batch, seqlen)
         assert seqlen == nchunks * chunk_size
         CB = _bmm_chunk_fwd(C, B, chunk_size, causal=True, output_dtype=torch.float32)
-        out, _ = _chunk_scan_fwd(CB, x, dt, dA_cumsum, C, prev_states, D=D, z=z)
+        out, out_x = _chunk_scan_fwd(CB, x, dt, dA_cumsum, C, prev_states, D=D, z=z)
+        ctx.save_for_backward(out if z is None else out_x, B, C, x, dt, dA_cumsum, prev_states, D, z)
         return out
 
     @staticmethod
     def backward(ctx, dout):
-        st.forward_only("chunk_scan")
+        from mamba_amd.ops.triton._ssd_stage_bwd import chunk_scan_bwd
+        y, B, C, x, dt, dA_cumsum, prev_states, D, z = ctx.saved_tensors
+        return chunk_scan_bwd(B, C, x, dt, dA_cumsum, prev_states, D, z, y, dout)
 
 
 def chunk_scan(B, C, x, dt, dA_cumsum, prev_states, D=None, z=None):

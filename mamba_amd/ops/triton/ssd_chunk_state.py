@@ -37,6 +37,39 @@ def _chunk_cumsum_fwd(dt, A, chunk_size, dt_bias=None, dt_softplus=False, dt_lim
     return dA_cumsum, dt_out
 
 
+def _chunk_cumsum_bwd(ddA, ddt_out, dt, A, dt_bias=None, dt_softplus=False, dt_limit=(0.0, float("inf")), ddt=None):
+    """Backward of _chunk_cumsum_fwd (ssd_chunk_state.py:744): ddA, ddt_out (batch, nheads, nchunks, chunk_size) are the
+    gradients with respect to dA_cumsum and the processed dt; dt (batch, seqlen, nheads) and A, dt_bias (nheads,) the
+    forward inputs.  Returns (ddt like dt, dA (nheads,) fp32, ddt_bias (nheads,) fp32 or None)."""
+    batch, seqlen, nheads = dt.shape
+    _, _, nchunks, chunk_size = ddA.shape
+    assert ddA.shape == (batch, nheads, nchunks, chunk_size) and ddt_out.shape == ddA.shape
+    assert A.shape == (nheads,)
+    _lib.require_gpu(ddA, ddt_out, dt, A, dt_bias, ddt)
+    if dt.dtype not in _lib.DTYPE_CODE:
+        dt = dt.float()
+    A32 = st.f32c(A)
+    bias32 = st.f32c(dt_bias) if dt_bias is not None else None
+    _, dt_proc = _chunk_cumsum_fwd(dt, A32, chunk_size, dt_bias=bias32, dt_softplus=dt_softplus, dt_limit=dt_limit)
+    ddA, ddt_out = st.f32c(ddA), st.f32c(ddt_out)
+    out = torch.empty(batch, seqlen, nheads, device=dt.device, dtype=dt.dtype)
+    sums = torch.zeros(2, nheads, device=dt.device, dtype=torch.float32)
+    p, _keep = st.stage_params(dt.device, batch=batch, seqlen=seqlen, nheads=nheads, headdim=1, dstate=1, ngroups=1,
+                               chunk_size=chunk_size, dt_dtype=dt.dtype, backward=True)
+    p.dt, p.A, p.dt_bias = dt.data_ptr(), A32.data_ptr(), _lib.ptr(bias32)
+    p.dt_bs, p.dt_ls, p.dt_hs = dt.stride()
+    p.dt_softplus = int(bool(dt_softplus))
+    p.dt_min, p.dt_max = float(dt_limit[0]), float(min(dt_limit[1], 3.0e38))
+    p.dt_out, p.ddA_cumsum, p.ddt_out = dt_proc.data_ptr(), ddA.data_ptr(), ddt_out.data_ptr()
+    p.ddt, p.dA = out.data_ptr(), sums[0].data_ptr()
+    p.ddt_bias = sums[1].data_ptr() if dt_bias is not None else None
+    st.run("ssd_chunk_cumsum_bwd", p, dt.device)
+    if ddt is not None:
+        ddt.copy_(out)
+        out = ddt
+    return out, sums[0], (sums[1] if dt_bias is not None else None)
+
+
 def _chunk_state_fwd(B, x, dt, dA_cumsum, seq_idx=None, states=None, states_in_fp32=True):
     """Chunk-local states sum_l B[l] x[l] dt[l] exp(a_end - a_l): (batch, nchunks, nheads, headdim, dstate)
     (ssd_chunk_state.py:812-842).  The kernel writes fp32; another `states` dtype is a cast of that."""
@@ -112,15 +145,19 @@ def chunk_state_varlen(B, x, dt, dA_cumsum, cu_seqlens, chunk_states):
 
 
 class ChunkStateFn(torch.autograd.Function):
-    """Forward of ssd_chunk_state.py:1047 ChunkStateFn."""
+    """ssd_chunk_state.py:1047 ChunkStateFn."""
 
     @staticmethod
     def forward(ctx, B, x, dt, dA_cumsum, states_in_fp32=True):
+        ctx.save_for_backward(B, x, dt, dA_cumsum)
         return _chunk_state_fwd(B, x, dt, dA_cumsum, states_in_fp32=states_in_fp32)
 
     @staticmethod
     def backward(ctx, dstates):
-        st.forward_only("chunk_state")
+        from mamba_amd.ops.triton._ssd_stage_bwd import chunk_state_bwd
+        B, x, dt, dA_cumsum = ctx.saved_tensors
+        dB, dx, ddt, ddA_cumsum = chunk_state_bwd(B, x, dt, dA_cumsum, dstates)
+        return dB, dx, ddt, ddA_cumsum, None
 
 
 def chunk_state(B, x, dt, dA_cumsum, states_in_fp32=True):

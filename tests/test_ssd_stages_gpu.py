@@ -247,9 +247,59 @@ def test_chunk_scan_function_and_ref():
     ref = chunk_scan_ref(t["B"].double(), t["C"].double(), t["x"].double(), dt_out.cpu().double(), dA.cpu().double(),
                          prev.cpu().double(), D=t["D"].double(), z=t["z"].double())
     _close("chunk_scan", out, ref, *_tol(torch.float32))
-    leaf = cu(t["x"]).requires_grad_()
-    with pytest.raises(NotImplementedError):
-        chunk_scan(cu(t["B"]), cu(t["C"]), leaf, dt_out, dA, prev).sum().backward()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("seqlen,chunk,headdim,dstate,ngroups", [(256, 64, 32, 64, 2), (512, 256, 64, 128, 1), (384, 128, 64, 16, 4)])
+def test_chunk_state_backward(seqlen, chunk, headdim, dstate, ngroups, dtype):
+    """chunk_state is differentiable (reference ChunkStateFn.backward, ssd_chunk_state.py:1060-1078): dB, dx, ddt,
+    ddA_cumsum against autograd through the plain-torch form of the stage in float64."""
+    from mamba_amd.ops.triton.ssd_chunk_state import _chunk_cumsum_fwd, chunk_state, chunk_state_ref
+    t = ssd_inputs(2, seqlen, 4, headdim, dstate, ngroups, dtype, seed=21)
+    cu = lambda v: v.cuda()
+    dA, dt_out = _chunk_cumsum_fwd(cu(t["dt"]), cu(t["A"]), chunk, dt_bias=cu(t["dt_bias"]), dt_softplus=True)
+    g = torch.Generator().manual_seed(2)
+    dstates = torch.randn(2, seqlen // chunk, 4, headdim, dstate, generator=g)
+    leaves = [cu(t["B"]).requires_grad_(), cu(t["x"]).requires_grad_(), dt_out.clone().requires_grad_(), dA.clone().requires_grad_()]
+    (chunk_state(*leaves) * dstates.cuda()).sum().backward()
+    ref_leaves = [t["B"].double().requires_grad_(), t["x"].double().requires_grad_(), dt_out.cpu().double().requires_grad_(),
+                  dA.cpu().double().requires_grad_()]
+    (chunk_state_ref(*ref_leaves) * dstates.double()).sum().backward()
+    rtol, atol = _tol(dtype)
+    for name, a, b in zip(("dB", "dx", "ddt", "ddA_cumsum"), leaves, ref_leaves):
+        scale = max(1.0, float(b.grad.abs().max())) if name in ("ddt", "ddA_cumsum") else 1.0
+        _close(name, a.grad, b.grad, 2 * rtol, 2 * atol * scale)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("seqlen,chunk,headdim,dstate,ngroups,has_z,d_hdim", [
+    (256, 64, 32, 64, 2, True, False), (512, 256, 64, 128, 1, True, False), (384, 128, 64, 16, 4, False, True)])
+def test_chunk_scan_backward(seqlen, chunk, headdim, dstate, ngroups, has_z, d_hdim, dtype):
+    """chunk_scan is differentiable (reference ChunkScanFn.backward, ssd_chunk_scan.py:1786-1825): dB, dC, dx, ddt,
+    ddA_cumsum, dprev_states, dD, dz against autograd through the plain-torch form in float64."""
+    from mamba_amd.ops.triton.ssd_chunk_scan import chunk_scan, chunk_scan_ref
+    from mamba_amd.ops.triton.ssd_chunk_state import _chunk_cumsum_fwd
+    H = 4
+    t = ssd_inputs(2, seqlen, H, headdim, dstate, ngroups, dtype, seed=22, D_has_hdim=d_hdim)
+    cu = lambda v: v.cuda()
+    dA, dt_out = _chunk_cumsum_fwd(cu(t["dt"]), cu(t["A"]), chunk, dt_bias=cu(t["dt_bias"]), dt_softplus=True)
+    prev = 0.1 * torch.randn(2, seqlen // chunk, H, headdim, dstate, generator=torch.Generator().manual_seed(3))
+    names = ["B", "C", "x", "dt", "dA_cumsum", "prev_states", "D"] + (["z"] if has_z else [])
+    gpu = dict(B=cu(t["B"]), C=cu(t["C"]), x=cu(t["x"]), dt=dt_out.clone(), dA_cumsum=dA.clone(), prev_states=prev.cuda(),
+               D=cu(t["D"]), z=cu(t["z"]) if has_z else None)
+    ref = dict(B=t["B"].double(), C=t["C"].double(), x=t["x"].double(), dt=dt_out.cpu().double(), dA_cumsum=dA.cpu().double(),
+               prev_states=prev.double(), D=t["D"].double(), z=t["z"].double() if has_z else None)
+    for d in (gpu, ref):
+        for k in names:
+            d[k].requires_grad_()
+    call = lambda fn, d: fn(d["B"], d["C"], d["x"], d["dt"], d["dA_cumsum"], d["prev_states"], D=d["D"], z=d["z"])
+    out = call(chunk_scan, gpu)
+    out.backward(cu(t["dout"]))
+    call(chunk_scan_ref, ref).backward(t["dout"].double())
+    rtol, atol = _tol(dtype)
+    for k in names:
+        scale = max(1.0, float(ref[k].grad.abs().max())) if k in ("dt", "dA_cumsum", "D") else 1.0
+        _close("d" + k, gpu[k].grad, ref[k].grad, 2 * rtol, 2 * atol * scale)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -299,3 +349,28 @@ def test_stage_functions_reject_cpu_tensors():
     from mamba_amd.ops.triton.ssd_chunk_state import _chunk_cumsum_fwd
     with pytest.raises(RuntimeError):
         _chunk_cumsum_fwd(torch.randn(1, 64, 2), -torch.rand(2), 64)
+
+
+@pytest.mark.parametrize("softplus,limit", [(True, (0.0, float("inf"))), (False, (0.0, float("inf"))), (True, (0.01, 0.5))])
+def test_chunk_cumsum_backward(softplus, limit):
+    """_chunk_cumsum_bwd (reference ssd_chunk_state.py:744) against autograd through the dt pipeline and the
+    per-chunk running sum written out in float64."""
+    import torch.nn.functional as F
+    from mamba_amd.ops.triton.ssd_chunk_state import _chunk_cumsum_bwd
+    batch, L, H, Q = 2, 320, 6, 128
+    g = torch.Generator().manual_seed(5)
+    dt = torch.randn(batch, L, H, generator=g)
+    A, bias = -(1 + torch.rand(H, generator=g)), torch.randn(H, generator=g) - 2
+    nc = (L + Q - 1) // Q
+    ddA, ddt_out = torch.randn(batch, H, nc, Q, generator=g), torch.randn(batch, H, nc, Q, generator=g)
+    got = _chunk_cumsum_bwd(ddA.cuda(), ddt_out.cuda(), dt.cuda(), A.cuda(), dt_bias=bias.cuda(), dt_softplus=softplus,
+                            dt_limit=limit)
+    dtr, Ar, br = dt.double().requires_grad_(), A.double().requires_grad_(), bias.double().requires_grad_()
+    v = dtr + br
+    v = F.softplus(v) if softplus else v
+    v = v.clamp(limit[0], limit[1])
+    v = F.pad(v, (0, 0, 0, nc * Q - L)).reshape(batch, nc, Q, H).permute(0, 3, 1, 2)        # (b, h, c, Q)
+    dA_cs = torch.cumsum(v * Ar[None, :, None, None], dim=-1)
+    ((dA_cs * ddA.double()).sum() + (v * ddt_out.double()).sum()).backward()
+    for name, a, b in zip(("ddt", "dA", "ddt_bias"), got, (dtr.grad, Ar.grad, br.grad)):
+        _close(name, a, b, 6e-4, 2e-3 * max(1.0, float(b.abs().max())))
