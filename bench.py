@@ -637,14 +637,16 @@ def bench_mamba1(dev, steps, warmup):
                 "fwd_traffic": profile_traffic(prof + "_hbm_counters.txt", "scan_fwd_kernel"),
                 "fwd_bwd_frac": (fwd_bytes + bwd_bytes) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS}
     vs_measured_copy(roofline, dev)
-    # The binding resource of both scan kernels is fp32 vector-ALU issue, not HBM: instruction slots per
-    # (position, channel, state) from the hardware counters of the committed profile (a transcendental
-    # takes two slots), times the elements of this launch, over the event time, beside the rate a bare
-    # v_fma_f32 loop reaches in this run.
+    # The binding resource of both scan kernels is fp32 vector-ALU issue, not HBM.  A SIMD issues one plain
+    # wave64 fp32 instruction every 2 cycles when at least two of its waves are ready (one wave alone: every 4),
+    # which is the published 157.3 TFLOP/s = 78.6 T lane-FMA/s; a transcendental (v_exp_f32) holds the port four
+    # times as long (measured: 19 T/s).  Slots per (position, channel, state) = the VALU instruction count of the
+    # committed counter profile with every transcendental counted four times, over the event time of this run,
+    # beside the rate a bare v_fma_f32 loop reaches in this run.
     elems = batch * dim * seqlen * dstate
     probe = measured_valu(dev)
     valu = {"unit": "T lane-instruction slots/s", "measured_fma_probe": probe,
-            "nominal_peak": 256 * 4 * 16 * 2.4e9 / 1e12, "element_states": elems}
+            "nominal_peak": 256 * 4 * 32 * 2.4e9 / 1e12, "element_states": elems}
     for name, ms in (("bwd", bwd_ms), ("fwd", fwd_ms)):
         kern = "scan_%s_kernel" % name
         insts = profile_counter(prof + "_valu_counters.txt", kern, "SQ_INSTS_VALU")
@@ -652,8 +654,10 @@ def bench_mamba1(dev, steps, warmup):
         if insts is None or trans is None:
             valu[name] = None
             continue
-        slots = (insts + trans) * 64 / elems
-        valu[name] = {"slots_per_element_state": slots, "achieved": slots * elems / (ms * 1e-3) / 1e12,
+        slots = (insts + 3 * trans) * 64 / elems
+        valu[name] = {"valu_instructions_per_element_state": insts * 64 / elems,
+                      "transcendentals_per_element_state": trans * 64 / elems,
+                      "slots_per_element_state": slots, "achieved": slots * elems / (ms * 1e-3) / 1e12,
                       "frac_of_probe": slots * elems / (ms * 1e-3) / 1e12 / probe}
     roofline["valu"] = valu
     return {
