@@ -42,8 +42,10 @@ DEVI int64_t chunk_off(const SsdParams &p, int b, int h, int c) {
 // shadow of the buffer; integer addition is associative, so the sum is the same in every order, and
 // det_convert_kernel turns the shadow into the float buffer before its first reader runs.
 DEVI float det_scale_of(const SsdParams &p) { return p.det_scale ? p.det_scale[0] : 0.f; }
-DEVI void acc_add(float *dst, int64_t *shadow, int64_t idx, float v, float dsc) {
-  if (dsc != 0.f) {
+// MODE: -1 decides at run time from dsc (the small kernels), 0 / 1 are compiled for one form (the kernels whose inner
+// loops hold these adds: carrying both forms costs them registers and ~10 % of their time).
+template <int MODE = -1> DEVI void acc_add(float *dst, int64_t *shadow, int64_t idx, float v, float dsc) {
+  if (MODE == 1 || (MODE < 0 && dsc != 0.f)) {
     const float q = fminf(fmaxf(v * dsc, -9.0e18f), 9.0e18f);
     __hip_atomic_fetch_add(reinterpret_cast<unsigned long long *>(shadow + idx),
                            static_cast<unsigned long long>(static_cast<long long>(__builtin_rintf(q))), __ATOMIC_RELAXED,
@@ -386,7 +388,7 @@ template <int W> __global__ __launch_bounds__(256) void state_passing_bwd_kernel
 // acc[s, p] = exp(a_last - a_s) [s in the chunk's last sequence] sum_n B[s, n] dS[p, n]
 //           + sum_{l >= s} CB[l, s] exp(a_l - a_s) g[l, p]
 // dx = dt_s acc + D g;  ddt_out[s] += <x_s, acc_s>;  chunk-state terms of ddA_cumsum.
-template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_kernel(const SsdParams p) {
+template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256) void bwd_dx_kernel(const SsdParams p) {
   __shared__ GemmLds lds;
   __shared__ float a_s[256], dt_s[256], kdec[256], rdec[GB], wrow[GB];
   const int tid = threadIdx.x;
@@ -533,12 +535,12 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
   const int64_t row_off = chunk_off(p, b, h, c);
   const float dsc = det_scale_of(p);
   if (lead) {
-    acc_add(p.ddt_out, p.det_ddt_out, row_off + s, q2, dsc);
-    acc_add(p.ddA_cumsum, p.det_ddA_cumsum, row_off + s, -dts * q1, dsc);  // chunk-state terms: -dt_s <x_s, acc1_s> at s ...
+    acc_add<DET ? 1 : 0>(p.ddt_out, p.det_ddt_out, row_off + s, q2, dsc);
+    acc_add<DET ? 1 : 0>(p.ddA_cumsum, p.det_ddA_cumsum, row_off + s, -dts * q1, dsc);  // chunk-state terms: -dt_s <x_s, acc1_s> at s ...
   }
   // ... and + at the chunk end: one address for the whole tile, so one atomic per wave
   const float endsum = wave_sum_to_last(lead ? dts * q1 : 0.f);
-  if ((tid & 63) == 63) acc_add(p.ddA_cumsum, p.det_ddA_cumsum, row_off + Q - 1, endsum, dsc);
+  if ((tid & 63) == 63) acc_add<DET ? 1 : 0>(p.ddA_cumsum, p.det_ddA_cumsum, row_off + Q - 1, endsum, dsc);
 }
 
 // ---------------------------------------------- state-path parts of dB, dC
@@ -548,7 +550,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dx_
 // both sums in registers (no atomics); the per-head row factor is folded into the A operand.
 // The carried-state share of ddA_cumsum, sum_n dC_h[l, n] C[l, n], is taken per head on the way.
 // PARTS: bit 0 = the dB product, bit 1 = the dC product.
-template <typename T, bool SPLIT, int PARTS> DEVI void dBC_state_body(const SsdParams &p) {
+template <typename T, bool SPLIT, bool DET, int PARTS> DEVI void dBC_state_body(const SsdParams &p) {
   constexpr int MAXH = 8;  // heads per workgroup (head_splits keeps it at or below 8)
   __shared__ GemmLds lds;
   __shared__ float wB[MAXH][GB], wC[MAXH][GB];  // per-head row factors
@@ -615,7 +617,7 @@ template <typename T, bool SPLIT, int PARTS> DEVI void dBC_state_body(const SsdP
         tid);
     acc_foreach(accB, tid, [&](int m, int n, float v) {
       const int s = st * GB + m, nn = nt * GB + n;
-      if (s < qlim && nn < N) acc_add(p.dB32, p.det_dB, (((int64_t)b * L + t0 + s) * G + g) * N + nn, v, det_scale_of(p));
+      if (s < qlim && nn < N) acc_add<DET ? 1 : 0>(p.dB32, p.det_dB, (((int64_t)b * L + t0 + s) * G + g) * N + nn, v, det_scale_of(p));
       return v;
     });
   }
@@ -675,7 +677,7 @@ template <typename T, bool SPLIT, int PARTS> DEVI void dBC_state_body(const SsdP
         });
     acc_foreach(accC, tid, [&](int m, int n, float v) {
       const int l = st * GB + m, nn = nt * GB + n;
-      if (l < qlim && nn < N) acc_add(p.dC32, p.det_dC, (((int64_t)b * L + t0 + l) * G + g) * N + nn, v, det_scale_of(p));
+      if (l < qlim && nn < N) acc_add<DET ? 1 : 0>(p.dC32, p.det_dC, (((int64_t)b * L + t0 + l) * G + g) * N + nn, v, det_scale_of(p));
       return v;
     });
     __syncthreads();
@@ -683,21 +685,21 @@ template <typename T, bool SPLIT, int PARTS> DEVI void dBC_state_body(const SsdP
       const int hl = idx / GB, r = idx % GB, l = st * GB + r;
       const float d = dda_s[0][hl][r] + dda_s[1][hl][r];
       if (l < qlim && d != 0.f)
-        acc_add(p.ddA_cumsum, p.det_ddA_cumsum, chunk_off(p, b, g * hpg + hs + hl * nsplit, c) + l, d, det_scale_of(p));
+        acc_add<DET ? 1 : 0>(p.ddA_cumsum, p.det_ddA_cumsum, chunk_off(p, b, g * hpg + hs + hl * nsplit, c) + l, d, det_scale_of(p));
     }
   }
 }
 
-template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_dBC_state_kernel(const SsdParams p) {
-  dBC_state_body<T, SPLIT, 3>(p);
+template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256, 4) void bwd_dBC_state_kernel(const SsdParams p) {
+  dBC_state_body<T, SPLIT, DET, 3>(p);
 }
-template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_dC_state_kernel(const SsdParams p) {
-  dBC_state_body<T, SPLIT, 2>(p);
+template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256, 4) void bwd_dC_state_kernel(const SsdParams p) {
+  dBC_state_body<T, SPLIT, DET, 2>(p);
 }
 
 // The dB product alone with a 64 x 128 tile per workgroup (whole 128-state blocks, headdim in whole
 // k steps, aligned x): k runs through (head, p) as above.
-template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dB_state_wide_kernel(const SsdParams p) {
+template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256) void bwd_dB_state_wide_kernel(const SsdParams p) {
   constexpr int MAXH = 8;
   __shared__ GemmLdsWide<SPLIT> lds;
   __shared__ float wB[MAXH][GB];
@@ -751,13 +753,13 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dB_
       if (s >= qlim) continue;
       const int64_t row = (((int64_t)b * L + t0 + s) * G + g) * N + nt * WB + wn * 64 + i;
 #pragma unroll
-      for (int tn = 0; tn < 4; ++tn) acc_add(p.dB32, p.det_dB, row + tn * 16, accB.v[tm][tn][r], det_scale_of(p));
+      for (int tn = 0; tn < 4; ++tn) acc_add<DET ? 1 : 0>(p.dB32, p.det_dB, row + tn * 16, accB.v[tm][tn][r], det_scale_of(p));
     }
 }
 
 // The dC product alone with a 64 x 128 tile per workgroup (same conditions, aligned g rows); the row sums
 // of the tile against C after each head give the heads' ddA_cumsum rows.
-template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_dC_state_wide_kernel(const SsdParams p) {
+template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256, 4) void bwd_dC_state_wide_kernel(const SsdParams p) {
   constexpr int MAXH = 8;
   __shared__ GemmLdsWide<SPLIT> lds;
   __shared__ float wC[MAXH][GB];
@@ -855,7 +857,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_
     const int hl = idx / GB, r = idx % GB, l = st * GB + r;
     const float d = dda_s[0][hl][r] + dda_s[1][hl][r] - (hl > 0 ? dda_s[0][hl - 1][r] + dda_s[1][hl - 1][r] : 0.f);
     if (l < qlim && d != 0.f)
-      acc_add(p.ddA_cumsum, p.det_ddA_cumsum, chunk_off(p, b, g * hpg + hs + hl * nsplit, c) + l, d, det_scale_of(p));
+      acc_add<DET ? 1 : 0>(p.ddA_cumsum, p.det_ddA_cumsum, chunk_off(p, b, g * hpg + hs + hl * nsplit, c) + l, d, det_scale_of(p));
   }
 #pragma unroll
   for (int tm = 0; tm < 2; ++tm)
@@ -865,7 +867,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_
       if (l >= qlim) continue;
       const int64_t row = (((int64_t)b * L + t0 + l) * G + g) * N + nt * WB + wn * 64 + i;
 #pragma unroll
-      for (int tn = 0; tn < 4; ++tn) acc_add(p.dC32, p.det_dC, row + tn * 16, acc.v[tm][tn][r], det_scale_of(p));
+      for (int tn = 0; tn < 4; ++tn) acc_add<DET ? 1 : 0>(p.dC32, p.det_dC, row + tn * 16, acc.v[tm][tn][r], det_scale_of(p));
     }
 }
 
@@ -874,7 +876,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_
 // one sequence.  One workgroup per (batch, chunk, group, lower-triangular 64 x 64 tile pair) loops
 // over the heads of the group with the sum in registers.  Per head, w = (head's term) * CB gives
 // the in-chunk share of ddA_cumsum: + row sums at l, - column sums at s.
-template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_dcb_kernel(const SsdParams p) {
+template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256, 4) void bwd_dcb_kernel(const SsdParams p) {
   __shared__ GemmLds lds;
   __shared__ float hA_l[2][GB], hA_s[2][GB], hdt[2][GB];  // per-head rows, double-buffered over the head loop
   // the heads' ddA_cumsum shares (row sums per column half, column sums per row half), flushed at the end: a
@@ -994,12 +996,12 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256, 4) void bwd_
     const int hl = idx / GB, r = idx % GB;
     const int64_t dda = chunk_off(p, b, g * hpg + hs + hl * nsplit, c);
     const float row = rs_s[0][hl][r] + rs_s[1][hl][r], col = cs_s[0][hl][r] + cs_s[1][hl][r];
-    if (lt * GB + r < Q && row != 0.f) acc_add(p.ddA_cumsum, p.det_ddA_cumsum, dda + lt * GB + r, row, det_scale_of(p));
-    if (st * GB + r < Q && col != 0.f) acc_add(p.ddA_cumsum, p.det_ddA_cumsum, dda + st * GB + r, -col, det_scale_of(p));
+    if (lt * GB + r < Q && row != 0.f) acc_add<DET ? 1 : 0>(p.ddA_cumsum, p.det_ddA_cumsum, dda + lt * GB + r, row, det_scale_of(p));
+    if (st * GB + r < Q && col != 0.f) acc_add<DET ? 1 : 0>(p.ddA_cumsum, p.det_ddA_cumsum, dda + st * GB + r, -col, det_scale_of(p));
   }
   acc_foreach(sum, tid, [&](int m, int n, float v) {
     const int l = lt * GB + m, s = st * GB + n;
-    if (l < Q && s < Q && v != 0.f) acc_add(p.dCB, p.det_dCB, dCB_off + (int64_t)l * Q + s, v, det_scale_of(p));  // dCB starts zeroed
+    if (l < Q && s < Q && v != 0.f) acc_add<DET ? 1 : 0>(p.dCB, p.det_dCB, dCB_off + (int64_t)l * Q + s, v, det_scale_of(p));  // dCB starts zeroed
     return v;
   });
 }
@@ -1161,6 +1163,22 @@ int launched() { return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAU
     default: hipLaunchKernelGGL((KERNEL<float, true>), GRID, dim3(256), 0, s, *p); break;            \
   }
 
+// the same for kernels compiled per summation mode (float atomics / fixed-point integer atomics)
+#define SSD_DISPATCH_DET(KERNEL, GRID)                                                                          \
+  if (p->det_scale) {                                                                                           \
+    switch (p->dtype) {                                                                                         \
+      case MAMBA_BF16: hipLaunchKernelGGL((KERNEL<bf16_t, false, true>), GRID, dim3(256), 0, s, *p); break;     \
+      case MAMBA_F16: hipLaunchKernelGGL((KERNEL<f16_t, true, true>), GRID, dim3(256), 0, s, *p); break;        \
+      default: hipLaunchKernelGGL((KERNEL<float, true, true>), GRID, dim3(256), 0, s, *p); break;               \
+    }                                                                                                           \
+  } else {                                                                                                      \
+    switch (p->dtype) {                                                                                         \
+      case MAMBA_BF16: hipLaunchKernelGGL((KERNEL<bf16_t, false, false>), GRID, dim3(256), 0, s, *p); break;    \
+      case MAMBA_F16: hipLaunchKernelGGL((KERNEL<f16_t, true, false>), GRID, dim3(256), 0, s, *p); break;       \
+      default: hipLaunchKernelGGL((KERNEL<float, true, false>), GRID, dim3(256), 0, s, *p); break;              \
+    }                                                                                                           \
+  }
+
 inline int tiles(int n) { return (n + GB - 1) / GB; }
 
 }  // namespace
@@ -1220,7 +1238,7 @@ extern "C" int ssd_bwd_dx(const SsdParams *p, mamba_stream_t stream) {
   if (p->dx_ls < (int64_t)p->headdim || p->dx_hs < (int64_t)p->headdim) return MAMBA_E_BADARG;  // strides not filled in
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid(tiles(p->chunk_size) * tiles(p->headdim), p->nchunks, p->batch * p->nheads);
-  SSD_DISPATCH(bwd_dx_kernel, grid)
+  SSD_DISPATCH_DET(bwd_dx_kernel, grid)
   return launched();
 }
 
@@ -1238,14 +1256,14 @@ extern "C" int ssd_bwd_dBC_state(const SsdParams *p, mamba_stream_t stream) {
     const bool g_ok = p->z ? (p->headdim % 8 == 0 && reinterpret_cast<uintptr_t>(p->gbuf) % 16 == 0)
                            : wide_operand_ok(p->dout, p->dtype, p->dout_bs, p->dout_ls, p->dout_hs);
     if (g_ok) {
-      SSD_DISPATCH(bwd_dC_state_wide_kernel, gridw)
+      SSD_DISPATCH_DET(bwd_dC_state_wide_kernel, gridw)
     } else {
-      SSD_DISPATCH(bwd_dC_state_kernel, grid)
+      SSD_DISPATCH_DET(bwd_dC_state_kernel, grid)
     }
-    SSD_DISPATCH(bwd_dB_state_wide_kernel, gridw)
+    SSD_DISPATCH_DET(bwd_dB_state_wide_kernel, gridw)
     return launched();
   }
-  SSD_DISPATCH(bwd_dBC_state_kernel, grid)
+  SSD_DISPATCH_DET(bwd_dBC_state_kernel, grid)
   return launched();
 }
 
@@ -1255,7 +1273,7 @@ extern "C" int ssd_bwd_dcb(const SsdParams *p, mamba_stream_t stream) {
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int nt = tiles(p->chunk_size);
   dim3 grid(nt * (nt + 1) / 2, p->nchunks, p->batch * p->ngroups * head_splits(p->nheads / p->ngroups));
-  SSD_DISPATCH(bwd_dcb_kernel, grid)
+  SSD_DISPATCH_DET(bwd_dcb_kernel, grid)
   return launched();
 }
 
