@@ -88,9 +88,16 @@ template <> DEVI void st8<f16_t>(f16_t *p, const float (&v)[8]) {
 
 // 8 values kept in registers in the storage format of T (exact round trip for values that were
 // loaded from T): 4 registers for 16-bit types, 8 for fp32.
+// Accesses that name the global address space.  A pointer that a kernel reads back from LDS or from
+// memory has lost its address space, and plain accesses through it become flat instructions, which
+// count in the LDS counter as well as in the memory counter: every wait for an LDS read then also waits
+// for the flat accesses in flight.
+#define GLOBAL_AS __attribute__((address_space(1)))
+
 template <typename T> struct Pack8 {
   u32x4 w;
   DEVI void load(const T *p) { w = *reinterpret_cast<const u32x4 *>(p); }  // 16-byte aligned
+  DEVI void load_global(const T *p) { w = *(const GLOBAL_AS u32x4 *)p; }
   DEVI void zero() { w = u32x4{0, 0, 0, 0}; }
   DEVI void pack(const float (&v)[8]) {
     if constexpr (DT<T>::id == MAMBA_BF16) {
@@ -113,6 +120,11 @@ template <> struct Pack8<float> {
   float v[8];
   DEVI void load(const float *p) {
     const f32x4 a = *reinterpret_cast<const f32x4 *>(p), b = *reinterpret_cast<const f32x4 *>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  }
+  DEVI void load_global(const float *p) {
+    const f32x4 a = *(const GLOBAL_AS f32x4 *)p, b = *(const GLOBAL_AS f32x4 *)(p + 4);
     v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
     v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
   }
@@ -152,6 +164,24 @@ template <typename T, bool VEC> DEVI void st8_guard(T *p, int nvalid, const floa
 #pragma unroll
     for (int i = 0; i < 8; ++i)
       if (i < nvalid) st1<T>(p + i, v[i]);
+  }
+}
+
+// The same through the global address space: 8 values stored as T with 16-byte accesses (all or nothing), or
+// element by element through the generic path.
+template <typename T, bool VEC> DEVI void st8_guard_global(T *p, int nvalid, const float (&v)[8]) {
+  if constexpr (VEC) {
+    if (nvalid < 8) return;
+    if constexpr (DT<T>::id == MAMBA_F32) {
+      *(GLOBAL_AS f32x4 *)p = f32x4{v[0], v[1], v[2], v[3]};
+      *(GLOBAL_AS f32x4 *)(p + 4) = f32x4{v[4], v[5], v[6], v[7]};
+    } else {
+      Pack8<T> k;
+      k.pack(v);
+      *(GLOBAL_AS u32x4 *)p = k.w;
+    }
+  } else {
+    st8_guard<T, false>(p, nvalid, v);
   }
 }
 

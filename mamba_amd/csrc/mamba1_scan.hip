@@ -74,7 +74,7 @@ DEVI void stage_bc(float *Bs, float *Cs, const T *Bg, int64_t B_ns, const T *Cg,
 // clamped position (the caller masks lanes past the end), else element by element.
 template <typename T, bool VEC> DEVI void load_items(Pack8<T> &k, const T *row, int tl, int L, int nvalid) {
   if constexpr (VEC) {
-    k.load(row + min(tl, L - KI));
+    k.load_global(row + min(tl, L - KI));
   } else {
     float v[8];
     ld8_guard<T, false>(row + tl, nvalid, 0.f, v);
@@ -254,7 +254,8 @@ __global__ __launch_bounds__(NTHREADS, 4) void scan_fwd_kernel(const MambaScanPa
 // ----------------------------------------------------------------- backward
 // Row starts of one channel of the workgroup, kept in LDS: every (tile, pass) step needs nine
 // addresses per lane, and as kernel arguments next to the loop state they did not fit the scalar
-// registers (each step then re-read hundreds of spilled scalars through v_readlane).
+// registers (each step then re-read hundreds of spilled scalars through v_readlane).  Pointers read back
+// from LDS carry no address space, so the rows are accessed through the helpers that name the global one.
 template <typename T> struct BwdRow {
   const T *u, *delta, *dout, *z;
   T *du, *ddelta, *dz, *out_z;
@@ -348,7 +349,7 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
     const int nvalid = min(max(L - tl, 0), KI);
     k.z.zero();
     k.ck = 0.f;
-    if (NBLK == 1 && tile > 0) k.ck = w.ckpt[(int64_t)(tile - 1) * N + min(c, N - 1)];
+    if (NBLK == 1 && tile > 0) k.ck = *(const GLOBAL_AS float *)(w.ckpt + (int64_t)(tile - 1) * N + min(c, N - 1));
     load_items<T, VEC>(k.u, w.u, tl, L, nvalid);
     load_items<T, VEC>(k.delta, w.delta, tl, L, nvalid);
     load_items<T, VEC>(k.dout, w.dout, tl, L, nvalid);
@@ -408,7 +409,7 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
         } else {
           for (int n = c; n < NP; n += RL) {
             float v = 0.f;
-            if (tile > 0 && n < N) v = rows[chw].ckpt[(int64_t)(tile - 1) * N + n];
+            if (tile > 0 && n < N) v = *(const GLOBAL_AS float *)(rows[chw].ckpt + (int64_t)(tile - 1) * N + n);
             hcar[chl * NP + n] = v;
           }
         }
@@ -599,7 +600,7 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
         float dbs = 0.f, dDs = 0.f;
 #pragma unroll
         for (int i = 0; i < KI; ++i) o[i] = __builtin_fmaf(dl[i], acc[i], Dd * dy[i]);
-        st8_guard<T, VEC>(w.du + tl, nvalid, o);
+        st8_guard_global<T, VEC>(w.du + tl, nvalid, o);
 #pragma unroll
         for (int i = 0; i < KI; ++i) {
           float gd = __builtin_fmaf(u[i], acc[i], dd[i]);
@@ -609,7 +610,7 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
           dbs += gd;
           dDs = __builtin_fmaf(dy[i], u[i], dDs);
         }
-        st8_guard<T, VEC>(w.ddelta + tl, nvalid, o);
+        st8_guard_global<T, VEC>(w.ddelta + tl, nvalid, o);
         if (has_z) {
           float z[8], dout[8], oz[8];
           z_k.unpack(z);
@@ -621,8 +622,8 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
             o[i] = dout[i] * yf * s * (1.f + z[i] * (1.f - s));
             oz[i] = yf * z[i] * s;
           }
-          st8_guard<T, VEC>(w.dz + tl, nvalid, o);
-          if (w.out_z) st8_guard<T, VEC>(w.out_z + tl, nvalid, oz);
+          st8_guard_global<T, VEC>(w.dz + tl, nvalid, o);
+          if (w.out_z) st8_guard_global<T, VEC>(w.out_z + tl, nvalid, oz);
         }
         dbs = row_sum_to_last(dbs);
         dDs = row_sum_to_last(dDs);
