@@ -213,7 +213,8 @@ int ssm_state_update(const MambaStepParams *p, mamba_stream_t stream);
  *                laid out [x (nheads * dim) | B (ngroups * dstate) | C (ngroups * dstate)]
  *   conv_state : (conv_state_rows >= batch, conv_dim, state_len) of ssm.x_dtype through element strides, updated in place
  *                to the last state_len positions of [conv_state, xBC]; width - 1 <= state_len <= 4
- *   conv_weight: (conv_dim, width) fp32 contiguous; conv_bias: (conv_dim) fp32, nullable; width 2..4
+ *   conv_weight: (conv_dim, width) of conv_weight_dtype, contiguous; conv_bias: (conv_dim) of the same dtype, nullable;
+ *                width 2..4
  *   sync       : int32 (mamba2_decode_step_sync_ints(p)), all zero on entry and again on return (the workgroups of a
  *                (batch entry, group) count themselves off here; the last one shifts the conv state of the group's
  *                shared B / C channels once every other one has read it).  Calls that share `sync` must not overlap.
@@ -225,11 +226,12 @@ int ssm_state_update(const MambaStepParams *p, mamba_stream_t stream);
 typedef struct MambaDecodeStepParams {
   MambaStepParams ssm;
   int32_t conv_dim, width, state_len, silu;
-  int32_t conv_state_rows, reserved;
+  int32_t conv_state_rows;
+  int32_t conv_weight_dtype; /* dtype code of conv_weight and conv_bias (MAMBA_F32 = 0 / MAMBA_BF16 / MAMBA_F16) */
   const void *xBC;
   void *conv_state;
-  const float *conv_weight;
-  const float *conv_bias; /* nullable */
+  const void *conv_weight;
+  const void *conv_bias; /* nullable */
   int32_t *sync;
   int64_t xBC_bs;
   int64_t cs_bs, cs_cs, cs_ls; /* conv_state strides: row, channel, position */
@@ -423,11 +425,11 @@ typedef struct CausalConvUpdateParams {
   int32_t dtype, state_dtype;
   int32_t silu;
   int32_t state_rows; /* rows of conv_state; an index outside [0, state_rows) is a padding entry */
-  int32_t reserved;
+  int32_t weight_dtype; /* dtype code of weight and bias (MAMBA_F32 = 0 / MAMBA_BF16 / MAMBA_F16) */
   const void *x;
   void *conv_state;
-  const float *weight;
-  const float *bias; /* nullable */
+  const void *weight; /* (dim, width) of weight_dtype, contiguous */
+  const void *bias;   /* nullable; (dim) of weight_dtype */
   void *out;
   const int32_t *conv_state_indices; /* nullable */
   int64_t x_bs, x_cs, x_ls;

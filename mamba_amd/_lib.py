@@ -47,7 +47,7 @@ class MambaStepParams(ctypes.Structure):
 class MambaDecodeStepParams(ctypes.Structure):
     _fields_ = (
         [("ssm", MambaStepParams)]
-        + [(n, c_i32) for n in ("conv_dim", "width", "state_len", "silu", "conv_state_rows", "reserved")]
+        + [(n, c_i32) for n in ("conv_dim", "width", "state_len", "silu", "conv_state_rows", "conv_weight_dtype")]
         + [(n, c_vp) for n in ("xBC", "conv_state", "conv_weight", "conv_bias", "sync")]
         + [(n, c_i64) for n in ("xBC_bs", "cs_bs", "cs_cs", "cs_ls")]
     )
@@ -84,7 +84,7 @@ class CausalConvParams(ctypes.Structure):
 class CausalConvUpdateParams(ctypes.Structure):
     _fields_ = (
         [(n, c_i32) for n in ("batch", "dim", "seqlen", "width", "state_len", "dtype", "state_dtype", "silu",
-                                "state_rows", "reserved")]
+                                "state_rows", "weight_dtype")]
         + [(n, c_vp) for n in ("x", "conv_state", "weight", "bias", "out", "conv_state_indices")]
         + [(n, c_i64) for n in ("x_bs", "x_cs", "x_ls", "out_bs", "out_cs", "out_ls", "state_bs", "state_cs", "state_ls")]
         + [("cache_seqlens", c_vp)]
@@ -204,6 +204,28 @@ def check(rc, what):
 
 def ptr(t):
     return None if t is None else t.data_ptr()
+
+
+_torch_ext = False  # False: not tried yet; None: not built or switched off
+
+
+def torch_ext():
+    """The C++ host side of the decode-step operators (mamba_amd/_torch_ext.so, built by
+    `python -m mamba_amd.build` from csrc/torch_ext.cpp), or None when it has not been built or
+    MAMBA_AMD_NO_TORCH_EXT=1 is set.  It only shortens the host time of a call: with or without it
+    the same kernels of the same library run."""
+    global _torch_ext
+    if _torch_ext is False:
+        _torch_ext = None
+        if os.environ.get("MAMBA_AMD_NO_TORCH_EXT", "0") != "1":
+            load()  # the extension links against the kernel library: fail on that first, and loudly
+            try:
+                from mamba_amd import _torch_ext as ext
+                if ext.abi_version() == _lib.mamba_hip_query(0):
+                    _torch_ext = ext
+            except ImportError:
+                pass
+    return _torch_ext
 
 
 def current_stream(device):

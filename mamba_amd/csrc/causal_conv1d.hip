@@ -391,6 +391,15 @@ template <typename T, bool VEC> __global__ __launch_bounds__(256) void conv_cl_b
 // (what the reference spells, for one new position and state_len = W, as roll + insert + dot:
 // mamba_ssm/modules/mamba2.py:291-296).  The shift runs in place in ascending order, which is safe
 // because every entry is written from a higher index of the same thread's own row.
+// one filter tap or bias value of the dtype the caller's parameters have
+DEVI float ld_param(const void *base, int dtype, int64_t i) {
+  switch (dtype) {
+    case MAMBA_BF16: return ld1<bf16_t>(static_cast<const bf16_t *>(base) + i);
+    case MAMBA_F16: return ld1<f16_t>(static_cast<const f16_t *>(base) + i);
+    default: return static_cast<const float *>(base)[i];
+  }
+}
+
 template <typename T, typename S> __global__ __launch_bounds__(256) void conv_update_kernel(const CausalConvUpdateParams p) {
   const int c = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
   if (c >= p.dim) return;
@@ -406,9 +415,9 @@ template <typename T, typename S> __global__ __launch_bounds__(256) void conv_up
 #pragma unroll
   for (int k = 0; k < MAXW; ++k) {
     const int j = k - (MAXW - p.width);
-    w[k] = j >= 0 ? p.weight[(int64_t)c * p.width + j] : 0.f;
+    w[k] = j >= 0 ? ld_param(p.weight, p.weight_dtype, (int64_t)c * p.width + j) : 0.f;
   }
-  bias = p.bias ? p.bias[c] : 0.f;
+  bias = p.bias ? ld_param(p.bias, p.weight_dtype, c) : 0.f;
   const int SL = p.state_len;
   float win[MAXW];  // win[0..2]: the three positions before the next output, win[3]: the new one
   if (p.cache_seqlens) {
@@ -542,6 +551,7 @@ extern "C" int causal_conv1d_update(const CausalConvUpdateParams *p, mamba_strea
   if (p->state_len < p->width - 1 || p->state_rows <= 0) return MAMBA_E_BADARG;
   if (!p->conv_state_indices && p->state_rows < p->batch) return MAMBA_E_BADARG;
   if (p->batch > 65535) return MAMBA_E_UNSUPPORTED;
+  if (p->weight_dtype < MAMBA_F32 || p->weight_dtype > MAMBA_F16) return MAMBA_E_BADARG;
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (p->dtype) {
     case MAMBA_F32: return launch_update<float>(*p, s);

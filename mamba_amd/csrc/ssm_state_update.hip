@@ -329,6 +329,15 @@ DEVI float conv_tap(const float (&sv)[3], float xn, const float (&w)[4], float b
   return silu ? silu_act(v) : v;
 }
 
+// one filter tap or bias value of the dtype the caller's parameters have
+DEVI float param_at(const void *base, int dtype, int64_t i) {
+  switch (dtype) {
+    case MAMBA_BF16: return ld1<bf16_t>(static_cast<const bf16_t *>(base) + i);
+    case MAMBA_F16: return ld1<f16_t>(static_cast<const f16_t *>(base) + i);
+    default: return static_cast<const float *>(base)[i];
+  }
+}
+
 // this thread's conv state taps and filter of channel c (element loads from valid addresses)
 template <typename TX>
 DEVI void conv_loads(const MambaDecodeStepParams &q, const TX *cstate, const TX *xBC, int c, float (&sv)[3], float &xn,
@@ -341,18 +350,26 @@ DEVI void conv_loads(const MambaDecodeStepParams &q, const TX *cstate, const TX 
     sv[i] = j >= 0 ? v : 0.f;
   }
   xn = ld1<TX>(xBC + c);
-  if (W == CW) {
-    const f32x4 wq = *reinterpret_cast<const f32x4 *>(q.conv_weight + (int64_t)c * CW);
+  const int wd = q.conv_weight_dtype;
+  if (wd == MAMBA_F32 && W == CW) {
+    const f32x4 wq = *reinterpret_cast<const f32x4 *>(static_cast<const float *>(q.conv_weight) + (int64_t)c * CW);
     w[0] = wq.x; w[1] = wq.y; w[2] = wq.z; w[3] = wq.w;
+  } else if (wd != MAMBA_F32 && W == CW) {  // four 16-bit taps: one 8-byte load
+    const u32x2 wq = *reinterpret_cast<const u32x2 *>(static_cast<const uint16_t *>(q.conv_weight) + (int64_t)c * CW);
+    if (wd == MAMBA_BF16) {
+      w[0] = bf16_lo(wq.x); w[1] = bf16_hi(wq.x); w[2] = bf16_lo(wq.y); w[3] = bf16_hi(wq.y);
+    } else {
+      w[0] = f16_lo(wq.x); w[1] = f16_hi(wq.x); w[2] = f16_lo(wq.y); w[3] = f16_hi(wq.y);
+    }
   } else {
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const int j = k - (CW - W);
-      const float v = q.conv_weight[(int64_t)c * W + max(j, 0)];
+      const float v = param_at(q.conv_weight, wd, (int64_t)c * W + max(j, 0));
       w[k] = j >= 0 ? v : 0.f;
     }
   }
-  bias = q.conv_bias ? q.conv_bias[c] : 0.f;
+  bias = q.conv_bias ? param_at(q.conv_bias, wd, c) : 0.f;
 }
 // conv state of one channel after the step: the old positions moved down by one, the new value last
 template <typename TX> DEVI void conv_shift(TX *st, int SL, int cs_ls, const float (&sv)[3], float xn) {
@@ -582,7 +599,8 @@ extern "C" int mamba2_decode_step(const MambaDecodeStepParams *q, mamba_stream_t
   if (p->nheads % p->ngroups != 0) return MAMBA_E_BADARG;
   if (q->conv_dim != p->nheads * p->dim + 2 * p->ngroups * p->dstate) return MAMBA_E_BADARG;
   if (p->state_rows < p->batch || q->conv_state_rows < p->batch) return MAMBA_E_BADARG;
-  if (!dtype_ok(p->state_dtype) || !dtype_ok(p->x_dtype) || !dtype_ok(p->dt_dtype)) return MAMBA_E_BADARG;
+  if (!dtype_ok(p->state_dtype) || !dtype_ok(p->x_dtype) || !dtype_ok(p->dt_dtype) || !dtype_ok(q->conv_weight_dtype))
+    return MAMBA_E_BADARG;
   // the form served here; anything else is for the two separate calls
   if (p->state_batch_indices) return MAMBA_E_UNSUPPORTED;
   if (reinterpret_cast<uintptr_t>(q->conv_weight) % 16 != 0) return MAMBA_E_UNSUPPORTED;

@@ -195,6 +195,13 @@ def causal_conv1d_update(x, conv_state, weight, bias=None, activation=None, cach
     Returns out with x's shape and dtype."""
     if activation not in (None, "silu", "swish"):
         raise NotImplementedError("activation must be None, silu, or swish")
+    ext = _lib.torch_ext()
+    if ext is not None:
+        # the same checks and launch in C++; None = it declined, and the code below handles the call
+        out = ext.causal_conv1d_update(x, conv_state, weight.detach(), None if bias is None else bias.detach(),
+                                       activation is not None, cache_seqlens, conv_state_indices)
+        if out is not None:
+            return out
     _lib.require_gpu(x, conv_state, weight, bias, conv_state_indices)
     squeeze = x.dim() == 2
     if squeeze:
@@ -224,13 +231,17 @@ def causal_conv1d_update(x, conv_state, weight, bias=None, activation=None, cach
     out = torch.empty_like(x)
     if batch == 0:
         return out.squeeze(-1) if squeeze else out
-    w32 = weight.detach().float().contiguous()
-    b32 = bias.detach().float().contiguous() if bias is not None else None
+    # the kernel reads the filter in fp32, bf16 or fp16 as it is (weight and bias in one dtype)
+    w, bv = weight.detach(), bias.detach() if bias is not None else None
+    if w.dtype not in _lib.DTYPE_CODE or (bv is not None and bv.dtype != w.dtype):
+        w, bv = w.float(), bv.float() if bv is not None else None
+    w, bv = w.contiguous(), bv.contiguous() if bv is not None else None
     p = _lib.CausalConvUpdateParams()
     p.batch, p.dim, p.seqlen, p.width, p.state_len = batch, dim, seqlen, width, conv_state.shape[2]
     p.dtype, p.state_dtype = _lib.DTYPE_CODE[x.dtype], _lib.DTYPE_CODE[conv_state.dtype]
+    p.weight_dtype = _lib.DTYPE_CODE[w.dtype]
     p.silu, p.state_rows = int(activation in ("silu", "swish")), conv_state.shape[0]
-    p.x, p.conv_state, p.weight, p.bias, p.out = x.data_ptr(), conv_state.data_ptr(), w32.data_ptr(), _lib.ptr(b32), out.data_ptr()
+    p.x, p.conv_state, p.weight, p.bias, p.out = x.data_ptr(), conv_state.data_ptr(), w.data_ptr(), _lib.ptr(bv), out.data_ptr()
     p.conv_state_indices = _lib.ptr(conv_state_indices)
     p.cache_seqlens = _lib.ptr(cache_seqlens)
     p.x_bs, p.x_cs, p.x_ls = _strides_bcl(x)

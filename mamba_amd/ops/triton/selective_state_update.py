@@ -28,6 +28,13 @@ def selective_state_update(state, x, dt, A, B, C, D=None, z=None, dt_bias=None, 
     Return:
         out: (batch, dim) or (batch, nheads, dim)
     """
+    ext = _lib.torch_ext()
+    if ext is not None:
+        # the same checks and launch in C++ (a few us of host time instead of ~15); it declines (None)
+        # whatever needs a conversion or an error message, which the code below then handles
+        out = ext.selective_state_update(state, x, dt, A, B, C, D, z, dt_bias, bool(dt_softplus), state_batch_indices)
+        if out is not None:
+            return out
     has_heads = state.dim() > 3
     if state.dim() == 3:
         state = state.unsqueeze(1)
@@ -172,11 +179,14 @@ def mamba2_decode_step(ssm_state, conv_state, xBC, dt, A, conv_weight, conv_bias
                and xBC.stride(1) == 1 and ssm_state.stride(3) == 1 and (z is None or z.dtype == xBC.dtype))
     explicit = fuse is True
     if fuse is None:
-        # Measured (80 heads x 64, 128 states, one MI355X): replayed from a captured graph the fused kernel takes as
-        # long as the two launches at batch 1 (12 us) and 2-16 us longer above (its ordered hand-over of the shared
-        # B / C conv state costs what the second launch costs); called eagerly it saves one host call (27 us against
-        # 47 us per token up to batch ~16, after which kernel time decides).
-        fuse = fusable and batch <= FUSE_MAX_BATCH and not torch.cuda.is_current_stream_capturing()
+        # Measured (80 heads x 64, 128 states, bf16 filter, one MI355X), per token: replayed from a captured graph
+        # the two launches take 8.7 us at batch 1 and the fused kernel 9.2 us (13.6 against 16.2 us at batch 8: its
+        # ordered hand-over of the shared B / C conv state costs more than the second launch).  Called eagerly the
+        # fused kernel saves one host call: 17.6 against 37.9 us through the Python + ctypes host side, but nothing
+        # once the C++ host side (mamba_amd/_torch_ext.so) is there: 15.4 against 15.0 us.  So it is picked only for
+        # eager calls at small batch without that extension.
+        fuse = (fusable and batch <= FUSE_MAX_BATCH and _lib.torch_ext() is None
+                and not torch.cuda.is_current_stream_capturing())
         if not fuse:
             return two_calls()
     if fuse is False:
@@ -188,8 +198,11 @@ def mamba2_decode_step(ssm_state, conv_state, xBC, dt, A, conv_weight, conv_bias
     dtb32 = dt_bias.float() if dt_bias is not None else None
     if dt.dtype != xBC.dtype:
         dt = dt.float()
-    w32 = conv_weight.detach().float().contiguous()
-    b32 = conv_bias.detach().float().contiguous() if conv_bias is not None else None
+    # the filter is read in fp32, bf16 or fp16 as it is (weight and bias in one dtype)
+    w32, b32 = conv_weight.detach(), conv_bias.detach() if conv_bias is not None else None
+    if w32.dtype not in code or (b32 is not None and b32.dtype != w32.dtype):
+        w32, b32 = w32.float(), b32.float() if b32 is not None else None
+    w32, b32 = w32.contiguous(), b32.contiguous() if b32 is not None else None
     out = torch.empty(batch, nheads, headdim, dtype=xBC.dtype, device=xBC.device)
     q = _lib.MambaDecodeStepParams()
     p = q.ssm
@@ -219,6 +232,7 @@ def mamba2_decode_step(ssm_state, conv_state, xBC, dt, A, conv_weight, conv_bias
         p.z_bs, p.z_hs, p.z_ps = z.stride()
     p.out_bs, p.out_hs, p.out_ps = out.stride()
     q.conv_dim, q.width, q.state_len = conv_dim, width, state_len
+    q.conv_weight_dtype = code[w32.dtype]
     q.silu, q.conv_state_rows = int(activation in ("silu", "swish")), conv_state.shape[0]
     q.xBC, q.conv_state, q.conv_weight, q.conv_bias = xBC.data_ptr(), conv_state.data_ptr(), w32.data_ptr(), _lib.ptr(b32)
     q.sync = sync.data_ptr()

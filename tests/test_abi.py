@@ -109,3 +109,17 @@ def test_shape_errors_match_the_reference_behaviour():
     with pytest.raises(AssertionError):   # nheads % ngroups, ssd_combined.py:346
         mamba_chunk_scan_combined(torch.randn(1, 8, 3, 4), torch.randn(1, 8, 3), -torch.ones(3),
                                   torch.randn(1, 8, 2, 4), torch.randn(1, 8, 2, 4), 4)
+
+
+def test_torch_extension_loads_and_declines_cpu_tensors():
+    """mamba_amd/_torch_ext.so (C++ host side of the decode-step operators): imports without a GPU, reports
+    the library's ABI version, and declines (None) instead of launching on CPU tensors."""
+    import torch
+    from mamba_amd import _lib
+    ext = _lib.torch_ext()
+    assert ext is not None, "mamba_amd/_torch_ext.so is not built (python -m mamba_amd.build)"
+    assert ext.abi_version() == _lib.load().mamba_hip_query(0)
+    s, x = torch.zeros(2, 4, 8), torch.zeros(2, 4)
+    A, B = -torch.ones(4, 8), torch.zeros(2, 8)
+    assert ext.selective_state_update(s, x, x, A, B, B, None, None, None, False, None) is None
+    assert ext.causal_conv1d_update(x, torch.zeros(2, 4, 3), torch.zeros(4, 4), None, True, None, None) is None

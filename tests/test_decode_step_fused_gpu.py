@@ -125,3 +125,18 @@ def test_fused_in_a_captured_graph():
         _ = (got.float() * 2).sum().item()   # eager work and a synchronisation between the replays
         assert torch.equal(got, want[i]), f"replay {i}"
     assert torch.equal(ssm, ssm_w) and torch.equal(conv, conv_w)
+
+
+@pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("W", [2, 3, 4])
+@pytest.mark.parametrize("fuse", [False, True])
+def test_filter_dtypes_same_bits_as_their_fp32_copies(wdtype, W, fuse):
+    """The kernels read a bf16 / fp16 filter as it is: same bits as with its exact fp32 copy."""
+    t, steps = _setup(2, 4, 64, 64, 2, W, 4, torch.bfloat16, torch.float32, True, True, True, True, True, seed=W)
+    t["conv_w"], t["conv_b"] = t["conv_w"].to(wdtype), t["conv_b"].to(wdtype)
+    got, ssm_g, conv_g = _run(t, steps, 2, fuse)
+    t["conv_w"], t["conv_b"] = t["conv_w"].float(), t["conv_b"].float()
+    want, ssm_w, conv_w = _run(t, steps, 2, fuse)
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+    assert torch.equal(ssm_g, ssm_w) and torch.equal(conv_g, conv_w)
