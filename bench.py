@@ -276,7 +276,7 @@ def bench_ssd(dev, steps, warmup):
     nc = L // Q
     mfma_tflops = measured_mfma(dev)
     flops = batch * nc * (H * (Q * Q * P + 2 * Q * N * P) + G * Q * Q * N)   # causal halves counted once
-    nbytes = 2 * (4 * batch * L * H * P + 2 * batch * L * G * N) + 4 * batch * nc * H * P * N  # x z out out_x B C states
+    nbytes = 2 * (4 * batch * L * H * P + 2 * batch * L * G * N) + 2 * batch * nc * H * P * N  # x z out out_x B C, bf16 states
     return ({
         "metric": "SSD mamba_chunk_scan_combined fwd+bwd tokens/s at 1 GPU", "value": batch * L / sec,
         "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": sec * 1e3,

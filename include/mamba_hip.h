@@ -314,6 +314,15 @@ typedef struct SsdParams {
    * Counterpart of the reference's deterministic mode, mamba_ssm/utils/determinism.py:21-27. */
   const float *det_scale;
   int64_t *det_dD, *det_ddA_cumsum, *det_ddt_out, *det_dCB, *det_dB, *det_dC, *det_dA, *det_ddt_bias;
+  /* With dtype MAMBA_BF16 the states carried between chunks and their gradients pass between the kernels in bf16
+   * (the matrix products take only the bf16 part of them anyway; the reference hands them on in the operands' dtype
+   * too, ssd_combined.py:384-386 out_dtype=C.dtype and :455-466 dstates_dtype=x.dtype), both (b, c, H, P, N):
+   *   states_lp   written by ssd_state_passing_fwd (`states` then keeps the chunks' own states and is not needed
+   *               afterwards), read by the scan, ssd_chunk_state_varlen, ssd_state_passing_bwd and ssd_bwd_dBC_state;
+   *   dstates_lp  takes the place of `dstates` in every backward stage.
+   * Required (non-NULL) for MAMBA_BF16, ignored for the other dtypes, which keep the fp32 `states` (in place) and
+   * `dstates`. */
+  void *states_lp, *dstates_lp;
 } SsdParams;
 
 /* forward stages, in launch order */

@@ -66,7 +66,7 @@ class SsdParams(ctypes.Structure):
                                "dinitial_states", "dstates", "ddA_cumsum", "ddt_out", "dCB", "dB32", "dC32", "gbuf")]
         + [(n, c_i64) for n in ("dout_bs", "dout_ls", "dout_hs", "dx_bs", "dx_ls", "dx_hs")]
         + [(n, c_vp) for n in ("det_scale", "det_dD", "det_ddA_cumsum", "det_ddt_out", "det_dCB", "det_dB", "det_dC",
-                               "det_dA", "det_ddt_bias")]
+                               "det_dA", "det_ddt_bias", "states_lp", "dstates_lp")]
     )
 
 

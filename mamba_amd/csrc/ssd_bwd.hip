@@ -255,10 +255,10 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dst
       TrStager<SPLIT, T>(lds.ah, lds.al, ga, gv.ls, P - pt * GB, qlim, nullptr, nullptr, va, tid),
       TrStager<SPLIT, T>(lds.bh, lds.bl, Ca, p.C_ls, N - nt * GB, qlim, rs, nullptr, vb, tid),
       tid);
-  float *ds = p.dstates + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
+  carried_t<T> *ds = carried_dstates<T>(p) + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
   acc_foreach(acc, tid, [&](int m, int n, float v) {
     const int pp = pt * GB + m, nn = nt * GB + n;
-    if (pp < P && nn < N) ds[(int64_t)pp * N + nn] = v;
+    if (pp < P && nn < N) st_carried(ds + (int64_t)pp * N + nn, v);
     return v;
   });
 }
@@ -295,7 +295,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dst
   WideTrStager<SPLIT, T, 64> sa(lds.ah, lds.al, ga, gv.ls, P - pt * GB, nullptr, tid);
   WideTrStager<SPLIT, T, WB> sb(lds.bh, lds.bl, Ca, p.C_ls, WB, rs, tid);
   block_gemm_wide<SPLIT>(acc, lds, qlim, sa, sb, tid);  // the first barrier inside publishes rs
-  float *ds = p.dstates + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
+  carried_t<T> *ds = carried_dstates<T>(p) + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
   store_wide(acc, ds + (int64_t)pt * GB * N + nt * WB, N, P - pt * GB, tid);
 }
 
@@ -312,6 +312,8 @@ template <> struct VecG<1> {
   float v[1];
   DEVI void load(const float *p) { v[0] = *p; }
   DEVI void store(float *p) const { *p = v[0]; }
+  DEVI void load(const bf16_t *p) { v[0] = ld1<bf16_t>(p); }
+  DEVI void store(bf16_t *p) const { st1<bf16_t>(p, v[0]); }
 };
 template <> struct VecG<4> {
   float v[4];
@@ -320,9 +322,17 @@ template <> struct VecG<4> {
     v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
   }
   DEVI void store(float *p) const { *reinterpret_cast<f32x4 *>(p) = f32x4{v[0], v[1], v[2], v[3]}; }
+  DEVI void load(const bf16_t *p) {
+    const u32x2 t = *reinterpret_cast<const u32x2 *>(p);
+    v[0] = bf16_lo(t.x); v[1] = bf16_hi(t.x); v[2] = bf16_lo(t.y); v[3] = bf16_hi(t.y);
+  }
+  DEVI void store(bf16_t *p) const { *reinterpret_cast<u32x2 *>(p) = u32x2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])}; }
 };
 
-template <int W> __global__ __launch_bounds__(256) void state_passing_bwd_kernel(const SsdParams p) {
+// CT: dtype of the carried states and of dstates (float, or bf16_t next to bf16 operands)
+template <int W, typename CT> __global__ __launch_bounds__(256) void state_passing_bwd_kernel(const SsdParams p) {
+  CT *const dst_p = std::is_same_v<CT, float> ? reinterpret_cast<CT *>(p.dstates) : static_cast<CT *>(p.dstates_lp);
+  const CT *const st_p = std::is_same_v<CT, float> ? reinterpret_cast<const CT *>(p.states) : static_cast<const CT *>(p.states_lp);
   const int PN = p.headdim * p.dstate, H = p.nheads, nc = p.nchunks, Q = p.chunk_size, L = p.seqlen;
   const int e = (blockIdx.x * 256 + threadIdx.x) * W;
   const int lane = threadIdx.x & 63;
@@ -351,8 +361,8 @@ template <int W> __global__ __launch_bounds__(256) void state_passing_bwd_kernel
   for (int j = 0; j < SPB_PF; ++j) {
     const int c = nc - 1 - j;
     if (c >= 0) {
-      direct[j].load(p.dstates + offset(c));
-      state[j].load(p.states + offset(c));
+      direct[j].load(dst_p + offset(c));
+      state[j].load(st_p + offset(c));
       scale[j] = decay(c);
     }
   }
@@ -361,12 +371,12 @@ template <int W> __global__ __launch_bounds__(256) void state_passing_bwd_kernel
     for (int j = 0; j < SPB_PF; ++j) {
       const int c = c0 - j;
       if (c < 0) break;
-      if (live) G.store(p.dstates + offset(c));
+      if (live) G.store(dst_p + offset(c));
       const VecG<W> dir = direct[j], st = state[j];
       const float sc = scale[j];
       if (c - SPB_PF >= 0) {
-        direct[j].load(p.dstates + offset(c - SPB_PF));
-        state[j].load(p.states + offset(c - SPB_PF));
+        direct[j].load(dst_p + offset(c - SPB_PF));
+        state[j].load(st_p + offset(c - SPB_PF));
         scale[j] = decay(c - SPB_PF);
       }
       float part = 0.f;
@@ -432,7 +442,7 @@ template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256) vo
   }
   const View4 gv = g_view(p);
   const int64_t gb = b * gv.bs + h * gv.hs, xb = b * p.x_bs + h * p.x_hs, Bb = b * p.B_bs + g * p.B_gs;
-  const float *dS = p.dstates + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
+  const carried_t<T> *dS = carried_dstates<T>(p) + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
   const float *CB = p.CB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
   GemmAcc acc1, acc2;  // carried-state part, in-chunk part
   acc1.zero();
@@ -440,12 +450,12 @@ template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256) vo
   {
     // A = B rows (s, k = n), B = dS rows (p, k = n): both k-contiguous
     const T *Ba = static_cast<const T *>(p.B) + Bb + (int64_t)(t0 + st * GB) * p.B_ls;
-    const float *dSa = dS + (int64_t)pt * GB * N;
+    const carried_t<T> *dSa = dS + (int64_t)pt * GB * N;
     const bool va = rows_aligned16(Ba, p.B_ls), vb = rows_aligned16(dSa, N);
     block_gemm_pipe<SPLIT>(
         acc1, lds, 0, N,
         KcStager<SPLIT, T>(lds.ah, lds.al, Ba, p.B_ls, qlim - st * GB, N, nullptr, nullptr, va, tid),
-        KcStager<SPLIT, float>(lds.bh, lds.bl, dSa, N, P - pt * GB, N, nullptr, nullptr, vb, tid),
+        KcStager<SPLIT, carried_t<T>>(lds.bh, lds.bl, dSa, N, P - pt * GB, N, nullptr, nullptr, vb, tid),
         tid);
   }
   {
@@ -608,9 +618,9 @@ template <typename T, bool SPLIT, bool DET, int PARTS> DEVI void dBC_state_body(
                      q.rscale = wB[hl];
                    },
                    seg_k),
-        seg_stager(TrStager<SPLIT, float>(lds.bh, lds.bl, nullptr, N, N - nt * GB, P, nullptr, nullptr, false, tid),
-                   [&](TrStager<SPLIT, float> &q, int hl) {
-                     q.base = p.dstates + state_off(hl);
+        seg_stager(TrStager<SPLIT, carried_t<T>>(lds.bh, lds.bl, nullptr, N, N - nt * GB, P, nullptr, nullptr, false, tid),
+                   [&](TrStager<SPLIT, carried_t<T>> &q, int hl) {
+                     q.base = carried_dstates<T>(p) + state_off(hl);
                      q.vec = rows_aligned16(q.base, N);
                    },
                    seg_k),
@@ -647,9 +657,9 @@ template <typename T, bool SPLIT, bool DET, int PARTS> DEVI void dBC_state_body(
                      q.rscale = wC[hl];
                    },
                    seg_k),
-        seg_stager(TrStager<SPLIT, float>(lds.bh, lds.bl, nullptr, N, N - nt * GB, P, nullptr, nullptr, false, tid),
-                   [&](TrStager<SPLIT, float> &q, int hl) {
-                     q.base = p.states + state_off(hl);
+        seg_stager(TrStager<SPLIT, carried_t<T>>(lds.bh, lds.bl, nullptr, N, N - nt * GB, P, nullptr, nullptr, false, tid),
+                   [&](TrStager<SPLIT, carried_t<T>> &q, int hl) {
+                     q.base = carried_states<T>(p) + state_off(hl);
                      q.vec = rows_aligned16(q.base, N);
                    },
                    seg_k),
@@ -738,9 +748,9 @@ template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256) vo
                          q.rscale = wB[hl];
                        },
                        P);
-  auto sb = seg_stager(WideTrStager<SPLIT, float, WB>(lds.bh, lds.bl, nullptr, N, WB, nullptr, tid),
-                       [&](WideTrStager<SPLIT, float, WB> &q, int hl) {
-                         q.base = p.dstates + (((int64_t)b * p.nchunks + c) * H + g * hpg + hs + hl * nsplit) * P * N + nt * WB;
+  auto sb = seg_stager(WideTrStager<SPLIT, carried_t<T>, WB>(lds.bh, lds.bl, nullptr, N, WB, nullptr, tid),
+                       [&](WideTrStager<SPLIT, carried_t<T>, WB> &q, int hl) {
+                         q.base = carried_dstates<T>(p) + (((int64_t)b * p.nchunks + c) * H + g * hpg + hs + hl * nsplit) * P * N + nt * WB;
                        },
                        P);
   block_gemm_wide<SPLIT>(accB, lds, nh * P, sa, sb, tid);  // the first barrier inside publishes wB
@@ -830,9 +840,9 @@ template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256, 4)
                          q.rscale = wC[hl];
                        },
                        P);
-  auto sb = seg_stager(WideTrStager<SPLIT, float, WB>(lds.bh, lds.bl, nullptr, N, WB, nullptr, tid),
-                       [&](WideTrStager<SPLIT, float, WB> &q, int hl) {
-                         q.base = p.states + (((int64_t)b * p.nchunks + c) * H + g * hpg + hs + hl * nsplit) * P * N + nt * WB;
+  auto sb = seg_stager(WideTrStager<SPLIT, carried_t<T>, WB>(lds.bh, lds.bl, nullptr, N, WB, nullptr, tid),
+                       [&](WideTrStager<SPLIT, carried_t<T>, WB> &q, int hl) {
+                         q.base = carried_states<T>(p) + (((int64_t)b * p.nchunks + c) * H + g * hpg + hs + hl * nsplit) * P * N + nt * WB;
                        },
                        P);
   block_gemm_wide<SPLIT>(acc, lds, nh * P, sa, sb, tid, [&](int k0) {  // the first barrier inside publishes wC
@@ -1146,9 +1156,16 @@ int check_bwd(const SsdParams *p) {
   if (p->chunk_size > 256 || p->dstate > 256 || p->headdim > 256) return MAMBA_E_UNSUPPORTED;
   if ((int64_t)p->batch * p->nheads > 65535 || p->nchunks > 65535) return MAMBA_E_UNSUPPORTED;
   if (p->dtype != MAMBA_F32 && p->dtype != MAMBA_BF16 && p->dtype != MAMBA_F16) return MAMBA_E_BADARG;
-  if (!p->dt_out || !p->dA_cumsum || !p->states || !p->CB || !p->dstates || !p->ddA_cumsum || !p->ddt_out ||
-      !p->dCB || !p->dB32 || !p->dC32 || !p->dx || !p->ddt || !p->dA)
+  if (!p->dt_out || !p->dA_cumsum || !p->CB || !p->ddA_cumsum || !p->ddt_out || !p->dCB || !p->dB32 || !p->dC32 ||
+      !p->dx || !p->ddt || !p->dA)
     return MAMBA_E_BADARG;
+  // the carried states and their gradients: bf16 buffers next to bf16 operands, the fp32 ones otherwise
+  if (p->dtype == MAMBA_BF16) {
+    if (!p->states_lp || !p->dstates_lp) return MAMBA_E_BADARG;
+    if ((reinterpret_cast<uintptr_t>(p->states_lp) | reinterpret_cast<uintptr_t>(p->dstates_lp)) & 15) return MAMBA_E_BADARG;
+  } else if (!p->states || !p->dstates) {
+    return MAMBA_E_BADARG;
+  }
   if (p->z && (!p->dz || !p->gbuf || !p->out_x)) return MAMBA_E_BADARG;
   if (!p->z && !p->out) return MAMBA_E_BADARG;
   if (p->D && !p->dD) return MAMBA_E_BADARG;
@@ -1222,12 +1239,17 @@ extern "C" int ssd_state_passing_bwd(const SsdParams *p, mamba_stream_t stream) 
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int PN = p->headdim * p->dstate;
   auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
-  if (PN % 4 == 0 && al16(p->states) && al16(p->dstates) && al16(p->dfinal_states) && al16(p->dinitial_states)) {
+  const bool lp = p->dtype == MAMBA_BF16;
+  const bool vec = PN % 4 == 0 && al16(p->dfinal_states) && al16(p->dinitial_states) &&
+                   (lp ? true : al16(p->states) && al16(p->dstates));
+  if (vec) {
     dim3 grid((PN / 4 + 255) / 256, p->nheads, p->batch);
-    hipLaunchKernelGGL(state_passing_bwd_kernel<4>, grid, dim3(256), 0, s, *p);
+    if (lp) hipLaunchKernelGGL((state_passing_bwd_kernel<4, bf16_t>), grid, dim3(256), 0, s, *p);
+    else hipLaunchKernelGGL((state_passing_bwd_kernel<4, float>), grid, dim3(256), 0, s, *p);
   } else {
     dim3 grid((PN + 255) / 256, p->nheads, p->batch);
-    hipLaunchKernelGGL(state_passing_bwd_kernel<1>, grid, dim3(256), 0, s, *p);
+    if (lp) hipLaunchKernelGGL((state_passing_bwd_kernel<1, bf16_t>), grid, dim3(256), 0, s, *p);
+    else hipLaunchKernelGGL((state_passing_bwd_kernel<1, float>), grid, dim3(256), 0, s, *p);
   }
   return launched();
 }

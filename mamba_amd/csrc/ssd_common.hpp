@@ -418,7 +418,21 @@ DEVI void block_gemm_wide(GemmAccWide &acc, GemmLdsWide<SPLIT> &s, int k_end, SA
 }
 
 // Stores the wide tile as fp32 rows of dst (the tile's origin, row pitch ld); rows >= rows_valid are skipped.
-DEVI void store_wide(const GemmAccWide &acc, float *dst, int64_t ld, int rows_valid, int tid) {
+// dtype in which the states carried between chunks, and their gradients, pass between kernels: bf16 next to bf16
+// operands (the matrix products only take that part of them), fp32 otherwise.
+template <typename T> using carried_t = std::conditional_t<std::is_same_v<T, bf16_t>, bf16_t, float>;
+template <typename T> DEVI carried_t<T> *carried_states(const SsdParams &p) {
+  if constexpr (std::is_same_v<T, bf16_t>) return static_cast<bf16_t *>(p.states_lp);
+  else return p.states;
+}
+template <typename T> DEVI carried_t<T> *carried_dstates(const SsdParams &p) {
+  if constexpr (std::is_same_v<T, bf16_t>) return static_cast<bf16_t *>(p.dstates_lp);
+  else return p.dstates;
+}
+DEVI void st_carried(float *p, float v) { *p = v; }
+DEVI void st_carried(bf16_t *p, float v) { st1<bf16_t>(p, v); }
+
+template <typename D> DEVI void store_wide(const GemmAccWide &acc, D *dst, int64_t ld, int rows_valid, int tid) {
   const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1, i = lane & 15, g = lane >> 4;
 #pragma unroll
   for (int tm = 0; tm < 2; ++tm)
@@ -427,7 +441,7 @@ DEVI void store_wide(const GemmAccWide &acc, float *dst, int64_t ld, int rows_va
       const int m = wm * 32 + tm * 16 + g * 4 + r;
       if (m >= rows_valid) continue;
 #pragma unroll
-      for (int tn = 0; tn < 4; ++tn) dst[(int64_t)m * ld + wn * 64 + tn * 16 + i] = acc.v[tm][tn][r];
+      for (int tn = 0; tn < 4; ++tn) st_carried(dst + (int64_t)m * ld + wn * 64 + tn * 16 + i, acc.v[tm][tn][r]);
     }
 }
 // Host side: a (batch, position, head/group, row) operand can feed WideTrStager.

@@ -230,11 +230,11 @@ __global__ __launch_bounds__(256) void chunk_state_varlen_kernel(const SsdParams
         TrStager<SPLIT, T>(lds.bh, lds.bl, Ba, p.B_ls, N - nt * GB, kend, w, nullptr, vb, tid),
         tid);
     if (start < t0) {
-      const float *Hc = p.states + ((int64_t)c * H + h) * P * N;
+      const carried_t<T> *Hc = carried_states<T>(p) + ((int64_t)c * H + h) * P * N;
       const float sc = fast_exp(a_end);
       acc_foreach(acc, tid, [&](int m, int n, float v) {
         const int pp = pt * GB + m, nn = nt * GB + n;
-        return (pp < P && nn < N) ? __builtin_fmaf(sc, Hc[(int64_t)pp * N + nn], v) : v;
+        return (pp < P && nn < N) ? __builtin_fmaf(sc, ld1<carried_t<T>>(Hc + (int64_t)pp * N + nn), v) : v;
       });
     }
   }
@@ -268,7 +268,9 @@ template <> struct VecF<4> {
   DEVI void store(float *p) const { *reinterpret_cast<f32x4 *>(p) = f32x4{v[0], v[1], v[2], v[3]}; }
 };
 
-template <int W> __global__ __launch_bounds__(256) void state_passing_fwd_kernel(const SsdParams p) {
+// CT float: in place, slot c of `states` receives the state entering chunk c.  CT bf16_t: that state goes to
+// states_lp in bf16 and `states` is only read.
+template <int W, typename CT> __global__ __launch_bounds__(256) void state_passing_fwd_kernel(const SsdParams p) {
   const int PN = p.headdim * p.dstate, H = p.nheads, nc = p.nchunks, Q = p.chunk_size, L = p.seqlen;
   const int e = (blockIdx.x * 256 + threadIdx.x) * W;
   const int h = blockIdx.y, b = blockIdx.z;
@@ -301,7 +303,16 @@ template <int W> __global__ __launch_bounds__(256) void state_passing_fwd_kernel
     for (int j = 0; j < SP_PF; ++j) {
       const int c = c0 + j;
       if (c >= nc) break;
-      s.store(slot(c));
+      if constexpr (std::is_same_v<CT, float>) {
+        s.store(slot(c));
+      } else {
+        CT *o = static_cast<CT *>(p.states_lp) + (((int64_t)b * nc + c) * H + h) * PN + e;
+        if constexpr (W == 4) {
+          *reinterpret_cast<u32x2 *>(o) = u32x2{pack_bf16(s.v[0], s.v[1]), pack_bf16(s.v[2], s.v[3])};
+        } else {
+          st1<CT>(o, s.v[0]);
+        }
+      }
       const VecF<W> loc = local[j];
       const float sc = scale[j];
       if (c + SP_PF < nc) {
@@ -350,7 +361,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void chunk_s
     rscale[tid] = sc;
   }
   const int64_t xb = b * p.x_bs + h * p.x_hs, Cb = b * p.C_bs + g * p.C_gs;
-  const float *Hc = p.states + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
+  const carried_t<T> *Hc = carried_states<T>(p) + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
   const float *CB = p.CB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
   GemmAcc acc;
   acc.zero();
@@ -361,7 +372,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void chunk_s
     };
     auto fb = [&](int r, int k) {  // (p, n)
       const int pp = pt * GB + r;
-      return (pp < P && k < N) ? Hc[(int64_t)pp * N + k] : 0.f;
+      return (pp < P && k < N) ? ld1<carried_t<T>>(Hc + (int64_t)pp * N + k) : 0.f;
     };
     block_gemm<SPLIT, true, true>(acc, lds, 0, N, fa, fb, tid);
     acc_foreach(acc, tid, [&](int m, int n, float v) { return v * rscale[m]; });
@@ -470,7 +481,8 @@ extern "C" int ssd_chunk_state_varlen(const SsdParams *p, const int32_t *cu_seql
                                       mamba_stream_t stream) {
   int rc = check(p);
   if (rc) return rc;
-  if (!p->states || !p->dt_out || !p->dA_cumsum || !cu_seqlens || !varlen_states) return MAMBA_E_BADARG;
+  if (!p->dt_out || !p->dA_cumsum || !cu_seqlens || !varlen_states) return MAMBA_E_BADARG;
+  if (!(p->dtype == MAMBA_BF16 ? p->states_lp : (void *)p->states)) return MAMBA_E_BADARG;  // the carried states
   if (p->batch != 1 || nseq < 0 || nseq > 65535) return MAMBA_E_BADARG;
   if (nseq == 0) return MAMBA_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -496,12 +508,16 @@ extern "C" int ssd_state_passing_fwd(const SsdParams *p, mamba_stream_t stream) 
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int PN = p->headdim * p->dstate;
   auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
-  if (PN % 4 == 0 && al16(p->states) && al16(p->final_states) && al16(p->initial_states)) {
+  const bool lp = p->dtype == MAMBA_BF16;
+  if (lp && !p->states_lp) return MAMBA_E_BADARG;
+  if (PN % 4 == 0 && al16(p->states) && al16(p->final_states) && al16(p->initial_states) && al16(p->states_lp)) {
     dim3 grid((PN / 4 + 255) / 256, p->nheads, p->batch);
-    hipLaunchKernelGGL(state_passing_fwd_kernel<4>, grid, dim3(256), 0, s, *p);
+    if (lp) hipLaunchKernelGGL((state_passing_fwd_kernel<4, bf16_t>), grid, dim3(256), 0, s, *p);
+    else hipLaunchKernelGGL((state_passing_fwd_kernel<4, float>), grid, dim3(256), 0, s, *p);
   } else {
     dim3 grid((PN + 255) / 256, p->nheads, p->batch);
-    hipLaunchKernelGGL(state_passing_fwd_kernel<1>, grid, dim3(256), 0, s, *p);
+    if (lp) hipLaunchKernelGGL((state_passing_fwd_kernel<1, bf16_t>), grid, dim3(256), 0, s, *p);
+    else hipLaunchKernelGGL((state_passing_fwd_kernel<1, float>), grid, dim3(256), 0, s, *p);
   }
   return launched();
 }
@@ -509,7 +525,8 @@ extern "C" int ssd_state_passing_fwd(const SsdParams *p, mamba_stream_t stream) 
 extern "C" int ssd_chunk_scan_fwd(const SsdParams *p, mamba_stream_t stream) {
   int rc = check(p);
   if (rc) return rc;
-  if (!p->states || !p->CB || !p->out || !p->dt_out || !p->dA_cumsum || (p->z && !p->out_x)) return MAMBA_E_BADARG;
+  if (!p->CB || !p->out || !p->dt_out || !p->dA_cumsum || (p->z && !p->out_x)) return MAMBA_E_BADARG;
+  if (!(p->dtype == MAMBA_BF16 ? p->states_lp : (void *)p->states)) return MAMBA_E_BADARG;  // the carried states
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid(((p->chunk_size + GB - 1) / GB) * ((p->headdim + GB - 1) / GB), p->nchunks, p->batch * p->nheads);
   SSD_DISPATCH(chunk_scan_fwd_kernel, grid)

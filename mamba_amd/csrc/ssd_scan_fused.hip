@@ -157,19 +157,16 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
       Cf[k][kk] = __builtin_bit_cast(bf16x8_t, v);
     }
   }
-  // carried state, fp32 -> bf16, rows p, k = n
+  // carried state (bf16 in memory), rows p, k = n
   constexpr int HCH = (P * N / 8 + NT - 1) / NT;
-  f32x4 hraw[HCH][2];
+  u32x4 hraw[HCH];
   {
-    const float *Hc = p.states + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
+    const bf16_t *Hc = static_cast<const bf16_t *>(p.states_lp) + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
 #pragma unroll
     for (int q = 0; q < HCH; ++q) {
       const int id = tid + q * NT;
-      hraw[q][0] = hraw[q][1] = f32x4{0.f, 0.f, 0.f, 0.f};
-      if (id < P * N / 8) {
-        hraw[q][0] = *reinterpret_cast<const f32x4 *>(Hc + (int64_t)id * 8);
-        hraw[q][1] = *reinterpret_cast<const f32x4 *>(Hc + (int64_t)id * 8 + 4);
-      }
+      hraw[q] = u32x4{0, 0, 0, 0};
+      if (id < P * N / 8) hraw[q] = *reinterpret_cast<const u32x4 *>(Hc + (int64_t)id * 8);
     }
   }
   // ---- per-position scalars of this (batch, head, chunk)
@@ -197,9 +194,7 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
 #pragma unroll
   for (int q = 0; q < HCH; ++q) {
     const int id = tid + q * NT, pp = id / (N / 8), c8 = id % (N / 8);
-    const f32x4 v0 = hraw[q][0], v1 = hraw[q][1];
-    const u32x4 o = {pack_bf16(v0.x, v0.y), pack_bf16(v0.z, v0.w), pack_bf16(v1.x, v1.y), pack_bf16(v1.z, v1.w)};
-    if (id < P * N / 8) *reinterpret_cast<u32x4 *>(&Hs[pp * BP + c8 * 8]) = o;
+    if (id < P * N / 8) *reinterpret_cast<u32x4 *>(&Hs[pp * BP + c8 * 8]) = hraw[q];
   }
   store_block(0, bregs[0], xregs[0]);
   __syncthreads();
@@ -383,12 +378,13 @@ extern "C" int ssd_chunk_scan_fwd_fused_supported(const SsdParams *p) {
     return 0;
   if (p->out_bs % 8 || p->out_ls % 8 || p->out_hs % 8) return 0;
   if (p->z && (!aligned(p->z, 16) || !aligned(p->out_x, 16) || p->z_bs % 8 || p->z_ls % 8 || p->z_hs % 8)) return 0;
+  if (p->states_lp && !aligned(p->states_lp, 16)) return 0;
   if (p->batch > 65535 || p->nheads > 65535) return 0;
   return 1;
 }
 
 extern "C" int ssd_chunk_scan_fwd_fused(const SsdParams *p, mamba_stream_t stream) {
-  if (!p || !p->x || !p->B || !p->C || !p->states || !p->out || !p->dt_out || !p->dA_cumsum || (p->z && !p->out_x))
+  if (!p || !p->x || !p->B || !p->C || !p->states_lp || !p->out || !p->dt_out || !p->dA_cumsum || (p->z && !p->out_x))
     return MAMBA_E_BADARG;
   if (!ssd_chunk_scan_fwd_fused_supported(p)) return MAMBA_E_UNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);

@@ -27,7 +27,25 @@ def stage_params(device, *, batch, seqlen, nheads, headdim, dstate, ngroups, chu
     blank = torch.zeros(64, device=device, dtype=torch.float32)
     for name in _ALWAYS + (_ALWAYS_BWD if backward else ()):
         setattr(p, name, blank.data_ptr())
+    if backward and dtype == torch.bfloat16:
+        p.states_lp = p.dstates_lp = blank.data_ptr()
     return p, blank
+
+
+def carried_dtype(x_dtype):
+    """dtype in which the states carried between chunks, and their gradients, pass between the kernels: bf16 next to
+    bf16 operands, fp32 otherwise."""
+    return torch.bfloat16 if x_dtype == torch.bfloat16 else torch.float32
+
+
+def set_carried(p, field, t, x_dtype):
+    """Hands the kernels a (batch, nchunks, nheads, headdim, dstate) tensor of carried states (`field` = "states") or
+    of their gradients ("dstates") in the dtype they take it in: bf16 through the *_lp field next to bf16 operands,
+    fp32 through the field itself otherwise.  Returns the tensor handed over (a kernel that writes fills this one)."""
+    want = carried_dtype(x_dtype)
+    t = t if (t.dtype == want and t.is_contiguous()) else t.to(want).contiguous()
+    setattr(p, field + "_lp" if want == torch.bfloat16 else field, t.data_ptr())
+    return t
 
 
 def f32c(t):

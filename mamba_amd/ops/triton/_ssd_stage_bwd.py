@@ -40,8 +40,8 @@ def chunk_state_bwd(B, x, dt, dA_cumsum, dstates):
     _lib.require_gpu(B, x, dt, dA_cumsum, dstates)
     dev, f32 = x.device, dict(device=x.device, dtype=torch.float32)
     xr, Br = _rows(x), _rows(B.to(x.dtype))
-    dtf, daf, dS = st.f32c(dt), st.f32c(dA_cumsum), st.f32c(dstates)
-    zeros_states = torch.zeros(batch, nchunks, nheads, headdim, dstate, **f32)
+    dtf, daf = st.f32c(dt), st.f32c(dA_cumsum)
+    zeros_states = torch.zeros(batch, nchunks, nheads, headdim, dstate, device=dev, dtype=st.carried_dtype(x.dtype))
     zeros_cb = torch.zeros(batch, nchunks, ngroups, Q, Q, **f32)
     acc = torch.zeros(2 * batch * nheads * nchunks * Q + 2 * batch * seqlen * ngroups * dstate, **f32)
     nrow, nbc = batch * nheads * nchunks * Q, batch * seqlen * ngroups * dstate
@@ -53,7 +53,8 @@ def chunk_state_bwd(B, x, dt, dA_cumsum, dstates):
     _common(p, xr, Br, Br, dtf, daf)
     p.dout = xr.data_ptr()  # stands in for g: it only meets the zero C B^T and the zero states
     p.dout_bs, p.dout_ls, p.dout_hs = xr.stride(0), xr.stride(1), xr.stride(2)
-    p.states, p.CB, p.dstates = zeros_states.data_ptr(), zeros_cb.data_ptr(), dS.data_ptr()
+    p.CB = zeros_cb.data_ptr()
+    _kept = (st.set_carried(p, "states", zeros_states, x.dtype), st.set_carried(p, "dstates", dstates, x.dtype))
     p.ddA_cumsum, p.ddt_out, p.dB32, p.dC32 = ddA.data_ptr(), ddt_out.data_ptr(), dB32.data_ptr(), dC32.data_ptr()
     p.dx = dx.data_ptr()
     p.dx_bs, p.dx_ls, p.dx_hs = dx.stride(0), dx.stride(1), dx.stride(2)
@@ -77,7 +78,7 @@ def chunk_scan_bwd(B, C, x, dt, dA_cumsum, prev_states, D, z, y, dout):
     xr, Br, Cr = _rows(x), _rows(B.to(x.dtype)), _rows(C.to(x.dtype))
     zr = _rows(z.to(x.dtype)) if z is not None else None
     dor, yr = _rows(dout.to(x.dtype)), _rows(y.to(x.dtype))
-    dtf, daf, Hc = st.f32c(dt), st.f32c(dA_cumsum), st.f32c(prev_states)
+    dtf, daf = st.f32c(dt), st.f32c(dA_cumsum)
     Df = st.f32c(D) if D is not None else None
     CB = _bmm_chunk_fwd(Cr, Br, Q, causal=True, output_dtype=torch.float32)
     nrow, nbc, ncb = batch * nheads * nchunks * Q, batch * seqlen * ngroups * dstate, batch * nchunks * ngroups * Q * Q
@@ -87,7 +88,7 @@ def chunk_scan_bwd(B, C, x, dt, dA_cumsum, prev_states, D, z, y, dout):
     dB32, dC32 = acc[2 * nrow:2 * nrow + nbc], acc[2 * nrow + nbc:2 * nrow + 2 * nbc]
     dCB = acc[2 * nrow + 2 * nbc:2 * nrow + 2 * nbc + ncb]
     dD = acc[2 * nrow + 2 * nbc + ncb:] if nD else None
-    dprev = torch.empty(batch, nchunks, nheads, headdim, dstate, **f32)
+    dprev = torch.empty(batch, nchunks, nheads, headdim, dstate, device=dev, dtype=st.carried_dtype(x.dtype))
     zeros_states = torch.zeros_like(dprev)
     dx = torch.empty(batch, seqlen, nheads, headdim, device=dev, dtype=x.dtype)
     dz = torch.empty_like(dx) if zr is not None else None
@@ -105,15 +106,16 @@ def chunk_scan_bwd(B, C, x, dt, dA_cumsum, prev_states, D, z, y, dout):
     p.out_bs, p.out_ls, p.out_hs = yr.stride(0), yr.stride(1), yr.stride(2)
     p.dout = dor.data_ptr()
     p.dout_bs, p.dout_ls, p.dout_hs = dor.stride(0), dor.stride(1), dor.stride(2)
-    p.states, p.CB = Hc.data_ptr(), CB.data_ptr()
+    p.CB = CB.data_ptr()
+    _Hc = st.set_carried(p, "states", prev_states, x.dtype)
     p.ddA_cumsum, p.ddt_out, p.dB32, p.dC32, p.dCB = (t.data_ptr() for t in (ddA, ddt_out, dB32, dC32, dCB))
     p.dD = _lib.ptr(dD)
     p.dx, p.dz, p.gbuf = dx.data_ptr(), _lib.ptr(dz), _lib.ptr(gbuf)
     p.dx_bs, p.dx_ls, p.dx_hs = dx.stride(0), dx.stride(1), dx.stride(2)
-    p.dstates = dprev.data_ptr()
+    st.set_carried(p, "dstates", dprev, x.dtype)
     st.run("ssd_bwd_dz", p, dev)
     st.run("ssd_bwd_dstates", p, dev)          # the direct gradient of the state entering each chunk
-    p.dstates = zeros_states.data_ptr()        # no chunk-state path in this function
+    st.set_carried(p, "dstates", zeros_states, x.dtype)  # no chunk-state path in this function
     for stage in ("ssd_bwd_dBC_state", "ssd_bwd_dx", "ssd_bwd_dcb", "ssd_bmm_chunk_bwd"):
         st.run(stage, p, dev)
     shape = (batch, nheads, nchunks, Q)

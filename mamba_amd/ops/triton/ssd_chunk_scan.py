@@ -41,7 +41,7 @@ def _chunk_scan_fwd(cb, x, dt, dA_cumsum, C, states, D=None, z=None, seq_idx=Non
     if z is not None:
         z = z.to(x.dtype)
         z = z if z.stride(-1) == 1 else z.contiguous()
-    cb, dt, dA_cumsum, states = st.f32c(cb), st.f32c(dt), st.f32c(dA_cumsum), st.f32c(states)
+    cb, dt, dA_cumsum = st.f32c(cb), st.f32c(dt), st.f32c(dA_cumsum)
     D = st.f32c(D) if D is not None else None
     seq_idx = st.seq_idx_i32(seq_idx)
     out = torch.empty(batch, seqlen, nheads, headdim, device=x.device, dtype=x.dtype)
@@ -54,7 +54,8 @@ def _chunk_scan_fwd(cb, x, dt, dA_cumsum, C, states, D=None, z=None, seq_idx=Non
     p.C_bs, p.C_ls, p.C_gs = C.stride(0), C.stride(1), C.stride(2)
     if z is not None:
         p.z_bs, p.z_ls, p.z_hs = z.stride(0), z.stride(1), z.stride(2)
-    p.CB, p.dt_out, p.dA_cumsum, p.states = cb.data_ptr(), dt.data_ptr(), dA_cumsum.data_ptr(), states.data_ptr()
+    p.CB, p.dt_out, p.dA_cumsum = cb.data_ptr(), dt.data_ptr(), dA_cumsum.data_ptr()
+    _states = st.set_carried(p, "states", states, x.dtype)
     p.out, p.out_x = out.data_ptr(), _lib.ptr(out_x)
     p.out_bs, p.out_ls, p.out_hs = out.stride(0), out.stride(1), out.stride(2)
     st.run("ssd_chunk_scan_fwd", p, x.device)

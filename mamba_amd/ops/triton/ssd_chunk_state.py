@@ -129,7 +129,7 @@ def chunk_state_varlen(B, x, dt, dA_cumsum, cu_seqlens, chunk_states):
     x = x if x.stride(-1) == 1 else x.contiguous()
     B = B.to(x.dtype)
     B = B if B.stride(-1) == 1 else B.contiguous()
-    dt, dA_cumsum, entering = st.f32c(dt), st.f32c(dA_cumsum), st.f32c(chunk_states)
+    dt, dA_cumsum = st.f32c(dt), st.f32c(dA_cumsum)
     cu = cu_seqlens.to(torch.int32).contiguous()
     out = torch.empty(nseq, nheads, headdim, dstate, device=x.device, dtype=torch.float32)
     p, _keep = st.stage_params(x.device, batch=1, seqlen=total_seqlen, nheads=nheads, headdim=headdim, dstate=dstate,
@@ -137,7 +137,8 @@ def chunk_state_varlen(B, x, dt, dA_cumsum, cu_seqlens, chunk_states):
     p.x, p.B = x.data_ptr(), B.data_ptr()
     p.x_ls, p.x_hs = x.stride(0), x.stride(1)
     p.B_ls, p.B_gs = B.stride(0), B.stride(1)
-    p.dt_out, p.dA_cumsum, p.states = dt.data_ptr(), dA_cumsum.data_ptr(), entering.data_ptr()
+    p.dt_out, p.dA_cumsum = dt.data_ptr(), dA_cumsum.data_ptr()
+    _entering = st.set_carried(p, "states", chunk_states.unsqueeze(0), x.dtype)
     with torch.cuda.device(x.device):
         _lib.check(_lib.load().ssd_chunk_state_varlen(p, cu.data_ptr(), nseq, out.data_ptr(),
                                                       _lib.current_stream(x.device)), "ssd_chunk_state_varlen")

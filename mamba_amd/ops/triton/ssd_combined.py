@@ -29,7 +29,8 @@ def _fill_fwd(p, x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, seq_
     p.D, p.z, p.dt_bias = _lib.ptr(D), _lib.ptr(z), _lib.ptr(dt_bias)
     p.initial_states, p.seq_idx = _lib.ptr(initial_states), _lib.ptr(seq_idx)
     p.dt_out, p.dA_cumsum = ws["dt_out"].data_ptr(), ws["dA_cumsum"].data_ptr()
-    p.states, p.final_states, p.CB = ws["states"].data_ptr(), ws["final_states"].data_ptr(), ws["CB"].data_ptr()
+    p.states, p.final_states, p.CB = _lib.ptr(ws["states"]), ws["final_states"].data_ptr(), ws["CB"].data_ptr()
+    p.states_lp = _lib.ptr(ws["states_lp"])
     p.x_bs, p.x_ls, p.x_hs = x.stride(0), x.stride(1), x.stride(2)
     if z is not None:
         p.z_bs, p.z_ls, p.z_hs = z.stride(0), z.stride(1), z.stride(2)
@@ -83,26 +84,37 @@ def _prepare(x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, seq_idx)
 
 
 def _workspace(x, B, chunk_size, forward_state=None):
-    """fp32 workspaces of the forward stages; forward_state = (dt_out, dA_cumsum, states) re-uses the
-    ones a forward pass has filled."""
+    """Workspaces of the forward stages.  `states` (fp32) receives the chunks' own states and, for fp32 / fp16
+    operands, in place the state entering each chunk; next to bf16 operands the entering states go to `states_lp`
+    in bf16 instead (the dtype the reference hands them on in, ssd_combined.py:384-386).  `carried` names whichever
+    of the two holds the entering states.  forward_state = (dt_out, dA_cumsum, carried) re-uses what a forward
+    pass has filled; `states` is then only allocated when the stages that fill it are run again."""
     batch, seqlen, nheads, headdim = x.shape
     ngroups, dstate = B.shape[2], B.shape[3]
     nchunks = math.ceil(seqlen / chunk_size)
     f32 = dict(device=x.device, dtype=torch.float32)
+    lp = x.dtype == torch.bfloat16
+    shape = (batch, nchunks, nheads, headdim, dstate)
     if forward_state is not None:
-        dt_out, dA_cumsum, states = forward_state
+        dt_out, dA_cumsum, carried = forward_state
         assert dt_out.shape == (batch, nheads, nchunks, chunk_size) and dA_cumsum.shape == dt_out.shape
-        assert states.shape == (batch, nchunks, nheads, headdim, dstate)
-        assert all(t.dtype == torch.float32 and t.is_contiguous() for t in forward_state)
+        assert carried.shape == shape and carried.is_contiguous()
+        assert carried.dtype == (torch.bfloat16 if lp else torch.float32)
+        assert all(t.dtype == torch.float32 and t.is_contiguous() for t in (dt_out, dA_cumsum))
+        states = None if lp else carried
+        states_lp = carried if lp else None
     else:
         dt_out = torch.empty(batch, nheads, nchunks, chunk_size, **f32)
         dA_cumsum = torch.empty(batch, nheads, nchunks, chunk_size, **f32)
-        states = torch.empty(batch, nchunks, nheads, headdim, dstate, **f32)
+        states = torch.empty(shape, **f32)
+        states_lp = torch.empty(shape, device=x.device, dtype=torch.bfloat16) if lp else None
     return dict(
         nchunks=nchunks,
         dt_out=dt_out,
         dA_cumsum=dA_cumsum,
         states=states,
+        states_lp=states_lp,
+        carried=states_lp if lp else states,
         final_states=torch.empty(batch, nheads, headdim, dstate, **f32),
         CB=torch.empty(batch, nchunks, ngroups, chunk_size, chunk_size, **f32),
     )
@@ -112,7 +124,8 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
                                    seq_idx=None, cu_seqlens=None, dt_softplus=False, dt_limit=(0.0, float("inf")),
                                    state_dtype=None):
     """Counterpart of ssd_combined.py:343.  Returns (out, out_x, dt_out, dA_cumsum, states, final_states)
-    where `states[:, c]` is the state entering chunk c, in fp32; with cu_seqlens a seventh element,
+    where `states[:, c]` is the state entering chunk c (bf16 next to bf16 operands, else fp32); with cu_seqlens a
+    seventh element,
     varlen_states (nseq, nheads, headdim, dstate): the state at the end of every packed sequence
     (ssd_combined.py:390-394), in state_dtype, else C's dtype, as the reference returns it."""
     state_out_dtype = state_dtype if state_dtype is not None else C.dtype
@@ -137,9 +150,9 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
             varlen = torch.empty(nseq, x.shape[2], x.shape[3], B.shape[3], device=x.device, dtype=torch.float32)
             _lib.check(_lib.load().ssd_chunk_state_varlen(p, cu_seqlens.data_ptr(), nseq, varlen.data_ptr(),
                                                           _lib.current_stream(x.device)), "ssd_chunk_state_varlen")
-            return (out, out_x, ws["dt_out"], ws["dA_cumsum"], ws["states"], ws["final_states"],
+            return (out, out_x, ws["dt_out"], ws["dA_cumsum"], ws["carried"], ws["final_states"],
                     varlen.to(state_out_dtype))
-    return out, out_x, ws["dt_out"], ws["dA_cumsum"], ws["states"], ws["final_states"]
+    return out, out_x, ws["dt_out"], ws["dA_cumsum"], ws["carried"], ws["final_states"]
 
 
 def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None, z=None, dt_bias=None,
@@ -187,7 +200,8 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
     for k, n in sizes.items():
         acc[k] = arena[off:off + n]
         off += n
-    dstates = torch.empty(batch, nchunks, nheads, headdim, dstate, **f32)
+    lp = x.dtype == torch.bfloat16  # the carried states' gradients pass between the stages in bf16 too
+    dstates = torch.empty(batch, nchunks, nheads, headdim, dstate, device=dev, dtype=torch.bfloat16 if lp else torch.float32)
     dinit = torch.empty(batch, nheads, headdim, dstate, **f32) if initial_states is not None else None
     dfinal = dfinal_states.float().contiguous() if dfinal_states is not None else None
 
@@ -204,7 +218,11 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
     p.dx_bs, p.dx_ls, p.dx_hs = dx.stride(0), dx.stride(1), dx.stride(2)
     p.dA, p.ddt_bias = acc["dA"].data_ptr(), acc["ddt_bias"].data_ptr()
     p.dD = acc["dD"].data_ptr() if D is not None else None
-    p.dinitial_states, p.dstates = _lib.ptr(dinit), dstates.data_ptr()
+    p.dinitial_states = _lib.ptr(dinit)
+    if lp:
+        p.dstates_lp = dstates.data_ptr()
+    else:
+        p.dstates = dstates.data_ptr()
     p.ddA_cumsum, p.ddt_out, p.dCB = acc["ddA_cumsum"].data_ptr(), acc["ddt_out"].data_ptr(), acc["dCB"].data_ptr()
     p.dB32, p.dC32 = acc["dB32"].data_ptr(), acc["dC32"].data_ptr()
     if use_deterministic_mode():
