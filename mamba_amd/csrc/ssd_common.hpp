@@ -417,7 +417,6 @@ DEVI void block_gemm_wide(GemmAccWide &acc, GemmLdsWide<SPLIT> &s, int k_end, SA
   block_gemm_wide<SPLIT>(acc, s, k_end, sa, sb, tid, [](int) {});
 }
 
-// Stores the wide tile as fp32 rows of dst (the tile's origin, row pitch ld); rows >= rows_valid are skipped.
 // dtype in which the states carried between chunks, and their gradients, pass between kernels: bf16 next to bf16
 // operands (the matrix products only take that part of them), fp32 otherwise.
 template <typename T> using carried_t = std::conditional_t<std::is_same_v<T, bf16_t>, bf16_t, float>;
@@ -432,6 +431,7 @@ template <typename T> DEVI carried_t<T> *carried_dstates(const SsdParams &p) {
 DEVI void st_carried(float *p, float v) { *p = v; }
 DEVI void st_carried(bf16_t *p, float v) { st1<bf16_t>(p, v); }
 
+// Stores the wide tile as rows of dst (the tile's origin, row pitch ld; fp32 or bf16); rows >= rows_valid are skipped.
 template <typename D> DEVI void store_wide(const GemmAccWide &acc, D *dst, int64_t ld, int rows_valid, int tid) {
   const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1, i = lane & 15, g = lane >> 4;
 #pragma unroll
