@@ -205,6 +205,14 @@ DEVI float softplus_f(float x) {
   return x <= 20.f ? r : x;
 }
 DEVI float sigmoid_f(float x) { return fast_rcp(1.f + fast_exp(-x)); }
+// d softplus(x) / dx = sigmoid(x), from y = softplus(x) alone: 1 - exp(-y) (= 1 / (1 + exp(-x)); above the softplus
+// threshold, where y = x, it differs from the slope 1 by less than exp(-20)).  For small y the difference is taken
+// from the series so that tiny steps keep their relative precision.
+DEVI float softplus_slope_f(float y) {
+  const float big = 1.f - fast_exp(-y);
+  const float small = y * (1.f - y * (0.5f - y * (0.16666667f - 0.041666668f * y)));
+  return y < 0.03f ? small : big;
+}
 
 // ------------------------------------------------------------------- DPP
 // dpp_ctrl encodings of the GFX9 family.

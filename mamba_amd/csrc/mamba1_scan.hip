@@ -368,17 +368,14 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
       const int d = min(d0 + chw, q.dend - 1);
       const int nvalid = valid ? min(max(L - tl, 0), KI) : 0;
       float u[8], dl[8], du[8], dy[8], acc[8], dd[8], y[8], dsum = 0.f, dtail = 0.f;
-      // raw delta, z and dout stay in registers in their storage format for the epilogue
-      const Rows cur = nxt;
-      Pack8<T> draw_k = cur.delta, z_k = cur.z, dout_k = cur.dout;
-      if (r + 1 < npass) fetch_rows(nxt, tile, r + 1);
-      else if (tile > 0) fetch_rows(nxt, tile - 1, 0);
       const float Dd = rows[chw].D, bias = rows[chw].bias;
       {
-        const Pack8<T> u_k = cur.u;
-        u_k.unpack(u);
-        draw_k.unpack(dl);
-        dout_k.unpack(dy);
+        // The rows requested during the previous step are unpacked where they were loaded, and only then are the
+        // next step's rows requested into the same registers: nothing of them has to be copied (a copy held
+        // across the loop's back edge went through scratch memory).  The epilogue reads z and dout again.
+        nxt.u.unpack(u);
+        nxt.delta.unpack(dl);
+        nxt.dout.unpack(dy);
 #pragma unroll
         for (int i = 0; i < KI; ++i) {  // lanes past the end read a clamped position: mask them
           u[i] = (i < nvalid) ? u[i] : 0.f;
@@ -386,7 +383,7 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
         }
         if (has_z) {
           float z[8];
-          z_k.unpack(z);
+          nxt.z.unpack(z);
 #pragma unroll
           for (int i = 0; i < KI; ++i) dy[i] *= z[i] * sigmoid_f(z[i]);
         }
@@ -405,7 +402,7 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
         dsum = dtail + dl[0];
         // state entering this tile (a row's own lanes write and read its slots)
         if (NBLK == 1) {
-          hcar[chl * NP + c] = c < N ? cur.ck : 0.f;
+          hcar[chl * NP + c] = c < N ? nxt.ck : 0.f;
         } else {
           for (int n = c; n < NP; n += RL) {
             float v = 0.f;
@@ -413,6 +410,8 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
             hcar[chl * NP + n] = v;
           }
         }
+        if (r + 1 < npass) fetch_rows(nxt, tile, r + 1);
+        else if (tile > 0) fetch_rows(nxt, tile - 1, 0);
       }
       for (int nb = 0; nb < NBLK; ++nb) {
         if (BC != 3 && (NBLK > 1 || r == 0)) {
@@ -594,9 +593,14 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
         }
       }
       {
-        float draw[8], o[8];
-        draw_k.unpack(draw);
+        float o[8];
         const BwdRow<T> w = rows[chw];
+        Pack8<T> z_k, dout_k;  // read again here rather than held through the state loop: they come from the caches
+        z_k.zero();
+        if (has_z) {
+          load_items<T, VEC>(z_k, w.z, tl, L, nvalid);
+          load_items<T, VEC>(dout_k, w.dout, tl, L, nvalid);
+        }
         float dbs = 0.f, dDs = 0.f;
 #pragma unroll
         for (int i = 0; i < KI; ++i) o[i] = __builtin_fmaf(dl[i], acc[i], Dd * dy[i]);
@@ -604,7 +608,7 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
 #pragma unroll
         for (int i = 0; i < KI; ++i) {
           float gd = __builtin_fmaf(u[i], acc[i], dd[i]);
-          if (p.delta_softplus) gd *= sigmoid_f(draw[i] + bias);  // (above the softplus threshold of 20 it rounds to 1)
+          if (p.delta_softplus) gd *= softplus_slope_f(dl[i]);
           gd = (i < nvalid) ? gd : 0.f;
           o[i] = gd;
           dbs += gd;
