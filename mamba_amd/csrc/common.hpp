@@ -214,6 +214,13 @@ DEVI float softplus_slope_f(float y) {
   return y < 0.03f ? small : big;
 }
 
+// Workgroup barrier for code that hands data from wave to wave through LDS only.  __syncthreads() is a fence
+// as well: it waits for every outstanding global access of the wave, stores included, so a barrier that follows a
+// burst of row stores sits through their whole write latency.  This one waits for the wave's LDS accesses alone;
+// global stores keep draining behind it.  (Nothing read through it may come from global memory written by another
+// wave of the workgroup.)
+DEVI void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // ------------------------------------------------------------------- DPP
 // dpp_ctrl encodings of the GFX9 family.
 enum : int {

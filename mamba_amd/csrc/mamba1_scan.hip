@@ -151,7 +151,7 @@ __global__ __launch_bounds__(NTHREADS, 4) void scan_fwd_kernel(const MambaScanPa
     A2s[i] = (d < q.dend && n < N) ? Ag[(int64_t)d * N + n] * kLog2e : 0.f;
     hcar[i] = 0.f;
   }
-  __syncthreads();
+  lds_barrier();
 
   for (int tile = 0; tile < q.ntiles; ++tile) {
     const int t0 = tile * TILE, tl = t0 + c * KI;
@@ -183,9 +183,9 @@ __global__ __launch_bounds__(NTHREADS, 4) void scan_fwd_kernel(const MambaScanPa
       for (int i = 0; i < KI; ++i) dsum += dl[i];
       for (int nb = 0; nb < NBLK; ++nb) {
         if (BC != 3 && (NBLK > 1 || r == 0)) {
-          __syncthreads();
+          lds_barrier();
           stage_bc<T, VEC, BC>(Bs, Cs, Bg, p.B_ns, Cg, p.C_ns, nb * NB16, N, t0, L, tid);
-          __syncthreads();
+          lds_barrier();
         }
         const float *A2row = A2s + chw * NP + nb * NB16;
         float *hrow = hcar + chw * NP + nb * NB16;
@@ -333,7 +333,7 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
     w.bias = p.delta_bias ? ((const float *)p.delta_bias)[d] : 0.f;
     rows[i] = w;
   }
-  __syncthreads();
+  lds_barrier();
 
   constexpr int NPP = NB16 / NWAVES;  // state rows per wave and phase (see the state loop)
   constexpr int NPH = NB16 / NPP;
@@ -415,11 +415,11 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
       }
       for (int nb = 0; nb < NBLK; ++nb) {
         if (BC != 3 && (NBLK > 1 || r == 0)) {
-          __syncthreads();
+          lds_barrier();
           stage_bc<T, VEC, BC>(Bs, Cs, Bg, p.B_ns, Cg, p.C_ns, nb * NB16, N, t0, L, tid);
           for (int i = tid * 4; i < 2 * ACC_FLOATS; i += NTHREADS * 4)  // dBs and dCs are adjacent
             *reinterpret_cast<f32x4 *>(dBs + i) = f32x4{0.f, 0.f, 0.f, 0.f};
-          __syncthreads();
+          lds_barrier();
         }
         {
           // The 8 waves add their channels' dB/dC terms into the shared LDS sums without atomics: between
@@ -516,7 +516,7 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
 #pragma unroll
               for (int s = 0; s < 2; ++s) gfirst[s] = __builtin_fmaf(ra[s], gc[s], rb[s]);
             }
-            if (early) __syncthreads();  // the early waves meet the others here, between the two halves
+            if (early) lds_barrier();  // the early waves meet the others here, between the two halves
             if (active) {
 #pragma unroll
               for (int s = 0; s < 2; ++s) {
@@ -559,11 +559,11 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
               }
             }
             if (ph + 1 < NPH) fetch_operands(ops, ph + 1);
-            if (!early) __syncthreads();
+            if (!early) lds_barrier();
           }
         }
         if (BC != 3 && (NBLK > 1 || r == npass - 1)) {
-          __syncthreads();  // waves 0-3 add their last sums after the last barrier of the phases
+          lds_barrier();  // waves 0-3 add their last sums after the last barrier of the phases
           // One partial per workgroup: the sum over the 4 channel slots of every (state, position), written
           // with plain stores (positions past the end and padded states are skipped).
           const int n0 = nb * NB16;
@@ -638,7 +638,7 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
       }
     }
   }
-  __syncthreads();
+  lds_barrier();
   // per-(batch, channel) partial sums; the caller reduces over batch
   for (int i = tid; i < WCH * N; i += NTHREADS) {
     const int ch = i / N, n = i % N, d = d0 + ch;
