@@ -1,20 +1,22 @@
 // SSD chunk_scan forward, fused with the C B^T contraction, for bf16 on gfx950.
 //
-// One workgroup (8 waves) computes the whole (chunk_size x headdim) output tile of one
-// (batch, chunk, head).  It is organised like a causal attention forward pass whose softmax
-// is replaced by the decay mask:
+// One workgroup (one wave per 16 positions of the chunk) computes the whole (chunk_size x headdim) output
+// tile of one (batch, chunk, head), and then that of the next head of its list: a workgroup works through
+// several heads of one group, whose C rows are the same and stay in registers, and fetches a head's first
+// blocks, carried state and scalars before the previous head's epilogue.  A tile is organised like a causal
+// attention forward pass whose softmax is replaced by the decay mask:
 //     S^T[s, l] = sum_n B[s, n] C[l, n]                       (MFMA; C rows live in registers)
 //     M^T[s, l] = S^T[s, l] * dt_s * exp(a_l - a_s)   (s <= l, same sequence)
 //     y^T[p, l] += sum_s X^T[p, s] M^T[s, l]                 (MFMA)
 // plus the carried state  y^T[p, l] += exp(a_l) sum_n H[p, n] C[l, n].
 // Working on the transposes makes the accumulator layout of the first MFMA (4 consecutive s per
 // lane for one l) equal to the B-operand layout of the second one, so M never leaves registers
-// and CB never goes to memory.  The k index of the second MFMA is permuted accordingly when X
-// is staged (transposed) into LDS.  For positions more than one 16-tile apart the decay is
+// and CB never goes to memory.  X is staged as it lies in memory (rows of positions) and the second
+// MFMA's X^T fragments, with the k order that M^T has, come out of it through the transposing LDS load.
+// For positions more than one 16-tile apart the decay is
 // factored as exp(a_l - a_end) * exp(a_end - a_s) with a_end the last a of the s tile (both
 // exponents <= 0), so the inner loop has one multiply per element instead of an exponential;
-// diagonal tiles use the exact form.  Each wave owns a balanced set of 16-row l tiles
-// (tile i paired with tile QT-1-i) so that the causal work is the same for all waves.
+// diagonal tiles use the exact form.
 #include "ssd_common.hpp"
 
 namespace {
@@ -36,16 +38,16 @@ template <int QT, int NWV> DEVI int l_tile(int w, int k) {
 // of NWV / SPLIT waves each (the pairing of tile i with tile QT-1-i keeps the workgroups balanced
 // as well).  Smaller workgroups let several of them, at different stages, share a CU.
 template <int PT, int NK, int QT, int NWV, int SPLIT>
-__global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(const SsdParams p) {
+__global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(const SsdParams p, const int hb) {
   constexpr int P = 16 * PT, N = 32 * NK, Q = 16 * QT, LT = QT / NWV, NSB = Q / 32, NWG = NWV / SPLIT, NT = 64 * NWG;
   static_assert(LT >= 1 && LT * NWV == QT, "l tiles divide evenly over the waves");
   static_assert(NWG * SPLIT == NWV, "waves divide evenly over the workgroups");
   constexpr int BP = N + 8;  // LDS pitch of a B row / H row (bf16): 16-byte aligned, bank-spread
-  constexpr int XP = 40;     // LDS pitch of an X^T row (32 k values + pad)
+  constexpr int XP = P + 16; // LDS pitch of an X row (one position, P values + pad), as it lies in memory
   constexpr int YP = P + 4;  // fp32 pitch of the epilogue's per-wave transpose patch (rows 4 banks apart)
   struct Stage {
     uint16_t Bs[2][32 * BP];
-    uint16_t Xs[2][P * XP];
+    uint16_t Xs[2][32 * XP];
     uint16_t Hs[P * BP];
   };
   union __align__(16) Shared {
@@ -59,13 +61,18 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
   __shared__ float a2_s[Q], dt_s[Q], cs_s[Q], rs_s[Q];
   __shared__ int seq_s[Q];
 
-  const int tid = threadIdx.x, lane = tid & 63;
+  int tid = threadIdx.x, lane = tid & 63;
   const int lwave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave inside this workgroup
-  const int j = lane & 15, g = lane >> 4;
+  int j = lane & 15, g = lane >> 4;
   const int H = p.nheads, G = p.ngroups, L = p.seqlen;
   // heads vary fastest over the grid: workgroups in flight together then read and write whole
   // (position, all heads) rows of x, z and out between them
-  const int h = blockIdx.x, c = blockIdx.y / SPLIT, part = blockIdx.y % SPLIT, b = blockIdx.z;
+  // A workgroup works through hb heads of one group, one after the other (their C rows are the same and stay in
+  // registers); its heads are `per` apart, so that workgroups in flight together, which sit at about the same place
+  // in their lists, touch neighbouring heads.
+  const int hpg = H / G, per = hpg / hb;
+  const int grp = blockIdx.x / per, h_first = grp * hpg + blockIdx.x % per;
+  const int c = blockIdx.y / SPLIT, part = blockIdx.y % SPLIT, b = blockIdx.z;
   const int wave = part * NWG + lwave;  // wave among the NWV that share the chunk
   // s blocks this workgroup needs: up to its last l tile
   int last_tile = 0;
@@ -73,24 +80,22 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
   for (int k = 0; k < LT; ++k)
     last_tile = max(last_tile, max(l_tile<QT, NWV>(part * NWG, k), l_tile<QT, NWV>(part * NWG + NWG - 1, k)));
   const int nsb = SPLIT == 1 ? NSB : min(NSB, (last_tile * 16 + 15) / 32 + 1);
-  const int grp = h / (H / G);
   const int t0 = c * Q;
   const int qlim = min(Q, L - t0);
-  const bf16_t *xg = static_cast<const bf16_t *>(p.x) + b * p.x_bs + h * p.x_hs;
+  const bf16_t *xg = static_cast<const bf16_t *>(p.x) + b * p.x_bs + h_first * p.x_hs;  // of the head being staged
   const bf16_t *Bg = static_cast<const bf16_t *>(p.B) + b * p.B_bs + grp * p.B_gs;
   const bf16_t *Cg = static_cast<const bf16_t *>(p.C) + b * p.C_bs + grp * p.C_gs;
   const bool has_seq = p.seq_idx != nullptr;
 
   // ---- staging helpers (global -> registers -> LDS), one s block of 32 positions
   constexpr int BCH = (32 * N / 8 + NT - 1) / NT;    // 16-byte chunks of B per thread
-  // X tasks: 4 consecutive positions x 8 consecutive p (four 16-byte loads, eight 8-byte
-  // transposed LDS stores); 8 * P / 8 tasks per block, taken by the first threads
-  constexpr int XTASKS = 8 * (P / 8);
+  // X: raw 16-byte pieces of the block's 32 rows, taken by the first threads; the second MFMA reads its
+  // X^T fragments out of these rows with the transposing LDS load
+  constexpr int XTASKS = 32 * (P / 8);
   static_assert(XTASKS <= NT, "one X task per thread at most");
-  struct XRegs { u32x4 v[4]; };
   u32x4 bregs[2][BCH];
-  XRegs xregs[2];  // two blocks in flight: global loads run two blocks ahead
-  auto load_block = [&](int sb, u32x4 (&breg)[BCH], XRegs &xreg) {
+  u32x4 xregs[2];  // two blocks in flight: global loads run two blocks ahead
+  auto load_block = [&](int sb, u32x4 (&breg)[BCH], u32x4 &xreg) {
 #pragma unroll
     for (int q = 0; q < BCH; ++q) {
       const int id = tid + q * NT, r = id / (N / 8), c8 = id % (N / 8);
@@ -99,52 +104,73 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
       if (id < 32 * N / 8 && s < qlim) breg[q] = *reinterpret_cast<const u32x4 *>(Bg + (int64_t)(t0 + s) * p.B_ls + c8 * 8);
     }
     if (tid < XTASKS) {
-      const int q4 = tid / (P / 8), p8 = tid % (P / 8);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int s = sb * 32 + q4 * 4 + e;
-        xreg.v[e] = u32x4{0, 0, 0, 0};
-        if (s < qlim) xreg.v[e] = *reinterpret_cast<const u32x4 *>(xg + (int64_t)(t0 + s) * p.x_ls + p8 * 8);
-      }
+      const int s = sb * 32 + tid / (P / 8), p8 = tid % (P / 8);
+      xreg = u32x4{0, 0, 0, 0};
+      if (s < qlim) xreg = *reinterpret_cast<const u32x4 *>(xg + (int64_t)(t0 + s) * p.x_ls + p8 * 8);
     }
   };
-  auto store_block = [&](int buf, const u32x4 (&breg)[BCH], const XRegs &xreg) {
+  auto store_block = [&](int buf, const u32x4 (&breg)[BCH], const u32x4 &xreg) {
 #pragma unroll
     for (int q = 0; q < BCH; ++q) {
       const int id = tid + q * NT, r = id / (N / 8), c8 = id % (N / 8);
       if (id < 32 * N / 8) *reinterpret_cast<u32x4 *>(&Bs[buf][r * BP + c8 * 8]) = breg[q];
     }
-    if (tid < XTASKS) {
-      const int q4 = tid / (P / 8), p8 = tid % (P / 8);
-      // k slots of positions 4 q4 .. 4 q4 + 3 inside the 32-block: the second MFMA's lane group gq
-      // holds positions 4 gq .. 4 gq + 3 of both 16-tiles.  The 8-element group is XOR-swizzled with the
-      // row's 16-tile index: the stores spread over the banks, and the 16 rows a quarter wave reads
-      // together share one swizzle, so their 16-byte pieces fall into 16 different bank groups.
-      const int pos = (((q4 & 3) ^ ((p8 >> 1) & 3)) << 3) + ((q4 >> 2) << 2);
-      const uint32_t w[4][4] = {{xreg.v[0].x, xreg.v[0].y, xreg.v[0].z, xreg.v[0].w},
-                                {xreg.v[1].x, xreg.v[1].y, xreg.v[1].z, xreg.v[1].w},
-                                {xreg.v[2].x, xreg.v[2].y, xreg.v[2].z, xreg.v[2].w},
-                                {xreg.v[3].x, xreg.v[3].y, xreg.v[3].z, xreg.v[3].w}};
-#pragma unroll
-      for (int pp = 0; pp < 8; ++pp) {  // p = p8 * 8 + pp: element pp of each of the 4 positions
-        const int d = pp >> 1;
-        uint32_t lo, hi;
-        if (pp & 1) {
-          lo = (w[0][d] >> 16) | (w[1][d] & 0xffff0000u);
-          hi = (w[2][d] >> 16) | (w[3][d] & 0xffff0000u);
-        } else {
-          lo = (w[0][d] & 0xffffu) | (w[1][d] << 16);
-          hi = (w[2][d] & 0xffffu) | (w[3][d] << 16);
-        }
-        *reinterpret_cast<u32x2 *>(&Xs[buf][(p8 * 8 + pp) * XP + pos]) = u32x2{lo, hi};
-      }
-    }
+    if (tid < XTASKS) *reinterpret_cast<u32x4 *>(&Xs[buf][(tid / (P / 8)) * XP + (tid % (P / 8)) * 8]) = xreg;
+  };
+  // X^T fragment of p tile pt: lane (j, g) gets row p = 16 pt + j and the k slots of lane group g, which are
+  // positions 4 g .. 4 g + 3 of the block's first 16-tile, then of its second: the layout in which the first
+  // MFMA leaves M^T.  Each half is one transposing load of a 4 x 16 patch.
+  auto x_frag = [&](int buf, int pt) {
+    typedef __attribute__((address_space(3))) i16x4_t *lds_ptr;
+    typedef short i16x8_t __attribute__((ext_vector_type(8)));
+    const uint16_t *src = &Xs[buf][(4 * g + (j >> 2)) * XP + pt * 16 + 4 * (j & 3)];
+    const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)src);
+    const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(src + 16 * XP));
+    return __builtin_bit_cast(bf16x8_t, (i16x8_t)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
   };
 
-  // Prologue: every global load is issued before anything waits, so the workgroup pays one
-  // memory latency: the first two s blocks, the wave's C rows, the carried state, the scalars.
-  load_block(0, bregs[0], xregs[0]);
-  if (nsb > 1) load_block(1, bregs[1], xregs[1]);
+  // carried state (bf16 in memory), rows p, k = n
+  constexpr int HCH = (P * N / 8 + NT - 1) / NT;
+  u32x4 hraw[HCH];
+  // Everything a head needs from memory before its first block: the first two s blocks, the carried state and the
+  // per-position scalars.  For the first head this is issued together with the C rows, so that the workgroup pays one
+  // memory latency; for every later head it is issued before the previous head's epilogue and arrives behind it.
+  static_assert(NT >= Q, "one position per thread");
+  float sc_a = 0.f, sc_aend = 0.f, sc_dt = 0.f;
+  bool carried_ok = false;
+  auto load_head = [&](int h) {
+    xg = static_cast<const bf16_t *>(p.x) + b * p.x_bs + h * p.x_hs;
+    load_block(0, bregs[0], xregs[0]);
+    if (nsb > 1) load_block(1, bregs[1], xregs[1]);
+    const bf16_t *Hc = static_cast<const bf16_t *>(p.states_lp) + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
+#pragma unroll
+    for (int q = 0; q < HCH; ++q) {
+      const int id = tid + q * NT;
+      hraw[q] = u32x4{0, 0, 0, 0};
+      if (id < P * N / 8) hraw[q] = *reinterpret_cast<const u32x4 *>(Hc + (int64_t)id * 8);
+    }
+    if (tid < Q) {
+      const float *dA = p.dA_cumsum + (((int64_t)b * H + h) * p.nchunks + c) * Q;
+      const float *dt = p.dt_out + (((int64_t)b * H + h) * p.nchunks + c) * Q;
+      sc_a = dA[tid];
+      sc_aend = dA[tid | 15];
+      sc_dt = dt[tid];
+    }
+  };
+  load_head(h_first);
+  // sequence ids of the chunk's positions (the same for every head), and whether the state entering the chunk
+  // belongs to the position's sequence
+  if (tid < Q) {
+    bool ok = tid < qlim;
+    int id = 0;
+    if (has_seq) {
+      const int32_t *seq = p.seq_idx + (int64_t)b * L + t0;
+      id = tid < qlim ? seq[tid] : -2;
+      ok = ok && id == (c > 0 ? seq[-1] : 0);
+    }
+    seq_s[tid] = id;
+    carried_ok = ok;
+  }
   // C rows of this wave's l tiles: B operand of both contractions (col l = j, k = n)
   bf16x8_t Cf[LT][NK];
 #pragma unroll
@@ -157,38 +183,20 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
       Cf[k][kk] = __builtin_bit_cast(bf16x8_t, v);
     }
   }
-  // carried state (bf16 in memory), rows p, k = n
-  constexpr int HCH = (P * N / 8 + NT - 1) / NT;
-  u32x4 hraw[HCH];
-  {
-    const bf16_t *Hc = static_cast<const bf16_t *>(p.states_lp) + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
-#pragma unroll
-    for (int q = 0; q < HCH; ++q) {
-      const int id = tid + q * NT;
-      hraw[q] = u32x4{0, 0, 0, 0};
-      if (id < P * N / 8) hraw[q] = *reinterpret_cast<const u32x4 *>(Hc + (int64_t)id * 8);
-    }
-  }
-  // ---- per-position scalars of this (batch, head, chunk)
-  {
-    const float *dA = p.dA_cumsum + (((int64_t)b * H + h) * p.nchunks + c) * Q;
-    const float *dt = p.dt_out + (((int64_t)b * H + h) * p.nchunks + c) * Q;
-    const int32_t *seq = has_seq ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
-    for (int s = tid; s < Q; s += NT) {
-      const float a = dA[s];
-      const float aend = dA[(s | 15)];
-      a2_s[s] = a * kLog2e;
-      dt_s[s] = dt[s];
-      cs_s[s] = dt[s] * fast_exp(aend - a);
-      bool ok = s < qlim;
-      int id = 0;
-      if (has_seq) {
-        id = s < qlim ? seq[s] : -2;
-        ok = ok && id == (c > 0 ? seq[-1] : 0);
-      }
-      seq_s[s] = id;
-      rs_s[s] = ok ? fast_exp(a) : 0.f;
-    }
+  const float *Dp = static_cast<const float *>(p.D);
+#pragma unroll 1
+  for (int hh = 0; hh < hb; ++hh) {
+  const int h = h_first + hh * per;
+  // The thread's indices pass through an empty asm once per head: to the compiler they are new values, so the
+  // addresses derived from them are computed where they are used, as in a kernel without this loop, instead of
+  // being kept in registers (or spilled) across it.
+  asm volatile("" : "+v"(tid), "+v"(lane), "+v"(j), "+v"(g));
+  // ---- per-position scalars of this (batch, head, chunk): thread s holds position s
+  if (tid < Q) {
+    a2_s[tid] = sc_a * kLog2e;
+    dt_s[tid] = sc_dt;
+    cs_s[tid] = sc_dt * fast_exp(sc_aend - sc_a);
+    rs_s[tid] = carried_ok ? fast_exp(sc_a) : 0.f;
   }
 
 #pragma unroll
@@ -197,7 +205,7 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
     if (id < P * N / 8) *reinterpret_cast<u32x4 *>(&Hs[pp * BP + c8 * 8]) = hraw[q];
   }
   store_block(0, bregs[0], xregs[0]);
-  __syncthreads();
+  lds_barrier();
 
   f32x4 acc[LT][PT];
   // ---- carried state: y^T[p, l] = rs_l * sum_n H[p, n] C[l, n]
@@ -215,7 +223,7 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
   // The epilogue's x (for D) and z rows are fetched a few blocks before the main loop ends, so
   // that their latency is covered by the remaining blocks.
   constexpr int EQ = (16 * P / 8 + 63) / 64;  // 16-byte chunks per lane of one 16 x P tile
-  const float *Dp = static_cast<const float *>(p.D);
+  const bf16_t *xe_g = static_cast<const bf16_t *>(p.x) + b * p.x_bs + h * p.x_hs;
   const bf16_t *zg = p.z ? static_cast<const bf16_t *>(p.z) + b * p.z_bs + h * p.z_hs : nullptr;
   u32x4 xe[LT][EQ], ze[LT][EQ];
   auto epilogue_prefetch = [&]() {
@@ -228,7 +236,7 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
         xe[k][q] = u32x4{0, 0, 0, 0};
         ze[k][q] = u32x4{0, 0, 0, 0};
         if (id < 16 * P / 8 && l < qlim) {
-          if (Dp) xe[k][q] = *reinterpret_cast<const u32x4 *>(xg + (int64_t)(t0 + l) * p.x_ls + c8 * 8);
+          if (Dp) xe[k][q] = *reinterpret_cast<const u32x4 *>(xe_g + (int64_t)(t0 + l) * p.x_ls + c8 * 8);
           if (zg) ze[k][q] = *reinterpret_cast<const u32x4 *>(zg + (int64_t)(t0 + l) * p.z_ls + c8 * 8);
         }
       }
@@ -284,15 +292,16 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
       const bf16x8_t Mf = __builtin_bit_cast(bf16x8_t, mp);
 #pragma unroll
       for (int pt = 0; pt < PT; ++pt)
-        acc[k][pt] = mfma_bf16(ld_frag(&Xs[buf][(pt * 16 + j) * XP + ((g ^ (pt & 3)) << 3)]), Mf, acc[k][pt]);
+        acc[k][pt] = mfma_bf16(x_frag(buf, pt), Mf, acc[k][pt]);
     }
     if (sb + 1 < nsb) store_block(buf ^ 1, bregs[(sb + 1) & 1], xregs[(sb + 1) & 1]);
-    __syncthreads();
+    lds_barrier();
   }
 
   // ---- epilogue: + D x, pre-gate copy, gate.  Each wave transposes its 16-row tiles through a
   // private LDS patch so that x / z loads and out / out_x stores are 16-byte pieces of
   // contiguous rows (the accumulator layout itself would scatter 8-byte pieces over 16 rows).
+  if (hh + 1 < hb) load_head(h + per);
   float *Ys = shm.ypatch + lwave * 16 * YP;
   bf16_t *og = static_cast<bf16_t *>(p.out) + b * p.out_bs + h * p.out_hs;
   bf16_t *oxg = p.z ? static_cast<bf16_t *>(p.out_x) + b * p.out_bs + h * p.out_hs : nullptr;
@@ -334,22 +343,48 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
   }
+  lds_barrier();  // the next head's staging overwrites the patches
+  }
 }
 
-#ifndef FUSED_SPLIT
-#define FUSED_SPLIT 1
-#endif
 bool aligned(const void *ptr, int a) { return (reinterpret_cast<uintptr_t>(ptr) % a) == 0; }
 
+int cu_count() {
+  static int cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    cached[dev] = (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) ? n : 256;
+  }
+  return cached[dev];
+}
+
+// Heads per workgroup: a divisor of the heads per group, 20 at most.  One workgroup fills a CU, so the launch runs in
+// ceil(workgroups / CUs) rounds, each as long as what a workgroup pays once (launch, arguments, C rows, the first
+// head's exposed memory latency: measured at about 0.15 of a head's work) plus its heads; the divisor with the
+// shortest estimate wins.
+int heads_per_workgroup(const SsdParams &p) {
+  const int hpg = p.nheads / p.ngroups, cus = cu_count();
+  const int64_t tiles = (int64_t)p.nchunks * p.batch;
+  int best = 1;
+  double best_cost = 1e30;
+  for (int hb = 1; hb <= 20 && hb <= hpg; ++hb) {
+    if (hpg % hb) continue;
+    const int64_t wgs = tiles * (p.nheads / hb);
+    const double cost = (double)((wgs + cus - 1) / cus) * (0.15 + hb);
+    if (cost < best_cost - 1e-9) best = hb, best_cost = cost;
+  }
+  return best;
+}
+
 template <int PT, int NK> int launch_q(const SsdParams &p, hipStream_t s) {
-  dim3 grid(p.nheads, p.nchunks, p.batch);
+  const int hb = heads_per_workgroup(p);
+  dim3 grid(p.nheads / hb, p.nchunks, p.batch);
   switch (p.chunk_size) {
-    case 256:
-      grid.y *= FUSED_SPLIT;
-      hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 16, 16, FUSED_SPLIT>), grid, dim3(1024 / FUSED_SPLIT), 0, s, p);
-      break;
-    case 128: hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 8, 8, 1>), grid, dim3(512), 0, s, p); break;
-    case 64: hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 4, 4, 1>), grid, dim3(256), 0, s, p); break;
+    case 256: hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 16, 16, 1>), grid, dim3(1024), 0, s, p, hb); break;
+    case 128: hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 8, 8, 1>), grid, dim3(512), 0, s, p, hb); break;
+    case 64: hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 4, 4, 1>), grid, dim3(256), 0, s, p, hb); break;
     default: return MAMBA_E_UNSUPPORTED;
   }
   return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
