@@ -60,6 +60,7 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
   auto &Hs = shm.st.Hs;
   __shared__ float a2_s[Q], dt_s[Q], cs_s[Q], rs_s[Q];
   __shared__ int seq_s[Q];
+  __shared__ __align__(16) float d_s[P];
 
   int tid = threadIdx.x, lane = tid & 63;
   const int lwave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave inside this workgroup
@@ -87,35 +88,41 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
   const bf16_t *Cg = static_cast<const bf16_t *>(p.C) + b * p.C_bs + grp * p.C_gs;
   const bool has_seq = p.seq_idx != nullptr;
 
-  // ---- staging helpers (global -> registers -> LDS), one s block of 32 positions
-  constexpr int BCH = (32 * N / 8 + NT - 1) / NT;    // 16-byte chunks of B per thread
-  // X: raw 16-byte pieces of the block's 32 rows, taken by the first threads; the second MFMA reads its
-  // X^T fragments out of these rows with the transposing LDS load
-  constexpr int XTASKS = 32 * (P / 8);
-  static_assert(XTASKS <= NT, "one X task per thread at most");
-  u32x4 bregs[2][BCH];
-  u32x4 xregs[2];  // two blocks in flight: global loads run two blocks ahead
-  auto load_block = [&](int sb, u32x4 (&breg)[BCH], u32x4 &xreg) {
+  // ---- staging (global -> registers -> LDS), one s block of 32 positions: the 16-byte pieces of its B rows and of
+  // its X rows (X as it lies in memory: the second MFMA reads its X^T fragments with the transposing LDS load) are
+  // one list of tasks, dealt to the threads.  Every thread issues the same number of loads whatever its task (an
+  // idle thread or a row past the end re-reads a valid piece that is dropped or zeroed at the commit): with no
+  // branch around a global load the compiler counts the loads in flight exactly, and the wait before a commit
+  // lets the loads of the blocks behind it stay in flight.
+  constexpr int TB = 32 * N / 8, TX = 32 * P / 8, TPT = (TB + TX + NT - 1) / NT;
+  u32x4 sregs[2][TPT];  // two blocks in flight: global loads run two blocks ahead
+  uint16_t *const stage0 = &shm.st.Bs[0][0];
+  static_assert(offsetof(Stage, Xs) == sizeof(uint16_t) * 2 * 32 * BP, "X tiles follow the B tiles");
+  const int64_t B_ls = p.B_ls, x_ls = p.x_ls;  // in registers: a select between them must not become a load
+  auto load_block = [&](int sb, u32x4 (&reg)[TPT]) {
 #pragma unroll
-    for (int q = 0; q < BCH; ++q) {
-      const int id = tid + q * NT, r = id / (N / 8), c8 = id % (N / 8);
-      const int s = sb * 32 + r;
-      breg[q] = u32x4{0, 0, 0, 0};
-      if (id < 32 * N / 8 && s < qlim) breg[q] = *reinterpret_cast<const u32x4 *>(Bg + (int64_t)(t0 + s) * p.B_ls + c8 * 8);
-    }
-    if (tid < XTASKS) {
-      const int s = sb * 32 + tid / (P / 8), p8 = tid % (P / 8);
-      xreg = u32x4{0, 0, 0, 0};
-      if (s < qlim) xreg = *reinterpret_cast<const u32x4 *>(xg + (int64_t)(t0 + s) * p.x_ls + p8 * 8);
+    for (int q = 0; q < TPT; ++q) {
+      const int t = tid + q * NT;
+      const bool is_b = t < TB;
+      const int u = is_b ? t : min(t - TB, TX - 1);
+      const int r = is_b ? u / (N / 8) : u / (P / 8), c8 = is_b ? u % (N / 8) : u % (P / 8);
+      const int64_t row = t0 + min(sb * 32 + r, qlim - 1);
+      const bf16_t *base = is_b ? Bg : xg;
+      reg[q] = *(const GLOBAL_AS u32x4 *)(base + row * (is_b ? B_ls : x_ls) + c8 * 8);
     }
   };
-  auto store_block = [&](int buf, const u32x4 (&breg)[BCH], const u32x4 &xreg) {
+  auto store_block = [&](int sb, int buf, const u32x4 (&reg)[TPT]) {
 #pragma unroll
-    for (int q = 0; q < BCH; ++q) {
-      const int id = tid + q * NT, r = id / (N / 8), c8 = id % (N / 8);
-      if (id < 32 * N / 8) *reinterpret_cast<u32x4 *>(&Bs[buf][r * BP + c8 * 8]) = breg[q];
+    for (int q = 0; q < TPT; ++q) {
+      const int t = tid + q * NT;
+      const bool is_b = t < TB;
+      const int u = t - (is_b ? 0 : TB);
+      const int r = is_b ? u / (N / 8) : u / (P / 8), c8 = is_b ? u % (N / 8) : u % (P / 8);
+      const bool live = sb * 32 + r < qlim;
+      const u32x4 v = {live ? reg[q].x : 0u, live ? reg[q].y : 0u, live ? reg[q].z : 0u, live ? reg[q].w : 0u};
+      const int off = is_b ? buf * 32 * BP + r * BP + c8 * 8 : 2 * 32 * BP + buf * 32 * XP + r * XP + c8 * 8;
+      if (t < TB + TX) *reinterpret_cast<u32x4 *>(stage0 + off) = v;
     }
-    if (tid < XTASKS) *reinterpret_cast<u32x4 *>(&Xs[buf][(tid / (P / 8)) * XP + (tid % (P / 8)) * 8]) = xreg;
   };
   // X^T fragment of p tile pt: lane (j, g) gets row p = 16 pt + j and the k slots of lane group g, which are
   // positions 4 g .. 4 g + 3 of the block's first 16-tile, then of its second: the layout in which the first
@@ -135,27 +142,28 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
   // Everything a head needs from memory before its first block: the first two s blocks, the carried state and the
   // per-position scalars.  For the first head this is issued together with the C rows, so that the workgroup pays one
   // memory latency; for every later head it is issued before the previous head's epilogue and arrives behind it.
-  static_assert(NT >= Q, "one position per thread");
+  static_assert(NT >= Q && NT >= P, "one position / one channel per thread");
+  const float *Dp = static_cast<const float *>(p.D);
   float sc_a = 0.f, sc_aend = 0.f, sc_dt = 0.f;
   bool carried_ok = false;
+  float sc_d = 0.f;
   auto load_head = [&](int h) {
     xg = static_cast<const bf16_t *>(p.x) + b * p.x_bs + h * p.x_hs;
-    load_block(0, bregs[0], xregs[0]);
-    if (nsb > 1) load_block(1, bregs[1], xregs[1]);
+    load_block(0, sregs[0]);
+    if (nsb > 1) load_block(1, sregs[1]);
     const bf16_t *Hc = static_cast<const bf16_t *>(p.states_lp) + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
 #pragma unroll
-    for (int q = 0; q < HCH; ++q) {
-      const int id = tid + q * NT;
-      hraw[q] = u32x4{0, 0, 0, 0};
-      if (id < P * N / 8) hraw[q] = *reinterpret_cast<const u32x4 *>(Hc + (int64_t)id * 8);
-    }
-    if (tid < Q) {
-      const float *dA = p.dA_cumsum + (((int64_t)b * H + h) * p.nchunks + c) * Q;
-      const float *dt = p.dt_out + (((int64_t)b * H + h) * p.nchunks + c) * Q;
-      sc_a = dA[tid];
-      sc_aend = dA[tid | 15];
-      sc_dt = dt[tid];
-    }
+    for (int q = 0; q < HCH; ++q)
+      hraw[q] = *(const GLOBAL_AS u32x4 *)(Hc + (int64_t)min(tid + q * NT, P * N / 8 - 1) * 8);
+    const float *dA = p.dA_cumsum + (((int64_t)b * H + h) * p.nchunks + c) * Q;
+    const float *dt = p.dt_out + (((int64_t)b * H + h) * p.nchunks + c) * Q;
+    const int pos = min(tid, Q - 1);
+    sc_a = *(const GLOBAL_AS float *)(dA + pos);
+    sc_aend = *(const GLOBAL_AS float *)(dA + (pos | 15));
+    sc_dt = *(const GLOBAL_AS float *)(dt + pos);
+    // D of channel min(tid, P - 1) of this head (0 without D); any valid address stands in when there is no D
+    const float *dsrc = Dp ? Dp + (p.D_has_hdim ? h * P + min(tid, P - 1) : h) : dA;
+    sc_d = *(const GLOBAL_AS float *)dsrc;
   };
   load_head(h_first);
   // sequence ids of the chunk's positions (the same for every head), and whether the state entering the chunk
@@ -183,7 +191,6 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
       Cf[k][kk] = __builtin_bit_cast(bf16x8_t, v);
     }
   }
-  const float *Dp = static_cast<const float *>(p.D);
 #pragma unroll 1
   for (int hh = 0; hh < hb; ++hh) {
   const int h = h_first + hh * per;
@@ -198,13 +205,14 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
     cs_s[tid] = sc_dt * fast_exp(sc_aend - sc_a);
     rs_s[tid] = carried_ok ? fast_exp(sc_a) : 0.f;
   }
+  if (tid < P) d_s[tid] = Dp ? sc_d : 0.f;
 
 #pragma unroll
   for (int q = 0; q < HCH; ++q) {
     const int id = tid + q * NT, pp = id / (N / 8), c8 = id % (N / 8);
     if (id < P * N / 8) *reinterpret_cast<u32x4 *>(&Hs[pp * BP + c8 * 8]) = hraw[q];
   }
-  store_block(0, bregs[0], xregs[0]);
+  store_block(0, 0, sregs[0]);
   lds_barrier();
 
   f32x4 acc[LT][PT];
@@ -233,12 +241,12 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
       for (int q = 0; q < EQ; ++q) {
         const int id = lane + q * 64, rr = id / (P / 8), c8 = id % (P / 8);
         const int l = l_tile<QT, NWV>(wave, k) * 16 + rr;
-        xe[k][q] = u32x4{0, 0, 0, 0};
-        ze[k][q] = u32x4{0, 0, 0, 0};
-        if (id < 16 * P / 8 && l < qlim) {
-          if (Dp) xe[k][q] = *reinterpret_cast<const u32x4 *>(xe_g + (int64_t)(t0 + l) * p.x_ls + c8 * 8);
-          if (zg) ze[k][q] = *reinterpret_cast<const u32x4 *>(zg + (int64_t)(t0 + l) * p.z_ls + c8 * 8);
-        }
+        // no branch around these loads either (rows past the end re-read the last row and are not stored;
+        // without z the x row stands in and is not used)
+        static_assert(EQ * 64 == 16 * P / 8, "whole 16-byte pieces per lane");
+        const int64_t row = t0 + min(l, qlim - 1);
+        xe[k][q] = *(const GLOBAL_AS u32x4 *)(xe_g + row * p.x_ls + c8 * 8);
+        ze[k][q] = *(const GLOBAL_AS u32x4 *)(zg ? zg + row * p.z_ls + c8 * 8 : xe_g + row * p.x_ls + c8 * 8);
       }
   };
 
@@ -248,7 +256,7 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
     const int buf = sb & 1;
     if (SPLIT > 1 && sb >= nsb) break;
     if (sb == max(nsb - 3, 0)) epilogue_prefetch();
-    if (sb + 2 < nsb) load_block(sb + 2, bregs[sb & 1], xregs[sb & 1]);
+    if (sb + 2 < nsb) load_block(sb + 2, sregs[sb & 1]);
 #pragma unroll
     for (int k = 0; k < LT; ++k) {
       const int lt = l_tile<QT, NWV>(wave, k);
@@ -294,7 +302,7 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
       for (int pt = 0; pt < PT; ++pt)
         acc[k][pt] = mfma_bf16(x_frag(buf, pt), Mf, acc[k][pt]);
     }
-    if (sb + 1 < nsb) store_block(buf ^ 1, bregs[(sb + 1) & 1], xregs[(sb + 1) & 1]);
+    if (sb + 1 < nsb) store_block(sb + 1, buf ^ 1, sregs[(sb + 1) & 1]);
     lds_barrier();
   }
 
@@ -327,7 +335,7 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
         const float xf[8] = {bf16_lo(xw.x), bf16_hi(xw.x), bf16_lo(xw.y), bf16_hi(xw.y),
                              bf16_lo(xw.z), bf16_hi(xw.z), bf16_lo(xw.w), bf16_hi(xw.w)};
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = __builtin_fmaf(p.D_has_hdim ? Dp[h * P + c8 * 8 + e] : Dp[h], xf[e], v[e]);
+        for (int e = 0; e < 8; ++e) v[e] = __builtin_fmaf(d_s[c8 * 8 + e], xf[e], v[e]);
       }
       const int64_t oi = (int64_t)(t0 + l) * p.out_ls + c8 * 8;
       if (zg) {
