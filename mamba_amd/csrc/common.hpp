@@ -185,6 +185,27 @@ template <typename T, bool VEC> DEVI void st8_guard_global(T *p, int nvalid, con
   }
 }
 
+// The same with no branch around the store on the 16-byte path: a lane with nothing to store (too few valid values, or
+// a destination that is not wanted) writes to `spare`, 32 bytes of its own that nobody reads.  A branch around a
+// store makes the compiler's count of the memory operations in flight inexact after it, and the next wait for an
+// older load then waits for the stores as well.
+template <typename T, bool VEC>
+DEVI void st8_or_spare_global(T *p, int nvalid, bool wanted, T *spare, const float (&v)[8]) {
+  if constexpr (VEC) {
+    T *dst = (wanted && nvalid >= 8) ? p : spare;
+    if constexpr (DT<T>::id == MAMBA_F32) {
+      *(GLOBAL_AS f32x4 *)dst = f32x4{v[0], v[1], v[2], v[3]};
+      *(GLOBAL_AS f32x4 *)(dst + 4) = f32x4{v[4], v[5], v[6], v[7]};
+    } else {
+      Pack8<T> k;
+      k.pack(v);
+      *(GLOBAL_AS u32x4 *)dst = k.w;
+    }
+  } else {
+    if (wanted) st8_guard<T, false>(p, nvalid, v);
+  }
+}
+
 // ------------------------------------------------------------------- math
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;

@@ -263,6 +263,10 @@ template <typename T> struct BwdRow {
   float D, bias;
 };
 
+// 32 bytes per thread that nobody reads: a lane with nothing to store (past the end of the sequence, no z)
+// stores there instead of branching around the store.  Shared by all workgroups.
+static __device__ __align__(16) float bwd_spare[NTHREADS * 8];
+
 // `passes` passes of PASS_CH channels per tile; the dB / dC sums of all of them leave once per tile as
 // partial number (workgroup's place in its group), or after every pass and block when the states come
 // in blocks of 16 (the host side then asks for one pass).
@@ -296,6 +300,7 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
   const int d0 = q.g * q.Dg + q.cb * WCH;
   const int ntiles = q.ntiles;
   const bool has_z = p.z != nullptr;
+  T *const spare = reinterpret_cast<T *>(bwd_spare + tid * 8);  // where this thread's unwanted row stores go
 
   const T *Bg = (const T *)p.B + b * p.B_bs + q.g * p.B_gs;
   const T *Cg = (const T *)p.C + b * p.C_bs + q.g * p.C_gs;
@@ -323,7 +328,7 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
     w.u = (const T *)p.u + b * p.u_bs + d * p.u_ds;
     w.delta = (const T *)p.delta + b * p.delta_bs + d * p.delta_ds;
     w.dout = (const T *)p.dout + b * p.dout_bs + d * p.dout_ds;
-    w.z = has_z ? (const T *)p.z + b * p.z_bs + d * p.z_ds : nullptr;
+    w.z = has_z ? (const T *)p.z + b * p.z_bs + d * p.z_ds : w.u;  // without z the u row stands in, read and unused
     w.du = (T *)p.du + b * p.du_bs + d * p.du_ds;
     w.ddelta = (T *)p.ddelta + b * p.ddelta_bs + d * p.ddelta_ds;
     w.dz = has_z ? (T *)p.dz + b * p.dz_bs + d * p.dz_ds : nullptr;
@@ -347,13 +352,14 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
     const BwdRow<T> &w = rows[r * PASS_CH + chl];
     const int tl = tile * TILE + c * KI;
     const int nvalid = min(max(L - tl, 0), KI);
-    k.z.zero();
-    k.ck = 0.f;
-    if (NBLK == 1 && tile > 0) k.ck = *(const GLOBAL_AS float *)(w.ckpt + (int64_t)(tile - 1) * N + min(c, N - 1));
+    // No branch around any of these loads (the checkpoint of tile 0 stands in where there is none to read, the u
+    // row where there is no z): with the same memory operations on every path through a step the compiler counts
+    // those in flight exactly, and a wait for these rows leaves the younger stores of the step before draining.
+    k.ck = *(const GLOBAL_AS float *)(w.ckpt + (int64_t)max(tile - 1, 0) * N + min(c, N - 1));
     load_items<T, VEC>(k.u, w.u, tl, L, nvalid);
     load_items<T, VEC>(k.delta, w.delta, tl, L, nvalid);
     load_items<T, VEC>(k.dout, w.dout, tl, L, nvalid);
-    if (has_z) load_items<T, VEC>(k.z, w.z, tl, L, nvalid);
+    load_items<T, VEC>(k.z, w.z, tl, L, nvalid);
   };
   int npass = 0;  // passes that hold at least one channel of the group (the same in every wave)
   while (npass < passes && d0 + npass * PASS_CH < q.dend) ++npass;
@@ -402,7 +408,7 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
         dsum = dtail + dl[0];
         // state entering this tile (a row's own lanes write and read its slots)
         if (NBLK == 1) {
-          hcar[chl * NP + c] = c < N ? nxt.ck : 0.f;
+          hcar[chl * NP + c] = (c < N && tile > 0) ? nxt.ck : 0.f;
         } else {
           for (int n = c; n < NP; n += RL) {
             float v = 0.f;
@@ -410,8 +416,10 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
             hcar[chl * NP + n] = v;
           }
         }
-        if (r + 1 < npass) fetch_rows(nxt, tile, r + 1);
-        else if (tile > 0) fetch_rows(nxt, tile - 1, 0);
+        {  // the very last step fetches tile 0 once more rather than branch around the loads
+          const bool more = r + 1 < npass;
+          fetch_rows(nxt, more ? tile : max(tile - 1, 0), more ? r + 1 : 0);
+        }
       }
       for (int nb = 0; nb < NBLK; ++nb) {
         if (BC != 3 && (NBLK > 1 || r == 0)) {
@@ -596,15 +604,12 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
         float o[8];
         const BwdRow<T> w = rows[chw];
         Pack8<T> z_k, dout_k;  // read again here rather than held through the state loop: they come from the caches
-        z_k.zero();
-        if (has_z) {
-          load_items<T, VEC>(z_k, w.z, tl, L, nvalid);
-          load_items<T, VEC>(dout_k, w.dout, tl, L, nvalid);
-        }
+        load_items<T, VEC>(z_k, w.z, tl, L, nvalid);
+        load_items<T, VEC>(dout_k, w.dout, tl, L, nvalid);
         float dbs = 0.f, dDs = 0.f;
 #pragma unroll
         for (int i = 0; i < KI; ++i) o[i] = __builtin_fmaf(dl[i], acc[i], Dd * dy[i]);
-        st8_guard_global<T, VEC>(w.du + tl, nvalid, o);
+        st8_or_spare_global<T, VEC>(w.du + tl, nvalid, true, spare, o);
 #pragma unroll
         for (int i = 0; i < KI; ++i) {
           float gd = __builtin_fmaf(u[i], acc[i], dd[i]);
@@ -614,9 +619,10 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
           dbs += gd;
           dDs = __builtin_fmaf(dy[i], u[i], dDs);
         }
-        st8_guard_global<T, VEC>(w.ddelta + tl, nvalid, o);
+        st8_or_spare_global<T, VEC>(w.ddelta + tl, nvalid, true, spare, o);
+        float oz[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         if (has_z) {
-          float z[8], dout[8], oz[8];
+          float z[8], dout[8];
           z_k.unpack(z);
           dout_k.unpack(dout);
 #pragma unroll
@@ -626,9 +632,9 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
             o[i] = dout[i] * yf * s * (1.f + z[i] * (1.f - s));
             oz[i] = yf * z[i] * s;
           }
-          st8_guard_global<T, VEC>(w.dz + tl, nvalid, o);
-          if (w.out_z) st8_guard_global<T, VEC>(w.out_z + tl, nvalid, oz);
         }
+        st8_or_spare_global<T, VEC>(w.dz + tl, nvalid, has_z, spare, o);
+        st8_or_spare_global<T, VEC>(w.out_z + tl, nvalid, w.out_z != nullptr, spare, oz);
         dbs = row_sum_to_last(dbs);
         dDs = row_sum_to_last(dDs);
         if (c == RL - 1) {
