@@ -753,7 +753,7 @@ template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256) vo
                          q.base = carried_dstates<T>(p) + (((int64_t)b * p.nchunks + c) * H + g * hpg + hs + hl * nsplit) * P * N + nt * WB;
                        },
                        P);
-  block_gemm_wide<SPLIT>(accB, lds, nh * P, sa, sb, tid);  // the first barrier inside publishes wB
+  block_gemm_wide<SPLIT, true>(accB, lds, nh * P, sa, sb, tid);  // the first barrier inside publishes wB
   const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1, i = lane & 15, gq = lane >> 4;
 #pragma unroll
   for (int tm = 0; tm < 2; ++tm)
@@ -845,7 +845,8 @@ template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256, 4)
                          q.base = carried_states<T>(p) + (((int64_t)b * p.nchunks + c) * H + g * hpg + hs + hl * nsplit) * P * N + nt * WB;
                        },
                        P);
-  block_gemm_wide<SPLIT>(acc, lds, nh * P, sa, sb, tid, [&](int k0) {  // the first barrier inside publishes wC
+  // (one pair of stagers: the kernel has no registers to spare for a second)
+  block_gemm_wide<SPLIT, false>(acc, lds, nh * P, sa, sb, tid, [&](int k0) {  // the first barrier inside publishes wC
     if ((k0 + GK) % P != 0) return;
     const int hl = k0 / P;
 #pragma unroll

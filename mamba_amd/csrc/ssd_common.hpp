@@ -374,20 +374,21 @@ template <bool SPLIT, typename S, int ROWS> struct WideTrStager {
 // acc[m][n] += sum_k A[m][k] B[n][k] over k in [0, k_end), k_end a multiple of 32.  The A stager is
 // a 64-row stager of either layout on its fast path, the B stager a 128-row WideTrStager (possibly
 // inside a SegStager).
-template <bool SPLIT, typename SA, typename SB, typename AFTER>
+template <bool SPLIT, bool RING, typename SA, typename SB, typename AFTER>
 DEVI void block_gemm_wide(GemmAccWide &acc, GemmLdsWide<SPLIT> &s, int k_end, SA &sa, SB &sb, int tid, AFTER after_step) {
   constexpr bool ATR = SA::transposed;
   const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
   const int i = lane & 15, g = lane >> 4;
-  sa.template fetch<true>(0);
-  sb.template fetch<true>(0);
-  for (int k0 = 0; k0 < k_end; k0 += GK) {
-    __syncthreads();
-    sa.template commit<true>(k0);
-    sb.template commit<true>(k0);
-    __syncthreads();
-    sa.template fetch<true>(min(k0 + GK, k_end - GK));
-    sb.template fetch<true>(min(k0 + GK, k_end - GK));
+  // One k step: commit the step's operands (fetched earlier into fa / fb) to LDS, request those of step k_next
+  // into the same registers, multiply.  The barriers wait for LDS only, so the loads requested here, and those
+  // the other pair of stagers has in flight, stay in flight across them.
+  auto step = [&](int k0, SA &fa, SB &fb, int k_next) {
+    lds_barrier();
+    fa.template commit<true>(k0);
+    fb.template commit<true>(k0);
+    lds_barrier();
+    fa.template fetch<true>(k_next);
+    fb.template fetch<true>(k_next);
     bf16x8_t a[2], b[4], al[2], bl[4];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
@@ -410,11 +411,30 @@ DEVI void block_gemm_wide(GemmAccWide &acc, GemmLdsWide<SPLIT> &s, int k_end, SA
         }
       }
     after_step(k0);
+  };
+  if (RING && !SPLIT && (k_end / GK) % 2 == 0) {
+    // Two pairs of stagers take the even and the odd steps: the operands of two steps are in flight, and a
+    // step's loads have two steps of work to arrive behind.  (Measured: the head loop of the state-path dB
+    // product gains 7 %, chunk_state loses as much to the registers, bwd_dstates is unchanged.)
+    SA sa2 = sa;
+    SB sb2 = sb;
+    sa.template fetch<true>(0);
+    sb.template fetch<true>(0);
+    sa2.template fetch<true>(GK);
+    sb2.template fetch<true>(GK);
+    for (int k0 = 0; k0 < k_end; k0 += 2 * GK) {
+      step(k0, sa, sb, min(k0 + 2 * GK, k_end - GK));
+      step(k0 + GK, sa2, sb2, min(k0 + 3 * GK, k_end - GK));
+    }
+  } else {
+    sa.template fetch<true>(0);
+    sb.template fetch<true>(0);
+    for (int k0 = 0; k0 < k_end; k0 += GK) step(k0, sa, sb, min(k0 + GK, k_end - GK));
   }
 }
-template <bool SPLIT, typename SA, typename SB>
+template <bool SPLIT, bool RING = false, typename SA, typename SB>
 DEVI void block_gemm_wide(GemmAccWide &acc, GemmLdsWide<SPLIT> &s, int k_end, SA &sa, SB &sb, int tid) {
-  block_gemm_wide<SPLIT>(acc, s, k_end, sa, sb, tid, [](int) {});
+  block_gemm_wide<SPLIT, RING>(acc, s, k_end, sa, sb, tid, [](int) {});
 }
 
 // dtype in which the states carried between chunks, and their gradients, pass between kernels: bf16 next to bf16
@@ -514,12 +534,15 @@ template <typename Inner, typename PT> struct SegStager {
   static constexpr bool transposed = Inner::transposed;
   Inner inner;
   PT point;
-  int seg_k;
-  DEVI SegStager(Inner inner_, PT point_, int seg_k_) : inner(inner_), point(point_), seg_k(seg_k_) { point(inner, 0); }
+  int seg_k, cur_seg;  // cur_seg: the segment the wrapped stager points at (the one of this object's last fetch)
+  DEVI SegStager(Inner inner_, PT point_, int seg_k_) : inner(inner_), point(point_), seg_k(seg_k_), cur_seg(0) { point(inner, 0); }
   DEVI bool fast() const { return inner.fast(); }
   template <bool FAST> DEVI void fetch(int k0) {
     const int seg = k0 / seg_k, kk = k0 - seg * seg_k;
-    if (kk == 0) point(inner, seg);
+    if (seg != cur_seg) {
+      point(inner, seg);
+      cur_seg = seg;
+    }
     inner.template fetch<FAST>(kk);
   }
   template <bool FAST> DEVI void commit(int k0) { inner.template commit<FAST>(k0 % seg_k); }
