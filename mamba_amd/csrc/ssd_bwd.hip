@@ -452,7 +452,7 @@ template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256) vo
     const T *Ba = static_cast<const T *>(p.B) + Bb + (int64_t)(t0 + st * GB) * p.B_ls;
     const carried_t<T> *dSa = dS + (int64_t)pt * GB * N;
     const bool va = rows_aligned16(Ba, p.B_ls), vb = rows_aligned16(dSa, N);
-    block_gemm_pipe<SPLIT>(
+    block_gemm_pipe<SPLIT, !SPLIT>(
         acc1, lds, 0, N,
         KcStager<SPLIT, T>(lds.ah, lds.al, Ba, p.B_ls, qlim - st * GB, N, nullptr, nullptr, va, tid),
         KcStager<SPLIT, carried_t<T>>(lds.bh, lds.bl, dSa, N, P - pt * GB, N, nullptr, nullptr, vb, tid),
@@ -468,7 +468,7 @@ template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256) vo
     const bool vb = rows_aligned16(ga, gv.ls);
     const float *CBa = CB + st * GB;  // A rows s are contiguous in the source, k = l strides by Q
     const bool va = rows_aligned16(CBa, Q);
-    block_gemm_pipe<SPLIT>(
+    block_gemm_pipe<SPLIT, !SPLIT>(
         acc2, lds, st * GB, qlim,
         // diagonal block: causal mask and the exact decay; below it CB^T with the rank-1 decays
         diag_stager<SPLIT>(fa, (st + 1) * GB,

@@ -514,15 +514,56 @@ DEVI void block_gemm_run(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, SA &s
     after_step(k0);  // e.g. to consume and clear the accumulator at segment ends
   }
 }
+// The fast path with two pairs of stagers, for an even number of steps: the pairs take the even and the odd steps,
+// so the operands of two steps are in flight and a step's loads have two steps of work to arrive behind.  The
+// barriers wait for LDS only (a barrier that also waited for the loads would put them back in step).
 template <bool SPLIT, typename SA, typename SB, typename AFTER>
+DEVI void block_gemm_run_ring(GemmAcc &acc, GemmLds &s, int k_begin, int k_last, SA &sa, SB &sb, int tid, AFTER &after_step) {
+  constexpr bool ATR = SA::transposed, BTR = SB::transposed;
+  const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+  std::remove_reference_t<SA> sa2 = sa;
+  std::remove_reference_t<SB> sb2 = sb;
+  auto step = [&](int k0, auto &fa, auto &fb) {
+    lds_barrier();
+    fa.template commit<true>(k0);
+    fb.template commit<true>(k0);
+    lds_barrier();
+    fa.template fetch<true>(min(k0 + 2 * GK, k_last));
+    fb.template fetch<true>(min(k0 + 2 * GK, k_last));
+    mma_step<SPLIT, ATR, BTR>(acc, s, wm, wn, lane);
+    after_step(k0);
+  };
+  sa.template fetch<true>(k_begin);
+  sb.template fetch<true>(k_begin);
+  sa2.template fetch<true>(k_begin + GK);
+  sb2.template fetch<true>(k_begin + GK);
+  for (int k0 = k_begin; k0 <= k_last; k0 += 2 * GK) {
+    step(k0, sa, sb);
+    step(k0 + GK, sa2, sb2);
+  }
+}
+template <bool SPLIT, bool RING, typename SA, typename SB, typename AFTER>
 DEVI void block_gemm_pipe(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, SA &&sa, SB &&sb, int tid, AFTER after_step) {
   if (k_begin >= k_end) return;
-  if (sa.fast() && sb.fast()) block_gemm_run<SPLIT, true>(acc, s, k_begin, k_end, sa, sb, tid, after_step);
-  else block_gemm_run<SPLIT, false>(acc, s, k_begin, k_end, sa, sb, tid, after_step);
+  if (sa.fast() && sb.fast()) {
+    const int k_last = k_begin + (k_end - k_begin - 1) / GK * GK;
+    if (RING && ((k_last - k_begin) / GK) % 2 == 1) block_gemm_run_ring<SPLIT>(acc, s, k_begin, k_last, sa, sb, tid, after_step);
+    else block_gemm_run<SPLIT, true>(acc, s, k_begin, k_end, sa, sb, tid, after_step);
+  } else {
+    block_gemm_run<SPLIT, false>(acc, s, k_begin, k_end, sa, sb, tid, after_step);
+  }
+}
+template <bool SPLIT, typename SA, typename SB, typename AFTER>
+DEVI void block_gemm_pipe(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, SA &&sa, SB &&sb, int tid, AFTER after_step) {
+  block_gemm_pipe<SPLIT, false>(acc, s, k_begin, k_end, sa, sb, tid, after_step);
 }
 template <bool SPLIT, typename SA, typename SB>
 DEVI void block_gemm_pipe(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, SA &&sa, SB &&sb, int tid) {
-  block_gemm_pipe<SPLIT>(acc, s, k_begin, k_end, sa, sb, tid, [](int) {});
+  block_gemm_pipe<SPLIT, false>(acc, s, k_begin, k_end, sa, sb, tid, [](int) {});
+}
+template <bool SPLIT, bool RING, typename SA, typename SB>
+DEVI void block_gemm_pipe(GemmAcc &acc, GemmLds &s, int k_begin, int k_end, SA &&sa, SB &&sb, int tid) {
+  block_gemm_pipe<SPLIT, RING>(acc, s, k_begin, k_end, sa, sb, tid, [](int) {});
 }
 
 // A k axis made of equal segments (one per head, say), each `seg_k` long (a multiple of the k step):
