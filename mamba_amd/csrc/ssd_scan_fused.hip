@@ -26,131 +26,72 @@ DEVI f32x4 mfma_bf16(bf16x8_t a, bf16x8_t b, f32x4 c) {
 }
 DEVI bf16x8_t ld_frag(const uint16_t *p) { return *reinterpret_cast<const bf16x8_t *>(p); }
 
-// l tile k (0 .. LT-1) of wave w, QT tiles in all, NWV waves
-template <int QT, int NWV> DEVI int l_tile(int w, int k) {
-  constexpr int LT = QT / NWV;
-  if (LT == 1) return w;
-  constexpr int HALF = LT / 2;
-  return k < HALF ? HALF * w + k : QT - 1 - (HALF * w + (k - HALF));
-}
-
-// NWV waves share the l tiles of one (batch, chunk, head); they are spread over SPLIT workgroups
-// of NWV / SPLIT waves each (the pairing of tile i with tile QT-1-i keeps the workgroups balanced
-// as well).  Smaller workgroups let several of them, at different stages, share a CU.
-template <int PT, int NK, int QT, int NWV, int SPLIT>
-__global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(const SsdParams p, const int hb) {
-  constexpr int P = 16 * PT, N = 32 * NK, Q = 16 * QT, LT = QT / NWV, NSB = Q / 32, NWG = NWV / SPLIT, NT = 64 * NWG;
-  static_assert(LT >= 1 && LT * NWV == QT, "l tiles divide evenly over the waves");
-  static_assert(NWG * SPLIT == NWV, "waves divide evenly over the workgroups");
-  constexpr int BP = N + 8;  // LDS pitch of a B row / H row (bf16): 16-byte aligned, bank-spread
-  constexpr int XP = P + 16; // LDS pitch of an X row (one position, P values + pad), as it lies in memory
-  constexpr int YP = P + 4;  // fp32 pitch of the epilogue's per-wave transpose patch (rows 4 banks apart)
-  struct Stage {
-    uint16_t Bs[2][32 * BP];
-    uint16_t Xs[2][32 * XP];
-    uint16_t Hs[P * BP];
+// One workgroup of QT waves; wave w owns the 16 positions l of tile w.  The chunk's B rows (the same for every head
+// of the group) are put into LDS once, a head's X rows, carried state and scalars once per head, all requested
+// before the previous head's epilogue; between the barrier that publishes them and the one before the epilogue the
+// waves run free: no staging and no barrier inside the causal loop, so that waves at different places in it keep
+// the LDS, matrix and vector pipes busy at the same time (in step, every wave read its fragments, then multiplied,
+// then masked, and each pipe idled two thirds of the time).
+template <int PT, int NK, int QT>
+__global__ __launch_bounds__(64 * QT) void chunk_scan_fwd_fused_kernel(const SsdParams p, const int hb) {
+  constexpr int P = 16 * PT, N = 32 * NK, Q = 16 * QT, NSB = Q / 32, NT = 64 * QT;
+  constexpr int BP = N + 8;   // LDS pitch of a B row / H row (bf16): 16-byte aligned, bank-spread
+  constexpr int XP = P + 16;  // LDS pitch of an X row (one position, P values + pad), as it lies in memory
+  constexpr int YP = P + 4;   // fp32 pitch of the epilogue's per-wave transpose patch (rows 4 banks apart)
+  __shared__ __align__(16) uint16_t Bs[Q * BP];  // the chunk's B rows
+  struct Head {
+    uint16_t Xs[Q * XP];  // the head's X rows
+    uint16_t Hs[P * BP];  // its carried state, rows p
   };
   union __align__(16) Shared {
-    Stage st;                       // main loop
-    float ypatch[NWG * 16 * YP];    // epilogue (the staging buffers are dead by then)
+    Head hd;                    // state product and causal loop
+    float ypatch[QT * 16 * YP]; // epilogue (X and the state are dead by then)
   };
   __shared__ Shared shm;
-  auto &Bs = shm.st.Bs;
-  auto &Xs = shm.st.Xs;
-  auto &Hs = shm.st.Hs;
+  auto &Xs = shm.hd.Xs;
+  auto &Hs = shm.hd.Hs;
   __shared__ float a2_s[Q], dt_s[Q], cs_s[Q], rs_s[Q];
   __shared__ int seq_s[Q];
   __shared__ __align__(16) float d_s[P];
 
   int tid = threadIdx.x, lane = tid & 63;
-  const int lwave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave inside this workgroup
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   int j = lane & 15, g = lane >> 4;
   const int H = p.nheads, G = p.ngroups, L = p.seqlen;
-  // heads vary fastest over the grid: workgroups in flight together then read and write whole
-  // (position, all heads) rows of x, z and out between them
-  // A workgroup works through hb heads of one group, one after the other (their C rows are the same and stay in
-  // registers); its heads are `per` apart, so that workgroups in flight together, which sit at about the same place
-  // in their lists, touch neighbouring heads.
+  // A workgroup works through hb heads of one group, one after the other; its heads are `per` apart, so that
+  // workgroups in flight together, which sit at about the same place in their lists, touch neighbouring heads.
   const int hpg = H / G, per = hpg / hb;
   const int grp = blockIdx.x / per, h_first = grp * hpg + blockIdx.x % per;
-  const int c = blockIdx.y / SPLIT, part = blockIdx.y % SPLIT, b = blockIdx.z;
-  const int wave = part * NWG + lwave;  // wave among the NWV that share the chunk
-  // s blocks this workgroup needs: up to its last l tile
-  int last_tile = 0;
-#pragma unroll
-  for (int k = 0; k < LT; ++k)
-    last_tile = max(last_tile, max(l_tile<QT, NWV>(part * NWG, k), l_tile<QT, NWV>(part * NWG + NWG - 1, k)));
-  const int nsb = SPLIT == 1 ? NSB : min(NSB, (last_tile * 16 + 15) / 32 + 1);
+  const int c = blockIdx.y, b = blockIdx.z;
+  const int lt = wave, last = lt >> 1;  // this wave's l tile; the s block that holds its diagonal
   const int t0 = c * Q;
   const int qlim = min(Q, L - t0);
-  const bf16_t *xg = static_cast<const bf16_t *>(p.x) + b * p.x_bs + h_first * p.x_hs;  // of the head being staged
   const bf16_t *Bg = static_cast<const bf16_t *>(p.B) + b * p.B_bs + grp * p.B_gs;
   const bf16_t *Cg = static_cast<const bf16_t *>(p.C) + b * p.C_bs + grp * p.C_gs;
   const bool has_seq = p.seq_idx != nullptr;
-
-  // ---- staging (global -> registers -> LDS), one s block of 32 positions: the 16-byte pieces of its B rows and of
-  // its X rows (X as it lies in memory: the second MFMA reads its X^T fragments with the transposing LDS load) are
-  // one list of tasks, dealt to the threads.  Every thread issues the same number of loads whatever its task (an
-  // idle thread or a row past the end re-reads a valid piece that is dropped or zeroed at the commit): with no
-  // branch around a global load the compiler counts the loads in flight exactly, and the wait before a commit
-  // lets the loads of the blocks behind it stay in flight.
-  constexpr int TB = 32 * N / 8, TX = 32 * P / 8, TPT = (TB + TX + NT - 1) / NT;
-  u32x4 sregs[2][TPT];  // two blocks in flight: global loads run two blocks ahead
-  uint16_t *const stage0 = &shm.st.Bs[0][0];
-  static_assert(offsetof(Stage, Xs) == sizeof(uint16_t) * 2 * 32 * BP, "X tiles follow the B tiles");
-  const int64_t B_ls = p.B_ls, x_ls = p.x_ls;  // in registers: a select between them must not become a load
-  auto load_block = [&](int sb, u32x4 (&reg)[TPT]) {
-#pragma unroll
-    for (int q = 0; q < TPT; ++q) {
-      const int t = tid + q * NT;
-      const bool is_b = t < TB;
-      const int u = is_b ? t : min(t - TB, TX - 1);
-      const int r = is_b ? u / (N / 8) : u / (P / 8), c8 = is_b ? u % (N / 8) : u % (P / 8);
-      const int64_t row = t0 + min(sb * 32 + r, qlim - 1);
-      const bf16_t *base = is_b ? Bg : xg;
-      reg[q] = *(const GLOBAL_AS u32x4 *)(base + row * (is_b ? B_ls : x_ls) + c8 * 8);
-    }
-  };
-  auto store_block = [&](int sb, int buf, const u32x4 (&reg)[TPT]) {
-#pragma unroll
-    for (int q = 0; q < TPT; ++q) {
-      const int t = tid + q * NT;
-      const bool is_b = t < TB;
-      const int u = t - (is_b ? 0 : TB);
-      const int r = is_b ? u / (N / 8) : u / (P / 8), c8 = is_b ? u % (N / 8) : u % (P / 8);
-      const bool live = sb * 32 + r < qlim;
-      const u32x4 v = {live ? reg[q].x : 0u, live ? reg[q].y : 0u, live ? reg[q].z : 0u, live ? reg[q].w : 0u};
-      const int off = is_b ? buf * 32 * BP + r * BP + c8 * 8 : 2 * 32 * BP + buf * 32 * XP + r * XP + c8 * 8;
-      if (t < TB + TX) *reinterpret_cast<u32x4 *>(stage0 + off) = v;
-    }
-  };
-  // X^T fragment of p tile pt: lane (j, g) gets row p = 16 pt + j and the k slots of lane group g, which are
-  // positions 4 g .. 4 g + 3 of the block's first 16-tile, then of its second: the layout in which the first
-  // MFMA leaves M^T.  Each half is one transposing load of a 4 x 16 patch.
-  auto x_frag = [&](int buf, int pt) {
-    typedef __attribute__((address_space(3))) i16x4_t *lds_ptr;
-    typedef short i16x8_t __attribute__((ext_vector_type(8)));
-    const uint16_t *src = &Xs[buf][(4 * g + (j >> 2)) * XP + pt * 16 + 4 * (j & 3)];
-    const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)src);
-    const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(src + 16 * XP));
-    return __builtin_bit_cast(bf16x8_t, (i16x8_t)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-  };
-
-  // carried state (bf16 in memory), rows p, k = n
-  constexpr int HCH = (P * N / 8 + NT - 1) / NT;
-  u32x4 hraw[HCH];
-  // Everything a head needs from memory before its first block: the first two s blocks, the carried state and the
-  // per-position scalars.  For the first head this is issued together with the C rows, so that the workgroup pays one
-  // memory latency; for every later head it is issued before the previous head's epilogue and arrives behind it.
-  static_assert(NT >= Q && NT >= P, "one position / one channel per thread");
+  const bool has_z = p.z != nullptr;
   const float *Dp = static_cast<const float *>(p.D);
-  float sc_a = 0.f, sc_aend = 0.f, sc_dt = 0.f;
+
+  // ---- global -> registers -> LDS in 16-byte pieces, every piece of a tensor dealt to a thread: no thread is idle
+  // and no branch surrounds a load (rows past the end of the sequence re-read its last row and are zeroed at the
+  // commit), so the compiler's count of the loads in flight is exact.
+  constexpr int BCH = Q * N / 8 / NT, XCH = Q * P / 8 / NT;
+  static_assert(BCH * NT * 8 == Q * N && XCH * NT * 8 == Q * P, "whole pieces per thread");
+  constexpr int HCH = (P * N / 8 + NT - 1) / NT;
+  static_assert(NT >= Q && NT >= P, "one position / one channel per thread");
+  u32x4 xregs[XCH], hraw[HCH];
+  float sc_a = 0.f, sc_aend = 0.f, sc_dt = 0.f, sc_d = 0.f;
   bool carried_ok = false;
-  float sc_d = 0.f;
+  // Everything a head needs from memory: its X rows, the carried state, the per-position scalars, D.  For the
+  // first head this is requested together with the B and C rows; for every later head as soon as a wave has left
+  // the previous head's causal loop, and it arrives behind the epilogue.
   auto load_head = [&](int h) {
-    xg = static_cast<const bf16_t *>(p.x) + b * p.x_bs + h * p.x_hs;
-    load_block(0, sregs[0]);
-    if (nsb > 1) load_block(1, sregs[1]);
+    const bf16_t *xg = static_cast<const bf16_t *>(p.x) + b * p.x_bs + h * p.x_hs;
+#pragma unroll
+    for (int q = 0; q < XCH; ++q) {
+      const int id = tid + q * NT, r = id / (P / 8), c8 = id % (P / 8);
+      xregs[q] = *(const GLOBAL_AS u32x4 *)(xg + (int64_t)(t0 + min(r, qlim - 1)) * p.x_ls + c8 * 8);
+    }
     const bf16_t *Hc = static_cast<const bf16_t *>(p.states_lp) + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
 #pragma unroll
     for (int q = 0; q < HCH; ++q)
@@ -165,102 +106,124 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
     const float *dsrc = Dp ? Dp + (p.D_has_hdim ? h * P + min(tid, P - 1) : h) : dA;
     sc_d = *(const GLOBAL_AS float *)dsrc;
   };
+  auto commit_head = [&]() {
+#pragma unroll
+    for (int q = 0; q < XCH; ++q) {
+      const int id = tid + q * NT, r = id / (P / 8), c8 = id % (P / 8);
+      const bool live = r < qlim;
+      const u32x4 v = {live ? xregs[q].x : 0u, live ? xregs[q].y : 0u, live ? xregs[q].z : 0u, live ? xregs[q].w : 0u};
+      *reinterpret_cast<u32x4 *>(&Xs[r * XP + c8 * 8]) = v;
+    }
+#pragma unroll
+    for (int q = 0; q < HCH; ++q) {
+      const int id = tid + q * NT, pp = id / (N / 8), c8 = id % (N / 8);
+      if (id < P * N / 8) *reinterpret_cast<u32x4 *>(&Hs[pp * BP + c8 * 8]) = hraw[q];
+    }
+    if (tid < Q) {
+      a2_s[tid] = sc_a * kLog2e;
+      dt_s[tid] = sc_dt;
+      cs_s[tid] = sc_dt * fast_exp(sc_aend - sc_a);
+      rs_s[tid] = carried_ok ? fast_exp(sc_a) : 0.f;
+    }
+    if (tid < P) d_s[tid] = Dp ? sc_d : 0.f;
+  };
+  // X^T fragment of p tile pt for block sb: lane (j, g) gets row p = 16 pt + j and the k slots of lane group g,
+  // which are positions 4 g .. 4 g + 3 of the block's first 16-tile, then of its second: the layout in which the
+  // first MFMA leaves M^T.  Each half is one transposing load of a 4 x 16 patch.
+  auto x_frag = [&](int sb, int pt) {
+    typedef __attribute__((address_space(3))) i16x4_t *lds_ptr;
+    typedef short i16x8_t __attribute__((ext_vector_type(8)));
+    const uint16_t *src = &Xs[(sb * 32 + 4 * g + (j >> 2)) * XP + pt * 16 + 4 * (j & 3)];
+    const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)src);
+    const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(src + 16 * XP));
+    return __builtin_bit_cast(bf16x8_t, (i16x8_t)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+  };
+
+  // ---- prologue: every global load is issued before anything waits
   load_head(h_first);
-  // sequence ids of the chunk's positions (the same for every head), and whether the state entering the chunk
-  // belongs to the position's sequence
-  if (tid < Q) {
-    bool ok = tid < qlim;
-    int id = 0;
-    if (has_seq) {
-      const int32_t *seq = p.seq_idx + (int64_t)b * L + t0;
-      id = tid < qlim ? seq[tid] : -2;
-      ok = ok && id == (c > 0 ? seq[-1] : 0);
-    }
-    seq_s[tid] = id;
-    carried_ok = ok;
-  }
-  // C rows of this wave's l tiles: B operand of both contractions (col l = j, k = n)
-  bf16x8_t Cf[LT][NK];
+  bf16x8_t Cf[NK];  // C rows of this wave's l tile: B operand of both contractions (col l = j, k = n)
+  {
+    const int l = min(lt * 16 + j, qlim - 1);  // rows past the end are never stored
 #pragma unroll
-  for (int k = 0; k < LT; ++k) {
-    const int l = l_tile<QT, NWV>(wave, k) * 16 + j;
+    for (int kk = 0; kk < NK; ++kk)
+      Cf[kk] = __builtin_bit_cast(bf16x8_t, *(const GLOBAL_AS u32x4 *)(Cg + (int64_t)(t0 + l) * p.C_ls + kk * 32 + g * 8));
+  }
+  {
+    u32x4 braw[BCH];
 #pragma unroll
-    for (int kk = 0; kk < NK; ++kk) {
-      u32x4 v = {0, 0, 0, 0};
-      if (l < qlim) v = *reinterpret_cast<const u32x4 *>(Cg + (int64_t)(t0 + l) * p.C_ls + kk * 32 + g * 8);
-      Cf[k][kk] = __builtin_bit_cast(bf16x8_t, v);
+    for (int q = 0; q < BCH; ++q) {
+      const int id = tid + q * NT, r = id / (N / 8), c8 = id % (N / 8);
+      braw[q] = *(const GLOBAL_AS u32x4 *)(Bg + (int64_t)(t0 + min(r, qlim - 1)) * p.B_ls + c8 * 8);
+    }
+    // sequence ids of the chunk's positions (the same for every head), and whether the state entering the chunk
+    // belongs to the position's sequence
+    if (tid < Q) {
+      bool ok = tid < qlim;
+      int id = 0;
+      if (has_seq) {
+        const int32_t *seq = p.seq_idx + (int64_t)b * L + t0;
+        id = tid < qlim ? seq[tid] : -2;
+        ok = ok && id == (c > 0 ? seq[-1] : 0);
+      }
+      seq_s[tid] = id;
+      carried_ok = ok;
+    }
+#pragma unroll
+    for (int q = 0; q < BCH; ++q) {
+      const int id = tid + q * NT, r = id / (N / 8), c8 = id % (N / 8);
+      const bool live = r < qlim;
+      const u32x4 v = {live ? braw[q].x : 0u, live ? braw[q].y : 0u, live ? braw[q].z : 0u, live ? braw[q].w : 0u};
+      *reinterpret_cast<u32x4 *>(&Bs[r * BP + c8 * 8]) = v;
     }
   }
+
+  constexpr int EQ = 16 * P / 8 / 64;  // 16-byte pieces per lane of one 16 x P tile
+  static_assert(EQ * 64 * 8 == 16 * P, "whole pieces per lane");
+  float *Ys = shm.ypatch + wave * 16 * YP;
+
 #pragma unroll 1
   for (int hh = 0; hh < hb; ++hh) {
-  const int h = h_first + hh * per;
-  // The thread's indices pass through an empty asm once per head: to the compiler they are new values, so the
-  // addresses derived from them are computed where they are used, as in a kernel without this loop, instead of
-  // being kept in registers (or spilled) across it.
-  asm volatile("" : "+v"(tid), "+v"(lane), "+v"(j), "+v"(g));
-  // ---- per-position scalars of this (batch, head, chunk): thread s holds position s
-  if (tid < Q) {
-    a2_s[tid] = sc_a * kLog2e;
-    dt_s[tid] = sc_dt;
-    cs_s[tid] = sc_dt * fast_exp(sc_aend - sc_a);
-    rs_s[tid] = carried_ok ? fast_exp(sc_a) : 0.f;
-  }
-  if (tid < P) d_s[tid] = Dp ? sc_d : 0.f;
+    const int h = h_first + hh * per;
+    // The thread's indices pass through an empty asm once per head: to the compiler they are new values, so the
+    // addresses derived from them are computed where they are used, as in a kernel without this loop, instead of
+    // being kept in registers (or spilled) across it.
+    asm volatile("" : "+v"(tid), "+v"(lane), "+v"(j), "+v"(g));
+    commit_head();
+    lds_barrier();
 
+    f32x4 acc[PT];
+    // ---- carried state: y^T[p, l] = rs_l * sum_n H[p, n] C[l, n]
+    {
+      const float rs = rs_s[lt * 16 + j];
 #pragma unroll
-  for (int q = 0; q < HCH; ++q) {
-    const int id = tid + q * NT, pp = id / (N / 8), c8 = id % (N / 8);
-    if (id < P * N / 8) *reinterpret_cast<u32x4 *>(&Hs[pp * BP + c8 * 8]) = hraw[q];
-  }
-  store_block(0, 0, sregs[0]);
-  lds_barrier();
-
-  f32x4 acc[LT][PT];
-  // ---- carried state: y^T[p, l] = rs_l * sum_n H[p, n] C[l, n]
+      for (int pt = 0; pt < PT; ++pt) {
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int k = 0; k < LT; ++k) {
-#pragma unroll
-    for (int pt = 0; pt < PT; ++pt) {
-      f32x4 v = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int kk = 0; kk < NK; ++kk) v = mfma_bf16(ld_frag(&Hs[(pt * 16 + j) * BP + kk * 32 + g * 8]), Cf[k][kk], v);
-      acc[k][pt] = v * rs_s[l_tile<QT, NWV>(wave, k) * 16 + j];
+        for (int kk = 0; kk < NK; ++kk) v = mfma_bf16(ld_frag(&Hs[(pt * 16 + j) * BP + kk * 32 + g * 8]), Cf[kk], v);
+        acc[pt] = v * rs;
+      }
     }
-  }
-
-  // The epilogue's x (for D) and z rows are fetched a few blocks before the main loop ends, so
-  // that their latency is covered by the remaining blocks.
-  constexpr int EQ = (16 * P / 8 + 63) / 64;  // 16-byte chunks per lane of one 16 x P tile
-  const bf16_t *xe_g = static_cast<const bf16_t *>(p.x) + b * p.x_bs + h * p.x_hs;
-  const bf16_t *zg = p.z ? static_cast<const bf16_t *>(p.z) + b * p.z_bs + h * p.z_hs : nullptr;
-  u32x4 xe[LT][EQ], ze[LT][EQ];
-  auto epilogue_prefetch = [&]() {
-#pragma unroll
-    for (int k = 0; k < LT; ++k)
+    // The epilogue's x (for D) and z rows are requested two blocks before the wave's last one.  No branch around
+    // these loads either (rows past the end re-read the last row and are not stored; without z the x row stands in).
+    const bf16_t *xt = static_cast<const bf16_t *>(p.x) + b * p.x_bs + h * p.x_hs + (int64_t)t0 * p.x_ls;
+    const bf16_t *zt = has_z ? static_cast<const bf16_t *>(p.z) + b * p.z_bs + h * p.z_hs + (int64_t)t0 * p.z_ls : xt;
+    const int64_t zls = has_z ? p.z_ls : p.x_ls;
+    u32x4 xe[EQ], ze[EQ];
+    auto epilogue_prefetch = [&]() {
 #pragma unroll
       for (int q = 0; q < EQ; ++q) {
         const int id = lane + q * 64, rr = id / (P / 8), c8 = id % (P / 8);
-        const int l = l_tile<QT, NWV>(wave, k) * 16 + rr;
-        // no branch around these loads either (rows past the end re-read the last row and are not stored;
-        // without z the x row stands in and is not used)
-        static_assert(EQ * 64 == 16 * P / 8, "whole 16-byte pieces per lane");
-        const int64_t row = t0 + min(l, qlim - 1);
-        xe[k][q] = *(const GLOBAL_AS u32x4 *)(xe_g + row * p.x_ls + c8 * 8);
-        ze[k][q] = *(const GLOBAL_AS u32x4 *)(zg ? zg + row * p.z_ls + c8 * 8 : xe_g + row * p.x_ls + c8 * 8);
+        const int64_t row = min(lt * 16 + rr, qlim - 1);
+        xe[q] = *(const GLOBAL_AS u32x4 *)(xt + row * p.x_ls + c8 * 8);
+        ze[q] = *(const GLOBAL_AS u32x4 *)(zt + row * zls + c8 * 8);
       }
-  };
+    };
 
-  // ---- inside the chunk
+    // ---- inside the chunk: the wave's blocks, up to the one that holds its diagonal
 #pragma unroll
-  for (int sb = 0; sb < NSB; ++sb) {
-    const int buf = sb & 1;
-    if (SPLIT > 1 && sb >= nsb) break;
-    if (sb == max(nsb - 3, 0)) epilogue_prefetch();
-    if (sb + 2 < nsb) load_block(sb + 2, sregs[sb & 1]);
-#pragma unroll
-    for (int k = 0; k < LT; ++k) {
-      const int lt = l_tile<QT, NWV>(wave, k);
-      if (lt * 16 + 15 < sb * 32) continue;  // every position of the block is after the tile
+    for (int sb = 0; sb < NSB; ++sb) {
+      if (sb > last) break;
+      if (sb == max(last - 2, 0)) epilogue_prefetch();
       const int l = lt * 16 + j;
       const float al2 = a2_s[l];
       const int lid = seq_s[l];
@@ -275,8 +238,7 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
         }
         f32x4 S = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int kk = 0; kk < NK; ++kk)
-          S = mfma_bf16(ld_frag(&Bs[buf][(h2 * 16 + j) * BP + kk * 32 + g * 8]), Cf[k][kk], S);
+        for (int kk = 0; kk < NK; ++kk) S = mfma_bf16(ld_frag(&Bs[(st * 16 + j) * BP + kk * 32 + g * 8]), Cf[kk], S);
         const int s0 = st * 16 + 4 * g;
         if (st < lt) {
           const float rl = fast_exp2(al2 - a2_s[st * 16 + 15]);
@@ -299,59 +261,52 @@ __global__ __launch_bounds__(64 * NWV / SPLIT) void chunk_scan_fwd_fused_kernel(
       const u32x4 mp = {pack_bf16(m[0], m[1]), pack_bf16(m[2], m[3]), pack_bf16(m[4], m[5]), pack_bf16(m[6], m[7])};
       const bf16x8_t Mf = __builtin_bit_cast(bf16x8_t, mp);
 #pragma unroll
-      for (int pt = 0; pt < PT; ++pt)
-        acc[k][pt] = mfma_bf16(x_frag(buf, pt), Mf, acc[k][pt]);
+      for (int pt = 0; pt < PT; ++pt) acc[pt] = mfma_bf16(x_frag(sb, pt), Mf, acc[pt]);
     }
-    if (sb + 1 < nsb) store_block(sb + 1, buf ^ 1, sregs[(sb + 1) & 1]);
-    lds_barrier();
-  }
 
-  // ---- epilogue: + D x, pre-gate copy, gate.  Each wave transposes its 16-row tiles through a
-  // private LDS patch so that x / z loads and out / out_x stores are 16-byte pieces of
-  // contiguous rows (the accumulator layout itself would scatter 8-byte pieces over 16 rows).
-  if (hh + 1 < hb) load_head(h + per);
-  float *Ys = shm.ypatch + lwave * 16 * YP;
-  bf16_t *og = static_cast<bf16_t *>(p.out) + b * p.out_bs + h * p.out_hs;
-  bf16_t *oxg = p.z ? static_cast<bf16_t *>(p.out_x) + b * p.out_bs + h * p.out_hs : nullptr;
+    // ---- the next head's operands are requested by each wave as it leaves the loop; the epilogue's patches lie
+    // over X and the state, so it starts once every wave has left
+    if (hh + 1 < hb) load_head(h + per);
+    lds_barrier();
+    // epilogue: + D x, pre-gate copy, gate.  Each wave transposes its 16 rows through a private LDS patch so that
+    // out / out_x stores are 16-byte pieces of contiguous rows (the accumulator layout itself would scatter 8-byte
+    // pieces over 16 rows).
+    {
+      const int64_t otile = b * p.out_bs + h * p.out_hs + (int64_t)(t0 + lt * 16) * p.out_ls;
+      bf16_t *og = static_cast<bf16_t *>(p.out) + otile;
+      bf16_t *oxg = has_z ? static_cast<bf16_t *>(p.out_x) + otile : nullptr;
 #pragma unroll
-  for (int k = 0; k < LT; ++k) {
-    const int ltile = l_tile<QT, NWV>(wave, k);
+      for (int pt = 0; pt < PT; ++pt) *reinterpret_cast<f32x4 *>(&Ys[j * YP + pt * 16 + 4 * g]) = acc[pt];
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-    for (int pt = 0; pt < PT; ++pt) *reinterpret_cast<f32x4 *>(&Ys[j * YP + pt * 16 + 4 * g]) = acc[k][pt];
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    // 16 rows x P/8 chunks of 8 columns
+      for (int q = 0; q < EQ; ++q) {  // 16 rows x P/8 pieces of 8 columns
+        const int id = lane + q * 64, rr = id / (P / 8), c8 = id % (P / 8);
+        if (lt * 16 + rr >= qlim) continue;
+        const f32x4 y0 = *reinterpret_cast<const f32x4 *>(&Ys[rr * YP + c8 * 8]);
+        const f32x4 y1 = *reinterpret_cast<const f32x4 *>(&Ys[rr * YP + c8 * 8 + 4]);
+        float v[8] = {y0.x, y0.y, y0.z, y0.w, y1.x, y1.y, y1.z, y1.w};
+        if (Dp) {
+          const u32x4 xw = xe[q];
+          const float xf[8] = {bf16_lo(xw.x), bf16_hi(xw.x), bf16_lo(xw.y), bf16_hi(xw.y),
+                               bf16_lo(xw.z), bf16_hi(xw.z), bf16_lo(xw.w), bf16_hi(xw.w)};
 #pragma unroll
-    for (int q = 0; q < EQ; ++q) {
-      const int id = lane + q * 64, rr = id / (P / 8), c8 = id % (P / 8);
-      const int l = ltile * 16 + rr;
-      if (id >= 16 * P / 8 || l >= qlim) continue;
-      const f32x4 y0 = *reinterpret_cast<const f32x4 *>(&Ys[rr * YP + c8 * 8]);
-      const f32x4 y1 = *reinterpret_cast<const f32x4 *>(&Ys[rr * YP + c8 * 8 + 4]);
-      float v[8] = {y0.x, y0.y, y0.z, y0.w, y1.x, y1.y, y1.z, y1.w};
-      if (Dp) {
-        const u32x4 xw = xe[k][q];
-        const float xf[8] = {bf16_lo(xw.x), bf16_hi(xw.x), bf16_lo(xw.y), bf16_hi(xw.y),
-                             bf16_lo(xw.z), bf16_hi(xw.z), bf16_lo(xw.w), bf16_hi(xw.w)};
+          for (int e = 0; e < 8; ++e) v[e] = __builtin_fmaf(d_s[c8 * 8 + e], xf[e], v[e]);
+        }
+        const int64_t oi = (int64_t)rr * p.out_ls + c8 * 8;
+        if (has_z) {
+          st8<bf16_t>(oxg + oi, v);
+          const u32x4 zw = ze[q];
+          const float zf[8] = {bf16_lo(zw.x), bf16_hi(zw.x), bf16_lo(zw.y), bf16_hi(zw.y),
+                               bf16_lo(zw.z), bf16_hi(zw.z), bf16_lo(zw.w), bf16_hi(zw.w)};
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = __builtin_fmaf(d_s[c8 * 8 + e], xf[e], v[e]);
+          for (int e = 0; e < 8; ++e) v[e] *= zf[e] * sigmoid_f(zf[e]);
+        }
+        st8<bf16_t>(og + oi, v);
       }
-      const int64_t oi = (int64_t)(t0 + l) * p.out_ls + c8 * 8;
-      if (zg) {
-        st8<bf16_t>(oxg + oi, v);
-        const u32x4 zw = ze[k][q];
-        const float zf[8] = {bf16_lo(zw.x), bf16_hi(zw.x), bf16_lo(zw.y), bf16_hi(zw.y),
-                             bf16_lo(zw.z), bf16_hi(zw.z), bf16_lo(zw.w), bf16_hi(zw.w)};
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] *= zf[e] * sigmoid_f(zf[e]);
-      }
-      st8<bf16_t>(og + oi, v);
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-  }
-  lds_barrier();  // the next head's staging overwrites the patches
+    lds_barrier();  // the next head's operands overwrite the patches
   }
 }
 
@@ -390,9 +345,9 @@ template <int PT, int NK> int launch_q(const SsdParams &p, hipStream_t s) {
   const int hb = heads_per_workgroup(p);
   dim3 grid(p.nheads / hb, p.nchunks, p.batch);
   switch (p.chunk_size) {
-    case 256: hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 16, 16, 1>), grid, dim3(1024), 0, s, p, hb); break;
-    case 128: hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 8, 8, 1>), grid, dim3(512), 0, s, p, hb); break;
-    case 64: hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 4, 4, 1>), grid, dim3(256), 0, s, p, hb); break;
+    case 256: hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 16>), grid, dim3(1024), 0, s, p, hb); break;
+    case 128: hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 8>), grid, dim3(512), 0, s, p, hb); break;
+    case 64: hipLaunchKernelGGL((chunk_scan_fwd_fused_kernel<PT, NK, 4>), grid, dim3(256), 0, s, p, hb); break;
     default: return MAMBA_E_UNSUPPORTED;
   }
   return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
