@@ -16,44 +16,10 @@
 
 namespace {
 
-struct View4 {  // (b, L, H, P) tensor, P stride 1
-  const void *ptr;
-  int64_t bs, ls, hs;
-};
-DEVI View4 g_view(const SsdParams &p) {
-  if (p.z) return {p.gbuf, (int64_t)p.seqlen * p.nheads * p.headdim, (int64_t)p.nheads * p.headdim, p.headdim};
-  return {p.dout, p.dout_bs, p.dout_ls, p.dout_hs};
-}
-
 // The heads of a group are spread over this many workgroups (each sums ~8 heads in registers and
 // adds its partial result atomically).
 __host__ __device__ inline int head_splits(int heads_per_group) { return (heads_per_group + 7) / 8; }
 
-DEVI float *chunk_row(float *base, const SsdParams &p, int b, int h, int c) {
-  return base + (((int64_t)b * p.nheads + h) * p.nchunks + c) * p.chunk_size;
-}
-DEVI int64_t chunk_off(const SsdParams &p, int b, int h, int c) {
-  return (((int64_t)b * p.nheads + h) * p.nchunks + c) * p.chunk_size;
-}
-
-// Sums that several workgroups add into one address.  Default: float atomics (the order of the adds, hence the
-// last bits of the sum, changes from run to run).  Deterministic mode (p.det_scale set): the term is scaled by a
-// power of two common to the whole call, rounded to an integer and added with a 64-bit integer atomic into the
-// shadow of the buffer; integer addition is associative, so the sum is the same in every order, and
-// det_convert_kernel turns the shadow into the float buffer before its first reader runs.
-DEVI float det_scale_of(const SsdParams &p) { return p.det_scale ? p.det_scale[0] : 0.f; }
-// MODE: -1 decides at run time from dsc (the small kernels), 0 / 1 are compiled for one form (the kernels whose inner
-// loops hold these adds: carrying both forms costs them registers and ~10 % of their time).
-template <int MODE = -1> DEVI void acc_add(float *dst, int64_t *shadow, int64_t idx, float v, float dsc) {
-  if (MODE == 1 || (MODE < 0 && dsc != 0.f)) {
-    const float q = fminf(fmaxf(v * dsc, -9.0e18f), 9.0e18f);
-    __hip_atomic_fetch_add(reinterpret_cast<unsigned long long *>(shadow + idx),
-                           static_cast<unsigned long long>(static_cast<long long>(__builtin_rintf(q))), __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
-  } else {
-    unsafeAtomicAdd(dst + idx, v);
-  }
-}
 __global__ __launch_bounds__(256) void det_convert_kernel(const int64_t *__restrict__ src, float *__restrict__ dst, int64_t n,
                                                           const float *__restrict__ scale) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -1260,6 +1226,9 @@ extern "C" int ssd_bwd_dx(const SsdParams *p, mamba_stream_t stream) {
   if (rc) return rc;
   if (p->dx_ls < (int64_t)p->headdim || p->dx_hs < (int64_t)p->headdim) return MAMBA_E_BADARG;  // strides not filled in
   hipStream_t s = static_cast<hipStream_t>(stream);
+  // bf16 on the common shapes: the fused kernel, which forms C B^T itself (p->CB is not read); else the tiled one
+  rc = ssd_bwd_dx_fused_launch(p, s);
+  if (rc != MAMBA_E_UNSUPPORTED) return rc;
   dim3 grid(tiles(p->chunk_size) * tiles(p->headdim), p->nchunks, p->batch * p->nheads);
   SSD_DISPATCH_DET(bwd_dx_kernel, grid)
   return launched();

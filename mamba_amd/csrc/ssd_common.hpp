@@ -670,3 +670,76 @@ DEVI Block3 xcd_block() {
   const int lid = xcd_linear_block();
   return {lid % nx, (lid / nx) % ny, lid / (nx * ny)};
 }
+
+// ---- pieces shared by the backward kernels
+struct View4 {  // (b, L, H, P) tensor, P stride 1
+  const void *ptr;
+  int64_t bs, ls, hs;
+};
+DEVI View4 g_view(const SsdParams &p) {
+  if (p.z) return {p.gbuf, (int64_t)p.seqlen * p.nheads * p.headdim, (int64_t)p.nheads * p.headdim, p.headdim};
+  return {p.dout, p.dout_bs, p.dout_ls, p.dout_hs};
+}
+
+
+DEVI float *chunk_row(float *base, const SsdParams &p, int b, int h, int c) {
+  return base + (((int64_t)b * p.nheads + h) * p.nchunks + c) * p.chunk_size;
+}
+DEVI int64_t chunk_off(const SsdParams &p, int b, int h, int c) {
+  return (((int64_t)b * p.nheads + h) * p.nchunks + c) * p.chunk_size;
+}
+
+// Sums that several workgroups add into one address.  Default: float atomics (the order of the adds, hence the
+// last bits of the sum, changes from run to run).  Deterministic mode (p.det_scale set): the term is scaled by a
+// power of two common to the whole call, rounded to an integer and added with a 64-bit integer atomic into the
+// shadow of the buffer; integer addition is associative, so the sum is the same in every order, and
+// det_convert_kernel turns the shadow into the float buffer before its first reader runs.
+DEVI float det_scale_of(const SsdParams &p) { return p.det_scale ? p.det_scale[0] : 0.f; }
+// MODE: -1 decides at run time from dsc (the small kernels), 0 / 1 are compiled for one form (the kernels whose inner
+// loops hold these adds: carrying both forms costs them registers and ~10 % of their time).
+template <int MODE = -1> DEVI void acc_add(float *dst, int64_t *shadow, int64_t idx, float v, float dsc) {
+  if (MODE == 1 || (MODE < 0 && dsc != 0.f)) {
+    const float q = fminf(fmaxf(v * dsc, -9.0e18f), 9.0e18f);
+    __hip_atomic_fetch_add(reinterpret_cast<unsigned long long *>(shadow + idx),
+                           static_cast<unsigned long long>(static_cast<long long>(__builtin_rintf(q))), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+  } else {
+    unsafeAtomicAdd(dst + idx, v);
+  }
+}
+
+// The fused dx kernel (ssd_dx_fused.hip): launches it and returns MAMBA_OK, or returns MAMBA_E_UNSUPPORTED when it has
+// no kernel for the problem (the caller then runs the tiled bwd_dx_kernel).
+__attribute__((visibility("hidden"))) int ssd_bwd_dx_fused_launch(const SsdParams *p, hipStream_t stream);
+
+// ---- host side of the kernels that work through the heads of a group in one workgroup
+inline bool aligned(const void *ptr, int a) { return (reinterpret_cast<uintptr_t>(ptr) % a) == 0; }
+
+inline int cu_count() {
+  static int cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    cached[dev] = (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) ? n : 256;
+  }
+  return cached[dev];
+}
+
+// Heads per workgroup: a divisor of the heads per group, 20 at most.  One workgroup fills a CU, so the launch runs in
+// ceil(workgroups / CUs) rounds, each as long as what a workgroup pays once (launch, arguments, C rows, the first
+// head's exposed memory latency: measured at about 0.15 of a head's work) plus its heads; the divisor with the
+// shortest estimate wins.
+inline int heads_per_workgroup(const SsdParams &p) {
+  const int hpg = p.nheads / p.ngroups, cus = cu_count();
+  const int64_t tiles = (int64_t)p.nchunks * p.batch;
+  int best = 1;
+  double best_cost = 1e30;
+  for (int hb = 1; hb <= 20 && hb <= hpg; ++hb) {
+    if (hpg % hb) continue;
+    const int64_t wgs = tiles * (p.nheads / hb);
+    const double cost = (double)((wgs + cus - 1) / cus) * (0.15 + hb);
+    if (cost < best_cost - 1e-9) best = hb, best_cost = cost;
+  }
+  return best;
+}

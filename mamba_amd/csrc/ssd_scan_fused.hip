@@ -310,37 +310,6 @@ __global__ __launch_bounds__(64 * QT) void chunk_scan_fwd_fused_kernel(const Ssd
   }
 }
 
-bool aligned(const void *ptr, int a) { return (reinterpret_cast<uintptr_t>(ptr) % a) == 0; }
-
-int cu_count() {
-  static int cached[64] = {};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cached[dev] == 0) {
-    int n = 0;
-    cached[dev] = (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) ? n : 256;
-  }
-  return cached[dev];
-}
-
-// Heads per workgroup: a divisor of the heads per group, 20 at most.  One workgroup fills a CU, so the launch runs in
-// ceil(workgroups / CUs) rounds, each as long as what a workgroup pays once (launch, arguments, C rows, the first
-// head's exposed memory latency: measured at about 0.15 of a head's work) plus its heads; the divisor with the
-// shortest estimate wins.
-int heads_per_workgroup(const SsdParams &p) {
-  const int hpg = p.nheads / p.ngroups, cus = cu_count();
-  const int64_t tiles = (int64_t)p.nchunks * p.batch;
-  int best = 1;
-  double best_cost = 1e30;
-  for (int hb = 1; hb <= 20 && hb <= hpg; ++hb) {
-    if (hpg % hb) continue;
-    const int64_t wgs = tiles * (p.nheads / hb);
-    const double cost = (double)((wgs + cus - 1) / cus) * (0.15 + hb);
-    if (cost < best_cost - 1e-9) best = hb, best_cost = cost;
-  }
-  return best;
-}
-
 template <int PT, int NK> int launch_q(const SsdParams &p, hipStream_t s) {
   const int hb = heads_per_workgroup(p);
   dim3 grid(p.nheads / hb, p.nchunks, p.batch);

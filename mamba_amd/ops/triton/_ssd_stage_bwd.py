@@ -5,7 +5,7 @@ ssd_chunk_scan.py:1786-1825), composed from the library's backward stage entry p
 The library cuts the backward pass differently from the reference (dx of the carried-state path and of the
 in-chunk path in one kernel; the dB / dC state products in one family), so each function below runs the
 stages it needs with the other path's operand set to zero:
-  chunk_state:  ssd_bwd_dBC_state (forward states = 0: no dC term), ssd_bwd_dx (C B^T = 0: no in-chunk term)
+  chunk_state:  ssd_bwd_dBC_state (forward states = 0: no dC term), ssd_bwd_dx (C = 0 and C B^T = 0: no in-chunk term)
   chunk_scan:   ssd_bwd_dz, ssd_bwd_dstates (-> dprev_states), then with dstates = 0: ssd_bwd_dBC_state,
                 ssd_bwd_dx, ssd_bwd_dcb, ssd_bmm_chunk_bwd
 """
@@ -50,7 +50,8 @@ def chunk_state_bwd(B, x, dt, dA_cumsum, dstates):
     dx = torch.empty(batch, seqlen, nheads, headdim, device=dev, dtype=x.dtype)
     p, _keep = st.stage_params(dev, batch=batch, seqlen=seqlen, nheads=nheads, headdim=headdim, dstate=dstate,
                                ngroups=ngroups, chunk_size=Q, dtype=x.dtype, backward=True)
-    _common(p, xr, Br, Br, dtf, daf)
+    Czero = torch.zeros_like(Br)  # C = 0: the dx stage forms C B^T itself on some shapes (kept alive to the end)
+    _common(p, xr, Br, Czero, dtf, daf)
     p.dout = xr.data_ptr()  # stands in for g: it only meets the zero C B^T and the zero states
     p.dout_bs, p.dout_ls, p.dout_hs = xr.stride(0), xr.stride(1), xr.stride(2)
     p.CB = zeros_cb.data_ptr()
