@@ -354,7 +354,9 @@ int ssd_chunk_state_varlen(const SsdParams *p, const int32_t *cu_seqlens, int ns
  *   ssd_state_passing_bwd  reverse recurrence over chunks (in place on dstates -> gradient
  *                     of the chunk-local states), dinitial_states, ddA_cumsum at chunk ends
  *   ssd_bwd_dBC_state state-path parts of dB32 / dC32
- *   ssd_bwd_dx        dx, ddt_out (direct part) and the matching ddA_cumsum terms
+ *   ssd_bwd_dx        dx, ddt_out (direct part) and the matching ddA_cumsum terms.  For bf16 with headdim
+ *                     32 / 64, dstate 64 / 128, chunk 64 / 128 / 256 and 16-byte aligned rows it forms C B^T
+ *                     itself from B and C (CB is not read); every other problem reads CB
  *   ssd_bwd_dcb       dCB
  *   ssd_bmm_chunk_bwd dB32 / dC32 += dCB contractions
  *   ssd_chunk_cumsum_bwd  ddt, dA, ddt_bias from ddA_cumsum and ddt_out
