@@ -902,8 +902,9 @@ template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256, 4)
     const int h = g * hpg + hs + hl * nsplit, par = hl & 1;
     const float *dA = chunk_row(p.dA_cumsum, p, b, h, c);
     const float *dt = chunk_row(p.dt_out, p, b, h, c);
-    if (tid < GB) hA_l[par][tid] = lt * GB + tid < Q ? dA[lt * GB + tid] : 0.f;
-    else if (tid < 2 * GB) hA_s[par][tid - GB] = st * GB + tid - GB < Q ? dA[st * GB + tid - GB] : 0.f;
+    // the exponents' rows are kept times log2(e): the decay of an element is then one v_exp_f32 of a difference
+    if (tid < GB) hA_l[par][tid] = lt * GB + tid < Q ? dA[lt * GB + tid] * kLog2e : 0.f;
+    else if (tid < 2 * GB) hA_s[par][tid - GB] = st * GB + tid - GB < Q ? dA[st * GB + tid - GB] * kLog2e : 0.f;
     else if (tid < 3 * GB) hdt[par][tid - 2 * GB] = st * GB + tid - 2 * GB < Q ? dt[st * GB + tid - 2 * GB] : 0.f;
   };
   load_rows(0);
@@ -946,8 +947,8 @@ template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256, 4)
             float rsum = 0.f;
 #pragma unroll
             for (int tn = 0; tn < 2; ++tn) {
-              float d = acc.v[tm][tn][r] * dt_s[tn] * fast_exp(fminf(a_l - a_s[tn], 0.f));
-              d = (live >> ((tm * 2 + tn) * 4 + r)) & 1 ? d : 0.f;
+              // (not masked here: cbr is zero at the masked positions, so w is, and sum is masked once at the end)
+              const float d = acc.v[tm][tn][r] * dt_s[tn] * fast_exp2(fminf(a_l - a_s[tn], 0.f));
               acc.v[tm][tn][r] = 0.f;
               sum.v[tm][tn][r] += d;
               const float w = d * cbr[tm][tn][r];
@@ -976,6 +977,13 @@ template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256, 4)
     if (lt * GB + r < Q && row != 0.f) acc_add<DET ? 1 : 0>(p.ddA_cumsum, p.det_ddA_cumsum, dda + lt * GB + r, row, det_scale_of(p));
     if (st * GB + r < Q && col != 0.f) acc_add<DET ? 1 : 0>(p.ddA_cumsum, p.det_ddA_cumsum, dda + st * GB + r, -col, det_scale_of(p));
   }
+#pragma unroll
+  for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+    for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (!((live >> ((tm * 2 + tn) * 4 + r)) & 1)) sum.v[tm][tn][r] = 0.f;  // causal / same-sequence mask
   acc_foreach(sum, tid, [&](int m, int n, float v) {
     const int l = lt * GB + m, s = st * GB + n;
     if (l < Q && s < Q && v != 0.f) acc_add<DET ? 1 : 0>(p.dCB, p.det_dCB, dCB_off + (int64_t)l * Q + s, v, det_scale_of(p));  // dCB starts zeroed
