@@ -520,10 +520,16 @@ int norm_gated_bwd(const NormGatedParams *p, mamba_stream_t stream);
  * LayerNorm / RMSNorm of (x + residual) with the sum handed on: the norm in front of every mixer
  * of the reference's Block (mamba_ssm/modules/block.py:57-66).  Replaces the Triton launches of
  * mamba_ssm/ops/triton/layer_norm.py:291 (_layer_norm_fwd) and :589 (_layer_norm_bwd) for the
- * arguments the Block uses (residual, prenorm, residual_in_fp32; no dropout, rowscale or second
- * branch).
- *   forward:  s = x + residual;  residual_out = s;  out = (s - mean) * rstd * weight + bias
- *   backward: dx = d_norm(dy) + dresidual, written as dx (dtype) and dresidual_in (res_dtype)
+ * arguments the Block uses (residual, prenorm, residual_in_fp32) and, through the optional fields at
+ * the end of the struct, for the rest of that operator (rowscale, dropout, the second input x1 and the
+ * second set of norm parameters weight1 / bias1; layer_norm.py:130-237 forward, :393-518 backward).
+ *   forward:  s = drop(x * rowscale) + drop1(x1) + residual;  residual_out = s;
+ *             out = (s - mean) * rstd * weight + bias;  out1 = (s - mean) * rstd * weight1 + bias1
+ *   backward: d = d_norm(dy, dy1) + dresidual is the gradient of s, written as dresidual_in (res_dtype);
+ *             dx = drop'(d) * rowscale and dx1 = drop1'(d) (dtype); without the optional parts dx = d
+ * drop keeps an element with probability 1 - dropout_p and scales it by 1 / (1 - dropout_p); the draw is a
+ * function of (seeds[0] for x, seeds[1] for x1; row; channel) that the backward call repeats, and the
+ * forward call writes it out as bytes (1 = kept) where mask / mask1 are given.
  * x, out, dy, dx are (rows, dim) of `dtype`; residual, residual_out, dresidual, dresidual_in of
  * `res_dtype` (equal to dtype, or fp32); unit channel stride, row strides given.  In the backward
  * call `x` is the summed input the forward call wrote (residual_out, or x itself when there was
@@ -557,6 +563,24 @@ typedef struct NormResidualParams {
   float *dw_part;
   float *db_part; /* null iff bias is null */
   int64_t dy_rs, dresidual_rs, dx_rs, dresidual_in_rs;
+  /* ---- optional parts, all null / 0 when unused ---- */
+  const void *x1;        /* (rows, dim) of dtype; not together with rowscale */
+  const float *rowscale; /* (rows) */
+  const int64_t *seeds;  /* 2 device words, required when dropout_p > 0 */
+  uint8_t *mask;         /* forward, nullable: (rows, dim) bytes, dense */
+  uint8_t *mask1;        /* forward, nullable: the same for x1 */
+  const float *weight1;  /* (dim) */
+  const float *bias1;    /* (dim), nullable */
+  void *out1;            /* forward, required with weight1 */
+  const void *dy1;       /* backward, required with weight1 */
+  void *dx1;             /* backward, required with x1 */
+  float *dweight1;       /* backward, required with weight1, like dweight */
+  float *dbias1;         /* null iff bias1 is null */
+  float *dw1_part;       /* (nparts, dim) workspaces like dw_part / db_part */
+  float *db1_part;
+  int64_t x1_rs, out1_rs, dy1_rs, dx1_rs;
+  float dropout_p;
+  int32_t reserved2;
 } NormResidualParams;
 
 int norm_residual_fwd(const NormResidualParams *p, mamba_stream_t stream);

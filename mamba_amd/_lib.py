@@ -118,6 +118,10 @@ class NormResidualParams(ctypes.Structure):
         + [(n, c_i64) for n in ("x_rs", "residual_rs", "out_rs", "residual_out_rs")]
         + [(n, c_vp) for n in ("dy", "dresidual", "dx", "dresidual_in", "dweight", "dbias", "dw_part", "db_part")]
         + [(n, c_i64) for n in ("dy_rs", "dresidual_rs", "dx_rs", "dresidual_in_rs")]
+        + [(n, c_vp) for n in ("x1", "rowscale", "seeds", "mask", "mask1", "weight1", "bias1", "out1", "dy1", "dx1",
+                               "dweight1", "dbias1", "dw1_part", "db1_part")]
+        + [(n, c_i64) for n in ("x1_rs", "out1_rs", "dy1_rs", "dx1_rs")]
+        + [("dropout_p", ctypes.c_float), ("reserved2", c_i32)]
     )
 
 
