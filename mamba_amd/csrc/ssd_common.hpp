@@ -451,17 +451,42 @@ template <typename T> DEVI carried_t<T> *carried_dstates(const SsdParams &p) {
 DEVI void st_carried(float *p, float v) { *p = v; }
 DEVI void st_carried(bf16_t *p, float v) { st1<bf16_t>(p, v); }
 
-// Stores the wide tile as rows of dst (the tile's origin, row pitch ld; fp32 or bf16); rows >= rows_valid are skipped.
-template <typename D> DEVI void store_wide(const GemmAccWide &acc, D *dst, int64_t ld, int rows_valid, int tid) {
+// Stores the wide tile as rows of dst (the tile's origin, row pitch ld; fp32 or bf16; dst 16-byte aligned, ld a
+// multiple of 8), rows >= rows_valid skipped, in whole 128-byte pieces of rows: each wave turns its 32 x 64 part
+// around through a patch of its own in the operand tiles' LDS, 16 rows by 128 bytes at a time, so that a lane
+// stores 16 contiguous bytes and eight lanes a whole line (single elements straight from the accumulator layout
+// are 32-byte runs in bf16: the state-gradient product measured 83 us with those, 71 us with these).  All 256 threads must call (one barrier: the last
+// step's operand reads end before the patches overwrite them).
+template <bool SPLIT, typename D>
+DEVI void store_wide_rows(const GemmAccWide &acc, GemmLdsWide<SPLIT> &s, D *dst, int64_t ld, int rows_valid, int tid) {
+  constexpr int CP = 128 / sizeof(D);      // columns per pass
+  constexpr int PP = CP + 16 / sizeof(D);  // patch pitch in elements (144 bytes)
+  constexpr int E16 = 16 / sizeof(D);      // elements per 16-byte piece
+  static_assert(sizeof(GemmLdsWide<SPLIT>) >= 4 * 16 * 144, "the four waves' patches fit in the operand tiles");
   const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1, i = lane & 15, g = lane >> 4;
+  D *patch = reinterpret_cast<D *>(&s) + wave * 16 * PP;
+  lds_barrier();
 #pragma unroll
   for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int m = wm * 32 + tm * 16 + g * 4 + r;
-      if (m >= rows_valid) continue;
+    for (int pass = 0; pass < 64 / CP; ++pass) {
 #pragma unroll
-      for (int tn = 0; tn < 4; ++tn) st_carried(dst + (int64_t)m * ld + wn * 64 + tn * 16 + i, acc.v[tm][tn][r]);
+      for (int t = 0; t < CP / 16; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) st_carried(patch + (g * 4 + r) * PP + t * 16 + i, acc.v[tm][pass * (CP / 16) + t][r]);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        const int row = q * 8 + (lane >> 3), piece = lane & 7;
+        const u32x4 v = *reinterpret_cast<const u32x4 *>(patch + row * PP + piece * E16);
+        const int m = wm * 32 + tm * 16 + row;
+        if (m < rows_valid) *reinterpret_cast<u32x4 *>(dst + (int64_t)m * ld + wn * 64 + pass * CP + piece * E16) = v;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
 }
 // Host side: a (batch, position, head/group, row) operand can feed WideTrStager.
@@ -711,6 +736,9 @@ template <int MODE = -1> DEVI void acc_add(float *dst, int64_t *shadow, int64_t 
 // The fused dx kernel (ssd_dx_fused.hip): launches it and returns MAMBA_OK, or returns MAMBA_E_UNSUPPORTED when it has
 // no kernel for the problem (the caller then runs the tiled bwd_dx_kernel).
 __attribute__((visibility("hidden"))) int ssd_bwd_dx_fused_launch(const SsdParams *p, hipStream_t stream);
+// The fused chunk-state dB / dC kernels (ssd_dbc_fused.hip), under the same convention (the caller then runs the
+// tiled bwd_d*_state kernels).
+__attribute__((visibility("hidden"))) int ssd_bwd_dbc_fused_launch(const SsdParams *p, hipStream_t stream);
 
 // ---- host side of the kernels that work through the heads of a group in one workgroup
 inline bool aligned(const void *ptr, int a) { return (reinterpret_cast<uintptr_t>(ptr) % a) == 0; }

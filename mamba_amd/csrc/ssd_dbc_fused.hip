@@ -1,0 +1,254 @@
+// SSD backward, the chunk-state parts of dB and dC (and the ddA_cumsum rows that come with dC), for bf16 on gfx950
+// (reference mamba_ssm/ops/triton/ssd_chunk_state.py:902 _chunk_state_bwd_db and ssd_chunk_scan.py:1451
+// _chunk_scan_bwd_dC; the same sums as bwd_dB_state_wide_kernel / bwd_dC_state_wide_kernel in ssd_bwd.hip):
+//     dB[s, n] += sum_{h in group} w_h[s] sum_p x[s, h, p] dS[h, p, n],   w_h[s] = dt_s exp(a_last - a_s), s in the
+//                                                                          chunk's last sequence, else 0
+//     dC[l, n] += sum_{h in group} v_h[l] sum_p g[l, h, p] H[h, p, n],    v_h[l] = exp(a_l), l in the sequence the
+//                                                                          chunk was entered in, else 0
+//     ddA_cumsum[h, l] += sum_n (v_h[l] sum_p g[l, h, p] H[h, p, n]) C[l, n]
+// with dS the gradient of the state a chunk hands on and H the state it was entered with.  One workgroup of one wave
+// per 16 positions works through a list of heads of one (batch, chunk, group): a head's rows (x or g, as they lie in
+// memory) and its P x N matrix are staged in LDS, two heads deep, so that a single barrier per head separates the
+// waves' products from the next commit and the loads of the head after next are in flight meanwhile.  Wave w owns
+// positions 16 w .. 16 w + 15 and keeps their sum over the heads in registers (fp32, N / 16 tiles); the per-position
+// weight is applied to the fp32 product of each head, not to the bf16 operand.  The matrix is the B operand with
+// k = p: its fragments come from transposing LDS reads.
+#include "ssd_common.hpp"
+
+namespace {
+
+DEVI f32x4 mfma_bf16(bf16x8_t a, bf16x8_t b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+constexpr int MAXHB = 20;  // heads per workgroup at most (heads_per_workgroup never picks more)
+
+template <int PT, int NK, int QT, bool IS_C, bool DET>
+__global__ __launch_bounds__(64 * QT) void bwd_dbc_fused_kernel(const SsdParams p, const int hb) {
+  constexpr int P = 16 * PT, N = 32 * NK, Q = 16 * QT, NT = 64 * QT, NTL = N / 16, KK = P / 32;
+  constexpr int XP = P + 8;   // LDS pitch of a row of x / g (bf16): 16-byte aligned pieces
+  constexpr int BP = N + 16;  // LDS pitch of a matrix row: the transposing reads of a half-wave cover all 64 banks once
+  struct Buf {
+    uint16_t Rs[Q * XP];  // the head's rows, one per position
+    uint16_t Ms[P * BP];  // the head's matrix, rows p
+    float w[Q];           // the head's weight per position
+  };
+  __shared__ __align__(16) Buf buf[2];
+  __shared__ float dda_s[IS_C ? MAXHB : 1][Q];  // the heads' ddA_cumsum rows, flushed at the end
+
+  int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  int j = lane & 15, g = lane >> 4;
+  const int H = p.nheads, G = p.ngroups, L = p.seqlen;
+  // the heads of a workgroup are `per` apart: workgroups in flight together touch neighbouring heads
+  const int hpg = H / G, per = hpg / hb;
+  const int grp = blockIdx.x / per, h_first = grp * hpg + blockIdx.x % per;
+  const int c = blockIdx.y, b = blockIdx.z;
+  const int t0 = c * Q;
+  const int qlim = min(Q, L - t0);
+  const float dsc = det_scale_of(p);
+  const View4 gv = g_view(p);
+  const bf16_t *rows_base = IS_C ? static_cast<const bf16_t *>(gv.ptr) + b * gv.bs : static_cast<const bf16_t *>(p.x) + b * p.x_bs;
+  const int64_t r_ls = IS_C ? gv.ls : p.x_ls, r_hs = IS_C ? gv.hs : p.x_hs;
+  const bf16_t *mats = static_cast<const bf16_t *>(IS_C ? p.states_lp : p.dstates_lp) + ((int64_t)b * p.nchunks + c) * H * P * N;
+
+  // position tid takes part: inside the sequence, and in the sequence the carried state belongs to
+  bool row_ok = false;
+  if (tid < Q) {
+    row_ok = tid < qlim;
+    if (p.seq_idx && row_ok) {
+      const int32_t *seq = p.seq_idx + (int64_t)b * L + t0;
+      if (IS_C) {
+        row_ok = seq[tid] == (c > 0 ? seq[-1] : 0);
+      } else {
+        const int last = seq[qlim - 1];
+        row_ok = last >= 0 && seq[tid] == last;
+      }
+    }
+  }
+
+  // ---- global -> registers -> LDS in 16-byte pieces, no branch around a load (rows past the end of the sequence
+  // re-read its last row; their weight is zero)
+  constexpr int GCH = Q * P / 8 / NT;
+  static_assert(GCH * NT * 8 == Q * P, "whole pieces per thread");
+  constexpr int HCH = (P * N / 8 + NT - 1) / NT;
+  static_assert(NT >= Q, "one position per thread");
+  u32x4 rregs[GCH], mregs[HCH];
+  float sc_a = 0.f, sc_alast = 0.f, sc_dt = 0.f;
+  auto load_head = [&](int h) {
+    const bf16_t *rr = rows_base + h * r_hs;
+#pragma unroll
+    for (int q = 0; q < GCH; ++q) {
+      const int id = tid + q * NT, r = id / (P / 8), c8 = id % (P / 8);
+      rregs[q] = *(const GLOBAL_AS u32x4 *)(rr + (int64_t)(t0 + min(r, qlim - 1)) * r_ls + c8 * 8);
+    }
+    const bf16_t *mm = mats + (int64_t)h * P * N;
+#pragma unroll
+    for (int q = 0; q < HCH; ++q) mregs[q] = *(const GLOBAL_AS u32x4 *)(mm + (int64_t)min(tid + q * NT, P * N / 8 - 1) * 8);
+    const float *dA = p.dA_cumsum + (((int64_t)b * H + h) * p.nchunks + c) * Q;
+    const int pos = min(tid, Q - 1);
+    sc_a = *(const GLOBAL_AS float *)(dA + pos);
+    if (!IS_C) {
+      sc_alast = *(const GLOBAL_AS float *)(dA + Q - 1);
+      sc_dt = *(const GLOBAL_AS float *)(p.dt_out + (((int64_t)b * H + h) * p.nchunks + c) * Q + pos);
+    }
+  };
+  auto commit_head = [&](Buf &B) {
+#pragma unroll
+    for (int q = 0; q < GCH; ++q) {
+      const int id = tid + q * NT, r = id / (P / 8), c8 = id % (P / 8);
+      *reinterpret_cast<u32x4 *>(&B.Rs[r * XP + c8 * 8]) = rregs[q];
+    }
+#pragma unroll
+    for (int q = 0; q < HCH; ++q) {
+      const int id = tid + q * NT, pp = id / (N / 8), c8 = id % (N / 8);
+      if (id < P * N / 8) *reinterpret_cast<u32x4 *>(&B.Ms[pp * BP + c8 * 8]) = mregs[q];
+    }
+    if (tid < Q) {
+      const float wv = IS_C ? fast_exp(sc_a) : fast_exp(fminf(sc_alast - sc_a, 0.f)) * sc_dt;
+      B.w[tid] = row_ok ? wv : 0.f;
+    }
+  };
+
+  load_head(h_first);
+
+  // C at this lane's accumulator positions (rows 16 wave + 4 g + r, columns 16 nt + j), packed in pairs
+  uint32_t crp[IS_C ? NTL / 2 : 1][4] = {};
+  if (IS_C) {
+    const uint16_t *Cg = static_cast<const uint16_t *>(p.C) + b * p.C_bs + grp * p.C_gs;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int l = wave * 16 + 4 * g + r;
+#pragma unroll
+      for (int nt = 0; nt < NTL; ++nt) {
+        const uint32_t raw = *(const GLOBAL_AS uint16_t *)(Cg + (int64_t)(t0 + min(l, qlim - 1)) * p.C_ls + nt * 16 + j);
+        crp[nt >> 1][r] |= raw << (16 * (nt & 1));
+      }
+    }
+  }
+
+  f32x4 sum[NTL];
+#pragma unroll
+  for (int nt = 0; nt < NTL; ++nt) sum[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  commit_head(buf[0]);
+  load_head(h_first + min(1, hb - 1) * per);
+  lds_barrier();
+
+#pragma unroll 1
+  for (int hh = 0; hh < hb; ++hh) {
+    // the thread's indices pass through an empty asm once per head, so that the addresses derived from them are
+    // computed where they are used instead of being carried (or spilled) across the loop over the heads
+    asm volatile("" : "+v"(tid), "+v"(lane), "+v"(j), "+v"(g));
+    Buf &B = buf[hh & 1];
+    f32x4 acc[NTL];
+#pragma unroll
+    for (int nt = 0; nt < NTL; ++nt) acc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      // k slots of lane group g: p = 32 kk + 4 g .. + 3, then 16 further on (both operands alike)
+      const uint16_t *ar = &B.Rs[(wave * 16 + j) * XP + kk * 32 + 4 * g];
+      const u32x2 a_lo = *reinterpret_cast<const u32x2 *>(ar), a_hi = *reinterpret_cast<const u32x2 *>(ar + 16);
+      const bf16x8_t af = __builtin_bit_cast(bf16x8_t, u32x4{a_lo.x, a_lo.y, a_hi.x, a_hi.y});
+#pragma unroll
+      for (int nt = 0; nt < NTL; ++nt) {
+        typedef __attribute__((address_space(3))) i16x4_t *lds_ptr;
+        typedef short i16x8_t __attribute__((ext_vector_type(8)));
+        const uint16_t *src = &B.Ms[(kk * 32 + 4 * g + (j >> 2)) * BP + nt * 16 + 4 * (j & 3)];
+        const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)src);
+        const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(src + 16 * BP));
+        const bf16x8_t bfr = __builtin_bit_cast(bf16x8_t, (i16x8_t)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        acc[nt] = mfma_bf16(af, bfr, acc[nt]);
+      }
+    }
+    const f32x4 wv = *reinterpret_cast<const f32x4 *>(&B.w[wave * 16 + 4 * g]);
+    if (IS_C) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float rs = 0.f;
+#pragma unroll
+        for (int nt = 0; nt < NTL; ++nt) {
+          const uint32_t cw = crp[nt >> 1][r];
+          rs = __builtin_fmaf(acc[nt][r], (nt & 1) ? bf16_hi(cw) : bf16_lo(cw), rs);
+        }
+        rs *= wv[r];
+        rs += dpp_f<DPP_ROW_SHR + 1>(0.f, rs);
+        rs += dpp_f<DPP_ROW_SHR + 2>(0.f, rs);
+        rs += dpp_f<DPP_ROW_SHR + 4>(0.f, rs);
+        rs += dpp_f<DPP_ROW_SHR + 8>(0.f, rs);
+        if (j == 15) dda_s[hh][wave * 16 + 4 * g + r] = rs;
+      }
+    }
+#pragma unroll
+    for (int nt = 0; nt < NTL; ++nt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) sum[nt][r] = __builtin_fmaf(acc[nt][r], wv[r], sum[nt][r]);
+
+    // the next head's operands go to the other buffer (last read one head ago, before the barrier that ended that
+    // head); the loads of the head after it follow, then the one barrier of this head
+    commit_head(buf[(hh + 1) & 1]);
+    load_head(h_first + min(hh + 2, hb - 1) * per);
+    lds_barrier();
+  }
+
+  // ---- the sums over this workgroup's heads join those of the others
+  float *dst = IS_C ? p.dC32 : p.dB32;
+  int64_t *shadow = IS_C ? p.det_dC : p.det_dB;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int l = wave * 16 + 4 * g + r;
+    if (l >= qlim) continue;
+    const int64_t row = (((int64_t)b * L + t0 + l) * G + grp) * N + j;
+#pragma unroll
+    for (int nt = 0; nt < NTL; ++nt) acc_add<DET ? 1 : 0>(dst, shadow, row + nt * 16, sum[nt][r], dsc);
+  }
+  if (IS_C) {
+    for (int idx = tid; idx < hb * Q; idx += NT) {
+      const int hh = idx / Q, l = idx % Q;
+      const float d = dda_s[hh][l];
+      if (l < qlim && d != 0.f)
+        acc_add<DET ? 1 : 0>(p.ddA_cumsum, p.det_ddA_cumsum, chunk_off(p, b, h_first + hh * per, c) + l, d, dsc);
+    }
+  }
+}
+
+template <int PT, int NK, bool IS_C, bool DET> int launch_q(const SsdParams &p, hipStream_t s) {
+  const int hb = heads_per_workgroup(p);
+  if (hb > MAXHB) return MAMBA_E_UNSUPPORTED;
+  dim3 grid(p.nheads / hb, p.nchunks, p.batch);
+  switch (p.chunk_size) {
+    case 256: hipLaunchKernelGGL((bwd_dbc_fused_kernel<PT, NK, 16, IS_C, DET>), grid, dim3(1024), 0, s, p, hb); break;
+    case 128: hipLaunchKernelGGL((bwd_dbc_fused_kernel<PT, NK, 8, IS_C, DET>), grid, dim3(512), 0, s, p, hb); break;
+    case 64: hipLaunchKernelGGL((bwd_dbc_fused_kernel<PT, NK, 4, IS_C, DET>), grid, dim3(256), 0, s, p, hb); break;
+    default: return MAMBA_E_UNSUPPORTED;
+  }
+  return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
+}
+template <bool IS_C, bool DET> int launch_pn(const SsdParams &p, hipStream_t s) {
+  if (p.headdim == 64) return p.dstate == 128 ? launch_q<4, 4, IS_C, DET>(p, s) : launch_q<4, 2, IS_C, DET>(p, s);
+  return p.dstate == 128 ? launch_q<2, 4, IS_C, DET>(p, s) : launch_q<2, 2, IS_C, DET>(p, s);
+}
+
+bool supported(const SsdParams *p) {
+  if (p->dtype != MAMBA_BF16 || !p->dstates_lp || !p->states_lp) return false;
+  if (p->headdim != 32 && p->headdim != 64) return false;
+  if (p->dstate != 64 && p->dstate != 128) return false;
+  if (p->chunk_size != 64 && p->chunk_size != 128 && p->chunk_size != 256) return false;
+  // 16-byte pieces of the x and g rows
+  const void *gptr = p->z ? static_cast<const void *>(p->gbuf) : p->dout;
+  if (!gptr || !p->dB32 || !p->dC32 || !p->ddA_cumsum) return false;
+  if (!aligned(p->x, 16) || !aligned(gptr, 16) || !aligned(p->dstates_lp, 16) || !aligned(p->states_lp, 16)) return false;
+  if (p->x_bs % 8 || p->x_ls % 8 || p->x_hs % 8) return false;
+  if (!p->z && (p->dout_bs % 8 || p->dout_ls % 8 || p->dout_hs % 8)) return false;
+  if (p->batch > 65535 || p->nchunks > 65535) return false;
+  return true;
+}
+
+}  // namespace
+
+int ssd_bwd_dbc_fused_launch(const SsdParams *p, hipStream_t stream) {
+  if (!supported(p)) return MAMBA_E_UNSUPPORTED;
+  int rc = p->det_scale ? launch_pn<true, true>(*p, stream) : launch_pn<true, false>(*p, stream);
+  if (rc) return rc;
+  return p->det_scale ? launch_pn<false, true>(*p, stream) : launch_pn<false, false>(*p, stream);
+}

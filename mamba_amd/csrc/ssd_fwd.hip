@@ -191,7 +191,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void chunk_s
   WideTrStager<SPLIT, T, WB> sb(lds.bh, lds.bl, Ba, p.B_ls, WB, w, tid);
   block_gemm_wide<SPLIT>(acc, lds, qlim, sa, sb, tid);  // the first barrier inside publishes w
   float *st = p.states + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
-  store_wide(acc, st + (int64_t)pt * GB * N + nt * WB, N, P - pt * GB, tid);
+  store_wide_rows(acc, lds, st + (int64_t)pt * GB * N + nt * WB, N, P - pt * GB, tid);
 }
 
 // ---------------------------------------------------- chunk_state_varlen
