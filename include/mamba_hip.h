@@ -276,7 +276,7 @@ typedef struct SsdParams {
   const float *initial_states;          /* nullable */
   const int32_t *seq_idx;               /* nullable */
   void *out;
-  void *out_x;                          /* pre-gate output, written iff z != NULL */
+  void *out_x;                          /* pre-gate output, written iff z != NULL; nullable (forward only: the backward pass reads it) */
   float *dt_out, *dA_cumsum, *states, *final_states, *CB;
 
   int64_t x_bs, x_ls, x_hs;

@@ -401,7 +401,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void chunk_s
     }
     const int64_t oi = b * p.out_bs + (int64_t)(t0 + l) * p.out_ls + h * p.out_hs + pp;
     if (p.z) {
-      stg<T>(p.out_x, oi, o);
+      if (p.out_x) stg<T>(p.out_x, oi, o);
       const float z = ldg<T>(p.z, b * p.z_bs + (int64_t)(t0 + l) * p.z_ls + h * p.z_hs + pp);
       o *= z * sigmoid_f(z);
     }
@@ -525,7 +525,7 @@ extern "C" int ssd_state_passing_fwd(const SsdParams *p, mamba_stream_t stream) 
 extern "C" int ssd_chunk_scan_fwd(const SsdParams *p, mamba_stream_t stream) {
   int rc = check(p);
   if (rc) return rc;
-  if (!p->CB || !p->out || !p->dt_out || !p->dA_cumsum || (p->z && !p->out_x)) return MAMBA_E_BADARG;
+  if (!p->CB || !p->out || !p->dt_out || !p->dA_cumsum) return MAMBA_E_BADARG;
   if (!(p->dtype == MAMBA_BF16 ? p->states_lp : (void *)p->states)) return MAMBA_E_BADARG;  // the carried states
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid(((p->chunk_size + GB - 1) / GB) * ((p->headdim + GB - 1) / GB), p->nchunks, p->batch * p->nheads);

@@ -274,7 +274,9 @@ __global__ __launch_bounds__(64 * QT) void chunk_scan_fwd_fused_kernel(const Ssd
     {
       const int64_t otile = b * p.out_bs + h * p.out_hs + (int64_t)(t0 + lt * 16) * p.out_ls;
       bf16_t *og = static_cast<bf16_t *>(p.out) + otile;
-      bf16_t *oxg = has_z ? static_cast<bf16_t *>(p.out_x) + otile : nullptr;
+      // without a pre-gate buffer (a forward pass nobody differentiates) the pre-gate store lands on the out row
+      // and the gated one after it replaces it in the cache: no branch around a store
+      bf16_t *oxg = has_z && p.out_x ? static_cast<bf16_t *>(p.out_x) + otile : og;
 #pragma unroll
       for (int pt = 0; pt < PT; ++pt) *reinterpret_cast<f32x4 *>(&Ys[j * YP + pt * 16 + 4 * g]) = acc[pt];
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -344,15 +346,14 @@ extern "C" int ssd_chunk_scan_fwd_fused_supported(const SsdParams *p) {
       p->C_ls % 8 || p->C_gs % 8)
     return 0;
   if (p->out_bs % 8 || p->out_ls % 8 || p->out_hs % 8) return 0;
-  if (p->z && (!aligned(p->z, 16) || !aligned(p->out_x, 16) || p->z_bs % 8 || p->z_ls % 8 || p->z_hs % 8)) return 0;
+  if (p->z && (!aligned(p->z, 16) || !aligned(p->out_x, 16) || p->z_bs % 8 || p->z_ls % 8 || p->z_hs % 8)) return 0;  // (a null out_x is aligned)
   if (p->states_lp && !aligned(p->states_lp, 16)) return 0;
   if (p->batch > 65535 || p->nheads > 65535) return 0;
   return 1;
 }
 
 extern "C" int ssd_chunk_scan_fwd_fused(const SsdParams *p, mamba_stream_t stream) {
-  if (!p || !p->x || !p->B || !p->C || !p->states_lp || !p->out || !p->dt_out || !p->dA_cumsum || (p->z && !p->out_x))
-    return MAMBA_E_BADARG;
+  if (!p || !p->x || !p->B || !p->C || !p->states_lp || !p->out || !p->dt_out || !p->dA_cumsum) return MAMBA_E_BADARG;
   if (!ssd_chunk_scan_fwd_fused_supported(p)) return MAMBA_E_UNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
   return p->headdim == 64 ? launch_n<4>(*p, s) : launch_n<2>(*p, s);

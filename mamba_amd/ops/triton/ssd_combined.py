@@ -122,9 +122,10 @@ def _workspace(x, B, chunk_size, forward_state=None):
 
 def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initial_states=None,
                                    seq_idx=None, cu_seqlens=None, dt_softplus=False, dt_limit=(0.0, float("inf")),
-                                   state_dtype=None):
+                                   state_dtype=None, want_out_x=True):
     """Counterpart of ssd_combined.py:343.  Returns (out, out_x, dt_out, dA_cumsum, states, final_states)
-    where `states[:, c]` is the state entering chunk c (bf16 next to bf16 operands, else fp32); with cu_seqlens a
+    where `states[:, c]` is the state entering chunk c (bf16 next to bf16 operands, else fp32) and out_x the output
+    before the gate (None without z, and with want_out_x=False: only the backward pass reads it); with cu_seqlens a
     seventh element,
     varlen_states (nseq, nheads, headdim, dstate): the state at the end of every packed sequence
     (ssd_combined.py:390-394), in state_dtype, else C's dtype, as the reference returns it."""
@@ -138,7 +139,7 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
         cu_seqlens = cu_seqlens.to(torch.int32).contiguous()
     ws = _workspace(x, B, chunk_size)
     out = torch.empty_like(x, memory_format=torch.contiguous_format)
-    out_x = torch.empty_like(out) if z is not None else None
+    out_x = torch.empty_like(out) if z is not None and want_out_x else None
     p = _lib.SsdParams()
     _fill_fwd(p, x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, seq_idx, dt_softplus, dt_limit, ws)
     p.out, p.out_x = out.data_ptr(), _lib.ptr(out_x)
@@ -276,7 +277,8 @@ class MambaChunkScanCombinedFn(torch.autograd.Function):
             assert cu_seqlens is not None, "cu_seqlens must be provided if return_varlen_states is True"
         out, out_x, dt_out, dA_cumsum, states, final_states, *rest = _mamba_chunk_scan_combined_fwd(
             x, dt, A, B, C, chunk_size, D=D, z=z, dt_bias=dt_bias, initial_states=initial_states, seq_idx=seq_idx,
-            cu_seqlens=cu_seqlens, dt_softplus=dt_softplus, dt_limit=dt_limit, state_dtype=state_dtype)
+            cu_seqlens=cu_seqlens, dt_softplus=dt_softplus, dt_limit=dt_limit, state_dtype=state_dtype,
+            want_out_x=any(ctx.needs_input_grad))  # no gradient asked for: the pre-gate copy is not written
         # with KEEP_FORWARD_STATE the fp32 dt, cumulative decay and chunk states of the forward pass
         # stay alive for the backward pass (batch*nchunks*nheads*headdim*dstate*4 bytes) instead of
         # being re-computed there as in the reference (ssd_combined.py:441-448)

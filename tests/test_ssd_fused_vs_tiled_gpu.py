@@ -1,10 +1,11 @@
-"""The fused SSD kernels (forward scan, backward dx: chosen for bf16 on 16-byte aligned rows) against the tiled
+"""The fused SSD kernels (forward scan, backward dx and chunk-state dB / dC: chosen for bf16 on 16-byte aligned rows) against the tiled
 kernels the same entry points fall back to: the same problem is run twice through mamba_chunk_scan_combined, once
 on ordinary tensors and once on copies of x and z whose rows start 8 bytes off a 16-byte boundary, which the fused
 kernels decline.  Both pipelines compute the same sums in fp32 from the same bf16 operands, so outputs and
 gradients agree to the rounding of the bf16 results (the oracle comparisons of each pipeline are in
 test_ssd_gpu.py and test_random_configs_gpu.py; this test pins the two against each other on shapes those draw
-rarely: several heads per workgroup, groups, packed sequences, a ragged last chunk)."""
+rarely: several heads per workgroup, groups, packed sequences, a ragged last chunk; the fused chunk-state dB / dC
+kernels decline the same copies, so their sums are pinned against the tiled ones here too)."""
 import pytest
 import torch
 
@@ -69,3 +70,28 @@ def test_fused_and_tiled_agree(batch, seqlen, nheads, headdim, ngroups, dstate, 
     close(out_f, out_t, "out")
     for name, gf, gt in zip(("dx", "dz", "ddt", "dA", "dB", "dC", "dD", "ddt_bias"), grads_f, grads_t):
         close(gf, gt, name)
+
+
+@pytest.mark.parametrize("misaligned", [False, True])
+def test_forward_without_gradients_skips_the_pre_gate_copy(misaligned):
+    """Under torch.no_grad() the scan is not handed a buffer for the output before the gate (only the backward pass
+    reads it): the gated output is bit for bit the one of a differentiated call, on the fused and on the tiled
+    kernels."""
+    torch.manual_seed(5)
+    dev, dt16 = "cuda", torch.bfloat16
+    batch, seqlen, nheads, headdim, ngroups, dstate, chunk = 2, 600, 8, 64, 2, 128, 256
+    x = torch.randn(batch, seqlen, nheads, headdim, device=dev, dtype=dt16)
+    z = torch.randn_like(x)
+    if misaligned:
+        x, z = _off_alignment(x), _off_alignment(z)
+    dt = (torch.rand(batch, seqlen, nheads, device=dev) * 0.5).to(dt16)
+    A = -(torch.rand(nheads, device=dev) + 0.5)
+    B = torch.randn(batch, seqlen, ngroups, dstate, device=dev, dtype=dt16)
+    C = torch.randn(batch, seqlen, ngroups, dstate, device=dev, dtype=dt16)
+    D = torch.randn(nheads, device=dev)
+    with torch.no_grad():
+        plain = mamba_chunk_scan_combined(x, dt, A, B, C, chunk, D=D, z=z, dt_softplus=True)
+    xg = x.detach().requires_grad_(True)
+    tracked = mamba_chunk_scan_combined(xg, dt, A, B, C, chunk, D=D, z=z, dt_softplus=True)
+    assert tracked.requires_grad and not plain.requires_grad
+    assert torch.equal(plain, tracked.detach())
