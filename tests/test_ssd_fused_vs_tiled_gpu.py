@@ -39,6 +39,10 @@ def _run(x, dt, A, B, C, D, z, dt_bias, seq_idx, chunk, dout):
     (1, 700, 8, 64, 2, 64, 128, False),     # ragged last chunk, two groups
     (1, 1024, 12, 32, 3, 128, 256, True),   # packed sequences, headdim 32
     (2, 256, 4, 64, 4, 64, 64, False),      # one head per group: one head per workgroup
+    (1, 384, 6, 32, 2, 64, 64, False),      # the smallest tiles of every fused kernel
+    (1, 640, 4, 64, 1, 128, 128, True),     # chunk 128 with 128 states, packed
+    (2, 200, 8, 32, 1, 128, 64, False),     # headdim 32 with 128 states, ragged
+    (1, 512, 10, 32, 1, 64, 256, False),    # headdim 32 with 64 states, chunk 256
 ])
 def test_fused_and_tiled_agree(batch, seqlen, nheads, headdim, ngroups, dstate, chunk, packed):
     torch.manual_seed(batch * 1000 + seqlen + nheads)
@@ -53,7 +57,7 @@ def test_fused_and_tiled_agree(batch, seqlen, nheads, headdim, ngroups, dstate, 
     dt_bias = torch.rand(nheads, device=dev) - 1.0
     seq_idx = None
     if packed:
-        cuts = torch.tensor([0, 130, 131, 400, 777, seqlen], device=dev)
+        cuts = torch.tensor([c for c in (0, 130, 131, 400, 777) if c < seqlen] + [seqlen], device=dev)
         seq_idx = (torch.arange(seqlen, device=dev)[None, :] >= cuts[1:-1, None]).sum(0).to(torch.int32)[None].expand(batch, -1).contiguous()
     dout = torch.randn_like(x)
 
