@@ -351,6 +351,8 @@ int ssd_chunk_state_varlen(const SsdParams *p, const int32_t *cu_seqlens, int ns
  * ssd_combined_bwd runs, in order:
  *   ssd_bwd_dz        dz, gbuf = dout silu(z), dD
  *   ssd_bwd_dstates   dstates[c] = direct gradient of the state entering chunk c
+ *                     (for bf16 with a gate, 128 states and 16-byte aligned rows ssd_combined_bwd runs these two
+ *                     stages as one kernel: the pass that makes gbuf feeds the product; same outputs)
  *   ssd_state_passing_bwd  reverse recurrence over chunks (in place on dstates -> gradient
  *                     of the chunk-local states), dinitial_states, ddA_cumsum at chunk ends
  *   ssd_bwd_dBC_state state-path parts of dB32 / dC32

@@ -266,6 +266,123 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dst
   store_wide_rows(acc, lds, ds + (int64_t)pt * GB * N + nt * WB, N, P - pt * GB, tid);
 }
 
+// dz, g = dout silu(z), dD and the state-gradient product of a (batch, chunk, head) in one pass (bf16 operands,
+// 128 states, a gate): the stager of the product's A operand makes g from dout and z on its way to LDS, stores it
+// and dz, and sums g x for dD; the product takes the stored (rounded) g, as the separate kernel does.  A thread's
+// task per k step is one 16-byte piece of a position's row, the task of bwd_dz_kernel.
+template <typename T> struct DzStager {
+  static constexpr bool transposed = true;
+  static constexpr int PITCH = WideTrStager<false, T, 64>::PITCH;
+  uint16_t *hi;
+  const T *dout, *z, *y, *x;  // at (batch, first position of the chunk, head, first p of the tile)
+  T *dz, *g;
+  int64_t dout_ls, z_ls, y_ls, x_ls, o_ls;
+  int rows_valid, t;
+  Pack8<T> qd, qz, qy, qx;
+  float dD[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  DEVI bool fast() const { return true; }
+  template <bool FAST = true> DEVI void fetch(int k0) {
+    const int l = k0 + (t >> 3), r8 = min((t & 7) * 8, rows_valid - 8);
+    qd.load(dout + (int64_t)l * dout_ls + r8);
+    qz.load(z + (int64_t)l * z_ls + r8);
+    qy.load(y + (int64_t)l * y_ls + r8);
+    qx.load(x + (int64_t)l * x_ls + r8);
+  }
+  template <bool FAST = true> DEVI void commit(int k0) {
+    const int kk = t >> 3, r8 = (t & 7) * 8, off = kk * PITCH + r8;
+    Pack8<T> gq;
+    gq.zero();
+    if (r8 < rows_valid) {
+      float d[8], zz[8], yy[8], xx[8], gv[8], dzv[8];
+      qd.unpack(d);
+      qz.unpack(zz);
+      qy.unpack(yy);
+      qx.unpack(xx);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float sg = sigmoid_f(zz[e]);
+        gv[e] = d[e] * zz[e] * sg;
+        dzv[e] = d[e] * yy[e] * sg * (1.f + zz[e] * (1.f - sg));
+        dD[e] = __builtin_fmaf(gv[e], xx[e], dD[e]);
+      }
+      gq.pack(gv);
+      Pack8<T> dq;
+      dq.pack(dzv);
+      const int64_t o = (int64_t)(k0 + kk) * o_ls + r8;
+      *reinterpret_cast<u32x4 *>(dz + o) = dq.w;
+      *reinterpret_cast<u32x4 *>(g + o) = gq.w;
+    }
+    *reinterpret_cast<u32x4 *>(hi + off) = gq.w;  // bf16 as it is: the MFMA operand
+  }
+};
+
+
+template <typename T> __global__ __launch_bounds__(256) void bwd_dz_dstates_kernel(const SsdParams p) {
+  __shared__ GemmLdsWide<false> lds;
+  __shared__ float rs[256];
+  const int tid = threadIdx.x;
+  const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads;
+  const Block3 blk = xcd_block();
+  const int pt = blk.x;  // one 128-state tile: a p tile's rows are read by one workgroup only
+  const int c = blk.y, b = blk.z / H, h = blk.z % H;
+  const int g = h / (H / p.ngroups);
+  const int t0 = c * Q, qlim = min(Q, L - t0);
+  const float *dA = chunk_row(p.dA_cumsum, p, b, h, c);
+  const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
+  for (int l = tid; l < Q; l += 256) {
+    float v = 0.f;
+    if (l < qlim) {
+      bool ok = true;
+      if (seq) ok = seq[l] == (c > 0 ? seq[-1] : 0);
+      if (ok) v = fast_exp(dA[l]);
+    }
+    rs[l] = v;
+  }
+  DzStager<T> sa;
+  sa.hi = lds.ah;
+  sa.dout = static_cast<const T *>(p.dout) + b * p.dout_bs + h * p.dout_hs + (int64_t)t0 * p.dout_ls + pt * GB;
+  sa.z = static_cast<const T *>(p.z) + b * p.z_bs + h * p.z_hs + (int64_t)t0 * p.z_ls + pt * GB;
+  sa.y = static_cast<const T *>(p.out_x) + b * p.out_bs + h * p.out_hs + (int64_t)t0 * p.out_ls + pt * GB;
+  sa.x = static_cast<const T *>(p.x) + b * p.x_bs + h * p.x_hs + (int64_t)t0 * p.x_ls + pt * GB;
+  const int64_t o0 = (((int64_t)b * L + t0) * H + h) * P + pt * GB;
+  sa.dz = static_cast<T *>(p.dz) + o0;
+  sa.g = static_cast<T *>(p.gbuf) + o0;
+  sa.dout_ls = p.dout_ls, sa.z_ls = p.z_ls, sa.y_ls = p.out_ls, sa.x_ls = p.x_ls, sa.o_ls = (int64_t)H * P;
+  sa.rows_valid = P - pt * GB;
+  sa.t = tid;
+  const T *Ca = static_cast<const T *>(p.C) + b * p.C_bs + g * p.C_gs + (int64_t)t0 * p.C_ls;
+  GemmAccWide acc;
+  acc.zero();
+  WideTrStager<false, T, WB> sb(lds.bh, lds.bl, Ca, p.C_ls, WB, rs, tid);
+  block_gemm_wide<false>(acc, lds, qlim, sa, sb, tid);  // the first barrier inside publishes rs
+  if (p.D) {
+    // a thread's 8 columns are the same in every step: column group tid % 8, summed over the 32 threads that share it
+    float *red = reinterpret_cast<float *>(&lds);  // row stride 9: conflict-free column reads
+    static_assert(sizeof(lds) >= 256 * 9 * sizeof(float), "the partial sums fit in the operand tiles");
+    lds_barrier();  // the last step's operand reads end before the sums overwrite them
+#pragma unroll
+    for (int e = 0; e < 8; ++e) red[tid * 9 + e] = sa.dD[e];
+    lds_barrier();
+    if (p.D_has_hdim) {
+      if (tid < GB && pt * GB + tid < P) {
+        float sacc = 0.f;
+        for (int r = tid / 8; r < 256; r += 8) sacc += red[r * 9 + (tid & 7)];
+        acc_add(p.dD, p.det_dD, h * P + pt * GB + tid, sacc, det_scale_of(p));
+      }
+    } else if (tid < 64) {
+      float sacc = 0.f;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sacc += red[(tid * 4 + r) * 9 + e];
+      sacc = wave_sum(sacc);
+      if (tid == 0) acc_add(p.dD, p.det_dD, h, sacc, det_scale_of(p));
+    }
+  }
+  carried_t<T> *ds = carried_dstates<T>(p) + (((int64_t)b * p.nchunks + c) * H + h) * P * N;
+  store_wide_rows(acc, lds, ds + (int64_t)pt * GB * N, N, P - pt * GB, tid);
+}
+
 // ---------------------------------------------------- state_passing bwd
 // Reverse recurrence over chunks.  On entry dstates[c] is the direct gradient of the state
 // entering chunk c; on exit it is the gradient of chunk c's local state.
@@ -1307,6 +1424,31 @@ extern "C" int ssd_det_convert(const int64_t *shadow, float *dst, int64_t n, con
   return launched();
 }
 
+// The first two stages: one kernel where the gate's pass over dout, z and the pre-gate output can feed the
+// state-gradient product directly (bf16 operands, one 128-state tile, whole k steps, 16-byte aligned rows), else
+// ssd_bwd_dz and ssd_bwd_dstates.
+static int dz_and_dstates(const SsdParams *p, mamba_stream_t stream) {
+  int rc = check_bwd(p);
+  if (rc) return rc;
+  auto rows16 = [&](const void *q, int64_t bs, int64_t ls, int64_t hs) {
+    return q && reinterpret_cast<uintptr_t>(q) % 16 == 0 && bs % 8 == 0 && ls % 8 == 0 && hs % 8 == 0;
+  };
+  const bool fused = p->z && p->out_x && p->dz && p->gbuf && p->dtype == MAMBA_BF16 && p->dstates_lp &&
+                     p->dstate == WB && p->headdim % 8 == 0 && whole_k_steps(p) &&
+                     rows16(p->dout, p->dout_bs, p->dout_ls, p->dout_hs) && rows16(p->z, p->z_bs, p->z_ls, p->z_hs) &&
+                     rows16(p->out_x, p->out_bs, p->out_ls, p->out_hs) && rows16(p->x, p->x_bs, p->x_ls, p->x_hs) &&
+                     rows16(p->dz, 0, 0, 0) && rows16(p->gbuf, 0, 0, 0) &&
+                     wide_operand_ok(p->C, p->dtype, p->C_bs, p->C_ls, p->C_gs);
+  if (fused) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    dim3 grid(tiles(p->headdim), p->nchunks, p->batch * p->nheads);
+    hipLaunchKernelGGL(bwd_dz_dstates_kernel<bf16_t>, grid, dim3(256), 0, s, *p);
+    return launched();
+  }
+  if ((rc = ssd_bwd_dz(p, stream))) return rc;
+  return ssd_bwd_dstates(p, stream);
+}
+
 extern "C" int ssd_combined_bwd(const SsdParams *p, mamba_stream_t stream) {
   int rc;
   if (p && p->det_scale) {
@@ -1317,8 +1459,7 @@ extern "C" int ssd_combined_bwd(const SsdParams *p, mamba_stream_t stream) {
     const int64_t rows = (int64_t)p->batch * p->nheads * p->nchunks * p->chunk_size;
     const int64_t bc = (int64_t)p->batch * p->seqlen * p->ngroups * p->dstate;
     const int64_t cb = (int64_t)p->batch * p->nchunks * p->ngroups * p->chunk_size * p->chunk_size;
-    if ((rc = ssd_bwd_dz(p, stream))) return rc;
-    if ((rc = ssd_bwd_dstates(p, stream))) return rc;
+    if ((rc = dz_and_dstates(p, stream))) return rc;
     if ((rc = ssd_state_passing_bwd(p, stream))) return rc;
     if ((rc = ssd_bwd_dBC_state(p, stream))) return rc;
     if ((rc = ssd_bwd_dx(p, stream))) return rc;
@@ -1338,8 +1479,7 @@ extern "C" int ssd_combined_bwd(const SsdParams *p, mamba_stream_t stream) {
     if (p->ddt_bias) return ssd_det_convert(p->det_ddt_bias, p->ddt_bias, p->nheads, p->det_scale, stream);
     return MAMBA_OK;
   }
-  if ((rc = ssd_bwd_dz(p, stream))) return rc;
-  if ((rc = ssd_bwd_dstates(p, stream))) return rc;
+  if ((rc = dz_and_dstates(p, stream))) return rc;
   if ((rc = ssd_state_passing_bwd(p, stream))) return rc;
   // dC reads the forward states, which the state-passing kernel has just read, and dB and dx the dstates it has just
   // written: in this order each finds them in the last-level cache

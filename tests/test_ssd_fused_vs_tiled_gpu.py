@@ -45,6 +45,16 @@ def _run(x, dt, A, B, C, D, z, dt_bias, seq_idx, chunk, dout):
     (1, 512, 10, 32, 1, 64, 256, False),    # headdim 32 with 64 states, chunk 256
 ])
 def test_fused_and_tiled_agree(batch, seqlen, nheads, headdim, ngroups, dstate, chunk, packed):
+    _compare(batch, seqlen, nheads, headdim, ngroups, dstate, chunk, packed)
+
+
+def test_fused_and_tiled_agree_with_a_D_per_channel():
+    """D of shape (nheads, headdim): dD per channel leaves the fused dz / state-gradient kernel as column sums."""
+    _compare(2, 512, 8, 64, 2, 128, 256, False, d_per_channel=True)
+    _compare(1, 256, 4, 32, 1, 128, 128, False, d_per_channel=True)
+
+
+def _compare(batch, seqlen, nheads, headdim, ngroups, dstate, chunk, packed, d_per_channel=False):
     torch.manual_seed(batch * 1000 + seqlen + nheads)
     dev, dt16 = "cuda", torch.bfloat16
     x = torch.randn(batch, seqlen, nheads, headdim, device=dev, dtype=dt16)
@@ -53,7 +63,7 @@ def test_fused_and_tiled_agree(batch, seqlen, nheads, headdim, ngroups, dstate, 
     A = -(torch.rand(nheads, device=dev) + 0.5)
     B = torch.randn(batch, seqlen, ngroups, dstate, device=dev, dtype=dt16)
     C = torch.randn(batch, seqlen, ngroups, dstate, device=dev, dtype=dt16)
-    D = torch.randn(nheads, device=dev)
+    D = torch.randn(nheads, headdim, device=dev) if d_per_channel else torch.randn(nheads, device=dev)
     dt_bias = torch.rand(nheads, device=dev) - 1.0
     seq_idx = None
     if packed:
