@@ -19,6 +19,8 @@ namespace {
 // The heads of a group are spread over this many workgroups (each sums ~8 heads in registers and
 // adds its partial result atomically).
 __host__ __device__ inline int head_splits(int heads_per_group) { return (heads_per_group + 7) / 8; }
+// The dCB kernel's lists are twice as long (~16 heads).
+__host__ __device__ inline int dcb_head_splits(int heads_per_group) { return (heads_per_group + 15) / 16; }
 
 __global__ __launch_bounds__(256) void det_convert_kernel(const int64_t *__restrict__ src, float *__restrict__ dst, int64_t n,
                                                           const float *__restrict__ scale) {
@@ -976,7 +978,7 @@ template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256, 4)
   __shared__ float hA_l[2][GB], hA_s[2][GB], hdt[2][GB];  // per-head rows, double-buffered over the head loop
   // the heads' ddA_cumsum shares (row sums per column half, column sums per row half), flushed at the end: a
   // global atomic per head would sit in the memory queue in front of the next head's loads
-  constexpr int MAXH = 8;  // heads per workgroup (head_splits keeps it at or below 8)
+  constexpr int MAXH = 16;  // heads per workgroup (dcb_head_splits keeps it at or below 16)
   __shared__ float rs_s[2][MAXH][GB], cs_s[2][MAXH][GB];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
@@ -986,7 +988,7 @@ template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256, 4)
   int lt = 0, rem = blk.x;
   while (rem > lt) { rem -= lt + 1; ++lt; }
   const int st = rem;
-  const int hpg = H / G, nsplit = head_splits(hpg);
+  const int hpg = H / G, nsplit = dcb_head_splits(hpg);
   const int c = blk.y, bg = blk.z / nsplit, hs = blk.z % nsplit, b = bg / G, g = bg % G;
   const int t0 = c * Q, qlim = min(Q, L - t0);
   const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
@@ -1393,7 +1395,7 @@ extern "C" int ssd_bwd_dcb(const SsdParams *p, mamba_stream_t stream) {
   if (rc) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int nt = tiles(p->chunk_size);
-  dim3 grid(nt * (nt + 1) / 2, p->nchunks, p->batch * p->ngroups * head_splits(p->nheads / p->ngroups));
+  dim3 grid(nt * (nt + 1) / 2, p->nchunks, p->batch * p->ngroups * dcb_head_splits(p->nheads / p->ngroups));
   SSD_DISPATCH_DET(bwd_dcb_kernel, grid)
   return launched();
 }
