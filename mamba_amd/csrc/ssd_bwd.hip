@@ -1163,6 +1163,56 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bmm_chu
   }
 }
 
+// The same two products on 64 x 128 tiles (whole 128-state blocks, chunks of whole k steps, 16-byte aligned B / C
+// rows): half the workgroups, each k step of dCB staged once for twice the columns.
+template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bmm_chunk_bwd_wide_kernel(const SsdParams p) {
+  __shared__ GemmLdsWide<SPLIT> lds;
+  const int tid = threadIdx.x;
+  const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, G = p.ngroups;
+  const int ntn = N / WB;
+  const int mt = blockIdx.x / ntn, nt = blockIdx.x % ntn;
+  const int c = blockIdx.y, b = blockIdx.z / G, g = blockIdx.z % G;
+  const int t0 = c * Q, qlim = min(Q, L - t0);
+  if (mt * GB >= qlim) return;
+  const float *dCB = p.dCB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
+  const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1, i = lane & 15, gq = lane >> 4;
+  auto add_tile = [&](const GemmAccWide &acc, float *dst) {  // dst[(row of the chunk) * G * N + column] += tile
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = mt * GB + wm * 32 + tm * 16 + gq * 4 + r;
+        if (m >= qlim) continue;
+        float *row = dst + (((int64_t)b * L + t0 + m) * G + g) * N + nt * WB + wn * 64 + i;
+#pragma unroll
+        for (int tn = 0; tn < 4; ++tn) row[tn * 16] += acc.v[tm][tn][r];
+      }
+  };
+  {
+    // dC: A = dCB rows (l, k = s), k-contiguous fp32, s up to the end of the l tile; B = B rows (k = s, n)
+    GemmAccWide acc;
+    acc.zero();
+    const int kend = min((mt + 1) * GB, qlim);
+    KcStager<SPLIT, float> sa(lds.ah, lds.al, dCB + (int64_t)mt * GB * Q, Q, qlim - mt * GB, kend, nullptr, nullptr, true, tid);
+    const T *Ba = static_cast<const T *>(p.B) + b * p.B_bs + g * p.B_gs + (int64_t)t0 * p.B_ls + nt * WB;
+    WideTrStager<SPLIT, T, WB> sb(lds.bh, lds.bl, Ba, p.B_ls, WB, nullptr, tid);
+    block_gemm_wide<SPLIT>(acc, lds, kend, sa, sb, tid);
+    add_tile(acc, p.dC32);
+  }
+  lds_barrier();  // the first product's last operand reads end before the second one's first commit
+  {
+    // dB: A = dCB^T (rows s, k = l from the s tile on), row-contiguous fp32; B = C rows (k = l, n)
+    GemmAccWide acc;
+    acc.zero();
+    const int k0 = mt * GB;
+    WideTrStager<SPLIT, float, 64> sa(lds.ah, lds.al, dCB + (int64_t)k0 * Q + mt * GB, Q, min(GB, Q - mt * GB), nullptr, tid);
+    const T *Ca = static_cast<const T *>(p.C) + b * p.C_bs + g * p.C_gs + (int64_t)(t0 + k0) * p.C_ls + nt * WB;
+    WideTrStager<SPLIT, T, WB> sb(lds.bh, lds.bl, Ca, p.C_ls, WB, nullptr, tid);
+    block_gemm_wide<SPLIT>(acc, lds, qlim - k0, sa, sb, tid);
+    add_tile(acc, p.dB32);
+  }
+}
+
 // --------------------------------------------------------- cumsum bwd
 // One workgroup per (batch, chunk, 16 heads); thread tid handles position Q-1-tid, so that the
 // reverse running sum of dL/da over the chunk (-> dL/d(dt A)) is a forward wave scan.  Then the
@@ -1404,6 +1454,13 @@ extern "C" int ssd_bmm_chunk_bwd(const SsdParams *p, mamba_stream_t stream) {
   int rc = check_bwd(p);
   if (rc) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (p->dstate % WB == 0 && p->chunk_size % GB == 0 && whole_k_steps(p) &&
+      wide_operand_ok(p->B, p->dtype, p->B_bs, p->B_ls, p->B_gs) && wide_operand_ok(p->C, p->dtype, p->C_bs, p->C_ls, p->C_gs) &&
+      reinterpret_cast<uintptr_t>(p->dCB) % 16 == 0) {
+    dim3 gridw(tiles(p->chunk_size) * (p->dstate / WB), p->nchunks, p->batch * p->ngroups);
+    SSD_DISPATCH(bmm_chunk_bwd_wide_kernel, gridw)
+    return launched();
+  }
   dim3 grid(tiles(p->chunk_size) * tiles(p->dstate), p->nchunks, p->batch * p->ngroups);
   SSD_DISPATCH(bmm_chunk_bwd_kernel, grid)
   return launched();
