@@ -112,20 +112,42 @@ __global__ __launch_bounds__(64 * QT) void bwd_dbc_fused_kernel(const SsdParams 
 
   load_head(h_first);
 
-  // C at this lane's accumulator positions (rows 16 wave + 4 g + r, columns 16 nt + j), packed in pairs
-  uint32_t crp[IS_C ? NTL / 2 : 1][4] = {};
+  // C at this lane's accumulator positions (rows 16 wave + 4 g + r, columns 16 nt + j): the wave's 16 rows go to
+  // LDS as they lie in memory (the staging buffers are still empty) and a transposing read hands lane (j, g) column
+  // 16 nt + j of rows 4 g .. 4 g + 3, which is that layout; cr(nt, r) is then one half of a register.
+  u32x2 crp[IS_C ? NTL : 1];
   if (IS_C) {
-    const uint16_t *Cg = static_cast<const uint16_t *>(p.C) + b * p.C_bs + grp * p.C_gs;
+    constexpr int CPP = 64 + 16;  // pitch of the patch (bf16): 16 rows x 64 columns at a time
+    static_assert(sizeof(Buf) * 2 >= (size_t)(Q / 16) * 16 * CPP * 2, "the waves' patches fit in the staging buffers");
+    uint16_t *Cw = reinterpret_cast<uint16_t *>(&buf[0]) + wave * 16 * CPP;
+    const bf16_t *Cg = static_cast<const bf16_t *>(p.C) + b * p.C_bs + grp * p.C_gs;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int l = wave * 16 + 4 * g + r;
+    for (int half = 0; half < N / 64; ++half) {
 #pragma unroll
-      for (int nt = 0; nt < NTL; ++nt) {
-        const uint32_t raw = *(const GLOBAL_AS uint16_t *)(Cg + (int64_t)(t0 + min(l, qlim - 1)) * p.C_ls + nt * 16 + j);
-        crp[nt >> 1][r] |= raw << (16 * (nt & 1));
+      for (int q = 0; q < 2; ++q) {  // 16 rows x 8 pieces of 8 columns
+        const int id = lane + q * 64, rr = id >> 3, c8 = id & 7;
+        const u32x4 v = *(const GLOBAL_AS u32x4 *)(Cg + (int64_t)(t0 + min(wave * 16 + rr, qlim - 1)) * p.C_ls + half * 64 + c8 * 8);
+        *reinterpret_cast<u32x4 *>(&Cw[rr * CPP + c8 * 8]) = v;
       }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        typedef __attribute__((address_space(3))) i16x4_t *lds_ptr;
+        const i16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)&Cw[(4 * g + (j >> 2)) * CPP + t * 16 + 4 * (j & 3)]);
+        crp[half * 4 + t] = __builtin_bit_cast(u32x2, v);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
+    lds_barrier();  // every wave has its C values before the first head is committed over the patches
   }
+  auto cr = [&](int nt, int r) {
+    const uint32_t w = (r & 2) ? crp[nt].y : crp[nt].x;
+    return (r & 1) ? bf16_hi(w) : bf16_lo(w);
+  };
 
   f32x4 sum[NTL];
 #pragma unroll
@@ -167,10 +189,7 @@ __global__ __launch_bounds__(64 * QT) void bwd_dbc_fused_kernel(const SsdParams 
       for (int r = 0; r < 4; ++r) {
         float rs = 0.f;
 #pragma unroll
-        for (int nt = 0; nt < NTL; ++nt) {
-          const uint32_t cw = crp[nt >> 1][r];
-          rs = __builtin_fmaf(acc[nt][r], (nt & 1) ? bf16_hi(cw) : bf16_lo(cw), rs);
-        }
+        for (int nt = 0; nt < NTL; ++nt) rs = __builtin_fmaf(acc[nt][r], cr(nt, r), rs);
         rs *= wv[r];
         rs += dpp_f<DPP_ROW_SHR + 1>(0.f, rs);
         rs += dpp_f<DPP_ROW_SHR + 2>(0.f, rs);
@@ -194,6 +213,8 @@ __global__ __launch_bounds__(64 * QT) void bwd_dbc_fused_kernel(const SsdParams 
   // ---- the sums over this workgroup's heads join those of the others
   float *dst = IS_C ? p.dC32 : p.dB32;
   int64_t *shadow = IS_C ? p.det_dC : p.det_dB;
+  // (the same adds as whole 128-byte lines of a row, through a patch per wave, measured no faster: 20 of a launch's
+  // ~85 us go into these atomics, and it is their number that costs)
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int l = wave * 16 + 4 * g + r;
