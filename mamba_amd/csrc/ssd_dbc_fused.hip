@@ -214,14 +214,21 @@ __global__ __launch_bounds__(64 * QT) void bwd_dbc_fused_kernel(const SsdParams 
   float *dst = IS_C ? p.dC32 : p.dB32;
   int64_t *shadow = IS_C ? p.det_dC : p.det_dB;
   // (the same adds as whole 128-byte lines of a row, through a patch per wave, measured no faster: 20 of a launch's
-  // ~85 us go into these atomics, and it is their number that costs)
+  // ~85 us go into these atomics, and it is their number that costs).  A workgroup that holds all heads of its group
+  // is the only one to touch its rows of dB / dC: it adds without atomics.
+  const bool alone = per == 1 && !DET;
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int l = wave * 16 + 4 * g + r;
     if (l >= qlim) continue;
     const int64_t row = (((int64_t)b * L + t0 + l) * G + grp) * N + j;
+    if (alone) {
 #pragma unroll
-    for (int nt = 0; nt < NTL; ++nt) acc_add<DET ? 1 : 0>(dst, shadow, row + nt * 16, sum[nt][r], dsc);
+      for (int nt = 0; nt < NTL; ++nt) dst[row + nt * 16] += sum[nt][r];
+    } else {
+#pragma unroll
+      for (int nt = 0; nt < NTL; ++nt) acc_add<DET ? 1 : 0>(dst, shadow, row + nt * 16, sum[nt][r], dsc);
+    }
   }
   if (IS_C) {
     for (int idx = tid; idx < hb * Q; idx += NT) {
