@@ -6,7 +6,8 @@
 //     dC[l, n] += sum_{h in group} v_h[l] sum_p g[l, h, p] H[h, p, n],    v_h[l] = exp(a_l), l in the sequence the
 //                                                                          chunk was entered in, else 0
 //     ddA_cumsum[h, l] += sum_n (v_h[l] sum_p g[l, h, p] H[h, p, n]) C[l, n]
-// with dS the gradient of the state a chunk hands on and H the state it was entered with.  One workgroup of one wave
+// with dS the gradient of the state a chunk hands on and H the state it was entered with.  One launch does both: half
+// of its workgroups take dC, half dB.  One workgroup of one wave
 // per 16 positions works through a list of heads of one (batch, chunk, group): a head's rows (x or g, as they lie in
 // memory) and its P x N matrix are staged in LDS, two heads deep, so that a single barrier per head separates the
 // waves' products from the next commit and the loads of the head after next are in flight meanwhile.  Wave w owns
@@ -21,20 +22,22 @@ DEVI f32x4 mfma_bf16(bf16x8_t a, bf16x8_t b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
 
-constexpr int MAXHB = 20;  // heads per workgroup at most (heads_per_workgroup never picks more)
+constexpr int MAXHB = 40;  // heads per workgroup at most (dbc_heads_per_workgroup never picks more)
 
+// LDS of one staged head: rows of x / g (pitch P + 8: 16-byte aligned pieces), the matrix (pitch N + 16: the
+// transposing reads of a half-wave cover all 64 banks once), the weight per position.
+template <int PT, int NK, int QT> struct DbcBuf {
+  uint16_t Rs[16 * QT * (16 * PT + 8)];
+  uint16_t Ms[16 * PT * (32 * NK + 16)];
+  float w[16 * QT];
+};
+
+// One of the two products for the workgroup's list of heads (list number `lb` of those of the launch).
 template <int PT, int NK, int QT, bool IS_C, bool DET>
-__global__ __launch_bounds__(64 * QT) void bwd_dbc_fused_kernel(const SsdParams p, const int hb) {
+DEVI void dbc_body(const SsdParams &p, const int hb, const int lb, DbcBuf<PT, NK, QT> *buf, float (*dda_s)[16 * QT]) {
   constexpr int P = 16 * PT, N = 32 * NK, Q = 16 * QT, NT = 64 * QT, NTL = N / 16, KK = P / 32;
-  constexpr int XP = P + 8;   // LDS pitch of a row of x / g (bf16): 16-byte aligned pieces
-  constexpr int BP = N + 16;  // LDS pitch of a matrix row: the transposing reads of a half-wave cover all 64 banks once
-  struct Buf {
-    uint16_t Rs[Q * XP];  // the head's rows, one per position
-    uint16_t Ms[P * BP];  // the head's matrix, rows p
-    float w[Q];           // the head's weight per position
-  };
-  __shared__ __align__(16) Buf buf[2];
-  __shared__ float dda_s[IS_C ? MAXHB : 1][Q];  // the heads' ddA_cumsum rows, flushed at the end
+  constexpr int XP = P + 8, BP = N + 16;
+  using Buf = DbcBuf<PT, NK, QT>;
 
   int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -42,7 +45,7 @@ __global__ __launch_bounds__(64 * QT) void bwd_dbc_fused_kernel(const SsdParams 
   const int H = p.nheads, G = p.ngroups, L = p.seqlen;
   // the heads of a workgroup are `per` apart: workgroups in flight together touch neighbouring heads
   const int hpg = H / G, per = hpg / hb;
-  const int grp = blockIdx.x / per, h_first = grp * hpg + blockIdx.x % per;
+  const int grp = lb / per, h_first = grp * hpg + lb % per;
   const int c = blockIdx.y, b = blockIdx.z;
   const int t0 = c * Q;
   const int qlim = min(Q, L - t0);
@@ -240,21 +243,48 @@ __global__ __launch_bounds__(64 * QT) void bwd_dbc_fused_kernel(const SsdParams 
   }
 }
 
-template <int PT, int NK, bool IS_C, bool DET> int launch_q(const SsdParams &p, hipStream_t s) {
-  const int hb = heads_per_workgroup(p);
-  if (hb > MAXHB) return MAMBA_E_UNSUPPORTED;
-  dim3 grid(p.nheads / hb, p.nchunks, p.batch);
+// Both products in one launch: the first half of the workgroups along x takes dC, the second dB, each for one list
+// of heads.  With lists twice as long as a launch per product would use to fill the chip there are half as many
+// lists to add up with atomics, the two prologues run side by side, and the whole chip is busy to the end.
+template <int PT, int NK, int QT, bool DET>
+__global__ __launch_bounds__(64 * QT) void bwd_dbc_fused_kernel(const SsdParams p, const int hb) {
+  __shared__ __align__(16) DbcBuf<PT, NK, QT> buf[2];
+  __shared__ float dda_s[MAXHB][16 * QT];  // the heads' ddA_cumsum rows of the dC product, flushed at the end
+  const int nlists = gridDim.x / 2;
+  if ((int)blockIdx.x < nlists) dbc_body<PT, NK, QT, true, DET>(p, hb, blockIdx.x, buf, dda_s);
+  else dbc_body<PT, NK, QT, false, DET>(p, hb, blockIdx.x - nlists, buf, dda_s);
+}
+
+// Heads per workgroup for that launch: a divisor of the heads per group, MAXHB at most, by the same estimate as
+// heads_per_workgroup with the fixed cost these kernels measure (prologue and final adds: about 8 heads' worth).
+inline int dbc_heads_per_workgroup(const SsdParams &p) {
+  const int hpg = p.nheads / p.ngroups, cus = cu_count();
+  const int64_t tiles = (int64_t)p.nchunks * p.batch;
+  int best = 1;
+  double best_cost = 1e30;
+  for (int hb = 1; hb <= MAXHB && hb <= hpg; ++hb) {
+    if (hpg % hb) continue;
+    const int64_t wgs = 2 * tiles * (p.nheads / hb);
+    const double cost = (double)((wgs + cus - 1) / cus) * (8.0 + hb);
+    if (cost < best_cost - 1e-9) best = hb, best_cost = cost;
+  }
+  return best;
+}
+
+template <int PT, int NK, bool DET> int launch_q(const SsdParams &p, hipStream_t s) {
+  const int hb = dbc_heads_per_workgroup(p);
+  dim3 grid(2 * (p.nheads / hb), p.nchunks, p.batch);
   switch (p.chunk_size) {
-    case 256: hipLaunchKernelGGL((bwd_dbc_fused_kernel<PT, NK, 16, IS_C, DET>), grid, dim3(1024), 0, s, p, hb); break;
-    case 128: hipLaunchKernelGGL((bwd_dbc_fused_kernel<PT, NK, 8, IS_C, DET>), grid, dim3(512), 0, s, p, hb); break;
-    case 64: hipLaunchKernelGGL((bwd_dbc_fused_kernel<PT, NK, 4, IS_C, DET>), grid, dim3(256), 0, s, p, hb); break;
+    case 256: hipLaunchKernelGGL((bwd_dbc_fused_kernel<PT, NK, 16, DET>), grid, dim3(1024), 0, s, p, hb); break;
+    case 128: hipLaunchKernelGGL((bwd_dbc_fused_kernel<PT, NK, 8, DET>), grid, dim3(512), 0, s, p, hb); break;
+    case 64: hipLaunchKernelGGL((bwd_dbc_fused_kernel<PT, NK, 4, DET>), grid, dim3(256), 0, s, p, hb); break;
     default: return MAMBA_E_UNSUPPORTED;
   }
   return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
 }
-template <bool IS_C, bool DET> int launch_pn(const SsdParams &p, hipStream_t s) {
-  if (p.headdim == 64) return p.dstate == 128 ? launch_q<4, 4, IS_C, DET>(p, s) : launch_q<4, 2, IS_C, DET>(p, s);
-  return p.dstate == 128 ? launch_q<2, 4, IS_C, DET>(p, s) : launch_q<2, 2, IS_C, DET>(p, s);
+template <bool DET> int launch_pn(const SsdParams &p, hipStream_t s) {
+  if (p.headdim == 64) return p.dstate == 128 ? launch_q<4, 4, DET>(p, s) : launch_q<4, 2, DET>(p, s);
+  return p.dstate == 128 ? launch_q<2, 4, DET>(p, s) : launch_q<2, 2, DET>(p, s);
 }
 
 bool supported(const SsdParams *p) {
@@ -276,7 +306,6 @@ bool supported(const SsdParams *p) {
 
 int ssd_bwd_dbc_fused_launch(const SsdParams *p, hipStream_t stream) {
   if (!supported(p)) return MAMBA_E_UNSUPPORTED;
-  int rc = p->det_scale ? launch_pn<true, true>(*p, stream) : launch_pn<true, false>(*p, stream);
-  if (rc) return rc;
-  return p->det_scale ? launch_pn<false, true>(*p, stream) : launch_pn<false, false>(*p, stream);
+  if (2 * (p->nheads / dbc_heads_per_workgroup(*p)) > 65535) return MAMBA_E_UNSUPPORTED;
+  return p->det_scale ? launch_pn<true>(*p, stream) : launch_pn<false>(*p, stream);
 }
