@@ -1165,13 +1165,13 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bmm_chu
 
 // The same two products on 64 x 128 tiles (whole 128-state blocks, chunks of whole k steps, 16-byte aligned B / C
 // rows): half the workgroups, each k step of dCB staged once for twice the columns.
-template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bmm_chunk_bwd_wide_kernel(const SsdParams p) {
+template <typename T, bool SPLIT> DEVI void bmm_chunk_bwd_wide_body(const SsdParams &p, int bx, int by, int bz) {
   __shared__ GemmLdsWide<SPLIT> lds;
   const int tid = threadIdx.x;
   const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, G = p.ngroups;
   const int ntn = N / WB;
-  const int mt = blockIdx.x / ntn, nt = blockIdx.x % ntn;
-  const int c = blockIdx.y, b = blockIdx.z / G, g = blockIdx.z % G;
+  const int mt = bx / ntn, nt = bx % ntn;
+  const int c = by, b = bz / G, g = bz % G;
   const int t0 = c * Q, qlim = min(Q, L - t0);
   if (mt * GB >= qlim) return;
   const float *dCB = p.dCB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
@@ -1213,6 +1213,10 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bmm_chu
   }
 }
 
+template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bmm_chunk_bwd_wide_kernel(const SsdParams p) {
+  bmm_chunk_bwd_wide_body<T, SPLIT>(p, blockIdx.x, blockIdx.y, blockIdx.z);
+}
+
 // --------------------------------------------------------- cumsum bwd
 // One workgroup per (batch, chunk, 16 heads); thread tid handles position Q-1-tid, so that the
 // reverse running sum of dL/da over the chunk (-> dL/d(dt A)) is a forward wave scan.  Then the
@@ -1230,12 +1234,12 @@ DEVI float wave_incl_sum(float x) {
 
 constexpr int CSB_HT = 4;  // heads per workgroup in the backward kernel (more, smaller workgroups)
 
-__global__ __launch_bounds__(256) void chunk_cumsum_bwd_kernel(const SsdParams p) {
+DEVI void chunk_cumsum_bwd_body(const SsdParams &p, int bx, int by, int bz) {
   __shared__ float wtot[4][CSB_HT], part[2][4][CSB_HT];
   const int H = p.nheads, Q = p.chunk_size, L = p.seqlen;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l = Q - 1 - tid;
-  const int c = blockIdx.x, h0 = blockIdx.y * CSB_HT, b = blockIdx.z;
+  const int c = bx, h0 = by * CSB_HT, b = bz;
   const int t = c * Q + l;
   const bool inq = l >= 0, live = inq && t < L;
   const int lc = max(l, 0), tc = min(c * Q + lc, L - 1);  // clamped: every load below is unconditional
@@ -1289,6 +1293,23 @@ __global__ __launch_bounds__(256) void chunk_cumsum_bwd_kernel(const SsdParams p
       if (which == 0) acc_add(p.dA, p.det_dA, h, v, det_scale_of(p));
       else if (p.ddt_bias) acc_add(p.ddt_bias, p.det_ddt_bias, h, v, det_scale_of(p));
     }
+  }
+}
+
+__global__ __launch_bounds__(256) void chunk_cumsum_bwd_kernel(const SsdParams p) {
+  chunk_cumsum_bwd_body(p, blockIdx.x, blockIdx.y, blockIdx.z);
+}
+
+// The last two stages read disjoint results of the stages before them (dCB; ddA_cumsum and ddt_out) and neither
+// fills the chip for long: one launch deals the wide-tile bmm workgroups first and the cumsum workgroups behind them.
+template <typename T, bool SPLIT>
+__global__ __launch_bounds__(256) void bmm_cumsum_bwd_kernel(const SsdParams p, int n_bmm, int bmm_x, int bmm_y, int cs_x, int cs_y) {
+  const int id = blockIdx.x;
+  if (id < n_bmm) {
+    bmm_chunk_bwd_wide_body<T, SPLIT>(p, id % bmm_x, (id / bmm_x) % bmm_y, id / (bmm_x * bmm_y));
+  } else {
+    const int k = id - n_bmm;
+    chunk_cumsum_bwd_body(p, k % cs_x, (k / cs_x) % cs_y, k / (cs_x * cs_y));
   }
 }
 
@@ -1483,6 +1504,36 @@ extern "C" int ssd_det_convert(const int64_t *shadow, float *dst, int64_t n, con
   return launched();
 }
 
+static bool bmm_bwd_wide_ok(const SsdParams *p) {
+  return p->dstate % WB == 0 && p->chunk_size % GB == 0 && whole_k_steps(p) &&
+         wide_operand_ok(p->B, p->dtype, p->B_bs, p->B_ls, p->B_gs) && wide_operand_ok(p->C, p->dtype, p->C_bs, p->C_ls, p->C_gs) &&
+         reinterpret_cast<uintptr_t>(p->dCB) % 16 == 0;
+}
+
+// The last two stages as one launch where the bmm stage runs on wide tiles, else one after the other.
+static int bmm_and_cumsum_bwd(const SsdParams *p, mamba_stream_t stream) {
+  int rc = check_bwd(p);
+  if (rc) return rc;
+  const int64_t bmm_x = tiles(p->chunk_size) * (p->dstate / WB), bmm_y = p->nchunks, bmm_z = (int64_t)p->batch * p->ngroups;
+  const int64_t cs_x = p->nchunks, cs_y = (p->nheads + CSB_HT - 1) / CSB_HT, cs_z = p->batch;
+  const int64_t n_bmm = bmm_x * bmm_y * bmm_z, total = n_bmm + cs_x * cs_y * cs_z;
+  if (bmm_bwd_wide_ok(p) && p->dCB && total <= 0x7fffffff) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    dim3 grid((unsigned)total);
+#define SSD_LAUNCH_BMM_CS(T, SPLIT) \
+  hipLaunchKernelGGL((bmm_cumsum_bwd_kernel<T, SPLIT>), grid, dim3(256), 0, s, *p, (int)n_bmm, (int)bmm_x, (int)bmm_y, (int)cs_x, (int)cs_y)
+    switch (p->dtype) {
+      case MAMBA_BF16: SSD_LAUNCH_BMM_CS(bf16_t, false); break;
+      case MAMBA_F16: SSD_LAUNCH_BMM_CS(f16_t, true); break;
+      default: SSD_LAUNCH_BMM_CS(float, true); break;
+    }
+#undef SSD_LAUNCH_BMM_CS
+    return launched();
+  }
+  if ((rc = ssd_bmm_chunk_bwd(p, stream))) return rc;
+  return ssd_chunk_cumsum_bwd(p, stream);
+}
+
 // The first two stages: one kernel where the gate's pass over dout, z and the pre-gate output can feed the
 // state-gradient product directly (bf16 operands, one 128-state tile, whole k steps, 16-byte aligned rows), else
 // ssd_bwd_dz and ssd_bwd_dstates.
@@ -1532,8 +1583,7 @@ extern "C" int ssd_combined_bwd(const SsdParams *p, mamba_stream_t stream) {
     if (p->D && (rc = ssd_det_convert(p->det_dD, p->dD, p->D_has_hdim ? (int64_t)p->nheads * p->headdim : p->nheads,
                                       p->det_scale, stream)))
       return rc;
-    if ((rc = ssd_bmm_chunk_bwd(p, stream))) return rc;  // one workgroup per output tile: plain adds
-    if ((rc = ssd_chunk_cumsum_bwd(p, stream))) return rc;
+    if ((rc = bmm_and_cumsum_bwd(p, stream))) return rc;  // bmm: one workgroup per output tile, plain adds
     if ((rc = ssd_det_convert(p->det_dA, p->dA, p->nheads, p->det_scale, stream))) return rc;
     if (p->ddt_bias) return ssd_det_convert(p->det_ddt_bias, p->ddt_bias, p->nheads, p->det_scale, stream);
     return MAMBA_OK;
@@ -1545,6 +1595,5 @@ extern "C" int ssd_combined_bwd(const SsdParams *p, mamba_stream_t stream) {
   if ((rc = ssd_bwd_dBC_state(p, stream))) return rc;
   if ((rc = ssd_bwd_dx(p, stream))) return rc;
   if ((rc = ssd_bwd_dcb(p, stream))) return rc;
-  if ((rc = ssd_bmm_chunk_bwd(p, stream))) return rc;
-  return ssd_chunk_cumsum_bwd(p, stream);
+  return bmm_and_cumsum_bwd(p, stream);
 }
