@@ -362,6 +362,8 @@ int ssd_chunk_state_varlen(const SsdParams *p, const int32_t *cu_seqlens, int ns
  *   ssd_bwd_dcb       dCB
  *   ssd_bmm_chunk_bwd dB32 / dC32 += dCB contractions
  *   ssd_chunk_cumsum_bwd  ddt, dA, ddt_bias from ddA_cumsum and ddt_out
+ *                     (ssd_combined_bwd deals the workgroups of these last two stages to one launch where the bmm
+ *                     stage runs on its 64 x 128 tiles: they read disjoint results of the stages before them)
  * ddA_cumsum holds the gradient with respect to the cumulative sums a_l; the last
  * stage turns it into the gradient of the per-position dt * A. */
 int ssd_bwd_dz(const SsdParams *p, mamba_stream_t stream);
