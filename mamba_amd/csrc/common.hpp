@@ -357,6 +357,32 @@ DEVI void row_scan_rev2(float &a0, float &b0, float &a1, float &b1) {
 }
 #undef MAMBA_DPP2
 
+// The same row scans for one recurrence: a step reads through DPP what the step before wrote, which needs two
+// wait states between the write and the read (the other instruction of the step plus s_nop 0).
+#define MAMBA_DPP1(CTRL)                                                       \
+  "v_fmac_f32_dpp %1, %1, %0 " CTRL " bank_mask:0xf\n\t"                      \
+  "v_mul_f32_dpp %0, %0, %0 " CTRL " bank_mask:0xf\n\t"                       \
+  "s_nop 0\n\t"
+DEVI void row_scan_fwd1(float &a, float &b) {
+  asm volatile("s_nop 1\n\t"
+               MAMBA_DPP1("row_shr:1 row_mask:0xf")
+               MAMBA_DPP1("row_shr:2 row_mask:0xf")
+               MAMBA_DPP1("row_shr:4 row_mask:0xf")
+               MAMBA_DPP1("row_shr:8 row_mask:0xf")
+               "s_nop 0\n\t"
+               : "+v"(a), "+v"(b));
+}
+DEVI void row_scan_rev1(float &a, float &b) {
+  asm volatile("s_nop 1\n\t"
+               MAMBA_DPP1("row_shl:1 row_mask:0xf")
+               MAMBA_DPP1("row_shl:2 row_mask:0xf")
+               MAMBA_DPP1("row_shl:4 row_mask:0xf")
+               MAMBA_DPP1("row_shl:8 row_mask:0xf")
+               "s_nop 0\n\t"
+               : "+v"(a), "+v"(b));
+}
+#undef MAMBA_DPP1
+
 // Completes a lane-reversed scan whose rows have been scanned by row_scan_rev2: appends to every
 // row the composition of the rows after it.
 DEVI void wave_scan_rev_finish(float &a, float &b, int lane) {

@@ -611,6 +611,13 @@ extern "C" int mamba2_decode_step(const MambaDecodeStepParams *q, mamba_stream_t
     return MAMBA_E_UNSUPPORTED;
   if (p->batch > 65535 || p->nheads > 65535 || p->dstate > 256 || p->dstate % 4 != 0) return MAMBA_E_UNSUPPORTED;
   {
+    // lane j of a wave convolves the x channel of the wave's row j, so a wave may hold at most 64 rows:
+    // fewer than 16 states (more than 16 rows per pass) are for the two separate calls
+    int lpr_log2 = 0;
+    (void)fused_grid_x(*p, &lpr_log2);
+    if ((64 >> lpr_log2) * UNR > 64) return MAMBA_E_UNSUPPORTED;
+  }
+  {
     const int es = p->state_dtype == MAMBA_F32 ? 4 : 2;
     const int64_t vb = 4 * es;
     if (p->state_ns != 1 || reinterpret_cast<uintptr_t>(p->state) % vb != 0 || (p->state_bs * es) % vb != 0 ||

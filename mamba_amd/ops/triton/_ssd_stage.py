@@ -60,9 +60,3 @@ def seq_idx_i32(seq_idx):
 def run(name, p, device):
     with torch.cuda.device(device):
         _lib.check(getattr(_lib.load(), name)(p, _lib.current_stream(device)), name)
-
-
-def forward_only(name):
-    raise NotImplementedError(
-        f"{name}: the stage-level function has no backward pass of its own here; gradients go through "
-        "mamba_chunk_scan_combined, whose backward stages are fused across chunk_state and chunk_scan")

@@ -175,7 +175,7 @@ def mamba2_decode_step(ssm_state, conv_state, xBC, dt, A, conv_weight, conv_bias
     width, state_len = conv_weight.shape[1], conv_state.shape[2]
     code = _lib.DTYPE_CODE
     fusable = (activation in (None, "silu", "swish") and xBC.dtype in code and conv_state.dtype == xBC.dtype
-               and ssm_state.dtype in code and 2 <= width <= 4 and width - 1 <= state_len <= 4 and dstate % 4 == 0
+               and ssm_state.dtype in code and 2 <= width <= 4 and width - 1 <= state_len <= 4 and dstate % 4 == 0 and dstate >= 16
                and xBC.stride(1) == 1 and ssm_state.stride(3) == 1 and (z is None or z.dtype == xBC.dtype))
     explicit = fuse is True
     if fuse is None:

@@ -72,29 +72,46 @@ def test_fused_optional_operands(has_z, has_D, has_bias, has_dtb):
     assert torch.equal(ssm_g, ssm_w) and torch.equal(conv_g, conv_w)
 
 
-def test_fused_against_the_oracle():
+@pytest.mark.parametrize("dtype,rtol,atol", [(torch.float32, 6e-4, 2e-3), (torch.bfloat16, 3e-2, 5e-2)])
+@pytest.mark.parametrize("batch,H,P,N,G", [(2, 4, 64, 128, 1), (3, 8, 64, 64, 2)])
+def test_fused_against_the_oracle(batch, H, P, N, G, dtype, rtol, atol):
     """The fused step alone against the CPU restatement: F.conv1d over [conv_state, x] + SiLU, then the
-    oracle's state update."""
+    oracle's state update (the oracle runs in fp32 on the same, already rounded, inputs; its conv output is
+    rounded to the activations' dtype as the operator's is)."""
     import torch.nn.functional as F
     from oracle.step import selective_state_update_oracle
-    batch, H, P, N, G, W = 2, 4, 64, 128, 1, 4
-    t, steps = _setup(batch, H, P, N, G, W, W, torch.float32, torch.float32, True, True, True, True, True, seed=5)
+    W = 4
+    t, steps = _setup(batch, H, P, N, G, W, W, dtype, torch.float32, True, True, True, True, True, seed=5)
     got, ssm_g, conv_g = _run(t, steps, G, True)
-    ssm, conv = t["ssm"].cpu().clone(), t["conv"].cpu().clone()
-    cw, cb = t["conv_w"].cpu(), t["conv_b"].cpu()
+    ssm, conv = t["ssm"].cpu().clone(), t["conv"].cpu().float().clone()
+    cw, cb = t["conv_w"].cpu().float(), t["conv_b"].cpu().float()
     for i, s in enumerate(steps):
-        full = torch.cat([conv, s["xBC"].cpu()[:, :, None]], dim=2)              # (batch, conv_dim, W + 1)
-        xc = F.silu(F.conv1d(full, cw[:, None, :], cb, groups=cw.shape[0])[:, :, -1])
+        full = torch.cat([conv, s["xBC"].cpu().float()[:, :, None]], dim=2)      # (batch, conv_dim, W + 1)
+        xc = F.silu(F.conv1d(full, cw[:, None, :], cb, groups=cw.shape[0])[:, :, -1]).to(dtype).float()
         conv = full[:, :, 1:].clone()
         x, B, C = torch.split(xc, [H * P, G * N, G * N], dim=-1)
         ref = selective_state_update_oracle(
-            ssm, x.reshape(batch, H, P), s["dt"].cpu()[:, :, None].expand(batch, H, P),
+            ssm, x.reshape(batch, H, P), s["dt"].cpu().float()[:, :, None].expand(batch, H, P),
             t["A"].cpu()[:, None, None].expand(H, P, N), B.reshape(batch, G, N), C.reshape(batch, G, N),
-            D=t["D"].cpu()[:, None].expand(H, P), z=s["z"].cpu(), dt_bias=t["dtb"].cpu()[:, None].expand(H, P),
+            D=t["D"].cpu()[:, None].expand(H, P), z=s["z"].cpu().float(), dt_bias=t["dtb"].cpu()[:, None].expand(H, P),
             dt_softplus=True)
-        assert torch.allclose(got[i].cpu(), ref, rtol=6e-4, atol=2e-3), f"step {i}"
-    assert torch.allclose(ssm_g.cpu(), ssm, rtol=6e-4, atol=2e-3)
-    assert torch.allclose(conv_g.cpu(), conv)
+        assert torch.allclose(got[i].cpu().float(), ref, rtol=rtol, atol=atol), f"step {i}"
+    assert torch.allclose(ssm_g.cpu(), ssm, rtol=rtol, atol=atol)
+    assert torch.equal(conv_g.cpu().float(), conv)
+
+
+@pytest.mark.parametrize("N,P", [(8, 128), (4, 64), (8, 64)])
+def test_few_states_take_the_two_calls(N, P):
+    """Fewer than 16 states put more than 64 rows into a wave of the fused kernel, which it does not serve: the
+    C entry point refuses, `fuse=True` raises, and `fuse=None` gives the two-call result."""
+    t, steps = _setup(2, 2, P, N, 1, 4, 4, torch.bfloat16, torch.float32, True, True, True, True, True, seed=N + P)
+    want, ssm_w, conv_w = _run(t, steps, 1, False)
+    got, ssm_g, conv_g = _run(t, steps, 1, None)
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+    assert torch.equal(ssm_g, ssm_w) and torch.equal(conv_g, conv_w)
+    with pytest.raises(RuntimeError):
+        _run(t, steps, 1, True)
 
 
 def test_fused_in_a_captured_graph():
