@@ -96,10 +96,11 @@ def _bwd_case(batch, seqlen, nheads, headdim, dstate, ngroups, chunk, dtype, seq
     names = ["x", "dt", "A", "B", "C", "D", "z", "dt_bias", "initial_states"]
     ref_in = {k: (t[k].clone().requires_grad_() if t[k] is not None else None) for k in names}
     gpu_in = {k: (t[k].cuda().requires_grad_() if t[k] is not None else None) for k in names}
+    # the oracle runs in float64 on the same (already rounded) inputs, so its own rounding is no part of the error
     out_ref, fin_ref = ssd_oracle(ref_in["x"], ref_in["dt"], ref_in["A"], ref_in["B"], ref_in["C"], D=ref_in["D"],
                                   z=ref_in["z"], dt_bias=ref_in["dt_bias"], initial_states=ref_in["initial_states"],
                                   seq_idx=t["seq_idx"], dt_softplus=True, dt_limit=dt_limit,
-                                  return_final_states=True)
+                                  return_final_states=True, compute_dtype=torch.float64)
     cu = lambda v: None if v is None else v.cuda()
     out, fin = mamba_chunk_scan_combined(gpu_in["x"], gpu_in["dt"], gpu_in["A"], gpu_in["B"], gpu_in["C"], chunk,
                                          D=gpu_in["D"], z=gpu_in["z"], dt_bias=gpu_in["dt_bias"],
@@ -107,18 +108,32 @@ def _bwd_case(batch, seqlen, nheads, headdim, dstate, ngroups, chunk, dtype, seq
                                          dt_softplus=True, dt_limit=dt_limit, return_final_states=True)
     _close("out", out, out_ref, rtol, atol)
     dfin = t["dfinal"] if with_dfinal else torch.zeros_like(t["dfinal"])
-    (out_ref.float() * t["dout"].float()).sum().add((fin_ref * dfin).sum()).backward()
+    (out_ref.double() * t["dout"].double()).sum().add((fin_ref * dfin.double()).sum()).backward()
     (out.float() * t["dout"].cuda().float()).sum().add((fin * dfin.cuda()).sum()).backward()
-    # gradient magnitudes grow with the sequence length; scale the absolute tolerance of the
-    # reduced (weight-like) gradients with their reference magnitude
+    # Every gradient at the base tolerance of its dtype, with two stated exceptions for 16-bit inputs:
+    #  * ddt: x LOOSE_DDT.  The gate gradient g = dout * silu(z) reaches the matrix cores rounded to the inputs'
+    #    dtype (the reference stores it the same way, ssd_chunk_scan.py:1386 `dout_x = torch.empty_like(dout)`),
+    #    and ddt sums ~headdim * chunk products of it with mixed signs; with fp32 kernels on the same values, or
+    #    without a gate, ddt holds the base tolerance (tests/test_ssd_rounding_sites_gpu.py).
+    #  * dA, dD, ddt_bias: fp32 sums over every position of a head; the absolute part of the tolerance follows the
+    #    largest entry of the reference (summation of 16-bit-rounded terms).
+    #  * fp16 inputs (no tolerance of their own in the benchmark; (3e-3, 5e-3) is the reference's fp16 setting for
+    #    the Mamba-1 scan, tests/ops/test_selective_scan.py:43-47): every gradient x 2, measured 1.5 on dx.
+    lowp = dtype != torch.float32
+    if dtype == torch.float16:
+        rtol, atol = 2 * rtol, 2 * atol
     for k in names:
         if ref_in[k] is None:
             continue
         gr, rr = gpu_in[k].grad, ref_in[k].grad
         assert gr is not None, f"no gradient for {k}"
         assert gr.dtype == gpu_in[k].dtype and gr.shape == gpu_in[k].shape
-        scale = max(1.0, float(rr.abs().max())) if k in ("A", "D", "dt_bias", "dt") else 1.0
-        _close("d" + k, gr, rr, rtol * 2, atol * 2 * scale * grad_scale)
+        f = LOOSE_DDT if (lowp and k == "dt") else 1.0
+        scale = max(1.0, float(rr.abs().max())) if (lowp and k in ("A", "D", "dt_bias")) else 1.0
+        _close("d" + k, gr, rr, rtol * f, atol * f * scale * grad_scale)
+
+
+LOOSE_DDT = 3.0
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
