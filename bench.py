@@ -35,10 +35,46 @@ HBM_PEAK_GBS = 8000.0
 PROFILES = os.path.join(ROOT, "profiles")
 
 
+def source_id():
+    """First 16 hex digits of the SHA-256 over the library's sources (mamba_amd/csrc/*.hip, *.hpp, *.cpp and
+    include/*.h, in name order).  The counter summaries under profiles/ carry the id of the sources they were
+    taken with; figures parsed from a summary whose id differs are reported as null."""
+    import hashlib
+    h = hashlib.sha256()
+    files = []
+    for d, exts in ((os.path.join(ROOT, "mamba_amd", "csrc"), (".hip", ".hpp", ".cpp")), (os.path.join(ROOT, "include"), (".h",))):
+        files += [os.path.join(d, n) for n in os.listdir(d) if n.endswith(exts)]
+    for p in sorted(files):
+        h.update(os.path.basename(p).encode())
+        h.update(open(p, "rb").read())
+    return h.hexdigest()[:16]
+
+
+_FRESH = {}
+
+
+def profile_fresh(filename):
+    """True when profiles/<filename> says it was taken with the sources this tree holds (a line
+    `library sources: <id>`)."""
+    if filename not in _FRESH:
+        ok = False
+        try:
+            for line in open(os.path.join(PROFILES, filename)):
+                if line.startswith("library sources:"):
+                    ok = line.split(":", 1)[1].strip() == source_id()
+                    break
+        except OSError:
+            pass
+        _FRESH[filename] = ok
+    return _FRESH[filename]
+
+
 def profile_traffic(filename, kernel):
     """HBM bytes per launch of `kernel` as the FETCH_SIZE / WRITE_SIZE counter runs measured them: the row of
     that kernel in profiles/<filename> (columns ... read MB (scaled), written MB (scaled)).  None when the
-    summary or the row is missing, e.g. after a kernel was renamed and before the counters were taken again."""
+    summary or the row is missing or the summary was taken with other sources than this tree's."""
+    if not profile_fresh(filename):
+        return None
     try:
         for line in open(os.path.join(PROFILES, filename)):
             cols = line.split()
@@ -49,8 +85,34 @@ def profile_traffic(filename, kernel):
     return None
 
 
+def profile_traffic_sum(filename):
+    """Sum of the scaled read + written bytes over every kernel row of an HBM-counter summary (one step)."""
+    if not profile_fresh(filename):
+        return None
+    total, rows = 0.0, 0
+    try:
+        seen = False
+        for line in open(os.path.join(PROFILES, filename)):
+            cols = line.split()
+            if cols[:1] == ["kernel"]:
+                seen = True
+                continue
+            if seen and len(cols) >= 5:
+                try:
+                    total += (float(cols[-2]) + float(cols[-1])) * 1e6
+                    rows += 1
+                except ValueError:
+                    pass
+    except OSError:
+        return None
+    return total if rows else None
+
+
 def profile_counter(filename, kernel, counter):
-    """Average per-launch value of one hardware counter from profiles/<filename> (lines `kernel counter value`)."""
+    """Average per-launch value of one hardware counter from profiles/<filename> (lines `kernel counter value`);
+    None when missing or stale."""
+    if not profile_fresh(filename):
+        return None
     try:
         for line in open(os.path.join(PROFILES, filename)):
             cols = line.split()
@@ -84,15 +146,15 @@ def cpu_model():
 
 
 def cpu_baseline(seqlen, dstate, full_dim):
-    """Oracle (a PyTorch restatement of the reference's selective_scan_ref) on the host cores, forward alone and
-    forward + backward, median of 3 each, on a batch-1 / 32-channel slice of the workload; channels and batch
-    rows are independent in the scan, so tokens/s is scaled by (32 / full_dim)."""
+    """Oracle (a PyTorch restatement of the reference's selective_scan_ref) on the host cores: forward alone (median
+    of 3) and forward + backward (median of 2), on a batch-1 slice of one sixteenth of the channels; channels and
+    batch rows are independent in the scan, so tokens/s of the whole workload is the slice's rate x slice / whole."""
     import statistics
     import torch
     from oracle.mamba1 import selective_scan_oracle, scan_inputs
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
-    dim = 32
+    dim = full_dim // 16
     t = scan_inputs(1, dim, seqlen, dstate, 1, torch.bfloat16, seed=0)
     names = ("u", "delta", "A", "B", "C", "D", "z", "delta_bias")
 
@@ -106,12 +168,66 @@ def cpu_baseline(seqlen, dstate, full_dim):
         return time.perf_counter() - t0
 
     fwd = statistics.median(run(False) for _ in range(3))
-    both = statistics.median(run(True) for _ in range(3))
+    both = statistics.median(run(True) for _ in range(2))
     scale = dim / full_dim
     return {"value": seqlen * scale / both, "unit": "tokens/s", "cores": cores, "kind": "port",
             "fwd_only_value": seqlen * scale / fwd, "cpu": cpu_model(),
-            "sample": f"oracle, batch 1 x {dim} of {full_dim} channels x seqlen {seqlen}, median of 3: forward "
-                      f"{fwd:.2f} s, forward + backward {both:.2f} s, scaled by {dim}/{full_dim}"}
+            "slice_seconds": {"forward": fwd, "forward_backward": both},
+            "sample": f"oracle.mamba1.selective_scan_oracle, batch 1 x {dim} of {full_dim} channels x seqlen {seqlen} "
+                      f"(1/16 of the channels of one of 8 batch rows): forward {fwd:.2f} s (median of 3), forward + "
+                      f"backward {both:.2f} s (median of 2); tokens/s of the whole workload = {seqlen} x {dim}/{full_dim} / seconds"}
+
+
+def cpu_baseline_ssd():
+    """The chunked SSD oracle (oracle.ssd.ssd_chunked, the four-step form of the reference's ssd_minimal.py) with
+    autograd on the host cores, on one batch row and one sixteenth of configuration 2's heads (heads and batch rows
+    are independent); forward + backward, median of 2."""
+    import statistics
+    import torch
+    from oracle.ssd import ssd_chunked, ssd_inputs, dt_pipeline
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    L, H, Hs, P, N, Q = 4096, 80, 5, 64, 128, 256
+    t = ssd_inputs(1, L, Hs, P, N, 1, torch.bfloat16, 0)
+
+    def run():
+        ins = {k: t[k].clone().float().requires_grad_() for k in ("x", "dt", "B", "C", "z")}
+        t0 = time.perf_counter()
+        dtv = dt_pipeline(ins["dt"], t["dt_bias"], True)
+        out = ssd_chunked(ins["x"], dtv, t["A"], ins["B"], ins["C"], Q, D=t["D"], z=ins["z"])
+        out.backward(t["dout"].float())
+        return time.perf_counter() - t0
+
+    sec = statistics.median(run() for _ in range(2))
+    return {"value": L * (Hs / H) / sec, "unit": "tokens/s", "cores": cores, "kind": "port", "slice_seconds": sec,
+            "sample": f"oracle.ssd.ssd_chunked forward + backward, batch 1 x {Hs} of {H} heads x seqlen {L}: {sec:.2f} s "
+                      f"(median of 2); tokens/s of the whole workload = {L} x {Hs}/{H} / seconds"}
+
+
+def cpu_baseline_decode():
+    """The decode-step oracle on the host cores: 16 of configuration 3's 256 batch rows, 20 consecutive steps."""
+    import torch
+    from oracle.step import selective_state_update_oracle
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    rows, batch, H, P, N, steps = 16, 256, 80, 64, 128, 20
+    g = torch.Generator().manual_seed(0)
+    state = 0.1 * torch.randn(rows, H, P, N, generator=g)
+    x, z = (torch.randn(rows, H, P, generator=g).bfloat16() for _ in range(2))
+    dt = torch.randn(rows, H, generator=g).bfloat16()[:, :, None].expand(rows, H, P)
+    B, C = (torch.randn(rows, 1, N, generator=g).bfloat16() for _ in range(2))
+    A = (-(1 + 15 * torch.rand(H, generator=g)))[:, None, None].expand(H, P, N)
+    D = torch.rand(H, generator=g)[:, None].expand(H, P)
+    dtb = (torch.rand(H, generator=g) - 4)[:, None].expand(H, P)
+    one = lambda: selective_state_update_oracle(state, x, dt, A, B, C, D=D, z=z, dt_bias=dtb, dt_softplus=True)
+    one()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        one()
+    sec = (time.perf_counter() - t0) / steps
+    return {"value": rows / sec, "unit": "tokens/s", "cores": cores, "kind": "port", "slice_seconds_per_step": sec,
+            "sample": f"oracle.step.selective_state_update_oracle, {rows} of {batch} batch rows, {steps} consecutive "
+                      f"steps: {sec * 1e3:.1f} ms per step; batch rows are independent, so tokens/s = rows / seconds"}
 
 
 def measured_copy(dev):
@@ -191,10 +307,15 @@ def vs_measured_copy(roofline, dev):
     return roofline
 
 
-def event_ms(fn, n, pre=None):
-    """Average HIP-event time of fn() on torch's current stream (where the library launches);
-    pre() runs outside the event pair."""
+KERNEL_ITERS = 100  # launches per event-timed kernel or pass; the median is reported
+
+
+def event_stats(fn, n=None, pre=None):
+    """HIP-event times of n single calls of fn() on torch's current stream (where the library launches), each
+    call in its own event pair; pre() runs outside the pairs.  Returns {"median", "min", "max", "n"} in ms."""
+    import statistics
     import torch
+    n = n or KERNEL_ITERS
     if pre:
         pre()
     fn()
@@ -207,7 +328,29 @@ def event_ms(fn, n, pre=None):
         fn()
         b.record()
     torch.cuda.synchronize()
-    return sum(a.elapsed_time(b) for a, b in ev) / n
+    ts = [a.elapsed_time(b) for a, b in ev]
+    return {"median": statistics.median(ts), "min": min(ts), "max": max(ts), "n": n}
+
+
+def event_ms(fn, n=None, pre=None):
+    """Median HIP-event time of one call of fn(), in ms."""
+    return event_stats(fn, n, pre)["median"]
+
+
+def timed_steps(step, steps, warmup):
+    """The contract's timing: `warmup` untimed steps, then exactly `steps` steps between two device
+    synchronisations; returns seconds per step.  Then every step of a second pass of max(steps, KERNEL_ITERS)
+    steps in its own event pair: {"median", "min", "max", "n"} in ms."""
+    import torch
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / steps
+    return sec, event_stats(step, max(steps, KERNEL_ITERS))
 
 
 def bench_ssd(dev, steps, warmup):
@@ -237,14 +380,7 @@ def bench_ssd(dev, steps, warmup):
             v.grad = None
         fwd().backward(dout)
 
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    torch.cuda.synchronize()
-    sec = (time.perf_counter() - t0) / steps
+    sec, step_stats = timed_steps(step, steps, warmup)
     # the same step in the deterministic mode (integer atomics on fixed-point terms in the backward pass)
     from mamba_amd.utils.determinism import set_deterministic_mode
     set_deterministic_mode(True)
@@ -259,7 +395,7 @@ def bench_ssd(dev, steps, warmup):
     finally:
         set_deterministic_mode(None)
     with torch.no_grad():
-        fwd_ms = event_ms(fwd, max(5, min(steps, 50)))
+        fwd_ms = event_ms(fwd)
         # the fused scan kernel alone, on the buffers of one forward pass
         lib = _lib.load()
         a = sc._prepare(x, dt, A, B, C, Q, D, z, dtb, None, None)
@@ -271,29 +407,48 @@ def bench_ssd(dev, steps, warmup):
         p.out_bs, p.out_ls, p.out_hs = out.stride(0), out.stride(1), out.stride(2)
         stream = _lib.current_stream(dev)
         _lib.check(lib.ssd_combined_fwd(p, stream), "ssd_combined_fwd")   # fills dA_cumsum and the chunk states
-        scan_ms = event_ms(lambda: _lib.check(lib.ssd_chunk_scan_fwd_fused(p, stream), "ssd_chunk_scan_fwd_fused"),
-                           max(5, min(steps, 50)))
+        scan = event_stats(lambda: _lib.check(lib.ssd_chunk_scan_fwd_fused(p, stream), "ssd_chunk_scan_fwd_fused"))
+        scan_ms = scan["median"]
     nc = L // Q
     mfma_tflops = measured_mfma(dev)
     flops = batch * nc * (H * (Q * Q * P + 2 * Q * N * P) + G * Q * Q * N)   # causal halves counted once
     nbytes = 2 * (4 * batch * L * H * P + 2 * batch * L * G * N) + 2 * batch * nc * H * P * N  # x z out out_x B C, bf16 states
+    prof = "ssd_combined_b4_l4096_h80_p64_n128_q256_bf16"
+    step_bytes = 2 * (8 * batch * L * H * P + 6 * batch * L * G * N + 3 * batch * L * H)  # fwd+bwd: 8 X + 6 BC + 3 T
     return ({
         "metric": "SSD mamba_chunk_scan_combined fwd+bwd tokens/s at 1 GPU", "value": batch * L / sec,
         "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": sec * 1e3,
-        "fwd_ms": fwd_ms, "deterministic_ms_per_step": det_sec * 1e3, "higher_is_better": True,
+        "step_ms": step_stats, "fwd_ms": fwd_ms, "deterministic_ms_per_step": det_sec * 1e3, "higher_is_better": True,
+        "step_roofline": {"bound": "hbm", "algorithmic_bytes": step_bytes, "achieved": step_bytes / sec / 1e9,
+                          "frac": step_bytes / sec / 1e9 / HBM_PEAK_GBS, "unit": "GB/s",
+                          "traffic": profile_traffic_sum(prof + "_hbm_counters.txt")},
         "dtype": "bf16 in/out, fp32 accumulation", "data": "synthetic",
         "config": {"workload": f"Mamba-2 SSD fwd+bwd: batch {batch}, seqlen {L}, {H} heads x {P}, d_state {N}, "
                                f"{G} group, chunk {Q}, bf16 (benchmark configuration 2)"},
         "roofline": vs_measured_copy({"bound": "hbm", "kernel": "chunk_scan_fwd_fused_kernel", "achieved": nbytes / scan_ms / 1e6,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / scan_ms / 1e6 / HBM_PEAK_GBS,
-                     "traffic": profile_traffic("ssd_combined_b4_l4096_h80_p64_n128_q256_bf16_hbm_counters.txt", "chunk_scan_fwd_fused_kernel"),
-                     "kernel_ms": scan_ms, "algorithmic_bytes": nbytes,
+                     "traffic": profile_traffic(prof + "_hbm_counters.txt", "chunk_scan_fwd_fused_kernel"),
+                     "kernel_ms": scan_ms, "kernel_ms_min_max_n": [scan["min"], scan["max"], scan["n"]],
+                     "algorithmic_bytes": nbytes,
                      "algorithmic_flops": flops, "mfma_tflops": flops / scan_ms / 1e9,
                      "mfma_frac_of_bf16_peak": flops / scan_ms / 1e9 / 2500.0,
                      # the kernel moves `algorithmic_bytes` for `algorithmic_flops`: at the HBM peak that caps it at
                      "flop_per_byte": flops / nbytes, "mfma_cap_from_hbm_tflops": flops / nbytes * HBM_PEAK_GBS / 1e3,
                      "measured_mfma_tflops": mfma_tflops,
-                     "mfma_frac_of_measured": flops / scan_ms / 1e9 / mfma_tflops}, dev)})
+                     "mfma_frac_of_measured": flops / scan_ms / 1e9 / mfma_tflops,
+                     "mfma_counters": mfma_counters(prof + "_mfma_counters.txt", "chunk_scan_fwd_fused_kernel")}, dev)})
+
+
+def mfma_counters(filename, kernel):
+    """Matrix-core counters of `kernel` from profiles/<filename> (per launch, summed over the chip): bf16 MFMA
+    instructions, and the share of the busy cycles of the compute units in which a matrix core was executing."""
+    n = profile_counter(filename, kernel, "SQ_INSTS_VALU_MFMA_BF16")
+    busy = profile_counter(filename, kernel, "SQ_VALU_MFMA_BUSY_CYCLES")
+    cu = profile_counter(filename, kernel, "SQ_BUSY_CU_CYCLES")
+    if n is None or busy is None or cu is None:
+        return None
+    return {"mfma_bf16_instructions": n, "mfma_busy_cycles": busy, "cu_busy_cycles": cu,
+            "mfma_busy_frac_of_cu_busy": busy / cu if cu else None}
 
 
 def bench_decode(dev, steps, warmup, batch=256):
@@ -422,18 +577,6 @@ def bench_decode_step(dev, steps, warmup, batch):
             **out}
 
 
-def _timed(step, steps, warmup):
-    import torch
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    torch.cuda.synchronize()
-    return (time.perf_counter() - t0) / steps
-
-
 def bench_varlen(dev, steps, warmup):
     """Configuration 4: one packed row of 16 sequences (lengths uniform in [512, 4096], rescaled to sum to
     32768), seq_idx, nonzero initial states, final states returned; forward + backward."""
@@ -466,19 +609,47 @@ def bench_varlen(dev, steps, warmup):
             v.grad = None
         fwd()[0].backward(dout)
 
-    sec = _timed(step, steps, warmup)
+    sec, step_stats = timed_steps(step, steps, warmup)
     with torch.no_grad():
-        fwd_ms = event_ms(fwd, max(5, min(steps, 50)))
-    nbytes = 2 * (5 * batch * L * H * P + 4 * batch * L * G * N)   # x z dout in, dx dz out, B C in, dB dC out (bf16)
+        fwd_ms = event_ms(fwd)
+        # the fused scan kernel alone (the kernel the roofline entry of configuration 2 names), on the buffers of one
+        # forward pass of this packed problem
+        from mamba_amd import _lib
+        lib = _lib.load()
+        a = sc._prepare(x, dt, A, B, C, Q, D, z, dtb, init, seq_idx)
+        ws = sc._workspace(a[0], a[3], Q)
+        out, out_x = torch.empty_like(a[0]), torch.empty_like(a[0])
+        p = _lib.SsdParams()
+        sc._fill_fwd(p, a[0], a[1], a[2], a[3], a[4], Q, a[5], a[6], a[7], a[8], a[9], True, (0.0, float("inf")), ws)
+        p.out, p.out_x = out.data_ptr(), out_x.data_ptr()
+        p.out_bs, p.out_ls, p.out_hs = out.stride(0), out.stride(1), out.stride(2)
+        stream = _lib.current_stream(dev)
+        _lib.check(lib.ssd_combined_fwd(p, stream), "ssd_combined_fwd")
+        scan = event_stats(lambda: _lib.check(lib.ssd_chunk_scan_fwd_fused(p, stream), "ssd_chunk_scan_fwd_fused"))
+    nc = L // Q
+    scan_bytes = 2 * (4 * batch * L * H * P + 2 * batch * L * G * N) + 2 * batch * nc * H * P * N
+    flops = batch * nc * (H * (Q * Q * P + 2 * Q * N * P) + G * Q * Q * N)
+    # fwd+bwd, bf16: reads x, z (fwd), x, z, dout (bwd), writes out, dx, dz = 8 X; B, C read twice + dB, dC = 6 BC; dt 3 T
+    step_bytes = 2 * (8 * batch * L * H * P + 6 * batch * L * G * N + 3 * batch * L * H)
+    prof = "ssd_varlen_b1_l32768_h64_p64_n128_g8_q256_bf16"
+    scan_ms = scan["median"]
     return ({
         "metric": "SSD mamba_chunk_scan_combined packed varlen fwd+bwd tokens/s at 1 GPU", "value": batch * L / sec,
         "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": sec * 1e3,
-        "fwd_ms": fwd_ms, "higher_is_better": True, "dtype": "bf16 in/out, fp32 accumulation", "data": "synthetic",
+        "step_ms": step_stats, "fwd_ms": fwd_ms, "higher_is_better": True, "dtype": "bf16 in/out, fp32 accumulation",
+        "data": "synthetic",
         "config": {"workload": f"Mamba-2 SSD fwd+bwd, packed: 1 row of {nseq} sequences, {L} positions, {H} heads x {P}, "
                                f"d_state {N}, {G} groups, chunk {Q}, initial + final states (benchmark configuration 4)"},
-        "roofline": vs_measured_copy({"bound": "hbm", "kernel": "whole step", "achieved": nbytes / sec / 1e9, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": nbytes / sec / 1e9 / HBM_PEAK_GBS, "traffic": None,
-                     "algorithmic_bytes": nbytes}, dev)})
+        "step_roofline": {"bound": "hbm", "algorithmic_bytes": step_bytes, "achieved": step_bytes / sec / 1e9,
+                          "frac": step_bytes / sec / 1e9 / HBM_PEAK_GBS, "unit": "GB/s",
+                          "traffic": profile_traffic_sum(prof + "_hbm_counters.txt")},
+        "roofline": vs_measured_copy({"bound": "hbm", "kernel": "chunk_scan_fwd_fused_kernel",
+                     "achieved": scan_bytes / scan_ms / 1e6, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": scan_bytes / scan_ms / 1e6 / HBM_PEAK_GBS,
+                     "traffic": profile_traffic(prof + "_hbm_counters.txt", "chunk_scan_fwd_fused_kernel"),
+                     "kernel_ms": scan_ms, "kernel_ms_min_max_n": [scan["min"], scan["max"], scan["n"]],
+                     "algorithmic_bytes": scan_bytes, "algorithmic_flops": flops,
+                     "mfma_tflops": flops / scan_ms / 1e9, "mfma_frac_of_bf16_peak": flops / scan_ms / 1e9 / 2500.0}, dev)})
 
 
 def bench_inner(dev, steps, warmup):
@@ -512,16 +683,16 @@ def bench_inner(dev, steps, warmup):
             v.grad = None
         fwd().backward(dout)
 
-    sec = _timed(step, steps, warmup)
+    sec, step_stats = timed_steps(step, steps, warmup)
     with torch.no_grad():
-        fwd_ms = event_ms(fwd, max(5, min(steps, 50)))
+        fwd_ms = event_ms(fwd)
         xin = xz[:, :di]
         cw = conv_w.squeeze(1)
-        conv_ms = event_ms(lambda: causal_conv1d_fwd(xin, cw, conv_b, activation="silu"), max(5, min(steps, 50)))
+        conv_ms = event_ms(lambda: causal_conv1d_fwd(xin, cw, conv_b, activation="silu"))
     nbytes = 2 * 2 * batch * di * L   # the convolution reads x and writes its output once
     return ({
         "metric": "mamba_inner_fn fwd+bwd tokens/s at 1 GPU", "value": batch * L / sec, "unit": "tokens/s",
-        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": sec * 1e3, "fwd_ms": fwd_ms,
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": sec * 1e3, "step_ms": step_stats, "fwd_ms": fwd_ms,
         "higher_is_better": True, "dtype": "bf16 in/out, fp32 state and accumulation", "data": "synthetic",
         "config": {"workload": f"mamba_inner_fn fwd+bwd: batch {batch}, seqlen {L}, d_model {dm}, d_inner {di}, "
                                f"d_state {N}, dt_rank {R}, conv width {W}"},
@@ -562,17 +733,17 @@ def bench_block(dev, steps, warmup):
             v.grad = None
         fwd().backward(dout)
 
-    sec = _timed(step, steps, warmup)
+    sec, step_stats = timed_steps(step, steps, warmup)
     with torch.no_grad():
-        fwd_ms = event_ms(fwd, max(5, min(steps, 50)))
+        fwd_ms = event_ms(fwd)
         y = rn(batch * L, dim).to(bf)
         zz = rn(batch * L, dim).to(bf)
         norm_ms = event_ms(lambda: _layer_norm_fwd(y, norm_w, None, 1e-6, z=zz, group_size=dim // G,
-                                                   norm_before_gate=False, is_rms_norm=True), max(5, min(steps, 50)))
+                                                   norm_before_gate=False, is_rms_norm=True))
     nbytes = 3 * 2 * batch * L * dim   # the gated norm reads y and z and writes its output once
     return ({
         "metric": "mamba_split_conv1d_scan_combined fwd+bwd tokens/s at 1 GPU", "value": batch * L / sec,
-        "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": sec * 1e3, "fwd_ms": fwd_ms,
+        "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": sec * 1e3, "step_ms": step_stats, "fwd_ms": fwd_ms,
         "higher_is_better": True, "dtype": "bf16 in/out, fp32 accumulation", "data": "synthetic",
         "config": {"workload": f"Mamba-2 block body fwd+bwd: batch {batch}, seqlen {L}, {H} heads x {P}, d_state {N}, "
                                f"{G} group, chunk {Q}, conv width {W}, gated RMSNorm, out_proj to {dm}"},
@@ -598,16 +769,9 @@ def bench_mamba1(dev, steps, warmup):
                                 z=leaves["z"], delta_bias=leaves["delta_bias"], delta_softplus=True)
         out.backward(t["dout"])
 
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed / steps * 1e3
-    tokens_per_s = batch * seqlen / (elapsed / steps)
+    sec, step_stats = timed_steps(step, steps, warmup)
+    ms_per_step = sec * 1e3
+    tokens_per_s = batch * seqlen / sec
 
     # Dominant kernel (the backward scan, with the two small kernels that add up its dB / dC partials) alone,
     # HIP events on the launch stream.
@@ -619,9 +783,8 @@ def bench_mamba1(dev, steps, warmup):
         bufs = ssi.scan_bwd_launch(*bwd_args)
         bwd = lambda: ssi.scan_bwd_launch(*bwd_args, bufs=bufs)
         fwd = lambda: selective_scan_fwd(d["u"], d["delta"], d["A"], d["B"], d["C"], d["D"], d["z"], d["delta_bias"], True)
-        n = max(5, min(steps, 50))
-        bwd_ms = event_ms(bwd, n)
-        fwd_ms = event_ms(fwd, n)
+        bwd_st, fwd_st = event_stats(bwd), event_stats(fwd)
+        bwd_ms, fwd_ms = bwd_st["median"], fwd_st["median"]
     es = 2  # bf16
     E = batch * dim * seqlen * es
     BC = batch * dstate * seqlen * es
@@ -632,8 +795,9 @@ def bench_mamba1(dev, steps, warmup):
     roofline = {"bound": "hbm", "kernel": "scan_bwd_kernel (+ reduce_parts_kernel x 2)", "achieved": achieved,
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                 "traffic": profile_traffic(prof + "_hbm_counters.txt", "scan_bwd_kernel"),
-                "kernel_ms": bwd_ms, "algorithmic_bytes": bwd_bytes,
-                "fwd_kernel_ms": fwd_ms, "fwd_achieved": fwd_bytes / (fwd_ms * 1e-3) / 1e9,
+                "kernel_ms": bwd_ms, "kernel_ms_min_max_n": [bwd_st["min"], bwd_st["max"], bwd_st["n"]],
+                "algorithmic_bytes": bwd_bytes,
+                "fwd_kernel_ms": fwd_ms, "fwd_kernel_ms_min_max_n": [fwd_st["min"], fwd_st["max"], fwd_st["n"]], "fwd_achieved": fwd_bytes / (fwd_ms * 1e-3) / 1e9,
                 "fwd_traffic": profile_traffic(prof + "_hbm_counters.txt", "scan_fwd_kernel"),
                 "fwd_bwd_frac": (fwd_bytes + bwd_bytes) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS}
     vs_measured_copy(roofline, dev)
@@ -660,10 +824,11 @@ def bench_mamba1(dev, steps, warmup):
                       "slots_per_element_state": slots, "achieved": slots * elems / (ms * 1e-3) / 1e12,
                       "frac_of_probe": slots * elems / (ms * 1e-3) / 1e12 / probe}
     roofline["valu"] = valu
+    roofline["profile_is_of_these_sources"] = profile_fresh(prof + "_hbm_counters.txt")
     return {
         "metric": "scan fwd+bwd tokens/s at 1 GPU; achieved HBM GB/s and % bf16 MFMA peak",
         "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": ms_per_step, "step_ms": step_stats, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16 in/out, fp32 state and accumulation", "data": "synthetic",
         "config": {"workload": "Mamba-1 selective_scan_fn fwd+bwd: batch 8, d_inner 5120, seqlen 4096, d_state 16, "
                                "bf16 u/delta/B/C/z, fp32 A/D/delta_bias (benchmark configuration 1)",
@@ -714,7 +879,7 @@ def main():
         # the other benchmark configurations, timed in the same run (each entry is the line its own
         # --workload prints): configuration 2 (SSD, with the MFMA figures), 3 (decode, 1000 consecutive
         # steps) and 4 (packed SSD)
-        keep = ("value", "unit", "ms_per_step", "fwd_ms", "deterministic_ms_per_step", "event_ms_per_step", "steps",
+        keep = ("value", "unit", "ms_per_step", "step_ms", "step_roofline", "fwd_ms", "deterministic_ms_per_step", "event_ms_per_step", "steps",
                 "config", "roofline")
         extra = {}
         for name, fn in (("ssd", lambda: bench_ssd(dev, args.steps, args.warmup)),
@@ -725,6 +890,9 @@ def main():
         result["extra"] = extra
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(4096, 16, 5120)
+        if "extra" in result:
+            result["extra"]["ssd"]["cpu_baseline"] = cpu_baseline_ssd()
+            result["extra"]["decode"]["cpu_baseline"] = cpu_baseline_decode()
     print(json.dumps(result))
 
 

@@ -56,10 +56,13 @@ def selective_scan_oracle(u, delta, A, B, C, D=None, z=None, delta_bias=None, de
     C = per_channel(C)
     h = torch.zeros(batch, dim, n, dtype=A.dtype, device=u.device)
     ys = []
+    # the time axis is taken apart once (unbind) rather than indexed per step: the same arithmetic, but autograd then
+    # gathers the per-step gradients in one pass instead of writing a full-size tensor per step
+    dts, us, Bts, Cts = delta.unbind(2), u.unbind(2), B.unbind(-1), C.unbind(-1)
     for t in range(L):
-        dt = delta[:, :, t, None]                              # (b, d, 1)
-        h = torch.exp(dt * A[None]) * h + (dt * u[:, :, t, None]) * B[:, :, :, t]
-        yt = (h * C[:, :, :, t]).sum(-1)
+        dt = dts[t][:, :, None]                                # (b, d, 1)
+        h = torch.exp(dt * A[None]) * h + (dt * us[t][:, :, None]) * Bts[t]
+        yt = (h * Cts[t]).sum(-1)
         ys.append(2 * yt.real if is_complex else yt)
     y = torch.stack(ys, dim=2)
     if D is not None:
