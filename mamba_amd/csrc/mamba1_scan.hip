@@ -20,6 +20,12 @@
 
 #include <stdlib.h>
 
+#include <algorithm>
+#include <map>
+#include <mutex>
+#include <type_traits>
+#include <utility>
+
 size_t mamba1_bwd_mx_lds(int passes, int np);                                                       // mamba1_scan_bwd_mx.hip
 int mamba1_bwd_mx_launch(const MambaScanParams &p, int passes, bool vec, hipStream_t stream);  // likewise
 
@@ -645,16 +651,37 @@ int bwd_nparts(const MambaScanParams &p) {
   return (Dg + PASS_CH * r - 1) / (PASS_CH * r) * (p.dstate > NB16 ? r : 1);
 }
 
+// Raises a kernel's dynamic LDS limit to `lds` bytes on the current device, once: the largest size granted so far is
+// remembered per (device, kernel), so that repeated launches (and launches under stream capture) make no runtime call.
+}  // namespace
+
+bool mamba1_allow_lds(const void *kernel, size_t lds) {
+  static std::mutex mu;
+  static std::map<std::pair<int, const void *>, size_t> granted;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  size_t &have = granted[{dev, kernel}];
+  if (lds <= have) return true;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  have = lds;
+  return true;
+}
+
+namespace {
+
 template <typename KernelT>
 int launch(KernelT kernel, const MambaScanParams &p, int passes, size_t lds, hipStream_t stream) {
   const int Dg = p.dim / p.ngroups;
   const int cblocks = (Dg + PASS_CH * passes - 1) / (PASS_CH * passes);
   if (lds > LDS_LIMIT) return MAMBA_E_UNSUPPORTED;
-  if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                          (int)lds) != hipSuccess) {
-    (void)hipGetLastError();
-    return MAMBA_E_LAUNCH;
-  }
+  if (!mamba1_allow_lds(reinterpret_cast<const void *>(kernel), lds)) return MAMBA_E_LAUNCH;
   dim3 grid(p.ngroups * cblocks, p.batch), block(NTHREADS);
   hipLaunchKernelGGL(kernel, grid, block, lds, stream, p, passes);
   return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
@@ -664,7 +691,6 @@ int check_common(const MambaScanParams *p) {
   if (!p || !p->u || !p->delta || !p->A || !p->B || !p->C || !p->ckpt) return MAMBA_E_BADARG;
   if (p->batch <= 0 || p->dim <= 0 || p->seqlen <= 0 || p->dstate <= 0 || p->ngroups <= 0) return MAMBA_E_BADARG;
   if (p->dim % p->ngroups != 0) return MAMBA_E_BADARG;
-  if (p->batch > 65535) return MAMBA_E_UNSUPPORTED;
   if (p->dstate > MAX_DSTATE) return MAMBA_E_UNSUPPORTED;
   if (p->dtype != MAMBA_F32 && p->dtype != MAMBA_BF16 && p->dtype != MAMBA_F16) return MAMBA_E_BADARG;
   return MAMBA_OK;
@@ -709,7 +735,9 @@ template <typename T> int reduce_dBC(const MambaScanParams &p, int nparts, hipSt
   return rc;
 }
 
-template <typename T, bool BWD, int BC> int dispatch_bc(const MambaScanParams &p, hipStream_t stream) {
+// `plan`: the whole problem, of which p may be a slice of batch rows; it decides the passes per workgroup and with
+// them the number of dB / dC partials, which must be the same for every slice.
+template <typename T, bool BWD, int BC> int dispatch_bc(const MambaScanParams &p, const MambaScanParams &plan, hipStream_t stream) {
   const int np = (p.dstate + NB16 - 1) / NB16 * NB16;
   const bool vec = vec_ok(p, BWD);
   if (!BWD) {
@@ -717,24 +745,51 @@ template <typename T, bool BWD, int BC> int dispatch_bc(const MambaScanParams &p
     return vec ? launch(scan_fwd_kernel<T, true, BC>, p, 1, lds, stream)
                : launch(scan_fwd_kernel<T, false, BC>, p, 1, lds, stream);
   }
-  const int passes = bwd_passes(p);
+  const int passes = bwd_passes(plan);
   if (use_mx(p)) {
     const int rc = mamba1_bwd_mx_launch(p, passes, vec, stream);
-    return rc != MAMBA_OK ? rc : reduce_dBC<T>(p, bwd_nparts(p), stream);
+    return rc != MAMBA_OK ? rc : reduce_dBC<T>(p, bwd_nparts(plan), stream);
   }
   const size_t lds = bwd_lds(passes, np, BC);
   const int rc = vec ? launch(scan_bwd_kernel<T, true, BC>, p, passes, lds, stream)
                      : launch(scan_bwd_kernel<T, false, BC>, p, passes, lds, stream);
-  return rc != MAMBA_OK ? rc : reduce_dBC<T>(p, bwd_nparts(p), stream);
+  return rc != MAMBA_OK ? rc : reduce_dBC<T>(p, bwd_nparts(plan), stream);
 }
 
-template <typename T, bool BWD> int dispatch(const MambaScanParams &p, hipStream_t stream) {
+template <typename T, bool BWD> int dispatch(const MambaScanParams &p, const MambaScanParams &plan, hipStream_t stream) {
   switch (p.bc_const & 3) {
-    case 0: return dispatch_bc<T, BWD, 0>(p, stream);
-    case 1: return dispatch_bc<T, BWD, 1>(p, stream);
-    case 2: return dispatch_bc<T, BWD, 2>(p, stream);
-    default: return dispatch_bc<T, BWD, 3>(p, stream);
+    case 0: return dispatch_bc<T, BWD, 0>(p, plan, stream);
+    case 1: return dispatch_bc<T, BWD, 1>(p, plan, stream);
+    case 2: return dispatch_bc<T, BWD, 2>(p, plan, stream);
+    default: return dispatch_bc<T, BWD, 3>(p, plan, stream);
   }
+}
+
+// The grid's batch coordinate is 16 bits wide: a larger batch is served in slices of rows (rows are independent; every
+// per-row pointer is advanced, the per-(batch, channel) partial sums included).
+constexpr int MAX_GRID_BATCH = 65535;
+
+MambaScanParams batch_slice(const MambaScanParams &p, int64_t b0, int nb, int nparts) {
+  MambaScanParams q = p;
+  q.batch = nb;
+  const int64_t es = p.dtype == MAMBA_F32 ? 4 : 2, cx = p.a_complex ? 2 : 1;
+  const int tile = p.a_complex ? TILE_COMPLEX : TILE;
+  const int64_t ntiles = (p.seqlen + tile - 1) / tile, N = p.dstate, L = p.seqlen, G = p.ngroups, D = p.dim;
+  auto adv = [&](auto *&ptr, int64_t elems, int64_t size) {
+    if (ptr) ptr = reinterpret_cast<std::remove_reference_t<decltype(ptr)>>(
+                 reinterpret_cast<uintptr_t>(ptr) + (uintptr_t)(b0 * elems * size));
+  };
+  adv(q.u, p.u_bs, es), adv(q.delta, p.delta_bs, es), adv(q.z, p.z_bs, es), adv(q.out, p.out_bs, es);
+  if (!(p.bc_const & 1)) adv(q.B, p.B_bs, es);
+  if (!(p.bc_const & 2)) adv(q.C, p.C_bs, es);
+  adv(q.ckpt, D * ntiles * N * cx, 4);
+  adv(q.dout, p.dout_bs, es), adv(q.du, p.du_bs, es), adv(q.ddelta, p.ddelta_bs, es), adv(q.dz, p.dz_bs, es);
+  adv(q.out_z, p.outz_bs, es);
+  adv(q.dB32, (p.bc_const & 1) ? D * N * cx : G * nparts * N * L * cx, 4);
+  adv(q.dC32, (p.bc_const & 2) ? D * N * cx : G * nparts * N * L * cx, 4);
+  adv(q.dA_part, D * N * cx, 4), adv(q.dD_part, D, 4), adv(q.ddelta_bias_part, D, 4);
+  adv(q.dB, G * N * L * cx, es), adv(q.dC, G * N * L * cx, es);
+  return q;
 }
 
 }  // namespace
@@ -743,17 +798,51 @@ int mamba1_scan_complex(const MambaScanParams *p, hipStream_t s, bool bwd);  // 
 
 int mamba1_scan_tile(bool a_complex) { return a_complex ? TILE_COMPLEX : TILE; }  // positions per checkpoint tile
 
+namespace {
+int scan_fwd_one(const MambaScanParams &p, hipStream_t s) {
+  if (p.a_complex) return mamba1_scan_complex(&p, s, false);
+  switch (p.dtype) {
+    case MAMBA_F32: return dispatch<float, false>(p, p, s);
+    case MAMBA_BF16: return dispatch<bf16_t, false>(p, p, s);
+    default: return dispatch<f16_t, false>(p, p, s);
+  }
+}
+
+int scan_bwd_one(const MambaScanParams &p, const MambaScanParams &plan, mamba_stream_t stream) {
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (p.a_complex) {
+    // the complex kernels add their dB / dC terms into one fp32 copy with atomics: clear it, run, convert
+    const int64_t bytes = (int64_t)p.batch * p.ngroups * p.dstate * 2 * p.seqlen * 4;
+    int rc = MAMBA_OK;
+    if (!(p.bc_const & 1)) rc = mamba_hip_zero(p.dB32, bytes, stream);
+    if (rc == MAMBA_OK && !(p.bc_const & 2)) rc = mamba_hip_zero(p.dC32, bytes, stream);
+    if (rc == MAMBA_OK) rc = mamba1_scan_complex(&p, s, true);
+    if (rc != MAMBA_OK) return rc;
+    switch (p.dtype) {
+      case MAMBA_F32: return reduce_dBC<float>(p, 1, s);
+      case MAMBA_BF16: return reduce_dBC<bf16_t>(p, 1, s);
+      default: return reduce_dBC<f16_t>(p, 1, s);
+    }
+  }
+  switch (p.dtype) {
+    case MAMBA_F32: return dispatch<float, true>(p, plan, s);
+    case MAMBA_BF16: return dispatch<bf16_t, true>(p, plan, s);
+    default: return dispatch<f16_t, true>(p, plan, s);
+  }
+}
+}  // namespace
+
 extern "C" int mamba1_scan_fwd(const MambaScanParams *p, mamba_stream_t stream) {
   int rc = check_common(p);
   if (rc != MAMBA_OK) return rc;
   if (!p->out) return MAMBA_E_BADARG;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (p->a_complex) return mamba1_scan_complex(p, s, false);
-  switch (p->dtype) {
-    case MAMBA_F32: return dispatch<float, false>(*p, s);
-    case MAMBA_BF16: return dispatch<bf16_t, false>(*p, s);
-    default: return dispatch<f16_t, false>(*p, s);
+  for (int64_t b0 = 0; b0 < p->batch; b0 += MAX_GRID_BATCH) {
+    const int nb = (int)std::min<int64_t>(MAX_GRID_BATCH, p->batch - b0);
+    rc = p->batch <= MAX_GRID_BATCH ? scan_fwd_one(*p, s) : scan_fwd_one(batch_slice(*p, b0, nb, 1), s);
+    if (rc != MAMBA_OK) return rc;
   }
+  return MAMBA_OK;
 }
 
 // ----------------------------------------------------- forward without a caller workspace
@@ -833,23 +922,11 @@ extern "C" int mamba1_scan_bwd(const MambaScanParams *p, mamba_stream_t stream) 
     return MAMBA_E_BADARG;
   if ((!(p->bc_const & 1) && !p->dB) || (!(p->bc_const & 2) && !p->dC)) return MAMBA_E_BADARG;
   if (p->z && !p->dz) return MAMBA_E_BADARG;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  if (p->a_complex) {
-    // the complex kernels add their dB / dC terms into one fp32 copy with atomics: clear it, run, convert
-    const int64_t bytes = (int64_t)p->batch * p->ngroups * p->dstate * 2 * p->seqlen * 4;
-    if (!(p->bc_const & 1)) rc = mamba_hip_zero(p->dB32, bytes, stream);
-    if (rc == MAMBA_OK && !(p->bc_const & 2)) rc = mamba_hip_zero(p->dC32, bytes, stream);
-    if (rc == MAMBA_OK) rc = mamba1_scan_complex(p, s, true);
+  const int nparts = p->a_complex ? 1 : bwd_nparts(*p);
+  for (int64_t b0 = 0; b0 < p->batch; b0 += MAX_GRID_BATCH) {
+    const int nb = (int)std::min<int64_t>(MAX_GRID_BATCH, p->batch - b0);
+    rc = p->batch <= MAX_GRID_BATCH ? scan_bwd_one(*p, *p, stream) : scan_bwd_one(batch_slice(*p, b0, nb, nparts), *p, stream);
     if (rc != MAMBA_OK) return rc;
-    switch (p->dtype) {
-      case MAMBA_F32: return reduce_dBC<float>(*p, 1, s);
-      case MAMBA_BF16: return reduce_dBC<bf16_t>(*p, 1, s);
-      default: return reduce_dBC<f16_t>(*p, 1, s);
-    }
   }
-  switch (p->dtype) {
-    case MAMBA_F32: return dispatch<float, true>(*p, s);
-    case MAMBA_BF16: return dispatch<bf16_t, true>(*p, s);
-    default: return dispatch<f16_t, true>(*p, s);
-  }
+  return MAMBA_OK;
 }

@@ -409,6 +409,8 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_mx_kernel(const MambaScanPa
 
 }  // namespace
 
+bool mamba1_allow_lds(const void *kernel, size_t lds);  // mamba1_scan.hip
+
 // LDS bytes of the kernel above for `passes` passes of PASS_CH channels and `np` padded states.
 size_t mamba1_bwd_mx_lds(int passes, int np) {
   const int wch = passes * PASS_CH;
@@ -425,11 +427,7 @@ int mamba1_bwd_mx_launch(const MambaScanParams &p, int passes, bool vec, hipStre
   const int cblocks = (Dg + PASS_CH * passes - 1) / (PASS_CH * passes);
   auto kernel = p.z ? (vec ? scan_bwd_mx_kernel<bf16_t, true, true> : scan_bwd_mx_kernel<bf16_t, false, true>)
                     : (vec ? scan_bwd_mx_kernel<bf16_t, true, false> : scan_bwd_mx_kernel<bf16_t, false, false>);
-  if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                          (int)lds) != hipSuccess) {
-    (void)hipGetLastError();
-    return MAMBA_E_LAUNCH;
-  }
+  if (!mamba1_allow_lds(reinterpret_cast<const void *>(kernel), lds)) return MAMBA_E_LAUNCH;
   dim3 grid(p.ngroups * cblocks, p.batch), block(NTHREADS);
   hipLaunchKernelGGL(kernel, grid, block, lds, stream, p, passes);
   return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;

@@ -1366,7 +1366,7 @@ inline int tiles(int n) { return (n + GB - 1) / GB; }
 
 }  // namespace
 
-extern "C" int ssd_bwd_dz(const SsdParams *p, mamba_stream_t stream) {
+static int ssd_bwd_dz_one(const SsdParams *p, mamba_stream_t stream) {
   int rc = check_bwd(p);
   if (rc) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -1379,7 +1379,7 @@ extern "C" int ssd_bwd_dz(const SsdParams *p, mamba_stream_t stream) {
   return launched();
 }
 
-extern "C" int ssd_bwd_dstates(const SsdParams *p, mamba_stream_t stream) {
+static int ssd_bwd_dstates_one(const SsdParams *p, mamba_stream_t stream) {
   int rc = check_bwd(p);
   if (rc) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -1399,7 +1399,7 @@ extern "C" int ssd_bwd_dstates(const SsdParams *p, mamba_stream_t stream) {
   return launched();
 }
 
-extern "C" int ssd_state_passing_bwd(const SsdParams *p, mamba_stream_t stream) {
+static int ssd_state_passing_bwd_one(const SsdParams *p, mamba_stream_t stream) {
   int rc = check_bwd(p);
   if (rc) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -1420,7 +1420,7 @@ extern "C" int ssd_state_passing_bwd(const SsdParams *p, mamba_stream_t stream) 
   return launched();
 }
 
-extern "C" int ssd_bwd_dx(const SsdParams *p, mamba_stream_t stream) {
+static int ssd_bwd_dx_one(const SsdParams *p, mamba_stream_t stream) {
   int rc = check_bwd(p);
   if (rc) return rc;
   if (p->dx_ls < (int64_t)p->headdim || p->dx_hs < (int64_t)p->headdim) return MAMBA_E_BADARG;  // strides not filled in
@@ -1433,7 +1433,7 @@ extern "C" int ssd_bwd_dx(const SsdParams *p, mamba_stream_t stream) {
   return launched();
 }
 
-extern "C" int ssd_bwd_dBC_state(const SsdParams *p, mamba_stream_t stream) {
+static int ssd_bwd_dBC_state_one(const SsdParams *p, mamba_stream_t stream) {
   int rc = check_bwd(p);
   if (rc) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -1461,7 +1461,7 @@ extern "C" int ssd_bwd_dBC_state(const SsdParams *p, mamba_stream_t stream) {
   return launched();
 }
 
-extern "C" int ssd_bwd_dcb(const SsdParams *p, mamba_stream_t stream) {
+static int ssd_bwd_dcb_one(const SsdParams *p, mamba_stream_t stream) {
   int rc = check_bwd(p);
   if (rc) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -1471,7 +1471,7 @@ extern "C" int ssd_bwd_dcb(const SsdParams *p, mamba_stream_t stream) {
   return launched();
 }
 
-extern "C" int ssd_bmm_chunk_bwd(const SsdParams *p, mamba_stream_t stream) {
+static int ssd_bmm_chunk_bwd_one(const SsdParams *p, mamba_stream_t stream) {
   int rc = check_bwd(p);
   if (rc) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -1487,7 +1487,7 @@ extern "C" int ssd_bmm_chunk_bwd(const SsdParams *p, mamba_stream_t stream) {
   return launched();
 }
 
-extern "C" int ssd_chunk_cumsum_bwd(const SsdParams *p, mamba_stream_t stream) {
+static int ssd_chunk_cumsum_bwd_one(const SsdParams *p, mamba_stream_t stream) {
   int rc = check_bwd(p);
   if (rc) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -1559,7 +1559,7 @@ static int dz_and_dstates(const SsdParams *p, mamba_stream_t stream) {
   return ssd_bwd_dstates(p, stream);
 }
 
-extern "C" int ssd_combined_bwd(const SsdParams *p, mamba_stream_t stream) {
+static int ssd_combined_bwd_one(const SsdParams *p, mamba_stream_t stream) {
   int rc;
   if (p && p->det_scale) {
     // deterministic mode: every shared sum goes through its integer shadow
@@ -1597,3 +1597,14 @@ extern "C" int ssd_combined_bwd(const SsdParams *p, mamba_stream_t stream) {
   if ((rc = ssd_bwd_dcb(p, stream))) return rc;
   return bmm_and_cumsum_bwd(p, stream);
 }
+
+// Public entry points: the whole problem in one go when one launch can index it, else in slices of batch rows.
+extern "C" int ssd_bwd_dz(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_bwd_dz_one); }
+extern "C" int ssd_bwd_dstates(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_bwd_dstates_one); }
+extern "C" int ssd_state_passing_bwd(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_state_passing_bwd_one); }
+extern "C" int ssd_bwd_dx(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_bwd_dx_one); }
+extern "C" int ssd_bwd_dBC_state(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_bwd_dBC_state_one); }
+extern "C" int ssd_bwd_dcb(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_bwd_dcb_one); }
+extern "C" int ssd_bmm_chunk_bwd(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_bmm_chunk_bwd_one); }
+extern "C" int ssd_chunk_cumsum_bwd(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_chunk_cumsum_bwd_one); }
+extern "C" int ssd_combined_bwd(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_combined_bwd_one); }

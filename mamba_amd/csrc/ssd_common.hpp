@@ -11,6 +11,7 @@
 // (hi*hi + hi*lo + lo*hi); bf16 inputs need one.
 #pragma once
 #include "common.hpp"
+#include <algorithm>
 #include <type_traits>
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -770,4 +771,49 @@ inline int heads_per_workgroup(const SsdParams &p) {
     if (cost < best_cost - 1e-9) best = hb, best_cost = cost;
   }
   return best;
+}
+
+// ------------------------------------------------------------------ batch slices
+// The kernels index (batch, head) pairs with one 16-bit grid coordinate.  A larger problem is served by the entry
+// points in slices of whole batch rows (rows are independent; the sums shared by all rows -- dA, dD, ddt_bias and
+// their integer shadows -- are added into by every slice): the same parameters with every per-row pointer advanced.
+constexpr int64_t SSD_MAX_GRID_ROWS = 65535;
+
+inline SsdParams ssd_batch_slice(const SsdParams &p, int64_t b0, int nb) {
+  SsdParams q = p;
+  q.batch = nb;
+  const int64_t es = p.dtype == MAMBA_F32 ? 4 : 2, ds = p.dt_dtype == MAMBA_F32 ? 4 : 2;
+  const int64_t H = p.nheads, P = p.headdim, N = p.dstate, G = p.ngroups, L = p.seqlen, Q = p.chunk_size, c = p.nchunks;
+  auto adv = [&](auto *&ptr, int64_t elems, int64_t size) {
+    if (ptr) ptr = reinterpret_cast<std::remove_reference_t<decltype(ptr)>>(
+                 reinterpret_cast<uintptr_t>(ptr) + (uintptr_t)(b0 * elems * size));
+  };
+  adv(q.x, p.x_bs, es), adv(q.z, p.z_bs, es), adv(q.out, p.out_bs, es), adv(q.out_x, p.out_bs, es);
+  adv(q.B, p.B_bs, es), adv(q.C, p.C_bs, es), adv(q.dt, p.dt_bs, ds);
+  adv(q.initial_states, H * P * N, 4), adv(q.seq_idx, L, 4);
+  adv(q.dt_out, H * c * Q, 4), adv(q.dA_cumsum, H * c * Q, 4);
+  adv(q.states, c * H * P * N, 4), adv(q.states_lp, c * H * P * N, 2), adv(q.final_states, H * P * N, 4);
+  adv(q.CB, c * G * Q * Q, 4);
+  adv(q.dout, p.dout_bs, es), adv(q.dfinal_states, H * P * N, 4), adv(q.dx, p.dx_bs, es), adv(q.dz, L * H * P, es);
+  adv(q.ddt, L * H, ds), adv(q.dB, L * G * N, es), adv(q.dC, L * G * N, es), adv(q.dinitial_states, H * P * N, 4);
+  adv(q.dstates, c * H * P * N, 4), adv(q.dstates_lp, c * H * P * N, 2);
+  adv(q.ddA_cumsum, H * c * Q, 4), adv(q.ddt_out, H * c * Q, 4), adv(q.dCB, c * G * Q * Q, 4);
+  adv(q.dB32, L * G * N, 4), adv(q.dC32, L * G * N, 4), adv(q.gbuf, L * H * P, es);
+  adv(q.det_ddA_cumsum, H * c * Q, 8), adv(q.det_ddt_out, H * c * Q, 8), adv(q.det_dCB, c * G * Q * Q, 8);
+  adv(q.det_dB, L * G * N, 8), adv(q.det_dC, L * G * N, 8);
+  return q;
+}
+
+// Runs `one` on the whole problem when one launch can index it, else on slices of whole batch rows.
+template <typename F> inline int ssd_sliced(const SsdParams *p, mamba_stream_t stream, F one) {
+  if (!p || p->batch <= 0 || p->nheads <= 0 || p->nheads > SSD_MAX_GRID_ROWS ||
+      (int64_t)p->batch * p->nheads <= SSD_MAX_GRID_ROWS)
+    return one(p, stream);
+  const int rows = (int)(SSD_MAX_GRID_ROWS / p->nheads);
+  for (int64_t b0 = 0; b0 < p->batch; b0 += rows) {
+    const SsdParams q = ssd_batch_slice(*p, b0, (int)std::min<int64_t>(rows, p->batch - b0));
+    const int rc = one(&q, stream);
+    if (rc) return rc;
+  }
+  return MAMBA_OK;
 }

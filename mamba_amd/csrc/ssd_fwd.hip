@@ -436,7 +436,7 @@ int launched() { return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAU
 
 }  // namespace
 
-extern "C" int ssd_chunk_cumsum_fwd(const SsdParams *p, mamba_stream_t stream) {
+static int ssd_chunk_cumsum_fwd_one(const SsdParams *p, mamba_stream_t stream) {
   int rc = check(p);
   if (rc) return rc;
   if (!p->dt_out || !p->dA_cumsum) return MAMBA_E_BADARG;
@@ -446,7 +446,7 @@ extern "C" int ssd_chunk_cumsum_fwd(const SsdParams *p, mamba_stream_t stream) {
   return launched();
 }
 
-extern "C" int ssd_bmm_chunk_fwd(const SsdParams *p, mamba_stream_t stream) {
+static int ssd_bmm_chunk_fwd_one(const SsdParams *p, mamba_stream_t stream) {
   int rc = check(p);
   if (rc) return rc;
   if (!p->CB) return MAMBA_E_BADARG;
@@ -457,7 +457,7 @@ extern "C" int ssd_bmm_chunk_fwd(const SsdParams *p, mamba_stream_t stream) {
   return launched();
 }
 
-extern "C" int ssd_chunk_state_fwd(const SsdParams *p, mamba_stream_t stream) {
+static int ssd_chunk_state_fwd_one(const SsdParams *p, mamba_stream_t stream) {
   int rc = check(p);
   if (rc) return rc;
   if (!p->states || !p->dt_out || !p->dA_cumsum) return MAMBA_E_BADARG;
@@ -502,7 +502,7 @@ extern "C" int ssd_chunk_state_varlen(const SsdParams *p, const int32_t *cu_seql
   return launched();
 }
 
-extern "C" int ssd_state_passing_fwd(const SsdParams *p, mamba_stream_t stream) {
+static int ssd_state_passing_fwd_one(const SsdParams *p, mamba_stream_t stream) {
   int rc = check(p);
   if (rc) return rc;
   if (!p->states || !p->final_states || !p->dA_cumsum) return MAMBA_E_BADARG;
@@ -523,7 +523,7 @@ extern "C" int ssd_state_passing_fwd(const SsdParams *p, mamba_stream_t stream) 
   return launched();
 }
 
-extern "C" int ssd_chunk_scan_fwd(const SsdParams *p, mamba_stream_t stream) {
+static int ssd_chunk_scan_fwd_one(const SsdParams *p, mamba_stream_t stream) {
   int rc = check(p);
   if (rc) return rc;
   if (!p->CB || !p->out || !p->dt_out || !p->dA_cumsum) return MAMBA_E_BADARG;
@@ -534,7 +534,7 @@ extern "C" int ssd_chunk_scan_fwd(const SsdParams *p, mamba_stream_t stream) {
   return launched();
 }
 
-extern "C" int ssd_combined_fwd(const SsdParams *p, mamba_stream_t stream) {
+static int ssd_combined_fwd_one(const SsdParams *p, mamba_stream_t stream) {
   int rc;
   if ((rc = ssd_chunk_cumsum_fwd(p, stream))) return rc;
   if ((rc = ssd_chunk_state_fwd(p, stream))) return rc;
@@ -543,3 +543,11 @@ extern "C" int ssd_combined_fwd(const SsdParams *p, mamba_stream_t stream) {
   if ((rc = ssd_bmm_chunk_fwd(p, stream))) return rc;
   return ssd_chunk_scan_fwd(p, stream);
 }
+
+// Public entry points: the whole problem in one go when one launch can index it, else in slices of batch rows.
+extern "C" int ssd_chunk_cumsum_fwd(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_chunk_cumsum_fwd_one); }
+extern "C" int ssd_bmm_chunk_fwd(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_bmm_chunk_fwd_one); }
+extern "C" int ssd_chunk_state_fwd(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_chunk_state_fwd_one); }
+extern "C" int ssd_state_passing_fwd(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_state_passing_fwd_one); }
+extern "C" int ssd_chunk_scan_fwd(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_chunk_scan_fwd_one); }
+extern "C" int ssd_combined_fwd(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_combined_fwd_one); }

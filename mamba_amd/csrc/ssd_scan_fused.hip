@@ -352,9 +352,12 @@ extern "C" int ssd_chunk_scan_fwd_fused_supported(const SsdParams *p) {
   return 1;
 }
 
-extern "C" int ssd_chunk_scan_fwd_fused(const SsdParams *p, mamba_stream_t stream) {
+static int ssd_chunk_scan_fwd_fused_one(const SsdParams *p, mamba_stream_t stream) {
   if (!p || !p->x || !p->B || !p->C || !p->states_lp || !p->out || !p->dt_out || !p->dA_cumsum) return MAMBA_E_BADARG;
   if (!ssd_chunk_scan_fwd_fused_supported(p)) return MAMBA_E_UNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
   return p->headdim == 64 ? launch_n<4>(*p, s) : launch_n<2>(*p, s);
 }
+
+// Public entry points: the whole problem in one go when one launch can index it, else in slices of batch rows.
+extern "C" int ssd_chunk_scan_fwd_fused(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_chunk_scan_fwd_fused_one); }

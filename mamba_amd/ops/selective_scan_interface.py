@@ -109,6 +109,12 @@ def selective_scan_fwd(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta
     `ckpt` is (batch, dim, ntiles, dstate) fp32, the state after each tile of `scan_tile()` positions
     (ckpt[:, :, -1] is the last state).  The ungated y is not stored: the backward pass re-computes it.
     """
+    ext = _lib.torch_ext()
+    if ext is not None and not A.is_complex():
+        # the same checks, allocations and launch in C++ (csrc/torch_ext.cpp); None = a case for the code below
+        r = ext.scan_fwd(u, delta, A, B, C, D, z, delta_bias, bool(delta_softplus))
+        if r is not None:
+            return r
     dims = _check_inputs(u, delta, A, B, C, D, z, delta_bias)
     batch, dim, seqlen, dstate, _ = dims
     A = A.contiguous()
@@ -199,6 +205,11 @@ def selective_scan_bwd(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, dz=None,
     Returns (du, ddelta, dA, dB, dC, dD, ddelta_bias, dz, out_z).  No float atomics are involved: the
     same inputs give the same bits every time.
     """
+    ext = _lib.torch_ext()
+    if ext is not None and not A.is_complex():
+        r = ext.scan_bwd(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, dz, bool(delta_softplus), bool(recompute_out_z))
+        if r is not None:
+            return tuple(r)
     dims = _check_inputs(u, delta, A, B, C, D, z, delta_bias)
     batch, dim, seqlen, dstate, ngroups = dims
     _lib.require_gpu(dout, ckpt, dz)
@@ -271,27 +282,13 @@ class SelectiveScanFn(torch.autograd.Function):
         return (du, ddelta, dA, dB, dC, dD, dz, ddelta_bias, None, None)
 
 
-MAX_GRID_BATCH = 65535  # batch rows per launch of the scan kernels
-
-
 def selective_scan_fn(u, delta, A, B, C, D=None, z=None, delta_bias=None, delta_softplus=False,
                       return_last_state=False):
     """if return_last_state is True, returns (out, last_state)
     last_state has shape (batch, dim, dstate). The gradient of the last state is not
     considered in the backward pass (as in the reference, selective_scan_interface.py:118-124).
     """
-    if u.shape[0] > MAX_GRID_BATCH:
-        # the kernels index the batch with one 16-bit grid coordinate: larger batches go in slices (batch rows
-        # are independent; autograd adds up the gradients of the shared A, D, delta_bias and constant B / C)
-        outs = []
-        for i in range(0, u.shape[0], MAX_GRID_BATCH):
-            sl = slice(i, i + MAX_GRID_BATCH)
-            cut = lambda t: t if t is None or t.dim() == 2 else t[sl]
-            outs.append(selective_scan_fn(u[sl], delta[sl], A, cut(B), cut(C), D, None if z is None else z[sl],
-                                          delta_bias, delta_softplus, return_last_state))
-        if return_last_state:
-            return torch.cat([o[0] for o in outs]), torch.cat([o[1] for o in outs])
-        return torch.cat(outs)
+    # (batches beyond the 65535 rows one launch's grid can index are served in slices inside the C entry points)
     return SelectiveScanFn.apply(u, delta, A, B, C, D, z, delta_bias, delta_softplus, return_last_state)
 
 

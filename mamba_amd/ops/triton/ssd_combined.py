@@ -129,6 +129,13 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
     seventh element,
     varlen_states (nseq, nheads, headdim, dstate): the state at the end of every packed sequence
     (ssd_combined.py:390-394), in state_dtype, else C's dtype, as the reference returns it."""
+    ext = _lib.torch_ext()
+    if ext is not None and cu_seqlens is None:
+        # the same checks, allocations and launch in C++ (csrc/torch_ext.cpp); None = a case for the code below
+        r = ext.ssd_fwd(x, dt, A, B, C, int(chunk_size), D, z, dt_bias, initial_states, seq_idx, bool(dt_softplus),
+                        float(dt_limit[0]), float(dt_limit[1]), bool(want_out_x))
+        if r is not None:
+            return tuple(r)
     state_out_dtype = state_dtype if state_dtype is not None else C.dtype
     x, dt, A, B, C, D, z, dt_bias, initial_states, seq_idx = _prepare(
         x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, seq_idx)
@@ -165,6 +172,13 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
     be caller-owned views (slices of a wider gradient buffer, unit stride in the last dimension), as the
     reference's fused block function passes them (ssd_combined.py:934-944).
     Returns (dx, ddt, dA, dB, dC, dD, dz, ddt_bias, dinitial_states)."""
+    ext = _lib.torch_ext()
+    if (ext is not None and saved is not None and dx is None and ddt is None and dB is None and dC is None
+            and not use_deterministic_mode()):
+        r = ext.ssd_bwd(dout, x, dt, A, B, C, out, int(chunk_size), D, z, dt_bias, initial_states, dfinal_states, seq_idx,
+                        bool(dt_softplus), float(dt_limit[0]), float(dt_limit[1]), saved[0], saved[1], saved[2])
+        if r is not None:
+            return tuple(r)
     in_dtypes = (A.dtype, D.dtype if D is not None else None, dt_bias.dtype if dt_bias is not None else None,
                  initial_states.dtype if initial_states is not None else None, B.dtype, C.dtype)
     D_shape = D.shape if D is not None else None
@@ -310,9 +324,6 @@ class MambaChunkScanCombinedFn(torch.autograd.Function):
                 None)
 
 
-MAX_GRID_ROWS = 65535  # (batch, head) pairs per launch of the SSD kernels
-
-
 def mamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, initial_states=None,
                               seq_idx=None, cu_seqlens=None, dt_softplus=False, dt_limit=(0.0, float("inf")),
                               return_final_states=False, return_varlen_states=False, state_dtype=None):
@@ -335,22 +346,7 @@ def mamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bia
     Return:
         out: (batch, seqlen, nheads, headdim) [, final_states (batch, nheads, headdim, dstate) fp32]
     """
-    batch, nheads = x.shape[0], x.shape[2]
-    rows = MAX_GRID_ROWS // max(nheads, 1)
-    if batch > rows >= 1 and not return_varlen_states:
-        # the kernels index (batch, head) pairs with one 16-bit grid coordinate: larger batches go in slices
-        # (batch rows are independent; autograd adds up the gradients of the shared A, D, dt_bias)
-        outs = []
-        for i in range(0, batch, rows):
-            sl = slice(i, i + rows)
-            cut = lambda t: None if t is None else t[sl]
-            outs.append(mamba_chunk_scan_combined(x[sl], dt[sl], A, B[sl], C[sl], chunk_size, D=D, z=cut(z), dt_bias=dt_bias,
-                                                  initial_states=cut(initial_states), seq_idx=cut(seq_idx),
-                                                  dt_softplus=dt_softplus, dt_limit=dt_limit,
-                                                  return_final_states=return_final_states, state_dtype=state_dtype))
-        if return_final_states:
-            return torch.cat([o[0] for o in outs]), torch.cat([o[1] for o in outs])
-        return torch.cat(outs)
+    # (more than 65535 (batch, head) pairs are served in slices of batch rows inside the C entry points)
     return MambaChunkScanCombinedFn.apply(x, dt, A, B, C, chunk_size, D, z, dt_bias, initial_states, seq_idx,
                                           cu_seqlens, dt_softplus, dt_limit, return_final_states,
                                           return_varlen_states, state_dtype)
