@@ -98,7 +98,8 @@ int64_t mamba_hip_valu_probe(float *sink, int iters, int blocks, mamba_stream_t 
  * backward pass re-computes the states inside a tile from ckpt.
  *
  * Backward: no float atomics are used for a real A, so every gradient repeats bit for bit from run to
- * run (the reference's deterministic mode, mamba_ssm/utils/determinism.py:21-27, is the only mode).
+ * run (the reference's deterministic mode, mamba_ssm/utils/determinism.py:21-27, is the only mode); with a
+ * complex A the det_* fields at the end of the struct select it.
  * ------------------------------------------------------------------------- */
 typedef struct MambaScanParams {
   int32_t batch, dim, seqlen, dstate, ngroups;
@@ -140,6 +141,16 @@ typedef struct MambaScanParams {
   /* gradients of per-position B and C: (batch, ngroups, dstate, seqlen) of `dtype`, contiguous
    * ((..., 2 * seqlen) with a complex A) */
   void *dB, *dC;
+  /* ---- deterministic backward with a complex A (all null: float atomics there; a real A needs none of this, its
+   * backward pass has no atomics) ----
+   * The complex kernels add every channel's dB / dC terms into one sum per (batch, group, state, position).  With
+   * det_scale set (device, {s, 1 / s}, s a power of two chosen by the caller as for SsdParams.det_scale) every term
+   * is multiplied by s, rounded to an integer and added with a 64-bit integer atomic into det_dB / det_dC, int64
+   * shadows of dB32 / dC32 (same shape, zero on entry; used for per-position operands only); the call converts them
+   * into dB32 / dC32 before it forms dB / dC.  Counterpart of the reference's deterministic mode,
+   * mamba_ssm/utils/determinism.py:21-27. */
+  const float *det_scale;
+  int64_t *det_dB, *det_dC;
 } MambaScanParams;
 
 int mamba1_scan_fwd(const MambaScanParams *p, mamba_stream_t stream);

@@ -28,7 +28,7 @@ class MambaScanParams(ctypes.Structure):
                                "ddelta_bias_part")]
         + [(n, c_i64) for n in ("dout_bs", "dout_ds", "du_bs", "du_ds", "ddelta_bs", "ddelta_ds", "dz_bs", "dz_ds",
                                 "outz_bs", "outz_ds")]
-        + [("dB", c_vp), ("dC", c_vp)]
+        + [("dB", c_vp), ("dC", c_vp), ("det_scale", c_vp), ("det_dB", c_vp), ("det_dC", c_vp)]
     )
 
 

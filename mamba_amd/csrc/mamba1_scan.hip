@@ -789,6 +789,7 @@ MambaScanParams batch_slice(const MambaScanParams &p, int64_t b0, int nb, int np
   adv(q.dC32, (p.bc_const & 2) ? D * N * cx : G * nparts * N * L * cx, 4);
   adv(q.dA_part, D * N * cx, 4), adv(q.dD_part, D, 4), adv(q.ddelta_bias_part, D, 4);
   adv(q.dB, G * N * L * cx, es), adv(q.dC, G * N * L * cx, es);
+  adv(q.det_dB, G * N * L * cx, 8), adv(q.det_dC, G * N * L * cx, 8);
   return q;
 }
 
@@ -816,7 +817,12 @@ int scan_bwd_one(const MambaScanParams &p, const MambaScanParams &plan, mamba_st
     int rc = MAMBA_OK;
     if (!(p.bc_const & 1)) rc = mamba_hip_zero(p.dB32, bytes, stream);
     if (rc == MAMBA_OK && !(p.bc_const & 2)) rc = mamba_hip_zero(p.dC32, bytes, stream);
+    if (p.det_scale && ((!(p.bc_const & 1) && !p.det_dB) || (!(p.bc_const & 2) && !p.det_dC))) return MAMBA_E_BADARG;
     if (rc == MAMBA_OK) rc = mamba1_scan_complex(&p, s, true);
+    if (rc == MAMBA_OK && p.det_scale) {  // the integer sums -> the fp32 sums the conversion below reads
+      if (!(p.bc_const & 1)) rc = ssd_det_convert(p.det_dB, p.dB32, bytes / 4, p.det_scale, stream);
+      if (rc == MAMBA_OK && !(p.bc_const & 2)) rc = ssd_det_convert(p.det_dC, p.dC32, bytes / 4, p.det_scale, stream);
+    }
     if (rc != MAMBA_OK) return rc;
     switch (p.dtype) {
       case MAMBA_F32: return reduce_dBC<float>(p, 1, s);

@@ -116,6 +116,19 @@ DEVI Geo geometry(const MambaScanParams &p, int wave) {
   return q;
 }
 
+// One term of a sum that every channel of a group adds into: a float atomic, or (dsc != 0) a 64-bit integer atomic
+// on the term scaled to a fixed point, whose result does not depend on the order of the adds.
+DEVI void add_term(float *dst, int64_t *shadow, int64_t idx, float v, float dsc) {
+  if (dsc != 0.f) {
+    const float q = fminf(fmaxf(v * dsc, -9.0e18f), 9.0e18f);
+    __hip_atomic_fetch_add(reinterpret_cast<unsigned long long *>(shadow + idx),
+                           static_cast<unsigned long long>(static_cast<long long>(__builtin_rintf(q))), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+  } else {
+    unsafeAtomicAdd(dst + idx, v);
+  }
+}
+
 // ------------------------------------------------------------------ forward
 template <typename T, bool VEC, int BC> __global__ __launch_bounds__(NW * 64) void cscan_fwd_kernel(const MambaScanParams p) {
   __shared__ cx hcar[NW][MAXN];  // state carried across tiles
@@ -207,6 +220,10 @@ template <typename T, bool VEC, int BC> __global__ __launch_bounds__(NW * 64) vo
   const float *Ad = (const float *)p.A + (int64_t)d * N * 2;
   float *dBg = p.dB32 + ((int64_t)b * p.ngroups + q.g) * N * 2 * L;  // (batch, ngroups, dstate, 2 L)
   float *dCg = p.dC32 + ((int64_t)b * p.ngroups + q.g) * N * 2 * L;
+  // deterministic mode: the same sums as 64-bit integers of fixed-point terms (order-independent)
+  const float dsc = p.det_scale ? p.det_scale[0] : 0.f;
+  int64_t *det_dBg = p.det_dB ? p.det_dB + ((int64_t)b * p.ngroups + q.g) * N * 2 * L : nullptr;
+  int64_t *det_dCg = p.det_dC ? p.det_dC + ((int64_t)b * p.ngroups + q.g) * N * 2 * L : nullptr;
   for (int n = lane; n < N; n += 64) {
     gcar[wave][n] = anx[wave][n] = dAacc[wave][n] = dBcacc[wave][n] = dCcacc[wave][n] = {0.f, 0.f};
   }
@@ -296,15 +313,15 @@ template <typename T, bool VEC, int BC> __global__ __launch_bounds__(NW * 64) vo
           dCp.r += dC.r;
           dCp.i += dC.i;
         } else if (i < nvalid) {
-          unsafeAtomicAdd(dCg + (int64_t)n * 2 * L + 2 * (tl + i), dC.r);
-          unsafeAtomicAdd(dCg + (int64_t)n * 2 * L + 2 * (tl + i) + 1, dC.i);
+          add_term(dCg, det_dCg, (int64_t)n * 2 * L + 2 * (tl + i), dC.r, dsc);
+          add_term(dCg, det_dCg, (int64_t)n * 2 * L + 2 * (tl + i) + 1, dC.i, dsc);
         }
         if constexpr (BC & 1) {
           dBp.r += dB.r;
           dBp.i += dB.i;
         } else if (i < nvalid) {
-          unsafeAtomicAdd(dBg + (int64_t)n * 2 * L + 2 * (tl + i), dB.r);
-          unsafeAtomicAdd(dBg + (int64_t)n * 2 * L + 2 * (tl + i) + 1, dB.i);
+          add_term(dBg, det_dBg, (int64_t)n * 2 * L + 2 * (tl + i), dB.r, dsc);
+          add_term(dBg, det_dBg, (int64_t)n * 2 * L + 2 * (tl + i) + 1, dB.i, dsc);
         }
         acc[i] += Bv[i].r * g.r + Bv[i].i * g.i;                      // Re(conj(B) g)
         const cx w = cmul(cconj(cx{h[i].r - bb[i].r, h[i].i - bb[i].i}), g);  // conj(a h[t-1]) g

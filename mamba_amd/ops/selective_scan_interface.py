@@ -16,6 +16,7 @@ from einops import rearrange
 
 from mamba_amd import _lib
 from mamba_amd.ops.causal_conv1d import causal_conv1d_bwd, causal_conv1d_fwd
+from mamba_amd.utils.determinism import fixed_point_scale, use_deterministic_mode
 
 _FLOAT_TYPES = (torch.float32, torch.bfloat16, torch.float16)
 
@@ -184,6 +185,15 @@ def scan_bwd_launch(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, delta_softp
     p.dB, p.dC = _lib.ptr(bufs.dB), _lib.ptr(bufs.dC)
     p.dA_part, p.dD_part = bufs.dA_part.data_ptr(), bufs.dD_part.data_ptr()
     p.ddelta_bias_part = bufs.dbias_part.data_ptr()
+    keep = None
+    if A.is_complex() and use_deterministic_mode():
+        # the complex kernels add every channel's dB / dC terms into one sum: as 64-bit integers of fixed-point terms
+        # the sum does not depend on the order of the adds (a real A's backward pass has no such sums)
+        scale = fixed_point_scale(dout)
+        shadows = [torch.zeros_like(t, dtype=torch.int64) if o.dim() == 4 else None
+                   for t, o in ((bufs.dB32, B), (bufs.dC32, C))]
+        p.det_scale, p.det_dB, p.det_dC = scale.data_ptr(), _lib.ptr(shadows[0]), _lib.ptr(shadows[1])
+        keep = (scale, shadows)
     p.dout_bs, p.dout_ds = dout.stride(0), dout.stride(1)
     p.du_bs, p.du_ds = bufs.du.stride(0), bufs.du.stride(1)
     p.ddelta_bs, p.ddelta_ds = bufs.ddelta.stride(0), bufs.ddelta.stride(1)
@@ -193,6 +203,7 @@ def scan_bwd_launch(u, delta, A, B, C, D, z, delta_bias, dout, ckpt, delta_softp
         p.outz_bs, p.outz_ds = out_z.stride(0), out_z.stride(1)
     with torch.cuda.device(u.device):
         _lib.check(lib.mamba1_scan_bwd(p, _lib.current_stream(u.device)), "mamba1_scan_bwd")
+    del keep  # (stream-ordered allocator: the buffers stay valid for the launches already queued)
     return bufs
 
 

@@ -203,3 +203,37 @@ def test_conv_and_block_backward_deterministic_mode(deterministic_mode):
     a, b = _twice(block)
     for ga, gb in zip(a, b):
         assert torch.equal(ga, gb)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_complex_scan_backward_deterministic_mode(deterministic_mode, dtype):
+    """A complex A (the S4D-style variant): its kernels add every channel's dB / dC terms into one sum per position.
+    In the deterministic mode those adds are integer adds of fixed-point terms: every gradient repeats bit for bit,
+    and agrees with the default mode's float sums to rounding noise."""
+    from mamba_amd.ops.selective_scan_interface import selective_scan_fn
+    from mamba_amd.utils.determinism import set_deterministic_mode
+    g = torch.Generator().manual_seed(7)
+    b, d, L, n = 2, 96, 700, 8
+    u, delta, z, dout = (torch.randn(b, d, L, generator=g).to(dtype).cuda() for _ in range(4))
+    delta = (0.5 * torch.rand(b, d, L, generator=g)).to(dtype).cuda()
+    A = torch.complex(-0.5 * torch.rand(d, n, generator=g), 2.0 * torch.randn(d, n, generator=g)).cuda()
+    B, C = (torch.randn(b, 2, n, 2 * L, generator=g).to(dtype).cuda() for _ in range(2))
+    D, bias = torch.rand(d, generator=g).cuda(), (0.5 * torch.rand(d, generator=g)).cuda()
+
+    def grads():
+        leaves = [t.clone().requires_grad_() for t in (u, delta, A, B, C, D, z, bias)]
+        out = selective_scan_fn(leaves[0], leaves[1], leaves[2], leaves[3], leaves[4], leaves[5], z=leaves[6],
+                                delta_bias=leaves[7], delta_softplus=True)
+        out.backward(dout)
+        return [torch.view_as_real(t.grad) if t.grad.is_complex() else t.grad for t in leaves]
+
+    a, bb = _twice(grads)
+    for i, (x, y) in enumerate(zip(a, bb)):
+        assert torch.equal(x, y), f"gradient {i} does not repeat bit for bit in the deterministic mode"
+    set_deterministic_mode(False)
+    try:
+        c = grads()
+    finally:
+        set_deterministic_mode(True)
+    for i, (x, y) in enumerate(zip(a, c)):
+        assert _noise(x, y) <= (1e-2 if dtype == torch.bfloat16 else 1e-4), (i, _noise(x, y))
