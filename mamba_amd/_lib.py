@@ -221,7 +221,9 @@ def torch_ext():
     global _torch_ext
     if _torch_ext is False:
         _torch_ext = None
-        if os.environ.get("MAMBA_AMD_NO_TORCH_EXT", "0") != "1":
+        # with MAMBA_AMD_LIB set the extension stays off: it is linked against the in-tree library and would run
+        # that one's kernels beside the override's
+        if os.environ.get("MAMBA_AMD_NO_TORCH_EXT", "0") != "1" and not os.environ.get("MAMBA_AMD_LIB"):
             load()  # the extension links against the kernel library: fail on that first, and loudly
             try:
                 from mamba_amd import _torch_ext as ext

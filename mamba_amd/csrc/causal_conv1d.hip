@@ -26,10 +26,7 @@ DEVI float silu_f(float v) { return v * sigmoid_f(v); }
 // on terms scaled to a fixed point, whose result does not depend on the order of the adds (see SsdParams).
 DEVI void conv_acc_add(const CausalConvParams &p, float *dst, int64_t *shadow, int64_t idx, float v) {
   if (p.det_scale) {
-    const float q = fminf(fmaxf(v * p.det_scale[0], -9.0e18f), 9.0e18f);
-    __hip_atomic_fetch_add(reinterpret_cast<unsigned long long *>(shadow + idx),
-                           static_cast<unsigned long long>(static_cast<long long>(__builtin_rintf(q))), __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
+    det_add(shadow, idx, v, p.det_scale[0]);
   } else {
     unsafeAtomicAdd(dst + idx, v);
   }

@@ -242,6 +242,29 @@ DEVI float softplus_slope_f(float y) {
 // wave of the workgroup.)
 DEVI void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// ------------------------------------------------------------------- fixed-point sums
+// One term of a sum kept as a 64-bit integer of fixed-point terms (the deterministic mode): v * scale rounded to an
+// integer and added with an integer atomic, whose result does not depend on the order of the adds.  A finite term is
+// clamped to +-2^59; a term that is not finite (NaN, Inf) replaces the sum by 2^62, which later adds cannot bring back
+// below 2^61 in magnitude: det_value() turns every sum of magnitude >= 2^61 -- poisoned, or overflowed -- into NaN, so
+// that non-finite gradients stay visible as they do with float atomics.
+DEVI void det_add(int64_t *shadow, int64_t idx, float v, float scale) {
+  unsigned long long *dst = reinterpret_cast<unsigned long long *>(shadow + idx);
+  const float q = v * scale;
+  if (__builtin_fabsf(q) <= 3.4e38f) {  // finite
+    const float c = fminf(fmaxf(q, -5.7e17f), 5.7e17f);
+    __hip_atomic_fetch_add(dst, static_cast<unsigned long long>(static_cast<long long>(__builtin_rintf(c))), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+  } else {
+    __hip_atomic_exchange(dst, 1ull << 62, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+DEVI float det_value(int64_t sum, float inv_scale) {
+  const int64_t mag = sum < 0 ? -sum : sum;
+  if (mag >= (int64_t(1) << 61) || sum == INT64_MIN) return __builtin_nanf("");
+  return (float)((double)sum * (double)inv_scale);
+}
+
 // ------------------------------------------------------------------- DPP
 // dpp_ctrl encodings of the GFX9 family.
 enum : int {

@@ -120,10 +120,7 @@ DEVI Geo geometry(const MambaScanParams &p, int wave) {
 // on the term scaled to a fixed point, whose result does not depend on the order of the adds.
 DEVI void add_term(float *dst, int64_t *shadow, int64_t idx, float v, float dsc) {
   if (dsc != 0.f) {
-    const float q = fminf(fmaxf(v * dsc, -9.0e18f), 9.0e18f);
-    __hip_atomic_fetch_add(reinterpret_cast<unsigned long long *>(shadow + idx),
-                           static_cast<unsigned long long>(static_cast<long long>(__builtin_rintf(q))), __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
+    det_add(shadow, idx, v, dsc);
   } else {
     unsafeAtomicAdd(dst + idx, v);
   }

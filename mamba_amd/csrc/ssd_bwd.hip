@@ -25,7 +25,7 @@ __host__ __device__ inline int dcb_head_splits(int heads_per_group) { return (he
 __global__ __launch_bounds__(256) void det_convert_kernel(const int64_t *__restrict__ src, float *__restrict__ dst, int64_t n,
                                                           const float *__restrict__ scale) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i < n) dst[i] = (float)((double)src[i] * (double)scale[1]);
+  if (i < n) dst[i] = det_value(src[i], scale[1]);
 }
 
 // Sums acc[m][n] * fx(m, n) over n for every row m of the block tile into rows[64] (LDS, zeroed

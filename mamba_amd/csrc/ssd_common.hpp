@@ -725,10 +725,7 @@ DEVI float det_scale_of(const SsdParams &p) { return p.det_scale ? p.det_scale[0
 // loops hold these adds: carrying both forms costs them registers and ~10 % of their time).
 template <int MODE = -1> DEVI void acc_add(float *dst, int64_t *shadow, int64_t idx, float v, float dsc) {
   if (MODE == 1 || (MODE < 0 && dsc != 0.f)) {
-    const float q = fminf(fmaxf(v * dsc, -9.0e18f), 9.0e18f);
-    __hip_atomic_fetch_add(reinterpret_cast<unsigned long long *>(shadow + idx),
-                           static_cast<unsigned long long>(static_cast<long long>(__builtin_rintf(q))), __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
+    det_add(shadow, idx, v, dsc);
   } else {
     unsafeAtomicAdd(dst + idx, v);
   }

@@ -143,7 +143,8 @@ def causal_conv1d_fn(x, weight, bias=None, seq_idx=None, initial_states=None, re
     x's layout.
     Streaming (the causal_conv1d package's arguments of the same names):
         initial_states: (batch, dim, width - 1), the positions in front of x; the output is that of the
-            convolution over [initial_states, x], cut to x's positions (not together with seq_idx)
+            convolution over [initial_states, x], cut to x's positions; with seq_idx they belong to the row's
+            first sequence
         return_final_states: also return (batch, dim, width - 1), the last width - 1 positions of
             [initial_states, x] (zero-filled on the left when there are fewer); no gradient flows through them
         final_states_out: a tensor to receive them
@@ -154,8 +155,6 @@ def causal_conv1d_fn(x, weight, bias=None, seq_idx=None, initial_states=None, re
     batch, dim, seqlen = x.shape
     joined = x
     if initial_states is not None:
-        if seq_idx is not None:
-            raise RuntimeError("causal_conv1d_fn: initial_states cannot be combined with seq_idx")
         if tuple(initial_states.shape) != (batch, dim, width - 1):
             raise RuntimeError("causal_conv1d_fn: initial_states must be (batch, dim, width - 1)")
         _lib.require_gpu(x, initial_states)
@@ -163,7 +162,12 @@ def causal_conv1d_fn(x, weight, bias=None, seq_idx=None, initial_states=None, re
             joined = torch.cat([initial_states.to(x.dtype).transpose(1, 2), x.transpose(1, 2)], dim=1).transpose(1, 2)
         else:
             joined = torch.cat([initial_states.to(x.dtype), x], dim=2)
-        out = CausalConv1dFn.apply(joined, weight, bias, None, activation)[:, :, width - 1:]
+        joined_idx = None
+        if seq_idx is not None:
+            # the carried positions continue the row's first sequence (a prefill cut into pieces hands them on):
+            # they take that sequence's id, so its first positions see them and no other sequence does
+            joined_idx = torch.cat([seq_idx[:, :1].expand(batch, width - 1), seq_idx], dim=1).to(torch.int32).contiguous()
+        out = CausalConv1dFn.apply(joined, weight, bias, joined_idx, activation)[:, :, width - 1:]
     else:
         out = CausalConv1dFn.apply(x, weight, bias, seq_idx, activation)
     if not return_final_states and final_states_out is None:

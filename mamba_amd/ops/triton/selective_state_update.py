@@ -126,7 +126,9 @@ def selective_state_update(state, x, dt, A, B, C, D=None, z=None, dt_bias=None, 
     return out
 
 
-_SYNC = {}  # (device index, size) -> zeroed int32 counters of mamba2_decode_step (left zero by every call)
+# (device index, stream, size) -> zeroed int32 counters of mamba2_decode_step (every call leaves them zero).  One buffer per
+# stream: calls on one stream run one after the other, calls on two streams may overlap and must not share counters.
+_SYNC = {}
 
 E_UNSUPPORTED = -2
 FUSE_MAX_BATCH = 16  # largest batch for which mamba2_decode_step picks the fused kernel by itself
@@ -148,6 +150,8 @@ def mamba2_decode_step(ssm_state, conv_state, xBC, dt, A, conv_weight, conv_bias
         xBC: (batch, conv_dim); dt: (batch, nheads); A, dt_bias, D: (nheads,); z: (batch, nheads, headdim)
         conv_weight: (conv_dim, width); conv_bias: (conv_dim,)
         fuse: None = one launch where served, False = always the two calls, True = one launch or an error
+    The fused launch keeps a small zeroed counter buffer per (device, stream, size), allocated on the first such call:
+    to capture `fuse=True` in a HIP graph, make one eager call on the capturing stream first.
     Returns y: (batch, nheads, headdim) in xBC's dtype."""
     from mamba_amd.ops.causal_conv1d import causal_conv1d_update
     _, nheads, headdim, dstate = ssm_state.shape
@@ -210,7 +214,7 @@ def mamba2_decode_step(ssm_state, conv_state, xBC, dt, A, conv_weight, conv_bias
     nsync = int(_lib.load().mamba2_decode_step_sync_ints(q))
     if nsync <= 0:
         _lib.check(nsync or -1, "mamba2_decode_step_sync_ints")
-    key = (xBC.device.index, nsync)
+    key = (xBC.device.index, _lib.current_stream(xBC.device), nsync)
     sync = _SYNC.get(key)
     if sync is None:
         sync = _SYNC[key] = torch.zeros(nsync, dtype=torch.int32, device=xBC.device)

@@ -180,6 +180,45 @@ def test_causal_conv1d_streaming_states(width, seqlen, channel_last):
     _close("final_states_out", buf, want, 0, 0)
 
 
+@pytest.mark.parametrize("channel_last", [False, True])
+def test_causal_conv1d_initial_states_with_seq_idx(channel_last):
+    """A packed row that continues a sequence (a prefill cut into pieces): initial_states carry the last width - 1
+    positions of the row's first sequence, seq_idx separates the sequences.  Checked against F.conv1d per
+    sequence, the first one convolved behind the carried positions, with every gradient.  (No call site of the
+    reference passes both arguments and the causal_conv1d package's own tests are not in it: this combination is
+    pinned by that arithmetic, not by a reference vector.)"""
+    import torch.nn.functional as F
+    from mamba_amd.ops.causal_conv1d import causal_conv1d_fn
+    g = torch.Generator().manual_seed(11)
+    batch, dim, width, lens = 2, 16, 4, [5, 2, 30, 11]
+    L = sum(lens)
+    x = torch.randn(batch, dim, L, generator=g)
+    init = torch.randn(batch, dim, width - 1, generator=g)
+    w, bias = 0.5 * torch.randn(dim, width, generator=g), torch.randn(dim, generator=g)
+    dout = torch.randn(batch, dim, L, generator=g)
+    seq_idx = torch.cat([torch.full((n,), i + 3, dtype=torch.int32) for i, n in enumerate(lens)])[None].expand(batch, L).contiguous()
+    xr, ir, wr, br = (t.clone().requires_grad_() for t in (x, init, w, bias))
+    pieces, start = [], 0
+    for i, n in enumerate(lens):
+        seg = xr[:, :, start:start + n]
+        front = ir if i == 0 else torch.zeros(batch, dim, width - 1)
+        pieces.append(F.silu(F.conv1d(torch.cat([front, seg], dim=2), wr[:, None, :], br, groups=dim)))
+        start += n
+    ref = torch.cat(pieces, dim=2)
+    (ref * dout).sum().backward()
+    lay = (lambda t: t.cuda().transpose(1, 2).contiguous().transpose(1, 2)) if channel_last else (lambda t: t.cuda())
+    xg, ig = lay(x).requires_grad_(), lay(init).requires_grad_()
+    wg, bg = w.cuda().requires_grad_(), bias.cuda().requires_grad_()
+    out, fin = causal_conv1d_fn(xg, wg, bg, seq_idx=seq_idx.cuda(), initial_states=ig, return_final_states=True,
+                                activation="silu")
+    (out * dout.cuda()).sum().backward()
+    _close("out", out, ref, 6e-4, 2e-3)
+    _close("final_states", fin, x[:, :, -(width - 1):], 0, 0)
+    for name, a, b in (("dx", xg.grad, xr.grad), ("dinitial_states", ig.grad, ir.grad), ("dweight", wg.grad, wr.grad),
+                       ("dbias", bg.grad, br.grad)):
+        _close(name, a, b, 6e-4, 2e-3)
+
+
 @pytest.mark.parametrize("width,state_len", [(4, 4), (4, 7), (3, 2), (2, 5)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_causal_conv1d_update_circular_buffer(width, state_len, dtype):
