@@ -302,7 +302,9 @@ typedef struct SsdParams {
   const float *dfinal_states;           /* nullable, (b, H, P, N) */
   void *dx, *dz;                        /* `dtype`, (b, L, H, P): dz contiguous, dx with the strides below */
   void *ddt;                            /* `dt_dtype`, contiguous (b, L, H) */
-  void *dB, *dC;                        /* `dtype`, contiguous (b, L, G, N) */
+  void *dB, *dC;                        /* `dtype`, contiguous (b, L, G, N); nullable: when set, ssd_combined_bwd leaves the
+                                           finished sums of dB32 / dC32 here in the operands' dtype (its last stage writes
+                                           them, so no conversion pass over the fp32 sums is needed) */
   float *dA, *ddt_bias;                 /* (H) fp32, zero on entry */
   float *dD;                            /* (H) or (H, P) fp32, zero on entry */
   float *dinitial_states;               /* nullable, (b, H, P, N) fp32 */
@@ -310,7 +312,8 @@ typedef struct SsdParams {
   float *dstates;                       /* (b, c, H, P, N) */
   float *ddA_cumsum;                    /* (b, H, c, Q), zero on entry */
   float *ddt_out;                       /* (b, H, c, Q), zero on entry */
-  float *dCB;                           /* (b, c, G, Q, Q), zero on entry when H/G > 1 */
+  float *dCB;                           /* (b, c, G, Q, Q), zero on entry when H/G > 16 or in the deterministic mode (several
+                                           workgroups then add into a tile); otherwise contents ignored on entry */
   float *dB32, *dC32;                   /* (b, L, G, N), zero on entry */
   void *gbuf;                           /* (b, L, H, P) of `dtype`: dout * silu(z); used iff z != NULL */
   int64_t dout_bs, dout_ls, dout_hs;

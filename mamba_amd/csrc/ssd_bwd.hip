@@ -1104,9 +1104,15 @@ template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256, 4)
 #pragma unroll
       for (int r = 0; r < 4; ++r)
         if (!((live >> ((tm * 2 + tn) * 4 + r)) & 1)) sum.v[tm][tn][r] = 0.f;  // causal / same-sequence mask
+  // Several workgroups (head lists) add into one tile: dCB starts zeroed.  One list per group: this workgroup owns the
+  // tile and stores it whole, zeros included, so the caller need not clear dCB (the later stages read these tiles only).
+  const bool own_tile = !DET && nsplit == 1;
   acc_foreach(sum, tid, [&](int m, int n, float v) {
     const int l = lt * GB + m, s = st * GB + n;
-    if (l < Q && s < Q && v != 0.f) acc_add<DET ? 1 : 0>(p.dCB, p.det_dCB, dCB_off + (int64_t)l * Q + s, v, det_scale_of(p));  // dCB starts zeroed
+    if (l < Q && s < Q) {
+      if (own_tile) p.dCB[dCB_off + (int64_t)l * Q + s] = v;
+      else if (v != 0.f) acc_add<DET ? 1 : 0>(p.dCB, p.det_dCB, dCB_off + (int64_t)l * Q + s, v, det_scale_of(p));
+    }
     return v;
   });
 }
@@ -1176,16 +1182,24 @@ template <typename T, bool SPLIT> DEVI void bmm_chunk_bwd_wide_body(const SsdPar
   if (mt * GB >= qlim) return;
   const float *dCB = p.dCB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
   const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1, i = lane & 15, gq = lane >> 4;
-  auto add_tile = [&](const GemmAccWide &acc, float *dst) {  // dst[(row of the chunk) * G * N + column] += tile
+  // dst[(row of the chunk) * G * N + column] += tile.  This stage is the last one to add into dB32 / dC32 and its
+  // tiles cover every row once: with `fin` set the sum leaves here in the operands' dtype as well (dB / dC), and no
+  // separate conversion pass over the fp32 sums is needed.
+  auto add_tile = [&](const GemmAccWide &acc, float *dst, void *fin) {
 #pragma unroll
     for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int m = mt * GB + wm * 32 + tm * 16 + gq * 4 + r;
         if (m >= qlim) continue;
-        float *row = dst + (((int64_t)b * L + t0 + m) * G + g) * N + nt * WB + wn * 64 + i;
+        const int64_t at = (((int64_t)b * L + t0 + m) * G + g) * N + nt * WB + wn * 64 + i;
+        float *row = dst + at;
 #pragma unroll
-        for (int tn = 0; tn < 4; ++tn) row[tn * 16] += acc.v[tm][tn][r];
+        for (int tn = 0; tn < 4; ++tn) {
+          const float v = row[tn * 16] + acc.v[tm][tn][r];
+          row[tn * 16] = v;
+          if (fin) st1<T>(static_cast<T *>(fin) + at + tn * 16, v);
+        }
       }
   };
   {
@@ -1197,7 +1211,7 @@ template <typename T, bool SPLIT> DEVI void bmm_chunk_bwd_wide_body(const SsdPar
     const T *Ba = static_cast<const T *>(p.B) + b * p.B_bs + g * p.B_gs + (int64_t)t0 * p.B_ls + nt * WB;
     WideTrStager<SPLIT, T, WB> sb(lds.bh, lds.bl, Ba, p.B_ls, WB, nullptr, tid);
     block_gemm_wide<SPLIT>(acc, lds, kend, sa, sb, tid);
-    add_tile(acc, p.dC32);
+    add_tile(acc, p.dC32, p.dC);
   }
   lds_barrier();  // the first product's last operand reads end before the second one's first commit
   {
@@ -1209,7 +1223,7 @@ template <typename T, bool SPLIT> DEVI void bmm_chunk_bwd_wide_body(const SsdPar
     const T *Ca = static_cast<const T *>(p.C) + b * p.C_bs + g * p.C_gs + (int64_t)(t0 + k0) * p.C_ls + nt * WB;
     WideTrStager<SPLIT, T, WB> sb(lds.bh, lds.bl, Ca, p.C_ls, WB, nullptr, tid);
     block_gemm_wide<SPLIT>(acc, lds, qlim - k0, sa, sb, tid);
-    add_tile(acc, p.dB32);
+    add_tile(acc, p.dB32, p.dB);
   }
 }
 
@@ -1471,9 +1485,13 @@ static int ssd_bwd_dcb_one(const SsdParams *p, mamba_stream_t stream) {
   return launched();
 }
 
-static int ssd_bmm_chunk_bwd_one(const SsdParams *p, mamba_stream_t stream) {
-  int rc = check_bwd(p);
+static int ssd_bmm_chunk_bwd_one(const SsdParams *p_in, mamba_stream_t stream) {
+  int rc = check_bwd(p_in);
   if (rc) return rc;
+  // the stage on its own only adds into dB32 / dC32; dB / dC are written by ssd_combined_bwd, whose last stage this is
+  SsdParams q = *p_in;
+  q.dB = q.dC = nullptr;
+  const SsdParams *p = &q;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (p->dstate % WB == 0 && p->chunk_size % GB == 0 && whole_k_steps(p) &&
       wide_operand_ok(p->B, p->dtype, p->B_bs, p->B_ls, p->B_gs) && wide_operand_ok(p->C, p->dtype, p->C_bs, p->C_ls, p->C_gs) &&
@@ -1510,7 +1528,33 @@ static bool bmm_bwd_wide_ok(const SsdParams *p) {
          reinterpret_cast<uintptr_t>(p->dCB) % 16 == 0;
 }
 
-// The last two stages as one launch where the bmm stage runs on wide tiles, else one after the other.
+// dst[i] = T(src[i]): the fp32 sums of dB / dC in the operands' dtype, for the paths whose last stage does not
+// write them itself
+template <typename T> __global__ __launch_bounds__(256) void cast_sum_kernel(const float *__restrict__ src, T *__restrict__ dst, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) st1<T>(dst + i, src[i]);
+}
+static int cast_sums(const SsdParams *p, mamba_stream_t stream) {
+  const int64_t n = (int64_t)p->batch * p->seqlen * p->ngroups * p->dstate;
+  if ((!p->dB && !p->dC) || n == 0) return MAMBA_OK;
+  if ((n + 255) / 256 > 0x7fffffff) return MAMBA_E_UNSUPPORTED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)((n + 255) / 256));
+  for (int k = 0; k < 2; ++k) {
+    void *dst = k ? p->dC : p->dB;
+    const float *src = k ? p->dC32 : p->dB32;
+    if (!dst) continue;
+    switch (p->dtype) {
+      case MAMBA_BF16: hipLaunchKernelGGL(cast_sum_kernel<bf16_t>, grid, dim3(256), 0, s, src, static_cast<bf16_t *>(dst), n); break;
+      case MAMBA_F16: hipLaunchKernelGGL(cast_sum_kernel<f16_t>, grid, dim3(256), 0, s, src, static_cast<f16_t *>(dst), n); break;
+      default: hipLaunchKernelGGL(cast_sum_kernel<float>, grid, dim3(256), 0, s, src, static_cast<float *>(dst), n); break;
+    }
+  }
+  return launched();
+}
+
+// The last two stages as one launch where the bmm stage runs on wide tiles, else one after the other.  Either way
+// dB / dC (when the caller passes them) hold the finished sums in the operands' dtype afterwards.
 static int bmm_and_cumsum_bwd(const SsdParams *p, mamba_stream_t stream) {
   int rc = check_bwd(p);
   if (rc) return rc;
@@ -1531,7 +1575,8 @@ static int bmm_and_cumsum_bwd(const SsdParams *p, mamba_stream_t stream) {
     return launched();
   }
   if ((rc = ssd_bmm_chunk_bwd(p, stream))) return rc;
-  return ssd_chunk_cumsum_bwd(p, stream);
+  if ((rc = ssd_chunk_cumsum_bwd(p, stream))) return rc;
+  return cast_sums(p, stream);
 }
 
 // The first two stages: one kernel where the gate's pass over dout, z and the pre-gate output can feed the

@@ -469,11 +469,15 @@ std::optional<TensorList> ssd_bwd_fast(const at::Tensor &dout, const at::Tensor 
   // one zeroed arena for every accumulator the kernels add into
   const int64_t nD = D ? D->numel() : 0, nHcQ = d.batch * d.H * d.nchunks * d.Q;
   const int64_t nCB = d.batch * d.nchunks * d.G * d.Q * d.Q, nBC = d.batch * d.L * d.G * d.N;
-  const int64_t sizes[8] = {d.H, d.H, nD, nHcQ, nHcQ, nCB, nBC, nBC};
+  // (dCB needs no clearing when one workgroup owns each of its tiles: at most 16 heads per group)
+  const bool dcb_owned = d.H / d.G <= 16;
+  const int64_t sizes[8] = {d.H, d.H, nD, nHcQ, nHcQ, dcb_owned ? 0 : nCB, nBC, nBC};
   int64_t total = 0, off[8];
   for (int i = 0; i < 8; ++i) off[i] = total, total += sizes[i];
   at::Tensor arena = at::zeros({total}, f32);
   float *base = arena.data_ptr<float>();
+  OptTensor dCB_own;
+  if (dcb_owned) dCB_own = at::empty({nCB}, f32);
   at::Tensor dstates = at::empty({d.batch, d.nchunks, d.H, d.P, d.N}, d.lp ? x.options() : f32);
   if (initial_states) dinit = at::empty({d.batch, d.H, d.P, d.N}, f32);
   p.dt_out = dt_out.data_ptr<float>(), p.dA_cumsum = dA_cumsum.data_ptr<float>();
@@ -486,9 +490,13 @@ std::optional<TensorList> ssd_bwd_fast(const at::Tensor &dout, const at::Tensor 
   p.dx = dx.data_ptr(), p.dz = dz ? dz->data_ptr() : nullptr, p.ddt = ddt.data_ptr(), p.gbuf = gbuf ? gbuf->data_ptr() : nullptr;
   p.dx_bs = dx.stride(0), p.dx_ls = dx.stride(1), p.dx_hs = dx.stride(2);
   p.dA = base + off[0], p.ddt_bias = base + off[1], p.dD = D ? base + off[2] : nullptr;
-  p.ddA_cumsum = base + off[3], p.ddt_out = base + off[4], p.dCB = base + off[5], p.dB32 = base + off[6], p.dC32 = base + off[7];
+  p.ddA_cumsum = base + off[3], p.ddt_out = base + off[4], p.dB32 = base + off[6], p.dC32 = base + off[7];
+  p.dCB = dcb_owned ? dCB_own->data_ptr<float>() : base + off[5];
   p.dinitial_states = dinit ? dinit->data_ptr<float>() : nullptr;
   if (d.lp) p.dstates_lp = dstates.data_ptr(); else p.dstates = dstates.data_ptr<float>();
+  // dB / dC in the operands' dtype: written by the call's last stage
+  at::Tensor dB = at::empty({d.batch, d.L, d.G, d.N}, B.options()), dC = at::empty({d.batch, d.L, d.G, d.N}, C.options());
+  p.dB = dB.data_ptr(), p.dC = dC.data_ptr();
   c10::DeviceGuard guard(dev);
   void *stream = stream_of(dev);
   check_rc(ssd_bmm_chunk_fwd(&p, stream), "ssd_bmm_chunk_fwd");  // CB: the fused forward never forms it
@@ -496,8 +504,7 @@ std::optional<TensorList> ssd_bwd_fast(const at::Tensor &dout, const at::Tensor 
   auto piece = [&](int i, at::IntArrayRef shape) { return arena.narrow(0, off[i], sizes[i]).view(shape); };
   TensorList r(9);
   r[0] = dx, r[1] = ddt, r[2] = piece(0, {d.H});
-  r[3] = piece(6, {d.batch, d.L, d.G, d.N}).to(B.scalar_type());
-  r[4] = piece(7, {d.batch, d.L, d.G, d.N}).to(C.scalar_type());
+  r[3] = dB, r[4] = dC;
   if (D) r[5] = piece(2, D->sizes());
   r[6] = dz;
   if (dt_bias) r[7] = piece(1, {d.H});

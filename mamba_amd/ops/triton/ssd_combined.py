@@ -210,9 +210,14 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
                  ddA_cumsum=batch * nheads * nchunks * chunk_size, ddt_out=batch * nheads * nchunks * chunk_size,
                  dCB=batch * nchunks * ngroups * chunk_size * chunk_size,
                  dB32=batch * seqlen * ngroups * dstate, dC32=batch * seqlen * ngroups * dstate)
-    arena = torch.zeros(sum(sizes.values()), **f32)
+    # dCB needs no clearing when one workgroup owns each of its tiles (at most 16 heads per group, float sums)
+    dcb_owned = nheads // ngroups <= 16 and not use_deterministic_mode()
+    arena = torch.zeros(sum(n for k, n in sizes.items() if not (k == "dCB" and dcb_owned)), **f32)
     acc, off = {}, 0
     for k, n in sizes.items():
+        if k == "dCB" and dcb_owned:
+            acc[k] = torch.empty(n, **f32)
+            continue
         acc[k] = arena[off:off + n]
         off += n
     lp = x.dtype == torch.bfloat16  # the carried states' gradients pass between the stages in bf16 too
@@ -240,6 +245,11 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
         p.dstates = dstates.data_ptr()
     p.ddA_cumsum, p.ddt_out, p.dCB = acc["ddA_cumsum"].data_ptr(), acc["ddt_out"].data_ptr(), acc["dCB"].data_ptr()
     p.dB32, p.dC32 = acc["dB32"].data_ptr(), acc["dC32"].data_ptr()
+    # dB / dC in the operands' dtype are written by the call's last stage; a caller's own (strided) views are filled
+    # from the fp32 sums afterwards instead
+    dB_own = torch.empty(batch, seqlen, ngroups, dstate, device=dev, dtype=x.dtype) if dB is None and in_dtypes[4] == x.dtype else None
+    dC_own = torch.empty(batch, seqlen, ngroups, dstate, device=dev, dtype=x.dtype) if dC is None and in_dtypes[5] == x.dtype else None
+    p.dB, p.dC = _lib.ptr(dB_own), _lib.ptr(dC_own)
     if use_deterministic_mode():
         # integer shadows of the shared sums, laid out like the float arena, and the call's fixed-point scale
         shadow = torch.zeros(sum(sizes.values()), device=dev, dtype=torch.int64)
@@ -266,8 +276,14 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
     dinit_out = dinit.to(in_dtypes[3]) if dinit is not None else None
     dB32 = acc["dB32"].view(batch, seqlen, ngroups, dstate)
     dC32 = acc["dC32"].view(batch, seqlen, ngroups, dstate)
-    dB = dB32.to(in_dtypes[4]) if dB is None else dB.copy_(dB32)     # the copy is the cast
-    dC = dC32.to(in_dtypes[5]) if dC is None else dC.copy_(dC32)
+    if dB_own is not None:
+        dB = dB_own
+    else:
+        dB = dB32.to(in_dtypes[4]) if dB is None else dB.copy_(dB32)     # the copy is the cast
+    if dC_own is not None:
+        dC = dC_own
+    else:
+        dC = dC32.to(in_dtypes[5]) if dC is None else dC.copy_(dC32)
     if ddt_out_view is not None:
         ddt = ddt_out_view.copy_(ddt)
     return dx, ddt, dA, dB, dC, dD, dz, ddt_bias, dinit_out
