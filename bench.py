@@ -441,14 +441,15 @@ def bench_ssd(dev, steps, warmup):
 
 def mfma_counters(filename, kernel):
     """Matrix-core counters of `kernel` from profiles/<filename> (per launch, summed over the chip): bf16 MFMA
-    instructions, and the share of the busy cycles of the compute units in which a matrix core was executing."""
+    instructions, and the share of the busy cycles of the compute units in which their matrix cores were
+    executing (one matrix core per SIMD, four SIMDs per compute unit)."""
     n = profile_counter(filename, kernel, "SQ_INSTS_VALU_MFMA_BF16")
     busy = profile_counter(filename, kernel, "SQ_VALU_MFMA_BUSY_CYCLES")
     cu = profile_counter(filename, kernel, "SQ_BUSY_CU_CYCLES")
     if n is None or busy is None or cu is None:
         return None
     return {"mfma_bf16_instructions": n, "mfma_busy_cycles": busy, "cu_busy_cycles": cu,
-            "mfma_busy_frac_of_cu_busy": busy / cu if cu else None}
+            "mfma_busy_frac_of_cu_busy": busy / (4 * cu) if cu else None}
 
 
 def bench_decode(dev, steps, warmup, batch=256):
