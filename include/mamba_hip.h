@@ -312,9 +312,11 @@ typedef struct SsdParams {
   float *dstates;                       /* (b, c, H, P, N) */
   float *ddA_cumsum;                    /* (b, H, c, Q), zero on entry */
   float *ddt_out;                       /* (b, H, c, Q), zero on entry */
-  float *dCB;                           /* (b, c, G, Q, Q), zero on entry when H/G > 16 or in the deterministic mode (several
-                                           workgroups then add into a tile); otherwise contents ignored on entry */
-  float *dB32, *dC32;                   /* (b, L, G, N), zero on entry */
+  float *dCB;                           /* (b, c, G, Q, Q), zero on entry unless ssd_bwd_overwrites() has
+                                           SSD_OVERWRITES_DCB (one workgroup then owns each tile and stores it) */
+  float *dB32, *dC32;                   /* (b, L, G, N), zero on entry unless ssd_bwd_overwrites() has
+                                           SSD_OVERWRITES_DBC (the first stage that touches them then stores them).  With
+                                           dB / dC set the finished sums are only in dB / dC */
   void *gbuf;                           /* (b, L, H, P) of `dtype`: dout * silu(z); used iff z != NULL */
   int64_t dout_bs, dout_ls, dout_hs;
   int64_t dx_bs, dx_ls, dx_hs;          /* dx may be a slice of a wider buffer; unit headdim stride */
@@ -381,6 +383,14 @@ int ssd_chunk_state_varlen(const SsdParams *p, const int32_t *cu_seqlens, int ns
  * ddA_cumsum holds the gradient with respect to the cumulative sums a_l; the last
  * stage turns it into the gradient of the per-position dt * A. */
 int ssd_bwd_dz(const SsdParams *p, mamba_stream_t stream);
+/* Which of the sum buffers the backward pass of this (completely filled) problem writes whole instead of adding
+ * into, so that the caller may hand them over uncleared: a set of the flags below; 0 in the deterministic mode, for a
+ * problem run in batch slices, or for a bad argument.  Clearing a buffer that is reported here is harmless.  No
+ * counterpart in the reference, whose Triton kernels write partial sums to fresh buffers and add them up with
+ * torch (mamba_ssm/ops/triton/ssd_combined.py:441-509). */
+#define SSD_OVERWRITES_DCB 1 /* dCB: at most 16 heads per group */
+#define SSD_OVERWRITES_DBC 2 /* dB32 and dC32: one workgroup of the state-path stage holds all heads of a group */
+int ssd_bwd_overwrites(const SsdParams *p);
 /* dst[i] = shadow[i] / s for i < n (det_scale = {s, 1 / s} on the device): the step between the stages of a
  * deterministic backward pass that ssd_combined_bwd inserts by itself */
 int ssd_det_convert(const int64_t *shadow, float *dst, int64_t n, const float *det_scale, mamba_stream_t stream);

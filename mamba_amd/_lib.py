@@ -164,6 +164,8 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = [ctypes.POINTER(SsdParams), c_vp]
         fn.restype = ctypes.c_int
+    lib.ssd_bwd_overwrites.argtypes = [ctypes.POINTER(SsdParams)]
+    lib.ssd_bwd_overwrites.restype = ctypes.c_int
     lib.ssd_det_convert.argtypes = [c_vp, c_vp, c_i64, c_vp, c_vp]
     lib.ssd_det_convert.restype = ctypes.c_int
     lib.ssd_chunk_state_varlen.argtypes = [ctypes.POINTER(SsdParams), c_vp, ctypes.c_int, c_vp, c_vp]

@@ -390,8 +390,11 @@ template <typename T> __global__ __launch_bounds__(256) void bwd_dz_dstates_kern
 // entering chunk c; on exit it is the gradient of chunk c's local state.
 // A thread owns W consecutive elements; the direct gradients and states of the next SPB_PF chunks
 // are always in flight (the serial recurrence only needs them one chunk at a time, and the
-// compiler cannot hoist the loads over the in-place stores by itself).
+// compiler cannot hoist the loads over the in-place stores by itself).  TABLE: the per-chunk decay factors come from
+// an LDS table filled before the loop, as in the forward kernel (no scalar loads, and their waits, inside the loop),
+// and the ddA_cumsum terms of the chunks are kept in LDS until the loop is over.
 constexpr int SPB_PF = 4;
+constexpr size_t SPB_TABLE_BYTES = 40960;
 
 template <int W> struct VecG;
 template <> struct VecG<1> {
@@ -414,16 +417,42 @@ template <> struct VecG<4> {
   }
   DEVI void store(bf16_t *p) const { *reinterpret_cast<u32x2 *>(p) = u32x2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])}; }
 };
+// W elements as they lie in memory: what the prefetch holds.  They are converted when the chunk is processed; a
+// conversion placed at the load makes the wave wait for the load it has just issued, i.e. no prefetch at all.
+template <int W, typename CT> struct RawG;
+template <> struct RawG<1, float> {
+  float r;
+  DEVI void load(const float *p) { r = *p; }
+  DEVI void unpack(float (&v)[1]) const { v[0] = r; }
+};
+template <> struct RawG<4, float> {
+  f32x4 r;
+  DEVI void load(const float *p) { r = *reinterpret_cast<const f32x4 *>(p); }
+  DEVI void unpack(float (&v)[4]) const { v[0] = r.x; v[1] = r.y; v[2] = r.z; v[3] = r.w; }
+};
+template <> struct RawG<1, bf16_t> {
+  uint16_t r;
+  DEVI void load(const bf16_t *p) { r = *reinterpret_cast<const uint16_t *>(p); }
+  DEVI void unpack(float (&v)[1]) const { v[0] = __builtin_bit_cast(float, (uint32_t)r << 16); }
+};
+template <> struct RawG<4, bf16_t> {
+  u32x2 r;
+  DEVI void load(const bf16_t *p) { r = *reinterpret_cast<const u32x2 *>(p); }
+  DEVI void unpack(float (&v)[4]) const { v[0] = bf16_lo(r.x); v[1] = bf16_hi(r.x); v[2] = bf16_lo(r.y); v[3] = bf16_hi(r.y); }
+};
 
 // CT: dtype of the carried states and of dstates (float, or bf16_t next to bf16 operands)
-template <int W, typename CT> __global__ __launch_bounds__(256) void state_passing_bwd_kernel(const SsdParams p) {
+template <int W, typename CT, bool TABLE, bool FULL = false> __global__ __launch_bounds__(256) void state_passing_bwd_kernel(const SsdParams p) {
+  extern __shared__ float spb_decay[];
   CT *const dst_p = std::is_same_v<CT, float> ? reinterpret_cast<CT *>(p.dstates) : static_cast<CT *>(p.dstates_lp);
   const CT *const st_p = std::is_same_v<CT, float> ? reinterpret_cast<const CT *>(p.states) : static_cast<const CT *>(p.states_lp);
   const int PN = p.headdim * p.dstate, H = p.nheads, nc = p.nchunks, Q = p.chunk_size, L = p.seqlen;
   const int e = (blockIdx.x * 256 + threadIdx.x) * W;
   const int lane = threadIdx.x & 63;
   const int h = blockIdx.y, b = blockIdx.z;
-  const bool live = e < PN;
+  // FULL: the state is a whole number of workgroups (no idle thread, and so no branch around the stores of the
+  // loop: with one the compiler counts the memory operations in flight for the worst path and waits for all)
+  const bool live = FULL || e < PN;
   const int ec = live ? e : 0;  // clamped: idle threads read valid memory and add nothing
   VecG<W> G;
 #pragma unroll
@@ -432,7 +461,7 @@ template <int W, typename CT> __global__ __launch_bounds__(256) void state_passi
   const float *dA = p.dA_cumsum + ((int64_t)b * H + h) * nc * Q;
   const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L : nullptr;
   auto offset = [&](int c) { return (((int64_t)b * nc + c) * H + h) * PN + ec; };
-  auto decay = [&](int c) {
+  auto decay_of = [&](int c) {
     float scale = fast_exp(dA[c * Q + Q - 1]);
     if (seq) {
       const int end_c = seq[min((c + 1) * Q, L) - 1];
@@ -441,39 +470,66 @@ template <int W, typename CT> __global__ __launch_bounds__(256) void state_passi
     }
     return scale;
   };
-  VecG<W> direct[SPB_PF], state[SPB_PF];
+  if constexpr (TABLE) {
+    for (int c = threadIdx.x; c < nc; c += 256) spb_decay[c] = decay_of(c);
+    lds_barrier();
+  }
+  auto decay = [&](int c) { return TABLE ? spb_decay[c] : decay_of(c); };
+  float *const parts = spb_decay + nc;  // [nc][4 waves] (TABLE)
+  RawG<W, CT> direct[SPB_PF], state[SPB_PF];
   float scale[SPB_PF];
 #pragma unroll
   for (int j = 0; j < SPB_PF; ++j) {
-    const int c = nc - 1 - j;
-    if (c >= 0) {
-      direct[j].load(dst_p + offset(c));
-      state[j].load(st_p + offset(c));
-      scale[j] = decay(c);
-    }
+    const int c = max(nc - 1 - j, 0);
+    direct[j].load(dst_p + offset(c));
+    state[j].load(st_p + offset(c));
+    scale[j] = decay(c);
   }
-  for (int c0 = nc - 1; c0 >= 0; c0 -= SPB_PF) {
+  // one chunk, its operands in slot j of the prefetch; `more`: request chunk c - SPB_PF into the slot
+  auto step = [&](int c, int j, bool more) {
+    if (live) G.store(dst_p + offset(c));
+    float dir[W], st[W];
+    direct[j].unpack(dir);
+    state[j].unpack(st);
+    const float sc = scale[j];
+    if (more) {  // past the first chunk the loads repeat chunk 0 and nobody uses them: no branch, so no register
+                 // copies (which would wait for the loads in flight) where the paths meet
+      const int cn = max(c - SPB_PF, 0);
+      direct[j].load(dst_p + offset(cn));
+      state[j].load(st_p + offset(cn));
+      scale[j] = decay(cn);
+    }
+    float part = 0.f;
 #pragma unroll
-    for (int j = 0; j < SPB_PF; ++j) {
-      const int c = c0 - j;
-      if (c < 0) break;
-      if (live) G.store(dst_p + offset(c));
-      const VecG<W> dir = direct[j], st = state[j];
-      const float sc = scale[j];
-      if (c - SPB_PF >= 0) {
-        direct[j].load(dst_p + offset(c - SPB_PF));
-        state[j].load(st_p + offset(c - SPB_PF));
-        scale[j] = decay(c - SPB_PF);
-      }
-      float part = 0.f;
-#pragma unroll
-      for (int i = 0; i < W; ++i) {
-        part = __builtin_fmaf(G.v[i], st.v[i], part);
-        G.v[i] = __builtin_fmaf(sc, G.v[i], dir.v[i]);
-      }
-      part = live ? part * sc : 0.f;
-      part = wave_sum_to_last(part);
+    for (int i = 0; i < W; ++i) {
+      part = __builtin_fmaf(G.v[i], st[i], part);
+      G.v[i] = __builtin_fmaf(sc, G.v[i], dir[i]);
+    }
+    part = live ? part * sc : 0.f;
+    part = wave_sum_to_last(part);
+    if constexpr (TABLE) {
+      if (lane == 63) parts[c * 4 + (threadIdx.x >> 6)] = part;  // the wave's own slot
+    } else {
       if (lane == 63 && part != 0.f)
+        acc_add(p.ddA_cumsum, p.det_ddA_cumsum, (((int64_t)b * H + h) * nc + c) * Q + Q - 1, part, det_scale_of(p));
+    }
+  };
+  // whole groups of SPB_PF chunks without a branch inside, then the chunks left over from what the slots hold
+  int c0 = nc - 1;
+  for (; c0 >= SPB_PF - 1; c0 -= SPB_PF) {
+#pragma unroll
+    for (int j = 0; j < SPB_PF; ++j) step(c0 - j, j, true);
+  }
+#pragma unroll
+  for (int j = 0; j < SPB_PF - 1; ++j)
+    if (c0 - j >= 0) step(c0 - j, j, false);
+  if constexpr (TABLE) {
+    // one add per chunk and workgroup, after the loop: an atomic inside it is counted with the loads, and the wait
+    // for a chunk's loads then sat through the round trips of the adds before them
+    lds_barrier();
+    for (int c = threadIdx.x; c < nc; c += 256) {
+      const float part = (parts[c * 4] + parts[c * 4 + 1]) + (parts[c * 4 + 2] + parts[c * 4 + 3]);
+      if (part != 0.f)
         acc_add(p.ddA_cumsum, p.det_ddA_cumsum, (((int64_t)b * H + h) * nc + c) * Q + Q - 1, part, det_scale_of(p));
     }
   }
@@ -1197,8 +1253,8 @@ template <typename T, bool SPLIT> DEVI void bmm_chunk_bwd_wide_body(const SsdPar
 #pragma unroll
         for (int tn = 0; tn < 4; ++tn) {
           const float v = row[tn * 16] + acc.v[tm][tn][r];
-          row[tn * 16] = v;
-          if (fin) st1<T>(static_cast<T *>(fin) + at + tn * 16, v);
+          if (fin) st1<T>(static_cast<T *>(fin) + at + tn * 16, v);  // the finished sum: nobody reads the fp32 one
+          else row[tn * 16] = v;
         }
       }
   };
@@ -1422,14 +1478,24 @@ static int ssd_state_passing_bwd_one(const SsdParams *p, mamba_stream_t stream) 
   const bool lp = p->dtype == MAMBA_BF16;
   const bool vec = PN % 4 == 0 && al16(p->dfinal_states) && al16(p->dinitial_states) &&
                    (lp ? true : al16(p->states) && al16(p->dstates));
+  const size_t tbytes = (size_t)p->nchunks * 5 * sizeof(float);  // decay factors + the four waves' partial sums
+  const bool table = tbytes <= SPB_TABLE_BYTES;
   if (vec) {
     dim3 grid((PN / 4 + 255) / 256, p->nheads, p->batch);
-    if (lp) hipLaunchKernelGGL((state_passing_bwd_kernel<4, bf16_t>), grid, dim3(256), 0, s, *p);
-    else hipLaunchKernelGGL((state_passing_bwd_kernel<4, float>), grid, dim3(256), 0, s, *p);
+    if (table && PN % 1024 == 0) {
+      if (lp) hipLaunchKernelGGL((state_passing_bwd_kernel<4, bf16_t, true, true>), grid, dim3(256), tbytes, s, *p);
+      else hipLaunchKernelGGL((state_passing_bwd_kernel<4, float, true, true>), grid, dim3(256), tbytes, s, *p);
+    } else if (table) {
+      if (lp) hipLaunchKernelGGL((state_passing_bwd_kernel<4, bf16_t, true>), grid, dim3(256), tbytes, s, *p);
+      else hipLaunchKernelGGL((state_passing_bwd_kernel<4, float, true>), grid, dim3(256), tbytes, s, *p);
+    } else {
+      if (lp) hipLaunchKernelGGL((state_passing_bwd_kernel<4, bf16_t, false>), grid, dim3(256), 0, s, *p);
+      else hipLaunchKernelGGL((state_passing_bwd_kernel<4, float, false>), grid, dim3(256), 0, s, *p);
+    }
   } else {
     dim3 grid((PN + 255) / 256, p->nheads, p->batch);
-    if (lp) hipLaunchKernelGGL((state_passing_bwd_kernel<1, bf16_t>), grid, dim3(256), 0, s, *p);
-    else hipLaunchKernelGGL((state_passing_bwd_kernel<1, float>), grid, dim3(256), 0, s, *p);
+    if (lp) hipLaunchKernelGGL((state_passing_bwd_kernel<1, bf16_t, false>), grid, dim3(256), 0, s, *p);
+    else hipLaunchKernelGGL((state_passing_bwd_kernel<1, float, false>), grid, dim3(256), 0, s, *p);
   }
   return launched();
 }
@@ -1641,6 +1707,14 @@ static int ssd_combined_bwd_one(const SsdParams *p, mamba_stream_t stream) {
   if ((rc = ssd_bwd_dx(p, stream))) return rc;
   if ((rc = ssd_bwd_dcb(p, stream))) return rc;
   return bmm_and_cumsum_bwd(p, stream);
+}
+
+extern "C" int ssd_bwd_overwrites(const SsdParams *p) {
+  if (!p || check_bwd(p) != MAMBA_OK || p->det_scale || (int64_t)p->batch * p->nheads > SSD_MAX_GRID_ROWS) return 0;
+  int flags = 0;
+  if (dcb_head_splits(p->nheads / p->ngroups) == 1) flags |= SSD_OVERWRITES_DCB;
+  if (ssd_bwd_dbc_fused_owns(p)) flags |= SSD_OVERWRITES_DBC;
+  return flags;
 }
 
 // Public entry points: the whole problem in one go when one launch can index it, else in slices of batch rows.

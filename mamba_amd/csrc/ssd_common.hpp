@@ -737,6 +737,7 @@ __attribute__((visibility("hidden"))) int ssd_bwd_dx_fused_launch(const SsdParam
 // The fused chunk-state dB / dC kernels (ssd_dbc_fused.hip), under the same convention (the caller then runs the
 // tiled bwd_d*_state kernels).
 __attribute__((visibility("hidden"))) int ssd_bwd_dbc_fused_launch(const SsdParams *p, hipStream_t stream);
+__attribute__((visibility("hidden"))) bool ssd_bwd_dbc_fused_owns(const SsdParams *p);
 
 // ---- host side of the kernels that work through the heads of a group in one workgroup
 inline bool aligned(const void *ptr, int a) { return (reinterpret_cast<uintptr_t>(ptr) % a) == 0; }

@@ -218,7 +218,8 @@ DEVI void dbc_body(const SsdParams &p, const int hb, const int lb, DbcBuf<PT, NK
   int64_t *shadow = IS_C ? p.det_dC : p.det_dB;
   // (the same adds as whole 128-byte lines of a row, through a patch per wave, measured no faster: 20 of a launch's
   // ~85 us go into these atomics, and it is their number that costs).  A workgroup that holds all heads of its group
-  // is the only one to touch its rows of dB / dC: it adds without atomics.
+  // is the only one to touch its rows of dB / dC, and the first of the backward pass to do so: it stores them, so
+  // the caller need not clear them (ssd_bwd_overwrites reports this case).
   const bool alone = per == 1 && !DET;
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
@@ -227,7 +228,7 @@ DEVI void dbc_body(const SsdParams &p, const int hb, const int lb, DbcBuf<PT, NK
     const int64_t row = (((int64_t)b * L + t0 + l) * G + grp) * N + j;
     if (alone) {
 #pragma unroll
-      for (int nt = 0; nt < NTL; ++nt) dst[row + nt * 16] += sum[nt][r];
+      for (int nt = 0; nt < NTL; ++nt) dst[row + nt * 16] = sum[nt][r];
     } else {
 #pragma unroll
       for (int nt = 0; nt < NTL; ++nt) acc_add<DET ? 1 : 0>(dst, shadow, row + nt * 16, sum[nt][r], dsc);
@@ -303,6 +304,14 @@ bool supported(const SsdParams *p) {
 }
 
 }  // namespace
+
+// True when ssd_bwd_dbc_fused_launch runs for this problem with one workgroup per (chunk, group): that workgroup
+// stores its rows of dB32 / dC32.
+bool ssd_bwd_dbc_fused_owns(const SsdParams *p) {
+  if (p->det_scale || !supported(p)) return false;
+  const int hb = dbc_heads_per_workgroup(*p);
+  return hb == p->nheads / p->ngroups && 2 * (p->nheads / hb) <= 65535;
+}
 
 int ssd_bwd_dbc_fused_launch(const SsdParams *p, hipStream_t stream) {
   if (!supported(p)) return MAMBA_E_UNSUPPORTED;

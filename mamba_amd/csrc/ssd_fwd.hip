@@ -251,8 +251,11 @@ __global__ __launch_bounds__(256) void chunk_state_varlen_kernel(const SsdParams
 // after the last chunk goes to final_states.  A thread owns W consecutive elements of the
 // (headdim x dstate) state; the chunk loop is a serial recurrence, so the local states of the
 // next SP_PF chunks are always in flight (the compiler cannot hoist those loads over the in-place
-// stores by itself).
+// stores by itself).  TABLE: the per-chunk decay factors are put in LDS before the loop; read one by one inside
+// it they are scalar loads, each waited for with everything else the scalar unit has in flight, and with few rows
+// per chunk (one long packed batch) that wait was the time of a step.
 constexpr int SP_PF = 4;
+constexpr size_t SP_TABLE_BYTES = 32768;
 
 template <int W> struct VecF;
 template <> struct VecF<1> {
@@ -271,19 +274,14 @@ template <> struct VecF<4> {
 
 // CT float: in place, slot c of `states` receives the state entering chunk c.  CT bf16_t: that state goes to
 // states_lp in bf16 and `states` is only read.
-template <int W, typename CT> __global__ __launch_bounds__(256) void state_passing_fwd_kernel(const SsdParams p) {
+template <int W, typename CT, bool TABLE> __global__ __launch_bounds__(256) void state_passing_fwd_kernel(const SsdParams p) {
+  extern __shared__ float sp_decay[];
   const int PN = p.headdim * p.dstate, H = p.nheads, nc = p.nchunks, Q = p.chunk_size, L = p.seqlen;
   const int e = (blockIdx.x * 256 + threadIdx.x) * W;
   const int h = blockIdx.y, b = blockIdx.z;
-  if (e >= PN) return;
-  VecF<W> s;
-#pragma unroll
-  for (int i = 0; i < W; ++i) s.v[i] = 0.f;
-  if (p.initial_states) s.load(p.initial_states + ((int64_t)b * H + h) * PN + e);
   const float *dA = p.dA_cumsum + ((int64_t)b * H + h) * nc * Q;
   const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L : nullptr;
-  auto slot = [&](int c) { return p.states + (((int64_t)b * nc + c) * H + h) * PN + e; };
-  auto decay = [&](int c) {  // carried-state factor of chunk c: 0 across a sequence boundary
+  auto decay_of = [&](int c) {  // carried-state factor of chunk c: 0 across a sequence boundary
     float scale = fast_exp(dA[c * Q + Q - 1]);
     if (seq) {
       const int seq_new = seq[min((c + 1) * Q, L) - 1], seq_prev = c > 0 ? seq[c * Q - 1] : 0;
@@ -291,39 +289,56 @@ template <int W, typename CT> __global__ __launch_bounds__(256) void state_passi
     }
     return scale;
   };
+  if constexpr (TABLE) {
+    for (int c = threadIdx.x; c < nc; c += 256) sp_decay[c] = decay_of(c);
+    lds_barrier();
+  }
+  if (e >= PN) return;
+  auto decay = [&](int c) { return TABLE ? sp_decay[c] : decay_of(c); };
+  VecF<W> s;
+#pragma unroll
+  for (int i = 0; i < W; ++i) s.v[i] = 0.f;
+  if (p.initial_states) s.load(p.initial_states + ((int64_t)b * H + h) * PN + e);
+  auto slot = [&](int c) { return p.states + (((int64_t)b * nc + c) * H + h) * PN + e; };
   VecF<W> local[SP_PF];
   float scale[SP_PF];
 #pragma unroll
-  for (int j = 0; j < SP_PF; ++j)
-    if (j < nc) {
-      local[j].load(slot(j));
-      scale[j] = decay(j);
-    }
-  for (int c0 = 0; c0 < nc; c0 += SP_PF) {
-#pragma unroll
-    for (int j = 0; j < SP_PF; ++j) {
-      const int c = c0 + j;
-      if (c >= nc) break;
-      if constexpr (std::is_same_v<CT, float>) {
-        s.store(slot(c));
-      } else {
-        CT *o = static_cast<CT *>(p.states_lp) + (((int64_t)b * nc + c) * H + h) * PN + e;
-        if constexpr (W == 4) {
-          *reinterpret_cast<u32x2 *>(o) = u32x2{pack_bf16(s.v[0], s.v[1]), pack_bf16(s.v[2], s.v[3])};
-        } else {
-          st1<CT>(o, s.v[0]);
-        }
-      }
-      const VecF<W> loc = local[j];
-      const float sc = scale[j];
-      if (c + SP_PF < nc) {
-        local[j].load(slot(c + SP_PF));
-        scale[j] = decay(c + SP_PF);
-      }
-#pragma unroll
-      for (int i = 0; i < W; ++i) s.v[i] = __builtin_fmaf(sc, s.v[i], loc.v[i]);
-    }
+  for (int j = 0; j < SP_PF; ++j) {
+    local[j].load(slot(min(j, nc - 1)));
+    scale[j] = decay(min(j, nc - 1));
   }
+  // one chunk, its local state in slot j of the prefetch; `more`: request chunk c + SP_PF into the slot
+  auto step = [&](int c, int j, bool more) {
+    if constexpr (std::is_same_v<CT, float>) {
+      s.store(slot(c));
+    } else {
+      CT *o = static_cast<CT *>(p.states_lp) + (((int64_t)b * nc + c) * H + h) * PN + e;
+      if constexpr (W == 4) {
+        *reinterpret_cast<u32x2 *>(o) = u32x2{pack_bf16(s.v[0], s.v[1]), pack_bf16(s.v[2], s.v[3])};
+      } else {
+        st1<CT>(o, s.v[0]);
+      }
+    }
+    const VecF<W> loc = local[j];
+    const float sc = scale[j];
+    if (more) {  // past the last chunk the loads repeat it and nobody uses them: no branch, so no register copies
+                 // (which would wait for the loads in flight) where the paths meet
+      const int cn = min(c + SP_PF, nc - 1);
+      local[j].load(slot(cn));
+      scale[j] = decay(cn);
+    }
+#pragma unroll
+    for (int i = 0; i < W; ++i) s.v[i] = __builtin_fmaf(sc, s.v[i], loc.v[i]);
+  };
+  // whole groups of SP_PF chunks without a branch inside, then the chunks left over from what the slots hold
+  int c0 = 0;
+  for (; c0 + SP_PF <= nc; c0 += SP_PF) {
+#pragma unroll
+    for (int j = 0; j < SP_PF; ++j) step(c0 + j, j, true);
+  }
+#pragma unroll
+  for (int j = 0; j < SP_PF - 1; ++j)
+    if (c0 + j < nc) step(c0 + j, j, false);
   s.store(p.final_states + ((int64_t)b * H + h) * PN + e);
 }
 
@@ -511,14 +526,21 @@ static int ssd_state_passing_fwd_one(const SsdParams *p, mamba_stream_t stream) 
   auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
   const bool lp = p->dtype == MAMBA_BF16;
   if (lp && !p->states_lp) return MAMBA_E_BADARG;
+  const size_t tbytes = (size_t)p->nchunks * sizeof(float);
+  const bool table = tbytes <= SP_TABLE_BYTES;
   if (PN % 4 == 0 && al16(p->states) && al16(p->final_states) && al16(p->initial_states) && al16(p->states_lp)) {
     dim3 grid((PN / 4 + 255) / 256, p->nheads, p->batch);
-    if (lp) hipLaunchKernelGGL((state_passing_fwd_kernel<4, bf16_t>), grid, dim3(256), 0, s, *p);
-    else hipLaunchKernelGGL((state_passing_fwd_kernel<4, float>), grid, dim3(256), 0, s, *p);
+    if (table) {
+      if (lp) hipLaunchKernelGGL((state_passing_fwd_kernel<4, bf16_t, true>), grid, dim3(256), tbytes, s, *p);
+      else hipLaunchKernelGGL((state_passing_fwd_kernel<4, float, true>), grid, dim3(256), tbytes, s, *p);
+    } else {
+      if (lp) hipLaunchKernelGGL((state_passing_fwd_kernel<4, bf16_t, false>), grid, dim3(256), 0, s, *p);
+      else hipLaunchKernelGGL((state_passing_fwd_kernel<4, float, false>), grid, dim3(256), 0, s, *p);
+    }
   } else {
     dim3 grid((PN + 255) / 256, p->nheads, p->batch);
-    if (lp) hipLaunchKernelGGL((state_passing_fwd_kernel<1, bf16_t>), grid, dim3(256), 0, s, *p);
-    else hipLaunchKernelGGL((state_passing_fwd_kernel<1, float>), grid, dim3(256), 0, s, *p);
+    if (lp) hipLaunchKernelGGL((state_passing_fwd_kernel<1, bf16_t, false>), grid, dim3(256), 0, s, *p);
+    else hipLaunchKernelGGL((state_passing_fwd_kernel<1, float, false>), grid, dim3(256), 0, s, *p);
   }
   return launched();
 }

@@ -466,18 +466,16 @@ std::optional<TensorList> ssd_bwd_fast(const at::Tensor &dout, const at::Tensor 
   OptTensor dz, gbuf, dinit;
   if (z) dz = at::empty(x.sizes(), x.options()), gbuf = at::empty(x.sizes(), x.options());
   at::Tensor ddt = at::empty({d.batch, d.L, d.H}, dt.options());
-  // one zeroed arena for every accumulator the kernels add into
+  // one zeroed arena for the small accumulators the kernels add into; the three large ones (dCB, dB32, dC32) are
+  // cleared below, and only where the library does not write them whole (ssd_bwd_overwrites)
   const int64_t nD = D ? D->numel() : 0, nHcQ = d.batch * d.H * d.nchunks * d.Q;
   const int64_t nCB = d.batch * d.nchunks * d.G * d.Q * d.Q, nBC = d.batch * d.L * d.G * d.N;
-  // (dCB needs no clearing when one workgroup owns each of its tiles: at most 16 heads per group)
-  const bool dcb_owned = d.H / d.G <= 16;
-  const int64_t sizes[8] = {d.H, d.H, nD, nHcQ, nHcQ, dcb_owned ? 0 : nCB, nBC, nBC};
-  int64_t total = 0, off[8];
-  for (int i = 0; i < 8; ++i) off[i] = total, total += sizes[i];
+  const int64_t sizes[5] = {d.H, d.H, nD, nHcQ, nHcQ};
+  int64_t total = 0, off[5];
+  for (int i = 0; i < 5; ++i) off[i] = total, total += sizes[i];
   at::Tensor arena = at::zeros({total}, f32);
   float *base = arena.data_ptr<float>();
-  OptTensor dCB_own;
-  if (dcb_owned) dCB_own = at::empty({nCB}, f32);
+  at::Tensor dCB = at::empty({nCB}, f32), dB32 = at::empty({nBC}, f32), dC32 = at::empty({nBC}, f32);
   at::Tensor dstates = at::empty({d.batch, d.nchunks, d.H, d.P, d.N}, d.lp ? x.options() : f32);
   if (initial_states) dinit = at::empty({d.batch, d.H, d.P, d.N}, f32);
   p.dt_out = dt_out.data_ptr<float>(), p.dA_cumsum = dA_cumsum.data_ptr<float>();
@@ -490,14 +488,17 @@ std::optional<TensorList> ssd_bwd_fast(const at::Tensor &dout, const at::Tensor 
   p.dx = dx.data_ptr(), p.dz = dz ? dz->data_ptr() : nullptr, p.ddt = ddt.data_ptr(), p.gbuf = gbuf ? gbuf->data_ptr() : nullptr;
   p.dx_bs = dx.stride(0), p.dx_ls = dx.stride(1), p.dx_hs = dx.stride(2);
   p.dA = base + off[0], p.ddt_bias = base + off[1], p.dD = D ? base + off[2] : nullptr;
-  p.ddA_cumsum = base + off[3], p.ddt_out = base + off[4], p.dB32 = base + off[6], p.dC32 = base + off[7];
-  p.dCB = dcb_owned ? dCB_own->data_ptr<float>() : base + off[5];
+  p.ddA_cumsum = base + off[3], p.ddt_out = base + off[4];
+  p.dB32 = dB32.data_ptr<float>(), p.dC32 = dC32.data_ptr<float>(), p.dCB = dCB.data_ptr<float>();
   p.dinitial_states = dinit ? dinit->data_ptr<float>() : nullptr;
   if (d.lp) p.dstates_lp = dstates.data_ptr(); else p.dstates = dstates.data_ptr<float>();
   // dB / dC in the operands' dtype: written by the call's last stage
   at::Tensor dB = at::empty({d.batch, d.L, d.G, d.N}, B.options()), dC = at::empty({d.batch, d.L, d.G, d.N}, C.options());
   p.dB = dB.data_ptr(), p.dC = dC.data_ptr();
   c10::DeviceGuard guard(dev);
+  const int owned = ssd_bwd_overwrites(&p);
+  if (!(owned & SSD_OVERWRITES_DCB)) dCB.zero_();
+  if (!(owned & SSD_OVERWRITES_DBC)) dB32.zero_(), dC32.zero_();
   void *stream = stream_of(dev);
   check_rc(ssd_bmm_chunk_fwd(&p, stream), "ssd_bmm_chunk_fwd");  // CB: the fused forward never forms it
   check_rc(ssd_combined_bwd(&p, stream), "ssd_combined_bwd");

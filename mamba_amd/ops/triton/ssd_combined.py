@@ -205,17 +205,17 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
     gbuf = torch.empty_like(dz) if z is not None else None
     ddt_out_view = ddt
     ddt = torch.empty(batch, seqlen, nheads, device=dev, dtype=dt.dtype)
-    # one zeroed arena for every accumulator the kernels add into
+    # one zeroed arena for the small accumulators the kernels add into; the three large ones (dCB, dB32, dC32) are
+    # cleared further down, and only where the library does not write them whole (ssd_bwd_overwrites)
     sizes = dict(dA=nheads, ddt_bias=nheads, dD=(D.numel() if D is not None else 0),
                  ddA_cumsum=batch * nheads * nchunks * chunk_size, ddt_out=batch * nheads * nchunks * chunk_size,
                  dCB=batch * nchunks * ngroups * chunk_size * chunk_size,
                  dB32=batch * seqlen * ngroups * dstate, dC32=batch * seqlen * ngroups * dstate)
-    # dCB needs no clearing when one workgroup owns each of its tiles (at most 16 heads per group, float sums)
-    dcb_owned = nheads // ngroups <= 16 and not use_deterministic_mode()
-    arena = torch.zeros(sum(n for k, n in sizes.items() if not (k == "dCB" and dcb_owned)), **f32)
+    large = ("dCB", "dB32", "dC32")
+    arena = torch.zeros(sum(n for k, n in sizes.items() if k not in large), **f32)
     acc, off = {}, 0
     for k, n in sizes.items():
-        if k == "dCB" and dcb_owned:
+        if k in large:
             acc[k] = torch.empty(n, **f32)
             continue
         acc[k] = arena[off:off + n]
@@ -262,6 +262,12 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
             off += n
     lib = _lib.load()
     with torch.cuda.device(dev):
+        owned = lib.ssd_bwd_overwrites(p)  # which of the large sum buffers the kernels store rather than add into
+        if not owned & 1:
+            acc["dCB"].zero_()
+        if not owned & 2:
+            acc["dB32"].zero_()
+            acc["dC32"].zero_()
         stream = _lib.current_stream(dev)
         # forward workspaces: kept from the forward pass, or re-computed as the reference does
         # (ssd_combined.py:441-448); CB is always re-computed (the fused forward never forms it)
