@@ -470,12 +470,14 @@ std::optional<TensorList> ssd_bwd_fast(const at::Tensor &dout, const at::Tensor 
   // cleared below, and only where the library does not write them whole (ssd_bwd_overwrites)
   const int64_t nD = D ? D->numel() : 0, nHcQ = d.batch * d.H * d.nchunks * d.Q;
   const int64_t nCB = d.batch * d.nchunks * d.G * d.Q * d.Q, nBC = d.batch * d.L * d.G * d.N;
-  const int64_t sizes[5] = {d.H, d.H, nD, nHcQ, nHcQ};
-  int64_t total = 0, off[5];
-  for (int i = 0; i < 5; ++i) off[i] = total, total += sizes[i];
-  at::Tensor arena = at::zeros({total}, f32);
+  const int64_t sizes[8] = {d.H, d.H, nD, nHcQ, nHcQ, nCB, nBC, nBC};  // the five small ones first
+  int64_t total = 0, off[8];
+  for (int i = 0; i < 8; ++i) {
+    if (i == 5) total = (total + 63) / 64 * 64;  // the large ones start on 256 bytes
+    off[i] = total, total += sizes[i];
+  }
+  at::Tensor arena = at::empty({total}, f32);
   float *base = arena.data_ptr<float>();
-  at::Tensor dCB = at::empty({nCB}, f32), dB32 = at::empty({nBC}, f32), dC32 = at::empty({nBC}, f32);
   at::Tensor dstates = at::empty({d.batch, d.nchunks, d.H, d.P, d.N}, d.lp ? x.options() : f32);
   if (initial_states) dinit = at::empty({d.batch, d.H, d.P, d.N}, f32);
   p.dt_out = dt_out.data_ptr<float>(), p.dA_cumsum = dA_cumsum.data_ptr<float>();
@@ -489,7 +491,7 @@ std::optional<TensorList> ssd_bwd_fast(const at::Tensor &dout, const at::Tensor 
   p.dx_bs = dx.stride(0), p.dx_ls = dx.stride(1), p.dx_hs = dx.stride(2);
   p.dA = base + off[0], p.ddt_bias = base + off[1], p.dD = D ? base + off[2] : nullptr;
   p.ddA_cumsum = base + off[3], p.ddt_out = base + off[4];
-  p.dB32 = dB32.data_ptr<float>(), p.dC32 = dC32.data_ptr<float>(), p.dCB = dCB.data_ptr<float>();
+  p.dCB = base + off[5], p.dB32 = base + off[6], p.dC32 = base + off[7];
   p.dinitial_states = dinit ? dinit->data_ptr<float>() : nullptr;
   if (d.lp) p.dstates_lp = dstates.data_ptr(); else p.dstates = dstates.data_ptr<float>();
   // dB / dC in the operands' dtype: written by the call's last stage
@@ -497,8 +499,13 @@ std::optional<TensorList> ssd_bwd_fast(const at::Tensor &dout, const at::Tensor 
   p.dB = dB.data_ptr(), p.dC = dC.data_ptr();
   c10::DeviceGuard guard(dev);
   const int owned = ssd_bwd_overwrites(&p);
-  if (!(owned & SSD_OVERWRITES_DCB)) dCB.zero_();
-  if (!(owned & SSD_OVERWRITES_DBC)) dB32.zero_(), dC32.zero_();
+  if (owned == 0) {
+    arena.zero_();  // one fill
+  } else {
+    arena.narrow(0, 0, off[5]).zero_();
+    if (!(owned & SSD_OVERWRITES_DCB)) arena.narrow(0, off[5], nCB).zero_();
+    if (!(owned & SSD_OVERWRITES_DBC)) arena.narrow(0, off[6], 2 * nBC).zero_();  // dB32 and dC32 are neighbours
+  }
   void *stream = stream_of(dev);
   check_rc(ssd_bmm_chunk_fwd(&p, stream), "ssd_bmm_chunk_fwd");  // CB: the fused forward never forms it
   check_rc(ssd_combined_bwd(&p, stream), "ssd_combined_bwd");

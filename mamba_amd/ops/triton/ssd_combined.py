@@ -212,14 +212,14 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
                  dCB=batch * nchunks * ngroups * chunk_size * chunk_size,
                  dB32=batch * seqlen * ngroups * dstate, dC32=batch * seqlen * ngroups * dstate)
     large = ("dCB", "dB32", "dC32")
-    arena = torch.zeros(sum(n for k, n in sizes.items() if k not in large), **f32)
+    n_small = -(-sum(n for k, n in sizes.items() if k not in large) // 64) * 64  # the large ones start on 256 bytes
+    arena = torch.empty(n_small + sum(sizes[k] for k in large), **f32)  # the small accumulators first
     acc, off = {}, 0
-    for k, n in sizes.items():
-        if k in large:
-            acc[k] = torch.empty(n, **f32)
-            continue
-        acc[k] = arena[off:off + n]
-        off += n
+    for k in sizes:
+        if k == large[0]:
+            off = n_small
+        acc[k] = arena[off:off + sizes[k]]
+        off += sizes[k]
     lp = x.dtype == torch.bfloat16  # the carried states' gradients pass between the stages in bf16 too
     dstates = torch.empty(batch, nchunks, nheads, headdim, dstate, device=dev, dtype=torch.bfloat16 if lp else torch.float32)
     dinit = torch.empty(batch, nheads, headdim, dstate, **f32) if initial_states is not None else None
@@ -263,11 +263,14 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
     lib = _lib.load()
     with torch.cuda.device(dev):
         owned = lib.ssd_bwd_overwrites(p)  # which of the large sum buffers the kernels store rather than add into
-        if not owned & 1:
-            acc["dCB"].zero_()
-        if not owned & 2:
-            acc["dB32"].zero_()
-            acc["dC32"].zero_()
+        if owned == 0:
+            arena.zero_()  # one fill
+        else:
+            arena[:n_small].zero_()
+            if not owned & 1:
+                acc["dCB"].zero_()
+            if not owned & 2:
+                arena[n_small + sizes["dCB"]:].zero_()  # dB32 and dC32 are neighbours
         stream = _lib.current_stream(dev)
         # forward workspaces: kept from the forward pass, or re-computed as the reference does
         # (ssd_combined.py:441-448); CB is always re-computed (the fused forward never forms it)
