@@ -146,9 +146,10 @@ def cpu_model():
 
 
 def cpu_baseline(seqlen, dstate, full_dim):
-    """Oracle (a PyTorch restatement of the reference's selective_scan_ref) on the host cores: forward alone (median
-    of 3) and forward + backward (median of 2), on a batch-1 slice of one sixteenth of the channels; channels and
-    batch rows are independent in the scan, so tokens/s of the whole workload is the slice's rate x slice / whole."""
+    """Oracle (a PyTorch restatement of the reference's selective_scan_ref) on the host cores: forward alone and
+    forward + backward, each the median of 5 runs (~10 s of CPU work in all), on a batch-1 slice of one sixteenth of
+    the channels; channels and batch rows are independent in the scan, so tokens/s of the whole workload is the
+    slice's rate x slice / whole."""
     import statistics
     import torch
     from oracle.mamba1 import selective_scan_oracle, scan_inputs
@@ -167,15 +168,15 @@ def cpu_baseline(seqlen, dstate, full_dim):
                 out.backward(t["dout"])
         return time.perf_counter() - t0
 
-    fwd = statistics.median(run(False) for _ in range(3))
-    both = statistics.median(run(True) for _ in range(2))
+    fwd = statistics.median(run(False) for _ in range(5))
+    both = statistics.median(run(True) for _ in range(5))
     scale = dim / full_dim
     return {"value": seqlen * scale / both, "unit": "tokens/s", "cores": cores, "kind": "port",
             "fwd_only_value": seqlen * scale / fwd, "cpu": cpu_model(),
             "slice_seconds": {"forward": fwd, "forward_backward": both},
             "sample": f"oracle.mamba1.selective_scan_oracle, batch 1 x {dim} of {full_dim} channels x seqlen {seqlen} "
-                      f"(1/16 of the channels of one of 8 batch rows): forward {fwd:.2f} s (median of 3), forward + "
-                      f"backward {both:.2f} s (median of 2); tokens/s of the whole workload = {seqlen} x {dim}/{full_dim} / seconds"}
+                      f"(1/16 of the channels of one of 8 batch rows): forward {fwd:.2f} s, forward + "
+                      f"backward {both:.2f} s (medians of 5); tokens/s of the whole workload = {seqlen} x {dim}/{full_dim} / seconds"}
 
 
 def cpu_baseline_ssd():

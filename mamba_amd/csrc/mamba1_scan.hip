@@ -741,7 +741,10 @@ template <typename T, bool BWD, int BC> int dispatch_bc(const MambaScanParams &p
   const int np = (p.dstate + NB16 - 1) / NB16 * NB16;
   const bool vec = vec_ok(p, BWD);
   if (!BWD) {
-    const size_t lds = fwd_lds(1, np);
+    // MAMBA_AMD_FWD_MIN_LDS (bytes): a measurement hook.  A workgroup that asks for more LDS shares its CU with fewer
+    // others (160 KB per CU), which is how the kernel's speed against resident waves per SIMD is measured.
+    static const size_t min_lds = getenv("MAMBA_AMD_FWD_MIN_LDS") ? (size_t)atol(getenv("MAMBA_AMD_FWD_MIN_LDS")) : 0;
+    const size_t lds = fwd_lds(1, np) > min_lds ? fwd_lds(1, np) : min_lds;
     return vec ? launch(scan_fwd_kernel<T, true, BC>, p, 1, lds, stream)
                : launch(scan_fwd_kernel<T, false, BC>, p, 1, lds, stream);
   }
