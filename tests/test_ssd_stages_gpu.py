@@ -118,7 +118,8 @@ def _passing_ref64(states, dAc, init, seq_chunk=None):
 
 
 @pytest.mark.parametrize("has_init", [False, True])
-@pytest.mark.parametrize("nchunks,dim", [(1, 64), (7, 2048), (33, 1000), (16, 8192), (5, 77)])
+# (2100 and 8300 chunks are beyond what the kernels keep as per-chunk tables in LDS: backward only, then both)
+@pytest.mark.parametrize("nchunks,dim", [(1, 64), (7, 2048), (33, 1000), (16, 8192), (5, 77), (2100, 1024), (8300, 64)])
 def test_state_passing_fwd_bwd(nchunks, dim, has_init):
     from mamba_amd.ops.triton.ssd_state_passing import state_passing, state_passing_ref
     g = torch.Generator().manual_seed(nchunks * 1000 + dim)
