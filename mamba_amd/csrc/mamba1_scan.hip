@@ -28,13 +28,19 @@
 
 size_t mamba1_bwd_mx_lds(int passes, int np);                                                       // mamba1_scan_bwd_mx.hip
 int mamba1_bwd_mx_launch(const MambaScanParams &p, int passes, bool vec, hipStream_t stream);  // likewise
+size_t mamba1_bwd_k4_lds(int passes);                                                          // mamba1_scan_bwd_k4.hip
+bool mamba1_bwd_k4_serves(const MambaScanParams &p);                                           // likewise
+int mamba1_bwd_k4_launch(const MambaScanParams &p, int pa, int pb, int nparts, hipStream_t stream);  // likewise
 
 namespace {
 
 // ------------------------------------------------------------------ forward
 // BC: bit 0 = B is an input-independent (dim, dstate) fp32 matrix, bit 1 = C likewise
 // (selective_scan_fwd_kernel.cuh:74 kIsVariableB / kIsVariableC false).
-template <typename T, bool VEC, int BC>
+// HALF: a checkpoint every 64 positions instead of every 128 (the state entering lane 8 of a row is the state after
+// the tile's first 64 positions): ckpt is then (batch, dim, ceil(L / 64), N).  For the backward kernel that walks
+// 64-position tiles (mamba1_scan_bwd_k4.hip).
+template <typename T, bool VEC, int BC, bool HALF>
 __global__ __launch_bounds__(NTHREADS, 4) void scan_fwd_kernel(const MambaScanParams p, const int passes) {
   extern __shared__ __align__(16) float smem[];
   const int N = p.dstate, L = p.seqlen;
@@ -43,6 +49,7 @@ __global__ __launch_bounds__(NTHREADS, 4) void scan_fwd_kernel(const MambaScanPa
   float *Cs = Bs + BC_FLOATS;
   float *A2s = Cs + BC_FLOATS;                 // [passes * PASS_CH][NP]  A * log2(e)
   float *hcar = A2s + passes * PASS_CH * NP;   // [passes * PASS_CH][NP]  state carried across tiles
+  float *hmid = hcar + passes * PASS_CH * NP;  // [passes * PASS_CH][NP]  state after the tile's first half (HALF)
 
   const int tid = threadIdx.x, lane = tid & 63, c = lane & (RL - 1), rsel = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -97,6 +104,7 @@ __global__ __launch_bounds__(NTHREADS, 4) void scan_fwd_kernel(const MambaScanPa
         }
         const float *A2row = A2s + chw * NP + nb * NB16;
         float *hrow = hcar + chw * NP + nb * NB16;
+        float *mrow = hmid + chw * NP + nb * NB16;
         const int nmax = min(NB16, N - nb * NB16);
         // two states per iteration: their row scans are interleaved (padded rows are inert:
         // A = 0, B = C = 0)
@@ -130,6 +138,9 @@ __global__ __launch_bounds__(NTHREADS, 4) void scan_fwd_kernel(const MambaScanPa
           for (int s = 0; s < 2; ++s) {
             float h = dpp_f<DPP_ROW_SHR + 1>(hc[s], hend[s]);  // state entering this lane
             if (c == RL - 1) hrow[n + s] = hend[s];            // state after the tile
+            if constexpr (HALF) {
+              if (c == RL / 2) mrow[n + s] = h;                // state after the tile's first half
+            }
 #pragma unroll
             for (int i = 0; i < KI; ++i) {
               h = __builtin_fmaf(a[s][i], h, bb[s][i]);
@@ -151,9 +162,18 @@ __global__ __launch_bounds__(NTHREADS, 4) void scan_fwd_kernel(const MambaScanPa
       }
       st8_guard<T, VEC>((T *)p.out + b * p.out_bs + d * p.out_ds + tl, nvalid, y);
       if (valid) {  // a row's own lanes wrote its slots of hcar: no other wave touches them
-        float *ck = p.ckpt + (((int64_t)b * p.dim + d) * q.ntiles + tile) * N;
         const float *hfin = hcar + chw * NP;
-        for (int n = c; n < N; n += RL) ck[n] = hfin[n];
+        if constexpr (HALF) {
+          const int nhalf = (L + TILE / 2 - 1) / (TILE / 2);
+          float *ck = p.ckpt + (((int64_t)b * p.dim + d) * nhalf + 2 * tile) * N;
+          const float *hm = hmid + chw * NP;
+          for (int n = c; n < N; n += RL) ck[n] = hm[n];
+          if (2 * tile + 1 < nhalf)
+            for (int n = c; n < N; n += RL) ck[N + n] = hfin[n];
+        } else {
+          float *ck = p.ckpt + (((int64_t)b * p.dim + d) * q.ntiles + tile) * N;
+          for (int n = c; n < N; n += RL) ck[n] = hfin[n];
+        }
       }
     }
   }
@@ -164,8 +184,9 @@ __global__ __launch_bounds__(NTHREADS, 4) void scan_fwd_kernel(const MambaScanPa
 // `passes` passes of PASS_CH channels per tile; the dB / dC sums of all of them leave once per tile as
 // partial number (workgroup's place in its group), or after every pass and block when the states come
 // in blocks of 16 (the host side then asks for one pass).
+// ck_half: the checkpoints come every 64 positions (see scan_fwd_kernel): the state entering tile t is slot 2 t - 1.
 template <typename T, bool VEC, int BC>
-__global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParams p, const int passes) {
+__global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParams p, const int passes, const int ck_half) {
   extern __shared__ __align__(16) float smem[];
   const int N = p.dstate, L = p.seqlen;
   const int NBLK = (N + NB16 - 1) / NB16, NP = NBLK * NB16;
@@ -227,7 +248,7 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
     w.ddelta = (T *)p.ddelta + b * p.ddelta_bs + d * p.ddelta_ds;
     w.dz = has_z ? (T *)p.dz + b * p.dz_bs + d * p.dz_ds : nullptr;
     w.out_z = (has_z && p.out_z) ? (T *)p.out_z + b * p.outz_bs + d * p.outz_ds : nullptr;
-    w.ckpt = p.ckpt + ((int64_t)b * p.dim + d) * ntiles * N;
+    w.ckpt = p.ckpt + ((int64_t)b * p.dim + d) * (ck_half ? (L + TILE / 2 - 1) / (TILE / 2) : ntiles) * N;
     w.D = p.D ? ((const float *)p.D)[d] : 0.f;
     w.bias = p.delta_bias ? ((const float *)p.delta_bias)[d] : 0.f;
     rows[i] = w;
@@ -249,7 +270,7 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
     // No branch around any of these loads (the checkpoint of tile 0 stands in where there is none to read, the u
     // row where there is no z): with the same memory operations on every path through a step the compiler counts
     // those in flight exactly, and a wait for these rows leaves the younger stores of the step before draining.
-    k.ck = *(const GLOBAL_AS float *)(w.ckpt + (int64_t)max(tile - 1, 0) * N + min(c, N - 1));
+    k.ck = *(const GLOBAL_AS float *)(w.ckpt + (int64_t)max(ck_half ? 2 * tile - 1 : tile - 1, 0) * N + min(c, N - 1));
     load_items<T, VEC>(k.u, w.u, tl, L, nvalid);
     load_items<T, VEC>(k.delta, w.delta, tl, L, nvalid);
     load_items<T, VEC>(k.dout, w.dout, tl, L, nvalid);
@@ -306,7 +327,8 @@ __global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParam
         } else {
           for (int n = c; n < NP; n += RL) {
             float v = 0.f;
-            if (tile > 0 && n < N) v = *(const GLOBAL_AS float *)(rows[chw].ckpt + (int64_t)(tile - 1) * N + n);
+            if (tile > 0 && n < N)
+              v = *(const GLOBAL_AS float *)(rows[chw].ckpt + (int64_t)(ck_half ? 2 * tile - 1 : tile - 1) * N + n);
             hcar[chl * NP + n] = v;
           }
         }
@@ -591,7 +613,9 @@ __global__ __launch_bounds__(256) void reduce_parts_kernel(const float *__restri
 // ------------------------------------------------------------------ launch
 inline bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
 
-inline size_t fwd_lds(int passes, int np) { return sizeof(float) * (2 * BC_FLOATS + 2 * passes * PASS_CH * np); }
+inline size_t fwd_lds(int passes, int np, bool half) {
+  return sizeof(float) * (2 * BC_FLOATS + (half ? 3 : 2) * passes * PASS_CH * np);
+}
 inline size_t bwd_lds(int passes, int np, int bc) {
   const int wch = passes * PASS_CH;
   return sizeof(float) * (2 * BC_FLOATS + 2 * ACC_FLOATS + PASS_CH * np + (bc ? 6 : 4) * wch * np + 2 * wch) +
@@ -616,6 +640,18 @@ int compute_units() {
 // default.  MAMBA_AMD_M1_BWD=mx in the environment (read once) sends bf16 rows with per-position B and C to the kernel
 // whose dB / dC sums are formed by the matrix cores (mamba1_scan_bwd_mx.hip): measured 8 % slower at batch 8 x 5120
 // channels x 4096 positions x 16 states, kept for comparisons.
+// MAMBA_AMD_M1_BWD=k4 (read once): checkpoints every 64 positions from the forward kernel, and the backward kernel
+// that walks 64-position tiles with 4 items per lane (mamba1_scan_bwd_k4.hip) where it serves the problem; the default
+// backward kernel reads the denser checkpoints everywhere else.
+bool k4_mode() {
+  static const int want = [] {
+    const char *e = getenv("MAMBA_AMD_M1_BWD");
+    return (e && e[0] == 'k') ? 1 : 0;
+  }();
+  return want != 0;
+}
+int ckpt_tile(bool a_complex) { return a_complex ? TILE_COMPLEX : (k4_mode() ? TILE / 2 : TILE); }
+
 bool use_mx(const MambaScanParams &p) {
   static const int want_mx = [] {
     const char *e = getenv("MAMBA_AMD_M1_BWD");
@@ -646,7 +682,32 @@ int bwd_passes(const MambaScanParams &p) {
   return best;
 }
 
+// The 4-items-per-lane backward kernel (k4 mode): two workgroups share a compute unit, so its workgroups may take
+// pa and pb passes alternately (the long and the short one of a unit); pa == pb: all the same.  Chosen like
+// bwd_passes: rounds of workgroups over the units' two places, times the mean passes of a round.
+struct K4Plan {
+  int pa, pb, nparts;
+};
+K4Plan k4_plan(const MambaScanParams &p) {
+  const int Dg = p.dim / p.ngroups, cus = compute_units();
+  static const int cand[6][2] = {{1, 1}, {2, 1}, {2, 2}, {3, 1}, {3, 2}, {3, 3}};
+  K4Plan best{1, 1, 1};
+  double best_cost = -1;
+  for (const auto &c : cand) {
+    const int pa = c[0], pb = c[1];
+    if (mamba1_bwd_k4_lds(pa) > LDS_LIMIT / 2) continue;
+    if (pa > 1 && (pa - 1) * PASS_CH >= Dg) continue;
+    const int per = pa == pb ? (Dg + PASS_CH * pa - 1) / (PASS_CH * pa) : 2 * ((Dg + PASS_CH * (pa + pb) - 1) / (PASS_CH * (pa + pb)));
+    const int64_t wgs = (int64_t)p.batch * p.ngroups * per;
+    const double cost = (double)((wgs + 2 * cus - 1) / (2 * cus)) * 0.5 * (pa + pb);
+    if (best_cost < 0 || cost <= best_cost) best_cost = cost, best = K4Plan{pa, pb, per};
+  }
+  return best;
+}
+bool use_k4(const MambaScanParams &p) { return k4_mode() && mamba1_bwd_k4_serves(p); }
+
 int bwd_nparts(const MambaScanParams &p) {
+  if (use_k4(p)) return k4_plan(p).nparts;
   const int Dg = p.dim / p.ngroups, r = bwd_passes(p);
   return (Dg + PASS_CH * r - 1) / (PASS_CH * r) * (p.dstate > NB16 ? r : 1);
 }
@@ -676,14 +737,14 @@ bool mamba1_allow_lds(const void *kernel, size_t lds) {
 
 namespace {
 
-template <typename KernelT>
-int launch(KernelT kernel, const MambaScanParams &p, int passes, size_t lds, hipStream_t stream) {
+template <typename KernelT, typename... Extra>
+int launch(KernelT kernel, const MambaScanParams &p, int passes, size_t lds, hipStream_t stream, Extra... extra) {
   const int Dg = p.dim / p.ngroups;
   const int cblocks = (Dg + PASS_CH * passes - 1) / (PASS_CH * passes);
   if (lds > LDS_LIMIT) return MAMBA_E_UNSUPPORTED;
   if (!mamba1_allow_lds(reinterpret_cast<const void *>(kernel), lds)) return MAMBA_E_LAUNCH;
   dim3 grid(p.ngroups * cblocks, p.batch), block(NTHREADS);
-  hipLaunchKernelGGL(kernel, grid, block, lds, stream, p, passes);
+  hipLaunchKernelGGL(kernel, grid, block, lds, stream, p, passes, extra...);
   return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
 }
 
@@ -744,9 +805,31 @@ template <typename T, bool BWD, int BC> int dispatch_bc(const MambaScanParams &p
     // MAMBA_AMD_FWD_MIN_LDS (bytes): a measurement hook.  A workgroup that asks for more LDS shares its CU with fewer
     // others (160 KB per CU), which is how the kernel's speed against resident waves per SIMD is measured.
     static const size_t min_lds = getenv("MAMBA_AMD_FWD_MIN_LDS") ? (size_t)atol(getenv("MAMBA_AMD_FWD_MIN_LDS")) : 0;
-    const size_t lds = fwd_lds(1, np) > min_lds ? fwd_lds(1, np) : min_lds;
-    return vec ? launch(scan_fwd_kernel<T, true, BC>, p, 1, lds, stream)
-               : launch(scan_fwd_kernel<T, false, BC>, p, 1, lds, stream);
+    const bool half = k4_mode();
+    const size_t lds = fwd_lds(1, np, half) > min_lds ? fwd_lds(1, np, half) : min_lds;
+    if (half)
+      return vec ? launch(scan_fwd_kernel<T, true, BC, true>, p, 1, lds, stream)
+                 : launch(scan_fwd_kernel<T, false, BC, true>, p, 1, lds, stream);
+    return vec ? launch(scan_fwd_kernel<T, true, BC, false>, p, 1, lds, stream)
+               : launch(scan_fwd_kernel<T, false, BC, false>, p, 1, lds, stream);
+  }
+  if (use_k4(plan)) {
+    const K4Plan k = k4_plan(plan);
+    if (vec) {
+      if constexpr (std::is_same_v<T, bf16_t> && BC == 0) {
+        const int rc = mamba1_bwd_k4_launch(p, k.pa, k.pb, k.nparts, stream);
+        return rc != MAMBA_OK ? rc : reduce_dBC<T>(p, k.nparts, stream);
+      }
+    }
+    // rows the 4-item kernel does not take (unaligned views): the default kernel with as many passes as a long and a
+    // short workgroup together, whose partials are fewer than the workspace was sized for: the others are cleared
+    const int64_t bytes = (int64_t)p.batch * p.ngroups * k.nparts * p.dstate * p.seqlen * 4;
+    int rc = mamba_hip_zero(p.dB32, bytes, stream);
+    if (rc == MAMBA_OK) rc = mamba_hip_zero(p.dC32, bytes, stream);
+    if (rc != MAMBA_OK) return rc;
+    const int passes = k.pa == k.pb ? k.pa : k.pa + k.pb;
+    rc = launch(scan_bwd_kernel<T, false, BC>, p, passes, bwd_lds(passes, np, BC), stream, 1);
+    return rc != MAMBA_OK ? rc : reduce_dBC<T>(p, k.nparts, stream);
   }
   const int passes = bwd_passes(plan);
   if (use_mx(p)) {
@@ -754,8 +837,9 @@ template <typename T, bool BWD, int BC> int dispatch_bc(const MambaScanParams &p
     return rc != MAMBA_OK ? rc : reduce_dBC<T>(p, bwd_nparts(plan), stream);
   }
   const size_t lds = bwd_lds(passes, np, BC);
-  const int rc = vec ? launch(scan_bwd_kernel<T, true, BC>, p, passes, lds, stream)
-                     : launch(scan_bwd_kernel<T, false, BC>, p, passes, lds, stream);
+  const int ck_half = k4_mode() ? 1 : 0;
+  const int rc = vec ? launch(scan_bwd_kernel<T, true, BC>, p, passes, lds, stream, ck_half)
+                     : launch(scan_bwd_kernel<T, false, BC>, p, passes, lds, stream, ck_half);
   return rc != MAMBA_OK ? rc : reduce_dBC<T>(p, bwd_nparts(plan), stream);
 }
 
@@ -776,7 +860,7 @@ MambaScanParams batch_slice(const MambaScanParams &p, int64_t b0, int nb, int np
   MambaScanParams q = p;
   q.batch = nb;
   const int64_t es = p.dtype == MAMBA_F32 ? 4 : 2, cx = p.a_complex ? 2 : 1;
-  const int tile = p.a_complex ? TILE_COMPLEX : TILE;
+  const int tile = ckpt_tile(p.a_complex);
   const int64_t ntiles = (p.seqlen + tile - 1) / tile, N = p.dstate, L = p.seqlen, G = p.ngroups, D = p.dim;
   auto adv = [&](auto *&ptr, int64_t elems, int64_t size) {
     if (ptr) ptr = reinterpret_cast<std::remove_reference_t<decltype(ptr)>>(
@@ -800,7 +884,7 @@ MambaScanParams batch_slice(const MambaScanParams &p, int64_t b0, int nb, int np
 
 int mamba1_scan_complex(const MambaScanParams *p, hipStream_t s, bool bwd);  // mamba1_scan_complex.hip
 
-int mamba1_scan_tile(bool a_complex) { return a_complex ? TILE_COMPLEX : TILE; }  // positions per checkpoint tile
+int mamba1_scan_tile(bool a_complex) { return ckpt_tile(a_complex); }  // positions per checkpoint tile
 
 namespace {
 int scan_fwd_one(const MambaScanParams &p, hipStream_t s) {
@@ -898,7 +982,7 @@ extern "C" int mamba_hip_init(void) { return scratch_for_current_device() ? MAMB
 extern "C" int mamba1_scan_fwd_noalloc(const MambaScanParams *p, float *last_state, mamba_stream_t stream) {
   if (!p) return MAMBA_E_BADARG;
   if (p->batch <= 0 || p->dim <= 0 || p->seqlen <= 0 || p->dstate <= 0) return MAMBA_E_BADARG;
-  const int tile = p->a_complex ? TILE_COMPLEX : TILE;
+  const int tile = ckpt_tile(p->a_complex);
   const int ntiles = (p->seqlen + tile - 1) / tile;
   const int width = p->dstate * (p->a_complex ? 2 : 1);
   const int64_t rows = (int64_t)p->batch * p->dim;
