@@ -383,13 +383,17 @@ int ssd_chunk_state_varlen(const SsdParams *p, const int32_t *cu_seqlens, int ns
  * ddA_cumsum holds the gradient with respect to the cumulative sums a_l; the last
  * stage turns it into the gradient of the per-position dt * A. */
 int ssd_bwd_dz(const SsdParams *p, mamba_stream_t stream);
-/* Which of the sum buffers the backward pass of this (completely filled) problem writes whole instead of adding
- * into, so that the caller may hand them over uncleared: a set of the flags below; 0 in the deterministic mode, for a
- * problem run in batch slices, or for a bad argument.  Clearing a buffer that is reported here is harmless.  No
+/* What the caller may leave out for the backward pass of this (completely filled, CB apart) problem: which of the sum
+ * buffers the kernels write whole instead of adding into, so that they may be handed over uncleared, and whether CB
+ * is needed at all: a set of the flags below; 0 in the deterministic mode, for a problem run in batch slices, or for
+ * a bad argument.  Clearing a buffer that is reported here is harmless.  No
  * counterpart in the reference, whose Triton kernels write partial sums to fresh buffers and add them up with
  * torch (mamba_ssm/ops/triton/ssd_combined.py:441-509). */
 #define SSD_OVERWRITES_DCB 1 /* dCB: at most 16 heads per group */
 #define SSD_OVERWRITES_DBC 2 /* dB32 and dC32: one workgroup of the state-path stage holds all heads of a group */
+#define SSD_BWD_FORMS_CB 4   /* not about clearing: the backward pass does not need CB from the caller (who may skip
+                                ssd_bmm_chunk_fwd and pass CB = NULL): the dCB stage forms its tiles of C B^T itself and
+                                the dx stage runs its fused kernel.  Passing CB anyway is always correct. */
 int ssd_bwd_overwrites(const SsdParams *p);
 /* dst[i] = shadow[i] / s for i < n (det_scale = {s, 1 / s} on the device): the step between the stages of a
  * deterministic backward pass that ssd_combined_bwd inserts by itself */

@@ -1029,7 +1029,9 @@ template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256, 4)
 // one sequence.  One workgroup per (batch, chunk, group, lower-triangular 64 x 64 tile pair) loops
 // over the heads of the group with the sum in registers.  Per head, w = (head's term) * CB gives
 // the in-chunk share of ddA_cumsum: + row sums at l, - column sums at s.
-template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256, 4) void bwd_dcb_kernel(const SsdParams p) {
+// FORM_CB: no CB buffer (p.CB null), the workgroup forms its tile of C B^T itself.
+template <typename T, bool SPLIT, bool DET, bool FORM_CB = false>
+__global__ __launch_bounds__(256, 4) void bwd_dcb_kernel(const SsdParams p) {
   __shared__ GemmLds lds;
   __shared__ float hA_l[2][GB], hA_s[2][GB], hdt[2][GB];  // per-head rows, double-buffered over the head loop
   // the heads' ddA_cumsum shares (row sums per column half, column sums per row half), flushed at the end: a
@@ -1050,11 +1052,25 @@ template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256, 4)
   const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L + t0 : nullptr;
   const View4 gv = g_view(p);
   const int64_t dCB_off = (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
-  const float *CB = p.CB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
   // This lane's 16 accumulator positions: CB there (the same for every head) and the causal /
-  // same-sequence mask, kept as zeros in cbr and a bit per position.
+  // same-sequence mask, kept as zeros in cbr and a bit per position.  Without a CB buffer (p.CB null: the caller
+  // skipped ssd_bmm_chunk_fwd, see ssd_bwd_overwrites) the workgroup forms its tile of C B^T itself, with the same
+  // pipeline, before the heads' products.
   float cbr[2][2][4];
   uint32_t live = 0;
+  GemmAcc sum, acc;
+  sum.zero();
+  acc.zero();
+  if constexpr (FORM_CB) {
+    const T *Cl = static_cast<const T *>(p.C) + b * p.C_bs + g * p.C_gs + (int64_t)(t0 + lt * GB) * p.C_ls;
+    const T *Bsr = static_cast<const T *>(p.B) + b * p.B_bs + g * p.B_gs + (int64_t)(t0 + st * GB) * p.B_ls;
+    block_gemm_pipe<SPLIT>(
+        acc, lds, 0, p.dstate,
+        KcStager<SPLIT, T>(lds.ah, lds.al, Cl, p.C_ls, qlim - lt * GB, p.dstate, nullptr, nullptr, rows_aligned16(Cl, p.C_ls), tid),
+        KcStager<SPLIT, T>(lds.bh, lds.bl, Bsr, p.B_ls, qlim - st * GB, p.dstate, nullptr, nullptr, rows_aligned16(Bsr, p.B_ls), tid),
+        tid);
+  }
+  const float *CB = FORM_CB ? nullptr : p.CB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
 #pragma unroll
   for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
@@ -1063,12 +1079,14 @@ template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256, 4)
       for (int r = 0; r < 4; ++r) {
         const int l = lt * GB + wm * 32 + tm * 16 + gq * 4 + r, s = st * GB + wn * 32 + tn * 16 + i;
         const bool ok = l < qlim && s <= l && (!seq || seq[l] == seq[s]);
-        cbr[tm][tn][r] = ok ? CB[(int64_t)l * Q + s] : 0.f;
+        if constexpr (FORM_CB) {
+          cbr[tm][tn][r] = ok ? acc.v[tm][tn][r] : 0.f;
+          acc.v[tm][tn][r] = 0.f;
+        } else {
+          cbr[tm][tn][r] = ok ? CB[(int64_t)l * Q + s] : 0.f;
+        }
         live |= (uint32_t)ok << ((tm * 2 + tn) * 4 + r);
       }
-  GemmAcc sum, acc;
-  sum.zero();
-  acc.zero();
   // One pipeline over the heads of this workgroup: k runs over (head, p), a head's product is
   // finished, weighted and added to the sum at its last k step, and the loads of the next head are
   // already in flight then.
@@ -1392,9 +1410,9 @@ int check_bwd(const SsdParams *p) {
   if (p->chunk_size > 256 || p->dstate > 256 || p->headdim > 256) return MAMBA_E_UNSUPPORTED;
   if ((int64_t)p->batch * p->nheads > 65535 || p->nchunks > 65535) return MAMBA_E_UNSUPPORTED;
   if (p->dtype != MAMBA_F32 && p->dtype != MAMBA_BF16 && p->dtype != MAMBA_F16) return MAMBA_E_BADARG;
-  if (!p->dt_out || !p->dA_cumsum || !p->CB || !p->ddA_cumsum || !p->ddt_out || !p->dCB || !p->dB32 || !p->dC32 ||
+  if (!p->dt_out || !p->dA_cumsum || !p->ddA_cumsum || !p->ddt_out || !p->dCB || !p->dB32 || !p->dC32 ||
       !p->dx || !p->ddt || !p->dA)
-    return MAMBA_E_BADARG;
+    return MAMBA_E_BADARG;  // (CB may be null: ssd_bwd_dcb then forms its tiles itself; the tiled dx kernel refuses)
   // the carried states and their gradients: bf16 buffers next to bf16 operands, the fp32 ones otherwise
   if (p->dtype == MAMBA_BF16) {
     if (!p->states_lp || !p->dstates_lp) return MAMBA_E_BADARG;
@@ -1508,6 +1526,7 @@ static int ssd_bwd_dx_one(const SsdParams *p, mamba_stream_t stream) {
   // bf16 on the common shapes: the fused kernel, which forms C B^T itself (p->CB is not read); else the tiled one
   rc = ssd_bwd_dx_fused_launch(p, s);
   if (rc != MAMBA_E_UNSUPPORTED) return rc;
+  if (!p->CB) return MAMBA_E_BADARG;  // the tiled kernel reads C B^T
   dim3 grid(tiles(p->chunk_size) * tiles(p->headdim), p->nchunks, p->batch * p->nheads);
   SSD_DISPATCH_DET(bwd_dx_kernel, grid)
   return launched();
@@ -1547,6 +1566,15 @@ static int ssd_bwd_dcb_one(const SsdParams *p, mamba_stream_t stream) {
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int nt = tiles(p->chunk_size);
   dim3 grid(nt * (nt + 1) / 2, p->nchunks, p->batch * p->ngroups * dcb_head_splits(p->nheads / p->ngroups));
+  if (!p->CB) {  // the workgroups form their tiles of C B^T themselves (default mode only: ssd_bwd_overwrites)
+    if (p->det_scale) return MAMBA_E_BADARG;
+    switch (p->dtype) {
+      case MAMBA_BF16: hipLaunchKernelGGL((bwd_dcb_kernel<bf16_t, false, false, true>), grid, dim3(256), 0, s, *p); break;
+      case MAMBA_F16: hipLaunchKernelGGL((bwd_dcb_kernel<f16_t, true, false, true>), grid, dim3(256), 0, s, *p); break;
+      default: hipLaunchKernelGGL((bwd_dcb_kernel<float, true, false, true>), grid, dim3(256), 0, s, *p); break;
+    }
+    return launched();
+  }
   SSD_DISPATCH_DET(bwd_dcb_kernel, grid)
   return launched();
 }
@@ -1714,6 +1742,9 @@ extern "C" int ssd_bwd_overwrites(const SsdParams *p) {
   int flags = 0;
   if (dcb_head_splits(p->nheads / p->ngroups) == 1) flags |= SSD_OVERWRITES_DCB;
   if (ssd_bwd_dbc_fused_owns(p)) flags |= SSD_OVERWRITES_DBC;
+  // CB: only the dCB stage and the tiled dx kernel read it.  Where the fused dx kernel runs and a group is one head
+  // list (so that each tile of C B^T would be formed once), the dCB stage can form its tiles itself.
+  if (dcb_head_splits(p->nheads / p->ngroups) == 1 && ssd_bwd_dx_fused_supported(p)) flags |= SSD_BWD_FORMS_CB;
   return flags;
 }
 

@@ -355,6 +355,8 @@ bool supported(const SsdParams *p) {
 
 }  // namespace
 
+bool ssd_bwd_dx_fused_supported(const SsdParams *p) { return supported(p); }
+
 int ssd_bwd_dx_fused_launch(const SsdParams *p, hipStream_t stream) {
   if (!supported(p)) return MAMBA_E_UNSUPPORTED;
   return p->det_scale ? launch_p<true>(*p, stream) : launch_p<false>(*p, stream);

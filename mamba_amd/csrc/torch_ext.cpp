@@ -507,7 +507,9 @@ std::optional<TensorList> ssd_bwd_fast(const at::Tensor &dout, const at::Tensor 
     if (!(owned & SSD_OVERWRITES_DBC)) arena.narrow(0, off[6], 2 * nBC).zero_();  // dB32 and dC32 are neighbours
   }
   void *stream = stream_of(dev);
-  check_rc(ssd_bmm_chunk_fwd(&p, stream), "ssd_bmm_chunk_fwd");  // CB: the fused forward never forms it
+  // CB: the fused forward never forms it; the backward kernels may not need it either
+  if (owned & SSD_BWD_FORMS_CB) p.CB = nullptr;
+  else check_rc(ssd_bmm_chunk_fwd(&p, stream), "ssd_bmm_chunk_fwd");
   check_rc(ssd_combined_bwd(&p, stream), "ssd_combined_bwd");
   auto piece = [&](int i, at::IntArrayRef shape) { return arena.narrow(0, off[i], sizes[i]).view(shape); };
   TensorList r(9);

@@ -273,9 +273,13 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
                 arena[n_small + sizes["dCB"]:].zero_()  # dB32 and dC32 are neighbours
         stream = _lib.current_stream(dev)
         # forward workspaces: kept from the forward pass, or re-computed as the reference does
-        # (ssd_combined.py:441-448); CB is always re-computed (the fused forward never forms it)
-        stages = ("ssd_bmm_chunk_fwd",) if saved is not None else (
-            "ssd_chunk_cumsum_fwd", "ssd_chunk_state_fwd", "ssd_state_passing_fwd", "ssd_bmm_chunk_fwd")
+        # (ssd_combined.py:441-448); CB is re-computed (the fused forward never forms it) unless the library says
+        # that its backward kernels do not read it (flag 4: the dCB stage then forms its tiles of C B^T itself)
+        stages = () if saved is not None else ("ssd_chunk_cumsum_fwd", "ssd_chunk_state_fwd", "ssd_state_passing_fwd")
+        if owned & 4:
+            p.CB = None
+        else:
+            stages += ("ssd_bmm_chunk_fwd",)
         for stage in stages:
             _lib.check(getattr(lib, stage)(p, stream), stage)
         _lib.check(lib.ssd_combined_bwd(p, stream), "ssd_combined_bwd")

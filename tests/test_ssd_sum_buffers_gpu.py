@@ -1,6 +1,6 @@
-"""Which sum buffers of the SSD backward pass need clearing (ssd_bwd_overwrites in include/mamba_hip.h): the host
-sides hand the large ones (dCB, dB32 / dC32) over uncleared where the library reports that its kernels store them
-whole.  Here the allocator's free blocks are filled with NaN first, so an entry that a kernel adds into, or never
+"""Which sum buffers of the SSD backward pass need clearing, and whether it needs CB (ssd_bwd_overwrites in
+include/mamba_hip.h): the host sides hand the large buffers (dCB, dB32 / dC32) over uncleared where the library reports
+that its kernels store them whole, and skip the C B^T stage where the dCB kernel forms its tiles itself.  Here the allocator's free blocks are filled with NaN first, so an entry that a kernel adds into, or never
 writes, although it was reported as stored would come back as NaN; the gradients are then held to the oracle."""
 import pytest
 import torch
@@ -21,10 +21,11 @@ def _poison(nbytes):
 
 
 # flags: 8 heads per group and enough (batch, chunk) pairs that the state-path stage gives a whole group to one
-# workgroup (2; with few pairs it prefers more, shorter head lists) and one head list owns each dCB tile (1); 16 heads
-# per group = the dCB tiles only; 32 per group = neither
+# workgroup (2; with few pairs it prefers more, shorter head lists), one head list owns each dCB tile (1) and forms
+# its tile of C B^T itself, so that CB is not passed at all (4); 16 heads per group = the dCB tiles and CB only; 32 per
+# group = none
 @pytest.mark.parametrize("host", ["extension", "python"])
-@pytest.mark.parametrize("H,G,L,Q,expect", [(16, 2, 4096, 64, 3), (16, 1, 1024, 256, 1), (32, 1, 1024, 256, 0)])
+@pytest.mark.parametrize("H,G,L,Q,expect", [(16, 2, 4096, 64, 7), (16, 1, 1024, 256, 5), (32, 1, 1024, 256, 0)])
 @pytest.mark.parametrize("packed", [False, True])
 def test_uncleared_sum_buffers(monkeypatch, H, G, L, Q, expect, packed, host):
     from mamba_amd import _lib
