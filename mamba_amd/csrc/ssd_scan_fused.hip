@@ -203,8 +203,9 @@ __global__ __launch_bounds__(64 * QT) void chunk_scan_fwd_fused_kernel(const Ssd
         acc[pt] = v * rs;
       }
     }
-    // The epilogue's x (for D) and z rows are requested two blocks before the wave's last one.  No branch around
-    // these loads either (rows past the end re-read the last row and are not stored; without z the x row stands in).
+    // The epilogue's z rows are requested two blocks before the wave's last one.  No branch around these loads
+    // either (rows past the end re-read the last row and are not stored; without z the x row stands in).  Its x rows
+    // (for D) are taken from the head's X rows in LDS when the wave leaves the loop, before the patches overlay them.
     const bf16_t *xt = static_cast<const bf16_t *>(p.x) + b * p.x_bs + h * p.x_hs + (int64_t)t0 * p.x_ls;
     const bf16_t *zt = has_z ? static_cast<const bf16_t *>(p.z) + b * p.z_bs + h * p.z_hs + (int64_t)t0 * p.z_ls : xt;
     const int64_t zls = has_z ? p.z_ls : p.x_ls;
@@ -214,7 +215,6 @@ __global__ __launch_bounds__(64 * QT) void chunk_scan_fwd_fused_kernel(const Ssd
       for (int q = 0; q < EQ; ++q) {
         const int id = lane + q * 64, rr = id / (P / 8), c8 = id % (P / 8);
         const int64_t row = min(lt * 16 + rr, qlim - 1);
-        xe[q] = *(const GLOBAL_AS u32x4 *)(xt + row * p.x_ls + c8 * 8);
         ze[q] = *(const GLOBAL_AS u32x4 *)(zt + row * zls + c8 * 8);
       }
     };
@@ -267,6 +267,11 @@ __global__ __launch_bounds__(64 * QT) void chunk_scan_fwd_fused_kernel(const Ssd
     // ---- the next head's operands are requested by each wave as it leaves the loop; the epilogue's patches lie
     // over X and the state, so it starts once every wave has left
     if (hh + 1 < hb) load_head(h + per);
+#pragma unroll
+    for (int q = 0; q < EQ; ++q) {
+      const int id = lane + q * 64, rr = id / (P / 8), c8 = id % (P / 8);
+      xe[q] = *reinterpret_cast<const u32x4 *>(&Xs[(lt * 16 + rr) * XP + c8 * 8]);
+    }
     lds_barrier();
     // epilogue: + D x, pre-gate copy, gate.  Each wave transposes its 16 rows through a private LDS patch so that
     // out / out_x stores are 16-byte pieces of contiguous rows (the accumulator layout itself would scatter 8-byte
