@@ -97,6 +97,8 @@ def profile_traffic_sum(filename):
             if cols[:1] == ["kernel"]:
                 seen = True
                 continue
+            if cols[:2] == ["rows", "below:"] or cols[:1] == ["sum"]:
+                break  # what follows is not part of a default step
             if seen and len(cols) >= 5:
                 try:
                     total += (float(cols[-2]) + float(cols[-1])) * 1e6
