@@ -206,17 +206,10 @@ __global__ __launch_bounds__(64 * QT) void bwd_dx_fused_kernel(const SsdParams p
     };
     const float q1 = x_dot(acc);
 
-    // The epilogue's g rows (for D) and this lane's x values (for ddt) are requested before the wave's last two
-    // blocks; no branch around the loads.
-    const bf16_t *gt = static_cast<const bf16_t *>(gv.ptr) + b * gv.bs + h * gv.hs + (int64_t)t0 * gv.ls;
+    // This lane's x values (for ddt) are requested again before the wave's last two blocks; no branch around the loads.
     const bf16_t *xcol = static_cast<const bf16_t *>(p.x) + b * p.x_bs + h * p.x_hs + (int64_t)(t0 + s_row) * p.x_ls + 4 * g;
     u32x4 ge[EQ];
     auto epilogue_prefetch = [&]() {
-#pragma unroll
-      for (int q = 0; q < EQ; ++q) {
-        const int id = lane + q * 64, rr = id / (P / 8), c8 = id % (P / 8);
-        ge[q] = *(const GLOBAL_AS u32x4 *)(gt + (int64_t)min(lt * 16 + rr, qlim - 1) * gv.ls + c8 * 8);
-      }
 #pragma unroll
       for (int pt = 0; pt < PT; ++pt) xl[pt] = *(const GLOBAL_AS u32x2 *)(xcol + pt * 16);  // again, for ddt
     };
@@ -280,6 +273,12 @@ __global__ __launch_bounds__(64 * QT) void bwd_dx_fused_kernel(const SsdParams p
     // ---- each wave requests the next head's operands as it leaves the loop; the epilogue's patches lie over g and
     // the state gradient, so it starts once every wave has left
     if (hh + 1 < hb) load_head(h + per);
+    // the epilogue's g rows (for D) come from the head's rows in LDS, before the patches overlay them
+#pragma unroll
+    for (int q = 0; q < EQ; ++q) {
+      const int id = lane + q * 64, rr = id / (P / 8), c8 = id % (P / 8);
+      ge[q] = *reinterpret_cast<const u32x4 *>(&Gs[(lt * 16 + rr) * XP + c8 * 8]);
+    }
     lds_barrier();
     {
       bf16_t *dxg = static_cast<bf16_t *>(p.dx) + b * p.dx_bs + h * p.dx_hs + (int64_t)(t0 + lt * 16) * p.dx_ls;
