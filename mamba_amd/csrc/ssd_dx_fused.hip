@@ -206,13 +206,7 @@ __global__ __launch_bounds__(64 * QT) void bwd_dx_fused_kernel(const SsdParams p
     };
     const float q1 = x_dot(acc);
 
-    // This lane's x values (for ddt) are requested again before the wave's last two blocks; no branch around the loads.
-    const bf16_t *xcol = static_cast<const bf16_t *>(p.x) + b * p.x_bs + h * p.x_hs + (int64_t)(t0 + s_row) * p.x_ls + 4 * g;
     u32x4 ge[EQ];
-    auto epilogue_prefetch = [&]() {
-#pragma unroll
-      for (int pt = 0; pt < PT; ++pt) xl[pt] = *(const GLOBAL_AS u32x2 *)(xcol + pt * 16);  // again, for ddt
-    };
 
     // ---- inside the chunk: the l blocks from the one that holds the wave's diagonal on
     const float as2 = a2_s[s_own];
@@ -220,7 +214,6 @@ __global__ __launch_bounds__(64 * QT) void bwd_dx_fused_kernel(const SsdParams p
 #pragma unroll
     for (int sb = 0; sb < NSB; ++sb) {
       if (sb < first) continue;
-      if (sb == max(NSB - 3, first)) epilogue_prefetch();
       float m[8];
 #pragma unroll
       for (int h2 = 0; h2 < 2; ++h2) {
