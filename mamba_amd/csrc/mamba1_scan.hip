@@ -184,9 +184,10 @@ __global__ __launch_bounds__(NTHREADS, 4) void scan_fwd_kernel(const MambaScanPa
 // `passes` passes of PASS_CH channels per tile; the dB / dC sums of all of them leave once per tile as
 // partial number (workgroup's place in its group), or after every pass and block when the states come
 // in blocks of 16 (the host side then asks for one pass).
-// ck_half: the checkpoints come every 64 positions (see scan_fwd_kernel): the state entering tile t is slot 2 t - 1.
-template <typename T, bool VEC, int BC>
-__global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParams p, const int passes, const int ck_half) {
+// CKH: the checkpoints come every 64 positions (see scan_fwd_kernel): the state entering tile t is slot 2 t - 1.
+template <typename T, bool VEC, int BC, bool CKH>
+__global__ __launch_bounds__(NTHREADS) void scan_bwd_kernel(const MambaScanParams p, const int passes) {
+  constexpr bool ck_half = CKH;
   extern __shared__ __align__(16) float smem[];
   const int N = p.dstate, L = p.seqlen;
   const int NBLK = (N + NB16 - 1) / NB16, NP = NBLK * NB16;
@@ -737,14 +738,14 @@ bool mamba1_allow_lds(const void *kernel, size_t lds) {
 
 namespace {
 
-template <typename KernelT, typename... Extra>
-int launch(KernelT kernel, const MambaScanParams &p, int passes, size_t lds, hipStream_t stream, Extra... extra) {
+template <typename KernelT>
+int launch(KernelT kernel, const MambaScanParams &p, int passes, size_t lds, hipStream_t stream) {
   const int Dg = p.dim / p.ngroups;
   const int cblocks = (Dg + PASS_CH * passes - 1) / (PASS_CH * passes);
   if (lds > LDS_LIMIT) return MAMBA_E_UNSUPPORTED;
   if (!mamba1_allow_lds(reinterpret_cast<const void *>(kernel), lds)) return MAMBA_E_LAUNCH;
   dim3 grid(p.ngroups * cblocks, p.batch), block(NTHREADS);
-  hipLaunchKernelGGL(kernel, grid, block, lds, stream, p, passes, extra...);
+  hipLaunchKernelGGL(kernel, grid, block, lds, stream, p, passes);
   return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
 }
 
@@ -828,7 +829,7 @@ template <typename T, bool BWD, int BC> int dispatch_bc(const MambaScanParams &p
     if (rc == MAMBA_OK) rc = mamba_hip_zero(p.dC32, bytes, stream);
     if (rc != MAMBA_OK) return rc;
     const int passes = k.pa == k.pb ? k.pa : k.pa + k.pb;
-    rc = launch(scan_bwd_kernel<T, false, BC>, p, passes, bwd_lds(passes, np, BC), stream, 1);
+    rc = launch(scan_bwd_kernel<T, false, BC, true>, p, passes, bwd_lds(passes, np, BC), stream);
     return rc != MAMBA_OK ? rc : reduce_dBC<T>(p, k.nparts, stream);
   }
   const int passes = bwd_passes(plan);
@@ -837,9 +838,13 @@ template <typename T, bool BWD, int BC> int dispatch_bc(const MambaScanParams &p
     return rc != MAMBA_OK ? rc : reduce_dBC<T>(p, bwd_nparts(plan), stream);
   }
   const size_t lds = bwd_lds(passes, np, BC);
-  const int ck_half = k4_mode() ? 1 : 0;
-  const int rc = vec ? launch(scan_bwd_kernel<T, true, BC>, p, passes, lds, stream, ck_half)
-                     : launch(scan_bwd_kernel<T, false, BC>, p, passes, lds, stream, ck_half);
+  int rc;
+  if (k4_mode())
+    rc = vec ? launch(scan_bwd_kernel<T, true, BC, true>, p, passes, lds, stream)
+             : launch(scan_bwd_kernel<T, false, BC, true>, p, passes, lds, stream);
+  else
+    rc = vec ? launch(scan_bwd_kernel<T, true, BC, false>, p, passes, lds, stream)
+             : launch(scan_bwd_kernel<T, false, BC, false>, p, passes, lds, stream);
   return rc != MAMBA_OK ? rc : reduce_dBC<T>(p, bwd_nparts(plan), stream);
 }
 
