@@ -195,7 +195,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dst
   const int tid = threadIdx.x;
   const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads;
   const int ntn = cdiv(N, GB);
-  const Block3 blk = xcd_block();  // the tiles of one (chunk, head) share its x / g rows: same L2
+  const Block3 blk = xcd_block_heads(H);  // the tiles of one (chunk, head) share its x / g rows: same L2
   const int pt = blk.x / ntn, nt = blk.x % ntn;
   const int c = blk.y, b = blk.z / H, h = blk.z % H;
   const int g = h / (H / p.ngroups);
@@ -240,7 +240,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bwd_dst
   const int tid = threadIdx.x;
   const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads;
   const int ntn = N / WB;
-  const Block3 blk = xcd_block();
+  const Block3 blk = xcd_block_heads(H);
   const int pt = blk.x / ntn, nt = blk.x % ntn;
   const int c = blk.y, b = blk.z / H, h = blk.z % H;
   const int g = h / (H / p.ngroups);
@@ -324,7 +324,7 @@ template <typename T> __global__ __launch_bounds__(256) void bwd_dz_dstates_kern
   __shared__ float rs[256];
   const int tid = threadIdx.x;
   const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads;
-  const Block3 blk = xcd_block();
+  const Block3 blk = xcd_block_heads(H);
   const int pt = blk.x;  // one 128-state tile: a p tile's rows are read by one workgroup only
   const int c = blk.y, b = blk.z / H, h = blk.z % H;
   const int g = h / (H / p.ngroups);

@@ -696,6 +696,17 @@ DEVI Block3 xcd_block() {
   const int lid = xcd_linear_block();
   return {lid % nx, (lid / nx) % ny, lid / (nx * ny)};
 }
+// For a grid of (tiles, chunks, batch * heads) whose workgroups of one (batch, chunk) share that chunk's B / C rows of
+// their group: {tile, chunk, batch * H + head} with the heads next to each other in the logical order, then the
+// chunks, then the batch rows.  With the chunks next to each other instead (xcd_block) a group's rows of a chunk come
+// round again only after every other chunk of the sequence, and on a long sequence (128 chunks) they have left the L2
+// by then: the product kernels of the packed benchmark read them once per head from memory.
+DEVI Block3 xcd_block_heads(int H) {
+  const int nx = gridDim.x, ny = gridDim.y;
+  const int lid = xcd_linear_block();
+  const int rest = lid / nx, h = rest % H, c = (rest / H) % ny, b = rest / (H * ny);
+  return {lid % nx, c, b * H + h};
+}
 
 // ---- pieces shared by the backward kernels
 struct View4 {  // (b, L, H, P) tensor, P stride 1

@@ -112,7 +112,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void chunk_s
   const int tid = threadIdx.x;
   const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads;
   const int ntn = cdiv(N, GB);
-  const Block3 blk = xcd_block();  // the tiles of one (chunk, head) share its x / g rows: same L2
+  const Block3 blk = xcd_block_heads(H);  // the tiles of one (chunk, head) share its x / g rows: same L2
   const int pt = blk.x / ntn, nt = blk.x % ntn;
   const int c = blk.y, b = blk.z / H, h = blk.z % H;
   const int g = h / (H / p.ngroups);
@@ -162,7 +162,7 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void chunk_s
   const int tid = threadIdx.x;
   const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, P = p.headdim, H = p.nheads;
   const int ntn = N / WB;
-  const Block3 blk = xcd_block();
+  const Block3 blk = xcd_block_heads(H);
   const int pt = blk.x / ntn, nt = blk.x % ntn;
   const int c = blk.y, b = blk.z / H, h = blk.z % H;
   const int g = h / (H / p.ngroups);
