@@ -428,9 +428,9 @@ def bench_ssd(dev, steps, warmup):
         "dtype": "bf16 in/out, fp32 accumulation", "data": "synthetic",
         "config": {"workload": f"Mamba-2 SSD fwd+bwd: batch {batch}, seqlen {L}, {H} heads x {P}, d_state {N}, "
                                f"{G} group, chunk {Q}, bf16 (benchmark configuration 2)"},
-        "roofline": vs_measured_copy({"bound": "hbm", "kernel": "chunk_scan_fwd_fused_kernel", "achieved": nbytes / scan_ms / 1e6,
+        "roofline": vs_measured_copy({"bound": "hbm", "kernel": "chunk_scan_fwd_paired_kernel", "achieved": nbytes / scan_ms / 1e6,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / scan_ms / 1e6 / HBM_PEAK_GBS,
-                     "traffic": profile_traffic(prof + "_hbm_counters.txt", "chunk_scan_fwd_fused_kernel"),
+                     "traffic": profile_traffic(prof + "_hbm_counters.txt", "chunk_scan_fwd_paired_kernel"),
                      "kernel_ms": scan_ms, "kernel_ms_min_max_n": [scan["min"], scan["max"], scan["n"]],
                      "algorithmic_bytes": nbytes,
                      "algorithmic_flops": flops, "mfma_tflops": flops / scan_ms / 1e9,
@@ -439,7 +439,7 @@ def bench_ssd(dev, steps, warmup):
                      "flop_per_byte": flops / nbytes, "mfma_cap_from_hbm_tflops": flops / nbytes * HBM_PEAK_GBS / 1e3,
                      "measured_mfma_tflops": mfma_tflops,
                      "mfma_frac_of_measured": flops / scan_ms / 1e9 / mfma_tflops,
-                     "mfma_counters": mfma_counters(prof + "_mfma_counters.txt", "chunk_scan_fwd_fused_kernel")}, dev)})
+                     "mfma_counters": mfma_counters(prof + "_mfma_counters.txt", "chunk_scan_fwd_paired_kernel")}, dev)})
 
 
 def mfma_counters(filename, kernel):
@@ -647,10 +647,10 @@ def bench_varlen(dev, steps, warmup):
         "step_roofline": {"bound": "hbm", "algorithmic_bytes": step_bytes, "achieved": step_bytes / sec / 1e9,
                           "frac": step_bytes / sec / 1e9 / HBM_PEAK_GBS, "unit": "GB/s",
                           "traffic": profile_traffic_sum(prof + "_hbm_counters.txt")},
-        "roofline": vs_measured_copy({"bound": "hbm", "kernel": "chunk_scan_fwd_fused_kernel",
+        "roofline": vs_measured_copy({"bound": "hbm", "kernel": "chunk_scan_fwd_paired_kernel",
                      "achieved": scan_bytes / scan_ms / 1e6, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": scan_bytes / scan_ms / 1e6 / HBM_PEAK_GBS,
-                     "traffic": profile_traffic(prof + "_hbm_counters.txt", "chunk_scan_fwd_fused_kernel"),
+                     "traffic": profile_traffic(prof + "_hbm_counters.txt", "chunk_scan_fwd_paired_kernel"),
                      "kernel_ms": scan_ms, "kernel_ms_min_max_n": [scan["min"], scan["max"], scan["n"]],
                      "algorithmic_bytes": scan_bytes, "algorithmic_flops": flops,
                      "mfma_tflops": flops / scan_ms / 1e9, "mfma_frac_of_bf16_peak": flops / scan_ms / 1e9 / 2500.0}, dev)})

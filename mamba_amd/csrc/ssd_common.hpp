@@ -783,6 +783,11 @@ inline int heads_per_workgroup(const SsdParams &p) {
   return best;
 }
 
+// The fused chunk scan with two tiles per wave (ssd_scan_paired.hip), for problems that
+// ssd_chunk_scan_fwd_fused_supported accepts.
+bool ssd_scan_paired_serves(const SsdParams &p);
+int ssd_scan_paired_launch(const SsdParams &p, hipStream_t s);
+
 // ------------------------------------------------------------------ batch slices
 // The kernels index (batch, head) pairs with one 16-bit grid coordinate.  A larger problem is served by the entry
 // points in slices of whole batch rows (rows are independent; the sums shared by all rows -- dA, dD, ddt_bias and

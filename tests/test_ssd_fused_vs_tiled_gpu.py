@@ -43,6 +43,8 @@ def _run(x, dt, A, B, C, D, z, dt_bias, seq_idx, chunk, dout):
     (1, 640, 4, 64, 1, 128, 128, True),     # chunk 128 with 128 states, packed
     (2, 200, 8, 32, 1, 128, 64, False),     # headdim 32 with 128 states, ragged
     (1, 512, 10, 32, 1, 64, 256, False),    # headdim 32 with 64 states, chunk 256
+    (1, 900, 8, 64, 2, 64, 256, True),      # chunk 256, packed, a ragged last chunk with whole tiles past the end
+    (2, 300, 4, 64, 1, 128, 256, False),    # chunk 256, second chunk of 44 positions
 ])
 def test_fused_and_tiled_agree(batch, seqlen, nheads, headdim, ngroups, dstate, chunk, packed):
     _compare(batch, seqlen, nheads, headdim, ngroups, dstate, chunk, packed)

@@ -68,6 +68,9 @@ def test_ssd_fwd_fused_scan_shapes(headdim, dstate, chunk, seqlen):
 def test_ssd_fwd_fused_scan_packed():
     _fwd_case(1, 1024, 4, 64, 128, 2, 256, torch.bfloat16, seq_lens=[300, 212, 100, 156, 256], has_init=True)
     _fwd_case(1, 700, 4, 32, 64, 1, 128, torch.bfloat16, seq_lens=[1, 127, 129, 443])
+    # chunk 256 (two tiles of the chunk per wave): a ragged last chunk with whole tiles past the end, no gate, no D
+    _fwd_case(1, 900, 4, 64, 64, 2, 256, torch.bfloat16, seq_lens=[255, 257, 388], has_z=False, has_D=False)
+    _fwd_case(2, 300, 4, 32, 128, 1, 256, torch.bfloat16, has_init=True)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
