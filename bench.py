@@ -254,6 +254,44 @@ def measured_copy(dev):
     return ms, 2 * nbytes / ms / 1e6
 
 
+def measured_row_pass(dev, batch, seqlen, nheads, n_in):
+    """Runs mamba_hip_rows_probe: a bare pass over (batch, seqlen, nheads, 64) bf16 tensors in the order the SSD
+    kernels visit them (one workgroup per (batch, 256 positions, head); 128-byte rows, nheads * 128 bytes from one
+    position to the next), n_in tensors read and two written.  Returns GB/s: what the layout allows a kernel that
+    touches every row once, beside the rate of the linear copy."""
+    import ctypes
+    import torch
+    from mamba_amd import _lib
+    seqlen = seqlen // 256 * 256
+    t = [torch.empty(batch, seqlen, nheads, 64, dtype=torch.bfloat16, device=dev).fill_(1.0) for _ in range(n_in + 2)]
+    ins = (ctypes.c_void_p * n_in)(*[x.data_ptr() for x in t[:n_in]])
+    outs = (ctypes.c_void_p * 2)(*[x.data_ptr() for x in t[n_in:]])
+    lib = _lib.load()
+    stream = _lib.current_stream(dev)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    nbytes = 0
+    for i in range(11):
+        if i == 1:
+            ev[0].record()
+        nbytes = lib.mamba_hip_rows_probe(ins, n_in, outs, batch, seqlen, nheads, stream)
+        if nbytes <= 0:
+            _lib.check(int(nbytes), "mamba_hip_rows_probe")
+    ev[1].record()
+    torch.cuda.synchronize()
+    return nbytes / (ev[0].elapsed_time(ev[1]) / 10) / 1e6
+
+
+def vs_row_pass(roofline, dev, batch, seqlen, nheads, n_in, moved_bytes):
+    """Adds the rate of the bare row pass with this problem's layout (n_in row tensors read, two written) and the
+    kernel's own rate over the bytes it moves (`moved_bytes` per launch) as a fraction of it."""
+    gbs = measured_row_pass(dev, batch, seqlen, nheads, n_in)
+    roofline["row_pass"] = {"gbs": gbs, "tensors_read": n_in, "tensors_written": 2,
+                            "kernel_moved_bytes": moved_bytes,
+                            "kernel_gbs": moved_bytes / roofline["kernel_ms"] / 1e6,
+                            "frac_of_row_pass": moved_bytes / roofline["kernel_ms"] / 1e6 / gbs}
+    return roofline
+
+
 def copy_calibration(dev):
     ms, gbs = measured_copy(dev)
     print(json.dumps({"kernel": "copy_kernel", "bytes_read": 1 << 30, "bytes_written": 1 << 30, "ms": ms, "GB/s": gbs}))
@@ -428,7 +466,7 @@ def bench_ssd(dev, steps, warmup):
         "dtype": "bf16 in/out, fp32 accumulation", "data": "synthetic",
         "config": {"workload": f"Mamba-2 SSD fwd+bwd: batch {batch}, seqlen {L}, {H} heads x {P}, d_state {N}, "
                                f"{G} group, chunk {Q}, bf16 (benchmark configuration 2)"},
-        "roofline": vs_measured_copy({"bound": "hbm", "kernel": "chunk_scan_fwd_paired_kernel", "achieved": nbytes / scan_ms / 1e6,
+        "roofline": vs_row_pass(vs_measured_copy({"bound": "hbm", "kernel": "chunk_scan_fwd_paired_kernel", "achieved": nbytes / scan_ms / 1e6,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / scan_ms / 1e6 / HBM_PEAK_GBS,
                      "traffic": profile_traffic(prof + "_hbm_counters.txt", "chunk_scan_fwd_paired_kernel"),
                      "kernel_ms": scan_ms, "kernel_ms_min_max_n": [scan["min"], scan["max"], scan["n"]],
@@ -439,7 +477,8 @@ def bench_ssd(dev, steps, warmup):
                      "flop_per_byte": flops / nbytes, "mfma_cap_from_hbm_tflops": flops / nbytes * HBM_PEAK_GBS / 1e3,
                      "measured_mfma_tflops": mfma_tflops,
                      "mfma_frac_of_measured": flops / scan_ms / 1e9 / mfma_tflops,
-                     "mfma_counters": mfma_counters(prof + "_mfma_counters.txt", "chunk_scan_fwd_paired_kernel")}, dev)})
+                     "mfma_counters": mfma_counters(prof + "_mfma_counters.txt", "chunk_scan_fwd_paired_kernel")}, dev),
+                     dev, batch, L, H, 2, nbytes)})
 
 
 def mfma_counters(filename, kernel):
@@ -647,13 +686,14 @@ def bench_varlen(dev, steps, warmup):
         "step_roofline": {"bound": "hbm", "algorithmic_bytes": step_bytes, "achieved": step_bytes / sec / 1e9,
                           "frac": step_bytes / sec / 1e9 / HBM_PEAK_GBS, "unit": "GB/s",
                           "traffic": profile_traffic_sum(prof + "_hbm_counters.txt")},
-        "roofline": vs_measured_copy({"bound": "hbm", "kernel": "chunk_scan_fwd_paired_kernel",
+        "roofline": vs_row_pass(vs_measured_copy({"bound": "hbm", "kernel": "chunk_scan_fwd_paired_kernel",
                      "achieved": scan_bytes / scan_ms / 1e6, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": scan_bytes / scan_ms / 1e6 / HBM_PEAK_GBS,
                      "traffic": profile_traffic(prof + "_hbm_counters.txt", "chunk_scan_fwd_paired_kernel"),
                      "kernel_ms": scan_ms, "kernel_ms_min_max_n": [scan["min"], scan["max"], scan["n"]],
                      "algorithmic_bytes": scan_bytes, "algorithmic_flops": flops,
-                     "mfma_tflops": flops / scan_ms / 1e9, "mfma_frac_of_bf16_peak": flops / scan_ms / 1e9 / 2500.0}, dev)})
+                     "mfma_tflops": flops / scan_ms / 1e9, "mfma_frac_of_bf16_peak": flops / scan_ms / 1e9 / 2500.0}, dev),
+                     dev, batch, L, H, 2, scan_bytes)})
 
 
 def bench_inner(dev, steps, warmup):

@@ -60,6 +60,15 @@ int mamba_hip_copy(void *dst, const void *src, int64_t nbytes, mamba_stream_t st
  * of device memory that is never written. */
 int64_t mamba_hip_mfma_probe(float *sink, int iters, int blocks, mamba_stream_t stream);
 
+/* Measurement yardstick for the SSD kernels, whose operands are (batch, seqlen, nheads, 64) 16-bit tensors of which a
+ * workgroup visits one head's 128-byte rows: a bare pass in that order, one workgroup per (batch, 256 positions,
+ * head), which reads every row of `n_in` (2 or 4) such tensors and writes every row of the two tensors `out`
+ * (xor / sum of the inputs; no LDS, no barrier, two steps of 32 positions in flight).  Its rate is what the layout
+ * allows a kernel that touches each row once.  seqlen must be a multiple of 256, all pointers 16-byte aligned.
+ * Returns the bytes the launch reads and writes (> 0), or an error code (< 0).  No counterpart in the reference. */
+int64_t mamba_hip_rows_probe(const void *const *in, int n_in, void *const *out, int batch, int seqlen, int nheads,
+                             mamba_stream_t stream);
+
 /* Measurement yardstick for the scan kernels, whose time is fp32 vector-ALU issue: launches `blocks` workgroups of
  * 4 waves, each lane running `iters` rounds of 64 v_fma_f32 in sixteen independent chains on register operands.
  * Returns the per-lane instructions of the launch (> 0), or an error code (< 0).  `sink` as above. */

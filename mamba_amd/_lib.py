@@ -194,6 +194,9 @@ def load():
     lib.mamba_hip_mfma_probe.restype = ctypes.c_int64
     lib.mamba_hip_valu_probe.argtypes = [c_vp, ctypes.c_int, ctypes.c_int, c_vp]
     lib.mamba_hip_valu_probe.restype = ctypes.c_int64
+    lib.mamba_hip_rows_probe.argtypes = [ctypes.POINTER(c_vp), ctypes.c_int, ctypes.POINTER(c_vp), ctypes.c_int,
+                                         ctypes.c_int, ctypes.c_int, c_vp]
+    lib.mamba_hip_rows_probe.restype = ctypes.c_int64
     for name in ("norm_residual_fwd", "norm_residual_bwd"):
         fn = getattr(lib, name)
         fn.argtypes = [ctypes.POINTER(NormResidualParams), c_vp]

@@ -51,7 +51,72 @@ __global__ __launch_bounds__(256) void valu_probe_kernel(float *sink, int iters)
   for (int j = 0; j < 16; ++j) s += a[j];
   if (s == -1.f) sink[0] = s;  // never true: keeps the loop alive
 }
+// A bare pass over (batch, position, head, 64 values) 16-bit tensors in the order the SSD kernels visit them: one
+// workgroup per (batch, 256 positions, head) reads the 128-byte rows of NI tensors and writes those of two, 32
+// positions per step with two steps in flight, and the heads of a (batch, chunk) are neighbours in launch order on
+// one XCD.  No arithmetic to speak of, no LDS, no barrier: its rate is what this layout allows a kernel that touches
+// every row once (a row of one head is 128 bytes, the next position's row lies nheads * 128 bytes further).
+struct RowsProbeArgs {
+  const uint16_t *in[4];
+  uint16_t *out[2];
+  int nheads, nchunks;
+};
+template <int NI> __global__ __launch_bounds__(256) void rows_probe_kernel(const RowsProbeArgs a) {
+  const int t = threadIdx.x;
+  const int n = gridDim.x, k = blockIdx.x;
+  const int lid = n % 8 == 0 ? (k % 8) * (n / 8) + k / 8 : k;
+  const int h = lid % a.nheads, c = (lid / a.nheads) % a.nchunks, b = lid / (a.nheads * a.nchunks);
+  const int64_t row = (int64_t)a.nheads * 64;
+  const int64_t base = ((int64_t)b * a.nchunks + c) * 256 * row + h * 64 + (t & 7) * 8 + (int64_t)(t >> 3) * row;
+  constexpr int PF = 2, STEPS = 8;
+  u32x4 q[PF][NI];
+#pragma unroll
+  for (int s = 0; s < PF; ++s)
+#pragma unroll
+    for (int i = 0; i < NI; ++i) q[s][i] = *reinterpret_cast<const u32x4 *>(a.in[i] + base + (int64_t)s * 32 * row);
+#pragma unroll
+  for (int st = 0; st < STEPS; ++st) {
+    const int s = st % PF;
+    u32x4 x = q[s][0], y = q[s][NI - 1];
+#pragma unroll
+    for (int i = 1; i < NI - 1; ++i) {
+      if (i & 1) x ^= q[s][i];
+      else y += q[s][i];
+    }
+    if (st + PF < STEPS) {
+#pragma unroll
+      for (int i = 0; i < NI; ++i) q[s][i] = *reinterpret_cast<const u32x4 *>(a.in[i] + base + (int64_t)(st + PF) * 32 * row);
+    }
+    const int64_t o = base + (int64_t)st * 32 * row;
+    *reinterpret_cast<u32x4 *>(a.out[0] + o) = x;
+    *reinterpret_cast<u32x4 *>(a.out[1] + o) = y;
+  }
+}
 }  // namespace
+
+extern "C" int64_t mamba_hip_rows_probe(const void *const *in, int n_in, void *const *out, int batch, int seqlen,
+                                        int nheads, mamba_stream_t stream) {
+  if (!in || !out || (n_in != 2 && n_in != 4) || batch <= 0 || nheads <= 0 || seqlen <= 0 || seqlen % 256) return MAMBA_E_BADARG;
+  RowsProbeArgs a;
+  for (int i = 0; i < 4; ++i) {
+    a.in[i] = static_cast<const uint16_t *>(in[i < n_in ? i : 0]);
+    if (!a.in[i] || (reinterpret_cast<uintptr_t>(a.in[i]) & 15)) return MAMBA_E_BADARG;
+  }
+  for (int i = 0; i < 2; ++i) {
+    a.out[i] = static_cast<uint16_t *>(out[i]);
+    if (!a.out[i] || (reinterpret_cast<uintptr_t>(a.out[i]) & 15)) return MAMBA_E_BADARG;
+  }
+  a.nheads = nheads, a.nchunks = seqlen / 256;
+  const int64_t wgs = (int64_t)batch * a.nchunks * nheads;
+  if (wgs > 0x7fffffff) return MAMBA_E_UNSUPPORTED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (n_in == 4)
+    hipLaunchKernelGGL(rows_probe_kernel<4>, dim3((unsigned)wgs), dim3(256), 0, s, a);
+  else
+    hipLaunchKernelGGL(rows_probe_kernel<2>, dim3((unsigned)wgs), dim3(256), 0, s, a);
+  if (hipGetLastError() != hipSuccess) return MAMBA_E_LAUNCH;
+  return (int64_t)(n_in + 2) * batch * seqlen * nheads * 64 * 2;  // bytes this launch reads and writes
+}
 
 extern "C" int64_t mamba_hip_valu_probe(float *sink, int iters, int blocks, mamba_stream_t stream) {
   if (!sink || iters <= 0 || blocks <= 0) return MAMBA_E_BADARG;

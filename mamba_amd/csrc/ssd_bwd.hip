@@ -1030,22 +1030,32 @@ template <typename T, bool SPLIT, bool DET> __global__ __launch_bounds__(256, 4)
 // over the heads of the group with the sum in registers.  Per head, w = (head's term) * CB gives
 // the in-chunk share of ddA_cumsum: + row sums at l, - column sums at s.
 // FORM_CB: no CB buffer (p.CB null), the workgroup forms its tile of C B^T itself.
-template <typename T, bool SPLIT, bool DET, bool FORM_CB = false>
-__global__ __launch_bounds__(256, 4) void bwd_dcb_kernel(const SsdParams p) {
-  __shared__ GemmLds lds;
-  __shared__ float hA_l[2][GB], hA_s[2][GB], hdt[2][GB];  // per-head rows, double-buffered over the head loop
+constexpr int DCB_MAXH = 16;  // heads per workgroup (dcb_head_splits keeps it at or below 16)
+struct DcbShared {
+  GemmLds lds;
+  float hA_l[2][GB], hA_s[2][GB], hdt[2][GB];  // per-head rows, double-buffered over the head loop
   // the heads' ddA_cumsum shares (row sums per column half, column sums per row half), flushed at the end: a
   // global atomic per head would sit in the memory queue in front of the next head's loads
-  constexpr int MAXH = 16;  // heads per workgroup (dcb_head_splits keeps it at or below 16)
-  __shared__ float rs_s[2][MAXH][GB], cs_s[2][MAXH][GB];
+  float rs_s[2][DCB_MAXH][GB], cs_s[2][DCB_MAXH][GB];
+};
+// The tile pair (lt, st) of one workgroup.  BELOW: lt > st, the whole tile lies below the diagonal and the decay is
+// factored; the kernel holds both forms as separate bodies, so that each keeps its own registers.
+// FASTP (32 or 64 = headdim; bf16 operands on 16-byte aligned rows, no integer shadows): the heads' products run in a
+// loop of their own instead of the general k pipeline -- a head's two 64 x headdim tiles go from memory to registers
+// to LDS in 16-byte pieces at offsets computed once, one barrier pair and headdim / 32 MFMAs per 16 x 16 tile and
+// head, the next head's tiles in flight under the weights.
+template <typename T, bool SPLIT, bool DET, bool FORM_CB, bool BELOW, int FASTP>
+DEVI void dcb_tile(const SsdParams &p, DcbShared &sh, const Block3 blk, const int lt, const int st) {
+  GemmLds &lds = sh.lds;
+  auto &hA_l = sh.hA_l;
+  auto &hA_s = sh.hA_s;
+  auto &hdt = sh.hdt;
+  auto &rs_s = sh.rs_s;
+  auto &cs_s = sh.cs_s;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
   const int i = lane & 15, gq = lane >> 4;
   const int Q = p.chunk_size, L = p.seqlen, P = p.headdim, H = p.nheads, G = p.ngroups;
-  const Block3 blk = xcd_block();
-  int lt = 0, rem = blk.x;
-  while (rem > lt) { rem -= lt + 1; ++lt; }
-  const int st = rem;
   const int hpg = H / G, nsplit = dcb_head_splits(hpg);
   const int c = blk.y, bg = blk.z / nsplit, hs = blk.z % nsplit, b = bg / G, g = bg % G;
   const int t0 = c * Q, qlim = min(Q, L - t0);
@@ -1092,16 +1102,128 @@ __global__ __launch_bounds__(256, 4) void bwd_dcb_kernel(const SsdParams p) {
   // already in flight then.
   const int nh = (hpg - hs + nsplit - 1) / nsplit;
   const int seg_k = (P + GK - 1) / GK * GK;
-  auto load_rows = [&](int hl) {  // rows of head hl into buffer hl & 1; published by the next step's barriers
-    const int h = g * hpg + hs + hl * nsplit, par = hl & 1;
+  auto load_rows = [&](int hl, int par) {  // rows of head hl into buffer par; published by the next step's barriers
+    const int h = g * hpg + hs + hl * nsplit;
     const float *dA = chunk_row(p.dA_cumsum, p, b, h, c);
     const float *dt = chunk_row(p.dt_out, p, b, h, c);
-    // the exponents' rows are kept times log2(e): the decay of an element is then one v_exp_f32 of a difference
+    // On the diagonal tiles the exponents' rows are kept times log2(e): the decay of an element is then one v_exp_f32
+    // of a difference.  Below the diagonal every l lies after every s, and the decay is taken apart at the l tile's
+    // first position, exp(a_l - a_ref) * exp(a_ref - a_s) with both exponents <= 0: the rows hold the two factors
+    // (one exponential per row and head instead of one per element), the second one times dt_s.
+    if constexpr (BELOW) {
+      const float a_ref = dA[lt * GB] * kLog2e;
+      if (tid < GB) hA_l[par][tid] = lt * GB + tid < Q ? fast_exp2(fminf(dA[lt * GB + tid] * kLog2e - a_ref, 0.f)) : 0.f;
+      else if (tid < 2 * GB) hA_s[par][tid - GB] = dt[st * GB + tid - GB] * fast_exp2(fminf(a_ref - dA[st * GB + tid - GB] * kLog2e, 0.f));
+      return;
+    }
     if (tid < GB) hA_l[par][tid] = lt * GB + tid < Q ? dA[lt * GB + tid] * kLog2e : 0.f;
     else if (tid < 2 * GB) hA_s[par][tid - GB] = st * GB + tid - GB < Q ? dA[st * GB + tid - GB] * kLog2e : 0.f;
     else if (tid < 3 * GB) hdt[par][tid - 2 * GB] = st * GB + tid - 2 * GB < Q ? dt[st * GB + tid - 2 * GB] : 0.f;
   };
-  load_rows(0);
+  load_rows(0, 0);
+  // d = a head's dCB term (added to sum); w = d * CB, whose row / column sums go to ddA
+  auto weigh_head = [&](int hl) {
+    const int par = hl & 1;
+    float a_s[2], dt_s[2] = {0.f, 0.f}, csum[2] = {0.f, 0.f};
+#pragma unroll
+    for (int tn = 0; tn < 2; ++tn) {
+      a_s[tn] = hA_s[par][wn * 32 + tn * 16 + i];
+      if (!BELOW) dt_s[tn] = hdt[par][wn * 32 + tn * 16 + i];
+    }
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = wm * 32 + tm * 16 + gq * 4 + r;
+        const float a_l = hA_l[par][m];
+        float rsum = 0.f;
+#pragma unroll
+        for (int tn = 0; tn < 2; ++tn) {
+          // (not masked here: cbr is zero at the masked positions, so w is, and sum is masked once at the end)
+          const float d = BELOW ? acc.v[tm][tn][r] * a_s[tn] * a_l
+                                : acc.v[tm][tn][r] * dt_s[tn] * fast_exp2(fminf(a_l - a_s[tn], 0.f));
+          acc.v[tm][tn][r] = 0.f;
+          sum.v[tm][tn][r] += d;
+          const float w = d * cbr[tm][tn][r];
+          rsum += w;
+          csum[tn] += w;
+        }
+        rsum += dpp_f<DPP_ROW_SHR + 1>(0.f, rsum);
+        rsum += dpp_f<DPP_ROW_SHR + 2>(0.f, rsum);
+        rsum += dpp_f<DPP_ROW_SHR + 4>(0.f, rsum);
+        rsum += dpp_f<DPP_ROW_SHR + 8>(0.f, rsum);
+        if (i == 15) rs_s[wn][hl][m] = rsum;
+      }
+#pragma unroll
+    for (int tn = 0; tn < 2; ++tn) {
+      float cs = csum[tn];
+      cs += __shfl_xor(cs, 16, 64);
+      cs += __shfl_xor(cs, 32, 64);
+      if (gq == 0) cs_s[wm][hl][wn * 32 + tn * 16 + i] = cs;
+    }
+  };
+  if constexpr (FASTP != 0) {
+    constexpr int PITCH = FASTP + 8, NP = FASTP / 32, KS = FASTP / 32;  // LDS row pitch; pieces per thread and tile; k slices
+    static_assert(2 * GB * PITCH * sizeof(uint16_t) <= sizeof(GemmLds), "both tiles fit in the pipeline's LDS");
+    uint16_t *ga = reinterpret_cast<uint16_t *>(&lds), *xa = ga + GB * PITCH;
+    typedef const GLOBAL_AS char *gptr;
+    // this thread's pieces of a head's tiles: byte offsets from the chunk's first row (rows past the end of the
+    // sequence re-read its last row; what they produce is masked), the same for every head
+    uint32_t goff[NP], xoff[NP];
+    int loff[NP];
+#pragma unroll
+    for (int q = 0; q < NP; ++q) {
+      const int id = tid + q * 256, r = id / (FASTP / 8), c8 = id % (FASTP / 8);
+      goff[q] = (uint32_t)(min(lt * GB + r, qlim - 1) * (int)gv.ls + c8 * 8) * 2u;
+      xoff[q] = (uint32_t)(min(st * GB + r, qlim - 1) * (int)p.x_ls + c8 * 8) * 2u;
+      loff[q] = r * PITCH + c8 * 8;
+    }
+    u32x4 gr[NP], xr[NP];
+    // the first head's rows, and the distance to the next head of this workgroup's list
+    const int h0 = g * hpg + hs;
+    const gptr gb0 = (gptr)(static_cast<const T *>(gv.ptr) + b * gv.bs + h0 * gv.hs + (int64_t)t0 * gv.ls);
+    const gptr xb0 = (gptr)(static_cast<const T *>(p.x) + b * p.x_bs + h0 * p.x_hs + (int64_t)t0 * p.x_ls);
+    const int64_t gstep = (int64_t)nsplit * gv.hs * 2, xstep = (int64_t)nsplit * p.x_hs * 2;
+    auto fetch = [&](int hl) {
+      const gptr gb = gb0 + hl * gstep, xb = xb0 + hl * xstep;
+#pragma unroll
+      for (int q = 0; q < NP; ++q) {
+        gr[q] = *(const GLOBAL_AS u32x4 *)(gb + goff[q]);
+        xr[q] = *(const GLOBAL_AS u32x4 *)(xb + xoff[q]);
+      }
+    };
+    fetch(0);
+#pragma unroll 1
+    for (int hl = 0; hl < nh; ++hl) {
+      lds_barrier();  // every wave is done with the previous head's tiles and rows
+#pragma unroll
+      for (int q = 0; q < NP; ++q) {
+        *reinterpret_cast<u32x4 *>(ga + loff[q]) = gr[q];
+        *reinterpret_cast<u32x4 *>(xa + loff[q]) = xr[q];
+      }
+      load_rows(min(hl + 1, nh - 1), (hl + 1) & 1);  // (after the last head: its own rows again, into the idle buffer)
+      lds_barrier();
+      fetch(min(hl + 1, nh - 1));
+      bf16x8_t af[2][KS], bfr[2][KS];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) {
+          af[t][kk] = *reinterpret_cast<const bf16x8_t *>(&ga[(wm * 32 + t * 16 + i) * PITCH + kk * 32 + gq * 8]);
+          bfr[t][kk] = *reinterpret_cast<const bf16x8_t *>(&xa[(wn * 32 + t * 16 + i) * PITCH + kk * 32 + gq * 8]);
+        }
+#pragma unroll
+      for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < 2; ++tn) {
+          f32x4 v = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int kk = 0; kk < KS; ++kk) v = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[tm][kk], bfr[tn][kk], v, 0, 0, 0);
+          acc.v[tm][tn] = v;
+        }
+      weigh_head(hl);
+    }
+  } else
   // A = g rows (l, k = p), B = x rows (s, k = p): both k-contiguous
   block_gemm_pipe<SPLIT>(
       acc, lds, 0, nh * seg_k,
@@ -1122,46 +1244,9 @@ __global__ __launch_bounds__(256, 4) void bwd_dcb_kernel(const SsdParams p) {
       tid, [&](int k0) {
         const int hl = k0 / seg_k;
         // the buffer written here was last read one step ago, before this step's barriers
-        if (k0 % seg_k == 0 && hl + 1 < nh) load_rows(hl + 1);
+        if (k0 % seg_k == 0 && hl + 1 < nh) load_rows(hl + 1, (hl + 1) & 1);
         if ((k0 + GK) % seg_k != 0) return;
-        const int par = hl & 1;
-        // d = this head's dCB term (added to sum); w = d * CB, whose row / column sums go to ddA
-        float a_s[2], dt_s[2], csum[2] = {0.f, 0.f};
-#pragma unroll
-        for (int tn = 0; tn < 2; ++tn) {
-          a_s[tn] = hA_s[par][wn * 32 + tn * 16 + i];
-          dt_s[tn] = hdt[par][wn * 32 + tn * 16 + i];
-        }
-#pragma unroll
-        for (int tm = 0; tm < 2; ++tm)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int m = wm * 32 + tm * 16 + gq * 4 + r;
-            const float a_l = hA_l[par][m];
-            float rsum = 0.f;
-#pragma unroll
-            for (int tn = 0; tn < 2; ++tn) {
-              // (not masked here: cbr is zero at the masked positions, so w is, and sum is masked once at the end)
-              const float d = acc.v[tm][tn][r] * dt_s[tn] * fast_exp2(fminf(a_l - a_s[tn], 0.f));
-              acc.v[tm][tn][r] = 0.f;
-              sum.v[tm][tn][r] += d;
-              const float w = d * cbr[tm][tn][r];
-              rsum += w;
-              csum[tn] += w;
-            }
-            rsum += dpp_f<DPP_ROW_SHR + 1>(0.f, rsum);
-            rsum += dpp_f<DPP_ROW_SHR + 2>(0.f, rsum);
-            rsum += dpp_f<DPP_ROW_SHR + 4>(0.f, rsum);
-            rsum += dpp_f<DPP_ROW_SHR + 8>(0.f, rsum);
-            if (i == 15) rs_s[wn][hl][m] = rsum;
-          }
-#pragma unroll
-        for (int tn = 0; tn < 2; ++tn) {
-          float cs = csum[tn];
-          cs += __shfl_xor(cs, 16, 64);
-          cs += __shfl_xor(cs, 32, 64);
-          if (gq == 0) cs_s[wm][hl][wn * 32 + tn * 16 + i] = cs;
-        }
+        weigh_head(hl);
       });
   __syncthreads();
   for (int idx = tid; idx < nh * GB; idx += 256) {
@@ -1189,6 +1274,19 @@ __global__ __launch_bounds__(256, 4) void bwd_dcb_kernel(const SsdParams p) {
     }
     return v;
   });
+}
+
+template <typename T, bool SPLIT, bool DET, bool FORM_CB = false, int FASTP = 0>
+__global__ __launch_bounds__(256, 4) void bwd_dcb_kernel(const SsdParams p) {
+  __shared__ DcbShared sh;
+  const Block3 blk = xcd_block();
+  int lt = 0, rem = blk.x;
+  while (rem > lt) { rem -= lt + 1; ++lt; }
+  const int st = rem;
+  if (lt != st)
+    dcb_tile<T, SPLIT, DET, FORM_CB, true, FASTP>(p, sh, blk, lt, st);
+  else
+    dcb_tile<T, SPLIT, DET, FORM_CB, false, FASTP>(p, sh, blk, lt, st);
 }
 
 // ------------------------------------------------------------- bmm bwd
@@ -1566,6 +1664,23 @@ static int ssd_bwd_dcb_one(const SsdParams *p, mamba_stream_t stream) {
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int nt = tiles(p->chunk_size);
   dim3 grid(nt * (nt + 1) / 2, p->nchunks, p->batch * p->ngroups * dcb_head_splits(p->nheads / p->ngroups));
+  // bf16 operands on 16-byte aligned rows of 32 or 64 values, no integer shadows: the head loop of its own
+  const void *gp = p->z ? p->gbuf : p->dout;
+  const int64_t g_ls = p->z ? (int64_t)p->nheads * p->headdim : p->dout_ls, g_hs = p->z ? p->headdim : p->dout_hs,
+                g_bs = p->z ? (int64_t)p->seqlen * p->nheads * p->headdim : p->dout_bs;
+  const bool fast = p->dtype == MAMBA_BF16 && !p->det_scale && (p->headdim == 32 || p->headdim == 64) &&
+                    aligned(gp, 16) && aligned(p->x, 16) && !(g_ls % 8 || g_hs % 8 || g_bs % 8) &&
+                    !(p->x_ls % 8 || p->x_hs % 8 || p->x_bs % 8) && g_ls < (1 << 21) && p->x_ls < (1 << 21);
+  if (fast) {
+    if (p->headdim == 64) {
+      if (p->CB) hipLaunchKernelGGL((bwd_dcb_kernel<bf16_t, false, false, false, 64>), grid, dim3(256), 0, s, *p);
+      else hipLaunchKernelGGL((bwd_dcb_kernel<bf16_t, false, false, true, 64>), grid, dim3(256), 0, s, *p);
+    } else {
+      if (p->CB) hipLaunchKernelGGL((bwd_dcb_kernel<bf16_t, false, false, false, 32>), grid, dim3(256), 0, s, *p);
+      else hipLaunchKernelGGL((bwd_dcb_kernel<bf16_t, false, false, true, 32>), grid, dim3(256), 0, s, *p);
+    }
+    return launched();
+  }
   if (!p->CB) {  // the workgroups form their tiles of C B^T themselves (default mode only: ssd_bwd_overwrites)
     if (p->det_scale) return MAMBA_E_BADARG;
     switch (p->dtype) {
