@@ -1044,8 +1044,10 @@ struct DcbShared {
 // loop of their own instead of the general k pipeline -- a head's two 64 x headdim tiles go from memory to registers
 // to LDS in 16-byte pieces at offsets computed once, one barrier pair and headdim / 32 MFMAs per 16 x 16 tile and
 // head, the next head's tiles in flight under the weights.
+// lp: this workgroup owns its tile, and the next stage takes it as bf16 (what its MFMA operand would round the fp32
+// tile to anyway): the tile is stored as bf16, packed at the start of the dCB buffer.
 template <typename T, bool SPLIT, bool DET, bool FORM_CB, bool BELOW, int FASTP>
-DEVI void dcb_tile(const SsdParams &p, DcbShared &sh, const Block3 blk, const int lt, const int st) {
+DEVI void dcb_tile(const SsdParams &p, DcbShared &sh, const Block3 blk, const int lt, const int st, const bool lp) {
   GemmLds &lds = sh.lds;
   auto &hA_l = sh.hA_l;
   auto &hA_s = sh.hA_s;
@@ -1269,14 +1271,15 @@ DEVI void dcb_tile(const SsdParams &p, DcbShared &sh, const Block3 blk, const in
   acc_foreach(sum, tid, [&](int m, int n, float v) {
     const int l = lt * GB + m, s = st * GB + n;
     if (l < Q && s < Q) {
-      if (own_tile) p.dCB[dCB_off + (int64_t)l * Q + s] = v;
+      if (own_tile && lp) st1<bf16_t>(reinterpret_cast<bf16_t *>(p.dCB) + dCB_off + (int64_t)l * Q + s, v);
+      else if (own_tile) p.dCB[dCB_off + (int64_t)l * Q + s] = v;
       else if (v != 0.f) acc_add<DET ? 1 : 0>(p.dCB, p.det_dCB, dCB_off + (int64_t)l * Q + s, v, det_scale_of(p));
     }
     return v;
   });
 }
 
-template <typename T, bool SPLIT, bool DET, bool FORM_CB = false, int FASTP = 0>
+template <typename T, bool SPLIT, bool DET, bool FORM_CB = false>
 __global__ __launch_bounds__(256, 4) void bwd_dcb_kernel(const SsdParams p) {
   __shared__ DcbShared sh;
   const Block3 blk = xcd_block();
@@ -1284,9 +1287,22 @@ __global__ __launch_bounds__(256, 4) void bwd_dcb_kernel(const SsdParams p) {
   while (rem > lt) { rem -= lt + 1; ++lt; }
   const int st = rem;
   if (lt != st)
-    dcb_tile<T, SPLIT, DET, FORM_CB, true, FASTP>(p, sh, blk, lt, st);
+    dcb_tile<T, SPLIT, DET, FORM_CB, true, 0>(p, sh, blk, lt, st, false);
   else
-    dcb_tile<T, SPLIT, DET, FORM_CB, false, FASTP>(p, sh, blk, lt, st);
+    dcb_tile<T, SPLIT, DET, FORM_CB, false, 0>(p, sh, blk, lt, st, false);
+}
+// bf16 operands on 16-byte aligned rows of FASTP = 32 or 64 values, no integer shadows
+template <bool FORM_CB, int FASTP>
+__global__ __launch_bounds__(256, 4) void bwd_dcb_rows_kernel(const SsdParams p, const int lp) {
+  __shared__ DcbShared sh;
+  const Block3 blk = xcd_block();
+  int lt = 0, rem = blk.x;
+  while (rem > lt) { rem -= lt + 1; ++lt; }
+  const int st = rem;
+  if (lt != st)
+    dcb_tile<bf16_t, false, false, FORM_CB, true, FASTP>(p, sh, blk, lt, st, lp != 0);
+  else
+    dcb_tile<bf16_t, false, false, FORM_CB, false, FASTP>(p, sh, blk, lt, st, lp != 0);
 }
 
 // ------------------------------------------------------------- bmm bwd
@@ -1343,7 +1359,9 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bmm_chu
 
 // The same two products on 64 x 128 tiles (whole 128-state blocks, chunks of whole k steps, 16-byte aligned B / C
 // rows): half the workgroups, each k step of dCB staged once for twice the columns.
-template <typename T, bool SPLIT> DEVI void bmm_chunk_bwd_wide_body(const SsdParams &p, int bx, int by, int bz) {
+// LP: dCB holds bf16 tiles (packed at the start of the buffer; see dcb_tile), which go to LDS as they are.
+template <typename T, bool SPLIT, bool LP = false> DEVI void bmm_chunk_bwd_wide_body(const SsdParams &p, int bx, int by, int bz) {
+  using CBT = std::conditional_t<LP, bf16_t, float>;
   __shared__ GemmLdsWide<SPLIT> lds;
   const int tid = threadIdx.x;
   const int Q = p.chunk_size, N = p.dstate, L = p.seqlen, G = p.ngroups;
@@ -1352,7 +1370,7 @@ template <typename T, bool SPLIT> DEVI void bmm_chunk_bwd_wide_body(const SsdPar
   const int c = by, b = bz / G, g = bz % G;
   const int t0 = c * Q, qlim = min(Q, L - t0);
   if (mt * GB >= qlim) return;
-  const float *dCB = p.dCB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
+  const CBT *dCB = reinterpret_cast<const CBT *>(p.dCB) + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
   const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1, i = lane & 15, gq = lane >> 4;
   // dst[(row of the chunk) * G * N + column] += tile.  This stage is the last one to add into dB32 / dC32 and its
   // tiles cover every row once: with `fin` set the sum leaves here in the operands' dtype as well (dB / dC), and no
@@ -1379,7 +1397,7 @@ template <typename T, bool SPLIT> DEVI void bmm_chunk_bwd_wide_body(const SsdPar
     GemmAccWide acc;
     acc.zero();
     const int kend = min((mt + 1) * GB, qlim);
-    KcStager<SPLIT, float> sa(lds.ah, lds.al, dCB + (int64_t)mt * GB * Q, Q, qlim - mt * GB, kend, nullptr, nullptr, true, tid);
+    KcStager<SPLIT, CBT> sa(lds.ah, lds.al, dCB + (int64_t)mt * GB * Q, Q, qlim - mt * GB, kend, nullptr, nullptr, true, tid);
     const T *Ba = static_cast<const T *>(p.B) + b * p.B_bs + g * p.B_gs + (int64_t)t0 * p.B_ls + nt * WB;
     WideTrStager<SPLIT, T, WB> sb(lds.bh, lds.bl, Ba, p.B_ls, WB, nullptr, tid);
     block_gemm_wide<SPLIT>(acc, lds, kend, sa, sb, tid);
@@ -1391,7 +1409,7 @@ template <typename T, bool SPLIT> DEVI void bmm_chunk_bwd_wide_body(const SsdPar
     GemmAccWide acc;
     acc.zero();
     const int k0 = mt * GB;
-    WideTrStager<SPLIT, float, 64> sa(lds.ah, lds.al, dCB + (int64_t)k0 * Q + mt * GB, Q, min(GB, Q - mt * GB), nullptr, tid);
+    WideTrStager<SPLIT, CBT, 64> sa(lds.ah, lds.al, dCB + (int64_t)k0 * Q + mt * GB, Q, min(GB, Q - mt * GB), nullptr, tid);
     const T *Ca = static_cast<const T *>(p.C) + b * p.C_bs + g * p.C_gs + (int64_t)(t0 + k0) * p.C_ls + nt * WB;
     WideTrStager<SPLIT, T, WB> sb(lds.bh, lds.bl, Ca, p.C_ls, WB, nullptr, tid);
     block_gemm_wide<SPLIT>(acc, lds, qlim - k0, sa, sb, tid);
@@ -1488,11 +1506,11 @@ __global__ __launch_bounds__(256) void chunk_cumsum_bwd_kernel(const SsdParams p
 
 // The last two stages read disjoint results of the stages before them (dCB; ddA_cumsum and ddt_out) and neither
 // fills the chip for long: one launch deals the wide-tile bmm workgroups first and the cumsum workgroups behind them.
-template <typename T, bool SPLIT>
+template <typename T, bool SPLIT, bool LP = false>
 __global__ __launch_bounds__(256) void bmm_cumsum_bwd_kernel(const SsdParams p, int n_bmm, int bmm_x, int bmm_y, int cs_x, int cs_y) {
   const int id = blockIdx.x;
   if (id < n_bmm) {
-    bmm_chunk_bwd_wide_body<T, SPLIT>(p, id % bmm_x, (id / bmm_x) % bmm_y, id / (bmm_x * bmm_y));
+    bmm_chunk_bwd_wide_body<T, SPLIT, LP>(p, id % bmm_x, (id / bmm_x) % bmm_y, id / (bmm_x * bmm_y));
   } else {
     const int k = id - n_bmm;
     chunk_cumsum_bwd_body(p, k % cs_x, (k / cs_x) % cs_y, k / (cs_x * cs_y));
@@ -1658,26 +1676,39 @@ static int ssd_bwd_dBC_state_one(const SsdParams *p, mamba_stream_t stream) {
   return launched();
 }
 
-static int ssd_bwd_dcb_one(const SsdParams *p, mamba_stream_t stream) {
+// The head loop of its own in the dCB stage: bf16 operands on 16-byte aligned rows of 32 or 64 values, no integer
+// shadows.
+static bool dcb_rows_ok(const SsdParams *p) {
+  const void *gp = p->z ? p->gbuf : p->dout;
+  const int64_t g_ls = p->z ? (int64_t)p->nheads * p->headdim : p->dout_ls, g_hs = p->z ? p->headdim : p->dout_hs,
+                g_bs = p->z ? (int64_t)p->seqlen * p->nheads * p->headdim : p->dout_bs;
+  return p->dtype == MAMBA_BF16 && !p->det_scale && (p->headdim == 32 || p->headdim == 64) && gp && aligned(gp, 16) &&
+         aligned(p->x, 16) && !(g_ls % 8 || g_hs % 8 || g_bs % 8) && !(p->x_ls % 8 || p->x_hs % 8 || p->x_bs % 8) &&
+         g_ls < (1 << 21) && p->x_ls < (1 << 21);
+}
+static bool bmm_bwd_wide_ok(const SsdParams *p);
+// Inside ssd_combined_bwd the dCB tiles pass from the dCB stage to the bmm stage as bf16 where one workgroup owns each
+// tile and the bmm stage's operand is bf16 anyway (the stages on their own keep the fp32 tiles their interface names).
+static int64_t bmm_cumsum_workgroups(const SsdParams *p);
+static bool dcb_tiles_lp(const SsdParams *p) {
+  return dcb_rows_ok(p) && p->dCB && dcb_head_splits(p->nheads / p->ngroups) == 1 && bmm_bwd_wide_ok(p) &&
+         bmm_cumsum_workgroups(p) <= 0x7fffffff;  // (the one-launch form of the last two stages is the reader)
+}
+
+static int ssd_bwd_dcb_one(const SsdParams *p, mamba_stream_t stream, bool lp) {
   int rc = check_bwd(p);
   if (rc) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int nt = tiles(p->chunk_size);
   dim3 grid(nt * (nt + 1) / 2, p->nchunks, p->batch * p->ngroups * dcb_head_splits(p->nheads / p->ngroups));
-  // bf16 operands on 16-byte aligned rows of 32 or 64 values, no integer shadows: the head loop of its own
-  const void *gp = p->z ? p->gbuf : p->dout;
-  const int64_t g_ls = p->z ? (int64_t)p->nheads * p->headdim : p->dout_ls, g_hs = p->z ? p->headdim : p->dout_hs,
-                g_bs = p->z ? (int64_t)p->seqlen * p->nheads * p->headdim : p->dout_bs;
-  const bool fast = p->dtype == MAMBA_BF16 && !p->det_scale && (p->headdim == 32 || p->headdim == 64) &&
-                    aligned(gp, 16) && aligned(p->x, 16) && !(g_ls % 8 || g_hs % 8 || g_bs % 8) &&
-                    !(p->x_ls % 8 || p->x_hs % 8 || p->x_bs % 8) && g_ls < (1 << 21) && p->x_ls < (1 << 21);
-  if (fast) {
+  if (dcb_rows_ok(p)) {
+    const int lpi = lp ? 1 : 0;
     if (p->headdim == 64) {
-      if (p->CB) hipLaunchKernelGGL((bwd_dcb_kernel<bf16_t, false, false, false, 64>), grid, dim3(256), 0, s, *p);
-      else hipLaunchKernelGGL((bwd_dcb_kernel<bf16_t, false, false, true, 64>), grid, dim3(256), 0, s, *p);
+      if (p->CB) hipLaunchKernelGGL((bwd_dcb_rows_kernel<false, 64>), grid, dim3(256), 0, s, *p, lpi);
+      else hipLaunchKernelGGL((bwd_dcb_rows_kernel<true, 64>), grid, dim3(256), 0, s, *p, lpi);
     } else {
-      if (p->CB) hipLaunchKernelGGL((bwd_dcb_kernel<bf16_t, false, false, false, 32>), grid, dim3(256), 0, s, *p);
-      else hipLaunchKernelGGL((bwd_dcb_kernel<bf16_t, false, false, true, 32>), grid, dim3(256), 0, s, *p);
+      if (p->CB) hipLaunchKernelGGL((bwd_dcb_rows_kernel<false, 32>), grid, dim3(256), 0, s, *p, lpi);
+      else hipLaunchKernelGGL((bwd_dcb_rows_kernel<true, 32>), grid, dim3(256), 0, s, *p, lpi);
     }
     return launched();
   }
@@ -1693,6 +1724,8 @@ static int ssd_bwd_dcb_one(const SsdParams *p, mamba_stream_t stream) {
   SSD_DISPATCH_DET(bwd_dcb_kernel, grid)
   return launched();
 }
+
+static int ssd_bwd_dcb_stage(const SsdParams *p, mamba_stream_t stream) { return ssd_bwd_dcb_one(p, stream, false); }
 
 static int ssd_bmm_chunk_bwd_one(const SsdParams *p_in, mamba_stream_t stream) {
   int rc = check_bwd(p_in);
@@ -1764,7 +1797,11 @@ static int cast_sums(const SsdParams *p, mamba_stream_t stream) {
 
 // The last two stages as one launch where the bmm stage runs on wide tiles, else one after the other.  Either way
 // dB / dC (when the caller passes them) hold the finished sums in the operands' dtype afterwards.
-static int bmm_and_cumsum_bwd(const SsdParams *p, mamba_stream_t stream) {
+static int64_t bmm_cumsum_workgroups(const SsdParams *p) {
+  return (int64_t)tiles(p->chunk_size) * (p->dstate / WB) * p->nchunks * p->batch * p->ngroups +
+         (int64_t)p->nchunks * ((p->nheads + CSB_HT - 1) / CSB_HT) * p->batch;
+}
+static int bmm_and_cumsum_bwd(const SsdParams *p, mamba_stream_t stream, bool lp = false) {
   int rc = check_bwd(p);
   if (rc) return rc;
   const int64_t bmm_x = tiles(p->chunk_size) * (p->dstate / WB), bmm_y = p->nchunks, bmm_z = (int64_t)p->batch * p->ngroups;
@@ -1776,7 +1813,10 @@ static int bmm_and_cumsum_bwd(const SsdParams *p, mamba_stream_t stream) {
 #define SSD_LAUNCH_BMM_CS(T, SPLIT) \
   hipLaunchKernelGGL((bmm_cumsum_bwd_kernel<T, SPLIT>), grid, dim3(256), 0, s, *p, (int)n_bmm, (int)bmm_x, (int)bmm_y, (int)cs_x, (int)cs_y)
     switch (p->dtype) {
-      case MAMBA_BF16: SSD_LAUNCH_BMM_CS(bf16_t, false); break;
+      case MAMBA_BF16:
+        if (lp) hipLaunchKernelGGL((bmm_cumsum_bwd_kernel<bf16_t, false, true>), grid, dim3(256), 0, s, *p, (int)n_bmm, (int)bmm_x, (int)bmm_y, (int)cs_x, (int)cs_y);
+        else SSD_LAUNCH_BMM_CS(bf16_t, false);
+        break;
       case MAMBA_F16: SSD_LAUNCH_BMM_CS(f16_t, true); break;
       default: SSD_LAUNCH_BMM_CS(float, true); break;
     }
@@ -1848,8 +1888,9 @@ static int ssd_combined_bwd_one(const SsdParams *p, mamba_stream_t stream) {
   // written: in this order each finds them in the last-level cache
   if ((rc = ssd_bwd_dBC_state(p, stream))) return rc;
   if ((rc = ssd_bwd_dx(p, stream))) return rc;
-  if ((rc = ssd_bwd_dcb(p, stream))) return rc;
-  return bmm_and_cumsum_bwd(p, stream);
+  const bool lp = dcb_tiles_lp(p);
+  if ((rc = ssd_bwd_dcb_one(p, stream, lp))) return rc;
+  return bmm_and_cumsum_bwd(p, stream, lp);
 }
 
 extern "C" int ssd_bwd_overwrites(const SsdParams *p) {
@@ -1869,7 +1910,7 @@ extern "C" int ssd_bwd_dstates(const SsdParams *p, mamba_stream_t stream) { retu
 extern "C" int ssd_state_passing_bwd(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_state_passing_bwd_one); }
 extern "C" int ssd_bwd_dx(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_bwd_dx_one); }
 extern "C" int ssd_bwd_dBC_state(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_bwd_dBC_state_one); }
-extern "C" int ssd_bwd_dcb(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_bwd_dcb_one); }
+extern "C" int ssd_bwd_dcb(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_bwd_dcb_stage); }
 extern "C" int ssd_bmm_chunk_bwd(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_bmm_chunk_bwd_one); }
 extern "C" int ssd_chunk_cumsum_bwd(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_chunk_cumsum_bwd_one); }
 extern "C" int ssd_combined_bwd(const SsdParams *p, mamba_stream_t stream) { return ssd_sliced(p, stream, ssd_combined_bwd_one); }
