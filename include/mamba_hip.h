@@ -322,7 +322,9 @@ typedef struct SsdParams {
   float *ddA_cumsum;                    /* (b, H, c, Q), zero on entry */
   float *ddt_out;                       /* (b, H, c, Q), zero on entry */
   float *dCB;                           /* (b, c, G, Q, Q), zero on entry unless ssd_bwd_overwrites() has
-                                           SSD_OVERWRITES_DCB (one workgroup then owns each tile and stores it) */
+                                           SSD_OVERWRITES_DCB (one workgroup then owns each tile and stores it).  A
+                                           workspace: after ssd_bwd_dcb it holds fp32 tiles; what ssd_combined_bwd
+                                           leaves in it is unspecified (bf16 tiles where it hands them on as such) */
   float *dB32, *dC32;                   /* (b, L, G, N), zero on entry unless ssd_bwd_overwrites() has
                                            SSD_OVERWRITES_DBC (the first stage that touches them then stores them).  With
                                            dB / dC set the finished sums are only in dB / dC */

@@ -785,8 +785,16 @@ inline int heads_per_workgroup(const SsdParams &p) {
 
 // The fused chunk scan with two tiles per wave (ssd_scan_paired.hip), for problems that
 // ssd_chunk_scan_fwd_fused_supported accepts.
-bool ssd_scan_paired_serves(const SsdParams &p);
-int ssd_scan_paired_launch(const SsdParams &p, hipStream_t s);
+__attribute__((visibility("hidden"))) bool ssd_scan_paired_serves(const SsdParams &p);
+__attribute__((visibility("hidden"))) int ssd_scan_paired_launch(const SsdParams &p, hipStream_t s);
+// MAMBA_AMD_SSD_SCAN=single keeps the one-tile-per-wave kernel for every chunk size (for measurements).
+inline bool ssd_single_tile_only() {
+  static const bool v = [] {
+    const char *e = getenv("MAMBA_AMD_SSD_SCAN");
+    return e && e[0] == 's';
+  }();
+  return v;
+}
 
 // ------------------------------------------------------------------ batch slices
 // The kernels index (batch, head) pairs with one 16-bit grid coordinate.  A larger problem is served by the entry

@@ -317,17 +317,8 @@ __global__ __launch_bounds__(64 * QT) void chunk_scan_fwd_fused_kernel(const Ssd
   }
 }
 
-// MAMBA_AMD_SSD_SCAN=single keeps the one-tile-per-wave kernel for every chunk size (for measurements).
-bool single_tile_only() {
-  static const bool v = [] {
-    const char *e = getenv("MAMBA_AMD_SSD_SCAN");
-    return e && e[0] == 's';
-  }();
-  return v;
-}
-
 template <int PT, int NK> int launch_q(const SsdParams &p, hipStream_t s) {
-  if (ssd_scan_paired_serves(p) && !single_tile_only()) return ssd_scan_paired_launch(p, s);
+  if (ssd_scan_paired_serves(p) && !ssd_single_tile_only()) return ssd_scan_paired_launch(p, s);
   const int hb = heads_per_workgroup(p);
   dim3 grid(p.nheads / hb, p.nchunks, p.batch);
   switch (p.chunk_size) {
