@@ -1360,7 +1360,11 @@ template <typename T, bool SPLIT> __global__ __launch_bounds__(256) void bmm_chu
 // The same two products on 64 x 128 tiles (whole 128-state blocks, chunks of whole k steps, 16-byte aligned B / C
 // rows): half the workgroups, each k step of dCB staged once for twice the columns.
 // LP: dCB holds bf16 tiles (packed at the start of the buffer; see dcb_tile), which go to LDS as they are.
-template <typename T, bool SPLIT, bool LP = false> DEVI void bmm_chunk_bwd_wide_body(const SsdParams &p, int bx, int by, int bz) {
+// which: 0 = both products, one after the other; 1 = the dC product only; 2 = the dB product only (the two read
+// different operands and write different sums: dealt to two workgroups they halve a workgroup's serial work where
+// the tiles alone do not fill the chip).
+template <typename T, bool SPLIT, bool LP = false>
+DEVI void bmm_chunk_bwd_wide_body(const SsdParams &p, int bx, int by, int bz, int which = 0) {
   using CBT = std::conditional_t<LP, bf16_t, float>;
   __shared__ GemmLdsWide<SPLIT> lds;
   const int tid = threadIdx.x;
@@ -1392,7 +1396,7 @@ template <typename T, bool SPLIT, bool LP = false> DEVI void bmm_chunk_bwd_wide_
         }
       }
   };
-  {
+  if (which != 2) {
     // dC: A = dCB rows (l, k = s), k-contiguous fp32, s up to the end of the l tile; B = B rows (k = s, n)
     GemmAccWide acc;
     acc.zero();
@@ -1403,8 +1407,8 @@ template <typename T, bool SPLIT, bool LP = false> DEVI void bmm_chunk_bwd_wide_
     block_gemm_wide<SPLIT>(acc, lds, kend, sa, sb, tid);
     add_tile(acc, p.dC32, p.dC);
   }
-  lds_barrier();  // the first product's last operand reads end before the second one's first commit
-  {
+  if (which == 0) lds_barrier();  // the first product's last operand reads end before the second one's first commit
+  if (which != 1) {
     // dB: A = dCB^T (rows s, k = l from the s tile on), row-contiguous fp32; B = C rows (k = l, n)
     GemmAccWide acc;
     acc.zero();
@@ -1507,10 +1511,12 @@ __global__ __launch_bounds__(256) void chunk_cumsum_bwd_kernel(const SsdParams p
 // The last two stages read disjoint results of the stages before them (dCB; ddA_cumsum and ddt_out) and neither
 // fills the chip for long: one launch deals the wide-tile bmm workgroups first and the cumsum workgroups behind them.
 template <typename T, bool SPLIT, bool LP = false>
-__global__ __launch_bounds__(256) void bmm_cumsum_bwd_kernel(const SsdParams p, int n_bmm, int bmm_x, int bmm_y, int cs_x, int cs_y) {
+__global__ __launch_bounds__(256) void bmm_cumsum_bwd_kernel(const SsdParams p, int n_bmm, int bmm_x, int bmm_y, int cs_x, int cs_y, int split) {
   const int id = blockIdx.x;
   if (id < n_bmm) {
-    bmm_chunk_bwd_wide_body<T, SPLIT, LP>(p, id % bmm_x, (id / bmm_x) % bmm_y, id / (bmm_x * bmm_y));
+    // split: two workgroups per tile, one per product, neighbours in launch order (they share the dCB tile)
+    const int t = split ? id >> 1 : id, which = split ? 1 + (id & 1) : 0;
+    bmm_chunk_bwd_wide_body<T, SPLIT, LP>(p, t % bmm_x, (t / bmm_x) % bmm_y, t / (bmm_x * bmm_y), which);
   } else {
     const int k = id - n_bmm;
     chunk_cumsum_bwd_body(p, k % cs_x, (k / cs_x) % cs_y, k / (cs_x * cs_y));
@@ -1806,15 +1812,17 @@ static int bmm_and_cumsum_bwd(const SsdParams *p, mamba_stream_t stream, bool lp
   if (rc) return rc;
   const int64_t bmm_x = tiles(p->chunk_size) * (p->dstate / WB), bmm_y = p->nchunks, bmm_z = (int64_t)p->batch * p->ngroups;
   const int64_t cs_x = p->nchunks, cs_y = (p->nheads + CSB_HT - 1) / CSB_HT, cs_z = p->batch;
-  const int64_t n_bmm = bmm_x * bmm_y * bmm_z, total = n_bmm + cs_x * cs_y * cs_z;
+  // few tiles (fewer than four workgroups per CU): a workgroup per product instead of one per tile
+  const int split = bmm_x * bmm_y * bmm_z < 4 * (int64_t)cu_count() ? 1 : 0;
+  const int64_t n_bmm = bmm_x * bmm_y * bmm_z * (split ? 2 : 1), total = n_bmm + cs_x * cs_y * cs_z;
   if (bmm_bwd_wide_ok(p) && p->dCB && total <= 0x7fffffff) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     dim3 grid((unsigned)total);
 #define SSD_LAUNCH_BMM_CS(T, SPLIT) \
-  hipLaunchKernelGGL((bmm_cumsum_bwd_kernel<T, SPLIT>), grid, dim3(256), 0, s, *p, (int)n_bmm, (int)bmm_x, (int)bmm_y, (int)cs_x, (int)cs_y)
+  hipLaunchKernelGGL((bmm_cumsum_bwd_kernel<T, SPLIT>), grid, dim3(256), 0, s, *p, (int)n_bmm, (int)bmm_x, (int)bmm_y, (int)cs_x, (int)cs_y, split)
     switch (p->dtype) {
       case MAMBA_BF16:
-        if (lp) hipLaunchKernelGGL((bmm_cumsum_bwd_kernel<bf16_t, false, true>), grid, dim3(256), 0, s, *p, (int)n_bmm, (int)bmm_x, (int)bmm_y, (int)cs_x, (int)cs_y);
+        if (lp) hipLaunchKernelGGL((bmm_cumsum_bwd_kernel<bf16_t, false, true>), grid, dim3(256), 0, s, *p, (int)n_bmm, (int)bmm_x, (int)bmm_y, (int)cs_x, (int)cs_y, split);
         else SSD_LAUNCH_BMM_CS(bf16_t, false);
         break;
       case MAMBA_F16: SSD_LAUNCH_BMM_CS(f16_t, true); break;
