@@ -1076,11 +1076,69 @@ DEVI void dcb_tile(const SsdParams &p, DcbShared &sh, const Block3 blk, const in
   if constexpr (FORM_CB) {
     const T *Cl = static_cast<const T *>(p.C) + b * p.C_bs + g * p.C_gs + (int64_t)(t0 + lt * GB) * p.C_ls;
     const T *Bsr = static_cast<const T *>(p.B) + b * p.B_bs + g * p.B_gs + (int64_t)(t0 + st * GB) * p.B_ls;
-    block_gemm_pipe<SPLIT>(
-        acc, lds, 0, p.dstate,
-        KcStager<SPLIT, T>(lds.ah, lds.al, Cl, p.C_ls, qlim - lt * GB, p.dstate, nullptr, nullptr, rows_aligned16(Cl, p.C_ls), tid),
-        KcStager<SPLIT, T>(lds.bh, lds.bl, Bsr, p.B_ls, qlim - st * GB, p.dstate, nullptr, nullptr, rows_aligned16(Bsr, p.B_ls), tid),
-        tid);
+    bool formed = false;
+    if constexpr (FASTP != 0) {
+      // The tile of C B^T the way the heads' products are formed below: FASTP states at a time, a 64 x FASTP piece of
+      // the C rows and of the B rows from memory to LDS in 16-byte pieces, one barrier pair per piece.
+      if (p.dstate % FASTP == 0 && rows_aligned16(Cl, p.C_ls) && rows_aligned16(Bsr, p.B_ls) && p.C_ls < (1 << 21) && p.B_ls < (1 << 21)) {
+        constexpr int PITCH = FASTP + 8, NP = FASTP / 32, KS = FASTP / 32;
+        uint16_t *ca = reinterpret_cast<uint16_t *>(&lds), *ba = ca + GB * PITCH;
+        typedef const GLOBAL_AS char *gptr;
+        uint32_t coff[NP], boff[NP];
+        int loff[NP];
+#pragma unroll
+        for (int q = 0; q < NP; ++q) {
+          const int id = tid + q * 256, r = id / (FASTP / 8), c8 = id % (FASTP / 8);
+          // from the chunk's first row (rows past the end of the sequence re-read its last row: never negative)
+          coff[q] = (uint32_t)(min(lt * GB + r, qlim - 1) * (int)p.C_ls + c8 * 8) * 2u;
+          boff[q] = (uint32_t)(min(st * GB + r, qlim - 1) * (int)p.B_ls + c8 * 8) * 2u;
+          loff[q] = r * PITCH + c8 * 8;
+        }
+        u32x4 cr[NP], br[NP];
+        const T *Cc = static_cast<const T *>(p.C) + b * p.C_bs + g * p.C_gs + (int64_t)t0 * p.C_ls;
+        const T *Bc = static_cast<const T *>(p.B) + b * p.B_bs + g * p.B_gs + (int64_t)t0 * p.B_ls;
+        auto fetch_cb = [&](int n0) {
+#pragma unroll
+          for (int q = 0; q < NP; ++q) {
+            cr[q] = *(const GLOBAL_AS u32x4 *)((gptr)(Cc + n0) + coff[q]);
+            br[q] = *(const GLOBAL_AS u32x4 *)((gptr)(Bc + n0) + boff[q]);
+          }
+        };
+        fetch_cb(0);
+#pragma unroll 1
+        for (int n0 = 0; n0 < p.dstate; n0 += FASTP) {
+          lds_barrier();
+#pragma unroll
+          for (int q = 0; q < NP; ++q) {
+            *reinterpret_cast<u32x4 *>(ca + loff[q]) = cr[q];
+            *reinterpret_cast<u32x4 *>(ba + loff[q]) = br[q];
+          }
+          lds_barrier();
+          fetch_cb(min(n0 + FASTP, p.dstate - FASTP));
+#pragma unroll
+          for (int kk = 0; kk < KS; ++kk) {
+            bf16x8_t af[2], bfr[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+              af[t] = *reinterpret_cast<const bf16x8_t *>(&ca[(wm * 32 + t * 16 + i) * PITCH + kk * 32 + gq * 8]);
+              bfr[t] = *reinterpret_cast<const bf16x8_t *>(&ba[(wn * 32 + t * 16 + i) * PITCH + kk * 32 + gq * 8]);
+            }
+#pragma unroll
+            for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+              for (int tn = 0; tn < 2; ++tn)
+                acc.v[tm][tn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[tm], bfr[tn], acc.v[tm][tn], 0, 0, 0);
+          }
+        }
+        formed = true;
+      }
+    }
+    if (!formed)
+      block_gemm_pipe<SPLIT>(
+          acc, lds, 0, p.dstate,
+          KcStager<SPLIT, T>(lds.ah, lds.al, Cl, p.C_ls, qlim - lt * GB, p.dstate, nullptr, nullptr, rows_aligned16(Cl, p.C_ls), tid),
+          KcStager<SPLIT, T>(lds.bh, lds.bl, Bsr, p.B_ls, qlim - st * GB, p.dstate, nullptr, nullptr, rows_aligned16(Bsr, p.B_ls), tid),
+          tid);
   }
   const float *CB = FORM_CB ? nullptr : p.CB + (((int64_t)b * p.nchunks + c) * G + g) * Q * Q;
 #pragma unroll
