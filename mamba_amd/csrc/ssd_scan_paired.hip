@@ -472,7 +472,11 @@ template <int PT> int launch_n(const SsdParams &p, hipStream_t s) {
 
 // Whether the two-tiles-per-wave kernel serves a problem that ssd_chunk_scan_fwd_fused_supported accepts: chunk size
 // 256, where the one-tile form leaves the last wave eight blocks and the first one a single block.
-bool ssd_scan_paired_serves(const SsdParams &p) { return p.chunk_size == 256; }
+// (Its per-thread offsets are 32-bit byte offsets from a chunk's first row: rows up to 8 MB apart.)
+bool ssd_scan_paired_serves(const SsdParams &p) {
+  const int64_t lim = 1 << 22;
+  return p.chunk_size == 256 && p.x_ls < lim && p.out_ls < lim && (!p.z || p.z_ls < lim);
+}
 
 int ssd_scan_paired_launch(const SsdParams &p, hipStream_t s) {
   return p.headdim == 64 ? launch_n<4>(p, s) : launch_n<2>(p, s);
