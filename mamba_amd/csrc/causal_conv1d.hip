@@ -382,6 +382,189 @@ template <typename T, bool VEC> __global__ __launch_bounds__(256) void conv_cl_b
   }
 }
 
+// The backward pass with 4 channels per thread (rows whose 4-channel pieces are aligned: the VEC case).  The
+// 8-channel kernel above keeps two windows, the taps and their gradients for 8 channels in 232 registers, two waves
+// per SIMD; half the channels per thread is half the registers and twice the waves.  A thread's loads of the next
+// four steps are requested, and kept in their storage format, before it works on the current four: memory and the
+// SiLU re-computation overlap instead of alternating.
+template <typename T> struct Raw4 {
+  typedef u32x2 type;
+};
+template <> struct Raw4<float> {
+  typedef u32x4 type;
+};
+template <typename T> DEVI void unpack4(const typename Raw4<T>::type &r, float (&o)[4]);
+template <> DEVI void unpack4<bf16_t>(const u32x2 &r, float (&o)[4]) {
+  o[0] = bf16_lo(r.x); o[1] = bf16_hi(r.x); o[2] = bf16_lo(r.y); o[3] = bf16_hi(r.y);
+}
+template <> DEVI void unpack4<f16_t>(const u32x2 &r, float (&o)[4]) {
+  o[0] = f16_lo(r.x); o[1] = f16_hi(r.x); o[2] = f16_lo(r.y); o[3] = f16_hi(r.y);
+}
+template <> DEVI void unpack4<float>(const u32x4 &r, float (&o)[4]) {
+  const f32x4 f = __builtin_bit_cast(f32x4, r);  // (the whole vector: a bit cast of one element of it is not one)
+  o[0] = f.x; o[1] = f.y; o[2] = f.z; o[3] = f.w;
+}
+template <typename T> DEVI typename Raw4<T>::type pack4(const float (&v)[4]);
+template <> DEVI u32x2 pack4<bf16_t>(const float (&v)[4]) { return u32x2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])}; }
+template <> DEVI u32x2 pack4<f16_t>(const float (&v)[4]) { return u32x2{pack_f16(v[0], v[1]), pack_f16(v[2], v[3])}; }
+template <> DEVI u32x4 pack4<float>(const float (&v)[4]) {
+  const f32x4 f = {v[0], v[1], v[2], v[3]};
+  return __builtin_bit_cast(u32x4, f);
+}
+
+template <typename T> __global__ __launch_bounds__(256) void conv_cl_bwd4_kernel(const CausalConvParams p) {
+  typedef typename Raw4<T>::type raw_t;
+  constexpr int CPT = 4;
+  __shared__ float red[NRUN - 1][64][CPT * (MAXW + 1)];
+  const int L = p.seqlen, b = blockIdx.z;
+  const int cg = threadIdx.x & 63, run = threadIdx.x >> 6;
+  const int c0 = (blockIdx.x * 64 + cg) * CPT;
+  const bool live = c0 < p.dim;  // (dim is a multiple of 8 here: a thread has all of its 4 channels or none)
+  const int lbeg = (blockIdx.y * NRUN + run) * RUN, lend = min(lbeg + RUN, L);
+  float dw[CPT][MAXW], db[CPT];
+#pragma unroll
+  for (int e = 0; e < CPT; ++e) {
+    db[e] = 0.f;
+#pragma unroll
+    for (int k = 0; k < MAXW; ++k) dw[e][k] = 0.f;
+  }
+  if (live && lbeg < L) {
+    float w[CPT][MAXW], bias[CPT];
+#pragma unroll
+    for (int e = 0; e < CPT; ++e) load_taps(p, c0 + e, w[e], bias[e]);
+    const T *xb = static_cast<const T *>(p.x) + b * p.x_bs + c0;
+    const T *gb = static_cast<const T *>(p.dout) + b * p.dout_bs + c0;
+    T *dxb = static_cast<T *>(p.dx) + b * p.dx_bs + c0;
+    const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L : nullptr;
+    // Walk down from lend + 2: the first three steps only rebuild dpre at the positions after the run.
+    const int ltop = min(lend + 2, L - 1);
+    float xw[4][CPT];  // x at l - 3 .. l
+    float dp[4][CPT];  // dpre at l .. l + 3
+    int idx[7];        // sequence ids at l - 3 .. l + 3
+#pragma unroll
+    for (int j = 0; j < 7; ++j) {
+      const int l = ltop - 3 + j;
+      idx[j] = (seq && l >= 0 && l < L) ? seq[l] : -0x7fffffff;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int l = ltop - 3 + j;
+#pragma unroll
+      for (int e = 0; e < CPT; ++e) xw[j][e] = dp[j][e] = 0.f;
+      if (l >= 0) unpack4<T>(*reinterpret_cast<const raw_t *>(xb + (int64_t)l * p.x_ls), xw[j]);
+    }
+    // the loads of four steps (dout at l4 .. l4 - 3, x at l4 - 4 .. l4 - 7), one group ahead
+    raw_t gn[4], xn[4];
+    int idn[4];
+    auto fetch = [&](int l4) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int l = l4 - u;
+        gn[u] = *reinterpret_cast<const raw_t *>(gb + (int64_t)max(l, 0) * p.dout_ls);
+        xn[u] = *reinterpret_cast<const raw_t *>(xb + (int64_t)max(l - 4, 0) * p.x_ls);
+        idn[u] = (seq && l - 4 >= 0) ? seq[l - 4] : -0x7fffffff;
+      }
+    };
+    fetch(ltop);
+    for (int l4 = ltop; l4 >= lbeg; l4 -= 4) {
+      raw_t g4[4], x4[4];
+      int id4[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) g4[u] = gn[u], x4[u] = xn[u], id4[u] = idn[u];
+      fetch(l4 - 4);  // (below the run on the last turn: rows that exist, never used)
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int l = l4 - u;
+        if (l < lbeg) break;
+        float gu[CPT], xu[CPT];
+        unpack4<T>(g4[u], gu);
+        unpack4<T>(x4[u], xu);
+        // dpre at l
+        float dcur[CPT];
+#pragma unroll
+        for (int e = 0; e < CPT; ++e) {
+          float v = bias[e];
+#pragma unroll
+          for (int k = 0; k < MAXW; ++k) {
+            float t = xw[k][e];
+            if (seq && idx[k] != idx[3]) t = 0.f;
+            v = __builtin_fmaf(w[e][k], t, v);
+          }
+          dcur[e] = p.silu ? gu[e] * dsilu(v) : gu[e];
+        }
+#pragma unroll
+        for (int e = 0; e < CPT; ++e) {
+          dp[3][e] = dp[2][e];
+          dp[2][e] = dp[1][e];
+          dp[1][e] = dp[0][e];
+          dp[0][e] = dcur[e];
+        }
+        if (l < lend) {
+          float o[CPT];
+#pragma unroll
+          for (int e = 0; e < CPT; ++e) {
+            float v = 0.f;
+#pragma unroll
+            for (int k = 0; k < MAXW; ++k) {  // x[l] enters out[l + 3 - k] through tap k
+              float t = dp[3 - k][e];
+              if (seq && idx[3 + 3 - k] != idx[3]) t = 0.f;
+              v = __builtin_fmaf(w[e][k], t, v);
+            }
+            o[e] = v;
+#pragma unroll
+            for (int k = 0; k < MAXW; ++k) {
+              float t = xw[k][e];
+              if (seq && idx[k] != idx[3]) t = 0.f;
+              dw[e][k] = __builtin_fmaf(dcur[e], t, dw[e][k]);
+            }
+            db[e] += dcur[e];
+          }
+          *reinterpret_cast<raw_t *>(dxb + (int64_t)l * p.dx_ls) = pack4<T>(o);
+        }
+        // slide both windows one position down
+        const bool has = l - 4 >= 0;
+#pragma unroll
+        for (int e = 0; e < CPT; ++e) {
+          xw[3][e] = xw[2][e];
+          xw[2][e] = xw[1][e];
+          xw[1][e] = xw[0][e];
+          xw[0][e] = has ? xu[e] : 0.f;
+        }
+#pragma unroll
+        for (int j = 6; j > 0; --j) idx[j] = idx[j - 1];
+        idx[0] = id4[u];
+      }
+    }
+  }
+  // the four runs of a channel group are summed in LDS, then one atomic per channel and tap
+  if (run > 0) {
+#pragma unroll
+    for (int e = 0; e < CPT; ++e) {
+#pragma unroll
+      for (int k = 0; k < MAXW; ++k) red[run - 1][cg][e * (MAXW + 1) + k] = dw[e][k];
+      red[run - 1][cg][e * (MAXW + 1) + MAXW] = db[e];
+    }
+  }
+  __syncthreads();
+  if (run == 0 && live) {
+#pragma unroll
+    for (int e = 0; e < CPT; ++e) {
+#pragma unroll
+      for (int k = 0; k < MAXW; ++k) {
+        float v = dw[e][k];
+#pragma unroll
+        for (int r = 0; r < NRUN - 1; ++r) v += red[r][cg][e * (MAXW + 1) + k];
+        const int j = k - (MAXW - p.width);
+        if (j >= 0 && v != 0.f) conv_acc_add(p, p.dweight, p.det_dweight, (int64_t)(c0 + e) * p.width + j, v);
+      }
+      float v = db[e];
+#pragma unroll
+      for (int r = 0; r < NRUN - 1; ++r) v += red[r][cg][e * (MAXW + 1) + MAXW];
+      if (p.dbias && v != 0.f) conv_acc_add(p, p.dbias, p.det_dbias, c0 + e, v);
+    }
+  }
+}
+
 // ------------------------------------------------------------------ decode step
 // One thread per (batch entry, channel): with xn = [conv_state, x] along the position axis,
 //   out[t] = act(bias + sum_k w[k] xn[state_len + t - (W-1) + k]),  conv_state <- last state_len of xn
@@ -504,7 +687,7 @@ template <typename T> int launch_conv(const CausalConvParams &p, bool bwd, hipSt
     if (ygrid > 65535) return MAMBA_E_UNSUPPORTED;
     dim3 grid((p.dim + 511) / 512, ygrid, p.batch);
     if (bwd) {
-      if (vec) hipLaunchKernelGGL((conv_cl_bwd_kernel<T, true>), grid, dim3(256), 0, s, p);
+      if (vec) hipLaunchKernelGGL((conv_cl_bwd4_kernel<T>), dim3((p.dim + 255) / 256, ygrid, p.batch), dim3(256), 0, s, p);
       else hipLaunchKernelGGL((conv_cl_bwd_kernel<T, false>), grid, dim3(256), 0, s, p);
     } else {
       if (vec) hipLaunchKernelGGL((conv_cl_fwd_kernel<T, true>), grid, dim3(256), 0, s, p);
