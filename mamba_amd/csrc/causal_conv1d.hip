@@ -412,6 +412,83 @@ template <> DEVI u32x4 pack4<float>(const float (&v)[4]) {
   return __builtin_bit_cast(u32x4, f);
 }
 
+// The forward pass in the same form: 4 channels per thread, the next four positions requested before the current
+// four are worked on.
+template <typename T> __global__ __launch_bounds__(256) void conv_cl_fwd4_kernel(const CausalConvParams p) {
+  typedef typename Raw4<T>::type raw_t;
+  constexpr int CPT = 4;
+  const int L = p.seqlen, b = blockIdx.z;
+  const int cg = threadIdx.x & 63, run = threadIdx.x >> 6;
+  const int c0 = (blockIdx.x * 64 + cg) * CPT;
+  if (c0 >= p.dim) return;
+  const int lbeg = (blockIdx.y * NRUN + run) * RUN, lend = min(lbeg + RUN, L);
+  if (lbeg >= L) return;
+  float w[CPT][MAXW], bias[CPT];
+#pragma unroll
+  for (int e = 0; e < CPT; ++e) load_taps(p, c0 + e, w[e], bias[e]);
+  const T *xb = static_cast<const T *>(p.x) + b * p.x_bs + c0;
+  T *ob = static_cast<T *>(p.out) + b * p.out_bs + c0;
+  const int32_t *seq = p.seq_idx ? p.seq_idx + (int64_t)b * L : nullptr;
+  float xw[3][CPT];  // x at l - 3, l - 2, l - 1
+  int idw[3] = {-0x7fffffff, -0x7fffffff, -0x7fffffff};
+#pragma unroll
+  for (int j = 0; j < 3; ++j) {
+    const int l = lbeg - 3 + j;
+#pragma unroll
+    for (int e = 0; e < CPT; ++e) xw[j][e] = 0.f;
+    if (l >= 0) {
+      unpack4<T>(*reinterpret_cast<const raw_t *>(xb + (int64_t)l * p.x_ls), xw[j]);
+      if (seq) idw[j] = seq[l];
+    }
+  }
+  raw_t xn[4];
+  int idn[4];
+  auto fetch = [&](int l4) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int l = min(l4 + u, L - 1);
+      xn[u] = *reinterpret_cast<const raw_t *>(xb + (int64_t)l * p.x_ls);
+      idn[u] = seq ? seq[l] : 0;
+    }
+  };
+  fetch(lbeg);
+  for (int l4 = lbeg; l4 < lend; l4 += 4) {
+    raw_t x4[4];
+    int id4[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) x4[u] = xn[u], id4[u] = idn[u];
+    fetch(l4 + 4);  // (past the run on the last turn: rows that exist, never used)
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int l = l4 + u;
+      if (l >= lend) break;
+      float xin[CPT], o[CPT];
+      unpack4<T>(x4[u], xin);
+#pragma unroll
+      for (int e = 0; e < CPT; ++e) {
+        float v = __builtin_fmaf(w[e][3], xin[e], bias[e]);
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+          float t = xw[j][e];
+          if (seq && idw[j] != id4[u]) t = 0.f;
+          v = __builtin_fmaf(w[e][j], t, v);
+        }
+        o[e] = p.silu ? silu_f(v) : v;
+      }
+      *reinterpret_cast<raw_t *>(ob + (int64_t)l * p.out_ls) = pack4<T>(o);
+#pragma unroll
+      for (int e = 0; e < CPT; ++e) {
+        xw[0][e] = xw[1][e];
+        xw[1][e] = xw[2][e];
+        xw[2][e] = xin[e];
+      }
+      idw[0] = idw[1];
+      idw[1] = idw[2];
+      idw[2] = id4[u];
+    }
+  }
+}
+
 template <typename T> __global__ __launch_bounds__(256) void conv_cl_bwd4_kernel(const CausalConvParams p) {
   typedef typename Raw4<T>::type raw_t;
   constexpr int CPT = 4;
@@ -690,7 +767,7 @@ template <typename T> int launch_conv(const CausalConvParams &p, bool bwd, hipSt
       if (vec) hipLaunchKernelGGL((conv_cl_bwd4_kernel<T>), dim3((p.dim + 255) / 256, ygrid, p.batch), dim3(256), 0, s, p);
       else hipLaunchKernelGGL((conv_cl_bwd_kernel<T, false>), grid, dim3(256), 0, s, p);
     } else {
-      if (vec) hipLaunchKernelGGL((conv_cl_fwd_kernel<T, true>), grid, dim3(256), 0, s, p);
+      if (vec) hipLaunchKernelGGL((conv_cl_fwd4_kernel<T>), dim3((p.dim + 255) / 256, ygrid, p.batch), dim3(256), 0, s, p);
       else hipLaunchKernelGGL((conv_cl_fwd_kernel<T, false>), grid, dim3(256), 0, s, p);
     }
   }
