@@ -489,7 +489,9 @@ template <typename T> __global__ __launch_bounds__(256) void conv_cl_fwd4_kernel
   }
 }
 
-template <typename T> __global__ __launch_bounds__(256) void conv_cl_bwd4_kernel(const CausalConvParams p) {
+// RUN: positions per thread.  A run costs a 6-position warm-up, the taps, and its share of the reduction of the
+// filter gradients: long runs (128) where the grid still fills the chip, the forward kernel's 32 otherwise.
+template <typename T, int RUN> __global__ __launch_bounds__(256) void conv_cl_bwd4_kernel(const CausalConvParams p) {
   typedef typename Raw4<T>::type raw_t;
   constexpr int CPT = 4;
   __shared__ float red[NRUN - 1][64][CPT * (MAXW + 1)];
@@ -764,7 +766,14 @@ template <typename T> int launch_conv(const CausalConvParams &p, bool bwd, hipSt
     if (ygrid > 65535) return MAMBA_E_UNSUPPORTED;
     dim3 grid((p.dim + 511) / 512, ygrid, p.batch);
     if (bwd) {
-      if (vec) hipLaunchKernelGGL((conv_cl_bwd4_kernel<T>), dim3((p.dim + 255) / 256, ygrid, p.batch), dim3(256), 0, s, p);
+      if (vec) {
+        constexpr int LONG = 128;
+        const int xg = (p.dim + 255) / 256, ylong = (p.seqlen + LONG * NRUN - 1) / (LONG * NRUN);
+        if ((int64_t)xg * ylong * p.batch >= 2 * (int64_t)cu_count())
+          hipLaunchKernelGGL((conv_cl_bwd4_kernel<T, LONG>), dim3(xg, ylong, p.batch), dim3(256), 0, s, p);
+        else
+          hipLaunchKernelGGL((conv_cl_bwd4_kernel<T, RUN>), dim3(xg, ygrid, p.batch), dim3(256), 0, s, p);
+      }
       else hipLaunchKernelGGL((conv_cl_bwd_kernel<T, false>), grid, dim3(256), 0, s, p);
     } else {
       if (vec) hipLaunchKernelGGL((conv_cl_fwd4_kernel<T>), dim3((p.dim + 255) / 256, ygrid, p.batch), dim3(256), 0, s, p);

@@ -446,3 +446,15 @@ DEVI float wave_sum(float x) {
   for (int off = 32; off >= 1; off >>= 1) x += __shfl_xor(x, off, 64);
   return x;
 }
+
+// Compute units of the current device (256 when the query fails).
+inline int cu_count() {
+  static int cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    cached[dev] = (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) ? n : 256;
+  }
+  return cached[dev];
+}

@@ -754,17 +754,6 @@ __attribute__((visibility("hidden"))) bool ssd_bwd_dbc_fused_owns(const SsdParam
 // ---- host side of the kernels that work through the heads of a group in one workgroup
 inline bool aligned(const void *ptr, int a) { return (reinterpret_cast<uintptr_t>(ptr) % a) == 0; }
 
-inline int cu_count() {
-  static int cached[64] = {};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cached[dev] == 0) {
-    int n = 0;
-    cached[dev] = (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) ? n : 256;
-  }
-  return cached[dev];
-}
-
 // Heads per workgroup: a divisor of the heads per group, 20 at most.  One workgroup fills a CU, so the launch runs in
 // ceil(workgroups / CUs) rounds, each as long as what a workgroup pays once (launch, arguments, C rows, the first
 // head's exposed memory latency: measured at about 0.15 of a head's work) plus its heads; the divisor with the

@@ -72,6 +72,13 @@ def test_causal_conv1d_packed_sequences(dtype, channel_last):
     _case(2, 24, 100, 3, dtype, channel_last, seq_lens=[50, 50])
 
 
+@pytest.mark.parametrize("seq_lens", [None, [500, 574]])
+def test_causal_conv1d_channel_last_long_runs(seq_lens):
+    """A channel-last problem large enough for the backward kernel's long runs (128 positions per thread): a ragged
+    length, so that the last run of every row is cut short, with and without packed sequences."""
+    _case(11, 4096, 1074, 4, torch.bfloat16, True, seq_lens=seq_lens, seed=3)
+
+
 def test_causal_conv1d_strided_view():
     # the xBC slice of a wider projection output: channel-contiguous rows with a larger position stride
     from mamba_amd.ops.causal_conv1d import causal_conv1d_fn
