@@ -98,6 +98,7 @@ template <typename T> struct Pack8 {
   u32x4 w;
   DEVI void load(const T *p) { w = *reinterpret_cast<const u32x4 *>(p); }  // 16-byte aligned
   DEVI void load_global(const T *p) { w = *(const GLOBAL_AS u32x4 *)p; }
+  DEVI void store_global(T *p) const { *(GLOBAL_AS u32x4 *)p = w; }
   DEVI void zero() { w = u32x4{0, 0, 0, 0}; }
   DEVI void pack(const float (&v)[8]) {
     if constexpr (DT<T>::id == MAMBA_BF16) {
@@ -127,6 +128,10 @@ template <> struct Pack8<float> {
     const f32x4 a = *(const GLOBAL_AS f32x4 *)p, b = *(const GLOBAL_AS f32x4 *)(p + 4);
     v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
     v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  }
+  DEVI void store_global(float *p) const {
+    *(GLOBAL_AS f32x4 *)p = f32x4{v[0], v[1], v[2], v[3]};
+    *(GLOBAL_AS f32x4 *)(p + 4) = f32x4{v[4], v[5], v[6], v[7]};
   }
   DEVI void zero() {
 #pragma unroll

@@ -138,7 +138,12 @@ __global__ __launch_bounds__(TEAM < 256 ? 256 : TEAM) void norm_bwd_kernel(const
   const float inv_n = 1.f / (float)gs;
   const bool gate_after = zp && p.norm_before_gate, gate_before = zp && !p.norm_before_gate;
   RowBuf<T, VEC, K, TEAM> bx, bg, bz;
+  // the row's statistics are requested with the row, and before it: a load issued after the next row's would make
+  // its first use wait for that whole row as well
+  float mean_n = 0.f, rstd_n = 0.f;
   if (it.part < p.rows) {
+    if (!p.is_rms) mean_n = p.mean[(int64_t)it.part * ngroups + it.group];
+    rstd_n = p.rstd[(int64_t)it.part * ngroups + it.group];
     bx.fetch(xp + it.part * p.x_rs, it.col, gs);
     bg.fetch(gp + it.part * p.dy_rs, it.col, gs);
     if (zp) bz.fetch(zp + it.part * p.z_rs, it.col, gs);
@@ -149,14 +154,15 @@ __global__ __launch_bounds__(TEAM < 256 ? 256 : TEAM) void norm_bwd_kernel(const
     bg.get(g);
     if (zp) bz.get(z);
     const RowBuf<T, VEC, K, TEAM> xkeep = bx;  // x itself is needed again when the gate comes first
+    const float mean = mean_n, rstd = rstd_n;
+    float c1 = 0.f, c2 = 0.f;
     if (r + nparts < p.rows) {
+      if (!p.is_rms) mean_n = p.mean[(int64_t)(r + nparts) * ngroups + it.group];
+      rstd_n = p.rstd[(int64_t)(r + nparts) * ngroups + it.group];
       bx.fetch(xp + (r + nparts) * p.x_rs, it.col, gs);
       bg.fetch(gp + (r + nparts) * p.dy_rs, it.col, gs);
       if (zp) bz.fetch(zp + (r + nparts) * p.z_rs, it.col, gs);
     }
-    const float mean = p.is_rms ? 0.f : p.mean[(int64_t)r * ngroups + it.group];
-    const float rstd = p.rstd[(int64_t)r * ngroups + it.group];
-    float c1 = 0.f, c2 = 0.f;
     // after this loop: x = xhat (0 outside the group), g = w * dy', z = dz (gate after the norm) or
     // kept as z (gate before it, finished below)
 #pragma unroll
@@ -212,6 +218,208 @@ __global__ __launch_bounds__(TEAM < 256 ? 256 : TEAM) void norm_bwd_kernel(const
   if (p.db_part) store_row<float, VEC, K, TEAM>(p.db_part + (int64_t)it.part * p.dim + g0, it.col, gs, db);
 }
 
+// The forward pass in the same form as norm_bwd_wide_kernel (below): a part of the rows per workgroup, the next
+// row requested before the current one is used, no branch around a row's loads or stores.
+template <typename T, int TEAM, bool HAS_Z>
+__global__ __launch_bounds__(TEAM, 8) void norm_fwd_wide_kernel(const NormGatedParams p, int nparts) {
+  __shared__ float lds[2 * (TEAM / 64) * 2];
+  TeamSum<TEAM> ts(lds);
+  const int gs = p.group_size, ngroups = p.dim / gs, rows = p.rows;
+  const int group = blockIdx.x % ngroups, part = blockIdx.x / ngroups;
+  const int col = threadIdx.x * 8;
+  if (__builtin_amdgcn_readfirstlane(col) >= gs) {
+    for (int r = part; r < rows; r += nparts) {
+      float a = 0.f, b = 0.f;
+      if (!p.is_rms) ts.sum2(a, b);
+      a = b = 0.f;  // sum2 hands back the team's totals
+      ts.sum2(a, b);
+    }
+    return;
+  }
+  if (part >= rows) return;
+  const int64_t c0 = (int64_t)group * gs + col;
+  float w[8], b[8];
+  ld8<float>(p.weight + c0, w);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) b[e] = 0.f;
+  if (p.bias) ld8<float>(p.bias + c0, b);
+  const T *xp = static_cast<const T *>(p.x) + c0;
+  const T *zp = HAS_Z ? static_cast<const T *>(p.z) + c0 : xp;
+  T *op = static_cast<T *>(p.out) + c0;
+  const float inv_n = 1.f / (float)gs;
+  const bool gate_after = HAS_Z && p.norm_before_gate, gate_before = HAS_Z && !p.norm_before_gate;
+  const int last = part + (rows - 1 - part) / nparts * nparts;  // the last row of this part
+  Pack8<T> cx, cz;
+  cx.load_global(xp + (int64_t)part * p.x_rs);
+  if (HAS_Z) cz.load_global(zp + (int64_t)part * p.z_rs);
+  for (int r = part; r < rows; r += nparts) {
+    const int rn = min(r + nparts, last);
+    Pack8<T> nx, nz;
+    nx.load_global(xp + (int64_t)rn * p.x_rs);
+    if (HAS_Z) nz.load_global(zp + (int64_t)rn * p.z_rs);
+    float x[8], sz[8];
+    cx.unpack(x);
+    if (HAS_Z) {
+      cz.unpack(sz);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float sig;
+        sz[e] = silu_g(sz[e], sig);
+        if (gate_before) x[e] *= sz[e];
+      }
+    }
+    float mean = 0.f, dummy = 0.f;
+    if (!p.is_rms) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) mean += x[e];
+      ts.sum2(mean, dummy);
+      mean *= inv_n;
+    }
+    float var = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      x[e] -= mean;
+      var = __builtin_fmaf(x[e], x[e], var);
+    }
+    dummy = 0.f;
+    ts.sum2(var, dummy);
+    const float rstd = 1.f / sqrtf(var * inv_n + p.eps);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float y = __builtin_fmaf(x[e] * rstd, w[e], b[e]);
+      if (gate_after) y *= sz[e];
+      x[e] = y;
+    }
+    Pack8<T> o;
+    o.pack(x);
+    o.store_global(op + (int64_t)r * p.out_rs);
+    if (threadIdx.x == 0) {
+      if (p.mean) p.mean[(int64_t)r * ngroups + group] = mean;
+      p.rstd[(int64_t)r * ngroups + group] = rstd;
+    }
+    cx = nx;
+    if (HAS_Z) cz = nz;
+  }
+}
+
+// The backward pass for groups of 1024 < group_size <= 8192 channels in whole waves' worth (multiples of 512), rows
+// of 16-byte pieces: a workgroup of 256 / 512 / 1024 threads per (part, group), one piece per thread, so that a
+// wave holds either 512 channels or none (5120 channels on 1024 threads: 10 waves of 16 work, 6 only take part in the
+// team's sums, in a loop of their own).  No branch surrounds a load or a store of the loop over the rows: the row
+// after next's operands are requested (the last row again at the end) before the current row's are used, and the
+// waits the compiler places then name exactly the loads they need.  With the guarded accesses of norm_bwd_kernel
+// every wait was for everything in flight, the row just requested included, and a row cost its whole latency.
+template <typename T, int TEAM, bool HAS_Z>
+__global__ __launch_bounds__(TEAM) void norm_bwd_wide_kernel(const NormGatedParams p) {
+  __shared__ float lds[2 * (TEAM / 64) * 2];
+  TeamSum<TEAM> ts(lds);
+  const int gs = p.group_size, ngroups = p.dim / gs, nparts = p.nparts, rows = p.rows;
+  const int group = blockIdx.x % ngroups, part = blockIdx.x / ngroups;
+  const int col = threadIdx.x * 8;
+  if (__builtin_amdgcn_readfirstlane(col) >= gs) {
+    for (int r = part; r < rows; r += nparts) {
+      float a = 0.f, b = 0.f;
+      ts.sum2(a, b);
+    }
+    return;
+  }
+  const int64_t c0 = (int64_t)group * gs + col;
+  float w[8], b[8], dw[8], db[8];
+  ld8<float>(p.weight + c0, w);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) b[e] = dw[e] = db[e] = 0.f;
+  if (p.bias) ld8<float>(p.bias + c0, b);
+  const T *xp = static_cast<const T *>(p.x) + c0;
+  const T *gp = static_cast<const T *>(p.dy) + c0;
+  const T *zp = HAS_Z ? static_cast<const T *>(p.z) + c0 : xp;
+  T *dxp = static_cast<T *>(p.dx) + c0;
+  T *dzp = HAS_Z ? static_cast<T *>(p.dz) + c0 : dxp;
+  const float *rstdp = p.rstd + group, *meanp = p.is_rms ? rstdp : p.mean + group;
+  const float inv_n = 1.f / (float)gs;
+  const bool gate_after = HAS_Z && p.norm_before_gate, gate_before = HAS_Z && !p.norm_before_gate;
+  if (part < rows) {
+    const int last = part + (rows - 1 - part) / nparts * nparts;  // the last row of this part
+    Pack8<T> cx, cg, cz;
+    float cmean = *(const GLOBAL_AS float *)(meanp + (int64_t)part * ngroups);
+    float crstd = *(const GLOBAL_AS float *)(rstdp + (int64_t)part * ngroups);
+    cx.load_global(xp + (int64_t)part * p.x_rs);
+    cg.load_global(gp + (int64_t)part * p.dy_rs);
+    if (HAS_Z) cz.load_global(zp + (int64_t)part * p.z_rs);
+    for (int r = part; r < rows; r += nparts) {
+      const int rn = min(r + nparts, last);
+      Pack8<T> nx, ng, nz;
+      const float nmean = *(const GLOBAL_AS float *)(meanp + (int64_t)rn * ngroups);
+      const float nrstd = *(const GLOBAL_AS float *)(rstdp + (int64_t)rn * ngroups);
+      nx.load_global(xp + (int64_t)rn * p.x_rs);
+      ng.load_global(gp + (int64_t)rn * p.dy_rs);
+      if (HAS_Z) nz.load_global(zp + (int64_t)rn * p.z_rs);
+      float x[8], g[8], z[8], xr[8];
+      cx.unpack(x);
+      cg.unpack(g);
+      if (HAS_Z) cz.unpack(z);
+      const float mean = p.is_rms ? 0.f : cmean, rstd = crstd;
+      float c1 = 0.f, c2 = 0.f;
+      // after this loop: x = xhat, g = w * dy', z = dz (gate after the norm) or kept as z (gate before it), xr = x
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float xv = x[e], gv = g[e];
+        float sig = 0.f, sz = 1.f;
+        if (HAS_Z) sz = silu_g(z[e], sig);
+        xr[e] = xv;
+        if (gate_before) xv *= sz;
+        const float xhat = (xv - mean) * rstd;
+        if (gate_after) {
+          const float y = __builtin_fmaf(xhat, w[e], b[e]);
+          z[e] = gv * y * sig * (1.f + z[e] * (1.f - sig));
+          gv *= sz;
+        }
+        dw[e] = __builtin_fmaf(gv, xhat, dw[e]);
+        db[e] += gv;
+        const float wdy = w[e] * gv;
+        c1 = __builtin_fmaf(xhat, wdy, c1);
+        c2 += wdy;
+        x[e] = xhat;
+        g[e] = wdy;
+      }
+      ts.sum2(c1, c2);
+      c1 *= inv_n;
+      c2 = p.is_rms ? 0.f : c2 * inv_n;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float d = (g[e] - (x[e] * c1 + c2)) * rstd;
+        if (gate_before) {  // dz = dx' * x * dsilu(z), dx = dx' * silu(z)
+          float sig;
+          const float sz = silu_g(z[e], sig);
+          z[e] = d * xr[e] * sig * (1.f + z[e] * (1.f - sig));
+          x[e] = d * sz;
+        } else {
+          x[e] = d;
+        }
+      }
+      Pack8<T> ox, oz;
+      ox.pack(x);
+      ox.store_global(dxp + (int64_t)r * p.dx_rs);
+      if (HAS_Z) {
+        oz.pack(z);
+        oz.store_global(dzp + (int64_t)r * p.dz_rs);
+      }
+      cx = nx;
+      cg = ng;
+      if (HAS_Z) cz = nz;
+      cmean = nmean;
+      crstd = nrstd;
+    }
+  }
+  float *dwp = p.dw_part + (int64_t)part * p.dim + c0;
+  *(GLOBAL_AS f32x4 *)dwp = f32x4{dw[0], dw[1], dw[2], dw[3]};
+  *(GLOBAL_AS f32x4 *)(dwp + 4) = f32x4{dw[4], dw[5], dw[6], dw[7]};
+  if (p.db_part) {
+    float *dbp = p.db_part + (int64_t)part * p.dim + c0;
+    *(GLOBAL_AS f32x4 *)dbp = f32x4{db[0], db[1], db[2], db[3]};
+    *(GLOBAL_AS f32x4 *)(dbp + 4) = f32x4{db[4], db[5], db[6], db[7]};
+  }
+}
+
 template <typename T> bool vec_ok(const NormGatedParams &p, bool bwd) {
   constexpr int per16 = 16 / (int)sizeof(T);  // elements per 16 bytes: loads of 8 need 8-element alignment of fp32 too
   (void)per16;
@@ -240,7 +448,9 @@ template <typename T, int TEAM, int K, bool VEC> int launch(const NormGatedParam
 }
 
 // The smallest team that holds the group in at most two steps of 8 channels per thread (more steps
-// cost registers, hence waves in flight); only groups beyond 16384 channels take 3 or 4 steps.
+// cost registers, hence waves in flight); only groups beyond 16384 channels take 3 or 4 steps.  Above 4096
+// channels a whole workgroup of 1024 threads: one step up to 8192 channels keeps the backward pass at 114
+// registers (a team of 512 with two steps needs 240 and measured 10 % slower on 5120 channels).
 template <typename T, int TEAM, bool VEC> int pick_k(const NormGatedParams &p, bool bwd, hipStream_t st) {
   const int k = (p.group_size + TEAM * 8 - 1) / (TEAM * 8);
   if (k == 1) return launch<T, TEAM, 1, VEC>(p, bwd, st);
@@ -258,12 +468,34 @@ template <typename T, bool VEC> int pick_team(const NormGatedParams &p, bool bwd
   if (p.group_size <= 512) return pick_k<T, 32, VEC>(p, bwd, st);
   if (p.group_size <= 1024) return pick_k<T, 64, VEC>(p, bwd, st);
   if (p.group_size <= 4096) return pick_k<T, 256, VEC>(p, bwd, st);
-  if (p.group_size <= 8192) return pick_k<T, 512, VEC>(p, bwd, st);
   return pick_k<T, 1024, VEC>(p, bwd, st);
 }
 
+template <typename T, int TEAM> int launch_wide(const NormGatedParams &p, bool bwd, hipStream_t st) {
+  // forward: as many parts as workgroups the chip holds at once (2048 threads per CU), never more than rows
+  const int ngroups = p.dim / p.group_size;
+  const int nparts = bwd ? p.nparts : max(1, min(p.rows, cu_count() * (2048 / TEAM) / ngroups));
+  const int64_t wgs = (int64_t)ngroups * nparts;
+  if (wgs > 0x7fffffff) return MAMBA_E_UNSUPPORTED;
+  const dim3 grid((unsigned)wgs), block(TEAM);
+  if (bwd) {
+    if (p.z) norm_bwd_wide_kernel<T, TEAM, true><<<grid, block, 0, st>>>(p);
+    else norm_bwd_wide_kernel<T, TEAM, false><<<grid, block, 0, st>>>(p);
+  } else {
+    if (p.z) norm_fwd_wide_kernel<T, TEAM, true><<<grid, block, 0, st>>>(p, nparts);
+    else norm_fwd_wide_kernel<T, TEAM, false><<<grid, block, 0, st>>>(p, nparts);
+  }
+  return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
+}
+
 template <typename T> int run(const NormGatedParams &p, bool bwd, hipStream_t st) {
-  return vec_ok<T>(p, bwd) ? pick_team<T, true>(p, bwd, st) : pick_team<T, false>(p, bwd, st);
+  const bool vec = vec_ok<T>(p, bwd);
+  if (vec && p.rows > 0 && p.group_size > 1024 && p.group_size <= 8192 && p.group_size % 512 == 0) {
+    if (p.group_size <= 2048) return launch_wide<T, 256>(p, bwd, st);
+    if (p.group_size <= 4096) return launch_wide<T, 512>(p, bwd, st);
+    return launch_wide<T, 1024>(p, bwd, st);
+  }
+  return vec ? pick_team<T, true>(p, bwd, st) : pick_team<T, false>(p, bwd, st);
 }
 
 int check(const NormGatedParams *p, bool bwd) {

@@ -1637,6 +1637,7 @@ inline int tiles(int n) { return (n + GB - 1) / GB; }
 static int ssd_bwd_dz_one(const SsdParams *p, mamba_stream_t stream) {
   int rc = check_bwd(p);
   if (rc) return rc;
+  if (!p->z && !p->D) return MAMBA_OK;  // neither a gate nor a skip term: nothing to compute
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid((p->seqlen + 63) / 64, p->nheads, p->batch);
   switch (p->dtype) {
@@ -1698,19 +1699,27 @@ static int ssd_state_passing_bwd_one(const SsdParams *p, mamba_stream_t stream) 
   return launched();
 }
 
-static int ssd_bwd_dx_one(const SsdParams *p, mamba_stream_t stream) {
+// Without a gate dD is sum g x with g = dout, and the fused dx kernel holds both operands: where it runs and D is
+// one value per head it adds dD up on its way, and the pass of bwd_dz_kernel over dout and x is not needed.
+static bool dD_with_dx(const SsdParams *p) {
+  return !p->z && p->D && p->dD && !p->D_has_hdim && ssd_bwd_dx_fused_supported(p);
+}
+
+static int ssd_bwd_dx_with(const SsdParams *p, mamba_stream_t stream, bool sum_dD) {
   int rc = check_bwd(p);
   if (rc) return rc;
   if (p->dx_ls < (int64_t)p->headdim || p->dx_hs < (int64_t)p->headdim) return MAMBA_E_BADARG;  // strides not filled in
   hipStream_t s = static_cast<hipStream_t>(stream);
   // bf16 on the common shapes: the fused kernel, which forms C B^T itself (p->CB is not read); else the tiled one
-  rc = ssd_bwd_dx_fused_launch(p, s);
+  rc = ssd_bwd_dx_fused_launch(p, s, sum_dD);
   if (rc != MAMBA_E_UNSUPPORTED) return rc;
+  if (sum_dD) return MAMBA_E_UNSUPPORTED;  // dD_with_dx promised the fused kernel
   if (!p->CB) return MAMBA_E_BADARG;  // the tiled kernel reads C B^T
   dim3 grid(tiles(p->chunk_size) * tiles(p->headdim), p->nchunks, p->batch * p->nheads);
   SSD_DISPATCH_DET(bwd_dx_kernel, grid)
   return launched();
 }
+static int ssd_bwd_dx_one(const SsdParams *p, mamba_stream_t stream) { return ssd_bwd_dx_with(p, stream, false); }
 
 static int ssd_bwd_dBC_state_one(const SsdParams *p, mamba_stream_t stream) {
   int rc = check_bwd(p);
@@ -1915,7 +1924,7 @@ static int dz_and_dstates(const SsdParams *p, mamba_stream_t stream) {
     hipLaunchKernelGGL(bwd_dz_dstates_kernel<bf16_t>, grid, dim3(256), 0, s, *p);
     return launched();
   }
-  if ((rc = ssd_bwd_dz(p, stream))) return rc;
+  if (!dD_with_dx(p) && (rc = ssd_bwd_dz(p, stream))) return rc;
   return ssd_bwd_dstates(p, stream);
 }
 
@@ -1932,7 +1941,7 @@ static int ssd_combined_bwd_one(const SsdParams *p, mamba_stream_t stream) {
     if ((rc = dz_and_dstates(p, stream))) return rc;
     if ((rc = ssd_state_passing_bwd(p, stream))) return rc;
     if ((rc = ssd_bwd_dBC_state(p, stream))) return rc;
-    if ((rc = ssd_bwd_dx(p, stream))) return rc;
+    if ((rc = ssd_bwd_dx_with(p, stream, dD_with_dx(p)))) return rc;
     if ((rc = ssd_bwd_dcb(p, stream))) return rc;
     // every term of these sums is in: shadows -> the float buffers their readers take
     if ((rc = ssd_det_convert(p->det_dCB, p->dCB, cb, p->det_scale, stream))) return rc;
@@ -1953,7 +1962,7 @@ static int ssd_combined_bwd_one(const SsdParams *p, mamba_stream_t stream) {
   // dC reads the forward states, which the state-passing kernel has just read, and dB and dx the dstates it has just
   // written: in this order each finds them in the last-level cache
   if ((rc = ssd_bwd_dBC_state(p, stream))) return rc;
-  if ((rc = ssd_bwd_dx(p, stream))) return rc;
+  if ((rc = ssd_bwd_dx_with(p, stream, dD_with_dx(p)))) return rc;
   const bool lp = dcb_tiles_lp(p);
   if ((rc = ssd_bwd_dcb_one(p, stream, lp))) return rc;
   return bmm_and_cumsum_bwd(p, stream, lp);

@@ -744,7 +744,7 @@ template <int MODE = -1> DEVI void acc_add(float *dst, int64_t *shadow, int64_t 
 
 // The fused dx kernel (ssd_dx_fused.hip): launches it and returns MAMBA_OK, or returns MAMBA_E_UNSUPPORTED when it has
 // no kernel for the problem (the caller then runs the tiled bwd_dx_kernel).
-__attribute__((visibility("hidden"))) int ssd_bwd_dx_fused_launch(const SsdParams *p, hipStream_t stream);
+__attribute__((visibility("hidden"))) int ssd_bwd_dx_fused_launch(const SsdParams *p, hipStream_t stream, bool sum_dD);
 __attribute__((visibility("hidden"))) bool ssd_bwd_dx_fused_supported(const SsdParams *p);
 // The fused chunk-state dB / dC kernels (ssd_dbc_fused.hip), under the same convention (the caller then runs the
 // tiled bwd_d*_state kernels).

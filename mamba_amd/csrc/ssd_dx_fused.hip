@@ -23,7 +23,7 @@ DEVI f32x4 mfma_bf16(bf16x8_t a, bf16x8_t b, f32x4 c) {
 DEVI bf16x8_t ld_frag(const uint16_t *p) { return *reinterpret_cast<const bf16x8_t *>(p); }
 
 template <int PT, int NK, int QT, bool DET>
-__global__ __launch_bounds__(64 * QT) void bwd_dx_fused_kernel(const SsdParams p, const int hb) {
+__global__ __launch_bounds__(64 * QT) void bwd_dx_fused_kernel(const SsdParams p, const int hb, const int sum_dD) {
   constexpr int P = 16 * PT, N = 32 * NK, Q = 16 * QT, NSB = Q / 32, NT = 64 * QT;
   constexpr int BP = N + 8;   // LDS pitch of a C row / dS row (bf16): 16-byte aligned, bank-spread
   constexpr int XP = P + 16;  // LDS pitch of a g row (one position, P values + pad), as it lies in memory
@@ -43,6 +43,7 @@ __global__ __launch_bounds__(64 * QT) void bwd_dx_fused_kernel(const SsdParams p
   __shared__ __align__(16) float a2_s[Q], el_s[Q], dt_s[Q], w_s[Q];
   __shared__ int seq_s[Q];
   __shared__ __align__(16) float d_s[P];
+  __shared__ float dd_s[QT];  // sum_dD: each wave's <g, x> of the head over its 16 positions
 
   int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -263,6 +264,22 @@ __global__ __launch_bounds__(64 * QT) void bwd_dx_fused_kernel(const SsdParams p
       if (lane == 63) acc_add<DET ? 1 : 0>(p.ddA_cumsum, p.det_ddA_cumsum, row_off + Q - 1, e, dsc);
     }
 
+    // ---- dD[h] += sum_{s, p} g[s, p] x[s, p] (a D per head and no gate: g is dout): x in this lane's registers,
+    // g of the same column and rows from the head's rows in LDS (zero past the end of the sequence)
+    if (sum_dD) {
+      float dd = 0.f;
+#pragma unroll
+      for (int pt = 0; pt < PT; ++pt) {
+        const u32x2 gw = *reinterpret_cast<const u32x2 *>(&Gs[s_own * XP + pt * 16 + 4 * g]);
+        dd = __builtin_fmaf(bf16_lo(xl[pt].x), bf16_lo(gw.x), dd);
+        dd = __builtin_fmaf(bf16_hi(xl[pt].x), bf16_hi(gw.x), dd);
+        dd = __builtin_fmaf(bf16_lo(xl[pt].y), bf16_lo(gw.y), dd);
+        dd = __builtin_fmaf(bf16_hi(xl[pt].y), bf16_hi(gw.y), dd);
+      }
+      dd = wave_sum_to_last(dd);
+      if (lane == 63) dd_s[wave] = dd;
+    }
+
     // ---- each wave requests the next head's operands as it leaves the loop; the epilogue's patches lie over g and
     // the state gradient, so it starts once every wave has left
     if (hh + 1 < hb) load_head(h + per);
@@ -273,6 +290,12 @@ __global__ __launch_bounds__(64 * QT) void bwd_dx_fused_kernel(const SsdParams p
       ge[q] = *reinterpret_cast<const u32x4 *>(&Gs[(lt * 16 + rr) * XP + c8 * 8]);
     }
     lds_barrier();
+    if (sum_dD && tid == 0) {  // every wave's part is in (added in a fixed order); the next head's follow two barriers on
+      float dd = 0.f;
+#pragma unroll
+      for (int w = 0; w < QT; ++w) dd += dd_s[w];
+      acc_add<DET ? 1 : 0>(p.dD, p.det_dD, h, dd, dsc);
+    }
     {
       bf16_t *dxg = static_cast<bf16_t *>(p.dx) + b * p.dx_bs + h * p.dx_hs + (int64_t)(t0 + lt * 16) * p.dx_ls;
 #pragma unroll
@@ -304,26 +327,26 @@ __global__ __launch_bounds__(64 * QT) void bwd_dx_fused_kernel(const SsdParams p
   }
 }
 
-template <int PT, int NK, bool DET> int launch_q(const SsdParams &p, hipStream_t s) {
+template <int PT, int NK, bool DET> int launch_q(const SsdParams &p, hipStream_t s, int dd) {
   const int hb = heads_per_workgroup(p);
   dim3 grid(p.nheads / hb, p.nchunks, p.batch);
   switch (p.chunk_size) {
-    case 256: hipLaunchKernelGGL((bwd_dx_fused_kernel<PT, NK, 16, DET>), grid, dim3(1024), 0, s, p, hb); break;
-    case 128: hipLaunchKernelGGL((bwd_dx_fused_kernel<PT, NK, 8, DET>), grid, dim3(512), 0, s, p, hb); break;
-    case 64: hipLaunchKernelGGL((bwd_dx_fused_kernel<PT, NK, 4, DET>), grid, dim3(256), 0, s, p, hb); break;
+    case 256: hipLaunchKernelGGL((bwd_dx_fused_kernel<PT, NK, 16, DET>), grid, dim3(1024), 0, s, p, hb, dd); break;
+    case 128: hipLaunchKernelGGL((bwd_dx_fused_kernel<PT, NK, 8, DET>), grid, dim3(512), 0, s, p, hb, dd); break;
+    case 64: hipLaunchKernelGGL((bwd_dx_fused_kernel<PT, NK, 4, DET>), grid, dim3(256), 0, s, p, hb, dd); break;
     default: return MAMBA_E_UNSUPPORTED;
   }
   return hipGetLastError() == hipSuccess ? MAMBA_OK : MAMBA_E_LAUNCH;
 }
-template <int PT, bool DET> int launch_n(const SsdParams &p, hipStream_t s) {
+template <int PT, bool DET> int launch_n(const SsdParams &p, hipStream_t s, int dd) {
   switch (p.dstate) {
-    case 64: return launch_q<PT, 2, DET>(p, s);
-    case 128: return launch_q<PT, 4, DET>(p, s);
+    case 64: return launch_q<PT, 2, DET>(p, s, dd);
+    case 128: return launch_q<PT, 4, DET>(p, s, dd);
     default: return MAMBA_E_UNSUPPORTED;
   }
 }
-template <bool DET> int launch_p(const SsdParams &p, hipStream_t s) {
-  return p.headdim == 64 ? launch_n<4, DET>(p, s) : launch_n<2, DET>(p, s);
+template <bool DET> int launch_p(const SsdParams &p, hipStream_t s, int dd) {
+  return p.headdim == 64 ? launch_n<4, DET>(p, s, dd) : launch_n<2, DET>(p, s, dd);
 }
 
 bool supported(const SsdParams *p) {
@@ -349,7 +372,10 @@ bool supported(const SsdParams *p) {
 
 bool ssd_bwd_dx_fused_supported(const SsdParams *p) { return supported(p); }
 
-int ssd_bwd_dx_fused_launch(const SsdParams *p, hipStream_t stream) {
+// With sum_dD the launch also adds the heads' <g, x> to dD (one D per head): the whole of dD where no gate stands
+// between dout and g.
+int ssd_bwd_dx_fused_launch(const SsdParams *p, hipStream_t stream, bool sum_dD) {
   if (!supported(p)) return MAMBA_E_UNSUPPORTED;
-  return p->det_scale ? launch_p<true>(*p, stream) : launch_p<false>(*p, stream);
+  if (sum_dD && (!p->dD || p->D_has_hdim || (p->det_scale && !p->det_dD))) return MAMBA_E_BADARG;
+  return p->det_scale ? launch_p<true>(*p, stream, sum_dD) : launch_p<false>(*p, stream, sum_dD);
 }

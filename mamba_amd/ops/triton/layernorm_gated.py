@@ -116,7 +116,10 @@ def _layer_norm_bwd(dy, x, weight, bias, eps, mean, rstd, z=None, group_size=Non
     if M == 0:
         return dx, torch.zeros_like(weight), torch.zeros_like(bias) if bias is not None else None, dz
     # enough teams of threads to fill the GPU several times over, never more parts than rows
-    team = next((t for t in (8, 16, 32, 64, 256, 512) if group_size <= 16 * t), 1024)
+    # the threads per (row, group) norm_gated.hip picks
+    team = next((t for t in (8, 16, 32, 64, 256) if group_size <= 16 * t), 1024)
+    if group_size % 512 == 0 and 2048 < group_size <= 4096:
+        team = 512
     nparts = max(1, min(M, (4096 * 64 // team) // ngroups, 65536))
     nb = 2 if bias is not None else 1
     parts = torch.empty(nb, nparts, N, dtype=torch.float32, device=x.device)

@@ -157,6 +157,22 @@ def test_ssd_backward_deterministic_mode(deterministic_mode, headdim, dstate, ng
         assert torch.allclose(default[k].float(), runs[0][k].float(), rtol=1e-2, atol=1e-2), k
 
 
+def test_ssd_backward_deterministic_mode_no_gate(deterministic_mode):
+    """Without z, dD (one value per head) is summed by the dx kernel: the same requirement."""
+    from mamba_amd.utils.determinism import set_deterministic_mode
+    names = ("x", "dt", "A", "B", "C", "D", "dt_bias")
+    t = {k: (v.cuda() if torch.is_tensor(v) else v)
+         for k, v in ssd_inputs(2, 640, 16, 64, 128, 1, torch.bfloat16, 9, has_z=False).items()}
+    runs = [_ssd_grads(t, names, 256, return_final_states=True) for _ in range(3)]
+    for r in runs[1:]:
+        for k in runs[0]:
+            assert torch.equal(runs[0][k], r[k]), k
+    set_deterministic_mode(False)
+    default = _ssd_grads(t, names, 256, return_final_states=True)
+    for k in default:
+        assert torch.allclose(default[k].float(), runs[0][k].float(), rtol=1e-2, atol=1e-2), k
+
+
 def test_ssd_backward_deterministic_mode_packed(deterministic_mode):
     names = ("x", "dt", "A", "B", "C", "D", "z", "dt_bias", "initial_states")
     t = {k: (v.cuda() if torch.is_tensor(v) else v)

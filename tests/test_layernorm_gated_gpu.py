@@ -102,6 +102,19 @@ def test_many_rows_bf16():
     _case(3000, 1024, 128, torch.bfloat16, norm_before_gate=False, seed=7)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_wide_groups_walk_rows(dtype):
+    """Groups of 1024 < n <= 8192 channels in multiples of 512 take the kernels that keep one 16-byte piece per thread
+    and request the next row ahead: several rows per workgroup, waves past the end of the group (5120 channels on
+    1024 threads, 3072 on 512) that only join the sums, two groups per row, LayerNorm's two sums, no gate, padded
+    rows."""
+    _case(1500, 5120, None, dtype, has_z=False, seed=9)
+    _case(1300, 4096, 2048, dtype, norm_before_gate=True, is_rms=False, has_bias=True, row_pad=8, seed=10)
+    _case(2100, 3072, None, dtype, norm_before_gate=False, seed=11)
+    _case(1100, 8192, None, dtype, norm_before_gate=False, is_rms=False, has_bias=True, seed=12)
+    _case(3, 1536, None, dtype, seed=13)
+
+
 def test_module_and_empty():
     from mamba_amd.ops.triton.layernorm_gated import RMSNorm, LayerNorm, rmsnorm_fn, rms_norm_ref
     m = RMSNorm(256, eps=1e-5, group_size=64, norm_before_gate=False, device="cuda", dtype=torch.float32)
