@@ -791,7 +791,7 @@ def bench_block(dev, steps, warmup):
         "higher_is_better": True, "dtype": "bf16 in/out, fp32 accumulation", "data": "synthetic",
         "config": {"workload": f"Mamba-2 block body fwd+bwd: batch {batch}, seqlen {L}, {H} heads x {P}, d_state {N}, "
                                f"{G} group, chunk {Q}, conv width {W}, gated RMSNorm, out_proj to {dm}"},
-        "roofline": vs_measured_copy({"bound": "hbm", "kernel": "norm_fwd_kernel", "achieved": nbytes / norm_ms / 1e6,
+        "roofline": vs_measured_copy({"bound": "hbm", "kernel": "norm_fwd_wide_kernel", "achieved": nbytes / norm_ms / 1e6,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / norm_ms / 1e6 / HBM_PEAK_GBS,
                      "traffic": None, "kernel_ms": norm_ms, "algorithmic_bytes": nbytes}, dev)})
 
