@@ -345,7 +345,7 @@ typedef struct SsdParams {
    * (the matrix products take only the bf16 part of them anyway; the reference hands them on in the operands' dtype
    * too, ssd_combined.py:384-386 out_dtype=C.dtype and :455-466 dstates_dtype=x.dtype), both (b, c, H, P, N):
    *   states_lp   written by ssd_state_passing_fwd (`states` then keeps the chunks' own states and is not needed
-   *               afterwards), read by the scan, ssd_chunk_state_varlen, ssd_state_passing_bwd and ssd_bwd_dBC_state;
+   *               afterwards) or by ssd_chunk_state_passing_fwd (`states` is then not written at all), read by the scan, ssd_chunk_state_varlen, ssd_state_passing_bwd and ssd_bwd_dBC_state;
    *   dstates_lp  takes the place of `dstates` in every backward stage.
    * Required (non-NULL) for MAMBA_BF16, ignored for the other dtypes, which keep the fp32 `states` (in place) and
    * `dstates`. */
@@ -363,7 +363,14 @@ int ssd_chunk_scan_fwd(const SsdParams *p, mamba_stream_t stream);
  * ssd_chunk_scan_fwd_fused_supported returns 1 when it applies. */
 int ssd_chunk_scan_fwd_fused_supported(const SsdParams *p);
 int ssd_chunk_scan_fwd_fused(const SsdParams *p, mamba_stream_t stream);
-/* cumsum, chunk_state, state_passing, then the fused scan when supported, else bmm + chunk_scan */
+/* ssd_chunk_state_fwd and ssd_state_passing_fwd in one launch, for MAMBA_BF16 with headdim 64, dstate 128,
+ * chunk_size 128 / 256, seqlen a multiple of chunk_size and 16-byte aligned x / B rows; MAMBA_E_UNSUPPORTED otherwise.
+ * One workgroup per (batch, head) walks the sequence: writes states_lp (the state entering each chunk) and
+ * final_states, reads dt_out / dA_cumsum, initial_states, seq_idx; `states` is not touched.  Replaces the pair
+ * _chunk_state_fwd + _state_passing_fwd of mamba_ssm/ops/triton/ssd_combined.py:375-382. */
+int ssd_chunk_state_passing_fwd(const SsdParams *p, mamba_stream_t stream);
+/* cumsum; chunk_state + state_passing (in one launch, ssd_chunk_state_passing_fwd, where it applies and batch x heads
+ * is at least three quarters of the compute units); then the fused scan when supported, else bmm + chunk_scan */
 int ssd_combined_fwd(const SsdParams *p, mamba_stream_t stream);
 /* Packed batch (p->batch == 1): the state after the last position of each of the nseq sequences
  * [cu_seqlens[i], cu_seqlens[i+1]) into varlen_states (nseq, H, P, N) fp32.  Needs dt_out,

@@ -157,7 +157,8 @@ def load():
     lib.mamba1_scan_fwd_noalloc.restype = ctypes.c_int
     lib.mamba_hip_init.argtypes = []
     lib.mamba_hip_init.restype = ctypes.c_int
-    for name in ("ssd_chunk_cumsum_fwd", "ssd_chunk_state_fwd", "ssd_state_passing_fwd", "ssd_bmm_chunk_fwd",
+    for name in ("ssd_chunk_cumsum_fwd", "ssd_chunk_state_fwd", "ssd_state_passing_fwd", "ssd_chunk_state_passing_fwd",
+                 "ssd_bmm_chunk_fwd",
                  "ssd_chunk_scan_fwd", "ssd_combined_fwd", "ssd_chunk_scan_fwd_fused", "ssd_bwd_dz", "ssd_bwd_dstates",
                  "ssd_state_passing_bwd", "ssd_bwd_dx", "ssd_bwd_dBC_state", "ssd_bwd_dcb", "ssd_bmm_chunk_bwd",
                  "ssd_chunk_cumsum_bwd", "ssd_combined_bwd"):

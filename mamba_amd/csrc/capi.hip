@@ -148,7 +148,7 @@ int mamba1_scan_tile(bool a_complex);  // mamba1_scan.hip
 
 extern "C" int mamba_hip_query(int what) {
   switch (what) {
-    case MAMBA_Q_ABI_VERSION: return 13;
+    case MAMBA_Q_ABI_VERSION: return 14;
     case MAMBA_Q_SCAN_TILE: return mamba1_scan_tile(false);
     case MAMBA_Q_SCAN_TILE_COMPLEX: return mamba1_scan_tile(true);
     case MAMBA_Q_MAX_DSTATE: return 256;

@@ -342,6 +342,7 @@ template <bool SPLIT, typename S, int ROWS> struct WideTrStager {
   const float *kscale;
   int t;
   Pack8<S> q[NT];
+  WideTrStager() = default;  // for arrays of stagers, each assigned from a constructed one
   DEVI WideTrStager(uint16_t *hi_, uint16_t *lo_, const S *base_, int64_t kstride_, int rows_valid_, const float *kscale_, int t_)
       : hi(hi_), lo(lo_), base(base_), kstride(kstride_), rows_valid(rows_valid_), kscale(kscale_), t(t_) {}
   static constexpr bool transposed = true;
@@ -437,6 +438,30 @@ template <bool SPLIT, bool RING = false, typename SA, typename SB>
 DEVI void block_gemm_wide(GemmAccWide &acc, GemmLdsWide<SPLIT> &s, int k_end, SA &sa, SB &sb, int tid) {
   block_gemm_wide<SPLIT, RING>(acc, s, k_end, sa, sb, tid, [](int) {});
 }
+// One k step of that product by itself, for callers that keep more than two pairs of stagers in flight: commits
+// the operands fa / fb hold (requested earlier for step k0), requests those of step k_next into the same registers,
+// multiplies.
+template <typename SA, typename SB>
+DEVI void wide_step(GemmAccWide &acc, GemmLdsWide<false> &s, int k0, SA &fa, SB &fb, int k_next, int tid) {
+  const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+  const int i = lane & 15, g = lane >> 4;
+  lds_barrier();
+  fa.template commit<true>(k0);
+  fb.template commit<true>(k0);
+  lds_barrier();
+  fa.template fetch<true>(k_next);
+  fb.template fetch<true>(k_next);
+  bf16x8_t a[2], b[4];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) a[t] = load_frag<SA::transposed>(s.ah, wm * 32 + t * 16, i, g);
+#pragma unroll
+  for (int t = 0; t < 4; ++t) b[t] = load_frag_tr<WLD>(s.bh, wn * 64 + t * 16, i, g);
+#pragma unroll
+  for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+    for (int tn = 0; tn < 4; ++tn)
+      acc.v[tm][tn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[tm], b[tn], acc.v[tm][tn], 0, 0, 0);
+}
 
 // dtype in which the states carried between chunks, and their gradients, pass between kernels: bf16 next to bf16
 // operands (the matrix products only take that part of them), fp32 otherwise.
@@ -458,7 +483,7 @@ DEVI void st_carried(bf16_t *p, float v) { st1<bf16_t>(p, v); }
 // stores 16 contiguous bytes and eight lanes a whole line (single elements straight from the accumulator layout
 // are 32-byte runs in bf16: the state-gradient product measured 83 us with those, 71 us with these).  All 256 threads must call (one barrier: the last
 // step's operand reads end before the patches overwrite them).
-template <bool SPLIT, typename D>
+template <bool SPLIT, typename D, bool GUARD = true>
 DEVI void store_wide_rows(const GemmAccWide &acc, GemmLdsWide<SPLIT> &s, D *dst, int64_t ld, int rows_valid, int tid) {
   constexpr int CP = 128 / sizeof(D);      // columns per pass
   constexpr int PP = CP + 16 / sizeof(D);  // patch pitch in elements (144 bytes)
@@ -483,7 +508,8 @@ DEVI void store_wide_rows(const GemmAccWide &acc, GemmLdsWide<SPLIT> &s, D *dst,
         const int row = q * 8 + (lane >> 3), piece = lane & 7;
         const u32x4 v = *reinterpret_cast<const u32x4 *>(patch + row * PP + piece * E16);
         const int m = wm * 32 + tm * 16 + row;
-        if (m < rows_valid) *reinterpret_cast<u32x4 *>(dst + (int64_t)m * ld + wn * 64 + pass * CP + piece * E16) = v;
+        // (GUARD false: all 64 rows exist, and no branch stands between the caller's loads in flight and its waits)
+        if (!GUARD || m < rows_valid) *(GLOBAL_AS u32x4 *)(dst + (int64_t)m * ld + wn * 64 + pass * CP + piece * E16) = v;
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();

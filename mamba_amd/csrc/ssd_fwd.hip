@@ -342,6 +342,117 @@ template <int W, typename CT, bool TABLE> __global__ __launch_bounds__(256) void
   s.store(p.final_states + ((int64_t)b * H + h) * PN + e);
 }
 
+// ------------------------------------------- chunk states and state passing in one pass
+// bf16, headdim 64, 128 states, chunks of Q = 32 R positions that tile the sequence: one workgroup per (batch, head)
+// walks the sequence once.  Per chunk it forms the chunk's own state (the product of chunk_state_fwd_wide_kernel,
+// a 64 x 128 tile, k = position), writes the state ENTERING the chunk (bf16, what the scan and the backward pass
+// read) and carries H <- decay_c H + S_c in fp32 registers; after the last chunk H is final_states.  The fp32
+// per-chunk states never exist in memory (configuration 2: 168 MB written and read again), and the recurrence over
+// the chunks costs no pass of its own.  With few workgroups (batch x heads) the loads must be deep instead: R pairs
+// of stagers hold the operands of the next R steps -- one chunk ahead -- and no branch surrounds a load or a store
+// of the walk, so each step waits for exactly its own operands.  The per-position weights w_s of chunk c + 1 are
+// computed while chunk c is multiplied (two tables in LDS), the per-chunk decay factors once at the start.
+constexpr int CSP_MAX_CHUNKS = 2048;
+template <int R, bool HAS_SEQ> __global__ __launch_bounds__(256) void chunk_state_passing_fwd_kernel(const SsdParams p) {
+  using T = bf16_t;
+  using SA = WideTrStager<false, T, 64>;
+  using SB = WideTrStager<false, T, WB>;
+  constexpr int Q = 32 * R, P = 64, N = WB;
+  static_assert(Q <= 256, "one table entry per thread");
+  __shared__ GemmLdsWide<false> lds;
+  __shared__ float wtab[2][Q];
+  __shared__ float dec[CSP_MAX_CHUNKS];
+  const int tid = threadIdx.x;
+  const int L = p.seqlen, H = p.nheads, nc = p.nchunks;
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int g = h / (H / p.ngroups);
+  const float *dA = p.dA_cumsum + ((int64_t)b * H + h) * nc * Q;
+  const float *dtp = p.dt_out + ((int64_t)b * H + h) * nc * Q;
+  const int32_t *seq = HAS_SEQ ? p.seq_idx + (int64_t)b * L : nullptr;
+  for (int c = tid; c < nc; c += 256) {  // carried-state factor of chunk c: 0 across a sequence boundary
+    float scale = fast_exp(dA[c * Q + Q - 1]);
+    if (HAS_SEQ) {
+      const int seq_new = seq[(c + 1) * Q - 1], seq_prev = c > 0 ? seq[c * Q - 1] : 0;
+      if (seq_new != seq_prev) scale = 0.f;
+    }
+    dec[c] = scale;
+  }
+  // w_s = dt_s exp(a_last - a_s) for the positions of the chunk's last sequence, else 0; entry min(tid, Q - 1)
+  const int ts = min(tid, Q - 1);
+  float t_a, t_alast, t_dt;
+  int t_sid = 0, t_slast = 0;
+  auto table_request = [&](int c) {
+    t_a = *(const GLOBAL_AS float *)(dA + c * Q + ts);
+    t_alast = *(const GLOBAL_AS float *)(dA + c * Q + Q - 1);
+    t_dt = *(const GLOBAL_AS float *)(dtp + c * Q + ts);
+    if (HAS_SEQ) {
+      t_sid = *(const GLOBAL_AS int32_t *)(seq + c * Q + ts);
+      t_slast = *(const GLOBAL_AS int32_t *)(seq + c * Q + Q - 1);
+    }
+  };
+  auto table_write = [&](int c) {
+    float v = fast_exp(fminf(t_alast - t_a, 0.f)) * t_dt;
+    if (HAS_SEQ && !(t_slast >= 0 && t_sid == t_slast)) v = 0.f;
+    if (tid < Q) wtab[c & 1][tid] = v;
+  };
+  table_request(0);
+  table_write(0);
+
+  // H in the accumulator layout: rows 32 wm + 16 tm + 4 g + r, columns 64 wn + 16 tn + i
+  GemmAccWide Hs, acc;
+  Hs.zero();
+  if (p.initial_states) {
+    const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1, i = lane & 15, gq = lane >> 4;
+    const float *init = p.initial_states + ((int64_t)b * H + h) * P * N;
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < 4; ++tn)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          Hs.v[tm][tn][r] = init[(wm * 32 + tm * 16 + gq * 4 + r) * N + wn * 64 + tn * 16 + i];
+  }
+
+  const T *xa = static_cast<const T *>(p.x) + b * p.x_bs + h * p.x_hs;
+  const T *Ba = static_cast<const T *>(p.B) + b * p.B_bs + g * p.B_gs;
+  SA sa[R];
+  SB sb[R];
+  {
+    const SA sa0(lds.ah, lds.al, xa, p.x_ls, P, nullptr, tid);
+    const SB sb0(lds.bh, lds.bl, Ba, p.B_ls, WB, wtab[0], tid);
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      sa[j] = sa0;
+      sb[j] = sb0;
+      sa[j].template fetch<true>(j * GK);
+      sb[j].template fetch<true>(j * GK);
+      // the requests leave in the order the walk consumes them: the waits in the loop are counted from the order
+      // on either way into it, and the compiler would otherwise issue these independent loads last pair first
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  bf16_t *carried = static_cast<bf16_t *>(p.states_lp) + ((int64_t)b * nc * H + h) * P * N;
+#pragma unroll 1
+  for (int c = 0; c < nc; ++c) {
+    table_request(min(c + 1, nc - 1));
+    acc.zero();
+    const float *ks = &wtab[c & 1][0] - c * Q;  // the stagers index their weights by position in the sequence
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      sb[j].kscale = ks;
+      wide_step(acc, lds, c * Q + j * GK, sa[j], sb[j], min(c * Q + (j + R) * GK, L - GK), tid);
+    }
+    table_write(c + 1);  // read from the next step's first barrier on; last read two chunks ago
+    store_wide_rows<false, bf16_t, false>(Hs, lds, carried + (int64_t)c * H * P * N, N, P, tid);
+    const float d = dec[c];
+#pragma unroll
+    for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < 4; ++tn) Hs.v[tm][tn] = Hs.v[tm][tn] * d + acc.v[tm][tn];
+  }
+  store_wide_rows<false, float, false>(Hs, lds, p.final_states + ((int64_t)b * H + h) * P * N, N, P, tid);
+}
+
 // ------------------------------------------------------------- chunk_scan
 // out[l, p] = exp(a_l) [seq_l == seq before the chunk] sum_n C[l, n] Hc[p, n]
 //           + sum_{s <= l} CB[l, s] exp(a_l - a_s) dt_s x[s, p] + D x[l, p];   out *= silu(z)
@@ -556,11 +667,49 @@ static int ssd_chunk_scan_fwd_one(const SsdParams *p, mamba_stream_t stream) {
   return launched();
 }
 
+// chunk_state + state_passing in one launch (chunk_state_passing_fwd_kernel): the shapes it is compiled for, whole
+// chunks, 16-byte aligned operands.
+static bool chunk_state_passing_shapes_ok(const SsdParams *p) {
+  auto al16 = [](const void *q) { return q && (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+  return p->dtype == MAMBA_BF16 && p->headdim == 64 && p->dstate == WB && (p->chunk_size == 256 || p->chunk_size == 128) &&
+         p->seqlen % p->chunk_size == 0 && p->nchunks <= CSP_MAX_CHUNKS && p->nheads <= 65535 && p->batch <= 65535 &&
+         al16(p->states_lp) && al16(p->final_states) && p->dt_out && p->dA_cumsum &&
+         wide_operand_ok(p->x, p->dtype, p->x_bs, p->x_ls, p->x_hs) && wide_operand_ok(p->B, p->dtype, p->B_bs, p->B_ls, p->B_gs);
+}
+// The combined forward pass takes it where there are enough (batch, head) pairs for one workgroup each to keep the
+// chip busy: a workgroup takes ~3.7 us per chunk of 256 whatever their number (its LDS traffic per k step is that of
+// chunk_state_fwd_wide_kernel, and that is what bounds both), the two-kernel path ~24 ns per (batch, head, chunk).
+// Measured at 80 heads x 4096 positions, walk / two kernels: batch 2 61 / 51 us, batch 3 65 / 95, batch 4 95 / 128
+// (320 workgroups on 256 CUs: a quarter of the CUs do double duty), batch 8 169 / 252; one packed row of 64 heads x
+// 32768 positions 436 / 195.
+static bool chunk_state_passing_pays(const SsdParams *p) {
+  return chunk_state_passing_shapes_ok(p) && (int64_t)p->batch * p->nheads >= cu_count() * 3 / 4;
+}
+extern "C" int ssd_chunk_state_passing_fwd(const SsdParams *p, mamba_stream_t stream) {
+  int rc = check(p);
+  if (rc) return rc;
+  if (!chunk_state_passing_shapes_ok(p)) return MAMBA_E_UNSUPPORTED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  dim3 grid(p->nheads, p->batch);
+  if (p->chunk_size == 256) {
+    if (p->seq_idx) hipLaunchKernelGGL((chunk_state_passing_fwd_kernel<8, true>), grid, dim3(256), 0, s, *p);
+    else hipLaunchKernelGGL((chunk_state_passing_fwd_kernel<8, false>), grid, dim3(256), 0, s, *p);
+  } else {
+    if (p->seq_idx) hipLaunchKernelGGL((chunk_state_passing_fwd_kernel<4, true>), grid, dim3(256), 0, s, *p);
+    else hipLaunchKernelGGL((chunk_state_passing_fwd_kernel<4, false>), grid, dim3(256), 0, s, *p);
+  }
+  return launched();
+}
+
 static int ssd_combined_fwd_one(const SsdParams *p, mamba_stream_t stream) {
   int rc;
   if ((rc = ssd_chunk_cumsum_fwd(p, stream))) return rc;
-  if ((rc = ssd_chunk_state_fwd(p, stream))) return rc;
-  if ((rc = ssd_state_passing_fwd(p, stream))) return rc;
+  if (check(p) == MAMBA_OK && chunk_state_passing_pays(p)) {
+    if ((rc = ssd_chunk_state_passing_fwd(p, stream))) return rc;
+  } else {
+    if ((rc = ssd_chunk_state_fwd(p, stream))) return rc;
+    if ((rc = ssd_state_passing_fwd(p, stream))) return rc;
+  }
   if (ssd_chunk_scan_fwd_fused_supported(p)) return ssd_chunk_scan_fwd_fused(p, stream);
   if ((rc = ssd_bmm_chunk_fwd(p, stream))) return rc;
   return ssd_chunk_scan_fwd(p, stream);
